@@ -1,0 +1,19 @@
+"""Table builders and index helpers (the tensor-product subset of ``equitorch.utils``)."""
+from ._indices import expand_left, extract_batch_segments, extract_scatter_indices, sort_by_column_key
+from ._random import rand_spherical_xyz
+from ._structs import (
+    create_tp_info,
+    generate_fully_connected_tp_paths,
+    prepare_so3,
+    sparse_product_info,
+    sparse_product_infos,
+    sparse_scale_info,
+    sparse_scale_infos,
+    tp_infos,
+)
+
+__all__ = [
+    "rand_spherical_xyz", "expand_left", "extract_batch_segments", "sort_by_column_key",
+    "extract_scatter_indices", "sparse_scale_info", "sparse_scale_infos", "sparse_product_info",
+    "sparse_product_infos", "generate_fully_connected_tp_paths", "tp_infos",
+]
