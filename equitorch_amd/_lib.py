@@ -1,0 +1,101 @@
+"""ctypes binding of ``libcgtp.so`` (the C ABI declared in ``include/cgtp.h``).
+
+The library is built in-tree by ``python -m equitorch_amd.csrc.build``; importing this module without it
+raises — there is no fallback implementation.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libcgtp.so")
+
+F32, F64, BF16, F16 = 0, 1, 2, 3
+OPERAND_NONE, OPERAND_VEC, OPERAND_SCALAR = 0, 1, 2
+_DTYPES = {torch.float32: F32, torch.float64: F64, torch.bfloat16: BF16, torch.float16: F16}
+
+
+class CgtpError(RuntimeError):
+    pass
+
+
+class Operand(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("rows", C.c_void_p), ("row_stride", C.c_int64),
+                ("idx_stride", C.c_int64), ("kind", C.c_int32), ("_pad", C.c_int32)]
+
+
+class TriArgs(C.Structure):
+    _fields_ = [("a", Operand), ("b", Operand), ("w", Operand),
+                ("coef", C.c_void_p), ("idx", C.c_void_p), ("seg", C.c_void_p),
+                ("n_out", C.c_int32), ("nnz", C.c_int32),
+                ("out", C.c_void_p), ("workspace", C.c_void_p), ("n_rows", C.c_int64),
+                ("C", C.c_int32), ("dtype", C.c_int32), ("reduce_c", C.c_int32), ("reduce_rows", C.c_int32)]
+
+
+class UvuArgs(C.Structure):
+    _fields_ = [("cfg", C.c_int32), ("dtype", C.c_int32), ("C", C.c_int32), ("w_shared", C.c_int32),
+                ("n_rows", C.c_int64), ("n_x_rows", C.c_int64), ("n_seg", C.c_int64),
+                ("ptr", C.c_void_p), ("perm", C.c_void_p), ("gather", C.c_void_p),
+                ("x", C.c_void_p), ("y", C.c_void_p), ("w", C.c_void_p),
+                ("out", C.c_void_p),
+                ("grad_out", C.c_void_p), ("grad_x", C.c_void_p), ("grad_y", C.c_void_p),
+                ("grad_w", C.c_void_p), ("workspace", C.c_void_p)]
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        raise ImportError(
+            f"{_LIB_PATH} is missing: build the HIP library first (python -m equitorch_amd.csrc.build). "
+            "equitorch_amd has no non-HIP implementation of its operators.")
+    lib = C.CDLL(_LIB_PATH)
+    lib.cgtp_status_string.restype = C.c_char_p
+    lib.cgtp_status_string.argtypes = [C.c_int]
+    lib.cgtp_version.restype = C.c_int
+    lib.cgtp_tri_workspace_bytes.restype = C.c_int64
+    lib.cgtp_tri_workspace_bytes.argtypes = [C.POINTER(TriArgs)]
+    lib.cgtp_tri_validate.argtypes = [C.POINTER(TriArgs)]
+    lib.cgtp_tri_contract.argtypes = [C.POINTER(TriArgs), C.c_void_p]
+    lib.cgtp_segment_sum.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                     C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p]
+    lib.cgtp_uvu_num_configs.restype = C.c_int
+    lib.cgtp_uvu_find.argtypes = [C.c_uint64]
+    lib.cgtp_uvu_describe.restype = C.c_uint64
+    lib.cgtp_uvu_describe.argtypes = [C.c_int, C.POINTER(C.c_int32)]
+    lib.cgtp_uvu_validate.argtypes = [C.POINTER(UvuArgs), C.c_int]
+    lib.cgtp_uvu_bwd_workspace_bytes.restype = C.c_int64
+    lib.cgtp_uvu_bwd_workspace_bytes.argtypes = [C.POINTER(UvuArgs)]
+    lib.cgtp_uvu_fwd.argtypes = [C.POINTER(UvuArgs), C.c_void_p]
+    lib.cgtp_uvu_bwd.argtypes = [C.POINTER(UvuArgs), C.c_void_p]
+    return lib
+
+
+lib = _load()
+
+
+def check(status: int, what: str = "cgtp"):
+    if status != 0:
+        raise CgtpError(f"{what}: {lib.cgtp_status_string(status).decode()} (status {status})")
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise CgtpError(f"unsupported dtype {dtype}") from None
+
+
+def stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def ptr(t) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def require_gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise CgtpError("equitorch_amd operators run on the GPU only (got a CPU tensor); "
+                            "there is no CPU implementation in this package")

@@ -1,0 +1,34 @@
+// Host-side declarations shared by the translation units of libcgtp.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "cgtp.h"
+
+namespace cgtp {
+
+// The 160 KB of LDS of a gfx950 compute unit; a workgroup may claim all of it.
+constexpr int64_t kLdsBytes = 160 * 1024;
+
+inline int elem_size(int dtype) {
+  switch (dtype) {
+    case CGTP_F32: return 4;
+    case CGTP_F64: return 8;
+    case CGTP_BF16: return 2;
+    case CGTP_F16: return 2;
+    default: return 0;
+  }
+}
+
+// out[i] = sum_k ws[k * n + i], accumulated in double in a fixed order (deterministic).
+template <typename T>
+__global__ void partial_sum_kernel(const T* __restrict__ ws, T* __restrict__ out, int64_t n_part, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  double s = 0.0;
+  for (int64_t k = 0; k < n_part; ++k) s += (double)ws[k * n + i];
+  out[i] = (T)s;
+}
+
+}  // namespace cgtp

@@ -1,0 +1,258 @@
+// Generic sparse trilinear contraction with the coefficient / index table staged in LDS, and the indexed
+// scale-segment reduction.  These kernels take the tables at run time, so they serve every irreps
+// configuration (and the reference's table-driven operator API); configurations with a compiled-in table
+// use the kernels of uvu_kernels.hip instead.
+#include "cgtp_device.h"
+#include "cgtp_host.h"
+
+namespace cgtp {
+
+template <typename T>
+struct OperandDev {
+  const T* data;
+  const int64_t* rows;
+  int64_t row_stride, idx_stride;
+  int kind;
+};
+
+template <typename T>
+struct TriDev {
+  OperandDev<T> a, b, w;
+  const T* coef;
+  const uint32_t* idx;
+  const int32_t* seg;
+  int n_out, nnz;
+  T* out;  // or the workspace when rows are reduced
+  int64_t n_rows;
+  int C, reduce_rows;
+};
+
+template <typename T>
+__device__ __forceinline__ const T* row_ptr(const OperandDev<T>& o, int64_t r) {
+  const int64_t rr = o.rows ? o.rows[r] : r;
+  return o.data + rr * o.row_stride;
+}
+
+// One wavefront per row (or per contiguous share of the rows when they are reduced); lanes run over
+// channels.  The table is read from LDS with wave-uniform addresses (broadcast reads).
+template <typename T, bool REDUCE_C>
+__global__ void __launch_bounds__(256) tri_kernel(const TriDev<T> a, int64_t n_waves) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  T* s_coef = reinterpret_cast<T*>(smem);
+  uint32_t* s_idx = reinterpret_cast<uint32_t*>(s_coef + a.nnz);
+  int32_t* s_seg = reinterpret_cast<int32_t*>(s_idx + a.nnz);
+  for (int t = threadIdx.x; t < a.nnz; t += blockDim.x) {
+    s_coef[t] = a.coef ? a.coef[t] : T(1);
+    s_idx[t] = a.idx[t];
+  }
+  for (int t = threadIdx.x; t <= a.n_out; t += blockDim.x) s_seg[t] = a.seg[t];
+  __syncthreads();
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (wave >= n_waves) return;
+
+  const int64_t per = a.reduce_rows ? (a.n_rows + n_waves - 1) / n_waves : 1;
+  const int64_t stride = a.reduce_rows ? n_waves * per : n_waves;  // reduce_rows: a single pass
+  for (int64_t r0 = wave * per; r0 < a.n_rows; r0 += stride) {
+    const int64_t r1 = (r0 + per < a.n_rows) ? r0 + per : a.n_rows;
+    const int64_t orow = a.reduce_rows ? wave : r0;
+    for (int o = 0; o < a.n_out; ++o) {
+      const int tb = s_seg[o], te = s_seg[o + 1];
+      T total = T(0);
+      for (int cb = 0; cb < a.C; cb += kWave) {
+        const int c = cb + lane;
+        const bool ok = c < a.C;
+        T acc = T(0);
+        if (ok) {
+          for (int64_t r = r0; r < r1; ++r) {
+            const T* pa = a.a.kind ? row_ptr(a.a, r) + (a.a.kind == CGTP_OPERAND_VEC ? c : 0) : nullptr;
+            const T* pb = a.b.kind ? row_ptr(a.b, r) + (a.b.kind == CGTP_OPERAND_VEC ? c : 0) : nullptr;
+            const T* pw = a.w.kind ? row_ptr(a.w, r) + (a.w.kind == CGTP_OPERAND_VEC ? c : 0) : nullptr;
+            for (int t = tb; t < te; ++t) {
+              const uint32_t u = s_idx[t];
+              T v = s_coef[t];
+              if (pa) v *= pa[(int64_t)(u & 1023u) * a.a.idx_stride];
+              if (pb) v *= pb[(int64_t)((u >> 10) & 1023u) * a.b.idx_stride];
+              if (pw) v *= pw[(int64_t)(u >> 20) * a.w.idx_stride];
+              acc += v;
+            }
+          }
+        }
+        if constexpr (REDUCE_C) {
+          total += acc;
+        } else {
+          if (ok) a.out[(orow * a.n_out + o) * a.C + c] = acc;
+        }
+      }
+      if constexpr (REDUCE_C) {
+        total = group_sum(total, kWave);
+        if (lane == 0) a.out[orow * a.n_out + o] = total;
+      }
+    }
+    if (a.reduce_rows) break;
+  }
+}
+
+// out[n, m, c] = sum_{t in [seg[m], seg[m+1])} scale[t] * in[n, index[t], c]; one wavefront per (n, m).
+template <typename T, int V>
+__global__ void __launch_bounds__(256) segment_sum_kernel(const T* __restrict__ in, const T* __restrict__ scale,
+                                                          const int64_t* __restrict__ index,
+                                                          const int64_t* __restrict__ seg, T* __restrict__ out,
+                                                          int64_t n_batch, int64_t in_size, int64_t out_size,
+                                                          int64_t C) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (wave >= n_batch * out_size) return;
+  const int64_t n = wave / out_size, m = wave % out_size;
+  const int64_t tb = seg ? seg[m] : m, te = seg ? seg[m + 1] : m + 1;
+  const T* base = in + n * in_size * C;
+  T* dst = out + (n * out_size + m) * C;
+  for (int64_t c = (int64_t)lane * V; c < C; c += kWave * V) {
+    T acc[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) acc[v] = T(0);
+    for (int64_t t = tb; t < te; ++t) {
+      const int64_t i = index ? index[t] : t;
+      const T s = scale ? scale[t] : T(1);
+      T x[V];
+      load_vec<T, V>(x, base + i * C + c);
+      fmav<T, V>(acc, s, x);
+    }
+    store_vec<T, V>(dst + c, acc);
+  }
+}
+
+static int tri_check(const cgtp_tri_args* a, int64_t* lds_bytes, int64_t* n_waves) {
+  if (!a) return CGTP_ERR_NULL;
+  if (a->dtype != CGTP_F32 && a->dtype != CGTP_F64) return CGTP_ERR_DTYPE;
+  if (a->n_out < 0 || a->nnz < 0 || a->n_rows < 0 || a->C <= 0) return CGTP_ERR_SHAPE;
+  if (!a->idx || !a->seg || !a->out) return CGTP_ERR_NULL;
+  const cgtp_operand* ops[3] = {&a->a, &a->b, &a->w};
+  for (const cgtp_operand* o : ops) {
+    if (o->kind < CGTP_OPERAND_NONE || o->kind > CGTP_OPERAND_SCALAR) return CGTP_ERR_SHAPE;
+    if (o->kind != CGTP_OPERAND_NONE && !o->data) return CGTP_ERR_NULL;
+    if (o->kind != CGTP_OPERAND_NONE && (o->row_stride < 0 || o->idx_stride < 0)) return CGTP_ERR_SHAPE;
+  }
+  const int64_t esz = elem_size(a->dtype);
+  *lds_bytes = (int64_t)a->nnz * (esz + 4) + ((int64_t)a->n_out + 1) * 4;
+  if (*lds_bytes > kLdsBytes) return CGTP_ERR_LDS;
+  if (a->reduce_rows) {
+    int64_t nw = a->n_rows < 1024 ? a->n_rows : 1024;
+    *n_waves = nw;
+    if (nw > 0 && !a->workspace) return CGTP_ERR_WORKSPACE;
+  } else {
+    *n_waves = a->n_rows < 16384 ? a->n_rows : 16384;
+  }
+  return CGTP_OK;
+}
+
+template <typename T>
+static OperandDev<T> op_dev(const cgtp_operand& o) {
+  return OperandDev<T>{(const T*)o.data, o.rows, o.row_stride, o.idx_stride, o.kind};
+}
+
+template <typename T>
+static int tri_launch(const cgtp_tri_args* a, int64_t lds, int64_t n_waves, hipStream_t stream) {
+  const int64_t per_row = (int64_t)a->n_out * (a->reduce_c ? 1 : a->C);
+  if (n_waves == 0) {
+    if (a->reduce_rows && per_row > 0) (void)hipMemsetAsync(a->out, 0, sizeof(T) * per_row, stream);
+    return CGTP_OK;
+  }
+  TriDev<T> d;
+  d.a = op_dev<T>(a->a); d.b = op_dev<T>(a->b); d.w = op_dev<T>(a->w);
+  d.coef = (const T*)a->coef; d.idx = a->idx; d.seg = a->seg;
+  d.n_out = a->n_out; d.nnz = a->nnz;
+  d.out = a->reduce_rows ? (T*)a->workspace : (T*)a->out;
+  d.n_rows = a->n_rows; d.C = a->C; d.reduce_rows = a->reduce_rows;
+  auto kern = a->reduce_c ? tri_kernel<T, true> : tri_kernel<T, false>;
+  if (lds > 48 * 1024) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return CGTP_ERR_LDS;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)((n_waves + 3) / 4)), dim3(256), (size_t)lds, stream, d, n_waves);
+  if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
+  if (a->reduce_rows) {
+    hipLaunchKernelGGL(partial_sum_kernel<T>, dim3((unsigned)((per_row + 255) / 256)), dim3(256), 0, stream,
+                       (const T*)a->workspace, (T*)a->out, n_waves, per_row);
+    if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
+  }
+  return CGTP_OK;
+}
+
+template <typename T, int VW>
+static int segsum_launch(const void* in, const void* scale, const int64_t* index, const int64_t* seg, void* out,
+                         int64_t n_batch, int64_t in_size, int64_t out_size, int64_t C, hipStream_t stream) {
+  const int64_t waves = n_batch * out_size;
+  if (waves == 0) return CGTP_OK;
+  const bool vec = (C % VW) == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+  dim3 grid((unsigned)((waves + 3) / 4));
+  if (vec)
+    hipLaunchKernelGGL((segment_sum_kernel<T, VW>), grid, dim3(256), 0, stream, (const T*)in, (const T*)scale,
+                       index, seg, (T*)out, n_batch, in_size, out_size, C);
+  else
+    hipLaunchKernelGGL((segment_sum_kernel<T, 1>), grid, dim3(256), 0, stream, (const T*)in, (const T*)scale,
+                       index, seg, (T*)out, n_batch, in_size, out_size, C);
+  return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
+}
+
+}  // namespace cgtp
+
+using namespace cgtp;
+
+extern "C" {
+
+const char* cgtp_status_string(int status) {
+  switch (status) {
+    case CGTP_OK: return "ok";
+    case CGTP_ERR_NULL: return "required pointer is NULL";
+    case CGTP_ERR_SHAPE: return "invalid or inconsistent extent";
+    case CGTP_ERR_ALIGN: return "pointer or stride misaligned";
+    case CGTP_ERR_DTYPE: return "unsupported element type";
+    case CGTP_ERR_CONFIG: return "unknown specialised-table id";
+    case CGTP_ERR_LDS: return "table does not fit in LDS";
+    case CGTP_ERR_LAUNCH: return "kernel launch failed";
+    case CGTP_ERR_WORKSPACE: return "workspace missing or too small";
+    default: return "unknown status";
+  }
+}
+
+int cgtp_version(void) { return 1; }
+
+int cgtp_tri_validate(const cgtp_tri_args* args) {
+  int64_t lds = 0, nw = 0;
+  cgtp_tri_args tmp;
+  if (args) {
+    tmp = *args;
+    if (tmp.reduce_rows && !tmp.workspace) tmp.workspace = (void*)&tmp;  // size query / dry run
+    return tri_check(&tmp, &lds, &nw);
+  }
+  return CGTP_ERR_NULL;
+}
+
+int64_t cgtp_tri_workspace_bytes(const cgtp_tri_args* a) {
+  if (!a || !a->reduce_rows) return 0;
+  const int64_t nw = a->n_rows < 1024 ? a->n_rows : 1024;
+  return nw * (int64_t)a->n_out * (a->reduce_c ? 1 : a->C) * elem_size(a->dtype);
+}
+
+int cgtp_tri_contract(const cgtp_tri_args* a, void* stream) {
+  int64_t lds = 0, nw = 0;
+  const int st = tri_check(a, &lds, &nw);
+  if (st != CGTP_OK) return st;
+  return a->dtype == CGTP_F32 ? tri_launch<float>(a, lds, nw, (hipStream_t)stream)
+                              : tri_launch<double>(a, lds, nw, (hipStream_t)stream);
+}
+
+int cgtp_segment_sum(const void* in, const void* scale, const int64_t* index, const int64_t* seg, void* out,
+                     int64_t n_batch, int64_t in_size, int64_t out_size, int64_t C, int32_t dtype, void* stream) {
+  if (!in || !out) return CGTP_ERR_NULL;
+  if (n_batch < 0 || in_size < 0 || out_size < 0 || C <= 0) return CGTP_ERR_SHAPE;
+  if (dtype == CGTP_F32)
+    return segsum_launch<float, 4>(in, scale, index, seg, out, n_batch, in_size, out_size, C, (hipStream_t)stream);
+  if (dtype == CGTP_F64)
+    return segsum_launch<double, 2>(in, scale, index, seg, out, n_batch, in_size, out_size, C, (hipStream_t)stream);
+  return CGTP_ERR_DTYPE;
+}
+
+}  // extern "C"

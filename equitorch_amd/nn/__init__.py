@@ -1,0 +1,6 @@
+"""Module layer (``equitorch.nn``) of the sparse tensor-product path."""
+from . import functional
+from .linears import SO3Linear
+from .tensor_products import TensorProduct
+
+__all__ = ["SO3Linear", "TensorProduct", "functional"]

@@ -1,0 +1,103 @@
+"""Fused edge message passing: gather at the source node, channel-wise tensor product with the edge
+harmonics and per-edge (or shared) weights, and scatter-sum to the destination node, in one kernel.
+
+In reference terms this is the composition
+
+    msg = SO3Linear('uu')(x.index_select(0, src), sh, W)                      (equitorch/nn/linears.py:145-187)
+    out = indexed_scale_segment(msg.view(1, E, -1), None, perm, ptr, N)       (ops/indexed_scale_segment_op.py)
+
+with ``perm`` / ``ptr`` the dst-sorted tables of ``sparse_scale_info(index_out=dst)``.  Neither the gathered
+features nor the messages touch memory here; the backward walks the src-sorted edge list so that the
+gradient with respect to the node features is a register-level segment sum as well.
+"""
+from typing import Optional
+
+import torch
+from torch import Tensor
+from torch.autograd import Function
+
+from ... import _lib
+from ...ops import kernels
+from ...structs import TensorProductInfo
+from .linears import tensor_product_u1u
+from .sparse_scale import sparse_scale
+from ...structs import SparseScaleInfo
+
+
+class EdgePlan:
+    """Sorted views of an edge list ``(src, dst)`` over ``num_nodes`` nodes.
+
+    ``perm_dst`` is the stable ascending sort of the edges by ``dst`` and ``ptr_dst`` its CSR pointer
+    (``ptr_dst[v] .. ptr_dst[v+1]`` are the sorted positions whose edges end at ``v``) — bit for bit the
+    ``index`` and ``seg_out`` of ``sparse_scale_info(index=range(E), index_out=dst, out_size=num_nodes)``
+    (``equitorch/utils/_structs.py:22-71``; a tuple sort on ``(dst, e)`` is a stable sort on ``dst``).
+    ``perm_src`` / ``ptr_src`` are the same for ``src``.  All tensors are int64 on ``src.device``.
+    """
+
+    def __init__(self, src: Tensor, dst: Tensor, num_nodes: int, num_src_nodes: Optional[int] = None):
+        assert src.ndim == 1 and src.shape == dst.shape and src.dtype == dst.dtype == torch.int64
+        self.src, self.dst = src.contiguous(), dst.contiguous()
+        self.num_nodes = int(num_nodes)
+        self.num_src_nodes = int(num_src_nodes if num_src_nodes is not None else num_nodes)
+        self.num_edges = src.shape[0]
+        self.perm_dst, self.ptr_dst = self._sorted(self.dst, self.num_nodes)
+        self.perm_src, self.ptr_src = self._sorted(self.src, self.num_src_nodes)
+
+    @staticmethod
+    def _sorted(key: Tensor, n: int):
+        perm = torch.sort(key, stable=True).indices
+        ptr = torch.zeros(n + 1, dtype=torch.int64, device=key.device)
+        ptr[1:] = torch.cumsum(torch.bincount(key, minlength=n), 0)
+        return perm.contiguous(), ptr
+
+    def scale_infos(self):
+        """(forward, transposed) ``SparseScaleInfo`` of the scatter-sum, for ``sparse_scale``."""
+        return (SparseScaleInfo(None, self.perm_dst, self.ptr_dst, None, self.num_nodes),
+                SparseScaleInfo(None, self.dst, None, None, self.num_edges))
+
+
+class _EdgeUvuCompiled(Function):
+    @staticmethod
+    def forward(ctx, x: Tensor, sh: Tensor, w: Tensor, plan: EdgePlan, tp_info: TensorProductInfo, cfg: int):
+        dims = kernels.uvu_dims(cfg)
+        out = kernels.uvu_forward(cfg, dims, x, sh, w, ptr_=plan.ptr_dst, perm=plan.perm_dst, gather=plan.src)
+        if out is None:
+            raise _lib.CgtpError("fused edge tensor product not launchable for these shapes")
+        ctx.save_for_backward(x, sh, w)
+        ctx.plan, ctx.cfg, ctx.dims = plan, cfg, dims
+        return out
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, g):
+        x, sh, w = ctx.saved_tensors
+        plan = ctx.plan
+        res = kernels.uvu_backward(ctx.cfg, ctx.dims, x, sh, w, g.contiguous(), ctx.needs_input_grad[:3],
+                                   ptr_=plan.ptr_src, perm=plan.perm_src, gather=plan.dst)
+        if res is None:
+            raise _lib.CgtpError("fused edge backward not launchable for these shapes")
+        return (*res, None, None, None)
+
+
+def edge_tensor_product_uu(x: Tensor, sh: Tensor, weight: Tensor, plan: EdgePlan,
+                           tp_info_forward: TensorProductInfo,
+                           tp_info_backward1: Optional[TensorProductInfo] = None,
+                           tp_info_backward2: Optional[TensorProductInfo] = None) -> Tensor:
+    """``out[v] = sum_{e: dst[e]=v} TP_uu(x[src[e]], sh[e], W[e])``.
+
+    ``x (N_src, D1, C)``, ``sh (E, D2)``, ``weight (E, P, C) | (P, C)`` -> ``(N, DO, C)``.  Uses the fused
+    kernel when the table of ``tp_info_forward`` is compiled in and one wavefront slot covers the channels;
+    otherwise runs the same three steps as separate launches.
+    """
+    _lib.require_gpu(x, sh, weight)
+    if plan.num_src_nodes != x.shape[0]:
+        raise _lib.CgtpError(f"plan was built for {plan.num_src_nodes} source nodes, x has {x.shape[0]}")
+    cfg = kernels.uvu_config_of(tp_info_forward)
+    if cfg >= 0 and x.dtype == sh.dtype == weight.dtype and x.dtype in (torch.float32, torch.float64):
+        xc, yc, wc = x.contiguous(), sh.contiguous(), weight.contiguous()
+        if kernels.uvu_launchable(cfg, xc, yc, wc, segments=True):
+            return _EdgeUvuCompiled.apply(xc, yc, wc, plan, tp_info_forward, cfg)
+    msg = tensor_product_u1u(x.index_select(0, plan.src), sh, weight, tp_info_forward)
+    e, d, c = msg.shape
+    fwd, bwd = plan.scale_infos()
+    return sparse_scale(msg.view(1, e, d * c), fwd, bwd).view(plan.num_nodes, d, c)

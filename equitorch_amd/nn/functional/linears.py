@@ -1,0 +1,94 @@
+"""Channel-wise tensor products where one operand has no channel axis (the ``SO3Linear('uu')`` family).
+
+Reference: ``equitorch/nn/functional/linears.py:16-252``.  There each product is two kernel launches with the
+``(N, n_segments, C)`` intermediate ``inter`` written to memory, saved for the backward and returned as a
+second output; here each product is one fused launch and nothing but the inputs is saved.
+
+    u1u : out[n,M,c] = sum_t c_t x[n,M1_t,c] y[n,M2_t]   W[(n),p_t,c]
+    1uu : out[n,M,c] = sum_t c_t x[n,M1_t]   y[n,M2_t,c] W[(n),p_t,c]
+    uu1 : out[n,M]   = sum_t c_t sum_c x[n,M1_t,c] y[n,M2_t,c] W[(n),p_t,c]
+
+``weight`` is shared ``(P, C)`` or per-sample ``(N, P, C)``.  Only ``tp_info_forward`` is read; the two
+backward tables are accepted for signature compatibility.
+"""
+from typing import Optional
+
+import torch
+from torch import Tensor
+from torch.autograd import Function
+
+from ... import _lib
+from ..._lib import OPERAND_SCALAR as S, OPERAND_VEC as V
+from ...ops import kernels
+from ...structs import TensorProductInfo
+from ._tri import spec_from_tp_info, tri
+
+
+class _UvuCompiled(Function):
+    """u1u on the kernels with a compiled-in table (``cgtp_uvu_fwd`` / ``cgtp_uvu_bwd``)."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, y: Tensor, w: Tensor, tp_info: TensorProductInfo, cfg: int):
+        out = kernels.uvu_forward(cfg, kernels.uvu_dims(cfg), x, y, w)
+        if out is None:
+            raise _lib.CgtpError("specialised forward not launchable")
+        ctx.save_for_backward(x, y, w)
+        ctx.tp_info, ctx.cfg = tp_info, cfg
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        x, y, w = ctx.saved_tensors
+        need = ctx.needs_input_grad[:3]
+        if torch.is_grad_enabled():
+            # higher-order derivative requested: re-express through the differentiable contraction
+            with torch.enable_grad():
+                spec = spec_from_tp_info(ctx.tp_info)
+                gx = tri(spec.grad_spec(0), (V, S, V), V, g, y, w) if need[0] else None
+                gy = tri(spec.grad_spec(1), (V, V, V), S, x, g, w) if need[1] else None
+                gw = tri(spec.grad_spec(2), (V, S, V), V, x, y, g, out_shared=(w.ndim == 2)) if need[2] else None
+            return gx, gy, gw, None, None
+        res = kernels.uvu_backward(ctx.cfg, kernels.uvu_dims(ctx.cfg), x, y, w, g.contiguous(), need)
+        if res is None:
+            raise _lib.CgtpError("specialised backward not launchable after a specialised forward")
+        return (*res, None, None)
+
+
+def _check_batch(input1, input2, weight):
+    _lib.require_gpu(input1, input2, weight)
+
+
+def tensor_product_u1u(input1: Tensor, input2: Tensor, weight: Tensor,
+                       tp_info_forward: TensorProductInfo,
+                       tp_info_backward1: Optional[TensorProductInfo] = None,
+                       tp_info_backward2: Optional[TensorProductInfo] = None) -> Tensor:
+    """``input1 (N, D1, C)``, ``input2 (N, D2)``, ``weight (P, C) | (N, P, C)`` -> ``(N, DO, C)``."""
+    _check_batch(input1, input2, weight)
+    if (input1.ndim == 3 and input2.ndim == 2 and input1.dtype == input2.dtype == weight.dtype
+            and input1.dtype in (torch.float32, torch.float64)):
+        cfg = kernels.uvu_config_of(tp_info_forward)
+        x, y, w = input1.contiguous(), input2.contiguous(), weight.contiguous()
+        if cfg >= 0 and kernels.uvu_launchable(cfg, x, y, w):
+            return _UvuCompiled.apply(x, y, w, tp_info_forward, cfg)
+    return tri(spec_from_tp_info(tp_info_forward), (V, S, V), V, input1, input2, weight)
+
+
+so3_linear_uu = tensor_product_u1u
+
+
+def tensor_product_1uu(input1: Tensor, input2: Tensor, weight: Tensor,
+                       tp_info_forward: TensorProductInfo,
+                       tp_info_backward1: Optional[TensorProductInfo] = None,
+                       tp_info_backward2: Optional[TensorProductInfo] = None) -> Tensor:
+    """``input1 (N, D1)``, ``input2 (N, D2, C)`` -> ``(N, DO, C)``."""
+    _check_batch(input1, input2, weight)
+    return tri(spec_from_tp_info(tp_info_forward), (S, V, V), V, input1, input2, weight)
+
+
+def tensor_product_uu1(input1: Tensor, input2: Tensor, weight: Tensor,
+                       tp_info_forward: TensorProductInfo,
+                       tp_info_backward1: Optional[TensorProductInfo] = None,
+                       tp_info_backward2: Optional[TensorProductInfo] = None) -> Tensor:
+    """``input1 (N, D1, C)``, ``input2 (N, D2, C)`` -> ``(N, DO)`` (summed over channels)."""
+    _check_batch(input1, input2, weight)
+    return tri(spec_from_tp_info(tp_info_forward), (V, V, V), S, input1, input2, weight)

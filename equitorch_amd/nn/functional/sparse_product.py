@@ -1,0 +1,50 @@
+"""Differentiable sparse products (element-wise members of ``equitorch/nn/functional/sparse_product.py``).
+
+Signatures follow the reference (``sparse_mul`` :71-99, ``sparse_inner`` :211-233, ``sparse_vecsca``
+:345-365, ``sparse_scavec`` :412-432).  ``info_bwd1`` / ``info_bwd2`` are accepted and unused: the gradient
+tables are derived from ``info_fwd`` itself.  ``out_accumulated=True`` sums the result over the batch axis.
+"""
+from typing import Optional
+
+from torch import Tensor
+
+from ..._lib import OPERAND_SCALAR as S, OPERAND_VEC as V
+from ...structs import SparseProductInfo
+from ._tri import spec_from_product_info, tri
+
+
+def _size(t: Tensor, kind: int) -> int:
+    return t.shape[-2] if kind == V else t.shape[-1]
+
+
+def _binary(k1, k2, ko, input1, input2, info_fwd, out_accumulated):
+    spec = spec_from_product_info(info_fwd, _size(input1, k1), _size(input2, k2))
+    return tri(spec, (k1, k2, 0), ko, input1, input2, None, out_shared=out_accumulated)
+
+
+def sparse_mul(input1: Tensor, input2: Tensor, info_fwd: SparseProductInfo,
+               info_bwd1: Optional[SparseProductInfo] = None, info_bwd2: Optional[SparseProductInfo] = None,
+               out_accumulated: bool = False) -> Tensor:
+    """``z[n,M,c] = sum_t s_t x[n,i1_t,c] y[n,i2_t,c]``."""
+    return _binary(V, V, V, input1, input2, info_fwd, out_accumulated)
+
+
+def sparse_inner(input1: Tensor, input2: Tensor, info_fwd: SparseProductInfo,
+                 info_bwd1: Optional[SparseProductInfo] = None, info_bwd2: Optional[SparseProductInfo] = None,
+                 out_accumulated: bool = False) -> Tensor:
+    """``z[n,M] = sum_t s_t sum_c x[n,i1_t,c] y[n,i2_t,c]``."""
+    return _binary(V, V, S, input1, input2, info_fwd, out_accumulated)
+
+
+def sparse_vecsca(input1: Tensor, input2: Tensor, info_fwd: SparseProductInfo,
+                  info_bwd1: Optional[SparseProductInfo] = None, info_bwd2: Optional[SparseProductInfo] = None,
+                  out_accumulated: bool = False) -> Tensor:
+    """``z[n,M,c] = sum_t s_t x[n,i1_t,c] y[n,i2_t]``."""
+    return _binary(V, S, V, input1, input2, info_fwd, out_accumulated)
+
+
+def sparse_scavec(input1: Tensor, input2: Tensor, info_fwd: SparseProductInfo,
+                  info_bwd1: Optional[SparseProductInfo] = None, info_bwd2: Optional[SparseProductInfo] = None,
+                  out_accumulated: bool = False) -> Tensor:
+    """``z[n,M,c] = sum_t s_t x[n,i1_t] y[n,i2_t,c]``."""
+    return _binary(S, V, V, input1, input2, info_fwd, out_accumulated)

@@ -1,0 +1,106 @@
+"""``SO3Linear``: tensor product of a channelled feature with a channel-less one (edge harmonics).
+
+Constructor, attributes, ``forward`` contract and ``repr`` follow ``equitorch/nn/linears.py:26-212``.
+"""
+import math
+from typing import Optional
+
+import torch
+import torch.nn as nn
+from torch import Tensor
+from torch.nn import Parameter
+
+from ..irreps import check_irreps
+from ..structs import TensorProductInfo
+from ..utils._structs import tp_infos
+from .functional.linears import so3_linear_uu
+from .init import initialize_so3_so2_linear
+
+
+class SO3Linear(nn.Module):
+    r"""``feature_mode='uu'``: ``input1 (N, irreps_in1.dim, C)``, ``input2 (N, irreps_in2.dim)``, weight
+    ``(num_paths, C)`` (shared) or ``(N, num_paths, C)`` (per sample) -> ``(N, irreps_out.dim, C)``.
+
+    ``feature_mode='uv'``: weight ``(num_paths, C_in, C_out)`` (or with a leading ``N``), output
+    ``(N, irreps_out.dim, C_out)``.
+    """
+    tp_info_forward: TensorProductInfo
+    tp_info_backward1: TensorProductInfo
+    tp_info_backward2: TensorProductInfo
+
+    def __init__(self, irreps_in1, irreps_in2, irreps_out, channels_in=None, channels_out=None,
+                 internal_weights=True, feature_mode='uu', path_norm=True, channel_norm=False, path=None):
+        super().__init__()
+        self.irreps_in1 = check_irreps(irreps_in1)
+        self.irreps_in2 = check_irreps(irreps_in2)
+        self.irreps_out = check_irreps(irreps_out)
+        self.irreps_in1_dim = self.irreps_in1.dim
+        self.irreps_in2_dim = self.irreps_in2.dim
+        self.irreps_out_dim = self.irreps_out.dim
+        assert not internal_weights or (channels_in is not None and channels_out is not None)
+        if feature_mode not in ('uu', 'uv'):
+            raise ValueError(f'Feature_mode should be in ["uv", "uu"], got {feature_mode}.')
+        self.channels_in = channels_in
+        self.channels_out = channels_out
+        self.feature_mode = feature_mode
+        self.path_norm = path_norm
+        self.channel_norm = channel_norm and (feature_mode == 'uv')
+        fan_in = self.channels_in if feature_mode == 'uv' else 1
+        (self.tp_info_forward, self.tp_info_backward1, self.tp_info_backward2, self.num_paths) = tp_infos(
+            self.irreps_out, self.irreps_in1, self.irreps_in2, path=path, path_norm=path_norm,
+            channel_norm=self.channel_norm, channel_scale=fan_in ** (-0.5))
+        if feature_mode == 'uv':
+            self.weight_shape = (self.num_paths, self.channels_in, self.channels_out)
+        else:
+            self.weight_shape = (self.num_paths, self.channels_out)
+        self.weight_numel = math.prod(self.weight_shape) if None not in self.weight_shape else None
+        self.internal_weights = internal_weights
+        if internal_weights:
+            self.weight = Parameter(torch.empty(*self.weight_shape))
+            initialize_so3_so2_linear(self.weight, feature_mode, channel_normed=self.channel_norm)
+        else:
+            self.weight = None
+
+    def _resolve_weight(self, input1: Tensor, weight: Optional[Tensor]) -> Tensor:
+        if self.internal_weights:
+            assert weight is None, 'Do not pass the weight when self.internal_weights is True.'
+            return self.weight
+        assert weight is not None, 'Please pass the weight when self.internal_weights is False.'
+        shape = self.weight_shape
+        if None in shape:  # channels were not given at construction: take them from the input
+            shape = ((self.num_paths, input1.shape[-1], weight.shape[-1]) if self.feature_mode == 'uv'
+                     else (self.num_paths, input1.shape[-1]))
+        numel = math.prod(shape)
+        return weight.view(-1, *shape) if weight.numel() > numel else weight.view(*shape)
+
+    def forward(self, input1: Tensor, input2: Tensor, weight: Optional[Tensor] = None):
+        assert input1.shape[-2] == self.irreps_in1_dim, \
+            f"Input1 spherical dim mismatch: expected {self.irreps_in1_dim}, got {input1.shape[-2]}"
+        assert input2.shape[-1] == self.irreps_in2_dim, \
+            f"Input2 spherical dim mismatch: expected {self.irreps_in2_dim}, got {input2.shape[-1]}"
+        assert input2.ndim == input1.ndim - 1, \
+            f"Input2 should have one less dimension than Input1. Got input1 ndim={input1.ndim}, input2 ndim={input2.ndim}"
+        assert self.channels_in is None or input1.shape[-1] == self.channels_in, \
+            f"Input1 channel dim mismatch: expected {self.channels_in}, got {input1.shape[-1]}"
+        weight = self._resolve_weight(input1, weight)
+        infos = (self.tp_info_forward, self.tp_info_backward1, self.tp_info_backward2)
+        if self.feature_mode == 'uu':
+            return so3_linear_uu(input1, input2, weight, *infos)
+        from .functional.linears_uv import so3_linear_uv
+        return so3_linear_uv(input1, input2, weight, *infos)
+
+    def _apply(self, *args, **kwargs):
+        mod = super()._apply(*args, **kwargs)
+        mod.tp_info_forward = self.tp_info_forward._apply(*args, **kwargs)
+        mod.tp_info_backward1 = self.tp_info_backward1._apply(*args, **kwargs)
+        mod.tp_info_backward2 = self.tp_info_backward2._apply(*args, **kwargs)
+        return mod
+
+    def __repr__(self):
+        ch = (f"channels={self.channels_in}" if self.feature_mode == 'uu'
+              else f"channels_in={self.channels_in}, channels_out={self.channels_out}")
+        return (f"{self.__class__.__name__}(irreps_in1={self.irreps_in1.short_repr()}, "
+                f"irreps_in2={self.irreps_in2.short_repr()}, irreps_out={self.irreps_out.short_repr()}, {ch}, "
+                f"feature_mode={self.feature_mode}, path_norm={self.path_norm}, "
+                f"channel_norm={self.channel_norm}, internal_weights={self.internal_weights}, "
+                f"num_paths={self.num_paths})")

@@ -1,0 +1,14 @@
+"""Operator layer (``equitorch.ops``): table-driven sparse products and the indexed scale-segment reduction,
+backed by the HIP kernels of ``libcgtp``."""
+from .batched_sparse_dense_op import (
+    indexed_inner_scale_gather,
+    indexed_mul_scale_gather,
+    indexed_scavec_scale_gather,
+    indexed_vecsca_scale_gather,
+)
+from .indexed_scale_segment_op import indexed_scale_segment
+
+__all__ = [
+    "indexed_mul_scale_gather", "indexed_vecsca_scale_gather", "indexed_scavec_scale_gather",
+    "indexed_inner_scale_gather", "indexed_scale_segment",
+]

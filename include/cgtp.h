@@ -1,0 +1,144 @@
+/*
+ * cgtp — sparse Clebsch-Gordan tensor-product kernels for AMD gfx950 (MI355X), C ABI.
+ *
+ * Every entry point takes raw device pointers, extents and a HIP stream (passed as void*; NULL = the null
+ * stream), enqueues its kernels on that stream and returns immediately with a status code.  Nothing here
+ * allocates, frees or synchronises; buffers (including workspaces) are owned by the caller.  Tensors use
+ * the Equitorch layout (batch, irreps_dim, channels), channel-last and contiguous unless a stride is given.
+ *
+ * The reference (GTML-LAB/Equitorch) has no FFI: its boundary is the Python signature of the Triton launch
+ * wrappers.  Each declaration below names the wrapper it stands in for.
+ */
+#ifndef CGTP_H
+#define CGTP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status codes ---------------------------------------------------------------------------------- */
+enum {
+  CGTP_OK = 0,
+  CGTP_ERR_NULL = 1,        /* a required pointer is NULL                                   */
+  CGTP_ERR_SHAPE = 2,       /* negative / zero / inconsistent extent                        */
+  CGTP_ERR_ALIGN = 3,       /* pointer or stride not aligned for the requested vector width */
+  CGTP_ERR_DTYPE = 4,       /* unsupported element type                                     */
+  CGTP_ERR_CONFIG = 5,      /* unknown specialised-table id                                 */
+  CGTP_ERR_LDS = 6,         /* table does not fit the 160 KB LDS of a CU                    */
+  CGTP_ERR_LAUNCH = 7,      /* hipLaunchKernel reported an error                            */
+  CGTP_ERR_WORKSPACE = 8    /* workspace missing or too small                               */
+};
+
+enum { CGTP_F32 = 0, CGTP_F64 = 1, CGTP_BF16 = 2, CGTP_F16 = 3 };
+
+const char* cgtp_status_string(int status);
+/* ABI version; bumped on any signature change. */
+int cgtp_version(void);
+
+/* ---- generic sparse trilinear contraction -------------------------------------------------------------
+ *
+ *   out[r, o, c] = sum_{t in [seg[o], seg[o+1])} coef[t] * A[ra(r), ia[t], c] * B[rb(r), ib[t], (c)]
+ *                                                        * W[rw(r), iw[t], c]
+ *
+ * with each operand optional, per-channel ("vec") or channel-less ("scalar"), per-row or shared, and
+ * optionally row-gathered.  Covers, with the reference's own tables, indexed_mul / vecsca / scavec / inner
+ * _scale_gather (equitorch/ops/batched_sparse_dense_op.py:156-232, 1665-1750, 994-1035, 713-788) and both
+ * stages of the u1u / 1uu / uu1 / uuu tensor products (equitorch/nn/functional/linears.py:16-252,
+ * equitorch/nn/functional/tensor_products.py:9-90) in one launch.  The table (coef, packed indices, seg)
+ * is staged into LDS by every workgroup.
+ */
+enum { CGTP_OPERAND_NONE = 0, CGTP_OPERAND_VEC = 1, CGTP_OPERAND_SCALAR = 2 };
+
+typedef struct cgtp_operand {
+  const void* data;        /* element type = args.dtype                                         */
+  const int64_t* rows;     /* optional: row r reads data row rows[r]; NULL = identity           */
+  int64_t row_stride;      /* elements between rows; 0 = one row shared by every r              */
+  int64_t idx_stride;      /* elements between consecutive sparse indices (C for vec, 1 scalar) */
+  int32_t kind;            /* CGTP_OPERAND_*                                                    */
+  int32_t _pad;
+} cgtp_operand;
+
+typedef struct cgtp_tri_args {
+  cgtp_operand a, b, w;
+  /* table, all device pointers */
+  const void* coef;        /* [nnz] element type = dtype (f32 or f64); NULL = all ones           */
+  const uint32_t* idx;     /* [nnz] packed ia | ib << 10 | iw << 20 (each < 1024, iw < 4096)     */
+  const int32_t* seg;      /* [n_out + 1]                                                        */
+  int32_t n_out, nnz;
+  /* output */
+  void* out;               /* (n_rows, n_out, C), (n_rows, n_out) if reduce_c, row axis dropped if reduce_rows */
+  void* workspace;         /* reduce_rows only: cgtp_tri_workspace_bytes() bytes                   */
+  int64_t n_rows;
+  int32_t C;
+  int32_t dtype;           /* CGTP_F32 | CGTP_F64                                                  */
+  int32_t reduce_c;        /* sum over channels (inner-product family)                             */
+  int32_t reduce_rows;     /* sum over rows (gradient of an operand shared across the batch)      */
+} cgtp_tri_args;
+
+int64_t cgtp_tri_workspace_bytes(const cgtp_tri_args* args);
+/* Host-only validation of the same conditions the launch checks; needs no device. */
+int cgtp_tri_validate(const cgtp_tri_args* args);
+int cgtp_tri_contract(const cgtp_tri_args* args, void* stream);
+
+/* ---- indexed scale-segment: out[n, m, c] = sum_{t in seg m} scale[t] * in[n, index[t], c] --------------
+ * Stands in for indexed_scale_segment_gpu (equitorch/ops/indexed_scale_segment_op.py:110-141), including the
+ * seg == NULL mode (pure scaled gather, one term per output) and optional scale / index.  With N == 1,
+ * in = messages viewed as (1, E, D*C), index = dst-sorted edge permutation, seg = dst CSR pointer, this is
+ * the edge -> node scatter-sum.  index / seg are int64 as in the reference's tables.
+ */
+int cgtp_segment_sum(const void* in, const void* scale, const int64_t* index, const int64_t* seg, void* out,
+                     int64_t n_batch, int64_t in_size, int64_t out_size, int64_t C, int32_t dtype,
+                     void* stream);
+
+/* ---- specialised channel-wise ("uvu") tensor product -----------------------------------------------------
+ *
+ *   out[n, M, c] = sum_t coef_t * x[xr(n), M1_t, c] * y[n, M2_t] * W[(n), p_t, c]
+ *
+ * Fused replacement for the two launches of TensorProductU1UDummy.forward
+ * (equitorch/nn/functional/linears.py:18-42: indexed_vecsca_scale_gather then indexed_mul_scale_gather) and,
+ * in the backward entry, for the seven launches of its backward (:44-83).  The Clebsch-Gordan table is
+ * compiled into the kernel; cgtp_uvu_find() maps a table fingerprint to a config id (or -1).
+ *
+ * Segment mode (ptr != NULL) additionally fuses the gather x[xrow[e]] and the scatter-sum over a sorted edge
+ * list: segment s owns sorted positions [ptr[s], ptr[s+1]); position q is edge e = perm ? perm[q] : q.
+ */
+int cgtp_uvu_num_configs(void);
+int cgtp_uvu_find(uint64_t fingerprint);
+/* Describes config `cfg`: dims (D1, D2, DO, P, NNZ) written to dims[5]; returns its fingerprint (0 if bad). */
+uint64_t cgtp_uvu_describe(int cfg, int32_t* dims);
+
+typedef struct cgtp_uvu_args {
+  int32_t cfg;             /* from cgtp_uvu_find                                                   */
+  int32_t dtype;           /* CGTP_F32 | CGTP_F64                                                  */
+  int32_t C;               /* channels                                                             */
+  int32_t w_shared;        /* 1: W is (P, C); 0: W is (n_rows, P, C)                               */
+  int64_t n_rows;          /* batch rows / edges                                                   */
+  int64_t n_x_rows;        /* rows of x (== n_rows unless gathered / segment-owned)                */
+  int64_t n_seg;           /* number of segments (nodes); 0 = no segment mode                      */
+  const int64_t* ptr;      /* [n_seg + 1] sorted-position CSR pointer, or NULL                     */
+  const int64_t* perm;     /* [n_rows] sorted position -> edge id, or NULL = identity              */
+  const int64_t* gather;   /* [n_rows] fwd: x row per edge; bwd: grad_out row per edge; or NULL    */
+  const void* x;           /* fwd: (n_x_rows, D1, C).  bwd: same; in segment mode row = segment id */
+  const void* y;           /* (n_rows, D2)                                                         */
+  const void* w;           /* (n_rows | 1, P, C)                                                   */
+  /* forward */
+  void* out;               /* (n_seg ? n_seg : n_rows, DO, C)                                      */
+  /* backward */
+  const void* grad_out;    /* (rows addressed by gather / row id, DO, C)                           */
+  void* grad_x;            /* (n_seg ? n_seg : n_rows, D1, C) or NULL                              */
+  void* grad_y;            /* (n_rows, D2) or NULL                                                 */
+  void* grad_w;            /* (n_rows | 1, P, C) or NULL                                           */
+  void* workspace;         /* bwd with w_shared && grad_w: cgtp_uvu_bwd_workspace_bytes() bytes    */
+} cgtp_uvu_args;
+
+int cgtp_uvu_validate(const cgtp_uvu_args* args, int backward);
+int64_t cgtp_uvu_bwd_workspace_bytes(const cgtp_uvu_args* args);
+int cgtp_uvu_fwd(const cgtp_uvu_args* args, void* stream);
+int cgtp_uvu_bwd(const cgtp_uvu_args* args, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CGTP_H */

@@ -1,0 +1,213 @@
+"""TEST INFRASTRUCTURE ONLY: CPU numerics of the sparse tensor-product path.
+
+Two independent restatements:
+
+* ``dense_*`` — float64 einsum straight from the dense Clebsch-Gordan blocks (no sparse table involved),
+  differentiated by torch autograd.  This is the arbiter for parity.
+* ``cpu_*`` — step-for-step restatement of the reference's CPU fallbacks in torch CPU ops
+  (``index_select`` both operands to nnz length -> product -> ``* scale`` -> CSR segment-sum), composed as the
+  reference's Functions compose them.  ``torch_geometric.utils.segment`` (PyG 2.5.3, absent here; used at
+  ``equitorch/ops/batched_sparse_dense_op.py:262,818,1495,1781`` and ``indexed_scale_segment_op.py:167``) is a
+  CSR sum along dim 1 and is restated as ``index_add_`` over expanded segment ids.  This is the timed
+  "reference CPU path" of the benchmark.
+
+Pinned by: agreement of the two restatements with each other (tests/test_oracle.py), and for the dense one
+by O(3)-equivariance, the l2=0 scaling identity, the 1x1->0 dot product, the 1x1->1 cross product and
+``torch.autograd.gradcheck``.  No stored output vectors exist in the reference for this path.
+"""
+import torch
+
+from . import ref_constants, ref_tables
+
+
+# ---- dense float64 oracle -----------------------------------------------------------------------------------
+def dense_coupling(irreps_out, irreps1, irreps2, path=None, path_norm=True, channel_norm=False,
+                   channel_scale=1.0) -> torch.Tensor:
+    """``T[p, M, M1, M2]`` float64 with the path normalisation of ``prepare_so3``
+    (``equitorch/utils/_structs.py:177-206``) folded in."""
+    io, i1, i2 = ref_tables.parse(irreps_out), ref_tables.parse(irreps1), ref_tables.parse(irreps2)
+    if not path:
+        path = ref_tables.fully_connected_paths(io, i1, i2)
+    so, s1, s2 = ref_tables.segments(io), ref_tables.segments(i1), ref_tables.segments(i2)
+    count, cur = {}, None
+    for k, _, _ in path:
+        count[k] = count[k] + 1 if k == cur else 1
+        cur = k
+    T = torch.zeros(len(path), so[-1], s1[-1], s2[-1], dtype=torch.float64)
+    for p, (k, i, j) in enumerate(path):
+        cg = ref_constants.so3_cg(io[k][0], i1[i][0], i2[j][0])
+        blk = torch.tensor([[[float(v) for v in r] for r in m] for m in cg], dtype=torch.float64)
+        norm = (count[k] ** -0.5 if path_norm else 1.0) * (channel_scale if channel_norm else 1.0)
+        T[p, so[k]:so[k + 1], s1[i]:s1[i + 1], s2[j]:s2[j + 1]] = blk * norm
+    return T
+
+
+def dense_u1u(T, x, y, w):
+    """``out[n,M,c] = sum T[p,M,a,b] x[n,a,c] y[n,b] w[(n),p,c]`` in float64."""
+    x, y, w = x.double(), y.double(), w.double()
+    if w.ndim == 2:
+        return torch.einsum("pmab,nac,nb,pc->nmc", T, x, y, w)
+    return torch.einsum("pmab,nac,nb,npc->nmc", T, x, y, w)
+
+
+def dense_uuu(T, x, y, w):
+    x, y, w = x.double(), y.double(), w.double()
+    if w.ndim == 2:
+        return torch.einsum("pmab,nac,nbc,pc->nmc", T, x, y, w)
+    return torch.einsum("pmab,nac,nbc,npc->nmc", T, x, y, w)
+
+
+def dense_u1v(T, x, y, w):
+    """``out[n,M,v] = sum T[p,M,a,b] y[n,b] x[n,a,u] w[(n),p,u,v]``."""
+    x, y, w = x.double(), y.double(), w.double()
+    if w.ndim == 3:
+        return torch.einsum("pmab,nau,nb,puv->nmv", T, x, y, w)
+    return torch.einsum("pmab,nau,nb,npuv->nmv", T, x, y, w)
+
+
+def dense_uvw(T, x, y, w):
+    x, y, w = x.double(), y.double(), w.double()
+    if w.ndim == 4:
+        return torch.einsum("pmab,nau,nbv,puvw->nmw", T, x, y, w)
+    return torch.einsum("pmab,nau,nbv,npuvw->nmw", T, x, y, w)
+
+
+def dense_grads(fn, T, inputs, cotangent):
+    """Gradients of ``(fn(T, *inputs) * cotangent).sum()`` w.r.t. every input, float64."""
+    leaves = [t.detach().double().requires_grad_(True) for t in inputs]
+    out = fn(T, *leaves)
+    return out.detach(), torch.autograd.grad((out * cotangent.double()).sum(), leaves)
+
+
+def scatter_sum(msg, dst, num_nodes):
+    """``node[v] = sum_{e: dst[e]=v} msg[e]`` in the dtype of ``msg``."""
+    out = torch.zeros((num_nodes,) + msg.shape[1:], dtype=msg.dtype)
+    return out.index_add_(0, dst, msg)
+
+
+# ---- structural restatement of the reference CPU path ------------------------------------------------------
+def _tt(v, dtype=None):
+    return None if v is None else torch.tensor(v, dtype=dtype)
+
+
+def tables_to_torch(info: dict, float_dtype=torch.float32) -> dict:
+    """Lists of ``oracle.ref_tables`` -> tensors as ``torch.tensor(list)`` makes them in the reference."""
+    out = {}
+    for k, v in info.items():
+        if isinstance(v, dict):
+            out[k] = tables_to_torch(v, float_dtype)
+        elif isinstance(v, list):
+            out[k] = torch.tensor(v, dtype=float_dtype if k == "scale" else torch.int64)
+        else:
+            out[k] = v
+    return out
+
+
+def segment_csr(src: torch.Tensor, ptr: torch.Tensor, dim: int) -> torch.Tensor:
+    """Sum of ``src`` over ``[ptr[i], ptr[i+1])`` along ``dim`` (what PyG's ``segment(src, ptr[None])`` does)."""
+    n_seg = ptr.shape[0] - 1
+    ids = torch.repeat_interleave(torch.arange(n_seg), ptr[1:] - ptr[:-1])
+    shape = list(src.shape)
+    shape[dim] = n_seg
+    return torch.zeros(shape, dtype=src.dtype).index_add_(dim, ids, src)
+
+
+def cpu_mul(x, y, info, out_accumulated=False):
+    """``indexed_mul_scale_gather_cpu`` (batched_sparse_dense_op.py:234-275)."""
+    if info["index1"] is not None:
+        x = x.index_select(-2, info["index1"])
+    if info["index2"] is not None:
+        y = y.index_select(-2, info["index2"])
+    inter = x * y
+    if info["scale"] is not None:
+        inter = inter * info["scale"].unsqueeze(-1)
+    if info["seg_out"] is not None:
+        inter = segment_csr(inter, info["seg_out"], inter.ndim - 2)
+    return inter.sum(0) if out_accumulated else inter
+
+
+def cpu_vecsca(x, y, info, out_accumulated=False):
+    """``indexed_vecsca_scale_gather_cpu`` (:1752-1794): x vector, y scalar."""
+    if info["index1"] is not None:
+        x = x.index_select(-2, info["index1"])
+    if info["index2"] is not None:
+        y = y.index_select(-1, info["index2"])
+    inter = x * y.unsqueeze(-1)
+    if info["scale"] is not None:
+        inter = inter * info["scale"].unsqueeze(-1)
+    if info["seg_out"] is not None:
+        inter = segment_csr(inter, info["seg_out"], inter.ndim - 2)
+    return inter.sum(0) if out_accumulated else inter
+
+
+def cpu_scavec(x, y, info, out_accumulated=False):
+    """``indexed_scavec_scale_gather`` (:994-1035): operands and their index columns swapped into vecsca."""
+    swapped = dict(info, index1=info["index2"], index2=info["index1"])
+    return cpu_vecsca(y, x, swapped, out_accumulated)
+
+
+def cpu_inner(x, y, info, out_accumulated=False):
+    """``indexed_inner_scale_gather_cpu`` (:790-831)."""
+    if info["index1"] is not None:
+        x = x.index_select(-2, info["index1"])
+    if info["index2"] is not None:
+        y = y.index_select(-2, info["index2"])
+    inter = (x * y).sum(-1)
+    if info["scale"] is not None:
+        inter = inter * info["scale"]
+    if info["seg_out"] is not None:
+        inter = segment_csr(inter, info["seg_out"], inter.ndim - 1)
+    return inter.sum(0) if out_accumulated else inter
+
+
+def cpu_scale_segment(inp, scale, index, seg):
+    """``indexed_scale_segment_cpu`` (indexed_scale_segment_op.py:143-170)."""
+    if index is not None:
+        inp = inp.index_select(-2, index)
+    if scale is not None:
+        inp = inp * scale.unsqueeze(-1)
+    if seg is not None:
+        inp = segment_csr(inp, seg, inp.ndim - 2)
+    return inp
+
+
+def cpu_u1u_forward(x, y, w, tp_fwd):
+    """``TensorProductU1UDummy.forward`` (nn/functional/linears.py:24-25) -> (ret, inter)."""
+    inter = cpu_vecsca(x, y, tp_fwd["info_Mij_fwd"])
+    return cpu_mul(inter, w, tp_fwd["info_M_fwd"]), inter
+
+
+def cpu_1uu_forward(x, y, w, tp_fwd):
+    """``TensorProduct1UUDummy.forward`` (:104-105): x scalar, y vector."""
+    inter = cpu_scavec(x, y, tp_fwd["info_Mij_fwd"])
+    return cpu_mul(inter, w, tp_fwd["info_M_fwd"])
+
+
+def cpu_uu1_forward(x, y, w, tp_fwd):
+    """``TensorProductUU1Dummy.forward`` (:184-185): both vectors, inner product with the weight."""
+    inter = cpu_mul(x, y, tp_fwd["info_Mij_fwd"])
+    return cpu_inner(inter, w, tp_fwd["info_M_fwd"])
+
+
+def cpu_u1u_backward(g, x, y, w, inter, tp_fwd, tp_bwd1, tp_bwd2):
+    """First-order part of ``TensorProductU1UDummy.backward`` (:44-83); the ``grad_inter`` terms vanish."""
+    gx = cpu_1uu_forward(y, g, w, tp_bwd1)
+    gy = cpu_uu1_forward(g, x, w, tp_bwd2)
+    gw = cpu_mul(g, inter, tp_fwd["info_M_bwd2"], out_accumulated=(w.ndim == 2))
+    return gx, gy, gw
+
+
+def cpu_edge_forward(x, sh, w, src, perm, ptr, tp_fwd):
+    """``x.index_select(0, src)`` -> u1u -> ``indexed_scale_segment(msg.view(1,E,-1), None, perm, ptr)``."""
+    msg, inter = cpu_u1u_forward(x.index_select(0, src), sh, w, tp_fwd)
+    e, d, c = msg.shape
+    out = cpu_scale_segment(msg.view(1, e, d * c), None, perm, ptr)
+    return out.view(-1, d, c), inter
+
+
+def cpu_edge_backward(ct, x, sh, w, inter, src, dst, tp_fwd, tp_bwd1, tp_bwd2):
+    """Transposed direction: gather the cotangent at dst, TP backward per edge, scatter grad_x to src."""
+    g = ct.index_select(0, dst)
+    gxs, gy, gw = cpu_u1u_backward(g, x.index_select(0, src), sh, w, inter, tp_fwd, tp_bwd1, tp_bwd2)
+    gx = torch.zeros_like(x).index_add_(0, src, gxs)
+    return gx, gy, gw
