@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Benchmark of the edge tensor-product hot path on one MI355X.
+
+Default workload (``edge_fwd_bwd``): the lmax=2, C=64 edge message-passing step of BASELINE.json —
+N=4096 nodes, E=65536 uniformly random edges, per-edge weights (E, 11, 64), fp32 — forward
+(gather x[src] -> channel-wise CG tensor product -> scatter-sum to dst) plus full backward (gradients
+w.r.t. node features, edge harmonics and per-edge weights).  A "step" is one forward + backward through
+the public autograd API on synthetic seeded inputs resident in HBM.  Weight tensors rotate over several
+buffers so that consecutive steps cannot be served from the 256 MB last-level cache.
+
+Prints ONE JSON line: throughput in Medges/s, the roofline record of the dominant kernel (backward),
+measured with events on the launch stream, and the CPU baseline (the oracle's restatement of the
+reference's CPU path, timed on a bounded sample of the same workload).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
+
+WORKLOADS = {
+    # name: (lmax, channels, nodes, edges)
+    "edge_fwd_bwd": (2, 64, 4096, 65536),
+    "edge_fwd": (2, 64, 4096, 65536),
+    # streaming kernels of known traffic (1 GiB): counter calibration and achievable-bandwidth reference
+    "copy": None,
+    "read": None,
+}
+
+
+def membench(kind, steps, warmup):
+    """Plain 1 GiB device copy (reads 1 GiB, writes 1 GiB) or read; one JSON line with the achieved GB/s."""
+    from equitorch_amd import _lib
+    dev = torch.device("cuda:0")
+    n_bytes = 1 << 30
+    src = torch.empty(n_bytes, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty(n_bytes if kind == "copy" else 16, dtype=torch.uint8, device=dev)
+    stream = _lib.stream_ptr(dev)
+
+    def launch():
+        if kind == "copy":
+            _lib.check(_lib.lib.cgtp_membench_copy(dst.data_ptr(), src.data_ptr(), n_bytes, stream))
+        else:
+            _lib.check(_lib.lib.cgtp_membench_read(src.data_ptr(), dst.data_ptr(), n_bytes, stream))
+    for _ in range(warmup):
+        launch()
+    evs = []
+    for _ in range(steps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(); launch(); b.record()
+        evs.append((a, b))
+    torch.cuda.synchronize()
+    ms = sum(a.elapsed_time(b) for a, b in evs) / steps
+    moved = n_bytes * (2 if kind == "copy" else 1)
+    print(json.dumps({"metric": f"membench_{kind}", "value": round(moved / ms / 1e6, 1), "unit": "GB/s",
+                      "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 5),
+                      "bytes_read": n_bytes, "bytes_written": n_bytes if kind == "copy" else 0,
+                      "config": {"workload": f"{kind} of 1 GiB, float4 grid-stride, 4096 workgroups"}}))
+
+
+def make_inputs(lmax, ch, n_nodes, n_edges, n_rot, device):
+    """Seeded CPU generation in the fixed order src, dst, x, vec -> sh, W, ct; then moved to the device."""
+    from equitorch_amd.utils._sh import spherical_harmonics
+    gen = torch.Generator().manual_seed(0)
+    d = (lmax + 1) ** 2
+    src = torch.randint(0, n_nodes, (n_edges,), generator=gen)
+    dst = torch.randint(0, n_nodes, (n_edges,), generator=gen)
+    x = torch.randn(n_nodes, d, ch, generator=gen)
+    vec = torch.randn(n_edges, 3, generator=gen)
+    sh = spherical_harmonics(vec / vec.norm(dim=-1, keepdim=True), lmax)
+    return dict(src=src, dst=dst, x=x, sh=sh, gen=gen, d=d)
+
+
+def algorithmic_bytes(n_nodes, n_edges, d, p, ch):
+    """Compulsory HBM traffic of one launch: every distinct input byte once, every output byte once, int64
+    index tables as in the reference."""
+    f = 4
+    w = n_edges * p * ch * f
+    node = n_nodes * d * ch * f
+    edge_sh = n_edges * d * f
+    idx = 2 * n_edges * 8 + (n_nodes + 1) * 8
+    fwd = w + node + edge_sh + node + idx            # read W, x, sh, tables; write out
+    bwd = (w + node + node + edge_sh + idx) + (w + edge_sh + node)  # read W, ct, x, sh, tables; write gW, gsh, gx
+    return fwd, bwd
+
+
+def cpu_baseline(inp, lmax, ch, n_nodes, sample_edges, budget_s=12.0):
+    """The oracle's step-for-step restatement of the reference's CPU path (index_select -> product -> scale ->
+    CSR segment-sum; forward and backward), timed on the first ``sample_edges`` edges of the same graph."""
+    from oracle import ref_ops, ref_tables
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+    fwd, b1, b2, n_paths = ref_tables.tp_infos(irreps, irreps, irreps)
+    fwd, b1, b2 = (ref_ops.tables_to_torch(t) for t in (fwd, b1, b2))
+    e = sample_edges
+    src, dst = inp["src"][:e], inp["dst"][:e]
+    scale_fwd, _ = ref_tables.sparse_scale_infos(index=list(range(e)), index_out=dst.tolist(),
+                                                 out_size=n_nodes, in_size=e)
+    perm = torch.tensor(scale_fwd["index"]) if scale_fwd["index"] is not None else None
+    ptr = torch.tensor(scale_fwd["seg_out"])
+    gen = torch.Generator().manual_seed(1)
+    x, sh = inp["x"], inp["sh"][:e]
+    w = torch.randn(e, n_paths, ch, generator=gen)
+    ct = torch.randn(n_nodes, inp["d"], ch, generator=gen)
+
+    def step():
+        out, inter = ref_ops.cpu_edge_forward(x, sh, w, src, perm, ptr, fwd)
+        return out, ref_ops.cpu_edge_backward(ct, x, sh, w, inter, src, dst, fwd, b1, b2)
+
+    step()
+    t0 = time.perf_counter()
+    step()
+    one = time.perf_counter() - t0
+    iters = max(2, min(20, int(budget_s / max(one, 1e-3))))
+    times = []
+    for _ in range(iters):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    return {"value": round(e / med / 1e6, 4), "unit": "Medges/s", "cores": threads, "kind": "port",
+            "sample": f"first {e} of {inp['src'].shape[0]} edges of the same graph, fwd+bwd, median of {iters} "
+                      f"runs, {med * 1e3:.1f} ms/run, torch {torch.__version__} CPU ops"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="edge_fwd_bwd", choices=sorted(WORKLOADS))
+    ap.add_argument("--rotate", type=int, default=4, help="number of weight buffers cycled through")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-edges", type=int, default=16384)
+    ap.add_argument("--pos-per-wave", type=int, default=0,
+                    help="sorted positions per wavefront in the per-kernel timing (0 = library default)")
+    ap.add_argument("--kernel-reps", type=int, default=30, help="launches per kernel for the roofline timing")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on exactly one GPU (the path has no multi-GPU part); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    if args.workload in ("copy", "read"):
+        membench(args.workload, args.steps, args.warmup)
+        return
+
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu
+    from equitorch_amd.ops import kernels
+
+    lmax, ch, n_nodes, n_edges = WORKLOADS[args.workload]
+    backward = args.workload == "edge_fwd_bwd"
+    dev = torch.device("cuda:0")
+    irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+    mod = SO3Linear(irreps, irreps, irreps, ch, ch, internal_weights=False, feature_mode="uu").to(dev)
+    p = mod.num_paths
+    inp = make_inputs(lmax, ch, n_nodes, n_edges, args.rotate, dev)
+    d = inp["d"]
+    plan = EdgePlan(inp["src"].to(dev), inp["dst"].to(dev), n_nodes)
+    x = inp["x"].to(dev).requires_grad_(backward)
+    sh = inp["sh"].to(dev).requires_grad_(backward)
+    ws = [torch.randn(n_edges, p, ch, generator=inp["gen"]).to(dev).requires_grad_(backward)
+          for _ in range(args.rotate)]
+    ct = torch.randn(n_nodes, d, ch, generator=inp["gen"]).to(dev)
+
+    def step(i):
+        w = ws[i % args.rotate]
+        out = edge_tensor_product_uu(x, sh, w, plan, mod.tp_info_forward)
+        if backward:
+            gx, gsh, gw = torch.autograd.grad(out, (x, sh, w), ct)
+            return gw
+        return out
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    medges = n_edges / (elapsed / args.steps) / 1e6
+
+    # ---- per-kernel durations with events on the launch stream (torch's current stream) ----------------------
+    cfg = kernels.uvu_config_of(mod.tp_info_forward)
+    dims = kernels.uvu_dims(cfg)
+    xd, shd = x.detach(), sh.detach()
+
+    def time_kernel(fn):
+        evs = []
+        for i in range(args.kernel_reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            w = ws[i % args.rotate].detach()
+            a.record()
+            fn(w)
+            b.record()
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        ts = sorted(a.elapsed_time(b) for a, b in evs)
+        return sum(ts) / len(ts), ts[len(ts) // 2]
+
+    ppw = args.pos_per_wave
+    fwd_fn = lambda w: kernels.uvu_forward(cfg, dims, xd, shd, w, seg=plan.fwd_index, pos_per_wave=ppw)
+    bwd_fn = lambda w: kernels.uvu_backward(cfg, dims, xd, shd, w, ct, (True, True, True), seg=plan.bwd_index,
+                                            pos_per_wave=ppw)
+    fwd_fn(ws[0].detach()); bwd_fn(ws[0].detach())
+    fwd_avg, fwd_med = time_kernel(fwd_fn)
+    bwd_avg, bwd_med = time_kernel(bwd_fn)
+    fwd_bytes, bwd_bytes = algorithmic_bytes(n_nodes, n_edges, d, p, ch)
+    if backward:
+        dom, dom_bytes, dom_ms = "uvu_bwd_kernel<sh2,f32,V4,SEG>", bwd_bytes, bwd_avg
+    else:
+        dom, dom_bytes, dom_ms = "uvu_fwd_kernel<sh2,f32,V4,SEG>", fwd_bytes, fwd_avg
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+
+    rec = {
+        "metric": "edge-TP fwd+bwd Medges/s (lmax=2,C=64)" if backward else "edge-TP fwd Medges/s (lmax=2,C=64)",
+        "value": round(medges, 2), "unit": "Medges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: N={n_nodes} nodes, E={n_edges} edges, irreps {irreps}, "
+                               f"C={ch}, per-edge weights (E,{p},{ch}), {args.rotate} rotating weight buffers"},
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes": dom_bytes, "avg_ms": round(dom_ms, 5)},
+        "kernels": {"fwd_avg_ms": round(fwd_avg, 5), "fwd_med_ms": round(fwd_med, 5),
+                    "fwd_GBs": round(fwd_bytes / fwd_avg / 1e6, 1),
+                    "bwd_avg_ms": round(bwd_avg, 5), "bwd_med_ms": round(bwd_med, 5),
+                    "bwd_GBs": round(bwd_bytes / bwd_avg / 1e6, 1),
+                    "fwd_bwd_GBs": round((fwd_bytes + bwd_bytes) / (fwd_avg + bwd_avg) / 1e6, 1)},
+    }
+    if not args.no_cpu_baseline:
+        rec["cpu_baseline"] = cpu_baseline(inp, lmax, ch, n_nodes, min(args.cpu_sample_edges, n_edges))
+    print(json.dumps(rec))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,8 +1,9 @@
 """Emits ``generated/uvu_configs.inc``: straight-line device code for the channel-wise tensor product of
 each registered irreps configuration.
 
-For a configuration the Clebsch-Gordan table is a list of ``(coef, M, M1, M2, p)``.  The forward body
-evaluates, per output row ``M`` and weight path ``p``,
+For a configuration the Clebsch-Gordan table is a list of ``(coef, M, M1, M2, p)``.  Both bodies walk the
+table path by path (the weight row of a path is fetched when the path starts and its gradient handed over
+when the path ends).  The forward body evaluates, per weight path ``p`` and output row ``M``,
 
     t      = sum_{nnz in (p, M)} (coef * y[M2]) * x[M1]        (V channels per lane)
     out[M] += w[p] * t
@@ -49,45 +50,66 @@ def _lit(v: float) -> str:
     return float(np.float32(v)).hex() + "f"
 
 
+def _opaque(m2s) -> str:
+    """Per path, hide the harmonics it reads behind an empty asm statement.  Many (coefficient, harmonic)
+    products recur in several paths; without this the optimiser computes each once and keeps it alive across
+    the whole body, which costs far more registers than the multiplications it saves."""
+    return "    " + " ".join(f'asm volatile("" : "+v"(yy[{m}]));' for m in m2s)
+
+
 def emit_config(name: str, coo) -> str:
     T = coo.coef.shape[0]
-    # segments (p, M) in table order (k, M, i, j)
+    # (p, M) segments, path-major: the weight row of a path is needed only while that path is evaluated, and
+    # its gradient is complete when the path ends, so neither has to stay in registers.
     segs = OrderedDict()
     for t in range(T):
-        segs.setdefault((int(coo.q[t]), int(coo.p[t]), int(coo.M[t])), []).append(t)
+        segs.setdefault((int(coo.p[t]), int(coo.M[t])), []).append(t)
+    by_path = OrderedDict()
+    for (p, M), ts in sorted(segs.items()):
+        by_path.setdefault(p, []).append((M, ts))
     L = []
     a = L.append
     a(f"struct TP_{name} {{")
     a(f"  static constexpr int D1 = {coo.D1}, D2 = {coo.D2}, DO = {coo.DO}, P = {coo.P}, NNZ = {T};")
     a(f"  static constexpr unsigned long long FINGERPRINT = 0x{fingerprint(coo):016x}ull;")
     a(f"  static constexpr const char* NAME = \"{name}\";")
-    # ---- forward
-    a("  template <typename T, int V>")
-    a("  __device__ __forceinline__ static void fwd(const T (&x)[D1][V], const T (&y)[D2], const T (&w)[P][V],")
+    # ---- forward: o[M] += w[p] * sum_t (coef_t y[M2_t]) x[M1_t]
+    a("  // wload(p, w): fetch the V channels of weight path p")
+    a("  template <typename T, int V, class WLoad>")
+    a("  __device__ __forceinline__ static void fwd(const T (&x)[D1][V], const T (&y)[D2], WLoad&& wload,")
     a("                                             T (&o)[DO][V]) {")
-    a("    T t[V];")
-    for (q, p, M), ts in segs.items():
-        for n, t in enumerate(ts):
-            op = "mulv" if n == 0 else "fmav"
-            a(f"    {op}(t, T({_lit(coo.coef[t])}) * y[{coo.M2[t]}], x[{coo.M1[t]}]);")
-        a(f"    fmavv(o[{M}], w[{p}], t);")
+    a("    T t[V], w[V], yy[D2];")
+    a("    for (int j = 0; j < D2; ++j) yy[j] = y[j];")
+    for p, items in by_path.items():
+        a(f"    wload({p}, w);")
+        a(_opaque(sorted({int(coo.M2[t]) for _, ts in items for t in ts})))
+        for M, ts in items:
+            for n, t in enumerate(ts):
+                op = "mulv" if n == 0 else "fmav"
+                a(f"    {op}(t, T({_lit(coo.coef[t])}) * yy[{coo.M2[t]}], x[{coo.M1[t]}]);")
+            a(f"    fmavv(o[{M}], w, t);")
     a("  }")
-    # ---- backward; segments regrouped path-major so gw[p] completes early
-    a("  template <typename T, int V>")
-    a("  __device__ __forceinline__ static void bwd(const T (&x)[D1][V], const T (&y)[D2], const T (&w)[P][V],")
+    # ---- backward
+    a("  // gwsink(p, gw): consume the finished gradient of weight path p")
+    a("  template <typename T, int V, class WLoad, class GwSink>")
+    a("  __device__ __forceinline__ static void bwd(const T (&x)[D1][V], const T (&y)[D2], WLoad&& wload,")
     a("                                             const T (&g)[DO][V], T (&gx)[D1][V], T (&gy)[D2],")
-    a("                                             T (&gw)[P][V]) {")
-    a("    T t[V], gq[V], s;")
-    by_path = sorted(segs.items(), key=lambda kv: (kv[0][1], kv[0][2], kv[0][0]))
-    for (q, p, M), ts in by_path:
-        a(f"    mulvv(gq, g[{M}], w[{p}]);")
-        for n, t in enumerate(ts):
-            c, m1, m2 = _lit(coo.coef[t]), coo.M1[t], coo.M2[t]
-            a(f"    s = T({c}) * y[{m2}];")
-            a(f"    {'mulv' if n == 0 else 'fmav'}(t, s, x[{m1}]);")
-            a(f"    fmav(gx[{m1}], s, gq);")
-            a(f"    gy[{m2}] = fma(T({c}), dotv(x[{m1}], gq), gy[{m2}]);")
-        a(f"    fmavv(gw[{p}], g[{M}], t);")
+    a("                                             GwSink&& gwsink) {")
+    a("    T t[V], gq[V], w[V], gw[V], s, yy[D2];")
+    a("    for (int j = 0; j < D2; ++j) yy[j] = y[j];")
+    for p, items in by_path.items():
+        a(f"    wload({p}, w);")
+        a(_opaque(sorted({int(coo.M2[t]) for _, ts in items for t in ts})))
+        for k, (M, ts) in enumerate(items):
+            a(f"    mulvv(gq, g[{M}], w);")
+            for n, t in enumerate(ts):
+                c, m1, m2 = _lit(coo.coef[t]), coo.M1[t], coo.M2[t]
+                a(f"    s = T({c}) * yy[{m2}];")
+                a(f"    {'mulv' if n == 0 else 'fmav'}(t, s, x[{m1}]);")
+                a(f"    fmav(gx[{m1}], s, gq);")
+                a(f"    gy[{m2}] = fma(T({c}), dotv(x[{m1}], gq), gy[{m2}]);")
+            a(f"    {'mulvv' if k == 0 else 'fmavv'}(gw, g[{M}], t);")
+        a(f"    gwsink({p}, gw);")
     a("  }")
     a("};")
     return "\n".join(L)

@@ -2,10 +2,17 @@
 //
 // Work decomposition (wave64): a wavefront is split into 64/LPE "slots" of LPE lanes; a lane owns V
 // consecutive channels, so one slot covers LPE*V >= C channels of one row (edge) with V*sizeof(T)-byte
-// coalesced accesses.  In row mode every slot owns one batch row.  In segment mode a wavefront owns one
-// segment (destination node in the forward, source node in the backward) of a sorted edge list; its slots
-// walk the segment's edges round-robin, accumulate in registers, and the slots are summed with cross-lane
-// shuffles before a single store, so the edge -> node reduction needs no atomics and is deterministic.
+// coalesced accesses.  In row mode every slot owns one batch row.
+//
+// In segment mode (fused gather + tensor product + scatter-sum over an edge list sorted by segment id:
+// destination node in the forward, source node in the backward) every wavefront owns the same number of
+// consecutive sorted positions, so the load is balanced whatever the degree distribution.  In every step its
+// slots take the next consecutive positions that belong to one segment (a step never straddles a segment
+// boundary; slots past the boundary idle and the next step starts at the boundary), the per-edge result is
+// accumulated in registers, and when the segment id changes the accumulator is summed over the slots with
+// cross-lane shuffles and stored once.  A segment that lies entirely inside the wavefront's range is written to the
+// output directly; the (at most two) segments cut by the range boundary are written as partial rows to a
+// workspace and summed in a fixed order by uvu_fixup_kernel.  No atomics: results are deterministic.
 #include "cgtp_device.h"
 #include "cgtp_host.h"
 
@@ -22,235 +29,466 @@ struct UvuDev {
   T* gx;
   T* gy;
   T* gw;
-  T* ws;
+  T* ws;   // segment mode: partial rows (n_waves, 2, D, C)
+  T* wsw;  // per-wavefront partial sums of a shared weight's gradient (n_waves, P, C)
   const int64_t* ptr;
   const int64_t* perm;
   const int64_t* gather;
+  const int64_t* seg_ids;
+  const int32_t* wave_seg;  // segment mode: optional wavefront -> first segment table (segment-aligned ranges)
   int64_t n_rows, n_seg;
-  int C, lpe_log2, w_shared;
+  int C, lpe_log2, w_shared, pos_per_wave;
 };
 
-template <class TP, typename T, int V, bool SEG>
-__global__ void __launch_bounds__(256) uvu_fwd_kernel(const UvuDev<T> a) {
-  constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
-  const int lpe = 1 << a.lpe_log2, slots = kWave >> a.lpe_log2;
-  const int slot = lane >> a.lpe_log2, cl = lane & (lpe - 1);
-  const int c0 = (blockIdx.y * lpe + cl) * V;
-  const bool cok = c0 < a.C;
-  const int64_t C = a.C;
-
-  T w[P][V];
-  if (a.w_shared && cok) {
-#pragma unroll
-    for (int p = 0; p < P; ++p) load_vec<T, V>(w[p], a.w + p * C + c0);
+struct Lanes {
+  int lane, lpe, slots, slot, cl;
+  __device__ __forceinline__ explicit Lanes(int lpe_log2) {
+    lane = threadIdx.x & (kWave - 1);
+    lpe = 1 << lpe_log2;
+    slots = kWave >> lpe_log2;
+    slot = lane >> lpe_log2;
+    cl = lane & (lpe - 1);
   }
-  T acc[DO][V];
-#pragma unroll
-  for (int m = 0; m < DO; ++m)
-#pragma unroll
-    for (int v = 0; v < V; ++v) acc[m][v] = T(0);
+};
 
-  auto one_row = [&](int64_t e, int64_t xr) {
-    T x[D1][V], y[D2];
+template <typename T, int D, int V>
+__device__ __forceinline__ void zero_rows(T (&a)[D][V]) {
 #pragma unroll
-    for (int j = 0; j < D2; ++j) y[j] = a.y[e * D2 + j];
-    if (cok) {
+  for (int m = 0; m < D; ++m)
 #pragma unroll
-      for (int i = 0; i < D1; ++i) load_vec<T, V>(x[i], a.x + (xr * D1 + i) * C + c0);
-      if (!a.w_shared) {
-#pragma unroll
-        for (int p = 0; p < P; ++p) load_vec_stream<T, V>(w[p], a.w + (e * P + p) * C + c0);
-      }
-      TP::template fwd<T, V>(x, y, w, acc);
-    }
-  };
-
-  if constexpr (SEG) {
-    if (wave >= a.n_seg) return;
-    const int64_t beg = a.ptr[wave], end = a.ptr[wave + 1];
-    for (int64_t pos = beg + slot; pos < end; pos += slots) {
-      const int64_t e = a.perm ? a.perm[pos] : pos;
-      one_row(e, a.gather ? a.gather[e] : e);
-    }
-#pragma unroll
-    for (int m = 0; m < DO; ++m)
-#pragma unroll
-      for (int v = 0; v < V; ++v) acc[m][v] = cross_group_sum(acc[m][v], lpe);
-    if (slot == 0 && cok) {
-#pragma unroll
-      for (int m = 0; m < DO; ++m) store_vec<T, V>(a.out + (wave * DO + m) * C + c0, acc[m]);
-    }
-  } else {
-    const int64_t r = wave * slots + slot;
-    if (r < a.n_rows) {
-      one_row(r, a.gather ? a.gather[r] : r);
-      if (cok) {
-#pragma unroll
-        for (int m = 0; m < DO; ++m) store_vec_stream<T, V>(a.out + (r * DO + m) * C + c0, acc[m]);
-      }
-    }
-  }
+    for (int v = 0; v < V; ++v) a[m][v] = T(0);
 }
 
-// Backward.  WRED: the weight is shared over rows, so its gradient is summed over every row a wavefront
-// visits and written as one partial per wavefront into the workspace (partial_sum_kernel finishes the sum).
-template <class TP, typename T, int V, bool SEG, bool WRED>
-__global__ void __launch_bounds__(256) uvu_bwd_kernel(const UvuDev<T> a, int64_t n_waves) {
+// ---- row mode ------------------------------------------------------------------------------------------------
+template <class TP, typename T, int V>
+__global__ void __launch_bounds__(256) uvu_fwd_kernel(const UvuDev<T> a) {
   constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
-  const int lane = threadIdx.x & (kWave - 1);
+  const Lanes L(a.lpe_log2);
   const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
-  const int lpe = 1 << a.lpe_log2, slots = kWave >> a.lpe_log2;
-  const int slot = lane >> a.lpe_log2, cl = lane & (lpe - 1);
-  const int c0 = cl * V;
+  const int c0 = (blockIdx.y * L.lpe + L.cl) * V;
+  const int64_t C = a.C;
+  const int64_t r = wave * L.slots + L.slot;
+  if (r >= a.n_rows || c0 >= a.C) return;
+  const int64_t xr = a.gather ? a.gather[r] : r;
+  const int64_t wr = a.w_shared ? 0 : r;
+  T x[D1][V], y[D2], acc[DO][V];
+#pragma unroll
+  for (int j = 0; j < D2; ++j) y[j] = a.y[r * D2 + j];
+#pragma unroll
+  for (int i = 0; i < D1; ++i) load_vec<T, V>(x[i], a.x + (xr * D1 + i) * C + c0);
+  const T* wrow = a.w + wr * P * C + c0;
+  T w[P][V];  // every weight row is requested before the arithmetic starts: maximal memory-level parallelism
+#pragma unroll
+  for (int p = 0; p < P; ++p) load_vec_stream<T, V>(w[p], wrow + p * C);
+  zero_rows(acc);
+  TP::template fwd<T, V>(x, y, [&](int p, T (&wp)[V]) {
+#pragma unroll
+          for (int v = 0; v < V; ++v) wp[v] = w[p][v];
+        }, acc);
+#pragma unroll
+  for (int m = 0; m < DO; ++m) store_vec_stream<T, V>(a.out + (r * DO + m) * C + c0, acc[m]);
+}
+
+// What the backward does with the weight gradient.  kGwReduce: the weight is shared over rows, so its gradient
+// is summed over every row a wavefront visits and written as one partial per wavefront into the workspace
+// (partial_sum_kernel finishes the sum).  A compile-time choice keeps the generated body free of branches.
+enum { kGwNone = 0, kGwStore = 1, kGwReduce = 2 };
+
+template <class TP, typename T, int V, int GW>
+__global__ void __launch_bounds__(256, 2) uvu_bwd_kernel(const UvuDev<T> a, int64_t n_waves) {
+  constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
+  const Lanes L(a.lpe_log2);
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  const int c0 = L.cl * V;
   const bool cok = c0 < a.C;
   const int64_t C = a.C;
   if (wave >= n_waves) return;
 
-  T w[P][V], x[D1][V], gx[D1][V], gw[P][V];
-  if (a.w_shared && cok) {
-#pragma unroll
-    for (int p = 0; p < P; ++p) load_vec<T, V>(w[p], a.w + p * C + c0);
-  }
-  auto zero_gx = [&]() {
-#pragma unroll
-    for (int i = 0; i < D1; ++i)
-#pragma unroll
-      for (int v = 0; v < V; ++v) gx[i][v] = T(0);
-  };
-  auto zero_gw = [&]() {
-#pragma unroll
-    for (int p = 0; p < P; ++p)
-#pragma unroll
-      for (int v = 0; v < V; ++v) gw[p][v] = T(0);
-  };
-  zero_gx();
-  zero_gw();
-
-  // one edge / row: e = row of y, w, gy, gw; gr = row of grad_out; x already in registers
-  auto one_row = [&](int64_t e, int64_t gr) {
-    T g[DO][V], y[D2], gy[D2];
+  T gwacc[GW == kGwReduce ? P : 1][V], gx[D1][V];
+  zero_rows(gwacc);
+  zero_rows(gx);
+#pragma unroll 1
+  for (int64_t r = wave * L.slots + L.slot; r < a.n_rows; r += n_waves * L.slots) {
+    const int64_t gr = a.gather ? a.gather[r] : r;
+    T x[D1][V], g[DO][V], y[D2], gy[D2];
 #pragma unroll
     for (int j = 0; j < D2; ++j) {
-      y[j] = a.y[e * D2 + j];
+      y[j] = a.y[r * D2 + j];
       gy[j] = T(0);
     }
     if (cok) {
 #pragma unroll
+      for (int i = 0; i < D1; ++i) load_vec<T, V>(x[i], a.x + (r * D1 + i) * C + c0);
+#pragma unroll
       for (int m = 0; m < DO; ++m) load_vec<T, V>(g[m], a.g + (gr * DO + m) * C + c0);
-      if (!a.w_shared) {
+      const T* wrow = a.w + (a.w_shared ? 0 : r) * P * C + c0;
+      T w[P][V];  // every weight row is requested before the arithmetic starts: maximal memory-level parallelism
 #pragma unroll
-        for (int p = 0; p < P; ++p) load_vec_stream<T, V>(w[p], a.w + (e * P + p) * C + c0);
-      }
-      if constexpr (!WRED) zero_gw();
-      TP::template bwd<T, V>(x, y, w, g, gx, gy, gw);
-      if constexpr (!WRED) {
-        if (a.gw) {
+      for (int p = 0; p < P; ++p) load_vec_stream<T, V>(w[p], wrow + p * C);
+      T* gwrow = a.gw + r * P * C + c0;
+      TP::template bwd<T, V>(
+          x, y, [&](int p, T (&wp)[V]) {
 #pragma unroll
-          for (int p = 0; p < P; ++p) store_vec_stream<T, V>(a.gw + (e * P + p) * C + c0, gw[p]);
-        }
+          for (int v = 0; v < V; ++v) wp[v] = w[p][v];
+        }, g, gx, gy,
+          [&](int p, const T (&gwp)[V]) {
+            if constexpr (GW == kGwReduce) {
+#pragma unroll
+              for (int v = 0; v < V; ++v) gwacc[p][v] += gwp[v];
+            } else if constexpr (GW == kGwStore) {
+              store_vec_stream<T, V>(gwrow + p * C, gwp);
+            }
+          });
+      if (a.gx) {
+#pragma unroll
+        for (int i = 0; i < D1; ++i) store_vec_stream<T, V>(a.gx + (r * D1 + i) * C + c0, gx[i]);
       }
+      zero_rows(gx);
     }
     if (a.gy) {
 #pragma unroll
       for (int j = 0; j < D2; ++j) {
-        const T s = group_sum(gy[j], lpe);
-        if (cl == (j & (lpe - 1))) a.gy[e * D2 + j] = s;
-      }
-    }
-  };
-
-  if constexpr (SEG) {
-    if (cok) {
-#pragma unroll
-      for (int i = 0; i < D1; ++i) load_vec<T, V>(x[i], a.x + (wave * D1 + i) * C + c0);
-    }
-    const int64_t beg = a.ptr[wave], end = a.ptr[wave + 1];
-    for (int64_t pos = beg + slot; pos < end; pos += slots) {
-      const int64_t e = a.perm ? a.perm[pos] : pos;
-      one_row(e, a.gather ? a.gather[e] : e);
-    }
-    if (a.gx) {
-#pragma unroll
-      for (int i = 0; i < D1; ++i)
-#pragma unroll
-        for (int v = 0; v < V; ++v) gx[i][v] = cross_group_sum(gx[i][v], lpe);
-      if (slot == 0 && cok) {
-#pragma unroll
-        for (int i = 0; i < D1; ++i) store_vec<T, V>(a.gx + (wave * D1 + i) * C + c0, gx[i]);
-      }
-    }
-  } else {
-    for (int64_t r = wave * slots + slot; r < a.n_rows; r += n_waves * slots) {
-      if (cok) {
-#pragma unroll
-        for (int i = 0; i < D1; ++i) load_vec<T, V>(x[i], a.x + (r * D1 + i) * C + c0);
-      }
-      zero_gx();
-      one_row(r, a.gather ? a.gather[r] : r);
-      if (a.gx && cok) {
-#pragma unroll
-        for (int i = 0; i < D1; ++i) store_vec_stream<T, V>(a.gx + (r * D1 + i) * C + c0, gx[i]);
+        const T s = group_sum(gy[j], L.lpe);
+        if (L.cl == (j & (L.lpe - 1))) a.gy[r * D2 + j] = s;
       }
     }
   }
-  if constexpr (WRED) {
+  if constexpr (GW == kGwReduce) {
 #pragma unroll
     for (int p = 0; p < P; ++p)
 #pragma unroll
-      for (int v = 0; v < V; ++v) gw[p][v] = cross_group_sum(gw[p][v], lpe);
-    if (slot == 0 && cok) {
+      for (int v = 0; v < V; ++v) gwacc[p][v] = cross_group_sum(gwacc[p][v], L.lpe);
+    if (L.slot == 0 && cok) {
 #pragma unroll
-      for (int p = 0; p < P; ++p) store_vec<T, V>(a.ws + (wave * P + p) * C + c0, gw[p]);
+      for (int p = 0; p < P; ++p) store_vec<T, V>(a.wsw + (wave * P + p) * C + c0, gwacc[p]);
     }
+  }
+}
+
+// ---- segment mode ----------------------------------------------------------------------------------------------
+// Range [p0, p1) of sorted positions owned by one wavefront.  Two ways to cut the edge list:
+//  * aligned (wave_seg given): the wavefront owns the whole segments [s0, s1); every row it produces is final,
+//    and it also zero-fills the rows of empty segments in [s0, s1);
+//  * by position (wave_seg == nullptr): exactly per_wave positions each; the first / last segment of a range may
+//    continue in a neighbouring wavefront and then goes through a partial row (see uvu_fixup_kernel).
+struct SegRange {
+  int64_t p0, p1;
+  int s0, s1;                          // aligned mode: owned segments; else -1
+  bool first_complete, last_complete;  // does the first / last segment of the range begin / end inside it?
+  __device__ __forceinline__ SegRange(const int64_t* __restrict__ seg_ids, const int64_t* __restrict__ ptr,
+                                      const int32_t* __restrict__ wave_seg, int64_t wave, int per_wave,
+                                      int64_t n_rows) {
+    if (wave_seg) {
+      s0 = wave_seg[wave];
+      s1 = wave_seg[wave + 1];
+      p0 = ptr[s0];
+      p1 = ptr[s1];
+      first_complete = last_complete = true;
+    } else {
+      s0 = s1 = -1;
+      p0 = wave * per_wave;
+      p1 = p0 + per_wave < n_rows ? p0 + per_wave : n_rows;
+      first_complete = p0 == 0 || seg_ids[p0 - 1] != seg_ids[p0];
+      last_complete = p1 == n_rows || seg_ids[p1 - 1] != seg_ids[p1];
+    }
+  }
+};
+
+// Progress of a wavefront through its range.
+struct SegStep {
+  int cur = -1;       // segment being accumulated (-1: none yet)
+  bool first = true;  // no segment of this range has been flushed yet
+  int next_row;       // aligned mode: lowest owned segment whose row has not been written yet
+};
+
+// Rows [from, to) := 0, all lanes of the wavefront cooperating.
+template <typename T>
+__device__ __forceinline__ void zero_fill_rows(T* __restrict__ rows, int from, int to, int64_t row_len, int lane) {
+  if (!rows || from >= to) return;
+  T* p = rows + (int64_t)from * row_len;
+  const int64_t n = (int64_t)(to - from) * row_len;
+  for (int64_t i = lane; i < n; i += kWave) p[i] = T(0);
+}
+
+// Sum `acc` over the slots and store it as the row of segment `st.cur`: to `final_rows` if the segment is
+// complete in this wavefront's range, else to the wavefront's partial row 0 (range's first segment) or 1 (last).
+template <typename T, int D, int V>
+__device__ __forceinline__ void flush_segment(SegStep& st, T (&acc)[D][V], T* __restrict__ final_rows,
+                                              T* __restrict__ ws, int64_t wave, bool complete, const SegRange& R,
+                                              const Lanes& L, bool cok, int64_t C, int c0) {
+#pragma unroll
+  for (int m = 0; m < D; ++m)
+#pragma unroll
+    for (int v = 0; v < V; ++v) acc[m][v] = cross_group_sum(acc[m][v], L.lpe);
+  T* dst = complete ? final_rows + (int64_t)st.cur * D * C : ws + (wave * 2 + (st.first ? 0 : 1)) * D * C;
+  if (L.slot == 0 && cok && final_rows) {  // final_rows == nullptr: this result was not requested
+#pragma unroll
+    for (int m = 0; m < D; ++m) store_vec<T, V>(dst + m * C + c0, acc[m]);
+  }
+  if (R.s0 >= 0) {
+    zero_fill_rows(final_rows, st.next_row, st.cur, D * C, L.lane);
+    st.next_row = st.cur + 1;
+  }
+  st.first = false;
+  zero_rows(acc);
+}
+
+// Index data of up to 64 consecutive sorted positions [c0, c1), fetched with one coalesced load per array (lane i
+// holds position c0 + i) and handed to the slots with cross-lane shuffles, so that no step waits on a chain of
+// dependent index loads.
+struct SegIndexRegs {
+  int sid, edge, other;  // segment id, edge id, row of the gathered operand
+  int npos;
+  __device__ __forceinline__ SegIndexRegs(const int64_t* __restrict__ seg_ids, const int64_t* __restrict__ perm,
+                                          const int64_t* __restrict__ gather, int64_t c0, int64_t c1, int lane) {
+    npos = (int)(c1 - c0);
+    const int64_t p = c0 + (lane < npos ? lane : 0);
+    sid = (int)seg_ids[p];
+    edge = (int)(perm ? perm[p] : p);
+    other = (int)gather[p];
+  }
+};
+
+// One step of a wavefront's walk over its sorted positions: slot s looks at offset off0 + s of the current index
+// chunk; the step covers the leading slots whose segment id equals that of off0.  Flushes the accumulator when
+// the segment changes.
+template <typename T, int D, int V>
+__device__ __forceinline__ bool seg_step_begin(SegStep& st, T (&acc)[D][V], T* __restrict__ final_rows,
+                                               T* __restrict__ ws, const SegIndexRegs& I, int& off0, int& edge,
+                                               int& other, int64_t wave, const SegRange& R, const Lanes& L,
+                                               int lpe_log2, bool cok, int64_t C, int c0) {
+  const int off = off0 + L.slot;
+  const int src = off < I.npos ? off : off0;
+  const int sid = __shfl(I.sid, src, kWave);
+  edge = __shfl(I.edge, src, kWave);
+  other = __shfl(I.other, src, kWave);
+  const int lead = __shfl(I.sid, off0, kWave);
+  if (lead != st.cur) {
+    if (st.cur >= 0)
+      flush_segment<T, D, V>(st, acc, final_rows, ws, wave, st.first ? R.first_complete : true, R, L, cok, C, c0);
+    st.cur = lead;
+  }
+  const bool valid = off < I.npos && sid == lead;
+  off0 += __popcll(__ballot(valid)) >> lpe_log2;
+  return valid;
+}
+
+// End of a wavefront's range: flush the open segment and zero-fill the remaining owned empty segments.
+template <typename T, int D, int V>
+__device__ __forceinline__ void seg_finish(SegStep& st, T (&acc)[D][V], T* __restrict__ final_rows,
+                                           T* __restrict__ ws, int64_t wave, const SegRange& R, const Lanes& L,
+                                           bool cok, int64_t C, int c0) {
+  if (st.cur >= 0)
+    flush_segment<T, D, V>(st, acc, final_rows, ws, wave, (st.first ? R.first_complete : true) && R.last_complete, R,
+                           L, cok, C, c0);
+  if (R.s0 >= 0) zero_fill_rows(final_rows, st.next_row, R.s1, (int64_t)D * C, L.lane);
+}
+
+template <class TP, typename T, int V>
+__global__ void __launch_bounds__(256) uvu_seg_fwd_kernel(const UvuDev<T> a, int64_t n_waves) {
+  constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
+  const Lanes L(a.lpe_log2);
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (wave >= n_waves) return;
+  const int c0 = L.cl * V;
+  const bool cok = c0 < a.C;
+  const int64_t C = a.C;
+  const SegRange R(a.seg_ids, a.ptr, a.wave_seg, wave, a.pos_per_wave, a.n_rows);
+
+  T acc[DO][V];
+  zero_rows(acc);
+  SegStep st;
+  st.next_row = R.s0;
+  for (int64_t cb = R.p0; cb < R.p1; cb += kWave) {
+  const SegIndexRegs I(a.seg_ids, a.perm, a.gather, cb, cb + kWave < R.p1 ? cb + kWave : R.p1, L.lane);
+  for (int off0 = 0; off0 < I.npos;) {
+    int ei, oi;
+    if (seg_step_begin<T, DO, V>(st, acc, a.out, a.ws, I, off0, ei, oi, wave, R, L, a.lpe_log2, cok, C, c0)) {
+      const int64_t e = ei, xr = oi;
+      T x[D1][V], y[D2];
+#pragma unroll
+      for (int j = 0; j < D2; ++j) y[j] = a.y[e * D2 + j];
+      if (cok) {
+#pragma unroll
+        for (int i = 0; i < D1; ++i) load_vec<T, V>(x[i], a.x + (xr * D1 + i) * C + c0);
+        const T* wrow = a.w + (a.w_shared ? 0 : e) * P * C + c0;
+        T w[P][V];  // every weight row is requested before the arithmetic starts: maximal memory-level parallelism
+#pragma unroll
+        for (int p = 0; p < P; ++p) load_vec_stream<T, V>(w[p], wrow + p * C);
+        TP::template fwd<T, V>(x, y, [&](int p, T (&wp)[V]) {
+#pragma unroll
+          for (int v = 0; v < V; ++v) wp[v] = w[p][v];
+        }, acc);
+      }
+    }
+  }
+  }
+  seg_finish<T, DO, V>(st, acc, a.out, a.ws, wave, R, L, cok, C, c0);
+}
+
+template <class TP, typename T, int V, int GW>
+__global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, int64_t n_waves) {
+  constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
+  const Lanes L(a.lpe_log2);
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (wave >= n_waves) return;
+  const int c0 = L.cl * V;
+  const bool cok = c0 < a.C;
+  const int64_t C = a.C;
+  const SegRange R(a.seg_ids, a.ptr, a.wave_seg, wave, a.pos_per_wave, a.n_rows);
+
+  T gwacc[GW == kGwReduce ? P : 1][V], acc[D1][V];
+  zero_rows(gwacc);
+  zero_rows(acc);
+  SegStep st;
+  st.next_row = R.s0;
+  for (int64_t cb = R.p0; cb < R.p1; cb += kWave) {
+  const SegIndexRegs I(a.seg_ids, a.perm, a.gather, cb, cb + kWave < R.p1 ? cb + kWave : R.p1, L.lane);
+  for (int off0 = 0; off0 < I.npos;) {
+    int ei, oi;
+    if (seg_step_begin<T, D1, V>(st, acc, a.gx, a.ws, I, off0, ei, oi, wave, R, L, a.lpe_log2, cok, C, c0)) {
+      const int64_t e = ei, gr = oi;
+      T x[D1][V], g[DO][V], y[D2], gy[D2];
+#pragma unroll
+      for (int j = 0; j < D2; ++j) {
+        y[j] = a.y[e * D2 + j];
+        gy[j] = T(0);
+      }
+      if (cok) {
+#pragma unroll
+        for (int i = 0; i < D1; ++i) load_vec<T, V>(x[i], a.x + ((int64_t)st.cur * D1 + i) * C + c0);
+#pragma unroll
+        for (int m = 0; m < DO; ++m) load_vec<T, V>(g[m], a.g + (gr * DO + m) * C + c0);
+        const T* wrow = a.w + (a.w_shared ? 0 : e) * P * C + c0;
+        T w[P][V];  // every weight row is requested before the arithmetic starts: maximal memory-level parallelism
+#pragma unroll
+        for (int p = 0; p < P; ++p) load_vec_stream<T, V>(w[p], wrow + p * C);
+        T* gwrow = a.gw + e * P * C + c0;
+        TP::template bwd<T, V>(
+            x, y, [&](int p, T (&wp)[V]) {
+#pragma unroll
+          for (int v = 0; v < V; ++v) wp[v] = w[p][v];
+        }, g, acc, gy,
+            [&](int p, const T (&gwp)[V]) {
+              if constexpr (GW == kGwReduce) {
+#pragma unroll
+                for (int v = 0; v < V; ++v) gwacc[p][v] += gwp[v];
+              } else if constexpr (GW == kGwStore) {
+                store_vec_stream<T, V>(gwrow + p * C, gwp);
+              }
+            });
+      }
+      if (a.gy) {
+#pragma unroll
+        for (int j = 0; j < D2; ++j) {
+          const T s = group_sum(gy[j], L.lpe);
+          if (L.cl == (j & (L.lpe - 1))) a.gy[e * D2 + j] = s;
+        }
+      }
+    }
+  }
+  }
+  seg_finish<T, D1, V>(st, acc, a.gx, a.ws, wave, R, L, cok, C, c0);
+  if constexpr (GW == kGwReduce) {
+#pragma unroll
+    for (int p = 0; p < P; ++p)
+#pragma unroll
+      for (int v = 0; v < V; ++v) gwacc[p][v] = cross_group_sum(gwacc[p][v], L.lpe);
+    if (L.slot == 0 && cok) {
+#pragma unroll
+      for (int p = 0; p < P; ++p) store_vec<T, V>(a.wsw + (wave * P + p) * C + c0, gwacc[p]);
+    }
+  }
+}
+
+// Rows of segments cut by a wavefront boundary: rows[v] = sum of the partial rows of the wavefronts that
+// touch v, in ascending wavefront order; rows of empty segments are zeroed.  One wavefront per segment.
+template <typename T>
+__global__ void __launch_bounds__(256) uvu_fixup_kernel(T* __restrict__ rows, const T* __restrict__ ws,
+                                                        const int64_t* __restrict__ ptr, int64_t n_seg,
+                                                        int64_t row_len, int per_wave) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t v = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (v >= n_seg) return;
+  const int64_t b = ptr[v], e = ptr[v + 1];
+  T* dst = rows + v * row_len;
+  if (e == b) {
+    for (int64_t i = lane; i < row_len; i += kWave) dst[i] = T(0);
+    return;
+  }
+  const int64_t ka = b / per_wave, kb = (e - 1) / per_wave;
+  if (ka == kb) return;  // written in full by wavefront ka
+  const int64_t slot_a = (b % per_wave == 0) ? 0 : 1;
+  for (int64_t i = lane; i < row_len; i += kWave) {
+    T s = ws[(ka * 2 + slot_a) * row_len + i];
+    for (int64_t k = ka + 1; k <= kb; ++k) s += ws[(k * 2) * row_len + i];
+    dst[i] = s;
   }
 }
 
 // ---- host side ----------------------------------------------------------------------------------------------
 struct UvuPlan {
-  int V, lpe_log2;
-  int64_t n_waves;  // backward: wavefronts launched (== partial count when the weight gradient is reduced)
+  int V, lpe_log2, pos_per_wave;
+  int64_t n_waves;    // wavefronts of the main kernel
+  int64_t ws_elems;   // segment mode: elements of partial rows at the start of the workspace
+  int64_t wsw_elems;  // elements of shared-weight-gradient partials after them
 };
 
 template <typename T>
 using FwdFn = void (*)(const UvuDev<T>);
 template <typename T>
-using BwdFn = void (*)(const UvuDev<T>, int64_t);
+using WaveFn = void (*)(const UvuDev<T>, int64_t);
 
 template <typename T>
 struct UvuEntry {
   uint64_t fingerprint;
   int dims[5];
   const char* name;
-  FwdFn<T> fwd[2][2];     // [vector path][SEG]
-  BwdFn<T> bwd[2][2][2];  // [vector path][SEG][WRED]
+  int v_fwd, v_bwd;         // channels per lane of the vector paths
+  FwdFn<T> fwd[2];          // [vector path]
+  WaveFn<T> bwd[2][3];      // [vector path][weight-gradient mode]
+  WaveFn<T> seg_fwd[2];     // [vector path]
+  WaveFn<T> seg_bwd[2][3];  // [vector path][weight-gradient mode]
 };
 
+// Channels per lane of the vector path: the widest 16-byte-or-narrower vector whose per-lane register arrays
+// (inputs, weights, accumulators; two registers per double) leave room for at least two wavefronts per SIMD.
 template <typename T>
-struct VecWidth;
-template <> struct VecWidth<float> { static constexpr int value = 4; };
-template <> struct VecWidth<double> { static constexpr int value = 2; };
+constexpr int pick_v(int rows, int scalars, int budget) {
+  const int regs = sizeof(T) / 4;
+  for (int v = 16 / (int)sizeof(T); v > 1; v /= 2)
+    if ((rows * v + scalars) * regs <= budget) return v;
+  return 1;
+}
+template <class TP, typename T>
+constexpr int v_fwd() { return pick_v<T>(TP::D1 + TP::P + TP::DO, TP::D2, 150); }
+template <class TP, typename T>
+constexpr int v_bwd() { return pick_v<T>(2 * TP::D1 + TP::DO + 2 * TP::P, 2 * TP::D2, 236); }
 
 template <class TP, typename T>
 static UvuEntry<T> make_entry() {
-  constexpr int VW = VecWidth<T>::value;
+  constexpr int VF = v_fwd<TP, T>(), VB = v_bwd<TP, T>();
   UvuEntry<T> e;
   e.fingerprint = TP::FINGERPRINT;
   e.dims[0] = TP::D1; e.dims[1] = TP::D2; e.dims[2] = TP::DO; e.dims[3] = TP::P; e.dims[4] = TP::NNZ;
   e.name = TP::NAME;
-  e.fwd[0][0] = uvu_fwd_kernel<TP, T, 1, false>;
-  e.fwd[0][1] = uvu_fwd_kernel<TP, T, 1, true>;
-  e.fwd[1][0] = uvu_fwd_kernel<TP, T, VW, false>;
-  e.fwd[1][1] = uvu_fwd_kernel<TP, T, VW, true>;
-  e.bwd[0][0][0] = uvu_bwd_kernel<TP, T, 1, false, false>;
-  e.bwd[0][0][1] = uvu_bwd_kernel<TP, T, 1, false, true>;
-  e.bwd[0][1][0] = uvu_bwd_kernel<TP, T, 1, true, false>;
-  e.bwd[0][1][1] = uvu_bwd_kernel<TP, T, 1, true, true>;
-  e.bwd[1][0][0] = uvu_bwd_kernel<TP, T, VW, false, false>;
-  e.bwd[1][0][1] = uvu_bwd_kernel<TP, T, VW, false, true>;
-  e.bwd[1][1][0] = uvu_bwd_kernel<TP, T, VW, true, false>;
-  e.bwd[1][1][1] = uvu_bwd_kernel<TP, T, VW, true, true>;
+  e.v_fwd = VF; e.v_bwd = VB;
+  e.fwd[0] = uvu_fwd_kernel<TP, T, 1>;
+  e.fwd[1] = uvu_fwd_kernel<TP, T, VF>;
+  e.bwd[0][0] = uvu_bwd_kernel<TP, T, 1, kGwNone>;
+  e.bwd[0][1] = uvu_bwd_kernel<TP, T, 1, kGwStore>;
+  e.bwd[0][2] = uvu_bwd_kernel<TP, T, 1, kGwReduce>;
+  e.bwd[1][0] = uvu_bwd_kernel<TP, T, VB, kGwNone>;
+  e.bwd[1][1] = uvu_bwd_kernel<TP, T, VB, kGwStore>;
+  e.bwd[1][2] = uvu_bwd_kernel<TP, T, VB, kGwReduce>;
+  e.seg_fwd[0] = uvu_seg_fwd_kernel<TP, T, 1>;
+  e.seg_fwd[1] = uvu_seg_fwd_kernel<TP, T, VF>;
+  e.seg_bwd[0][0] = uvu_seg_bwd_kernel<TP, T, 1, kGwNone>;
+  e.seg_bwd[0][1] = uvu_seg_bwd_kernel<TP, T, 1, kGwStore>;
+  e.seg_bwd[0][2] = uvu_seg_bwd_kernel<TP, T, 1, kGwReduce>;
+  e.seg_bwd[1][0] = uvu_seg_bwd_kernel<TP, T, VB, kGwNone>;
+  e.seg_bwd[1][1] = uvu_seg_bwd_kernel<TP, T, VB, kGwStore>;
+  e.seg_bwd[1][2] = uvu_seg_bwd_kernel<TP, T, VB, kGwReduce>;
   return e;
 }
 
@@ -266,48 +504,73 @@ static const UvuEntry<T>* entries(int* count) {
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 static constexpr int64_t kMaxRowWaves = 2048;
+static constexpr int kDefaultPosPerWave = 32;
 
-static int uvu_plan(const cgtp_uvu_args* a, int backward, UvuPlan* plan) {
+static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan* plan) {
   if (!a) return CGTP_ERR_NULL;
   int n_cfg = 0;
-  entries<float>(&n_cfg);
+  const UvuEntry<float>* tab = entries<float>(&n_cfg);
   if (a->cfg < 0 || a->cfg >= n_cfg) return CGTP_ERR_CONFIG;
   if (a->dtype != CGTP_F32 && a->dtype != CGTP_F64) return CGTP_ERR_DTYPE;
-  if (a->C <= 0 || a->n_rows < 0 || a->n_seg < 0 || a->n_x_rows < 0) return CGTP_ERR_SHAPE;
+  if (a->C <= 0 || a->n_rows < 0 || a->n_seg < 0 || a->n_x_rows < 0 || a->pos_per_wave < 0) return CGTP_ERR_SHAPE;
   if (!a->x || !a->y || !a->w) return CGTP_ERR_NULL;
-  if (a->n_seg > 0 && !a->ptr) return CGTP_ERR_NULL;
-  if (a->n_seg == 0 && (a->ptr || a->perm)) return CGTP_ERR_SHAPE;
+  const bool seg = a->n_seg > 0;
+  if (seg && (!a->ptr || !a->seg_ids || !a->gather)) return CGTP_ERR_NULL;
+  if (!seg && (a->ptr || a->perm || a->seg_ids)) return CGTP_ERR_SHAPE;
+  if (seg && (a->n_seg >= (int64_t)1 << 31 || a->n_rows >= (int64_t)1 << 31 || a->n_x_rows >= (int64_t)1 << 31))
+    return CGTP_ERR_SHAPE;  // segment mode keeps ids and rows in 32-bit registers
+  if (seg && a->wave_seg && a->n_waves <= 0) return CGTP_ERR_SHAPE;
   if (backward) {
     if (!a->grad_out) return CGTP_ERR_NULL;
-    if (a->n_seg > 0 && a->n_x_rows != a->n_seg) return CGTP_ERR_SHAPE;
-    if (a->n_seg == 0 && a->n_x_rows != a->n_rows) return CGTP_ERR_SHAPE;
+    if (seg && a->n_x_rows != a->n_seg) return CGTP_ERR_SHAPE;
+    if (!seg && a->n_x_rows != a->n_rows) return CGTP_ERR_SHAPE;
   } else {
     if (!a->out) return CGTP_ERR_NULL;
-    if (!a->gather && a->n_x_rows != a->n_rows) return CGTP_ERR_SHAPE;
+    if (!seg && !a->gather && a->n_x_rows != a->n_rows) return CGTP_ERR_SHAPE;
   }
-  const int vw = a->dtype == CGTP_F32 ? 4 : 2;
-  bool vec = (a->C % vw) == 0 && aligned16(a->x) && aligned16(a->w);
+  int vw;
+  if (a->dtype == CGTP_F32) {
+    vw = backward ? tab[a->cfg].v_bwd : tab[a->cfg].v_fwd;
+  } else {
+    int n64 = 0;
+    const UvuEntry<double>* tab64 = entries<double>(&n64);
+    vw = backward ? tab64[a->cfg].v_bwd : tab64[a->cfg].v_fwd;
+  }
+  bool vec = vw > 1 && (a->C % vw) == 0 && aligned16(a->x) && aligned16(a->w);
   if (backward) {
     vec = vec && aligned16(a->grad_out) && (!a->grad_x || aligned16(a->grad_x)) &&
-          (!a->grad_w || aligned16(a->grad_w)) && (!a->workspace || aligned16(a->workspace));
+          (!a->grad_w || aligned16(a->grad_w));
   } else {
     vec = vec && aligned16(a->out);
   }
+  if (a->workspace) vec = vec && aligned16(a->workspace);
   plan->V = vec ? vw : 1;
   const int lanes = (a->C + plan->V - 1) / plan->V;
   int lg = 0;
   while ((1 << lg) < lanes && lg < 6) ++lg;
   plan->lpe_log2 = lg;
-  if (backward && lanes > kWave) return CGTP_ERR_SHAPE;  // channel reduction of grad_y stays inside one slot
+  // channel reduction of grad_y and the segment accumulators stay inside one slot
+  if ((backward || seg) && lanes > kWave) return CGTP_ERR_SHAPE;
   const int slots = kWave >> lg;
-  if (a->n_seg > 0) {
-    plan->n_waves = a->n_seg;
+  const int64_t row_d = backward ? tab[a->cfg].dims[0] : tab[a->cfg].dims[2];
+  const bool wred = backward && a->w_shared && a->grad_w;
+  plan->ws_elems = plan->wsw_elems = 0;
+  plan->pos_per_wave = 0;
+  if (seg && a->wave_seg) {
+    plan->n_waves = a->n_waves;  // segment-aligned ranges: every row is final, no partial rows
+  } else if (seg) {
+    int ppw = a->pos_per_wave > 0 ? a->pos_per_wave : kDefaultPosPerWave;
+    ppw = ((ppw + slots - 1) / slots) * slots;
+    plan->pos_per_wave = ppw;
+    plan->n_waves = (a->n_rows + ppw - 1) / ppw;
+    if (!backward || a->grad_x) plan->ws_elems = plan->n_waves * 2 * row_d * a->C;
   } else {
     int64_t nw = (a->n_rows + slots - 1) / slots;
-    if (backward && a->w_shared && a->grad_w && nw > kMaxRowWaves) nw = kMaxRowWaves;
+    if (wred && nw > kMaxRowWaves) nw = kMaxRowWaves;
     plan->n_waves = nw;
   }
-  if (backward && a->w_shared && a->grad_w && !a->workspace && plan->n_waves > 0) return CGTP_ERR_WORKSPACE;
+  if (wred) plan->wsw_elems = plan->n_waves * tab[a->cfg].dims[3] * a->C;
+  if (need_ws && plan->ws_elems + plan->wsw_elems > 0 && !a->workspace) return CGTP_ERR_WORKSPACE;
   return CGTP_OK;
 }
 
@@ -317,46 +580,66 @@ static UvuDev<T> to_dev(const cgtp_uvu_args* a, const UvuPlan& plan) {
   d.x = (const T*)a->x; d.y = (const T*)a->y; d.w = (const T*)a->w; d.out = (T*)a->out;
   d.g = (const T*)a->grad_out; d.gx = (T*)a->grad_x; d.gy = (T*)a->grad_y; d.gw = (T*)a->grad_w;
   d.ws = (T*)a->workspace;
-  d.ptr = a->ptr; d.perm = a->perm; d.gather = a->gather;
+  d.wsw = d.ws ? d.ws + plan.ws_elems : nullptr;
+  d.ptr = a->ptr; d.perm = a->perm; d.gather = a->gather; d.seg_ids = a->seg_ids; d.wave_seg = a->wave_seg;
   d.n_rows = a->n_rows; d.n_seg = a->n_seg;
-  d.C = a->C; d.lpe_log2 = plan.lpe_log2; d.w_shared = a->w_shared;
+  d.C = a->C; d.lpe_log2 = plan.lpe_log2; d.w_shared = a->w_shared; d.pos_per_wave = plan.pos_per_wave;
   return d;
+}
+
+static inline int launched() { return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH; }
+
+template <typename T>
+static int launch_fixup(T* rows, const UvuDev<T>& d, int64_t row_len, hipStream_t stream) {
+  hipLaunchKernelGGL(uvu_fixup_kernel<T>, dim3((unsigned)((d.n_seg + 3) / 4)), dim3(256), 0, stream, rows,
+                     (const T*)d.ws, d.ptr, d.n_seg, row_len, d.pos_per_wave);
+  return launched();
 }
 
 template <typename T>
 static int launch_fwd(const cgtp_uvu_args* a, const UvuPlan& plan, hipStream_t stream) {
   int n = 0;
   const UvuEntry<T>& e = entries<T>(&n)[a->cfg];
-  const bool seg = a->n_seg > 0;
-  const int slots = kWave >> plan.lpe_log2;
-  const int64_t waves = seg ? a->n_seg : (a->n_rows + slots - 1) / slots;
-  if (waves == 0) return CGTP_OK;
+  const UvuDev<T> d = to_dev<T>(a, plan);
+  const int vi = plan.V > 1;
+  if (a->n_seg > 0) {
+    if (plan.n_waves > 0) {
+      hipLaunchKernelGGL(e.seg_fwd[vi], dim3((unsigned)((plan.n_waves + 3) / 4)), dim3(256), 0, stream, d,
+                         plan.n_waves);
+      if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
+    }
+    return a->wave_seg ? CGTP_OK : launch_fixup<T>(d.out, d, (int64_t)e.dims[2] * a->C, stream);
+  }
+  if (plan.n_waves == 0) return CGTP_OK;
   const int chunk = (1 << plan.lpe_log2) * plan.V;
-  dim3 grid((unsigned)((waves + 3) / 4), (unsigned)((a->C + chunk - 1) / chunk));
-  hipLaunchKernelGGL(e.fwd[plan.V > 1][seg], grid, dim3(256), 0, stream, to_dev<T>(a, plan));
-  return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
+  dim3 grid((unsigned)((plan.n_waves + 3) / 4), (unsigned)((a->C + chunk - 1) / chunk));
+  hipLaunchKernelGGL(e.fwd[vi], grid, dim3(256), 0, stream, d);
+  return launched();
 }
 
 template <typename T>
 static int launch_bwd(const cgtp_uvu_args* a, const UvuPlan& plan, hipStream_t stream) {
   int n = 0;
   const UvuEntry<T>& e = entries<T>(&n)[a->cfg];
+  const UvuDev<T> d = to_dev<T>(a, plan);
+  const int vi = plan.V > 1;
   const bool seg = a->n_seg > 0;
   const bool wred = a->w_shared && a->grad_w;
+  const int64_t w_elems = (int64_t)e.dims[3] * a->C;
   if (plan.n_waves == 0) {
-    if (wred) (void)hipMemsetAsync(a->grad_w, 0, sizeof(T) * e.dims[3] * a->C, stream);
-    return CGTP_OK;
+    if (wred) (void)hipMemsetAsync(a->grad_w, 0, sizeof(T) * w_elems, stream);
+  } else {
+    const int gwm = !a->grad_w ? kGwNone : (wred ? kGwReduce : kGwStore);
+    hipLaunchKernelGGL(seg ? e.seg_bwd[vi][gwm] : e.bwd[vi][gwm], dim3((unsigned)((plan.n_waves + 3) / 4)),
+                       dim3(256), 0, stream, d, plan.n_waves);
+    if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
+    if (wred) {
+      hipLaunchKernelGGL(partial_sum_kernel<T>, dim3((unsigned)((w_elems + 255) / 256)), dim3(256), 0, stream,
+                         (const T*)d.wsw, (T*)a->grad_w, plan.n_waves, w_elems);
+      if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
+    }
   }
-  dim3 grid((unsigned)((plan.n_waves + 3) / 4));
-  hipLaunchKernelGGL(e.bwd[plan.V > 1][seg][wred], grid, dim3(256), 0, stream, to_dev<T>(a, plan),
-                     plan.n_waves);
-  if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
-  if (wred) {
-    const int64_t nel = (int64_t)e.dims[3] * a->C;
-    hipLaunchKernelGGL(partial_sum_kernel<T>, dim3((unsigned)((nel + 255) / 256)), dim3(256), 0, stream,
-                       (const T*)a->workspace, (T*)a->grad_w, plan.n_waves, nel);
-    if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
-  }
+  if (seg && a->grad_x && !a->wave_seg) return launch_fixup<T>(d.gx, d, (int64_t)e.dims[0] * a->C, stream);
   return CGTP_OK;
 }
 
@@ -391,25 +674,18 @@ uint64_t cgtp_uvu_describe(int cfg, int32_t* dims) {
 
 int cgtp_uvu_validate(const cgtp_uvu_args* args, int backward) {
   UvuPlan plan;
-  return uvu_plan(args, backward, &plan);
+  return uvu_plan(args, backward, false, &plan);
 }
 
-int64_t cgtp_uvu_bwd_workspace_bytes(const cgtp_uvu_args* a) {
-  if (!a || !(a->w_shared && a->grad_w)) return 0;
-  cgtp_uvu_args tmp = *a;
-  static char dummy[16] __attribute__((aligned(16)));
-  if (!tmp.workspace) tmp.workspace = dummy;
+int64_t cgtp_uvu_workspace_bytes(const cgtp_uvu_args* a, int backward) {
   UvuPlan plan;
-  if (uvu_plan(&tmp, 1, &plan) != CGTP_OK) return 0;
-  int32_t dims[5];
-  cgtp_uvu_describe(a->cfg, dims);
-  const int64_t esz = a->dtype == CGTP_F32 ? 4 : 8;
-  return plan.n_waves * dims[3] * (int64_t)a->C * esz;
+  if (uvu_plan(a, backward, false, &plan) != CGTP_OK) return 0;
+  return (plan.ws_elems + plan.wsw_elems) * (a->dtype == CGTP_F32 ? 4 : 8);
 }
 
 int cgtp_uvu_fwd(const cgtp_uvu_args* a, void* stream) {
   UvuPlan plan;
-  const int st = uvu_plan(a, 0, &plan);
+  const int st = uvu_plan(a, 0, true, &plan);
   if (st != CGTP_OK) return st;
   return a->dtype == CGTP_F32 ? launch_fwd<float>(a, plan, (hipStream_t)stream)
                               : launch_fwd<double>(a, plan, (hipStream_t)stream);
@@ -417,7 +693,7 @@ int cgtp_uvu_fwd(const cgtp_uvu_args* a, void* stream) {
 
 int cgtp_uvu_bwd(const cgtp_uvu_args* a, void* stream) {
   UvuPlan plan;
-  const int st = uvu_plan(a, 1, &plan);
+  const int st = uvu_plan(a, 1, true, &plan);
   if (st != CGTP_OK) return st;
   return a->dtype == CGTP_F32 ? launch_bwd<float>(a, plan, (hipStream_t)stream)
                               : launch_bwd<double>(a, plan, (hipStream_t)stream);

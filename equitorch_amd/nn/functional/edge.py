@@ -42,6 +42,11 @@ class EdgePlan:
         self.num_edges = src.shape[0]
         self.perm_dst, self.ptr_dst = self._sorted(self.dst, self.num_nodes)
         self.perm_src, self.ptr_src = self._sorted(self.src, self.num_src_nodes)
+        # per-sorted-position views for the fused kernels: segment id and the row gathered at the other end
+        self.fwd_index = kernels.SegIndex(self.ptr_dst, self.perm_dst, self.dst[self.perm_dst].contiguous(),
+                                          self.src[self.perm_dst].contiguous())
+        self.bwd_index = kernels.SegIndex(self.ptr_src, self.perm_src, self.src[self.perm_src].contiguous(),
+                                          self.dst[self.perm_src].contiguous())
 
     @staticmethod
     def _sorted(key: Tensor, n: int):
@@ -60,9 +65,7 @@ class _EdgeUvuCompiled(Function):
     @staticmethod
     def forward(ctx, x: Tensor, sh: Tensor, w: Tensor, plan: EdgePlan, tp_info: TensorProductInfo, cfg: int):
         dims = kernels.uvu_dims(cfg)
-        out = kernels.uvu_forward(cfg, dims, x, sh, w, ptr_=plan.ptr_dst, perm=plan.perm_dst, gather=plan.src)
-        if out is None:
-            raise _lib.CgtpError("fused edge tensor product not launchable for these shapes")
+        out = kernels.uvu_forward(cfg, dims, x, sh, w, seg=plan.fwd_index)
         ctx.save_for_backward(x, sh, w)
         ctx.plan, ctx.cfg, ctx.dims = plan, cfg, dims
         return out
@@ -73,9 +76,7 @@ class _EdgeUvuCompiled(Function):
         x, sh, w = ctx.saved_tensors
         plan = ctx.plan
         res = kernels.uvu_backward(ctx.cfg, ctx.dims, x, sh, w, g.contiguous(), ctx.needs_input_grad[:3],
-                                   ptr_=plan.ptr_src, perm=plan.perm_src, gather=plan.dst)
-        if res is None:
-            raise _lib.CgtpError("fused edge backward not launchable for these shapes")
+                                   seg=plan.bwd_index)
         return (*res, None, None, None)
 
 

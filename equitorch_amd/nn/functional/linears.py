@@ -30,8 +30,6 @@ class _UvuCompiled(Function):
     @staticmethod
     def forward(ctx, x: Tensor, y: Tensor, w: Tensor, tp_info: TensorProductInfo, cfg: int):
         out = kernels.uvu_forward(cfg, kernels.uvu_dims(cfg), x, y, w)
-        if out is None:
-            raise _lib.CgtpError("specialised forward not launchable")
         ctx.save_for_backward(x, y, w)
         ctx.tp_info, ctx.cfg = tp_info, cfg
         return out
@@ -49,8 +47,6 @@ class _UvuCompiled(Function):
                 gw = tri(spec.grad_spec(2), (V, S, V), V, x, y, g, out_shared=(w.ndim == 2)) if need[2] else None
             return gx, gy, gw, None, None
         res = kernels.uvu_backward(ctx.cfg, kernels.uvu_dims(ctx.cfg), x, y, w, g.contiguous(), need)
-        if res is None:
-            raise _lib.CgtpError("specialised backward not launchable after a specialised forward")
         return (*res, None, None)
 
 

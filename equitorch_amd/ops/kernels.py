@@ -110,70 +110,100 @@ def segment_sum(inp: Tensor, scale: Optional[Tensor], index: Optional[Tensor], s
 
 
 # ---- specialised uvu ----------------------------------------------------------------------------------------
-def _uvu_args(cfg: int, x: Tensor, y: Tensor, w: Tensor, n_rows: int, ptr_, perm, gather) -> UvuArgs:
+class SegIndex:
+    """Per-sorted-position index arrays of the segment mode (all int64, same device)."""
+
+    def __init__(self, ptr: Tensor, perm: Optional[Tensor], seg_ids: Tensor, gather: Tensor,
+                 positions_per_wave: int = 32):
+        self.ptr, self.perm, self.seg_ids, self.gather = ptr, perm, seg_ids, gather
+        self.wave_seg = self.aligned_ranges(ptr, positions_per_wave)
+
+    @staticmethod
+    def aligned_ranges(ptr: Tensor, positions_per_wave: int) -> Optional[Tensor]:
+        """Cut the sorted list at segment boundaries into ranges of about ``positions_per_wave`` positions:
+        int32 ``[n_ranges + 1]`` segment indices (first 0, last n_seg).  Range k starts at the first segment
+        whose first position is >= k * positions_per_wave.  Returns None (ranges by position are used instead)
+        when a segment is so large that aligned ranges would be badly unbalanced."""
+        n_seg, n_pos = ptr.shape[0] - 1, int(ptr[-1])
+        if n_seg == 0:
+            return None
+        if n_pos and int((ptr[1:] - ptr[:-1]).max()) > 8 * positions_per_wave:
+            return None
+        targets = torch.arange(0, max(n_pos, 1), positions_per_wave, device=ptr.device, dtype=ptr.dtype)
+        cuts = torch.searchsorted(ptr[:-1].contiguous(), targets)
+        cuts = torch.unique_consecutive(torch.cat([cuts.new_zeros(1), cuts, cuts.new_full((1,), n_seg)]))
+        return cuts.to(torch.int32).contiguous()
+
+
+def _uvu_args(cfg: int, x: Tensor, y: Tensor, w: Tensor, seg: Optional[SegIndex], gather: Optional[Tensor],
+              pos_per_wave: int = 0) -> UvuArgs:
     a = UvuArgs()
     a.cfg, a.dtype, a.C = cfg, _lib.dtype_code(x.dtype), x.shape[-1]
     a.w_shared = int(w.ndim == 2)
-    a.n_rows, a.n_x_rows = n_rows, x.shape[0]
-    a.n_seg = 0 if ptr_ is None else ptr_.shape[0] - 1
-    a.ptr, a.perm, a.gather = _lib.ptr(ptr_), _lib.ptr(perm), _lib.ptr(gather)
+    a.n_rows, a.n_x_rows = y.shape[0], x.shape[0]
+    if seg is not None:
+        a.n_seg = seg.ptr.shape[0] - 1
+        a.ptr, a.perm, a.seg_ids, a.gather = seg.ptr.data_ptr(), _lib.ptr(seg.perm), seg.seg_ids.data_ptr(), \
+            seg.gather.data_ptr()
+        a.pos_per_wave = pos_per_wave
+        if seg.wave_seg is not None and pos_per_wave == 0:
+            a.wave_seg, a.n_waves = seg.wave_seg.data_ptr(), seg.wave_seg.shape[0] - 1
+    else:
+        a.gather = _lib.ptr(gather)
     a.x, a.y, a.w = x.data_ptr(), y.data_ptr(), w.data_ptr()
     return a
+
+
+def _workspace(a: UvuArgs, backward: int, device):
+    nbytes = int(_lib.lib.cgtp_uvu_workspace_bytes(C.byref(a), backward))
+    if nbytes == 0:
+        return None
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    a.workspace = ws.data_ptr()
+    return ws
 
 
 def uvu_launchable(cfg: int, x: Tensor, y: Tensor, w: Tensor, segments: bool = False) -> bool:
     """True when both the specialised forward and backward accept these operands (dtype, channel count,
     alignment); outputs are torch allocations and therefore always aligned."""
+    if x.shape[0] == 0 or y.shape[0] == 0:
+        return False
     a = UvuArgs()
     a.cfg, a.dtype, a.C = cfg, _lib.dtype_code(x.dtype), x.shape[-1]
     a.w_shared = int(w.ndim == 2)
     a.n_rows = y.shape[0]
     dummy = 256
+    a.n_x_rows = x.shape[0]
     if segments:
-        a.n_seg, a.n_x_rows, a.ptr, a.gather = x.shape[0], x.shape[0], dummy, dummy
-    else:
-        a.n_x_rows = x.shape[0]
+        a.n_seg, a.ptr, a.gather, a.seg_ids = x.shape[0], dummy, dummy, dummy
     a.x, a.y, a.w = x.data_ptr() or dummy, y.data_ptr() or dummy, w.data_ptr() or dummy
-    a.out = a.grad_out = a.grad_x = a.grad_y = a.grad_w = a.workspace = dummy
-    if x.shape[0] == 0 or y.shape[0] == 0:
-        return False
-    if _lib.lib.cgtp_uvu_validate(C.byref(a), 1) != 0:
-        return False
-    return True
+    a.out = a.grad_out = a.grad_x = a.grad_y = a.grad_w = dummy
+    return _lib.lib.cgtp_uvu_validate(C.byref(a), 1) == 0
 
 
-def uvu_forward(cfg: int, dims, x: Tensor, y: Tensor, w: Tensor, ptr_: Optional[Tensor] = None,
-                perm: Optional[Tensor] = None, gather: Optional[Tensor] = None) -> Optional[Tensor]:
-    """Specialised forward; returns None when the launch conditions are not met (caller falls back to the
-    table-driven kernel)."""
-    n_rows = y.shape[0]
-    a = _uvu_args(cfg, x, y, w, n_rows, ptr_, perm, gather)
-    n_out_rows = a.n_seg if ptr_ is not None else n_rows
+def uvu_forward(cfg: int, dims, x: Tensor, y: Tensor, w: Tensor, seg: Optional[SegIndex] = None,
+                gather: Optional[Tensor] = None, pos_per_wave: int = 0) -> Tensor:
+    """Compiled-table forward.  Row mode: ``out[r] = TP(x[gather[r] | r], y[r], w[r])``.  Segment mode:
+    ``out[s] = sum_{q in segment s} TP(x[seg.gather[q]], y[e_q], w[e_q])``."""
+    a = _uvu_args(cfg, x, y, w, seg, gather, pos_per_wave)
+    n_out_rows = a.n_seg if seg is not None else y.shape[0]
     out = torch.empty((n_out_rows, dims[2], x.shape[-1]), dtype=x.dtype, device=x.device)
     a.out = out.data_ptr()
-    if _lib.lib.cgtp_uvu_validate(C.byref(a), 0) != 0:
-        return None
+    ws = _workspace(a, 0, x.device)
     _lib.check(_lib.lib.cgtp_uvu_fwd(C.byref(a), _lib.stream_ptr(x.device)), "cgtp_uvu_fwd")
     return out
 
 
-def uvu_backward(cfg: int, dims, x: Tensor, y: Tensor, w: Tensor, g: Tensor, need, ptr_=None, perm=None,
-                 gather=None):
-    """Specialised backward -> (grad_x, grad_y, grad_w) (None where not needed), or None if not launchable."""
-    n_rows = y.shape[0]
-    a = _uvu_args(cfg, x, y, w, n_rows, ptr_, perm, gather)
+def uvu_backward(cfg: int, dims, x: Tensor, y: Tensor, w: Tensor, g: Tensor, need, seg: Optional[SegIndex] = None,
+                 gather: Optional[Tensor] = None, pos_per_wave: int = 0):
+    """Compiled-table backward -> (grad_x, grad_y, grad_w), None where ``need`` is False."""
+    a = _uvu_args(cfg, x, y, w, seg, gather, pos_per_wave)
     a.grad_out = g.data_ptr()
     gx = torch.empty_like(x) if need[0] else None
     gy = torch.empty_like(y) if need[1] else None
     gw = torch.empty_like(w) if need[2] else None
     a.grad_x, a.grad_y, a.grad_w = _lib.ptr(gx), _lib.ptr(gy), _lib.ptr(gw)
-    ws = None
-    if a.w_shared and need[2]:
-        nbytes = int(_lib.lib.cgtp_uvu_bwd_workspace_bytes(C.byref(a)))
-        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
-        a.workspace = ws.data_ptr()
-    if _lib.lib.cgtp_uvu_validate(C.byref(a), 1) != 0:
-        return None
+    ws = _workspace(a, 1, x.device)
     _lib.check(_lib.lib.cgtp_uvu_bwd(C.byref(a), _lib.stream_ptr(x.device)), "cgtp_uvu_bwd")
     return gx, gy, gw
 

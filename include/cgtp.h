@@ -101,8 +101,17 @@ int cgtp_segment_sum(const void* in, const void* scale, const int64_t* index, co
  * in the backward entry, for the seven launches of its backward (:44-83).  The Clebsch-Gordan table is
  * compiled into the kernel; cgtp_uvu_find() maps a table fingerprint to a config id (or -1).
  *
- * Segment mode (ptr != NULL) additionally fuses the gather x[xrow[e]] and the scatter-sum over a sorted edge
- * list: segment s owns sorted positions [ptr[s], ptr[s+1]); position q is edge e = perm ? perm[q] : q.
+ * Segment mode (n_seg > 0) additionally fuses a gather of the node operand and the scatter-sum over an edge
+ * list sorted by segment id (destination node in the forward, source node in the backward).  All per-edge
+ * index arrays are then indexed by SORTED POSITION q: the edge is e = perm ? perm[q] : q (rows of y, W, grad_y,
+ * grad_w), seg_ids[q] is its (ascending) segment id, gather[q] the row of the gathered operand (forward: row
+ * of x; backward: row of grad_out; in the backward x is read at row seg_ids[q]).  ptr is the CSR pointer of
+ * seg_ids.  The sorted list is cut into one range per wavefront in one of two ways.  With wave_seg (n_waves + 1
+ * ascending segment indices, first 0, last n_seg) wavefront k owns the whole segments [wave_seg[k],
+ * wave_seg[k+1]) and writes their rows directly (zero rows for empty segments); the caller balances the ranges
+ * (about 32 positions each works well).  Without it every wavefront owns pos_per_wave consecutive positions and
+ * segments cut by a range boundary go through partial rows in the workspace and a fix-up kernel.  Either way
+ * there are no atomics and results are deterministic.
  */
 int cgtp_uvu_num_configs(void);
 int cgtp_uvu_find(uint64_t fingerprint);
@@ -116,11 +125,17 @@ typedef struct cgtp_uvu_args {
   int32_t w_shared;        /* 1: W is (P, C); 0: W is (n_rows, P, C)                               */
   int64_t n_rows;          /* batch rows / edges                                                   */
   int64_t n_x_rows;        /* rows of x (== n_rows unless gathered / segment-owned)                */
-  int64_t n_seg;           /* number of segments (nodes); 0 = no segment mode                      */
-  const int64_t* ptr;      /* [n_seg + 1] sorted-position CSR pointer, or NULL                     */
-  const int64_t* perm;     /* [n_rows] sorted position -> edge id, or NULL = identity              */
-  const int64_t* gather;   /* [n_rows] fwd: x row per edge; bwd: grad_out row per edge; or NULL    */
-  const void* x;           /* fwd: (n_x_rows, D1, C).  bwd: same; in segment mode row = segment id */
+  int64_t n_seg;           /* number of segments (nodes); 0 = row mode                             */
+  const int64_t* ptr;      /* segment mode: [n_seg + 1] CSR pointer over sorted positions          */
+  const int64_t* perm;     /* segment mode: [n_rows] sorted position -> edge id, NULL = identity   */
+  const int64_t* seg_ids;  /* segment mode: [n_rows] sorted position -> segment id, ascending      */
+  const int64_t* gather;   /* [n_rows] row of the gathered operand (fwd: x, bwd: grad_out); row mode: per
+                              row, optional; segment mode: per sorted position, required           */
+  int32_t pos_per_wave;    /* segment mode without wave_seg: positions per wavefront; 0 = 32       */
+  int32_t _pad;
+  const int32_t* wave_seg; /* segment mode, optional: [n_waves + 1] first segment of every wavefront */
+  int64_t n_waves;         /* number of ranges in wave_seg                                         */
+  const void* x;           /* (n_x_rows, D1, C); bwd segment mode: n_x_rows == n_seg               */
   const void* y;           /* (n_rows, D2)                                                         */
   const void* w;           /* (n_rows | 1, P, C)                                                   */
   /* forward */
@@ -130,13 +145,21 @@ typedef struct cgtp_uvu_args {
   void* grad_x;            /* (n_seg ? n_seg : n_rows, D1, C) or NULL                              */
   void* grad_y;            /* (n_rows, D2) or NULL                                                 */
   void* grad_w;            /* (n_rows | 1, P, C) or NULL                                           */
-  void* workspace;         /* bwd with w_shared && grad_w: cgtp_uvu_bwd_workspace_bytes() bytes    */
+  void* workspace;         /* cgtp_uvu_workspace_bytes() bytes (segment mode, or bwd of a shared W) */
 } cgtp_uvu_args;
 
 int cgtp_uvu_validate(const cgtp_uvu_args* args, int backward);
-int64_t cgtp_uvu_bwd_workspace_bytes(const cgtp_uvu_args* args);
+/* Bytes of workspace the forward (backward = 0) or backward (1) launch of `args` needs; 0 if none. */
+int64_t cgtp_uvu_workspace_bytes(const cgtp_uvu_args* args, int backward);
 int cgtp_uvu_fwd(const cgtp_uvu_args* args, void* stream);
 int cgtp_uvu_bwd(const cgtp_uvu_args* args, void* stream);
+
+/* ---- streaming kernels of known traffic (counter calibration, achievable-bandwidth reference) ------------
+ * No counterpart in the reference.  copy: reads n_bytes and writes n_bytes; read: reads n_bytes.
+ * n_bytes must be a multiple of 16 and the pointers 16-byte aligned.
+ */
+int cgtp_membench_copy(void* dst, const void* src, int64_t n_bytes, void* stream);
+int cgtp_membench_read(const void* src, void* sink, int64_t n_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -98,3 +98,42 @@ def test_edge_fused_small(device, shared_w):
     for name, g, r in zip(("out", "grad_x", "grad_sh", "grad_w"), (out, xd.grad, shd.grad, wd.grad),
                           (ref_out, *ref_grads)):
         assert_close(g, r, 1e-5, f"edge fused shared={shared_w} {name}")
+
+
+@pytest.mark.parametrize("pos_per_wave", [4, 8, 32, 60])
+@pytest.mark.parametrize("hub", [False, True])
+def test_edge_fused_range_modes(device, pos_per_wave, hub):
+    """Ranges cut by position (partial rows + fix-up kernel) must give the same rows as segment-aligned ranges,
+    including with a hub node whose segment spans many wavefronts and with empty segments."""
+    from equitorch_amd.nn.functional import EdgePlan
+    from equitorch_amd.ops import kernels
+    irreps = SH[2]
+    mod = _module(irreps, irreps, irreps).to(device)
+    cfg = kernels.uvu_config_of(mod.tp_info_forward)
+    dims = kernels.uvu_dims(cfg)
+    gen = torch.Generator().manual_seed(9)
+    n_nodes, n_edges, ch = 61, 900, 32
+    src = torch.randint(0, n_nodes, (n_edges,), generator=gen)
+    dst = torch.randint(0, n_nodes, (n_edges,), generator=gen)
+    if hub:
+        dst[100:600] = 17
+        src[300:700] = 5
+    x, sh, w = tp_inputs(n_edges, 9, 2, 11, ch, False, seed=10)
+    x = x[:n_nodes].contiguous()
+    ct = torch.randn(n_nodes, 9, ch, generator=gen)
+    plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
+    xd, shd, wd, ctd = (t.to(device) for t in (x, sh, w, ct))
+    T = ref_ops.dense_coupling(irreps, irreps, irreps)
+
+    def ref_fn(T, x, sh, w):
+        return ref_ops.scatter_sum(ref_ops.dense_u1u(T, x.index_select(0, src), sh, w), dst, n_nodes)
+    ref_out, ref_grads = ref_ops.dense_grads(ref_fn, T, (x, sh, w), ct)
+    out = kernels.uvu_forward(cfg, dims, xd, shd, wd, seg=plan.fwd_index, pos_per_wave=pos_per_wave)
+    gx, gy, gw = kernels.uvu_backward(cfg, dims, xd, shd, wd, ctd, (True, True, True), seg=plan.bwd_index,
+                                      pos_per_wave=pos_per_wave)
+    for name, g, r in zip(("out", "grad_x", "grad_sh", "grad_w"), (out, gx, gy, gw), (ref_out, *ref_grads)):
+        assert_close(g, r, 1e-5, f"ppw={pos_per_wave} hub={hub} {name}")
+    if not hub:
+        assert plan.fwd_index.wave_seg is not None
+    out_a = kernels.uvu_forward(cfg, dims, xd, shd, wd, seg=plan.fwd_index)
+    assert_close(out_a, ref_out, 1e-5, "aligned out")
