@@ -1,0 +1,96 @@
+"""The C-ABI library: loads, exports every symbol declared in include/cgtp.h, and its host-only validation
+entry points report the documented status codes (no kernel is launched here)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "equitorch_amd", "lib", "libcgtp.so")
+pytestmark = pytest.mark.skipif(not os.path.exists(LIB), reason="libcgtp.so not built (run __graft_entry__.build())")
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "cgtp.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cgtp_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported():
+    lib = C.CDLL(LIB)
+    names = declared_symbols()
+    assert len(names) >= 15
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/cgtp.h but not exported"
+
+
+def test_version_and_status_strings():
+    from equitorch_amd import _lib
+    assert _lib.lib.cgtp_version() >= 1
+    assert _lib.lib.cgtp_status_string(0) == b"ok"
+    assert len({_lib.lib.cgtp_status_string(i) for i in range(9)}) == 9
+
+
+def test_compiled_tables_match_python_fingerprints():
+    from equitorch_amd import _lib
+    from equitorch_amd._tables import fingerprint, tp_coo
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    n = _lib.lib.cgtp_uvu_num_configs()
+    assert n >= 3
+    irr = Irreps("0e+1o+2e")
+    coo = tp_coo(tp_infos(irr, irr, irr)[0])
+    cfg = _lib.lib.cgtp_uvu_find(C.c_uint64(fingerprint(coo)))
+    assert cfg >= 0
+    dims = (C.c_int32 * 5)()
+    assert _lib.lib.cgtp_uvu_describe(cfg, dims) == fingerprint(coo)
+    assert tuple(dims) == (9, 9, 9, 11, 83)
+    assert _lib.lib.cgtp_uvu_find(C.c_uint64(12345)) == -1
+
+
+def test_host_side_validation_codes():
+    from equitorch_amd import _lib
+    L = _lib.lib
+    a = _lib.UvuArgs()
+    assert L.cgtp_uvu_validate(None, 0) == 1                        # CGTP_ERR_NULL
+    a.cfg = 999
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 5                  # CGTP_ERR_CONFIG
+    a.cfg, a.dtype = 1, 7
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 4                  # CGTP_ERR_DTYPE
+    a.dtype, a.C = 0, 0
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 2                  # CGTP_ERR_SHAPE
+    a.C, a.n_rows, a.n_x_rows = 64, 10, 10
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 1                  # x / y / w missing
+    a.x = a.y = a.w = a.out = 256
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 0
+    a.n_x_rows = 9
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 2                  # rows of x without a gather table
+    a.n_x_rows, a.C = 10, 512
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 0                  # forward tiles channels over the grid
+    a.grad_out = 256
+    assert L.cgtp_uvu_validate(C.byref(a), 1) == 2                  # backward keeps a row inside one wavefront
+    a.C, a.w_shared, a.grad_w = 64, 1, 256
+    assert L.cgtp_uvu_workspace_bytes(C.byref(a), 1) == 3 * 11 * 64 * 4   # 10 rows / 4 slots = 3 partial rows
+    assert L.cgtp_uvu_bwd(C.byref(a), None) == 8                    # CGTP_ERR_WORKSPACE, nothing launched
+
+    t = _lib.TriArgs()
+    assert L.cgtp_tri_validate(C.byref(t)) == 2                     # C == 0
+    t.C, t.n_out, t.nnz, t.n_rows = 8, 4, 30000, 3
+    t.idx = t.seg = t.out = 256
+    assert L.cgtp_tri_validate(C.byref(t)) == 6                     # 30000 * 8 B of table > 160 KB of LDS
+    t.nnz = 100
+    assert L.cgtp_tri_validate(C.byref(t)) == 0
+    t.a.kind = 1
+    assert L.cgtp_tri_validate(C.byref(t)) == 1                     # operand declared but no data
+    assert L.cgtp_segment_sum(None, None, None, None, None, 1, 1, 1, 1, 0, None) == 1
+    assert L.cgtp_membench_copy(256, 256, 17, None) == 2
+
+
+def test_cpu_tensors_are_rejected_loudly():
+    import torch
+    from equitorch_amd import _lib
+    from equitorch_amd.nn import SO3Linear
+    m = SO3Linear("0e+1o", "0e+1o", "0e+1o", 4, 4)
+    with pytest.raises(_lib.CgtpError, match="GPU only"):
+        m(torch.randn(2, 4, 4), torch.randn(2, 4))
