@@ -26,6 +26,13 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 
+# HBM bytes per launch of the dominant kernels on the edge workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# scaled by the same counters on the 1 GiB copy kernel (profiles/uvu_seg_sh2_edge_fwd_bwd.md): KiB per dispatch.
+MEASURED_TRAFFIC_KIB = {
+    "edge_fwd_bwd": 158572.3 * 2.0 + 193595.3 * 1.0,  # uvu_seg_bwd_kernel<TP_sh2,float,4,1>
+    "edge_fwd": 147109.1 * 2.0 + 9216.0 * 1.0,        # uvu_seg_fwd_kernel<TP_sh2,float,4>
+}
+
 WORKLOADS = {
     # name: (lmax, channels, nodes, edges)
     "edge_fwd_bwd": (2, 64, 4096, 65536),
@@ -219,9 +226,9 @@ def main():
     bwd_avg, bwd_med = time_kernel(bwd_fn)
     fwd_bytes, bwd_bytes = algorithmic_bytes(n_nodes, n_edges, d, p, ch)
     if backward:
-        dom, dom_bytes, dom_ms = "uvu_bwd_kernel<sh2,f32,V4,SEG>", bwd_bytes, bwd_avg
+        dom, dom_bytes, dom_ms = "cgtp::uvu_seg_bwd_kernel<TP_sh2,float,4,1>", bwd_bytes, bwd_avg
     else:
-        dom, dom_bytes, dom_ms = "uvu_fwd_kernel<sh2,f32,V4,SEG>", fwd_bytes, fwd_avg
+        dom, dom_bytes, dom_ms = "cgtp::uvu_seg_fwd_kernel<TP_sh2,float,4>", fwd_bytes, fwd_avg
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
 
     rec = {
@@ -232,7 +239,8 @@ def main():
         "config": {"workload": f"{args.workload}: N={n_nodes} nodes, E={n_edges} edges, irreps {irreps}, "
                                f"C={ch}, per-edge weights (E,{p},{ch}), {args.rotate} rotating weight buffers"},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": int(MEASURED_TRAFFIC_KIB[args.workload] * 1024),
                      "algorithmic_bytes": dom_bytes, "avg_ms": round(dom_ms, 5)},
         "kernels": {"fwd_avg_ms": round(fwd_avg, 5), "fwd_med_ms": round(fwd_med, 5),
                     "fwd_GBs": round(fwd_bytes / fwd_avg / 1e6, 1),
