@@ -34,6 +34,19 @@ class TriArgs(C.Structure):
                 ("C", C.c_int32), ("dtype", C.c_int32), ("reduce_c", C.c_int32), ("reduce_rows", C.c_int32)]
 
 
+class GenOperand(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("row_stride", C.c_int64), ("idx_stride", C.c_int64),
+                ("u_stride", C.c_int64), ("w_stride", C.c_int64), ("present", C.c_int32), ("_pad", C.c_int32)]
+
+
+class GenArgs(C.Structure):
+    _fields_ = [("a", GenOperand), ("b", GenOperand), ("w", GenOperand),
+                ("coef", C.c_void_p), ("idx", C.c_void_p), ("seg", C.c_void_p),
+                ("n_out", C.c_int32), ("nnz", C.c_int32), ("out", C.c_void_p), ("n_rows", C.c_int64),
+                ("U", C.c_int32), ("W", C.c_int32), ("out_has_u", C.c_int32), ("out_has_w", C.c_int32),
+                ("reduce_rows", C.c_int32), ("dtype", C.c_int32)]
+
+
 class UvuArgs(C.Structure):
     _fields_ = [("cfg", C.c_int32), ("dtype", C.c_int32), ("C", C.c_int32), ("w_shared", C.c_int32),
                 ("n_rows", C.c_int64), ("n_x_rows", C.c_int64), ("n_seg", C.c_int64),
@@ -59,6 +72,8 @@ def _load():
     lib.cgtp_tri_workspace_bytes.argtypes = [C.POINTER(TriArgs)]
     lib.cgtp_tri_validate.argtypes = [C.POINTER(TriArgs)]
     lib.cgtp_tri_contract.argtypes = [C.POINTER(TriArgs), C.c_void_p]
+    lib.cgtp_gen_validate.argtypes = [C.POINTER(GenArgs)]
+    lib.cgtp_gen_contract.argtypes = [C.POINTER(GenArgs), C.c_void_p]
     lib.cgtp_segment_sum.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                      C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p]
     lib.cgtp_uvu_num_configs.restype = C.c_int

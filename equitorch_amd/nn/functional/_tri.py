@@ -1,4 +1,4 @@
-"""Autograd wrapper of the table-driven trilinear kernel.
+"""Autograd wrapper of the table-driven contraction kernels.
 
 ``out[r, o, (c)] = sum_t coef_t * A[r, ia_t, (c)] * B[r, ib_t, (c)] * W[r, iw_t, (c)]`` is linear in each
 operand, and its gradient with respect to one operand is the same contraction with that operand's index
@@ -54,51 +54,116 @@ class TriSpec:
         return self._packed[key]
 
 
-def _is_shared(t: Tensor, kind: int) -> bool:
-    return t.ndim == (2 if kind == OPERAND_VEC else 1)
+def _axes(kind) -> str:
+    """Operand kind -> channel axes it carries: '' (channel-less), 'u', 'w' or 'uw'.  The integer kinds of the
+    single-axis family map to 'u' (per-channel) and '' (channel-less)."""
+    if kind is None or isinstance(kind, str):
+        return kind
+    return {OPERAND_NONE: None, OPERAND_VEC: "u", OPERAND_SCALAR: ""}[kind]
+
+
+def _is_shared(t: Tensor, axes: str) -> bool:
+    return t.ndim == 1 + len(axes)
+
+
+def _gen_operand(t: Optional[Tensor], axes: Optional[str]) -> "_lib.GenOperand":
+    op = _lib.GenOperand()
+    if t is None or axes is None:
+        return op
+    op.present, op.data = 1, t.data_ptr()
+    shared = _is_shared(t, axes)
+    op.row_stride = 0 if shared else t.stride(0)
+    op.idx_stride = t.stride(0 if shared else 1)
+    pos = 1 if shared else 2
+    for ax in axes:
+        setattr(op, f"{ax}_stride", t.stride(pos))
+        pos += 1
+    return op
+
+
+def _gen_contract(spec: "TriSpec", ops, axes, out_axes: str, out_shared: bool, n_rows: int, U: int, W: int,
+                  dtype, device) -> Tensor:
+    import ctypes as C
+    table = spec.packed(dtype, device)
+    a = _lib.GenArgs()
+    a.a, a.b, a.w = (_gen_operand(t, ax) for t, ax in zip(ops, axes))
+    a.coef, a.idx, a.seg = _lib.ptr(table["coef"]), table["idx"].data_ptr(), table["seg"].data_ptr()
+    a.n_out, a.nnz = spec.out_size, table["idx"].shape[0]
+    shape = (spec.out_size,) + ((U,) if "u" in out_axes else ()) + ((W,) if "w" in out_axes else ())
+    if not out_shared:
+        shape = (n_rows,) + shape
+    out = torch.empty(shape, dtype=dtype, device=device)
+    a.out, a.n_rows, a.U, a.W = out.data_ptr(), n_rows, U, W
+    a.out_has_u, a.out_has_w = int("u" in out_axes), int("w" in out_axes)
+    a.reduce_rows, a.dtype = int(out_shared), _lib.dtype_code(dtype)
+    _lib.check(_lib.lib.cgtp_gen_contract(C.byref(a), _lib.stream_ptr(device)), "cgtp_gen_contract")
+    return out
 
 
 class TriContract(Function):
-    """forward(spec, kinds, out_kind, out_shared, a, b, w) -> out; tensors with kind NONE are passed as None."""
+    """forward(spec, kinds, out_kind, out_shared, a, b, w) -> out.
+
+    ``kinds`` / ``out_kind`` name the channel axes of each operand ('' | 'u' | 'w' | 'uw', or the integer kinds
+    of the single-axis family; None / OPERAND_NONE = operand absent, passed as None).  An axis the output carries
+    is element-wise, the others are summed.  Half-precision inputs are computed in fp32 and rounded once."""
 
     @staticmethod
-    def forward(ctx, spec: TriSpec, kinds: Tuple[int, int, int], out_kind: int, out_shared: bool,
+    def forward(ctx, spec: TriSpec, kinds, out_kind, out_shared: bool,
                 a: Optional[Tensor], b: Optional[Tensor], w: Optional[Tensor]):
+        axes = [_axes(k) for k in kinds]
+        out_axes = _axes(out_kind)
         ops = [a, b, w]
-        present = [t for t, k in zip(ops, kinds) if k != OPERAND_NONE]
+        present = [t for t, ax in zip(ops, axes) if ax is not None]
         _lib.require_gpu(*present)
-        dtype = present[0].dtype
+        res_dtype = present[0].dtype
         for t in present[1:]:
-            dtype = torch.promote_types(dtype, t.dtype)
+            res_dtype = torch.promote_types(res_dtype, t.dtype)
+        dtype = res_dtype if res_dtype in (torch.float32, torch.float64) else torch.float32
         device = present[0].device
-        ops = [None if k == OPERAND_NONE else t.to(dtype).contiguous() for t, k in zip(ops, kinds)]
-        n_rows, channels = None, None
-        for t, k in zip(ops, kinds):
-            if k == OPERAND_NONE:
+        single_axis = all(ax in (None, "", "u") for ax in axes + [out_axes])
+        ops = [None if ax is None else (t.to(dtype).contiguous() if single_axis else t.to(dtype))
+               for t, ax in zip(ops, axes)]
+        n_rows, ext = None, {"u": None, "w": None}
+        for t, ax in zip(ops, axes):
+            if ax is None:
                 continue
-            if not _is_shared(t, k):
+            if t.ndim not in (1 + len(ax), 2 + len(ax)):
+                raise _lib.CgtpError(f"operand with axes '{ax}' must have {1 + len(ax)} or {2 + len(ax)} dims, "
+                                     f"got {t.ndim}")
+            if not _is_shared(t, ax):
                 if n_rows not in (None, t.shape[0]):
                     raise _lib.CgtpError(f"batch size mismatch: {n_rows} vs {t.shape[0]}")
                 n_rows = t.shape[0]
-            if k == OPERAND_VEC:
-                if channels not in (None, t.shape[-1]):
-                    raise _lib.CgtpError(f"channel mismatch: {channels} vs {t.shape[-1]}")
-                channels = t.shape[-1]
+            for i, name in enumerate(ax):
+                size = t.shape[t.ndim - len(ax) + i]
+                if ext[name] not in (None, size):
+                    raise _lib.CgtpError(f"extent mismatch on axis {name}: {ext[name]} vs {size}")
+                ext[name] = size
         any_batched = n_rows is not None
         n_rows = 1 if n_rows is None else n_rows
-        if channels is None:
-            raise _lib.CgtpError("at least one operand must carry a channel axis")
-        out = kernels.tri_contract(spec.packed(dtype, device), spec.out_size,
-                                   (ops[0], kinds[0]), (ops[1], kinds[1]), (ops[2], kinds[2]),
-                                   n_rows, channels, dtype, device,
-                                   reduce_c=(out_kind == OPERAND_SCALAR), reduce_rows=out_shared)
+        for name in out_axes:
+            if ext[name] is None:
+                raise _lib.CgtpError(f"output axis {name} is carried by no operand")
+        if single_axis:
+            if ext["u"] is None:
+                raise _lib.CgtpError("at least one operand must carry a channel axis")
+            code = {None: OPERAND_NONE, "": OPERAND_SCALAR, "u": OPERAND_VEC}
+            out = kernels.tri_contract(spec.packed(dtype, device), spec.out_size,
+                                       *[(t, code[ax]) for t, ax in zip(ops, axes)],
+                                       n_rows, ext["u"], dtype, device,
+                                       reduce_c=(out_axes == ""), reduce_rows=out_shared)
+        else:
+            out = _gen_contract(spec, ops, axes, out_axes, out_shared, n_rows, ext["u"] or 1, ext["w"] or 1, dtype,
+                                device)
         if not out_shared and not any_batched:
             out = out.squeeze(0)  # every operand shared -> result has no batch axis either
-        ctx.spec, ctx.kinds, ctx.out_kind, ctx.out_shared = spec, kinds, out_kind, out_shared
-        ctx.shared = [k != OPERAND_NONE and _is_shared(t, k) for t, k in zip(ops, kinds)]
+        ctx.spec, ctx.axes, ctx.out_axes = spec, axes, out_axes
+        ctx.shared = [ax is not None and _is_shared(t, ax) for t, ax in zip(ops, axes)]
         ctx.save_for_backward(*[t for t in ops if t is not None])
         ctx.present = [t is not None for t in ops]
-        return out
+        ctx.in_dtypes = [None if t is None else t.dtype for t in (a, b, w)]
+        ctx.in_shapes = [None if t is None else t.shape for t in (a, b, w)]
+        return out.to(res_dtype)
 
     @staticmethod
     def backward(ctx, g):
@@ -106,13 +171,16 @@ class TriContract(Function):
         ops = [saved.pop(0) if p else None for p in ctx.present]
         grads = [None, None, None]
         for s in range(3):
-            if ctx.kinds[s] == OPERAND_NONE or not ctx.needs_input_grad[4 + s]:
+            if ctx.axes[s] is None or not ctx.needs_input_grad[4 + s]:
                 continue
-            new_ops = list(ops)
-            new_kinds = list(ctx.kinds)
-            new_ops[s], new_kinds[s] = g, ctx.out_kind
-            grads[s] = TriContract.apply(ctx.spec.grad_spec(s), tuple(new_kinds), ctx.kinds[s], ctx.shared[s],
-                                         *new_ops)
+            new_ops, new_axes = list(ops), list(ctx.axes)
+            new_ops[s], new_axes[s] = g, ctx.out_axes
+            grads[s] = TriContract.apply(ctx.spec.grad_spec(s), tuple(new_axes), ctx.axes[s], ctx.shared[s],
+                                         *new_ops).to(ctx.in_dtypes[s])
+            if grads[s].shape != ctx.in_shapes[s]:
+                # the output was summed over rows and every other operand is shared: the gradient of a batched
+                # operand is then the same for every row
+                grads[s] = grads[s].expand(ctx.in_shapes[s])
         return (None, None, None, None, *grads)
 
 

@@ -8,6 +8,9 @@ second output; here each product is one fused launch and nothing but the inputs 
     1uu : out[n,M,c] = sum_t c_t x[n,M1_t]   y[n,M2_t,c] W[(n),p_t,c]
     uu1 : out[n,M]   = sum_t c_t sum_c x[n,M1_t,c] y[n,M2_t,c] W[(n),p_t,c]
 
+and the fully connected siblings u1v / 1vu / vu1 (``SO3Linear('uv')`` family, reference ``:254-492``) at the end
+of the file.
+
 ``weight`` is shared ``(P, C)`` or per-sample ``(N, P, C)``.  Only ``tp_info_forward`` is read; the two
 backward tables are accepted for signature compatibility.
 """
@@ -18,7 +21,7 @@ from torch import Tensor
 from torch.autograd import Function
 
 from ... import _lib
-from ..._lib import OPERAND_SCALAR as S, OPERAND_VEC as V
+S, V = "", "u"  # channel axes of an operand: none / one
 from ...ops import kernels
 from ...structs import TensorProductInfo
 from ._tri import spec_from_tp_info, tri
@@ -88,3 +91,40 @@ def tensor_product_uu1(input1: Tensor, input2: Tensor, weight: Tensor,
     """``input1 (N, D1, C)``, ``input2 (N, D2, C)`` -> ``(N, DO)`` (summed over channels)."""
     _check_batch(input1, input2, weight)
     return tri(spec_from_tp_info(tp_info_forward), (V, V, V), S, input1, input2, weight)
+
+
+# ---- fully connected in the channels: weight (P, C_in, C_out) or (N, P, C_in, C_out) ---------------------------
+def tensor_product_u1v(input1: Tensor, input2: Tensor, weight: Tensor,
+                       tp_info_forward: TensorProductInfo,
+                       tp_info_backward1: Optional[TensorProductInfo] = None,
+                       tp_info_backward2: Optional[TensorProductInfo] = None) -> Tensor:
+    """``out[n,M,w] = sum_t c_t y[n,M2_t] sum_u x[n,M1_t,u] W[(n),p_t,u,w]`` — ``input1 (N, D1, C_in)``,
+    ``input2 (N, D2)`` -> ``(N, DO, C_out)`` (reference ``linears.py:254-336``)."""
+    _check_batch(input1, input2, weight)
+    from . import _uvw_mfma
+    fast = _uvw_mfma.try_forward(input1, input2, weight, tp_info_forward)
+    if fast is not None:
+        return fast
+    return tri(spec_from_tp_info(tp_info_forward), ("u", "", "uw"), "w", input1, input2, weight)
+
+
+so3_linear_uv = tensor_product_u1v
+
+
+def tensor_product_1vu(input1: Tensor, input2: Tensor, weight: Tensor,
+                       tp_info_forward: TensorProductInfo,
+                       tp_info_backward1: Optional[TensorProductInfo] = None,
+                       tp_info_backward2: Optional[TensorProductInfo] = None) -> Tensor:
+    """``input1 (N, D1)``, ``input2 (N, D2, C_in)`` -> ``(N, DO, C_out)`` (reference ``:338-412``)."""
+    _check_batch(input1, input2, weight)
+    return tri(spec_from_tp_info(tp_info_forward), ("", "u", "uw"), "w", input1, input2, weight)
+
+
+def tensor_product_vu1(input1: Tensor, input2: Tensor, weight: Tensor,
+                       tp_info_forward: TensorProductInfo,
+                       tp_info_backward1: Optional[TensorProductInfo] = None,
+                       tp_info_backward2: Optional[TensorProductInfo] = None) -> Tensor:
+    """``out[n,M] = sum_t c_t sum_{u,w} x[n,M1_t,u] W[(n),p_t,u,w] y[n,M2_t,w]`` — ``input1 (N, D1, C1)``,
+    ``input2 (N, D2, C2)``, ``weight (P, C1, C2)`` -> ``(N, DO)`` (reference ``:414-492``)."""
+    _check_batch(input1, input2, weight)
+    return tri(spec_from_tp_info(tp_info_forward), ("u", "w", "uw"), "", input1, input2, weight)

@@ -1,15 +1,16 @@
 """Tensor products where both operands carry channels (``equitorch/nn/functional/tensor_products.py``).
 
-    uuu : out[n,M,c] = sum_t c_t x[n,M1_t,c] y[n,M2_t,c] W[(n),p_t,c]        (:9-90)
+    uuu : out[n,M,c] = sum_t c_t x[n,M1_t,c] y[n,M2_t,c] W[(n),p_t,c]                 (:9-90)
+    uvw : out[n,M,o] = sum_t c_t sum_{u,v} x[n,M1_t,u] y[n,M2_t,v] W[(n),p_t,u,v,o]   (:92-172)
 """
 from typing import Optional
 
 from torch import Tensor
 
 from ... import _lib
-from ..._lib import OPERAND_VEC as V
+V = "u"  # channel axes of a per-channel operand
 from ...structs import TensorProductInfo
-from ._tri import spec_from_tp_info, tri
+from ._tri import spec_from_product_info, spec_from_tp_info, tri
 
 
 def tensor_product_uuu(input1: Tensor, input2: Tensor, weight: Tensor,
@@ -19,3 +20,20 @@ def tensor_product_uuu(input1: Tensor, input2: Tensor, weight: Tensor,
     """``input1 (N, D1, C)``, ``input2 (N, D2, C)``, ``weight (P, C) | (N, P, C)`` -> ``(N, DO, C)``."""
     _lib.require_gpu(input1, input2, weight)
     return tri(spec_from_tp_info(tp_info_forward), (V, V, V), V, input1, input2, weight)
+
+
+def tensor_product_uvw(input1: Tensor, input2: Tensor, weight: Tensor,
+                       tp_info_forward: TensorProductInfo,
+                       tp_info_backward1: Optional[TensorProductInfo] = None,
+                       tp_info_backward2: Optional[TensorProductInfo] = None) -> Tensor:
+    """``input1 (N, D1, C1)``, ``input2 (N, D2, C2)``, ``weight (P, C1, C2, C_out) | (N, P, C1, C2, C_out)`` ->
+    ``(N, DO, C_out)``.  Two stages as in the reference (``tensor_products.py:100-101``): the outer products per
+    stage-1 segment, flattened to ``C1*C2`` channels, then one matrix product per segment with the flattened
+    weight of its path."""
+    _lib.require_gpu(input1, input2, weight)
+    s1, s2 = tp_info_forward.info_Mij_fwd, tp_info_forward.info_M_fwd
+    inter = tri(spec_from_product_info(s1, input1.shape[-2], input2.shape[-2]), ("u", "w", None), "uw",
+                input1, input2)
+    inter = inter.flatten(-2)
+    w2 = weight.flatten(-3, -2)
+    return tri(spec_from_product_info(s2, inter.shape[-2], w2.shape[-3]), ("u", "uw", None), "w", inter, w2)

@@ -13,7 +13,7 @@ from torch.nn import Parameter
 from ..irreps import check_irreps
 from ..structs import TensorProductInfo
 from ..utils._structs import tp_infos
-from .functional.linears import so3_linear_uu
+from .functional.linears import so3_linear_uu, so3_linear_uv
 from .init import initialize_so3_so2_linear
 
 
@@ -86,7 +86,6 @@ class SO3Linear(nn.Module):
         infos = (self.tp_info_forward, self.tp_info_backward1, self.tp_info_backward2)
         if self.feature_mode == 'uu':
             return so3_linear_uu(input1, input2, weight, *infos)
-        from .functional.linears_uv import so3_linear_uv
         return so3_linear_uv(input1, input2, weight, *infos)
 
     def _apply(self, *args, **kwargs):

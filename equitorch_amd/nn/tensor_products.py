@@ -11,7 +11,7 @@ from torch.nn import Parameter
 from ..irreps import check_irreps
 from ..structs import TensorProductInfo
 from ..utils._structs import tp_infos
-from .functional.tensor_products import tensor_product_uuu
+from .functional.tensor_products import tensor_product_uuu, tensor_product_uvw
 from .init import initialize_tensor_product
 
 
@@ -79,7 +79,6 @@ class TensorProduct(nn.Module):
         infos = (self.tp_info_forward, self.tp_info_backward1, self.tp_info_backward2)
         if self.feature_mode == 'uuu':
             return tensor_product_uuu(input1, input2, weight, *infos)
-        from .functional.tensor_products_uvw import tensor_product_uvw
         return tensor_product_uvw(input1, input2, weight, *infos)
 
     def _apply(self, *args, **kwargs):

@@ -1,5 +1,6 @@
-"""The element-wise members of the reference's batched sparse-dense product family
-(``equitorch/ops/batched_sparse_dense_op.py``) on the table-driven HIP kernel.
+"""The reference's batched sparse-dense product family (``equitorch/ops/batched_sparse_dense_op.py``) on the
+table-driven HIP kernels: the element-wise members below on the single-axis kernel, the matrix members
+(outer, vecmat, mat_t_vec; end of file) on the two-axis kernel.
 
     mul    : z[n,M,c] = sum_t s_t x[n,i1_t,c] y[n,i2_t,c]          (:156-299)
     vecsca : z[n,M,c] = sum_t s_t x[n,i1_t,c] y[n,i2_t]            (:1665-1818)
@@ -90,3 +91,47 @@ def indexed_inner_scale_gather(input1, input2, scale=None, index1=None, index2=N
                                loop_unroll_factor=4):
     return _product(input1, OPERAND_VEC, input2, OPERAND_VEC, scale, index1, index2, seg, gather_index,
                     index_out, out, out_accumulated, out_size, reduce_c=True)
+
+
+def _matrix_product(input1, axes1, input2, axes2, out_axes, scale, index1, index2, seg, gather_index, index_out,
+                    out, out_accumulated, out_size):
+    """Matrix members of the family on the two-axis contraction kernel (no autograd at this layer)."""
+    if gather_index is not None or index_out is not None:
+        raise NotImplementedError("gather_index / index_out tables are not supported")
+    from ..nn.functional._tri import spec_from_product_info, tri
+    from ..structs import SparseProductInfo
+    info = SparseProductInfo(scale, index1, index2, seg, None, None, out_size)
+    size1, size2 = input1.shape[-1 - len(axes1)], input2.shape[-1 - len(axes2)]
+    with torch.no_grad():
+        res = tri(spec_from_product_info(info, size1, size2), (axes1, axes2, None), out_axes, input1, input2,
+                  None, out_shared=out_accumulated)
+    if out is not None:
+        out.copy_(res)
+        return out
+    return res
+
+
+def indexed_outer_scale_gather(input1, input2, scale=None, index1=None, index2=None, seg=None,
+                               gather_index=None, index_out=None, out=None, out_accumulated=False,
+                               out_size=None, block_size_n=8, block_size_c1=32, block_size_c2=32, num_stages=2):
+    """``z[n,M,c1,c2] = sum_t s_t x[n,i1_t,c1] y[n,i2_t,c2]`` (reference ``:436-579``)."""
+    return _matrix_product(input1, "u", input2, "w", "uw", scale, index1, index2, seg, gather_index, index_out,
+                           out, out_accumulated, out_size)
+
+
+def indexed_vecmat_scale_gather(input1, input2, scale=None, index1=None, index2=None, seg=None,
+                                gather_index=None, index_out=None, out=None, out_accumulated=False,
+                                out_size=None, block_size_n=8, block_size_c_out=32, block_size_c_in=32,
+                                num_stages=1, loop_unroll_factor=4):
+    """``z[n,M,w] = sum_t s_t sum_u x[n,i1_t,u] Y[(n),i2_t,u,w]`` (reference ``:1383-1534``)."""
+    return _matrix_product(input1, "u", input2, "uw", "w", scale, index1, index2, seg, gather_index, index_out,
+                           out, out_accumulated, out_size)
+
+
+def indexed_mat_t_vec_scale_gather(input1, input2, scale=None, index1=None, index2=None, seg=None,
+                                   gather_index=None, index_out=None, out=None, out_accumulated=False,
+                                   out_size=None, block_size_n=8, block_size_c_out=32, block_size_c_in=32,
+                                   num_stages=1, loop_unroll_factor=4):
+    """``z[n,M,u] = sum_t s_t sum_w Y[(n),i1_t,u,w] x[n,i2_t,w]`` (reference ``:1200-1238``)."""
+    return _matrix_product(input1, "uw", input2, "w", "u", scale, index1, index2, seg, gather_index, index_out,
+                           out, out_accumulated, out_size)

@@ -82,6 +82,44 @@ int64_t cgtp_tri_workspace_bytes(const cgtp_tri_args* args);
 int cgtp_tri_validate(const cgtp_tri_args* args);
 int cgtp_tri_contract(const cgtp_tri_args* args, void* stream);
 
+/* ---- general contraction over two channel axes (u, w) ----------------------------------------------------
+ *
+ *   out[r, o, (u), (w)] = sum_{t in seg[o]} coef[t] * sum_{axes not in out} A[r, ia_t, ..] * B[r, ib_t, ..] * W[r, iw_t, ..]
+ *
+ * Each operand carries any subset of {u, w} (stride 0 for an axis it lacks); an axis the output carries is
+ * element-wise, the others are summed.  Any-shape path for the matrix members of the reference's operator
+ * family — indexed_vecmat / outer / mat_t_vec _scale_gather (equitorch/ops/batched_sparse_dense_op.py:1383-1459,
+ * 436-512, 1200-1238) — for the fully connected products built from them (TensorProductU1VDummy and siblings,
+ * equitorch/nn/functional/linears.py:254-492; TensorProductUVWDummy, nn/functional/tensor_products.py:92-172)
+ * and for all their gradients.  Same packed table as cgtp_tri_contract.  reduce_rows sums over rows.
+ */
+typedef struct cgtp_gen_operand {
+  const void* data;
+  int64_t row_stride;      /* 0: shared over rows */
+  int64_t idx_stride;      /* elements between sparse indices */
+  int64_t u_stride;        /* 0: operand has no u axis */
+  int64_t w_stride;        /* 0: operand has no w axis */
+  int32_t present;
+  int32_t _pad;
+} cgtp_gen_operand;
+
+typedef struct cgtp_gen_args {
+  cgtp_gen_operand a, b, w;
+  const void* coef;        /* [nnz] dtype; NULL = ones */
+  const uint32_t* idx;     /* [nnz] ia | ib << 10 | iw << 20 */
+  const int32_t* seg;      /* [n_out + 1] */
+  int32_t n_out, nnz;
+  void* out;               /* (n_rows | 1, n_out, [U], [W]) contiguous */
+  int64_t n_rows;
+  int32_t U, W;            /* extents of the two channel axes */
+  int32_t out_has_u, out_has_w;
+  int32_t reduce_rows;
+  int32_t dtype;           /* CGTP_F32 | CGTP_F64 */
+} cgtp_gen_args;
+
+int cgtp_gen_validate(const cgtp_gen_args* args);
+int cgtp_gen_contract(const cgtp_gen_args* args, void* stream);
+
 /* ---- indexed scale-segment: out[n, m, c] = sum_{t in seg m} scale[t] * in[n, index[t], c] --------------
  * Stands in for indexed_scale_segment_gpu (equitorch/ops/indexed_scale_segment_op.py:110-141), including the
  * seg == NULL mode (pure scaled gather, one term per output) and optional scale / index.  With N == 1,

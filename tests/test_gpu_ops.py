@@ -1,0 +1,197 @@
+"""GPU parity of the table-driven operator family and of the uv / uvw tensor products against the oracle.
+
+The operator sweep follows the reference's own test procedure (test/test_op/test_sparse_structs.py:668-733):
+Irreps((1,3)) tables, N=135, every shared / accumulated flag combination, forward and gradients, here against
+the oracle's restatement of the reference CPU ops (and dense einsum for the matrix members)."""
+import itertools
+
+import pytest
+import torch
+
+from helpers import assert_close
+from oracle import ref_ops, ref_tables
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tables13():
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    irr = Irreps((1, 3))
+    mine = tp_infos(irr, irr, irr)[0]
+    ref = ref_ops.tables_to_torch(ref_tables.tp_infos((1, 3), (1, 3), (1, 3))[0], torch.float64)
+    return mine, ref
+
+
+def _dense_from_info(info, size1, size2):
+    """(out, size1, size2) float64 coupling of one sparse product table."""
+    n = info["scale"].shape[0]
+    i1 = info["index1"] if info["index1"] is not None else torch.arange(n)
+    i2 = info["index2"] if info["index2"] is not None else torch.arange(n)
+    seg = info["seg_out"]
+    out_idx = torch.repeat_interleave(torch.arange(seg.shape[0] - 1), seg[1:] - seg[:-1])
+    T = torch.zeros(seg.shape[0] - 1, size1, size2, dtype=torch.float64)
+    T.index_put_((out_idx, i1, i2), info["scale"].double(), accumulate=True)
+    return T
+
+
+EW = {  # name: (oracle fn, axes1, axes2)
+    "mul": (ref_ops.cpu_mul, "u", "u"), "inner": (ref_ops.cpu_inner, "u", "u"),
+    "vecsca": (ref_ops.cpu_vecsca, "u", ""), "scavec": (ref_ops.cpu_scavec, "", "u"),
+}
+
+
+@pytest.mark.parametrize("op", sorted(EW))
+@pytest.mark.parametrize("shared1,shared2,acc", [s for s in itertools.product([False, True], repeat=3)
+                                                 if not (s[0] and s[1] and s[2])])
+@pytest.mark.parametrize("channels", [97, 35])
+def test_elementwise_ops_sweep(device, tables13, op, shared1, shared2, acc, channels):
+    import equitorch_amd.nn.functional as F
+    mine, ref = tables13
+    oracle, ax1, ax2 = EW[op]
+    info_m, info_r = mine.info_Mij_fwd.to(device), ref["info_Mij_fwd"]
+    g = torch.Generator().manual_seed(hash((op, shared1, shared2, acc, channels)) % 2 ** 31)
+    n, d = 135, 15
+
+    def mk(axes, shared):
+        shape = (() if shared else (n,)) + (d,) + ((channels,) if axes else ())
+        return torch.randn(*shape, generator=g, dtype=torch.float64)
+    x, y = mk(ax1, shared1), mk(ax2, shared2)
+    fn = getattr(F, f"sparse_{op}")
+    xd, yd = (t.float().to(device).requires_grad_(True) for t in (x, y))
+    out = fn(xd, yd, info_m, out_accumulated=acc)
+    xr, yr = (t.float().double().requires_grad_(True) for t in (x, y))
+    ref_out = oracle(xr, yr, info_r, out_accumulated=acc)
+    assert_close(out, ref_out, 1e-5, f"{op} forward")
+    ct = torch.randn(ref_out.shape, generator=g, dtype=torch.float64)
+    gx, gy = torch.autograd.grad(out, (xd, yd), ct.float().to(device))
+    rgx, rgy = torch.autograd.grad(ref_out, (xr, yr), ct.float().double())
+    assert_close(gx, rgx, 1e-5, f"{op} grad1")
+    assert_close(gy, rgy, 1e-5, f"{op} grad2")
+
+
+MAT = {  # name: (axes1, axes2, out axes, einsum)
+    "outer": ("u", "w", "uw", "mab,{a}au,{b}bw->{o}muw"),
+    "vecmat": ("u", "uw", "w", "mab,{a}au,{b}buw->{o}mw"),
+    "mat_t_vec": ("uw", "w", "u", "mab,{a}auw,{b}bw->{o}mu"),
+}
+
+
+@pytest.mark.parametrize("op", sorted(MAT))
+@pytest.mark.parametrize("shared1,shared2,acc", [(False, False, False), (False, True, False), (True, False, False),
+                                                 (False, False, True), (False, True, True)])
+def test_matrix_ops_sweep(device, tables13, op, shared1, shared2, acc):
+    import equitorch_amd.nn.functional as F
+    mine, ref = tables13
+    ax1, ax2, axo, eq = MAT[op]
+    info_m = mine.info_Mij_fwd.to(device)
+    T = _dense_from_info(ref["info_Mij_fwd"], 15, 15)
+    g = torch.Generator().manual_seed(hash((op, shared1, shared2, acc)) % 2 ** 31)
+    n, d, U, W = 37, 15, 21, 13
+    ext = {"u": U, "w": W}
+
+    def mk(axes, shared):
+        return torch.randn(*((() if shared else (n,)) + (d,) + tuple(ext[a] for a in axes)), generator=g,
+                           dtype=torch.float64)
+    x, y = mk(ax1, shared1), mk(ax2, shared2)
+    xd, yd = (t.float().to(device).requires_grad_(True) for t in (x, y))
+    out = getattr(F, f"sparse_{op}")(xd, yd, info_m, out_accumulated=acc)
+    xr, yr = (t.float().double().requires_grad_(True) for t in (x, y))
+    eq = eq.format(a="" if shared1 else "n", b="" if shared2 else "n", o="" if (shared1 and shared2) else "n")
+    ref_out = torch.einsum(eq, T, xr, yr)
+    if acc:
+        ref_out = ref_out.sum(0)
+    assert_close(out, ref_out, 1e-5, f"{op} forward")
+    ct = torch.randn(ref_out.shape, generator=g, dtype=torch.float64)
+    gx, gy = torch.autograd.grad(out, (xd, yd), ct.float().to(device))
+    rgx, rgy = torch.autograd.grad(ref_out, (xr, yr), ct.float().double())
+    assert_close(gx, rgx, 1e-5, f"{op} grad1")
+    assert_close(gy, rgy, 1e-5, f"{op} grad2")
+
+
+@pytest.mark.parametrize("scaled,indexed,segmented", [(True, True, True), (False, True, True), (True, False, True),
+                                                      (True, True, False), (False, False, False)])
+def test_indexed_scale_segment(device, scaled, indexed, segmented):
+    from equitorch_amd.ops import indexed_scale_segment
+    g = torch.Generator().manual_seed(3)
+    n, in_size, c, n_out = 3, 50, 37, 11
+    x = torch.randn(n, in_size, c, generator=g)
+    if segmented:
+        counts = torch.randint(0, 9, (n_out,), generator=g)
+        seg = torch.cat([torch.zeros(1, dtype=torch.int64), torch.cumsum(counts, 0)])
+        t = int(seg[-1])
+    else:
+        seg, t = None, n_out
+    index = torch.randint(0, in_size, (t,), generator=g) if indexed else None
+    scale = torch.randn(t, generator=g) if scaled else None
+    if not indexed:
+        x = x[:, :t].contiguous()
+    dev = lambda v: None if v is None else v.to(device)
+    out = indexed_scale_segment(x.to(device), dev(scale), dev(index), dev(seg), out_size=n_out)
+    ref = ref_ops.cpu_scale_segment(x.double(), None if scale is None else scale.double(), index, seg)
+    assert_close(out, ref, 1e-5, "indexed_scale_segment")
+
+
+@pytest.mark.parametrize("mode", ["u1v", "1vu", "vu1", "uvw", "uuu", "1uu", "uu1"])
+@pytest.mark.parametrize("shared_w", [True, False])
+def test_tensor_product_family_vs_dense(device, mode, shared_w):
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    io, i1, i2 = "0e+1o+2e", "0e+1o+2e", "0e+1o"
+    infos = [t.to(device) for t in tp_infos(Irreps(io), Irreps(i1), Irreps(i2))[:3]]
+    T = ref_ops.dense_coupling(io, i1, i2)
+    p = T.shape[0]
+    g = torch.Generator().manual_seed(hash((mode, shared_w)) % 2 ** 31)
+    n, u, v, w = 29, 12, 5, 9
+    shapes = {  # mode: (x channels, y channels, weight channels, einsum)
+        "u1v": ((u,), (), (u, w), "pmab,nau,nb,{W}puw->nmw"), "1vu": ((), (u,), (u, w), "pmab,na,nbu,{W}puw->nmw"),
+        "vu1": ((u,), (w,), (u, w), "pmab,nau,nbw,{W}puw->nm"), "uvw": ((u,), (v,), (u, v, w), "pmab,nau,nbv,{W}puvw->nmw"),
+        "uuu": ((u,), (u,), (u,), "pmab,nau,nbu,{W}pu->nmu"), "1uu": ((), (u,), (u,), "pmab,na,nbu,{W}pu->nmu"),
+        "uu1": ((u,), (u,), (u,), "pmab,nau,nbu,{W}pu->nm"),
+    }
+    cx, cy, cw, eq = shapes[mode]
+    x = torch.randn(n, 9, *cx, generator=g, dtype=torch.float64)
+    y = torch.randn(n, 4, *cy, generator=g, dtype=torch.float64)
+    wt = torch.randn(*(() if shared_w else (n,)), p, *cw, generator=g, dtype=torch.float64)
+    xd, yd, wd = (t.float().to(device).requires_grad_(True) for t in (x, y, wt))
+    out = getattr(F, f"tensor_product_{mode}")(xd, yd, wd, *infos)
+    xr, yr, wr = (t.float().double().requires_grad_(True) for t in (x, y, wt))
+    ref_out = torch.einsum(eq.format(W="" if shared_w else "n"), T, xr, yr, wr)
+    assert_close(out, ref_out, 1e-5, f"{mode} forward")
+    ct = torch.randn(ref_out.shape, generator=g, dtype=torch.float64)
+    grads = torch.autograd.grad(out, (xd, yd, wd), ct.float().to(device))
+    refs = torch.autograd.grad(ref_out, (xr, yr, wr), ct.float().double())
+    for name, a, b in zip(("grad1", "grad2", "grad_w"), grads, refs):
+        assert_close(a, b, 1e-5, f"{mode} {name}")
+
+
+def test_modules_uv_uvw_and_gradgradcheck(device):
+    """Module API for the fully connected modes, and second-order correctness (the reference checks gradcheck and
+    gradgradcheck in float64 on 0e+1e+2e x 0e+1e+2e -> 0e+1e+2e+3e, test/test_tp/test_grad_tp.py:57-103)."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.nn import SO3Linear, TensorProduct
+    io, i1, i2 = "0e+1e+2e+3e", "0e+1e+2e", "0e+1e+2e"
+    g = torch.Generator().manual_seed(1)
+    n = 6
+    for mode, ch in (("uu", (3, 3)), ("uv", (3, 4))):
+        mod = SO3Linear(i1, i2, io, ch[0], ch[1], feature_mode=mode).to(device).double()
+        x = torch.randn(n, 9, ch[0], generator=g, dtype=torch.float64).to(device).requires_grad_(True)
+        y = torch.randn(n, 9, generator=g, dtype=torch.float64).to(device).requires_grad_(True)
+        assert mod(x, y).shape == (n, 16, ch[1])
+        op = getattr(F, "so3_linear_" + mode)
+        fn = lambda x, y, w: op(x, y, w, mod.tp_info_forward)
+        w = mod.weight.detach().clone().requires_grad_(True)
+        assert torch.autograd.gradcheck(fn, (x, y, w), eps=1e-6, atol=1e-5, rtol=1e-5, nondet_tol=1e-9)
+        assert torch.autograd.gradgradcheck(fn, (x, y, w), eps=1e-6, atol=1e-5, rtol=1e-5, nondet_tol=1e-9)
+    for mode, ch in (("uuu", (3, 3, 3)), ("uvw", (3, 2, 4))):
+        mod = TensorProduct(i1, i2, io, *ch, feature_mode=mode).to(device).double()
+        x = torch.randn(n, 9, ch[0], generator=g, dtype=torch.float64).to(device).requires_grad_(True)
+        y = torch.randn(n, 9, ch[1], generator=g, dtype=torch.float64).to(device).requires_grad_(True)
+        assert mod(x, y).shape == (n, 16, ch[2])
+        tp = getattr(F, "tensor_product_" + mode)
+        w = mod.weight.detach().clone().requires_grad_(True)
+        fn = lambda x, y, w: tp(x, y, w, mod.tp_info_forward)
+        assert torch.autograd.gradcheck(fn, (x, y, w), eps=1e-6, atol=1e-5, rtol=1e-5, nondet_tol=1e-9)
+        assert torch.autograd.gradgradcheck(fn, (x, y, w), eps=1e-6, atol=1e-5, rtol=1e-5, nondet_tol=1e-9)
