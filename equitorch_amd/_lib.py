@@ -85,6 +85,11 @@ def _load():
     lib.cgtp_uvu_workspace_bytes.argtypes = [C.POINTER(UvuArgs), C.c_int]
     lib.cgtp_uvu_fwd.argtypes = [C.POINTER(UvuArgs), C.c_void_p]
     lib.cgtp_uvu_bwd.argtypes = [C.POINTER(UvuArgs), C.c_void_p]
+    lib.cgtp_uv_find.argtypes = [C.c_uint64]
+    _uv = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32,
+           C.c_int32]
+    lib.cgtp_uv_validate.argtypes = _uv
+    lib.cgtp_uv_apply.argtypes = _uv + [C.c_void_p]
     lib.cgtp_membench_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
     lib.cgtp_membench_read.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
     return lib

@@ -1,9 +1,78 @@
-"""Dispatch of the fully connected product to the bf16 matrix-core kernel (when it applies)."""
+"""Dispatch of the fully connected ("uv") product to the bf16 matrix-core kernel (``cgtp_uv_apply``)."""
+import ctypes as C
 from typing import Optional
 
+import torch
 from torch import Tensor
+from torch.autograd import Function
+
+from ... import _lib
+from ..._tables import fingerprint
+from ...ops import kernels
+from ._tri import spec_from_tp_info, tri
+
+
+def uv_config_of(tp_info) -> int:
+    return kernels.cached(tp_info.info_Mij_fwd.scale, "uv_cfg",
+                          lambda: int(_lib.lib.cgtp_uv_find(C.c_uint64(fingerprint(kernels.coo_of(tp_info))))))
+
+
+def _apply(cfg: int, direction: int, x: Tensor, y: Tensor, wt: Tensor, d_out: int) -> Tensor:
+    n, _, cin = x.shape
+    cout = wt.shape[1]
+    out = torch.empty((n, d_out, cout), dtype=x.dtype, device=x.device)
+    _lib.check(_lib.lib.cgtp_uv_apply(cfg, direction, x.data_ptr(), y.data_ptr(), wt.data_ptr(), out.data_ptr(), n,
+                                      cin, cout, _lib.BF16, _lib.stream_ptr(x.device)), "cgtp_uv_apply")
+    return out
+
+
+class _UvMfma(Function):
+    """u1v with a shared weight on the matrix cores.  Forward and the gradient w.r.t. input1 run the MFMA kernel;
+    the gradients w.r.t. the harmonics and the weight go through the general contraction kernel."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, y: Tensor, w: Tensor, tp_info, cfg: int):
+        coo = kernels.coo_of(tp_info)
+        out = _apply(cfg, 0, x, y, w.transpose(-1, -2).contiguous(), coo.DO)
+        ctx.save_for_backward(x, y, w)
+        ctx.tp_info, ctx.cfg, ctx.d1 = tp_info, cfg, coo.D1
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        x, y, w = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        spec = spec_from_tp_info(ctx.tp_info)
+        gx = gy = gw = None
+        with torch.enable_grad() if torch.is_grad_enabled() else torch.no_grad():
+            if need[0]:
+                if torch.is_grad_enabled():
+                    gx = tri(spec.grad_spec(0), ("w", "", "uw"), "u", g, y, w)
+                else:
+                    gx = _apply(ctx.cfg, 1, g.contiguous(), y, w.contiguous(), ctx.d1)
+            if need[1]:
+                gy = tri(spec.grad_spec(1), ("u", "w", "uw"), "", x, g, w)
+            if need[2]:
+                gw = tri(spec.grad_spec(2), ("u", "", "w"), "uw", x, y, g, out_shared=True)
+        return gx, gy, gw, None, None
 
 
 def try_forward(input1: Tensor, input2: Tensor, weight: Tensor, tp_info) -> Optional[Tensor]:
-    """Returns the product computed by the MFMA kernel, or None if the operands are outside its domain."""
-    return None
+    """The product on the MFMA kernel, or None if the operands are outside its domain (bf16, shared weight,
+    C_in in {32, 64, 128} both ways, C_out a multiple of 32, table compiled in, input rows fit in LDS)."""
+    if not (input1.dtype == input2.dtype == weight.dtype == torch.bfloat16):
+        return None
+    if input1.ndim != 3 or input2.ndim != 2 or weight.ndim != 3 or input1.shape[0] == 0:
+        return None
+    cin, cout = weight.shape[-2:]
+    if cin not in (32, 64, 128) or cout not in (32, 64, 128):
+        return None
+    cfg = uv_config_of(tp_info)
+    if cfg < 0:
+        return None
+    x, y = input1.contiguous(), input2.contiguous()
+    dummy = 256
+    for direction, (ci, co) in enumerate(((cin, cout), (cout, cin))):
+        if _lib.lib.cgtp_uv_validate(cfg, direction, dummy, dummy, dummy, dummy, x.shape[0], ci, co, _lib.BF16) != 0:
+            return None
+    return _UvMfma.apply(x, y, weight, tp_info, cfg)

@@ -192,6 +192,26 @@ int64_t cgtp_uvu_workspace_bytes(const cgtp_uvu_args* args, int backward);
 int cgtp_uvu_fwd(const cgtp_uvu_args* args, void* stream);
 int cgtp_uvu_bwd(const cgtp_uvu_args* args, void* stream);
 
+/* ---- fully connected ("uv") tensor product on the matrix cores --------------------------------------------
+ *
+ *   out[n, m, w] = sum_t coef_t * y[n, b_t] * sum_u x[n, a_t, u] * Wt[p_t, w, u]        bf16 in, fp32 accumulate
+ *
+ * Fused replacement for TensorProductU1VDummy.forward (equitorch/nn/functional/linears.py:257-280:
+ * indexed_vecsca_scale_gather then indexed_vecmat_scale_gather, with the (N, segments, C_in) intermediate in
+ * memory) and, with direction = 1, for the grad-input1 product of its backward (:290-293).  The table is compiled
+ * in; cgtp_uv_find() maps the fingerprint of the forward table to a config id (or -1).
+ *   direction 0: x = input1 (n_rows, D1, cin), out (n_rows, DO, cout), wt = W transposed to (P, cout, cin);
+ *   direction 1: x = grad_out (n_rows, DO, cin), out = grad_input1 (n_rows, D1, cout), wt = W as stored
+ *                (P, C_in, C_out) (here cin = C_out of the module and cout = its C_in).
+ * y is (n_rows, D2).  cin in {32, 64, 128}, cout a multiple of 32, dtype CGTP_BF16, 16-byte aligned pointers.
+ */
+int cgtp_uv_num_configs(void);
+int cgtp_uv_find(uint64_t fingerprint);
+int cgtp_uv_validate(int cfg, int direction, const void* x, const void* y, const void* wt, const void* out,
+                     int64_t n_rows, int32_t cin, int32_t cout, int32_t dtype);
+int cgtp_uv_apply(int cfg, int direction, const void* x, const void* y, const void* wt, void* out, int64_t n_rows,
+                  int32_t cin, int32_t cout, int32_t dtype, void* stream);
+
 /* ---- streaming kernels of known traffic (counter calibration, achievable-bandwidth reference) ------------
  * No counterpart in the reference.  copy: reads n_bytes and writes n_bytes; read: reads n_bytes.
  * n_bytes must be a multiple of 16 and the pointers 16-byte aligned.

@@ -195,3 +195,32 @@ def test_modules_uv_uvw_and_gradgradcheck(device):
         fn = lambda x, y, w: tp(x, y, w, mod.tp_info_forward)
         assert torch.autograd.gradcheck(fn, (x, y, w), eps=1e-6, atol=1e-5, rtol=1e-5, nondet_tol=1e-9)
         assert torch.autograd.gradgradcheck(fn, (x, y, w), eps=1e-6, atol=1e-5, rtol=1e-5, nondet_tol=1e-9)
+
+
+@pytest.mark.parametrize("lmax,cin,cout,n", [(1, 32, 32, 70), (2, 64, 128, 100), (3, 128, 128, 257), (3, 128, 64, 33)])
+def test_uv_mfma_bf16(device, lmax, cin, cout, n):
+    """bf16 matrix-core path of SO3Linear('uv'): forward and all gradients against the dense float64 oracle
+    evaluated on the bf16-rounded inputs; tolerance rel 1e-2 of the tensor's largest magnitude (bf16 output)."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import _uvw_mfma
+    from equitorch_amd.utils._sh import spherical_harmonics
+    from helpers import unit_vectors
+    irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+    mod = SO3Linear(irreps, irreps, irreps, cin, cout, internal_weights=False, feature_mode="uv").to(device)
+    assert _uvw_mfma.uv_config_of(mod.tp_info_forward) >= 0
+    d = (lmax + 1) ** 2
+    g = torch.Generator().manual_seed(lmax * 1000 + cin + cout)
+    x = torch.randn(n, d, cin, generator=g).bfloat16()
+    y = spherical_harmonics(unit_vectors(n, g), lmax).bfloat16()
+    w = (torch.randn(mod.num_paths, cin, cout, generator=g) / (cin * mod.num_paths) ** 0.5).bfloat16()
+    ct = torch.randn(n, d, cout, generator=g).bfloat16()
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    out = mod(xd, yd, wd)
+    assert out.dtype == torch.bfloat16
+    gx, gy, gw = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
+    T = ref_ops.dense_coupling(irreps, irreps, irreps).float().double()
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x, y, w), ct)
+    for name, a, b in zip(("out", "grad_x", "grad_sh", "grad_w"), (out, gx, gy, gw), (ref_out, *ref_grads)):
+        a, b = a.detach().double().cpu(), b.double()
+        err = float((a - b).abs().max())
+        assert err <= 1e-2 * float(b.abs().max()), f"lmax={lmax} {name}: max abs err {err:.3e} vs scale {float(b.abs().max()):.3e}"
