@@ -37,6 +37,8 @@ WORKLOADS = {
     # name: (lmax, channels, nodes, edges)
     "edge_fwd_bwd": (2, 64, 4096, 65536),
     "edge_fwd": (2, 64, 4096, 65536),
+    # fully connected product on the matrix cores (BASELINE configs[3]): (lmax, C_in = C_out, batch)
+    "uvw_fwd": (3, 128, 32768),
     # streaming kernels of known traffic (1 GiB): counter calibration and achievable-bandwidth reference
     "copy": None,
     "read": None,
@@ -71,6 +73,59 @@ def membench(kind, steps, warmup):
                       "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 5),
                       "bytes_read": n_bytes, "bytes_written": n_bytes if kind == "copy" else 0,
                       "config": {"workload": f"{kind} of 1 GiB, float4 grid-stride, 4096 workgroups"}}))
+
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, vendor figure
+
+
+def uvw_bench(args):
+    """BASELINE configs[3], forward: bf16 x (B,16,128), sh (B,16), shared W (23,128,128), fp32 accumulation;
+    algorithmic flops 2*B*99*128*128 (the Clebsch-Gordan stage is not counted)."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import _uvw_mfma
+    from equitorch_amd.utils._sh import spherical_harmonics
+    lmax, ch, n = WORKLOADS["uvw_fwd"]
+    dev = torch.device("cuda:0")
+    irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+    mod = SO3Linear(irreps, irreps, irreps, ch, ch, internal_weights=False, feature_mode="uv").to(dev)
+    d = (lmax + 1) ** 2
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(n, d, ch, generator=gen).bfloat16().to(dev)
+    vec = torch.randn(n, 3, generator=gen)
+    sh = spherical_harmonics(vec / vec.norm(dim=-1, keepdim=True), lmax).bfloat16().to(dev)
+    w = (torch.randn(mod.num_paths, ch, ch, generator=gen) / (ch * mod.num_paths) ** 0.5).bfloat16().to(dev)
+    cfg = _uvw_mfma.uv_config_of(mod.tp_info_forward)
+    wt = w.transpose(-1, -2).contiguous()
+    s1 = int(mod.tp_info_forward.info_Mij_fwd.out_size)
+    flops = 2.0 * n * s1 * ch * ch
+
+    def step():
+        return mod(x, sh, w)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) / args.steps * 1e3
+    evs = []
+    for _ in range(args.kernel_reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(); _uvw_mfma._apply(cfg, 0, x, sh, wt, d); b.record()
+        evs.append((a, b))
+    torch.cuda.synchronize()
+    k_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    tf = flops / (k_ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "uvw fwd TFLOP/s (lmax=3,C=128,bf16)", "value": round(flops / (ms_step * 1e-3) / 1e12, 2),
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"uvw_fwd: B={n}, irreps {irreps}, C_in=C_out={ch}, shared W ({mod.num_paths},{ch},{ch}), "
+                               f"bf16 in / fp32 accumulate / bf16 out, forward through SO3Linear('uv')"},
+        "roofline": {"bound": "mfma", "kernel": "cgtp::uv_kernel<UV_sh3_d0,128>", "achieved": round(tf, 2),
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "traffic": None, "algorithmic_flops": flops, "avg_ms": round(k_ms, 5)}}))
 
 
 def make_inputs(lmax, ch, n_nodes, n_edges, n_rot, device):
@@ -159,6 +214,9 @@ def main():
 
     if args.workload in ("copy", "read"):
         membench(args.workload, args.steps, args.warmup)
+        return
+    if args.workload == "uvw_fwd":
+        uvw_bench(args)
         return
 
     from equitorch_amd.nn import SO3Linear
