@@ -2,7 +2,7 @@
 on the matrix cores.
 
 Evaluation order is weight-first: for every weight path ``p`` and every row ``a`` of the channelled input that the
-path reads, one accumulator tile ``Z[w, n] = sum_u Wt[p][w, u] * x[n, a, u]`` (32 output channels x 32 samples,
+path reads, two accumulator tiles ``Z[w, n] = sum_u Wt[p][w, u] * x[n, a, u]`` (2 x 16 output channels x 16 samples,
 K = C_in, bf16 MFMA with fp32 accumulation), then the Clebsch-Gordan stage as fp32 FMAs on accumulator tiles,
 ``out[m] += (coef * y[n, b]) * Z`` — in the MFMA accumulator layout every lane belongs to one sample, so the
 harmonic ``y[n, b]`` is a per-lane scalar and the stage needs no data movement.  Nothing of size
@@ -47,9 +47,9 @@ def emit_direction(name: str, direction: int, coo, seg_out, seg_in1) -> str:
     a("  template <int CIN, class LoadA, class Store>")
     a("  __device__ __forceinline__ static void run(const unsigned char* xs, LoadA&& load_a, const float (&y)[D2],")
     a("                                             Store&& store) {")
-    a("    constexpr int KS = CIN / 16;")
-    a("    bf16x8 wa[KS], wb[KS];")
-    a("    floatx16 za, zb;")
+    a("    constexpr int KS = CIN / 32;")
+    a("    bf16x8 wa[2][KS], wb[2][KS];")
+    a("    floatx4 za0, za1, zb0, zb1;")
     a("    float yy[D2];")
     a("    for (int j = 0; j < D2; ++j) yy[j] = y[j];")
     for b0, b1 in zip(blocks[:-1], blocks[1:]):
@@ -57,9 +57,9 @@ def emit_direction(name: str, direction: int, coo, seg_out, seg_in1) -> str:
         nnz = [t for t in range(T) if b0 <= out_idx[t] < b1]
         if not nnz:
             a("    {")
-            a("      floatx16 zero = {0};")
+            a("      floatx4 zero = {0};")
             for r in rows:
-                a(f"      store({r}, zero);")
+                a(f"      store({r}, zero, zero);")
             a("    }")
             continue
         # tiles of this block: (path, input row) -> [(out row, y index, coef)]
@@ -70,13 +70,13 @@ def emit_direction(name: str, direction: int, coo, seg_out, seg_in1) -> str:
         paths = list(OrderedDict.fromkeys(p for p, _ in keys))
         a("    {")
         for r in rows:
-            a(f"      floatx16 o{r} = {{0}};")
+            a(f"      floatx4 o{r}_0 = {{0}}, o{r}_1 = {{0}};")
         a(f"      load_a({paths[0]}, wa);")
         # software pipeline: the MFMA chain of tile k+1 is issued before the FMAs that consume tile k
         def chain(dst, key):
             p, row = key
             frag = "wa" if paths.index(p) % 2 == 0 else "wb"
-            a(f"      {dst} = mfma_chain<KS>({frag}, xs + {row} * CIN * 2);")
+            a(f"      mfma_chain<KS>({frag}, xs + {row} * CIN * 2, {dst}0, {dst}1);")
         prev_path = None
         for k, key in enumerate(keys):
             p = key[0]
@@ -95,12 +95,16 @@ def emit_direction(name: str, direction: int, coo, seg_out, seg_in1) -> str:
             # tiles and would otherwise be computed once and kept in registers across the whole body
             a("      " + " ".join(f'asm volatile("" : "+v"(yy[{m}]));' for m in sorted({m2 for _, m2, _ in tiles[key]})))
             for (o, m2, c) in tiles[key]:
-                a(f"      o{o} += ({_lit(c)} * yy[{m2}]) * {cur};")
+                a(f"      {{ const float s = {_lit(c)} * yy[{m2}]; o{o}_0 += s * {cur}0; o{o}_1 += s * {cur}1; }}")
+            # pin the updated accumulators: an output row is read again only when it is stored, and without this the
+            # optimiser sinks every update of a block to its end, keeping all the block's tiles alive until then
+            touched = sorted({o for o, _, _ in tiles[key]})
+            a("      asm volatile(\"\" : " + ", ".join(f'"+v"(o{o}_0), "+v"(o{o}_1)' for o in touched) + ");")
             # the scheduler may interleave the MFMA chain above with these FMAs, but nothing crosses this point:
             # without it weight-fragment loads and whole chains are hoisted until thousands of registers are live
             a("      __builtin_amdgcn_sched_barrier(0);")
         for r in rows:
-            a(f"      store({r}, o{r});")
+            a(f"      store({r}, o{r}_0, o{r}_1);")
         a("    }")
     a("  }")
     a("};")

@@ -2,13 +2,16 @@
 //
 //   out[n, m, w] = sum_t coef_t * y[n, b_t] * sum_u x[n, a_t, u] * W[p_t, u, w]
 //
-// A workgroup owns 32 samples and stages their whole input rows (DIN x C_in bf16 per sample) in LDS once; each
-// of its four wavefronts owns 32-wide blocks of output channels.  Per weight path and input row the wavefront
-// forms one 32(channels) x 32(samples) accumulator tile with C_in/16 MFMAs (v_mfma_f32_32x32x16_bf16: A = 16-byte
-// weight fragments held in registers for the whole path, B = 16-byte fragments of the staged input read from
-// LDS), and then applies the Clebsch-Gordan coefficients as fp32 FMAs between accumulator tiles: in the
-// accumulator layout a lane belongs to exactly one sample, so coef * y[n, b] is a per-lane scalar.  The staged
-// rows are padded by 16 bytes per sample so that the 16 lanes of one LDS phase hit distinct banks.
+// A workgroup owns 16 samples and stages their whole input rows (DIN x C_in bf16 per sample) in LDS once; each
+// of its four wavefronts owns a 32-wide block of output channels.  Per weight path and input row the wavefront
+// forms two 16(channels) x 16(samples) accumulator tiles with 2 * C_in/32 MFMAs (v_mfma_f32_16x16x32_bf16: A =
+// 16-byte weight fragments held in registers for the whole path, B = 16-byte fragments of the staged input read
+// from LDS and shared by both tiles), and then applies the Clebsch-Gordan coefficients as fp32 FMAs between
+// accumulator tiles: in the accumulator layout a lane belongs to exactly one sample, so coef * y[n, b] is a
+// per-lane scalar.  Output rows are finished one output irrep at a time, which keeps the live accumulators to
+// (2l+1) * 8 registers; the whole wavefront fits 256 registers, so two workgroups share a compute unit and one
+// stages its input while the other computes.  The staged rows are padded by 16 bytes per sample so that the 16
+// lanes of one LDS phase hit distinct banks.
 #include "cgtp_device.h"
 #include "cgtp_host.h"
 
@@ -18,28 +21,29 @@
 namespace cgtp {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-// Z[w, n] = sum_k A[w, k] * B[k, n] over KS steps of 16; xs points at this lane's 8 consecutive k of step 0.
+// Z_t[w, n] = sum_k A_t[w, k] * B[k, n] for the two channel tiles t over KS steps of 32; xs points at this lane's
+// 8 consecutive k of step 0.
 template <int KS>
-__device__ __forceinline__ floatx16 mfma_chain(const bf16x8 (&a)[KS], const unsigned char* xs) {
-  floatx16 z = {0};
+__device__ __forceinline__ void mfma_chain(const bf16x8 (&a)[2][KS], const unsigned char* xs, floatx4& z0,
+                                           floatx4& z1) {
+  z0 = floatx4{0.f, 0.f, 0.f, 0.f};
+  z1 = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int k = 0; k < KS; ++k) {
-    const bf16x8 b = *reinterpret_cast<const bf16x8*>(xs + k * 32);
-    z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[k], b, z, 0, 0, 0);
+    const bf16x8 b = *reinterpret_cast<const bf16x8*>(xs + k * 64);
+    z0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[0][k], b, z0, 0, 0, 0);
+    z1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[1][k], b, z1, 0, 0, 0);
   }
-  return z;
 }
 
 #include "generated/uv_configs.inc"
 
-constexpr int kUvSamples = 32;
+constexpr int kUvSamples = 16;
 
 template <class CFG, int CIN>
-__global__ void __launch_bounds__(256, 1) uv_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ y,
+__global__ void __launch_bounds__(256, 2) uv_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ y,
                                                     const __bf16* __restrict__ wt, __bf16* __restrict__ out,
                                                     int64_t n_rows, int cout) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -48,7 +52,7 @@ __global__ void __launch_bounds__(256, 1) uv_kernel(const __bf16* __restrict__ x
   constexpr int ROW_PITCH = ROW_BYTES + 16;     // + pad: consecutive samples start 16 B further in the banks
   const int64_t n0 = (int64_t)blockIdx.x * kUvSamples;
 
-  // stage the 32 samples' rows: 16-byte pieces, coalesced in global memory
+  // stage the 16 samples' rows: 16-byte pieces, coalesced in global memory
   constexpr int PIECES = ROW_BYTES / 16;
   for (int i = threadIdx.x; i < kUvSamples * PIECES; i += blockDim.x) {
     const int s = i / PIECES, c = i % PIECES;
@@ -60,40 +64,43 @@ __global__ void __launch_bounds__(256, 1) uv_kernel(const __bf16* __restrict__ x
   __syncthreads();
 
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  const int n = lane & 31, half = lane >> 5;
+  const int n = lane & 15, q = lane >> 4;
   const bool valid = n0 + n < n_rows;
   float yv[D2];
 #pragma unroll
   for (int j = 0; j < D2; ++j) yv[j] = valid ? (float)y[(n0 + n) * D2 + j] : 0.f;
-  const unsigned char* xs = smem + n * ROW_PITCH + half * 16;
+  const unsigned char* xs = smem + n * ROW_PITCH + q * 16;
 
-  // one 32-channel block per wavefront, blockIdx.y tiles wider outputs (a loop over blocks here would let the
-  // compiler hoist every loop-invariant LDS fragment read of the body out of it, thousands of registers)
+  // one 32-channel block per wavefront, blockIdx.y tiles wider outputs
   const int wblk = blockIdx.y * (blockDim.x / kWave) + wave;
   if (wblk * 32 >= cout) return;
-  {
-    // A fragment: lane holds Wt[p][w = wblk*32 + n][k*16 + half*8 .. +8]
-    const __bf16* wrow = wt + (int64_t)(wblk * 32 + n) * CIN + half * 8;
-    const int64_t path_stride = (int64_t)cout * CIN;
-    __bf16* orow = out + (n0 + n) * DOUT * cout + wblk * 32 + 4 * half;
-    CFG::template run<CIN>(
-        xs,
-        [&](int p, bf16x8(&frag)[CIN / 16]) __attribute__((always_inline)) {
+  // Row r = 4*g + i of channel tile t is output channel wblk*32 + 8*g + 4*t + i, so that in the accumulator layout
+  // (lane (n, q) holds rows 4*q .. 4*q+3 of column n) a lane ends up with 8 consecutive channels of its sample.
+  // A fragment: lane (r = lane & 15, q) holds Wt[p][channel(t, r)][k*32 + q*8 .. +8]
+  const __bf16* wrow = wt + (int64_t)(wblk * 32 + 8 * (n >> 2) + (n & 3)) * CIN + q * 8;
+  const int64_t path_stride = (int64_t)cout * CIN;
+  __bf16* orow = out + (n0 + n) * DOUT * cout + wblk * 32 + 8 * q;
+  CFG::template run<CIN>(
+      xs,
+      [&](int p, bf16x8(&frag)[2][CIN / 32]) __attribute__((always_inline)) {
 #pragma unroll
-          for (int k = 0; k < CIN / 16; ++k) frag[k] = *reinterpret_cast<const bf16x8*>(wrow + p * path_stride + k * 16);
-        },
-        yv,
-        [&](int row, const floatx16& o) __attribute__((always_inline)) {
-          // accumulator element i is output channel 8*(i/4) + 4*half + i%4 of this block
-          if (valid) {
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const floatx4 f = {o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
-              *reinterpret_cast<bf16x4*>(orow + row * cout + 8 * j) = __builtin_convertvector(f, bf16x4);
-            }
+          for (int k = 0; k < CIN / 32; ++k)
+            frag[t][k] = *reinterpret_cast<const bf16x8*>(wrow + p * path_stride + t * 4 * CIN + k * 32);
+      },
+      yv,
+      [&](int row, const floatx4& o0, const floatx4& o1) __attribute__((always_inline)) {
+        if (valid) {
+          bf16x8 v;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            v[i] = (__bf16)o0[i];
+            v[4 + i] = (__bf16)o1[i];
           }
-        });
-  }
+          *reinterpret_cast<bf16x8*>(orow + row * cout) = v;
+        }
+      });
 }
 
 using UvFn = void (*)(const __bf16*, const __bf16*, const __bf16*, __bf16*, int64_t, int);
