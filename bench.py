@@ -95,7 +95,7 @@ def uvw_bench(args):
     sh = spherical_harmonics(vec / vec.norm(dim=-1, keepdim=True), lmax).bfloat16().to(dev)
     w = (torch.randn(mod.num_paths, ch, ch, generator=gen) / (ch * mod.num_paths) ** 0.5).bfloat16().to(dev)
     cfg = _uvw_mfma.uv_config_of(mod.tp_info_forward)
-    wt = w.transpose(-1, -2).contiguous()
+    wt = _uvw_mfma.pack_weights(0, w)
     s1 = int(mod.tp_info_forward.info_Mij_fwd.out_size)
     flops = 2.0 * n * s1 * ch * ch
 

@@ -88,6 +88,8 @@ def _load():
     lib.cgtp_uv_find.argtypes = [C.c_uint64]
     _uv = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32,
            C.c_int32]
+    lib.cgtp_uv_pack_weights.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
+                                         C.c_void_p]
     lib.cgtp_uv_validate.argtypes = _uv
     lib.cgtp_uv_apply.argtypes = _uv + [C.c_void_p]
     lib.cgtp_membench_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]

@@ -38,74 +38,99 @@ def emit_direction(name: str, direction: int, coo, seg_out, seg_in1) -> str:
     else:
         out_idx, in_idx, blocks, din, dout = coo.M1, coo.M, seg_in1, coo.DO, coo.D1
     T = coo.coef.shape[0]
+    # tiles in execution order: output irrep by output irrep (an output row is live only while its block runs),
+    # inside a block path by path; tile = (path, input row) -> [(out row, y index, coef)]
+    tiles, first_of_block, last_of_block, empty_rows = [], {}, {}, []
+    for b0, b1 in zip(blocks[:-1], blocks[1:]):
+        nnz = [t for t in range(T) if b0 <= out_idx[t] < b1]
+        if not nnz:
+            empty_rows += list(range(b0, b1))
+            continue
+        d = OrderedDict()
+        for t in sorted(nnz, key=lambda t: (coo.p[t], in_idx[t], out_idx[t], coo.M2[t])):
+            d.setdefault((int(coo.p[t]), int(in_idx[t])), []).append((int(out_idx[t]), int(coo.M2[t]), coo.coef[t]))
+        first_of_block[len(tiles)] = list(range(b0, b1))
+        tiles += list(d.items())
+        last_of_block[len(tiles) - 1] = list(range(b0, b1))
+    # weight fragments live in a ring of three buffers, fetched two path-runs ahead of their first use
+    runs = []  # (path, first tile)
+    for k, ((p, _), _) in enumerate(tiles):
+        if not runs or runs[-1][0] != p or k in first_of_block:
+            runs.append((p, k))
+    run_of_tile = {}
+    for j, (p, k0) in enumerate(runs):
+        k1 = runs[j + 1][1] if j + 1 < len(runs) else len(tiles)
+        for k in range(k0, k1):
+            run_of_tile[k] = j
     L = []
     a = L.append
     a(f"struct UV_{name}_d{direction} {{")
     a(f"  static constexpr int DIN = {din}, DOUT = {dout}, D2 = {coo.D2}, P = {coo.P};")
     a("  // xs: this lane's base into the staged input tile (row a of the sample at byte a * CIN * 2);")
-    a("  // load_a(p, frag): fetch the weight fragments of path p; store(row, tile): emit one finished output row.")
+    a("  // load_a(p, frag): fetch the weight fragments of path p; store(row, t0, t1): emit one finished output row.")
     a("  template <int CIN, class LoadA, class Store>")
     a("  __device__ __forceinline__ static void run(const unsigned char* xs, LoadA&& load_a, const float (&y)[D2],")
     a("                                             Store&& store) {")
     a("    constexpr int KS = CIN / 32;")
-    a("    bf16x8 wa[2][KS], wb[2][KS];")
+    a("    bf16x8 w0[2][KS], w1[2][KS], w2[2][KS], b0[KS], b1[KS];")
     a("    floatx4 za0, za1, zb0, zb1;")
     a("    float yy[D2];")
     a("    for (int j = 0; j < D2; ++j) yy[j] = y[j];")
-    for b0, b1 in zip(blocks[:-1], blocks[1:]):
-        rows = list(range(b0, b1))
-        nnz = [t for t in range(T) if b0 <= out_idx[t] < b1]
-        if not nnz:
-            a("    {")
-            a("      floatx4 zero = {0};")
-            for r in rows:
-                a(f"      store({r}, zero, zero);")
-            a("    }")
-            continue
-        # tiles of this block: (path, input row) -> [(out row, y index, coef)]
-        tiles = OrderedDict()
-        for t in sorted(nnz, key=lambda t: (coo.p[t], in_idx[t], out_idx[t], coo.M2[t])):
-            tiles.setdefault((int(coo.p[t]), int(in_idx[t])), []).append((int(out_idx[t]), int(coo.M2[t]), coo.coef[t]))
-        keys = list(tiles)
-        paths = list(OrderedDict.fromkeys(p for p, _ in keys))
+    if empty_rows:
         a("    {")
-        for r in rows:
-            a(f"      floatx4 o{r}_0 = {{0}}, o{r}_1 = {{0}};")
-        a(f"      load_a({paths[0]}, wa);")
-        # software pipeline: the MFMA chain of tile k+1 is issued before the FMAs that consume tile k
-        def chain(dst, key):
-            p, row = key
-            frag = "wa" if paths.index(p) % 2 == 0 else "wb"
-            a(f"      mfma_chain<KS>({frag}, xs + {row} * CIN * 2, {dst}0, {dst}1);")
-        prev_path = None
-        for k, key in enumerate(keys):
-            p = key[0]
-            if p != prev_path:
-                nxt = paths.index(p) + 1
-                if nxt < len(paths):
-                    a(f"      load_a({paths[nxt]}, {'wa' if nxt % 2 == 0 else 'wb'});")
-                prev_path = p
-            if k == 0:
-                chain("za", key)
-            cur = "za" if k % 2 == 0 else "zb"
-            if k + 1 < len(keys):
-                # weight fragments of the next tile's path were requested one path earlier
-                chain("zb" if k % 2 == 0 else "za", keys[k + 1])
-            # hide the harmonics behind an empty asm per tile: equal (coefficient, harmonic) products recur in many
-            # tiles and would otherwise be computed once and kept in registers across the whole body
-            a("      " + " ".join(f'asm volatile("" : "+v"(yy[{m}]));' for m in sorted({m2 for _, m2, _ in tiles[key]})))
-            for (o, m2, c) in tiles[key]:
-                a(f"      {{ const float s = {_lit(c)} * yy[{m2}]; o{o}_0 += s * {cur}0; o{o}_1 += s * {cur}1; }}")
-            # pin the updated accumulators: an output row is read again only when it is stored, and without this the
-            # optimiser sinks every update of a block to its end, keeping all the block's tiles alive until then
-            touched = sorted({o for o, _, _ in tiles[key]})
-            a("      asm volatile(\"\" : " + ", ".join(f'"+v"(o{o}_0), "+v"(o{o}_1)' for o in touched) + ");")
-            # the scheduler may interleave the MFMA chain above with these FMAs, but nothing crosses this point:
-            # without it weight-fragment loads and whole chains are hoisted until thousands of registers are live
-            a("      __builtin_amdgcn_sched_barrier(0);")
-        for r in rows:
-            a(f"      store({r}, o{r}_0, o{r}_1);")
+        a("      floatx4 zero = {0};")
+        for r in empty_rows:
+            a(f"      store({r}, zero, zero);")
         a("    }")
+
+    def load_b(k):
+        a(f"    load_b<KS>(b{k % 2}, xs + {tiles[k][0][1]} * CIN * 2);")
+
+    def chain(k):
+        z = "za" if k % 2 == 0 else "zb"
+        a(f"    mfma_chain<KS>(w{run_of_tile[k] % 3}, b{k % 2}, {z}0, {z}1);")
+        j = run_of_tile[k]
+        if runs[j][1] == k and j + 2 < len(runs):
+            a(f"    load_a({runs[j + 2][0]}, w{(j + 2) % 3});")
+
+    if tiles:
+        a(f"    load_a({runs[0][0]}, w0);")
+        if len(runs) > 1:
+            a(f"    load_a({runs[1][0]}, w1);")
+        load_b(0)
+        if len(tiles) > 1:
+            load_b(1)
+        chain(0)
+        a("    __builtin_amdgcn_sched_barrier(0);")
+    for k, (key, terms) in enumerate(tiles):
+        # slot k: fetch the input fragments of tile k+2, run the MFMA chain of tile k+1, and apply the Clebsch-Gordan
+        # coefficients to tile k, whose chain ran in the previous slot
+        if k in first_of_block:
+            for r in first_of_block[k]:
+                a(f"    floatx4 o{r}_0 = {{0}}, o{r}_1 = {{0}};")
+        if k + 1 < len(tiles):
+            chain(k + 1)
+        if k + 2 < len(tiles):
+            load_b(k + 2)
+        cur = "za" if k % 2 == 0 else "zb"
+        # hide the harmonics behind an empty asm per tile: equal (coefficient, harmonic) products recur in many
+        # tiles and would otherwise be computed once and kept in registers across the whole body
+        a("    " + " ".join(f'asm volatile("" : "+v"(yy[{m}]));' for m in sorted({m2 for _, m2, _ in terms})))
+        a("#ifndef UV_ABL_NOFMA")
+        for (o, m2, c) in terms:
+            a(f"    {{ const float s = {_lit(c)} * yy[{m2}]; o{o}_0 += s * {cur}0; o{o}_1 += s * {cur}1; }}")
+        a("#else")
+        a(f'    asm volatile("" :: "v"({cur}0), "v"({cur}1));')
+        a("#endif")
+        # pin the updated accumulators: an output row is read again only when it is stored, and without this the
+        # optimiser sinks every update of a block to its end, keeping all the block's tiles alive until then
+        touched = sorted({o for o, _, _ in terms})
+        a("    asm volatile(\"\" : " + ", ".join(f'"+v"(o{o}_0), "+v"(o{o}_1)' for o in touched) + ");")
+        # the scheduler may interleave the MFMA chain above with these FMAs, but nothing crosses this point
+        a("    __builtin_amdgcn_sched_barrier(0);")
+        if k in last_of_block:
+            for r in last_of_block[k]:
+                a(f"    store({r}, o{r}_0, o{r}_1);")
     a("  }")
     a("};")
     return "\n".join(L)

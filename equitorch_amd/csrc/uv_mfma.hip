@@ -23,18 +23,32 @@ namespace cgtp {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-// Z_t[w, n] = sum_k A_t[w, k] * B[k, n] for the two channel tiles t over KS steps of 32; xs points at this lane's
-// 8 consecutive k of step 0.
+// this lane's 8 consecutive k of every K step of one staged input row
 template <int KS>
-__device__ __forceinline__ void mfma_chain(const bf16x8 (&a)[2][KS], const unsigned char* xs, floatx4& z0,
-                                           floatx4& z1) {
-  z0 = floatx4{0.f, 0.f, 0.f, 0.f};
-  z1 = floatx4{0.f, 0.f, 0.f, 0.f};
+__device__ __forceinline__ void load_b(bf16x8 (&b)[KS], const unsigned char* xs) {
 #pragma unroll
   for (int k = 0; k < KS; ++k) {
-    const bf16x8 b = *reinterpret_cast<const bf16x8*>(xs + k * 64);
-    z0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[0][k], b, z0, 0, 0, 0);
-    z1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[1][k], b, z1, 0, 0, 0);
+#ifdef UV_ABL_NOB
+    asm volatile("" : "=v"(b[k]) : "v"(xs));
+#else
+    b[k] = *reinterpret_cast<const bf16x8*>(xs + k * 64);
+#endif
+  }
+}
+
+// Z_t[w, n] = sum_k A_t[w, k] * B[k, n] for the two channel tiles t over KS steps of 32
+template <int KS>
+__device__ __forceinline__ void mfma_chain(const bf16x8 (&a)[2][KS], const bf16x8 (&b)[KS], floatx4& z0, floatx4& z1) {
+  z0 = floatx4{0.f, 0.f, 0.f, 0.f};
+  z1 = floatx4{0.f, 0.f, 0.f, 0.f};
+#ifdef UV_ABL_NOMFMA
+  asm volatile("" : "+v"(z0), "+v"(z1) : "v"(a[0][0]), "v"(a[1][KS-1]), "v"(b[0]), "v"(b[KS-1]));
+  return;
+#endif
+#pragma unroll
+  for (int k = 0; k < KS; ++k) {
+    z0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[0][k], b[k], z0, 0, 0, 0);
+    z1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[1][k], b[k], z1, 0, 0, 0);
   }
 }
 
@@ -42,33 +56,52 @@ __device__ __forceinline__ void mfma_chain(const bf16x8 (&a)[2][KS], const unsig
 
 constexpr int kUvSamples = 16;
 
+#ifdef CGTP_UV_TRACE
+__device__ unsigned long long* g_uv_trace;
+#define UV_MARK(k) do { if ((threadIdx.x & 63) == 0) g_uv_trace[((int64_t)blockIdx.x * 4 + threadIdx.x / 64) * 8 + (k)] = clock64(); } while (0)
+#else
+#define UV_MARK(k)
+#endif
+
 template <class CFG, int CIN>
 __global__ void __launch_bounds__(256, 2) uv_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ y,
-                                                    const __bf16* __restrict__ wt, __bf16* __restrict__ out,
+                                                    const __bf16* __restrict__ wp, __bf16* __restrict__ out,
                                                     int64_t n_rows, int cout) {
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int DIN = CFG::DIN, DOUT = CFG::DOUT, D2 = CFG::D2;
   constexpr int ROW_BYTES = DIN * CIN * 2;      // one sample's input rows
   constexpr int ROW_PITCH = ROW_BYTES + 16;     // + pad: consecutive samples start 16 B further in the banks
   const int64_t n0 = (int64_t)blockIdx.x * kUvSamples;
+  UV_MARK(0);
 
-  // stage the 16 samples' rows: 16-byte pieces, coalesced in global memory
-  constexpr int PIECES = ROW_BYTES / 16;
-  for (int i = threadIdx.x; i < kUvSamples * PIECES; i += blockDim.x) {
-    const int s = i / PIECES, c = i % PIECES;
-    f32x4 v = {0.f, 0.f, 0.f, 0.f};
-    if (n0 + s < n_rows)
-      v = *reinterpret_cast<const f32x4*>(reinterpret_cast<const unsigned char*>(x) + (n0 + s) * ROW_BYTES + c * 16);
-    *reinterpret_cast<f32x4*>(smem + s * ROW_PITCH + c * 16) = v;
+  // stage the 16 samples' rows: 16-byte pieces, coalesced in global memory; every load is issued before the
+  // first LDS write.  Rows past the end of the batch re-read the last row (their results are never stored).
+  constexpr int PIECES = ROW_BYTES / 16, TOTAL = kUvSamples * PIECES, PER_THREAD = (TOTAL + 255) / 256;
+  constexpr int UNROLL = PER_THREAD < 16 ? PER_THREAD : 16;
+  for (int base = 0; base < TOTAL; base += 256 * UNROLL) {
+    f32x4 v[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int i = min(base + u * 256 + (int)threadIdx.x, TOTAL - 1), s = i / PIECES, c = i % PIECES;
+      const int64_t row = min(n0 + s, n_rows - 1);
+      v[u] = *reinterpret_cast<const f32x4*>(reinterpret_cast<const unsigned char*>(x) + row * ROW_BYTES + c * 16);
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int i = min(base + u * 256 + (int)threadIdx.x, TOTAL - 1), s = i / PIECES, c = i % PIECES;
+      *reinterpret_cast<f32x4*>(smem + s * ROW_PITCH + c * 16) = v[u];
+    }
   }
+  UV_MARK(1);
   __syncthreads();
+  UV_MARK(2);
 
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int n = lane & 15, q = lane >> 4;
   const bool valid = n0 + n < n_rows;
   float yv[D2];
 #pragma unroll
-  for (int j = 0; j < D2; ++j) yv[j] = valid ? (float)y[(n0 + n) * D2 + j] : 0.f;
+  for (int j = 0; j < D2; ++j) yv[j] = (float)y[min(n0 + n, n_rows - 1) * D2 + j];
   const unsigned char* xs = smem + n * ROW_PITCH + q * 16;
 
   // one 32-channel block per wavefront, blockIdx.y tiles wider outputs
@@ -76,8 +109,9 @@ __global__ void __launch_bounds__(256, 2) uv_kernel(const __bf16* __restrict__ x
   if (wblk * 32 >= cout) return;
   // Row r = 4*g + i of channel tile t is output channel wblk*32 + 8*g + 4*t + i, so that in the accumulator layout
   // (lane (n, q) holds rows 4*q .. 4*q+3 of column n) a lane ends up with 8 consecutive channels of its sample.
-  // A fragment: lane (r = lane & 15, q) holds Wt[p][channel(t, r)][k*32 + q*8 .. +8]
-  const __bf16* wrow = wt + (int64_t)(wblk * 32 + 8 * (n >> 2) + (n & 3)) * CIN + q * 8;
+  // The weights arrive packed in fragment order (uv_pack_kernel): per (path, channel block) 2 * KS chunks of 1 KB,
+  // chunk t * KS + k holding the 16 bytes of every lane, so that a wavefront's load is one contiguous KB.
+  const __bf16* wfrag = wp + (int64_t)wblk * (2 * (CIN / 32) * 512) + lane * 8;
   const int64_t path_stride = (int64_t)cout * CIN;
   __bf16* orow = out + (n0 + n) * DOUT * cout + wblk * 32 + 8 * q;
   CFG::template run<CIN>(
@@ -87,7 +121,13 @@ __global__ void __launch_bounds__(256, 2) uv_kernel(const __bf16* __restrict__ x
         for (int t = 0; t < 2; ++t)
 #pragma unroll
           for (int k = 0; k < CIN / 32; ++k)
-            frag[t][k] = *reinterpret_cast<const bf16x8*>(wrow + p * path_stride + t * 4 * CIN + k * 32);
+#ifdef UV_ABL_NOA
+            asm volatile("" : "=v"(frag[t][k]) : "v"(wfrag));
+#elif defined(UV_ABL_A0)
+            frag[t][k] = *reinterpret_cast<const volatile bf16x8*>(wfrag + (p & 1) * path_stride + (t * (CIN / 32) + k) * 512);
+#else
+            frag[t][k] = *reinterpret_cast<const bf16x8*>(wfrag + p * path_stride + (t * (CIN / 32) + k) * 512);
+#endif
       },
       yv,
       [&](int row, const floatx4& o0, const floatx4& o1) __attribute__((always_inline)) {
@@ -100,7 +140,33 @@ __global__ void __launch_bounds__(256, 2) uv_kernel(const __bf16* __restrict__ x
           }
           *reinterpret_cast<bf16x8*>(orow + row * cout) = v;
         }
+        if (row == 0) UV_MARK(3);
+        if (row == 3) UV_MARK(4);
+        if (row == 8) UV_MARK(5);
       });
+  UV_MARK(6);
+}
+
+// packed[p][blk][t][k][lane = 16*q + r][e] = Wt[p][blk*32 + 8*(r/4) + 4*t + r%4][k*32 + 8*q + e], where
+// Wt[p][row][col] = w[p * rows * cols + row * row_stride + col * col_stride]; one thread per 16-byte piece.
+__global__ void uv_pack_kernel(const __bf16* __restrict__ w, __bf16* __restrict__ packed, int64_t n_pieces, int rows,
+                               int cols, int64_t row_stride, int64_t col_stride) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_pieces) return;
+  const int ks = cols / 32, nblk = rows / 32;
+  const int lane = (int)(i & 63);
+  int64_t c = i >> 6;
+  const int k = (int)(c % ks); c /= ks;
+  const int t = (int)(c & 1); c >>= 1;
+  const int blk = (int)(c % nblk);
+  const int64_t p = c / nblk;
+  const int r = lane & 15, q = lane >> 4;
+  const int64_t row = blk * 32 + 8 * (r >> 2) + 4 * t + (r & 3), col = k * 32 + 8 * q;
+  const __bf16* src = w + p * rows * cols + row * row_stride + col * col_stride;
+  bf16x8 v;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = src[e * col_stride];
+  *reinterpret_cast<bf16x8*>(packed + i * 8) = v;
 }
 
 using UvFn = void (*)(const __bf16*, const __bf16*, const __bf16*, __bf16*, int64_t, int);
@@ -131,18 +197,18 @@ static const UvEntry* uv_entries(int* count) {
   return table;
 }
 
-static int uv_check(int cfg, int direction, const void* x, const void* y, const void* wt, const void* out,
+static int uv_check(int cfg, int direction, const void* x, const void* y, const void* wp, const void* out,
                     int64_t n_rows, int cin, int cout, int dtype, int* ci, int64_t* lds) {
   int n = 0;
   const UvEntry* t = uv_entries(&n);
   if (cfg < 0 || cfg >= n) return CGTP_ERR_CONFIG;
   if (direction != 0 && direction != 1) return CGTP_ERR_SHAPE;
   if (dtype != CGTP_BF16) return CGTP_ERR_DTYPE;
-  if (!x || !y || !wt || !out) return CGTP_ERR_NULL;
+  if (!x || !y || !wp || !out) return CGTP_ERR_NULL;
   if (n_rows < 0 || cout <= 0 || cout % 32 != 0) return CGTP_ERR_SHAPE;
   *ci = cin == 32 ? 0 : cin == 64 ? 1 : cin == 128 ? 2 : -1;
   if (*ci < 0) return CGTP_ERR_SHAPE;
-  const uintptr_t al = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(wt) | reinterpret_cast<uintptr_t>(out);
+  const uintptr_t al = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(wp) | reinterpret_cast<uintptr_t>(out);
   if (al & 15u) return CGTP_ERR_ALIGN;
   *lds = (int64_t)kUvSamples * ((int64_t)t[cfg].din[direction] * cin * 2 + 16);
   if (*lds > kLdsBytes) return CGTP_ERR_LDS;
@@ -169,18 +235,35 @@ int cgtp_uv_find(uint64_t fingerprint) {
   return -1;
 }
 
-int cgtp_uv_validate(int cfg, int direction, const void* x, const void* y, const void* wt, const void* out,
+int cgtp_uv_pack_weights(int direction, const void* w, void* packed, int32_t n_paths, int32_t cin, int32_t cout,
+                         int32_t dtype, void* stream) {
+  if (direction != 0 && direction != 1) return CGTP_ERR_SHAPE;
+  if (dtype != CGTP_BF16) return CGTP_ERR_DTYPE;
+  if (!w || !packed) return CGTP_ERR_NULL;
+  if (n_paths < 0 || cin <= 0 || cout <= 0 || cin % 32 != 0 || cout % 32 != 0) return CGTP_ERR_SHAPE;
+  if ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(packed)) & 15u) return CGTP_ERR_ALIGN;
+  if (n_paths == 0) return CGTP_OK;
+  // rows = result channels, cols = contracted channels; direction 0 reads W (P, cin, cout) transposed, direction 1
+  // reads W (P, cout, cin) as stored
+  const int64_t n_pieces = (int64_t)n_paths * cin * cout / 8;
+  const int64_t row_stride = direction == 0 ? 1 : cin, col_stride = direction == 0 ? cout : 1;
+  hipLaunchKernelGGL(uv_pack_kernel, dim3((unsigned)((n_pieces + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const __bf16*)w, (__bf16*)packed, n_pieces, (int)cout, (int)cin, row_stride, col_stride);
+  return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
+}
+
+int cgtp_uv_validate(int cfg, int direction, const void* x, const void* y, const void* wp, const void* out,
                      int64_t n_rows, int32_t cin, int32_t cout, int32_t dtype) {
   int ci = 0;
   int64_t lds = 0;
-  return uv_check(cfg, direction, x, y, wt, out, n_rows, cin, cout, dtype, &ci, &lds);
+  return uv_check(cfg, direction, x, y, wp, out, n_rows, cin, cout, dtype, &ci, &lds);
 }
 
-int cgtp_uv_apply(int cfg, int direction, const void* x, const void* y, const void* wt, void* out, int64_t n_rows,
+int cgtp_uv_apply(int cfg, int direction, const void* x, const void* y, const void* wp, void* out, int64_t n_rows,
                   int32_t cin, int32_t cout, int32_t dtype, void* stream) {
   int ci = 0;
   int64_t lds = 0;
-  const int st = uv_check(cfg, direction, x, y, wt, out, n_rows, cin, cout, dtype, &ci, &lds);
+  const int st = uv_check(cfg, direction, x, y, wp, out, n_rows, cin, cout, dtype, &ci, &lds);
   if (st != CGTP_OK) return st;
   if (n_rows == 0) return CGTP_OK;
   int n = 0;
@@ -189,7 +272,7 @@ int cgtp_uv_apply(int cfg, int direction, const void* x, const void* y, const vo
     return CGTP_ERR_LDS;
   hipLaunchKernelGGL(fn, dim3((unsigned)((n_rows + kUvSamples - 1) / kUvSamples), (unsigned)((cout + 127) / 128)),
                      dim3(256), (size_t)lds,
-                     (hipStream_t)stream, (const __bf16*)x, (const __bf16*)y, (const __bf16*)wt, (__bf16*)out, n_rows,
+                     (hipStream_t)stream, (const __bf16*)x, (const __bf16*)y, (const __bf16*)wp, (__bf16*)out, n_rows,
                      (int)cout);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }

@@ -1,5 +1,6 @@
 """Dispatch of the fully connected ("uv") product to the bf16 matrix-core kernel (``cgtp_uv_apply``)."""
 import ctypes as C
+import weakref
 from typing import Optional
 
 import torch
@@ -17,11 +18,41 @@ def uv_config_of(tp_info) -> int:
                           lambda: int(_lib.lib.cgtp_uv_find(C.c_uint64(fingerprint(kernels.coo_of(tp_info))))))
 
 
-def _apply(cfg: int, direction: int, x: Tensor, y: Tensor, wt: Tensor, d_out: int) -> Tensor:
+_packed = {}  # (id(w), direction) -> (weakref to w, its version counter, packed copy)
+
+
+def pack_weights(direction: int, w: Tensor) -> Tensor:
+    """W as stored by the module, (P, C_in, C_out), rewritten in the fragment order the kernel reads.  The packed
+    copy is kept until the weight tensor is modified in place (its version counter moves) or dies."""
+    key = (id(w), direction)
+    hit = _packed.get(key)
+    if hit is not None and hit[0]() is w and hit[1] == w._version:
+        return hit[2]
+    packed = _pack(direction, w)
+    if len(_packed) >= 64:
+        for k in [k for k, v in _packed.items() if v[0]() is None]:
+            del _packed[k]
+        if len(_packed) >= 64:
+            _packed.clear()
+    _packed[key] = (weakref.ref(w), w._version, packed)
+    return packed
+
+
+def _pack(direction: int, w: Tensor) -> Tensor:
+    w = w.contiguous()
+    cin, cout = (w.shape[1], w.shape[2]) if direction == 0 else (w.shape[2], w.shape[1])
+    packed = torch.empty_like(w)
+    _lib.check(_lib.lib.cgtp_uv_pack_weights(direction, w.data_ptr(), packed.data_ptr(), w.shape[0], cin, cout,
+                                             _lib.BF16, _lib.stream_ptr(w.device)), "cgtp_uv_pack_weights")
+    return packed
+
+
+def _apply(cfg: int, direction: int, x: Tensor, y: Tensor, wp: Tensor, d_out: int) -> Tensor:
+    """``wp`` = ``pack_weights(direction, W)``."""
     n, _, cin = x.shape
-    cout = wt.shape[1]
+    cout = wp.numel() // (wp.shape[0] * cin)
     out = torch.empty((n, d_out, cout), dtype=x.dtype, device=x.device)
-    _lib.check(_lib.lib.cgtp_uv_apply(cfg, direction, x.data_ptr(), y.data_ptr(), wt.data_ptr(), out.data_ptr(), n,
+    _lib.check(_lib.lib.cgtp_uv_apply(cfg, direction, x.data_ptr(), y.data_ptr(), wp.data_ptr(), out.data_ptr(), n,
                                       cin, cout, _lib.BF16, _lib.stream_ptr(x.device)), "cgtp_uv_apply")
     return out
 
@@ -33,7 +64,7 @@ class _UvMfma(Function):
     @staticmethod
     def forward(ctx, x: Tensor, y: Tensor, w: Tensor, tp_info, cfg: int):
         coo = kernels.coo_of(tp_info)
-        out = _apply(cfg, 0, x, y, w.transpose(-1, -2).contiguous(), coo.DO)
+        out = _apply(cfg, 0, x, y, pack_weights(0, w), coo.DO)
         ctx.save_for_backward(x, y, w)
         ctx.tp_info, ctx.cfg, ctx.d1 = tp_info, cfg, coo.D1
         return out
@@ -49,7 +80,7 @@ class _UvMfma(Function):
                 if torch.is_grad_enabled():
                     gx = tri(spec.grad_spec(0), ("w", "", "uw"), "u", g, y, w)
                 else:
-                    gx = _apply(ctx.cfg, 1, g.contiguous(), y, w.contiguous(), ctx.d1)
+                    gx = _apply(ctx.cfg, 1, g.contiguous(), y, pack_weights(1, w), ctx.d1)
             if need[1]:
                 gy = tri(spec.grad_spec(1), ("u", "w", "uw"), "", x, g, w)
             if need[2]:

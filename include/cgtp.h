@@ -200,16 +200,22 @@ int cgtp_uvu_bwd(const cgtp_uvu_args* args, void* stream);
  * indexed_vecsca_scale_gather then indexed_vecmat_scale_gather, with the (N, segments, C_in) intermediate in
  * memory) and, with direction = 1, for the grad-input1 product of its backward (:290-293).  The table is compiled
  * in; cgtp_uv_find() maps the fingerprint of the forward table to a config id (or -1).
- *   direction 0: x = input1 (n_rows, D1, cin), out (n_rows, DO, cout), wt = W transposed to (P, cout, cin);
- *   direction 1: x = grad_out (n_rows, DO, cin), out = grad_input1 (n_rows, D1, cout), wt = W as stored
- *                (P, C_in, C_out) (here cin = C_out of the module and cout = its C_in).
+ *   direction 0: x = input1 (n_rows, D1, cin), out (n_rows, DO, cout), W stored (P, cin, cout);
+ *   direction 1: x = grad_out (n_rows, DO, cin), out = grad_input1 (n_rows, D1, cout), W stored (P, cout, cin)
+ *                (here cin = C_out of the module and cout = its C_in).
  * y is (n_rows, D2).  cin in {32, 64, 128}, cout a multiple of 32, dtype CGTP_BF16, 16-byte aligned pointers.
+ *
+ * The kernel reads the weight in matrix-core fragment order, wp: cgtp_uv_pack_weights() rewrites W as stored by the
+ * module (same element count, one small launch per weight update and direction) so that every wavefront load of
+ * weight fragments is one contiguous KB; strided 64-byte pieces reach a third of that rate from L2.
  */
 int cgtp_uv_num_configs(void);
 int cgtp_uv_find(uint64_t fingerprint);
-int cgtp_uv_validate(int cfg, int direction, const void* x, const void* y, const void* wt, const void* out,
+int cgtp_uv_pack_weights(int direction, const void* w, void* packed, int32_t n_paths, int32_t cin, int32_t cout,
+                         int32_t dtype, void* stream);
+int cgtp_uv_validate(int cfg, int direction, const void* x, const void* y, const void* wp, const void* out,
                      int64_t n_rows, int32_t cin, int32_t cout, int32_t dtype);
-int cgtp_uv_apply(int cfg, int direction, const void* x, const void* y, const void* wt, void* out, int64_t n_rows,
+int cgtp_uv_apply(int cfg, int direction, const void* x, const void* y, const void* wp, void* out, int64_t n_rows,
                   int32_t cin, int32_t cout, int32_t dtype, void* stream);
 
 /* ---- streaming kernels of known traffic (counter calibration, achievable-bandwidth reference) ------------
