@@ -32,7 +32,10 @@ CONFIGS = OrderedDict([
 ])
 
 
-def emit_direction(name: str, direction: int, coo, seg_out, seg_in1) -> str:
+def emit_direction(name: str, direction: int, coo, seg_out, seg_in1, gy: bool = False) -> str:
+    """Body of one configuration.  ``gy``: instead of accumulating output rows, contract every tile with the rows of
+    a second channelled operand ``g`` (the output gradient) into the gradient w.r.t. the harmonics,
+    ``gy[b] += coef * sum_w g[m, w] * Z[w]`` (forward tables only)."""
     if direction == 0:
         out_idx, in_idx, blocks, din, dout = coo.M, coo.M1, seg_out, coo.D1, coo.DO
     else:
@@ -64,19 +67,26 @@ def emit_direction(name: str, direction: int, coo, seg_out, seg_in1) -> str:
             run_of_tile[k] = j
     L = []
     a = L.append
-    a(f"struct UV_{name}_d{direction} {{")
+    a(f"struct UV_{name}_{'gy' if gy else 'd' + str(direction)} {{")
     a(f"  static constexpr int DIN = {din}, DOUT = {dout}, D2 = {coo.D2}, P = {coo.P};")
     a("  // xs: this lane's base into the staged input tile (row a of the sample at byte a * CIN * 2);")
-    a("  // load_a(p, frag): fetch the weight fragments of path p; store(row, t0, t1): emit one finished output row.")
-    a("  template <int CIN, class LoadA, class Store>")
-    a("  __device__ __forceinline__ static void run(const unsigned char* xs, LoadA&& load_a, const float (&y)[D2],")
-    a("                                             Store&& store) {")
+    a("  // load_a(p, frag): fetch the weight fragments of path p;")
+    if gy:
+        a("  // load_g(row, t0, t1): this lane's 8 channels of row `row` of g; y receives this lane's partial sums.")
+        a("  template <int CIN, class LoadA, class LoadG>")
+        a("  __device__ __forceinline__ static void run(const unsigned char* xs, LoadA&& load_a, float (&y)[D2],")
+        a("                                             LoadG&& load_g) {")
+    else:
+        a("  // store(row, t0, t1): emit one finished output row.")
+        a("  template <int CIN, class LoadA, class Store>")
+        a("  __device__ __forceinline__ static void run(const unsigned char* xs, LoadA&& load_a, const float (&y)[D2],")
+        a("                                             Store&& store) {")
     a("    constexpr int KS = CIN / 32;")
     a("    bf16x8 w0[2][KS], w1[2][KS], w2[2][KS], b0[KS], b1[KS];")
     a("    floatx4 za0, za1, zb0, zb1;")
     a("    float yy[D2];")
-    a("    for (int j = 0; j < D2; ++j) yy[j] = y[j];")
-    if empty_rows:
+    a("    for (int j = 0; j < D2; ++j) yy[j] = " + ("0.f;" if gy else "y[j];"))
+    if empty_rows and not gy:
         a("    {")
         a("      floatx4 zero = {0};")
         for r in empty_rows:
@@ -107,12 +117,22 @@ def emit_direction(name: str, direction: int, coo, seg_out, seg_in1) -> str:
         # coefficients to tile k, whose chain ran in the previous slot
         if k in first_of_block:
             for r in first_of_block[k]:
-                a(f"    floatx4 o{r}_0 = {{0}}, o{r}_1 = {{0}};")
+                if gy:
+                    a(f"    floatx4 o{r}_0, o{r}_1; load_g({r}, o{r}_0, o{r}_1);")
+                else:
+                    a(f"    floatx4 o{r}_0 = {{0}}, o{r}_1 = {{0}};")
         if k + 1 < len(tiles):
             chain(k + 1)
         if k + 2 < len(tiles):
             load_b(k + 2)
         cur = "za" if k % 2 == 0 else "zb"
+        if gy:
+            for (o, m2, c) in terms:
+                a(f"    yy[{m2}] += {_lit(c)} * dot8(o{o}_0, o{o}_1, {cur}0, {cur}1);")
+            # pin the partial sums (see the accumulators of the forward body)
+            a("    asm volatile(\"\" : " + ", ".join(f'"+v"(yy[{m}])' for m in sorted({m2 for _, m2, _ in terms})) + ");")
+            a("    __builtin_amdgcn_sched_barrier(0);")
+            continue
         # hide the harmonics behind an empty asm per tile: equal (coefficient, harmonic) products recur in many
         # tiles and would otherwise be computed once and kept in registers across the whole body
         a("    " + " ".join(f'asm volatile("" : "+v"(yy[{m}]));' for m in sorted({m2 for _, m2, _ in terms})))
@@ -131,6 +151,8 @@ def emit_direction(name: str, direction: int, coo, seg_out, seg_in1) -> str:
         if k in last_of_block:
             for r in last_of_block[k]:
                 a(f"    store({r}, o{r}_0, o{r}_1);")
+    if gy:
+        a("    for (int j = 0; j < D2; ++j) y[j] = yy[j];")
     a("  }")
     a("};")
     return "\n".join(L)
@@ -147,10 +169,11 @@ def main(out_dir: str = None) -> str:
         chunks.append(f"// {name}: {i1} x {i2} -> {io}")
         for d in (0, 1):
             chunks.append(emit_direction(name, d, coo, seg_out, seg_in1))
+        chunks.append(emit_direction(name, 0, coo, seg_out, seg_in1, gy=True))
         entries.append((name, fingerprint(coo)))
         chunks.append("")
     chunks.append("#define CGTP_FOREACH_UV_CONFIG(X) \\")
-    chunks.append(" \\\n".join(f"  X(UV_{n}_d0, UV_{n}_d1, 0x{fp:016x}ull, \"{n}\")" for n, fp in entries))
+    chunks.append(" \\\n".join(f"  X(UV_{n}_d0, UV_{n}_d1, UV_{n}_gy, 0x{fp:016x}ull, \"{n}\")" for n, fp in entries))
     chunks.append("")
     path = os.path.join(out_dir, "uv_configs.inc")
     text = "\n".join(chunks)

@@ -52,6 +52,13 @@ __device__ __forceinline__ void mfma_chain(const bf16x8 (&a)[2][KS], const bf16x
   }
 }
 
+__device__ __forceinline__ float dot8(const floatx4& g0, const floatx4& g1, const floatx4& z0, const floatx4& z1) {
+  float s = g0[0] * z0[0];
+  s += g0[1] * z0[1]; s += g0[2] * z0[2]; s += g0[3] * z0[3];
+  s += g1[0] * z1[0]; s += g1[1] * z1[1]; s += g1[2] * z1[2]; s += g1[3] * z1[3];
+  return s;
+}
+
 #include "generated/uv_configs.inc"
 
 constexpr int kUvSamples = 16;
@@ -63,19 +70,11 @@ __device__ unsigned long long* g_uv_trace;
 #define UV_MARK(k)
 #endif
 
-template <class CFG, int CIN>
-__global__ void __launch_bounds__(256, 2) uv_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ y,
-                                                    const __bf16* __restrict__ wp, __bf16* __restrict__ out,
-                                                    int64_t n_rows, int cout) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  constexpr int DIN = CFG::DIN, DOUT = CFG::DOUT, D2 = CFG::D2;
-  constexpr int ROW_BYTES = DIN * CIN * 2;      // one sample's input rows
-  constexpr int ROW_PITCH = ROW_BYTES + 16;     // + pad: consecutive samples start 16 B further in the banks
-  const int64_t n0 = (int64_t)blockIdx.x * kUvSamples;
-  UV_MARK(0);
-
-  // stage the 16 samples' rows: 16-byte pieces, coalesced in global memory; every load is issued before the
-  // first LDS write.  Rows past the end of the batch re-read the last row (their results are never stored).
+// Stage the 16 samples' rows of one workgroup: 16-byte pieces, coalesced in global memory; every load is issued
+// before the first LDS write.  Rows past the end of the batch re-read the last row (their results are never stored).
+template <int ROW_BYTES>
+__device__ __forceinline__ void uv_stage(const __bf16* __restrict__ x, int64_t n0, int64_t n_rows, unsigned char* smem) {
+  constexpr int ROW_PITCH = ROW_BYTES + 16;
   constexpr int PIECES = ROW_BYTES / 16, TOTAL = kUvSamples * PIECES, PER_THREAD = (TOTAL + 255) / 256;
   constexpr int UNROLL = PER_THREAD < 16 ? PER_THREAD : 16;
   for (int base = 0; base < TOTAL; base += 256 * UNROLL) {
@@ -92,6 +91,43 @@ __global__ void __launch_bounds__(256, 2) uv_kernel(const __bf16* __restrict__ x
       *reinterpret_cast<f32x4*>(smem + s * ROW_PITCH + c * 16) = v[u];
     }
   }
+}
+
+// Weight fragments of one 32-channel block.  Row r = 4*g + i of channel tile t is output channel blk*32 + 8*g + 4*t
+// + i, so that in the accumulator layout (lane (n, q) holds rows 4*q .. 4*q+3 of column n) a lane ends up with 8
+// consecutive channels of its sample.  The weights arrive packed in fragment order (uv_pack_kernel): per (path,
+// channel block) 2 * KS chunks of 1 KB, chunk t * KS + k holding the 16 bytes of every lane, so that a wavefront's
+// load is one contiguous KB.
+template <int CIN>
+struct UvWeights {
+  const __bf16* base;
+  int64_t path_stride;
+  __device__ __forceinline__ UvWeights(const __bf16* wp, int wblk, int lane, int cout)
+      : base(wp + (int64_t)wblk * (2 * (CIN / 32) * 512) + lane * 8), path_stride((int64_t)cout * CIN) {}
+  __device__ __forceinline__ void operator()(int p, bf16x8 (&frag)[2][CIN / 32]) const {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int k = 0; k < CIN / 32; ++k)
+#ifdef UV_ABL_NOA
+        asm volatile("" : "=v"(frag[t][k]) : "v"(base));
+#else
+        frag[t][k] = *reinterpret_cast<const bf16x8*>(base + p * path_stride + (t * (CIN / 32) + k) * 512);
+#endif
+  }
+};
+
+template <class CFG, int CIN>
+__global__ void __launch_bounds__(256, 2) uv_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ y,
+                                                    const __bf16* __restrict__ wp, __bf16* __restrict__ out,
+                                                    int64_t n_rows, int cout) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  constexpr int DIN = CFG::DIN, DOUT = CFG::DOUT, D2 = CFG::D2;
+  constexpr int ROW_BYTES = DIN * CIN * 2;      // one sample's input rows
+  constexpr int ROW_PITCH = ROW_BYTES + 16;     // + pad: consecutive samples start 16 B further in the banks
+  const int64_t n0 = (int64_t)blockIdx.x * kUvSamples;
+  UV_MARK(0);
+  uv_stage<ROW_BYTES>(x, n0, n_rows, smem);
   UV_MARK(1);
   __syncthreads();
   UV_MARK(2);
@@ -107,29 +143,9 @@ __global__ void __launch_bounds__(256, 2) uv_kernel(const __bf16* __restrict__ x
   // one 32-channel block per wavefront, blockIdx.y tiles wider outputs
   const int wblk = blockIdx.y * (blockDim.x / kWave) + wave;
   if (wblk * 32 >= cout) return;
-  // Row r = 4*g + i of channel tile t is output channel wblk*32 + 8*g + 4*t + i, so that in the accumulator layout
-  // (lane (n, q) holds rows 4*q .. 4*q+3 of column n) a lane ends up with 8 consecutive channels of its sample.
-  // The weights arrive packed in fragment order (uv_pack_kernel): per (path, channel block) 2 * KS chunks of 1 KB,
-  // chunk t * KS + k holding the 16 bytes of every lane, so that a wavefront's load is one contiguous KB.
-  const __bf16* wfrag = wp + (int64_t)wblk * (2 * (CIN / 32) * 512) + lane * 8;
-  const int64_t path_stride = (int64_t)cout * CIN;
   __bf16* orow = out + (n0 + n) * DOUT * cout + wblk * 32 + 8 * q;
   CFG::template run<CIN>(
-      xs,
-      [&](int p, bf16x8(&frag)[2][CIN / 32]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int k = 0; k < CIN / 32; ++k)
-#ifdef UV_ABL_NOA
-            asm volatile("" : "=v"(frag[t][k]) : "v"(wfrag));
-#elif defined(UV_ABL_A0)
-            frag[t][k] = *reinterpret_cast<const volatile bf16x8*>(wfrag + (p & 1) * path_stride + (t * (CIN / 32) + k) * 512);
-#else
-            frag[t][k] = *reinterpret_cast<const bf16x8*>(wfrag + p * path_stride + (t * (CIN / 32) + k) * 512);
-#endif
-      },
-      yv,
+      xs, UvWeights<CIN>(wp, wblk, lane, cout), yv,
       [&](int row, const floatx4& o0, const floatx4& o1) __attribute__((always_inline)) {
         if (valid) {
           bf16x8 v;
@@ -145,6 +161,59 @@ __global__ void __launch_bounds__(256, 2) uv_kernel(const __bf16* __restrict__ x
         if (row == 8) UV_MARK(5);
       });
   UV_MARK(6);
+}
+
+// Gradient w.r.t. the harmonics: gy[n, b] = sum_t coef_t * sum_w g[n, m_t, w] * Z[p_t, a_t][w, n] with the same
+// tiles Z as the forward.  Every lane sums over its 8 channels, the four lanes of a sample and the four wavefronts
+// (channel blocks) are then added through LDS in a fixed order.  cout <= 128: one workgroup sees all channels.
+template <class CFG, int CIN>
+__global__ void __launch_bounds__(256, 2) uv_gy_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ g,
+                                                       const __bf16* __restrict__ wp, __bf16* __restrict__ gy,
+                                                       int64_t n_rows, int cout) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  constexpr int DIN = CFG::DIN, DOUT = CFG::DOUT, D2 = CFG::D2;
+  constexpr int ROW_BYTES = DIN * CIN * 2, ROW_PITCH = ROW_BYTES + 16;
+  const int64_t n0 = (int64_t)blockIdx.x * kUvSamples;
+  uv_stage<ROW_BYTES>(x, n0, n_rows, smem);
+  __syncthreads();
+
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int n = lane & 15, q = lane >> 4;
+  const unsigned char* xs = smem + n * ROW_PITCH + q * 16;
+  const int n_blk = cout / 32;
+  float part[D2];
+#pragma unroll
+  for (int j = 0; j < D2; ++j) part[j] = 0.f;
+  if (wave < n_blk) {
+    const __bf16* grow = g + min(n0 + n, n_rows - 1) * DOUT * cout + wave * 32 + 8 * q;
+    CFG::template run<CIN>(
+        xs, UvWeights<CIN>(wp, wave, lane, cout), part,
+        [&](int row, floatx4& g0, floatx4& g1) __attribute__((always_inline)) {
+          const bf16x8 v = *reinterpret_cast<const bf16x8*>(grow + row * cout);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            g0[i] = (float)v[i];
+            g1[i] = (float)v[4 + i];
+          }
+        });
+#pragma unroll
+    for (int j = 0; j < D2; ++j) {
+      part[j] += __shfl_xor(part[j], 16, kWave);
+      part[j] += __shfl_xor(part[j], 32, kWave);
+    }
+  }
+  __syncthreads();  // every wavefront is done with the staged rows; reuse the front of LDS for the partial sums
+  float* red = reinterpret_cast<float*>(smem);
+  if (wave < n_blk && q == 0) {
+#pragma unroll
+    for (int j = 0; j < D2; ++j) red[(wave * kUvSamples + n) * D2 + j] = part[j];
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < kUvSamples * D2; i += blockDim.x) {
+    float s = 0.f;
+    for (int w = 0; w < n_blk; ++w) s += red[w * kUvSamples * D2 + i];
+    if (n0 + i / D2 < n_rows) gy[n0 * D2 + i] = (__bf16)s;
+  }
 }
 
 // packed[p][blk][t][k][lane = 16*q + r][e] = Wt[p][blk*32 + 8*(r/4) + 4*t + r%4][k*32 + 8*q + e], where
@@ -175,10 +244,10 @@ struct UvEntry {
   uint64_t fingerprint;
   const char* name;
   int din[2], dout[2], d2, p;
-  UvFn fn[2][3];  // [direction][C_in = 32, 64, 128]
+  UvFn fn[3][3];  // [direction 0, direction 1, grad y][C_in = 32, 64, 128]
 };
 
-template <class D0, class D1>
+template <class D0, class D1, class GY>
 static UvEntry make_uv_entry(uint64_t fp, const char* name) {
   UvEntry e;
   e.fingerprint = fp; e.name = name;
@@ -186,11 +255,12 @@ static UvEntry make_uv_entry(uint64_t fp, const char* name) {
   e.d2 = D0::D2; e.p = D0::P;
   e.fn[0][0] = uv_kernel<D0, 32>; e.fn[0][1] = uv_kernel<D0, 64>; e.fn[0][2] = uv_kernel<D0, 128>;
   e.fn[1][0] = uv_kernel<D1, 32>; e.fn[1][1] = uv_kernel<D1, 64>; e.fn[1][2] = uv_kernel<D1, 128>;
+  e.fn[2][0] = uv_gy_kernel<GY, 32>; e.fn[2][1] = uv_gy_kernel<GY, 64>; e.fn[2][2] = uv_gy_kernel<GY, 128>;
   return e;
 }
 
 static const UvEntry* uv_entries(int* count) {
-#define CGTP_X(D0, D1, FP, NAME) make_uv_entry<D0, D1>(FP, NAME),
+#define CGTP_X(D0, D1, GY, FP, NAME) make_uv_entry<D0, D1, GY>(FP, NAME),
   static const UvEntry table[] = {CGTP_FOREACH_UV_CONFIG(CGTP_X)};
 #undef CGTP_X
   *count = (int)(sizeof(table) / sizeof(table[0]));
@@ -273,6 +343,25 @@ int cgtp_uv_apply(int cfg, int direction, const void* x, const void* y, const vo
   hipLaunchKernelGGL(fn, dim3((unsigned)((n_rows + kUvSamples - 1) / kUvSamples), (unsigned)((cout + 127) / 128)),
                      dim3(256), (size_t)lds,
                      (hipStream_t)stream, (const __bf16*)x, (const __bf16*)y, (const __bf16*)wp, (__bf16*)out, n_rows,
+                     (int)cout);
+  return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
+}
+
+int cgtp_uv_grad_y(int cfg, const void* x, const void* g, const void* wp, void* gy, int64_t n_rows, int32_t cin,
+                   int32_t cout, int32_t dtype, void* stream) {
+  int ci = 0;
+  int64_t lds = 0;
+  const int st = uv_check(cfg, 0, x, g, wp, gy, n_rows, cin, cout, dtype, &ci, &lds);
+  if (st != CGTP_OK) return st;
+  if (cout > 128) return CGTP_ERR_SHAPE;
+  if (reinterpret_cast<uintptr_t>(g) & 15u) return CGTP_ERR_ALIGN;
+  if (n_rows == 0) return CGTP_OK;
+  int n = 0;
+  UvFn fn = uv_entries(&n)[cfg].fn[2][ci];
+  if (hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return CGTP_ERR_LDS;
+  hipLaunchKernelGGL(fn, dim3((unsigned)((n_rows + kUvSamples - 1) / kUvSamples)), dim3(256), (size_t)lds,
+                     (hipStream_t)stream, (const __bf16*)x, (const __bf16*)g, (const __bf16*)wp, (__bf16*)gy, n_rows,
                      (int)cout);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }

@@ -57,6 +57,16 @@ def _apply(cfg: int, direction: int, x: Tensor, y: Tensor, wp: Tensor, d_out: in
     return out
 
 
+def _grad_y(cfg: int, x: Tensor, g: Tensor, wp: Tensor, d2: int) -> Tensor:
+    """Gradient w.r.t. the harmonics; ``wp`` = ``pack_weights(0, W)``."""
+    n, _, cin = x.shape
+    cout = g.shape[-1]
+    gy = torch.empty((n, d2), dtype=x.dtype, device=x.device)
+    _lib.check(_lib.lib.cgtp_uv_grad_y(cfg, x.data_ptr(), g.data_ptr(), wp.data_ptr(), gy.data_ptr(), n, cin, cout,
+                                       _lib.BF16, _lib.stream_ptr(x.device)), "cgtp_uv_grad_y")
+    return gy
+
+
 class _UvMfma(Function):
     """u1v with a shared weight on the matrix cores.  Forward and the gradient w.r.t. input1 run the MFMA kernel;
     the gradients w.r.t. the harmonics and the weight go through the general contraction kernel."""
@@ -82,7 +92,10 @@ class _UvMfma(Function):
                 else:
                     gx = _apply(ctx.cfg, 1, g.contiguous(), y, pack_weights(1, w), ctx.d1)
             if need[1]:
-                gy = tri(spec.grad_spec(1), ("u", "w", "uw"), "", x, g, w)
+                if torch.is_grad_enabled() or g.shape[-1] > 128:
+                    gy = tri(spec.grad_spec(1), ("u", "w", "uw"), "", x, g, w)
+                else:
+                    gy = _grad_y(ctx.cfg, x, g.contiguous(), pack_weights(0, w), y.shape[-1])
             if need[2]:
                 gw = tri(spec.grad_spec(2), ("u", "", "w"), "uw", x, y, g, out_shared=True)
         return gx, gy, gw, None, None

@@ -217,6 +217,13 @@ int cgtp_uv_validate(int cfg, int direction, const void* x, const void* y, const
                      int64_t n_rows, int32_t cin, int32_t cout, int32_t dtype);
 int cgtp_uv_apply(int cfg, int direction, const void* x, const void* y, const void* wp, void* out, int64_t n_rows,
                   int32_t cin, int32_t cout, int32_t dtype, void* stream);
+/* Gradient w.r.t. the harmonics of direction 0 (the uu1/vu1 product of the reference's backward,
+ * equitorch/nn/functional/linears.py:294-300, without its (N, segments, C) intermediates):
+ *   gy[n, b] = sum_t [b_t = b] coef_t * sum_w g[n, m_t, w] * sum_u x[n, a_t, u] * W[p_t, u, w]
+ * x (n_rows, D1, cin), g = grad_out (n_rows, DO, cout), wp = direction-0 packed weights, gy (n_rows, D2);
+ * cout <= 128.  Sums run in a fixed order (no atomics). */
+int cgtp_uv_grad_y(int cfg, const void* x, const void* g, const void* wp, void* gy, int64_t n_rows, int32_t cin,
+                   int32_t cout, int32_t dtype, void* stream);
 
 /* ---- streaming kernels of known traffic (counter calibration, achievable-bandwidth reference) ------------
  * No counterpart in the reference.  copy: reads n_bytes and writes n_bytes; read: reads n_bytes.
