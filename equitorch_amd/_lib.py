@@ -92,6 +92,10 @@ def _load():
                                          C.c_void_p]
     lib.cgtp_uv_grad_y.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32,
                                    C.c_int32, C.c_int32, C.c_void_p]
+    lib.cgtp_uv_grad_w_workspace_bytes.restype = C.c_int64
+    lib.cgtp_uv_grad_w_workspace_bytes.argtypes = [C.c_int, C.c_int64, C.c_int32, C.c_int32]
+    lib.cgtp_uv_grad_w.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
+                                   C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
     lib.cgtp_uv_validate.argtypes = _uv
     lib.cgtp_uv_apply.argtypes = _uv + [C.c_void_p]
     lib.cgtp_membench_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]

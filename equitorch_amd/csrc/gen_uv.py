@@ -158,6 +158,55 @@ def emit_direction(name: str, direction: int, coo, seg_out, seg_in1, gy: bool = 
     return "\n".join(L)
 
 
+def emit_gw(name: str, coo, seg_out, seg_in1) -> str:
+    """Per-path Clebsch-Gordan mixing for the weight gradient: ``G[a] = sum_(m,b) coef * y[b] * g[m]`` for every
+    input row ``a`` the path reads, on 8-channel fp32 vectors (the matrix cores then contract ``x[a]`` with ``G[a]``
+    over the samples)."""
+    T = coo.coef.shape[0]
+    L = []
+    w = L.append
+    a0, na = [], []
+    for p in range(coo.P):
+        rows = sorted({int(coo.M1[t]) for t in range(T) if coo.p[t] == p})
+        assert rows == list(range(rows[0], rows[0] + len(rows)))
+        a0.append(rows[0])
+        na.append(len(rows))
+    w(f"struct UV_{name}_gw {{")
+    w(f"  static constexpr int D1 = {coo.D1}, DO = {coo.DO}, D2 = {coo.D2}, P = {coo.P}, MAX_ROWS = {max(na)};")
+    w("  // rows of the channelled input read by every path: first row and count")
+    w(f"  static constexpr unsigned char A0[P] = {{{', '.join(map(str, a0))}}};")
+    w(f"  static constexpr unsigned char NA[P] = {{{', '.join(map(str, na))}}};")
+    w("  // src(h, m): 8 channels (pass h of 2) of row m of g as floats; dst(h, r, v): the mixed row for input row")
+    w("  // A0[p] + r.  Both passes of a path sit in one case so that the coef * y products are formed once per path")
+    w("  // and only for the path at hand.")
+    w("  template <class Src, class Dst>")
+    w("  __device__ __forceinline__ static void mix(int p, const float (&y)[D2], Src&& src, Dst&& dst) {")
+    w("    switch (p) {")
+    for p in range(coo.P):
+        nnz = [t for t in range(T) if coo.p[t] == p]
+        w(f"      case {p}: {{")
+        prods = OrderedDict()
+        for t in nnz:
+            prods.setdefault((int(coo.M2[t]), _lit(coo.coef[t])), len(prods))
+        for (b, c), i in prods.items():
+            w(f"        const float s{i} = {c} * y[{b}];")
+        for h in (0, 1):
+            w("        {")
+            for m in sorted({int(coo.M[t]) for t in nnz}):
+                w(f"          const floatx8 g{m} = src({h}, {m});")
+            for r in range(na[p]):
+                terms = sorted((int(coo.M[t]), int(coo.M2[t]), _lit(coo.coef[t])) for t in nnz if coo.M1[t] == a0[p] + r)
+                expr = " + ".join(f"s{prods[(b, c)]} * g{m}" for m, b, c in terms)
+                w(f"          dst({h}, {r}, {expr});")
+            w("        }")
+        w("      } break;")
+    w("      default: break;")
+    w("    }")
+    w("  }")
+    w("};")
+    return "\n".join(L)
+
+
 def main(out_dir: str = None) -> str:
     out_dir = out_dir or os.path.join(HERE, "generated")
     os.makedirs(out_dir, exist_ok=True)
@@ -170,10 +219,11 @@ def main(out_dir: str = None) -> str:
         for d in (0, 1):
             chunks.append(emit_direction(name, d, coo, seg_out, seg_in1))
         chunks.append(emit_direction(name, 0, coo, seg_out, seg_in1, gy=True))
+        chunks.append(emit_gw(name, coo, seg_out, seg_in1))
         entries.append((name, fingerprint(coo)))
         chunks.append("")
     chunks.append("#define CGTP_FOREACH_UV_CONFIG(X) \\")
-    chunks.append(" \\\n".join(f"  X(UV_{n}_d0, UV_{n}_d1, UV_{n}_gy, 0x{fp:016x}ull, \"{n}\")" for n, fp in entries))
+    chunks.append(" \\\n".join(f"  X(UV_{n}_d0, UV_{n}_d1, UV_{n}_gy, UV_{n}_gw, 0x{fp:016x}ull, \"{n}\")" for n, fp in entries))
     chunks.append("")
     path = os.path.join(out_dir, "uv_configs.inc")
     text = "\n".join(chunks)

@@ -22,6 +22,8 @@ namespace cgtp {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
 
 // this lane's 8 consecutive k of every K step of one staged input row
 template <int KS>
@@ -216,6 +218,140 @@ __global__ void __launch_bounds__(256, 2) uv_gy_kernel(const __bf16* __restrict_
   }
 }
 
+// ---- weight gradient ---------------------------------------------------------------------------------------
+//   gW[p, u, w] = sum_n sum_a x[n, a, u] * G[n, p, a, w],   G[n, p, a, w] = sum_(m, b) coef * y[n, b] * g[n, m, w]
+// A workgroup owns one path and one chunk of samples and keeps the whole (C_in x C_out) fp32 accumulator in
+// registers (four wavefronts, 64 x 64 each).  Per step of 32 samples it stages the path's rows of x in LDS as they
+// lie in memory ([sample][channel]), forms the mixed rows G on the vector ALUs into LDS in the same layout, and then
+// contracts over the samples on the matrix cores: both MFMA operands need 8 consecutive samples of one channel per
+// lane, which ds_read_b64_tr_b16 delivers from the [sample][channel] tiles (within 16 lanes, lane L receives the
+// four 16-bit elements that lanes L/4, L/4 + 4, L/4 + 8, L/4 + 12 addressed at position L % 4).  Chunk partials go
+// to a workspace and are summed in a fixed order by uv_gw_reduce_kernel.
+constexpr int kGwStep = 32;    // samples per MFMA step (K of v_mfma_f32_16x16x32_bf16)
+constexpr int kGwChunk = 512;  // samples per workgroup
+constexpr int kGwPad = 32;     // bytes added to a tile row: the four rows a 16-lane transpose read touches land in
+                               // distinct banks
+
+struct UvGwMeta {              // per configuration, passed by value: workgroup -> path, and the x rows of a path
+  unsigned char order[64], a0[64], na[64];
+};
+
+__device__ __forceinline__ bf16x8 lds_read_tr(const unsigned char* p0, const unsigned char* p1) {
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p1));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+template <class CFG>
+__global__ void __launch_bounds__(256, 1) uv_gw_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ y,
+                                                       const __bf16* __restrict__ g, float* __restrict__ part,
+                                                       int64_t n_rows, int cin, int cout, UvGwMeta meta) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  constexpr int D1 = CFG::D1, DO = CFG::DO, D2 = CFG::D2, P = CFG::P;
+  // the same for every lane: keep them in scalar registers so that the switch over paths is a scalar branch
+  const int p = __builtin_amdgcn_readfirstlane(meta.order[blockIdx.x % P]);
+  const int64_t c = blockIdx.x / P;
+  const int a0 = __builtin_amdgcn_readfirstlane(meta.a0[p]), na = __builtin_amdgcn_readfirstlane(meta.na[p]);
+  const int pu = cin * 2 + kGwPad, pw = cout * 2 + kGwPad;   // tile row pitches
+  unsigned char* xt = smem;                           // [na][32][pu]  rows of x
+  unsigned char* gt = smem + CFG::MAX_ROWS * kGwStep * pu;  // [na][32][pw]  mixed rows
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int vu = wave >> 1, vw = wave & 1;            // this wavefront's 64 x 64 block of the accumulator
+  floatx4 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int64_t n_begin = c * kGwChunk, n_end = min(n_begin + (int64_t)kGwChunk, n_rows);
+  const int sn = tid >> 3, cg = tid & 7;              // mixing: sample of the step and 8-channel group (two passes)
+  const int ls = lane & 15, lq = lane >> 4;           // fragment reads
+  for (int64_t nb = n_begin; nb < n_end; nb += kGwStep) {
+    __syncthreads();  // the previous step's fragment reads are done
+    // rows of x: per sample one contiguous run of na * cin elements
+    {
+      const int pieces = na * cin / 8;                // 16-byte pieces per sample
+      for (int i = tid; i < kGwStep * pieces; i += 256) {
+        const int s_ = i / pieces, k = i % pieces;
+        const int64_t row = min(nb + s_, n_rows - 1);
+        const f32x4 v = *reinterpret_cast<const f32x4*>(x + (row * D1 + a0) * cin + k * 8);
+        const int r = (k * 8) / cin, ch = (k * 8) % cin;
+        *reinterpret_cast<f32x4*>(xt + (r * kGwStep + s_) * pu + ch * 2) = v;
+      }
+    }
+    // mixed rows; samples past the end get y = 0 and so contribute nothing
+    {
+      const int64_t n = nb + sn;
+      const int64_t row = min(n, n_rows - 1);
+      float yv[D2];
+#pragma unroll
+      for (int j = 0; j < D2; ++j) yv[j] = n < n_end ? (float)y[row * D2 + j] : 0.f;
+      // two passes of 8 channels per thread; a pass beyond cout re-reads the last group and stores nothing
+      const __bf16* grow = g + row * DO * cout;
+      unsigned char* drow = gt + sn * pw;
+      CFG::mix(
+          p, yv,
+          [&](int h, int m) __attribute__((always_inline)) {
+            const int ch = min((cg + 8 * h) * 8, cout - 8);
+            const bf16x8 v = *reinterpret_cast<const bf16x8*>(grow + m * cout + ch);
+            floatx8 f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[e] = (float)v[e];
+            return f;
+          },
+          [&](int h, int r, const floatx8& v) __attribute__((always_inline)) {
+            const int ch = (cg + 8 * h) * 8;
+            bf16x8 o;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (__bf16)v[e];
+            if (ch < cout) *reinterpret_cast<bf16x8*>(drow + r * kGwStep * pw + ch * 2) = o;
+          });
+    }
+    __syncthreads();
+    // contract over the 32 samples of the step, row by row
+    for (int r = 0; r < na; ++r) {
+      const unsigned char* xa = xt + (r * kGwStep + 8 * lq + (ls >> 2)) * pu + (ls & 3) * 8;
+      const unsigned char* gb = gt + (r * kGwStep + 8 * lq + (ls >> 2)) * pw + (ls & 3) * 8;
+      bf16x8 fa[4], fb[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int ut = vu * 4 + i, wt = vw * 4 + i;
+        if (ut * 16 < cin) fa[i] = lds_read_tr(xa + ut * 32, xa + ut * 32 + 4 * pu);
+        if (wt * 16 < cout) fb[i] = lds_read_tr(gb + wt * 32, gb + wt * 32 + 4 * pw);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if ((vu * 4 + i) * 16 < cin && (vw * 4 + j) * 16 < cout)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+  }
+  // accumulator element e of lane (col = lane & 15, q) is row 4*q + e of the tile
+  float* out = part + (c * P + p) * (int64_t)cin * cout;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int u0 = (vu * 4 + i) * 16 + 4 * lq, w_ = (vw * 4 + j) * 16 + ls;
+      if (u0 < cin && w_ < cout) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[(int64_t)(u0 + e) * cout + w_] = acc[i][j][e];
+      }
+    }
+}
+
+__global__ void uv_gw_reduce_kernel(const float* __restrict__ part, __bf16* __restrict__ gw, int64_t n_chunks, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float s = 0.f;
+  for (int64_t k = 0; k < n_chunks; ++k) s += part[k * n + i];
+  gw[i] = (__bf16)s;
+}
+
 // packed[p][blk][t][k][lane = 16*q + r][e] = Wt[p][blk*32 + 8*(r/4) + 4*t + r%4][k*32 + 8*q + e], where
 // Wt[p][row][col] = w[p * rows * cols + row * row_stride + col * col_stride]; one thread per 16-byte piece.
 __global__ void uv_pack_kernel(const __bf16* __restrict__ w, __bf16* __restrict__ packed, int64_t n_pieces, int rows,
@@ -239,15 +375,19 @@ __global__ void uv_pack_kernel(const __bf16* __restrict__ w, __bf16* __restrict_
 }
 
 using UvFn = void (*)(const __bf16*, const __bf16*, const __bf16*, __bf16*, int64_t, int);
+using UvGwFn = void (*)(const __bf16*, const __bf16*, const __bf16*, float*, int64_t, int, int, UvGwMeta);
 
 struct UvEntry {
   uint64_t fingerprint;
   const char* name;
   int din[2], dout[2], d2, p;
   UvFn fn[3][3];  // [direction 0, direction 1, grad y][C_in = 32, 64, 128]
+  UvGwFn gw_fn;
+  int gw_max_rows;
+  UvGwMeta gw_meta;  // order: paths with the most rows first, so that long workgroups start first
 };
 
-template <class D0, class D1, class GY>
+template <class D0, class D1, class GY, class GW>
 static UvEntry make_uv_entry(uint64_t fp, const char* name) {
   UvEntry e;
   e.fingerprint = fp; e.name = name;
@@ -256,11 +396,22 @@ static UvEntry make_uv_entry(uint64_t fp, const char* name) {
   e.fn[0][0] = uv_kernel<D0, 32>; e.fn[0][1] = uv_kernel<D0, 64>; e.fn[0][2] = uv_kernel<D0, 128>;
   e.fn[1][0] = uv_kernel<D1, 32>; e.fn[1][1] = uv_kernel<D1, 64>; e.fn[1][2] = uv_kernel<D1, 128>;
   e.fn[2][0] = uv_gy_kernel<GY, 32>; e.fn[2][1] = uv_gy_kernel<GY, 64>; e.fn[2][2] = uv_gy_kernel<GY, 128>;
+  static_assert(GW::P <= 64, "path order table too small");
+  e.gw_fn = uv_gw_kernel<GW>;
+  e.gw_max_rows = GW::MAX_ROWS;
+  int k = 0;
+  for (int rows = GW::MAX_ROWS; rows >= 1; --rows)
+    for (int p = 0; p < GW::P; ++p)
+      if (GW::NA[p] == rows) e.gw_meta.order[k++] = (unsigned char)p;
+  for (int p = 0; p < GW::P; ++p) {
+    e.gw_meta.a0[p] = GW::A0[p];
+    e.gw_meta.na[p] = GW::NA[p];
+  }
   return e;
 }
 
 static const UvEntry* uv_entries(int* count) {
-#define CGTP_X(D0, D1, GY, FP, NAME) make_uv_entry<D0, D1, GY>(FP, NAME),
+#define CGTP_X(D0, D1, GY, GW, FP, NAME) make_uv_entry<D0, D1, GY, GW>(FP, NAME),
   static const UvEntry table[] = {CGTP_FOREACH_UV_CONFIG(CGTP_X)};
 #undef CGTP_X
   *count = (int)(sizeof(table) / sizeof(table[0]));
@@ -363,6 +514,44 @@ int cgtp_uv_grad_y(int cfg, const void* x, const void* g, const void* wp, void* 
   hipLaunchKernelGGL(fn, dim3((unsigned)((n_rows + kUvSamples - 1) / kUvSamples)), dim3(256), (size_t)lds,
                      (hipStream_t)stream, (const __bf16*)x, (const __bf16*)g, (const __bf16*)wp, (__bf16*)gy, n_rows,
                      (int)cout);
+  return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
+}
+
+int64_t cgtp_uv_grad_w_workspace_bytes(int cfg, int64_t n_rows, int32_t cin, int32_t cout) {
+  int n = 0;
+  const UvEntry* t = uv_entries(&n);
+  if (cfg < 0 || cfg >= n || n_rows <= 0 || cin <= 0 || cout <= 0) return 0;
+  const int64_t n_chunks = (n_rows + kGwChunk - 1) / kGwChunk;
+  return n_chunks * t[cfg].p * (int64_t)cin * cout * (int64_t)sizeof(float);
+}
+
+int cgtp_uv_grad_w(int cfg, const void* x, const void* y, const void* g, void* gw, void* workspace, int64_t n_rows,
+                   int32_t cin, int32_t cout, int32_t dtype, void* stream) {
+  int n = 0;
+  const UvEntry* t = uv_entries(&n);
+  if (cfg < 0 || cfg >= n) return CGTP_ERR_CONFIG;
+  if (dtype != CGTP_BF16) return CGTP_ERR_DTYPE;
+  if (!x || !y || !g || !gw) return CGTP_ERR_NULL;
+  if (n_rows < 0 || cin <= 0 || cout <= 0 || cin % 32 != 0 || cout % 32 != 0 || cin > 128 || cout > 128)
+    return CGTP_ERR_SHAPE;
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(workspace)) & 15u)
+    return CGTP_ERR_ALIGN;
+  const UvEntry& e = t[cfg];
+  const int64_t n_out = (int64_t)e.p * cin * cout;
+  hipStream_t st = (hipStream_t)stream;
+  if (n_rows == 0) {
+    return hipMemsetAsync(gw, 0, n_out * 2, st) == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
+  }
+  if (!workspace) return CGTP_ERR_WORKSPACE;
+  const int64_t lds = (int64_t)e.gw_max_rows * kGwStep * ((int64_t)cin * 2 + cout * 2 + 2 * kGwPad);
+  if (lds > kLdsBytes) return CGTP_ERR_LDS;
+  if (hipFuncSetAttribute((const void*)e.gw_fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return CGTP_ERR_LDS;
+  const int64_t n_chunks = (n_rows + kGwChunk - 1) / kGwChunk;
+  hipLaunchKernelGGL(e.gw_fn, dim3((unsigned)(n_chunks * e.p)), dim3(256), (size_t)lds, st, (const __bf16*)x,
+                     (const __bf16*)y, (const __bf16*)g, (float*)workspace, n_rows, (int)cin, (int)cout, e.gw_meta);
+  hipLaunchKernelGGL(uv_gw_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, st,
+                     (const float*)workspace, (__bf16*)gw, n_chunks, n_out);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 

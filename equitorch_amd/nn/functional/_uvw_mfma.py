@@ -67,9 +67,21 @@ def _grad_y(cfg: int, x: Tensor, g: Tensor, wp: Tensor, d2: int) -> Tensor:
     return gy
 
 
+def _grad_w(cfg: int, x: Tensor, y: Tensor, g: Tensor, n_paths: int) -> Tensor:
+    """Gradient w.r.t. the shared weight, (P, C_in, C_out)."""
+    n, _, cin = x.shape
+    cout = g.shape[-1]
+    gw = torch.empty((n_paths, cin, cout), dtype=x.dtype, device=x.device)
+    ws_bytes = int(_lib.lib.cgtp_uv_grad_w_workspace_bytes(cfg, n, cin, cout))
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=x.device)
+    _lib.check(_lib.lib.cgtp_uv_grad_w(cfg, x.data_ptr(), y.data_ptr(), g.data_ptr(), gw.data_ptr(), ws.data_ptr(), n,
+                                       cin, cout, _lib.BF16, _lib.stream_ptr(x.device)), "cgtp_uv_grad_w")
+    return gw
+
+
 class _UvMfma(Function):
-    """u1v with a shared weight on the matrix cores.  Forward and the gradient w.r.t. input1 run the MFMA kernel;
-    the gradients w.r.t. the harmonics and the weight go through the general contraction kernel."""
+    """u1v with a shared weight on the matrix cores: forward and the three first-order gradients.  Under
+    ``create_graph`` the gradients are formed by the general contraction kernel, which is differentiable again."""
 
     @staticmethod
     def forward(ctx, x: Tensor, y: Tensor, w: Tensor, tp_info, cfg: int):
@@ -97,7 +109,10 @@ class _UvMfma(Function):
                 else:
                     gy = _grad_y(ctx.cfg, x, g.contiguous(), pack_weights(0, w), y.shape[-1])
             if need[2]:
-                gw = tri(spec.grad_spec(2), ("u", "", "w"), "uw", x, y, g, out_shared=True)
+                if torch.is_grad_enabled():
+                    gw = tri(spec.grad_spec(2), ("u", "", "w"), "uw", x, y, g, out_shared=True)
+                else:
+                    gw = _grad_w(ctx.cfg, x, y, g.contiguous(), w.shape[0])
         return gx, gy, gw, None, None
 
 

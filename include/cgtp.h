@@ -224,6 +224,15 @@ int cgtp_uv_apply(int cfg, int direction, const void* x, const void* y, const vo
  * cout <= 128.  Sums run in a fixed order (no atomics). */
 int cgtp_uv_grad_y(int cfg, const void* x, const void* g, const void* wp, void* gy, int64_t n_rows, int32_t cin,
                    int32_t cout, int32_t dtype, void* stream);
+/* Gradient w.r.t. the shared weight (the reference accumulates batch outer products with atomics,
+ * indexed_outer_scale_gather with out_accumulated, equitorch/nn/functional/linears.py:301-307):
+ *   gw[p, u, w] = sum_n sum_t [p_t = p] coef_t * y[n, b_t] * x[n, a_t, u] * g[n, m_t, w]
+ * x (n_rows, D1, cin), y (n_rows, D2), g = grad_out (n_rows, DO, cout), gw (P, cin, cout) as the module stores W;
+ * cin, cout multiples of 32 up to 128.  The samples are contracted on the matrix cores in chunks; the fp32 chunk
+ * partials live in `workspace` (cgtp_uv_grad_w_workspace_bytes bytes) and are added in a fixed order. */
+int64_t cgtp_uv_grad_w_workspace_bytes(int cfg, int64_t n_rows, int32_t cin, int32_t cout);
+int cgtp_uv_grad_w(int cfg, const void* x, const void* y, const void* g, void* gw, void* workspace, int64_t n_rows,
+                   int32_t cin, int32_t cout, int32_t dtype, void* stream);
 
 /* ---- streaming kernels of known traffic (counter calibration, achievable-bandwidth reference) ------------
  * No counterpart in the reference.  copy: reads n_bytes and writes n_bytes; read: reads n_bytes.
