@@ -39,6 +39,7 @@ WORKLOADS = {
     "edge_fwd": (2, 64, 4096, 65536),
     # fully connected product on the matrix cores (BASELINE configs[3]): (lmax, C_in = C_out, batch)
     "uvw_fwd": (3, 128, 32768),
+    "uvw_fwd_bwd": (3, 128, 32768),
     # streaming kernels of known traffic (1 GiB): counter calibration and achievable-bandwidth reference
     "copy": None,
     "read": None,
@@ -84,7 +85,8 @@ def uvw_bench(args):
     from equitorch_amd.nn import SO3Linear
     from equitorch_amd.nn.functional import _uvw_mfma
     from equitorch_amd.utils._sh import spherical_harmonics
-    lmax, ch, n = WORKLOADS["uvw_fwd"]
+    lmax, ch, n = WORKLOADS[args.workload]
+    backward = args.workload == "uvw_fwd_bwd"
     dev = torch.device("cuda:0")
     irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
     mod = SO3Linear(irreps, irreps, irreps, ch, ch, internal_weights=False, feature_mode="uv").to(dev)
@@ -98,6 +100,8 @@ def uvw_bench(args):
     wt = _uvw_mfma.pack_weights(0, w)
     s1 = int(mod.tp_info_forward.info_Mij_fwd.out_size)
     flops = 2.0 * n * s1 * ch * ch
+    if backward:
+        return uvw_fwd_bwd_bench(args, mod, x, sh, w, cfg, flops, irreps, gen)
 
     def step():
         return mod(x, sh, w)
@@ -126,6 +130,57 @@ def uvw_bench(args):
         "roofline": {"bound": "mfma", "kernel": "cgtp::uv_kernel<UV_sh3_d0,128>", "achieved": round(tf, 2),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
                      "traffic": None, "algorithmic_flops": flops, "avg_ms": round(k_ms, 5)}}))
+
+
+def uvw_fwd_bwd_bench(args, mod, x, sh, w, cfg, flops, irreps, gen):
+    """BASELINE configs[3], forward and backward (gx, gsh, gW).  Each of the four products contracts the 99
+    (path, row) tiles with a 128 x 128 weight once, so the step is priced at 4 x the forward's flops."""
+    from equitorch_amd.nn.functional import _uvw_mfma
+    n, d, ch = x.shape
+    ct = torch.randn(n, d, ch, generator=gen).bfloat16().to(x.device)
+    xg, shg, wg = (t.clone().requires_grad_(True) for t in (x, sh, w))
+
+    def step():
+        out = mod(xg, shg, wg)
+        return torch.autograd.grad(out, (xg, shg, wg), ct)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) / args.steps * 1e3
+
+    def timed(fn):
+        evs = []
+        for _ in range(args.kernel_reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(); fn(); b.record()
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        return sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    w0, w1 = _uvw_mfma.pack_weights(0, w), _uvw_mfma.pack_weights(1, w)
+    kern = {
+        "fwd_ms": timed(lambda: _uvw_mfma._apply(cfg, 0, x, sh, w0, d)),
+        "grad_x_ms": timed(lambda: _uvw_mfma._apply(cfg, 1, ct, sh, w1, d)),
+        "grad_sh_ms": timed(lambda: _uvw_mfma._grad_y(cfg, x, ct, w0, sh.shape[-1])),
+        "grad_w_ms": timed(lambda: _uvw_mfma._grad_w(cfg, x, sh, ct, w.shape[0])),
+    }
+    dom = max(kern, key=kern.get)
+    tf = flops / (kern[dom] * 1e-3) / 1e12
+    names = {"fwd_ms": "cgtp::uv_kernel<UV_sh3_d0,128>", "grad_x_ms": "cgtp::uv_kernel<UV_sh3_d1,128>",
+             "grad_sh_ms": "cgtp::uv_gy_kernel<UV_sh3_gy,128>", "grad_w_ms": "cgtp::uv_gw_kernel<UV_sh3_gw>"}
+    print(json.dumps({
+        "metric": "uvw fwd+bwd TFLOP/s (lmax=3,C=128,bf16)", "value": round(4 * flops / (ms_step * 1e-3) / 1e12, 2),
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"uvw_fwd_bwd: B={n}, irreps {irreps}, C_in=C_out={ch}, shared W ({w.shape[0]},{ch},{ch}), "
+                               f"bf16 in / fp32 accumulate / bf16 out, SO3Linear('uv') forward + grads of x, sh, W"},
+        "roofline": {"bound": "mfma", "kernel": names[dom], "achieved": round(tf, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "algorithmic_flops": flops, "avg_ms": round(kern[dom], 5)},
+        "kernels": {k: round(v, 5) for k, v in kern.items()}}))
 
 
 def make_inputs(lmax, ch, n_nodes, n_edges, n_rot, device):
@@ -215,7 +270,7 @@ def main():
     if args.workload in ("copy", "read"):
         membench(args.workload, args.steps, args.warmup)
         return
-    if args.workload == "uvw_fwd":
+    if args.workload in ("uvw_fwd", "uvw_fwd_bwd"):
         uvw_bench(args)
         return
 

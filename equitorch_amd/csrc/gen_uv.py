@@ -136,12 +136,8 @@ def emit_direction(name: str, direction: int, coo, seg_out, seg_in1, gy: bool = 
         # hide the harmonics behind an empty asm per tile: equal (coefficient, harmonic) products recur in many
         # tiles and would otherwise be computed once and kept in registers across the whole body
         a("    " + " ".join(f'asm volatile("" : "+v"(yy[{m}]));' for m in sorted({m2 for _, m2, _ in terms})))
-        a("#ifndef UV_ABL_NOFMA")
         for (o, m2, c) in terms:
             a(f"    {{ const float s = {_lit(c)} * yy[{m2}]; o{o}_0 += s * {cur}0; o{o}_1 += s * {cur}1; }}")
-        a("#else")
-        a(f'    asm volatile("" :: "v"({cur}0), "v"({cur}1));')
-        a("#endif")
         # pin the updated accumulators: an output row is read again only when it is stored, and without this the
         # optimiser sinks every update of a block to its end, keeping all the block's tiles alive until then
         touched = sorted({o for o, _, _ in terms})
@@ -165,18 +161,22 @@ def emit_gw(name: str, coo, seg_out, seg_in1) -> str:
     T = coo.coef.shape[0]
     L = []
     w = L.append
-    a0, na = [], []
+    a0, na, m0, nm = [], [], [], []
     for p in range(coo.P):
-        rows = sorted({int(coo.M1[t]) for t in range(T) if coo.p[t] == p})
-        assert rows == list(range(rows[0], rows[0] + len(rows)))
-        a0.append(rows[0])
-        na.append(len(rows))
+        for col, first, count in ((coo.M1, a0, na), (coo.M, m0, nm)):
+            rows = sorted({int(col[t]) for t in range(T) if coo.p[t] == p})
+            assert rows == list(range(rows[0], rows[0] + len(rows)))
+            first.append(rows[0])
+            count.append(len(rows))
     w(f"struct UV_{name}_gw {{")
-    w(f"  static constexpr int D1 = {coo.D1}, DO = {coo.DO}, D2 = {coo.D2}, P = {coo.P}, MAX_ROWS = {max(na)};")
+    w(f"  static constexpr int D1 = {coo.D1}, DO = {coo.DO}, D2 = {coo.D2}, P = {coo.P}, MAX_ROWS = {max(na + nm)};")
     w("  // rows of the channelled input read by every path: first row and count")
     w(f"  static constexpr unsigned char A0[P] = {{{', '.join(map(str, a0))}}};")
     w(f"  static constexpr unsigned char NA[P] = {{{', '.join(map(str, na))}}};")
-    w("  // src(h, m): 8 channels (pass h of 2) of row m of g as floats; dst(h, r, v): the mixed row for input row")
+    w("  // rows of g (the output irrep) of every path: first row and count")
+    w(f"  static constexpr unsigned char M0[P] = {{{', '.join(map(str, m0))}}};")
+    w(f"  static constexpr unsigned char NM[P] = {{{', '.join(map(str, nm))}}};")
+    w("  // src(h, j): 8 channels (pass h of 2) of row M0[p] + j of g as floats; dst(h, r, v): the mixed row for input row")
     w("  // A0[p] + r.  Both passes of a path sit in one case so that the coef * y products are formed once per path")
     w("  // and only for the path at hand.")
     w("  template <class Src, class Dst>")
@@ -193,7 +193,7 @@ def emit_gw(name: str, coo, seg_out, seg_in1) -> str:
         for h in (0, 1):
             w("        {")
             for m in sorted({int(coo.M[t]) for t in nnz}):
-                w(f"          const floatx8 g{m} = src({h}, {m});")
+                w(f"          const floatx8 g{m} = src({h}, {m - m0[p]});")
             for r in range(na[p]):
                 terms = sorted((int(coo.M[t]), int(coo.M2[t]), _lit(coo.coef[t])) for t in nnz if coo.M1[t] == a0[p] + r)
                 expr = " + ".join(f"s{prods[(b, c)]} * g{m}" for m, b, c in terms)

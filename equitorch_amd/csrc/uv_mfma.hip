@@ -30,11 +30,7 @@ template <int KS>
 __device__ __forceinline__ void load_b(bf16x8 (&b)[KS], const unsigned char* xs) {
 #pragma unroll
   for (int k = 0; k < KS; ++k) {
-#ifdef UV_ABL_NOB
-    asm volatile("" : "=v"(b[k]) : "v"(xs));
-#else
     b[k] = *reinterpret_cast<const bf16x8*>(xs + k * 64);
-#endif
   }
 }
 
@@ -43,10 +39,6 @@ template <int KS>
 __device__ __forceinline__ void mfma_chain(const bf16x8 (&a)[2][KS], const bf16x8 (&b)[KS], floatx4& z0, floatx4& z1) {
   z0 = floatx4{0.f, 0.f, 0.f, 0.f};
   z1 = floatx4{0.f, 0.f, 0.f, 0.f};
-#ifdef UV_ABL_NOMFMA
-  asm volatile("" : "+v"(z0), "+v"(z1) : "v"(a[0][0]), "v"(a[1][KS-1]), "v"(b[0]), "v"(b[KS-1]));
-  return;
-#endif
 #pragma unroll
   for (int k = 0; k < KS; ++k) {
     z0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[0][k], b[k], z0, 0, 0, 0);
@@ -65,12 +57,6 @@ __device__ __forceinline__ float dot8(const floatx4& g0, const floatx4& g1, cons
 
 constexpr int kUvSamples = 16;
 
-#ifdef CGTP_UV_TRACE
-__device__ unsigned long long* g_uv_trace;
-#define UV_MARK(k) do { if ((threadIdx.x & 63) == 0) g_uv_trace[((int64_t)blockIdx.x * 4 + threadIdx.x / 64) * 8 + (k)] = clock64(); } while (0)
-#else
-#define UV_MARK(k)
-#endif
 
 // Stage the 16 samples' rows of one workgroup: 16-byte pieces, coalesced in global memory; every load is issued
 // before the first LDS write.  Rows past the end of the batch re-read the last row (their results are never stored).
@@ -111,11 +97,7 @@ struct UvWeights {
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int k = 0; k < CIN / 32; ++k)
-#ifdef UV_ABL_NOA
-        asm volatile("" : "=v"(frag[t][k]) : "v"(base));
-#else
         frag[t][k] = *reinterpret_cast<const bf16x8*>(base + p * path_stride + (t * (CIN / 32) + k) * 512);
-#endif
   }
 };
 
@@ -128,11 +110,8 @@ __global__ void __launch_bounds__(256, 2) uv_kernel(const __bf16* __restrict__ x
   constexpr int ROW_BYTES = DIN * CIN * 2;      // one sample's input rows
   constexpr int ROW_PITCH = ROW_BYTES + 16;     // + pad: consecutive samples start 16 B further in the banks
   const int64_t n0 = (int64_t)blockIdx.x * kUvSamples;
-  UV_MARK(0);
   uv_stage<ROW_BYTES>(x, n0, n_rows, smem);
-  UV_MARK(1);
   __syncthreads();
-  UV_MARK(2);
 
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int n = lane & 15, q = lane >> 4;
@@ -158,11 +137,7 @@ __global__ void __launch_bounds__(256, 2) uv_kernel(const __bf16* __restrict__ x
           }
           *reinterpret_cast<bf16x8*>(orow + row * cout) = v;
         }
-        if (row == 0) UV_MARK(3);
-        if (row == 3) UV_MARK(4);
-        if (row == 8) UV_MARK(5);
       });
-  UV_MARK(6);
 }
 
 // Gradient w.r.t. the harmonics: gy[n, b] = sum_t coef_t * sum_w g[n, m_t, w] * Z[p_t, a_t][w, n] with the same
@@ -232,8 +207,8 @@ constexpr int kGwChunk = 512;  // samples per workgroup
 constexpr int kGwPad = 32;     // bytes added to a tile row: the four rows a 16-lane transpose read touches land in
                                // distinct banks
 
-struct UvGwMeta {              // per configuration, passed by value: workgroup -> path, and the x rows of a path
-  unsigned char order[64], a0[64], na[64];
+struct UvGwMeta {              // per configuration, passed by value: workgroup -> path; x rows and g rows of a path
+  unsigned char order[64], a0[64], na[64], m0[64], nm[64];
 };
 
 __device__ __forceinline__ bf16x8 lds_read_tr(const unsigned char* p0, const unsigned char* p1) {
@@ -269,37 +244,74 @@ __global__ void __launch_bounds__(256, 1) uv_gw_kernel(const __bf16* __restrict_
   const int64_t n_begin = c * kGwChunk, n_end = min(n_begin + (int64_t)kGwChunk, n_rows);
   const int sn = tid >> 3, cg = tid & 7;              // mixing: sample of the step and 8-channel group (two passes)
   const int ls = lane & 15, lq = lane >> 4;           // fragment reads
+  // Operands of a step are fetched into registers one step ahead, row by row between the matrix work of the step
+  // before, so that neither their issue nor their latency is exposed.  x: per input row 32 samples x cin/8 16-byte
+  // pieces, thread = (sample, piece) in at most two passes; g: this thread's sample, two 8-channel groups of every
+  // row of the path's output irrep.  Row counts are the same for every lane: the guards are scalar branches.
+  constexpr int MR = CFG::MAX_ROWS;
+  const int m0 = __builtin_amdgcn_readfirstlane(meta.m0[p]), nm = __builtin_amdgcn_readfirstlane(meta.nm[p]);
+  const int lp = 31 - __builtin_clz(cin / 8);          // log2 of the pieces per row and sample
+  const int xpiece = tid & ((1 << lp) - 1), xs0 = tid >> lp, xstride = 256 >> lp;   // samples per pass
+  f32x4 xpre[MR][2];
+  bf16x8 gpre[2][MR];
+  float ypre[D2];
+  const __bf16 *xsrc[2], *gsrc[2];
+  auto prefetch_begin = [&](int64_t nb) __attribute__((always_inline)) {
+#pragma unroll
+    for (int v = 0; v < 2; ++v)
+      xsrc[v] = x + (min(nb + min(xs0 + v * xstride, kGwStep - 1), n_rows - 1) * D1 + a0) * cin + xpiece * 8;
+    const int64_t row = min(nb + sn, n_rows - 1);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) gsrc[h] = g + (row * DO + m0) * cout + min((cg + 8 * h) * 8, cout - 8);
+    if constexpr (D2 % 8 == 0) {
+#pragma unroll
+      for (int j = 0; j < D2; j += 8) {
+        const bf16x8 v = *reinterpret_cast<const bf16x8*>(y + row * D2 + j);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ypre[j + e] = (float)v[e];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < D2; ++j) ypre[j] = (float)y[row * D2 + j];
+    }
+  };
+  auto prefetch_row = [&](int r) __attribute__((always_inline)) {
+    if (r < na) {
+#pragma unroll
+      for (int v = 0; v < 2; ++v) xpre[r][v] = *reinterpret_cast<const f32x4*>(xsrc[v] + r * cin);
+    }
+    if (r < nm) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) gpre[h][r] = *reinterpret_cast<const bf16x8*>(gsrc[h] + r * cout);
+    }
+  };
+  prefetch_begin(n_begin);
+#pragma unroll
+  for (int r = 0; r < MR; ++r) prefetch_row(r);
+  const unsigned char* xa = xt + (8 * lq + (ls >> 2)) * pu + (ls & 3) * 8;
+  const unsigned char* gb = gt + (8 * lq + (ls >> 2)) * pw + (ls & 3) * 8;
   for (int64_t nb = n_begin; nb < n_end; nb += kGwStep) {
     __syncthreads();  // the previous step's fragment reads are done
-    // rows of x: per sample one contiguous run of na * cin elements
-    {
-      const int pieces = na * cin / 8;                // 16-byte pieces per sample
-      for (int i = tid; i < kGwStep * pieces; i += 256) {
-        const int s_ = i / pieces, k = i % pieces;
-        const int64_t row = min(nb + s_, n_rows - 1);
-        const f32x4 v = *reinterpret_cast<const f32x4*>(x + (row * D1 + a0) * cin + k * 8);
-        const int r = (k * 8) / cin, ch = (k * 8) % cin;
-        *reinterpret_cast<f32x4*>(xt + (r * kGwStep + s_) * pu + ch * 2) = v;
-      }
+#pragma unroll
+    for (int v = 0; v < 2; ++v) {
+      const int s_ = min(xs0 + v * xstride, kGwStep - 1);
+#pragma unroll
+      for (int r = 0; r < MR; ++r)
+        if (r < na) *reinterpret_cast<f32x4*>(xt + (r * kGwStep + s_) * pu + xpiece * 16) = xpre[r][v];
     }
     // mixed rows; samples past the end get y = 0 and so contribute nothing
     {
-      const int64_t n = nb + sn;
-      const int64_t row = min(n, n_rows - 1);
       float yv[D2];
+      const float live = nb + sn < n_end ? 1.f : 0.f;
 #pragma unroll
-      for (int j = 0; j < D2; ++j) yv[j] = n < n_end ? (float)y[row * D2 + j] : 0.f;
-      // two passes of 8 channels per thread; a pass beyond cout re-reads the last group and stores nothing
-      const __bf16* grow = g + row * DO * cout;
+      for (int j = 0; j < D2; ++j) yv[j] = ypre[j] * live;
       unsigned char* drow = gt + sn * pw;
       CFG::mix(
           p, yv,
-          [&](int h, int m) __attribute__((always_inline)) {
-            const int ch = min((cg + 8 * h) * 8, cout - 8);
-            const bf16x8 v = *reinterpret_cast<const bf16x8*>(grow + m * cout + ch);
+          [&](int h, int j) __attribute__((always_inline)) {
             floatx8 f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) f[e] = (float)v[e];
+            for (int e = 0; e < 8; ++e) f[e] = (float)gpre[h][j][e];
             return f;
           },
           [&](int h, int r, const floatx8& v) __attribute__((always_inline)) {
@@ -311,23 +323,30 @@ __global__ void __launch_bounds__(256, 1) uv_gw_kernel(const __bf16* __restrict_
           });
     }
     __syncthreads();
-    // contract over the 32 samples of the step, row by row
-    for (int r = 0; r < na; ++r) {
-      const unsigned char* xa = xt + (r * kGwStep + 8 * lq + (ls >> 2)) * pu + (ls & 3) * 8;
-      const unsigned char* gb = gt + (r * kGwStep + 8 * lq + (ls >> 2)) * pw + (ls & 3) * 8;
-      bf16x8 fa[4], fb[4];
+    // contract over the 32 samples of the step, row by row, fetching the next step's rows in between
+    const bool more = nb + kGwStep < n_end;
+    if (more) prefetch_begin(nb + kGwStep);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int ut = vu * 4 + i, wt = vw * 4 + i;
-        if (ut * 16 < cin) fa[i] = lds_read_tr(xa + ut * 32, xa + ut * 32 + 4 * pu);
-        if (wt * 16 < cout) fb[i] = lds_read_tr(gb + wt * 32, gb + wt * 32 + 4 * pw);
-      }
+    for (int r = 0; r < MR; ++r) {
+      if (more) prefetch_row(r);
+      if (r < na) {
+        const unsigned char* xr = xa + r * kGwStep * pu;
+        const unsigned char* gr = gb + r * kGwStep * pw;
+        bf16x8 fa[4], fb[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 4; ++i) {
+          // tiles past the channel count repeat the last one; their products are never stored.  No branches
+          // here: a branch per read would make every read wait for the one before.
+          const int ut = min(vu * 4 + i, cin / 16 - 1), wt = min(vw * 4 + i, cout / 16 - 1);
+          fa[i] = lds_read_tr(xr + ut * 32, xr + ut * 32 + 4 * pu);
+          fb[i] = lds_read_tr(gr + wt * 32, gr + wt * 32 + 4 * pw);
+        }
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if ((vu * 4 + i) * 16 < cin && (vw * 4 + j) * 16 < cout)
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      }
     }
   }
   // accumulator element e of lane (col = lane & 15, q) is row 4*q + e of the tile
@@ -406,6 +425,8 @@ static UvEntry make_uv_entry(uint64_t fp, const char* name) {
   for (int p = 0; p < GW::P; ++p) {
     e.gw_meta.a0[p] = GW::A0[p];
     e.gw_meta.na[p] = GW::NA[p];
+    e.gw_meta.m0[p] = GW::M0[p];
+    e.gw_meta.nm[p] = GW::NM[p];
   }
   return e;
 }

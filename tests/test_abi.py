@@ -87,6 +87,40 @@ def test_host_side_validation_codes():
     assert L.cgtp_membench_copy(256, 256, 17, None) == 2
 
 
+def test_uv_matrix_core_entry_points_validate_on_the_host():
+    """cgtp_uv_*: config lookup by fingerprint and argument checks, no launch (n_rows = 0 or a failing check)."""
+    from equitorch_amd import _lib
+    from equitorch_amd._tables import fingerprint, tp_coo
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    L = _lib.lib
+    sh3 = "0e+1o+2e+3o"
+    coo = tp_coo(tp_infos(Irreps(sh3), Irreps(sh3), Irreps(sh3))[0])
+    cfg = L.cgtp_uv_find(C.c_uint64(fingerprint(coo)))
+    assert 0 <= cfg < L.cgtp_uv_num_configs()
+    assert L.cgtp_uv_find(C.c_uint64(12345)) == -1
+    p16 = 4096  # any non-null, 16-byte aligned address: nothing is dereferenced by the checks
+    assert L.cgtp_uv_validate(cfg, 0, p16, p16, p16, p16, 100, 128, 128, _lib.BF16) == 0
+    assert L.cgtp_uv_validate(cfg, 2, p16, p16, p16, p16, 100, 128, 128, _lib.BF16) == 2       # direction
+    assert L.cgtp_uv_validate(cfg, 0, p16, p16, p16, p16, 100, 128, 128, _lib.F32) == 4        # dtype
+    assert L.cgtp_uv_validate(cfg, 0, p16, p16, p16, p16, 100, 48, 128, _lib.BF16) == 2        # C_in not 32/64/128
+    assert L.cgtp_uv_validate(cfg, 0, p16, p16, p16, p16, 100, 128, 80, _lib.BF16) == 2        # C_out % 32
+    assert L.cgtp_uv_validate(cfg, 0, p16 + 2, p16, p16, p16, 100, 128, 128, _lib.BF16) == 3   # alignment
+    assert L.cgtp_uv_validate(cfg, 0, None, p16, p16, p16, 100, 128, 128, _lib.BF16) == 1      # null
+    assert L.cgtp_uv_validate(99, 0, p16, p16, p16, p16, 100, 128, 128, _lib.BF16) == 5        # config
+    assert L.cgtp_uv_apply(cfg, 0, p16, p16, p16, p16, 0, 128, 128, _lib.BF16, None) == 0      # empty batch
+    assert L.cgtp_uv_grad_y(cfg, p16, p16, p16, p16, 0, 128, 128, _lib.BF16, None) == 0
+    assert L.cgtp_uv_grad_y(cfg, p16, p16, p16, p16, 10, 128, 256, _lib.BF16, None) == 2       # C_out > 128
+    assert L.cgtp_uv_pack_weights(0, p16, p16, 0, 128, 128, _lib.BF16, None) == 0
+    assert L.cgtp_uv_pack_weights(0, p16, p16, 23, 100, 128, _lib.BF16, None) == 2
+    assert L.cgtp_uv_pack_weights(3, p16, p16, 23, 128, 128, _lib.BF16, None) == 2
+    # weight gradient: one fp32 partial of (P, C_in, C_out) per chunk of 512 samples
+    assert L.cgtp_uv_grad_w_workspace_bytes(cfg, 32768, 128, 128) == 64 * 23 * 128 * 128 * 4
+    assert L.cgtp_uv_grad_w_workspace_bytes(cfg, 513, 32, 64) == 2 * 23 * 32 * 64 * 4
+    assert L.cgtp_uv_grad_w(cfg, p16, p16, p16, p16, None, 100, 128, 128, _lib.BF16, None) == 8  # workspace missing
+    assert L.cgtp_uv_grad_w(cfg, p16, p16, p16, p16, p16, 100, 128, 160, _lib.BF16, None) == 2
+
+
 def test_cpu_tensors_are_rejected_loudly():
     import torch
     from equitorch_amd import _lib

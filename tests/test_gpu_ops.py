@@ -197,7 +197,8 @@ def test_modules_uv_uvw_and_gradgradcheck(device):
         assert torch.autograd.gradgradcheck(fn, (x, y, w), eps=1e-6, atol=1e-5, rtol=1e-5, nondet_tol=1e-9)
 
 
-@pytest.mark.parametrize("lmax,cin,cout,n", [(1, 32, 32, 70), (2, 64, 128, 100), (3, 128, 128, 257), (3, 128, 64, 33)])
+@pytest.mark.parametrize("lmax,cin,cout,n", [(1, 32, 32, 70), (2, 64, 128, 100), (3, 128, 128, 257), (3, 128, 64, 33),
+                                             (3, 128, 128, 1100), (2, 32, 64, 700)])
 def test_uv_mfma_bf16(device, lmax, cin, cout, n):
     """bf16 matrix-core path of SO3Linear('uv'): forward and all gradients against the dense float64 oracle
     evaluated on the bf16-rounded inputs; tolerance rel 1e-2 of the tensor's largest magnitude (bf16 output)."""
@@ -224,3 +225,49 @@ def test_uv_mfma_bf16(device, lmax, cin, cout, n):
         a, b = a.detach().double().cpu(), b.double()
         err = float((a - b).abs().max())
         assert err <= 1e-2 * float(b.abs().max()), f"lmax={lmax} {name}: max abs err {err:.3e} vs scale {float(b.abs().max()):.3e}"
+
+
+def test_uv_mfma_full_size_properties(device):
+    """BASELINE configs[3] shapes (B = 32768, lmax = 3, C = 128, bf16).  The dense oracle is run on a strided
+    subset of the rows for out / grad_x / grad_sh (each row depends on its own sample only); the weight gradient
+    sums over the batch, so it is checked through additivity over two halves of the batch (bf16 rounding of the
+    three results bounds the difference) and against the oracle's sum over the subset when the other rows'
+    output gradients are zero."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.utils._sh import spherical_harmonics
+    from helpers import unit_vectors
+    lmax, ch, n = 3, 128, 32768
+    irreps = "0e+1o+2e+3o"
+    mod = SO3Linear(irreps, irreps, irreps, ch, ch, internal_weights=False, feature_mode="uv").to(device)
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(n, 16, ch, generator=g).bfloat16()
+    y = spherical_harmonics(unit_vectors(n, g), lmax).bfloat16()
+    w = (torch.randn(mod.num_paths, ch, ch, generator=g) / (ch * mod.num_paths) ** 0.5).bfloat16()
+    ct = torch.randn(n, 16, ch, generator=g).bfloat16()
+    sub = torch.arange(5, n, 257)                      # 128 rows spread over all chunks
+    mask = torch.zeros(n, 1, 1, dtype=torch.bfloat16)
+    mask[sub] = 1
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    out = mod(xd, yd, wd)
+    gx, gy, gw = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
+    T = ref_ops.dense_coupling(irreps, irreps, irreps).float().double()
+    ref_out, (rgx, rgy, rgw_sub) = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x[sub], y[sub], w), ct[sub])
+    for name, a, b in (("out", out[sub.to(device)], ref_out), ("grad_x", gx[sub.to(device)], rgx),
+                       ("grad_sh", gy[sub.to(device)], rgy)):
+        a, b = a.detach().double().cpu(), b.double()
+        assert float((a - b).abs().max()) <= 1e-2 * float(b.abs().max()), name
+    # weight gradient restricted to the subset (all other output gradients zero) against the oracle
+    out = mod(xd, yd, wd)
+    (gw_sub,) = torch.autograd.grad(out, (wd,), (ct * mask).to(device))
+    a, b = gw_sub.double().cpu(), rgw_sub.double()
+    assert float((a - b).abs().max()) <= 1e-2 * float(b.abs().max())
+    # additivity over the batch
+    half = n // 2
+    parts = []
+    for lo, hi in ((0, half), (half, n)):
+        xs, ys = xd[lo:hi].detach(), yd[lo:hi].detach()
+        ws = wd.detach().requires_grad_(True)
+        (gp,) = torch.autograd.grad(mod(xs, ys, ws), (ws,), ct[lo:hi].to(device))
+        parts.append(gp.double())
+    scale = float(gw.double().abs().max())
+    assert float((gw.double() - parts[0] - parts[1]).abs().max()) <= 2e-2 * scale
