@@ -40,8 +40,9 @@ def _compile(src: str) -> str:
 
 
 def build(jobs: int = 8) -> str:
-    from . import gen_uv, gen_uvu
+    from . import gen_uv, gen_uvu, gen_uvu_big
     gen_uvu.main()
+    gen_uvu_big.main()
     gen_uv.main()
     os.makedirs(OBJ_DIR, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)

@@ -1,0 +1,188 @@
+"""Emits ``generated/uvu_big_configs.inc``: the channel-wise tensor product for configurations whose table is too
+large for the register-resident bodies of ``gen_uvu`` (hundreds of weight rows, thousands of coefficients).
+
+One lane owns one channel.  The bodies walk the table output irrep by output irrep (only the 2l+1 rows of that
+irrep are live as accumulators or gradient rows) and inside an irrep path by path.  A path's weight is a single
+register, taken from a ring of ``RING`` registers that is refilled ``RING`` paths ahead so that the per-row weight
+stream never waits for memory.  Per path the forward evaluates
+
+    t = y[b] * x[a]   once per (a, b) pair,      i[M] += coef * t,      o[M] += w[p] * i[M]
+
+and the backward, with ``u[M] = w[p] * g[M]``,
+
+    gw[p] = sum_M i[M] * g[M]        gx[a] += coef * (y[b] * u[M])        gy[b] += coef * (x[a] * u[M])
+
+the pair products again formed once per pair.  Every index is a literal and every coefficient the hexadecimal
+literal of the fp32 table value.
+"""
+from __future__ import annotations
+
+import os
+from collections import OrderedDict
+
+from .._tables import fingerprint, tp_coo
+from ..irreps import Irreps, irrep_segments
+from ..utils import tp_infos
+from .gen_uvu import _lit, _sh
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+RING = 8
+
+CONFIGS = OrderedDict([
+    ("sh6", (_sh(6), _sh(6), _sh(6), {})),
+])
+
+
+def _pin(names) -> str:
+    """An empty asm that takes the accumulators as in/out operands, in chunks of 12: without it the optimiser
+    sinks updates towards the final store and keeps whole paths of temporaries alive."""
+    names = list(names)
+    out = []
+    for i in range(0, len(names), 12):
+        out.append('asm volatile("" : ' + ", ".join(f'"+v"({n})' for n in names[i:i + 12]) + ");")
+    return " ".join(out)
+
+
+def _grouped(terms, key):
+    d = OrderedDict()
+    for t in sorted(terms, key=key):
+        d.setdefault(key(t), []).append(t)
+    return d
+
+
+def emit_config(name: str, coo, seg_out) -> str:
+    T = coo.coef.shape[0]
+    term = [(int(coo.p[t]), int(coo.M[t]), int(coo.M1[t]), int(coo.M2[t]), _lit(coo.coef[t])) for t in range(T)]
+    # execution order: output irrep blocks, inside a block the paths in table order
+    blocks = []
+    for b0, b1 in zip(seg_out[:-1], seg_out[1:]):
+        paths = sorted({p for p, M, _, _, _ in term if b0 <= M < b1})
+        if paths:
+            blocks.append((list(range(b0, b1)), paths))
+    order = [p for _, paths in blocks for p in paths]
+    assert sorted(order) == list(range(coo.P))
+    pos = {p: k for k, p in enumerate(order)}
+    by_path = {p: [t for t in term if t[0] == p] for p in order}
+
+    L = []
+    a = L.append
+    a(f"struct TPB_{name} {{")
+    a(f"  static constexpr int D1 = {coo.D1}, D2 = {coo.D2}, DO = {coo.DO}, P = {coo.P}, NNZ = {T};")
+    a(f"  static constexpr unsigned long long FINGERPRINT = 0x{fingerprint(coo):016x}ull;")
+    a(f"  static constexpr const char* NAME = \"{name}\";")
+
+    def ring_prologue():
+        for k in range(min(RING, len(order))):
+            a(f"    float wq{k} = wload({order[k]});")
+
+    def ring_take(p):
+        k = pos[p]
+        a(f"      const float w = wq{k % RING};")
+        if k + RING < len(order):
+            a(f"      wq{k % RING} = wload({order[k + RING]});")
+
+    def opaque(ys):
+        a("      " + " ".join(f'asm volatile("" : "+v"(yy[{m}]));' for m in sorted(ys)))
+
+    # ---- forward ---------------------------------------------------------------------------------------------
+    a("  // wload(p): this lane's channel of weight path p; store(M, v): one finished output row")
+    a("  template <class WLoad, class Store>")
+    a("  __device__ __forceinline__ static void fwd(const float (&x)[D1], const float (&y)[D2], WLoad&& wload,")
+    a("                                             Store&& store) {")
+    a("    float yy[D2];")
+    a("    for (int j = 0; j < D2; ++j) yy[j] = y[j];")
+    ring_prologue()
+    for rows, paths in blocks:
+        a("    {")
+        a("      float " + ", ".join(f"o{M} = 0.f" for M in rows) + ";")
+        for p in paths:
+            ms = sorted({M for _, M, _, _, _ in by_path[p]})
+            a("      {")
+            ring_take(p)
+            opaque({b for _, _, _, b, _ in by_path[p]})
+            a("      float " + ", ".join(f"i{M}" for M in ms) + ";")
+            seen = set()
+            for (aa, b), ts in _grouped(by_path[p], lambda t: (t[2], t[3])).items():
+                ops = []
+                for _, M, _, _, c in ts:
+                    ops.append(f"i{M} {'+=' if M in seen else '='} {c} * t;")
+                    seen.add(M)
+                a(f"      {{ const float t = yy[{b}] * x[{aa}]; " + " ".join(ops) + " }")
+            a("      " + " ".join(f"o{M} += w * i{M};" for M in ms))
+            a("      " + _pin(f"o{M}" for M in ms))
+            a("      }")
+        for M in rows:
+            a(f"      store({M}, o{M});")
+        a("    }")
+    a("  }")
+
+    # ---- backward --------------------------------------------------------------------------------------------
+    a("  // gload(M): this lane's channel of row M of grad_out; gwsink(p, v): gradient of weight path p;")
+    a("  // gx / gy: accumulated in place (gy holds this lane's channel only, the caller sums over channels)")
+    a("  template <class WLoad, class GLoad, class GwSink>")
+    a("  __device__ __forceinline__ static void bwd(const float (&x)[D1], const float (&y)[D2], WLoad&& wload,")
+    a("                                             GLoad&& gload, float (&gx)[D1], float (&gy)[D2],")
+    a("                                             GwSink&& gwsink) {")
+    a("    float yy[D2], xx[D1];")
+    a("    for (int j = 0; j < D2; ++j) yy[j] = y[j];")
+    a("    for (int j = 0; j < D1; ++j) xx[j] = x[j];")
+    ring_prologue()
+    for M in blocks[0][0]:
+        a(f"    const float g{M} = gload({M});")
+    for bi, (rows, paths) in enumerate(blocks):
+        if bi + 1 < len(blocks):  # rows of the next irrep are requested one block ahead
+            for M in blocks[bi + 1][0]:
+                a(f"    const float g{M} = gload({M});")
+        a("    {")
+        for p in paths:
+            ts_p = by_path[p]
+            ms = sorted({M for _, M, _, _, _ in ts_p})
+            a("      {")
+            ring_take(p)
+            opaque({b for _, _, _, b, _ in ts_p})
+            a("      " + " ".join(f'asm volatile("" : "+v"(xx[{m}]));' for m in sorted({t[2] for t in ts_p})))
+            a("      float " + ", ".join(f"i{M}" for M in ms) + ";")
+            a("      " + " ".join(f"const float u{M} = w * g{M};" for M in ms))
+            seen = set()
+            for (aa, b), ts in _grouped(ts_p, lambda t: (t[2], t[3])).items():
+                ops = []
+                for _, M, _, _, c in ts:
+                    ops.append(f"i{M} {'+=' if M in seen else '='} {c} * t;")
+                    seen.add(M)
+                a(f"      {{ const float t = yy[{b}] * xx[{aa}]; " + " ".join(ops) + " }")
+            a(f"      gwsink({p}, " + " + ".join(f"i{M} * g{M}" for M in ms) + ");")
+            for (b, M), ts in _grouped(ts_p, lambda t: (t[3], t[1])).items():
+                a(f"      {{ const float t = yy[{b}] * u{M}; " + " ".join(f"gx[{aa}] += {c} * t;" for _, _, aa, _, c in ts) + " }")
+            a("      " + _pin(f"gx[{m}]" for m in sorted({t[2] for t in ts_p})))
+            for (aa, M), ts in _grouped(ts_p, lambda t: (t[2], t[1])).items():
+                a(f"      {{ const float t = xx[{aa}] * u{M}; " + " ".join(f"gy[{b}] += {c} * t;" for _, _, _, b, c in ts) + " }")
+            a("      " + _pin(f"gy[{m}]" for m in sorted({t[3] for t in ts_p})))
+            a("      }")
+        a("    }")
+    a("  }")
+    a("};")
+    return "\n".join(L)
+
+
+def main(out_dir: str = None) -> str:
+    out_dir = out_dir or os.path.join(HERE, "generated")
+    os.makedirs(out_dir, exist_ok=True)
+    chunks = ["// Generated by equitorch_amd/csrc/gen_uvu_big.py; do not edit.", ""]
+    for name, (io, i1, i2, kw) in CONFIGS.items():
+        coo = tp_coo(tp_infos(Irreps(io), Irreps(i1), Irreps(i2), **kw)[0])
+        chunks.append(f"// {name}: {i1} x {i2} -> {io}")
+        chunks.append(emit_config(name, coo, irrep_segments(Irreps(io))))
+        chunks.append("")
+    chunks.append("#define CGTP_FOREACH_UVU_BIG_CONFIG(X) \\")
+    chunks.append(" \\\n".join(f"  X(TPB_{n})" for n in CONFIGS))
+    chunks.append("")
+    path = os.path.join(out_dir, "uvu_big_configs.inc")
+    text = "\n".join(chunks)
+    if not os.path.exists(path) or open(path).read() != text:
+        with open(path, "w") as f:
+            f.write(text)
+    return path
+
+
+if __name__ == "__main__":
+    print(main())

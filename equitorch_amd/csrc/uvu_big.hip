@@ -1,0 +1,108 @@
+// Channel-wise ("uvu") tensor product for configurations with very large tables (lmax = 6: 106 weight paths, 6460
+// coefficients): fp32, one batch row per group of lanes, one channel per lane.  The arithmetic (about two vector
+// instructions per coefficient and channel) dominates the memory traffic here, so the kernels keep only what the
+// generated bodies need in registers: the input rows x and y, a ring of weight values fetched a few paths ahead,
+// and the 2l+1 output (or output-gradient) rows of the irrep being worked on.
+#include "uvu_common.h"
+
+namespace cgtp {
+#include "generated/uvu_big_configs.inc"
+
+// Lanes past the batch or the channel count re-read the last valid element and store nothing, so that every lane
+// runs the same code and the channel sum of grad_y can use full-width shuffles.
+template <class TP>
+__global__ void __launch_bounds__(256, 2) uvu_big_fwd_kernel(const UvuDev<float> a) {
+  constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
+  const Lanes L(a.lpe_log2);
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  const int64_t C = a.C;
+  const int c_raw = blockIdx.y * L.lpe + L.cl;
+  const int64_t r_raw = wave * L.slots + L.slot;
+  const bool live = r_raw < a.n_rows && c_raw < a.C;
+  const int64_t r = min(r_raw, a.n_rows - 1);
+  const int c = min(c_raw, a.C - 1);
+  const int64_t xr = a.gather ? a.gather[r] : r;
+  float x[D1], y[D2];
+#pragma unroll
+  for (int j = 0; j < D2; ++j) y[j] = a.y[r * D2 + j];
+#pragma unroll
+  for (int i = 0; i < D1; ++i) x[i] = a.x[(xr * D1 + i) * C + c];
+  const float* wrow = a.w + (a.w_shared ? 0 : r) * P * C + c;
+  float* orow = a.out + r * DO * C + c;
+  TP::fwd(
+      x, y, [&](int p) __attribute__((always_inline)) { return __builtin_nontemporal_load(wrow + p * C); },
+      [&](int m, float v) __attribute__((always_inline)) {
+        if (live) __builtin_nontemporal_store(v, orow + m * C);
+      });
+}
+
+template <class TP, int GW>
+__global__ void __launch_bounds__(256, 1) uvu_big_bwd_kernel(const UvuDev<float> a, int64_t n_waves) {
+  constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
+  const Lanes L(a.lpe_log2);
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (wave >= n_waves) return;
+  const int64_t C = a.C;
+  const int64_t r_raw = wave * L.slots + L.slot;
+  const bool row_ok = r_raw < a.n_rows, live = row_ok && L.cl < a.C;
+  const int64_t r = min(r_raw, a.n_rows - 1);
+  const int c = min(L.cl, a.C - 1);
+  const int64_t gr = a.gather ? a.gather[r] : r;
+  const int64_t xr = a.x_gather ? a.x_gather[r] : r;
+  float x[D1], y[D2], gx[D1], gy[D2];
+#pragma unroll
+  for (int j = 0; j < D2; ++j) {
+    y[j] = a.y[r * D2 + j];
+    gy[j] = 0.f;
+  }
+#pragma unroll
+  for (int i = 0; i < D1; ++i) {
+    x[i] = a.x[(xr * D1 + i) * C + c];
+    gx[i] = 0.f;
+  }
+  const float* wrow = a.w + (a.w_shared ? 0 : r) * P * C + c;
+  const float* grow = a.g + gr * DO * C + c;
+  float* gwrow = a.gw + r * P * C + c;
+  TP::bwd(
+      x, y, [&](int p) __attribute__((always_inline)) { return __builtin_nontemporal_load(wrow + p * C); },
+      [&](int m) __attribute__((always_inline)) { return grow[m * C]; }, gx, gy,
+      [&](int p, float v) __attribute__((always_inline)) {
+        if constexpr (GW == kGwStore) {
+          if (live) __builtin_nontemporal_store(v, gwrow + p * C);
+        }
+      });
+  if (a.gx && live) {
+#pragma unroll
+    for (int i = 0; i < D1; ++i) __builtin_nontemporal_store(gx[i], a.gx + (r * D1 + i) * C + c);
+  }
+  if (a.gy) {
+    const float keep = L.cl < a.C ? 1.f : 0.f;  // duplicate channels of the padding lanes do not count
+#pragma unroll
+    for (int j = 0; j < D2; ++j) {
+      const float s = group_sum(gy[j] * keep, L.lpe);
+      if (row_ok && L.cl == (j & (L.lpe - 1))) a.gy[r * D2 + j] = s;
+    }
+  }
+}
+
+template <class TP>
+static UvuBigEntry make_big_entry() {
+  UvuBigEntry e;
+  e.fingerprint = TP::FINGERPRINT;
+  e.dims[0] = TP::D1; e.dims[1] = TP::D2; e.dims[2] = TP::DO; e.dims[3] = TP::P; e.dims[4] = TP::NNZ;
+  e.name = TP::NAME;
+  e.fwd = uvu_big_fwd_kernel<TP>;
+  e.bwd[kGwNone] = uvu_big_bwd_kernel<TP, kGwNone>;
+  e.bwd[kGwStore] = uvu_big_bwd_kernel<TP, kGwStore>;
+  return e;
+}
+
+const UvuBigEntry* uvu_big_entries(int* count) {
+#define CGTP_X(TP) make_big_entry<TP>(),
+  static const UvuBigEntry table[] = {CGTP_FOREACH_UVU_BIG_CONFIG(CGTP_X)};
+#undef CGTP_X
+  *count = (int)(sizeof(table) / sizeof(table[0]));
+  return table;
+}
+
+}  // namespace cgtp

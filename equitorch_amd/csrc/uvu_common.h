@@ -1,0 +1,58 @@
+// Kernel-side argument block and lane decomposition shared by the channel-wise ("uvu") tensor-product kernels.
+#pragma once
+
+#include "cgtp_device.h"
+#include "cgtp_host.h"
+
+namespace cgtp {
+
+template <typename T>
+struct UvuDev {
+  const T* x;
+  const T* y;
+  const T* w;
+  T* out;
+  const T* g;
+  T* gx;
+  T* gy;
+  T* gw;
+  T* ws;   // segment mode: partial rows (n_waves, 2, D, C)
+  T* wsw;  // per-wavefront partial sums of a shared weight's gradient (n_waves, P, C)
+  const int64_t* ptr;
+  const int64_t* perm;
+  const int64_t* gather;
+  const int64_t* x_gather;  // row mode backward: optional row of x per batch row
+  const int64_t* seg_ids;
+  const int32_t* wave_seg;  // segment mode: optional wavefront -> first segment table (segment-aligned ranges)
+  int64_t n_rows, n_seg;
+  int C, lpe_log2, w_shared, pos_per_wave;
+};
+
+struct Lanes {
+  int lane, lpe, slots, slot, cl;
+  __device__ __forceinline__ explicit Lanes(int lpe_log2) {
+    lane = threadIdx.x & (kWave - 1);
+    lpe = 1 << lpe_log2;
+    slots = kWave >> lpe_log2;
+    slot = lane >> lpe_log2;
+    cl = lane & (lpe - 1);
+  }
+};
+
+// What the backward does with the weight gradient.  kGwReduce: the weight is shared over rows, so its gradient
+// is summed over every row a wavefront visits and written as one partial per wavefront into the workspace
+// (partial_sum_kernel finishes the sum).  A compile-time choice keeps the generated body free of branches.
+enum { kGwNone = 0, kGwStore = 1, kGwReduce = 2 };
+
+// Configurations too large for the register-resident bodies (uvu_big.hip): fp32, row mode, one channel per lane,
+// per-row weights or no weight gradient.
+struct UvuBigEntry {
+  uint64_t fingerprint;
+  int dims[5];
+  const char* name;
+  void (*fwd)(const UvuDev<float>);
+  void (*bwd[2])(const UvuDev<float>, int64_t);  // [kGwNone, kGwStore]
+};
+const UvuBigEntry* uvu_big_entries(int* count);
+
+}  // namespace cgtp

@@ -13,43 +13,10 @@
 // cross-lane shuffles and stored once.  A segment that lies entirely inside the wavefront's range is written to the
 // output directly; the (at most two) segments cut by the range boundary are written as partial rows to a
 // workspace and summed in a fixed order by uvu_fixup_kernel.  No atomics: results are deterministic.
-#include "cgtp_device.h"
-#include "cgtp_host.h"
+#include "uvu_common.h"
 
 namespace cgtp {
 #include "generated/uvu_configs.inc"
-
-template <typename T>
-struct UvuDev {
-  const T* x;
-  const T* y;
-  const T* w;
-  T* out;
-  const T* g;
-  T* gx;
-  T* gy;
-  T* gw;
-  T* ws;   // segment mode: partial rows (n_waves, 2, D, C)
-  T* wsw;  // per-wavefront partial sums of a shared weight's gradient (n_waves, P, C)
-  const int64_t* ptr;
-  const int64_t* perm;
-  const int64_t* gather;
-  const int64_t* seg_ids;
-  const int32_t* wave_seg;  // segment mode: optional wavefront -> first segment table (segment-aligned ranges)
-  int64_t n_rows, n_seg;
-  int C, lpe_log2, w_shared, pos_per_wave;
-};
-
-struct Lanes {
-  int lane, lpe, slots, slot, cl;
-  __device__ __forceinline__ explicit Lanes(int lpe_log2) {
-    lane = threadIdx.x & (kWave - 1);
-    lpe = 1 << lpe_log2;
-    slots = kWave >> lpe_log2;
-    slot = lane >> lpe_log2;
-    cl = lane & (lpe - 1);
-  }
-};
 
 template <typename T, int D, int V>
 __device__ __forceinline__ void zero_rows(T (&a)[D][V]) {
@@ -89,10 +56,6 @@ __global__ void __launch_bounds__(256) uvu_fwd_kernel(const UvuDev<T> a) {
   for (int m = 0; m < DO; ++m) store_vec_stream<T, V>(a.out + (r * DO + m) * C + c0, acc[m]);
 }
 
-// What the backward does with the weight gradient.  kGwReduce: the weight is shared over rows, so its gradient
-// is summed over every row a wavefront visits and written as one partial per wavefront into the workspace
-// (partial_sum_kernel finishes the sum).  A compile-time choice keeps the generated body free of branches.
-enum { kGwNone = 0, kGwStore = 1, kGwReduce = 2 };
 
 template <class TP, typename T, int V, int GW>
 __global__ void __launch_bounds__(256, 2) uvu_bwd_kernel(const UvuDev<T> a, int64_t n_waves) {
@@ -110,6 +73,7 @@ __global__ void __launch_bounds__(256, 2) uvu_bwd_kernel(const UvuDev<T> a, int6
 #pragma unroll 1
   for (int64_t r = wave * L.slots + L.slot; r < a.n_rows; r += n_waves * L.slots) {
     const int64_t gr = a.gather ? a.gather[r] : r;
+    const int64_t xr = a.x_gather ? a.x_gather[r] : r;
     T x[D1][V], g[DO][V], y[D2], gy[D2];
 #pragma unroll
     for (int j = 0; j < D2; ++j) {
@@ -118,7 +82,7 @@ __global__ void __launch_bounds__(256, 2) uvu_bwd_kernel(const UvuDev<T> a, int6
     }
     if (cok) {
 #pragma unroll
-      for (int i = 0; i < D1; ++i) load_vec<T, V>(x[i], a.x + (r * D1 + i) * C + c0);
+      for (int i = 0; i < D1; ++i) load_vec<T, V>(x[i], a.x + (xr * D1 + i) * C + c0);
 #pragma unroll
       for (int m = 0; m < DO; ++m) load_vec<T, V>(g[m], a.g + (gr * DO + m) * C + c0);
       const T* wrow = a.w + (a.w_shared ? 0 : r) * P * C + c0;
@@ -508,13 +472,18 @@ static constexpr int kDefaultPosPerWave = 32;
 
 static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan* plan) {
   if (!a) return CGTP_ERR_NULL;
-  int n_cfg = 0;
+  int n_cfg = 0, n_big = 0;
   const UvuEntry<float>* tab = entries<float>(&n_cfg);
-  if (a->cfg < 0 || a->cfg >= n_cfg) return CGTP_ERR_CONFIG;
+  const UvuBigEntry* big_tab = uvu_big_entries(&n_big);
+  if (a->cfg < 0 || a->cfg >= n_cfg + n_big) return CGTP_ERR_CONFIG;
+  const bool big = a->cfg >= n_cfg;  // large-table configurations follow the register-resident ones
+  const int* dims = big ? big_tab[a->cfg - n_cfg].dims : tab[a->cfg].dims;
   if (a->dtype != CGTP_F32 && a->dtype != CGTP_F64) return CGTP_ERR_DTYPE;
+  if (big && a->dtype != CGTP_F32) return CGTP_ERR_DTYPE;
   if (a->C <= 0 || a->n_rows < 0 || a->n_seg < 0 || a->n_x_rows < 0 || a->pos_per_wave < 0) return CGTP_ERR_SHAPE;
   if (!a->x || !a->y || !a->w) return CGTP_ERR_NULL;
   const bool seg = a->n_seg > 0;
+  if (big && (seg || (backward && a->w_shared && a->grad_w))) return CGTP_ERR_SHAPE;  // row mode, per-row weight gradient
   if (seg && (!a->ptr || !a->seg_ids || !a->gather)) return CGTP_ERR_NULL;
   if (!seg && (a->ptr || a->perm || a->seg_ids)) return CGTP_ERR_SHAPE;
   if (seg && (a->n_seg >= (int64_t)1 << 31 || a->n_rows >= (int64_t)1 << 31 || a->n_x_rows >= (int64_t)1 << 31))
@@ -523,13 +492,16 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
   if (backward) {
     if (!a->grad_out) return CGTP_ERR_NULL;
     if (seg && a->n_x_rows != a->n_seg) return CGTP_ERR_SHAPE;
-    if (!seg && a->n_x_rows != a->n_rows) return CGTP_ERR_SHAPE;
+    if (!seg && !a->x_gather && a->n_x_rows != a->n_rows) return CGTP_ERR_SHAPE;
+    if (seg && a->x_gather) return CGTP_ERR_SHAPE;
   } else {
     if (!a->out) return CGTP_ERR_NULL;
     if (!seg && !a->gather && a->n_x_rows != a->n_rows) return CGTP_ERR_SHAPE;
   }
   int vw;
-  if (a->dtype == CGTP_F32) {
+  if (big) {
+    vw = 1;
+  } else if (a->dtype == CGTP_F32) {
     vw = backward ? tab[a->cfg].v_bwd : tab[a->cfg].v_fwd;
   } else {
     int n64 = 0;
@@ -552,7 +524,7 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
   // channel reduction of grad_y and the segment accumulators stay inside one slot
   if ((backward || seg) && lanes > kWave) return CGTP_ERR_SHAPE;
   const int slots = kWave >> lg;
-  const int64_t row_d = backward ? tab[a->cfg].dims[0] : tab[a->cfg].dims[2];
+  const int64_t row_d = backward ? dims[0] : dims[2];
   const bool wred = backward && a->w_shared && a->grad_w;
   plan->ws_elems = plan->wsw_elems = 0;
   plan->pos_per_wave = 0;
@@ -569,7 +541,7 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
     if (wred && nw > kMaxRowWaves) nw = kMaxRowWaves;
     plan->n_waves = nw;
   }
-  if (wred) plan->wsw_elems = plan->n_waves * tab[a->cfg].dims[3] * a->C;
+  if (wred) plan->wsw_elems = plan->n_waves * dims[3] * a->C;
   if (need_ws && plan->ws_elems + plan->wsw_elems > 0 && !a->workspace) return CGTP_ERR_WORKSPACE;
   return CGTP_OK;
 }
@@ -581,7 +553,7 @@ static UvuDev<T> to_dev(const cgtp_uvu_args* a, const UvuPlan& plan) {
   d.g = (const T*)a->grad_out; d.gx = (T*)a->grad_x; d.gy = (T*)a->grad_y; d.gw = (T*)a->grad_w;
   d.ws = (T*)a->workspace;
   d.wsw = d.ws ? d.ws + plan.ws_elems : nullptr;
-  d.ptr = a->ptr; d.perm = a->perm; d.gather = a->gather; d.seg_ids = a->seg_ids; d.wave_seg = a->wave_seg;
+  d.ptr = a->ptr; d.perm = a->perm; d.gather = a->gather; d.x_gather = a->x_gather; d.seg_ids = a->seg_ids; d.wave_seg = a->wave_seg;
   d.n_rows = a->n_rows; d.n_seg = a->n_seg;
   d.C = a->C; d.lpe_log2 = plan.lpe_log2; d.w_shared = a->w_shared; d.pos_per_wave = plan.pos_per_wave;
   return d;
@@ -594,6 +566,29 @@ static int launch_fixup(T* rows, const UvuDev<T>& d, int64_t row_len, hipStream_
   hipLaunchKernelGGL(uvu_fixup_kernel<T>, dim3((unsigned)((d.n_seg + 3) / 4)), dim3(256), 0, stream, rows,
                      (const T*)d.ws, d.ptr, d.n_seg, row_len, d.pos_per_wave);
   return launched();
+}
+
+static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward, hipStream_t stream) {
+  int n = 0, n_big = 0;
+  entries<float>(&n);
+  const UvuBigEntry& e = uvu_big_entries(&n_big)[a->cfg - n];
+  if (plan.n_waves == 0) return CGTP_OK;
+  const UvuDev<float> d = to_dev<float>(a, plan);
+  if (backward) {
+    hipLaunchKernelGGL(e.bwd[a->grad_w ? kGwStore : kGwNone], dim3((unsigned)((plan.n_waves + 3) / 4)), dim3(256), 0,
+                       stream, d, plan.n_waves);
+  } else {
+    const int chunk = 1 << plan.lpe_log2;
+    dim3 grid((unsigned)((plan.n_waves + 3) / 4), (unsigned)((a->C + chunk - 1) / chunk));
+    hipLaunchKernelGGL(e.fwd, grid, dim3(256), 0, stream, d);
+  }
+  return launched();
+}
+
+static bool is_big(int cfg) {
+  int n = 0;
+  entries<float>(&n);
+  return cfg >= n;
 }
 
 template <typename T>
@@ -650,26 +645,32 @@ using namespace cgtp;
 extern "C" {
 
 int cgtp_uvu_num_configs(void) {
-  int n = 0;
+  int n = 0, n_big = 0;
   entries<float>(&n);
-  return n;
+  uvu_big_entries(&n_big);
+  return n + n_big;
 }
 
 int cgtp_uvu_find(uint64_t fingerprint) {
-  int n = 0;
+  int n = 0, n_big = 0;
   const UvuEntry<float>* t = entries<float>(&n);
   for (int i = 0; i < n; ++i)
     if (t[i].fingerprint == fingerprint) return i;
+  const UvuBigEntry* b = uvu_big_entries(&n_big);
+  for (int i = 0; i < n_big; ++i)
+    if (b[i].fingerprint == fingerprint) return n + i;
   return -1;
 }
 
 uint64_t cgtp_uvu_describe(int cfg, int32_t* dims) {
-  int n = 0;
+  int n = 0, n_big = 0;
   const UvuEntry<float>* t = entries<float>(&n);
-  if (cfg < 0 || cfg >= n) return 0;
+  const UvuBigEntry* b = uvu_big_entries(&n_big);
+  if (cfg < 0 || cfg >= n + n_big) return 0;
+  const int* d = cfg < n ? t[cfg].dims : b[cfg - n].dims;
   if (dims)
-    for (int i = 0; i < 5; ++i) dims[i] = t[cfg].dims[i];
-  return t[cfg].fingerprint;
+    for (int i = 0; i < 5; ++i) dims[i] = d[i];
+  return cfg < n ? t[cfg].fingerprint : b[cfg - n].fingerprint;
 }
 
 int cgtp_uvu_validate(const cgtp_uvu_args* args, int backward) {
@@ -687,6 +688,7 @@ int cgtp_uvu_fwd(const cgtp_uvu_args* a, void* stream) {
   UvuPlan plan;
   const int st = uvu_plan(a, 0, true, &plan);
   if (st != CGTP_OK) return st;
+  if (is_big(a->cfg)) return launch_big(a, plan, 0, (hipStream_t)stream);
   return a->dtype == CGTP_F32 ? launch_fwd<float>(a, plan, (hipStream_t)stream)
                               : launch_fwd<double>(a, plan, (hipStream_t)stream);
 }
@@ -695,6 +697,7 @@ int cgtp_uvu_bwd(const cgtp_uvu_args* a, void* stream) {
   UvuPlan plan;
   const int st = uvu_plan(a, 1, true, &plan);
   if (st != CGTP_OK) return st;
+  if (is_big(a->cfg)) return launch_big(a, plan, 1, (hipStream_t)stream);
   return a->dtype == CGTP_F32 ? launch_bwd<float>(a, plan, (hipStream_t)stream)
                               : launch_bwd<double>(a, plan, (hipStream_t)stream);
 }

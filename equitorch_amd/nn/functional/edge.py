@@ -80,6 +80,37 @@ class _EdgeUvuCompiled(Function):
         return (*res, None, None, None)
 
 
+class _EdgeUvuRows(Function):
+    """The same composition on the row-mode kernels, for tables the fused segment kernels do not cover: per-edge
+    messages from the gathered node rows, then a segment sum over the dst-sorted list; the backward forms the
+    per-edge gradient of the gathered rows and sums it over the src-sorted list."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, sh: Tensor, w: Tensor, plan: EdgePlan, tp_info: TensorProductInfo, cfg: int):
+        dims = kernels.uvu_dims(cfg)
+        msg = kernels.uvu_forward(cfg, dims, x, sh, w, gather=plan.src)
+        e, d, c = msg.shape
+        out = kernels.segment_sum(msg.view(1, e, d * c), None, plan.perm_dst, plan.ptr_dst, plan.num_nodes)
+        ctx.save_for_backward(x, sh, w)
+        ctx.plan, ctx.cfg, ctx.dims = plan, cfg, dims
+        return out.view(plan.num_nodes, d, c)
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, g):
+        x, sh, w = ctx.saved_tensors
+        plan = ctx.plan
+        need = ctx.needs_input_grad[:3]
+        gxe, gy, gw = kernels.uvu_backward(ctx.cfg, ctx.dims, x, sh, w, g.contiguous(), need, gather=plan.dst,
+                                           x_gather=plan.src)
+        gx = None
+        if need[0]:
+            e, d, c = gxe.shape
+            gx = kernels.segment_sum(gxe.view(1, e, d * c), None, plan.perm_src, plan.ptr_src,
+                                     plan.num_src_nodes).view(plan.num_src_nodes, d, c)
+        return gx, gy, gw, None, None, None
+
+
 def edge_tensor_product_uu(x: Tensor, sh: Tensor, weight: Tensor, plan: EdgePlan,
                            tp_info_forward: TensorProductInfo,
                            tp_info_backward1: Optional[TensorProductInfo] = None,
@@ -98,6 +129,8 @@ def edge_tensor_product_uu(x: Tensor, sh: Tensor, weight: Tensor, plan: EdgePlan
         xc, yc, wc = x.contiguous(), sh.contiguous(), weight.contiguous()
         if kernels.uvu_launchable(cfg, xc, yc, wc, segments=True):
             return _EdgeUvuCompiled.apply(xc, yc, wc, plan, tp_info_forward, cfg)
+        if kernels.uvu_launchable(cfg, xc, yc, wc, gathered=True):
+            return _EdgeUvuRows.apply(xc, yc, wc, plan, tp_info_forward, cfg)
     msg = tensor_product_u1u(x.index_select(0, plan.src), sh, weight, tp_info_forward)
     e, d, c = msg.shape
     fwd, bwd = plan.scale_infos()

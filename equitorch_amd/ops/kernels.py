@@ -163,9 +163,10 @@ def _workspace(a: UvuArgs, backward: int, device):
     return ws
 
 
-def uvu_launchable(cfg: int, x: Tensor, y: Tensor, w: Tensor, segments: bool = False) -> bool:
+def uvu_launchable(cfg: int, x: Tensor, y: Tensor, w: Tensor, segments: bool = False, gathered: bool = False) -> bool:
     """True when both the specialised forward and backward accept these operands (dtype, channel count,
-    alignment); outputs are torch allocations and therefore always aligned."""
+    alignment); outputs are torch allocations and therefore always aligned.  ``gathered``: row mode with the rows
+    of ``x`` picked by an index."""
     if x.shape[0] == 0 or y.shape[0] == 0:
         return False
     a = UvuArgs()
@@ -176,6 +177,8 @@ def uvu_launchable(cfg: int, x: Tensor, y: Tensor, w: Tensor, segments: bool = F
     a.n_x_rows = x.shape[0]
     if segments:
         a.n_seg, a.ptr, a.gather, a.seg_ids = x.shape[0], dummy, dummy, dummy
+    elif gathered:
+        a.gather = a.x_gather = dummy
     a.x, a.y, a.w = x.data_ptr() or dummy, y.data_ptr() or dummy, w.data_ptr() or dummy
     a.out = a.grad_out = a.grad_x = a.grad_y = a.grad_w = dummy
     return _lib.lib.cgtp_uvu_validate(C.byref(a), 1) == 0
@@ -195,11 +198,19 @@ def uvu_forward(cfg: int, dims, x: Tensor, y: Tensor, w: Tensor, seg: Optional[S
 
 
 def uvu_backward(cfg: int, dims, x: Tensor, y: Tensor, w: Tensor, g: Tensor, need, seg: Optional[SegIndex] = None,
-                 gather: Optional[Tensor] = None, pos_per_wave: int = 0):
-    """Compiled-table backward -> (grad_x, grad_y, grad_w), None where ``need`` is False."""
+                 gather: Optional[Tensor] = None, pos_per_wave: int = 0, x_gather: Optional[Tensor] = None):
+    """Compiled-table backward -> (grad_x, grad_y, grad_w), None where ``need`` is False.  Row mode: ``gather``
+    picks the row of ``g`` and ``x_gather`` the row of ``x`` of every batch row; with ``x_gather`` the returned
+    grad_x is per batch row, ``(n_rows, D1, C)``."""
     a = _uvu_args(cfg, x, y, w, seg, gather, pos_per_wave)
     a.grad_out = g.data_ptr()
-    gx = torch.empty_like(x) if need[0] else None
+    a.x_gather = _lib.ptr(x_gather)
+    if not need[0]:
+        gx = None
+    elif x_gather is not None:
+        gx = torch.empty((y.shape[0],) + x.shape[1:], dtype=x.dtype, device=x.device)
+    else:
+        gx = torch.empty_like(x)
     gy = torch.empty_like(y) if need[1] else None
     gw = torch.empty_like(w) if need[2] else None
     a.grad_x, a.grad_y, a.grad_w = _lib.ptr(gx), _lib.ptr(gy), _lib.ptr(gw)

@@ -184,6 +184,8 @@ typedef struct cgtp_uvu_args {
   void* grad_y;            /* (n_rows, D2) or NULL                                                 */
   void* grad_w;            /* (n_rows | 1, P, C) or NULL                                           */
   void* workspace;         /* cgtp_uvu_workspace_bytes() bytes (segment mode, or bwd of a shared W) */
+  const int64_t* x_gather; /* row mode backward, optional: [n_rows] row of x of every batch row (x then has
+                              n_x_rows rows; grad_x stays per batch row, (n_rows, D1, C))              */
 } cgtp_uvu_args;
 
 int cgtp_uvu_validate(const cgtp_uvu_args* args, int backward);

@@ -137,3 +137,65 @@ def test_edge_fused_range_modes(device, pos_per_wave, hub):
         assert plan.fwd_index.wave_seg is not None
     out_a = kernels.uvu_forward(cfg, dims, xd, shd, wd, seg=plan.fwd_index)
     assert_close(out_a, ref_out, 1e-5, "aligned out")
+
+
+SH6 = "0e+1o+2e+3o+4e+5o+6e"
+
+
+@pytest.mark.parametrize("channels", [32, 20, 64])
+def test_u1u_large_table_fp32(device, channels):
+    """lmax = 6 (106 paths, 6460 coefficients) on the large-table kernels: forward and all gradients, per-row
+    weights, against the dense float64 oracle."""
+    from equitorch_amd.ops import kernels
+    mod = _module(SH6, SH6, SH6).to(device)
+    cfg = kernels.uvu_config_of(mod.tp_info_forward)
+    assert cfg >= 0 and kernels.uvu_dims(cfg) == (49, 49, 49, 106, 6460)
+    n = 77
+    x, sh, w = tp_inputs(n, 49, 6, mod.num_paths, channels, False, seed=600 + channels)
+    ct = torch.randn(n, 49, channels, generator=torch.Generator().manual_seed(7))
+    assert kernels.uvu_launchable(cfg, x.to(device), sh.to(device), w.to(device))
+    got = _run(mod, x, sh, w, ct, device)
+    T = ref_ops.dense_coupling(SH6, SH6, SH6)
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1u, T, (x, sh, w), ct)
+    for name, g, r in zip(("out", "grad_x", "grad_sh", "grad_w"), got, (ref_out, *ref_grads)):
+        assert_close(g, r, 1e-5, f"lmax=6 C={channels} {name}")
+
+
+def test_u1u_large_table_shared_weight_uses_the_general_kernel(device):
+    """A shared weight's gradient is outside the large-table kernels: the product then runs on the table-driven
+    kernel, same results."""
+    mod = _module(SH6, SH6, SH6).to(device)
+    n, ch = 40, 16
+    x, sh, w = tp_inputs(n, 49, 6, mod.num_paths, ch, True, seed=66)
+    ct = torch.randn(n, 49, ch, generator=torch.Generator().manual_seed(7))
+    got = _run(mod, x, sh, w, ct, device)
+    T = ref_ops.dense_coupling(SH6, SH6, SH6)
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1u, T, (x, sh, w), ct)
+    for name, g, r in zip(("out", "grad_x", "grad_sh", "grad_w"), got, (ref_out, *ref_grads)):
+        assert_close(g, r, 1e-5, f"lmax=6 shared {name}")
+
+
+def test_edge_large_table(device):
+    """Edge message passing at lmax = 6, C = 32 (BASELINE configs[4] shapes, small graph): gathered row-mode
+    kernels plus segment sums against the dense oracle."""
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu
+    mod = _module(SH6, SH6, SH6).to(device)
+    gen = torch.Generator().manual_seed(15)
+    n_nodes, n_edges, ch = 41, 333, 32
+    src = torch.randint(0, n_nodes, (n_edges,), generator=gen)
+    dst = torch.randint(0, n_nodes - 2, (n_edges,), generator=gen)
+    x, sh, w = tp_inputs(n_edges, 49, 6, mod.num_paths, ch, False, seed=16)
+    x = x[:n_nodes].contiguous()
+    ct = torch.randn(n_nodes, 49, ch, generator=gen)
+    plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
+    xd, shd, wd = (t.to(device).requires_grad_(True) for t in (x, sh, w))
+    out = edge_tensor_product_uu(xd, shd, wd, plan, mod.tp_info_forward)
+    (out * ct.to(device)).sum().backward()
+    T = ref_ops.dense_coupling(SH6, SH6, SH6)
+
+    def ref_fn(T, x, sh, w):
+        return ref_ops.scatter_sum(ref_ops.dense_u1u(T, x.index_select(0, src), sh, w), dst, n_nodes)
+    ref_out, ref_grads = ref_ops.dense_grads(ref_fn, T, (x, sh, w), ct)
+    for name, g, r in zip(("out", "grad_x", "grad_sh", "grad_w"), (out, xd.grad, shd.grad, wd.grad),
+                          (ref_out, *ref_grads)):
+        assert_close(g, r, 1e-5, f"edge lmax=6 {name}")
