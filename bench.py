@@ -37,6 +37,8 @@ WORKLOADS = {
     # name: (lmax, channels, nodes, edges)
     "edge_fwd_bwd": (2, 64, 4096, 65536),
     "edge_fwd": (2, 64, 4096, 65536),
+    # BASELINE configs[4]: high-l channel-wise product, forward + backward, on the large-table kernels
+    "edge_l6_fwd_bwd": (6, 32, 20000, 200000),
     # fully connected product on the matrix cores (BASELINE configs[3]): (lmax, C_in = C_out, batch)
     "uvw_fwd": (3, 128, 32768),
     "uvw_fwd_bwd": (3, 128, 32768),
@@ -209,6 +211,88 @@ def algorithmic_bytes(n_nodes, n_edges, d, p, ch):
     return fwd, bwd
 
 
+FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X fp32, vendor figure
+
+
+def edge_rows_bench(args):
+    """BASELINE configs[4] (lmax = 6, C = 32, N = 20000, E = 200000, per-edge weights), forward + backward.  The
+    table (6460 coefficients) runs on the large-table row kernels: messages and per-edge input gradients go through
+    memory and are summed by the segment-sum kernel.  The arithmetic dominates here: about two vector instructions
+    per coefficient and channel, priced as 2 * (T + S1) * C flops per edge forward and three times that backward
+    (T coefficients, S1 = 826 (path, row) weight products)."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu
+    from equitorch_amd.ops import kernels
+    lmax, ch, n_nodes, n_edges = WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+    mod = SO3Linear(irreps, irreps, irreps, ch, ch, internal_weights=False, feature_mode="uu").to(dev)
+    p = mod.num_paths
+    n_rot = min(args.rotate, 2)
+    inp = make_inputs(lmax, ch, n_nodes, n_edges, n_rot, dev)
+    d = inp["d"]
+    plan = EdgePlan(inp["src"].to(dev), inp["dst"].to(dev), n_nodes)
+    x = inp["x"].to(dev).requires_grad_(True)
+    sh = inp["sh"].to(dev).requires_grad_(True)
+    ws = [torch.randn(n_edges, p, ch, generator=inp["gen"]).to(dev).requires_grad_(True) for _ in range(n_rot)]
+    ct = torch.randn(n_nodes, d, ch, generator=inp["gen"]).to(dev)
+
+    def step(i):
+        w = ws[i % n_rot]
+        out = edge_tensor_product_uu(x, sh, w, plan, mod.tp_info_forward)
+        return torch.autograd.grad(out, (x, sh, w), ct)
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) / args.steps * 1e3
+
+    cfg = kernels.uvu_config_of(mod.tp_info_forward)
+    dims = kernels.uvu_dims(cfg)
+    xd, shd = x.detach(), sh.detach()
+
+    def timed(fn):
+        evs = []
+        for i in range(max(3, args.kernel_reps // 3)):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            w = ws[i % n_rot].detach()
+            a.record(); fn(w); b.record()
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        return sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    fwd_ms = timed(lambda w: kernels.uvu_forward(cfg, dims, xd, shd, w, gather=plan.src))
+    bwd_ms = timed(lambda w: kernels.uvu_backward(cfg, dims, xd, shd, w, ct, (True, True, True), gather=plan.dst,
+                                                  x_gather=plan.src))
+    nnz, s1 = dims[4], int(mod.tp_info_forward.info_Mij_fwd.out_size)
+    flops_fwd = 2.0 * (nnz + s1) * ch * n_edges
+    fwd_bytes, bwd_bytes = algorithmic_bytes(n_nodes, n_edges, d, p, ch)
+    msg = n_edges * d * ch * 4  # the unfused path also writes the per-edge rows once
+    tf = 3 * flops_fwd / (bwd_ms * 1e-3) / 1e12
+    gbs = (bwd_bytes + msg) / (bwd_ms * 1e-3) / 1e9
+    rec = {
+        "metric": "edge-TP fwd+bwd Medges/s (lmax=6,C=32)", "value": round(n_edges / (ms_step * 1e-3) / 1e6, 2),
+        "unit": "Medges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: N={n_nodes} nodes, E={n_edges} edges, irreps {irreps}, C={ch}, "
+                               f"per-edge weights (E,{p},{ch}), {n_rot} rotating weight buffers"},
+        "roofline": {"bound": "hbm", "kernel": "cgtp::uvu_big_bwd_kernel<TPB_sh6,1>", "achieved": round(gbs, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes": bwd_bytes + msg, "avg_ms": round(bwd_ms, 4),
+                     "fp32_vector": {"achieved": round(tf, 2), "peak": FP32_VECTOR_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                     "frac": round(tf / FP32_VECTOR_PEAK_TFLOPS, 4),
+                                     "algorithmic_flops": 3 * flops_fwd}},
+        "kernels": {"fwd_ms": round(fwd_ms, 4), "bwd_ms": round(bwd_ms, 4),
+                    "fwd_TFLOPs": round(flops_fwd / (fwd_ms * 1e-3) / 1e12, 2),
+                    "fwd_GBs": round((fwd_bytes + msg) / (fwd_ms * 1e-3) / 1e9, 1)},
+    }
+    if not args.no_cpu_baseline:
+        rec["cpu_baseline"] = cpu_baseline(inp, lmax, ch, n_nodes, min(args.cpu_sample_edges, 1024))
+    print(json.dumps(rec))
+
+
 def cpu_baseline(inp, lmax, ch, n_nodes, sample_edges, budget_s=12.0):
     """The oracle's step-for-step restatement of the reference's CPU path (index_select -> product -> scale ->
     CSR segment-sum; forward and backward), timed on the first ``sample_edges`` edges of the same graph."""
@@ -272,6 +356,9 @@ def main():
         return
     if args.workload in ("uvw_fwd", "uvw_fwd_bwd"):
         uvw_bench(args)
+        return
+    if args.workload == "edge_l6_fwd_bwd":
+        edge_rows_bench(args)
         return
 
     from equitorch_amd.nn import SO3Linear

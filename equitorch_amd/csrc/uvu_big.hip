@@ -37,7 +37,7 @@ __global__ void __launch_bounds__(256, 2) uvu_big_fwd_kernel(const UvuDev<float>
 }
 
 template <class TP, int GW>
-__global__ void __launch_bounds__(256, 1) uvu_big_bwd_kernel(const UvuDev<float> a, int64_t n_waves) {
+__global__ void __launch_bounds__(256, 2) uvu_big_bwd_kernel(const UvuDev<float> a, int64_t n_waves) {
   constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
   const Lanes L(a.lpe_log2);
   const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
