@@ -227,8 +227,13 @@ __global__ void __launch_bounds__(256, 1) uv_gw_kernel(const __bf16* __restrict_
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int D1 = CFG::D1, DO = CFG::DO, D2 = CFG::D2, P = CFG::P;
   // the same for every lane: keep them in scalar registers so that the switch over paths is a scalar branch
-  const int p = __builtin_amdgcn_readfirstlane(meta.order[blockIdx.x % P]);
-  const int64_t c = blockIdx.x / P;
+  // Workgroups are dealt to the 8 XCDs round-robin by index.  The P workgroups of one chunk of samples read the same
+  // rows of x and g, so they are given indices that land on one XCD (one L2): index = 8 * slot + xcd, chunk =
+  // 8 * (slot / P) + xcd, path = order[slot % P].
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int p = __builtin_amdgcn_readfirstlane(meta.order[slot % P]);
+  const int64_t c = (int64_t)(slot / P) * 8 + xcd;
+  if (c * kGwChunk >= n_rows) return;
   const int a0 = __builtin_amdgcn_readfirstlane(meta.a0[p]), na = __builtin_amdgcn_readfirstlane(meta.na[p]);
   const int pu = cin * 2 + kGwPad, pw = cout * 2 + kGwPad;   // tile row pitches
   unsigned char* xt = smem;                           // [na][32][pu]  rows of x
@@ -569,7 +574,8 @@ int cgtp_uv_grad_w(int cfg, const void* x, const void* y, const void* g, void* g
   if (hipFuncSetAttribute((const void*)e.gw_fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
     return CGTP_ERR_LDS;
   const int64_t n_chunks = (n_rows + kGwChunk - 1) / kGwChunk;
-  hipLaunchKernelGGL(e.gw_fn, dim3((unsigned)(n_chunks * e.p)), dim3(256), (size_t)lds, st, (const __bf16*)x,
+  const int64_t n_chunks8 = (n_chunks + 7) / 8 * 8;  // whole rounds over the XCDs; the surplus workgroups exit
+  hipLaunchKernelGGL(e.gw_fn, dim3((unsigned)(n_chunks8 * e.p)), dim3(256), (size_t)lds, st, (const __bf16*)x,
                      (const __bf16*)y, (const __bf16*)g, (float*)workspace, n_rows, (int)cin, (int)cout, e.gw_meta);
   hipLaunchKernelGGL(uv_gw_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, st,
                      (const float*)workspace, (__bf16*)gw, n_chunks, n_out);
