@@ -29,6 +29,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 RING = 8
 
 CONFIGS = OrderedDict([
+    ("sh4", (_sh(4), _sh(4), _sh(4), {})),
+    ("sh5", (_sh(5), _sh(5), _sh(5), {})),
     ("sh6", (_sh(6), _sh(6), _sh(6), {})),
 ])
 

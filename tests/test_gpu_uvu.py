@@ -142,23 +142,27 @@ def test_edge_fused_range_modes(device, pos_per_wave, hub):
 SH6 = "0e+1o+2e+3o+4e+5o+6e"
 
 
-@pytest.mark.parametrize("channels", [32, 20, 64])
-def test_u1u_large_table_fp32(device, channels):
-    """lmax = 6 (106 paths, 6460 coefficients) on the large-table kernels: forward and all gradients, per-row
-    weights, against the dense float64 oracle."""
+@pytest.mark.parametrize("lmax,channels", [(6, 32), (6, 20), (6, 64), (4, 48), (5, 32)])
+def test_u1u_large_table_fp32(device, lmax, channels):
+    """lmax = 4..6 (lmax = 6: 106 paths, 6460 coefficients) on the large-table kernels: forward and all gradients,
+    per-row weights, against the dense float64 oracle."""
     from equitorch_amd.ops import kernels
-    mod = _module(SH6, SH6, SH6).to(device)
+    irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+    d = (lmax + 1) ** 2
+    mod = _module(irreps, irreps, irreps).to(device)
     cfg = kernels.uvu_config_of(mod.tp_info_forward)
-    assert cfg >= 0 and kernels.uvu_dims(cfg) == (49, 49, 49, 106, 6460)
+    assert cfg >= 0 and kernels.uvu_dims(cfg)[:4] == (d, d, d, mod.num_paths)
+    if lmax == 6:
+        assert kernels.uvu_dims(cfg) == (49, 49, 49, 106, 6460)
     n = 77
-    x, sh, w = tp_inputs(n, 49, 6, mod.num_paths, channels, False, seed=600 + channels)
-    ct = torch.randn(n, 49, channels, generator=torch.Generator().manual_seed(7))
+    x, sh, w = tp_inputs(n, d, lmax, mod.num_paths, channels, False, seed=100 * lmax + channels)
+    ct = torch.randn(n, d, channels, generator=torch.Generator().manual_seed(7))
     assert kernels.uvu_launchable(cfg, x.to(device), sh.to(device), w.to(device))
     got = _run(mod, x, sh, w, ct, device)
-    T = ref_ops.dense_coupling(SH6, SH6, SH6)
+    T = ref_ops.dense_coupling(irreps, irreps, irreps)
     ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1u, T, (x, sh, w), ct)
     for name, g, r in zip(("out", "grad_x", "grad_sh", "grad_w"), got, (ref_out, *ref_grads)):
-        assert_close(g, r, 1e-5, f"lmax=6 C={channels} {name}")
+        assert_close(g, r, 1e-5, f"lmax={lmax} C={channels} {name}")
 
 
 def test_u1u_large_table_shared_weight_uses_the_general_kernel(device):
