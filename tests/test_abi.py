@@ -87,6 +87,42 @@ def test_host_side_validation_codes():
     assert L.cgtp_membench_copy(256, 256, 17, None) == 2
 
 
+def test_large_table_configs_and_row_gathers_validate_on_the_host():
+    """lmax = 4..6 tables are served by the large-table kernels: fp32, row mode, no shared-weight gradient; the
+    row-mode backward accepts a separate gather for the rows of x."""
+    from equitorch_amd import _lib
+    from equitorch_amd._tables import fingerprint, tp_coo
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    L = _lib.lib
+    sh6 = "0e+1o+2e+3o+4e+5o+6e"
+    coo = tp_coo(tp_infos(Irreps(sh6), Irreps(sh6), Irreps(sh6))[0])
+    cfg = L.cgtp_uvu_find(C.c_uint64(fingerprint(coo)))
+    assert 0 <= cfg < L.cgtp_uvu_num_configs()
+    dims = (C.c_int32 * 5)()
+    assert L.cgtp_uvu_describe(cfg, dims) == fingerprint(coo) and tuple(dims) == (49, 49, 49, 106, 6460)
+    a = _lib.UvuArgs()
+    a.cfg, a.dtype, a.C, a.n_rows, a.n_x_rows = cfg, _lib.F32, 32, 10, 10
+    a.x = a.y = a.w = a.out = a.grad_out = a.grad_x = a.grad_y = a.grad_w = 4096
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 0 and L.cgtp_uvu_validate(C.byref(a), 1) == 0
+    assert L.cgtp_uvu_workspace_bytes(C.byref(a), 1) == 0
+    a.dtype = _lib.F64
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 4                  # fp32 only
+    a.dtype, a.w_shared = _lib.F32, 1
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 0                  # shared weight forward is fine
+    assert L.cgtp_uvu_validate(C.byref(a), 1) == 2                  # ... its gradient is not covered
+    a.grad_w = None
+    assert L.cgtp_uvu_validate(C.byref(a), 1) == 0
+    a.w_shared, a.grad_w, a.n_seg, a.ptr, a.seg_ids, a.gather = 0, 4096, 10, 4096, 4096, 4096
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 2                  # no segment mode
+    # row-mode backward with gathered x rows: x may then have any number of rows
+    a.n_seg, a.ptr, a.seg_ids = 0, None, None
+    a.n_x_rows = 4
+    assert L.cgtp_uvu_validate(C.byref(a), 1) == 2
+    a.x_gather = 4096
+    assert L.cgtp_uvu_validate(C.byref(a), 1) == 0
+
+
 def test_uv_matrix_core_entry_points_validate_on_the_host():
     """cgtp_uv_*: config lookup by fingerprint and argument checks, no launch (n_rows = 0 or a failing check)."""
     from equitorch_amd import _lib
