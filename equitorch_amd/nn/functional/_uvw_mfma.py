@@ -18,23 +18,24 @@ def uv_config_of(tp_info) -> int:
                           lambda: int(_lib.lib.cgtp_uv_find(C.c_uint64(fingerprint(kernels.coo_of(tp_info))))))
 
 
-_packed = {}  # (id(w), direction) -> (weakref to w, its version counter, packed copy)
+_packed = {}  # (id(w), direction) -> (weakref to w, its version counter, its data pointer, packed copy)
 
 
 def pack_weights(direction: int, w: Tensor) -> Tensor:
     """W as stored by the module, (P, C_in, C_out), rewritten in the fragment order the kernel reads.  The packed
-    copy is kept until the weight tensor is modified in place (its version counter moves) or dies."""
+    copy is kept until the weight tensor is modified in place (its version counter moves), is given other storage,
+    or dies."""
     key = (id(w), direction)
     hit = _packed.get(key)
-    if hit is not None and hit[0]() is w and hit[1] == w._version:
-        return hit[2]
+    if hit is not None and hit[0]() is w and hit[1] == w._version and hit[2] == w.data_ptr():
+        return hit[3]
     packed = _pack(direction, w)
     if len(_packed) >= 64:
         for k in [k for k, v in _packed.items() if v[0]() is None]:
             del _packed[k]
         if len(_packed) >= 64:
             _packed.clear()
-    _packed[key] = (weakref.ref(w), w._version, packed)
+    _packed[key] = (weakref.ref(w), w._version, w.data_ptr(), packed)
     return packed
 
 
