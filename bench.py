@@ -45,7 +45,32 @@ WORKLOADS = {
     # streaming kernels of known traffic (1 GiB): counter calibration and achievable-bandwidth reference
     "copy": None,
     "read": None,
+    # plain library GEMM (torch.matmul, bf16, 8192^3): the matrix rate the box reaches, next to the vendor peak
+    "gemm": None,
 }
+
+
+def gemm_bench(steps, warmup):
+    """bf16 8192 x 8192 x 8192 torch.matmul (hipBLASLt): achievable dense matrix rate on this box."""
+    dev = torch.device("cuda:0")
+    n = 8192
+    a = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
+    b = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
+    for _ in range(warmup):
+        a @ b
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        a @ b
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    tf = 2.0 * n ** 3 / (ms * 1e-3) / 1e12
+    print(json.dumps({"metric": "bf16 GEMM TFLOP/s (8192^3, torch.matmul)", "value": round(tf, 1), "unit": "TFLOP/s",
+                      "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 4),
+                      "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+                      "data": "synthetic", "config": {"workload": "gemm: library GEMM, calibration of the MFMA peak"},
+                      "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
+                                   "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None}}))
 
 
 def membench(kind, steps, warmup):
@@ -330,7 +355,19 @@ def cpu_baseline(inp, lmax, ch, n_nodes, sample_edges, budget_s=12.0):
     med = sorted(times)[len(times) // 2]
     return {"value": round(e / med / 1e6, 4), "unit": "Medges/s", "cores": threads, "kind": "port",
             "sample": f"first {e} of {inp['src'].shape[0]} edges of the same graph, fwd+bwd, median of {iters} "
-                      f"runs, {med * 1e3:.1f} ms/run, torch {torch.__version__} CPU ops"}
+                      f"runs, {med * 1e3:.1f} ms/run, torch {torch.__version__} CPU ops, {threads} threads on "
+                      f"{cpu_model()} ({os.cpu_count()} logical CPUs)"}
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown CPU"
 
 
 def main():
@@ -353,6 +390,9 @@ def main():
 
     if args.workload in ("copy", "read"):
         membench(args.workload, args.steps, args.warmup)
+        return
+    if args.workload == "gemm":
+        gemm_bench(args.steps, args.warmup)
         return
     if args.workload in ("uvw_fwd", "uvw_fwd_bwd"):
         uvw_bench(args)
