@@ -1,5 +1,6 @@
-"""Emits ``generated/uvu_big_configs.inc``: the channel-wise tensor product for configurations whose table is too
-large for the register-resident bodies of ``gen_uvu`` (hundreds of weight rows, thousands of coefficients).
+"""Emits ``generated/uvu_big_configs.inc``: the channel-wise tensor product, one channel per lane, for row-mode
+launches of every registered configuration and for configurations whose table is too large for the
+register-resident bodies of ``gen_uvu`` (hundreds of weight rows, thousands of coefficients).
 
 One lane owns one channel.  The bodies walk the table output irrep by output irrep (only the 2l+1 rows of that
 irrep are live as accumulators or gradient rows) and inside an irrep path by path.  A path's weight is a single
@@ -29,9 +30,13 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 RING = 8
 
 CONFIGS = OrderedDict([
+    ("sh1", (_sh(1), _sh(1), _sh(1), {})),
+    ("sh2", (_sh(2), _sh(2), _sh(2), {})),
+    ("sh3", (_sh(3), _sh(3), _sh(3), {})),
     ("sh4", (_sh(4), _sh(4), _sh(4), {})),
     ("sh5", (_sh(5), _sh(5), _sh(5), {})),
     ("sh6", (_sh(6), _sh(6), _sh(6), {})),
+    ("so3_012_to_0123", ("0e+1e+2e+3e", "0e+1e+2e", "0e+1e+2e", {})),
 ])
 
 

@@ -393,6 +393,7 @@ __global__ void __launch_bounds__(256) uvu_fixup_kernel(T* __restrict__ rows, co
 // ---- host side ----------------------------------------------------------------------------------------------
 struct UvuPlan {
   int V, lpe_log2, pos_per_wave;
+  int big_idx;        // >= 0: entry of the block-wise kernels that runs this launch
   int64_t n_waves;    // wavefronts of the main kernel
   int64_t ws_elems;   // segment mode: elements of partial rows at the start of the workspace
   int64_t wsw_elems;  // elements of shared-weight-gradient partials after them
@@ -476,14 +477,26 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
   const UvuEntry<float>* tab = entries<float>(&n_cfg);
   const UvuBigEntry* big_tab = uvu_big_entries(&n_big);
   if (a->cfg < 0 || a->cfg >= n_cfg + n_big) return CGTP_ERR_CONFIG;
-  const bool big = a->cfg >= n_cfg;  // large-table configurations follow the register-resident ones
-  const int* dims = big ? big_tab[a->cfg - n_cfg].dims : tab[a->cfg].dims;
+  const bool seg_mode = a->n_seg > 0;
+  // The block-wise kernels (one channel per lane) serve the configurations that have no register-resident body
+  // (indices n_cfg and up) and, because they are faster there, every fp32 row-mode launch of the others except
+  // the gradient of a shared weight and backward launches wider than one wavefront (C > 64).
+  int big_idx = a->cfg >= n_cfg ? a->cfg - n_cfg : -1;
+  if (big_idx < 0 && a->dtype == CGTP_F32 && !seg_mode && !(backward && a->w_shared && a->grad_w) &&
+      !(backward && a->C > kWave)) {
+    for (int i = 0; i < n_big; ++i)
+      if (big_tab[i].fingerprint == tab[a->cfg].fingerprint) big_idx = i;
+  }
+  const bool big = big_idx >= 0;
+  plan->big_idx = big_idx;
+  const int* dims = big ? big_tab[big_idx].dims : tab[a->cfg].dims;
   if (a->dtype != CGTP_F32 && a->dtype != CGTP_F64) return CGTP_ERR_DTYPE;
-  if (big && a->dtype != CGTP_F32) return CGTP_ERR_DTYPE;
+  if (a->cfg >= n_cfg && a->dtype != CGTP_F32) return CGTP_ERR_DTYPE;
   if (a->C <= 0 || a->n_rows < 0 || a->n_seg < 0 || a->n_x_rows < 0 || a->pos_per_wave < 0) return CGTP_ERR_SHAPE;
   if (!a->x || !a->y || !a->w) return CGTP_ERR_NULL;
   const bool seg = a->n_seg > 0;
-  if (big && (seg || (backward && a->w_shared && a->grad_w))) return CGTP_ERR_SHAPE;  // row mode, per-row weight gradient
+  if (a->cfg >= n_cfg && (seg || (backward && a->w_shared && a->grad_w)))
+    return CGTP_ERR_SHAPE;  // block-wise kernels only: row mode, per-row weight gradient
   if (seg && (!a->ptr || !a->seg_ids || !a->gather)) return CGTP_ERR_NULL;
   if (!seg && (a->ptr || a->perm || a->seg_ids)) return CGTP_ERR_SHAPE;
   if (seg && (a->n_seg >= (int64_t)1 << 31 || a->n_rows >= (int64_t)1 << 31 || a->n_x_rows >= (int64_t)1 << 31))
@@ -569,9 +582,8 @@ static int launch_fixup(T* rows, const UvuDev<T>& d, int64_t row_len, hipStream_
 }
 
 static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward, hipStream_t stream) {
-  int n = 0, n_big = 0;
-  entries<float>(&n);
-  const UvuBigEntry& e = uvu_big_entries(&n_big)[a->cfg - n];
+  int n_big = 0;
+  const UvuBigEntry& e = uvu_big_entries(&n_big)[plan.big_idx];
   if (plan.n_waves == 0) return CGTP_OK;
   const UvuDev<float> d = to_dev<float>(a, plan);
   if (backward) {
@@ -583,12 +595,6 @@ static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward,
     hipLaunchKernelGGL(e.fwd, grid, dim3(256), 0, stream, d);
   }
   return launched();
-}
-
-static bool is_big(int cfg) {
-  int n = 0;
-  entries<float>(&n);
-  return cfg >= n;
 }
 
 template <typename T>
@@ -654,9 +660,9 @@ int cgtp_uvu_num_configs(void) {
 int cgtp_uvu_find(uint64_t fingerprint) {
   int n = 0, n_big = 0;
   const UvuEntry<float>* t = entries<float>(&n);
+  const UvuBigEntry* b = uvu_big_entries(&n_big);
   for (int i = 0; i < n; ++i)
     if (t[i].fingerprint == fingerprint) return i;
-  const UvuBigEntry* b = uvu_big_entries(&n_big);
   for (int i = 0; i < n_big; ++i)
     if (b[i].fingerprint == fingerprint) return n + i;
   return -1;
@@ -688,7 +694,7 @@ int cgtp_uvu_fwd(const cgtp_uvu_args* a, void* stream) {
   UvuPlan plan;
   const int st = uvu_plan(a, 0, true, &plan);
   if (st != CGTP_OK) return st;
-  if (is_big(a->cfg)) return launch_big(a, plan, 0, (hipStream_t)stream);
+  if (plan.big_idx >= 0) return launch_big(a, plan, 0, (hipStream_t)stream);
   return a->dtype == CGTP_F32 ? launch_fwd<float>(a, plan, (hipStream_t)stream)
                               : launch_fwd<double>(a, plan, (hipStream_t)stream);
 }
@@ -697,7 +703,7 @@ int cgtp_uvu_bwd(const cgtp_uvu_args* a, void* stream) {
   UvuPlan plan;
   const int st = uvu_plan(a, 1, true, &plan);
   if (st != CGTP_OK) return st;
-  if (is_big(a->cfg)) return launch_big(a, plan, 1, (hipStream_t)stream);
+  if (plan.big_idx >= 0) return launch_big(a, plan, 1, (hipStream_t)stream);
   return a->dtype == CGTP_F32 ? launch_bwd<float>(a, plan, (hipStream_t)stream)
                               : launch_bwd<double>(a, plan, (hipStream_t)stream);
 }
