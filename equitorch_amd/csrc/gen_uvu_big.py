@@ -37,7 +37,25 @@ CONFIGS = OrderedDict([
     ("sh5", (_sh(5), _sh(5), _sh(5), {})),
     ("sh6", (_sh(6), _sh(6), _sh(6), {})),
     ("so3_012_to_0123", ("0e+1e+2e+3e", "0e+1e+2e", "0e+1e+2e", {})),
+    ("so3_2", ("0e+1e+2e", "0e+1e+2e", "0e+1e+2e", {})),
+    ("so3_3", ("0e+1e+2e+3e", "0e+1e+2e+3e", "0e+1e+2e+3e", {})),
 ])
+
+
+def extra_configs() -> OrderedDict:
+    """Configurations a user registers in ``extra_uvu_configs.json`` next to this file:
+    ``{"name": ["irreps_out", "irreps_in1", "irreps_in2"], ...}`` (names: C identifiers).  They are compiled into the
+    library by the next build like the ones above."""
+    import json
+    path = os.path.join(HERE, "extra_uvu_configs.json")
+    out = OrderedDict()
+    if os.path.exists(path):
+        with open(path) as f:
+            for name, (io, i1, i2) in json.load(f).items():
+                if not name.isidentifier():
+                    raise ValueError(f"{path}: configuration name {name!r} is not an identifier")
+                out[name] = (io, i1, i2, {})
+    return out
 
 
 def _pin(names) -> str:
@@ -175,13 +193,20 @@ def main(out_dir: str = None) -> str:
     out_dir = out_dir or os.path.join(HERE, "generated")
     os.makedirs(out_dir, exist_ok=True)
     chunks = ["// Generated by equitorch_amd/csrc/gen_uvu_big.py; do not edit.", ""]
-    for name, (io, i1, i2, kw) in CONFIGS.items():
+    configs = OrderedDict(CONFIGS)
+    configs.update(extra_configs())
+    seen = {}
+    for name, (io, i1, i2, kw) in configs.items():
         coo = tp_coo(tp_infos(Irreps(io), Irreps(i1), Irreps(i2), **kw)[0])
+        fp = fingerprint(coo)
+        if fp in seen:
+            raise ValueError(f"configuration {name} has the same table as {seen[fp]}")
+        seen[fp] = name
         chunks.append(f"// {name}: {i1} x {i2} -> {io}")
         chunks.append(emit_config(name, coo, irrep_segments(Irreps(io))))
         chunks.append("")
     chunks.append("#define CGTP_FOREACH_UVU_BIG_CONFIG(X) \\")
-    chunks.append(" \\\n".join(f"  X(TPB_{n})" for n in CONFIGS))
+    chunks.append(" \\\n".join(f"  X(TPB_{n})" for n in configs))
     chunks.append("")
     path = os.path.join(out_dir, "uvu_big_configs.inc")
     text = "\n".join(chunks)

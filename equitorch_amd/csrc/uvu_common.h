@@ -44,8 +44,8 @@ struct Lanes {
 // (partial_sum_kernel finishes the sum).  A compile-time choice keeps the generated body free of branches.
 enum { kGwNone = 0, kGwStore = 1, kGwReduce = 2 };
 
-// Configurations too large for the register-resident bodies (uvu_big.hip): fp32, row mode, one channel per lane,
-// per-row weights or no weight gradient.
+// Block-wise kernels (uvu_big.hip): fp32, row mode, one channel per lane.  They write the weight gradient per row;
+// for a shared weight the caller sums the rows.
 struct UvuBigEntry {
   uint64_t fingerprint;
   int dims[5];

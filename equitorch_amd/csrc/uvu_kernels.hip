@@ -470,6 +470,7 @@ static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t
 
 static constexpr int64_t kMaxRowWaves = 2048;
 static constexpr int kDefaultPosPerWave = 32;
+static constexpr int kBigSumRows = 256;  // rows per first-pass chunk of the shared-weight gradient sum
 
 static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan* plan) {
   if (!a) return CGTP_ERR_NULL;
@@ -480,10 +481,9 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
   const bool seg_mode = a->n_seg > 0;
   // The block-wise kernels (one channel per lane) serve the configurations that have no register-resident body
   // (indices n_cfg and up) and, because they are faster there, every fp32 row-mode launch of the others except
-  // the gradient of a shared weight and backward launches wider than one wavefront (C > 64).
+  // backward launches wider than one wavefront (C > 64).
   int big_idx = a->cfg >= n_cfg ? a->cfg - n_cfg : -1;
-  if (big_idx < 0 && a->dtype == CGTP_F32 && !seg_mode && !(backward && a->w_shared && a->grad_w) &&
-      !(backward && a->C > kWave)) {
+  if (big_idx < 0 && a->dtype == CGTP_F32 && !seg_mode && !(backward && a->C > kWave)) {
     for (int i = 0; i < n_big; ++i)
       if (big_tab[i].fingerprint == tab[a->cfg].fingerprint) big_idx = i;
   }
@@ -495,8 +495,7 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
   if (a->C <= 0 || a->n_rows < 0 || a->n_seg < 0 || a->n_x_rows < 0 || a->pos_per_wave < 0) return CGTP_ERR_SHAPE;
   if (!a->x || !a->y || !a->w) return CGTP_ERR_NULL;
   const bool seg = a->n_seg > 0;
-  if (a->cfg >= n_cfg && (seg || (backward && a->w_shared && a->grad_w)))
-    return CGTP_ERR_SHAPE;  // block-wise kernels only: row mode, per-row weight gradient
+  if (a->cfg >= n_cfg && seg) return CGTP_ERR_SHAPE;  // block-wise kernels only: row mode
   if (seg && (!a->ptr || !a->seg_ids || !a->gather)) return CGTP_ERR_NULL;
   if (!seg && (a->ptr || a->perm || a->seg_ids)) return CGTP_ERR_SHAPE;
   if (seg && (a->n_seg >= (int64_t)1 << 31 || a->n_rows >= (int64_t)1 << 31 || a->n_x_rows >= (int64_t)1 << 31))
@@ -554,7 +553,14 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
     if (wred && nw > kMaxRowWaves) nw = kMaxRowWaves;
     plan->n_waves = nw;
   }
-  if (wred) plan->wsw_elems = plan->n_waves * dims[3] * a->C;
+  if (wred && big) {
+    // block-wise kernels write the weight gradient of every row; two summation passes follow (kBigSumRows rows
+    // each, then the partials)
+    const int64_t chunks = (a->n_rows + kBigSumRows - 1) / kBigSumRows;
+    plan->wsw_elems = (a->n_rows + chunks) * dims[3] * a->C;
+  } else if (wred) {
+    plan->wsw_elems = plan->n_waves * dims[3] * a->C;
+  }
   if (need_ws && plan->ws_elems + plan->wsw_elems > 0 && !a->workspace) return CGTP_ERR_WORKSPACE;
   return CGTP_OK;
 }
@@ -581,14 +587,41 @@ static int launch_fixup(T* rows, const UvuDev<T>& d, int64_t row_len, hipStream_
   return launched();
 }
 
+// part[c * n + i] = sum of rows[r * n + i] over the rows r of chunk c (kBigSumRows rows), in row order.
+__global__ void __launch_bounds__(256) rows_sum_kernel(const float* __restrict__ rows, float* __restrict__ part,
+                                                       int64_t n_rows, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int64_t r0 = (int64_t)blockIdx.y * kBigSumRows, r1 = r0 + kBigSumRows < n_rows ? r0 + kBigSumRows : n_rows;
+  float s = 0.f;
+  for (int64_t r = r0; r < r1; ++r) s += rows[r * n + i];
+  part[blockIdx.y * n + i] = s;
+}
+
 static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward, hipStream_t stream) {
   int n_big = 0;
   const UvuBigEntry& e = uvu_big_entries(&n_big)[plan.big_idx];
-  if (plan.n_waves == 0) return CGTP_OK;
-  const UvuDev<float> d = to_dev<float>(a, plan);
+  const bool wred = backward && a->w_shared && a->grad_w;
+  const int64_t w_elems = (int64_t)e.dims[3] * a->C;
+  if (plan.n_waves == 0) {
+    if (wred) (void)hipMemsetAsync(a->grad_w, 0, sizeof(float) * w_elems, stream);
+    return CGTP_OK;
+  }
+  UvuDev<float> d = to_dev<float>(a, plan);
   if (backward) {
+    if (wred) d.gw = d.wsw;  // per-row gradients into the workspace, summed below
     hipLaunchKernelGGL(e.bwd[a->grad_w ? kGwStore : kGwNone], dim3((unsigned)((plan.n_waves + 3) / 4)), dim3(256), 0,
                        stream, d, plan.n_waves);
+    if (wred) {
+      if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
+      const int64_t chunks = (a->n_rows + kBigSumRows - 1) / kBigSumRows;
+      float* part = d.wsw + a->n_rows * w_elems;
+      hipLaunchKernelGGL(rows_sum_kernel, dim3((unsigned)((w_elems + 255) / 256), (unsigned)chunks), dim3(256), 0, stream,
+                         (const float*)d.wsw, part, a->n_rows, w_elems);
+      if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
+      hipLaunchKernelGGL(partial_sum_kernel<float>, dim3((unsigned)((w_elems + 255) / 256)), dim3(256), 0, stream,
+                         (const float*)part, (float*)a->grad_w, chunks, w_elems);
+    }
   } else {
     const int chunk = 1 << plan.lpe_log2;
     dim3 grid((unsigned)((plan.n_waves + 3) / 4), (unsigned)((a->C + chunk - 1) / chunk));

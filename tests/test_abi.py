@@ -71,7 +71,11 @@ def test_host_side_validation_codes():
     a.grad_out = 256
     assert L.cgtp_uvu_validate(C.byref(a), 1) == 2                  # backward keeps a row inside one wavefront
     a.C, a.w_shared, a.grad_w = 64, 1, 256
-    assert L.cgtp_uvu_workspace_bytes(C.byref(a), 1) == 3 * 11 * 64 * 4   # 10 rows / 4 slots = 3 partial rows
+    # fp32 row mode runs on the block-wise kernels: 10 per-row weight gradients + 1 chunk partial of (P, C)
+    assert L.cgtp_uvu_workspace_bytes(C.byref(a), 1) == (10 + 1) * 11 * 64 * 4
+    a.dtype = _lib.F64
+    assert L.cgtp_uvu_workspace_bytes(C.byref(a), 1) == 5 * 11 * 64 * 8   # fp64: 10 rows / 2 slots = 5 partial rows
+    a.dtype = _lib.F32
     assert L.cgtp_uvu_bwd(C.byref(a), None) == 8                    # CGTP_ERR_WORKSPACE, nothing launched
 
     t = _lib.TriArgs()
@@ -88,8 +92,8 @@ def test_host_side_validation_codes():
 
 
 def test_large_table_configs_and_row_gathers_validate_on_the_host():
-    """lmax = 4..6 tables are served by the large-table kernels: fp32, row mode, no shared-weight gradient; the
-    row-mode backward accepts a separate gather for the rows of x."""
+    """lmax = 4..6 tables are served by the block-wise kernels only: fp32, row mode; a shared weight's gradient goes
+    through per-row gradients in the workspace.  The row-mode backward accepts a separate gather for the rows of x."""
     from equitorch_amd import _lib
     from equitorch_amd._tables import fingerprint, tp_coo
     from equitorch_amd.irreps import Irreps
@@ -109,10 +113,10 @@ def test_large_table_configs_and_row_gathers_validate_on_the_host():
     a.dtype = _lib.F64
     assert L.cgtp_uvu_validate(C.byref(a), 0) == 4                  # fp32 only
     a.dtype, a.w_shared = _lib.F32, 1
-    assert L.cgtp_uvu_validate(C.byref(a), 0) == 0                  # shared weight forward is fine
-    assert L.cgtp_uvu_validate(C.byref(a), 1) == 2                  # ... its gradient is not covered
-    a.grad_w = None
-    assert L.cgtp_uvu_validate(C.byref(a), 1) == 0
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 0 and L.cgtp_uvu_validate(C.byref(a), 1) == 0
+    # shared weight: 10 per-row gradients + 1 chunk partial of (P, C) floats
+    assert L.cgtp_uvu_workspace_bytes(C.byref(a), 1) == (10 + 1) * 106 * 32 * 4
+    assert L.cgtp_uvu_bwd(C.byref(a), None) == 8                    # workspace missing, nothing launched
     a.w_shared, a.grad_w, a.n_seg, a.ptr, a.seg_ids, a.gather = 0, 4096, 10, 4096, 4096, 4096
     assert L.cgtp_uvu_validate(C.byref(a), 0) == 2                  # no segment mode
     # row-mode backward with gathered x rows: x may then have any number of rows

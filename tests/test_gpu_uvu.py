@@ -165,18 +165,20 @@ def test_u1u_large_table_fp32(device, lmax, channels):
         assert_close(g, r, 1e-5, f"lmax={lmax} C={channels} {name}")
 
 
-def test_u1u_large_table_shared_weight_uses_the_general_kernel(device):
-    """A shared weight's gradient is outside the large-table kernels: the product then runs on the table-driven
-    kernel, same results."""
-    mod = _module(SH6, SH6, SH6).to(device)
-    n, ch = 40, 16
-    x, sh, w = tp_inputs(n, 49, 6, mod.num_paths, ch, True, seed=66)
-    ct = torch.randn(n, 49, ch, generator=torch.Generator().manual_seed(7))
+@pytest.mark.parametrize("lmax,n,ch", [(6, 40, 16), (4, 700, 32), (2, 300, 64)])
+def test_u1u_block_wise_shared_weight(device, lmax, n, ch):
+    """Shared weight on the block-wise kernels: its gradient is written per row and summed in two fixed-order
+    passes (700 rows: three first-pass chunks)."""
+    irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+    d = (lmax + 1) ** 2
+    mod = _module(irreps, irreps, irreps).to(device)
+    x, sh, w = tp_inputs(n, d, lmax, mod.num_paths, ch, True, seed=66 + lmax)
+    ct = torch.randn(n, d, ch, generator=torch.Generator().manual_seed(7))
     got = _run(mod, x, sh, w, ct, device)
-    T = ref_ops.dense_coupling(SH6, SH6, SH6)
+    T = ref_ops.dense_coupling(irreps, irreps, irreps)
     ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1u, T, (x, sh, w), ct)
     for name, g, r in zip(("out", "grad_x", "grad_sh", "grad_w"), got, (ref_out, *ref_grads)):
-        assert_close(g, r, 1e-5, f"lmax=6 shared {name}")
+        assert_close(g, r, 1e-5, f"lmax={lmax} shared {name}")
 
 
 def test_edge_large_table(device):
