@@ -45,6 +45,8 @@ WORKLOADS = {
     # streaming kernels of known traffic (1 GiB): counter calibration and achievable-bandwidth reference
     "copy": None,
     "read": None,
+    # indexed scale-segment reduction alone: the messages of BASELINE configs[1] summed to their destination nodes
+    "scatter": None,
     # plain library GEMM (torch.matmul, bf16, 8192^3): the matrix rate the box reaches, next to the vendor peak
     "gemm": None,
 }
@@ -71,6 +73,41 @@ def gemm_bench(steps, warmup):
                       "data": "synthetic", "config": {"workload": "gemm: library GEMM, calibration of the MFMA peak"},
                       "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
                                    "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None}}))
+
+
+def scatter_bench(steps, warmup):
+    """`indexed_scale_segment(msg.view(1, E, 576), None, perm, ptr)` at N = 4096, E = 65536 (lmax = 2, C = 64): reads
+    every message once (151 MB) and the sorted tables, writes the node rows (9.4 MB)."""
+    from equitorch_amd.ops import indexed_scale_segment
+    dev = torch.device("cuda:0")
+    gen = torch.Generator().manual_seed(0)
+    n_nodes, n_edges, feat = 4096, 65536, 576
+    dst = torch.randint(0, n_nodes, (n_edges,), generator=gen)
+    perm = torch.sort(dst, stable=True).indices.to(dev)
+    ptr = torch.zeros(n_nodes + 1, dtype=torch.int64)
+    ptr[1:] = torch.cumsum(torch.bincount(dst, minlength=n_nodes), 0)
+    ptr = ptr.to(dev)
+    msgs = [torch.randn(1, n_edges, feat, generator=gen).to(dev) for _ in range(4)]
+    for i in range(warmup):
+        indexed_scale_segment(msgs[i % 4], None, perm, ptr, out_size=n_nodes)
+    evs = []
+    for i in range(steps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        indexed_scale_segment(msgs[i % 4], None, perm, ptr, out_size=n_nodes)
+        b.record()
+        evs.append((a, b))
+    torch.cuda.synchronize()
+    ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    nbytes = n_edges * feat * 4 + n_nodes * feat * 4 + n_edges * 8 + (n_nodes + 1) * 8
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    print(json.dumps({"metric": "scatter-sum Medges/s (576 floats per edge)", "value": round(n_edges / (ms * 1e-3) / 1e6, 1),
+                      "unit": "Medges/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 5),
+                      "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+                      "config": {"workload": f"scatter: indexed_scale_segment of (1, {n_edges}, {feat}) to {n_nodes} nodes"},
+                      "roofline": {"bound": "hbm", "kernel": "cgtp::segment_sum_kernel<float,4>", "achieved": round(gbs, 1),
+                                   "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                                   "traffic": None, "algorithmic_bytes": nbytes, "avg_ms": round(ms, 5)}}))
 
 
 def membench(kind, steps, warmup):
@@ -393,6 +430,9 @@ def main():
         return
     if args.workload == "gemm":
         gemm_bench(args.steps, args.warmup)
+        return
+    if args.workload == "scatter":
+        scatter_bench(args.steps, args.warmup)
         return
     if args.workload in ("uvw_fwd", "uvw_fwd_bwd"):
         uvw_bench(args)

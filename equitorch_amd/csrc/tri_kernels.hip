@@ -94,33 +94,56 @@ __global__ void __launch_bounds__(256) tri_kernel(const TriDev<T> a, int64_t n_w
   }
 }
 
-// out[n, m, c] = sum_{t in [seg[m], seg[m+1])} scale[t] * in[n, index[t], c]; one wavefront per (n, m).
+// out[n, m, c] = sum_{t in [seg[m], seg[m+1])} scale[t] * in[n, index[t], c].  One wavefront per (n, m, chunk of
+// 64 * V channels): wide rows are spread over several wavefronts, and the terms of a segment are fetched four at
+// a time (indices and scales first, then the four rows; the last one to three singly) and added in position
+// order, so the sum is the same whatever the launch shape.
 template <typename T, int V>
 __global__ void __launch_bounds__(256) segment_sum_kernel(const T* __restrict__ in, const T* __restrict__ scale,
                                                           const int64_t* __restrict__ index,
                                                           const int64_t* __restrict__ seg, T* __restrict__ out,
                                                           int64_t n_batch, int64_t in_size, int64_t out_size,
-                                                          int64_t C) {
+                                                          int64_t C, int chunks) {
+  constexpr int U = 4;
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
-  if (wave >= n_batch * out_size) return;
-  const int64_t n = wave / out_size, m = wave % out_size;
+  if (wave >= n_batch * out_size * chunks) return;
+  const int64_t row = wave / chunks;
+  const int64_t c = ((wave % chunks) * kWave + lane) * V;
+  const int64_t n = row / out_size, m = row % out_size;
   const int64_t tb = seg ? seg[m] : m, te = seg ? seg[m + 1] : m + 1;
-  const T* base = in + n * in_size * C;
-  T* dst = out + (n * out_size + m) * C;
-  for (int64_t c = (int64_t)lane * V; c < C; c += kWave * V) {
-    T acc[V];
+  const T* base = in + n * in_size * C + c;
+  const bool ok = c < C;
+  T acc[V];
 #pragma unroll
-    for (int v = 0; v < V; ++v) acc[v] = T(0);
-    for (int64_t t = tb; t < te; ++t) {
-      const int64_t i = index ? index[t] : t;
-      const T s = scale ? scale[t] : T(1);
-      T x[V];
-      load_vec<T, V>(x, base + i * C + c);
-      fmav<T, V>(acc, s, x);
+  for (int v = 0; v < V; ++v) acc[v] = T(0);
+  int64_t t0 = tb;
+  for (; t0 + U <= te; t0 += U) {
+    int64_t idx[U];
+    T sc[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      idx[u] = index ? index[t0 + u] : t0 + u;
+      sc[u] = scale ? scale[t0 + u] : T(1);
     }
-    store_vec<T, V>(dst + c, acc);
+    T x[U][V];
+    if (ok) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) load_vec<T, V>(x[u], base + idx[u] * C);
+#pragma unroll
+      for (int u = 0; u < U; ++u) fmav<T, V>(acc, sc[u], x[u]);
+    }
   }
+  for (; t0 < te; ++t0) {
+    const int64_t i = index ? index[t0] : t0;
+    const T sc = scale ? scale[t0] : T(1);
+    if (ok) {
+      T x[V];
+      load_vec<T, V>(x, base + i * C);
+      fmav<T, V>(acc, sc, x);
+    }
+  }
+  if (ok) store_vec<T, V>(out + (n * out_size + m) * C + c, acc);
 }
 
 static int tri_check(const cgtp_tri_args* a, int64_t* lds_bytes, int64_t* n_waves) {
@@ -183,16 +206,18 @@ static int tri_launch(const cgtp_tri_args* a, int64_t lds, int64_t n_waves, hipS
 template <typename T, int VW>
 static int segsum_launch(const void* in, const void* scale, const int64_t* index, const int64_t* seg, void* out,
                          int64_t n_batch, int64_t in_size, int64_t out_size, int64_t C, hipStream_t stream) {
-  const int64_t waves = n_batch * out_size;
-  if (waves == 0) return CGTP_OK;
+  if (n_batch * out_size == 0) return CGTP_OK;
   const bool vec = (C % VW) == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+  const int v = vec ? VW : 1;
+  const int chunks = (int)((C + (int64_t)kWave * v - 1) / ((int64_t)kWave * v));
+  const int64_t waves = n_batch * out_size * chunks;
   dim3 grid((unsigned)((waves + 3) / 4));
   if (vec)
     hipLaunchKernelGGL((segment_sum_kernel<T, VW>), grid, dim3(256), 0, stream, (const T*)in, (const T*)scale,
-                       index, seg, (T*)out, n_batch, in_size, out_size, C);
+                       index, seg, (T*)out, n_batch, in_size, out_size, C, chunks);
   else
     hipLaunchKernelGGL((segment_sum_kernel<T, 1>), grid, dim3(256), 0, stream, (const T*)in, (const T*)scale,
-                       index, seg, (T*)out, n_batch, in_size, out_size, C);
+                       index, seg, (T*)out, n_batch, in_size, out_size, C, chunks);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 
