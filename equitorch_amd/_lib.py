@@ -23,7 +23,7 @@ class CgtpError(RuntimeError):
 
 class Operand(C.Structure):
     _fields_ = [("data", C.c_void_p), ("rows", C.c_void_p), ("row_stride", C.c_int64),
-                ("idx_stride", C.c_int64), ("kind", C.c_int32), ("_pad", C.c_int32)]
+                ("idx_stride", C.c_int64), ("kind", C.c_int32), ("size", C.c_int32)]
 
 
 class TriArgs(C.Structure):

@@ -31,4 +31,18 @@ __global__ void partial_sum_kernel(const T* __restrict__ ws, T* __restrict__ out
   out[i] = (T)s;
 }
 
+// First pass of a sum over many rows: part[c * n + i] = sum of rows[r * n + i] over the rows r of chunk c
+// (kSumRows rows), in row order; partial_sum_kernel then adds the chunks.  Fixed order, no atomics.
+constexpr int kSumRows = 256;
+template <typename T>
+__global__ void __launch_bounds__(256) rows_sum_kernel(const T* __restrict__ rows, T* __restrict__ part, int64_t n_rows,
+                                                       int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int64_t r0 = (int64_t)blockIdx.y * kSumRows, r1 = r0 + kSumRows < n_rows ? r0 + kSumRows : n_rows;
+  T s = T(0);
+  for (int64_t r = r0; r < r1; ++r) s += rows[r * n + i];
+  part[blockIdx.y * n + i] = s;
+}
+
 }  // namespace cgtp

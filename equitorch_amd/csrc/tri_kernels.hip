@@ -12,7 +12,7 @@ struct OperandDev {
   const T* data;
   const int64_t* rows;
   int64_t row_stride, idx_stride;
-  int kind;
+  int kind, size;
 };
 
 template <typename T>
@@ -94,6 +94,96 @@ __global__ void __launch_bounds__(256) tri_kernel(const TriDev<T> a, int64_t n_w
   }
 }
 
+// The same contraction with the operands of a row staged in LDS first (the caller states the extent of every
+// operand's index axis): a wavefront copies the 64-channel slice of its row's operands into its own LDS region with
+// coalesced loads, then walks the table reading operands from LDS at wave-uniform row offsets — no global loads,
+// 64-bit address arithmetic or operand-kind branches per coefficient.  A per-channel operand occupies size x 64
+// elements, a channel-less one size elements, an absent one a single 1.  Writes one result per row (a sum over rows
+// is taken afterwards by the launcher).
+template <typename T>
+struct StagedOperand {
+  int offset;   // first element of the operand inside the wavefront's region
+  int stride;   // elements between sparse indices: 64 | 1 | 0
+};
+
+template <typename T, bool REDUCE_C>
+__global__ void __launch_bounds__(256) tri_staged_kernel(const TriDev<T> a, int64_t n_waves, int region_elems) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  T* s_coef = reinterpret_cast<T*>(smem);
+  uint32_t* s_idx = reinterpret_cast<uint32_t*>(s_coef + a.nnz);
+  int32_t* s_seg = reinterpret_cast<int32_t*>(s_idx + a.nnz);
+  const int table_elems = ((int)((a.nnz * (sizeof(T) + 4) + (a.n_out + 1) * 4 + 15) / 16)) * (16 / (int)sizeof(T));
+  for (int t = threadIdx.x; t < a.nnz; t += blockDim.x) {
+    s_coef[t] = a.coef ? a.coef[t] : T(1);
+    s_idx[t] = a.idx[t];
+  }
+  for (int t = threadIdx.x; t <= a.n_out; t += blockDim.x) s_seg[t] = a.seg[t];
+  __syncthreads();
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (wave >= n_waves) return;
+  T* region = reinterpret_cast<T*>(smem) + table_elems + (threadIdx.x / kWave) * region_elems;
+  const OperandDev<T>* ops[3] = {&a.a, &a.b, &a.w};
+  StagedOperand<T> so[3];
+  int off = 0;
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    const int kind = ops[k]->kind;
+    so[k].offset = off;
+    so[k].stride = kind == CGTP_OPERAND_VEC ? kWave : (kind == CGTP_OPERAND_SCALAR ? 1 : 0);
+    off += kind == CGTP_OPERAND_VEC ? ops[k]->size * kWave : (kind == CGTP_OPERAND_SCALAR ? ops[k]->size : 1);
+  }
+  // this lane's element of every operand: per-channel operands are read at [index * 64 + lane], the others at [index]
+  const T* la = region + so[0].offset + (so[0].stride == kWave ? lane : 0);
+  const T* lb = region + so[1].offset + (so[1].stride == kWave ? lane : 0);
+  const T* lw = region + so[2].offset + (so[2].stride == kWave ? lane : 0);
+
+  for (int64_t r = wave; r < a.n_rows; r += n_waves) {
+    for (int cb = 0; cb < a.C; cb += kWave) {
+      const int c = cb + lane;
+      const bool ok = c < a.C;
+#pragma unroll
+      for (int k = 0; k < 3; ++k) {
+        const OperandDev<T>& o = *ops[k];
+        T* dst = region + so[k].offset;
+        if (o.kind == CGTP_OPERAND_VEC) {
+          const T* src = row_ptr(o, r) + (ok ? c : 0);
+          for (int i = 0; i < o.size; ++i) dst[i * kWave + lane] = ok ? src[(int64_t)i * o.idx_stride] : T(0);
+        } else if (o.kind == CGTP_OPERAND_SCALAR) {
+          if (cb == 0) {
+            const T* src = row_ptr(o, r);
+            for (int i = lane; i < o.size; i += kWave) dst[i] = src[(int64_t)i * o.idx_stride];
+          }
+        } else if (cb == 0 && lane == 0) {
+          dst[0] = T(1);
+        }
+      }
+      // LDS operations of one wavefront complete in order: the reads below see the writes above
+      for (int o = 0; o < a.n_out; ++o) {
+        const int tb = __builtin_amdgcn_readfirstlane(s_seg[o]), te = __builtin_amdgcn_readfirstlane(s_seg[o + 1]);
+        T acc = T(0);
+#pragma unroll 4
+        for (int t = tb; t < te; ++t) {
+          const uint32_t u = __builtin_amdgcn_readfirstlane(s_idx[t]);
+          const int ia = (u & 1023u) * so[0].stride, ib = ((u >> 10) & 1023u) * so[1].stride, iw = (u >> 20) * so[2].stride;
+          acc += s_coef[t] * la[ia] * lb[ib] * lw[iw];
+        }
+        if constexpr (REDUCE_C) {
+          const T sum = group_sum(ok ? acc : T(0), kWave);
+          // channel blocks of one output row are accumulated by lane 0 in the output itself
+          if (lane == 0) {
+            T* dst = a.out + r * a.n_out + o;
+            *dst = cb == 0 ? sum : *dst + sum;
+          }
+        } else {
+          if (ok) a.out[(r * a.n_out + o) * a.C + c] = acc;
+        }
+      }
+    }
+  }
+}
+
 // out[n, m, c] = sum_{t in [seg[m], seg[m+1])} scale[t] * in[n, index[t], c].  One wavefront per (n, m, chunk of
 // 64 * V channels): wide rows are spread over several wavefronts, and the terms of a segment are fetched four at
 // a time (indices and scales first, then the four rows; the last one to three singly) and added in position
@@ -146,6 +236,30 @@ __global__ void __launch_bounds__(256) segment_sum_kernel(const T* __restrict__ 
   if (ok) store_vec<T, V>(out + (n * out_size + m) * C + c, acc);
 }
 
+static int64_t tri_table_bytes(const cgtp_tri_args* a) {
+  return (int64_t)a->nnz * (elem_size(a->dtype) + 4) + ((int64_t)a->n_out + 1) * 4;
+}
+
+// LDS bytes of the staged kernel (table + four operand regions) and elements per region, or 0 if the operands'
+// extents are unknown, the regions do not fit, or staging would not pay.
+static int64_t tri_staged_lds(const cgtp_tri_args* a, int64_t table_bytes, int64_t* region_elems) {
+  const cgtp_operand* ops[3] = {&a->a, &a->b, &a->w};
+  int64_t region = 0, vec_rows = 0;
+  for (const cgtp_operand* o : ops) {
+    if (o->kind != CGTP_OPERAND_NONE && o->size <= 0) return 0;
+    region += o->kind == CGTP_OPERAND_VEC ? (int64_t)o->size * kWave : (o->kind == CGTP_OPERAND_SCALAR ? o->size : 1);
+    if (o->kind == CGTP_OPERAND_VEC) vec_rows += o->size;
+  }
+  // staging pays when operand rows are read more than once; with about one coefficient per staged row (the
+  // second stage of the reference's two-launch products) the direct kernel is faster
+  if (a->nnz <= vec_rows) return 0;
+  region = (region + 3) / 4 * 4;
+  const int64_t lds = (table_bytes + 15) / 16 * 16 + 4 * region * elem_size(a->dtype);
+  if (lds > kLdsBytes) return 0;
+  *region_elems = region;
+  return lds;
+}
+
 static int tri_check(const cgtp_tri_args* a, int64_t* lds_bytes, int64_t* n_waves) {
   if (!a) return CGTP_ERR_NULL;
   if (a->dtype != CGTP_F32 && a->dtype != CGTP_F64) return CGTP_ERR_DTYPE;
@@ -157,8 +271,7 @@ static int tri_check(const cgtp_tri_args* a, int64_t* lds_bytes, int64_t* n_wave
     if (o->kind != CGTP_OPERAND_NONE && !o->data) return CGTP_ERR_NULL;
     if (o->kind != CGTP_OPERAND_NONE && (o->row_stride < 0 || o->idx_stride < 0)) return CGTP_ERR_SHAPE;
   }
-  const int64_t esz = elem_size(a->dtype);
-  *lds_bytes = (int64_t)a->nnz * (esz + 4) + ((int64_t)a->n_out + 1) * 4;
+  *lds_bytes = tri_table_bytes(a);
   if (*lds_bytes > kLdsBytes) return CGTP_ERR_LDS;
   if (a->reduce_rows) {
     int64_t nw = a->n_rows < 1024 ? a->n_rows : 1024;
@@ -172,7 +285,7 @@ static int tri_check(const cgtp_tri_args* a, int64_t* lds_bytes, int64_t* n_wave
 
 template <typename T>
 static OperandDev<T> op_dev(const cgtp_operand& o) {
-  return OperandDev<T>{(const T*)o.data, o.rows, o.row_stride, o.idx_stride, o.kind};
+  return OperandDev<T>{(const T*)o.data, o.rows, o.row_stride, o.idx_stride, o.kind, o.size};
 }
 
 template <typename T>
@@ -188,6 +301,29 @@ static int tri_launch(const cgtp_tri_args* a, int64_t lds, int64_t n_waves, hipS
   d.n_out = a->n_out; d.nnz = a->nnz;
   d.out = a->reduce_rows ? (T*)a->workspace : (T*)a->out;
   d.n_rows = a->n_rows; d.C = a->C; d.reduce_rows = a->reduce_rows;
+  // operands staged in LDS when their extents are known and four regions fit next to the table; a sum over rows
+  // then goes through per-row results in the workspace and two fixed-order passes
+  int64_t region = 0;
+  const int64_t staged_lds = tri_staged_lds(a, lds, &region);
+  if (staged_lds > 0) {
+    auto skern = a->reduce_c ? tri_staged_kernel<T, true> : tri_staged_kernel<T, false>;
+    if (staged_lds > 48 * 1024 &&
+        hipFuncSetAttribute((const void*)skern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)staged_lds) != hipSuccess)
+      return CGTP_ERR_LDS;
+    const int64_t nw = a->n_rows < 16384 ? a->n_rows : 16384;
+    hipLaunchKernelGGL(skern, dim3((unsigned)((nw + 3) / 4)), dim3(256), (size_t)staged_lds, stream, d, nw, (int)region);
+    if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
+    if (a->reduce_rows) {
+      const int64_t chunks = (a->n_rows + kSumRows - 1) / kSumRows;
+      T* part = (T*)a->workspace + a->n_rows * per_row;
+      hipLaunchKernelGGL(rows_sum_kernel<T>, dim3((unsigned)((per_row + 255) / 256), (unsigned)chunks), dim3(256), 0,
+                         stream, (const T*)a->workspace, part, a->n_rows, per_row);
+      hipLaunchKernelGGL(partial_sum_kernel<T>, dim3((unsigned)((per_row + 255) / 256)), dim3(256), 0, stream,
+                         (const T*)part, (T*)a->out, chunks, per_row);
+      if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
+    }
+    return CGTP_OK;
+  }
   auto kern = a->reduce_c ? tri_kernel<T, true> : tri_kernel<T, false>;
   if (lds > 48 * 1024) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -257,8 +393,12 @@ int cgtp_tri_validate(const cgtp_tri_args* args) {
 
 int64_t cgtp_tri_workspace_bytes(const cgtp_tri_args* a) {
   if (!a || !a->reduce_rows) return 0;
+  const int64_t per_row = (int64_t)a->n_out * (a->reduce_c ? 1 : a->C);
+  int64_t region = 0;
+  if (tri_staged_lds(a, tri_table_bytes(a), &region) > 0)  // per-row results + first-pass partials
+    return (a->n_rows + (a->n_rows + kSumRows - 1) / kSumRows) * per_row * elem_size(a->dtype);
   const int64_t nw = a->n_rows < 1024 ? a->n_rows : 1024;
-  return nw * (int64_t)a->n_out * (a->reduce_c ? 1 : a->C) * elem_size(a->dtype);
+  return nw * per_row * elem_size(a->dtype);
 }
 
 int cgtp_tri_contract(const cgtp_tri_args* a, void* stream) {

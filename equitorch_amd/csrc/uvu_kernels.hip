@@ -470,7 +470,6 @@ static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t
 
 static constexpr int64_t kMaxRowWaves = 2048;
 static constexpr int kDefaultPosPerWave = 32;
-static constexpr int kBigSumRows = 256;  // rows per first-pass chunk of the shared-weight gradient sum
 
 static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan* plan) {
   if (!a) return CGTP_ERR_NULL;
@@ -554,9 +553,9 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
     plan->n_waves = nw;
   }
   if (wred && big) {
-    // block-wise kernels write the weight gradient of every row; two summation passes follow (kBigSumRows rows
+    // block-wise kernels write the weight gradient of every row; two summation passes follow (kSumRows rows
     // each, then the partials)
-    const int64_t chunks = (a->n_rows + kBigSumRows - 1) / kBigSumRows;
+    const int64_t chunks = (a->n_rows + kSumRows - 1) / kSumRows;
     plan->wsw_elems = (a->n_rows + chunks) * dims[3] * a->C;
   } else if (wred) {
     plan->wsw_elems = plan->n_waves * dims[3] * a->C;
@@ -587,17 +586,6 @@ static int launch_fixup(T* rows, const UvuDev<T>& d, int64_t row_len, hipStream_
   return launched();
 }
 
-// part[c * n + i] = sum of rows[r * n + i] over the rows r of chunk c (kBigSumRows rows), in row order.
-__global__ void __launch_bounds__(256) rows_sum_kernel(const float* __restrict__ rows, float* __restrict__ part,
-                                                       int64_t n_rows, int64_t n) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const int64_t r0 = (int64_t)blockIdx.y * kBigSumRows, r1 = r0 + kBigSumRows < n_rows ? r0 + kBigSumRows : n_rows;
-  float s = 0.f;
-  for (int64_t r = r0; r < r1; ++r) s += rows[r * n + i];
-  part[blockIdx.y * n + i] = s;
-}
-
 static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward, hipStream_t stream) {
   int n_big = 0;
   const UvuBigEntry& e = uvu_big_entries(&n_big)[plan.big_idx];
@@ -614,9 +602,9 @@ static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward,
                        stream, d, plan.n_waves);
     if (wred) {
       if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
-      const int64_t chunks = (a->n_rows + kBigSumRows - 1) / kBigSumRows;
+      const int64_t chunks = (a->n_rows + kSumRows - 1) / kSumRows;
       float* part = d.wsw + a->n_rows * w_elems;
-      hipLaunchKernelGGL(rows_sum_kernel, dim3((unsigned)((w_elems + 255) / 256), (unsigned)chunks), dim3(256), 0, stream,
+      hipLaunchKernelGGL(rows_sum_kernel<float>, dim3((unsigned)((w_elems + 255) / 256), (unsigned)chunks), dim3(256), 0, stream,
                          (const float*)d.wsw, part, a->n_rows, w_elems);
       if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
       hipLaunchKernelGGL(partial_sum_kernel<float>, dim3((unsigned)((w_elems + 255) / 256)), dim3(256), 0, stream,

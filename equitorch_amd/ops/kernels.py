@@ -62,6 +62,7 @@ def _operand(t: Optional[Tensor], kind: int, rows: Optional[Tensor] = None) -> O
     op.data = t.data_ptr()
     op.rows = _lib.ptr(rows)
     op.kind = kind
+    op.size = t.shape[-2] if kind == OPERAND_VEC else t.shape[-1]
     return op
 
 

@@ -57,7 +57,8 @@ typedef struct cgtp_operand {
   int64_t row_stride;      /* elements between rows; 0 = one row shared by every r              */
   int64_t idx_stride;      /* elements between consecutive sparse indices (C for vec, 1 scalar) */
   int32_t kind;            /* CGTP_OPERAND_*                                                    */
-  int32_t _pad;
+  int32_t size;            /* extent of the sparse index axis, or 0 if unknown (known extents let the kernel
+                              stage the operand in LDS)                                            */
 } cgtp_operand;
 
 typedef struct cgtp_tri_args {
