@@ -1,0 +1,72 @@
+"""Fully connected ("uv") products in fp32 / fp64 with a shared weight: the channel mixing is a plain GEMM per weight
+path on the library (``torch.matmul``), the Clebsch-Gordan stage runs on the table-driven contraction kernel.
+
+Weight-first order, as in the matrix-core kernel: ``z[n, q, :] = x[n, a_q, :] @ W[p_q]`` for every (path, input row)
+pair ``q``, then ``out[n, M] = sum_t coef_t * y[n, b_t] * z[n, q_t]``.  Every piece is differentiable (``matmul``,
+``cat`` and the closed contraction family of ``_tri``), so gradients of any order come from autograd.  The bf16 case
+does not come here (``_uvw_mfma``); per-sample weights stay on the general two-axis kernel.
+"""
+from typing import List, Tuple
+
+import numpy as np
+import torch
+from torch import Tensor
+
+from ..._lib import OPERAND_NONE, OPERAND_SCALAR, OPERAND_VEC
+from ...ops import kernels
+from ._tri import TriSpec, tri
+
+
+class _Plan:
+    """Per table and channelled operand: the row range every path reads and the contraction of the second stage."""
+
+    def __init__(self, coo, chan_col: np.ndarray, other_col: np.ndarray, other_size: int):
+        self.ranges: List[Tuple[int, int]] = []
+        q_of = {}
+        n_q = 0
+        for p in range(coo.P):
+            rows = np.unique(chan_col[coo.p == p])
+            if not (rows.size and np.array_equal(rows, np.arange(rows[0], rows[0] + rows.size))):
+                raise ValueError("the rows a path reads must be contiguous (one irrep)")
+            self.ranges.append((int(rows[0]), int(rows.size)))
+            for a in rows:
+                q_of[(p, int(a))] = n_q
+                n_q += 1
+        q = np.array([q_of[(int(p), int(a))] for p, a in zip(coo.p, chan_col)], dtype=np.int64)
+        self.n_q = n_q
+        self.spec = TriSpec(coo.M, [q, other_col, None], coo.coef, coo.DO, [n_q, other_size, None])
+
+
+def _plan(tp_info, chan: int) -> _Plan:
+    def build():
+        coo = kernels.coo_of(tp_info)
+        if chan == 1:
+            return _Plan(coo, coo.M1, coo.M2, coo.D2)
+        return _Plan(coo, coo.M2, coo.M1, coo.D1)
+    return kernels.cached(tp_info.info_Mij_fwd.scale, ("uv_gemm", chan), build)
+
+
+def _mix(x: Tensor, weight: Tensor, plan: _Plan) -> Tensor:
+    """``z[n, q, :] = x[n, a_q, :] @ weight[p_q]``: one GEMM per path over the rows of its input irrep."""
+    return torch.cat([torch.matmul(x[:, a0:a0 + na, :], weight[p]) for p, (a0, na) in enumerate(plan.ranges)], dim=1)
+
+
+def supported(*tensors: Tensor) -> bool:
+    dtypes = {t.dtype for t in tensors}
+    return len(dtypes) == 1 and next(iter(dtypes)) in (torch.float32, torch.float64) and tensors[-1].ndim == 3
+
+
+def u1v(input1: Tensor, input2: Tensor, weight: Tensor, tp_info) -> Tensor:
+    plan = _plan(tp_info, 1)
+    return tri(plan.spec, (OPERAND_VEC, OPERAND_SCALAR, OPERAND_NONE), OPERAND_VEC, _mix(input1, weight, plan), input2)
+
+
+def one_vu(input1: Tensor, input2: Tensor, weight: Tensor, tp_info) -> Tensor:
+    plan = _plan(tp_info, 2)
+    return tri(plan.spec, (OPERAND_VEC, OPERAND_SCALAR, OPERAND_NONE), OPERAND_VEC, _mix(input2, weight, plan), input1)
+
+
+def vu1(input1: Tensor, input2: Tensor, weight: Tensor, tp_info) -> Tensor:
+    """``out[n, M] = sum_t coef_t * <x[n, a_t, :] @ W[p_t], y[n, b_t, :]>``."""
+    plan = _plan(tp_info, 1)
+    return tri(plan.spec, (OPERAND_VEC, OPERAND_VEC, OPERAND_NONE), OPERAND_SCALAR, _mix(input1, weight, plan), input2)

@@ -101,10 +101,12 @@ def tensor_product_u1v(input1: Tensor, input2: Tensor, weight: Tensor,
     """``out[n,M,w] = sum_t c_t y[n,M2_t] sum_u x[n,M1_t,u] W[(n),p_t,u,w]`` — ``input1 (N, D1, C_in)``,
     ``input2 (N, D2)`` -> ``(N, DO, C_out)`` (reference ``linears.py:254-336``)."""
     _check_batch(input1, input2, weight)
-    from . import _uvw_mfma
+    from . import _uv_gemm, _uvw_mfma
     fast = _uvw_mfma.try_forward(input1, input2, weight, tp_info_forward)
     if fast is not None:
         return fast
+    if input1.ndim == 3 and input2.ndim == 2 and _uv_gemm.supported(input1, input2, weight):
+        return _uv_gemm.u1v(input1, input2, weight, tp_info_forward)
     return tri(spec_from_tp_info(tp_info_forward), ("u", "", "uw"), "w", input1, input2, weight)
 
 
@@ -117,6 +119,9 @@ def tensor_product_1vu(input1: Tensor, input2: Tensor, weight: Tensor,
                        tp_info_backward2: Optional[TensorProductInfo] = None) -> Tensor:
     """``input1 (N, D1)``, ``input2 (N, D2, C_in)`` -> ``(N, DO, C_out)`` (reference ``:338-412``)."""
     _check_batch(input1, input2, weight)
+    from . import _uv_gemm
+    if input1.ndim == 2 and input2.ndim == 3 and _uv_gemm.supported(input1, input2, weight):
+        return _uv_gemm.one_vu(input1, input2, weight, tp_info_forward)
     return tri(spec_from_tp_info(tp_info_forward), ("", "u", "uw"), "w", input1, input2, weight)
 
 
@@ -127,4 +132,7 @@ def tensor_product_vu1(input1: Tensor, input2: Tensor, weight: Tensor,
     """``out[n,M] = sum_t c_t sum_{u,w} x[n,M1_t,u] W[(n),p_t,u,w] y[n,M2_t,w]`` — ``input1 (N, D1, C1)``,
     ``input2 (N, D2, C2)``, ``weight (P, C1, C2)`` -> ``(N, DO)`` (reference ``:414-492``)."""
     _check_batch(input1, input2, weight)
+    from . import _uv_gemm
+    if input1.ndim == 3 and input2.ndim == 3 and _uv_gemm.supported(input1, input2, weight):
+        return _uv_gemm.vu1(input1, input2, weight, tp_info_forward)
     return tri(spec_from_tp_info(tp_info_forward), ("u", "w", "uw"), "", input1, input2, weight)
