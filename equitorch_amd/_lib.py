@@ -98,6 +98,10 @@ def _load():
                                    C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
     lib.cgtp_uv_validate.argtypes = _uv
     lib.cgtp_uv_apply.argtypes = _uv + [C.c_void_p]
+    lib.cgtp_sh_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_double, C.c_int,
+                                    C.c_void_p]
+    lib.cgtp_sh_backward.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_double,
+                                     C.c_int, C.c_void_p]
     lib.cgtp_membench_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
     lib.cgtp_membench_read.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
     return lib

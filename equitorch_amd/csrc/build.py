@@ -40,7 +40,8 @@ def _compile(src: str) -> str:
 
 
 def build(jobs: int = 8) -> str:
-    from . import gen_uv, gen_uvu, gen_uvu_big
+    from . import gen_sh, gen_uv, gen_uvu, gen_uvu_big
+    gen_sh.main()
     gen_uvu.main()
     gen_uvu_big.main()
     gen_uv.main()

@@ -5,11 +5,13 @@ from .linears import (so3_linear_uu, so3_linear_uv, tensor_product_1uu, tensor_p
 from .sparse_product import (sparse_inner, sparse_mat_t_vec, sparse_mul, sparse_outer, sparse_scavec, sparse_vecmat,
                              sparse_vecsca)
 from .sparse_scale import sparse_scale
+from .sphericals import spherical_harmonics, spherical_to_xyz, xyz_to_spherical
 from .tensor_products import tensor_product_uuu, tensor_product_uvw
 
 __all__ = [
     "tensor_product_uuu", "tensor_product_uvw", "tensor_product_u1u", "tensor_product_1uu", "tensor_product_uu1",
     "tensor_product_u1v", "tensor_product_1vu", "tensor_product_vu1", "so3_linear_uu", "so3_linear_uv",
     "sparse_mul", "sparse_outer", "sparse_inner", "sparse_vecmat", "sparse_vecsca", "sparse_scavec",
-    "sparse_mat_t_vec", "sparse_scale", "EdgePlan", "edge_tensor_product_uu",
+    "sparse_mat_t_vec", "sparse_scale", "EdgePlan", "edge_tensor_product_uu", "spherical_harmonics",
+    "xyz_to_spherical", "spherical_to_xyz",
 ]

@@ -237,6 +237,23 @@ int64_t cgtp_uv_grad_w_workspace_bytes(int cfg, int64_t n_rows, int32_t cin, int
 int cgtp_uv_grad_w(int cfg, const void* x, const void* y, const void* g, void* gw, void* workspace, int64_t n_rows,
                    int32_t cin, int32_t cout, int32_t dtype, void* stream);
 
+/* ---- real spherical harmonics of vectors -----------------------------------------------------------------
+ * Stands in for spherical_harmonics (equitorch/ops/spherical_harmonics.py:68-640: explicit polynomials per
+ * degree, TorchScript, differentiated by autograd) together with its callers' pre- and post-processing:
+ * torch.nn.functional.normalize(input, dim=-1) of SphericalHarmonics.forward (equitorch/nn/sphericals.py:31-35)
+ * when normalize != 0, and the 1/sqrt(4 pi) factor of integral_normalize
+ * (equitorch/nn/functional/sphericals.py:9-14) passed as scale (1.0 otherwise).
+ * xyz: (n, 3); out / grad_out: (n, (lmax+1)^2), index l^2 + l + m; grad_xyz: (n, 3).  Component order and
+ * normalisation as in the reference: Y_1 = sqrt(3) (y, z, x), |Y_l|^2 = 2l+1 on the unit sphere, homogeneous
+ * of degree l when normalize == 0.  lmax <= cgtp_sh_max_degree() (17, the reference's limit).
+ * dtype: CGTP_F32 | CGTP_F64.  n == 0 returns CGTP_OK without a launch.
+ */
+int cgtp_sh_max_degree(void);
+int cgtp_sh_forward(const void* xyz, void* out, int64_t n, int lmax, int normalize, double scale, int dtype,
+                    void* stream);
+int cgtp_sh_backward(const void* xyz, const void* grad_out, void* grad_xyz, int64_t n, int lmax, int normalize,
+                     double scale, int dtype, void* stream);
+
 /* ---- streaming kernels of known traffic (counter calibration, achievable-bandwidth reference) ------------
  * No counterpart in the reference.  copy: reads n_bytes and writes n_bytes; read: reads n_bytes.
  * n_bytes must be a multiple of 16 and the pointers 16-byte aligned.

@@ -161,6 +161,19 @@ def test_uv_matrix_core_entry_points_validate_on_the_host():
     assert L.cgtp_uv_grad_w(cfg, p16, p16, p16, p16, p16, 100, 128, 160, _lib.BF16, None) == 2
 
 
+def test_spherical_harmonics_entry_points_validate_on_the_host():
+    from equitorch_amd import _lib
+    L = _lib.lib
+    assert L.cgtp_sh_max_degree() == 17
+    assert L.cgtp_sh_forward(None, None, 0, 3, 1, 1.0, _lib.F32, None) == 0          # empty batch: no launch
+    assert L.cgtp_sh_forward(None, 4096, 5, 3, 1, 1.0, _lib.F32, None) == 1          # null
+    assert L.cgtp_sh_forward(4096, 4096, 5, 18, 1, 1.0, _lib.F32, None) == 2         # degree above 17
+    assert L.cgtp_sh_forward(4096, 4096, -1, 2, 1, 1.0, _lib.F32, None) == 2
+    assert L.cgtp_sh_forward(4096, 4096, 5, 2, 1, 1.0, _lib.BF16, None) == 4         # fp32 / fp64 only
+    assert L.cgtp_sh_backward(4096, None, 4096, 5, 2, 1, 1.0, _lib.F64, None) == 1
+    assert L.cgtp_sh_backward(4096, 4096, 4096, 0, 2, 1, 1.0, _lib.F64, None) == 0
+
+
 def test_cpu_tensors_are_rejected_loudly():
     import torch
     from equitorch_amd import _lib

@@ -1,0 +1,97 @@
+"""GPU parity of the spherical-harmonics kernels (cgtp_sh_forward / cgtp_sh_backward) against the oracle."""
+import math
+
+import pytest
+import torch
+
+from helpers import assert_close
+from oracle import ref_sh
+
+pytestmark = pytest.mark.gpu
+
+
+def _vectors(n, seed, spread=True):
+    g = torch.Generator().manual_seed(seed)
+    v = torch.randn(n, 3, generator=g, dtype=torch.float64)
+    v = v / v.norm(dim=-1, keepdim=True)
+    if spread:   # lengths in [0.6, 1.4]: the polynomials are homogeneous, so this exercises r^l
+        v = v * (0.6 + 0.8 * torch.rand(n, 1, generator=g, dtype=torch.float64))
+    return v
+
+
+@pytest.mark.parametrize("l_max", [0, 1, 2, 3, 4, 6, 7, 8, 11, 17])
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+def test_forward_matches_oracle(device, l_max, dtype):
+    """Four, two or one wavefront tiles in LDS by degree; fp64 at degree 17 addresses global memory directly; n is not
+    a multiple of 64."""
+    from equitorch_amd.ops import spherical_harmonics
+    v = _vectors(1000 + l_max, seed=l_max)
+    ref = ref_sh.spherical_harmonics(v, l_max)
+    out = spherical_harmonics(v.to(device, dtype), l_max)
+    assert out.dtype == dtype and out.shape == ref.shape
+    if dtype == torch.float64:
+        assert_close(out, ref, tol=1e-12, what=f"Y lmax={l_max}")
+    else:
+        # fp32 parity bar: rel/abs 1e-5; inputs rounded to fp32 first so that only arithmetic differs
+        ref32 = ref_sh.spherical_harmonics(v.float().double(), l_max)
+        assert_close(out, ref32, tol=1e-5, what=f"Y lmax={l_max}")
+
+
+@pytest.mark.parametrize("l_max", [1, 2, 3, 6, 9])
+@pytest.mark.parametrize("normalize", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+def test_backward_matches_oracle_autograd(device, l_max, normalize, dtype):
+    from equitorch_amd.ops import spherical_harmonics
+    n = 333
+    v = _vectors(n, seed=50 + l_max).to(dtype).double().requires_grad_(True)
+    ct = torch.randn(n, (l_max + 1) ** 2, generator=torch.Generator().manual_seed(7), dtype=torch.float64)
+    ct = ct.to(dtype).double()
+    scale = 0.37
+    ref = scale * ref_sh.spherical_harmonics(ref_sh.normalize(v) if normalize else v, l_max)
+    (ref * ct).sum().backward()
+    vd = v.detach().to(device, dtype).requires_grad_(True)
+    out = spherical_harmonics(vd, l_max, normalize=normalize, scale=scale)
+    (out * ct.to(device, dtype)).sum().backward()
+    tol = 1e-11 if dtype == torch.float64 else 1e-5
+    assert_close(out, ref, tol=tol, what="Y")
+    assert_close(vd.grad, v.grad, tol=tol, what="grad_xyz")
+
+
+def test_module_layout_options_and_edge_cases(device):
+    from equitorch_amd.nn import SphericalHarmonics
+    from equitorch_amd.nn.functional import spherical_harmonics
+    v = _vectors(24, seed=3).reshape(2, 3, 4, 3)
+    mod = SphericalHarmonics(3, normalize_input=True, integral_normalize=True)
+    ref = ref_sh.spherical_harmonics(ref_sh.normalize(v.reshape(-1, 3)), 3).reshape(2, 3, 4, 16) / math.sqrt(4 * math.pi)
+    assert_close(mod(v.to(device)), ref, tol=1e-12, what="module")
+    # vectors stored along another dimension
+    out = spherical_harmonics(v.permute(0, 3, 1, 2).to(device), 3, dim=1)
+    assert out.shape == (2, 16, 3, 4)
+    assert_close(out.permute(0, 2, 3, 1), ref_sh.spherical_harmonics(v.reshape(-1, 3), 3).reshape(2, 3, 4, 16),
+                 tol=1e-12, what="dim=1")
+    # empty batch, single vector, the zero vector under normalisation (F.normalize maps it to zero: only Y_0 survives)
+    assert spherical_harmonics(torch.zeros(0, 3, device=device), 2).shape == (0, 9)
+    z = torch.zeros(1, 3, device=device, dtype=torch.float64, requires_grad=True)
+    y0 = SphericalHarmonics(2)(z)
+    assert_close(y0, torch.tensor([[1.0] + [0.0] * 8], dtype=torch.float64), tol=1e-12, what="zero vector")
+    y0.sum().backward()
+    assert torch.isfinite(z.grad).all()
+    with pytest.raises(ValueError):
+        spherical_harmonics(torch.zeros(4, 2, device=device), 2)
+    with pytest.raises(ValueError):
+        spherical_harmonics(torch.zeros(4, 3, device=device), 18)
+
+
+def test_full_size_properties(device):
+    """One million vectors, lmax = 6: |Y_l|^2 = 2l+1 for every vector and degree, and the result does not depend on
+    where in the batch a vector sits (rows of a permuted batch are the permuted rows)."""
+    from equitorch_amd.ops import spherical_harmonics
+    n = 1_000_003
+    g = torch.Generator(device=device).manual_seed(0)
+    v = torch.randn(n, 3, generator=g, device=device)
+    y = spherical_harmonics(v, 6, normalize=True)
+    for l in range(7):
+        nrm = (y[:, l * l:(l + 1) ** 2] ** 2).sum(-1)
+        assert float((nrm - (2 * l + 1)).abs().max()) < 1e-4 * (2 * l + 1)
+    perm = torch.randperm(n, generator=g, device=device)
+    assert torch.equal(spherical_harmonics(v[perm], 6, normalize=True), y[perm])
