@@ -51,7 +51,7 @@ class UvuArgs(C.Structure):
     _fields_ = [("cfg", C.c_int32), ("dtype", C.c_int32), ("C", C.c_int32), ("w_shared", C.c_int32),
                 ("n_rows", C.c_int64), ("n_x_rows", C.c_int64), ("n_seg", C.c_int64),
                 ("ptr", C.c_void_p), ("perm", C.c_void_p), ("seg_ids", C.c_void_p), ("gather", C.c_void_p),
-                ("pos_per_wave", C.c_int32), ("_pad", C.c_int32),
+                ("pos_per_wave", C.c_int32), ("y_vec", C.c_int32),
                 ("wave_seg", C.c_void_p), ("n_waves", C.c_int64),
                 ("x", C.c_void_p), ("y", C.c_void_p), ("w", C.c_void_p),
                 ("out", C.c_void_p),
@@ -80,6 +80,7 @@ def _load():
     lib.cgtp_uvu_find.argtypes = [C.c_uint64]
     lib.cgtp_uvu_describe.restype = C.c_uint64
     lib.cgtp_uvu_describe.argtypes = [C.c_int, C.POINTER(C.c_int32)]
+    lib.cgtp_uvu_sh_degree.argtypes = [C.c_int]
     lib.cgtp_uvu_validate.argtypes = [C.POINTER(UvuArgs), C.c_int]
     lib.cgtp_uvu_workspace_bytes.restype = C.c_int64
     lib.cgtp_uvu_workspace_bytes.argtypes = [C.POINTER(UvuArgs), C.c_int]

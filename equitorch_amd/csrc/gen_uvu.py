@@ -57,7 +57,14 @@ def _opaque(m2s) -> str:
     return "    " + " ".join(f'asm volatile("" : "+v"(yy[{m}]));' for m in m2s)
 
 
-def emit_config(name: str, coo) -> str:
+def sh_degree(irreps_in2) -> int:
+    """L when the second operand has the layout of spherical harmonics of degrees 0..L (one irrep per degree, in
+    order, any parity), else -1: only then can a kernel evaluate the operand from a vector."""
+    ls = [ir.l for ir in Irreps(irreps_in2)]
+    return len(ls) - 1 if ls == list(range(len(ls))) else -1
+
+
+def emit_config(name: str, coo, sh_lmax: int = -1) -> str:
     T = coo.coef.shape[0]
     # (p, M) segments, path-major: the weight row of a path is needed only while that path is evaluated, and
     # its gradient is complete when the path ends, so neither has to stay in registers.
@@ -73,6 +80,7 @@ def emit_config(name: str, coo) -> str:
     a(f"  static constexpr int D1 = {coo.D1}, D2 = {coo.D2}, DO = {coo.DO}, P = {coo.P}, NNZ = {T};")
     a(f"  static constexpr unsigned long long FINGERPRINT = 0x{fingerprint(coo):016x}ull;")
     a(f"  static constexpr const char* NAME = \"{name}\";")
+    a(f"  static constexpr int SH_LMAX = {sh_lmax};  // second operand = harmonics of degrees 0..SH_LMAX (-1: not)")
     # ---- forward: o[M] += w[p] * sum_t (coef_t y[M2_t]) x[M1_t]
     a("  // wload(p, w): fetch the V channels of weight path p")
     a("  template <typename T, int V, class WLoad>")
@@ -122,7 +130,7 @@ def main(out_dir: str = None) -> str:
     for name, (io, i1, i2, kw) in CONFIGS.items():
         coo = tp_coo(tp_infos(Irreps(io), Irreps(i1), Irreps(i2), **kw)[0])
         chunks.append(f"// {name}: {i1} x {i2} -> {io} {kw if kw else ''}")
-        chunks.append(emit_config(name, coo))
+        chunks.append(emit_config(name, coo, sh_degree(i2)))
         chunks.append("")
     chunks.append("#define CGTP_FOREACH_UVU_CONFIG(X) \\")
     chunks.append(" \\\n".join(f"  X(TP_{n})" for n in CONFIGS))

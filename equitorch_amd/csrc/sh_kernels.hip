@@ -15,25 +15,12 @@
 // global memory directly.
 #include "cgtp_host.h"
 
-#include "generated/sh_coef.inc"
+#include "sh_device.h"
 
 namespace cgtp {
 namespace {
 
-template <typename T> struct ShCoef;
-template <> struct ShCoef<float> {
-  __device__ static float step(int m) { return kShStepF[m]; }
-  __device__ static float a(int l, int m) { return kShAF[l][m]; }
-  __device__ static float b(int l, int m) { return kShBF[l][m]; }
-};
-template <> struct ShCoef<double> {
-  __device__ static double step(int m) { return kShStepD[m]; }
-  __device__ static double a(int l, int m) { return kShAD[l][m]; }
-  __device__ static double b(int l, int m) { return kShBD[l][m]; }
-};
-
 constexpr int kShBlock = 256;       // most vectors per workgroup, one per lane
-constexpr double kShEps = 1e-12;    // torch.nn.functional.normalize: v / max(|v|, eps)
 
 // Row `lane` of a (64 x D) tile: in LDS at pitch `pitch`, or straight in global memory at pitch D.
 template <typename T>

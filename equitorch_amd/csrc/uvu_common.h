@@ -26,6 +26,7 @@ struct UvuDev {
   const int32_t* wave_seg;  // segment mode: optional wavefront -> first segment table (segment-aligned ranges)
   int64_t n_rows, n_seg;
   int C, lpe_log2, w_shared, pos_per_wave;
+  int y_vec;  // segment mode: y holds edge vectors (kYUnitVector / kYRawVector) instead of harmonics
 };
 
 struct Lanes {

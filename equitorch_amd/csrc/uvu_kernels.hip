@@ -14,6 +14,7 @@
 // output directly; the (at most two) segments cut by the range boundary are written as partial rows to a
 // workspace and summed in a fixed order by uvu_fixup_kernel.  No atomics: results are deterministic.
 #include "uvu_common.h"
+#include "sh_device.h"
 
 namespace cgtp {
 #include "generated/uvu_configs.inc"
@@ -248,7 +249,8 @@ __device__ __forceinline__ void seg_finish(SegStep& st, T (&acc)[D][V], T* __res
   if (R.s0 >= 0) zero_fill_rows(final_rows, st.next_row, R.s1, (int64_t)D * C, L.lane);
 }
 
-template <class TP, typename T, int V>
+// YV: the second operand is an edge vector; its harmonics are evaluated here (sh_device.h).
+template <class TP, typename T, int V, bool YV = false>
 __global__ void __launch_bounds__(256) uvu_seg_fwd_kernel(const UvuDev<T> a, int64_t n_waves) {
   constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
   const Lanes L(a.lpe_log2);
@@ -270,8 +272,13 @@ __global__ void __launch_bounds__(256) uvu_seg_fwd_kernel(const UvuDev<T> a, int
     if (seg_step_begin<T, DO, V>(st, acc, a.out, a.ws, I, off0, ei, oi, wave, R, L, a.lpe_log2, cok, C, c0)) {
       const int64_t e = ei, xr = oi;
       T x[D1][V], y[D2];
+      if constexpr (YV) {
+        const ShPoint<T> pt(a.y[e * 3], a.y[e * 3 + 1], a.y[e * 3 + 2], a.y_vec == kYUnitVector);
+        sh_values<T, TP::SH_LMAX>(pt.x, pt.y, pt.z, y);
+      } else {
 #pragma unroll
-      for (int j = 0; j < D2; ++j) y[j] = a.y[e * D2 + j];
+        for (int j = 0; j < D2; ++j) y[j] = a.y[e * D2 + j];
+      }
       if (cok) {
 #pragma unroll
         for (int i = 0; i < D1; ++i) load_vec<T, V>(x[i], a.x + (xr * D1 + i) * C + c0);
@@ -290,7 +297,7 @@ __global__ void __launch_bounds__(256) uvu_seg_fwd_kernel(const UvuDev<T> a, int
   seg_finish<T, DO, V>(st, acc, a.out, a.ws, wave, R, L, cok, C, c0);
 }
 
-template <class TP, typename T, int V, int GW>
+template <class TP, typename T, int V, int GW, bool YV = false>
 __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, int64_t n_waves) {
   constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
   const Lanes L(a.lpe_log2);
@@ -313,11 +320,17 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, 
     if (seg_step_begin<T, D1, V>(st, acc, a.gx, a.ws, I, off0, ei, oi, wave, R, L, a.lpe_log2, cok, C, c0)) {
       const int64_t e = ei, gr = oi;
       T x[D1][V], g[DO][V], y[D2], gy[D2];
+      T ux = 0, uy = 0, uz = 0;
+      if constexpr (YV) {
+        ux = a.y[e * 3]; uy = a.y[e * 3 + 1]; uz = a.y[e * 3 + 2];
+        const ShPoint<T> pt(ux, uy, uz, a.y_vec == kYUnitVector);
+        sh_values<T, TP::SH_LMAX>(pt.x, pt.y, pt.z, y);
+      } else {
 #pragma unroll
-      for (int j = 0; j < D2; ++j) {
-        y[j] = a.y[e * D2 + j];
-        gy[j] = T(0);
+        for (int j = 0; j < D2; ++j) y[j] = a.y[e * D2 + j];
       }
+#pragma unroll
+      for (int j = 0; j < D2; ++j) gy[j] = T(0);
       if (cok) {
 #pragma unroll
         for (int i = 0; i < D1; ++i) load_vec<T, V>(x[i], a.x + ((int64_t)st.cur * D1 + i) * C + c0);
@@ -343,10 +356,21 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, 
             });
       }
       if (a.gy) {
+        if constexpr (YV) {
+          // chain rule through the harmonics (and the normalisation): three values per edge instead of D2
 #pragma unroll
-        for (int j = 0; j < D2; ++j) {
-          const T s = group_sum(gy[j], L.lpe);
-          if (L.cl == (j & (L.lpe - 1))) a.gy[e * D2 + j] = s;
+          for (int j = 0; j < D2; ++j) gy[j] = group_sum(gy[j], L.lpe);
+          const ShPoint<T> pt(ux, uy, uz, a.y_vec == kYUnitVector);
+          T vx, vy, vz;
+          sh_pull_back<T, TP::SH_LMAX>(pt.x, pt.y, pt.z, gy, vx, vy, vz);
+          pt.pull_back(vx, vy, vz, a.y_vec == kYUnitVector);
+          if (L.cl == 0) { a.gy[e * 3] = vx; a.gy[e * 3 + 1] = vy; a.gy[e * 3 + 2] = vz; }
+        } else {
+#pragma unroll
+          for (int j = 0; j < D2; ++j) {
+            const T s = group_sum(gy[j], L.lpe);
+            if (L.cl == (j & (L.lpe - 1))) a.gy[e * D2 + j] = s;
+          }
         }
       }
     }
@@ -414,6 +438,9 @@ struct UvuEntry {
   WaveFn<T> bwd[2][3];      // [vector path][weight-gradient mode]
   WaveFn<T> seg_fwd[2];     // [vector path]
   WaveFn<T> seg_bwd[2][3];  // [vector path][weight-gradient mode]
+  int sh_lmax;              // >= 0: the second operand is laid out like harmonics of degrees 0..sh_lmax, and
+  WaveFn<T> seg_fwd_vec[2]; // the segment kernels exist in a form that evaluates them from edge vectors
+  WaveFn<T> seg_bwd_vec[2][3];
 };
 
 // Channels per lane of the vector path: the widest 16-byte-or-narrower vector whose per-lane register arrays
@@ -454,6 +481,22 @@ static UvuEntry<T> make_entry() {
   e.seg_bwd[1][0] = uvu_seg_bwd_kernel<TP, T, VB, kGwNone>;
   e.seg_bwd[1][1] = uvu_seg_bwd_kernel<TP, T, VB, kGwStore>;
   e.seg_bwd[1][2] = uvu_seg_bwd_kernel<TP, T, VB, kGwReduce>;
+  e.sh_lmax = TP::SH_LMAX;
+  if constexpr (TP::SH_LMAX >= 0) {
+    static_assert((TP::SH_LMAX + 1) * (TP::SH_LMAX + 1) == TP::D2, "harmonics layout");
+    e.seg_fwd_vec[0] = uvu_seg_fwd_kernel<TP, T, 1, true>;
+    e.seg_fwd_vec[1] = uvu_seg_fwd_kernel<TP, T, VF, true>;
+    e.seg_bwd_vec[0][0] = uvu_seg_bwd_kernel<TP, T, 1, kGwNone, true>;
+    e.seg_bwd_vec[0][1] = uvu_seg_bwd_kernel<TP, T, 1, kGwStore, true>;
+    e.seg_bwd_vec[0][2] = uvu_seg_bwd_kernel<TP, T, 1, kGwReduce, true>;
+    e.seg_bwd_vec[1][0] = uvu_seg_bwd_kernel<TP, T, VB, kGwNone, true>;
+    e.seg_bwd_vec[1][1] = uvu_seg_bwd_kernel<TP, T, VB, kGwStore, true>;
+    e.seg_bwd_vec[1][2] = uvu_seg_bwd_kernel<TP, T, VB, kGwReduce, true>;
+  } else {
+    for (auto& f : e.seg_fwd_vec) f = nullptr;
+    for (auto& r : e.seg_bwd_vec)
+      for (auto& f : r) f = nullptr;
+  }
   return e;
 }
 
@@ -500,6 +543,11 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
   if (seg && (a->n_seg >= (int64_t)1 << 31 || a->n_rows >= (int64_t)1 << 31 || a->n_x_rows >= (int64_t)1 << 31))
     return CGTP_ERR_SHAPE;  // segment mode keeps ids and rows in 32-bit registers
   if (seg && a->wave_seg && a->n_waves <= 0) return CGTP_ERR_SHAPE;
+  if (a->y_vec) {  // harmonics evaluated in the kernel: fused segment kernels of a config laid out for them
+    if (a->y_vec != kYUnitVector && a->y_vec != kYRawVector) return CGTP_ERR_SHAPE;
+    if (!seg) return CGTP_ERR_SHAPE;
+    if (tab[a->cfg].sh_lmax < 0) return CGTP_ERR_CONFIG;
+  }
   if (backward) {
     if (!a->grad_out) return CGTP_ERR_NULL;
     if (seg && a->n_x_rows != a->n_seg) return CGTP_ERR_SHAPE;
@@ -574,6 +622,7 @@ static UvuDev<T> to_dev(const cgtp_uvu_args* a, const UvuPlan& plan) {
   d.ptr = a->ptr; d.perm = a->perm; d.gather = a->gather; d.x_gather = a->x_gather; d.seg_ids = a->seg_ids; d.wave_seg = a->wave_seg;
   d.n_rows = a->n_rows; d.n_seg = a->n_seg;
   d.C = a->C; d.lpe_log2 = plan.lpe_log2; d.w_shared = a->w_shared; d.pos_per_wave = plan.pos_per_wave;
+  d.y_vec = a->y_vec;
   return d;
 }
 
@@ -626,7 +675,7 @@ static int launch_fwd(const cgtp_uvu_args* a, const UvuPlan& plan, hipStream_t s
   const int vi = plan.V > 1;
   if (a->n_seg > 0) {
     if (plan.n_waves > 0) {
-      hipLaunchKernelGGL(e.seg_fwd[vi], dim3((unsigned)((plan.n_waves + 3) / 4)), dim3(256), 0, stream, d,
+      hipLaunchKernelGGL(a->y_vec ? e.seg_fwd_vec[vi] : e.seg_fwd[vi], dim3((unsigned)((plan.n_waves + 3) / 4)), dim3(256), 0, stream, d,
                          plan.n_waves);
       if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
     }
@@ -652,7 +701,7 @@ static int launch_bwd(const cgtp_uvu_args* a, const UvuPlan& plan, hipStream_t s
     if (wred) (void)hipMemsetAsync(a->grad_w, 0, sizeof(T) * w_elems, stream);
   } else {
     const int gwm = !a->grad_w ? kGwNone : (wred ? kGwReduce : kGwStore);
-    hipLaunchKernelGGL(seg ? e.seg_bwd[vi][gwm] : e.bwd[vi][gwm], dim3((unsigned)((plan.n_waves + 3) / 4)),
+    hipLaunchKernelGGL(seg ? (a->y_vec ? e.seg_bwd_vec[vi][gwm] : e.seg_bwd[vi][gwm]) : e.bwd[vi][gwm], dim3((unsigned)((plan.n_waves + 3) / 4)),
                        dim3(256), 0, stream, d, plan.n_waves);
     if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
     if (wred) {
@@ -698,6 +747,12 @@ uint64_t cgtp_uvu_describe(int cfg, int32_t* dims) {
   if (dims)
     for (int i = 0; i < 5; ++i) dims[i] = d[i];
   return cfg < n ? t[cfg].fingerprint : b[cfg - n].fingerprint;
+}
+
+int cgtp_uvu_sh_degree(int cfg) {
+  int n = 0;
+  const UvuEntry<float>* t = entries<float>(&n);
+  return cfg >= 0 && cfg < n ? t[cfg].sh_lmax : -1;
 }
 
 int cgtp_uvu_validate(const cgtp_uvu_args* args, int backward) {

@@ -80,6 +80,26 @@ class _EdgeUvuCompiled(Function):
         return (*res, None, None, None)
 
 
+class _EdgeUvuVectors(Function):
+    """The fused kernels with the harmonics evaluated inside them: the second operand is the edge vector."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, vec: Tensor, w: Tensor, plan: EdgePlan, cfg: int, y_vec: int):
+        dims = kernels.uvu_dims(cfg)
+        out = kernels.uvu_forward(cfg, dims, x, vec, w, seg=plan.fwd_index, y_vec=y_vec)
+        ctx.save_for_backward(x, vec, w)
+        ctx.plan, ctx.cfg, ctx.dims, ctx.y_vec = plan, cfg, dims, y_vec
+        return out
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, g):
+        x, vec, w = ctx.saved_tensors
+        res = kernels.uvu_backward(ctx.cfg, ctx.dims, x, vec, w, g.contiguous(), ctx.needs_input_grad[:3],
+                                   seg=ctx.plan.bwd_index, y_vec=ctx.y_vec)
+        return (*res, None, None, None)
+
+
 class _EdgeUvuRows(Function):
     """The same composition on the row-mode kernels, for tables the fused segment kernels do not cover: per-edge
     messages from the gathered node rows, then a segment sum over the dst-sorted list; the backward forms the
@@ -135,3 +155,35 @@ def edge_tensor_product_uu(x: Tensor, sh: Tensor, weight: Tensor, plan: EdgePlan
     e, d, c = msg.shape
     fwd, bwd = plan.scale_infos()
     return sparse_scale(msg.view(1, e, d * c), fwd, bwd).view(plan.num_nodes, d, c)
+
+
+def edge_tensor_product_uu_vectors(x: Tensor, edge_vec: Tensor, weight: Tensor, plan: EdgePlan,
+                                   tp_info_forward: TensorProductInfo, normalize_input: bool = True,
+                                   tp_info_backward1: Optional[TensorProductInfo] = None,
+                                   tp_info_backward2: Optional[TensorProductInfo] = None) -> Tensor:
+    """:func:`edge_tensor_product_uu` with ``sh = SphericalHarmonics(l_max, normalize_input)(edge_vec)``
+    (``equitorch/nn/sphericals.py:31-35``) evaluated inside the edge kernels: ``edge_vec (E, 3)`` replaces the
+    ``(E, (l_max+1)^2)`` harmonics as an input, and its gradient the harmonics' gradient as an output.  ``l_max`` is
+    the degree of the second operand of ``tp_info_forward``, which must be laid out like harmonics (degrees
+    ``0..l_max`` in order).  Tables without fused kernels take the harmonics kernel followed by
+    :func:`edge_tensor_product_uu`.
+    """
+    from .sphericals import spherical_harmonics
+    _lib.require_gpu(x, edge_vec, weight)
+    if edge_vec.ndim != 2 or edge_vec.shape[1] != 3:
+        raise ValueError(f"edge_vec must be (E, 3), got {tuple(edge_vec.shape)}")
+    if plan.num_src_nodes != x.shape[0]:
+        raise _lib.CgtpError(f"plan was built for {plan.num_src_nodes} source nodes, x has {x.shape[0]}")
+    cfg = kernels.uvu_config_of(tp_info_forward)
+    mode = kernels.Y_UNIT_VECTOR if normalize_input else kernels.Y_RAW_VECTOR
+    if (cfg >= 0 and kernels.uvu_sh_degree(cfg) >= 0 and x.dtype == edge_vec.dtype == weight.dtype
+            and x.dtype in (torch.float32, torch.float64)):
+        xc, vc, wc = x.contiguous(), edge_vec.contiguous(), weight.contiguous()
+        if kernels.uvu_launchable(cfg, xc, vc, wc, segments=True, y_vec=mode):
+            return _EdgeUvuVectors.apply(xc, vc, wc, plan, cfg, mode)
+    d2 = int(kernels.coo_of(tp_info_forward).D2)
+    l_max = int(round(d2 ** 0.5)) - 1
+    if (l_max + 1) ** 2 != d2:
+        raise ValueError(f"second operand of the table has {d2} components: not a set of harmonics 0..l_max")
+    sh = spherical_harmonics(edge_vec, l_max, normalize_input=normalize_input)
+    return edge_tensor_product_uu(x, sh, weight, plan, tp_info_forward, tp_info_backward1, tp_info_backward2)

@@ -137,8 +137,9 @@ class SegIndex:
 
 
 def _uvu_args(cfg: int, x: Tensor, y: Tensor, w: Tensor, seg: Optional[SegIndex], gather: Optional[Tensor],
-              pos_per_wave: int = 0) -> UvuArgs:
+              pos_per_wave: int = 0, y_vec: int = 0) -> UvuArgs:
     a = UvuArgs()
+    a.y_vec = y_vec
     a.cfg, a.dtype, a.C = cfg, _lib.dtype_code(x.dtype), x.shape[-1]
     a.w_shared = int(w.ndim == 2)
     a.n_rows, a.n_x_rows = y.shape[0], x.shape[0]
@@ -164,7 +165,8 @@ def _workspace(a: UvuArgs, backward: int, device):
     return ws
 
 
-def uvu_launchable(cfg: int, x: Tensor, y: Tensor, w: Tensor, segments: bool = False, gathered: bool = False) -> bool:
+def uvu_launchable(cfg: int, x: Tensor, y: Tensor, w: Tensor, segments: bool = False, gathered: bool = False,
+                   y_vec: int = 0) -> bool:
     """True when both the specialised forward and backward accept these operands (dtype, channel count,
     alignment); outputs are torch allocations and therefore always aligned.  ``gathered``: row mode with the rows
     of ``x`` picked by an index."""
@@ -174,6 +176,7 @@ def uvu_launchable(cfg: int, x: Tensor, y: Tensor, w: Tensor, segments: bool = F
     a.cfg, a.dtype, a.C = cfg, _lib.dtype_code(x.dtype), x.shape[-1]
     a.w_shared = int(w.ndim == 2)
     a.n_rows = y.shape[0]
+    a.y_vec = y_vec
     dummy = 256
     a.n_x_rows = x.shape[0]
     if segments:
@@ -185,11 +188,16 @@ def uvu_launchable(cfg: int, x: Tensor, y: Tensor, w: Tensor, segments: bool = F
     return _lib.lib.cgtp_uvu_validate(C.byref(a), 1) == 0
 
 
+Y_HARMONICS, Y_UNIT_VECTOR, Y_RAW_VECTOR = 0, 1, 2
+
+
 def uvu_forward(cfg: int, dims, x: Tensor, y: Tensor, w: Tensor, seg: Optional[SegIndex] = None,
-                gather: Optional[Tensor] = None, pos_per_wave: int = 0) -> Tensor:
+                gather: Optional[Tensor] = None, pos_per_wave: int = 0, y_vec: int = 0) -> Tensor:
     """Compiled-table forward.  Row mode: ``out[r] = TP(x[gather[r] | r], y[r], w[r])``.  Segment mode:
-    ``out[s] = sum_{q in segment s} TP(x[seg.gather[q]], y[e_q], w[e_q])``."""
-    a = _uvu_args(cfg, x, y, w, seg, gather, pos_per_wave)
+    ``out[s] = sum_{q in segment s} TP(x[seg.gather[q]], y[e_q], w[e_q])``.  With ``y_vec`` (segment mode), ``y``
+    holds ``(E, 3)`` edge vectors and the kernel evaluates their harmonics itself (``Y_UNIT_VECTOR``: after
+    normalising them, ``Y_RAW_VECTOR``: as they are)."""
+    a = _uvu_args(cfg, x, y, w, seg, gather, pos_per_wave, y_vec)
     n_out_rows = a.n_seg if seg is not None else y.shape[0]
     out = torch.empty((n_out_rows, dims[2], x.shape[-1]), dtype=x.dtype, device=x.device)
     a.out = out.data_ptr()
@@ -199,11 +207,12 @@ def uvu_forward(cfg: int, dims, x: Tensor, y: Tensor, w: Tensor, seg: Optional[S
 
 
 def uvu_backward(cfg: int, dims, x: Tensor, y: Tensor, w: Tensor, g: Tensor, need, seg: Optional[SegIndex] = None,
-                 gather: Optional[Tensor] = None, pos_per_wave: int = 0, x_gather: Optional[Tensor] = None):
+                 gather: Optional[Tensor] = None, pos_per_wave: int = 0, x_gather: Optional[Tensor] = None,
+                 y_vec: int = 0):
     """Compiled-table backward -> (grad_x, grad_y, grad_w), None where ``need`` is False.  Row mode: ``gather``
     picks the row of ``g`` and ``x_gather`` the row of ``x`` of every batch row; with ``x_gather`` the returned
     grad_x is per batch row, ``(n_rows, D1, C)``."""
-    a = _uvu_args(cfg, x, y, w, seg, gather, pos_per_wave)
+    a = _uvu_args(cfg, x, y, w, seg, gather, pos_per_wave, y_vec)
     a.grad_out = g.data_ptr()
     a.x_gather = _lib.ptr(x_gather)
     if not need[0]:
@@ -218,6 +227,11 @@ def uvu_backward(cfg: int, dims, x: Tensor, y: Tensor, w: Tensor, g: Tensor, nee
     ws = _workspace(a, 1, x.device)
     _lib.check(_lib.lib.cgtp_uvu_bwd(C.byref(a), _lib.stream_ptr(x.device)), "cgtp_uvu_bwd")
     return gx, gy, gw
+
+
+def uvu_sh_degree(cfg: int) -> int:
+    """Degree L when the fused kernels of ``cfg`` can evaluate the second operand from edge vectors, else -1."""
+    return int(_lib.lib.cgtp_uvu_sh_degree(cfg))
 
 
 def uvu_dims(cfg: int):

@@ -156,6 +156,9 @@ int cgtp_uvu_num_configs(void);
 int cgtp_uvu_find(uint64_t fingerprint);
 /* Describes config `cfg`: dims (D1, D2, DO, P, NNZ) written to dims[5]; returns its fingerprint (0 if bad). */
 uint64_t cgtp_uvu_describe(int cfg, int32_t* dims);
+/* Degree L if the second operand of config `cfg` is laid out like harmonics of degrees 0..L and the fused
+ * kernels can evaluate them from edge vectors (cgtp_uvu_args.y_vec); -1 otherwise. */
+int cgtp_uvu_sh_degree(int cfg);
 
 typedef struct cgtp_uvu_args {
   int32_t cfg;             /* from cgtp_uvu_find                                                   */
@@ -171,18 +174,23 @@ typedef struct cgtp_uvu_args {
   const int64_t* gather;   /* [n_rows] row of the gathered operand (fwd: x, bwd: grad_out); row mode: per
                               row, optional; segment mode: per sorted position, required           */
   int32_t pos_per_wave;    /* segment mode without wave_seg: positions per wavefront; 0 = 32       */
-  int32_t _pad;
+  int32_t y_vec;           /* segment mode: 0 = y holds harmonics (n_rows, D2); 1 / 2 = y holds edge vectors
+                              (n_rows, 3) and the kernel evaluates the harmonics of degrees 0..sqrt(D2)-1 itself,
+                              of y / max(|y|, 1e-12) (1) or of y as it is (2); grad_y is then (n_rows, 3).  Needs a
+                              config whose second operand is laid out like harmonics (cgtp_uvu_sh_degree >= 0).
+                              Fuses SphericalHarmonics.forward (equitorch/nn/sphericals.py:31-35) into the edge
+                              kernel; no counterpart as one call in the reference                             */
   const int32_t* wave_seg; /* segment mode, optional: [n_waves + 1] first segment of every wavefront */
   int64_t n_waves;         /* number of ranges in wave_seg                                         */
   const void* x;           /* (n_x_rows, D1, C); bwd segment mode: n_x_rows == n_seg               */
-  const void* y;           /* (n_rows, D2)                                                         */
+  const void* y;           /* (n_rows, D2); (n_rows, 3) if y_vec                                   */
   const void* w;           /* (n_rows | 1, P, C)                                                   */
   /* forward */
   void* out;               /* (n_seg ? n_seg : n_rows, DO, C)                                      */
   /* backward */
   const void* grad_out;    /* (rows addressed by gather / row id, DO, C)                           */
   void* grad_x;            /* (n_seg ? n_seg : n_rows, D1, C) or NULL                              */
-  void* grad_y;            /* (n_rows, D2) or NULL                                                 */
+  void* grad_y;            /* (n_rows, D2), (n_rows, 3) if y_vec, or NULL                          */
   void* grad_w;            /* (n_rows | 1, P, C) or NULL                                           */
   void* workspace;         /* cgtp_uvu_workspace_bytes() bytes (segment mode, or bwd of a shared W) */
   const int64_t* x_gather; /* row mode backward, optional: [n_rows] row of x of every batch row (x then has

@@ -95,3 +95,45 @@ def test_full_size_properties(device):
         assert float((nrm - (2 * l + 1)).abs().max()) < 1e-4 * (2 * l + 1)
     perm = torch.randperm(n, generator=g, device=device)
     assert torch.equal(spherical_harmonics(v[perm], 6, normalize=True), y[perm])
+
+
+SH = {1: "0e+1o", 2: "0e+1o+2e", 3: "0e+1o+2e+3o", 4: "0e+1o+2e+3o+4e"}
+
+
+@pytest.mark.parametrize("lmax,channels,dtype,normalize", [
+    (2, 64, torch.float32, True), (2, 64, torch.float32, False), (3, 32, torch.float32, True),
+    (2, 20, torch.float64, True), (1, 64, torch.float32, True), (4, 32, torch.float32, True)])
+def test_edge_product_with_harmonics_evaluated_in_the_kernel(device, lmax, channels, dtype, normalize):
+    """edge_tensor_product_uu_vectors(x, edge_vec, W) against the dense oracle applied to the oracle's harmonics of
+    the (normalised) edge vectors, gathered at src and summed at dst: output and the gradients with respect to the
+    node features, the edge vectors and the per-edge weights.  lmax = 4 has no fused kernels and takes the
+    harmonics kernel followed by the row-mode kernels."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu_vectors
+    from oracle import ref_ops
+    n_nodes, n_edges = 50, 600
+    g = torch.Generator().manual_seed(100 + lmax)
+    irr = SH[lmax]
+    mod = SO3Linear(irr, irr, irr, internal_weights=False, feature_mode="uu").to(device)
+    d = (lmax + 1) ** 2
+    src = torch.randint(0, n_nodes, (n_edges,), generator=g)
+    dst = torch.randint(0, n_nodes, (n_edges,), generator=g)
+    dst[dst == 7] = 8                                            # an empty segment
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).to(dtype).double()
+    vec = (rd(n_edges, 3) * (0.5 + torch.rand(n_edges, 1, generator=g, dtype=torch.float64))).to(dtype).double()
+    T = ref_ops.dense_coupling(irr, irr, irr)
+    if dtype == torch.float64:
+        T = T.float().double()          # the compiled tables hold the reference's fp32 coefficients
+    x, ct, w = rd(n_nodes, d, channels), rd(n_nodes, d, channels), rd(n_edges, mod.num_paths, channels)
+    xr, vr, wr = (t.clone().requires_grad_(True) for t in (x, vec, w))
+    sh = ref_sh.spherical_harmonics(ref_sh.normalize(vr) if normalize else vr, lmax)
+    ref = ref_ops.scatter_sum(ref_ops.dense_u1u(T, xr[src], sh, wr), dst, n_nodes)
+    (ref * ct).sum().backward()
+    plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
+    xd, vd, wd = (t.to(device, dtype).requires_grad_(True) for t in (x, vec, w))
+    out = edge_tensor_product_uu_vectors(xd, vd, wd, plan, mod.tp_info_forward, normalize_input=normalize)
+    (out * ct.to(device, dtype)).sum().backward()
+    tol = 1e-5 if dtype == torch.float32 else 1e-11
+    for name, a, b in (("out", out, ref), ("grad_x", xd.grad, xr.grad), ("grad_vec", vd.grad, vr.grad),
+                       ("grad_w", wd.grad, wr.grad)):
+        assert_close(a, b, tol=tol, what=f"lmax={lmax} {name}")
