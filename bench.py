@@ -47,6 +47,8 @@ WORKLOADS = {
     "read": None,
     # indexed scale-segment reduction alone: the messages of BASELINE configs[1] summed to their destination nodes
     "scatter": None,
+    # spherical harmonics of 2^20 vectors up to degree 6 (forward and gradient kernels), normalisation fused
+    "sh": None,
     # plain library GEMM (torch.matmul, bf16, 8192^3): the matrix rate the box reaches, next to the vendor peak
     "gemm": None,
 }
@@ -73,6 +75,70 @@ def gemm_bench(steps, warmup):
                       "data": "synthetic", "config": {"workload": "gemm: library GEMM, calibration of the MFMA peak"},
                       "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
                                    "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None}}))
+
+
+def sh_bench(steps, warmup):
+    """SphericalHarmonics(l_max=6, normalize_input=True) forward and its gradient on 2^20 vectors: a step is one
+    forward and one backward launch through the C ABI.  Per vector the forward reads 12 B and writes 196 B, the
+    backward reads 12 + 196 B and writes 12 B."""
+    from equitorch_amd import _lib
+    dev = torch.device("cuda:0")
+    n, lmax = 1 << 20, 6
+    d = (lmax + 1) ** 2
+    gen = torch.Generator().manual_seed(0)
+    v = torch.randn(n, 3, generator=gen).to(dev)
+    g = torch.randn(n, d, generator=gen).to(dev)
+    y, gv = torch.empty(n, d, device=dev), torch.empty(n, 3, device=dev)
+    st = _lib.stream_ptr(dev)
+    fwd = lambda: _lib.check(_lib.lib.cgtp_sh_forward(v.data_ptr(), y.data_ptr(), n, lmax, 1, 1.0, _lib.F32, st))
+    bwd = lambda: _lib.check(_lib.lib.cgtp_sh_backward(v.data_ptr(), g.data_ptr(), gv.data_ptr(), n, lmax, 1, 1.0,
+                                                       _lib.F32, st))
+
+    def timed(fn):
+        evs = []
+        for _ in range(steps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        return sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+
+    for _ in range(warmup):
+        fwd(); bwd()
+    f_ms, b_ms = timed(fwd), timed(bwd)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fwd(); bwd()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    f_bytes, b_bytes = n * (3 + d) * 4, n * (6 + d) * 4
+    gbs = f_bytes / (f_ms * 1e-3) / 1e9
+    # CPU baseline: the oracle's restatement of the reference recursion, forward + autograd backward, on a sample
+    from oracle import ref_sh
+    sample = 1 << 17
+    vc = v[:sample].cpu().double().requires_grad_(True)
+    gc = g[:sample].cpu().double()
+    ref_sh.spherical_harmonics(ref_sh.normalize(vc[:16]), lmax)
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < 10.0:
+        torch.autograd.grad(ref_sh.spherical_harmonics(ref_sh.normalize(vc), lmax), vc, gc)
+        reps += 1
+    cpu = {"value": round(sample * reps / (time.perf_counter() - t0) / 1e6, 3), "unit": "Mvectors/s",
+           "cores": torch.get_num_threads(), "kind": "port",
+           "sample": f"{sample} of the {n} vectors, oracle ref_sh (float64 torch) forward + autograd backward, {cpu_model()}"}
+    print(json.dumps({"cpu_baseline": cpu, "metric": "spherical harmonics fwd+bwd Mvectors/s (lmax=6)", "value": round(n / (ms * 1e-3) / 1e6, 1),
+                      "unit": "Mvectors/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 5),
+                      "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+                      "config": {"workload": f"sh: {n} vectors, degrees 0..{lmax}, input normalised in the kernel"},
+                      "roofline": {"bound": "hbm", "kernel": "cgtp::sh_kernel<float,false>", "achieved": round(gbs, 1),
+                                   "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                                   "traffic": None, "algorithmic_bytes": f_bytes, "avg_ms": round(f_ms, 5)},
+                      "kernels": {"fwd_avg_ms": round(f_ms, 5), "fwd_GBs": round(gbs, 1), "bwd_avg_ms": round(b_ms, 5),
+                                  "bwd_GBs": round(b_bytes / (b_ms * 1e-3) / 1e9, 1)}}))
 
 
 def scatter_bench(steps, warmup):
@@ -430,6 +496,9 @@ def main():
         return
     if args.workload == "gemm":
         gemm_bench(args.steps, args.warmup)
+        return
+    if args.workload == "sh":
+        sh_bench(args.steps, args.warmup)
         return
     if args.workload == "scatter":
         scatter_bench(args.steps, args.warmup)
