@@ -49,6 +49,8 @@ WORKLOADS = {
     "scatter": None,
     # spherical harmonics of 2^20 vectors up to degree 6 (forward and gradient kernels), normalisation fused
     "sh": None,
+    # IrrepsLinear 128 -> 128 channels on 32768 x (0e+1o+2e+3o), bf16, shared weight, forward + backward
+    "irreps_linear": None,
     # plain library GEMM (torch.matmul, bf16, 8192^3): the matrix rate the box reaches, next to the vendor peak
     "gemm": None,
 }
@@ -139,6 +141,56 @@ def sh_bench(steps, warmup):
                                    "traffic": None, "algorithmic_bytes": f_bytes, "avg_ms": round(f_ms, 5)},
                       "kernels": {"fwd_avg_ms": round(f_ms, 5), "fwd_GBs": round(gbs, 1), "bwd_avg_ms": round(b_ms, 5),
                                   "bwd_GBs": round(b_bytes / (b_ms * 1e-3) / 1e9, 1)}}))
+
+
+def irreps_linear_bench(steps, warmup):
+    """IrrepsLinear(0e+1o+2e+3o -> same, 128 -> 128 channels) on 32768 rows in bf16: a step is the forward and the
+    gradients of input and weight.  On the matrix-core kernels of the fully connected product (second operand = 1).
+    The forward reads x (134 MB) and the weight, writes out (134 MB): HBM-bound at 64 flops per byte."""
+    from equitorch_amd.nn import IrrepsLinear
+    dev = torch.device("cuda:0")
+    irr, n, c = "0e+1o+2e+3o", 32768, 128
+    torch.manual_seed(0)
+    mod = IrrepsLinear(irr, irr, c, c).to(dev).to(torch.bfloat16)
+    d = mod.irreps_in_dim
+    x = torch.randn(n, d, c, device=dev).bfloat16().requires_grad_(True)
+    ct = torch.randn(n, d, c, device=dev).bfloat16()
+
+    def step():
+        return torch.autograd.grad(mod(x), (x, mod.weight), ct)
+
+    def fwd():
+        with torch.no_grad():
+            return mod(x)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    evs = []
+    for _ in range(steps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fwd()
+        b.record()
+        evs.append((a, b))
+    torch.cuda.synchronize()
+    f_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    nbytes = 2 * n * d * c * 2 + mod.weight.numel() * 2
+    gbs = nbytes / (f_ms * 1e-3) / 1e9
+    flops = 2 * n * d * c * c
+    print(json.dumps({"metric": "IrrepsLinear fwd+bwd Mrows/s (lmax=3, 128->128, bf16)", "value": round(n / (ms * 1e-3) / 1e6, 2),
+                      "unit": "Mrows/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 5),
+                      "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                      "config": {"workload": f"irreps_linear: {n} rows of {irr}, {c} -> {c} channels, shared weight (4,{c},{c})"},
+                      "roofline": {"bound": "hbm", "kernel": "cgtp::uv_kernel<UV_lin_sh3_d0,128> (forward)",
+                                   "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                   "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": nbytes,
+                                   "avg_ms": round(f_ms, 5), "fwd_TFLOPs": round(flops / (f_ms * 1e-3) / 1e12, 1)}}))
 
 
 def scatter_bench(steps, warmup):
@@ -499,6 +551,9 @@ def main():
         return
     if args.workload == "sh":
         sh_bench(args.steps, args.warmup)
+        return
+    if args.workload == "irreps_linear":
+        irreps_linear_bench(args.steps, args.warmup)
         return
     if args.workload == "scatter":
         scatter_bench(args.steps, args.warmup)

@@ -29,6 +29,9 @@ CONFIGS = OrderedDict([
     ("sh1", (_sh(1), _sh(1), _sh(1), {})),
     ("sh2", (_sh(2), _sh(2), _sh(2), {})),
     ("sh3", (_sh(3), _sh(3), _sh(3), {})),
+    # second operand = the scalar 1: channel mixing per irrep (IrrepsLinear between equal irreps)
+    ("lin_sh2", (_sh(2), _sh(2), "0e", {})),
+    ("lin_sh3", (_sh(3), _sh(3), "0e", {})),
 ])
 
 

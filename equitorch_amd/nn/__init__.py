@@ -1,7 +1,7 @@
 """Module layer (``equitorch.nn``) of the sparse tensor-product path."""
 from . import functional
-from .linears import SO3Linear
+from .linears import IrrepsLinear, IrrepWiseLinear, SO3Linear
 from .sphericals import SphericalHarmonics, SphericalToXYZ, XYZToSpherical
 from .tensor_products import TensorProduct
 
-__all__ = ["SO3Linear", "TensorProduct", "SphericalHarmonics", "XYZToSpherical", "SphericalToXYZ", "functional"]
+__all__ = ["SO3Linear", "IrrepsLinear", "IrrepWiseLinear", "TensorProduct", "SphericalHarmonics", "XYZToSpherical", "SphericalToXYZ", "functional"]

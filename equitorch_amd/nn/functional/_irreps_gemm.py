@@ -1,0 +1,296 @@
+"""Irreps-preserving channel mixing (``IrrepsLinear`` / ``IrrepWiseLinear``) as library GEMMs on strided views.
+
+The reference runs these layers on its table-driven vector-matrix kernels (``indexed_vecmat_scale_segment`` plus
+a scatter, ``equitorch/nn/functional/linears.py:494-571``).  The tables have a simple structure: a path couples
+the ``2l+1`` consecutive components of one input irrep with those of one output irrep through one ``(C_in, C_out)``
+matrix and one scale.  So every path is a plain GEMM, and this module issues it as such — the one place where a
+library GEMM (``torch.baddbmm`` / ``torch.bmm`` -> rocBLAS / hipBLASLt) is the right kernel:
+
+* shared weight ``(P, C_in, C_out)``: a batch of ``2l+1`` GEMMs ``(N, C_in) @ (C_in, C_out)``, one per component,
+  reading ``x[:, M0, :]`` and writing ``out[:, M, :]`` in place through their row strides (no gather, no scatter,
+  no intermediate);
+* per-sample weight ``(N, P, C_in, C_out)``: a batch of ``N`` GEMMs ``(2l+1, C_in) @ (C_in, C_out)``.
+
+Gradients are the same two primitives again (``mix`` with the transposed weight and exchanged row ranges for the
+input, ``outer`` for the weight), each a :class:`torch.autograd.Function` whose backward is written in terms of
+the two, so gradients of every order are available as in the reference.
+"""
+from typing import List, NamedTuple, Tuple
+
+import torch
+from torch import Tensor
+from torch.autograd import Function
+
+from ... import _lib
+from ...ops.kernels import cached
+
+
+class Path(NamedTuple):
+    w: int          # weight index
+    o0: int         # first output component
+    i0: int         # first input component
+    k: int          # number of components (2l+1)
+    scale: float
+
+
+class Group(NamedTuple):
+    """Consecutive paths whose output and input ranges advance together: one batched GEMM over ``rows`` components,
+    component ``j`` using weight ``w_of_row[j]``."""
+    o0: int
+    i0: int
+    rows: int
+    w_of_row: Tuple[int, ...]
+    scale: float
+    accumulate: bool      # an earlier group already wrote these output rows
+
+
+class LinearPlan(NamedTuple):
+    paths: Tuple[Path, ...]
+    n_paths: int
+    out_size: int
+
+    def groups(self) -> Tuple[Group, ...]:
+        out: List[Group] = []
+        written: List[Tuple[int, int]] = []
+        for p in self.paths:
+            g = out[-1] if out else None
+            hit = any(a < p.o0 + p.k and p.o0 < b for a, b in written)
+            if (g is not None and g.scale == p.scale and g.o0 + g.rows == p.o0 and g.i0 + g.rows == p.i0
+                    and not g.accumulate and not hit):
+                out[-1] = Group(g.o0, g.i0, g.rows + p.k, g.w_of_row + (p.w,) * p.k, g.scale, False)
+                written[-1] = (g.o0, g.o0 + g.rows + p.k)
+            else:
+                out.append(Group(p.o0, p.i0, p.k, (p.w,) * p.k, p.scale, hit))
+                written.append((p.o0, p.o0 + p.k))
+        return tuple(out)
+
+
+def _plan_from_entries(M, M0, ii0, scale, out_size) -> LinearPlan:
+    """Group table entries ``(M, M0, path, scale)`` by path and check that each path is a pair of consecutive
+    ranges with one scale — true for every table ``irreps_linear_infos`` builds."""
+    by_path = {}
+    for m, m0, p, s in zip(M, M0, ii0, scale):
+        by_path.setdefault(int(p), []).append((int(m), int(m0), float(s)))
+    paths = []
+    for p in sorted(by_path):
+        ent = sorted(by_path[p])
+        o0, i0, s = ent[0]
+        for j, (m, m0, sj) in enumerate(ent):
+            if m != o0 + j or m0 != i0 + j or sj != s:
+                raise _lib.CgtpError("irreps_linear: a path of the table is not a pair of consecutive component "
+                                     "ranges with a single scale")
+        paths.append(Path(p, o0, i0, len(ent), s))
+    return LinearPlan(tuple(paths), (max(by_path) + 1) if by_path else 0, int(out_size))
+
+
+def plan_of_linear_info(info) -> LinearPlan:
+    return cached(info.M_MM0, "linear_plan", lambda: _plan_from_entries(
+        info.M_MM0.tolist(), info.M0_MM0.tolist(), info.ii0_MM0.tolist(), info.scale_MM0.tolist(), info.out_size))
+
+
+def plan_of_irreps_info(info) -> LinearPlan:
+    def build():
+        seg = info.irrep_seg.tolist()
+        return LinearPlan(tuple(Path(i, seg[i], seg[i], seg[i + 1] - seg[i], 1.0) for i in range(len(seg) - 1)),
+                          len(seg) - 1, seg[-1])
+    return cached(info.irrep_seg, "irrep_wise_plan", build)
+
+
+def transposed(plan: LinearPlan, in_size: int) -> LinearPlan:
+    return LinearPlan(tuple(Path(p.w, p.i0, p.o0, p.k, p.scale) for p in plan.paths), plan.n_paths, in_size)
+
+
+_GROUPS = {}
+
+
+def _groups(plan: LinearPlan) -> Tuple[Group, ...]:
+    g = _GROUPS.get(plan)
+    if g is None:
+        if len(_GROUPS) > 256:
+            _GROUPS.clear()
+        g = _GROUPS[plan] = plan.groups()
+    return g
+
+
+_ROW_WEIGHTS = {}
+
+
+def _row_weights(grp: Group, device) -> Tensor:
+    key = (grp.w_of_row, str(device))
+    t = _ROW_WEIGHTS.get(key)
+    if t is None:
+        if len(_ROW_WEIGHTS) > 256:
+            _ROW_WEIGHTS.clear()
+        t = _ROW_WEIGHTS[key] = torch.tensor(grp.w_of_row, dtype=torch.int64, device=device)
+    return t
+
+
+def _covered(plan: LinearPlan) -> bool:
+    rows = sorted((p.o0, p.o0 + p.k) for p in plan.paths)
+    end = 0
+    for a, b in rows:
+        if a > end:
+            return False
+        end = max(end, b)
+    return end >= plan.out_size
+
+
+def _mix_raw(x: Tensor, w: Tensor, plan: LinearPlan, w_t: bool) -> Tensor:
+    """``out[n, o0+j, :] += scale * x[n, i0+j, :] @ W[(n,) p]`` for every path; ``w_t``: use ``W^T``."""
+    n, _, cin = x.shape
+    shared = w.ndim == 3
+    cout = w.shape[-2] if w_t else w.shape[-1]
+    out = (torch.empty if _covered(plan) else torch.zeros)((n, plan.out_size, cout), dtype=x.dtype, device=x.device)
+    if n == 0:
+        return out
+    for grp in _groups(plan):
+        xs, os_ = x[:, grp.i0:grp.i0 + grp.rows, :], out[:, grp.o0:grp.o0 + grp.rows, :]
+        beta = 1.0 if grp.accumulate else 0.0
+        if shared:
+            # one GEMM (N, C_in) @ (C_in, C_out) per component, batched over the components of the group
+            wb = w.index_select(0, _row_weights(grp, w.device))
+            if w_t:
+                wb = wb.transpose(1, 2)
+            ot = os_.transpose(0, 1)                                   # (rows, N, cout), rows strided by D_out * cout
+            torch.baddbmm(ot, xs.transpose(0, 1), wb, beta=beta, alpha=grp.scale, out=ot)
+        else:
+            # per sample: (rows of one path, C_in) @ (C_in, C_out); paths of a group share nothing, so go one by one
+            at = 0
+            while at < grp.rows:
+                pw = grp.w_of_row[at]
+                k = next((j for j in range(at, grp.rows) if grp.w_of_row[j] != pw), grp.rows) - at
+                wp = w[:, pw].transpose(1, 2) if w_t else w[:, pw]
+                dst = os_[:, at:at + k, :]
+                torch.baddbmm(dst, xs[:, at:at + k, :], wp, beta=beta, alpha=grp.scale, out=dst)
+                at += k
+    return out
+
+
+def _outer_raw(x: Tensor, g: Tensor, plan: LinearPlan, shared: bool) -> Tensor:
+    """``gw[(n,) p] = scale * sum_j x[n, i0+j, :]^T (x) g[n, o0+j, :]`` (summed over ``n`` when ``shared``)."""
+    n, _, cin = x.shape
+    cout = g.shape[-1]
+    if shared:
+        gw = torch.zeros((plan.n_paths, cin, cout), dtype=x.dtype, device=x.device)
+        if n:
+            for grp in _groups(plan):
+                a = x[:, grp.i0:grp.i0 + grp.rows, :].permute(1, 2, 0)          # (rows, cin, N)
+                b = g[:, grp.o0:grp.o0 + grp.rows, :].transpose(0, 1)           # (rows, N, cout)
+                gw.index_add_(0, _row_weights(grp, x.device), torch.bmm(a, b), alpha=grp.scale)
+        return gw
+    gw = torch.zeros((n, plan.n_paths, cin, cout), dtype=x.dtype, device=x.device)
+    if n:
+        for p in plan.paths:
+            dst = gw[:, p.w]
+            torch.baddbmm(dst, x[:, p.i0:p.i0 + p.k, :].transpose(1, 2), g[:, p.o0:p.o0 + p.k, :], beta=0.0,
+                          alpha=p.scale, out=dst)
+    return gw
+
+
+class _Mix(Function):
+    """out = mix(x, W): the layer itself; also the gradient with respect to x (transposed plan and weight)."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, w: Tensor, plan: LinearPlan, w_t: bool, in_size: int):
+        ctx.save_for_backward(x, w)
+        ctx.plan, ctx.w_t, ctx.in_size = plan, w_t, in_size
+        return _mix_raw(x, w, plan, w_t)
+
+    @staticmethod
+    def backward(ctx, g: Tensor):
+        x, w = ctx.saved_tensors
+        plan, w_t = ctx.plan, ctx.w_t
+        gx = gw = None
+        if ctx.needs_input_grad[0]:
+            gx = _Mix.apply(g, w, transposed(plan, ctx.in_size), not w_t, plan.out_size)
+        if ctx.needs_input_grad[1]:
+            if w_t:   # out = x W^T: the gradient of W is the outer product with the operands exchanged
+                gw = _Outer.apply(g, x, transposed(plan, ctx.in_size), w.ndim == 3)
+            else:
+                gw = _Outer.apply(x, g, plan, w.ndim == 3)
+        return gx, gw, None, None, None
+
+
+class _Outer(Function):
+    """gw = outer(x, g): gradient with respect to the weight; linear in both arguments."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, g: Tensor, plan: LinearPlan, shared: bool):
+        ctx.save_for_backward(x, g)
+        ctx.plan, ctx.shared = plan, shared
+        return _outer_raw(x.contiguous(), g.contiguous(), plan, shared)
+
+    @staticmethod
+    def backward(ctx, ggw: Tensor):
+        x, g = ctx.saved_tensors
+        plan = ctx.plan
+        gx = gg = None
+        if ctx.needs_input_grad[0]:   # d/dx sum(ggw * gw) = mix^T(g, ggw^T)
+            gx = _Mix.apply(g, ggw, transposed(plan, x.shape[1]), True, g.shape[1])
+        if ctx.needs_input_grad[1]:   # d/dg = mix(x, ggw)
+            gg = _Mix.apply(x, ggw, LinearPlan(plan.paths, plan.n_paths, g.shape[1]), False, x.shape[1])
+        return gx, gg, None, None
+
+
+def _as_tensor_product(plan: LinearPlan, in_size: int):
+    """The layer as a fully connected product with the scalar 1 as second operand (``C(l; l, 0)`` is the identity):
+    forward ``TensorProductInfo`` over parity-free irreps laid out like the plan's row ranges, or None if the
+    plan's scales are not the path normalisation such a product would carry."""
+    from ...utils import tp_infos
+
+    def layout(blocks, size):
+        irreps, index, at = [], {}, 0
+        for start, k in sorted(set(blocks)):
+            if start < at:
+                return None, None            # overlapping ranges of different irreps
+            irreps += [0] * (start - at)     # rows no path touches: scalars
+            index[start] = len(irreps)
+            irreps.append((k - 1) // 2)
+            at = start + k
+        irreps += [0] * (size - at)
+        return irreps, index
+
+    irr_out, idx_out = layout([(p.o0, p.k) for p in plan.paths], plan.out_size)
+    irr_in, idx_in = layout([(p.i0, p.k) for p in plan.paths], in_size)
+    if irr_out is None or irr_in is None or [p.w for p in plan.paths] != list(range(len(plan.paths))):
+        return None
+    path = [(idx_out[p.o0], idx_in[p.i0], 0) for p in plan.paths]
+    if path != sorted(path):
+        return None
+    info = tp_infos(irr_out, irr_in, [0], path=path)[0]
+    return info
+
+
+def _matrix_core_path(x: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anchor: Tensor):
+    """bf16 with a shared weight: the hand-written MFMA kernels of the fully connected product, if a table equal to
+    this layer's is compiled in (cgtp_uv_find); None otherwise."""
+    from . import _uvw_mfma
+    if x.dtype != torch.bfloat16 or weight.ndim != 3 or x.shape[0] == 0:
+        return None
+    info = cached(anchor, ("linear_as_tp", in_size, str(x.device)), lambda: (
+        lambda t: t.to(x.device) if t is not None else None)(_as_tensor_product(plan, in_size)))
+    if info is None or _uvw_mfma.uv_config_of(info) < 0:
+        return None
+    ones = cached(anchor, ("ones", x.shape[0], str(x.device)),
+                  lambda: torch.ones(x.shape[0], 1, dtype=torch.bfloat16, device=x.device))
+    return _uvw_mfma.try_forward(x, ones, weight, info)
+
+
+def mix(input: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anchor: Tensor = None) -> Tensor:
+    """``(..., D_in, C_in) x (P, C_in, C_out) | (N, P, C_in, C_out) -> (..., D_out, C_out)``."""
+    _lib.require_gpu(input, weight)
+    if input.dtype != weight.dtype:
+        raise _lib.CgtpError(f"input is {input.dtype} but weight is {weight.dtype}")
+    if input.shape[-2] != in_size:
+        raise _lib.CgtpError(f"input has {input.shape[-2]} components, the table expects {in_size}")
+    if weight.ndim not in (3, 4) or weight.shape[-3] != plan.n_paths or weight.shape[-2] != input.shape[-1]:
+        raise _lib.CgtpError(f"weight {tuple(weight.shape)} does not fit {plan.n_paths} paths of "
+                             f"{input.shape[-1]} input channels")
+    lead = input.shape[:-2]
+    x = input.reshape(-1, *input.shape[-2:]).contiguous()
+    if weight.ndim == 4 and weight.shape[0] != x.shape[0]:
+        raise _lib.CgtpError(f"per-sample weight has {weight.shape[0]} samples, input has {x.shape[0]}")
+    out = _matrix_core_path(x, weight, plan, in_size, anchor) if anchor is not None else None
+    if out is None:
+        out = _Mix.apply(x, weight, plan, False, in_size)
+    return out.reshape(*lead, plan.out_size, out.shape[-1])

@@ -136,3 +136,24 @@ def tensor_product_vu1(input1: Tensor, input2: Tensor, weight: Tensor,
     if input1.ndim == 3 and input2.ndim == 3 and _uv_gemm.supported(input1, input2, weight):
         return _uv_gemm.vu1(input1, input2, weight, tp_info_forward)
     return tri(spec_from_tp_info(tp_info_forward), ("u", "w", "uw"), "", input1, input2, weight)
+
+
+# ---- irreps-preserving channel mixing (reference :494-571) ------------------------------------------------------
+def irreps_linear(input: Tensor, weight: Tensor, irreps_linear_info_forward, irreps_linear_info_backward=None):
+    r"""``out[n, M, :] = sum_{(M, M0, p)} scale * input[n, M0, :] @ weight[(n,) p]`` over the entries of the table
+    (``IrrepsLinear.forward``, reference ``:528-571``): channel mixing between input and output irreps of equal
+    degree and parity.  ``weight`` is ``(P, C_in, C_out)`` or ``(N, P, C_in, C_out)``.  Runs as library GEMMs on
+    the strided component rows (``_irreps_gemm``); only the forward table is read."""
+    from . import _irreps_gemm as G
+    plan = G.plan_of_linear_info(irreps_linear_info_forward)
+    in_size = (irreps_linear_info_backward.out_size if irreps_linear_info_backward is not None
+               else input.shape[-2])
+    return G.mix(input, weight, plan, in_size, anchor=irreps_linear_info_forward.M_MM0)
+
+
+def irrep_wise_linear(input: Tensor, weight: Tensor, irreps_info):
+    r"""``out[n, M, :] = input[n, M, :] @ weight[(n,) irrep_of(M)]`` (``IrrepWiseLinear.forward``, reference
+    ``:494-526``): one channel-mixing matrix per irrep, the irreps themselves unchanged."""
+    from . import _irreps_gemm as G
+    plan = G.plan_of_irreps_info(irreps_info)
+    return G.mix(input, weight, plan, plan.out_size, anchor=irreps_info.irrep_seg)

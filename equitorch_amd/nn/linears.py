@@ -1,6 +1,7 @@
-"""``SO3Linear``: tensor product of a channelled feature with a channel-less one (edge harmonics).
+"""``SO3Linear``: tensor product of a channelled feature with a channel-less one (edge harmonics);
+``IrrepWiseLinear`` / ``IrrepsLinear``: channel mixing that leaves the irreps structure alone.
 
-Constructor, attributes, ``forward`` contract and ``repr`` follow ``equitorch/nn/linears.py:26-212``.
+Constructors, attributes, ``forward`` contracts and ``repr`` follow ``equitorch/nn/linears.py:26-411``.
 """
 import math
 from typing import Optional
@@ -11,10 +12,10 @@ from torch import Tensor
 from torch.nn import Parameter
 
 from ..irreps import check_irreps
-from ..structs import TensorProductInfo
-from ..utils._structs import tp_infos
-from .functional.linears import so3_linear_uu, so3_linear_uv
-from .init import initialize_so3_so2_linear
+from ..structs import IrrepsInfo, IrrepsLinearInfo, TensorProductInfo
+from ..utils._structs import irreps_info, irreps_linear_infos, tp_infos
+from .functional.linears import irrep_wise_linear, irreps_linear, so3_linear_uu, so3_linear_uv
+from .init import initialize_linear, initialize_so3_so2_linear
 
 
 class SO3Linear(nn.Module):
@@ -103,3 +104,117 @@ class SO3Linear(nn.Module):
                 f"feature_mode={self.feature_mode}, path_norm={self.path_norm}, "
                 f"channel_norm={self.channel_norm}, internal_weights={self.internal_weights}, "
                 f"num_paths={self.num_paths})")
+
+
+def _view_weight(weight: Tensor, shape, numel: int) -> Tensor:
+    return weight.view(-1, *shape) if weight.numel() > numel else weight.view(*shape)
+
+
+class IrrepWiseLinear(nn.Module):
+    r"""One ``(channels_in, channels_out)`` matrix per irrep of ``irreps`` applied to the channels
+    (``equitorch/nn/linears.py:215-300``): ``(..., irreps.dim, channels_in) -> (..., irreps.dim, channels_out)``,
+    weight ``(len(irreps), channels_in, channels_out)`` (or with a leading sample axis).  ``channel_norm`` divides
+    the output by ``sqrt(channels_in)``."""
+    irreps_info: IrrepsInfo
+
+    def __init__(self, irreps, channels_in, channels_out, internal_weights=True, channel_norm: bool = False):
+        super().__init__()
+        self.irreps = check_irreps(irreps)
+        self.irreps_dim = self.irreps.dim
+        self.channels_in = channels_in
+        self.channels_out = channels_out
+        self.irreps_info = irreps_info(self.irreps)
+        self.channel_norm = channel_norm
+        self.num_paths = len(self.irreps)
+        self.weight_shape = (self.num_paths, self.channels_in, self.channels_out)
+        self.weight_numel = math.prod(self.weight_shape)
+        self.internal_weights = internal_weights
+        if internal_weights:
+            self.weight = Parameter(torch.empty(*self.weight_shape))
+            initialize_linear(self.weight, channel_normed=self.channel_norm)
+        else:
+            self.weight = None
+
+    def forward(self, input: Tensor, weight: Optional[Tensor] = None):
+        assert input.shape[-2] == self.irreps_dim, \
+            f"Input spherical dim mismatch: expected {self.irreps_dim}, got {input.shape[-2]}"
+        assert input.shape[-1] == self.channels_in, \
+            f"Input channel dim mismatch: expected {self.channels_in}, got {input.shape[-1]}"
+        if self.internal_weights:
+            assert weight is None, 'Do not pass the weight when self.internal_weights is True.'
+            weight = self.weight
+        else:
+            assert weight is not None, 'Please pass the weight when self.internal_weights is False.'
+            weight = _view_weight(weight, self.weight_shape, self.weight_numel)
+        output = irrep_wise_linear(input, weight, self.irreps_info)
+        if self.channel_norm:
+            output = output / (self.channels_in ** 0.5)
+        return output
+
+    def _apply(self, *args, **kwargs):
+        tp = super()._apply(*args, **kwargs)
+        tp.irreps_info = self.irreps_info._apply(*args, **kwargs)
+        return tp
+
+    def __repr__(self):
+        return (f"{self.__class__.__name__}(irreps={self.irreps.short_repr()}, channels_in={self.channels_in}, "
+                f"channels_out={self.channels_out}, channel_norm={self.channel_norm}, "
+                f"internal_weights={self.internal_weights})")
+
+
+class IrrepsLinear(nn.Module):
+    r"""Channel mixing between input and output irreps of equal degree and compatible parity
+    (``equitorch/nn/linears.py:302-411``): ``(..., irreps_in.dim, channels_in) -> (..., irreps_out.dim,
+    channels_out)``, weight ``(num_paths, channels_in, channels_out)`` (or with a leading sample axis), one path
+    per allowed ``(irrep_out, irrep_in)`` pair.  ``path_norm`` scales each path by ``count(paths into its output
+    irrep)^-1/2``.  As in the reference, ``channel_norm`` multiplies the table scales by ``channels_in`` (the
+    value its constructor hands to the table builder) and switches the initialiser to the un-normalised range."""
+    forward_info: IrrepsLinearInfo
+    backward_info: IrrepsLinearInfo
+
+    def __init__(self, irreps_in, irreps_out, channels_in, channels_out, internal_weights=True, path_norm=True,
+                 channel_norm=False, path=None):
+        super().__init__()
+        self.irreps_in = check_irreps(irreps_in)
+        self.irreps_out = check_irreps(irreps_out)
+        self.irreps_in_dim = self.irreps_in.dim
+        self.irreps_out_dim = self.irreps_out.dim
+        self.channels_in = channels_in
+        self.channels_out = channels_out
+        self.channel_norm = channel_norm
+        self.path_norm = path_norm
+        self.forward_info, self.backward_info, self.num_paths = irreps_linear_infos(
+            self.irreps_out, self.irreps_in, path, path_norm, channel_norm, self.channels_in)
+        self.weight_shape = (self.num_paths, self.channels_in, self.channels_out)
+        self.weight_numel = math.prod(self.weight_shape)
+        self.internal_weights = internal_weights
+        if internal_weights:
+            self.weight = Parameter(torch.empty(*self.weight_shape))
+            initialize_linear(self.weight, channel_normed=channel_norm)
+        else:
+            self.weight = None
+
+    def forward(self, input: Tensor, weight: Optional[Tensor] = None):
+        assert input.shape[-2] == self.irreps_in_dim, \
+            f"Input spherical dim mismatch: expected {self.irreps_in_dim}, got {input.shape[-2]}"
+        assert input.shape[-1] == self.channels_in, \
+            f"Input channel dim mismatch: expected {self.channels_in}, got {input.shape[-1]}"
+        if self.internal_weights:
+            assert weight is None, 'Do not pass the weight when self.internal_weights is True.'
+            weight = self.weight
+        else:
+            assert weight is not None, 'Please pass the weight when self.internal_weights is False.'
+            weight = _view_weight(weight, self.weight_shape, self.weight_numel)
+        return irreps_linear(input, weight, self.forward_info, self.backward_info)
+
+    def _apply(self, *args, **kwargs):
+        tp = super()._apply(*args, **kwargs)
+        tp.forward_info = self.forward_info._apply(*args, **kwargs)
+        tp.backward_info = self.backward_info._apply(*args, **kwargs)
+        return tp
+
+    def __repr__(self):
+        return (f"{self.__class__.__name__}(irreps_in={self.irreps_in.short_repr()}, "
+                f"irreps_out={self.irreps_out.short_repr()}, channels_in={self.channels_in}, "
+                f"channels_out={self.channels_out}, path_norm={self.path_norm}, channel_norm={self.channel_norm}, "
+                f"internal_weights={self.internal_weights}, num_paths={self.num_paths})")

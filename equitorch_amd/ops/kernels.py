@@ -29,7 +29,7 @@ def cached(anchor: Tensor, key, build):
         return hit[1]
     val = build()
     ident = id(anchor)
-    ref = weakref.ref(anchor, lambda _r, k=k: _CACHE.pop(k, None))
+    ref = weakref.ref(anchor, lambda _r, k=k: _CACHE.pop(k, None) if _CACHE is not None else None)
     _CACHE[k] = (ref, val)
     return val
 

@@ -78,3 +78,32 @@ class TensorProductInfo(NamedTuple):
     info_M_kM1M2_fwd: SparseScaleInfo
     info_M_kM1M2_bwd: SparseScaleInfo
     out_size: int
+
+
+@_movable
+class IrrepsInfo(NamedTuple):
+    """Per-irrep constants of an ``Irreps`` (``equitorch/structs/__init__.py:106-111``)."""
+    rsqrt_dims: Tensor      # (num_irreps,) (2l+1)^-1/2
+    rdims: Tensor           # (num_irreps,) 1/(2l+1)
+    irrep_index: Tensor     # (dim,) irrep of every component
+    irrep_seg: Tensor       # (num_irreps+1,) first component of every irrep
+    num_irreps: int
+
+
+@_movable
+class IrrepsLinearInfo(NamedTuple):
+    """Tables of the irreps-preserving channel mixing (``equitorch/structs/__init__.py:114-130``): entries
+    ``(M, M0, path)`` sorted by output component, and the same entries sorted by path for the weight gradient."""
+    scale_MM0: Tensor
+    M_seg_MM0: Tensor
+    ii0_MM0: Tensor
+    M0_MM0: Tensor
+    M_MM0: Tensor
+    M_out: Tensor
+
+    ii0_seg_ii0MM0: Tensor
+    M_ii0MM0: Tensor
+    M0_ii0MM0: Tensor
+    scales_ii0: Tensor
+
+    out_size: int

@@ -2,8 +2,13 @@
 from ._indices import expand_left, extract_batch_segments, extract_scatter_indices, sort_by_column_key
 from ._random import rand_spherical_xyz
 from ._structs import (
+    create_irreps_linear_info,
     create_tp_info,
+    generate_fully_connected_irreps_linear_paths,
     generate_fully_connected_tp_paths,
+    irreps_info,
+    irreps_linear_infos,
+    prepare_irreps_linear,
     prepare_so3,
     sparse_product_info,
     sparse_product_infos,
@@ -16,4 +21,5 @@ __all__ = [
     "rand_spherical_xyz", "expand_left", "extract_batch_segments", "sort_by_column_key",
     "extract_scatter_indices", "sparse_scale_info", "sparse_scale_infos", "sparse_product_info",
     "sparse_product_infos", "generate_fully_connected_tp_paths", "tp_infos",
+    "generate_fully_connected_irreps_linear_paths", "irreps_linear_infos", "irreps_info",
 ]

@@ -12,8 +12,8 @@ from torch import tensor
 
 from ..constants import so3_clebsch_gordan
 from ..irreps import Irreps, check_irreps, has_path, irrep_segments
-from ..structs import SparseProductInfo, SparseScaleInfo, TensorProductInfo
-from ._indices import _lex_order
+from ..structs import IrrepsInfo, IrrepsLinearInfo, SparseProductInfo, SparseScaleInfo, TensorProductInfo
+from ._indices import _lex_order, extract_batch_segments, sort_by_column_key
 
 
 def _csr_pointer(sorted_out: np.ndarray, out_size: Optional[int], shifted: bool):
@@ -208,3 +208,73 @@ def tp_infos(irreps_out, irreps1, irreps2, path: List[Tuple[int, int, int]] = No
             create_tp_info(cg, M1, M2, M, i, j, k, w, d1, d2, do),
             create_tp_info(cg, M2, M, M1, j, k, i, w, d2, do, d1),
             num_paths)
+
+
+# ---- irreps-preserving channel mixing (IrrepsLinear / IrrepWiseLinear) ---------------------------------------
+def generate_fully_connected_irreps_linear_paths(irreps_out: Irreps, irreps_in: Irreps) -> List[Tuple[int, int]]:
+    """All ``(i_out, i_in)`` with equal degree and compatible parity (reference ``:336-343``)."""
+    return [(i, i0) for i, ir_out in enumerate(irreps_out) for i0, ir_in in enumerate(irreps_in)
+            if has_path(ir_out, ir_in)]
+
+
+def prepare_irreps_linear(irreps_out, irreps_in, path, path_norm, channel_norm, channel_scale: float = 1.0):
+    """One entry ``(scale, M, M0, i, i0, path)`` per component of every path (reference ``:346-385``).  The scale
+    is ``count(paths into i)^-1/2`` under ``path_norm`` (the Python int ``1`` otherwise, which makes the scale
+    tensors integer-typed exactly as in the reference), times ``channel_scale`` under ``channel_norm``."""
+    if not path:
+        path = generate_fully_connected_irreps_linear_paths(irreps_out, irreps_in)
+    seg_out, seg_in = irrep_segments(irreps_out), irrep_segments(irreps_in)
+    current, path_count = None, {}
+    for i, _ in path:
+        path_count[i] = path_count[i] + 1 if i == current else 1
+        current = i
+    scales, M_s, M0_s, i_s, i0_s, ii0_s = [], [], [], [], [], []
+    for w_idx, (i, i0) in enumerate(path):
+        norm_scale = path_count[i] ** (-0.5) if path_norm else 1
+        if channel_norm:
+            norm_scale *= channel_scale
+        for m in range(2 * irreps_out[i].l + 1):
+            scales.append(norm_scale)
+            M_s.append(seg_out[i] + m)
+            M0_s.append(seg_in[i0] + m)
+            i_s.append(i)
+            i0_s.append(i0)
+            ii0_s.append(w_idx)
+    return scales, M_s, M0_s, i_s, i0_s, ii0_s, len(path)
+
+
+def create_irreps_linear_info(scales, M_s, M0_s, ii0_s, out_size) -> IrrepsLinearInfo:
+    """Reference ``:387-415``: the entries sorted by ``(M, M0, path, scale)`` with the CSR pointer over distinct
+    ``M``, and sorted by ``(path, M, M0, scale)`` with the CSR pointer over paths."""
+    M_MM0, M0_MM0, ii0_MM0, scales_MM0 = sort_by_column_key([M_s, M0_s, ii0_s, scales])
+    _, M_seg_MM0, (M,) = extract_batch_segments([M_MM0])
+    ii0_ii0MM0, M_ii0MM0, M0_ii0MM0, scales_ii0MM0 = sort_by_column_key([ii0_s, M_s, M0_s, scales])
+    _, ii0_seg_ii0MM0, (_, scales_ii0) = extract_batch_segments([ii0_ii0MM0, scales_ii0MM0])
+    return IrrepsLinearInfo(tensor(scales_MM0), tensor(M_seg_MM0), tensor(ii0_MM0), tensor(M0_MM0), tensor(M_MM0),
+                            tensor(M), tensor(ii0_seg_ii0MM0), tensor(M_ii0MM0), tensor(M0_ii0MM0),
+                            tensor(scales_ii0), out_size)
+
+
+def irreps_linear_infos(irreps_out, irreps_in, path: List[Tuple[int, int]] = None, path_norm: bool = True,
+                        channel_norm: bool = False, channel_scale: float = 1.0):
+    """``(forward_info, backward_info, num_paths)`` (reference ``:432-443``); the backward tables exchange the
+    roles of input and output components."""
+    irreps_out, irreps_in = check_irreps(irreps_out), check_irreps(irreps_in)
+    scales, M_s, M0_s, _, _, ii0_s, num_paths = prepare_irreps_linear(irreps_out, irreps_in, path, path_norm,
+                                                                      channel_norm, channel_scale)
+    return (create_irreps_linear_info(scales, M_s, M0_s, ii0_s, irreps_out.dim),
+            create_irreps_linear_info(scales, M0_s, M_s, ii0_s, irreps_in.dim), num_paths)
+
+
+def irreps_info(irreps) -> IrrepsInfo:
+    """Reference ``:446-459``."""
+    irreps = check_irreps(irreps)
+    seg, idx, rsqrt_dim, rdims, acc = [], [], [], [], 0
+    for i, irrep in enumerate(irreps):
+        seg.append(acc)
+        idx.extend(irrep.dim * [i])
+        acc += irrep.dim
+        rsqrt_dim.append(irrep.dim ** (-0.5))
+        rdims.append(1 / irrep.dim)
+    seg.append(acc)
+    return IrrepsInfo(tensor(rsqrt_dim), tensor(rdims), tensor(idx), tensor(seg), len(irreps))

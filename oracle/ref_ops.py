@@ -211,3 +211,31 @@ def cpu_edge_backward(ct, x, sh, w, inter, src, dst, tp_fwd, tp_bwd1, tp_bwd2):
     gxs, gy, gw = cpu_u1u_backward(g, x.index_select(0, src), sh, w, inter, tp_fwd, tp_bwd1, tp_bwd2)
     gx = torch.zeros_like(x).index_add_(0, src, gxs)
     return gx, gy, gw
+
+
+# ---- irreps-preserving channel mixing ------------------------------------------------------------------------
+def cpu_irreps_linear(x, w, info):
+    """``IrrepsLinear.forward`` (equitorch/nn/functional/linears.py:533-546): per table entry the vector-matrix
+    product ``scale * x[n, M0] @ W[(n,) path]`` summed over the entries of each output segment
+    (``indexed_vecmat_scale_segment``), then scattered to the rows ``M_out`` of a zero ``(N, out_size, C_out)``.
+    ``info``: dict from ``ref_tables.irreps_linear_infos``; float64 loops, small cases only."""
+    n = x.shape[0]
+    seg = torch.zeros(n, len(info["M_out"]), w.shape[-1], dtype=x.dtype)
+    ptr = info["M_seg_MM0"]
+    for s in range(len(ptr) - 1):
+        for t in range(ptr[s], ptr[s + 1]):
+            wp = w[info["ii0_MM0"][t]] if w.ndim == 3 else w[:, info["ii0_MM0"][t]]
+            vec = x[:, info["M0_MM0"][t], :]
+            prod = vec @ wp if w.ndim == 3 else torch.einsum("nu,nuw->nw", vec, wp)
+            seg[:, s] = seg[:, s] + info["scale_MM0"][t] * prod
+    out = torch.zeros(n, info["out_size"], w.shape[-1], dtype=x.dtype)
+    return out.index_add(1, torch.tensor(info["M_out"], dtype=torch.int64), seg)
+
+
+def cpu_irrep_wise_linear(x, w, info):
+    """``IrrepWiseLinear.forward`` (equitorch/nn/functional/linears.py:497-509): ``sparse_vecmat`` with
+    ``index2 = irrep_index``: ``out[n, M] = x[n, M] @ W[(n,) irrep_index[M]]``."""
+    rows = []
+    for M, i in enumerate(info["irrep_index"]):
+        rows.append(x[:, M, :] @ w[i] if w.ndim == 3 else torch.einsum("nu,nuw->nw", x[:, M, :], w[:, i]))
+    return torch.stack(rows, dim=1)

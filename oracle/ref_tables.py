@@ -227,3 +227,58 @@ def tp_infos(irreps_out, irreps1, irreps2, path=None, path_norm=True, channel_no
             create_tp_info(cg, M1, M2, M, i, j, k, w, d1, d2, do),
             create_tp_info(cg, M2, M, M1, j, k, i, w, d2, do, d1),
             n_paths)
+
+
+# ---- irreps-preserving channel mixing (equitorch/utils/_structs.py:336-459) --------------------------------
+def has_linear_path(out, a):
+    """``has_path`` with two arguments (equitorch/irreps/__init__.py:237-238)."""
+    return out[0] == a[0] and (out[1] == 0 or a[1] == out[1])
+
+
+def prepare_irreps_linear(irs_out, irs_in, path=None, path_norm=True, channel_norm=False, channel_scale=1.0):
+    """:346-385.  Pinned by closed forms (tests/test_tables.py): entry count ``sum over paths of 2l+1``, scale
+    ``count^-1/2``, and the layer reducing to ``x @ W`` per irrep when every output irrep has one path."""
+    if not path:
+        path = [(i, i0) for i, o in enumerate(irs_out) for i0, a in enumerate(irs_in) if has_linear_path(o, a)]
+    seg_out, seg_in = segments(irs_out), segments(irs_in)
+    current, count = None, {}
+    for i, _ in path:
+        count[i] = count[i] + 1 if i == current else 1
+        current = i
+    scales, M_s, M0_s, ii0_s = [], [], [], []
+    for w_idx, (i, i0) in enumerate(path):
+        norm = count[i] ** (-0.5) if path_norm else 1
+        if channel_norm:
+            norm *= channel_scale
+        for m in range(2 * irs_out[i][0] + 1):
+            scales.append(norm)
+            M_s.append(seg_out[i] + m)
+            M0_s.append(seg_in[i0] + m)
+            ii0_s.append(w_idx)
+    return scales, M_s, M0_s, ii0_s, len(path)
+
+
+def create_irreps_linear_info(scales, M_s, M0_s, ii0_s, out_size):
+    """:387-415, as a dict with the field names of ``IrrepsLinearInfo``."""
+    M_MM0, M0_MM0, ii0_MM0, scales_MM0 = sort_columns([M_s, M0_s, ii0_s, scales])
+    _, M_seg, (M,) = batch_segments([M_MM0])
+    ii0_k, M_k, M0_k, scales_k = sort_columns([ii0_s, M_s, M0_s, scales])
+    _, ii0_seg, (_, scales_ii0) = batch_segments([ii0_k, scales_k])
+    return dict(scale_MM0=scales_MM0, M_seg_MM0=M_seg, ii0_MM0=ii0_MM0, M0_MM0=M0_MM0, M_MM0=M_MM0, M_out=M,
+                ii0_seg_ii0MM0=ii0_seg, M_ii0MM0=M_k, M0_ii0MM0=M0_k, scales_ii0=scales_ii0, out_size=out_size)
+
+
+def irreps_linear_infos(irreps_out, irreps_in, path=None, path_norm=True, channel_norm=False, channel_scale=1.0):
+    """:432-443 -> (forward dict, backward dict, num_paths)."""
+    io, ii = parse(irreps_out), parse(irreps_in)
+    scales, M_s, M0_s, ii0_s, n = prepare_irreps_linear(io, ii, path, path_norm, channel_norm, channel_scale)
+    return (create_irreps_linear_info(scales, M_s, M0_s, ii0_s, segments(io)[-1]),
+            create_irreps_linear_info(scales, M0_s, M_s, ii0_s, segments(ii)[-1]), n)
+
+
+def irreps_info(irreps):
+    """:446-459."""
+    irs = parse(irreps)
+    idx = [i for i, (l, _) in enumerate(irs) for _ in range(2 * l + 1)]
+    return dict(rsqrt_dims=[(2 * l + 1) ** (-0.5) for l, _ in irs], rdims=[1 / (2 * l + 1) for l, _ in irs],
+                irrep_index=idx, irrep_seg=segments(irs), num_irreps=len(irs))

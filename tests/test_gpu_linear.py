@@ -1,0 +1,117 @@
+"""GPU parity of IrrepsLinear / IrrepWiseLinear against the oracle's restatement of the reference forward and its
+autograd gradients (first and second order)."""
+import pytest
+import torch
+
+from helpers import assert_close
+from oracle import ref_ops, ref_tables
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    ("0e+1o+2e", "0e+1o+2e", {}),
+    ("0e+1o+2e", "0e+1o+1o+2e+0e", {}),
+    ("2x0e+1o+3x2e", "0e+2x1o+2e+3e", {}),
+    ("0e+1o", "0e+1e+2e", {"path_norm": False}),          # 1o has no source: zero rows
+    ("0e+1o+2e", "0e+1o+2e", {"channel_norm": True}),
+]
+
+
+def _grads(out, inputs, ct):
+    return torch.autograd.grad(out, inputs, ct)
+
+
+@pytest.mark.parametrize("io,ii,kw", CASES)
+@pytest.mark.parametrize("shared", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_irreps_linear_matches_oracle(device, io, ii, kw, shared, dtype):
+    from equitorch_amd.nn import IrrepsLinear
+    n, cin, cout = 37, 24, 40
+    mod = IrrepsLinear(ii, io, cin, cout, internal_weights=False, **kw).to(device)
+    okw = dict(kw)
+    if okw.get("channel_norm"):
+        okw["channel_scale"] = cin            # what the reference's constructor passes (nn/linears.py:357-358)
+    info = ref_tables.irreps_linear_infos(io, ii, **okw)[0]
+    # the reference stores the scales with torch.tensor(list): fp32 values, also under fp64 inputs
+    info["scale_MM0"] = torch.tensor(info["scale_MM0"]).double().tolist()
+    g = torch.Generator().manual_seed(1)
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).to(dtype).double()
+    x = rd(n, mod.irreps_in_dim, cin)
+    w = rd(*(() if shared else (n,)), mod.num_paths, cin, cout)
+    ct = rd(n, mod.irreps_out_dim, cout)
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    ref = ref_ops.cpu_irreps_linear(xr, wr, info)
+    rgx, rgw = _grads(ref, (xr, wr), ct)
+    xd, wd = (t.to(device, dtype).requires_grad_(True) for t in (x, w))
+    out = mod(xd, wd)
+    gx, gw = _grads(out, (xd, wd), ct.to(device, dtype))
+    tol = 1e-5 if dtype == torch.float32 else 1e-12
+    for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
+        assert_close(a, b, tol=tol, what=f"{io}<-{ii} shared={shared} {name}")
+
+
+@pytest.mark.parametrize("shared", [True, False])
+def test_irrep_wise_linear_matches_oracle_and_leading_dims(device, shared):
+    from equitorch_amd.nn import IrrepWiseLinear
+    irr, cin, cout = "0e+1o+2e+1o", 16, 8
+    mod = IrrepWiseLinear(irr, cin, cout, internal_weights=False, channel_norm=True).to(device)
+    info = ref_tables.irreps_info(irr)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(3, 5, 12, cin, generator=g, dtype=torch.float64)
+    w = torch.randn(*(() if shared else (15,)), 4, cin, cout, generator=g, dtype=torch.float64)
+    ct = torch.randn(3, 5, 12, cout, generator=g, dtype=torch.float64)
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    ref = ref_ops.cpu_irrep_wise_linear(xr.reshape(15, 12, cin), wr, info).reshape(3, 5, 12, cout) / cin ** 0.5
+    rgx, rgw = _grads(ref, (xr, wr), ct)
+    xd, wd = (t.to(device).requires_grad_(True) for t in (x, w))
+    out = mod(xd, wd.reshape(-1) if shared else wd)       # a flat weight is viewed to (P, C_in, C_out)
+    gx, gw = _grads(out, (xd, wd), ct.to(device))
+    for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
+        assert_close(a, b, tol=1e-12, what=f"irrep-wise shared={shared} {name}")
+
+
+def test_internal_weights_bf16_and_second_order(device):
+    from equitorch_amd.nn import IrrepsLinear
+    torch.manual_seed(0)
+    mod = IrrepsLinear("0e+1o+2e", "0e+1o+2e", 32, 32).to(device)
+    assert mod.weight.shape == (3, 32, 32) and float(mod.weight.detach().abs().max()) <= (3.0 / 32) ** 0.5
+    x = torch.randn(64, 9, 32, device=device)
+    ref = torch.cat([x[:, a:b] @ mod.weight[p] for p, (a, b) in enumerate([(0, 1), (1, 4), (4, 9)])], dim=1)
+    assert_close(mod(x), ref, tol=1e-5, what="internal weights")
+    out16 = mod.to(torch.bfloat16)(x.bfloat16())
+    assert out16.dtype == torch.bfloat16
+    assert float((out16.float() - ref).detach().abs().max()) <= 1e-2 * max(1.0, float(ref.detach().abs().max()))
+    # second order: gradgradcheck of the two primitives in fp64 on a tiny case
+    mod64 = IrrepsLinear("0e+1o+1o", "0e+1o", 3, 2, internal_weights=False).to(device)
+    xs = torch.randn(4, 7, 3, device=device, dtype=torch.float64, requires_grad=True)
+    for shape in ((3, 3, 2), (4, 3, 3, 2)):
+        ws = torch.randn(*shape, device=device, dtype=torch.float64, requires_grad=True)
+        assert torch.autograd.gradcheck(mod64, (xs, ws))
+        assert torch.autograd.gradgradcheck(mod64, (xs, ws))
+    with pytest.raises(Exception):
+        mod64(torch.randn(4, 7, 3), torch.randn(3, 3, 2))     # CPU tensors are rejected
+
+
+@pytest.mark.parametrize("irr,cin,cout,n", [("0e+1o+2e+3o", 128, 128, 1100), ("0e+1o+2e", 64, 32, 700)])
+def test_bf16_shared_weight_runs_on_the_matrix_core_kernels(device, irr, cin, cout, n):
+    """bf16 with a shared weight and a compiled-in table: the MFMA kernels of the fully connected product with the
+    scalar 1 as second operand.  Output and both gradients within rel 1e-2 of the fp64 oracle."""
+    from equitorch_amd.nn import IrrepsLinear
+    from equitorch_amd.nn.functional import _irreps_gemm as G, _uvw_mfma
+    mod = IrrepsLinear(irr, irr, cin, cout, internal_weights=False).to(device)
+    plan = G.plan_of_linear_info(mod.forward_info)
+    assert _uvw_mfma.uv_config_of(G._as_tensor_product(plan, mod.irreps_in_dim)) >= 0
+    info = ref_tables.irreps_linear_infos(irr, irr)[0]
+    g = torch.Generator().manual_seed(3)
+    rd = lambda *s: torch.randn(*s, generator=g).bfloat16().double()
+    x, w, ct = rd(n, mod.irreps_in_dim, cin), rd(mod.num_paths, cin, cout) / cin ** 0.5, rd(n, mod.irreps_out_dim, cout)
+    w = w.bfloat16().double()
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    ref = ref_ops.cpu_irreps_linear(xr, wr, info)
+    rgx, rgw = _grads(ref, (xr, wr), ct)
+    xd, wd = (t.to(device, torch.bfloat16).requires_grad_(True) for t in (x, w))
+    out = mod(xd, wd)
+    gx, gw = _grads(out, (xd, wd), ct.to(device, torch.bfloat16))
+    for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
+        assert a.dtype == torch.bfloat16
+        assert_close(a.float(), b, tol=1e-2, what=f"bf16 {irr} {name}")
