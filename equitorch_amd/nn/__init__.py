@@ -1,7 +1,11 @@
 """Module layer (``equitorch.nn``) of the sparse tensor-product path."""
 from . import functional
+from .activations import Gate
 from .linears import IrrepsLinear, IrrepWiseLinear, SO3Linear
+from .norm import MeanSquaredNorm, Norm, SquaredNorm
+from .normalization import BatchRMSNorm, LayerRMSNorm
 from .sphericals import SphericalHarmonics, SphericalToXYZ, XYZToSpherical
 from .tensor_products import TensorProduct
 
-__all__ = ["SO3Linear", "IrrepsLinear", "IrrepWiseLinear", "TensorProduct", "SphericalHarmonics", "XYZToSpherical", "SphericalToXYZ", "functional"]
+__all__ = ["SO3Linear", "IrrepsLinear", "IrrepWiseLinear", "TensorProduct", "SphericalHarmonics", "XYZToSpherical", "SphericalToXYZ", "Gate", "SquaredNorm", "Norm", "MeanSquaredNorm",
+           "BatchRMSNorm", "LayerRMSNorm", "functional"]

@@ -1,7 +1,10 @@
 """Functional layer (``equitorch.nn.functional``) of the sparse tensor-product path."""
+from .activations import gating
 from .edge import EdgePlan, edge_tensor_product_uu, edge_tensor_product_uu_vectors
 from .linears import (irrep_wise_linear, irreps_linear, so3_linear_uu, so3_linear_uv, tensor_product_1uu, tensor_product_1vu, tensor_product_u1u,
                       tensor_product_u1v, tensor_product_uu1, tensor_product_vu1)
+from .norm import batch_mean_squared_norm, channel_mean_squared_norm, norm, squared_norm
+from .normalization import batch_rms_norm, layer_rms_norm
 from .sparse_product import (sparse_inner, sparse_mat_t_vec, sparse_mul, sparse_outer, sparse_scavec, sparse_vecmat,
                              sparse_vecsca)
 from .sparse_scale import sparse_scale
@@ -13,5 +16,6 @@ __all__ = [
     "tensor_product_u1v", "tensor_product_1vu", "tensor_product_vu1", "so3_linear_uu", "so3_linear_uv", "irreps_linear", "irrep_wise_linear",
     "sparse_mul", "sparse_outer", "sparse_inner", "sparse_vecmat", "sparse_vecsca", "sparse_scavec",
     "sparse_mat_t_vec", "sparse_scale", "EdgePlan", "edge_tensor_product_uu", "edge_tensor_product_uu_vectors", "spherical_harmonics",
-    "xyz_to_spherical", "spherical_to_xyz",
+    "xyz_to_spherical", "spherical_to_xyz", "gating", "squared_norm", "norm", "channel_mean_squared_norm",
+    "batch_mean_squared_norm", "batch_rms_norm", "layer_rms_norm",
 ]

@@ -239,3 +239,60 @@ def cpu_irrep_wise_linear(x, w, info):
     for M, i in enumerate(info["irrep_index"]):
         rows.append(x[:, M, :] @ w[i] if w.ndim == 3 else torch.einsum("nu,nuw->nw", x[:, M, :], w[:, i]))
     return torch.stack(rows, dim=1)
+
+
+# ---- gates, norms, RMS normalisation (pure torch float64; autograd gives the gradient oracle) -----------------
+def _block_sum(t, seg):
+    """``torch_geometric.utils.segment(t, ptr)`` along dim -2, as a slice-and-sum (cf. ``segment_csr`` above)."""
+    return torch.stack([t[..., seg[i]:seg[i + 1], :].sum(dim=-2) for i in range(len(seg) - 1)], dim=-2)
+
+
+def cpu_gating(x, gates, info):
+    """``gating`` (equitorch/nn/functional/activations.py:9-35): ``x[n, M, c] * gates[(n,) irrep_index[M], c]``."""
+    idx = torch.tensor(info["irrep_index"], dtype=torch.int64)
+    return x * gates.index_select(-2, idx)
+
+
+def cpu_squared_norm(x, info, scaled=True):
+    """``SquaredNorm.forward`` (equitorch/nn/functional/norm.py:22-37)."""
+    out = _block_sum(x.pow(2), info["irrep_seg"])
+    return out * torch.tensor(info["rdims"], dtype=x.dtype).unsqueeze(-1) if scaled else out
+
+
+def cpu_norm(x, info, scaled=True):
+    """``Norm.forward`` (:80-98); its backward (:100-126) puts a zero gradient at zero blocks."""
+    out = torch.sqrt(_block_sum(x.pow(2), info["irrep_seg"]))
+    return out * torch.tensor(info["rsqrt_dims"], dtype=x.dtype).unsqueeze(-1) if scaled else out
+
+
+def cpu_channel_mean_squared_norm(x, info, scaled=True):
+    """``ChannelMeanSquaredNorm.forward`` (:139-160)."""
+    out = _block_sum(x.pow(2), info["irrep_seg"]).sum(dim=-1) / x.shape[-1]
+    return out * torch.tensor(info["rdims"], dtype=x.dtype) if scaled else out
+
+
+def cpu_batch_mean_squared_norm(x, info, scaled=True):
+    """``BatchMeanSquaredNorm.forward`` (:200-224)."""
+    out = _block_sum(x.pow(2), info["irrep_seg"]).sum(dim=0) / x.shape[0]
+    return out * torch.tensor(info["rdims"], dtype=x.dtype).unsqueeze(-1) if scaled else out
+
+
+def cpu_batch_rms_norm(x, running, info, weight=None, scaled=True, training=False, momentum=0.1, eps=1e-5):
+    """``batch_rms_norm`` (equitorch/nn/functional/normalization.py:10-72) -> (output, updated running statistic)."""
+    if training:
+        stat = cpu_squared_norm(x, info, scaled).mean(dim=0)
+        running = torch.lerp(running, stat.detach(), momentum)
+    else:
+        stat = running
+    scale = torch.rsqrt(stat + eps)
+    if weight is not None:
+        scale = weight * scale
+    return cpu_gating(x, scale, info), running
+
+
+def cpu_layer_rms_norm(x, info, weight=None, scaled=True, eps=1e-5):
+    """``layer_rms_norm`` (:75-118)."""
+    rsigma = torch.rsqrt(cpu_channel_mean_squared_norm(x, info, scaled) + eps)
+    idx = torch.tensor(info["irrep_index"], dtype=torch.int64)
+    out = x * rsigma.index_select(-1, idx).unsqueeze(-1)
+    return out if weight is None else cpu_gating(out, weight, info)

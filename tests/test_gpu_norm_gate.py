@@ -1,0 +1,117 @@
+"""GPU parity of Gate, the invariant norms and the RMS normalisation layers against the oracle (float64 torch
+restatement of the reference's forwards; autograd of the oracle for the gradients)."""
+import pytest
+import torch
+
+from helpers import assert_close
+from oracle import ref_ops, ref_tables
+
+pytestmark = pytest.mark.gpu
+
+IRR = "0e+1o+2e+1o"      # dim 12, 4 irreps
+
+
+def _info():
+    """The oracle's tables with 1/dim and dim^-1/2 rounded to fp32, which is how the reference stores them
+    (``torch.tensor(list)``), also when the features are fp64."""
+    info = ref_tables.irreps_info(IRR)
+    for k in ("rdims", "rsqrt_dims"):
+        info[k] = torch.tensor(info[k]).double().tolist()
+    return info
+
+
+def _data(n, c, dtype, seed=0, extra=0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(n, 12 + extra, c, generator=g, dtype=torch.float64).to(dtype).double(), g
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("shared", [False, True])
+def test_gate(device, dtype, shared):
+    from equitorch_amd.nn import Gate
+    info = _info()
+    x, g = _data(33, 20, dtype)
+    gate = torch.randn(*(() if shared else (33,)), 4, 20, generator=g, dtype=torch.float64).to(dtype).double()
+    ct = torch.randn(33, 12, 20, generator=g, dtype=torch.float64).to(dtype).double()
+    act = torch.nn.Sigmoid()
+    xr, gr = x.clone().requires_grad_(True), gate.clone().requires_grad_(True)
+    ref = ref_ops.cpu_gating(xr, act(gr), info)
+    rg = torch.autograd.grad(ref, (xr, gr), ct)
+    mod = Gate(IRR, activation=act).to(device)
+    xd, gd = (t.to(device, dtype).requires_grad_(True) for t in (x, gate))
+    out = mod(xd, gd)
+    got = torch.autograd.grad(out, (xd, gd), ct.to(device, dtype))
+    tol = 1e-5 if dtype == torch.float32 else 1e-12
+    for name, a, b in (("out", out, ref), ("grad_x", got[0], rg[0]), ("grad_gate", got[1], rg[1])):
+        assert_close(a, b, tol=tol, what=f"gate shared={shared} {name}")
+    if not shared:      # concatenated input and the global (not irrep-wise) gate
+        cat = torch.cat([x, gate], dim=1).to(device, dtype)
+        assert_close(mod(cat), ref, tol=tol, what="concatenated gates")
+        glob = Gate(IRR, irrep_wise=False).to(device)
+        assert_close(glob(xd, gd[:, :1]), x * gate[:, :1], tol=tol, what="global gate")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("scaled", [True, False])
+def test_norms(device, dtype, scaled):
+    from equitorch_amd.nn import MeanSquaredNorm, Norm, SquaredNorm
+    info = _info()
+    x, g = _data(41, 24, dtype, seed=1)
+    x[3, 1:4] = 0.0                      # a zero block: the norm's gradient there is zero, not nan
+    tol = 1e-5 if dtype == torch.float32 else 1e-12
+    cases = [("squared", SquaredNorm(IRR, scaled), ref_ops.cpu_squared_norm),
+             ("norm", Norm(IRR, scaled), ref_ops.cpu_norm),
+             ("channel mean", MeanSquaredNorm(IRR, scaled, dim=-1), ref_ops.cpu_channel_mean_squared_norm),
+             ("batch mean", MeanSquaredNorm(IRR, scaled, dim=0), ref_ops.cpu_batch_mean_squared_norm)]
+    for name, mod, ref_fn in cases:
+        xr = x.clone().requires_grad_(True)
+        ref = ref_fn(xr, info, scaled)
+        ct = torch.randn(ref.shape, generator=g, dtype=torch.float64).to(dtype).double()
+        (rgx,) = torch.autograd.grad(ref, xr, ct)
+        rgx = torch.nan_to_num(rgx, nan=0.0)            # sqrt at the zero block: the reference defines 0
+        xd = x.to(device, dtype).requires_grad_(True)
+        out = mod.to(device)(xd)
+        (gx,) = torch.autograd.grad(out, xd, ct.to(device, dtype))
+        assert torch.isfinite(gx).all()
+        assert_close(out, ref, tol=tol, what=f"{name} scaled={scaled}")
+        assert_close(gx, rgx, tol=tol, what=f"{name} scaled={scaled} grad")
+
+
+@pytest.mark.parametrize("affine", [True, False])
+def test_rms_normalisation_layers(device, affine):
+    from equitorch_amd.nn import BatchRMSNorm, LayerRMSNorm
+    info = _info()
+    x, g = _data(29, 16, torch.float64, seed=2)
+    ct = torch.randn(29, 12, 16, generator=g, dtype=torch.float64)
+    w = (1 + 0.3 * torch.randn(4, 16, generator=g, dtype=torch.float64)) if affine else None
+    # layer norm
+    mod = LayerRMSNorm(IRR, 16, affine=affine).to(device).double()
+    if affine:
+        mod.weight.data.copy_(w)
+    xr = x.clone().requires_grad_(True)
+    ref = ref_ops.cpu_layer_rms_norm(xr, info, w)
+    (rgx,) = torch.autograd.grad(ref, xr, ct)
+    xd = x.to(device).requires_grad_(True)
+    out = mod(xd)
+    (gx,) = torch.autograd.grad(out, xd, ct.to(device))
+    assert_close(out, ref, tol=1e-12, what="layer rms")
+    assert_close(gx, rgx, tol=1e-11, what="layer rms grad")
+    # batch norm: training step (statistics of the batch, running average updated), then evaluation
+    bn = BatchRMSNorm(IRR, 16, affine=affine, momentum=0.2).to(device).double()
+    if affine:
+        bn.weight.data.copy_(w)
+    xr = x.clone().requires_grad_(True)
+    ref, running = ref_ops.cpu_batch_rms_norm(xr, torch.ones(4, 16, dtype=torch.float64), info, w, training=True,
+                                              momentum=0.2)
+    (rgx,) = torch.autograd.grad(ref, xr, ct)
+    xd = x.to(device).requires_grad_(True)
+    out = bn(xd)
+    (gx,) = torch.autograd.grad(out, xd, ct.to(device))
+    assert_close(out, ref, tol=1e-12, what="batch rms (training)")
+    assert_close(gx, rgx, tol=1e-11, what="batch rms grad")
+    assert_close(bn.running_squared_norm, running, tol=1e-12, what="running statistic")
+    bn.eval()
+    ref_eval, _ = ref_ops.cpu_batch_rms_norm(x, running, info, w, training=False)
+    assert_close(bn(x.to(device)), ref_eval, tol=1e-12, what="batch rms (evaluation)")
+    with pytest.raises(ValueError):
+        bn(x.to(device)[:, :5])
