@@ -1,5 +1,6 @@
 """Functional layer (``equitorch.nn.functional``) of the sparse tensor-product path."""
 from .activations import gating
+from .cutoffs import cosine_cutoff, mollifier_cutoff, polynomial_cutoff, radial_standarize
 from .edge import EdgePlan, edge_tensor_product_uu, edge_tensor_product_uu_vectors
 from .linears import (irrep_wise_linear, irreps_linear, so3_linear_uu, so3_linear_uv, tensor_product_1uu, tensor_product_1vu, tensor_product_u1u,
                       tensor_product_u1v, tensor_product_uu1, tensor_product_vu1)
@@ -17,5 +18,6 @@ __all__ = [
     "sparse_mul", "sparse_outer", "sparse_inner", "sparse_vecmat", "sparse_vecsca", "sparse_scavec",
     "sparse_mat_t_vec", "sparse_scale", "EdgePlan", "edge_tensor_product_uu", "edge_tensor_product_uu_vectors", "spherical_harmonics",
     "xyz_to_spherical", "spherical_to_xyz", "gating", "squared_norm", "norm", "channel_mean_squared_norm",
-    "batch_mean_squared_norm", "batch_rms_norm", "layer_rms_norm",
+    "batch_mean_squared_norm", "batch_rms_norm", "layer_rms_norm", "radial_standarize", "polynomial_cutoff",
+    "cosine_cutoff", "mollifier_cutoff",
 ]

@@ -1,0 +1,26 @@
+"""Radial basis (``equitorch/nn/radials.py``)."""
+import math
+
+import torch
+from torch import Tensor, nn
+
+
+class BesselBasis(nn.Module):
+    r"""``b_n(r) = (2 / r_max) sin(n pi r / r_max) / r`` for ``n = 1..num_basis`` (reference ``:10-58``); the
+    frequencies ``n pi`` are a parameter when ``trainable``, a buffer otherwise.  ``(...,) -> (..., num_basis)``."""
+
+    def __init__(self, r_max, num_basis=8, trainable=True):
+        super().__init__()
+        self.trainable = trainable
+        self.num_basis = num_basis
+        self.r_max = float(r_max)
+        self.prefactor = 2.0 / self.r_max
+        freq = torch.linspace(start=1.0, end=num_basis, steps=num_basis) * math.pi
+        if trainable:
+            self.bessel_weights = nn.Parameter(freq)
+        else:
+            self.register_buffer("bessel_weights", freq)
+
+    def forward(self, x: Tensor) -> Tensor:
+        r = x.unsqueeze(-1)
+        return self.prefactor * (torch.sin(self.bessel_weights * r / self.r_max) / r)

@@ -1,0 +1,42 @@
+"""Radial basis and cutoff envelopes (plain tensor expressions, as in the reference) against what their definitions
+fix: boundary values, vanishing derivatives, known points, orthogonality of the Bessel functions."""
+import math
+
+import torch
+
+from equitorch_amd.nn.radials import BesselBasis
+from equitorch_amd.nn.cutoffs import CosineCutoff, MollifierCutoff, PolynomialCutoff
+
+
+def test_bessel_basis_values_and_orthogonality():
+    basis = BesselBasis(r_max=4.0, num_basis=6, trainable=False).double()
+    r = torch.tensor([0.5, 1.0, 2.0, 3.9], dtype=torch.float64)
+    out = basis(r)
+    n = torch.arange(1, 7, dtype=torch.float64)
+    torch.testing.assert_close(out, 0.5 * torch.sin(n * math.pi * r[:, None] / 4.0) / r[:, None])
+    # int_0^R b_n b_m r^2 dr = (2 / R) delta_nm for these functions (midpoint rule on a fine grid)
+    grid = (torch.arange(20000, dtype=torch.float64) + 0.5) * (4.0 / 20000)
+    b = basis(grid)
+    gram = (b[:, :, None] * b[:, None, :] * grid[:, None, None] ** 2).sum(0) * (4.0 / 20000)
+    torch.testing.assert_close(gram, 0.5 * torch.eye(6, dtype=torch.float64), atol=1e-6, rtol=0)
+    assert isinstance(BesselBasis(4.0).bessel_weights, torch.nn.Parameter)
+
+
+def test_cutoffs_boundary_behaviour():
+    r = torch.tensor([0.0, 1.0, 2.5, 4.0, 5.0], dtype=torch.float64, requires_grad=True)
+    poly = PolynomialCutoff(r_max=4.0, r_min=1.0, p=6)(r).detach()
+    assert poly[0] == 1 and poly[1] == 1 and abs(float(poly[3])) < 1e-12 and poly[4] == 0
+    u = torch.tensor(0.5, dtype=torch.float64)
+    expect = 1 - 28 * u ** 6 + 48 * u ** 7 - 21 * u ** 8
+    torch.testing.assert_close(poly[2], expect)
+    # first and second derivative vanish at both ends of the interval
+    x = torch.tensor([1.0 + 1e-9, 4.0 - 1e-9], dtype=torch.float64, requires_grad=True)
+    y = PolynomialCutoff(4.0, 1.0, 6)(x)
+    (g1,) = torch.autograd.grad(y.sum(), x, create_graph=True)
+    (g2,) = torch.autograd.grad(g1.sum(), x)
+    assert g1.abs().max() < 1e-6 and g2.abs().max() < 1e-5
+    cos = CosineCutoff(r_max=4.0)(r.detach())
+    torch.testing.assert_close(cos[:4], 0.5 * (1 + torch.cos(math.pi * r.detach()[:4] / 4.0)))
+    assert cos[4] == 0
+    mol = MollifierCutoff(r_max=4.0, eps=1e-7)(r.detach())
+    assert abs(float(mol[0]) - 1) < 1e-6 and float(mol[3]) < 1e-12 and float(mol[2]) == math.exp(1 - 1 / (1 - 0.625 ** 2 + 1e-7))
