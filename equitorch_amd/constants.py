@@ -116,3 +116,17 @@ def so3_clebsch_gordan(l: int, l1: int, l2: int) -> np.ndarray:
                 out[m, a, b] = _eval_sqrt_sum(re)
     out.setflags(write=False)
     return out
+
+
+@functools.lru_cache(maxsize=None)
+def j_matrix(l: int) -> np.ndarray:
+    """Real-basis Wigner matrix of the rotation that exchanges the y and z axes and reverses x
+    (``equitorch/constants/__init__.py:13-36``): ``J_1`` is written down, higher degrees follow from
+    ``J_l = C(l; 1, l-1) (J_1 (x) J_{l-1}) C(l; 1, l-1)^T``.  With it every rotation is
+    ``D(alpha, beta, gamma) = Z(alpha) J Z(beta) J Z(gamma)`` where ``Z`` mixes only the ``+-m`` pairs."""
+    if l == 0:
+        return np.ones((1, 1))
+    if l == 1:
+        return np.array([[0.0, 1.0, 0.0], [1.0, 0.0, 0.0], [0.0, 0.0, -1.0]])
+    cg = so3_clebsch_gordan(l, 1, l - 1)
+    return np.einsum("iI,jJ,kij,KIJ->kK", j_matrix(1), j_matrix(l - 1), cg, cg)

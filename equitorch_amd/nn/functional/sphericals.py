@@ -6,6 +6,7 @@ import torch
 from torch import Tensor
 
 from ...ops.spherical_harmonics import spherical_harmonics as _spherical_harmonics
+from .angular import sincos
 
 _INV_SQRT_4PI = 1.0 / (2.0 * math.sqrt(math.pi))
 
@@ -40,3 +41,12 @@ def spherical_to_xyz(theta: Tensor, phi: Tensor, r: Optional[Tensor] = None, dim
     st = torch.sin(theta)
     xyz = torch.stack([st * torch.cos(phi), st * torch.sin(phi), torch.cos(theta)], dim=dim)
     return xyz if r is None else xyz * r.unsqueeze(dim)
+
+
+def xyz_to_sincos(xyz: Tensor, max_m: int, normalize_input: bool = True, component_normalize: bool = False,
+                  eps: float = 1e-14, dim: int = -1):
+    """``(sincos(theta), sincos(phi))`` of the polar angles of ``xyz``
+    (``equitorch/nn/functional/sphericals.py:116-156``)."""
+    theta, phi = xyz_to_spherical(xyz, normalize_input=normalize_input, with_r=False, eps=eps, dim=dim)
+    return (sincos(theta, max_m, component_normalize=component_normalize),
+            sincos(phi, max_m, component_normalize=component_normalize))

@@ -13,8 +13,9 @@ from torch.nn import Parameter
 
 from ..irreps import check_irreps
 from ..structs import IrrepsInfo, IrrepsLinearInfo, TensorProductInfo
-from ..utils._structs import irreps_info, irreps_linear_infos, tp_infos
+from ..utils._structs import irreps_info, irreps_linear_infos, so2_linear_infos, tp_infos
 from .functional.linears import irrep_wise_linear, irreps_linear, so3_linear_uu, so3_linear_uv
+from .functional.sparse_product import sparse_mul, sparse_vecmat
 from .init import initialize_linear, initialize_so3_so2_linear
 
 
@@ -218,3 +219,70 @@ class IrrepsLinear(nn.Module):
                 f"irreps_out={self.irreps_out.short_repr()}, channels_in={self.channels_in}, "
                 f"channels_out={self.channels_out}, path_norm={self.path_norm}, channel_norm={self.channel_norm}, "
                 f"internal_weights={self.internal_weights}, num_paths={self.num_paths})")
+
+
+class SO2Linear(nn.Module):
+    r"""Linear map between features expressed in the frame where the edge points along z
+    (``equitorch/nn/linears.py:413-571``): components of equal ``|m|`` mix, with one weight for ``m = 0`` and a
+    ``(w_+, w_-)`` pair acting like a complex number on the ``(+m, -m)`` pair otherwise, for every path
+    ``(irrep_out, irrep_in)`` and ``m <= min(l_out, l_in)``.  ``feature_mode='uu'``: weight ``(num_weights, C)``,
+    channel-wise; ``'uv'``: weight ``(num_weights, C_in, C_out)``; either may carry a leading sample axis."""
+
+    def __init__(self, irreps_in, irreps_out, channels_in=None, channels_out=None, internal_weights=True,
+                 feature_mode='uu', path_norm=True, channel_norm=False, path=None):
+        super().__init__()
+        self.irreps_in = check_irreps(irreps_in)
+        self.irreps_out = check_irreps(irreps_out)
+        assert not internal_weights or (channels_in is not None and channels_out is not None)
+        if feature_mode not in ('uu', 'uv'):
+            raise ValueError(f'Feature_mode should be in ["uv", "uu"], got {feature_mode}.')
+        self.channels_in, self.channels_out = channels_in, channels_out
+        self.internal_weights = internal_weights
+        self.feature_mode = feature_mode
+        self.path_norm = path_norm
+        self.channel_norm = channel_norm and feature_mode == 'uv'
+        channel_scale = self.channels_in ** (-0.5) if self.channel_norm else 1.0
+        self.info_forward, self.info_backward1, self.info_backward2, self.num_weights = so2_linear_infos(
+            self.irreps_out, self.irreps_in, path=path, path_norm=path_norm, channel_norm=self.channel_norm,
+            channel_scale=channel_scale)
+        if feature_mode == 'uv':
+            self.weight_shape = (self.num_weights, self.channels_in, self.channels_out)
+        else:
+            self.weight_shape = (self.num_weights, self.channels_out)
+        self.weight_numel = math.prod(self.weight_shape) if None not in self.weight_shape else None
+        if internal_weights:
+            self.weight = Parameter(torch.empty(*self.weight_shape))
+            initialize_so3_so2_linear(self.weight, feature_mode, channel_normed=self.channel_norm)
+        else:
+            self.weight = None
+
+    def forward(self, input: Tensor, weight: Optional[Tensor] = None):
+        assert input.shape[-2] == self.irreps_in.dim, \
+            f"Input spherical dim mismatch: expected {self.irreps_in.dim}, got {input.shape[-2]}"
+        if self.channels_in is not None:
+            assert input.shape[-1] == self.channels_in, \
+                f"Input channel dim mismatch: expected {self.channels_in}, got {input.shape[-1]}"
+        if self.internal_weights:
+            assert weight is None, 'Do not pass the weight when self.internal_weights is True.'
+            weight = self.weight
+        else:
+            assert weight is not None, 'Please pass the weight when self.internal_weights is False.'
+            if self.weight_numel is not None:
+                weight = _view_weight(weight, self.weight_shape, self.weight_numel)
+        op = sparse_mul if self.feature_mode == 'uu' else sparse_vecmat
+        return op(input, weight, self.info_forward, self.info_backward1, self.info_backward2)
+
+    def _apply(self, *args, **kwargs):
+        lin = super()._apply(*args, **kwargs)
+        lin.info_forward = self.info_forward._apply(*args, **kwargs)
+        lin.info_backward1 = self.info_backward1._apply(*args, **kwargs)
+        lin.info_backward2 = self.info_backward2._apply(*args, **kwargs)
+        return lin
+
+    def __repr__(self):
+        channels = (f"channels={self.channels_in}" if self.feature_mode == 'uu'
+                    else f"channels_in={self.channels_in}, channels_out={self.channels_out}")
+        return (f"{self.__class__.__name__}(irreps_in={self.irreps_in.short_repr()}, "
+                f"irreps_out={self.irreps_out.short_repr()}, {channels}, feature_mode={self.feature_mode}, "
+                f"path_norm={self.path_norm}, channel_norm={self.channel_norm}, "
+                f"internal_weights={self.internal_weights}, num_weights={self.num_weights})")

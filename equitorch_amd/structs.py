@@ -107,3 +107,15 @@ class IrrepsLinearInfo(NamedTuple):
     scales_ii0: Tensor
 
     out_size: int
+
+
+@_movable
+class WignerRotationInfo(NamedTuple):
+    """Tables of a rotation applied as ``Z(alpha) J Z(beta) J Z(gamma)``
+    (``equitorch/structs/__init__.py:133-139``)."""
+    j_matrix_info: SparseScaleInfo
+    rotate_z_info_fwd: SparseProductInfo
+    rotate_z_info_bwd_input: Optional[SparseProductInfo] = None
+    rotate_z_info_bwd_cs: Optional[SparseProductInfo] = None
+    sign: Optional[Tensor] = None
+    max_m: Optional[int] = None

@@ -7,6 +7,10 @@ from ._structs import (
     generate_fully_connected_irreps_linear_paths,
     generate_fully_connected_tp_paths,
     irreps_info,
+    j_matrix_info,
+    so2_linear_infos,
+    wigner_d_info,
+    z_rotation_infos,
     irreps_linear_infos,
     prepare_irreps_linear,
     prepare_so3,
@@ -21,5 +25,5 @@ __all__ = [
     "rand_spherical_xyz", "expand_left", "extract_batch_segments", "sort_by_column_key",
     "extract_scatter_indices", "sparse_scale_info", "sparse_scale_infos", "sparse_product_info",
     "sparse_product_infos", "generate_fully_connected_tp_paths", "tp_infos",
-    "generate_fully_connected_irreps_linear_paths", "irreps_linear_infos", "irreps_info",
+    "generate_fully_connected_irreps_linear_paths", "irreps_linear_infos", "irreps_info", "z_rotation_infos", "j_matrix_info", "wigner_d_info", "so2_linear_infos",
 ]

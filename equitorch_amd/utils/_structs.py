@@ -10,9 +10,10 @@ from typing import List, Optional, Tuple
 import numpy as np
 from torch import tensor
 
-from ..constants import so3_clebsch_gordan
+from ..constants import j_matrix, so3_clebsch_gordan
 from ..irreps import Irreps, check_irreps, has_path, irrep_segments
-from ..structs import IrrepsInfo, IrrepsLinearInfo, SparseProductInfo, SparseScaleInfo, TensorProductInfo
+from ..structs import (IrrepsInfo, IrrepsLinearInfo, SparseProductInfo, SparseScaleInfo, TensorProductInfo,
+                       WignerRotationInfo)
 from ._indices import _lex_order, extract_batch_segments, sort_by_column_key
 
 
@@ -278,3 +279,117 @@ def irreps_info(irreps) -> IrrepsInfo:
         rdims.append(1 / irrep.dim)
     seg.append(acc)
     return IrrepsInfo(tensor(rsqrt_dim), tensor(rdims), tensor(idx), tensor(seg), len(irreps))
+
+
+# ---- rotations: D(alpha, beta, gamma) = Z(alpha) J Z(beta) J Z(gamma) ------------------------------------------
+def _component_index(irreps):
+    """``{(irrep index, m): component}`` for ``m = -l..l`` of every irrep."""
+    table, at = {}, 0
+    for i, ir in enumerate(irreps):
+        for m in range(-ir.l, ir.l + 1):
+            table[(i, m)] = at
+            at += 1
+    return table
+
+
+def prepare_z_rotation(irreps):
+    """Entries ``(x index, cs index, output, scale)`` of a rotation about z (reference ``:460-521``):
+    ``x'[m] = cos(m phi) x[m] - sign(m) sin(|m| phi) x[-m]`` with ``cs = [1, sin phi, cos phi, sin 2 phi, ...]``;
+    ``m = 0`` components are copied."""
+    where = _component_index(irreps)
+    index1, index2, index_out, scales = [], [], [], []
+    for (i, m), M in where.items():
+        if m == 0:
+            index_out.append(M); scales.append(1.0); index1.append(M); index2.append(0)
+        else:
+            index_out.append(M); scales.append(1.0); index1.append(M); index2.append(2 * abs(m))
+            index_out.append(M); scales.append(-(float(m > 0) - float(m < 0)))
+            index1.append(where[(i, -m)]); index2.append(2 * abs(m) - 1)
+    return index1, index2, index_out, scales, 1 + 2 * max((ir.l for ir in irreps), default=0)
+
+
+def z_rotation_infos(irreps):
+    """``(forward, gradient of x, gradient of cs)`` product tables of the z rotation (reference ``:536-585``)."""
+    irreps = check_irreps(irreps)
+    index1, index2, index_out, scales, cs_dim = prepare_z_rotation(irreps)
+    return sparse_product_infos(index1=index1, index2=index2, index=index_out, scale=scales, out_size=irreps.dim,
+                                in1_size=irreps.dim, in2_size=cs_dim)
+
+
+def j_matrix_info(irreps) -> SparseScaleInfo:
+    """Block-diagonal ``J`` as a sparse scale table; entries below 1e-9 are dropped (reference ``:587-636``)."""
+    irreps = check_irreps(irreps)
+    index_in, index_out, scales, offset = [], [], [], 0
+    for ir in irreps:
+        block = j_matrix(ir.l)
+        for row in range(ir.dim):
+            for col in range(ir.dim):
+                if abs(block[row, col]) > 1e-9:
+                    index_out.append(offset + row)
+                    index_in.append(offset + col)
+                    scales.append(float(block[row, col]))
+        offset += ir.dim
+    return sparse_scale_info(index=index_in, index_out=index_out, scale=scales, out_size=irreps.dim)
+
+
+def wigner_d_info(irreps) -> WignerRotationInfo:
+    """Reference ``:638-654``.  ``sign`` holds ``p^l`` twice per irrep, as the reference's comprehension over the
+    ``(l, p)`` pair of every irrep produces it."""
+    irreps = check_irreps(irreps)
+    fwd, bwd_x, bwd_cs = z_rotation_infos(irreps)
+    sign = [ir.p ** ir.l for ir in irreps for _ in range(2)]
+    return WignerRotationInfo(j_matrix_info=j_matrix_info(irreps), rotate_z_info_fwd=fwd,
+                              rotate_z_info_bwd_input=bwd_x, rotate_z_info_bwd_cs=bwd_cs,
+                              max_m=max(ir.l for ir in irreps), sign=tensor(sign))
+
+
+# ---- SO(2) linear layer (features in the frame where the edge points along z) -----------------------------------
+def prepare_so2_linear(irreps_out, irreps_in, path=None, path_norm=True, channel_norm=False, channel_scale=1.0):
+    """Entries of ``SO2Linear`` (reference ``:674-778``).  A path ``(k, i)`` carries one weight for ``m = 0`` and two
+    (``w_-``, ``w_+``) for every ``0 < m <= min(l_k, l_i)``:
+
+        out[+m] += s (w_+ x[+m] - w_- x[-m]),      out[-m] += s (w_+ x[-m] + w_- x[+m]),     s = 1 / sqrt(2 n),
+
+    ``out[0] += x[0] w_0 / sqrt(n0)``, where ``n0`` counts the paths into ``(k, 0)`` and — following the reference's
+    bookkeeping, which looks the running count up under ``(k, -m)`` while storing it under ``(k, m)`` — ``n`` is 1
+    for every ``m > 0``."""
+    if path is None:
+        path = [(k, i) for k in range(len(irreps_out)) for i in range(len(irreps_in))]
+    where_in, where_out = _component_index(irreps_in), _component_index(irreps_out)
+    weight_of, count = {}, {}
+    for k, i in path:
+        for m in range(min(irreps_out[k].l, irreps_in[i].l) + 1):
+            if m == 0:
+                weight_of[(k, i, 0)] = len(weight_of)
+                count[(k, 0)] = count.get((k, 0), 0) + 1
+            else:
+                weight_of[(k, i, -m)] = len(weight_of)
+                weight_of[(k, i, m)] = len(weight_of)
+                count[(k, m)] = count.get((k, -m), 0) + 1
+    index1, index2, index_out, scales = [], [], [], []
+
+    def entry(out, inp, w, s):
+        index_out.append(out); index1.append(inp); index2.append(w); scales.append(s)
+
+    for k, i in path:
+        for m in range(min(irreps_out[k].l, irreps_in[i].l) + 1):
+            if m == 0:
+                entry(where_out[(k, 0)], where_in[(i, 0)], weight_of[(k, i, 0)],
+                      count[(k, 0)] ** (-0.5) if path_norm else 1.0)
+                continue
+            s = (count[(k, m)] * 2) ** (-0.5) if path_norm else 2 ** (-0.5)
+            entry(where_out[(k, m)], where_in[(i, m)], weight_of[(k, i, m)], s)
+            entry(where_out[(k, -m)], where_in[(i, -m)], weight_of[(k, i, m)], s)
+            entry(where_out[(k, m)], where_in[(i, -m)], weight_of[(k, i, -m)], -s)
+            entry(where_out[(k, -m)], where_in[(i, m)], weight_of[(k, i, -m)], s)
+    if channel_norm:
+        scales = [s * channel_scale for s in scales]
+    return index1, index2, index_out, scales, len(weight_of)
+
+
+def so2_linear_infos(irreps_out, irreps_in, path=None, path_norm=True, channel_norm=False, channel_scale=1.0):
+    """``(forward, backward1, backward2, num_weights)`` (reference ``:784-786``)."""
+    irreps_out, irreps_in = check_irreps(irreps_out), check_irreps(irreps_in)
+    index1, index2, index_out, scales, n = prepare_so2_linear(irreps_out, irreps_in, path, path_norm, channel_norm,
+                                                              channel_scale)
+    return (*sparse_product_infos(index1, index2, index_out, scales, irreps_out.dim, irreps_in.dim, n), n)

@@ -64,3 +64,21 @@ def so3_cg(l, l1, l2):
                             acc = acc + qt * c[n][i][k] * q1[i][j] * q2[k][lp]
                 out[m][j][lp] = sympy.sympify(acc)
     return out
+
+
+@functools.lru_cache(maxsize=None)
+def j_matrix(l):
+    """``j_matrix`` (equitorch/constants/__init__.py:13-36) in exact arithmetic: nested lists of sympy numbers.
+    Pinned by the golden fixture ``tests/golden/rotation_tables.npz`` (entries as stored by the reference's
+    ``j_matrix_info``), by ``J^2 = 1`` and by ``Y(J v) = J Y(v)`` for ``J v = (-x, z, y)``."""
+    if l == 0:
+        return [[S(1)]]
+    if l == 1:
+        return [[S(0), S(1), S(0)], [S(1), S(0), S(0)], [S(0), S(0), S(-1)]]
+    cg, j1, jp = so3_cg(l, 1, l - 1), j_matrix(1), j_matrix(l - 1)
+    n, n1 = 2 * l + 1, 2 * l - 1
+    # 'iI,jJ,kij,KIJ->kK'
+    half = [[[sum(j1[i][I] * jp[j][J] * cg[k][i][j] for i in range(3) for j in range(n1))
+              for J in range(n1)] for I in range(3)] for k in range(n)]
+    return [[sympy.nsimplify(sum(half[k][I][J] * cg[K][I][J] for I in range(3) for J in range(n1)))
+             for K in range(n)] for k in range(n)]

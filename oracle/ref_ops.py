@@ -296,3 +296,65 @@ def cpu_layer_rms_norm(x, info, weight=None, scaled=True, eps=1e-5):
     idx = torch.tensor(info["irrep_index"], dtype=torch.int64)
     out = x * rsigma.index_select(-1, idx).unsqueeze(-1)
     return out if weight is None else cpu_gating(out, weight, info)
+
+
+# ---- rotations and the SO(2) linear layer --------------------------------------------------------------------
+def _product_entries(info):
+    """(out, i1, i2, scale) per entry of a ``sparse_product_info`` dict (None index = identity)."""
+    n = len(info["scale"])
+    i1 = info["index1"] if info["index1"] is not None else list(range(n))
+    i2 = info["index2"] if info["index2"] is not None else list(range(n))
+    seg = info["seg_out"] if info["seg_out"] is not None else list(range(n + 1))
+    out = [m for m in range(len(seg) - 1) for _ in range(seg[m], seg[m + 1])]
+    return list(zip(out, i1, i2, info["scale"]))
+
+
+def cpu_z_rotation(x, cs, info):
+    """``sparse_vecsca(x, cs, rotate_z_info_fwd)`` (equitorch/nn/functional/wigner_d.py:34-37):
+    ``out[n, M, c] = sum_t scale_t x[n, i1_t, c] cs[n, i2_t]``."""
+    rows = [torch.zeros_like(x[:, 0]) for _ in range(info["out_size"])]
+    for o, i1, i2, s in _product_entries(info):
+        rows[o] = rows[o] + s * x[:, i1] * cs[:, i2, None]
+    return torch.stack(rows, dim=1)
+
+
+def cpu_j(x, info):
+    """``sparse_scale(x, j_matrix_info)``: ``out[n, M] = sum_{t in seg M} scale_t x[n, index_t]``."""
+    seg, idx, sc = info["seg_out"], info["index"], info["scale"]
+    return torch.stack([sum(sc[t] * x[:, idx[t]] for t in range(seg[m], seg[m + 1])) for m in range(len(seg) - 1)],
+                       dim=1)
+
+
+def cpu_wigner_rotation(x, sc_alpha, sc_beta, sc_gamma, z_info, j_info):
+    """``sparse_wigner_rotation`` (equitorch/nn/functional/wigner_d.py:14-56): Z(alpha) J Z(beta) J Z(gamma) x."""
+    if sc_gamma is not None:
+        x = cpu_z_rotation(x, sc_gamma, z_info)
+    if sc_beta is not None:
+        x = cpu_j(cpu_z_rotation(cpu_j(x, j_info), sc_beta, z_info), j_info)
+    if sc_alpha is not None:
+        x = cpu_z_rotation(x, sc_alpha, z_info)
+    return x
+
+
+def cpu_sincos(angle, max_m):
+    """``sincos`` (equitorch/nn/functional/angular.py): [1, sin a, cos a, sin 2a, cos 2a, ...]."""
+    cols = [torch.ones_like(angle)]
+    for m in range(1, max_m + 1):
+        cols += [torch.sin(m * angle), torch.cos(m * angle)]
+    return torch.stack(cols, dim=-1)
+
+
+def cpu_so2_linear(x, w, info, per_sample=False):
+    """``SO2Linear.forward`` (equitorch/nn/linears.py:495-507): ``sparse_mul`` for a channel-wise weight
+    ``((N,) num_weights, C)``, ``sparse_vecmat`` for ``((N,) num_weights, C_in, C_out)``."""
+    rows = [None] * info["out_size"]
+    matrix = w.ndim - int(per_sample) == 3
+    for o, i1, i2, s in _product_entries(info):
+        wt = w[:, i2] if per_sample else w[i2]
+        if not matrix:
+            term = s * x[:, i1] * wt
+        else:
+            term = s * (torch.einsum("nu,nuw->nw", x[:, i1], wt) if per_sample else x[:, i1] @ wt)
+        rows[o] = term if rows[o] is None else rows[o] + term
+    some = next(r for r in rows if r is not None)
+    return torch.stack([r if r is not None else torch.zeros_like(some) for r in rows], dim=1)

@@ -282,3 +282,77 @@ def irreps_info(irreps):
     idx = [i for i, (l, _) in enumerate(irs) for _ in range(2 * l + 1)]
     return dict(rsqrt_dims=[(2 * l + 1) ** (-0.5) for l, _ in irs], rdims=[1 / (2 * l + 1) for l, _ in irs],
                 irrep_index=idx, irrep_seg=segments(irs), num_irreps=len(irs))
+
+
+# ---- rotations and the SO(2) linear layer (equitorch/utils/_structs.py:460-786) -----------------------------
+def _components(irs):
+    table, at = {}, 0
+    for i, (l, _) in enumerate(irs):
+        for m in range(-l, l + 1):
+            table[(i, m)] = at
+            at += 1
+    return table
+
+
+def z_rotation_infos(irreps):
+    """:460-585 -> (forward, gradient-of-x, gradient-of-cs) dicts of ``sparse_product_infos``."""
+    irs = parse(irreps)
+    where = _components(irs)
+    i1, i2, io, sc = [], [], [], []
+    for (i, m), M in where.items():
+        if m == 0:
+            io.append(M); sc.append(1.0); i1.append(M); i2.append(0)
+        else:
+            io.append(M); sc.append(1.0); i1.append(M); i2.append(2 * abs(m))
+            io.append(M); sc.append(-(float(m > 0) - float(m < 0))); i1.append(where[(i, -m)]); i2.append(2 * abs(m) - 1)
+    dim = segments(irs)[-1]
+    return sparse_product_infos(i1, i2, io, sc, dim, dim, 1 + 2 * max(l for l, _ in irs))
+
+
+def j_matrix_info(irreps):
+    """:587-636."""
+    irs = parse(irreps)
+    idx_in, idx_out, sc, off = [], [], [], 0
+    for l, _ in irs:
+        blk = ref_constants.j_matrix(l)
+        for r in range(2 * l + 1):
+            for c in range(2 * l + 1):
+                if abs(blk[r][c]) > 1e-9:
+                    idx_out.append(off + r); idx_in.append(off + c); sc.append(float(blk[r][c]))
+        off += 2 * l + 1
+    return sparse_scale_info(index=idx_in, index_out=idx_out, scale=sc, out_size=off)
+
+
+def so2_linear_infos(irreps_out, irreps_in, path=None, path_norm=True, channel_norm=False, channel_scale=1.0):
+    """:674-786 -> (forward, backward1, backward2 dicts, num_weights).  The count for ``m > 0`` is read under the key
+    ``(k, -m)``, which is never written, so it is always 1 — as in the reference."""
+    io_, ii_ = parse(irreps_out), parse(irreps_in)
+    if path is None:
+        path = [(k, i) for k in range(len(io_)) for i in range(len(ii_))]
+    w_in, w_out = _components(ii_), _components(io_)
+    widx, cnt = {}, {}
+    for k, i in path:
+        for m in range(min(io_[k][0], ii_[i][0]) + 1):
+            if m == 0:
+                widx[(k, i, 0)] = len(widx)
+                cnt[(k, 0)] = cnt.get((k, 0), 0) + 1
+            else:
+                widx[(k, i, -m)] = len(widx)
+                cnt[(k, m)] = cnt.get((k, -m), 0) + 1
+                widx[(k, i, m)] = len(widx)
+                cnt[(k, m)] = cnt.get((k, -m), 0) + 1
+    i1, i2, io, sc = [], [], [], []
+    for k, i in path:
+        for m in range(min(io_[k][0], ii_[i][0]) + 1):
+            if m == 0:
+                sc.append(cnt[(k, 0)] ** (-0.5) if path_norm else 1.0)
+                io.append(w_out[(k, 0)]); i1.append(w_in[(i, 0)]); i2.append(widx[(k, i, 0)])
+                continue
+            s = (cnt[(k, m)] * 2) ** (-0.5) if path_norm else 2 ** (-0.5)
+            for out_m, in_m, w_m, sign in ((m, m, m, 1), (-m, -m, m, 1), (m, -m, -m, -1), (-m, m, -m, 1)):
+                sc.append(sign * s)
+                io.append(w_out[(k, out_m)]); i1.append(w_in[(i, in_m)]); i2.append(widx[(k, i, w_m)])
+    if channel_norm:
+        sc = [s * channel_scale for s in sc]
+    n = len(widx)
+    return (*sparse_product_infos(i1, i2, io, sc, segments(io_)[-1], segments(ii_)[-1], n), n)

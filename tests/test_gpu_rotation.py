@@ -1,0 +1,95 @@
+"""GPU parity of the sparse Wigner rotation, the dense Wigner matrices and SO2Linear against the oracle."""
+import math
+
+import pytest
+import torch
+
+from helpers import assert_close
+from oracle import ref_ops, ref_sh, ref_tables
+
+pytestmark = pytest.mark.gpu
+
+IRR = "0e+1o+2e+3o"
+
+
+def _f32(d):
+    """Scale lists as the reference stores them: fp32 values."""
+    d = dict(d)
+    d["scale"] = torch.tensor(d["scale"]).double().tolist()
+    return d
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_sparse_rotation_and_its_gradients(device, dtype):
+    from equitorch_amd.nn import SparseWignerRotation
+    from equitorch_amd.nn.functional import sincos
+    z = _f32(ref_tables.z_rotation_infos(IRR)[0])
+    j = _f32(ref_tables.j_matrix_info(IRR))
+    g = torch.Generator().manual_seed(0)
+    n, c = 50, 12
+    x = torch.randn(n, 16, c, generator=g, dtype=torch.float64).to(dtype).double()
+    ang = ((torch.rand(3, n, generator=g, dtype=torch.float64) - 0.5) * 6).to(dtype).double()
+    ct = torch.randn(n, 16, c, generator=g, dtype=torch.float64).to(dtype).double()
+    xr, ar = x.clone().requires_grad_(True), ang.clone().requires_grad_(True)
+    ref = ref_ops.cpu_wigner_rotation(xr, *(ref_ops.cpu_sincos(ar[k], 3) for k in range(3)), z, j)
+    rgx, rga = torch.autograd.grad(ref, (xr, ar), ct)
+    mod = SparseWignerRotation(IRR).to(device)
+    xd, ad = x.to(device, dtype).requires_grad_(True), ang.to(device, dtype).requires_grad_(True)
+    out = mod(xd, *(sincos(ad[k], 3) for k in range(3)))
+    gx, ga = torch.autograd.grad(out, (xd, ad), ct.to(device, dtype))
+    tol = 1e-5 if dtype == torch.float32 else 1e-11
+    assert_close(out, ref, tol=tol, what="rotated features")
+    assert_close(gx, rgx, tol=tol, what="grad input")
+    assert_close(ga, rga, tol=10 * tol, what="grad angles")
+    # an angle given as None is skipped
+    ref0 = ref_ops.cpu_wigner_rotation(x, None, ref_ops.cpu_sincos(ang[1], 3), None, z, j)
+    assert_close(mod(xd, None, sincos(ad[1], 3), None), ref0, tol=tol, what="beta only")
+
+
+def test_dense_wigner_matrices_and_alignment(device):
+    from equitorch_amd.nn import AlignToZWignerD, DenseWignerRotation, WignerD
+    g = torch.Generator().manual_seed(1)
+    n = 9
+    ang = (torch.rand(3, n, generator=g, dtype=torch.float64) - 0.5) * 6
+    wd = WignerD(IRR).to(device).double()
+    D = wd(alpha=ang[0].to(device), beta=ang[1].to(device), gamma=ang[2].to(device))
+    assert D.shape == (n, 16, 16)
+    v = torch.randn(15, 3, generator=g, dtype=torch.float64)
+    v = v / v.norm(dim=-1, keepdim=True)
+    y = ref_sh.spherical_harmonics(v, 3)
+    for k in range(n):
+        Dk = D[k].cpu()
+        R = Dk[1:4, 1:4][[2, 0, 1]][:, [2, 0, 1]]          # degree-1 block, (y, z, x) -> (x, y, z)
+        assert_close(ref_sh.spherical_harmonics(v @ R.T, 3), y @ Dk.T, tol=1e-6, what="D transports harmonics")
+    single = wd(beta=ang[1, :1].to(device))
+    assert single.shape == (16, 16)                         # no batch of more than one: the batch axis is dropped
+    # alignment: D(v) Y(v) = Y(z axis) = sqrt(2l+1) on the m = 0 components
+    vz = v[:n].to(device)
+    Dz = AlignToZWignerD(IRR, normalized=True).to(device).double()(vz)
+    target = torch.zeros(16, dtype=torch.float64)
+    for l in range(4):
+        target[l * l + l] = math.sqrt(2 * l + 1)
+    yz = DenseWignerRotation(IRR)(y[:n].to(device).unsqueeze(-1), Dz).squeeze(-1)
+    assert_close(yz, target.expand(n, 16), tol=1e-6, what="aligned harmonics")
+
+
+@pytest.mark.parametrize("mode,per_sample", [("uu", False), ("uu", True), ("uv", False), ("uv", True)])
+def test_so2_linear(device, mode, per_sample):
+    from equitorch_amd.nn import SO2Linear
+    irr_in, irr_out = "0e+1o+2e+3o", "0e+1o+2e"
+    info = _f32(ref_tables.so2_linear_infos(irr_out, irr_in)[0])
+    n, cin, cout = 31, 8, 8 if mode == "uu" else 6
+    mod = SO2Linear(irr_in, irr_out, cin, cout, internal_weights=False, feature_mode=mode).to(device)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(n, 16, cin, generator=g, dtype=torch.float64)
+    wshape = (mod.num_weights, cout) if mode == "uu" else (mod.num_weights, cin, cout)
+    w = torch.randn(*((n,) if per_sample else ()), *wshape, generator=g, dtype=torch.float64)
+    ct = torch.randn(n, 9, cout, generator=g, dtype=torch.float64)
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    ref = ref_ops.cpu_so2_linear(xr, wr, info, per_sample=per_sample)
+    rgx, rgw = torch.autograd.grad(ref, (xr, wr), ct)
+    xd, wd = x.to(device).requires_grad_(True), w.to(device).requires_grad_(True)
+    out = mod(xd, wd)
+    gx, gw = torch.autograd.grad(out, (xd, wd), ct.to(device))
+    for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
+        assert_close(a, b, tol=1e-11, what=f"SO2Linear {mode} per_sample={per_sample} {name}")
