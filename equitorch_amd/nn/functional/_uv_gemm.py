@@ -1,10 +1,12 @@
-"""Fully connected ("uv") products in fp32 / fp64 with a shared weight: the channel mixing is a plain GEMM per weight
-path on the library (``torch.matmul``), the Clebsch-Gordan stage runs on the table-driven contraction kernel.
+"""Fully connected ("uv") products outside the matrix-core kernel's domain (fp32 / fp64, per-sample weights, channel
+counts it does not cover): the channel mixing is a plain GEMM per weight path on the library (``torch.matmul``), the
+Clebsch-Gordan stage runs on the table-driven contraction kernel.
 
 Weight-first order, as in the matrix-core kernel: ``z[n, q, :] = x[n, a_q, :] @ W[p_q]`` for every (path, input row)
 pair ``q``, then ``out[n, M] = sum_t coef_t * y[n, b_t] * z[n, q_t]``.  Every piece is differentiable (``matmul``,
 ``cat`` and the closed contraction family of ``_tri``), so gradients of any order come from autograd.  The bf16 case
-does not come here (``_uvw_mfma``); per-sample weights stay on the general two-axis kernel.
+with a shared weight does not come here (``_uvw_mfma``).  A per-sample weight ``(N, P, C_in, C_out)`` makes the
+path GEMMs batched over the samples.
 """
 from typing import List, Tuple
 
@@ -48,12 +50,14 @@ def _plan(tp_info, chan: int) -> _Plan:
 
 def _mix(x: Tensor, weight: Tensor, plan: _Plan) -> Tensor:
     """``z[n, q, :] = x[n, a_q, :] @ weight[p_q]``: one GEMM per path over the rows of its input irrep."""
-    return torch.cat([torch.matmul(x[:, a0:a0 + na, :], weight[p]) for p, (a0, na) in enumerate(plan.ranges)], dim=1)
+    pick = (lambda p: weight[p]) if weight.ndim == 3 else (lambda p: weight[:, p])
+    return torch.cat([torch.matmul(x[:, a0:a0 + na, :], pick(p)) for p, (a0, na) in enumerate(plan.ranges)], dim=1)
 
 
 def supported(*tensors: Tensor) -> bool:
+    """One floating dtype throughout and a weight ``(P, C_in, C_out)`` or ``(N, P, C_in, C_out)``."""
     dtypes = {t.dtype for t in tensors}
-    return len(dtypes) == 1 and next(iter(dtypes)) in (torch.float32, torch.float64) and tensors[-1].ndim == 3
+    return len(dtypes) == 1 and next(iter(dtypes)).is_floating_point and tensors[-1].ndim in (3, 4)
 
 
 def u1v(input1: Tensor, input2: Tensor, weight: Tensor, tp_info) -> Tensor:

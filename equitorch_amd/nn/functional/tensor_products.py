@@ -10,7 +10,7 @@ from torch import Tensor
 from ... import _lib
 V = "u"  # channel axes of a per-channel operand
 from ...structs import TensorProductInfo
-from ._tri import spec_from_product_info, spec_from_tp_info, tri
+from ._tri import spec_from_tp_info, tri
 
 
 def tensor_product_uuu(input1: Tensor, input2: Tensor, weight: Tensor,
@@ -28,12 +28,11 @@ def tensor_product_uvw(input1: Tensor, input2: Tensor, weight: Tensor,
                        tp_info_backward2: Optional[TensorProductInfo] = None) -> Tensor:
     """``input1 (N, D1, C1)``, ``input2 (N, D2, C2)``, ``weight (P, C1, C2, C_out) | (N, P, C1, C2, C_out)`` ->
     ``(N, DO, C_out)``.  Two stages as in the reference (``tensor_products.py:100-101``): the outer products per
-    stage-1 segment, flattened to ``C1*C2`` channels, then one matrix product per segment with the flattened
-    weight of its path."""
+    stage-1 segment on the table-driven kernel, then the contraction with the weights as one library GEMM per
+    output irrep (``_uvw_gemm``)."""
     _lib.require_gpu(input1, input2, weight)
-    s1, s2 = tp_info_forward.info_Mij_fwd, tp_info_forward.info_M_fwd
-    inter = tri(spec_from_product_info(s1, input1.shape[-2], input2.shape[-2]), ("u", "w", None), "uw",
-                input1, input2)
-    inter = inter.flatten(-2)
-    w2 = weight.flatten(-3, -2)
-    return tri(spec_from_product_info(s2, inter.shape[-2], w2.shape[-3]), ("u", "uw", None), "w", inter, w2)
+    if weight.ndim not in (4, 5) or input1.dtype != input2.dtype or input1.dtype != weight.dtype:
+        raise _lib.CgtpError(f"tensor_product_uvw: operands {input1.dtype}, {input2.dtype}, {weight.dtype} with "
+                             f"weight of {weight.ndim} dims")
+    from . import _uvw_gemm
+    return _uvw_gemm.uvw(input1.contiguous(), input2.contiguous(), weight, tp_info_forward)
