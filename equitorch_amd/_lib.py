@@ -56,7 +56,8 @@ class UvuArgs(C.Structure):
                 ("x", C.c_void_p), ("y", C.c_void_p), ("w", C.c_void_p),
                 ("out", C.c_void_p),
                 ("grad_out", C.c_void_p), ("grad_x", C.c_void_p), ("grad_y", C.c_void_p),
-                ("grad_w", C.c_void_p), ("workspace", C.c_void_p), ("x_gather", C.c_void_p)]
+                ("grad_w", C.c_void_p), ("workspace", C.c_void_p), ("x_gather", C.c_void_p),
+                ("y_channels", C.c_int32), ("reserved_", C.c_int32)]
 
 
 def _load():

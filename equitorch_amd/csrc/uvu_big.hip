@@ -10,7 +10,8 @@ namespace cgtp {
 
 // Lanes past the batch or the channel count re-read the last valid element and store nothing, so that every lane
 // runs the same code and the channel sum of grad_y can use full-width shuffles.
-template <class TP>
+// YC: the second operand carries channels, y (n_rows, D2, C); one value per lane like x.
+template <class TP, bool YC = false>
 __global__ void __launch_bounds__(256, 2) uvu_big_fwd_kernel(const UvuDev<float> a) {
   constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
   const Lanes L(a.lpe_log2);
@@ -24,7 +25,7 @@ __global__ void __launch_bounds__(256, 2) uvu_big_fwd_kernel(const UvuDev<float>
   const int64_t xr = a.gather ? a.gather[r] : r;
   float x[D1], y[D2];
 #pragma unroll
-  for (int j = 0; j < D2; ++j) y[j] = a.y[r * D2 + j];
+  for (int j = 0; j < D2; ++j) y[j] = YC ? a.y[(r * D2 + j) * C + c] : a.y[r * D2 + j];
 #pragma unroll
   for (int i = 0; i < D1; ++i) x[i] = a.x[(xr * D1 + i) * C + c];
   const float* wrow = a.w + (a.w_shared ? 0 : r) * P * C + c;
@@ -36,7 +37,7 @@ __global__ void __launch_bounds__(256, 2) uvu_big_fwd_kernel(const UvuDev<float>
       });
 }
 
-template <class TP, int GW>
+template <class TP, int GW, bool YC = false>
 __global__ void __launch_bounds__(256, 2) uvu_big_bwd_kernel(const UvuDev<float> a, int64_t n_waves) {
   constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
   const Lanes L(a.lpe_log2);
@@ -52,7 +53,7 @@ __global__ void __launch_bounds__(256, 2) uvu_big_bwd_kernel(const UvuDev<float>
   float x[D1], y[D2], gx[D1], gy[D2];
 #pragma unroll
   for (int j = 0; j < D2; ++j) {
-    y[j] = a.y[r * D2 + j];
+    y[j] = YC ? a.y[(r * D2 + j) * C + c] : a.y[r * D2 + j];
     gy[j] = 0.f;
   }
 #pragma unroll
@@ -75,7 +76,12 @@ __global__ void __launch_bounds__(256, 2) uvu_big_bwd_kernel(const UvuDev<float>
 #pragma unroll
     for (int i = 0; i < D1; ++i) __builtin_nontemporal_store(gx[i], a.gx + (r * D1 + i) * C + c);
   }
-  if (a.gy) {
+  if (YC) {
+    if (a.gy && live) {
+#pragma unroll
+      for (int j = 0; j < D2; ++j) __builtin_nontemporal_store(gy[j], a.gy + (r * D2 + j) * C + c);
+    }
+  } else if (a.gy) {
     const float keep = L.cl < a.C ? 1.f : 0.f;  // duplicate channels of the padding lanes do not count
 #pragma unroll
     for (int j = 0; j < D2; ++j) {
@@ -94,6 +100,9 @@ static UvuBigEntry make_big_entry() {
   e.fwd = uvu_big_fwd_kernel<TP>;
   e.bwd[kGwNone] = uvu_big_bwd_kernel<TP, kGwNone>;
   e.bwd[kGwStore] = uvu_big_bwd_kernel<TP, kGwStore>;
+  e.fwd_yc = uvu_big_fwd_kernel<TP, true>;
+  e.bwd_yc[kGwNone] = uvu_big_bwd_kernel<TP, kGwNone, true>;
+  e.bwd_yc[kGwStore] = uvu_big_bwd_kernel<TP, kGwStore, true>;
   return e;
 }
 

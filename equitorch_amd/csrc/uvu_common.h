@@ -53,6 +53,9 @@ struct UvuBigEntry {
   const char* name;
   void (*fwd)(const UvuDev<float>);
   void (*bwd[2])(const UvuDev<float>, int64_t);  // [kGwNone, kGwStore]
+  // the same with a channelled second operand, y (n_rows, D2, C) ("uuu"): grad_y is then per channel as well
+  void (*fwd_yc)(const UvuDev<float>);
+  void (*bwd_yc[2])(const UvuDev<float>, int64_t);
 };
 const UvuBigEntry* uvu_big_entries(int* count);
 

@@ -529,6 +529,17 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
     for (int i = 0; i < n_big; ++i)
       if (big_tab[i].fingerprint == tab[a->cfg].fingerprint) big_idx = i;
   }
+  if (a->y_channels) {  // channelled second operand: block-wise kernels only (fp32, row mode, one wavefront wide)
+    if (seg_mode || a->y_vec) return CGTP_ERR_SHAPE;
+    if (a->dtype != CGTP_F32) return CGTP_ERR_DTYPE;
+    if (a->cfg < n_cfg) {
+      big_idx = -1;
+      for (int i = 0; i < n_big; ++i)
+        if (big_tab[i].fingerprint == tab[a->cfg].fingerprint) big_idx = i;
+    }
+    if (big_idx < 0) return CGTP_ERR_CONFIG;
+    if (backward && a->C > kWave) return CGTP_ERR_SHAPE;
+  }
   const bool big = big_idx >= 0;
   plan->big_idx = big_idx;
   const int* dims = big ? big_tab[big_idx].dims : tab[a->cfg].dims;
@@ -647,8 +658,8 @@ static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward,
   UvuDev<float> d = to_dev<float>(a, plan);
   if (backward) {
     if (wred) d.gw = d.wsw;  // per-row gradients into the workspace, summed below
-    hipLaunchKernelGGL(e.bwd[a->grad_w ? kGwStore : kGwNone], dim3((unsigned)((plan.n_waves + 3) / 4)), dim3(256), 0,
-                       stream, d, plan.n_waves);
+    hipLaunchKernelGGL((a->y_channels ? e.bwd_yc : e.bwd)[a->grad_w ? kGwStore : kGwNone],
+                       dim3((unsigned)((plan.n_waves + 3) / 4)), dim3(256), 0, stream, d, plan.n_waves);
     if (wred) {
       if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
       const int64_t chunks = (a->n_rows + kSumRows - 1) / kSumRows;
@@ -662,7 +673,7 @@ static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward,
   } else {
     const int chunk = 1 << plan.lpe_log2;
     dim3 grid((unsigned)((plan.n_waves + 3) / 4), (unsigned)((a->C + chunk - 1) / chunk));
-    hipLaunchKernelGGL(e.fwd, grid, dim3(256), 0, stream, d);
+    hipLaunchKernelGGL(a->y_channels ? e.fwd_yc : e.fwd, grid, dim3(256), 0, stream, d);
   }
   return launched();
 }

@@ -5,12 +5,41 @@
 """
 from typing import Optional
 
+import torch
 from torch import Tensor
+from torch.autograd import Function
 
 from ... import _lib
 V = "u"  # channel axes of a per-channel operand
+from ...ops import kernels
 from ...structs import TensorProductInfo
 from ._tri import spec_from_tp_info, tri
+
+
+class _UuuCompiled(Function):
+    """uuu on the block-wise kernels with a compiled-in table (``cgtp_uvu_fwd`` / ``cgtp_uvu_bwd`` with
+    ``y_channels``); gradients of higher order go through the differentiable table-driven contraction."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, y: Tensor, w: Tensor, tp_info: TensorProductInfo, cfg: int):
+        out = kernels.uvu_forward(cfg, kernels.uvu_dims(cfg), x, y, w)
+        ctx.save_for_backward(x, y, w)
+        ctx.tp_info, ctx.cfg = tp_info, cfg
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        x, y, w = ctx.saved_tensors
+        need = ctx.needs_input_grad[:3]
+        if torch.is_grad_enabled():
+            with torch.enable_grad():
+                spec = spec_from_tp_info(ctx.tp_info)
+                gx = tri(spec.grad_spec(0), (V, V, V), V, g, y, w) if need[0] else None
+                gy = tri(spec.grad_spec(1), (V, V, V), V, x, g, w) if need[1] else None
+                gw = tri(spec.grad_spec(2), (V, V, V), V, x, y, g, out_shared=(w.ndim == 2)) if need[2] else None
+            return gx, gy, gw, None, None
+        res = kernels.uvu_backward(ctx.cfg, kernels.uvu_dims(ctx.cfg), x, y, w, g.contiguous(), need)
+        return (*res, None, None)
 
 
 def tensor_product_uuu(input1: Tensor, input2: Tensor, weight: Tensor,
@@ -19,6 +48,12 @@ def tensor_product_uuu(input1: Tensor, input2: Tensor, weight: Tensor,
                        tp_info_backward2: Optional[TensorProductInfo] = None) -> Tensor:
     """``input1 (N, D1, C)``, ``input2 (N, D2, C)``, ``weight (P, C) | (N, P, C)`` -> ``(N, DO, C)``."""
     _lib.require_gpu(input1, input2, weight)
+    if (input1.ndim == 3 and input2.ndim == 3 and input1.dtype == input2.dtype == weight.dtype == torch.float32
+            and input1.shape[-1] == input2.shape[-1]):
+        cfg = kernels.uvu_config_of(tp_info_forward)
+        x, y, w = input1.contiguous(), input2.contiguous(), weight.contiguous()
+        if cfg >= 0 and kernels.uvu_launchable(cfg, x, y, w):
+            return _UuuCompiled.apply(x, y, w, tp_info_forward, cfg)
     return tri(spec_from_tp_info(tp_info_forward), (V, V, V), V, input1, input2, weight)
 
 

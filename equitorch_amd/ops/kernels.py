@@ -140,6 +140,7 @@ def _uvu_args(cfg: int, x: Tensor, y: Tensor, w: Tensor, seg: Optional[SegIndex]
               pos_per_wave: int = 0, y_vec: int = 0) -> UvuArgs:
     a = UvuArgs()
     a.y_vec = y_vec
+    a.y_channels = int(y.ndim == 3)
     a.cfg, a.dtype, a.C = cfg, _lib.dtype_code(x.dtype), x.shape[-1]
     a.w_shared = int(w.ndim == 2)
     a.n_rows, a.n_x_rows = y.shape[0], x.shape[0]
@@ -177,6 +178,7 @@ def uvu_launchable(cfg: int, x: Tensor, y: Tensor, w: Tensor, segments: bool = F
     a.w_shared = int(w.ndim == 2)
     a.n_rows = y.shape[0]
     a.y_vec = y_vec
+    a.y_channels = int(y.ndim == 3)
     dummy = 256
     a.n_x_rows = x.shape[0]
     if segments:

@@ -195,6 +195,10 @@ typedef struct cgtp_uvu_args {
   void* workspace;         /* cgtp_uvu_workspace_bytes() bytes (segment mode, or bwd of a shared W) */
   const int64_t* x_gather; /* row mode backward, optional: [n_rows] row of x of every batch row (x then has
                               n_x_rows rows; grad_x stays per batch row, (n_rows, D1, C))              */
+  int32_t y_channels;      /* row mode, fp32: 1 = y and grad_y carry channels, (n_rows, D2, C): the "uuu" product
+                              TensorProductUUUDummy (equitorch/nn/functional/tensor_products.py:9-90), on the
+                              block-wise kernels; backward needs C <= 64                               */
+  int32_t reserved_;
 } cgtp_uvu_args;
 
 int cgtp_uvu_validate(const cgtp_uvu_args* args, int backward);

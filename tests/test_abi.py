@@ -125,6 +125,17 @@ def test_large_table_configs_and_row_gathers_validate_on_the_host():
     assert L.cgtp_uvu_validate(C.byref(a), 1) == 2
     a.x_gather = 4096
     assert L.cgtp_uvu_validate(C.byref(a), 1) == 0
+    # channelled second operand ("uuu"): block-wise kernels, fp32, row mode, backward one wavefront wide
+    b = _lib.UvuArgs()
+    b.cfg, b.dtype, b.C, b.n_rows, b.n_x_rows, b.y_channels = cfg, _lib.F32, 64, 10, 10, 1
+    b.x = b.y = b.w = b.out = b.grad_out = b.grad_x = b.grad_y = b.grad_w = 4096
+    assert L.cgtp_uvu_validate(C.byref(b), 0) == 0 and L.cgtp_uvu_validate(C.byref(b), 1) == 0
+    b.C = 128
+    assert L.cgtp_uvu_validate(C.byref(b), 0) == 0 and L.cgtp_uvu_validate(C.byref(b), 1) == 2
+    b.C, b.dtype = 64, _lib.F64
+    assert L.cgtp_uvu_validate(C.byref(b), 0) == 4
+    b.dtype, b.n_seg, b.ptr, b.seg_ids, b.gather = _lib.F32, 10, 4096, 4096, 4096
+    assert L.cgtp_uvu_validate(C.byref(b), 0) == 2                  # no segment mode
 
 
 def test_uv_matrix_core_entry_points_validate_on_the_host():

@@ -205,3 +205,43 @@ def test_edge_large_table(device):
     for name, g, r in zip(("out", "grad_x", "grad_sh", "grad_w"), (out, xd.grad, shd.grad, wd.grad),
                           (ref_out, *ref_grads)):
         assert_close(g, r, 1e-5, f"edge lmax=6 {name}")
+
+
+@pytest.mark.parametrize("lmax,channels", [(2, 64), (2, 20), (3, 48)])
+@pytest.mark.parametrize("shared_w", [False, True])
+def test_uuu_on_the_block_wise_kernels(device, lmax, channels, shared_w):
+    """TensorProduct('uuu') with a compiled table: both operands channelled, fp32, forward and all gradients against
+    the dense oracle; a second-order gradient goes through the table-driven contraction and must agree too."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.nn import TensorProduct
+    from equitorch_amd.ops import kernels
+    irr = SH[lmax]
+    d = (lmax + 1) ** 2
+    mod = TensorProduct(irr, irr, irr, channels, channels, channels, feature_mode="uuu", internal_weights=False).to(device)
+    assert kernels.uvu_config_of(mod.tp_info_forward) >= 0
+    g = torch.Generator().manual_seed(31 + lmax)
+    n = 77
+    x = torch.randn(n, d, channels, generator=g)
+    y = torch.randn(n, d, channels, generator=g)
+    w = torch.randn(*(() if shared_w else (n,)), mod.num_paths, channels, generator=g)
+    ct = torch.randn(n, d, channels, generator=g)
+    T = ref_ops.dense_coupling(irr, irr, irr)
+    xr, yr, wr = (t.double().requires_grad_(True) for t in (x, y, w))
+    ref = torch.einsum(f"pmab,nau,nbu,{'' if shared_w else 'n'}pu->nmu", T, xr, yr, wr)
+    rg = torch.autograd.grad(ref, (xr, yr, wr), ct.double(), create_graph=True)
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    out = F.tensor_product_uuu(xd, yd, wd, mod.tp_info_forward)
+    assert kernels.uvu_launchable(kernels.uvu_config_of(mod.tp_info_forward), xd.detach(), yd.detach(), wd.detach())
+    got = torch.autograd.grad(out, (xd, yd, wd), ct.to(device), create_graph=True)
+    assert_close(out, ref, 1e-5, "uuu out")
+    for name, a, b in zip(("grad_x", "grad_y", "grad_w"), got, rg):
+        assert_close(a, b, 1e-5, f"uuu lmax={lmax} shared={shared_w} {name}")
+    # first-order gradients without create_graph take the compiled backward kernel
+    plain = torch.autograd.grad(F.tensor_product_uuu(xd, yd, wd, mod.tp_info_forward), (xd, yd, wd), ct.to(device))
+    for name, a, b in zip(("grad_x", "grad_y", "grad_w"), plain, rg):
+        assert_close(a, b, 1e-5, f"uuu compiled backward {name}")
+    # second order: d/dx of <grad_y, ct2>
+    ct2 = torch.randn(n, d, channels, generator=g)
+    (hx,) = torch.autograd.grad((got[1] * ct2.to(device)).sum(), xd)
+    (rhx,) = torch.autograd.grad((rg[1] * ct2.double()).sum(), xr)
+    assert_close(hx, rhx, 1e-5, "uuu second order")
