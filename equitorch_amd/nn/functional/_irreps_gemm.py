@@ -267,9 +267,12 @@ def _matrix_core_path(x: Tensor, weight: Tensor, plan: LinearPlan, in_size: int,
     from . import _uvw_mfma
     if x.dtype != torch.bfloat16 or weight.ndim != 3 or x.shape[0] == 0:
         return None
-    info = cached(anchor, ("linear_as_tp", in_size, str(x.device)), lambda: (
-        lambda t: t.to(x.device) if t is not None else None)(_as_tensor_product(plan, in_size)))
-    if info is None or _uvw_mfma.uv_config_of(info) < 0:
+    def build():
+        info = _as_tensor_product(plan, in_size)
+        return False if info is None else info.to(x.device)     # False: memoised "no such product"
+
+    info = cached(anchor, ("linear_as_tp", in_size, str(x.device)), build)
+    if info is False or _uvw_mfma.uv_config_of(info) < 0:
         return None
     ones = cached(anchor, ("ones", x.shape[0], str(x.device)),
                   lambda: torch.ones(x.shape[0], 1, dtype=torch.bfloat16, device=x.device))
