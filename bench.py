@@ -365,13 +365,17 @@ def uvw_fwd_bwd_bench(args, mod, x, sh, w, cfg, flops, irreps, gen):
         "kernels": {k: round(v, 5) for k, v in kern.items()}}))
 
 
-def make_inputs(lmax, ch, n_nodes, n_edges, n_rot, device):
-    """Seeded CPU generation in the fixed order src, dst, x, vec -> sh, W, ct; then moved to the device."""
+def make_inputs(lmax, ch, n_nodes, n_edges, n_rot, device, graph="uniform"):
+    """Seeded CPU generation in the fixed order src, dst, x, vec -> sh, W, ct; then moved to the device.
+    ``graph='local'`` (not the BASELINE workload): every edge starts within 64 node ids of where it ends, the
+    locality a radius graph over spatially ordered atoms has."""
     from equitorch_amd.utils._sh import spherical_harmonics
     gen = torch.Generator().manual_seed(0)
     d = (lmax + 1) ** 2
     src = torch.randint(0, n_nodes, (n_edges,), generator=gen)
     dst = torch.randint(0, n_nodes, (n_edges,), generator=gen)
+    if graph == "local":
+        src = (dst + torch.randint(-64, 65, (n_edges,), generator=gen)) % n_nodes
     x = torch.randn(n_nodes, d, ch, generator=gen)
     vec = torch.randn(n_edges, 3, generator=gen)
     sh = spherical_harmonics(vec / vec.norm(dim=-1, keepdim=True), lmax)
@@ -532,6 +536,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="edge_fwd_bwd", choices=sorted(WORKLOADS))
     ap.add_argument("--rotate", type=int, default=4, help="number of weight buffers cycled through")
+    ap.add_argument("--graph", default="uniform", choices=["uniform", "local"],
+                    help="edge workloads: uniform random src/dst (BASELINE) or edges between nearby node ids")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-edges", type=int, default=16384)
     ap.add_argument("--pos-per-wave", type=int, default=0,
@@ -575,7 +581,7 @@ def main():
     irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
     mod = SO3Linear(irreps, irreps, irreps, ch, ch, internal_weights=False, feature_mode="uu").to(dev)
     p = mod.num_paths
-    inp = make_inputs(lmax, ch, n_nodes, n_edges, args.rotate, dev)
+    inp = make_inputs(lmax, ch, n_nodes, n_edges, args.rotate, dev, args.graph)
     d = inp["d"]
     plan = EdgePlan(inp["src"].to(dev), inp["dst"].to(dev), n_nodes)
     x = inp["x"].to(dev).requires_grad_(backward)
@@ -641,7 +647,8 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"{args.workload}: N={n_nodes} nodes, E={n_edges} edges, irreps {irreps}, "
-                               f"C={ch}, per-edge weights (E,{p},{ch}), {args.rotate} rotating weight buffers"},
+                               f"C={ch}, per-edge weights (E,{p},{ch}), {args.rotate} rotating weight buffers"
+                               + ("" if args.graph == "uniform" else f", {args.graph} graph")},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": int(MEASURED_TRAFFIC_KIB[args.workload] * 1024),

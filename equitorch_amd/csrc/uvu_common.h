@@ -29,6 +29,20 @@ struct UvuDev {
   int y_vec;  // segment mode: y holds edge vectors (kYUnitVector / kYRawVector) instead of harmonics
 };
 
+// Segment mode: which range of the sorted edge list a wavefront takes.  Workgroups are dispatched to the 8 XCDs
+// round-robin (workgroup b runs on XCD b % 8); handing XCD k the k-th contiguous eighth of the ranges keeps the rows
+// gathered by one XCD's wavefronts — rows near its own segments when edges connect nearby nodes — inside that
+// XCD's L2.  Returns -1 for the padding workgroups of the last eighth.
+__device__ __forceinline__ int64_t seg_wave_index(int64_t n_waves) {
+  const int waves_per_block = blockDim.x / kWave;
+  const int64_t blocks = (n_waves + waves_per_block - 1) / waves_per_block;
+  const int64_t per_xcd = (blocks + 7) / 8;
+  const int64_t block = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if ((int64_t)(blockIdx.x >> 3) >= per_xcd || block >= blocks) return -1;
+  const int64_t wave = block * waves_per_block + threadIdx.x / kWave;
+  return wave < n_waves ? wave : -1;
+}
+
 struct Lanes {
   int lane, lpe, slots, slot, cl;
   __device__ __forceinline__ explicit Lanes(int lpe_log2) {

@@ -254,8 +254,8 @@ template <class TP, typename T, int V, bool YV = false>
 __global__ void __launch_bounds__(256) uvu_seg_fwd_kernel(const UvuDev<T> a, int64_t n_waves) {
   constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
   const Lanes L(a.lpe_log2);
-  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
-  if (wave >= n_waves) return;
+  const int64_t wave = seg_wave_index(n_waves);
+  if (wave < 0) return;
   const int c0 = L.cl * V;
   const bool cok = c0 < a.C;
   const int64_t C = a.C;
@@ -301,8 +301,8 @@ template <class TP, typename T, int V, int GW, bool YV = false>
 __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, int64_t n_waves) {
   constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
   const Lanes L(a.lpe_log2);
-  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
-  if (wave >= n_waves) return;
+  const int64_t wave = seg_wave_index(n_waves);
+  if (wave < 0) return;
   const int c0 = L.cl * V;
   const bool cok = c0 < a.C;
   const int64_t C = a.C;
@@ -637,6 +637,12 @@ static UvuDev<T> to_dev(const cgtp_uvu_args* a, const UvuPlan& plan) {
   return d;
 }
 
+// Workgroups of a segment-mode launch: 4 wavefronts each, rounded up to whole eighths (see seg_wave_index).
+static inline unsigned seg_grid(int64_t n_waves) {
+  const int64_t blocks = (n_waves + 3) / 4;
+  return (unsigned)(((blocks + 7) / 8) * 8);
+}
+
 static inline int launched() { return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH; }
 
 template <typename T>
@@ -686,8 +692,8 @@ static int launch_fwd(const cgtp_uvu_args* a, const UvuPlan& plan, hipStream_t s
   const int vi = plan.V > 1;
   if (a->n_seg > 0) {
     if (plan.n_waves > 0) {
-      hipLaunchKernelGGL(a->y_vec ? e.seg_fwd_vec[vi] : e.seg_fwd[vi], dim3((unsigned)((plan.n_waves + 3) / 4)), dim3(256), 0, stream, d,
-                         plan.n_waves);
+      hipLaunchKernelGGL(a->y_vec ? e.seg_fwd_vec[vi] : e.seg_fwd[vi], dim3(seg_grid(plan.n_waves)), dim3(256), 0, stream,
+                         d, plan.n_waves);
       if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
     }
     return a->wave_seg ? CGTP_OK : launch_fixup<T>(d.out, d, (int64_t)e.dims[2] * a->C, stream);
@@ -712,8 +718,9 @@ static int launch_bwd(const cgtp_uvu_args* a, const UvuPlan& plan, hipStream_t s
     if (wred) (void)hipMemsetAsync(a->grad_w, 0, sizeof(T) * w_elems, stream);
   } else {
     const int gwm = !a->grad_w ? kGwNone : (wred ? kGwReduce : kGwStore);
-    hipLaunchKernelGGL(seg ? (a->y_vec ? e.seg_bwd_vec[vi][gwm] : e.seg_bwd[vi][gwm]) : e.bwd[vi][gwm], dim3((unsigned)((plan.n_waves + 3) / 4)),
-                       dim3(256), 0, stream, d, plan.n_waves);
+    hipLaunchKernelGGL(seg ? (a->y_vec ? e.seg_bwd_vec[vi][gwm] : e.seg_bwd[vi][gwm]) : e.bwd[vi][gwm],
+                       dim3(seg ? seg_grid(plan.n_waves) : (unsigned)((plan.n_waves + 3) / 4)), dim3(256), 0, stream, d,
+                       plan.n_waves);
     if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
     if (wred) {
       hipLaunchKernelGGL(partial_sum_kernel<T>, dim3((unsigned)((w_elems + 255) / 256)), dim3(256), 0, stream,
