@@ -16,8 +16,6 @@ from __future__ import annotations
 import os
 from collections import OrderedDict
 
-import numpy as np
-
 from .._tables import fingerprint, tp_coo
 from ..irreps import Irreps, irrep_segments
 from ..utils import tp_infos

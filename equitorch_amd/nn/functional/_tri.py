@@ -10,7 +10,7 @@ its sibling Functions and rotated tables, ``equitorch/nn/functional/sparse_produ
 """
 from __future__ import annotations
 
-from typing import Optional, Sequence, Tuple
+from typing import Optional, Sequence
 
 import numpy as np
 import torch

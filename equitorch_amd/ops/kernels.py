@@ -14,7 +14,7 @@ import torch
 from torch import Tensor
 
 from .. import _lib
-from .._lib import OPERAND_NONE, OPERAND_SCALAR, OPERAND_VEC, Operand, TriArgs, UvuArgs
+from .._lib import OPERAND_NONE, OPERAND_VEC, Operand, TriArgs, UvuArgs
 from .._tables import TpCoo, fingerprint, pack_tri_table, tp_coo
 
 # ---- per-table caches (keyed by the identity of a table tensor; dropped with it) --------------------------

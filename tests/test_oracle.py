@@ -1,7 +1,6 @@
 """Pins of the numeric oracle: the dense float64 einsum oracle against textbook identities, O(3)
 equivariance and autograd's own gradcheck, and the structural restatement of the reference's CPU path against
 the dense oracle."""
-import numpy as np
 import pytest
 import torch
 
