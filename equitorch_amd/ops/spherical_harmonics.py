@@ -48,9 +48,12 @@ def spherical_harmonics(input: Tensor, l_max: int, dim: int = -1, normalize: boo
     if input.shape[dim] != 3:
         raise ValueError(f"expected 3 components along dim {dim}, got shape {tuple(input.shape)}")
     _lib.require_gpu(input)
-    if input.dtype not in (torch.float32, torch.float64):
+    if not input.dtype.is_floating_point:
         raise _lib.CgtpError(f"spherical_harmonics: unsupported dtype {input.dtype}")
     moved = input.movedim(dim, -1)
     flat = moved.reshape(-1, 3).contiguous()
-    out = _SphericalHarmonics.apply(flat, l_max, normalize, scale)
+    if flat.dtype in (torch.float32, torch.float64):
+        out = _SphericalHarmonics.apply(flat, l_max, normalize, scale)
+    else:   # half precisions: evaluated in fp32, rounded once
+        out = _SphericalHarmonics.apply(flat.float(), l_max, normalize, scale).to(input.dtype)
     return out.reshape(*moved.shape[:-1], (l_max + 1) ** 2).movedim(-1, dim)

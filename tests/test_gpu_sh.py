@@ -76,6 +76,14 @@ def test_module_layout_options_and_edge_cases(device):
     assert_close(y0, torch.tensor([[1.0] + [0.0] * 8], dtype=torch.float64), tol=1e-12, what="zero vector")
     y0.sum().backward()
     assert torch.isfinite(z.grad).all()
+    # half precision: evaluated in fp32 and rounded once; gradients flow back in the input's dtype
+    vb = _vectors(10, seed=4).to(device, torch.bfloat16).requires_grad_(True)
+    yb = spherical_harmonics(vb, 2, normalize_input=True)
+    assert yb.dtype == torch.bfloat16
+    assert_close(yb.float(), ref_sh.spherical_harmonics(ref_sh.normalize(vb.detach().double().cpu()), 2), tol=1e-2,
+                 what="bf16")
+    yb.sum().backward()
+    assert vb.grad.dtype == torch.bfloat16 and torch.isfinite(vb.grad).all()
     with pytest.raises(ValueError):
         spherical_harmonics(torch.zeros(4, 2, device=device), 2)
     with pytest.raises(ValueError):
