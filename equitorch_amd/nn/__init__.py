@@ -2,6 +2,9 @@
 from . import functional
 from .activations import Gate
 from .angular import SinCos
+from .dropout import Dropout
+from .others import Separable, SplitIrreps
+from .rotations import AnglesToMatrix
 from .cutoffs import CosineCutoff, MollifierCutoff, PolynomialCutoff
 from .linears import IrrepsLinear, IrrepWiseLinear, SO2Linear, SO3Linear
 from .norm import MeanSquaredNorm, Norm, SquaredNorm
@@ -14,4 +17,4 @@ from .wigner_d import AlignToZWignerD, DenseWignerRotation, SparseWignerRotation
 __all__ = ["SO3Linear", "IrrepsLinear", "IrrepWiseLinear", "TensorProduct", "SphericalHarmonics", "XYZToSpherical", "SphericalToXYZ", "Gate", "SquaredNorm", "Norm", "MeanSquaredNorm",
            "BatchRMSNorm", "LayerRMSNorm", "BesselBasis", "PolynomialCutoff", "CosineCutoff", "MollifierCutoff",
            "SO2Linear", "SinCos", "SparseWignerRotation", "DenseWignerRotation", "WignerD", "AlignToZWignerD",
-           "functional"]
+           "Dropout", "SplitIrreps", "Separable", "AnglesToMatrix", "functional"]

@@ -2,6 +2,8 @@
 from .activations import gating
 from .angular import sincos
 from .cutoffs import cosine_cutoff, mollifier_cutoff, polynomial_cutoff, radial_standarize
+from .dropout import irrep_wise_dropout
+from .rotations import angles_to_matrix
 from .edge import EdgePlan, edge_tensor_product_uu, edge_tensor_product_uu_vectors
 from .linears import (irrep_wise_linear, irreps_linear, so3_linear_uu, so3_linear_uv, tensor_product_1uu, tensor_product_1vu, tensor_product_u1u,
                       tensor_product_u1v, tensor_product_uu1, tensor_product_vu1)
@@ -22,5 +24,5 @@ __all__ = [
     "xyz_to_spherical", "spherical_to_xyz", "gating", "squared_norm", "norm", "channel_mean_squared_norm",
     "batch_mean_squared_norm", "batch_rms_norm", "layer_rms_norm", "radial_standarize", "polynomial_cutoff",
     "cosine_cutoff", "mollifier_cutoff", "sincos", "xyz_to_sincos", "sparse_wigner_rotation",
-    "dense_wigner_rotation", "wigner_d_matrix", "align_to_z_wigner_d",
+    "dense_wigner_rotation", "wigner_d_matrix", "align_to_z_wigner_d", "irrep_wise_dropout", "angles_to_matrix",
 ]

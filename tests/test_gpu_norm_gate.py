@@ -115,3 +115,29 @@ def test_rms_normalisation_layers(device, affine):
     assert_close(bn(x.to(device)), ref_eval, tol=1e-12, what="batch rms (evaluation)")
     with pytest.raises(ValueError):
         bn(x.to(device)[:, :5])
+
+
+def test_irrep_wise_dropout(device):
+    """Whole irrep blocks of a channel are dropped together and the survivors scaled by 1 / (1 - p); evaluation mode
+    is the identity; the gradient is the mask itself."""
+    from equitorch_amd.nn import Dropout
+    torch.manual_seed(0)
+    drop = Dropout(p=0.4, irreps=IRR).to(device)
+    x = (1.0 + torch.rand(64, 12, 16, device=device)).requires_grad_(True)      # strictly positive entries
+    y = drop(x)
+    ratio = (y / x).detach()
+    assert torch.all((ratio - 0).abs().lt(1e-6) | (ratio - 1 / 0.6).abs().lt(1e-5))
+    seg = [0, 1, 4, 9, 12]
+    for a, b in zip(seg[:-1], seg[1:]):
+        block = ratio[:, a:b]
+        assert float((block - block[:, :1]).abs().max()) < 1e-5                  # one decision per irrep and channel
+    kept = float((ratio > 0).float().mean())
+    assert 0.5 < kept < 0.7
+    (g,) = torch.autograd.grad(y.sum(), x)
+    assert_close(g, ratio, tol=1e-5, what="dropout gradient")
+    drop.eval()
+    assert drop(x) is x
+    plain = Dropout(p=0.5, irrep_wise=False).to(device).train()
+    z = plain(x.detach())
+    per_channel = (z != 0).float().mean(dim=1)
+    assert torch.all((per_channel == 0) | (per_channel == 1))                     # whole channels
