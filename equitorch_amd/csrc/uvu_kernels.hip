@@ -313,13 +313,26 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, 
   zero_rows(acc);
   SegStep st;
   st.next_row = R.s0;
+  // The rows of x belong to the segment, not to the edge: they stay in registers over the steps of a segment (every
+  // load instruction costs delivery bandwidth, whether or not it hits in cache).
+  T x[D1][V];
+  zero_rows(x);
+  int x_seg = -1;
   for (int64_t cb = R.p0; cb < R.p1; cb += kWave) {
   const SegIndexRegs I(a.seg_ids, a.perm, a.gather, cb, cb + kWave < R.p1 ? cb + kWave : R.p1, L.lane);
   for (int off0 = 0; off0 < I.npos;) {
     int ei, oi;
-    if (seg_step_begin<T, D1, V>(st, acc, a.gx, a.ws, I, off0, ei, oi, wave, R, L, a.lpe_log2, cok, C, c0)) {
+    const bool valid = seg_step_begin<T, D1, V>(st, acc, a.gx, a.ws, I, off0, ei, oi, wave, R, L, a.lpe_log2, cok, C, c0);
+    if (st.cur != x_seg) {   // the same for all lanes of the wavefront
+      x_seg = st.cur;
+      if (cok) {
+#pragma unroll
+        for (int i = 0; i < D1; ++i) load_vec<T, V>(x[i], a.x + ((int64_t)x_seg * D1 + i) * C + c0);
+      }
+    }
+    if (valid) {
       const int64_t e = ei, gr = oi;
-      T x[D1][V], g[DO][V], y[D2], gy[D2];
+      T g[DO][V], y[D2], gy[D2];
       T ux = 0, uy = 0, uz = 0;
       if constexpr (YV) {
         ux = a.y[e * 3]; uy = a.y[e * 3 + 1]; uz = a.y[e * 3 + 2];
@@ -332,8 +345,6 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, 
 #pragma unroll
       for (int j = 0; j < D2; ++j) gy[j] = T(0);
       if (cok) {
-#pragma unroll
-        for (int i = 0; i < D1; ++i) load_vec<T, V>(x[i], a.x + ((int64_t)st.cur * D1 + i) * C + c0);
 #pragma unroll
         for (int m = 0; m < DO; ++m) load_vec<T, V>(g[m], a.g + (gr * DO + m) * C + c0);
         const T* wrow = a.w + (a.w_shared ? 0 : e) * P * C + c0;
