@@ -2,7 +2,8 @@
 
 Mirrors the public surface of ``equitorch/irreps/__init__.py`` that the sparse
 Clebsch-Gordan path touches (``Irrep``, ``Irreps``, ``check_irreps``, ``has_path``,
-``irrep_segments``; reference lines 12-158, 161-238, 240-338, 558-717, 889-921).
+``irrep_segments`` and the index helpers ``unique_irreps``, ``irrep_indices``, ``irrep_degrees``,
+``element_degrees``, ``element_orders``; reference lines 12-158, 161-238, 240-338, 558-717, 841-974).
 
 Conventions kept from the reference: a feature tensor is ``(batch, irreps.dim, channels)``
 and the multiplicity of an ``Irreps`` entry is *not* the channel count; parity is stored as
@@ -15,6 +16,7 @@ import re
 from typing import Iterator, List, Sequence, Tuple, Union
 
 _PARITY = {"e": 1, "o": -1, 1: 1, -1: -1, 0: 0, None: 0}
+p_mapping = _PARITY   # the reference's public name (``:8-10``)
 _TERM = re.compile(r"(?:(\d+)x)?(\d+)([eo]?)")
 
 
@@ -281,3 +283,38 @@ def irrep_segments(irreps) -> List[int]:
     for ir in check_irreps(irreps):
         seg.append(seg[-1] + ir.dim)
     return seg
+
+
+def unique_irreps(irreps):
+    """``(Irreps of the distinct irreps in order of first appearance, {irrep: positions in the expanded sequence})``
+    (reference ``:841-887``): ``unique_irreps("0+0e+1o+0e+0e") -> (Irreps(0+0e+1o), {0: [0], 0e: [1, 3, 4], 1o: [2]})``."""
+    positions = {}
+    for i, ir in enumerate(check_irreps(irreps)):
+        positions.setdefault(ir, []).append(i)
+    return Irreps(list(positions)), positions
+
+
+def _long_tensor(values):
+    import torch   # only these helpers return tensors; the rest of the module is torch-free
+    return torch.tensor(values, dtype=torch.long)
+
+
+def irrep_indices(irreps):
+    """For every component of the feature, the position of its irrep in the expanded sequence
+    (reference ``:923-952``): ``"0+2x1e+2e" -> [0, 1, 1, 1, 2, 2, 2, 3, 3, 3, 3, 3]``."""
+    return _long_tensor([i for i, ir in enumerate(check_irreps(irreps)) for _ in range(ir.dim)])
+
+
+def irrep_degrees(irreps):
+    """Degree ``l`` of every irrep of the expanded sequence (reference ``:954-959``)."""
+    return _long_tensor([ir.l for ir in check_irreps(irreps)])
+
+
+def element_degrees(irreps):
+    """Degree ``l`` of every component (reference ``:961-966``)."""
+    return _long_tensor([ir.l for ir in check_irreps(irreps) for _ in range(ir.dim)])
+
+
+def element_orders(irreps):
+    """Order ``m = -l .. l`` of every component (reference ``:968-974``)."""
+    return _long_tensor([m for ir in check_irreps(irreps) for m in range(-ir.l, ir.l + 1)])

@@ -157,3 +157,7 @@ def irrep_wise_linear(input: Tensor, weight: Tensor, irreps_info):
     from . import _irreps_gemm as G
     plan = G.plan_of_irreps_info(irreps_info)
     return G.mix(input, weight, plan, plan.out_size, anchor=irreps_info.irrep_seg)
+
+
+# ---- SO(2) linear maps are plain sparse products with the table of ``so2_linear_infos`` (reference :576-577) ----
+from .sparse_product import sparse_mul as so2_linear_uu, sparse_vecmat as so2_linear_uv  # noqa: E402

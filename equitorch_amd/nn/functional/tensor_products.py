@@ -2,6 +2,7 @@
 
     uuu : out[n,M,c] = sum_t c_t x[n,M1_t,c] y[n,M2_t,c] W[(n),p_t,c]                 (:9-90)
     uvw : out[n,M,o] = sum_t c_t sum_{u,v} x[n,M1_t,u] y[n,M2_t,v] W[(n),p_t,u,v,o]   (:92-172)
+    dot : out[n,k,c] = sum_{M in irrep k} x[n,M,c] y[n,M,c]                           (:173-237)
 """
 from typing import Optional
 
@@ -12,7 +13,7 @@ from torch.autograd import Function
 from ... import _lib
 V = "u"  # channel axes of a per-channel operand
 from ...ops import kernels
-from ...structs import TensorProductInfo
+from ...structs import IrrepsInfo, SparseProductInfo, TensorProductInfo
 from ._tri import spec_from_tp_info, tri
 
 
@@ -71,3 +72,23 @@ def tensor_product_uvw(input1: Tensor, input2: Tensor, weight: Tensor,
                              f"weight of {weight.ndim} dims")
     from . import _uvw_gemm
     return _uvw_gemm.uvw(input1.contiguous(), input2.contiguous(), weight, tp_info_forward)
+
+
+def tensor_dot_uu(input1: Tensor, input2: Tensor, irreps_info: IrrepsInfo, scaled: bool = True) -> Tensor:
+    """Irrep-wise, channel-wise dot product ``(..., dim, C), (..., dim, C) -> (..., num_irreps, C)``, divided by
+    ``sqrt(2l+1)`` when ``scaled`` (``TensorDotUU``, reference ``:173-223``).  One segmented product on the
+    table-driven kernel; its gradients of every order come from that kernel's autograd closure."""
+    from .sparse_product import sparse_mul
+    _lib.require_gpu(input1, input2)
+    lead = torch.broadcast_shapes(input1.shape[:-2], input2.shape[:-2])
+    x = input1.expand(*lead, *input1.shape[-2:]).reshape(-1, *input1.shape[-2:])
+    y = input2.expand(*lead, *input2.shape[-2:]).reshape(-1, *input2.shape[-2:])
+    out = sparse_mul(x, y, SparseProductInfo(seg_out=irreps_info.irrep_seg))
+    if scaled:
+        out = out * irreps_info.rsqrt_dims.unsqueeze(-1)
+    return out.reshape(*lead, *out.shape[-2:])
+
+
+def tensor_dot_uv(input1: Tensor, input2: Tensor, irreps_info: IrrepsInfo, scaled: bool = True) -> Tensor:
+    """Declared but not implemented by the reference (``TensorDotUV``, ``:225-237`` raises); same here."""
+    raise NotImplementedError()

@@ -1,5 +1,5 @@
 """``TensorProduct``: weighted tensor product of two channelled features
-(``equitorch/nn/tensor_products.py:19-198``)."""
+(``equitorch/nn/tensor_products.py:19-198``); ``TensorDot``: irrep-wise dot product (``:199-262``)."""
 import math
 from typing import Optional
 
@@ -9,9 +9,10 @@ from torch import Tensor
 from torch.nn import Parameter
 
 from ..irreps import check_irreps
-from ..structs import TensorProductInfo
+from ..structs import IrrepsInfo, TensorProductInfo
 from ..utils._structs import tp_infos
-from .functional.tensor_products import tensor_product_uuu, tensor_product_uvw
+from ._irreps_module import IrrepsModule
+from .functional.tensor_products import tensor_dot_uu, tensor_dot_uv, tensor_product_uuu, tensor_product_uvw
 from .init import initialize_tensor_product
 
 
@@ -96,3 +97,33 @@ class TensorProduct(nn.Module):
                 f"feature_mode={self.feature_mode}, path_norm={self.path_norm}, "
                 f"channel_norm={self.channel_norm}, internal_weights={self.internal_weights}, "
                 f"num_paths={self.num_paths})")
+
+
+class TensorDot(IrrepsModule):
+    r"""Irrep-wise dot product of two features with the same irreps (``equitorch/nn/tensor_products.py:199-262``).
+
+    ``feature_mode='uu'``: ``(..., irreps.dim, C), (..., irreps.dim, C) -> (..., len(irreps), C)``;
+    ``'uv'`` (``-> (..., len(irreps), C1, C2)``) is declared by the reference but raises ``NotImplementedError``
+    there, and does so here.  ``scaled`` divides by ``sqrt(2l+1)``.
+    """
+    irreps_info: IrrepsInfo
+
+    def __init__(self, irreps, feature_mode, scaled=False):
+        super().__init__(irreps)
+        assert feature_mode in ['uv', 'uu']
+        self.feature_mode = feature_mode
+        self.scaled = scaled
+
+    def forward(self, input1: Tensor, input2: Tensor) -> Tensor:
+        assert input1.shape[-2] == self.irreps_dim, \
+            f"Input1 spherical dim mismatch: expected {self.irreps_dim}, got {input1.shape[-2]}"
+        assert input2.shape[-2] == self.irreps_dim, \
+            f"Input2 spherical dim mismatch: expected {self.irreps_dim}, got {input2.shape[-2]}"
+        if self.feature_mode == 'uu':
+            assert input1.shape[-1] == input2.shape[-1], \
+                f"Input channel dims must match in 'uu' mode. Got {input1.shape[-1]} and {input2.shape[-1]}"
+            return tensor_dot_uu(input1, input2, self.irreps_info, self.scaled)
+        return tensor_dot_uv(input1, input2, self.irreps_info, self.scaled)
+
+    def extra_repr(self) -> str:
+        return f"irreps={self.irreps}, feature_mode={self.feature_mode}, scaled={self.scaled}"

@@ -393,3 +393,26 @@ def so2_linear_infos(irreps_out, irreps_in, path=None, path_norm=True, channel_n
     index1, index2, index_out, scales, n = prepare_so2_linear(irreps_out, irreps_in, path, path_norm, channel_norm,
                                                               channel_scale)
     return (*sparse_product_infos(index1, index2, index_out, scales, irreps_out.dim, irreps_in.dim, n), n)
+
+
+def so2_linear_info(irreps_out, irreps_in, path=None, path_norm=True, channel_norm=False, channel_scale=1.0):
+    """``(forward table, num_weights)`` (reference ``:780-782``)."""
+    irreps_out, irreps_in = check_irreps(irreps_out), check_irreps(irreps_in)
+    index1, index2, index_out, scales, n = prepare_so2_linear(irreps_out, irreps_in, path, path_norm, channel_norm,
+                                                              channel_scale)
+    return sparse_product_info(index1, index2, index_out, scales, irreps_out.dim), n
+
+
+def irreps_blocks_infos(irreps):
+    """Tables of the block-diagonal action of one dense ``(2l+1, 2l+1)`` matrix per irrep on a feature
+    (reference ``:656-671``): entry ``q`` multiplies matrix element ``q`` (blocks laid out one after the other,
+    row-major) with input component ``M_in`` into output component ``M_out``."""
+    irreps = check_irreps(irreps)
+    index_in, index_out, first = [], [], 0
+    for ir in irreps:
+        for m_out in range(first, first + ir.dim):
+            for m_in in range(first, first + ir.dim):
+                index_in.append(m_in)
+                index_out.append(m_out)
+        first += ir.dim
+    return sparse_product_infos(list(range(len(index_in))), index_in, index_out)

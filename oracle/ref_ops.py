@@ -259,6 +259,14 @@ def cpu_squared_norm(x, info, scaled=True):
     return out * torch.tensor(info["rdims"], dtype=x.dtype).unsqueeze(-1) if scaled else out
 
 
+def cpu_tensor_dot(x1, x2, info, scaled=True):
+    """``TensorDotUU.forward`` (equitorch/nn/functional/tensor_products.py:176-198): the products summed over the
+    components of each irrep, times ``dim^-1/2`` when ``scaled``.  Pinned in tests/test_oracle_norms.py by the
+    per-block dot product written out with slices and by ``dot(x, x) = squared norm``."""
+    out = _block_sum(x1 * x2, info["irrep_seg"])
+    return out * torch.tensor(info["rsqrt_dims"], dtype=out.dtype).unsqueeze(-1) if scaled else out
+
+
 def cpu_norm(x, info, scaled=True):
     """``Norm.forward`` (:80-98); its backward (:100-126) puts a zero gradient at zero blocks."""
     out = torch.sqrt(_block_sum(x.pow(2), info["irrep_seg"]))

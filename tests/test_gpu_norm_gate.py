@@ -141,3 +141,47 @@ def test_irrep_wise_dropout(device):
     z = plain(x.detach())
     per_channel = (z != 0).float().mean(dim=1)
     assert torch.all((per_channel == 0) | (per_channel == 1))                     # whole channels
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("scaled", [True, False])
+def test_tensor_dot(device, dtype, scaled):
+    """``TensorDot('uu')``: irrep-wise dot product and both gradients against the oracle; extra leading axes and a
+    broadcast second operand; ``'uv'`` raises as in the reference."""
+    from equitorch_amd.nn import TensorDot
+    info = _info()
+    x, g = _data(37, 24, dtype, seed=5)
+    y = torch.randn(37, 12, 24, generator=g, dtype=torch.float64).to(dtype).double()
+    ct = torch.randn(37, 4, 24, generator=g, dtype=torch.float64).to(dtype).double()
+    xr, yr = x.clone().requires_grad_(True), y.clone().requires_grad_(True)
+    ref = ref_ops.cpu_tensor_dot(xr, yr, info, scaled)
+    rg = torch.autograd.grad(ref, (xr, yr), ct)
+    mod = TensorDot(IRR, "uu", scaled=scaled).to(device)
+    xd, yd = (t.to(device, dtype).requires_grad_(True) for t in (x, y))
+    out = mod(xd, yd)
+    got = torch.autograd.grad(out, (xd, yd), ct.to(device, dtype))
+    tol = 1e-5 if dtype == torch.float32 else 1e-12
+    for name, a, b in (("out", out, ref), ("grad_1", got[0], rg[0]), ("grad_2", got[1], rg[1])):
+        assert_close(a, b, tol=tol, what=f"tensor dot scaled={scaled} {name}")
+    lead = mod(xd.detach().reshape(1, 37, 12, 24).expand(2, 37, 12, 24), yd.detach())
+    assert lead.shape == (2, 37, 4, 24)
+    assert_close(lead[1], ref, tol=tol, what="leading axes")
+    with pytest.raises(NotImplementedError):
+        TensorDot(IRR, "uv").to(device)(xd, yd)
+
+
+def test_xyz_to_sincos_module(device):
+    """``XYZToSinCos``: ``[1, sin(m a), cos(m a)]_m`` of the polar angles, against atan2 / acos in float64."""
+    from equitorch_amd.nn import XYZToSinCos
+    g = torch.Generator().manual_seed(6)
+    v = torch.randn(50, 3, generator=g, dtype=torch.float64)
+    u = v / v.norm(dim=-1, keepdim=True)
+    theta, phi = torch.acos(u[:, 2].clamp(-1, 1)), torch.atan2(u[:, 1], u[:, 0])
+    for normalised in (False, True):
+        st, sp = XYZToSinCos(3, component_normalize=normalised)(v.to(device))
+        scale = 2 ** 0.5 if normalised else 1.0
+        for got, ang in ((st, theta), (sp, phi)):
+            assert got.shape == (50, 7)
+            ref = torch.stack([torch.ones_like(ang)] + [f(m * ang) * scale for m in (1, 2, 3)
+                                                        for f in (torch.sin, torch.cos)], dim=-1)
+            assert_close(got, ref, tol=1e-10, what=f"sincos normalised={normalised}")

@@ -36,3 +36,18 @@ def test_gate_and_normalisation_oracle_properties():
     torch.testing.assert_close(ref_ops.cpu_batch_mean_squared_norm(z, info, True), torch.ones(3, 4, dtype=torch.float64))
     stat = ref_ops.cpu_batch_mean_squared_norm(x, info, True)
     torch.testing.assert_close(running, 0.75 * torch.ones(3, 4, dtype=torch.float64) + 0.25 * stat)
+
+
+def test_tensor_dot_oracle_against_hand_written_blocks():
+    info = ref_tables.irreps_info("0e+1o+2e")
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(6, 9, 5, generator=g, dtype=torch.float64)
+    y = torch.randn(6, 9, 5, generator=g, dtype=torch.float64)
+    dots = torch.stack([(x[:, a:b] * y[:, a:b]).sum(1) for a, b in ((0, 1), (1, 4), (4, 9))], dim=1)
+    dims = torch.tensor([1.0, 3.0, 5.0], dtype=torch.float64)
+    torch.testing.assert_close(ref_ops.cpu_tensor_dot(x, y, info, False), dots)
+    torch.testing.assert_close(ref_ops.cpu_tensor_dot(x, y, info, True), dots / dims.sqrt()[:, None])
+    torch.testing.assert_close(ref_ops.cpu_tensor_dot(x, x, info, False), ref_ops.cpu_squared_norm(x, info, False))
+    # the l = 1 block is the Euclidean dot product of the two vectors, whatever the component order
+    torch.testing.assert_close(ref_ops.cpu_tensor_dot(x, y, info, False)[:, 1],
+                               torch.einsum("nmc,nmc->nc", x[:, 1:4], y[:, 1:4]))
