@@ -37,6 +37,9 @@ def _movable(cls):
     return cls
 
 
+add_operation_methods = _movable   # the reference's name for this class decorator (``structs/__init__.py:7-47``)
+
+
 @_movable
 class SparseScaleInfo(NamedTuple):
     """``z[M] = sum_{t in seg_out[M]..seg_out[M+1]} scale[t] * x[index[t]]``."""

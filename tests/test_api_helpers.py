@@ -61,3 +61,33 @@ def test_irreps_blocks_and_so2_linear_tables():
     for f in ("scale", "index1", "index2", "seg_out", "gather_index", "index_out"):
         a, b = getattr(one, f), getattr(three[0], f)
         assert (a is None and b is None) or torch.equal(a, b)
+
+
+def test_transforms_without_pyg():
+    """The data transforms on a plain attribute container: the radius graph against a double loop (centres in index
+    order, first ``max_num_neighbors`` neighbours, examples of a batch kept apart), norms and length embeddings."""
+    from types import SimpleNamespace
+
+    from equitorch_amd import transforms as T
+    g = torch.Generator().manual_seed(3)
+    pos = torch.rand(40, 3, generator=g, dtype=torch.float64)
+    batch = (torch.arange(40) >= 25).long()
+    data = SimpleNamespace(pos=pos, batch=batch)
+    out = T.RadiusGraph(0.45, max_num_neighbors=4)(data)
+    assert not hasattr(data, "edge_index")                       # applied to a shallow copy
+    want = []
+    for i in range(40):
+        nb = [j for j in range(40) if j != i and batch[i] == batch[j] and (pos[i] - pos[j]).norm() < 0.45][:4]
+        want += [(j, i) for j in nb]
+    assert out.edge_index.dtype == torch.long
+    assert sorted(map(tuple, out.edge_index.t().tolist())) == sorted(want)
+    torch.testing.assert_close(out.edge_vec, pos[out.edge_index[1]] - pos[out.edge_index[0]])
+    flipped = T.RadiusGraph(0.45, max_num_neighbors=4, flow="target_to_source")(data)
+    assert torch.equal(flipped.edge_index, out.edge_index.flip(0))
+    loops = T.RadiusGraph(0.2, loop=True, max_num_neighbors=64)(SimpleNamespace(pos=pos, batch=None))
+    assert ((loops.edge_index[0] == loops.edge_index[1]).sum()) == 40
+    out = T.AddVectorNorm()(out)
+    torch.testing.assert_close(out.edge_norm, out.edge_vec.norm(dim=-1))
+    out = T.AddVectorLengthEmbedding(lambda d: torch.stack([d, d * d], dim=-1))(out)
+    torch.testing.assert_close(out.edge_emb[:, 1], out.edge_norm ** 2)
+    assert repr(T.RadiusGraph(0.5)) == "RadiusGraph(r=0.5)"

@@ -145,3 +145,19 @@ def test_edge_product_with_harmonics_evaluated_in_the_kernel(device, lmax, chann
     for name, a, b in (("out", out, ref), ("grad_x", xd.grad, xr.grad), ("grad_vec", vd.grad, vr.grad),
                        ("grad_w", wd.grad, wr.grad)):
         assert_close(a, b, tol=tol, what=f"lmax={lmax} {name}")
+
+
+def test_add_spherical_harmonics_transform(device):
+    """``transforms.AddSphericalHarmonics`` on a plain attribute container: the harmonics of the raw edge vectors
+    (``r^l`` scaling kept, as in the reference's transform), with and without the ``1 / sqrt(4 pi)`` factor."""
+    from types import SimpleNamespace
+
+    from equitorch_amd.transforms import AddSphericalHarmonics, AddVectorNorm
+    v = _vectors(257, seed=21)
+    data = SimpleNamespace(edge_vec=v.to(device))
+    out = AddVectorNorm()(AddSphericalHarmonics(3)(data))
+    assert out.edge_sh.shape == (257, 16) and not hasattr(data, "edge_sh")
+    assert_close(out.edge_sh, ref_sh.spherical_harmonics(v, 3), tol=1e-12, what="edge_sh")
+    assert_close(out.edge_norm, v.norm(dim=-1), tol=1e-12, what="edge_norm")
+    scaled = AddSphericalHarmonics(2, sh_attr="y", integral_normalize=True)(data)
+    assert_close(scaled.y, ref_sh.spherical_harmonics(v, 2) / math.sqrt(4 * math.pi), tol=1e-12, what="scaled")
