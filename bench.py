@@ -136,7 +136,7 @@ def sh_bench(steps, warmup):
                       "unit": "Mvectors/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 5),
                       "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
                       "config": {"workload": f"sh: {n} vectors, degrees 0..{lmax}, input normalised in the kernel"},
-                      "roofline": {"bound": "hbm", "kernel": "cgtp::sh_kernel<float,false>", "achieved": round(gbs, 1),
+                      "roofline": {"bound": "hbm", "kernel": "cgtp::sh_kernel<float,false,6>", "achieved": round(gbs, 1),
                                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                                    "traffic": None, "algorithmic_bytes": f_bytes, "avg_ms": round(f_ms, 5)},
                       "kernels": {"fwd_avg_ms": round(f_ms, 5), "fwd_GBs": round(gbs, 1), "bwd_avg_ms": round(b_ms, 5),

@@ -13,6 +13,8 @@
 // HBM-bound: 3 values in, (lmax+1)^2 out per vector.  Rows of 64 vectors are exchanged through a wavefront-private
 // LDS tile so that global loads and stores are contiguous; when a tile would not fit (high degree), lanes address
 // global memory directly.
+#include <utility>
+
 #include "cgtp_host.h"
 
 #include "sh_device.h"
@@ -21,6 +23,7 @@ namespace cgtp {
 namespace {
 
 constexpr int kShBlock = 256;       // most vectors per workgroup, one per lane
+constexpr int kShUnrolled = 8;      // degrees up to this one have kernels with the degree compiled in
 
 // Row `lane` of a (64 x D) tile: in LDS at pitch `pitch`, or straight in global memory at pitch D.
 template <typename T>
@@ -31,9 +34,41 @@ struct ShRow {
 
 // Copies the wavefront's `cnt` rows of D values between the LDS tile and the contiguous global range, eight
 // independent 256-byte row segments in flight per step (a global load per iteration would serialise on latency).
-template <typename T, bool TO_GLOBAL>
-__device__ __forceinline__ void sh_tile_copy(T* tile, int pitch, T* glob, int cnt, int D, int lane) {
+// Element j of the range is element j + (j / D) * (pitch - D) of the tile.  DC > 0: D is the compile-time constant
+// DC; a full tile (64 rows) is then copied by straight-line code with constant offsets.
+template <typename T, bool TO_GLOBAL, int DC>
+__device__ __forceinline__ void sh_tile_copy(T* tile, int pitch, T* glob, int cnt, int D_arg, int lane) {
   constexpr int kBatch = 8;
+  const int D = DC > 0 ? DC : D_arg;
+  if (DC > 0 && cnt == 64) {
+    const int pad = pitch - D;     // 0 or 1
+#pragma unroll
+    for (int t0 = 0; t0 < (DC > 0 ? DC : 1); t0 += kBatch) {
+      T v[kBatch];
+      int at[kBatch];
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) {
+        const int j = lane + 64 * (t0 + k);
+        at[k] = j + (pad ? j / D : 0);
+      }
+      if (TO_GLOBAL) {
+#pragma unroll
+        for (int k = 0; k < kBatch; ++k)
+          if (t0 + k < D) v[k] = tile[at[k]];
+#pragma unroll
+        for (int k = 0; k < kBatch; ++k)
+          if (t0 + k < D) glob[lane + 64 * (t0 + k)] = v[k];
+      } else {
+#pragma unroll
+        for (int k = 0; k < kBatch; ++k)
+          if (t0 + k < D) v[k] = glob[lane + 64 * (t0 + k)];
+#pragma unroll
+        for (int k = 0; k < kBatch; ++k)
+          if (t0 + k < D) tile[at[k]] = v[k];
+      }
+    }
+    return;
+  }
   const int total = cnt * D;
   const int dq = 64 / D, dr = 64 - dq * D;     // a step of 64 elements = dq rows and dr columns
   int r = lane / D, i = lane - r * D;
@@ -62,13 +97,17 @@ __device__ __forceinline__ void sh_tile_copy(T* tile, int pitch, T* glob, int cn
   }
 }
 
-template <typename T, bool BWD>
+// LT >= 0: the degree is LT, known at compile time (both loops unroll, the coefficients become literals and the
+// tile accesses independent); LT < 0: the degree is the run-time argument.
+template <typename T, bool BWD, int LT>
 __global__ void __launch_bounds__(kShBlock) sh_kernel(const T* __restrict__ xyz, const T* __restrict__ gout,
-                                                      T* __restrict__ out, int64_t n, int lmax, int normalize,
+                                                      T* __restrict__ out, int64_t n, int lmax_arg, int normalize,
                                                       T scale, int pitch) {
   extern __shared__ __align__(16) unsigned char sh_smem[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lmax = LT >= 0 ? LT : lmax_arg;
   const int D = (lmax + 1) * (lmax + 1);
+  constexpr int DC = LT >= 0 ? (LT + 1) * (LT + 1) : -1;
   const int64_t e0 = (int64_t)blockIdx.x * blockDim.x + wave * 64;   // first vector of this wavefront
   const int64_t e = e0 + lane;
   const bool live = e < n;
@@ -88,7 +127,7 @@ __global__ void __launch_bounds__(kShBlock) sh_kernel(const T* __restrict__ xyz,
   // the row this lane reads (backward: grad_out) or writes (forward: Y)
   T* base = BWD ? const_cast<T*>(gout) : out;
   if (BWD && tile) {
-    sh_tile_copy<T, false>(tile, pitch, base + e0 * D, cnt, D, lane);
+    sh_tile_copy<T, false, DC>(tile, pitch, base + e0 * D, cnt, D, lane);
     __syncthreads();
   }
   ShRow<T> row{tile ? tile + (size_t)lane * pitch : base + (live ? e : 0) * D};
@@ -96,6 +135,7 @@ __global__ void __launch_bounds__(kShBlock) sh_kernel(const T* __restrict__ xyz,
   T gx = 0, gy = 0, gz = 0;
   T C = 1, S = 0;            // C_m, S_m
   T Cp = 0, Sp = 0;          // C_{m-1}, S_{m-1}
+#pragma unroll
   for (int m = 0; m <= lmax; ++m) {
     T fm = 0;
     if (m > 0) {
@@ -109,6 +149,7 @@ __global__ void __launch_bounds__(kShBlock) sh_kernel(const T* __restrict__ xyz,
     T R1 = 0, R = 1;         // R_{l-1}, R_l (l = m)
     T Rz1 = 0, Rz = 0;       // dR/dz at fixed r^2
     T Rr1 = 0, Rr = 0;       // dR/d(r^2)
+#pragma unroll
     for (int l = m; l <= lmax; ++l) {
       if (l > m) {
         const T a = ShCoef<T>::a(l, m), b = ShCoef<T>::b(l, m);
@@ -141,7 +182,7 @@ __global__ void __launch_bounds__(kShBlock) sh_kernel(const T* __restrict__ xyz,
   if (!BWD) {
     if (tile) {
       __syncthreads();
-      sh_tile_copy<T, true>(tile, pitch, out + e0 * D, cnt, D, lane);
+      sh_tile_copy<T, true, DC>(tile, pitch, out + e0 * D, cnt, D, lane);
     }
   } else if (live) {
     gx *= scale; gy *= scale; gz *= scale;
@@ -179,6 +220,15 @@ int sh_check(const void* xyz, const void* a, const void* b, int64_t n, int lmax,
 }
 
 template <typename T, bool BWD>
+using ShKernel = void (*)(const T*, const T*, T*, int64_t, int, int, T, int);
+
+template <typename T, bool BWD, int... LS>
+ShKernel<T, BWD> sh_pick(int lmax, std::integer_sequence<int, LS...>) {
+  static const ShKernel<T, BWD> table[] = {sh_kernel<T, BWD, LS>...};
+  return lmax <= kShUnrolled ? table[lmax] : sh_kernel<T, BWD, -1>;
+}
+
+template <typename T, bool BWD>
 int sh_launch(const void* xyz, const void* gout, void* out, int64_t n, int lmax, int normalize, double scale,
               int dtype, hipStream_t stream) {
   if (n == 0) return CGTP_OK;
@@ -186,8 +236,9 @@ int sh_launch(const void* xyz, const void* gout, void* out, int64_t n, int lmax,
   const int block = sh.waves * 64;
   const size_t lds = (size_t)block * sh.pitch * sizeof(T);
   const unsigned grid = (unsigned)((n + block - 1) / block);
-  hipLaunchKernelGGL((sh_kernel<T, BWD>), dim3(grid), dim3(block), lds, stream, (const T*)xyz, (const T*)gout,
-                     (T*)out, n, lmax, normalize, (T)scale, sh.pitch);
+  const ShKernel<T, BWD> fn = sh_pick<T, BWD>(lmax, std::make_integer_sequence<int, kShUnrolled + 1>{});
+  hipLaunchKernelGGL(fn, dim3(grid), dim3(block), lds, stream, (const T*)xyz, (const T*)gout, (T*)out, n, lmax,
+                     normalize, (T)scale, sh.pitch);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 
