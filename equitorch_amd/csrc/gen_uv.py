@@ -137,8 +137,13 @@ def emit_direction(name: str, direction: int, coo, seg_out, seg_in1, gy: bool = 
         # hide the harmonics behind an empty asm per tile: equal (coefficient, harmonic) products recur in many
         # tiles and would otherwise be computed once and kept in registers across the whole body
         a("    " + " ".join(f'asm volatile("" : "+v"(yy[{m}]));' for m in sorted({m2 for _, m2, _ in terms})))
+        # one update per output row: the harmonics that couple the same (output row, input row) pair are summed first
+        by_row = OrderedDict()
         for (o, m2, c) in terms:
-            a(f"    {{ const float s = {_lit(c)} * yy[{m2}]; o{o}_0 += s * {cur}0; o{o}_1 += s * {cur}1; }}")
+            by_row.setdefault(o, []).append((m2, c))
+        for o, pairs in by_row.items():
+            s_expr = " + ".join(f"{_lit(c)} * yy[{m2}]" for m2, c in pairs)
+            a(f"    {{ const float s = {s_expr}; o{o}_0 += s * {cur}0; o{o}_1 += s * {cur}1; }}")
         # pin the updated accumulators: an output row is read again only when it is stored, and without this the
         # optimiser sinks every update of a block to its end, keeping all the block's tiles alive until then
         touched = sorted({o for o, _, _ in terms})
