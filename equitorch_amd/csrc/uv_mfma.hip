@@ -135,7 +135,8 @@ __global__ void __launch_bounds__(256, 2) uv_kernel(const __bf16* __restrict__ x
             v[i] = (__bf16)o0[i];
             v[4 + i] = (__bf16)o1[i];
           }
-          *reinterpret_cast<bf16x8*>(orow + row * cout) = v;
+          // written once and not read again by this launch: keep it out of the way of the weights in L2
+          __builtin_nontemporal_store(__builtin_bit_cast(f32x4, v), reinterpret_cast<f32x4*>(orow + row * cout));
         }
       });
 }
