@@ -21,14 +21,31 @@ inline int elem_size(int dtype) {
   }
 }
 
-// out[i] = sum_k ws[k * n + i], accumulated in double in a fixed order (deterministic).
+// out[i] = sum_k ws[k * n + i], accumulated in double in a fixed order (deterministic): 16 threads per column take
+// every 16th partial each, their sums are added in thread order.
+constexpr int kPartialSlices = 16, kPartialCols = 16;
 template <typename T>
-__global__ void partial_sum_kernel(const T* __restrict__ ws, T* __restrict__ out, int64_t n_part, int64_t n) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
+__global__ void __launch_bounds__(kPartialSlices * kPartialCols)
+partial_sum_kernel(const T* __restrict__ ws, T* __restrict__ out, int64_t n_part, int64_t n) {
+  __shared__ double part[kPartialSlices][kPartialCols];
+  const int col = threadIdx.x % kPartialCols, slice = threadIdx.x / kPartialCols;
+  const int64_t i = (int64_t)blockIdx.x * kPartialCols + col;
   double s = 0.0;
-  for (int64_t k = 0; k < n_part; ++k) s += (double)ws[k * n + i];
-  out[i] = (T)s;
+  if (i < n)
+    for (int64_t k = slice; k < n_part; k += kPartialSlices) s += (double)ws[k * n + i];
+  part[slice][col] = s;
+  __syncthreads();
+  if (slice == 0 && i < n) {
+    double total = 0.0;
+    for (int j = 0; j < kPartialSlices; ++j) total += part[j][col];
+    out[i] = (T)total;
+  }
+}
+
+template <typename T>
+inline void launch_partial_sum(const T* ws, T* out, int64_t n_part, int64_t n, hipStream_t stream) {
+  hipLaunchKernelGGL(partial_sum_kernel<T>, dim3((unsigned)((n + kPartialCols - 1) / kPartialCols)),
+                     dim3(kPartialSlices * kPartialCols), 0, stream, ws, out, n_part, n);
 }
 
 // First pass of a sum over many rows: part[c * n + i] = sum of rows[r * n + i] over the rows r of chunk c

@@ -184,6 +184,114 @@ __global__ void __launch_bounds__(256) tri_staged_kernel(const TriDev<T> a, int6
   }
 }
 
+// The same contraction for light tables (about one coefficient per operand row: gates, per-irrep scalings and
+// block sums, rotations about z), where staging cannot pay and the row-by-row kernel above is bound by latency.
+// A row takes LPR = next_pow2(C / V) lanes with V channels each (16-byte accesses), so a wavefront covers 64 / LPR
+// rows at once; the coefficients are walked in table order four at a time, all operand loads of the four issued
+// before any arithmetic, and a result row is stored when the output index changes (the indices are the same for
+// every lane: scalar branches).  No reduction over rows; C / V <= 64.
+template <typename T>
+struct LightOperand {
+  const T* p;        // this lane's row (+ channel for per-channel operands), or nullptr
+  int64_t stride;    // elements between sparse indices
+  bool vec;
+};
+
+template <typename T, int V>
+__device__ __forceinline__ void light_fetch(const LightOperand<T>& o, uint32_t i, T (&dst)[V]) {
+  if (!o.p) {
+#pragma unroll
+    for (int v = 0; v < V; ++v) dst[v] = T(1);
+  } else if (o.vec) {
+    load_vec<T, V>(dst, o.p + (int64_t)i * o.stride);
+  } else {
+    const T x = o.p[(int64_t)i * o.stride];
+#pragma unroll
+    for (int v = 0; v < V; ++v) dst[v] = x;
+  }
+}
+
+template <typename T, int V, bool REDUCE_C>
+__global__ void __launch_bounds__(256) tri_light_kernel(const TriDev<T> a, int lpr_log2) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  constexpr int U = 4;
+  T* s_coef = reinterpret_cast<T*>(smem);
+  uint32_t* s_idx = reinterpret_cast<uint32_t*>(s_coef + a.nnz);
+  int32_t* s_out = reinterpret_cast<int32_t*>(s_idx + a.nnz);      // output index of every coefficient
+  for (int t = threadIdx.x; t < a.nnz; t += blockDim.x) {
+    s_coef[t] = a.coef ? a.coef[t] : T(1);
+    s_idx[t] = a.idx[t];
+  }
+  for (int o = threadIdx.x; o < a.n_out; o += blockDim.x)
+    for (int t = a.seg[o]; t < a.seg[o + 1]; ++t) s_out[t] = o;
+  __syncthreads();
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int lpr = 1 << lpr_log2, slot = lane >> lpr_log2, sub = lane & (lpr - 1);
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  const int64_t r = wave * (kWave >> lpr_log2) + slot;
+  const int c = sub * V;
+  const bool ok = r < a.n_rows && c < a.C;
+  const int64_t rr = r < a.n_rows ? r : 0;       // idle lanes read row 0 and store nothing
+  const int cc = c < a.C ? c : 0;
+  LightOperand<T> ops[3];
+  const OperandDev<T>* src[3] = {&a.a, &a.b, &a.w};
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    ops[k].vec = src[k]->kind == CGTP_OPERAND_VEC;
+    ops[k].stride = src[k]->idx_stride;
+    ops[k].p = src[k]->kind ? row_ptr(*src[k], rr) + (ops[k].vec ? cc : 0) : nullptr;
+  }
+  auto emit = [&](int o, const T (&acc)[V]) __attribute__((always_inline)) {
+    if constexpr (REDUCE_C) {
+      T sum = T(0);
+#pragma unroll
+      for (int v = 0; v < V; ++v) sum += acc[v];
+      sum = group_sum(ok ? sum : T(0), lpr);
+      if (ok && sub == 0) a.out[r * a.n_out + o] = sum;
+    } else {
+      if (ok) store_vec<T, V>(a.out + (r * a.n_out + o) * a.C + c, acc);
+    }
+  };
+  T acc[V];
+#pragma unroll
+  for (int v = 0; v < V; ++v) acc[v] = T(0);
+  int cur = 0;      // outputs before `cur` are written; rows without coefficients are written as zeros
+  for (int t0 = 0; t0 < a.nnz; t0 += U) {
+    T xa[U][V], xb[U][V], xw[U][V], cf[U];
+    int oi[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const int t = min(t0 + k, a.nnz - 1);
+      const uint32_t u = __builtin_amdgcn_readfirstlane(s_idx[t]);
+      oi[k] = __builtin_amdgcn_readfirstlane(s_out[t]);
+      cf[k] = s_coef[t];
+      light_fetch<T, V>(ops[0], u & 1023u, xa[k]);
+      light_fetch<T, V>(ops[1], (u >> 10) & 1023u, xb[k]);
+      light_fetch<T, V>(ops[2], u >> 20, xw[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      if (t0 + k < a.nnz) {
+        while (cur < oi[k]) {
+          emit(cur, acc);
+#pragma unroll
+          for (int v = 0; v < V; ++v) acc[v] = T(0);
+          ++cur;
+        }
+#pragma unroll
+        for (int v = 0; v < V; ++v) acc[v] += cf[k] * xa[k][v] * xb[k][v] * xw[k][v];
+      }
+    }
+  }
+  while (cur < a.n_out) {
+    emit(cur, acc);
+#pragma unroll
+    for (int v = 0; v < V; ++v) acc[v] = T(0);
+    ++cur;
+  }
+}
+
 // out[n, m, c] = sum_{t in [seg[m], seg[m+1])} scale[t] * in[n, index[t], c].  One wavefront per (n, m, chunk of
 // 64 * V channels): wide rows are spread over several wavefronts, and the terms of a segment are fetched four at
 // a time (indices and scales first, then the four rows; the last one to three singly) and added in position
@@ -288,6 +396,57 @@ static OperandDev<T> op_dev(const cgtp_operand& o) {
   return OperandDev<T>{(const T*)o.data, o.rows, o.row_stride, o.idx_stride, o.kind, o.size};
 }
 
+// tri_light_kernel serves a launch when the shapes allow it: V channels per lane (16 bytes) if every per-channel
+// operand and the output keep 16-byte alignment from row to row and index to index, else one; at most 64 lanes per
+// row; table within the default LDS limit.  Returns V, or 0 when the kernel does not apply.
+template <typename T, int V>
+static bool light_aligned(const cgtp_tri_args* a, const void* out) {
+  if (V == 1) return true;
+  if (a->C % V) return false;
+  const cgtp_operand* ops[3] = {&a->a, &a->b, &a->w};
+  for (const cgtp_operand* o : ops)
+    if (o->kind == CGTP_OPERAND_VEC &&
+        ((reinterpret_cast<uintptr_t>(o->data) & (V * sizeof(T) - 1)) || o->row_stride % V || o->idx_stride % V))
+      return false;
+  return (reinterpret_cast<uintptr_t>(out) & (V * sizeof(T) - 1)) == 0;
+}
+
+template <typename T>
+static int light_width(const cgtp_tri_args* a) {
+  constexpr int VW = 16 / sizeof(T);
+  if (a->n_out == 0 || a->n_rows == 0) return 0;
+  if ((int64_t)a->nnz * (sizeof(T) + 8) > 48 * 1024) return 0;
+  // rows summed afterwards go through the workspace (allocated 256-byte aligned by the caller's allocator; checked)
+  const void* out = a->reduce_rows ? a->workspace : a->out;
+  if (light_aligned<T, VW>(a, out) && a->C / VW <= kWave) return VW;
+  return a->C <= kWave ? 1 : 0;
+}
+
+template <typename T, int V>
+static int tri_light_launch_v(const cgtp_tri_args* a, const TriDev<T>& d, hipStream_t stream) {
+  const int lanes = (a->C + V - 1) / V;
+  int lpr_log2 = 0;
+  while ((1 << lpr_log2) < lanes) ++lpr_log2;
+  const int64_t lds = (int64_t)a->nnz * (sizeof(T) + 8);
+  const int64_t rows_per_block = (int64_t)4 * (kWave >> lpr_log2);
+  const int64_t blocks = (a->n_rows + rows_per_block - 1) / rows_per_block;
+  if (blocks > 0x7fffffff) return CGTP_ERR_SHAPE;
+  auto kern = a->reduce_c ? tri_light_kernel<T, V, true> : tri_light_kernel<T, V, false>;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), (size_t)lds, stream, d, lpr_log2);
+  return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
+}
+
+// Sum over rows of per-row results in the workspace: chunks of kSumRows rows, then the chunks, both in a fixed order.
+template <typename T>
+static int tri_sum_rows(const cgtp_tri_args* a, int64_t per_row, hipStream_t stream) {
+  const int64_t chunks = (a->n_rows + kSumRows - 1) / kSumRows;
+  T* part = (T*)a->workspace + a->n_rows * per_row;
+  hipLaunchKernelGGL(rows_sum_kernel<T>, dim3((unsigned)((per_row + 255) / 256), (unsigned)chunks), dim3(256), 0,
+                     stream, (const T*)a->workspace, part, a->n_rows, per_row);
+  launch_partial_sum<T>((const T*)part, (T*)a->out, chunks, per_row, stream);
+  return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
+}
+
 template <typename T>
 static int tri_launch(const cgtp_tri_args* a, int64_t lds, int64_t n_waves, hipStream_t stream) {
   const int64_t per_row = (int64_t)a->n_out * (a->reduce_c ? 1 : a->C);
@@ -313,16 +472,13 @@ static int tri_launch(const cgtp_tri_args* a, int64_t lds, int64_t n_waves, hipS
     const int64_t nw = a->n_rows < 16384 ? a->n_rows : 16384;
     hipLaunchKernelGGL(skern, dim3((unsigned)((nw + 3) / 4)), dim3(256), (size_t)staged_lds, stream, d, nw, (int)region);
     if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
-    if (a->reduce_rows) {
-      const int64_t chunks = (a->n_rows + kSumRows - 1) / kSumRows;
-      T* part = (T*)a->workspace + a->n_rows * per_row;
-      hipLaunchKernelGGL(rows_sum_kernel<T>, dim3((unsigned)((per_row + 255) / 256), (unsigned)chunks), dim3(256), 0,
-                         stream, (const T*)a->workspace, part, a->n_rows, per_row);
-      hipLaunchKernelGGL(partial_sum_kernel<T>, dim3((unsigned)((per_row + 255) / 256)), dim3(256), 0, stream,
-                         (const T*)part, (T*)a->out, chunks, per_row);
-      if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
-    }
-    return CGTP_OK;
+    return a->reduce_rows ? tri_sum_rows<T>(a, per_row, stream) : CGTP_OK;
+  }
+  if (const int v = light_width<T>(a)) {
+    constexpr int VW = 16 / sizeof(T);
+    const int rc = v == 1 ? tri_light_launch_v<T, 1>(a, d, stream) : tri_light_launch_v<T, VW>(a, d, stream);
+    if (rc != CGTP_OK) return rc;
+    return a->reduce_rows ? tri_sum_rows<T>(a, per_row, stream) : CGTP_OK;
   }
   auto kern = a->reduce_c ? tri_kernel<T, true> : tri_kernel<T, false>;
   if (lds > 48 * 1024) {
@@ -332,8 +488,7 @@ static int tri_launch(const cgtp_tri_args* a, int64_t lds, int64_t n_waves, hipS
   hipLaunchKernelGGL(kern, dim3((unsigned)((n_waves + 3) / 4)), dim3(256), (size_t)lds, stream, d, n_waves);
   if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
   if (a->reduce_rows) {
-    hipLaunchKernelGGL(partial_sum_kernel<T>, dim3((unsigned)((per_row + 255) / 256)), dim3(256), 0, stream,
-                       (const T*)a->workspace, (T*)a->out, n_waves, per_row);
+    launch_partial_sum<T>((const T*)a->workspace, (T*)a->out, n_waves, per_row, stream);
     if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
   }
   return CGTP_OK;
@@ -395,7 +550,12 @@ int64_t cgtp_tri_workspace_bytes(const cgtp_tri_args* a) {
   if (!a || !a->reduce_rows) return 0;
   const int64_t per_row = (int64_t)a->n_out * (a->reduce_c ? 1 : a->C);
   int64_t region = 0;
-  if (tri_staged_lds(a, tri_table_bytes(a), &region) > 0)  // per-row results + first-pass partials
+  // per-row results + first-pass partials when the staged or the light kernel serves the launch (the light kernel's
+  // choice of vector width does not change the size; judge it with a workspace that is aligned)
+  cgtp_tri_args probe = *a;
+  probe.workspace = nullptr;
+  const bool light = a->dtype == CGTP_F32 ? light_width<float>(&probe) > 0 : light_width<double>(&probe) > 0;
+  if (tri_staged_lds(a, tri_table_bytes(a), &region) > 0 || light)
     return (a->n_rows + (a->n_rows + kSumRows - 1) / kSumRows) * per_row * elem_size(a->dtype);
   const int64_t nw = a->n_rows < 1024 ? a->n_rows : 1024;
   return nw * per_row * elem_size(a->dtype);

@@ -684,8 +684,7 @@ static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward,
       hipLaunchKernelGGL(rows_sum_kernel<float>, dim3((unsigned)((w_elems + 255) / 256), (unsigned)chunks), dim3(256), 0, stream,
                          (const float*)d.wsw, part, a->n_rows, w_elems);
       if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
-      hipLaunchKernelGGL(partial_sum_kernel<float>, dim3((unsigned)((w_elems + 255) / 256)), dim3(256), 0, stream,
-                         (const float*)part, (float*)a->grad_w, chunks, w_elems);
+      launch_partial_sum<float>((const float*)part, (float*)a->grad_w, chunks, w_elems, stream);
     }
   } else {
     const int chunk = 1 << plan.lpe_log2;
@@ -734,8 +733,7 @@ static int launch_bwd(const cgtp_uvu_args* a, const UvuPlan& plan, hipStream_t s
                        plan.n_waves);
     if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
     if (wred) {
-      hipLaunchKernelGGL(partial_sum_kernel<T>, dim3((unsigned)((w_elems + 255) / 256)), dim3(256), 0, stream,
-                         (const T*)d.wsw, (T*)a->grad_w, plan.n_waves, w_elems);
+      launch_partial_sum<T>((const T*)d.wsw, (T*)a->grad_w, plan.n_waves, w_elems, stream);
       if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
     }
   }
