@@ -29,8 +29,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 # HBM bytes per launch of the dominant kernels on the edge workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # scaled by the same counters on the 1 GiB copy kernel (profiles/uvu_seg_sh2_edge_fwd_bwd.md): KiB per dispatch.
 MEASURED_TRAFFIC_KIB = {
-    "edge_fwd_bwd": 158572.3 * 2.0 + 193595.3 * 1.0,  # uvu_seg_bwd_kernel<TP_sh2,float,4,1>
-    "edge_fwd": 147109.1 * 2.0 + 9216.0 * 1.0,        # uvu_seg_fwd_kernel<TP_sh2,float,4>
+    "edge_fwd_bwd": 153878.6 * 2.0 + 193584.8 * 1.0,  # uvu_seg_bwd_kernel<TP_sh2,float,4,1>
+    "edge_fwd": 146857.7 * 2.0 + 9216.0 * 1.0,        # uvu_seg_fwd_kernel<TP_sh2,float,4>
 }
 
 WORKLOADS = {
