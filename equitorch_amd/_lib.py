@@ -104,6 +104,16 @@ def _load():
                                     C.c_void_p]
     lib.cgtp_sh_backward.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_double,
                                      C.c_int, C.c_void_p]
+    _seg = C.POINTER(C.c_int32)
+    lib.cgtp_layer_rms_supported.argtypes = [_seg, C.c_int, C.c_int, C.c_int]
+    lib.cgtp_layer_rms_workspace_bytes.argtypes = [C.c_int64, C.c_int, C.c_int, C.c_int]
+    lib.cgtp_layer_rms_workspace_bytes.restype = C.c_int64
+    _rd = C.POINTER(C.c_float)
+    lib.cgtp_layer_rms_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, _seg, _rd, C.c_int,
+                                           C.c_int64, C.c_int, C.c_int, C.c_int, C.c_double, C.c_int, C.c_void_p]
+    lib.cgtp_layer_rms_backward.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                            C.c_void_p, _seg, _rd, C.c_int, C.c_int64, C.c_int, C.c_int, C.c_int,
+                                            C.c_int, C.c_void_p]
     lib.cgtp_membench_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
     lib.cgtp_membench_read.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
     return lib

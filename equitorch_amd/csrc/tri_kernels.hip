@@ -451,7 +451,7 @@ template <typename T>
 static int tri_launch(const cgtp_tri_args* a, int64_t lds, int64_t n_waves, hipStream_t stream) {
   const int64_t per_row = (int64_t)a->n_out * (a->reduce_c ? 1 : a->C);
   if (n_waves == 0) {
-    if (a->reduce_rows && per_row > 0) (void)hipMemsetAsync(a->out, 0, sizeof(T) * per_row, stream);
+    if (a->reduce_rows && per_row > 0) launch_partial_sum<T>(nullptr, (T*)a->out, 0, per_row, stream);  // writes 0
     return CGTP_OK;
   }
   TriDev<T> d;

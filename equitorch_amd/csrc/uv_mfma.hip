@@ -566,8 +566,11 @@ int cgtp_uv_grad_w(int cfg, const void* x, const void* y, const void* g, void* g
   const UvEntry& e = t[cfg];
   const int64_t n_out = (int64_t)e.p * cin * cout;
   hipStream_t st = (hipStream_t)stream;
-  if (n_rows == 0) {
-    return hipMemsetAsync(gw, 0, n_out * 2, st) == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
+  if (n_rows == 0) {  // no samples: the gradient is zero (the summation kernel over zero chunks writes it; a fill
+                      // kernel rather than a memset, so that the call can be captured into a graph)
+    hipLaunchKernelGGL(uv_gw_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, st,
+                       (const float*)nullptr, (__bf16*)gw, (int64_t)0, n_out);
+    return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
   }
   if (!workspace) return CGTP_ERR_WORKSPACE;
   const int64_t lds = (int64_t)e.gw_max_rows * kGwStep * ((int64_t)cin * 2 + cout * 2 + 2 * kGwPad);

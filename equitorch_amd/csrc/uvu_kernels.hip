@@ -669,7 +669,7 @@ static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward,
   const bool wred = backward && a->w_shared && a->grad_w;
   const int64_t w_elems = (int64_t)e.dims[3] * a->C;
   if (plan.n_waves == 0) {
-    if (wred) (void)hipMemsetAsync(a->grad_w, 0, sizeof(float) * w_elems, stream);
+    if (wred) launch_partial_sum<float>(nullptr, (float*)a->grad_w, 0, w_elems, stream);   // zero partials: writes 0
     return CGTP_OK;
   }
   UvuDev<float> d = to_dev<float>(a, plan);
@@ -725,7 +725,7 @@ static int launch_bwd(const cgtp_uvu_args* a, const UvuPlan& plan, hipStream_t s
   const bool wred = a->w_shared && a->grad_w;
   const int64_t w_elems = (int64_t)e.dims[3] * a->C;
   if (plan.n_waves == 0) {
-    if (wred) (void)hipMemsetAsync(a->grad_w, 0, sizeof(T) * w_elems, stream);
+    if (wred) launch_partial_sum<T>(nullptr, (T*)a->grad_w, 0, w_elems, stream);   // zero partials: writes 0
   } else {
     const int gwm = !a->grad_w ? kGwNone : (wred ? kGwReduce : kGwStore);
     hipLaunchKernelGGL(seg ? (a->y_vec ? e.seg_bwd_vec[vi][gwm] : e.seg_bwd[vi][gwm]) : e.bwd[vi][gwm],

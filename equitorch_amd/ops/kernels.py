@@ -110,6 +110,63 @@ def segment_sum(inp: Tensor, scale: Optional[Tensor], index: Optional[Tensor], s
     return out
 
 
+# ---- fused layer RMS normalisation ------------------------------------------------------------------------------
+def _seg_array(irrep_seg: Tensor):
+    """Host int32 array of the irrep boundaries (cached on the table tensor)."""
+    def build():
+        vals = [int(v) for v in irrep_seg.detach().cpu().tolist()]
+        return (C.c_int32 * len(vals))(*vals), len(vals) - 1
+    return cached(irrep_seg, "layer_rms_seg", build)
+
+
+def _rdims_array(rdims: Tensor):
+    """Host float array of the table's ``1 / dim`` factors (fp32, as the reference stores them)."""
+    def build():
+        vals = rdims.detach().to(torch.float32).cpu().tolist()
+        return (C.c_float * len(vals))(*vals)
+    return cached(rdims, "layer_rms_rdims", build)
+
+
+def layer_rms_supported(irrep_seg: Tensor, channels: int, dtype: torch.dtype) -> bool:
+    if dtype not in (torch.float32, torch.float64):
+        return False
+    arr, k = _seg_array(irrep_seg)
+    return bool(_lib.lib.cgtp_layer_rms_supported(arr, k, channels, _lib.dtype_code(dtype)))
+
+
+def layer_rms_forward(x: Tensor, weight: Optional[Tensor], irrep_seg: Tensor, rdims: Tensor, scaled: bool, eps: float,
+                      want_rsigma: bool):
+    """``(out, rsigma | None)`` of ``cgtp_layer_rms_forward``; ``x`` is ``(N, D, C)`` contiguous."""
+    arr, k = _seg_array(irrep_seg)
+    n, d, ch = x.shape
+    out = torch.empty_like(x)
+    rsigma = torch.empty((n, k), dtype=x.dtype, device=x.device) if want_rsigma else None
+    _lib.check(_lib.lib.cgtp_layer_rms_forward(x.data_ptr(), _lib.ptr(weight), out.data_ptr(), _lib.ptr(rsigma), arr,
+                                               _rdims_array(rdims), k, n, d, ch, int(scaled), float(eps),
+                                               _lib.dtype_code(x.dtype),
+                                               _lib.stream_ptr(x.device)), "cgtp_layer_rms_forward")
+    return out, rsigma
+
+
+def layer_rms_backward(x: Tensor, weight: Optional[Tensor], rsigma: Tensor, grad_out: Tensor, irrep_seg: Tensor,
+                       rdims: Tensor, scaled: bool, need_x: bool, need_w: bool):
+    """``(grad_x | None, grad_weight | None)`` of ``cgtp_layer_rms_backward``."""
+    arr, k = _seg_array(irrep_seg)
+    n, d, ch = x.shape
+    gx = torch.empty_like(x) if need_x else None
+    gw = ws = None
+    if need_w:
+        gw = torch.empty((k, ch), dtype=x.dtype, device=x.device)
+        nbytes = int(_lib.lib.cgtp_layer_rms_workspace_bytes(n, k, ch, _lib.dtype_code(x.dtype)))
+        ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+    _lib.check(_lib.lib.cgtp_layer_rms_backward(x.data_ptr(), _lib.ptr(weight), rsigma.data_ptr(), grad_out.data_ptr(),
+                                                _lib.ptr(gx), _lib.ptr(gw), _lib.ptr(ws), arr, _rdims_array(rdims), k,
+                                                n, d, ch, int(scaled), _lib.dtype_code(x.dtype),
+                                                _lib.stream_ptr(x.device)),
+               "cgtp_layer_rms_backward")
+    return gx, gw
+
+
 # ---- specialised uvu ----------------------------------------------------------------------------------------
 class SegIndex:
     """Per-sorted-position index arrays of the segment mode (all int64, same device)."""

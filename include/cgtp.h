@@ -266,6 +266,31 @@ int cgtp_sh_forward(const void* xyz, void* out, int64_t n, int lmax, int normali
 int cgtp_sh_backward(const void* xyz, const void* grad_out, void* grad_xyz, int64_t n, int lmax, int normalize,
                      double scale, int dtype, void* stream);
 
+/* ---- layer RMS normalisation of equivariant features ------------------------------------------------------
+ * Stands in for layer_rms_norm (equitorch/nn/functional/normalization.py:111-157: channel_mean_squared_norm,
+ * rsqrt, sparse_vecsca with the per-sample factors and sparse_mul with the weight; four launches and their
+ * autograd backward) with one launch per direction:
+ *   ms[n,k] = sum_{M in irrep k, c} x[n,M,c]^2 / (C * (scaled ? dim_k : 1)),  r = rsqrt(ms + eps),
+ *   out[n,M,c] = x[n,M,c] * r[n,k(M)] * weight[k(M),c]          (weight NULL = no scaling)
+ * x, out, grad_out, grad_x: (n_rows, D, C) contiguous; weight, grad_weight: (n_irreps, C); rsigma: (n_rows,
+ * n_irreps), written by the forward (NULL = not wanted) and read by the backward.  irrep_seg: HOST array of
+ * n_irreps + 1 block boundaries, irrep_seg[0] = 0, irrep_seg[n_irreps] = D (IrrepsInfo.irrep_seg); irrep_rdims:
+ * HOST array of the n_irreps factors 1 / dim_k as the table holds them (IrrepsInfo.rdims, fp32; NULL = computed
+ * here), read when scaled != 0; blocks of at most 13 components (l <= 6), at most 64 irreps, C <= 64 or C/4 (fp32) resp. C/2 (fp64) <= 64 with 16-byte
+ * aligned pointers: cgtp_layer_rms_supported tells.  grad_x and grad_weight may each be NULL; grad_weight needs a
+ * workspace of cgtp_layer_rms_workspace_bytes (per-row terms, summed over rows in a fixed order).
+ * dtype: CGTP_F32 | CGTP_F64.
+ */
+int cgtp_layer_rms_supported(const int32_t* irrep_seg, int n_irreps, int C, int dtype);
+int64_t cgtp_layer_rms_workspace_bytes(int64_t n_rows, int n_irreps, int C, int dtype);
+int cgtp_layer_rms_forward(const void* x, const void* weight, void* out, void* rsigma, const int32_t* irrep_seg,
+                           const float* irrep_rdims, int n_irreps, int64_t n_rows, int D, int C, int scaled,
+                           double eps, int dtype, void* stream);
+int cgtp_layer_rms_backward(const void* x, const void* weight, const void* rsigma, const void* grad_out,
+                            void* grad_x, void* grad_weight, void* workspace, const int32_t* irrep_seg,
+                            const float* irrep_rdims, int n_irreps, int64_t n_rows, int D, int C, int scaled,
+                            int dtype, void* stream);
+
 /* ---- streaming kernels of known traffic (counter calibration, achievable-bandwidth reference) ------------
  * No counterpart in the reference.  copy: reads n_bytes and writes n_bytes; read: reads n_bytes.
  * n_bytes must be a multiple of 16 and the pointers 16-byte aligned.

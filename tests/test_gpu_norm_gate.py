@@ -185,3 +185,71 @@ def test_xyz_to_sincos_module(device):
             ref = torch.stack([torch.ones_like(ang)] + [f(m * ang) * scale for m in (1, 2, 3)
                                                         for f in (torch.sin, torch.cos)], dim=-1)
             assert_close(got, ref, tol=1e-10, what=f"sincos normalised={normalised}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("channels", [64, 24, 10, 256])
+@pytest.mark.parametrize("scaled", [True, False])
+def test_layer_rms_fused_kernels(device, dtype, channels, scaled):
+    """``cgtp_layer_rms_forward`` / ``cgtp_layer_rms_backward`` against the oracle: 16-byte lanes (64, 24, 256
+    channels; 256 needs them in fp32 and is too wide in fp64, where the composed path takes over), one element per
+    lane (10), irreps up to l = 6, rows not a multiple of the rows per wavefront, gradients of x and of the weight."""
+    from equitorch_amd.nn.functional import layer_rms_norm
+    from equitorch_amd.utils import irreps_info
+    irr = "0e+1o+2e+6e+1o"
+    info = ref_tables.irreps_info(irr)
+    for k in ("rdims", "rsqrt_dims"):
+        info[k] = torch.tensor(info[k]).double().tolist()
+    d = 1 + 3 + 5 + 13 + 3
+    g = torch.Generator().manual_seed(11)
+    n = 131
+    x = torch.randn(n, d, channels, generator=g, dtype=torch.float64).to(dtype).double()
+    w = (1 + 0.3 * torch.randn(5, channels, generator=g, dtype=torch.float64)).to(dtype).double()
+    ct = torch.randn(n, d, channels, generator=g, dtype=torch.float64).to(dtype).double()
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    ref = ref_ops.cpu_layer_rms_norm(xr, info, wr, scaled=scaled, eps=1e-5)
+    rgx, rgw = torch.autograd.grad(ref, (xr, wr), ct)
+    dev_info = irreps_info(irr).to(device)
+    xd, wd = x.to(device, dtype).requires_grad_(True), w.to(device, dtype).requires_grad_(True)
+    out = layer_rms_norm(xd, dev_info, wd, scaled=scaled, eps=1e-5)
+    gx, gw = torch.autograd.grad(out, (xd, wd), ct.to(device, dtype))
+    tol = 1e-5 if dtype == torch.float32 else 1e-11
+    assert_close(out, ref, tol=tol, what="out")
+    assert_close(gx, rgx, tol=tol * 10, what="grad x")
+    # the weight gradient sums 131 x dim terms of either sign: judged against the sum of their magnitudes
+    assert_close(gw, rgw, tol=tol * 10, what="grad weight")
+    # no weight, only the input's gradient
+    out0 = layer_rms_norm(xd, dev_info, None, scaled=scaled, eps=1e-5)
+    ref0 = ref_ops.cpu_layer_rms_norm(xr, info, None, scaled=scaled, eps=1e-5)
+    assert_close(out0, ref0, tol=tol, what="out without weight")
+    (g0,) = torch.autograd.grad(out0, xd, ct.to(device, dtype))
+    (r0,) = torch.autograd.grad(ref0, xr, ct)
+    assert_close(g0, r0, tol=tol * 10, what="grad x without weight")
+
+
+def test_layer_rms_second_order_and_fallback(device):
+    """Gradients of gradients go through the composed, differentiable path and agree with the oracle's; an irrep of
+    degree 7 (15 components) is outside the fused kernel and runs composed."""
+    from equitorch_amd.nn.functional import layer_rms_norm
+    from equitorch_amd.ops import kernels
+    from equitorch_amd.utils import irreps_info
+    info = _info()
+    x, g = _data(9, 8, torch.float64, seed=12)
+    w = 1 + 0.3 * torch.randn(4, 8, generator=g, dtype=torch.float64)
+    ct = torch.randn(9, 12, 8, generator=g, dtype=torch.float64)
+    v = torch.randn(9, 12, 8, generator=g, dtype=torch.float64)
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    (rg,) = torch.autograd.grad(ref_ops.cpu_layer_rms_norm(xr, info, wr), xr, ct, create_graph=True)
+    rgg = torch.autograd.grad(rg, (xr, wr), v)
+    dev_info = irreps_info(IRR).to(device)
+    xd, wd = x.to(device).requires_grad_(True), w.to(device).requires_grad_(True)
+    (gd,) = torch.autograd.grad(layer_rms_norm(xd, dev_info, wd), xd, ct.to(device), create_graph=True)
+    assert_close(gd, rg, tol=1e-10, what="first order under create_graph")
+    gg = torch.autograd.grad(gd, (xd, wd), v.to(device))
+    assert_close(gg[0], rgg[0], tol=1e-9, what="second order x")
+    assert_close(gg[1], rgg[1], tol=1e-9, what="second order weight")
+    big = irreps_info("0e+7o").to(device)
+    assert not kernels.layer_rms_supported(big.irrep_seg, 8, torch.float64)
+    xb = torch.randn(5, 16, 8, generator=g, dtype=torch.float64)
+    ref = ref_ops.cpu_layer_rms_norm(xb, ref_tables.irreps_info("0e+7o"), None)
+    assert_close(layer_rms_norm(xb.to(device), big, None), ref, tol=1e-6, what="composed path")
