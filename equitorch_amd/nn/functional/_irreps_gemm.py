@@ -35,13 +35,18 @@ class Path(NamedTuple):
 
 class Group(NamedTuple):
     """Consecutive paths whose output and input ranges advance together: one batched GEMM over ``rows`` components,
-    component ``j`` using weight ``w_of_row[j]``."""
+    component ``j`` using weight ``w_of_row[j]`` times ``scale_of_row[j]``."""
     o0: int
     i0: int
     rows: int
     w_of_row: Tuple[int, ...]
-    scale: float
+    scale_of_row: Tuple[float, ...]
     accumulate: bool      # an earlier group already wrote these output rows
+
+    @property
+    def scale(self):
+        """The common scale of the rows, or None if they differ."""
+        return self.scale_of_row[0] if len(set(self.scale_of_row)) == 1 else None
 
 
 class LinearPlan(NamedTuple):
@@ -55,12 +60,13 @@ class LinearPlan(NamedTuple):
         for p in self.paths:
             g = out[-1] if out else None
             hit = any(a < p.o0 + p.k and p.o0 < b for a, b in written)
-            if (g is not None and g.scale == p.scale and g.o0 + g.rows == p.o0 and g.i0 + g.rows == p.i0
+            if (g is not None and g.o0 + g.rows == p.o0 and g.i0 + g.rows == p.i0
                     and not g.accumulate and not hit):
-                out[-1] = Group(g.o0, g.i0, g.rows + p.k, g.w_of_row + (p.w,) * p.k, g.scale, False)
+                out[-1] = Group(g.o0, g.i0, g.rows + p.k, g.w_of_row + (p.w,) * p.k,
+                                g.scale_of_row + (p.scale,) * p.k, False)
                 written[-1] = (g.o0, g.o0 + g.rows + p.k)
             else:
-                out.append(Group(p.o0, p.i0, p.k, (p.w,) * p.k, p.scale, hit))
+                out.append(Group(p.o0, p.i0, p.k, (p.w,) * p.k, (p.scale,) * p.k, hit))
                 written.append((p.o0, p.o0 + p.k))
         return tuple(out)
 
@@ -96,6 +102,33 @@ def plan_of_irreps_info(info) -> LinearPlan:
     return cached(info.irrep_seg, "irrep_wise_plan", build)
 
 
+def plan_of_product_info(info, in_size: int, n_weights: int) -> LinearPlan:
+    """Plan of ``out[n, M, :] = sum_t scale_t * x[n, index1_t, :] @ W[index2_t]`` for a ``SparseProductInfo`` (the
+    table of ``sparse_vecmat``; ``SO2Linear('uv')``): one single-component path per entry, ordered so that entries
+    on one diagonal (``M - index1`` fixed, ``M`` rising) follow each other and merge into batched GEMMs."""
+    anchor = next(t for t in (info.seg_out, info.index1, info.index2, info.scale) if t is not None)
+
+    def build():
+        n = next((t.shape[0] for t in (info.index1, info.index2, info.scale) if t is not None), None)
+        if n is None:
+            n = int(info.seg_out[-1]) if info.seg_out is not None else in_size
+        i1 = list(range(n)) if info.index1 is None else info.index1.tolist()
+        i2 = list(range(n)) if info.index2 is None else info.index2.tolist()
+        sc = [1.0] * n if info.scale is None else info.scale.tolist()
+        if info.seg_out is None:
+            out_of, n_out = list(range(n)), n
+        else:
+            seg = info.seg_out.tolist()
+            n_out = len(seg) - 1
+            out_of = [m for m in range(n_out) for _ in range(seg[m], seg[m + 1])]
+        if info.out_size is not None:
+            n_out = max(n_out, int(info.out_size))
+        entries = sorted(zip(out_of, i1, i2, sc), key=lambda e: (e[0] - e[1], e[0]))
+        return LinearPlan(tuple(Path(int(w), int(m), int(m0), 1, float(s)) for m, m0, w, s in entries), int(n_weights),
+                          int(n_out))
+    return cached(anchor, ("product_plan", in_size, n_weights), build)
+
+
 def transposed(plan: LinearPlan, in_size: int) -> LinearPlan:
     return LinearPlan(tuple(Path(p.w, p.i0, p.o0, p.k, p.scale) for p in plan.paths), plan.n_paths, in_size)
 
@@ -125,6 +158,20 @@ def _row_weights(grp: Group, device) -> Tensor:
     return t
 
 
+_ROW_SCALES = {}
+
+
+def _row_scales(grp: Group, like: Tensor) -> Tensor:
+    """``(rows, 1, 1)`` tensor of the rows' scales (only asked for when they differ)."""
+    key = (grp.scale_of_row, str(like.device), like.dtype)
+    t = _ROW_SCALES.get(key)
+    if t is None:
+        if len(_ROW_SCALES) > 256:
+            _ROW_SCALES.clear()
+        t = _ROW_SCALES[key] = torch.tensor(grp.scale_of_row, dtype=like.dtype, device=like.device).view(-1, 1, 1)
+    return t
+
+
 def _covered(plan: LinearPlan) -> bool:
     rows = sorted((p.o0, p.o0 + p.k) for p in plan.paths)
     end = 0
@@ -149,10 +196,13 @@ def _mix_raw(x: Tensor, w: Tensor, plan: LinearPlan, w_t: bool) -> Tensor:
         if shared:
             # one GEMM (N, C_in) @ (C_in, C_out) per component, batched over the components of the group
             wb = w.index_select(0, _row_weights(grp, w.device))
+            alpha = grp.scale
+            if alpha is None:                                          # rows with different scales: fold them in
+                wb, alpha = wb * _row_scales(grp, wb), 1.0
             if w_t:
                 wb = wb.transpose(1, 2)
             ot = os_.transpose(0, 1)                                   # (rows, N, cout), rows strided by D_out * cout
-            torch.baddbmm(ot, xs.transpose(0, 1), wb, beta=beta, alpha=grp.scale, out=ot)
+            torch.baddbmm(ot, xs.transpose(0, 1), wb, beta=beta, alpha=alpha, out=ot)
         else:
             # per sample: (rows of one path, C_in) @ (C_in, C_out); paths of a group share nothing, so go one by one
             at = 0
@@ -160,8 +210,9 @@ def _mix_raw(x: Tensor, w: Tensor, plan: LinearPlan, w_t: bool) -> Tensor:
                 pw = grp.w_of_row[at]
                 k = next((j for j in range(at, grp.rows) if grp.w_of_row[j] != pw), grp.rows) - at
                 wp = w[:, pw].transpose(1, 2) if w_t else w[:, pw]
+                k = next((j for j in range(at, at + k) if grp.scale_of_row[j] != grp.scale_of_row[at]), at + k) - at
                 dst = os_[:, at:at + k, :]
-                torch.baddbmm(dst, xs[:, at:at + k, :], wp, beta=beta, alpha=grp.scale, out=dst)
+                torch.baddbmm(dst, xs[:, at:at + k, :], wp, beta=beta, alpha=grp.scale_of_row[at], out=dst)
                 at += k
     return out
 
@@ -176,13 +227,17 @@ def _outer_raw(x: Tensor, g: Tensor, plan: LinearPlan, shared: bool) -> Tensor:
             for grp in _groups(plan):
                 a = x[:, grp.i0:grp.i0 + grp.rows, :].permute(1, 2, 0)          # (rows, cin, N)
                 b = g[:, grp.o0:grp.o0 + grp.rows, :].transpose(0, 1)           # (rows, N, cout)
-                gw.index_add_(0, _row_weights(grp, x.device), torch.bmm(a, b), alpha=grp.scale)
+                prod = torch.bmm(a, b)
+                if grp.scale is None:
+                    gw.index_add_(0, _row_weights(grp, x.device), prod * _row_scales(grp, prod))
+                else:
+                    gw.index_add_(0, _row_weights(grp, x.device), prod, alpha=grp.scale)
         return gw
     gw = torch.zeros((n, plan.n_paths, cin, cout), dtype=x.dtype, device=x.device)
     if n:
-        for p in plan.paths:
+        for p in plan.paths:      # gw starts at zero and a weight may serve several paths: accumulate
             dst = gw[:, p.w]
-            torch.baddbmm(dst, x[:, p.i0:p.i0 + p.k, :].transpose(1, 2), g[:, p.o0:p.o0 + p.k, :], beta=0.0,
+            torch.baddbmm(dst, x[:, p.i0:p.i0 + p.k, :].transpose(1, 2), g[:, p.o0:p.o0 + p.k, :], beta=1.0,
                           alpha=p.scale, out=dst)
     return gw
 

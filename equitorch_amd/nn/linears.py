@@ -11,6 +11,7 @@ import torch.nn as nn
 from torch import Tensor
 from torch.nn import Parameter
 
+from .._lib import require_gpu as _lib_require
 from ..irreps import check_irreps
 from ..structs import IrrepsInfo, IrrepsLinearInfo, TensorProductInfo
 from ..utils._structs import irreps_info, irreps_linear_infos, so2_linear_infos, tp_infos
@@ -269,8 +270,20 @@ class SO2Linear(nn.Module):
             assert weight is not None, 'Please pass the weight when self.internal_weights is False.'
             if self.weight_numel is not None:
                 weight = _view_weight(weight, self.weight_shape, self.weight_numel)
-        op = sparse_mul if self.feature_mode == 'uu' else sparse_vecmat
-        return op(input, weight, self.info_forward, self.info_backward1, self.info_backward2)
+        if self.feature_mode == 'uu':
+            return sparse_mul(input, weight, self.info_forward, self.info_backward1, self.info_backward2)
+        if (input.is_floating_point() and input.dtype == weight.dtype and weight.ndim in (3, 4)
+                and weight.shape[-3] == self.num_weights and input.ndim >= 3):
+            if weight.ndim == 3:
+                # one GEMM per order |m| over the components of that order side by side
+                from .functional._so2_gemm import so2_linear_uv_shared
+                _lib_require(input, weight)
+                return so2_linear_uv_shared(input, weight, self.info_forward, self.irreps_in.dim, self.num_weights)
+            # per-sample weights: every table entry is a (C_in, C_out) GEMM on one component, batched over samples
+            from .functional import _irreps_gemm as G
+            plan = G.plan_of_product_info(self.info_forward, self.irreps_in.dim, self.num_weights)
+            return G.mix(input, weight, plan, self.irreps_in.dim)
+        return sparse_vecmat(input, weight, self.info_forward, self.info_backward1, self.info_backward2)
 
     def _apply(self, *args, **kwargs):
         lin = super()._apply(*args, **kwargs)
