@@ -350,6 +350,8 @@ static int64_t tri_table_bytes(const cgtp_tri_args* a) {
 
 // LDS bytes of the staged kernel (table + four operand regions) and elements per region, or 0 if the operands'
 // extents are unknown, the regions do not fit, or staging would not pay.
+constexpr int64_t kLightReuse = 8;
+
 static int64_t tri_staged_lds(const cgtp_tri_args* a, int64_t table_bytes, int64_t* region_elems) {
   const cgtp_operand* ops[3] = {&a->a, &a->b, &a->w};
   int64_t region = 0, vec_rows = 0;
@@ -358,9 +360,10 @@ static int64_t tri_staged_lds(const cgtp_tri_args* a, int64_t table_bytes, int64
     region += o->kind == CGTP_OPERAND_VEC ? (int64_t)o->size * kWave : (o->kind == CGTP_OPERAND_SCALAR ? o->size : 1);
     if (o->kind == CGTP_OPERAND_VEC) vec_rows += o->size;
   }
-  // staging pays when operand rows are read more than once; with about one coefficient per staged row (the
-  // second stage of the reference's two-launch products) the direct kernel is faster
-  if (a->nnz <= vec_rows) return 0;
+  // staging pays when operand rows are read many times; with up to kLightReuse coefficients per staged row
+  // (gates, block sums, rotations, SO(2) maps, the second stage of the reference's two-launch products) reading the
+  // operands through the caches is faster
+  if (a->nnz <= kLightReuse * vec_rows) return 0;
   region = (region + 3) / 4 * 4;
   const int64_t lds = (table_bytes + 15) / 16 * 16 + 4 * region * elem_size(a->dtype);
   if (lds > kLdsBytes) return 0;
