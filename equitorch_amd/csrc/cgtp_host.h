@@ -49,17 +49,42 @@ inline void launch_partial_sum(const T* ws, T* out, int64_t n_part, int64_t n, h
 }
 
 // First pass of a sum over many rows: part[c * n + i] = sum of rows[r * n + i] over the rows r of chunk c
-// (kSumRows rows), in row order; partial_sum_kernel then adds the chunks.  Fixed order, no atomics.
-constexpr int kSumRows = 256;
+// (kSumRows rows); partial_sum_kernel then adds the chunks.  Fixed order, no atomics: four threads per column take
+// every fourth row of the chunk each, four loads in flight, and their sums are added in thread order.
+constexpr int kSumRows = 64;
+constexpr int kSumSlices = 4, kSumCols = 64;
 template <typename T>
-__global__ void __launch_bounds__(256) rows_sum_kernel(const T* __restrict__ rows, T* __restrict__ part, int64_t n_rows,
-                                                       int64_t n) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
+__global__ void __launch_bounds__(kSumSlices * kSumCols) rows_sum_kernel(const T* __restrict__ rows, T* __restrict__ part,
+                                                                         int64_t n_rows, int64_t n) {
+  __shared__ T acc[kSumSlices][kSumCols];
+  const int col = threadIdx.x % kSumCols, slice = threadIdx.x / kSumCols;
+  const int64_t i = (int64_t)blockIdx.x * kSumCols + col;
   const int64_t r0 = (int64_t)blockIdx.y * kSumRows, r1 = r0 + kSumRows < n_rows ? r0 + kSumRows : n_rows;
   T s = T(0);
-  for (int64_t r = r0; r < r1; ++r) s += rows[r * n + i];
-  part[blockIdx.y * n + i] = s;
+  if (i < n) {
+    int64_t r = r0 + slice;
+    for (; r + 3 * kSumSlices < r1; r += 4 * kSumSlices) {
+      const T a = rows[r * n + i], b = rows[(r + kSumSlices) * n + i], c = rows[(r + 2 * kSumSlices) * n + i],
+              d = rows[(r + 3 * kSumSlices) * n + i];
+      s += a; s += b; s += c; s += d;
+    }
+    for (; r < r1; r += kSumSlices) s += rows[r * n + i];
+  }
+  acc[slice][col] = s;
+  __syncthreads();
+  if (slice == 0 && i < n) {
+    T total = acc[0][col];
+#pragma unroll
+    for (int j = 1; j < kSumSlices; ++j) total += acc[j][col];
+    part[blockIdx.y * n + i] = total;
+  }
+}
+
+template <typename T>
+inline void launch_rows_sum(const T* rows, T* part, int64_t n_rows, int64_t n, hipStream_t stream) {
+  const int64_t chunks = (n_rows + kSumRows - 1) / kSumRows;
+  hipLaunchKernelGGL(rows_sum_kernel<T>, dim3((unsigned)((n + kSumCols - 1) / kSumCols), (unsigned)chunks),
+                     dim3(kSumSlices * kSumCols), 0, stream, rows, part, n_rows, n);
 }
 
 }  // namespace cgtp

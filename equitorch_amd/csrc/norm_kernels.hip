@@ -227,8 +227,7 @@ int bwd_launch(const void* x, const void* weight, const void* rsigma, const void
     const int64_t per_row = (int64_t)seg.n_irreps * C;
     const int64_t chunks = (n_rows + kSumRows - 1) / kSumRows;
     T* part = (T*)workspace + n_rows * per_row;
-    hipLaunchKernelGGL(rows_sum_kernel<T>, dim3((unsigned)((per_row + 255) / 256), (unsigned)chunks), dim3(256), 0,
-                       stream, (const T*)workspace, part, n_rows, per_row);
+    launch_rows_sum<T>((const T*)workspace, part, n_rows, per_row, stream);
     launch_partial_sum<T>((const T*)part, (T*)gweight, chunks, per_row, stream);
     if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
   }

@@ -444,8 +444,7 @@ template <typename T>
 static int tri_sum_rows(const cgtp_tri_args* a, int64_t per_row, hipStream_t stream) {
   const int64_t chunks = (a->n_rows + kSumRows - 1) / kSumRows;
   T* part = (T*)a->workspace + a->n_rows * per_row;
-  hipLaunchKernelGGL(rows_sum_kernel<T>, dim3((unsigned)((per_row + 255) / 256), (unsigned)chunks), dim3(256), 0,
-                     stream, (const T*)a->workspace, part, a->n_rows, per_row);
+  launch_rows_sum<T>((const T*)a->workspace, part, a->n_rows, per_row, stream);
   launch_partial_sum<T>((const T*)part, (T*)a->out, chunks, per_row, stream);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }

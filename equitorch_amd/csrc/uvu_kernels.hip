@@ -681,8 +681,7 @@ static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward,
       if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
       const int64_t chunks = (a->n_rows + kSumRows - 1) / kSumRows;
       float* part = d.wsw + a->n_rows * w_elems;
-      hipLaunchKernelGGL(rows_sum_kernel<float>, dim3((unsigned)((w_elems + 255) / 256), (unsigned)chunks), dim3(256), 0, stream,
-                         (const float*)d.wsw, part, a->n_rows, w_elems);
+      launch_rows_sum<float>((const float*)d.wsw, part, a->n_rows, w_elems, stream);
       if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
       launch_partial_sum<float>((const float*)part, (float*)a->grad_w, chunks, w_elems, stream);
     }

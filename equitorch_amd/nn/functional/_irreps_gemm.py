@@ -217,6 +217,20 @@ def _mix_raw(x: Tensor, w: Tensor, plan: LinearPlan, w_t: bool) -> Tensor:
     return out
 
 
+def _long_k_bmm(a: Tensor, b: Tensor) -> Tensor:
+    """``bmm(a (B, m, K), b (B, K, n))`` for small ``m x n`` and long ``K`` (a sum over samples): the library runs one
+    workgroup per output tile down the whole of ``K``, so the sum is cut into ``S`` slices that run as a larger batch
+    and are added afterwards."""
+    k = a.shape[-1]
+    s = 1
+    while s < 64 and k % (2 * s) == 0 and k // (2 * s) >= 512:
+        s *= 2
+    if s == 1:
+        return torch.bmm(a, b)
+    parts = torch.matmul(a.unflatten(2, (s, k // s)).permute(0, 2, 1, 3), b.unflatten(1, (s, k // s)))
+    return parts.sum(dim=1)
+
+
 def _outer_raw(x: Tensor, g: Tensor, plan: LinearPlan, shared: bool) -> Tensor:
     """``gw[(n,) p] = scale * sum_j x[n, i0+j, :]^T (x) g[n, o0+j, :]`` (summed over ``n`` when ``shared``)."""
     n, _, cin = x.shape
@@ -227,7 +241,7 @@ def _outer_raw(x: Tensor, g: Tensor, plan: LinearPlan, shared: bool) -> Tensor:
             for grp in _groups(plan):
                 a = x[:, grp.i0:grp.i0 + grp.rows, :].permute(1, 2, 0)          # (rows, cin, N)
                 b = g[:, grp.o0:grp.o0 + grp.rows, :].transpose(0, 1)           # (rows, N, cout)
-                prod = torch.bmm(a, b)
+                prod = _long_k_bmm(a, b)
                 if grp.scale is None:
                     gw.index_add_(0, _row_weights(grp, x.device), prod * _row_scales(grp, prod))
                 else:
