@@ -51,6 +51,8 @@ WORKLOADS = {
     "sh": None,
     # IrrepsLinear 128 -> 128 channels on 32768 x (0e+1o+2e+3o), bf16, shared weight, forward + backward
     "irreps_linear": None,
+    # element-wise and SO(2) modules on 65536 rows of 0e+1o+2e, 64 channels, fp32 (table of timings)
+    "modules": None,
     # plain library GEMM (torch.matmul, bf16, 8192^3): the matrix rate the box reaches, next to the vendor peak
     "gemm": None,
 }
@@ -191,6 +193,70 @@ def irreps_linear_bench(steps, warmup):
                                    "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                    "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": nbytes,
                                    "avg_ms": round(f_ms, 5), "fwd_TFLOPs": round(flops / (f_ms * 1e-3) / 1e12, 1)}}))
+
+
+def modules_bench(steps, warmup):
+    """Forward and forward + backward times of the element-wise and SO(2) modules on 65536 rows of 0e+1o+2e with 64
+    channels in fp32 (151 MB per feature tensor).  ``value`` is LayerRMSNorm forward + backward; the roofline entry is
+    its forward launch (reads and writes the feature tensor once); the other modules are listed under ``modules``."""
+    import math
+
+    from equitorch_amd import nn as enn
+    from equitorch_amd.nn.functional import sincos
+    dev = torch.device("cuda:0")
+    irr, n, c, d, k = "0e+1o+2e", 65536, 64, 9, 3
+    torch.manual_seed(0)
+    x = torch.randn(n, d, c, device=dev)
+    gates = torch.randn(n, k, c, device=dev)
+    sc = [sincos(torch.rand(n, device=dev) * 2 * math.pi, 2) for _ in range(3)]
+
+    def timed(fn, reps):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps
+
+    def both(mod, *extra):
+        xr = x.clone().requires_grad_(True)
+
+        def fwd():
+            with torch.no_grad():
+                return mod(x, *extra)
+
+        ct = torch.randn_like(fwd())
+
+        def step():
+            return torch.autograd.grad(mod(xr, *extra), xr, ct)
+        return round(timed(fwd, steps), 5), round(timed(step, steps), 5)
+
+    norm = enn.LayerRMSNorm(irr, c).to(dev)
+    table = {
+        "LayerRMSNorm": both(norm),
+        "Gate": both(enn.Gate(irr, activation=None).to(dev), gates),
+        "SquaredNorm": both(enn.SquaredNorm(irr).to(dev)),
+        "TensorDot_uu": both(enn.TensorDot(irr, "uu").to(dev), x),
+        "SO2Linear_uu": both(enn.SO2Linear(irr, irr, c, c, feature_mode="uu").to(dev)),
+        "SO2Linear_uv": both(enn.SO2Linear(irr, irr, c, c, feature_mode="uv").to(dev)),
+        "SparseWignerRotation": both(enn.SparseWignerRotation(irr).to(dev), *sc),
+        "copy": (round(timed(lambda: x.clone(), steps), 5), None),
+    }
+    f_ms, step_ms = table["LayerRMSNorm"]
+    nbytes = 2 * x.numel() * 4 + norm.weight.numel() * 4
+    gbs = nbytes / (f_ms * 1e-3) / 1e9
+    print(json.dumps({"metric": "LayerRMSNorm fwd+bwd Mrows/s (0e+1o+2e, C=64, fp32)", "value": round(n / (step_ms * 1e-3) / 1e6, 1),
+                      "unit": "Mrows/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": step_ms,
+                      "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+                      "config": {"workload": f"modules: {n} rows of {irr}, {c} channels"},
+                      "roofline": {"bound": "hbm", "kernel": "cgtp::layer_rms_fwd_kernel<float,4>", "achieved": round(gbs, 1),
+                                   "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                                   "traffic": None, "algorithmic_bytes": nbytes, "avg_ms": f_ms},
+                      "modules": {name: {"fwd_ms": f, "fwd_bwd_ms": fb} for name, (f, fb) in table.items()}}))
 
 
 def scatter_bench(steps, warmup):
@@ -563,6 +629,9 @@ def main():
         return
     if args.workload == "scatter":
         scatter_bench(args.steps, args.warmup)
+        return
+    if args.workload == "modules":
+        modules_bench(args.steps, args.warmup)
         return
     if args.workload in ("uvw_fwd", "uvw_fwd_bwd"):
         uvw_bench(args)
