@@ -8,7 +8,9 @@ from typing import Optional
 
 import torch
 from torch import Tensor
+from torch.autograd import Function
 
+from ...ops import kernels
 from ...structs import WignerRotationInfo
 from .angular import sincos
 from .sparse_product import sparse_vecsca
@@ -20,10 +22,8 @@ def _z(x: Tensor, cs: Tensor, info: WignerRotationInfo) -> Tensor:
     return sparse_vecsca(x, cs, info.rotate_z_info_fwd, info.rotate_z_info_bwd_input, info.rotate_z_info_bwd_cs)
 
 
-def sparse_wigner_rotation(input: Tensor, sincos_alpha: Optional[Tensor], sincos_beta: Optional[Tensor],
-                           sincos_gamma: Optional[Tensor], info: WignerRotationInfo) -> Tensor:
-    """``D(alpha, beta, gamma) input`` for ``input (N, irreps.dim, C)`` and ``sincos_* (N, 1 + 2 max_m)`` (reference
-    ``:14-56``); an angle given as ``None`` is zero and its factor is skipped."""
+def _composed_rotation(input: Tensor, sincos_alpha, sincos_beta, sincos_gamma, info: WignerRotationInfo) -> Tensor:
+    """The reference's five launches (``:14-56``); differentiable in every argument to any order."""
     x = input
     if sincos_gamma is not None:
         x = _z(x, sincos_gamma, info)
@@ -34,6 +34,51 @@ def sparse_wigner_rotation(input: Tensor, sincos_alpha: Optional[Tensor], sincos
     if sincos_alpha is not None:
         x = _z(x, sincos_alpha, info)
     return x
+
+
+class _FusedRotation(Function):
+    """One launch (``cgtp_wigner_rotate``); the gradient of the features is the transposed rotation, again one
+    launch.  Gradients with respect to the angles, and gradients of higher order, go through the composition."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, sa, sb, sg, info: WignerRotationInfo, layout):
+        ctx.save_for_backward(x, sa, sb, sg)
+        ctx.info, ctx.layout = info, layout
+        return kernels.wigner_rotate(x, sa, sb, sg, layout, transposed=False)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, sa, sb, sg = ctx.saved_tensors
+        angles_need = any(ctx.needs_input_grad[1:4])
+        if angles_need or torch.is_grad_enabled():
+            with torch.enable_grad():
+                out = _composed_rotation(x, sa, sb, sg, ctx.info)
+                wanted = [(i, t) for i, t in enumerate((x, sa, sb, sg)) if t is not None and ctx.needs_input_grad[i]]
+                grads = torch.autograd.grad(out, [t for _, t in wanted], g, create_graph=torch.is_grad_enabled())
+            res = [None] * 4
+            for (i, _), gr in zip(wanted, grads):
+                res[i] = gr
+            return (*res, None, None)
+        gx = kernels.wigner_rotate(g.contiguous(), sa, sb, sg, ctx.layout, transposed=True)
+        return gx, None, None, None, None, None
+
+
+def sparse_wigner_rotation(input: Tensor, sincos_alpha: Optional[Tensor], sincos_beta: Optional[Tensor],
+                           sincos_gamma: Optional[Tensor], info: WignerRotationInfo) -> Tensor:
+    """``D(alpha, beta, gamma) input`` for ``input (N, irreps.dim, C)`` and ``sincos_* (N, 1 + 2 max_m)`` (reference
+    ``:14-56``); an angle given as ``None`` is zero and its factor is skipped.  fp32 / fp64 features with one sincos
+    row per sample and irreps up to l = 6 take the fused kernel; other cases the composition."""
+    cs = [t for t in (sincos_alpha, sincos_beta, sincos_gamma) if t is not None]
+    if (cs and input.is_cuda and input.ndim == 3 and input.dtype in (torch.float32, torch.float64)
+            and all(t.ndim == 2 and t.shape[0] == input.shape[0] and t.dtype == input.dtype
+                    and t.shape[1] == cs[0].shape[1] for t in cs)):
+        layout = kernels.rotation_layout(info)
+        if (layout.ok and layout.dim == input.shape[1] and cs[0].shape[1] >= 1 + 2 * layout.max_degree
+                and kernels.wigner_rotate_supported(layout, input.shape[2], input.dtype)):
+            c = lambda t: None if t is None else t.contiguous()
+            return _FusedRotation.apply(input.contiguous(), c(sincos_alpha), c(sincos_beta), c(sincos_gamma), info,
+                                        layout)
+    return _composed_rotation(input, sincos_alpha, sincos_beta, sincos_gamma, info)
 
 
 def dense_wigner_rotation(input: Tensor, wigner_d: Tensor) -> Tensor:

@@ -167,6 +167,85 @@ def layer_rms_backward(x: Tensor, weight: Optional[Tensor], rsigma: Tensor, grad
     return gx, gw
 
 
+# ---- fused Wigner rotation ----------------------------------------------------------------------------------
+class RotationLayout:
+    """Irrep blocks and dense J blocks recovered from the tables of a ``WignerRotationInfo``: the z-rotation table
+    pairs component ``m`` with ``-m`` (so the partner of a block's first row is its last row), and the entries of the
+    sparse J table fill one dense block per irrep.  ``ok`` is False when the tables do not have that structure."""
+
+    def __init__(self, info):
+        z, j = info.rotate_z_info_fwd, info.j_matrix_info
+        self.ok = False
+        # tables with identity columns or one term per output arrive with those fields collapsed to None
+        n_z = next((t.shape[0] for t in (z.index1, z.index2, z.scale) if t is not None), None)
+        if n_z is None or z.out_size is None:
+            return
+        dim = int(z.out_size)
+        zi = list(range(n_z)) if z.index1 is None else z.index1.tolist()
+        zseg = list(range(dim + 1)) if z.seg_out is None else z.seg_out.tolist()
+        if len(zseg) - 1 != dim:
+            return
+        first, degree, at = [], [], 0
+        while at < dim:
+            partner = max(zi[zseg[at]:zseg[at + 1]], default=at)     # m = -l pairs with m = +l, the block's last row
+            size = partner - at + 1
+            if size < 1 or size % 2 == 0 or at + size > dim:
+                return
+            first.append(at)
+            degree.append((size - 1) // 2)
+            at += size
+        block_of = [k for k, l in enumerate(degree) for _ in range(2 * l + 1)]
+        blocks = [torch.zeros(2 * l + 1, 2 * l + 1, dtype=torch.float64) for l in degree]
+        n_j = next((t.shape[0] for t in (j.index, j.scale) if t is not None), dim)
+        jseg = list(range(dim + 1)) if j.seg_out is None else j.seg_out.tolist()
+        jidx = list(range(n_j)) if j.index is None else j.index.tolist()
+        jval = [1.0] * n_j if j.scale is None else j.scale.double().tolist()
+        if len(jseg) - 1 != dim or jseg[-1] != n_j:
+            return
+        for row in range(dim):
+            k = block_of[row]
+            for t in range(jseg[row], jseg[row + 1]):
+                col = jidx[t]
+                if block_of[col] != k:
+                    return
+                blocks[k][row - first[k], col - first[k]] = jval[t]
+        self.first = (C.c_int32 * len(first))(*first)
+        self.degree = (C.c_int32 * len(degree))(*degree)
+        self.n_irreps, self.dim, self.max_degree = len(first), dim, max(degree, default=0)
+        self._flat = torch.cat([b.reshape(-1) for b in blocks]) if blocks else torch.zeros(0, dtype=torch.float64)
+        self._on = {}
+        self.ok = True
+
+    def j_blocks(self, dtype, device) -> Tensor:
+        key = (dtype, str(device))
+        if key not in self._on:
+            self._on[key] = self._flat.to(device=device, dtype=dtype)
+        return self._on[key]
+
+
+def rotation_layout(info) -> RotationLayout:
+    return cached(info.j_matrix_info.scale, "rotation_layout", lambda: RotationLayout(info))
+
+
+def wigner_rotate_supported(layout: RotationLayout, channels: int, dtype: torch.dtype) -> bool:
+    return (layout.ok and dtype in (torch.float32, torch.float64) and bool(_lib.lib.cgtp_wigner_rotate_supported(
+        layout.first, layout.degree, layout.n_irreps, channels, _lib.dtype_code(dtype))))
+
+
+def wigner_rotate(x: Tensor, sincos_alpha: Optional[Tensor], sincos_beta: Optional[Tensor],
+                  sincos_gamma: Optional[Tensor], layout: RotationLayout, transposed: bool) -> Tensor:
+    """``cgtp_wigner_rotate`` on ``x (N, D, C)`` contiguous; the sincos tensors are ``(N, cs_dim)`` contiguous."""
+    n, _, ch = x.shape
+    out = torch.empty_like(x)
+    cs_dim = next(t.shape[-1] for t in (sincos_alpha, sincos_beta, sincos_gamma) if t is not None)
+    _lib.check(_lib.lib.cgtp_wigner_rotate(x.data_ptr(), out.data_ptr(), _lib.ptr(sincos_alpha), _lib.ptr(sincos_beta),
+                                           _lib.ptr(sincos_gamma), layout.j_blocks(x.dtype, x.device).data_ptr(),
+                                           layout.first, layout.degree, layout.n_irreps, n, ch, cs_dim,
+                                           int(transposed), _lib.dtype_code(x.dtype), _lib.stream_ptr(x.device)),
+               "cgtp_wigner_rotate")
+    return out
+
+
 # ---- specialised uvu ----------------------------------------------------------------------------------------
 class SegIndex:
     """Per-sorted-position index arrays of the segment mode (all int64, same device)."""

@@ -291,6 +291,26 @@ int cgtp_layer_rms_backward(const void* x, const void* weight, const void* rsigm
                             const float* irrep_rdims, int n_irreps, int64_t n_rows, int D, int C, int scaled,
                             int dtype, void* stream);
 
+/* ---- rotation of equivariant features by Euler angles -------------------------------------------------------
+ * Stands in for sparse_wigner_rotation (equitorch/nn/functional/wigner_d.py:14-56: three sparse_vecsca launches
+ * for the rotations about z and two sparse_scale launches for the constant matrix J) with one launch:
+ *   out[n] = Z(alpha_n) J Z(beta_n) J Z(gamma_n) x[n],   transposed != 0: the transpose of that matrix (the
+ * gradient with respect to x), Z(phi): y[m] = cs[2|m|] x[m] - sign(m) cs[2|m|-1] x[-m], y[0] = cs[0] x[0].
+ * x, out: (n_rows, D, C) contiguous; sincos_*: (n_rows, cs_dim) with cs = (1, sin phi, cos phi, sin 2 phi, ...),
+ * cs_dim >= 1 + 2 max l, NULL = that factor is skipped (a NULL beta skips both J as well); j_blocks: DEVICE array,
+ * the dense (2l+1) x (2l+1) row-major block of J for every irrep one after the other; irrep_first / irrep_degree:
+ * HOST arrays, first component and degree l of every irrep (consecutive blocks covering 0 .. D-1, l <= 6, at most 64
+ * irreps).  C <= 64, or C/4 (fp32) resp. C/2 (fp64) <= 64 with 16-byte aligned pointers:
+ * cgtp_wigner_rotate_supported tells.  dtype: CGTP_F32 | CGTP_F64.  Gradients with respect to the sincos
+ * tensors are not provided here.
+ */
+int cgtp_wigner_rotate_supported(const int32_t* irrep_first, const int32_t* irrep_degree, int n_irreps, int C,
+                                 int dtype);
+int cgtp_wigner_rotate(const void* x, void* out, const void* sincos_alpha, const void* sincos_beta,
+                       const void* sincos_gamma, const void* j_blocks, const int32_t* irrep_first,
+                       const int32_t* irrep_degree, int n_irreps, int64_t n_rows, int C, int cs_dim, int transposed,
+                       int dtype, void* stream);
+
 /* ---- streaming kernels of known traffic (counter calibration, achievable-bandwidth reference) ------------
  * No counterpart in the reference.  copy: reads n_bytes and writes n_bytes; read: reads n_bytes.
  * n_bytes must be a multiple of 16 and the pointers 16-byte aligned.

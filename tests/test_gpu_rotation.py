@@ -93,3 +93,47 @@ def test_so2_linear(device, mode, per_sample):
     gx, gw = torch.autograd.grad(out, (xd, wd), ct.to(device))
     for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
         assert_close(a, b, tol=1e-11, what=f"SO2Linear {mode} per_sample={per_sample} {name}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("channels", [64, 10])
+def test_fused_rotation_kernel(device, dtype, channels):
+    """``cgtp_wigner_rotate`` (forward and, with angles that need no gradient, the transposed launch for the gradient
+    of the features) against the oracle and against the five-launch composition: irreps up to l = 6 with a repeated
+    and an out-of-order degree, 16-byte and single-element lanes, rows not a multiple of the rows per wavefront,
+    every subset of the three angles."""
+    from equitorch_amd.nn.functional import sincos, sparse_wigner_rotation
+    from equitorch_amd.nn.functional.wigner_d import _composed_rotation
+    from equitorch_amd.ops import kernels
+    from equitorch_amd.utils import wigner_d_info
+    irr = "2e+0e+6e+1o+1o+4e"
+    dim = 5 + 1 + 13 + 3 + 3 + 9
+    z = _f32(ref_tables.z_rotation_infos(irr)[0])
+    j = _f32(ref_tables.j_matrix_info(irr))
+    info = wigner_d_info(irr).to(device)
+    layout = kernels.rotation_layout(info)
+    assert layout.ok and list(layout.degree) == [2, 0, 6, 1, 1, 4] and list(layout.first) == [0, 5, 6, 19, 22, 25]
+    assert kernels.wigner_rotate_supported(layout, channels, dtype)
+    g = torch.Generator().manual_seed(3)
+    n = 77
+    x = torch.randn(n, dim, channels, generator=g, dtype=torch.float64).to(dtype).double()
+    ang = ((torch.rand(3, n, generator=g, dtype=torch.float64) - 0.5) * 6).to(dtype).double()
+    ct = torch.randn(n, dim, channels, generator=g, dtype=torch.float64).to(dtype).double()
+    tol = 1e-5 if dtype == torch.float32 else 1e-11
+    for use in ((1, 1, 1), (1, 0, 0), (0, 1, 0), (0, 0, 1), (1, 0, 1)):
+        xr = x.clone().requires_grad_(True)
+        ref = ref_ops.cpu_wigner_rotation(xr, *(ref_ops.cpu_sincos(ang[k], 6) if use[k] else None for k in range(3)), z, j)
+        (rgx,) = torch.autograd.grad(ref, xr, ct)
+        xd = x.to(device, dtype).requires_grad_(True)
+        cs = [sincos(ang[k].to(device, dtype), 6) if use[k] else None for k in range(3)]
+        out = sparse_wigner_rotation(xd, *cs, info)
+        assert type(out.grad_fn).__name__ == "_FusedRotationBackward"
+        (gx,) = torch.autograd.grad(out, xd, ct.to(device, dtype))
+        assert_close(out, ref, tol=tol, what=f"rotation {use}")
+        assert_close(gx, rgx, tol=tol, what=f"transposed rotation {use}")
+        with torch.no_grad():
+            comp = _composed_rotation(xd, *cs, info)
+        assert_close(out, comp, tol=1e-6 if dtype == torch.float32 else 1e-13, what=f"against the composition {use}")
+    # degrees above 6 are outside the fused kernel
+    big = wigner_d_info("0e+7o").to(device)
+    assert not kernels.wigner_rotate_supported(kernels.rotation_layout(big), channels, dtype)
