@@ -67,9 +67,12 @@ def sparse_wigner_rotation(input: Tensor, sincos_alpha: Optional[Tensor], sincos
                            sincos_gamma: Optional[Tensor], info: WignerRotationInfo) -> Tensor:
     """``D(alpha, beta, gamma) input`` for ``input (N, irreps.dim, C)`` and ``sincos_* (N, 1 + 2 max_m)`` (reference
     ``:14-56``); an angle given as ``None`` is zero and its factor is skipped.  fp32 / fp64 features with one sincos
-    row per sample and irreps up to l = 6 take the fused kernel; other cases the composition."""
+    row per sample, angles that need no gradient and irreps up to l = 6 take the fused kernel; other cases the
+    composition."""
     cs = [t for t in (sincos_alpha, sincos_beta, sincos_gamma) if t is not None]
-    if (cs and input.is_cuda and input.ndim == 3 and input.dtype in (torch.float32, torch.float64)
+    # angles that need a gradient: the composition computes it without a second forward pass
+    angles_fixed = not (torch.is_grad_enabled() and any(t.requires_grad for t in cs))
+    if (cs and angles_fixed and input.is_cuda and input.ndim == 3 and input.dtype in (torch.float32, torch.float64)
             and all(t.ndim == 2 and t.shape[0] == input.shape[0] and t.dtype == input.dtype
                     and t.shape[1] == cs[0].shape[1] for t in cs)):
         layout = kernels.rotation_layout(info)
