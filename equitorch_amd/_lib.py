@@ -117,6 +117,8 @@ def _load():
     lib.cgtp_wigner_rotate_supported.argtypes = [_seg, _seg, C.c_int, C.c_int, C.c_int]
     lib.cgtp_wigner_rotate.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, _seg,
                                        _seg, C.c_int, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
+    lib.cgtp_wigner_rotate_backward.argtypes = [C.c_void_p] * 6 + [_seg, _seg, C.c_int, C.c_int64, C.c_int, C.c_int] + \
+        [C.c_void_p] * 4 + [C.c_int, C.c_void_p]
     lib.cgtp_membench_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
     lib.cgtp_membench_read.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
     return lib

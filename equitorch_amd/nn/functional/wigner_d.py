@@ -37,8 +37,9 @@ def _composed_rotation(input: Tensor, sincos_alpha, sincos_beta, sincos_gamma, i
 
 
 class _FusedRotation(Function):
-    """One launch (``cgtp_wigner_rotate``); the gradient of the features is the transposed rotation, again one
-    launch.  Gradients with respect to the angles, and gradients of higher order, go through the composition."""
+    """One launch (``cgtp_wigner_rotate``).  The gradient of the features alone is the transposed rotation, again one
+    launch; with gradients of the sincos tensors it is ``cgtp_wigner_rotate_backward``, which recomputes the
+    intermediate features in registers.  Gradients of higher order go through the composition."""
 
     @staticmethod
     def forward(ctx, x: Tensor, sa, sb, sg, info: WignerRotationInfo, layout):
@@ -49,30 +50,30 @@ class _FusedRotation(Function):
     @staticmethod
     def backward(ctx, g):
         x, sa, sb, sg = ctx.saved_tensors
-        angles_need = any(ctx.needs_input_grad[1:4])
-        if angles_need or torch.is_grad_enabled():
+        need_cs = [t is not None and ctx.needs_input_grad[1 + i] for i, t in enumerate((sa, sb, sg))]
+        if torch.is_grad_enabled():          # a gradient of this gradient is wanted
             with torch.enable_grad():
                 out = _composed_rotation(x, sa, sb, sg, ctx.info)
                 wanted = [(i, t) for i, t in enumerate((x, sa, sb, sg)) if t is not None and ctx.needs_input_grad[i]]
-                grads = torch.autograd.grad(out, [t for _, t in wanted], g, create_graph=torch.is_grad_enabled())
+                grads = torch.autograd.grad(out, [t for _, t in wanted], g, create_graph=True)
             res = [None] * 4
             for (i, _), gr in zip(wanted, grads):
                 res[i] = gr
             return (*res, None, None)
-        gx = kernels.wigner_rotate(g.contiguous(), sa, sb, sg, ctx.layout, transposed=True)
-        return gx, None, None, None, None, None
+        if not any(need_cs):                 # the transposed rotation; nothing to recompute
+            return kernels.wigner_rotate(g.contiguous(), sa, sb, sg, ctx.layout, transposed=True), None, None, None, None, None
+        gx, gcs = kernels.wigner_rotate_backward(x, g.contiguous(), (sa, sb, sg), ctx.layout, ctx.needs_input_grad[0],
+                                                 need_cs)
+        return (gx, *gcs, None, None)
 
 
 def sparse_wigner_rotation(input: Tensor, sincos_alpha: Optional[Tensor], sincos_beta: Optional[Tensor],
                            sincos_gamma: Optional[Tensor], info: WignerRotationInfo) -> Tensor:
     """``D(alpha, beta, gamma) input`` for ``input (N, irreps.dim, C)`` and ``sincos_* (N, 1 + 2 max_m)`` (reference
     ``:14-56``); an angle given as ``None`` is zero and its factor is skipped.  fp32 / fp64 features with one sincos
-    row per sample, angles that need no gradient and irreps up to l = 6 take the fused kernel; other cases the
-    composition."""
+    row per sample and irreps up to l = 6 take the fused kernels; other cases the composition."""
     cs = [t for t in (sincos_alpha, sincos_beta, sincos_gamma) if t is not None]
-    # angles that need a gradient: the composition computes it without a second forward pass
-    angles_fixed = not (torch.is_grad_enabled() and any(t.requires_grad for t in cs))
-    if (cs and angles_fixed and input.is_cuda and input.ndim == 3 and input.dtype in (torch.float32, torch.float64)
+    if (cs and input.is_cuda and input.ndim == 3 and input.dtype in (torch.float32, torch.float64)
             and all(t.ndim == 2 and t.shape[0] == input.shape[0] and t.dtype == input.dtype
                     and t.shape[1] == cs[0].shape[1] for t in cs)):
         layout = kernels.rotation_layout(info)

@@ -246,6 +246,21 @@ def wigner_rotate(x: Tensor, sincos_alpha: Optional[Tensor], sincos_beta: Option
     return out
 
 
+def wigner_rotate_backward(x: Tensor, grad_out: Tensor, sincos, layout: RotationLayout, need_x: bool, need_cs):
+    """``(grad_x | None, [grad of each sincos tensor | None])`` of ``cgtp_wigner_rotate_backward``; ``sincos`` is the
+    triple (alpha, beta, gamma) with ``None`` for a skipped factor, ``need_cs`` the matching triple of flags."""
+    n, _, ch = x.shape
+    cs_dim = next(t.shape[-1] for t in sincos if t is not None)
+    gx = torch.empty_like(x) if need_x else None
+    gcs = [torch.empty_like(t) if (t is not None and want) else None for t, want in zip(sincos, need_cs)]
+    _lib.check(_lib.lib.cgtp_wigner_rotate_backward(x.data_ptr(), grad_out.data_ptr(), *[_lib.ptr(t) for t in sincos],
+                                                    layout.j_blocks(x.dtype, x.device).data_ptr(), layout.first,
+                                                    layout.degree, layout.n_irreps, n, ch, cs_dim, _lib.ptr(gx),
+                                                    *[_lib.ptr(t) for t in gcs], _lib.dtype_code(x.dtype),
+                                                    _lib.stream_ptr(x.device)), "cgtp_wigner_rotate_backward")
+    return gx, gcs
+
+
 # ---- specialised uvu ----------------------------------------------------------------------------------------
 class SegIndex:
     """Per-sorted-position index arrays of the segment mode (all int64, same device)."""

@@ -301,8 +301,11 @@ int cgtp_layer_rms_backward(const void* x, const void* weight, const void* rsigm
  * the dense (2l+1) x (2l+1) row-major block of J for every irrep one after the other; irrep_first / irrep_degree:
  * HOST arrays, first component and degree l of every irrep (consecutive blocks covering 0 .. D-1, l <= 6, at most 64
  * irreps).  C <= 64, or C/4 (fp32) resp. C/2 (fp64) <= 64 with 16-byte aligned pointers:
- * cgtp_wigner_rotate_supported tells.  dtype: CGTP_F32 | CGTP_F64.  Gradients with respect to the sincos
- * tensors are not provided here.
+ * cgtp_wigner_rotate_supported tells.  dtype: CGTP_F32 | CGTP_F64.
+ * cgtp_wigner_rotate_backward: from x and grad_out (n_rows, D, C), the gradient of the features (grad_x, NULL = not
+ * wanted) and of the sincos tensors (grad_alpha / grad_beta / grad_gamma, each (n_rows, cs_dim) or NULL; columns
+ * beyond 1 + 2 max l are written as zeros) in one launch that recomputes the intermediate features in registers
+ * (the reference's autograd keeps them in memory).
  */
 int cgtp_wigner_rotate_supported(const int32_t* irrep_first, const int32_t* irrep_degree, int n_irreps, int C,
                                  int dtype);
@@ -310,6 +313,11 @@ int cgtp_wigner_rotate(const void* x, void* out, const void* sincos_alpha, const
                        const void* sincos_gamma, const void* j_blocks, const int32_t* irrep_first,
                        const int32_t* irrep_degree, int n_irreps, int64_t n_rows, int C, int cs_dim, int transposed,
                        int dtype, void* stream);
+int cgtp_wigner_rotate_backward(const void* x, const void* grad_out, const void* sincos_alpha, const void* sincos_beta,
+                                const void* sincos_gamma, const void* j_blocks, const int32_t* irrep_first,
+                                const int32_t* irrep_degree, int n_irreps, int64_t n_rows, int C, int cs_dim,
+                                void* grad_x, void* grad_alpha, void* grad_beta, void* grad_gamma, int dtype,
+                                void* stream);
 
 /* ---- streaming kernels of known traffic (counter calibration, achievable-bandwidth reference) ------------
  * No counterpart in the reference.  copy: reads n_bytes and writes n_bytes; read: reads n_bytes.

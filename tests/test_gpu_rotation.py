@@ -137,3 +137,51 @@ def test_fused_rotation_kernel(device, dtype, channels):
     # degrees above 6 are outside the fused kernel
     big = wigner_d_info("0e+7o").to(device)
     assert not kernels.wigner_rotate_supported(kernels.rotation_layout(big), channels, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("irr,channels", [("2e+0e+6e+1o+1o+4e", 64), ("2e+0e+6e+1o+1o+4e", 10), ("0e+1o+2e+1o", 64),
+                                          ("3o+4e", 24)])
+def test_fused_rotation_gradients_of_the_sincos_tensors(device, dtype, irr, channels):
+    """``cgtp_wigner_rotate_backward``: gradients of the features and of the three sincos tensors (leaves here, with
+    more columns than the largest degree needs) against the oracle's autograd, for largest degrees 2, 4 and 6 (four,
+    four and two channels per lane in fp32) and every subset of angles; a sincos tensor that is given but needs no
+    gradient gets none."""
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.nn.functional import sparse_wigner_rotation
+    from equitorch_amd.utils import wigner_d_info
+    dim, max_l = Irreps(irr).dim, max(ir.l for ir in Irreps(irr))
+    z = _f32(ref_tables.z_rotation_infos(irr)[0])
+    j = _f32(ref_tables.j_matrix_info(irr))
+    info = wigner_d_info(irr).to(device)
+    g = torch.Generator().manual_seed(4)
+    n, extra = 53, 2
+    x = torch.randn(n, dim, channels, generator=g, dtype=torch.float64).to(dtype).double()
+    ang = (torch.rand(3, n, generator=g, dtype=torch.float64) - 0.5) * 6
+    cs = [torch.cat([ref_ops.cpu_sincos(ang[k], max_l), torch.randn(n, extra, generator=g, dtype=torch.float64)], dim=1)
+          .to(dtype).double() for k in range(3)]
+    ct = torch.randn(n, dim, channels, generator=g, dtype=torch.float64).to(dtype).double()
+    tol = 2e-5 if dtype == torch.float32 else 1e-10
+    for use in ((1, 1, 1), (0, 1, 1), (1, 0, 0), (0, 0, 1)):
+        xr = x.clone().requires_grad_(True)
+        cr = [c[:, :1 + 2 * max_l].clone().requires_grad_(True) if u else None for c, u in zip(cs, use)]
+        ref = ref_ops.cpu_wigner_rotation(xr, *cr, z, j)
+        refs = torch.autograd.grad(ref, [xr] + [c for c in cr if c is not None], ct)
+        xd = x.to(device, dtype).requires_grad_(True)
+        cd = [c.to(device, dtype).requires_grad_(True) if u else None for c, u in zip(cs, use)]
+        out = sparse_wigner_rotation(xd, *cd, info)
+        assert type(out.grad_fn).__name__ == "_FusedRotationBackward"
+        got = torch.autograd.grad(out, [xd] + [c for c in cd if c is not None], ct.to(device, dtype))
+        assert_close(got[0], refs[0], tol=tol, what=f"grad x {use}")
+        for a, b in zip(got[1:], refs[1:]):
+            # sums over dim x channels products: judged relative to the largest entry
+            assert_close(a[:, :1 + 2 * max_l], b, tol=tol * 10, what=f"grad sincos {use}")
+            assert float(a[:, 1 + 2 * max_l:].abs().max()) == 0.0
+    # only one of two given sincos tensors needs a gradient
+    xd = x.to(device, dtype)
+    ca = cs[0].to(device, dtype).requires_grad_(True)
+    cb = cs[1].to(device, dtype)
+    (ga,) = torch.autograd.grad(sparse_wigner_rotation(xd, ca, cb, None, info), ca, ct.to(device, dtype))
+    cr = [cs[0][:, :1 + 2 * max_l].clone().requires_grad_(True), cs[1][:, :1 + 2 * max_l]]
+    (ra,) = torch.autograd.grad(ref_ops.cpu_wigner_rotation(x, cr[0], cr[1], None, z, j), cr[0], ct)
+    assert_close(ga[:, :1 + 2 * max_l], ra, tol=tol * 10, what="grad of alpha alone")
