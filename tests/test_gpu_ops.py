@@ -271,3 +271,35 @@ def test_uv_mfma_full_size_properties(device):
         parts.append(gp.double())
     scale = float(gw.double().abs().max())
     assert float((gw.double() - parts[0] - parts[1]).abs().max()) <= 2e-2 * scale
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("channels", [(8, 16, 4), (32, 32, 8), (6, 20, 5)])
+def test_uvw_on_the_two_operand_kernels(device, dtype, channels):
+    """``tensor_product_uvw`` on enough rows for the outer-product and contraction kernels of the two-axis family
+    (16-byte lanes along the contiguous axis; (6, 20, .): 5 lanes per row do not divide the workgroup, the general
+    kernel runs): forward and all three gradients against the dense einsum, shared weight."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    io, i1, i2 = "0e+1o+2e", "0e+1o+2e", "0e+1o"
+    infos = [t.to(device) for t in tp_infos(Irreps(io), Irreps(i1), Irreps(i2))[:3]]
+    T = ref_ops.dense_coupling(io, i1, i2).float().double()      # the tables hold fp32 coefficients
+    p = T.shape[0]
+    g = torch.Generator().manual_seed(7)
+    n = 301
+    u, v, w = channels
+    x = torch.randn(n, 9, u, generator=g, dtype=torch.float64).to(dtype).double()
+    y = torch.randn(n, 4, v, generator=g, dtype=torch.float64).to(dtype).double()
+    wt = (torch.randn(p, u, v, w, generator=g, dtype=torch.float64) / (u * v) ** 0.5).to(dtype).double()
+    xd, yd, wd = (t.to(device, dtype).requires_grad_(True) for t in (x, y, wt))
+    out = F.tensor_product_uvw(xd, yd, wd, *infos)
+    xr, yr, wr = (t.clone().requires_grad_(True) for t in (x, y, wt))
+    ref_out = torch.einsum("pmab,nau,nbv,puvw->nmw", T, xr, yr, wr)
+    tol = 1e-5 if dtype == torch.float32 else 1e-11
+    assert_close(out, ref_out, tol, "uvw forward")
+    ct = torch.randn(ref_out.shape, generator=g, dtype=torch.float64).to(dtype).double()
+    grads = torch.autograd.grad(out, (xd, yd, wd), ct.to(device, dtype))
+    refs = torch.autograd.grad(ref_out, (xr, yr, wr), ct)
+    for name, a, b in zip(("grad1", "grad2", "grad_w"), grads, refs):
+        assert_close(a, b, tol * 10, f"uvw {name}")
