@@ -241,6 +241,11 @@ def modules_bench(steps, warmup):
         "Gate": both(enn.Gate(irr, activation=None).to(dev), gates),
         "SquaredNorm": both(enn.SquaredNorm(irr).to(dev)),
         "TensorDot_uu": both(enn.TensorDot(irr, "uu").to(dev), x),
+        "Norm": both(enn.Norm(irr).to(dev)),
+        "BatchRMSNorm_train": both(enn.BatchRMSNorm(irr, c).to(dev).train()),
+        "BatchRMSNorm_eval": both(enn.BatchRMSNorm(irr, c).to(dev).eval()),
+        "IrrepsLinear_fp32": both(enn.IrrepsLinear(irr, irr, c, c).to(dev)),
+        "IrrepWiseLinear_fp32": both(enn.IrrepWiseLinear(irr, c, c).to(dev)),
         "SO2Linear_uu": both(enn.SO2Linear(irr, irr, c, c, feature_mode="uu").to(dev)),
         "SO2Linear_uv": both(enn.SO2Linear(irr, irr, c, c, feature_mode="uv").to(dev)),
         "SparseWignerRotation": both(enn.SparseWignerRotation(irr).to(dev), *sc),

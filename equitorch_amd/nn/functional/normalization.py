@@ -6,7 +6,7 @@ from torch.autograd import Function
 from ...ops import kernels
 from ...structs import IrrepsInfo
 from .activations import _broadcast_infos
-from .norm import channel_mean_squared_norm, squared_norm
+from .norm import batch_mean_squared_norm, channel_mean_squared_norm
 from .sparse_product import sparse_mul, sparse_vecsca
 
 
@@ -16,7 +16,7 @@ def batch_rms_norm(input: Tensor, running_squared_norm: Tensor, irreps_info: Irr
     ``s`` the batch mean of the per-sample squared norms when ``training`` (then also blended into
     ``running_squared_norm`` in place with ``momentum``), else ``running_squared_norm`` (reference ``:10-72``)."""
     if training:
-        stat = squared_norm(input, irreps_info, scaled).mean(dim=0)
+        stat = batch_mean_squared_norm(input, irreps_info, scaled)      # summed over the batch inside the launch
         running_squared_norm.data.lerp_(stat.detach().to(running_squared_norm.dtype), momentum)
     else:
         stat = running_squared_norm
