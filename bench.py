@@ -53,6 +53,9 @@ WORKLOADS = {
     "irreps_linear": None,
     # element-wise and SO(2) modules on 65536 rows of 0e+1o+2e, 64 channels, fp32 (table of timings)
     "modules": None,
+    # a whole message-passing layer (harmonics + radial MLP + fused edge product + mixing + gate + layer norm) at the
+    # shape of BASELINE configs[2], forward + backward, launched eagerly and replayed as one recorded HIP graph
+    "layer": None,
     # plain library GEMM (torch.matmul, bf16, 8192^3): the matrix rate the box reaches, next to the vendor peak
     "gemm": None,
 }
@@ -600,6 +603,84 @@ def cpu_model():
     return "unknown CPU"
 
 
+def layer_bench(steps, warmup):
+    """Forward + backward of a message-passing layer built from the public modules on 4096 nodes / 65536 edges,
+    0e+1o+2e, 64 channels, fp32: wall time per step launched eagerly from Python, and the same step recorded once
+    with ``torch.cuda.graph`` and replayed (the launches are host-bound when issued one by one)."""
+    import time
+
+    from equitorch_amd import nn as enn
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu_vectors
+    dev = torch.device("cuda:0")
+    irr, n_nodes, n_edges, c, num_basis, r_max = "0e+1o+2e", 4096, 65536, 64, 8, 3.0
+
+    class Layer(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.basis = enn.BesselBasis(r_max, num_basis, trainable=False)
+            self.cutoff = enn.PolynomialCutoff(r_max)
+            self.tp = enn.SO3Linear(irr, irr, irr, c, c, internal_weights=False, feature_mode="uu")
+            self.radial = torch.nn.Sequential(torch.nn.Linear(num_basis, 16), torch.nn.SiLU(),
+                                              torch.nn.Linear(16, self.tp.num_paths * c))
+            self.mix = enn.IrrepsLinear(irr, irr, c, c)
+            self.gate_lin = enn.IrrepsLinear(irr, "0e+0e+0e", c, c)
+            self.gate = enn.Gate(irr, activation=torch.nn.Sigmoid())
+            self.norm = enn.LayerRMSNorm(irr, c)
+
+        def forward(self, x, edge_vec, plan):
+            r = edge_vec.norm(dim=-1)
+            w = self.radial(self.basis(r) * self.cutoff(r)[:, None]).view(-1, self.tp.num_paths, c)
+            h = self.mix(edge_tensor_product_uu_vectors(x, edge_vec, w, plan, self.tp.tp_info_forward))
+            return self.norm(self.gate(h, self.gate_lin(h)))
+
+    torch.manual_seed(0)
+    layer = Layer().to(dev)
+    g = torch.Generator().manual_seed(1)
+    plan = EdgePlan(torch.randint(0, n_nodes, (n_edges,), generator=g).to(dev),
+                    torch.randint(0, n_nodes, (n_edges,), generator=g).to(dev), n_nodes)
+    x = torch.randn(n_nodes, 9, c, generator=g).to(dev).requires_grad_(True)
+    ev = (torch.randn(n_edges, 3, generator=g) * 1.2).to(dev).requires_grad_(True)
+    ct = torch.randn(n_nodes, 9, c, generator=g).to(dev)
+    wrt = [x, ev] + list(layer.parameters())
+
+    def step():
+        return torch.autograd.grad(layer(x, ev, plan), wrt, ct)
+
+    def wall(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3
+
+    eager_ms = wall(step)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        recorded = step()
+    graph_ms = wall(graph.replay)
+    expect = step()
+    torch.cuda.synchronize()
+    err = max(float((a - b).abs().max() / b.abs().max().clamp_min(1e-30)) for a, b in zip(recorded, expect))
+    print(json.dumps({"metric": "message-passing layer fwd+bwd Medges/s (lmax=2, C=64, fp32)",
+                      "value": round(n_edges / (graph_ms * 1e-3) / 1e6, 1), "unit": "Medges/s", "n_gpus": 1,
+                      "steps": steps, "warmup": warmup, "ms_per_step": round(graph_ms, 4), "higher_is_better": True,
+                      "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+                      "config": {"workload": f"layer: {n_nodes} nodes, {n_edges} edges, {irr}, {c} channels, "
+                                             "one recorded HIP graph per step"},
+                      "eager_ms_per_step": round(eager_ms, 4), "graph_ms_per_step": round(graph_ms, 4),
+                      "graph_vs_eager_max_rel_err": err}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -637,6 +718,9 @@ def main():
         return
     if args.workload == "modules":
         modules_bench(args.steps, args.warmup)
+        return
+    if args.workload == "layer":
+        layer_bench(args.steps, args.warmup)
         return
     if args.workload in ("uvw_fwd", "uvw_fwd_bwd"):
         uvw_bench(args)
