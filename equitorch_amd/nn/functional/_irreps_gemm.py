@@ -231,6 +231,24 @@ def _long_k_bmm(a: Tensor, b: Tensor) -> Tensor:
     return parts.sum(dim=1)
 
 
+def _all_rows_outer(x: Tensor, g: Tensor):
+    """``prod[j] = sum_n x[n, j, :]^T (x) g[n, j, :]`` for every component ``j`` of contiguous ``x (N, D, C_in)`` and
+    ``g (N, D, C_out)``, or None when ``N`` is too short to be worth cutting.  The sum over samples is cut into ``S``
+    interleaved slices (sample ``n`` belongs to slice ``n mod S``): seen as ``(N/S, S*D, C)`` the tensors then have
+    one batch axis ``(slice, component)`` of stride ``C``, so the ``S*D`` partial products are one batched GEMM on
+    the tensors as they lie in memory, and their sum over the slices is small."""
+    n, d, cin = x.shape
+    cout = g.shape[-1]
+    s = 1
+    while s < 64 and n % (2 * s) == 0 and n // (2 * s) >= 512:
+        s *= 2
+    if s == 1:
+        return None
+    a = x.view(n // s, s * d, cin).permute(1, 2, 0)             # (S*D, C_in, N/S), a transposed operand
+    b = g.view(n // s, s * d, cout).transpose(0, 1)             # (S*D, N/S, C_out)
+    return torch.bmm(a, b).view(s, d, cin, cout).sum(dim=0)
+
+
 def _outer_raw(x: Tensor, g: Tensor, plan: LinearPlan, shared: bool) -> Tensor:
     """``gw[(n,) p] = scale * sum_j x[n, i0+j, :]^T (x) g[n, o0+j, :]`` (summed over ``n`` when ``shared``)."""
     n, _, cin = x.shape
@@ -239,9 +257,13 @@ def _outer_raw(x: Tensor, g: Tensor, plan: LinearPlan, shared: bool) -> Tensor:
         gw = torch.zeros((plan.n_paths, cin, cout), dtype=x.dtype, device=x.device)
         if n:
             for grp in _groups(plan):
-                a = x[:, grp.i0:grp.i0 + grp.rows, :].permute(1, 2, 0)          # (rows, cin, N)
-                b = g[:, grp.o0:grp.o0 + grp.rows, :].transpose(0, 1)           # (rows, N, cout)
-                prod = _long_k_bmm(a, b)
+                prod = None
+                if grp.rows == x.shape[1] == g.shape[1] and x.is_contiguous() and g.is_contiguous():
+                    prod = _all_rows_outer(x, g)
+                if prod is None:
+                    a = x[:, grp.i0:grp.i0 + grp.rows, :].permute(1, 2, 0)      # (rows, cin, N)
+                    b = g[:, grp.o0:grp.o0 + grp.rows, :].transpose(0, 1)       # (rows, N, cout)
+                    prod = _long_k_bmm(a, b)
                 if grp.scale is None:
                     gw.index_add_(0, _row_weights(grp, x.device), prod * _row_scales(grp, prod))
                 else:
