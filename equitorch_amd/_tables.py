@@ -36,7 +36,7 @@ def _expand_seg(seg, n_rows_default: int) -> np.ndarray:
 def tp_coo(tp_info) -> TpCoo:
     """Flatten the forward tables of one ``TensorProductInfo`` into per-non-zero arrays (table order)."""
     s1, s2 = tp_info.info_Mij_fwd, tp_info.info_M_fwd
-    coef = s1.scale.detach().cpu().numpy().astype(np.float64)
+    coef = s1.scale.detach().cpu().double().numpy()
     T = coef.shape[0]
     ident = np.arange(T, dtype=np.int64)
     M1 = ident if s1.index1 is None else s1.index1.cpu().numpy()

@@ -38,7 +38,7 @@ class Gate(IrrepsModule):
             if self.activation is not None:
                 gate = self.activation(gate)
             return features * gate
-        shared = gate.numel() <= self.num_gates * channels
+        shared = gate.numel() == self.num_gates * channels          # an empty batch has an empty, batched gate
         gate = gate.reshape(self.num_gates, channels) if shared else gate.reshape(-1, self.num_gates, channels)
         if self.activation is not None:
             gate = self.activation(gate)

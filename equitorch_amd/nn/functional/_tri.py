@@ -93,6 +93,8 @@ def _gen_contract(spec: "TriSpec", ops, axes, out_axes: str, out_shared: bool, n
     if not out_shared:
         shape = (n_rows,) + shape
     out = torch.empty(shape, dtype=dtype, device=device)
+    if n_rows == 0 or out.numel() == 0:      # empty batch: nothing to launch; a sum over no rows is zero
+        return out.zero_()
     a.out, a.n_rows, a.U, a.W = out.data_ptr(), n_rows, U, W
     a.out_has_u, a.out_has_w = int("u" in out_axes), int("w" in out_axes)
     a.reduce_rows, a.dtype = int(out_shared), _lib.dtype_code(dtype)
@@ -212,7 +214,7 @@ def spec_from_product_info(info, size1: int, size2: int) -> TriSpec:
             out_idx = np.repeat(np.arange(n_out, dtype=np.int64), np.diff(s))
         if info.out_size is not None:
             n_out = max(n_out, int(info.out_size))
-        coef = None if info.scale is None else info.scale.detach().cpu().numpy().astype(np.float64)
+        coef = None if info.scale is None else info.scale.detach().cpu().double().numpy()
         return TriSpec(out_idx, [i1, i2, None], coef, n_out, [size1, size2, None])
 
     if anchor is None:

@@ -72,14 +72,16 @@ def tri_contract(table: dict, n_out: int, a: Tuple[Optional[Tensor], int], b: Tu
                  rows_a: Optional[Tensor] = None, rows_b: Optional[Tensor] = None,
                  rows_w: Optional[Tensor] = None) -> Tensor:
     """``out[r,o,c] = sum_t coef_t A[r,ia_t,c] B[r,ib_t,(c)] W[r,iw_t,c]`` with the packed ``table``."""
-    args = TriArgs()
-    args.a, args.b, args.w = _operand(*a, rows_a), _operand(*b, rows_b), _operand(*w, rows_w)
-    args.coef, args.idx, args.seg = _lib.ptr(table["coef"]), table["idx"].data_ptr(), table["seg"].data_ptr()
-    args.n_out, args.nnz = n_out, table["idx"].shape[0]
     shape = ((n_out,) if reduce_c else (n_out, channels))
     if not reduce_rows:
         shape = (n_rows,) + shape
     out = torch.empty(shape, dtype=dtype, device=device)
+    if n_rows == 0 or out.numel() == 0:      # empty batch: nothing to launch; a sum over no rows is zero
+        return out.zero_()
+    args = TriArgs()
+    args.a, args.b, args.w = _operand(*a, rows_a), _operand(*b, rows_b), _operand(*w, rows_w)
+    args.coef, args.idx, args.seg = _lib.ptr(table["coef"]), table["idx"].data_ptr(), table["seg"].data_ptr()
+    args.n_out, args.nnz = n_out, table["idx"].shape[0]
     args.out, args.n_rows, args.C = out.data_ptr(), n_rows, channels
     args.dtype, args.reduce_c, args.reduce_rows = _lib.dtype_code(dtype), int(reduce_c), int(reduce_rows)
     ws = None
@@ -95,9 +97,13 @@ def segment_sum(inp: Tensor, scale: Optional[Tensor], index: Optional[Tensor], s
                 out_size: int) -> Tensor:
     """``out[n,m,c] = sum_{t in seg m} scale[t] * inp[n, index[t], c]`` (``seg=None``: one term per row)."""
     _lib.require_gpu(inp, scale, index, seg)
+    if inp.dtype not in (torch.float32, torch.float64):      # reduced precision: summed in fp32, rounded once
+        return segment_sum(inp.float(), scale, index, seg, out_size).to(inp.dtype)
     inp = inp.contiguous()
     n, in_size, ch = inp.shape
     out = torch.empty((n, out_size, ch), dtype=inp.dtype, device=inp.device)
+    if inp.numel() == 0 or out.numel() == 0:      # nothing to sum: every output row is an empty sum
+        return out.zero_()
     n_seg = out_size if seg is None else seg.shape[0] - 1
     if n_seg < out_size:
         out.zero_()
@@ -432,7 +438,7 @@ def product_tri_table(scale, index1, index2, seg, n_entries: int, dtype, device)
             s = seg.detach().cpu().numpy().astype(np.int64)
             n_out = s.shape[0] - 1
             out_idx = np.repeat(np.arange(n_out, dtype=np.int64), np.diff(s))
-        coef = None if scale is None else scale.detach().cpu().numpy().astype(np.float64)
+        coef = None if scale is None else scale.detach().cpu().double().numpy()
         return pack_tri_table(out_idx, i1, i2, None, coef, n_out, dtype, device), n_out
     key = ("prod", id(scale), id(index1), id(index2), id(seg), n_entries, dtype, str(device))
     return cached(anchor, key, build)

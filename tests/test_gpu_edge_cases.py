@@ -1,0 +1,121 @@
+"""Degenerate inputs through the public modules: an empty batch, a single row, a graph without edges, and modules
+converted to bfloat16 (their coefficient tables are then bfloat16 tensors too, as after ``module.to(dtype)`` in the
+reference).  An empty batch yields empty outputs and zero parameter gradients without a launch; reduced precision
+is computed in float32 and rounded once, so it agrees with the float32 module to bfloat16 rounding."""
+import pytest
+import torch
+
+from helpers import assert_close
+
+pytestmark = pytest.mark.gpu
+
+IRR, C = "0e+1o+2e", 32
+
+
+def _modules(device):
+    from equitorch_amd import nn as enn
+    from equitorch_amd.nn.functional import sincos
+
+    def angles(n, dt):
+        return tuple(sincos(torch.linspace(-2.0, 2.5, n, device=device).to(dt) * (k + 1), 2) for k in range(3))
+
+    return {
+        "LayerRMSNorm": (lambda: enn.LayerRMSNorm(IRR, C), lambda n, dt: ()),
+        "Gate": (lambda: enn.Gate(IRR, activation=None), lambda n, dt: (torch.randn(n, 3, C, device=device, dtype=dt),)),
+        "SquaredNorm": (lambda: enn.SquaredNorm(IRR), lambda n, dt: ()),
+        "Norm": (lambda: enn.Norm(IRR), lambda n, dt: ()),
+        "TensorDot": (lambda: enn.TensorDot(IRR, "uu"),
+                      lambda n, dt: (torch.randn(n, 9, C, device=device, dtype=dt),)),
+        "IrrepsLinear": (lambda: enn.IrrepsLinear(IRR, IRR, C, C), lambda n, dt: ()),
+        "IrrepWiseLinear": (lambda: enn.IrrepWiseLinear(IRR, C, C), lambda n, dt: ()),
+        "SO2Linear_uu": (lambda: enn.SO2Linear(IRR, IRR, C, C, feature_mode="uu"), lambda n, dt: ()),
+        "SO2Linear_uv": (lambda: enn.SO2Linear(IRR, IRR, C, C, feature_mode="uv"), lambda n, dt: ()),
+        "SparseWignerRotation": (lambda: enn.SparseWignerRotation(IRR), angles),
+        "SO3Linear_uu": (lambda: enn.SO3Linear(IRR, IRR, IRR, C, C, feature_mode="uu"),
+                         lambda n, dt: (torch.randn(n, 9, device=device, dtype=dt),)),
+        "SO3Linear_uv": (lambda: enn.SO3Linear(IRR, IRR, IRR, C, C, feature_mode="uv"),
+                         lambda n, dt: (torch.randn(n, 9, device=device, dtype=dt),)),
+        "TensorProduct_uuu": (lambda: enn.TensorProduct(IRR, IRR, IRR, C, C, C, feature_mode="uuu"),
+                              lambda n, dt: (torch.randn(n, 9, C, device=device, dtype=dt),)),
+    }
+
+
+NAMES = ["LayerRMSNorm", "Gate", "SquaredNorm", "Norm", "TensorDot", "IrrepsLinear", "IrrepWiseLinear", "SO2Linear_uu",
+         "SO2Linear_uv", "SparseWignerRotation", "SO3Linear_uu", "SO3Linear_uv", "TensorProduct_uuu"]
+
+
+def _run(mod, x, extra):
+    out = mod(x, *extra)
+    params = list(mod.parameters())
+    grads = torch.autograd.grad(out.float().sum(), [x] + params, allow_unused=True)
+    return out, grads[0], grads[1:]
+
+
+@pytest.mark.parametrize("name", NAMES)
+def test_empty_batch_and_single_row(device, name):
+    torch.manual_seed(0)
+    make, extra = _modules(device)[name]
+    mod = make().to(device)
+    x = torch.randn(0, 9, C, device=device, requires_grad=True)
+    out, gx, gparams = _run(mod, x, extra(0, torch.float32))
+    assert out.shape[0] == 0 and gx.shape == x.shape
+    for p, g in zip(mod.parameters(), gparams):
+        assert g is None or (g.shape == p.shape and not g.any()), "a sum over no rows must be zero"
+    # one row against the same row inside a batch of five
+    xs = torch.randn(5, 9, C, device=device, requires_grad=True)
+    ex = extra(5, torch.float32)
+    full, _, _ = _run(mod, xs, ex)
+    one, _, _ = _run(mod, xs[2:3].detach().requires_grad_(True), tuple(e[2:3] for e in ex))
+    assert_close(one, full[2:3], tol=1e-6, what=f"{name}: row alone vs in a batch")
+
+
+@pytest.mark.parametrize("name", NAMES)
+def test_module_converted_to_bfloat16(device, name):
+    torch.manual_seed(1)
+    make, extra = _modules(device)[name]
+    ref = make().to(device)
+    low = make().to(device)
+    low.load_state_dict(ref.state_dict())
+    low = low.to(torch.bfloat16)
+    n = 70
+    x = torch.randn(n, 9, C, device=device)
+    torch.manual_seed(2)
+    ex = extra(n, torch.float32)
+    exl = tuple(e.to(torch.bfloat16) for e in ex)
+    xl = x.to(torch.bfloat16).requires_grad_(True)
+    out, gx, _ = _run(low, xl, exl)
+    assert out.dtype == torch.bfloat16 and gx.dtype == torch.bfloat16
+    # the float32 module on the same (rounded) inputs and parameters
+    for p, q in zip(ref.parameters(), low.parameters()):
+        p.data.copy_(q.data.float())
+    xr = xl.detach().float().requires_grad_(True)
+    want, gwant, _ = _run(ref, xr, tuple(e.float() for e in exl))
+    assert_close(out.float(), want, tol=3e-2, what=f"{name} bf16 output")
+    assert_close(gx.float(), gwant, tol=3e-2, what=f"{name} bf16 grad_x")
+
+
+@pytest.mark.parametrize("n_nodes,n_edges", [(10, 0), (0, 0), (10, 1)])
+@pytest.mark.parametrize("vectors", [False, True])
+def test_graph_without_edges(device, n_nodes, n_edges, vectors):
+    from equitorch_amd import nn as enn
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu, edge_tensor_product_uu_vectors
+    torch.manual_seed(3)
+    tp = enn.SO3Linear(IRR, IRR, IRR, C, C, internal_weights=False, feature_mode="uu").to(device)
+    src = torch.randint(0, max(n_nodes, 1), (n_edges,), device=device)
+    dst = torch.randint(0, max(n_nodes, 1), (n_edges,), device=device)
+    plan = EdgePlan(src, dst, n_nodes)
+    x = torch.randn(n_nodes, 9, C, device=device, requires_grad=True)
+    w = torch.randn(n_edges, tp.num_paths, C, device=device, requires_grad=True)
+    if vectors:
+        y = torch.randn(n_edges, 3, device=device, requires_grad=True)
+        out = edge_tensor_product_uu_vectors(x, y, w, plan, tp.tp_info_forward)
+    else:
+        y = torch.randn(n_edges, 9, device=device, requires_grad=True)
+        out = edge_tensor_product_uu(x, y, w, plan, tp.tp_info_forward)
+    gx, gy, gw = torch.autograd.grad(out.sum(), [x, y, w])
+    assert out.shape == (n_nodes, 9, C) and gx.shape == x.shape and gy.shape == y.shape and gw.shape == w.shape
+    touched = torch.zeros(n_nodes, dtype=torch.bool, device=device)
+    touched[dst] = True
+    assert not out[~touched].any(), "nodes without incoming edges receive zero"
+    if n_edges == 0:
+        assert not gx.any()
