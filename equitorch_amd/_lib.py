@@ -79,6 +79,7 @@ def _load():
                                      C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_void_p]
     lib.cgtp_uvu_num_configs.restype = C.c_int
     lib.cgtp_uvu_find.argtypes = [C.c_uint64]
+    lib.cgtp_uvu_find_rounded.argtypes = [C.c_uint64, C.c_int]
     lib.cgtp_uvu_describe.restype = C.c_uint64
     lib.cgtp_uvu_describe.argtypes = [C.c_int, C.POINTER(C.c_int32)]
     lib.cgtp_uvu_sh_degree.argtypes = [C.c_int]
@@ -88,6 +89,7 @@ def _load():
     lib.cgtp_uvu_fwd.argtypes = [C.POINTER(UvuArgs), C.c_void_p]
     lib.cgtp_uvu_bwd.argtypes = [C.POINTER(UvuArgs), C.c_void_p]
     lib.cgtp_uv_find.argtypes = [C.c_uint64]
+    lib.cgtp_uv_find_rounded.argtypes = [C.c_uint64, C.c_int]
     _uv = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32,
            C.c_int32]
     lib.cgtp_uv_pack_weights.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32,

@@ -58,13 +58,28 @@ def tp_coo(tp_info) -> TpCoo:
                  int(tp_info.out_size), int(p.max()) + 1)
 
 
-def fingerprint(coo: TpCoo, dtype=np.float32) -> int:
-    """64-bit FNV-1a over dims, indices and the coefficient bits rounded to ``dtype``; identifies a
-    compiled-in table."""
+def round_coefficients(coef: np.ndarray, precision: str) -> np.ndarray:
+    """fp32 array of the coefficients as they read after ``tensor.to(precision)`` of the fp32 table:
+    ``'f32'`` (unchanged), ``'bf16'`` or ``'f16'`` (round to nearest even from fp32)."""
+    c32 = np.ascontiguousarray(coef, dtype=np.float32)
+    if precision == "f32":
+        return c32
+    if precision == "f16":
+        return c32.astype(np.float16).astype(np.float32)
+    if precision == "bf16":
+        u = c32.view(np.uint32).astype(np.uint64)
+        u = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+        return u.astype(np.uint32).view(np.float32)
+    raise ValueError(precision)
+
+
+def fingerprint(coo: TpCoo, precision: str = "f32") -> int:
+    """64-bit FNV-1a over dims, indices and the fp32 bits of the coefficients rounded to ``precision``; identifies
+    a compiled-in table (``'bf16'`` / ``'f16'``: the table of a module converted to that type)."""
     blob = b"".join([
         np.array([coo.D1, coo.D2, coo.DO, coo.P, coo.coef.shape[0]], dtype=np.int32).tobytes(),
         coo.M.tobytes(), coo.M1.tobytes(), coo.M2.tobytes(), coo.p.tobytes(),
-        coo.coef.astype(dtype).tobytes(),
+        round_coefficients(coo.coef, precision).tobytes(),
     ])
     h = 0xCBF29CE484222325
     for b in blob:

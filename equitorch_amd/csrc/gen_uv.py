@@ -226,10 +226,11 @@ def main(out_dir: str = None) -> str:
             chunks.append(emit_direction(name, d, coo, seg_out, seg_in1))
         chunks.append(emit_direction(name, 0, coo, seg_out, seg_in1, gy=True))
         chunks.append(emit_gw(name, coo, seg_out, seg_in1))
-        entries.append((name, fingerprint(coo)))
+        entries.append((name, fingerprint(coo), fingerprint(coo, "bf16"), fingerprint(coo, "f16")))
         chunks.append("")
     chunks.append("#define CGTP_FOREACH_UV_CONFIG(X) \\")
-    chunks.append(" \\\n".join(f"  X(UV_{n}_d0, UV_{n}_d1, UV_{n}_gy, UV_{n}_gw, 0x{fp:016x}ull, \"{n}\")" for n, fp in entries))
+    chunks.append(" \\\n".join(f"  X(UV_{n}_d0, UV_{n}_d1, UV_{n}_gy, UV_{n}_gw, 0x{fp:016x}ull, 0x{fb:016x}ull, 0x{fh:016x}ull, \"{n}\")"
+                              for n, fp, fb, fh in entries))
     chunks.append("")
     path = os.path.join(out_dir, "uv_configs.inc")
     text = "\n".join(chunks)

@@ -79,6 +79,8 @@ def emit_config(name: str, coo, sh_lmax: int = -1) -> str:
     a(f"struct TP_{name} {{")
     a(f"  static constexpr int D1 = {coo.D1}, D2 = {coo.D2}, DO = {coo.DO}, P = {coo.P}, NNZ = {T};")
     a(f"  static constexpr unsigned long long FINGERPRINT = 0x{fingerprint(coo):016x}ull;")
+    a(f"  static constexpr unsigned long long FINGERPRINT_BF16 = 0x{fingerprint(coo, 'bf16'):016x}ull;")
+    a(f"  static constexpr unsigned long long FINGERPRINT_F16 = 0x{fingerprint(coo, 'f16'):016x}ull;")
     a(f"  static constexpr const char* NAME = \"{name}\";")
     a(f"  static constexpr int SH_LMAX = {sh_lmax};  // second operand = harmonics of degrees 0..SH_LMAX (-1: not)")
     # ---- forward: o[M] += w[p] * sum_t (coef_t y[M2_t]) x[M1_t]

@@ -94,6 +94,8 @@ def emit_config(name: str, coo, seg_out) -> str:
     a(f"struct TPB_{name} {{")
     a(f"  static constexpr int D1 = {coo.D1}, D2 = {coo.D2}, DO = {coo.DO}, P = {coo.P}, NNZ = {T};")
     a(f"  static constexpr unsigned long long FINGERPRINT = 0x{fingerprint(coo):016x}ull;")
+    a(f"  static constexpr unsigned long long FINGERPRINT_BF16 = 0x{fingerprint(coo, 'bf16'):016x}ull;")
+    a(f"  static constexpr unsigned long long FINGERPRINT_F16 = 0x{fingerprint(coo, 'f16'):016x}ull;")
     a(f"  static constexpr const char* NAME = \"{name}\";")
 
     def ring_prologue():

@@ -404,6 +404,7 @@ using UvGwFn = void (*)(const __bf16*, const __bf16*, const __bf16*, float*, int
 
 struct UvEntry {
   uint64_t fingerprint;
+  uint64_t fingerprint_rounded[2];  // of the table rounded to bf16 / fp16 (a module converted to that type)
   const char* name;
   int din[2], dout[2], d2, p;
   UvFn fn[3][3];  // [direction 0, direction 1, grad y][C_in = 32, 64, 128]
@@ -413,9 +414,9 @@ struct UvEntry {
 };
 
 template <class D0, class D1, class GY, class GW>
-static UvEntry make_uv_entry(uint64_t fp, const char* name) {
+static UvEntry make_uv_entry(uint64_t fp, uint64_t fp_bf16, uint64_t fp_f16, const char* name) {
   UvEntry e;
-  e.fingerprint = fp; e.name = name;
+  e.fingerprint = fp; e.fingerprint_rounded[0] = fp_bf16; e.fingerprint_rounded[1] = fp_f16; e.name = name;
   e.din[0] = D0::DIN; e.dout[0] = D0::DOUT; e.din[1] = D1::DIN; e.dout[1] = D1::DOUT;
   e.d2 = D0::D2; e.p = D0::P;
   e.fn[0][0] = uv_kernel<D0, 32>; e.fn[0][1] = uv_kernel<D0, 64>; e.fn[0][2] = uv_kernel<D0, 128>;
@@ -438,7 +439,7 @@ static UvEntry make_uv_entry(uint64_t fp, const char* name) {
 }
 
 static const UvEntry* uv_entries(int* count) {
-#define CGTP_X(D0, D1, GY, GW, FP, NAME) make_uv_entry<D0, D1, GY, GW>(FP, NAME),
+#define CGTP_X(D0, D1, GY, GW, FP, FP_BF16, FP_F16, NAME) make_uv_entry<D0, D1, GY, GW>(FP, FP_BF16, FP_F16, NAME),
   static const UvEntry table[] = {CGTP_FOREACH_UV_CONFIG(CGTP_X)};
 #undef CGTP_X
   *count = (int)(sizeof(table) / sizeof(table[0]));
@@ -480,6 +481,15 @@ int cgtp_uv_find(uint64_t fingerprint) {
   const UvEntry* t = uv_entries(&n);
   for (int i = 0; i < n; ++i)
     if (t[i].fingerprint == fingerprint) return i;
+  return -1;
+}
+
+int cgtp_uv_find_rounded(uint64_t fingerprint, int dtype) {
+  if (dtype != CGTP_BF16 && dtype != CGTP_F16) return -1;
+  int n = 0;
+  const UvEntry* t = uv_entries(&n);
+  for (int i = 0; i < n; ++i)
+    if (t[i].fingerprint_rounded[dtype == CGTP_F16] == fingerprint) return i;
   return -1;
 }
 

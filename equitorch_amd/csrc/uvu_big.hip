@@ -95,6 +95,7 @@ template <class TP>
 static UvuBigEntry make_big_entry() {
   UvuBigEntry e;
   e.fingerprint = TP::FINGERPRINT;
+  e.fingerprint_rounded[0] = TP::FINGERPRINT_BF16; e.fingerprint_rounded[1] = TP::FINGERPRINT_F16;
   e.dims[0] = TP::D1; e.dims[1] = TP::D2; e.dims[2] = TP::DO; e.dims[3] = TP::P; e.dims[4] = TP::NNZ;
   e.name = TP::NAME;
   e.fwd = uvu_big_fwd_kernel<TP>;

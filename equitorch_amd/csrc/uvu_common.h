@@ -63,6 +63,7 @@ enum { kGwNone = 0, kGwStore = 1, kGwReduce = 2 };
 // for a shared weight the caller sums the rows.
 struct UvuBigEntry {
   uint64_t fingerprint;
+  uint64_t fingerprint_rounded[2];  // of the table rounded to bf16 / fp16
   int dims[5];
   const char* name;
   void (*fwd)(const UvuDev<float>);

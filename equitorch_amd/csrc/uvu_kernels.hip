@@ -442,6 +442,7 @@ using WaveFn = void (*)(const UvuDev<T>, int64_t);
 template <typename T>
 struct UvuEntry {
   uint64_t fingerprint;
+  uint64_t fingerprint_rounded[2];  // of the table rounded to bf16 / fp16 (a module converted to that type)
   int dims[5];
   const char* name;
   int v_fwd, v_bwd;         // channels per lane of the vector paths
@@ -473,6 +474,7 @@ static UvuEntry<T> make_entry() {
   constexpr int VF = v_fwd<TP, T>(), VB = v_bwd<TP, T>();
   UvuEntry<T> e;
   e.fingerprint = TP::FINGERPRINT;
+  e.fingerprint_rounded[0] = TP::FINGERPRINT_BF16; e.fingerprint_rounded[1] = TP::FINGERPRINT_F16;
   e.dims[0] = TP::D1; e.dims[1] = TP::D2; e.dims[2] = TP::DO; e.dims[3] = TP::P; e.dims[4] = TP::NNZ;
   e.name = TP::NAME;
   e.v_fwd = VF; e.v_bwd = VB;
@@ -761,6 +763,19 @@ int cgtp_uvu_find(uint64_t fingerprint) {
     if (t[i].fingerprint == fingerprint) return i;
   for (int i = 0; i < n_big; ++i)
     if (b[i].fingerprint == fingerprint) return n + i;
+  return -1;
+}
+
+int cgtp_uvu_find_rounded(uint64_t fingerprint, int dtype) {
+  if (dtype != CGTP_BF16 && dtype != CGTP_F16) return -1;
+  const int k = dtype == CGTP_F16;
+  int n = 0, n_big = 0;
+  const UvuEntry<float>* t = entries<float>(&n);
+  const UvuBigEntry* b = uvu_big_entries(&n_big);
+  for (int i = 0; i < n; ++i)
+    if (t[i].fingerprint_rounded[k] == fingerprint) return i;
+  for (int i = 0; i < n_big; ++i)
+    if (b[i].fingerprint_rounded[k] == fingerprint) return n + i;
   return -1;
 }
 

@@ -8,14 +8,11 @@ from torch import Tensor
 from torch.autograd import Function
 
 from ... import _lib
-from ..._tables import fingerprint
 from ...ops import kernels
 from ._tri import spec_from_tp_info, tri
 
 
-def uv_config_of(tp_info) -> int:
-    return kernels.cached(tp_info.info_Mij_fwd.scale, "uv_cfg",
-                          lambda: int(_lib.lib.cgtp_uv_find(C.c_uint64(fingerprint(kernels.coo_of(tp_info))))))
+uv_config_of = kernels.uv_config_of
 
 
 _packed = {}  # (id(w), direction) -> (weakref to w, its version counter, its data pointer, packed copy)

@@ -38,10 +38,28 @@ def coo_of(tp_info) -> TpCoo:
     return cached(tp_info.info_Mij_fwd.scale, "coo", lambda: tp_coo(tp_info))
 
 
+_ROUNDED = {torch.bfloat16: ("bf16", 2), torch.float16: ("f16", 3)}     # precision name, dtype code of the library
+
+
+def _find_config(tp_info, find, find_rounded) -> int:
+    scale = tp_info.info_Mij_fwd.scale
+    if scale.dtype in _ROUNDED:      # table of a module converted to reduced precision
+        name, code = _ROUNDED[scale.dtype]
+        return int(find_rounded(C.c_uint64(fingerprint(coo_of(tp_info), name)), code))
+    return int(find(C.c_uint64(fingerprint(coo_of(tp_info)))))
+
+
 def uvu_config_of(tp_info) -> int:
-    """Index of the compiled-in table equal to this ``tp_info`` (fp32 coefficient bits), or -1."""
+    """Index of the compiled-in table equal to this ``tp_info`` (fp32 coefficient bits; for a bf16 / fp16 table:
+    equal after rounding the compiled coefficients to that type), or -1."""
     return cached(tp_info.info_Mij_fwd.scale, "cfg",
-                  lambda: int(_lib.lib.cgtp_uvu_find(C.c_uint64(fingerprint(coo_of(tp_info))))))
+                  lambda: _find_config(tp_info, _lib.lib.cgtp_uvu_find, _lib.lib.cgtp_uvu_find_rounded))
+
+
+def uv_config_of(tp_info) -> int:
+    """The same among the tables of the fully connected product on the matrix cores."""
+    return cached(tp_info.info_Mij_fwd.scale, "uv_cfg",
+                  lambda: _find_config(tp_info, _lib.lib.cgtp_uv_find, _lib.lib.cgtp_uv_find_rounded))
 
 
 # ---- operands ---------------------------------------------------------------------------------------------

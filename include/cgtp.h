@@ -154,6 +154,10 @@ int cgtp_segment_sum(const void* in, const void* scale, const int64_t* index, co
  */
 int cgtp_uvu_num_configs(void);
 int cgtp_uvu_find(uint64_t fingerprint);
+/* The same for the table of a module converted to reduced precision (reference: TensorProductInfo._apply moves
+ * the coefficient tensors with the module, equitorch/structs/__init__.py:7-102): `fingerprint` is taken over the
+ * coefficients as they read in `dtype` (CGTP_BF16 | CGTP_F16); matches the config whose fp32 table rounds to them. */
+int cgtp_uvu_find_rounded(uint64_t fingerprint, int dtype);
 /* Describes config `cfg`: dims (D1, D2, DO, P, NNZ) written to dims[5]; returns its fingerprint (0 if bad). */
 uint64_t cgtp_uvu_describe(int cfg, int32_t* dims);
 /* Degree L if the second operand of config `cfg` is laid out like harmonics of degrees 0..L and the fused
@@ -226,6 +230,8 @@ int cgtp_uvu_bwd(const cgtp_uvu_args* args, void* stream);
  */
 int cgtp_uv_num_configs(void);
 int cgtp_uv_find(uint64_t fingerprint);
+/* As cgtp_uvu_find_rounded, for the fully connected product. */
+int cgtp_uv_find_rounded(uint64_t fingerprint, int dtype);
 int cgtp_uv_pack_weights(int direction, const void* w, void* packed, int32_t n_paths, int32_t cin, int32_t cout,
                          int32_t dtype, void* stream);
 int cgtp_uv_validate(int cfg, int direction, const void* x, const void* y, const void* wp, const void* out,

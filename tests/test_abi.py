@@ -192,3 +192,36 @@ def test_cpu_tensors_are_rejected_loudly():
     m = SO3Linear("0e+1o", "0e+1o", "0e+1o", 4, 4)
     with pytest.raises(_lib.CgtpError, match="GPU only"):
         m(torch.randn(2, 4, 4), torch.randn(2, 4))
+
+
+def test_tables_of_a_module_in_reduced_precision_find_their_config():
+    """``module.to(torch.bfloat16)`` moves the coefficient tables too; such a table matches the compiled config whose
+    fp32 coefficients round to it (cgtp_uvu_find_rounded / cgtp_uv_find_rounded), and only that one."""
+    import torch
+    from equitorch_amd import _lib
+    from equitorch_amd._tables import fingerprint, round_coefficients, tp_coo
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.ops import kernels
+    from equitorch_amd.utils import tp_infos
+    L = _lib.lib
+    # the rounding is torch's
+    c = torch.randn(1000, dtype=torch.float64).numpy()
+    for name, dt in (("bf16", torch.bfloat16), ("f16", torch.float16)):
+        want = torch.from_numpy(c).float().to(dt).float().numpy()
+        assert (round_coefficients(c, name) == want).all()
+    for irreps, find, find_rounded, of in (
+            ("0e+1o+2e", L.cgtp_uvu_find, L.cgtp_uvu_find_rounded, kernels.uvu_config_of),
+            ("0e+1o+2e+3o", L.cgtp_uv_find, L.cgtp_uv_find_rounded, kernels.uv_config_of)):
+        irr = Irreps(irreps)
+        info = tp_infos(irr, irr, irr)[0]
+        cfg = find(C.c_uint64(fingerprint(tp_coo(info))))
+        assert cfg >= 0
+        for name, dt, code in (("bf16", torch.bfloat16, _lib.BF16), ("f16", torch.float16, 3)):
+            low = info._apply(lambda t: t.to(dt) if t.is_floating_point() else t)
+            assert low.info_Mij_fwd.scale.dtype == dt
+            fp = fingerprint(tp_coo(low), name)
+            assert fp == fingerprint(tp_coo(info), name) != fingerprint(tp_coo(info))
+            assert find_rounded(C.c_uint64(fp), code) == cfg == of(low)
+            assert find(C.c_uint64(fp)) == -1                            # not an fp32 table
+            assert find_rounded(C.c_uint64(fp), _lib.F32) == -1
+        assert find_rounded(C.c_uint64(fingerprint(tp_coo(info), "bf16")), 3) == -1

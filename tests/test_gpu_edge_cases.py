@@ -119,3 +119,36 @@ def test_graph_without_edges(device, n_nodes, n_edges, vectors):
     assert not out[~touched].any(), "nodes without incoming edges receive zero"
     if n_edges == 0:
         assert not gx.any()
+
+
+def test_converted_module_runs_on_the_compiled_kernels(device):
+    """``SO3Linear(..., 'uv').to(torch.bfloat16)`` carries bfloat16 tables; they still select the matrix-core
+    kernels, and the result agrees with the float32 module on the same rounded operands."""
+    from equitorch_amd import nn as enn
+    from equitorch_amd.nn.functional import _uvw_mfma
+    from equitorch_amd.ops import kernels
+    torch.manual_seed(4)
+    irr, c, n = "0e+1o+2e+3o", 64, 300
+    ref = enn.SO3Linear(irr, irr, irr, c, c, feature_mode="uv").to(device)
+    low = enn.SO3Linear(irr, irr, irr, c, c, feature_mode="uv").to(device)
+    low.load_state_dict(ref.state_dict())
+    low = low.to(torch.bfloat16)
+    assert low.tp_info_forward.info_Mij_fwd.scale.dtype == torch.bfloat16
+    assert kernels.uv_config_of(low.tp_info_forward) == kernels.uv_config_of(ref.tp_info_forward) >= 0
+    x = torch.randn(n, 16, c, device=device).bfloat16().requires_grad_(True)
+    y = torch.randn(n, 16, device=device).bfloat16().requires_grad_(True)
+    assert _uvw_mfma.try_forward(x, y, low.weight, low.tp_info_forward) is not None
+    out = low(x, y)
+    ct = torch.randn_like(out)
+    grads = torch.autograd.grad(out, [x, y, low.weight], ct)
+    with torch.no_grad():
+        ref.weight.copy_(low.weight.float())
+    xr, yr = x.detach().float().requires_grad_(True), y.detach().float().requires_grad_(True)
+    want = ref(xr, yr)
+    gwant = torch.autograd.grad(want, [xr, yr, ref.weight], ct.float())
+    assert_close(out.float(), want, tol=2e-2, what="bf16 module output")
+    for name, a, b in zip(("grad_x", "grad_y", "grad_w"), grads, gwant):
+        assert_close(a.float(), b, tol=2e-2, what=name)
+    # the channel-wise product of a float16 module finds its compiled table as well
+    half = enn.SO3Linear("0e+1o+2e", "0e+1o+2e", "0e+1o+2e", c, c, feature_mode="uu").to(device).half()
+    assert kernels.uvu_config_of(half.tp_info_forward) >= 0
