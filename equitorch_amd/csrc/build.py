@@ -19,7 +19,7 @@ LIB_PATH = os.path.join(LIB_DIR, "libcgtp.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
-    "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-ffp-contract=off",
+    "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-ffp-contract=fast",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
     f"-I{os.path.join(ROOT, 'include')}", f"-I{HERE}",

@@ -2,19 +2,22 @@
 launches of every registered configuration and for configurations whose table is too large for the
 register-resident bodies of ``gen_uvu`` (hundreds of weight rows, thousands of coefficients).
 
-One lane owns one channel.  The bodies walk the table output irrep by output irrep (only the 2l+1 rows of that
-irrep are live as accumulators or gradient rows) and inside an irrep path by path.  A path's weight is a single
+One lane owns one channel.  The forward walks the table output irrep by output irrep (only the 2l+1 accumulator
+rows of that irrep are live), the backward input irrep by input irrep (only that irrep's rows of x and grad_x are
+live, next to all of y, grad_y and grad_out: at lmax = 6 that is 173 registers instead of 209 for the walk by
+output irrep, and the body needs no scratch memory), inside an irrep path by path.  A path's weight is a single
 register, taken from a ring of ``RING`` registers that is refilled ``RING`` paths ahead so that the per-row weight
 stream never waits for memory.  Per path the forward evaluates
 
     t = y[b] * x[a]   once per (a, b) pair,      i[M] += coef * t,      o[M] += w[p] * i[M]
 
-and the backward, with ``u[M] = w[p] * g[M]``,
+and the backward contracts the coefficients with the rows of ``grad_out`` first, once per (a, b) pair,
 
-    gw[p] = sum_M i[M] * g[M]        gx[a] += coef * (y[b] * u[M])        gy[b] += coef * (x[a] * u[M])
+    v = sum_M coef * g[M]        s[a] += y[b] * v        gy[b] += (w[p] * x[a]) * v
+    gw[p] = sum_a x[a] * s[a]    gx[a] += w[p] * s[a]
 
-the pair products again formed once per pair.  Every index is a literal and every coefficient the hexadecimal
-literal of the fp32 table value.
+so that a coefficient costs one instruction and a pair two (the forward intermediate is not rebuilt).  Every
+index is a literal and every coefficient the hexadecimal literal of the fp32 table value.
 """
 from __future__ import annotations
 
@@ -75,7 +78,7 @@ def _grouped(terms, key):
     return d
 
 
-def emit_config(name: str, coo, seg_out) -> str:
+def emit_config(name: str, coo, seg_out, seg_in1) -> str:
     T = coo.coef.shape[0]
     term = [(int(coo.p[t]), int(coo.M[t]), int(coo.M1[t]), int(coo.M2[t]), _lit(coo.coef[t])) for t in range(T)]
     # execution order: output irrep blocks, inside a block the paths in table order
@@ -144,47 +147,54 @@ def emit_config(name: str, coo, seg_out) -> str:
     a("  }")
 
     # ---- backward --------------------------------------------------------------------------------------------
-    a("  // gload(M): this lane's channel of row M of grad_out; gwsink(p, v): gradient of weight path p;")
-    a("  // gx / gy: accumulated in place (gy holds this lane's channel only, the caller sums over channels)")
-    a("  template <class WLoad, class GLoad, class GwSink>")
-    a("  __device__ __forceinline__ static void bwd(const float (&x)[D1], const float (&y)[D2], WLoad&& wload,")
-    a("                                             GLoad&& gload, float (&gx)[D1], float (&gy)[D2],")
+    # Walks the table input irrep by input irrep: of x and grad_x only the 2l+1 rows of the current irrep are
+    # live (and the next irrep's rows of x, requested one block ahead); y, grad_y and grad_out stay whole.
+    blocks_in = []
+    for b0, b1 in zip(seg_in1[:-1], seg_in1[1:]):
+        paths = sorted({p for p, _, aa, _, _ in term if b0 <= aa < b1})
+        if paths:
+            blocks_in.append((list(range(b0, b1)), paths))
+    order = [p for _, paths in blocks_in for p in paths]
+    assert sorted(order) == list(range(coo.P))
+    pos = {p: k for k, p in enumerate(order)}
+    a("  // xload(a): this lane's channel of row a of x; wload(p): of weight path p; g: the rows of grad_out;")
+    a("  // gxstore(a, v): a finished row of grad_x; gwsink(p, v): gradient of weight path p; gy: accumulated in place")
+    a("  // (this lane's channel only, the caller sums over channels)")
+    a("  template <class XLoad, class WLoad, class GxStore, class GwSink>")
+    a("  __device__ __forceinline__ static void bwd(XLoad&& xload, const float (&y)[D2], WLoad&& wload,")
+    a("                                             const float (&g)[DO], GxStore&& gxstore, float (&gy)[D2],")
     a("                                             GwSink&& gwsink) {")
-    a("    float yy[D2], xx[D1];")
+    a("    float yy[D2], gg[DO];")
     a("    for (int j = 0; j < D2; ++j) yy[j] = y[j];")
-    a("    for (int j = 0; j < D1; ++j) xx[j] = x[j];")
+    a("    for (int j = 0; j < DO; ++j) gg[j] = g[j];")
     ring_prologue()
-    for M in blocks[0][0]:
-        a(f"    const float g{M} = gload({M});")
-    for bi, (rows, paths) in enumerate(blocks):
-        if bi + 1 < len(blocks):  # rows of the next irrep are requested one block ahead
-            for M in blocks[bi + 1][0]:
-                a(f"    const float g{M} = gload({M});")
+    for aa in blocks_in[0][0]:
+        a(f"    float x{aa} = xload({aa});")
+    for bi, (rows, paths) in enumerate(blocks_in):
+        if bi + 1 < len(blocks_in):
+            for aa in blocks_in[bi + 1][0]:
+                a(f"    float x{aa} = xload({aa});")
         a("    {")
+        a("      float " + ", ".join(f"gx{aa} = 0.f" for aa in rows) + ";")
         for p in paths:
             ts_p = by_path[p]
-            ms = sorted({M for _, M, _, _, _ in ts_p})
             a("      {")
             ring_take(p)
             opaque({b for _, _, _, b, _ in ts_p})
-            a("      " + " ".join(f'asm volatile("" : "+v"(xx[{m}]));' for m in sorted({t[2] for t in ts_p})))
-            a("      float " + ", ".join(f"i{M}" for M in ms) + ";")
-            a("      " + " ".join(f"const float u{M} = w * g{M};" for M in ms))
-            seen = set()
-            for (aa, b), ts in _grouped(ts_p, lambda t: (t[2], t[3])).items():
-                ops = []
-                for _, M, _, _, c in ts:
-                    ops.append(f"i{M} {'+=' if M in seen else '='} {c} * t;")
-                    seen.add(M)
-                a(f"      {{ const float t = yy[{b}] * xx[{aa}]; " + " ".join(ops) + " }")
-            a(f"      gwsink({p}, " + " + ".join(f"i{M} * g{M}" for M in ms) + ");")
-            for (b, M), ts in _grouped(ts_p, lambda t: (t[3], t[1])).items():
-                a(f"      {{ const float t = yy[{b}] * u{M}; " + " ".join(f"gx[{aa}] += {c} * t;" for _, _, aa, _, c in ts) + " }")
-            a("      " + _pin(f"gx[{m}]" for m in sorted({t[2] for t in ts_p})))
-            for (aa, M), ts in _grouped(ts_p, lambda t: (t[2], t[1])).items():
-                a(f"      {{ const float t = xx[{aa}] * u{M}; " + " ".join(f"gy[{b}] += {c} * t;" for _, _, _, b, c in ts) + " }")
-            a("      " + _pin(f"gy[{m}]" for m in sorted({t[3] for t in ts_p})))
+            a("      " + " ".join(f'asm volatile("" : "+v"(gg[{m}]));' for m in sorted({t[1] for t in ts_p})))
+            a("      float gwp;")
+            for ai, (aa, ts_a) in enumerate(_grouped(ts_p, lambda t: t[2]).items()):
+                a(f"      {{ const float xw = w * x{aa}; float s;")
+                for bi_, (b, ts) in enumerate(_grouped(ts_a, lambda t: t[3]).items()):
+                    v = " + ".join(f"{c} * gg[{M}]" for _, M, _, _, c in ts)
+                    pins = f' asm volatile("" : "+v"(s), "+v"(gy[{b}]));'
+                    a(f"        {{ const float v = {v}; s {'+=' if bi_ else '='} yy[{b}] * v; gy[{b}] += xw * v;{pins} }}")
+                a(f"        gwp {'+=' if ai else '='} x{aa} * s; gx{aa} += w * s; }}")
+            a(f"      gwsink({p}, gwp);")
+            a("      " + _pin(f"gx{m}" for m in sorted({t[2] for t in ts_p})))
             a("      }")
+        for aa in rows:
+            a(f"      gxstore({aa}, gx{aa});")
         a("    }")
     a("  }")
     a("};")
@@ -205,7 +215,7 @@ def main(out_dir: str = None) -> str:
             raise ValueError(f"configuration {name} has the same table as {seen[fp]}")
         seen[fp] = name
         chunks.append(f"// {name}: {i1} x {i2} -> {io}")
-        chunks.append(emit_config(name, coo, irrep_segments(Irreps(io))))
+        chunks.append(emit_config(name, coo, irrep_segments(Irreps(io)), irrep_segments(Irreps(i1))))
         chunks.append("")
     chunks.append("#define CGTP_FOREACH_UVU_BIG_CONFIG(X) \\")
     chunks.append(" \\\n".join(f"  X(TPB_{n})" for n in configs))

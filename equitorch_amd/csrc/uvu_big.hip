@@ -50,32 +50,32 @@ __global__ void __launch_bounds__(256, 2) uvu_big_bwd_kernel(const UvuDev<float>
   const int c = min(L.cl, a.C - 1);
   const int64_t gr = a.gather ? a.gather[r] : r;
   const int64_t xr = a.x_gather ? a.x_gather[r] : r;
-  float x[D1], y[D2], gx[D1], gy[D2];
+  float y[D2], gy[D2], g[DO];
 #pragma unroll
   for (int j = 0; j < D2; ++j) {
     y[j] = YC ? a.y[(r * D2 + j) * C + c] : a.y[r * D2 + j];
     gy[j] = 0.f;
   }
-#pragma unroll
-  for (int i = 0; i < D1; ++i) {
-    x[i] = a.x[(xr * D1 + i) * C + c];
-    gx[i] = 0.f;
-  }
-  const float* wrow = a.w + (a.w_shared ? 0 : r) * P * C + c;
   const float* grow = a.g + gr * DO * C + c;
+#pragma unroll
+  for (int m = 0; m < DO; ++m) g[m] = grow[m * C];
+  const float* xrow = a.x + xr * D1 * C + c;
+  const float* wrow = a.w + (a.w_shared ? 0 : r) * P * C + c;
   float* gwrow = a.gw + r * P * C + c;
+  float* gxrow = a.gx + r * D1 * C + c;
+  const bool gx_live = a.gx && live;
   TP::bwd(
-      x, y, [&](int p) __attribute__((always_inline)) { return __builtin_nontemporal_load(wrow + p * C); },
-      [&](int m) __attribute__((always_inline)) { return grow[m * C]; }, gx, gy,
+      [&](int i) __attribute__((always_inline)) { return xrow[i * C]; }, y,
+      [&](int p) __attribute__((always_inline)) { return __builtin_nontemporal_load(wrow + p * C); }, g,
+      [&](int i, float v) __attribute__((always_inline)) {
+        if (gx_live) __builtin_nontemporal_store(v, gxrow + i * C);
+      },
+      gy,
       [&](int p, float v) __attribute__((always_inline)) {
         if constexpr (GW == kGwStore) {
           if (live) __builtin_nontemporal_store(v, gwrow + p * C);
         }
       });
-  if (a.gx && live) {
-#pragma unroll
-    for (int i = 0; i < D1; ++i) __builtin_nontemporal_store(gx[i], a.gx + (r * D1 + i) * C + c);
-  }
   if (YC) {
     if (a.gy && live) {
 #pragma unroll
