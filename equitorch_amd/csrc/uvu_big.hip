@@ -45,9 +45,10 @@ __global__ void __launch_bounds__(256, 2) uvu_big_bwd_kernel(const UvuDev<float>
   if (wave >= n_waves) return;
   const int64_t C = a.C;
   const int64_t r_raw = wave * L.slots + L.slot;
-  const bool row_ok = r_raw < a.n_rows, live = row_ok && L.cl < a.C;
+  const int c_raw = blockIdx.y * L.lpe + L.cl;  // rows wider than one wavefront: one channel chunk per blockIdx.y
+  const bool row_ok = r_raw < a.n_rows, live = row_ok && c_raw < a.C;
   const int64_t r = min(r_raw, a.n_rows - 1);
-  const int c = min(L.cl, a.C - 1);
+  const int c = min(c_raw, a.C - 1);
   const int64_t gr = a.gather ? a.gather[r] : r;
   const int64_t xr = a.x_gather ? a.x_gather[r] : r;
   float y[D2], gy[D2], g[DO];
@@ -82,11 +83,13 @@ __global__ void __launch_bounds__(256, 2) uvu_big_bwd_kernel(const UvuDev<float>
       for (int j = 0; j < D2; ++j) __builtin_nontemporal_store(gy[j], a.gy + (r * D2 + j) * C + c);
     }
   } else if (a.gy) {
-    const float keep = L.cl < a.C ? 1.f : 0.f;  // duplicate channels of the padding lanes do not count
+    const float keep = c_raw < a.C ? 1.f : 0.f;  // duplicate channels of the padding lanes do not count
+    // several channel chunks: each writes its partial sums to the workspace, the host sums them in chunk order
+    float* gyrow = (gridDim.y > 1 ? a.ws + (int64_t)blockIdx.y * a.n_rows * D2 : a.gy) + r * D2;
 #pragma unroll
     for (int j = 0; j < D2; ++j) {
       const float s = group_sum(gy[j] * keep, L.lpe);
-      if (row_ok && L.cl == (j & (L.lpe - 1))) a.gy[r * D2 + j] = s;
+      if (row_ok && L.cl == (j & (L.lpe - 1))) gyrow[j] = s;
     }
   }
 }

@@ -535,10 +535,9 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
   if (a->cfg < 0 || a->cfg >= n_cfg + n_big) return CGTP_ERR_CONFIG;
   const bool seg_mode = a->n_seg > 0;
   // The block-wise kernels (one channel per lane) serve the configurations that have no register-resident body
-  // (indices n_cfg and up) and, because they are faster there, every fp32 row-mode launch of the others except
-  // backward launches wider than one wavefront (C > 64).
+  // (indices n_cfg and up) and, because they are faster there, every fp32 row-mode launch of the others.
   int big_idx = a->cfg >= n_cfg ? a->cfg - n_cfg : -1;
-  if (big_idx < 0 && a->dtype == CGTP_F32 && !seg_mode && !(backward && a->C > kWave)) {
+  if (big_idx < 0 && a->dtype == CGTP_F32 && !seg_mode) {
     for (int i = 0; i < n_big; ++i)
       if (big_tab[i].fingerprint == tab[a->cfg].fingerprint) big_idx = i;
   }
@@ -551,7 +550,6 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
         if (big_tab[i].fingerprint == tab[a->cfg].fingerprint) big_idx = i;
     }
     if (big_idx < 0) return CGTP_ERR_CONFIG;
-    if (backward && a->C > kWave) return CGTP_ERR_SHAPE;
   }
   const bool big = big_idx >= 0;
   plan->big_idx = big_idx;
@@ -605,7 +603,8 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
   while ((1 << lg) < lanes && lg < 6) ++lg;
   plan->lpe_log2 = lg;
   // channel reduction of grad_y and the segment accumulators stay inside one slot
-  if ((backward || seg) && lanes > kWave) return CGTP_ERR_SHAPE;
+  // (the block-wise kernels cut wider rows into chunks of one wavefront and sum grad_y over the chunks afterwards)
+  if (!big && (backward || seg) && lanes > kWave) return CGTP_ERR_SHAPE;
   const int slots = kWave >> lg;
   const int64_t row_d = backward ? dims[0] : dims[2];
   const bool wred = backward && a->w_shared && a->grad_w;
@@ -621,8 +620,11 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
     if (!backward || a->grad_x) plan->ws_elems = plan->n_waves * 2 * row_d * a->C;
   } else {
     int64_t nw = (a->n_rows + slots - 1) / slots;
-    if (wred && nw > kMaxRowWaves) nw = kMaxRowWaves;
+    if (wred && !big && nw > kMaxRowWaves) nw = kMaxRowWaves;  // the block-wise kernels take one pass per wavefront
     plan->n_waves = nw;
+    // block-wise backward wider than one wavefront: grad_y partials of every channel chunk, summed afterwards
+    if (big && backward && a->grad_y && !a->y_channels && a->C > kWave)
+      plan->ws_elems = (int64_t)((a->C + kWave - 1) / kWave) * a->n_rows * dims[1];
   }
   if (wred && big) {
     // block-wise kernels write the weight gradient of every row; two summation passes follow (kSumRows rows
@@ -677,8 +679,15 @@ static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward,
   UvuDev<float> d = to_dev<float>(a, plan);
   if (backward) {
     if (wred) d.gw = d.wsw;  // per-row gradients into the workspace, summed below
+    const int chunk = 1 << plan.lpe_log2;
+    const int64_t c_chunks = (a->C + chunk - 1) / chunk;
     hipLaunchKernelGGL((a->y_channels ? e.bwd_yc : e.bwd)[a->grad_w ? kGwStore : kGwNone],
-                       dim3((unsigned)((plan.n_waves + 3) / 4)), dim3(256), 0, stream, d, plan.n_waves);
+                       dim3((unsigned)((plan.n_waves + 3) / 4), (unsigned)c_chunks), dim3(256), 0, stream, d,
+                       plan.n_waves);
+    if (plan.ws_elems > 0) {  // grad_y: fixed-order sum of the channel chunks' partials
+      if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
+      launch_partial_sum<float>((const float*)d.ws, (float*)a->grad_y, c_chunks, a->n_rows * e.dims[1], stream);
+    }
     if (wred) {
       if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
       const int64_t chunks = (a->n_rows + kSumRows - 1) / kSumRows;

@@ -196,12 +196,13 @@ typedef struct cgtp_uvu_args {
   void* grad_x;            /* (n_seg ? n_seg : n_rows, D1, C) or NULL                              */
   void* grad_y;            /* (n_rows, D2), (n_rows, 3) if y_vec, or NULL                          */
   void* grad_w;            /* (n_rows | 1, P, C) or NULL                                           */
-  void* workspace;         /* cgtp_uvu_workspace_bytes() bytes (segment mode, or bwd of a shared W) */
+  void* workspace;         /* cgtp_uvu_workspace_bytes() bytes (segment mode, bwd of a shared W, fp32 row-mode
+                              bwd with grad_y and C > 64)                                          */
   const int64_t* x_gather; /* row mode backward, optional: [n_rows] row of x of every batch row (x then has
                               n_x_rows rows; grad_x stays per batch row, (n_rows, D1, C))              */
   int32_t y_channels;      /* row mode, fp32: 1 = y and grad_y carry channels, (n_rows, D2, C): the "uuu" product
                               TensorProductUUUDummy (equitorch/nn/functional/tensor_products.py:9-90), on the
-                              block-wise kernels; backward needs C <= 64                               */
+                              block-wise kernels                                                     */
   int32_t reserved_;
 } cgtp_uvu_args;
 

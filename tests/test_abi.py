@@ -69,7 +69,12 @@ def test_host_side_validation_codes():
     a.n_x_rows, a.C = 10, 512
     assert L.cgtp_uvu_validate(C.byref(a), 0) == 0                  # forward tiles channels over the grid
     a.grad_out = 256
-    assert L.cgtp_uvu_validate(C.byref(a), 1) == 2                  # backward keeps a row inside one wavefront
+    assert L.cgtp_uvu_validate(C.byref(a), 1) == 0                  # fp32 row mode: so does the backward ...
+    a.grad_y = 256
+    assert L.cgtp_uvu_workspace_bytes(C.byref(a), 1) == 8 * 10 * 9 * 4  # ... with grad_y partials of 8 channel chunks
+    a.dtype = _lib.F64
+    assert L.cgtp_uvu_validate(C.byref(a), 1) == 2                  # fp64 backward keeps a row inside one wavefront
+    a.dtype, a.grad_y = _lib.F32, None
     a.C, a.w_shared, a.grad_w = 64, 1, 256
     # fp32 row mode runs on the block-wise kernels: 10 per-row weight gradients + 1 chunk partial of (P, C)
     assert L.cgtp_uvu_workspace_bytes(C.byref(a), 1) == (10 + 1) * 11 * 64 * 4
@@ -131,7 +136,7 @@ def test_large_table_configs_and_row_gathers_validate_on_the_host():
     b.x = b.y = b.w = b.out = b.grad_out = b.grad_x = b.grad_y = b.grad_w = 4096
     assert L.cgtp_uvu_validate(C.byref(b), 0) == 0 and L.cgtp_uvu_validate(C.byref(b), 1) == 0
     b.C = 128
-    assert L.cgtp_uvu_validate(C.byref(b), 0) == 0 and L.cgtp_uvu_validate(C.byref(b), 1) == 2
+    assert L.cgtp_uvu_validate(C.byref(b), 0) == 0 and L.cgtp_uvu_validate(C.byref(b), 1) == 0   # chunks of 64
     b.C, b.dtype = 64, _lib.F64
     assert L.cgtp_uvu_validate(C.byref(b), 0) == 4
     b.dtype, b.n_seg, b.ptr, b.seg_ids, b.gather = _lib.F32, 10, 4096, 4096, 4096

@@ -165,10 +165,11 @@ def test_u1u_large_table_fp32(device, lmax, channels):
         assert_close(g, r, 1e-5, f"lmax={lmax} C={channels} {name}")
 
 
-@pytest.mark.parametrize("lmax,n,ch", [(6, 40, 16), (4, 700, 32), (2, 300, 64)])
+@pytest.mark.parametrize("lmax,n,ch", [(6, 40, 16), (4, 700, 32), (2, 300, 64), (2, 5000, 64), (1, 9000, 32)])
 def test_u1u_block_wise_shared_weight(device, lmax, n, ch):
     """Shared weight on the block-wise kernels: its gradient is written per row and summed in two fixed-order
-    passes (700 rows: three first-pass chunks)."""
+    passes (700 rows: three first-pass chunks; 5000 and 9000 rows: more wavefronts than the register-resident
+    kernels' grid-stride launch would use)."""
     irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
     d = (lmax + 1) ** 2
     mod = _module(irreps, irreps, irreps).to(device)
@@ -207,7 +208,24 @@ def test_edge_large_table(device):
         assert_close(g, r, 1e-5, f"edge lmax=6 {name}")
 
 
-@pytest.mark.parametrize("lmax,channels", [(2, 64), (2, 20), (3, 48)])
+@pytest.mark.parametrize("lmax,n,ch", [(3, 130, 128), (2, 257, 200), (2, 33, 65)])
+@pytest.mark.parametrize("shared_w", [False, True])
+def test_u1u_block_wise_wide_rows(device, lmax, n, ch, shared_w):
+    """More than 64 channels, fp32: forward and backward run one channel chunk per wavefront; grad_sh is summed over
+    the chunks' partial sums in a fixed order."""
+    irreps = SH[lmax]
+    d = (lmax + 1) ** 2
+    mod = _module(irreps, irreps, irreps).to(device)
+    x, sh, w = tp_inputs(n, d, lmax, mod.num_paths, ch, shared_w, seed=90 + lmax)
+    ct = torch.randn(n, d, ch, generator=torch.Generator().manual_seed(8))
+    got = _run(mod, x, sh, w, ct, device)
+    T = ref_ops.dense_coupling(irreps, irreps, irreps)
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1u, T, (x, sh, w), ct)
+    for name, g, r in zip(("out", "grad_x", "grad_sh", "grad_w"), got, (ref_out, *ref_grads)):
+        assert_close(g, r, 1e-5, f"lmax={lmax} C={ch} shared={shared_w} {name}")
+
+
+@pytest.mark.parametrize("lmax,channels", [(2, 64), (2, 20), (3, 48), (2, 96)])
 @pytest.mark.parametrize("shared_w", [False, True])
 def test_uuu_on_the_block_wise_kernels(device, lmax, channels, shared_w):
     """TensorProduct('uuu') with a compiled table: both operands channelled, fp32, forward and all gradients against
