@@ -304,7 +304,11 @@ def scatter_bench(steps, warmup):
 
 def membench(kind, steps, warmup):
     """Plain 1 GiB device copy (reads 1 GiB, writes 1 GiB) or read; one JSON line with the achieved GB/s."""
+    import ctypes
     from equitorch_amd import _lib
+    blib = ctypes.CDLL(os.path.join(ROOT, "equitorch_amd", "lib", "libcgtp_bench.so"))
+    for fn in (blib.cgtpbench_copy, blib.cgtpbench_read):
+        fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
     dev = torch.device("cuda:0")
     n_bytes = 1 << 30
     src = torch.empty(n_bytes, dtype=torch.uint8, device=dev).fill_(1)
@@ -313,9 +317,9 @@ def membench(kind, steps, warmup):
 
     def launch():
         if kind == "copy":
-            _lib.check(_lib.lib.cgtp_membench_copy(dst.data_ptr(), src.data_ptr(), n_bytes, stream))
+            _lib.check(blib.cgtpbench_copy(dst.data_ptr(), src.data_ptr(), n_bytes, stream))
         else:
-            _lib.check(_lib.lib.cgtp_membench_read(src.data_ptr(), dst.data_ptr(), n_bytes, stream))
+            _lib.check(blib.cgtpbench_read(src.data_ptr(), dst.data_ptr(), n_bytes, stream))
     for _ in range(warmup):
         launch()
     evs = []

@@ -121,8 +121,7 @@ def _load():
                                        _seg, C.c_int, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
     lib.cgtp_wigner_rotate_backward.argtypes = [C.c_void_p] * 6 + [_seg, _seg, C.c_int, C.c_int64, C.c_int, C.c_int] + \
         [C.c_void_p] * 4 + [C.c_int, C.c_void_p]
-    lib.cgtp_membench_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
-    lib.cgtp_membench_read.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
+    lib.cgtp_abi_layout.argtypes = [C.c_int, C.POINTER(C.c_int64), C.c_int]
     return lib
 
 

@@ -1,5 +1,7 @@
-// Plain streaming kernels of known traffic, used to calibrate hardware counters and to read the achievable
-// HBM bandwidth of the device next to the tensor-product kernels.
+// Plain streaming kernels of known traffic, used by the benchmark script to calibrate hardware counters and to read
+// the achievable HBM bandwidth of the device next to the tensor-product kernels.  Built into libcgtp_bench.so, which
+// is not part of the product's C ABI.  copy: reads n_bytes and writes n_bytes; read: reads n_bytes; n_bytes must be a
+// multiple of 16 and the pointers 16-byte aligned; status codes as in cgtp.h.
 #include "cgtp_device.h"
 #include "cgtp_host.h"
 
@@ -26,7 +28,7 @@ using namespace cgtp;
 
 extern "C" {
 
-int cgtp_membench_copy(void* dst, const void* src, int64_t n_bytes, void* stream) {
+int cgtpbench_copy(void* dst, const void* src, int64_t n_bytes, void* stream) {
   if (!dst || !src) return CGTP_ERR_NULL;
   if (n_bytes < 0 || (n_bytes & 15)) return CGTP_ERR_SHAPE;
   if (((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15u) != 0) return CGTP_ERR_ALIGN;
@@ -36,7 +38,7 @@ int cgtp_membench_copy(void* dst, const void* src, int64_t n_bytes, void* stream
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 
-int cgtp_membench_read(const void* src, void* sink, int64_t n_bytes, void* stream) {
+int cgtpbench_read(const void* src, void* sink, int64_t n_bytes, void* stream) {
   if (!src || !sink) return CGTP_ERR_NULL;
   if (n_bytes < 0 || (n_bytes & 15)) return CGTP_ERR_SHAPE;
   if ((reinterpret_cast<uintptr_t>(src) & 15u) != 0) return CGTP_ERR_ALIGN;

@@ -16,6 +16,7 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 LIB_DIR = os.path.join(os.path.dirname(HERE), "lib")
 OBJ_DIR = os.path.join(HERE, "_build")
 LIB_PATH = os.path.join(LIB_DIR, "libcgtp.so")
+BENCH_LIB_PATH = os.path.join(LIB_DIR, "libcgtp_bench.so")     # calibration kernels of bench.py, not the product ABI
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -50,10 +51,15 @@ def build(jobs: int = 8) -> str:
     sources = sorted(os.path.join(HERE, f) for f in os.listdir(HERE) if f.endswith(".hip"))
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
         objs = list(pool.map(_compile, sources))
-    cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB_PATH, *objs]
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
+    bench_dir = os.path.join(HERE, "bench")
+    bench_sources = sorted(os.path.join(bench_dir, f) for f in os.listdir(bench_dir) if f.endswith(".hip"))
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        bench_objs = list(pool.map(_compile, bench_sources))
+    for path, parts in ((LIB_PATH, objs), (BENCH_LIB_PATH, bench_objs)):
+        cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", path, *parts]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"link of {path} failed:\n{res.stdout}\n{res.stderr}")
     return LIB_PATH
 
 

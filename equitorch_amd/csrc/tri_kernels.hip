@@ -2,6 +2,7 @@
 // scale-segment reduction.  These kernels take the tables at run time, so they serve every irreps
 // configuration (and the reference's table-driven operator API); configurations with a compiled-in table
 // use the kernels of uvu_kernels.hip instead.
+#include <cstddef>
 #include "cgtp_device.h"
 #include "cgtp_host.h"
 
@@ -54,7 +55,9 @@ __global__ void __launch_bounds__(256) tri_kernel(const TriDev<T> a, int64_t n_w
 
   const int64_t per = a.reduce_rows ? (a.n_rows + n_waves - 1) / n_waves : 1;
   const int64_t stride = a.reduce_rows ? n_waves * per : n_waves;  // reduce_rows: a single pass
-  for (int64_t r0 = wave * per; r0 < a.n_rows; r0 += stride) {
+  // a wavefront of a row sum whose share is empty (wave * per >= n_rows) still writes its partial row, as zeros:
+  // the second pass adds all n_waves partial rows
+  for (int64_t r0 = wave * per; a.reduce_rows || r0 < a.n_rows; r0 += stride) {
     const int64_t r1 = (r0 + per < a.n_rows) ? r0 + per : a.n_rows;
     const int64_t orow = a.reduce_rows ? wave : r0;
     for (int o = 0; o < a.n_out; ++o) {
@@ -535,7 +538,51 @@ const char* cgtp_status_string(int status) {
   }
 }
 
-int cgtp_version(void) { return 1; }
+int cgtp_version(void) { return 2; }
+
+int cgtp_abi_layout(int which, int64_t* out, int capacity) {
+#define CGTP_OFF(S, f) (int64_t) offsetof(S, f)
+  static const int64_t operand[] = {sizeof(cgtp_operand), CGTP_OFF(cgtp_operand, data), CGTP_OFF(cgtp_operand, rows),
+                                    CGTP_OFF(cgtp_operand, row_stride), CGTP_OFF(cgtp_operand, idx_stride),
+                                    CGTP_OFF(cgtp_operand, kind), CGTP_OFF(cgtp_operand, size)};
+  static const int64_t tri[] = {sizeof(cgtp_tri_args), CGTP_OFF(cgtp_tri_args, a), CGTP_OFF(cgtp_tri_args, b),
+                                CGTP_OFF(cgtp_tri_args, w), CGTP_OFF(cgtp_tri_args, coef), CGTP_OFF(cgtp_tri_args, idx),
+                                CGTP_OFF(cgtp_tri_args, seg), CGTP_OFF(cgtp_tri_args, n_out), CGTP_OFF(cgtp_tri_args, nnz),
+                                CGTP_OFF(cgtp_tri_args, out), CGTP_OFF(cgtp_tri_args, workspace),
+                                CGTP_OFF(cgtp_tri_args, n_rows), CGTP_OFF(cgtp_tri_args, C), CGTP_OFF(cgtp_tri_args, dtype),
+                                CGTP_OFF(cgtp_tri_args, reduce_c), CGTP_OFF(cgtp_tri_args, reduce_rows)};
+  static const int64_t gen_operand[] = {sizeof(cgtp_gen_operand), CGTP_OFF(cgtp_gen_operand, data),
+                                        CGTP_OFF(cgtp_gen_operand, row_stride), CGTP_OFF(cgtp_gen_operand, idx_stride),
+                                        CGTP_OFF(cgtp_gen_operand, u_stride), CGTP_OFF(cgtp_gen_operand, w_stride),
+                                        CGTP_OFF(cgtp_gen_operand, present), CGTP_OFF(cgtp_gen_operand, _pad)};
+  static const int64_t gen[] = {sizeof(cgtp_gen_args), CGTP_OFF(cgtp_gen_args, a), CGTP_OFF(cgtp_gen_args, b),
+                                CGTP_OFF(cgtp_gen_args, w), CGTP_OFF(cgtp_gen_args, coef), CGTP_OFF(cgtp_gen_args, idx),
+                                CGTP_OFF(cgtp_gen_args, seg), CGTP_OFF(cgtp_gen_args, n_out), CGTP_OFF(cgtp_gen_args, nnz),
+                                CGTP_OFF(cgtp_gen_args, out), CGTP_OFF(cgtp_gen_args, n_rows), CGTP_OFF(cgtp_gen_args, U),
+                                CGTP_OFF(cgtp_gen_args, W), CGTP_OFF(cgtp_gen_args, out_has_u),
+                                CGTP_OFF(cgtp_gen_args, out_has_w), CGTP_OFF(cgtp_gen_args, reduce_rows),
+                                CGTP_OFF(cgtp_gen_args, dtype)};
+  static const int64_t uvu[] = {sizeof(cgtp_uvu_args), CGTP_OFF(cgtp_uvu_args, cfg), CGTP_OFF(cgtp_uvu_args, dtype),
+                                CGTP_OFF(cgtp_uvu_args, C), CGTP_OFF(cgtp_uvu_args, w_shared),
+                                CGTP_OFF(cgtp_uvu_args, n_rows), CGTP_OFF(cgtp_uvu_args, n_x_rows),
+                                CGTP_OFF(cgtp_uvu_args, n_seg), CGTP_OFF(cgtp_uvu_args, ptr), CGTP_OFF(cgtp_uvu_args, perm),
+                                CGTP_OFF(cgtp_uvu_args, seg_ids), CGTP_OFF(cgtp_uvu_args, gather),
+                                CGTP_OFF(cgtp_uvu_args, pos_per_wave), CGTP_OFF(cgtp_uvu_args, y_vec),
+                                CGTP_OFF(cgtp_uvu_args, wave_seg), CGTP_OFF(cgtp_uvu_args, n_waves),
+                                CGTP_OFF(cgtp_uvu_args, x), CGTP_OFF(cgtp_uvu_args, y), CGTP_OFF(cgtp_uvu_args, w),
+                                CGTP_OFF(cgtp_uvu_args, out), CGTP_OFF(cgtp_uvu_args, grad_out),
+                                CGTP_OFF(cgtp_uvu_args, grad_x), CGTP_OFF(cgtp_uvu_args, grad_y),
+                                CGTP_OFF(cgtp_uvu_args, grad_w), CGTP_OFF(cgtp_uvu_args, workspace),
+                                CGTP_OFF(cgtp_uvu_args, x_gather), CGTP_OFF(cgtp_uvu_args, y_channels),
+                                CGTP_OFF(cgtp_uvu_args, reserved_)};
+#undef CGTP_OFF
+  const int64_t* tabs[] = {operand, tri, gen_operand, gen, uvu};
+  const int counts[] = {(int)(sizeof(operand) / 8), (int)(sizeof(tri) / 8), (int)(sizeof(gen_operand) / 8),
+                        (int)(sizeof(gen) / 8), (int)(sizeof(uvu) / 8)};
+  if (which < 0 || which >= 5) return -1;
+  for (int i = 0; out && i < counts[which] && i < capacity; ++i) out[i] = tabs[which][i];
+  return counts[which];
+}
 
 int cgtp_tri_validate(const cgtp_tri_args* args) {
   int64_t lds = 0, nw = 0;

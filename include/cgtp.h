@@ -36,6 +36,12 @@ enum { CGTP_F32 = 0, CGTP_F64 = 1, CGTP_BF16 = 2, CGTP_F16 = 3 };
 const char* cgtp_status_string(int status);
 /* ABI version; bumped on any signature change. */
 int cgtp_version(void);
+/* Layout of the argument structs as this library was compiled, so that a binding that mirrors them by hand (ctypes,
+ * cgo, JNI) can check itself: which = CGTP_LAYOUT_*; writes sizeof(struct) followed by the byte offset of every field
+ * in declaration order to out[0 .. capacity) and returns how many numbers the full description has (-1: bad id). */
+enum { CGTP_LAYOUT_OPERAND = 0, CGTP_LAYOUT_TRI_ARGS = 1, CGTP_LAYOUT_GEN_OPERAND = 2, CGTP_LAYOUT_GEN_ARGS = 3,
+       CGTP_LAYOUT_UVU_ARGS = 4 };
+int cgtp_abi_layout(int which, int64_t* out, int capacity);
 
 /* ---- generic sparse trilinear contraction -------------------------------------------------------------
  *
@@ -325,13 +331,6 @@ int cgtp_wigner_rotate_backward(const void* x, const void* grad_out, const void*
                                 const int32_t* irrep_degree, int n_irreps, int64_t n_rows, int C, int cs_dim,
                                 void* grad_x, void* grad_alpha, void* grad_beta, void* grad_gamma, int dtype,
                                 void* stream);
-
-/* ---- streaming kernels of known traffic (counter calibration, achievable-bandwidth reference) ------------
- * No counterpart in the reference.  copy: reads n_bytes and writes n_bytes; read: reads n_bytes.
- * n_bytes must be a multiple of 16 and the pointers 16-byte aligned.
- */
-int cgtp_membench_copy(void* dst, const void* src, int64_t n_bytes, void* stream);
-int cgtp_membench_read(const void* src, void* sink, int64_t n_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -11,9 +11,13 @@ Two independent restatements:
   CSR sum along dim 1 and is restated as ``index_add_`` over expanded segment ids.  This is the timed
   "reference CPU path" of the benchmark.
 
-Pinned by: agreement of the two restatements with each other (tests/test_oracle.py), and for the dense one
-by O(3)-equivariance, the l2=0 scaling identity, the 1x1->0 dot product, the 1x1->1 cross product and
-``torch.autograd.gradcheck``.  No stored output vectors exist in the reference for this path.
+Pinned by: agreement of the two restatements with each other (tests/test_oracle.py, tests/test_oracle_uv.py),
+and for the dense one by O(3)-equivariance, the l2=0 scaling identity, the 1x1->0 dot product, the 1x1->1
+cross product and ``torch.autograd.gradcheck``; the fully connected members (``dense_u1v``, ``dense_uvw``)
+additionally by their reduction to ``x @ W`` at lmax = 0, by the ``l2 = 0`` paths being ``y0 * x[block] @ W[p]``,
+by ``dense_uvw`` with a single second-operand channel equal to ``dense_u1v`` and with diagonal weights equal to
+``dense_uuu``, and by the structural ``cpu_u1v_* / cpu_1vu_* / cpu_vu1_* / cpu_uvw_*`` chains.  No stored output
+vectors exist in the reference for this path.
 """
 import torch
 
@@ -160,6 +164,43 @@ def cpu_inner(x, y, info, out_accumulated=False):
     return inter.sum(0) if out_accumulated else inter
 
 
+def cpu_outer(x, y, info, out_accumulated=False):
+    """``indexed_outer_scale_gather_cpu`` (batched_sparse_dense_op.py:515-556): ``x (.., M1, U)``, ``y (.., M2, V)``
+    -> ``(.., M, U, V)``."""
+    if info["index1"] is not None:
+        x = x.index_select(-2, info["index1"])
+    if info["index2"] is not None:
+        y = y.index_select(-2, info["index2"])
+    inter = x.unsqueeze(-1) * y.unsqueeze(-2)
+    if info["scale"] is not None:
+        inter = inter * info["scale"].view(-1, 1, 1)
+    if info["seg_out"] is not None:
+        inter = segment_csr(inter, info["seg_out"], inter.ndim - 3)
+    return inter.sum(0) if out_accumulated else inter
+
+
+def cpu_vecmat(x, y, info, out_accumulated=False):
+    """``indexed_vecmat_scale_gather_cpu`` (:1461-1509): ``x (.., M1, U)`` vector, ``y (.., M2, U, V)`` matrix
+    -> ``(.., M, V)``."""
+    if info["index1"] is not None:
+        x = x.index_select(-2, info["index1"])
+    if info["index2"] is not None:
+        y = y.index_select(-3, info["index2"])
+    inter = torch.einsum("...ti,...tij->...tj", x, y)
+    if info["scale"] is not None:
+        inter = inter * info["scale"].unsqueeze(-1)
+    if info["seg_out"] is not None:
+        inter = segment_csr(inter, info["seg_out"], inter.ndim - 2)
+    return inter.sum(0) if out_accumulated else inter
+
+
+def cpu_mat_t_vec(x, y, info, out_accumulated=False):
+    """``indexed_mat_t_vec_scale_gather`` (:1200-1238): matrix first, vector second; calls vecmat with the operands
+    and their index columns exchanged."""
+    swapped = dict(info, index1=info["index2"], index2=info["index1"])
+    return cpu_vecmat(y, x, swapped, out_accumulated)
+
+
 def cpu_scale_segment(inp, scale, index, seg):
     """``indexed_scale_segment_cpu`` (indexed_scale_segment_op.py:143-170)."""
     if index is not None:
@@ -195,6 +236,65 @@ def cpu_u1u_backward(g, x, y, w, inter, tp_fwd, tp_bwd1, tp_bwd2):
     gy = cpu_uu1_forward(g, x, w, tp_bwd2)
     gw = cpu_mul(g, inter, tp_fwd["info_M_bwd2"], out_accumulated=(w.ndim == 2))
     return gx, gy, gw
+
+
+# fully connected family: ``TensorProductU1VDummy`` and siblings (nn/functional/linears.py:254-492) and
+# ``TensorProductUVWDummy`` (nn/functional/tensor_products.py:92-172), first-order parts
+def cpu_sparse_scale(x, info):
+    """``sparse_scale`` (nn/functional/sparse_scale.py:14-46) on a table dict with ``scale / index / seg_out``."""
+    return cpu_scale_segment(x, info["scale"], info["index"], info["seg_out"])
+
+
+def cpu_u1v_forward(x, y, w, tp_fwd):
+    """``TensorProductU1VDummy.forward`` (linears.py:257-280): vecsca then vecmat -> (ret, inter)."""
+    inter = cpu_vecsca(x, y, tp_fwd["info_Mij_fwd"])
+    return cpu_vecmat(inter, w, tp_fwd["info_M_fwd"]), inter
+
+
+def cpu_1vu_forward(x, y, w, tp_fwd):
+    """``TensorProduct1VUDummy.forward`` (:341-344): x channel-less, y carries the input channels."""
+    inter = cpu_scavec(x, y, tp_fwd["info_Mij_fwd"])
+    return cpu_vecmat(inter, w, tp_fwd["info_M_fwd"]), inter
+
+
+def cpu_vu1_forward(x, y, w, tp_fwd):
+    """``TensorProductVU1Dummy.forward`` (:419-422): weight first (``info_kM1j``), inner product with the second
+    operand (``info_kM1M2``), then the coefficient sum (``info_M_kM1M2``)."""
+    inter = cpu_vecmat(x, w, tp_fwd["info_kM1j_fwd"])
+    inter = cpu_inner(inter, y, tp_fwd["info_kM1M2_fwd"])
+    return cpu_sparse_scale(inter.unsqueeze(-1), tp_fwd["info_M_kM1M2_fwd"]).squeeze(-1)
+
+
+def cpu_u1v_backward(g, x, y, w, inter, tp_fwd, tp_bwd1, tp_bwd2):
+    """First-order part of ``TensorProductU1VDummy.backward`` (:282-324)."""
+    wt = w.transpose(-1, -2).contiguous()
+    gx, _ = cpu_1vu_forward(y, g, wt, tp_bwd1)
+    gy = cpu_vu1_forward(g, x, wt, tp_bwd2)
+    gw = cpu_outer(g, inter, tp_fwd["info_M_bwd2"], out_accumulated=(w.ndim == 3)).transpose(-1, -2).contiguous()
+    return gx, gy, gw
+
+
+def cpu_uvw_forward(x, y, w, tp_fwd):
+    """``TensorProductUVWDummy.forward`` (tensor_products.py:95-101): outer product of the operands' channels, then
+    vecmat with the weight flattened over (u, v) -> (ret, inter)."""
+    inter = cpu_outer(x, y, tp_fwd["info_Mij_fwd"])
+    return cpu_vecmat(inter.flatten(-2), w.flatten(-3, -2), tp_fwd["info_M_fwd"]), inter
+
+
+def cpu_uvw_backward(g, x, y, w, inter, tp_fwd, tp_bwd1, tp_bwd2):
+    """First-order part of ``TensorProductUVWDummy.backward`` (:120-161)."""
+    lead = tuple(range(w.ndim - 3))
+    gx, _ = cpu_uvw_forward(y, g, w.permute(*lead, -2, -1, -3).contiguous(), tp_bwd1)
+    gy, _ = cpu_uvw_forward(g, x, w.permute(*lead, -1, -3, -2).contiguous(), tp_bwd2)
+    gw = cpu_outer(g, inter.flatten(-2), tp_fwd["info_M_bwd2"], out_accumulated=(w.ndim == 4))
+    gw = gw.transpose(-1, -2).contiguous().unflatten(-2, w.shape[-3:-1])
+    return gx, gy, gw
+
+
+def cpu_uuu_forward(x, y, w, tp_fwd):
+    """``TensorProductUUUDummy.forward`` (tensor_products.py:12-18): both operands and the weight per channel."""
+    inter = cpu_mul(x, y, tp_fwd["info_Mij_fwd"])
+    return cpu_mul(inter, w, tp_fwd["info_M_fwd"]), inter
 
 
 def cpu_edge_forward(x, sh, w, src, perm, ptr, tp_fwd):

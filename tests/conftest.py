@@ -6,6 +6,9 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
+HERE = os.path.dirname(os.path.abspath(__file__))
+if HERE not in sys.path:
+    sys.path.insert(0, HERE)
 
 
 def pytest_configure(config):
@@ -18,3 +21,17 @@ def device():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     return torch.device("cuda:0")
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """With CGTP_PARITY_REPORT=<file>: one line per comparison made through helpers.assert_close — test, quantity,
+    tolerance, worst element-wise ratio |a-b| / (1 + |b|), worst norm-wise ratio max|a-b| / max(1, max|b|)."""
+    path = os.environ.get("CGTP_PARITY_REPORT")
+    if not path:
+        return
+    from helpers import PARITY_LOG
+    os.makedirs(os.path.dirname(os.path.abspath(path)), exist_ok=True)
+    with open(path, "w") as f:
+        f.write("test\twhat\ttol\telementwise\tnormwise\n")
+        for test, what, tol, elem, normwise in PARITY_LOG:
+            f.write(f"{test}\t{what}\t{tol:.0e}\t{elem:.3e}\t{normwise:.3e}\n")

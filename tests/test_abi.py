@@ -25,6 +25,21 @@ def test_every_declared_symbol_is_exported():
         assert hasattr(lib, n), f"{n} declared in include/cgtp.h but not exported"
 
 
+def test_struct_layouts_match_the_ctypes_mirror():
+    """The argument structs are mirrored by hand in ``equitorch_amd/_lib.py``; the library reports sizeof and every
+    field offset as compiled, in declaration order."""
+    from equitorch_amd import _lib
+    for which, cls in enumerate((_lib.Operand, _lib.TriArgs, _lib.GenOperand, _lib.GenArgs, _lib.UvuArgs)):
+        n = _lib.lib.cgtp_abi_layout(which, None, 0)
+        assert n == 1 + len(cls._fields_), f"{cls.__name__}: {n - 1} fields in the library, {len(cls._fields_)} here"
+        buf = (C.c_int64 * n)()
+        assert _lib.lib.cgtp_abi_layout(which, buf, n) == n
+        assert buf[0] == C.sizeof(cls), f"sizeof {cls.__name__}"
+        for k, (name, _) in enumerate(cls._fields_):
+            assert buf[1 + k] == getattr(cls, name).offset, f"{cls.__name__}.{name}"
+    assert _lib.lib.cgtp_abi_layout(99, None, 0) == -1
+
+
 def test_version_and_status_strings():
     from equitorch_amd import _lib
     assert _lib.lib.cgtp_version() >= 1
@@ -93,7 +108,6 @@ def test_host_side_validation_codes():
     t.a.kind = 1
     assert L.cgtp_tri_validate(C.byref(t)) == 1                     # operand declared but no data
     assert L.cgtp_segment_sum(None, None, None, None, None, 1, 1, 1, 1, 0, None) == 1
-    assert L.cgtp_membench_copy(256, 256, 17, None) == 2
 
 
 def test_large_table_configs_and_row_gathers_validate_on_the_host():

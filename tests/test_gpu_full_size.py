@@ -1,0 +1,199 @@
+"""GPU parity at the full sizes of the benchmark configurations: the fused edge tensor product at
+N = 4096 / E = 65536 (lmax = 2, C = 64) and the large-table edge product at N = 20000 / E = 200000 (lmax = 6,
+C = 32), forward and all gradients.
+
+The dense float64 oracle cannot run at these sizes in seconds, so it is run on sub-problems that are exact for a
+strided subset of the result rows: an output row depends only on the in-edges of its node, a ``grad_x`` row only on
+the out-edges of its node, ``grad_sh`` / ``grad_W`` rows only on their own edge.  The subsets are spread over the
+whole index range so that every wavefront range, every XCD share and the tail of the launch contribute rows.
+Inputs follow the benchmark's recipe (one CPU generator seeded 0; src, dst, x, unit vectors -> harmonics, W,
+cotangent, in that order)."""
+import pytest
+import torch
+
+from helpers import assert_close, unit_vectors
+from oracle import ref_ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _sh_irreps(lmax):
+    return "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+
+
+def _inputs(n_nodes, n_edges, lmax, channels, n_paths, hubs=0):
+    from equitorch_amd.utils._sh import spherical_harmonics
+    gen = torch.Generator().manual_seed(0)
+    src = torch.randint(0, n_nodes, (n_edges,), generator=gen)
+    dst = torch.randint(0, n_nodes, (n_edges,), generator=gen)
+    if hubs:
+        # a few nodes of very high in- and out-degree (several wavefront ranges each), the rest stay uniform
+        for h in range(hubs):
+            dst[1000 + 3000 * h: 1000 + 3000 * h + 700 * (h + 1)] = 97 * (h + 1)
+            src[20000 + 3000 * h: 20000 + 3000 * h + 500 * (h + 1)] = 11 * (h + 1)
+    d = (lmax + 1) ** 2
+    x = torch.randn(n_nodes, d, channels, generator=gen)
+    sh = spherical_harmonics(unit_vectors(n_edges, gen), lmax)
+    w = torch.randn(n_edges, n_paths, channels, generator=gen)
+    ct = torch.randn(n_nodes, d, channels, generator=gen)
+    return src, dst, x, sh, w, ct
+
+
+def _check_subsets(T, src, dst, x, sh, w, ct, got, n_dst, n_src, n_edge, tol=1e-5, tag=""):
+    """Compare ``got = (out, grad_x, grad_sh, grad_w)`` (device tensors) with the dense oracle on strided subsets."""
+    out, gx, gsh, gw = (t.detach().cpu() for t in got)
+    n_nodes, n_edges = x.shape[0], src.shape[0]
+    # output rows: all in-edges of a strided set of nodes (+ the first and the last node)
+    nodes = torch.unique(torch.cat([torch.arange(3, n_nodes, max(1, n_nodes // n_dst)), torch.tensor([0, n_nodes - 1])]))
+    mask = torch.zeros(n_nodes, dtype=torch.bool)
+    mask[nodes] = True
+    e_in = torch.nonzero(mask[dst]).flatten()
+    msg = ref_ops.dense_u1u(T, x[src[e_in]], sh[e_in], w[e_in])
+    ref_out = ref_ops.scatter_sum(msg, dst[e_in], n_nodes)[nodes]
+    # rows summed over ~16 (up to hundreds at a hub) edges x all coefficients: element-wise where it holds
+    assert_close(out[nodes], ref_out, tol, f"{tag} out rows", norm="max")
+    # grad_x rows: all out-edges of a strided set of nodes; grad_sh / grad_w: those edges and a strided set of edges
+    nodes = torch.unique(torch.cat([torch.arange(5, n_nodes, max(1, n_nodes // n_src)), torch.tensor([0, n_nodes - 1])]))
+    mask = torch.zeros(n_nodes, dtype=torch.bool)
+    mask[nodes] = True
+    emask = mask[src]
+    emask[torch.arange(7, n_edges, max(1, n_edges // n_edge))] = True
+    emask[0] = emask[n_edges - 1] = True
+    e_sub = torch.nonzero(emask).flatten()
+    xr = x.double().requires_grad_(True)
+    shr, wr = sh[e_sub].double().requires_grad_(True), w[e_sub].double().requires_grad_(True)
+    loss = (ref_ops.dense_u1u(T, xr[src[e_sub]], shr, wr) * ct[dst[e_sub]].double()).sum()
+    rgx, rgsh, rgw = torch.autograd.grad(loss, (xr, shr, wr))
+    assert_close(gx[nodes], rgx[nodes], tol, f"{tag} grad_x rows", norm="max")
+    assert_close(gsh[e_sub], rgsh, tol, f"{tag} grad_sh rows", norm="max")
+    assert_close(gw[e_sub], rgw, tol, f"{tag} grad_w rows")
+
+
+@pytest.mark.parametrize("graph", ["uniform", "hubs"])
+def test_edge_fused_full_size_lmax2(device, graph):
+    """BASELINE configs[1] / configs[2] shapes through the public autograd path (segment-aligned ranges on the
+    uniform graph; the graph with hub nodes takes ranges cut by position, partial rows and the fix-up kernel)."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu
+    irr = _sh_irreps(2)
+    n_nodes, n_edges, ch = 4096, 65536, 64
+    mod = SO3Linear(irr, irr, irr, ch, ch, internal_weights=False, feature_mode="uu").to(device)
+    src, dst, x, sh, w, ct = _inputs(n_nodes, n_edges, 2, ch, mod.num_paths, hubs=3 if graph == "hubs" else 0)
+    plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
+    if graph == "uniform":
+        assert plan.fwd_index.wave_seg is not None and plan.bwd_index.wave_seg is not None
+    else:
+        assert plan.fwd_index.wave_seg is None and plan.bwd_index.wave_seg is None
+    xd, shd, wd = (t.to(device).requires_grad_(True) for t in (x, sh, w))
+    out = edge_tensor_product_uu(xd, shd, wd, plan, mod.tp_info_forward)
+    (out * ct.to(device)).sum().backward()
+    T = ref_ops.dense_coupling(irr, irr, irr)
+    _check_subsets(T, src, dst, x, sh, w, ct, (out, xd.grad, shd.grad, wd.grad), 64, 64, 512, tag=f"lmax=2 {graph}")
+
+
+def test_edge_fused_full_size_by_position(device):
+    """The same uniform graph with the ranges cut by position (32 per wavefront) instead of at segment boundaries:
+    2048 ranges, almost every one starting and ending inside a segment."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import EdgePlan
+    from equitorch_amd.ops import kernels
+    irr = _sh_irreps(2)
+    n_nodes, n_edges, ch = 4096, 65536, 64
+    mod = SO3Linear(irr, irr, irr, ch, ch, internal_weights=False, feature_mode="uu").to(device)
+    cfg = kernels.uvu_config_of(mod.tp_info_forward)
+    dims = kernels.uvu_dims(cfg)
+    src, dst, x, sh, w, ct = _inputs(n_nodes, n_edges, 2, ch, mod.num_paths)
+    plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
+    xd, shd, wd, ctd = (t.to(device) for t in (x, sh, w, ct))
+    out = kernels.uvu_forward(cfg, dims, xd, shd, wd, seg=plan.fwd_index, pos_per_wave=32)
+    gx, gy, gw = kernels.uvu_backward(cfg, dims, xd, shd, wd, ctd, (True, True, True), seg=plan.bwd_index,
+                                      pos_per_wave=32)
+    T = ref_ops.dense_coupling(irr, irr, irr)
+    _check_subsets(T, src, dst, x, sh, w, ct, (out, gx, gy, gw), 64, 64, 512, tag="lmax=2 by position")
+
+
+def test_edge_fused_full_size_vectors(device):
+    """Full size with the harmonics evaluated inside the kernels (edge vectors in, gradient of the vectors out):
+    output and node / weight gradients against the same oracle; the vector gradient against the harmonics' own
+    backward applied to the oracle's ``grad_sh`` on the subset."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu, edge_tensor_product_uu_vectors
+    irr = _sh_irreps(2)
+    n_nodes, n_edges, ch = 4096, 65536, 64
+    mod = SO3Linear(irr, irr, irr, ch, ch, internal_weights=False, feature_mode="uu").to(device)
+    src, dst, x, _, w, ct = _inputs(n_nodes, n_edges, 2, ch, mod.num_paths)
+    vec = torch.randn(n_edges, 3, generator=torch.Generator().manual_seed(1)) * 1.7
+    plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
+    xd, vd, wd = (t.to(device).requires_grad_(True) for t in (x, vec, w))
+    out = edge_tensor_product_uu_vectors(xd, vd, wd, plan, mod.tp_info_forward)
+    (out * ct.to(device)).sum().backward()
+    from oracle import ref_sh
+    vr = vec.double().requires_grad_(True)
+    shr = ref_sh.spherical_harmonics(vr / vr.norm(dim=-1, keepdim=True), 2)
+    T = ref_ops.dense_coupling(irr, irr, irr)
+    e_sub = torch.arange(7, n_edges, 128)
+    xr, wr = x.double(), w[e_sub].double()
+    loss = (ref_ops.dense_u1u(T, xr[src[e_sub]], shr[e_sub], wr) * ct[dst[e_sub]].double()).sum()
+    (rgv,) = torch.autograd.grad(loss, vr)
+    assert_close(vd.grad.cpu()[e_sub], rgv[e_sub], 1e-5, "grad_vec rows", norm="max")
+    nodes = torch.arange(3, n_nodes, 64)
+    mask = torch.zeros(n_nodes, dtype=torch.bool)
+    mask[nodes] = True
+    e_in = torch.nonzero(mask[dst]).flatten()
+    msg = ref_ops.dense_u1u(T, xr[src[e_in]], shr.detach()[e_in], w[e_in])
+    assert_close(out.detach().cpu()[nodes], ref_ops.scatter_sum(msg, dst[e_in], n_nodes)[nodes], 1e-5,
+                 "out rows (vectors)", norm="max")
+
+
+def test_edge_full_size_lmax6(device):
+    """BASELINE configs[4] shapes: N = 20000, E = 200000, lmax = 6, C = 32, per-edge weights (2.7 GB), forward and
+    all gradients through the public autograd path (block-wise row-mode kernels + segment sums over 200000 rows)."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu
+    irr = _sh_irreps(6)
+    n_nodes, n_edges, ch = 20000, 200000, 32
+    mod = SO3Linear(irr, irr, irr, ch, ch, internal_weights=False, feature_mode="uu").to(device)
+    src, dst, x, sh, w, ct = _inputs(n_nodes, n_edges, 6, ch, mod.num_paths)
+    plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
+    xd, shd, wd = (t.to(device).requires_grad_(True) for t in (x, sh, w))
+    out = edge_tensor_product_uu(xd, shd, wd, plan, mod.tp_info_forward)
+    (out * ct.to(device)).sum().backward()
+    T = ref_ops.dense_coupling(irr, irr, irr)
+    _check_subsets(T, src, dst, x, sh, w, ct, (out, xd.grad, shd.grad, wd.grad), 12, 12, 96, tag="lmax=6")
+
+
+def test_row_mode_full_size_shared_weight(device):
+    """BASELINE configs[0] module (``SO3Linear('uu')``, shared weight) at 65536 rows, lmax = 2, C = 64: out / grad_x /
+    grad_sh rows on a strided subset; the shared weight's gradient (a sum over all rows) through linearity — the
+    gradient for a cotangent that is zero outside the subset equals the oracle's sum over the subset."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.utils._sh import spherical_harmonics
+    irr = _sh_irreps(2)
+    n, ch = 65536, 64
+    mod = SO3Linear(irr, irr, irr, ch, ch, internal_weights=False, feature_mode="uu").to(device)
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(n, 9, ch, generator=gen)
+    sh = spherical_harmonics(unit_vectors(n, gen), 2)
+    w = torch.randn(mod.num_paths, ch, generator=gen)
+    ct = torch.randn(n, 9, ch, generator=gen)
+    sub = torch.arange(11, n, 257)
+    xd, shd, wd = (t.to(device).requires_grad_(True) for t in (x, sh, w))
+    out = mod(xd, shd, wd)
+    gx, gsh, gw = torch.autograd.grad(out, (xd, shd, wd), ct.to(device))
+    T = ref_ops.dense_coupling(irr, irr, irr)
+    ref_out, (rgx, rgsh, rgw_sub) = ref_ops.dense_grads(ref_ops.dense_u1u, T, (x[sub], sh[sub], w), ct[sub])
+    assert_close(out[sub.to(device)], ref_out, 1e-5, "row mode out")
+    assert_close(gx[sub.to(device)], rgx, 1e-5, "row mode grad_x")
+    assert_close(gsh[sub.to(device)], rgsh, 1e-5, "row mode grad_sh", norm="max")   # sums over 64 channels x 83 terms
+    masked = torch.zeros_like(ct)
+    masked[sub] = ct[sub]
+    (gw_sub,) = torch.autograd.grad(mod(xd, shd, wd), (wd,), masked.to(device))
+    assert_close(gw_sub, rgw_sub, 1e-5, "row mode grad_w of the subset", norm="max")      # sum over 256 rows
+    # the full gradient is additive over two halves of the batch
+    half = n // 2
+    parts = []
+    for lo, hi in ((0, half), (half, n)):
+        ws = wd.detach().requires_grad_(True)
+        (gp,) = torch.autograd.grad(mod(xd[lo:hi].detach(), shd[lo:hi].detach(), ws), (ws,), ct[lo:hi].to(device))
+        parts.append(gp)
+    assert_close(gw, parts[0] + parts[1], 1e-5, "row mode grad_w additivity", norm="max")  # sums over 65536 rows

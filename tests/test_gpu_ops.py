@@ -71,6 +71,42 @@ def test_elementwise_ops_sweep(device, tables13, op, shared1, shared2, acc, chan
     assert_close(gy, rgy, 1e-5, f"{op} grad2")
 
 
+@pytest.mark.parametrize("table", ["info_Mij_fwd", "info_M_fwd"])
+@pytest.mark.parametrize("n,channels,dtype", [(1025, 97, torch.float32), (1500, 260, torch.float32),
+                                              (3000, 97, torch.float32), (1500, 130, torch.float64),
+                                              (2000, 64, torch.float32)])
+def test_row_sums_beyond_1024_rows(device, tables13, table, n, channels, dtype):
+    """Sums over the batch (``out_accumulated``, gradient of a shared operand) with more rows than the row-by-row
+    kernel has wavefronts (1024): shares of the rows are then uneven and the last wavefronts own none.  Heavy
+    (``info_Mij_fwd``) and light (``info_M_fwd``: one coefficient per row) tables, channel counts that take the
+    staged, the 16-byte and the one-channel-per-lane kernels, fp32 and fp64; against the CPU restatement."""
+    import equitorch_amd.nn.functional as F
+    mine, ref = tables13
+    info_m, info_r = getattr(mine, table).to(device), ref[table]
+    nnz = info_r["scale"].shape[0] if info_r["scale"] is not None else info_r["seg_out"][-1].item()
+    size = lambda idx: nnz if idx is None else int(idx.max()) + 1
+    d1, d2 = size(info_r["index1"]), size(info_r["index2"])
+    g = torch.Generator().manual_seed(n + channels)
+    x = torch.randn(n, d1, channels, generator=g, dtype=torch.float64).to(dtype)
+    tol = 1e-5 if dtype == torch.float32 else 1e-11
+    for op, oracle, y in (("mul", ref_ops.cpu_mul, torch.randn(n, d2, channels, generator=g, dtype=torch.float64)),
+                          ("inner", ref_ops.cpu_inner, torch.randn(n, d2, channels, generator=g, dtype=torch.float64)),
+                          ("vecsca", ref_ops.cpu_vecsca, torch.randn(n, d2, generator=g, dtype=torch.float64))):
+        y = y.to(dtype)
+        out = getattr(F, f"sparse_{op}")(x.to(device), y.to(device), info_m, out_accumulated=True)
+        # sums of n products of N(0,1) numbers: magnitude sqrt(n) * coefficients; compared norm-wise
+        assert_close(out, oracle(x.double(), y.double(), info_r, out_accumulated=True), tol, f"{op} row sum",
+                     norm="max")
+    # gradient of a shared second operand (the sum over rows happens in the backward launch)
+    w = torch.randn(d2, channels, generator=g, dtype=torch.float64).to(dtype)
+    wd = w.to(device).requires_grad_(True)
+    ct = torch.randn(n, info_r["seg_out"].shape[0] - 1, channels, generator=g, dtype=torch.float64).to(dtype)
+    (gw,) = torch.autograd.grad(F.sparse_mul(x.to(device), wd, info_m), (wd,), ct.to(device))
+    wr = w.double().requires_grad_(True)
+    (rgw,) = torch.autograd.grad(ref_ops.cpu_mul(x.double(), wr, info_r), (wr,), ct.double())
+    assert_close(gw, rgw, tol, "shared-operand gradient", norm="max")
+
+
 MAT = {  # name: (axes1, axes2, out axes, einsum)
     "outer": ("u", "w", "uw", "mab,{a}au,{b}bw->{o}muw"),
     "vecmat": ("u", "uw", "w", "mab,{a}au,{b}buw->{o}mw"),
