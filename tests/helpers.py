@@ -34,6 +34,12 @@ def assert_close(actual, expected, tol=1e-5, what="", norm="element"):
         assert err <= tol * scale, f"{what}: max abs err {err:.3e} > {tol:.0e} * {scale:.3e}"
 
 
+def stable_seed(*key) -> int:
+    """Seed derived from a test's parameters; the same in every process (``hash`` of a str is not)."""
+    import zlib
+    return zlib.crc32(repr(key).encode()) % 2 ** 31
+
+
 def unit_vectors(n, gen):
     v = torch.randn(n, 3, generator=gen)
     return v / v.norm(dim=-1, keepdim=True)

@@ -91,6 +91,8 @@ def test_message_passing_layer(device, fused_harmonics):
     mix_w, radial_w = (p.detach().double().cpu().requires_grad_(True) for p in params)
     ref = _reference(layer, xr, vr, src, dst, n_nodes, mix_w, radial_w)
     ref_grads = torch.autograd.grad(ref, [xr, vr, mix_w, radial_w], ct.double())
-    assert_close(out, ref, tol=2e-5, what="layer output")
+    assert_close(out, ref, tol=1e-5, what="layer output")
     for name, a, b in zip(("grad_x", "grad_edge_vec", "grad_mix_weight", "grad_radial_weight"), grads, ref_grads):
-        assert_close(a, b, tol=5e-5, what=name)
+        # the parameter gradients sum over all nodes / edges, grad_edge_vec over every channel and coefficient of
+        # the layer behind it: norm-wise; grad_x element-wise
+        assert_close(a, b, tol=1e-5, what=name, norm="element" if name == "grad_x" else "max")

@@ -47,7 +47,10 @@ def test_irreps_linear_matches_oracle(device, io, ii, kw, shared, dtype):
     gx, gw = _grads(out, (xd, wd), ct.to(device, dtype))
     tol = 1e-5 if dtype == torch.float32 else 1e-12
     for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
-        assert_close(a, b, tol=tol, what=f"{io}<-{ii} shared={shared} {name}")
+        # channel_norm as the reference passes it (channel_scale = C_in) gives terms of order 10^2 that cancel:
+        # that case is compared norm-wise in fp32
+        big = bool(kw.get("channel_norm")) and dtype == torch.float32
+        assert_close(a, b, tol=tol, what=f"{io}<-{ii} shared={shared} {name}", norm="max" if big else "element")
 
 
 @pytest.mark.parametrize("shared", [True, False])

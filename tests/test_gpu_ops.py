@@ -8,7 +8,7 @@ import itertools
 import pytest
 import torch
 
-from helpers import assert_close
+from helpers import assert_close, stable_seed
 from oracle import ref_ops, ref_tables
 
 pytestmark = pytest.mark.gpu
@@ -51,7 +51,7 @@ def test_elementwise_ops_sweep(device, tables13, op, shared1, shared2, acc, chan
     mine, ref = tables13
     oracle, ax1, ax2 = EW[op]
     info_m, info_r = mine.info_Mij_fwd.to(device), ref["info_Mij_fwd"]
-    g = torch.Generator().manual_seed(hash((op, shared1, shared2, acc, channels)) % 2 ** 31)
+    g = torch.Generator().manual_seed(stable_seed(op, shared1, shared2, acc, channels))
     n, d = 135, 15
 
     def mk(axes, shared):
@@ -82,7 +82,9 @@ def test_row_sums_beyond_1024_rows(device, tables13, table, n, channels, dtype):
     staged, the 16-byte and the one-channel-per-lane kernels, fp32 and fp64; against the CPU restatement."""
     import equitorch_amd.nn.functional as F
     mine, ref = tables13
-    info_m, info_r = getattr(mine, table).to(device), ref[table]
+    info_m, info_r = getattr(mine, table).to(device), dict(ref[table])
+    if info_r["scale"] is not None:
+        info_r["scale"] = info_r["scale"].float().double()      # the tables hold fp32 coefficients
     nnz = info_r["scale"].shape[0] if info_r["scale"] is not None else info_r["seg_out"][-1].item()
     size = lambda idx: nnz if idx is None else int(idx.max()) + 1
     d1, d2 = size(info_r["index1"]), size(info_r["index2"])
@@ -123,7 +125,7 @@ def test_matrix_ops_sweep(device, tables13, op, shared1, shared2, acc):
     ax1, ax2, axo, eq = MAT[op]
     info_m = mine.info_Mij_fwd.to(device)
     T = _dense_from_info(ref["info_Mij_fwd"], 15, 15)
-    g = torch.Generator().manual_seed(hash((op, shared1, shared2, acc)) % 2 ** 31)
+    g = torch.Generator().manual_seed(stable_seed(op, shared1, shared2, acc))
     n, d, U, W = 37, 15, 21, 13
     ext = {"u": U, "w": W}
 
@@ -138,12 +140,14 @@ def test_matrix_ops_sweep(device, tables13, op, shared1, shared2, acc):
     ref_out = torch.einsum(eq, T, xr, yr)
     if acc:
         ref_out = ref_out.sum(0)
-    assert_close(out, ref_out, 1e-5, f"{op} forward")
+    # results summed over the batch (accumulated output, gradient of a shared operand) and over up to 21 channels
+    # and ~40 coefficients per element: norm-wise; per-row results element-wise
+    assert_close(out, ref_out, 1e-5, f"{op} forward", norm="max" if acc else "element")
     ct = torch.randn(ref_out.shape, generator=g, dtype=torch.float64)
     gx, gy = torch.autograd.grad(out, (xd, yd), ct.float().to(device))
     rgx, rgy = torch.autograd.grad(ref_out, (xr, yr), ct.float().double())
-    assert_close(gx, rgx, 1e-5, f"{op} grad1")
-    assert_close(gy, rgy, 1e-5, f"{op} grad2")
+    assert_close(gx, rgx, 1e-5, f"{op} grad1", norm="max" if shared1 else "element")
+    assert_close(gy, rgy, 1e-5, f"{op} grad2", norm="max" if shared2 else "element")
 
 
 @pytest.mark.parametrize("scaled,indexed,segmented", [(True, True, True), (False, True, True), (True, False, True),
@@ -179,7 +183,7 @@ def test_tensor_product_family_vs_dense(device, mode, shared_w):
     infos = [t.to(device) for t in tp_infos(Irreps(io), Irreps(i1), Irreps(i2))[:3]]
     T = ref_ops.dense_coupling(io, i1, i2)
     p = T.shape[0]
-    g = torch.Generator().manual_seed(hash((mode, shared_w)) % 2 ** 31)
+    g = torch.Generator().manual_seed(stable_seed(mode, shared_w))
     n, u, v, w = 29, 12, 5, 9
     shapes = {  # mode: (x channels, y channels, weight channels, einsum)
         "u1v": ((u,), (), (u, w), "pmab,nau,nb,{W}puw->nmw"), "1vu": ((), (u,), (u, w), "pmab,na,nbu,{W}puw->nmw"),
@@ -194,7 +198,11 @@ def test_tensor_product_family_vs_dense(device, mode, shared_w):
     xd, yd, wd = (t.float().to(device).requires_grad_(True) for t in (x, y, wt))
     out = getattr(F, f"tensor_product_{mode}")(xd, yd, wd, *infos)
     xr, yr, wr = (t.float().double().requires_grad_(True) for t in (x, y, wt))
-    ref_out = torch.einsum(eq.format(W="" if shared_w else "n"), T, xr, yr, wr)
+    oracle = {"u1v": ref_ops.dense_u1v, "uvw": ref_ops.dense_uvw, "uuu": ref_ops.dense_uuu}.get(mode)
+    # the three members the oracle names directly (pinned on the CPU in tests/test_oracle_uv.py); the role-rotated
+    # siblings are the same contraction with the channel axes on other operands
+    ref_out = (oracle(T, xr, yr, wr) if oracle else
+               torch.einsum(eq.format(W="" if shared_w else "n"), T, xr, yr, wr))
     assert_close(out, ref_out, 1e-5, f"{mode} forward")
     ct = torch.randn(ref_out.shape, generator=g, dtype=torch.float64)
     grads = torch.autograd.grad(out, (xd, yd, wd), ct.float().to(device))
