@@ -26,12 +26,24 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
 
-# HBM bytes per launch of the dominant kernels on the edge workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# scaled by the same counters on the 1 GiB copy kernel (profiles/uvu_seg_sh2_edge_fwd_bwd.md): KiB per dispatch.
-MEASURED_TRAFFIC_KIB = {
-    "edge_fwd_bwd": 153878.6 * 2.0 + 193584.8 * 1.0,  # uvu_seg_bwd_kernel<TP_sh2,float,4,1>
-    "edge_fwd": 146857.7 * 2.0 + 9216.0 * 1.0,        # uvu_seg_fwd_kernel<TP_sh2,float,4>
-}
+def profiled_traffic(workload):
+    """HBM bytes per launch of the dominant kernel as a separate ``rocprofv3 --pmc FETCH_SIZE`` / ``WRITE_SIZE`` pair
+    of runs measured them (this run cannot read hardware counters itself): parsed from the committed summary
+    ``profiles/uvu_seg_sh2_edge_fwd_bwd.md`` (table row ``| backward | fetched MB | written MB | total MB | ...``).
+    Returns (bytes or None, where the figure comes from)."""
+    path = os.path.join(ROOT, "profiles", "uvu_seg_sh2_edge_fwd_bwd.md")
+    row = {"edge_fwd_bwd": "backward", "edge_fwd": "forward"}.get(workload)
+    try:
+        with open(path) as f:
+            for line in f:
+                cells = [c.strip() for c in line.strip().strip("|").split("|")]
+                if len(cells) >= 4 and cells[0] == row:
+                    return int(float(cells[3]) * 1e6), ("profiles/uvu_seg_sh2_edge_fwd_bwd.md (rocprofv3 --pmc "
+                                                        "FETCH_SIZE / WRITE_SIZE, separate runs, scaled by the copy kernel)")
+    except (OSError, ValueError):
+        pass
+    return None, "no counter run on record"
+
 
 WORKLOADS = {
     # name: (lmax, channels, nodes, edges)
@@ -357,7 +369,7 @@ def uvw_bench(args):
     sh = spherical_harmonics(vec / vec.norm(dim=-1, keepdim=True), lmax).bfloat16().to(dev)
     w = (torch.randn(mod.num_paths, ch, ch, generator=gen) / (ch * mod.num_paths) ** 0.5).bfloat16().to(dev)
     cfg = _uvw_mfma.uv_config_of(mod.tp_info_forward)
-    wt = _uvw_mfma.pack_weights(0, w)
+    wt = _uvw_mfma.pack_weights(0, w, cfg)
     s1 = int(mod.tp_info_forward.info_Mij_fwd.out_size)
     flops = 2.0 * n * s1 * ch * ch
     if backward:
@@ -381,7 +393,7 @@ def uvw_bench(args):
     torch.cuda.synchronize()
     k_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
     tf = flops / (k_ms * 1e-3) / 1e12
-    print(json.dumps({
+    return ({
         "metric": "uvw fwd TFLOP/s (lmax=3,C=128,bf16)", "value": round(flops / (ms_step * 1e-3) / 1e12, 2),
         "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
@@ -389,7 +401,7 @@ def uvw_bench(args):
                                f"bf16 in / fp32 accumulate / bf16 out, forward through SO3Linear('uv')"},
         "roofline": {"bound": "mfma", "kernel": "cgtp::uv_kernel<UV_sh3_d0,128>", "achieved": round(tf, 2),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "traffic": None, "algorithmic_flops": flops, "avg_ms": round(k_ms, 5)}}))
+                     "traffic": None, "algorithmic_flops": flops, "avg_ms": round(k_ms, 5)}})
 
 
 def uvw_fwd_bwd_bench(args, mod, x, sh, w, cfg, flops, irreps, gen):
@@ -420,18 +432,18 @@ def uvw_fwd_bwd_bench(args, mod, x, sh, w, cfg, flops, irreps, gen):
             evs.append((a, b))
         torch.cuda.synchronize()
         return sum(a.elapsed_time(b) for a, b in evs) / len(evs)
-    w0, w1 = _uvw_mfma.pack_weights(0, w), _uvw_mfma.pack_weights(1, w)
+    w0, w1 = _uvw_mfma.pack_weights(0, w, cfg), _uvw_mfma.pack_weights(1, w, cfg)
     kern = {
         "fwd_ms": timed(lambda: _uvw_mfma._apply(cfg, 0, x, sh, w0, d)),
         "grad_x_ms": timed(lambda: _uvw_mfma._apply(cfg, 1, ct, sh, w1, d)),
         "grad_sh_ms": timed(lambda: _uvw_mfma._grad_y(cfg, x, ct, w0, sh.shape[-1])),
-        "grad_w_ms": timed(lambda: _uvw_mfma._grad_w(cfg, x, sh, ct, w.shape[0])),
+        "grad_w_ms": timed(lambda: _uvw_mfma._grad_w(cfg, x, sh, ct)),
     }
     dom = max(kern, key=kern.get)
     tf = flops / (kern[dom] * 1e-3) / 1e12
     names = {"fwd_ms": "cgtp::uv_kernel<UV_sh3_d0,128>", "grad_x_ms": "cgtp::uv_kernel<UV_sh3_d1,128>",
              "grad_sh_ms": "cgtp::uv_gy_kernel<UV_sh3_gy,128>", "grad_w_ms": "cgtp::uv_gw_kernel<UV_sh3_gw>"}
-    print(json.dumps({
+    return ({
         "metric": "uvw fwd+bwd TFLOP/s (lmax=3,C=128,bf16)", "value": round(4 * flops / (ms_step * 1e-3) / 1e12, 2),
         "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
@@ -440,7 +452,7 @@ def uvw_fwd_bwd_bench(args, mod, x, sh, w, cfg, flops, irreps, gen):
         "roofline": {"bound": "mfma", "kernel": names[dom], "achieved": round(tf, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
                      "algorithmic_flops": flops, "avg_ms": round(kern[dom], 5)},
-        "kernels": {k: round(v, 5) for k, v in kern.items()}}))
+        "kernels": {k: round(v, 5) for k, v in kern.items()}})
 
 
 def make_inputs(lmax, ch, n_nodes, n_edges, n_rot, device, graph="uniform"):
@@ -552,7 +564,7 @@ def edge_rows_bench(args):
     }
     if not args.no_cpu_baseline:
         rec["cpu_baseline"] = cpu_baseline(inp, lmax, ch, n_nodes, min(args.cpu_sample_edges, 1024))
-    print(json.dumps(rec))
+    return rec
 
 
 def cpu_baseline(inp, lmax, ch, n_nodes, sample_edges, budget_s=12.0):
@@ -695,6 +707,8 @@ def main():
     ap.add_argument("--graph", default="uniform", choices=["uniform", "local"],
                     help="edge workloads: uniform random src/dst (BASELINE) or edges between nearby node ids")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="default workload: skip the compact records of the other BASELINE configurations")
     ap.add_argument("--cpu-sample-edges", type=int, default=16384)
     ap.add_argument("--pos-per-wave", type=int, default=0,
                     help="sorted positions per wavefront in the per-kernel timing (0 = library default)")
@@ -727,10 +741,10 @@ def main():
         layer_bench(args.steps, args.warmup)
         return
     if args.workload in ("uvw_fwd", "uvw_fwd_bwd"):
-        uvw_bench(args)
+        print(json.dumps(uvw_bench(args)))
         return
     if args.workload == "edge_l6_fwd_bwd":
-        edge_rows_bench(args)
+        print(json.dumps(edge_rows_bench(args)))
         return
 
     from equitorch_amd.nn import SO3Linear
@@ -802,6 +816,7 @@ def main():
     else:
         dom, dom_bytes, dom_ms = "cgtp::uvu_seg_fwd_kernel<TP_sh2,float,4>", fwd_bytes, fwd_avg
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    traffic, traffic_source = profiled_traffic(args.workload) if args.graph == "uniform" else (None, "not profiled")
 
     rec = {
         "metric": "edge-TP fwd+bwd Medges/s (lmax=2,C=64)" if backward else "edge-TP fwd Medges/s (lmax=2,C=64)",
@@ -813,7 +828,7 @@ def main():
                                + ("" if args.graph == "uniform" else f", {args.graph} graph")},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": int(MEASURED_TRAFFIC_KIB[args.workload] * 1024),
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "algorithmic_bytes": dom_bytes, "avg_ms": round(dom_ms, 5)},
         "kernels": {"fwd_avg_ms": round(fwd_avg, 5), "fwd_med_ms": round(fwd_med, 5),
                     "fwd_GBs": round(fwd_bytes / fwd_avg / 1e6, 1),
@@ -823,7 +838,94 @@ def main():
     }
     if not args.no_cpu_baseline:
         rec["cpu_baseline"] = cpu_baseline(inp, lmax, ch, n_nodes, min(args.cpu_sample_edges, n_edges))
+    if args.workload == "edge_fwd_bwd" and not args.no_configs and args.graph == "uniform":
+        del x, sh, ws, ct, plan
+        torch.cuda.empty_cache()
+        rec["configs"] = other_configs(args, rec)
     print(json.dumps(rec))
+
+
+def other_configs(args, headline):
+    """Compact records of the other BASELINE configurations, timed in the same run with a few steps each so that the
+    default command covers all five: [0] the CPU-reference module (B = 1024, C = 16, shared weight) on the oracle's
+    CPU path and on the GPU; [1] the edge forward; [3] the bf16 fully connected product; [4] the lmax = 6 edge step."""
+    import copy
+    out = {}
+    k = headline["kernels"]
+    out["cfg1_edge_fwd_lmax2_C64"] = {"kernel_ms": k["fwd_avg_ms"], "GBs": k["fwd_GBs"],
+                                      "hbm_frac": round(k["fwd_GBs"] / HBM_PEAK_GBS, 4),
+                                      "Medges_s": round(65536 / (k["fwd_avg_ms"] * 1e-3) / 1e6, 1)}
+    out["cfg0_uvu_B1024_C16_shared_w"] = config0_record(not args.no_cpu_baseline)
+    sub = copy.copy(args)
+    sub.steps, sub.warmup, sub.kernel_reps, sub.no_cpu_baseline = 10, 3, 12, True
+    sub.workload = "uvw_fwd_bwd"
+    r = uvw_bench(sub)
+    flops = r["roofline"]["algorithmic_flops"]
+    out["cfg3_uvw_bf16_B32768_C128"] = {
+        "step_ms": r["ms_per_step"], "step_TFLOPs": r["value"], "step_mfma_frac": round(r["value"] / MFMA_BF16_PEAK_TFLOPS, 4),
+        "fwd_ms": r["kernels"]["fwd_ms"], "fwd_TFLOPs": round(flops / (r["kernels"]["fwd_ms"] * 1e-3) / 1e12, 1),
+        "fwd_mfma_frac": round(flops / (r["kernels"]["fwd_ms"] * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+        "grad_x_ms": r["kernels"]["grad_x_ms"], "grad_sh_ms": r["kernels"]["grad_sh_ms"],
+        "grad_w_ms": r["kernels"]["grad_w_ms"]}
+    torch.cuda.empty_cache()
+    sub.workload, sub.steps, sub.warmup = "edge_l6_fwd_bwd", 4, 2
+    r = edge_rows_bench(sub)
+    out["cfg4_edge_fwd_bwd_lmax6_C32"] = {
+        "Medges_s": r["value"], "step_ms": r["ms_per_step"], "fwd_ms": r["kernels"]["fwd_ms"],
+        "bwd_ms": r["kernels"]["bwd_ms"], "bwd_hbm_frac": r["roofline"]["frac"],
+        "bwd_fp32_frac": r["roofline"]["fp32_vector"]["frac"], "fwd_TFLOPs": r["kernels"]["fwd_TFLOPs"]}
+    return out
+
+
+def config0_record(with_cpu):
+    """BASELINE configs[0]: ``SO3Linear('0e+1o+2e' x3, 16, 16, feature_mode='uu')`` with a shared weight on B = 1024
+    rows, forward + backward: the oracle's restatement of the reference CPU path (all host threads up to 16) next to
+    the same step on the GPU (wall time per step through the public API, launch-bound at this size)."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.utils._sh import spherical_harmonics
+    from oracle import ref_ops, ref_tables
+    irr, n, c = "0e+1o+2e", 1024, 16
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(n, 9, c, generator=gen)
+    v = torch.randn(n, 3, generator=gen)
+    sh = spherical_harmonics(v / v.norm(dim=-1, keepdim=True), 2)
+    w = torch.randn(11, c, generator=gen)
+    ct = torch.randn(n, 9, c, generator=gen)
+    rec = {}
+    dev = torch.device("cuda:0")
+    mod = SO3Linear(irr, irr, irr, c, c, internal_weights=False, feature_mode="uu").to(dev)
+    xd, shd, wd = (t.to(dev).requires_grad_(True) for t in (x, sh, w))
+    ctd = ct.to(dev)
+
+    def gstep():
+        return torch.autograd.grad(mod(xd, shd, wd), (xd, shd, wd), ctd)
+    for _ in range(5):
+        gstep()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(50):
+        gstep()
+    torch.cuda.synchronize()
+    rec["gpu_ms_per_step"] = round((time.perf_counter() - t0) / 50 * 1e3, 4)
+    if with_cpu:
+        threads = min(os.cpu_count() or 1, 16)
+        torch.set_num_threads(threads)
+        fwd, b1, b2, _ = ref_tables.tp_infos(irr, irr, irr)
+        fwd, b1, b2 = (ref_ops.tables_to_torch(t) for t in (fwd, b1, b2))
+
+        def cstep():
+            out, inter = ref_ops.cpu_u1u_forward(x, sh, w, fwd)
+            return out, ref_ops.cpu_u1u_backward(ct, x, sh, w, inter, fwd, b1, b2)
+        for _ in range(3):
+            cstep()
+        times = []
+        for _ in range(20):
+            t0 = time.perf_counter()
+            cstep()
+            times.append(time.perf_counter() - t0)
+        rec["cpu_ms_per_step"] = round(sorted(times)[10] * 1e3, 3)
+        rec["cpu"] = f"oracle ref_ops.cpu_u1u_forward/backward, median of 20, {threads} threads, {cpu_model()}"
+    return rec
 
 
 if __name__ == "__main__":

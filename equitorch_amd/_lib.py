@@ -57,7 +57,7 @@ class UvuArgs(C.Structure):
                 ("out", C.c_void_p),
                 ("grad_out", C.c_void_p), ("grad_x", C.c_void_p), ("grad_y", C.c_void_p),
                 ("grad_w", C.c_void_p), ("workspace", C.c_void_p), ("x_gather", C.c_void_p),
-                ("y_channels", C.c_int32), ("reserved_", C.c_int32)]
+                ("y_channels", C.c_int32), ("reserved_", C.c_int32), ("path_scale", C.c_void_p)]
 
 
 def _load():
@@ -73,6 +73,8 @@ def _load():
     lib.cgtp_tri_workspace_bytes.argtypes = [C.POINTER(TriArgs)]
     lib.cgtp_tri_validate.argtypes = [C.POINTER(TriArgs)]
     lib.cgtp_tri_contract.argtypes = [C.POINTER(TriArgs), C.c_void_p]
+    lib.cgtp_tri_contract_static.argtypes = [C.POINTER(TriArgs), C.c_void_p]
+    lib.cgtp_tri_static_scratch_bytes.restype = C.c_int64
     lib.cgtp_gen_validate.argtypes = [C.POINTER(GenArgs)]
     lib.cgtp_gen_contract.argtypes = [C.POINTER(GenArgs), C.c_void_p]
     lib.cgtp_segment_sum.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
@@ -83,6 +85,8 @@ def _load():
     lib.cgtp_uvu_describe.restype = C.c_uint64
     lib.cgtp_uvu_describe.argtypes = [C.c_int, C.POINTER(C.c_int32)]
     lib.cgtp_uvu_sh_degree.argtypes = [C.c_int]
+    lib.cgtp_uvu_table.argtypes = [C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_int32)]
+    lib.cgtp_uv_table.argtypes = [C.c_int, C.POINTER(C.c_int32), C.POINTER(C.c_float), C.POINTER(C.c_int32)]
     lib.cgtp_uvu_validate.argtypes = [C.POINTER(UvuArgs), C.c_int]
     lib.cgtp_uvu_workspace_bytes.restype = C.c_int64
     lib.cgtp_uvu_workspace_bytes.argtypes = [C.POINTER(UvuArgs), C.c_int]
@@ -93,13 +97,13 @@ def _load():
     _uv = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32,
            C.c_int32]
     lib.cgtp_uv_pack_weights.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
-                                         C.c_void_p]
+                                         C.c_void_p, C.c_void_p]
     lib.cgtp_uv_grad_y.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32,
                                    C.c_int32, C.c_int32, C.c_void_p]
     lib.cgtp_uv_grad_w_workspace_bytes.restype = C.c_int64
     lib.cgtp_uv_grad_w_workspace_bytes.argtypes = [C.c_int, C.c_int64, C.c_int32, C.c_int32]
     lib.cgtp_uv_grad_w.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
-                                   C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
+                                   C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
     lib.cgtp_uv_validate.argtypes = _uv
     lib.cgtp_uv_apply.argtypes = _uv + [C.c_void_p]
     lib.cgtp_sh_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_double, C.c_int,

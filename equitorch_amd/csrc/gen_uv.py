@@ -19,7 +19,7 @@ from collections import OrderedDict
 from .._tables import fingerprint, tp_coo
 from ..irreps import Irreps, irrep_segments
 from ..utils import tp_infos
-from .gen_uvu import _lit, _sh
+from .gen_uvu import _lit, _sh, table_arrays
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 
@@ -226,10 +226,13 @@ def main(out_dir: str = None) -> str:
             chunks.append(emit_direction(name, d, coo, seg_out, seg_in1))
         chunks.append(emit_direction(name, 0, coo, seg_out, seg_in1, gy=True))
         chunks.append(emit_gw(name, coo, seg_out, seg_in1))
+        chunks.append("\n".join([f"struct UV_{name}_tab {{",
+                                 f"  static constexpr int D1 = {coo.D1}, D2 = {coo.D2}, DO = {coo.DO}, P = {coo.P}, "
+                                 f"NNZ = {coo.coef.shape[0]};", *table_arrays(coo), "};"]))
         entries.append((name, fingerprint(coo), fingerprint(coo, "bf16"), fingerprint(coo, "f16")))
         chunks.append("")
     chunks.append("#define CGTP_FOREACH_UV_CONFIG(X) \\")
-    chunks.append(" \\\n".join(f"  X(UV_{n}_d0, UV_{n}_d1, UV_{n}_gy, UV_{n}_gw, 0x{fp:016x}ull, 0x{fb:016x}ull, 0x{fh:016x}ull, \"{n}\")"
+    chunks.append(" \\\n".join(f"  X(UV_{n}_d0, UV_{n}_d1, UV_{n}_gy, UV_{n}_gw, UV_{n}_tab, 0x{fp:016x}ull, 0x{fb:016x}ull, 0x{fh:016x}ull, \"{n}\")"
                               for n, fp, fb, fh in entries))
     chunks.append("")
     path = os.path.join(out_dir, "uv_configs.inc")

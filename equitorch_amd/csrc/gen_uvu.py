@@ -64,6 +64,16 @@ def sh_degree(irreps_in2) -> int:
     return len(ls) - 1 if ls == list(range(len(ls))) else -1
 
 
+def table_arrays(coo) -> list:
+    """The table itself as data members, so that the library can describe a compiled configuration to a caller
+    that wants to match another table against it: fp32 coefficients and (M, M1, M2, p) per entry, table order."""
+    T = coo.coef.shape[0]
+    coefs = ", ".join(_lit(coo.coef[t]) for t in range(T))
+    idx = ", ".join(f"{{{coo.M[t]}, {coo.M1[t]}, {coo.M2[t]}, {coo.p[t]}}}" for t in range(T))
+    return [f"  static constexpr float COEF[{T}] = {{{coefs}}};",
+            f"  static constexpr unsigned char IDX[{T}][4] = {{{idx}}};"]
+
+
 def emit_config(name: str, coo, sh_lmax: int = -1) -> str:
     T = coo.coef.shape[0]
     # (p, M) segments, path-major: the weight row of a path is needed only while that path is evaluated, and
@@ -83,6 +93,7 @@ def emit_config(name: str, coo, sh_lmax: int = -1) -> str:
     a(f"  static constexpr unsigned long long FINGERPRINT_F16 = 0x{fingerprint(coo, 'f16'):016x}ull;")
     a(f"  static constexpr const char* NAME = \"{name}\";")
     a(f"  static constexpr int SH_LMAX = {sh_lmax};  // second operand = harmonics of degrees 0..SH_LMAX (-1: not)")
+    L.extend(table_arrays(coo))
     # ---- forward: o[M] += w[p] * sum_t (coef_t y[M2_t]) x[M1_t]
     a("  // wload(p, w): fetch the V channels of weight path p")
     a("  template <typename T, int V, class WLoad>")

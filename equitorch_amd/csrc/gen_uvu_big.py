@@ -27,7 +27,7 @@ from collections import OrderedDict
 from .._tables import fingerprint, tp_coo
 from ..irreps import Irreps, irrep_segments
 from ..utils import tp_infos
-from .gen_uvu import _lit, _sh
+from .gen_uvu import _lit, _sh, table_arrays
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 RING = 8
@@ -42,6 +42,7 @@ CONFIGS = OrderedDict([
     ("so3_012_to_0123", ("0e+1e+2e+3e", "0e+1e+2e", "0e+1e+2e", {})),
     ("so3_2", ("0e+1e+2e", "0e+1e+2e", "0e+1e+2e", {})),
     ("so3_3", ("0e+1e+2e+3e", "0e+1e+2e+3e", "0e+1e+2e+3e", {})),
+    ("so3_4", ("0e+1e+2e+3e+4e", "0e+1e+2e+3e+4e", "0e+1e+2e+3e+4e", {})),
 ])
 
 
@@ -100,6 +101,7 @@ def emit_config(name: str, coo, seg_out, seg_in1) -> str:
     a(f"  static constexpr unsigned long long FINGERPRINT_BF16 = 0x{fingerprint(coo, 'bf16'):016x}ull;")
     a(f"  static constexpr unsigned long long FINGERPRINT_F16 = 0x{fingerprint(coo, 'f16'):016x}ull;")
     a(f"  static constexpr const char* NAME = \"{name}\";")
+    L.extend(table_arrays(coo))
 
     def ring_prologue():
         for k in range(min(RING, len(order))):

@@ -2,6 +2,7 @@
 // scale-segment reduction.  These kernels take the tables at run time, so they serve every irreps
 // configuration (and the reference's table-driven operator API); configurations with a compiled-in table
 // use the kernels of uvu_kernels.hip instead.
+#include <atomic>
 #include <cstddef>
 #include "cgtp_device.h"
 #include "cgtp_host.h"
@@ -534,11 +535,12 @@ const char* cgtp_status_string(int status) {
     case CGTP_ERR_LDS: return "table does not fit in LDS";
     case CGTP_ERR_LAUNCH: return "kernel launch failed";
     case CGTP_ERR_WORKSPACE: return "workspace missing or too small";
+    case CGTP_ERR_SCRATCH_LIMIT: return "partial results exceed the library's fixed scratch array";
     default: return "unknown status";
   }
 }
 
-int cgtp_version(void) { return 2; }
+int cgtp_version(void) { return 3; }
 
 int cgtp_abi_layout(int which, int64_t* out, int capacity) {
 #define CGTP_OFF(S, f) (int64_t) offsetof(S, f)
@@ -574,7 +576,7 @@ int cgtp_abi_layout(int which, int64_t* out, int capacity) {
                                 CGTP_OFF(cgtp_uvu_args, grad_x), CGTP_OFF(cgtp_uvu_args, grad_y),
                                 CGTP_OFF(cgtp_uvu_args, grad_w), CGTP_OFF(cgtp_uvu_args, workspace),
                                 CGTP_OFF(cgtp_uvu_args, x_gather), CGTP_OFF(cgtp_uvu_args, y_channels),
-                                CGTP_OFF(cgtp_uvu_args, reserved_)};
+                                CGTP_OFF(cgtp_uvu_args, reserved_), CGTP_OFF(cgtp_uvu_args, path_scale)};
 #undef CGTP_OFF
   const int64_t* tabs[] = {operand, tri, gen_operand, gen, uvu};
   const int counts[] = {(int)(sizeof(operand) / 8), (int)(sizeof(tri) / 8), (int)(sizeof(gen_operand) / 8),
@@ -616,6 +618,51 @@ int cgtp_tri_contract(const cgtp_tri_args* a, void* stream) {
   if (st != CGTP_OK) return st;
   return a->dtype == CGTP_F32 ? tri_launch<float>(a, lds, nw, (hipStream_t)stream)
                               : tri_launch<double>(a, lds, nw, (hipStream_t)stream);
+}
+
+// ---- the row-summing contraction for callers that cannot allocate ---------------------------------------------
+// The partial rows of a sum over rows live in a fixed device array instead of a caller-provided workspace.  Every
+// device that loads the library holds its own copy of the array at its own address; host code never uses the
+// array's name as a pointer, only the address hipGetSymbolAddress reports for the current device.
+constexpr int64_t kStaticScratchBytes = 16ll << 20;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static std::atomic<void*> g_scratch_of_device[kMaxDevices];
+
+static int static_scratch(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return CGTP_ERR_LAUNCH;
+  void* p = g_scratch_of_device[dev].load(std::memory_order_acquire);
+  if (!p) {
+    // first call on this device: ask the runtime where this device's copy of the array lives (no allocation: the
+    // array is part of the loaded code object).  Racing first calls obtain the same address.
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return CGTP_ERR_LAUNCH;
+    g_scratch_of_device[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return CGTP_OK;
+}
+
+int64_t cgtp_tri_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int cgtp_tri_contract_static(const cgtp_tri_args* a, void* stream) {
+  if (!a) return CGTP_ERR_NULL;
+  cgtp_tri_args b = *a;
+  b.workspace = nullptr;
+  if (b.reduce_rows) {
+    // validate with a placeholder first so that shape / dtype errors are reported as such
+    cgtp_tri_args probe = b;
+    probe.workspace = (void*)&probe;
+    int64_t lds = 0, nw = 0;
+    const int st = tri_check(&probe, &lds, &nw);
+    if (st != CGTP_OK) return st;
+    if (cgtp_tri_workspace_bytes(&b) > kStaticScratchBytes) return CGTP_ERR_SCRATCH_LIMIT;
+    void* p = nullptr;
+    const int rc = static_scratch(&p);
+    if (rc != CGTP_OK) return rc;
+    b.workspace = p;      // every partial row the second pass reads is written by the first: nothing to clear
+  }
+  return cgtp_tri_contract(&b, stream);
 }
 
 int cgtp_segment_sum(const void* in, const void* scale, const int64_t* index, const int64_t* seg, void* out,

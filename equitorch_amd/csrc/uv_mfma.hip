@@ -369,18 +369,22 @@ __global__ void __launch_bounds__(256, 1) uv_gw_kernel(const __bf16* __restrict_
     }
 }
 
-__global__ void uv_gw_reduce_kernel(const float* __restrict__ part, __bf16* __restrict__ gw, int64_t n_chunks, int64_t n) {
+// path_scale (one factor per weight path, or nullptr): the module's table is the compiled one with every path's
+// coefficients multiplied by that factor; per_path = elements of one path's weight matrix.
+__global__ void uv_gw_reduce_kernel(const float* __restrict__ part, __bf16* __restrict__ gw, int64_t n_chunks, int64_t n,
+                                    const float* __restrict__ path_scale, int64_t per_path) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   float s = 0.f;
   for (int64_t k = 0; k < n_chunks; ++k) s += part[k * n + i];
+  if (path_scale) s *= path_scale[i / per_path];
   gw[i] = (__bf16)s;
 }
 
 // packed[p][blk][t][k][lane = 16*q + r][e] = Wt[p][blk*32 + 8*(r/4) + 4*t + r%4][k*32 + 8*q + e], where
 // Wt[p][row][col] = w[p * rows * cols + row * row_stride + col * col_stride]; one thread per 16-byte piece.
 __global__ void uv_pack_kernel(const __bf16* __restrict__ w, __bf16* __restrict__ packed, int64_t n_pieces, int rows,
-                               int cols, int64_t row_stride, int64_t col_stride) {
+                               int cols, int64_t row_stride, int64_t col_stride, const float* __restrict__ path_scale) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n_pieces) return;
   const int ks = cols / 32, nblk = rows / 32;
@@ -396,6 +400,11 @@ __global__ void uv_pack_kernel(const __bf16* __restrict__ w, __bf16* __restrict_
   bf16x8 v;
 #pragma unroll
   for (int e = 0; e < 8; ++e) v[e] = src[e * col_stride];
+  if (path_scale) {      // folded in fp32, rounded to bf16 once
+    const float f = path_scale[p];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (__bf16)((float)v[e] * f);
+  }
   *reinterpret_cast<bf16x8*>(packed + i * 8) = v;
 }
 
@@ -411,11 +420,16 @@ struct UvEntry {
   UvGwFn gw_fn;
   int gw_max_rows;
   UvGwMeta gw_meta;  // order: paths with the most rows first, so that long workgroups start first
+  int dims[5];       // D1, D2, DO, P, NNZ
+  const float* coef;                 // the compiled table, table order
+  const unsigned char (*idx)[4];     // (M, M1, M2, p) per entry
 };
 
-template <class D0, class D1, class GY, class GW>
+template <class D0, class D1, class GY, class GW, class TAB>
 static UvEntry make_uv_entry(uint64_t fp, uint64_t fp_bf16, uint64_t fp_f16, const char* name) {
   UvEntry e;
+  e.dims[0] = TAB::D1; e.dims[1] = TAB::D2; e.dims[2] = TAB::DO; e.dims[3] = TAB::P; e.dims[4] = TAB::NNZ;
+  e.coef = TAB::COEF; e.idx = TAB::IDX;
   e.fingerprint = fp; e.fingerprint_rounded[0] = fp_bf16; e.fingerprint_rounded[1] = fp_f16; e.name = name;
   e.din[0] = D0::DIN; e.dout[0] = D0::DOUT; e.din[1] = D1::DIN; e.dout[1] = D1::DOUT;
   e.d2 = D0::D2; e.p = D0::P;
@@ -439,7 +453,8 @@ static UvEntry make_uv_entry(uint64_t fp, uint64_t fp_bf16, uint64_t fp_f16, con
 }
 
 static const UvEntry* uv_entries(int* count) {
-#define CGTP_X(D0, D1, GY, GW, FP, FP_BF16, FP_F16, NAME) make_uv_entry<D0, D1, GY, GW>(FP, FP_BF16, FP_F16, NAME),
+#define CGTP_X(D0, D1, GY, GW, TAB, FP, FP_BF16, FP_F16, NAME) \
+  make_uv_entry<D0, D1, GY, GW, TAB>(FP, FP_BF16, FP_F16, NAME),
   static const UvEntry table[] = {CGTP_FOREACH_UV_CONFIG(CGTP_X)};
 #undef CGTP_X
   *count = (int)(sizeof(table) / sizeof(table[0]));
@@ -493,8 +508,21 @@ int cgtp_uv_find_rounded(uint64_t fingerprint, int dtype) {
   return -1;
 }
 
+int cgtp_uv_table(int cfg, int32_t* dims, float* coef, int32_t* idx) {
+  int n = 0;
+  const UvEntry* t = uv_entries(&n);
+  if (cfg < 0 || cfg >= n) return -1;
+  const UvEntry& e = t[cfg];
+  for (int i = 0; dims && i < 5; ++i) dims[i] = e.dims[i];
+  for (int k = 0; k < e.dims[4]; ++k) {
+    if (coef) coef[k] = e.coef[k];
+    for (int j = 0; idx && j < 4; ++j) idx[4 * k + j] = e.idx[k][j];
+  }
+  return e.dims[4];
+}
+
 int cgtp_uv_pack_weights(int direction, const void* w, void* packed, int32_t n_paths, int32_t cin, int32_t cout,
-                         int32_t dtype, void* stream) {
+                         int32_t dtype, const float* path_scale, void* stream) {
   if (direction != 0 && direction != 1) return CGTP_ERR_SHAPE;
   if (dtype != CGTP_BF16) return CGTP_ERR_DTYPE;
   if (!w || !packed) return CGTP_ERR_NULL;
@@ -506,7 +534,8 @@ int cgtp_uv_pack_weights(int direction, const void* w, void* packed, int32_t n_p
   const int64_t n_pieces = (int64_t)n_paths * cin * cout / 8;
   const int64_t row_stride = direction == 0 ? 1 : cin, col_stride = direction == 0 ? cout : 1;
   hipLaunchKernelGGL(uv_pack_kernel, dim3((unsigned)((n_pieces + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                     (const __bf16*)w, (__bf16*)packed, n_pieces, (int)cout, (int)cin, row_stride, col_stride);
+                     (const __bf16*)w, (__bf16*)packed, n_pieces, (int)cout, (int)cin, row_stride, col_stride,
+                     path_scale);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 
@@ -563,7 +592,7 @@ int64_t cgtp_uv_grad_w_workspace_bytes(int cfg, int64_t n_rows, int32_t cin, int
 }
 
 int cgtp_uv_grad_w(int cfg, const void* x, const void* y, const void* g, void* gw, void* workspace, int64_t n_rows,
-                   int32_t cin, int32_t cout, int32_t dtype, void* stream) {
+                   int32_t cin, int32_t cout, int32_t dtype, const float* path_scale, void* stream) {
   int n = 0;
   const UvEntry* t = uv_entries(&n);
   if (cfg < 0 || cfg >= n) return CGTP_ERR_CONFIG;
@@ -579,7 +608,8 @@ int cgtp_uv_grad_w(int cfg, const void* x, const void* y, const void* g, void* g
   if (n_rows == 0) {  // no samples: the gradient is zero (the summation kernel over zero chunks writes it; a fill
                       // kernel rather than a memset, so that the call can be captured into a graph)
     hipLaunchKernelGGL(uv_gw_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, st,
-                       (const float*)nullptr, (__bf16*)gw, (int64_t)0, n_out);
+                       (const float*)nullptr, (__bf16*)gw, (int64_t)0, n_out, (const float*)nullptr,
+                       (int64_t)cin * cout);
     return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
   }
   if (!workspace) return CGTP_ERR_WORKSPACE;
@@ -592,7 +622,7 @@ int cgtp_uv_grad_w(int cfg, const void* x, const void* y, const void* g, void* g
   hipLaunchKernelGGL(e.gw_fn, dim3((unsigned)(n_chunks8 * e.p)), dim3(256), (size_t)lds, st, (const __bf16*)x,
                      (const __bf16*)y, (const __bf16*)g, (float*)workspace, n_rows, (int)cin, (int)cout, e.gw_meta);
   hipLaunchKernelGGL(uv_gw_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, st,
-                     (const float*)workspace, (__bf16*)gw, n_chunks, n_out);
+                     (const float*)workspace, (__bf16*)gw, n_chunks, n_out, path_scale, (int64_t)cin * cout);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 

@@ -11,7 +11,7 @@ namespace cgtp {
 // Lanes past the batch or the channel count re-read the last valid element and store nothing, so that every lane
 // runs the same code and the channel sum of grad_y can use full-width shuffles.
 // YC: the second operand carries channels, y (n_rows, D2, C); one value per lane like x.
-template <class TP, bool YC = false>
+template <class TP, bool PS, bool YC = false>
 __global__ void __launch_bounds__(256, 2) uvu_big_fwd_kernel(const UvuDev<float> a) {
   constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
   const Lanes L(a.lpe_log2);
@@ -30,14 +30,19 @@ __global__ void __launch_bounds__(256, 2) uvu_big_fwd_kernel(const UvuDev<float>
   for (int i = 0; i < D1; ++i) x[i] = a.x[(xr * D1 + i) * C + c];
   const float* wrow = a.w + (a.w_shared ? 0 : r) * P * C + c;
   float* orow = a.out + r * DO * C + c;
+  const float* __restrict__ ps = a.ps;
   TP::fwd(
-      x, y, [&](int p) __attribute__((always_inline)) { return __builtin_nontemporal_load(wrow + p * C); },
+      x, y,
+      [&](int p) __attribute__((always_inline)) {
+        const float w = __builtin_nontemporal_load(wrow + p * C);
+        if constexpr (PS) return w * ps[p]; else return w;
+      },
       [&](int m, float v) __attribute__((always_inline)) {
         if (live) __builtin_nontemporal_store(v, orow + m * C);
       });
 }
 
-template <class TP, int GW, bool YC = false>
+template <class TP, int GW, bool PS, bool YC = false>
 __global__ void __launch_bounds__(256, 2) uvu_big_bwd_kernel(const UvuDev<float> a, int64_t n_waves) {
   constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
   const Lanes L(a.lpe_log2);
@@ -65,16 +70,21 @@ __global__ void __launch_bounds__(256, 2) uvu_big_bwd_kernel(const UvuDev<float>
   float* gwrow = a.gw + r * P * C + c;
   float* gxrow = a.gx + r * D1 * C + c;
   const bool gx_live = a.gx && live;
+  const float* __restrict__ ps = a.ps;
   TP::bwd(
       [&](int i) __attribute__((always_inline)) { return xrow[i * C]; }, y,
-      [&](int p) __attribute__((always_inline)) { return __builtin_nontemporal_load(wrow + p * C); }, g,
+      [&](int p) __attribute__((always_inline)) {
+        const float w = __builtin_nontemporal_load(wrow + p * C);
+        if constexpr (PS) return w * ps[p]; else return w;
+      },
+      g,
       [&](int i, float v) __attribute__((always_inline)) {
         if (gx_live) __builtin_nontemporal_store(v, gxrow + i * C);
       },
       gy,
       [&](int p, float v) __attribute__((always_inline)) {
         if constexpr (GW == kGwStore) {
-          if (live) __builtin_nontemporal_store(v, gwrow + p * C);
+          if (live) __builtin_nontemporal_store(PS ? v * ps[p] : v, gwrow + p * C);
         }
       });
   if (YC) {
@@ -94,24 +104,32 @@ __global__ void __launch_bounds__(256, 2) uvu_big_bwd_kernel(const UvuDev<float>
   }
 }
 
-template <class TP>
+template <class TP, bool PS>
 static UvuBigEntry make_big_entry() {
   UvuBigEntry e;
   e.fingerprint = TP::FINGERPRINT;
   e.fingerprint_rounded[0] = TP::FINGERPRINT_BF16; e.fingerprint_rounded[1] = TP::FINGERPRINT_F16;
   e.dims[0] = TP::D1; e.dims[1] = TP::D2; e.dims[2] = TP::DO; e.dims[3] = TP::P; e.dims[4] = TP::NNZ;
   e.name = TP::NAME;
-  e.fwd = uvu_big_fwd_kernel<TP>;
-  e.bwd[kGwNone] = uvu_big_bwd_kernel<TP, kGwNone>;
-  e.bwd[kGwStore] = uvu_big_bwd_kernel<TP, kGwStore>;
-  e.fwd_yc = uvu_big_fwd_kernel<TP, true>;
-  e.bwd_yc[kGwNone] = uvu_big_bwd_kernel<TP, kGwNone, true>;
-  e.bwd_yc[kGwStore] = uvu_big_bwd_kernel<TP, kGwStore, true>;
+  e.coef = TP::COEF; e.idx = TP::IDX;
+  e.fwd = uvu_big_fwd_kernel<TP, PS>;
+  e.bwd[kGwNone] = uvu_big_bwd_kernel<TP, kGwNone, PS>;
+  e.bwd[kGwStore] = uvu_big_bwd_kernel<TP, kGwStore, PS>;
+  e.fwd_yc = uvu_big_fwd_kernel<TP, PS, true>;
+  e.bwd_yc[kGwNone] = uvu_big_bwd_kernel<TP, kGwNone, PS, true>;
+  e.bwd_yc[kGwStore] = uvu_big_bwd_kernel<TP, kGwStore, PS, true>;
   return e;
 }
 
+// Two sets, as for the register-resident kernels: uvu_big_ps.hip includes this file with CGTP_UVU_PS_UNIT defined and
+// provides the set that applies one factor per weight path.
+#ifdef CGTP_UVU_PS_UNIT
+const UvuBigEntry* uvu_big_entries_scaled(int* count) {
+#define CGTP_X(TP) make_big_entry<TP, true>(),
+#else
 const UvuBigEntry* uvu_big_entries(int* count) {
-#define CGTP_X(TP) make_big_entry<TP>(),
+#define CGTP_X(TP) make_big_entry<TP, false>(),
+#endif
   static const UvuBigEntry table[] = {CGTP_FOREACH_UVU_BIG_CONFIG(CGTP_X)};
 #undef CGTP_X
   *count = (int)(sizeof(table) / sizeof(table[0]));

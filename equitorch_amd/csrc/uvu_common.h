@@ -27,6 +27,7 @@ struct UvuDev {
   int64_t n_rows, n_seg;
   int C, lpe_log2, w_shared, pos_per_wave;
   int y_vec;  // segment mode: y holds edge vectors (kYUnitVector / kYRawVector) instead of harmonics
+  const T* ps;  // optional factor of every weight path (the caller's table = compiled table x ps[p]); nullptr = ones
 };
 
 // Segment mode: which range of the sorted edge list a wavefront takes.  Workgroups are dispatched to the 8 XCDs
@@ -66,6 +67,8 @@ struct UvuBigEntry {
   uint64_t fingerprint_rounded[2];  // of the table rounded to bf16 / fp16
   int dims[5];
   const char* name;
+  const float* coef;                // the compiled table, table order
+  const unsigned char (*idx)[4];    // (M, M1, M2, p) per entry
   void (*fwd)(const UvuDev<float>);
   void (*bwd[2])(const UvuDev<float>, int64_t);  // [kGwNone, kGwStore]
   // the same with a channelled second operand, y (n_rows, D2, C) ("uuu"): grad_y is then per channel as well
@@ -73,5 +76,6 @@ struct UvuBigEntry {
   void (*bwd_yc[2])(const UvuDev<float>, int64_t);
 };
 const UvuBigEntry* uvu_big_entries(int* count);
+const UvuBigEntry* uvu_big_entries_scaled(int* count);  // the same kernels applying UvuDev::ps
 
 }  // namespace cgtp

@@ -28,7 +28,7 @@ __device__ __forceinline__ void zero_rows(T (&a)[D][V]) {
 }
 
 // ---- row mode ------------------------------------------------------------------------------------------------
-template <class TP, typename T, int V>
+template <class TP, typename T, int V, bool PS>
 __global__ void __launch_bounds__(256) uvu_fwd_kernel(const UvuDev<T> a) {
   constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
   const Lanes L(a.lpe_log2);
@@ -48,6 +48,14 @@ __global__ void __launch_bounds__(256) uvu_fwd_kernel(const UvuDev<T> a) {
   T w[P][V];  // every weight row is requested before the arithmetic starts: maximal memory-level parallelism
 #pragma unroll
   for (int p = 0; p < P; ++p) load_vec_stream<T, V>(w[p], wrow + p * C);
+  if constexpr (PS) {  // this instantiation applies one factor per weight path
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      const T f = a.ps[p];
+#pragma unroll
+      for (int v = 0; v < V; ++v) w[p][v] *= f;
+    }
+  }
   zero_rows(acc);
   TP::template fwd<T, V>(x, y, [&](int p, T (&wp)[V]) {
 #pragma unroll
@@ -58,7 +66,7 @@ __global__ void __launch_bounds__(256) uvu_fwd_kernel(const UvuDev<T> a) {
 }
 
 
-template <class TP, typename T, int V, int GW>
+template <class TP, typename T, int V, int GW, bool PS>
 __global__ void __launch_bounds__(256, 2) uvu_bwd_kernel(const UvuDev<T> a, int64_t n_waves) {
   constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
   const Lanes L(a.lpe_log2);
@@ -90,6 +98,14 @@ __global__ void __launch_bounds__(256, 2) uvu_bwd_kernel(const UvuDev<T> a, int6
       T w[P][V];  // every weight row is requested before the arithmetic starts: maximal memory-level parallelism
 #pragma unroll
       for (int p = 0; p < P; ++p) load_vec_stream<T, V>(w[p], wrow + p * C);
+      if constexpr (PS) {  // this instantiation applies one factor per weight path
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+          const T f = a.ps[p];
+#pragma unroll
+          for (int v = 0; v < V; ++v) w[p][v] *= f;
+        }
+      }
       T* gwrow = a.gw + r * P * C + c0;
       TP::template bwd<T, V>(
           x, y, [&](int p, T (&wp)[V]) {
@@ -101,7 +117,15 @@ __global__ void __launch_bounds__(256, 2) uvu_bwd_kernel(const UvuDev<T> a, int6
 #pragma unroll
               for (int v = 0; v < V; ++v) gwacc[p][v] += gwp[v];
             } else if constexpr (GW == kGwStore) {
-              store_vec_stream<T, V>(gwrow + p * C, gwp);
+              if constexpr (PS) {
+                const T f = a.ps[p];
+                T sc[V];
+#pragma unroll
+                for (int v = 0; v < V; ++v) sc[v] = gwp[v] * f;
+                store_vec_stream<T, V>(gwrow + p * C, sc);
+              } else {
+                store_vec_stream<T, V>(gwrow + p * C, gwp);
+              }
             }
           });
       if (a.gx) {
@@ -122,7 +146,10 @@ __global__ void __launch_bounds__(256, 2) uvu_bwd_kernel(const UvuDev<T> a, int6
 #pragma unroll
     for (int p = 0; p < P; ++p)
 #pragma unroll
-      for (int v = 0; v < V; ++v) gwacc[p][v] = cross_group_sum(gwacc[p][v], L.lpe);
+      for (int v = 0; v < V; ++v) {
+        gwacc[p][v] = cross_group_sum(gwacc[p][v], L.lpe);
+        if constexpr (PS) gwacc[p][v] *= a.ps[p];
+      }
     if (L.slot == 0 && cok) {
 #pragma unroll
       for (int p = 0; p < P; ++p) store_vec<T, V>(a.wsw + (wave * P + p) * C + c0, gwacc[p]);
@@ -250,7 +277,7 @@ __device__ __forceinline__ void seg_finish(SegStep& st, T (&acc)[D][V], T* __res
 }
 
 // YV: the second operand is an edge vector; its harmonics are evaluated here (sh_device.h).
-template <class TP, typename T, int V, bool YV = false>
+template <class TP, typename T, int V, bool PS, bool YV = false>
 __global__ void __launch_bounds__(256) uvu_seg_fwd_kernel(const UvuDev<T> a, int64_t n_waves) {
   constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
   const Lanes L(a.lpe_log2);
@@ -286,6 +313,14 @@ __global__ void __launch_bounds__(256) uvu_seg_fwd_kernel(const UvuDev<T> a, int
         T w[P][V];  // every weight row is requested before the arithmetic starts: maximal memory-level parallelism
 #pragma unroll
         for (int p = 0; p < P; ++p) load_vec_stream<T, V>(w[p], wrow + p * C);
+        if constexpr (PS) {  // this instantiation applies one factor per weight path
+#pragma unroll
+          for (int p = 0; p < P; ++p) {
+            const T f = a.ps[p];
+#pragma unroll
+            for (int v = 0; v < V; ++v) w[p][v] *= f;
+          }
+        }
         TP::template fwd<T, V>(x, y, [&](int p, T (&wp)[V]) {
 #pragma unroll
           for (int v = 0; v < V; ++v) wp[v] = w[p][v];
@@ -297,7 +332,7 @@ __global__ void __launch_bounds__(256) uvu_seg_fwd_kernel(const UvuDev<T> a, int
   seg_finish<T, DO, V>(st, acc, a.out, a.ws, wave, R, L, cok, C, c0);
 }
 
-template <class TP, typename T, int V, int GW, bool YV = false>
+template <class TP, typename T, int V, int GW, bool PS, bool YV = false>
 __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, int64_t n_waves) {
   constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
   const Lanes L(a.lpe_log2);
@@ -351,6 +386,14 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, 
         T w[P][V];  // every weight row is requested before the arithmetic starts: maximal memory-level parallelism
 #pragma unroll
         for (int p = 0; p < P; ++p) load_vec_stream<T, V>(w[p], wrow + p * C);
+        if constexpr (PS) {  // this instantiation applies one factor per weight path
+#pragma unroll
+          for (int p = 0; p < P; ++p) {
+            const T f = a.ps[p];
+#pragma unroll
+            for (int v = 0; v < V; ++v) w[p][v] *= f;
+          }
+        }
         T* gwrow = a.gw + e * P * C + c0;
         TP::template bwd<T, V>(
             x, y, [&](int p, T (&wp)[V]) {
@@ -362,7 +405,15 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, 
 #pragma unroll
                 for (int v = 0; v < V; ++v) gwacc[p][v] += gwp[v];
               } else if constexpr (GW == kGwStore) {
-                store_vec_stream<T, V>(gwrow + p * C, gwp);
+                if constexpr (PS) {
+                  const T f = a.ps[p];
+                  T sc[V];
+#pragma unroll
+                  for (int v = 0; v < V; ++v) sc[v] = gwp[v] * f;
+                  store_vec_stream<T, V>(gwrow + p * C, sc);
+                } else {
+                  store_vec_stream<T, V>(gwrow + p * C, gwp);
+                }
               }
             });
       }
@@ -392,7 +443,10 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, 
 #pragma unroll
     for (int p = 0; p < P; ++p)
 #pragma unroll
-      for (int v = 0; v < V; ++v) gwacc[p][v] = cross_group_sum(gwacc[p][v], L.lpe);
+      for (int v = 0; v < V; ++v) {
+        gwacc[p][v] = cross_group_sum(gwacc[p][v], L.lpe);
+        if constexpr (PS) gwacc[p][v] *= a.ps[p];
+      }
     if (L.slot == 0 && cok) {
 #pragma unroll
       for (int p = 0; p < P; ++p) store_vec<T, V>(a.wsw + (wave * P + p) * C + c0, gwacc[p]);
@@ -445,6 +499,8 @@ struct UvuEntry {
   uint64_t fingerprint_rounded[2];  // of the table rounded to bf16 / fp16 (a module converted to that type)
   int dims[5];
   const char* name;
+  const float* coef;               // the compiled table, table order
+  const unsigned char (*idx)[4];   // (M, M1, M2, p) per entry
   int v_fwd, v_bwd;         // channels per lane of the vector paths
   FwdFn<T> fwd[2];          // [vector path]
   WaveFn<T> bwd[2][3];      // [vector path][weight-gradient mode]
@@ -469,7 +525,7 @@ constexpr int v_fwd() { return pick_v<T>(TP::D1 + TP::P + TP::DO, TP::D2, 150); 
 template <class TP, typename T>
 constexpr int v_bwd() { return pick_v<T>(2 * TP::D1 + TP::DO + 2 * TP::P, 2 * TP::D2, 236); }
 
-template <class TP, typename T>
+template <class TP, typename T, bool PS>
 static UvuEntry<T> make_entry() {
   constexpr int VF = v_fwd<TP, T>(), VB = v_bwd<TP, T>();
   UvuEntry<T> e;
@@ -477,34 +533,35 @@ static UvuEntry<T> make_entry() {
   e.fingerprint_rounded[0] = TP::FINGERPRINT_BF16; e.fingerprint_rounded[1] = TP::FINGERPRINT_F16;
   e.dims[0] = TP::D1; e.dims[1] = TP::D2; e.dims[2] = TP::DO; e.dims[3] = TP::P; e.dims[4] = TP::NNZ;
   e.name = TP::NAME;
+  e.coef = TP::COEF; e.idx = TP::IDX;
   e.v_fwd = VF; e.v_bwd = VB;
-  e.fwd[0] = uvu_fwd_kernel<TP, T, 1>;
-  e.fwd[1] = uvu_fwd_kernel<TP, T, VF>;
-  e.bwd[0][0] = uvu_bwd_kernel<TP, T, 1, kGwNone>;
-  e.bwd[0][1] = uvu_bwd_kernel<TP, T, 1, kGwStore>;
-  e.bwd[0][2] = uvu_bwd_kernel<TP, T, 1, kGwReduce>;
-  e.bwd[1][0] = uvu_bwd_kernel<TP, T, VB, kGwNone>;
-  e.bwd[1][1] = uvu_bwd_kernel<TP, T, VB, kGwStore>;
-  e.bwd[1][2] = uvu_bwd_kernel<TP, T, VB, kGwReduce>;
-  e.seg_fwd[0] = uvu_seg_fwd_kernel<TP, T, 1>;
-  e.seg_fwd[1] = uvu_seg_fwd_kernel<TP, T, VF>;
-  e.seg_bwd[0][0] = uvu_seg_bwd_kernel<TP, T, 1, kGwNone>;
-  e.seg_bwd[0][1] = uvu_seg_bwd_kernel<TP, T, 1, kGwStore>;
-  e.seg_bwd[0][2] = uvu_seg_bwd_kernel<TP, T, 1, kGwReduce>;
-  e.seg_bwd[1][0] = uvu_seg_bwd_kernel<TP, T, VB, kGwNone>;
-  e.seg_bwd[1][1] = uvu_seg_bwd_kernel<TP, T, VB, kGwStore>;
-  e.seg_bwd[1][2] = uvu_seg_bwd_kernel<TP, T, VB, kGwReduce>;
+  e.fwd[0] = uvu_fwd_kernel<TP, T, 1, PS>;
+  e.fwd[1] = uvu_fwd_kernel<TP, T, VF, PS>;
+  e.bwd[0][0] = uvu_bwd_kernel<TP, T, 1, kGwNone, PS>;
+  e.bwd[0][1] = uvu_bwd_kernel<TP, T, 1, kGwStore, PS>;
+  e.bwd[0][2] = uvu_bwd_kernel<TP, T, 1, kGwReduce, PS>;
+  e.bwd[1][0] = uvu_bwd_kernel<TP, T, VB, kGwNone, PS>;
+  e.bwd[1][1] = uvu_bwd_kernel<TP, T, VB, kGwStore, PS>;
+  e.bwd[1][2] = uvu_bwd_kernel<TP, T, VB, kGwReduce, PS>;
+  e.seg_fwd[0] = uvu_seg_fwd_kernel<TP, T, 1, PS>;
+  e.seg_fwd[1] = uvu_seg_fwd_kernel<TP, T, VF, PS>;
+  e.seg_bwd[0][0] = uvu_seg_bwd_kernel<TP, T, 1, kGwNone, PS>;
+  e.seg_bwd[0][1] = uvu_seg_bwd_kernel<TP, T, 1, kGwStore, PS>;
+  e.seg_bwd[0][2] = uvu_seg_bwd_kernel<TP, T, 1, kGwReduce, PS>;
+  e.seg_bwd[1][0] = uvu_seg_bwd_kernel<TP, T, VB, kGwNone, PS>;
+  e.seg_bwd[1][1] = uvu_seg_bwd_kernel<TP, T, VB, kGwStore, PS>;
+  e.seg_bwd[1][2] = uvu_seg_bwd_kernel<TP, T, VB, kGwReduce, PS>;
   e.sh_lmax = TP::SH_LMAX;
   if constexpr (TP::SH_LMAX >= 0) {
     static_assert((TP::SH_LMAX + 1) * (TP::SH_LMAX + 1) == TP::D2, "harmonics layout");
-    e.seg_fwd_vec[0] = uvu_seg_fwd_kernel<TP, T, 1, true>;
-    e.seg_fwd_vec[1] = uvu_seg_fwd_kernel<TP, T, VF, true>;
-    e.seg_bwd_vec[0][0] = uvu_seg_bwd_kernel<TP, T, 1, kGwNone, true>;
-    e.seg_bwd_vec[0][1] = uvu_seg_bwd_kernel<TP, T, 1, kGwStore, true>;
-    e.seg_bwd_vec[0][2] = uvu_seg_bwd_kernel<TP, T, 1, kGwReduce, true>;
-    e.seg_bwd_vec[1][0] = uvu_seg_bwd_kernel<TP, T, VB, kGwNone, true>;
-    e.seg_bwd_vec[1][1] = uvu_seg_bwd_kernel<TP, T, VB, kGwStore, true>;
-    e.seg_bwd_vec[1][2] = uvu_seg_bwd_kernel<TP, T, VB, kGwReduce, true>;
+    e.seg_fwd_vec[0] = uvu_seg_fwd_kernel<TP, T, 1, PS, true>;
+    e.seg_fwd_vec[1] = uvu_seg_fwd_kernel<TP, T, VF, PS, true>;
+    e.seg_bwd_vec[0][0] = uvu_seg_bwd_kernel<TP, T, 1, kGwNone, PS, true>;
+    e.seg_bwd_vec[0][1] = uvu_seg_bwd_kernel<TP, T, 1, kGwStore, PS, true>;
+    e.seg_bwd_vec[0][2] = uvu_seg_bwd_kernel<TP, T, 1, kGwReduce, PS, true>;
+    e.seg_bwd_vec[1][0] = uvu_seg_bwd_kernel<TP, T, VB, kGwNone, PS, true>;
+    e.seg_bwd_vec[1][1] = uvu_seg_bwd_kernel<TP, T, VB, kGwStore, PS, true>;
+    e.seg_bwd_vec[1][2] = uvu_seg_bwd_kernel<TP, T, VB, kGwReduce, PS, true>;
   } else {
     for (auto& f : e.seg_fwd_vec) f = nullptr;
     for (auto& r : e.seg_bwd_vec)
@@ -513,14 +570,33 @@ static UvuEntry<T> make_entry() {
   return e;
 }
 
-template <typename T>
-static const UvuEntry<T>* entries(int* count) {
-#define CGTP_X(TP) make_entry<TP, T>(),
+// The kernels exist twice: as they are for a table equal to the compiled one, and with one factor per weight path
+// applied to the weights and their gradient (PS).  The second set is instantiated in its own translation unit
+// (uvu_kernels_ps.hip includes this file with CGTP_UVU_PS_UNIT defined) so that both compile side by side.
+template <typename T, bool PS>
+static const UvuEntry<T>* make_entries(int* count) {
+#define CGTP_X(TP) make_entry<TP, T, PS>(),
   static const UvuEntry<T> table[] = {CGTP_FOREACH_UVU_CONFIG(CGTP_X)};
 #undef CGTP_X
   *count = (int)(sizeof(table) / sizeof(table[0]));
   return table;
 }
+const UvuEntry<float>* uvu_entries_scaled_f32(int* count);
+const UvuEntry<double>* uvu_entries_scaled_f64(int* count);
+
+#ifdef CGTP_UVU_PS_UNIT
+const UvuEntry<float>* uvu_entries_scaled_f32(int* count) { return make_entries<float, true>(count); }
+const UvuEntry<double>* uvu_entries_scaled_f64(int* count) { return make_entries<double, true>(count); }
+}  // namespace cgtp
+#else
+template <typename T>
+static const UvuEntry<T>* entries(int* count) { return make_entries<T, false>(count); }
+template <typename T>
+static const UvuEntry<T>* entries_scaled(int* count);
+template <>
+const UvuEntry<float>* entries_scaled<float>(int* count) { return uvu_entries_scaled_f32(count); }
+template <>
+const UvuEntry<double>* entries_scaled<double>(int* count) { return uvu_entries_scaled_f64(count); }
 
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -649,6 +725,7 @@ static UvuDev<T> to_dev(const cgtp_uvu_args* a, const UvuPlan& plan) {
   d.n_rows = a->n_rows; d.n_seg = a->n_seg;
   d.C = a->C; d.lpe_log2 = plan.lpe_log2; d.w_shared = a->w_shared; d.pos_per_wave = plan.pos_per_wave;
   d.y_vec = a->y_vec;
+  d.ps = (const T*)a->path_scale;
   return d;
 }
 
@@ -669,7 +746,7 @@ static int launch_fixup(T* rows, const UvuDev<T>& d, int64_t row_len, hipStream_
 
 static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward, hipStream_t stream) {
   int n_big = 0;
-  const UvuBigEntry& e = uvu_big_entries(&n_big)[plan.big_idx];
+  const UvuBigEntry& e = (a->path_scale ? uvu_big_entries_scaled(&n_big) : uvu_big_entries(&n_big))[plan.big_idx];
   const bool wred = backward && a->w_shared && a->grad_w;
   const int64_t w_elems = (int64_t)e.dims[3] * a->C;
   if (plan.n_waves == 0) {
@@ -707,7 +784,7 @@ static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward,
 template <typename T>
 static int launch_fwd(const cgtp_uvu_args* a, const UvuPlan& plan, hipStream_t stream) {
   int n = 0;
-  const UvuEntry<T>& e = entries<T>(&n)[a->cfg];
+  const UvuEntry<T>& e = (a->path_scale ? entries_scaled<T>(&n) : entries<T>(&n))[a->cfg];
   const UvuDev<T> d = to_dev<T>(a, plan);
   const int vi = plan.V > 1;
   if (a->n_seg > 0) {
@@ -728,7 +805,7 @@ static int launch_fwd(const cgtp_uvu_args* a, const UvuPlan& plan, hipStream_t s
 template <typename T>
 static int launch_bwd(const cgtp_uvu_args* a, const UvuPlan& plan, hipStream_t stream) {
   int n = 0;
-  const UvuEntry<T>& e = entries<T>(&n)[a->cfg];
+  const UvuEntry<T>& e = (a->path_scale ? entries_scaled<T>(&n) : entries<T>(&n))[a->cfg];
   const UvuDev<T> d = to_dev<T>(a, plan);
   const int vi = plan.V > 1;
   const bool seg = a->n_seg > 0;
@@ -799,6 +876,21 @@ uint64_t cgtp_uvu_describe(int cfg, int32_t* dims) {
   return cfg < n ? t[cfg].fingerprint : b[cfg - n].fingerprint;
 }
 
+int cgtp_uvu_table(int cfg, float* coef, int32_t* idx) {
+  int n = 0, n_big = 0;
+  const UvuEntry<float>* t = entries<float>(&n);
+  const UvuBigEntry* b = uvu_big_entries(&n_big);
+  if (cfg < 0 || cfg >= n + n_big) return -1;
+  const int nnz = cfg < n ? t[cfg].dims[4] : b[cfg - n].dims[4];
+  const float* c = cfg < n ? t[cfg].coef : b[cfg - n].coef;
+  const unsigned char (*ix)[4] = cfg < n ? t[cfg].idx : b[cfg - n].idx;
+  for (int k = 0; k < nnz; ++k) {
+    if (coef) coef[k] = c[k];
+    for (int j = 0; idx && j < 4; ++j) idx[4 * k + j] = ix[k][j];
+  }
+  return nnz;
+}
+
 int cgtp_uvu_sh_degree(int cfg) {
   int n = 0;
   const UvuEntry<float>* t = entries<float>(&n);
@@ -835,3 +927,4 @@ int cgtp_uvu_bwd(const cgtp_uvu_args* a, void* stream) {
 }
 
 }  // extern "C"
+#endif  // CGTP_UVU_PS_UNIT

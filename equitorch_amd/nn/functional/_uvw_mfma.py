@@ -1,6 +1,5 @@
 """Dispatch of the fully connected ("uv") product to the bf16 matrix-core kernel (``cgtp_uv_apply``)."""
 import ctypes as C
-import weakref
 from typing import Optional
 
 import torch
@@ -15,33 +14,17 @@ from ._tri import spec_from_tp_info, tri
 uv_config_of = kernels.uv_config_of
 
 
-_packed = {}  # (id(w), direction) -> (weakref to w, its version counter, its data pointer, packed copy)
-
-
-def pack_weights(direction: int, w: Tensor) -> Tensor:
-    """W as stored by the module, (P, C_in, C_out), rewritten in the fragment order the kernel reads.  The packed
-    copy is kept until the weight tensor is modified in place (its version counter moves), is given other storage,
-    or dies."""
-    key = (id(w), direction)
-    hit = _packed.get(key)
-    if hit is not None and hit[0]() is w and hit[1] == w._version and hit[2] == w.data_ptr():
-        return hit[3]
-    packed = _pack(direction, w)
-    if len(_packed) >= 64:
-        for k in [k for k, v in _packed.items() if v[0]() is None]:
-            del _packed[k]
-        if len(_packed) >= 64:
-            _packed.clear()
-    _packed[key] = (weakref.ref(w), w._version, w.data_ptr(), packed)
-    return packed
-
-
-def _pack(direction: int, w: Tensor) -> Tensor:
-    w = w.contiguous()
+def pack_weights(direction: int, w: Tensor, cfg) -> Tensor:
+    """W as stored by the module, (P, C_in, C_out), rewritten in the fragment order the kernel reads, with the
+    per-path factors of ``cfg`` folded in (fp32 product, rounded to bf16 once).  Packed anew on every call: one small
+    launch, and no cached copy that an in-place update through ``w.data`` could leave stale."""
+    w = kernels.expand_paths(w, cfg, 0).contiguous()
     cin, cout = (w.shape[1], w.shape[2]) if direction == 0 else (w.shape[2], w.shape[1])
     packed = torch.empty_like(w)
+    scale = cfg.scale_tensor(torch.float32, w.device) if isinstance(cfg, kernels.Cfg) else None
     _lib.check(_lib.lib.cgtp_uv_pack_weights(direction, w.data_ptr(), packed.data_ptr(), w.shape[0], cin, cout,
-                                             _lib.BF16, _lib.stream_ptr(w.device)), "cgtp_uv_pack_weights")
+                                             _lib.BF16, _lib.ptr(scale), _lib.stream_ptr(w.device)),
+               "cgtp_uv_pack_weights")
     return packed
 
 
@@ -65,16 +48,19 @@ def _grad_y(cfg: int, x: Tensor, g: Tensor, wp: Tensor, d2: int) -> Tensor:
     return gy
 
 
-def _grad_w(cfg: int, x: Tensor, y: Tensor, g: Tensor, n_paths: int) -> Tensor:
-    """Gradient w.r.t. the shared weight, (P, C_in, C_out)."""
+def _grad_w(cfg: int, x: Tensor, y: Tensor, g: Tensor) -> Tensor:
+    """Gradient w.r.t. the shared weight, (P, C_in, C_out) over the caller's own paths."""
     n, _, cin = x.shape
     cout = g.shape[-1]
+    n_paths = kernels._compiled_tables("uv")[int(cfg)][0][3]
     gw = torch.empty((n_paths, cin, cout), dtype=x.dtype, device=x.device)
+    scale = cfg.scale_tensor(torch.float32, x.device) if isinstance(cfg, kernels.Cfg) else None
     ws_bytes = int(_lib.lib.cgtp_uv_grad_w_workspace_bytes(cfg, n, cin, cout))
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=x.device)
     _lib.check(_lib.lib.cgtp_uv_grad_w(cfg, x.data_ptr(), y.data_ptr(), g.data_ptr(), gw.data_ptr(), ws.data_ptr(), n,
-                                       cin, cout, _lib.BF16, _lib.stream_ptr(x.device)), "cgtp_uv_grad_w")
-    return gw
+                                       cin, cout, _lib.BF16, _lib.ptr(scale), _lib.stream_ptr(x.device)),
+               "cgtp_uv_grad_w")
+    return kernels.contract_paths(gw, cfg, 0)
 
 
 class _UvMfma(Function):
@@ -84,7 +70,7 @@ class _UvMfma(Function):
     @staticmethod
     def forward(ctx, x: Tensor, y: Tensor, w: Tensor, tp_info, cfg: int):
         coo = kernels.coo_of(tp_info)
-        out = _apply(cfg, 0, x, y, pack_weights(0, w), coo.DO)
+        out = _apply(cfg, 0, x, y, pack_weights(0, w, cfg), coo.DO)
         ctx.save_for_backward(x, y, w)
         ctx.tp_info, ctx.cfg, ctx.d1 = tp_info, cfg, coo.D1
         return out
@@ -100,17 +86,17 @@ class _UvMfma(Function):
                 if torch.is_grad_enabled():
                     gx = tri(spec.grad_spec(0), ("w", "", "uw"), "u", g, y, w)
                 else:
-                    gx = _apply(ctx.cfg, 1, g.contiguous(), y, pack_weights(1, w), ctx.d1)
+                    gx = _apply(ctx.cfg, 1, g.contiguous(), y, pack_weights(1, w, ctx.cfg), ctx.d1)
             if need[1]:
                 if torch.is_grad_enabled() or g.shape[-1] > 128:
                     gy = tri(spec.grad_spec(1), ("u", "w", "uw"), "", x, g, w)
                 else:
-                    gy = _grad_y(ctx.cfg, x, g.contiguous(), pack_weights(0, w), y.shape[-1])
+                    gy = _grad_y(ctx.cfg, x, g.contiguous(), pack_weights(0, w, ctx.cfg), y.shape[-1])
             if need[2]:
                 if torch.is_grad_enabled():
                     gw = tri(spec.grad_spec(2), ("u", "", "w"), "uw", x, y, g, out_shared=True)
                 else:
-                    gw = _grad_w(ctx.cfg, x, y, g.contiguous(), w.shape[0])
+                    gw = _grad_w(ctx.cfg, x, y, g.contiguous())
         return gx, gy, gw, None, None
 
 

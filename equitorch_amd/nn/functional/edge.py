@@ -148,9 +148,12 @@ def edge_tensor_product_uu(x: Tensor, sh: Tensor, weight: Tensor, plan: EdgePlan
     if cfg >= 0 and x.dtype == sh.dtype == weight.dtype and x.dtype in (torch.float32, torch.float64):
         xc, yc, wc = x.contiguous(), sh.contiguous(), weight.contiguous()
         if kernels.uvu_launchable(cfg, xc, yc, wc, segments=True):
+            kernels.log_tier("edge_tensor_product_uu", "fused gather / product / segment sum", f"config {int(cfg)}")
             return _EdgeUvuCompiled.apply(xc, yc, wc, plan, tp_info_forward, cfg)
         if kernels.uvu_launchable(cfg, xc, yc, wc, gathered=True):
+            kernels.log_tier("edge_tensor_product_uu", "block-wise row kernels + segment sums", f"config {int(cfg)}")
             return _EdgeUvuRows.apply(xc, yc, wc, plan, tp_info_forward, cfg)
+    kernels.log_tier("edge_tensor_product_uu", "index_select + tensor_product_u1u + sparse_scale")
     msg = tensor_product_u1u(x.index_select(0, plan.src), sh, weight, tp_info_forward)
     e, d, c = msg.shape
     fwd, bwd = plan.scale_infos()

@@ -68,7 +68,9 @@ def tensor_product_u1u(input1: Tensor, input2: Tensor, weight: Tensor,
         cfg = kernels.uvu_config_of(tp_info_forward)
         x, y, w = input1.contiguous(), input2.contiguous(), weight.contiguous()
         if cfg >= 0 and kernels.uvu_launchable(cfg, x, y, w):
+            kernels.log_tier("tensor_product_u1u", "compiled table", f"config {int(cfg)}")
             return _UvuCompiled.apply(x, y, w, tp_info_forward, cfg)
+    kernels.log_tier("tensor_product_u1u", "table-driven kernel", str(input1.dtype))
     return tri(spec_from_tp_info(tp_info_forward), (V, S, V), V, input1, input2, weight)
 
 
@@ -104,9 +106,12 @@ def tensor_product_u1v(input1: Tensor, input2: Tensor, weight: Tensor,
     from . import _uv_gemm, _uvw_mfma
     fast = _uvw_mfma.try_forward(input1, input2, weight, tp_info_forward)
     if fast is not None:
+        kernels.log_tier("tensor_product_u1v", "matrix-core kernel (compiled table)")
         return fast
     if input1.ndim == 3 and input2.ndim == 2 and _uv_gemm.supported(input1, input2, weight):
+        kernels.log_tier("tensor_product_u1v", "library GEMM + table-driven kernel", str(input1.dtype))
         return _uv_gemm.u1v(input1, input2, weight, tp_info_forward)
+    kernels.log_tier("tensor_product_u1v", "general two-axis kernel", str(input1.dtype))
     return tri(spec_from_tp_info(tp_info_forward), ("u", "", "uw"), "w", input1, input2, weight)
 
 

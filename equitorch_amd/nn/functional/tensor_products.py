@@ -54,7 +54,9 @@ def tensor_product_uuu(input1: Tensor, input2: Tensor, weight: Tensor,
         cfg = kernels.uvu_config_of(tp_info_forward)
         x, y, w = input1.contiguous(), input2.contiguous(), weight.contiguous()
         if cfg >= 0 and kernels.uvu_launchable(cfg, x, y, w):
+            kernels.log_tier("tensor_product_uuu", "compiled table", f"config {int(cfg)}")
             return _UuuCompiled.apply(x, y, w, tp_info_forward, cfg)
+    kernels.log_tier("tensor_product_uuu", "table-driven kernel", str(input1.dtype))
     return tri(spec_from_tp_info(tp_info_forward), (V, V, V), V, input1, input2, weight)
 
 

@@ -38,28 +38,169 @@ def coo_of(tp_info) -> TpCoo:
     return cached(tp_info.info_Mij_fwd.scale, "coo", lambda: tp_coo(tp_info))
 
 
-_ROUNDED = {torch.bfloat16: ("bf16", 2), torch.float16: ("f16", 3)}     # precision name, dtype code of the library
+class Cfg(int):
+    """Index of a compiled-in table (an ``int``, -1: none), carrying how the caller's table maps onto the compiled one.
+
+    ``path_scale`` (float64 array over the compiled paths, or None = all ones): the caller's coefficients are the
+    compiled ones times one factor per weight path — what ``path_norm`` / ``channel_norm`` / ``channel_scale`` change
+    (``equitorch/utils/_structs.py:177-206``).  ``w_rows`` (int array over the compiled paths, or None = identity): the
+    caller's weight row of every compiled path, -1 for a path the caller's table does not have (an explicit ``path=``
+    subset); such weights are expanded with zero rows before the launch (:func:`expand_paths`)."""
+    path_scale: Optional[np.ndarray]
+    w_rows: Optional[np.ndarray]
+
+    def __new__(cls, value: int, path_scale=None, w_rows=None):
+        obj = super().__new__(cls, value)
+        obj.path_scale, obj.w_rows = path_scale, w_rows
+        obj._dev = {}
+        return obj
+
+    def scale_tensor(self, dtype: torch.dtype, device) -> Optional[Tensor]:
+        """``path_scale`` as a device tensor of ``dtype`` (cached), or None."""
+        if self.path_scale is None:
+            return None
+        key = (dtype, str(device))
+        if key not in self._dev:
+            self._dev[key] = torch.from_numpy(self.path_scale).to(device=device, dtype=dtype)
+        return self._dev[key]
+
+    def rows_tensor(self, device) -> Optional[Tensor]:
+        if self.w_rows is None:
+            return None
+        key = ("rows", str(device))
+        if key not in self._dev:
+            self._dev[key] = torch.from_numpy(self.w_rows.astype(np.int64)).to(device)
+        return self._dev[key]
 
 
-def _find_config(tp_info, find, find_rounded) -> int:
-    scale = tp_info.info_Mij_fwd.scale
-    if scale.dtype in _ROUNDED:      # table of a module converted to reduced precision
-        name, code = _ROUNDED[scale.dtype]
-        return int(find_rounded(C.c_uint64(fingerprint(coo_of(tp_info), name)), code))
-    return int(find(C.c_uint64(fingerprint(coo_of(tp_info)))))
+_COMPILED = {}   # family -> list of (dims, {(M, M1, M2): (p, coef)}) of every compiled configuration
 
 
-def uvu_config_of(tp_info) -> int:
-    """Index of the compiled-in table equal to this ``tp_info`` (fp32 coefficient bits; for a bf16 / fp16 table:
-    equal after rounding the compiled coefficients to that type), or -1."""
-    return cached(tp_info.info_Mij_fwd.scale, "cfg",
-                  lambda: _find_config(tp_info, _lib.lib.cgtp_uvu_find, _lib.lib.cgtp_uvu_find_rounded))
+def _compiled_tables(family: str):
+    """The tables compiled into the library, read back through ``cgtp_uvu_table`` / ``cgtp_uv_table`` (once)."""
+    if family in _COMPILED:
+        return _COMPILED[family]
+    L = _lib.lib
+    out = []
+    n = L.cgtp_uvu_num_configs() if family == "uvu" else L.cgtp_uv_num_configs()
+    for cfg in range(n):
+        dims = (C.c_int32 * 5)()
+        if family == "uvu":
+            L.cgtp_uvu_describe(cfg, dims)
+        else:
+            L.cgtp_uv_table(cfg, dims, None, None)
+        nnz = dims[4]
+        coef, idx = (C.c_float * nnz)(), (C.c_int32 * (4 * nnz))()
+        got = L.cgtp_uvu_table(cfg, coef, idx) if family == "uvu" else L.cgtp_uv_table(cfg, None, coef, idx)
+        assert got == nnz
+        ix = np.frombuffer(idx, dtype=np.int32).reshape(nnz, 4)
+        cf = np.frombuffer(coef, dtype=np.float32).astype(np.float64)
+        out.append((tuple(dims), {(int(m), int(a), int(b)): (int(p), float(c)) for (m, a, b, p), c in zip(ix, cf)}))
+    _COMPILED[family] = out
+    return out
 
 
-def uv_config_of(tp_info) -> int:
+_RATIO_TOL = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10}   # coefficient tensors converted with the module
+
+
+def _match_config(tp_info, family: str) -> Cfg:
+    """The compiled configuration whose table has the same entries as ``tp_info`` up to one factor per weight path
+    (and, for an explicit ``path=`` subset, a subset of its paths), or ``Cfg(-1)``.  Exact equality of the fp32
+    coefficients gives ``path_scale = None``."""
+    coo = coo_of(tp_info)
+    tol = _RATIO_TOL.get(tp_info.info_Mij_fwd.scale.dtype, 1e-6)
+    nnz = coo.coef.shape[0]
+    for cfg, (dims, table) in enumerate(_compiled_tables(family)):
+        if dims[:3] != (coo.D1, coo.D2, coo.DO) or nnz > dims[4] or coo.P > dims[3]:
+            continue
+        comp_of, row_of, ratios, ok = {}, {}, {}, True      # caller path -> compiled path and back; ratios per path
+        for t in range(nnz):
+            hit = table.get((int(coo.M[t]), int(coo.M1[t]), int(coo.M2[t])))
+            if hit is None:
+                ok = False
+                break
+            pc, cc = hit
+            pm = int(coo.p[t])
+            if comp_of.setdefault(pm, pc) != pc or row_of.setdefault(pc, pm) != pm:
+                ok = False
+                break
+            ratios.setdefault(pc, []).append(float(coo.coef[t]) / cc)
+        if not ok:
+            continue
+        # every entry of a matched compiled path must be present (a path is either taken whole or not at all)
+        count = {}
+        for (_, _, _), (pc, _) in table.items():
+            count[pc] = count.get(pc, 0) + 1
+        if any(len(r) != count[pc] for pc, r in ratios.items()):
+            continue
+        scale = np.zeros(dims[3], dtype=np.float64)
+        for pc, r in ratios.items():
+            r = np.asarray(r)
+            mid = float(np.median(r))
+            if mid == 0.0 or np.any(np.abs(r / mid - 1.0) > tol):
+                ok = False
+                break
+            scale[pc] = mid
+        if not ok:
+            continue
+        full = len(ratios) == dims[3]
+        identity = full and all(row_of[pc] == pc for pc in range(dims[3]))
+        ones = full and np.all(np.abs(scale - 1.0) <= tol)
+        rows = None if identity else np.array([row_of.get(pc, -1) for pc in range(dims[3])], dtype=np.int64)
+        return Cfg(cfg, None if ones else scale, rows)
+    return Cfg(-1)
+
+
+def uvu_config_of(tp_info) -> Cfg:
+    """The compiled-in channel-wise table this ``tp_info`` runs on (see :class:`Cfg`), or ``Cfg(-1)``."""
+    return cached(tp_info.info_Mij_fwd.scale, "cfg", lambda: _match_config(tp_info, "uvu"))
+
+
+def uv_config_of(tp_info) -> Cfg:
     """The same among the tables of the fully connected product on the matrix cores."""
-    return cached(tp_info.info_Mij_fwd.scale, "uv_cfg",
-                  lambda: _find_config(tp_info, _lib.lib.cgtp_uv_find, _lib.lib.cgtp_uv_find_rounded))
+    return cached(tp_info.info_Mij_fwd.scale, "uv_cfg", lambda: _match_config(tp_info, "uv"))
+
+
+def expand_paths(w: Tensor, cfg, path_dim: int) -> Tensor:
+    """Weights of a table that has only some of the compiled paths (``cfg.w_rows``), laid out over all compiled
+    paths with zeros for the missing ones; differentiable.  Identity when the table has all paths in order."""
+    rows = getattr(cfg, "w_rows", None)
+    if rows is None:
+        return w
+    idx = cfg.rows_tensor(w.device)
+    present = idx >= 0
+    full = w.index_select(path_dim, idx.clamp(min=0))
+    shape = [1] * w.ndim
+    shape[path_dim] = -1
+    return full * present.to(w.dtype).view(shape)
+
+
+def contract_paths(gw: Optional[Tensor], cfg, path_dim: int) -> Optional[Tensor]:
+    """Inverse of :func:`expand_paths` for a gradient: the rows of the caller's own paths, in the caller's order."""
+    rows = getattr(cfg, "w_rows", None)
+    if rows is None or gw is None:
+        return gw
+    key = ("inverse", str(gw.device))
+    if key not in cfg._dev:
+        inv = np.full(int(rows.max()) + 1, -1, dtype=np.int64)
+        for pc, pm in enumerate(rows):
+            if pm >= 0:
+                inv[pm] = pc
+        cfg._dev[key] = torch.from_numpy(inv).to(gw.device)
+    return gw.index_select(path_dim, cfg._dev[key]).contiguous()
+
+
+_TIER_LOG = bool(__import__("os").environ.get("CGTP_LOG_TIER"))
+_TIER_SEEN = set()
+
+
+def log_tier(op: str, tier: str, detail: str = ""):
+    """With ``CGTP_LOG_TIER=1`` in the environment: one line on stderr the first time an operator takes a kernel tier
+    (compiled table / block-wise / table-driven / library GEMM), so that a slow path is visible."""
+    if _TIER_LOG and (op, tier, detail) not in _TIER_SEEN:
+        _TIER_SEEN.add((op, tier, detail))
+        import sys
+        print(f"[cgtp] {op}: {tier}{' (' + detail + ')' if detail else ''}", file=sys.stderr, flush=True)
 
 
 # ---- operands ---------------------------------------------------------------------------------------------
@@ -88,12 +229,19 @@ def tri_contract(table: dict, n_out: int, a: Tuple[Optional[Tensor], int], b: Tu
                  w: Tuple[Optional[Tensor], int], n_rows: int, channels: int, dtype: torch.dtype, device,
                  reduce_c: bool = False, reduce_rows: bool = False,
                  rows_a: Optional[Tensor] = None, rows_b: Optional[Tensor] = None,
-                 rows_w: Optional[Tensor] = None) -> Tensor:
-    """``out[r,o,c] = sum_t coef_t A[r,ia_t,c] B[r,ib_t,(c)] W[r,iw_t,c]`` with the packed ``table``."""
+                 rows_w: Optional[Tensor] = None, out: Optional[Tensor] = None,
+                 static_scratch: bool = False) -> Tensor:
+    """``out[r,o,c] = sum_t coef_t A[r,ia_t,c] B[r,ib_t,(c)] W[r,iw_t,c]`` with the packed ``table``.
+    ``static_scratch``: launch through ``cgtp_tri_contract_static`` — no workspace is allocated here, the partial
+    rows of a sum over rows live in the library's fixed per-device array (and with ``out`` given, this call allocates
+    nothing at all)."""
     shape = ((n_out,) if reduce_c else (n_out, channels))
     if not reduce_rows:
         shape = (n_rows,) + shape
-    out = torch.empty(shape, dtype=dtype, device=device)
+    if out is None:
+        out = torch.empty(shape, dtype=dtype, device=device)
+    elif tuple(out.shape) != shape or out.dtype != dtype or not out.is_contiguous():
+        raise _lib.CgtpError(f"out must be a contiguous {dtype} tensor of shape {shape}")
     if n_rows == 0 or out.numel() == 0:      # empty batch: nothing to launch; a sum over no rows is zero
         return out.zero_()
     args = TriArgs()
@@ -102,6 +250,10 @@ def tri_contract(table: dict, n_out: int, a: Tuple[Optional[Tensor], int], b: Tu
     args.n_out, args.nnz = n_out, table["idx"].shape[0]
     args.out, args.n_rows, args.C = out.data_ptr(), n_rows, channels
     args.dtype, args.reduce_c, args.reduce_rows = _lib.dtype_code(dtype), int(reduce_c), int(reduce_rows)
+    if static_scratch:
+        _lib.check(_lib.lib.cgtp_tri_contract_static(C.byref(args), _lib.stream_ptr(device)),
+                   "cgtp_tri_contract_static")
+        return out
     ws = None
     if reduce_rows:
         nbytes = int(_lib.lib.cgtp_tri_workspace_bytes(C.byref(args)))
@@ -329,6 +481,9 @@ def _uvu_args(cfg: int, x: Tensor, y: Tensor, w: Tensor, seg: Optional[SegIndex]
     else:
         a.gather = _lib.ptr(gather)
     a.x, a.y, a.w = x.data_ptr(), y.data_ptr(), w.data_ptr()
+    scale = cfg.scale_tensor(x.dtype, x.device) if isinstance(cfg, Cfg) else None
+    a.path_scale = _lib.ptr(scale)
+    a._keep = scale
     return a
 
 
@@ -374,6 +529,7 @@ def uvu_forward(cfg: int, dims, x: Tensor, y: Tensor, w: Tensor, seg: Optional[S
     ``out[s] = sum_{q in segment s} TP(x[seg.gather[q]], y[e_q], w[e_q])``.  With ``y_vec`` (segment mode), ``y``
     holds ``(E, 3)`` edge vectors and the kernel evaluates their harmonics itself (``Y_UNIT_VECTOR``: after
     normalising them, ``Y_RAW_VECTOR``: as they are)."""
+    w = expand_paths(w, cfg, -2)
     a = _uvu_args(cfg, x, y, w, seg, gather, pos_per_wave, y_vec)
     n_out_rows = a.n_seg if seg is not None else y.shape[0]
     out = torch.empty((n_out_rows, dims[2], x.shape[-1]), dtype=x.dtype, device=x.device)
@@ -389,6 +545,7 @@ def uvu_backward(cfg: int, dims, x: Tensor, y: Tensor, w: Tensor, g: Tensor, nee
     """Compiled-table backward -> (grad_x, grad_y, grad_w), None where ``need`` is False.  Row mode: ``gather``
     picks the row of ``g`` and ``x_gather`` the row of ``x`` of every batch row; with ``x_gather`` the returned
     grad_x is per batch row, ``(n_rows, D1, C)``."""
+    w = expand_paths(w, cfg, -2)
     a = _uvu_args(cfg, x, y, w, seg, gather, pos_per_wave, y_vec)
     a.grad_out = g.data_ptr()
     a.x_gather = _lib.ptr(x_gather)
@@ -403,7 +560,7 @@ def uvu_backward(cfg: int, dims, x: Tensor, y: Tensor, w: Tensor, g: Tensor, nee
     a.grad_x, a.grad_y, a.grad_w = _lib.ptr(gx), _lib.ptr(gy), _lib.ptr(gw)
     ws = _workspace(a, 1, x.device)
     _lib.check(_lib.lib.cgtp_uvu_bwd(C.byref(a), _lib.stream_ptr(x.device)), "cgtp_uvu_bwd")
-    return gx, gy, gw
+    return gx, gy, contract_paths(gw, cfg, -2)
 
 
 def uvu_sh_degree(cfg: int) -> int:

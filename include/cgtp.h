@@ -28,7 +28,8 @@ enum {
   CGTP_ERR_CONFIG = 5,      /* unknown specialised-table id                                 */
   CGTP_ERR_LDS = 6,         /* table does not fit the 160 KB LDS of a CU                    */
   CGTP_ERR_LAUNCH = 7,      /* hipLaunchKernel reported an error                            */
-  CGTP_ERR_WORKSPACE = 8    /* workspace missing or too small                               */
+  CGTP_ERR_WORKSPACE = 8,   /* workspace missing or too small                               */
+  CGTP_ERR_SCRATCH_LIMIT = 9 /* cgtp_tri_contract_static: partial results beyond the fixed scratch array */
 };
 
 enum { CGTP_F32 = 0, CGTP_F64 = 1, CGTP_BF16 = 2, CGTP_F16 = 3 };
@@ -88,6 +89,17 @@ int64_t cgtp_tri_workspace_bytes(const cgtp_tri_args* args);
 /* Host-only validation of the same conditions the launch checks; needs no device. */
 int cgtp_tri_validate(const cgtp_tri_args* args);
 int cgtp_tri_contract(const cgtp_tri_args* args, void* stream);
+
+/* cgtp_tri_contract for callers that cannot allocate device memory or pass a workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  args->workspace
+ * is ignored; when reduce_rows != 0 the partial rows of the sum over rows live in a fixed device array inside the
+ * library (cgtp_tri_static_scratch_bytes() = 16 MiB per device, held until the process ends).  A launch whose
+ * cgtp_tri_workspace_bytes() exceeds that returns CGTP_ERR_SCRATCH_LIMIT without launching.  Calls nothing that
+ * allocates.  Results are bit-identical to cgtp_tri_contract.  All calls on one device share the array: two calls
+ * that overlap in time on one device (different streams or threads) race; calls on one stream do not.  The first call
+ * on a device looks the array's address up (hipGetSymbolAddress); make it outside graph capture. */
+int64_t cgtp_tri_static_scratch_bytes(void);
+int cgtp_tri_contract_static(const cgtp_tri_args* args, void* stream);
 
 /* ---- general contraction over two channel axes (u, w) ----------------------------------------------------
  *
@@ -166,6 +178,10 @@ int cgtp_uvu_find(uint64_t fingerprint);
 int cgtp_uvu_find_rounded(uint64_t fingerprint, int dtype);
 /* Describes config `cfg`: dims (D1, D2, DO, P, NNZ) written to dims[5]; returns its fingerprint (0 if bad). */
 uint64_t cgtp_uvu_describe(int cfg, int32_t* dims);
+/* The compiled table of config `cfg` (dims from cgtp_uvu_describe): coef[NNZ] fp32 values, idx[4 * NNZ] = (M, M1, M2,
+ * p) per entry in table order; either may be NULL.  Returns NNZ, -1 for a bad id.  Host only.  See
+ * cgtp_uvu_args.path_scale. */
+int cgtp_uvu_table(int cfg, float* coef, int32_t* idx);
 /* Degree L if the second operand of config `cfg` is laid out like harmonics of degrees 0..L and the fused
  * kernels can evaluate them from edge vectors (cgtp_uvu_args.y_vec); -1 otherwise. */
 int cgtp_uvu_sh_degree(int cfg);
@@ -210,6 +226,9 @@ typedef struct cgtp_uvu_args {
                               TensorProductUUUDummy (equitorch/nn/functional/tensor_products.py:9-90), on the
                               block-wise kernels                                                     */
   int32_t reserved_;
+  const void* path_scale;  /* optional, device, P values of dtype: the caller's table is the compiled one with the
+                              coefficients of weight path p multiplied by path_scale[p] (other path_norm / channel_norm
+                              than the compiled default, equitorch/utils/_structs.py:177-206); NULL = all ones        */
 } cgtp_uvu_args;
 
 int cgtp_uvu_validate(const cgtp_uvu_args* args, int backward);
@@ -239,8 +258,17 @@ int cgtp_uv_num_configs(void);
 int cgtp_uv_find(uint64_t fingerprint);
 /* As cgtp_uvu_find_rounded, for the fully connected product. */
 int cgtp_uv_find_rounded(uint64_t fingerprint, int dtype);
+/* path_scale (device, n_paths floats, or NULL): factor of every weight path, folded into the packed copy — for a
+ * table that equals the compiled one up to one factor per path (other path / channel normalisation, see
+ * cgtp_uv_table). */
 int cgtp_uv_pack_weights(int direction, const void* w, void* packed, int32_t n_paths, int32_t cin, int32_t cout,
-                         int32_t dtype, void* stream);
+                         int32_t dtype, const float* path_scale, void* stream);
+/* The compiled table of config `cfg`: dims[5] = (D1, D2, DO, P, NNZ), coef[NNZ] (fp32 values), idx[4 * NNZ] =
+ * (M, M1, M2, p) per entry, in table order; each output may be NULL.  Returns NNZ, -1 for a bad id.  Host only.  A
+ * caller whose table has the same entries with every path's coefficients multiplied by one factor per path (the
+ * reference's path_norm / channel_norm options, equitorch/utils/_structs.py:177-206) passes those factors as
+ * path_scale and runs on the same kernels. */
+int cgtp_uv_table(int cfg, int32_t* dims, float* coef, int32_t* idx);
 int cgtp_uv_validate(int cfg, int direction, const void* x, const void* y, const void* wp, const void* out,
                      int64_t n_rows, int32_t cin, int32_t cout, int32_t dtype);
 int cgtp_uv_apply(int cfg, int direction, const void* x, const void* y, const void* wp, void* out, int64_t n_rows,
@@ -260,7 +288,7 @@ int cgtp_uv_grad_y(int cfg, const void* x, const void* g, const void* wp, void* 
  * partials live in `workspace` (cgtp_uv_grad_w_workspace_bytes bytes) and are added in a fixed order. */
 int64_t cgtp_uv_grad_w_workspace_bytes(int cfg, int64_t n_rows, int32_t cin, int32_t cout);
 int cgtp_uv_grad_w(int cfg, const void* x, const void* y, const void* g, void* gw, void* workspace, int64_t n_rows,
-                   int32_t cin, int32_t cout, int32_t dtype, void* stream);
+                   int32_t cin, int32_t cout, int32_t dtype, const float* path_scale, void* stream);
 
 /* ---- real spherical harmonics of vectors -----------------------------------------------------------------
  * Stands in for spherical_harmonics (equitorch/ops/spherical_harmonics.py:68-640: explicit polynomials per

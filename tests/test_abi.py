@@ -44,7 +44,7 @@ def test_version_and_status_strings():
     from equitorch_amd import _lib
     assert _lib.lib.cgtp_version() >= 1
     assert _lib.lib.cgtp_status_string(0) == b"ok"
-    assert len({_lib.lib.cgtp_status_string(i) for i in range(9)}) == 9
+    assert len({_lib.lib.cgtp_status_string(i) for i in range(10)}) == 10
 
 
 def test_compiled_tables_match_python_fingerprints():
@@ -181,14 +181,14 @@ def test_uv_matrix_core_entry_points_validate_on_the_host():
     assert L.cgtp_uv_apply(cfg, 0, p16, p16, p16, p16, 0, 128, 128, _lib.BF16, None) == 0      # empty batch
     assert L.cgtp_uv_grad_y(cfg, p16, p16, p16, p16, 0, 128, 128, _lib.BF16, None) == 0
     assert L.cgtp_uv_grad_y(cfg, p16, p16, p16, p16, 10, 128, 256, _lib.BF16, None) == 2       # C_out > 128
-    assert L.cgtp_uv_pack_weights(0, p16, p16, 0, 128, 128, _lib.BF16, None) == 0
-    assert L.cgtp_uv_pack_weights(0, p16, p16, 23, 100, 128, _lib.BF16, None) == 2
-    assert L.cgtp_uv_pack_weights(3, p16, p16, 23, 128, 128, _lib.BF16, None) == 2
+    assert L.cgtp_uv_pack_weights(0, p16, p16, 0, 128, 128, _lib.BF16, None, None) == 0
+    assert L.cgtp_uv_pack_weights(0, p16, p16, 23, 100, 128, _lib.BF16, None, None) == 2
+    assert L.cgtp_uv_pack_weights(3, p16, p16, 23, 128, 128, _lib.BF16, None, None) == 2
     # weight gradient: one fp32 partial of (P, C_in, C_out) per chunk of 512 samples
     assert L.cgtp_uv_grad_w_workspace_bytes(cfg, 32768, 128, 128) == 64 * 23 * 128 * 128 * 4
     assert L.cgtp_uv_grad_w_workspace_bytes(cfg, 513, 32, 64) == 2 * 23 * 32 * 64 * 4
-    assert L.cgtp_uv_grad_w(cfg, p16, p16, p16, p16, None, 100, 128, 128, _lib.BF16, None) == 8  # workspace missing
-    assert L.cgtp_uv_grad_w(cfg, p16, p16, p16, p16, p16, 100, 128, 160, _lib.BF16, None) == 2
+    assert L.cgtp_uv_grad_w(cfg, p16, p16, p16, p16, None, 100, 128, 128, _lib.BF16, None, None) == 8  # workspace missing
+    assert L.cgtp_uv_grad_w(cfg, p16, p16, p16, p16, p16, 100, 128, 160, _lib.BF16, None, None) == 2
 
 
 def test_spherical_harmonics_entry_points_validate_on_the_host():

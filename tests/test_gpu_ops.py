@@ -271,6 +271,39 @@ def test_uv_mfma_bf16(device, lmax, cin, cout, n):
         assert err <= 1e-2 * float(b.abs().max()), f"lmax={lmax} {name}: max abs err {err:.3e} vs scale {float(b.abs().max()):.3e}"
 
 
+@pytest.mark.parametrize("kw", [{"path_norm": False}, {"channel_norm": True},
+                                {"channel_norm": True, "path_norm": False}])
+def test_uv_mfma_bf16_normalisation_options(device, kw):
+    """``channel_norm=True`` (the reference's channel-normalised comparison test) and ``path_norm=False`` only
+    rescale the coefficients of a path: the bf16 matrix-core kernels must still be selected (the factors are folded
+    into the packed weights and into the weight gradient), and agree with the dense oracle built with those options."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import _uvw_mfma
+    from equitorch_amd.utils._sh import spherical_harmonics
+    from helpers import unit_vectors
+    lmax, cin, cout, n = 3, 64, 128, 300
+    irreps = "0e+1o+2e+3o"
+    mod = SO3Linear(irreps, irreps, irreps, cin, cout, internal_weights=False, feature_mode="uv", **kw).to(device)
+    cfg = _uvw_mfma.uv_config_of(mod.tp_info_forward)
+    assert cfg >= 0 and cfg.path_scale is not None
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(n, 16, cin, generator=g).bfloat16()
+    y = spherical_harmonics(unit_vectors(n, g), lmax).bfloat16()
+    w = (torch.randn(mod.num_paths, cin, cout, generator=g) / mod.num_paths ** 0.5).bfloat16()
+    ct = torch.randn(n, 16, cout, generator=g).bfloat16()
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    assert _uvw_mfma.try_forward(xd.detach(), yd.detach(), wd.detach(), mod.tp_info_forward) is not None
+    out = mod(xd, yd, wd)
+    gx, gy, gw = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
+    T = ref_ops.dense_coupling(irreps, irreps, irreps, path_norm=kw.get("path_norm", True),
+                               channel_norm=kw.get("channel_norm", False), channel_scale=cin ** -0.5).float().double()
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x, y, w), ct)
+    for name, a, b in zip(("out", "grad_x", "grad_sh", "grad_w"), (out, gx, gy, gw), (ref_out, *ref_grads)):
+        a, b = a.detach().double().cpu(), b.double()
+        err = float((a - b).abs().max())
+        assert err <= 1e-2 * float(b.abs().max()), f"{kw} {name}: max abs err {err:.3e} vs {float(b.abs().max()):.3e}"
+
+
 def test_uv_mfma_full_size_properties(device):
     """BASELINE configs[3] shapes (B = 32768, lmax = 3, C = 128, bf16).  The dense oracle is run on a strided
     subset of the rows for out / grad_x / grad_sh (each row depends on its own sample only); the weight gradient

@@ -295,3 +295,81 @@ def test_edge_large_table_hub_and_shared_weight(device, hub):
         for name, g, r in zip(("out", "grad_x", "grad_sh", "grad_w"), (out, xd.grad, shd.grad, wd.grad),
                               (ref_out, *ref_grads)):
             assert_close(g, r, 1e-5, f"lmax=4 hub={hub} shared={shared} {name}")
+
+
+def _subset_paths(irreps, drop):
+    from oracle import ref_tables
+    full = ref_tables.fully_connected_paths(*(ref_tables.parse(irreps),) * 3)
+    return [p for n, p in enumerate(full) if n not in drop]
+
+
+@pytest.mark.parametrize("kw", [{"path_norm": False}, {"path": "subset"}, {"path": "subset", "path_norm": False}])
+@pytest.mark.parametrize("shared_w", [False, True])
+def test_u1u_options_that_rescale_or_drop_paths_stay_on_the_compiled_kernels(device, kw, shared_w):
+    """``path_norm=False`` and an explicit ``path=`` subset (``SO3Linear`` arguments of the reference,
+    ``equitorch/nn/linears.py:85-95``) give tables that differ from the compiled one by a factor per weight path and
+    by missing paths: they must select the same compiled kernels, in row mode and in the fused edge mode, and agree
+    with the dense oracle built with the same options."""
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu
+    from equitorch_amd.ops import kernels
+    irreps = SH[2]
+    kw = dict(kw)
+    if kw.get("path") == "subset":
+        kw["path"] = _subset_paths(irreps, (2, 5, 6))
+    mod = _module(irreps, irreps, irreps, **kw).to(device)
+    base = _module(irreps, irreps, irreps).to(device)
+    cfg = kernels.uvu_config_of(mod.tp_info_forward)
+    assert cfg >= 0 and int(cfg) == int(kernels.uvu_config_of(base.tp_info_forward))
+    assert cfg.path_scale is not None
+    n, ch = 300, 64
+    x, sh, w = tp_inputs(n, 9, 2, mod.num_paths, ch, shared_w, seed=77)
+    ct = torch.randn(n, 9, ch, generator=torch.Generator().manual_seed(7))
+    got = _run(mod, x, sh, w, ct, device)
+    T = ref_ops.dense_coupling(irreps, irreps, irreps, path=kw.get("path"), path_norm=kw.get("path_norm", True))
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1u, T, (x, sh, w), ct)
+    for name, g, r in zip(("out", "grad_x", "grad_sh", "grad_w"), got, (ref_out, *ref_grads)):
+        assert_close(g, r, 1e-5, f"{sorted(kw)} shared={shared_w} {name}")
+    # fused edge mode
+    gen = torch.Generator().manual_seed(5)
+    n_nodes = 40
+    src = torch.randint(0, n_nodes, (n,), generator=gen)
+    dst = torch.randint(0, n_nodes, (n,), generator=gen)
+    xn, ctn = x[:n_nodes].contiguous(), ct[:n_nodes].contiguous()
+    plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
+    xd, shd, wd = (t.to(device).requires_grad_(True) for t in (xn, sh, w))
+    out = edge_tensor_product_uu(xd, shd, wd, plan, mod.tp_info_forward)
+    (out * ctn.to(device)).sum().backward()
+
+    def ref_fn(T, x, sh, w):
+        return ref_ops.scatter_sum(ref_ops.dense_u1u(T, x.index_select(0, src), sh, w), dst, n_nodes)
+    ref_out, ref_grads = ref_ops.dense_grads(ref_fn, T, (xn, sh, w), ctn)
+    for name, g, r in zip(("out", "grad_x", "grad_sh", "grad_w"), (out, xd.grad, shd.grad, wd.grad),
+                          (ref_out, *ref_grads)):
+        # a shared weight's gradient sums over all edges: norm-wise
+        assert_close(g, r, 1e-5, f"edge {sorted(kw)} shared={shared_w} {name}",
+                     norm="max" if (shared_w and name == "grad_w") else "element")
+
+
+def test_u1u_so3_lmax4_reference_test_irreps(device):
+    """``0e+1e+2e+3e+4e`` for all three operands — the irreps of the reference's own comparison test
+    (``test/test_tp/test_tensor_product_channel_e3nn.py:639-646``) — runs on a compiled table, with and without
+    ``path_norm``."""
+    from equitorch_amd.ops import kernels
+    irreps = "0e+1e+2e+3e+4e"
+    for path_norm in (True, False):
+        mod = _module(irreps, irreps, irreps, path_norm=path_norm).to(device)
+        assert kernels.uvu_config_of(mod.tp_info_forward) >= 0
+        n, ch = 256, 16
+        g = torch.Generator().manual_seed(3)
+        x = torch.randn(n, 25, ch, generator=g)
+        y = torch.randn(n, 25, generator=g)
+        w = torch.randn(n, mod.num_paths, ch, generator=g)
+        ct = torch.randn(n, 25, ch, generator=g)
+        assert kernels.uvu_launchable(kernels.uvu_config_of(mod.tp_info_forward), x.to(device), y.to(device), w.to(device))
+        got = _run(mod, x, y, w, ct, device)
+        T = ref_ops.dense_coupling(irreps, irreps, irreps, path_norm=path_norm)
+        ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1u, T, (x, y, w), ct)
+        for name, a, b in zip(("out", "grad_x", "grad_y", "grad_w"), got, (ref_out, *ref_grads)):
+            # up to 61 paths x hundreds of coefficients per element, inputs not normalised: norm-wise for the sums
+            assert_close(a, b, 1e-5, f"so3 lmax=4 path_norm={path_norm} {name}",
+                         norm="element" if name == "grad_w" else "max")
