@@ -60,6 +60,20 @@ class UvuArgs(C.Structure):
                 ("y_channels", C.c_int32), ("reserved_", C.c_int32), ("path_scale", C.c_void_p)]
 
 
+class UvtItem(C.Structure):
+    _fields_ = [("p", C.c_int32), ("kb0", C.c_int32), ("nkb", C.c_int32), ("t0", C.c_int32), ("t1", C.c_int32),
+                ("out_row", C.c_int32), ("flags", C.c_int32), ("reserved_", C.c_int32)]
+
+
+class UvtArgs(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("y", C.c_void_p), ("wp", C.c_void_p), ("out", C.c_void_p),
+                ("items", C.c_void_p), ("term_a", C.c_void_p), ("term_b", C.c_void_p), ("term_c", C.c_void_p),
+                ("n_rows", C.c_int64), ("n_items", C.c_int32),
+                ("dx", C.c_int32), ("dy", C.c_int32), ("dout", C.c_int32),
+                ("cx", C.c_int32), ("cy", C.c_int32), ("cout", C.c_int32),
+                ("kbi", C.c_int32), ("dtype", C.c_int32), ("reserved_", C.c_int32)]
+
+
 def _load():
     if not os.path.exists(_LIB_PATH):
         raise ImportError(
@@ -106,6 +120,13 @@ def _load():
                                    C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]
     lib.cgtp_uv_validate.argtypes = _uv
     lib.cgtp_uv_apply.argtypes = _uv + [C.c_void_p]
+    lib.cgtp_uvt_packed_elems.restype = C.c_int64
+    lib.cgtp_uvt_packed_elems.argtypes = [C.c_int32, C.c_int64, C.c_int32]
+    lib.cgtp_uvt_pack_weights.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_int64, C.c_int64,
+                                          C.c_int64, C.c_int32, C.c_void_p]
+    lib.cgtp_uvt_chunk.argtypes = [C.c_int64] + [C.c_int32] * 5
+    lib.cgtp_uvt_validate.argtypes = [C.POINTER(UvtArgs)]
+    lib.cgtp_uvt_apply.argtypes = [C.POINTER(UvtArgs), C.c_void_p]
     lib.cgtp_sh_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_double, C.c_int,
                                     C.c_void_p]
     lib.cgtp_sh_backward.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_double,

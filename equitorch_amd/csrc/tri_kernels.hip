@@ -577,11 +577,24 @@ int cgtp_abi_layout(int which, int64_t* out, int capacity) {
                                 CGTP_OFF(cgtp_uvu_args, grad_w), CGTP_OFF(cgtp_uvu_args, workspace),
                                 CGTP_OFF(cgtp_uvu_args, x_gather), CGTP_OFF(cgtp_uvu_args, y_channels),
                                 CGTP_OFF(cgtp_uvu_args, reserved_), CGTP_OFF(cgtp_uvu_args, path_scale)};
+  static const int64_t uvt_item[] = {sizeof(cgtp_uvt_item), CGTP_OFF(cgtp_uvt_item, p), CGTP_OFF(cgtp_uvt_item, kb0),
+                                     CGTP_OFF(cgtp_uvt_item, nkb), CGTP_OFF(cgtp_uvt_item, t0), CGTP_OFF(cgtp_uvt_item, t1),
+                                     CGTP_OFF(cgtp_uvt_item, out_row), CGTP_OFF(cgtp_uvt_item, flags),
+                                     CGTP_OFF(cgtp_uvt_item, reserved_)};
+  static const int64_t uvt[] = {sizeof(cgtp_uvt_args), CGTP_OFF(cgtp_uvt_args, x), CGTP_OFF(cgtp_uvt_args, y),
+                                CGTP_OFF(cgtp_uvt_args, wp), CGTP_OFF(cgtp_uvt_args, out), CGTP_OFF(cgtp_uvt_args, items),
+                                CGTP_OFF(cgtp_uvt_args, term_a), CGTP_OFF(cgtp_uvt_args, term_b),
+                                CGTP_OFF(cgtp_uvt_args, term_c), CGTP_OFF(cgtp_uvt_args, n_rows),
+                                CGTP_OFF(cgtp_uvt_args, n_items), CGTP_OFF(cgtp_uvt_args, dx), CGTP_OFF(cgtp_uvt_args, dy),
+                                CGTP_OFF(cgtp_uvt_args, dout), CGTP_OFF(cgtp_uvt_args, cx), CGTP_OFF(cgtp_uvt_args, cy),
+                                CGTP_OFF(cgtp_uvt_args, cout), CGTP_OFF(cgtp_uvt_args, kbi), CGTP_OFF(cgtp_uvt_args, dtype),
+                                CGTP_OFF(cgtp_uvt_args, reserved_)};
 #undef CGTP_OFF
-  const int64_t* tabs[] = {operand, tri, gen_operand, gen, uvu};
+  const int64_t* tabs[] = {operand, tri, gen_operand, gen, uvu, uvt_item, uvt};
   const int counts[] = {(int)(sizeof(operand) / 8), (int)(sizeof(tri) / 8), (int)(sizeof(gen_operand) / 8),
-                        (int)(sizeof(gen) / 8), (int)(sizeof(uvu) / 8)};
-  if (which < 0 || which >= 5) return -1;
+                        (int)(sizeof(gen) / 8), (int)(sizeof(uvu) / 8), (int)(sizeof(uvt_item) / 8),
+                        (int)(sizeof(uvt) / 8)};
+  if (which < 0 || which >= 7) return -1;
   for (int i = 0; out && i < counts[which] && i < capacity; ++i) out[i] = tabs[which][i];
   return counts[which];
 }

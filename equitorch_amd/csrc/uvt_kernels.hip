@@ -1,0 +1,323 @@
+// Fully connected Clebsch-Gordan tensor products ("uv" / "uvw" families) in fp32 on the matrix cores, driven by
+// run-time tables (any irreps, any normalisation):
+//
+//   out[n, M, w] = sum_{segments s = (p, M)} sum_k inter_s[n, k] * W[p, k, w]
+//   inter_s[n, k] = sum_{t in s} coef_t * x[n, a_t, k] * y[n, b_t]                 (y without channels, k = u)
+//   inter_s[n, k] = sum_{t in s} coef_t * x[n, a_t, u] * y[n, b_t, v],  k = u * CY + v   (y with channels: "uvw")
+//
+// Order: coupling first.  The mixed operand inter_s (the reference's stage-1 intermediate, which it writes to memory
+// for the whole batch) is formed on the vector ALUs directly in the layout of an MFMA B operand — lane (n, g) holds
+// k = 16 kb + 4 g + i of sample n — from the rows of x and y staged once per workgroup in LDS, and is contracted
+// with the weights by v_mfma_f32_16x16x4_f32 into a 16 (w) x 16 (n) accumulator tile per block of output channels.
+// The walk is a flat list of items (segment, chunk of k) ordered by output row, so a wavefront keeps only the
+// accumulators of the row it is working on.  fp32 matrix instructions are slow enough (32 cycles each) that the
+// table walk, the mixing (a few dozen FMAs per item) and the LDS reads disappear behind them; weight fragments come
+// from a copy of W repacked in fragment order (one contiguous KB per wavefront load) and are requested one item
+// ahead.  The gradient with respect to the channelled operand is the same kernel with the roles of the rows
+// exchanged and the weight packed transposed; the other two gradients have kernels of their own below.
+#include "cgtp_device.h"
+#include "cgtp_host.h"
+
+#pragma clang fp contract(fast)
+
+namespace cgtp {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kUvtFirst = 1, kUvtLast = 2;   // item flags: first / last item of its output row
+
+struct UvtDev {
+  const float* x;
+  const float* y;
+  const float* wp;
+  float* out;
+  const cgtp_uvt_item* items;
+  const int32_t* ta;
+  const int32_t* tb;
+  const float* tc;
+  int64_t n_rows;
+  int n_items, dx, dy, dout, cx, cy, cout;
+  int kx;        // y without channels: cx rounded up to 16 (row length of the staged x); with: cx
+  int px, py;    // LDS pitch per sample of the x and y tiles, in elements
+  int kblocks;   // K / 16 (K padded to 16)
+  int wbp;       // blocks of 16 output channels, rounded up to a multiple of 4 (as packed)
+  int sb_log2;   // log2 of the 16-sample blocks per workgroup (1, 2 or 4 blocks)
+};
+
+// Rows of the workgroup's samples into LDS: x as [sample][row][kx] (zero-padded channels), y as [sample][row] or
+// [sample][row][cy].  Samples past the end of the batch are staged as zeros.
+template <bool YC>
+__device__ __forceinline__ void uvt_stage(const UvtDev& a, float* xs, float* ys, int64_t nb0, int n_samples) {
+  const int kx4 = a.kx / 4, per_sample = a.dx * kx4;
+  for (int i = threadIdx.x; i < n_samples * per_sample; i += blockDim.x) {
+    const int s = i / per_sample, rem = i - s * per_sample, row = rem / kx4, c4 = rem - row * kx4;
+    const int64_t n = nb0 + s;
+    floatx4 v = {0.f, 0.f, 0.f, 0.f};
+    if (n < a.n_rows && c4 * 4 < a.cx) v = *reinterpret_cast<const floatx4*>(a.x + (n * a.dx + row) * a.cx + c4 * 4);
+    *reinterpret_cast<floatx4*>(xs + (size_t)s * a.px + row * a.kx + c4 * 4) = v;
+  }
+  if constexpr (YC) {
+    const int cy4 = a.cy / 4, per_y = a.dy * cy4;
+    for (int i = threadIdx.x; i < n_samples * per_y; i += blockDim.x) {
+      const int s = i / per_y, rem = i - s * per_y;
+      const int64_t n = nb0 + s;
+      floatx4 v = {0.f, 0.f, 0.f, 0.f};
+      if (n < a.n_rows) v = *reinterpret_cast<const floatx4*>(a.y + n * a.dy * a.cy + rem * 4);
+      *reinterpret_cast<floatx4*>(ys + (size_t)s * a.py + rem * 4) = v;
+    }
+  } else {
+    for (int i = threadIdx.x; i < n_samples * a.dy; i += blockDim.x) {
+      const int s = i / a.dy, b = i - s * a.dy;
+      const int64_t n = nb0 + s;
+      ys[(size_t)s * a.py + b] = n < a.n_rows ? a.y[n * a.dy + b] : 0.f;
+    }
+  }
+}
+
+// This lane's part of the mixed operand of one item: bf[j][i] = inter_s[n, 16 (kb0 + j) + 4 g + i].
+template <bool YC, int KBI>
+__device__ __forceinline__ void uvt_mix(const UvtDev& a, const cgtp_uvt_item& it, const float* xl, const float* yl, int g,
+                                        floatx4 (&bf)[KBI]) {
+#pragma unroll
+  for (int j = 0; j < KBI; ++j) bf[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+  int xo[KBI], yo[KBI];   // with a channelled y: offsets of (u) in a row of x and of (v .. v+3) in a row of y
+  if constexpr (YC) {
+#pragma unroll
+    for (int j = 0; j < KBI; ++j) {
+      const int k0 = (it.kb0 + j) * 16 + 4 * g;
+      xo[j] = k0 / a.cy;
+      yo[j] = k0 - xo[j] * a.cy;
+    }
+  }
+  for (int t = it.t0; t < it.t1; ++t) {
+    const int ia = a.ta[t], ib = a.tb[t];
+    const float c = a.tc[t];
+    if constexpr (YC) {
+      const float* xr = xl + ia * a.cx;
+      const float* yr = yl + ib * a.cy;
+#pragma unroll
+      for (int j = 0; j < KBI; ++j)
+        if (j < it.nkb) bf[j] += (c * xr[xo[j]]) * *reinterpret_cast<const floatx4*>(yr + yo[j]);
+    } else {
+      const float s = c * yl[ib];
+      const floatx4* xr = reinterpret_cast<const floatx4*>(xl + ia * a.kx + it.kb0 * 16 + 4 * g);
+#pragma unroll
+      for (int j = 0; j < KBI; ++j)
+        if (j < it.nkb) bf[j] += s * xr[j * 4];
+    }
+  }
+}
+
+// WB: blocks of 16 output channels per wavefront; KBI: blocks of 16 k per item (the tables are built for it).
+template <bool YC, int WB, int KBI>
+__global__ void __launch_bounds__(256) uvt_apply_kernel(const UvtDev a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int sb_count = 1 << a.sb_log2;
+  float* xs = reinterpret_cast<float*>(smem);
+  float* ys = xs + (size_t)(16 * sb_count) * a.px;
+  const int64_t nb0 = (int64_t)blockIdx.x * (16 * sb_count);
+  uvt_stage<YC>(a, xs, ys, nb0, 16 * sb_count);
+  __syncthreads();
+
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), r = lane & 15, g = lane >> 4;
+  const int sb = wave & (sb_count - 1), wg = wave >> a.sb_log2, wgroups = 4 >> a.sb_log2;
+  const int wb0 = (blockIdx.y * wgroups + wg) * WB;
+  if (wb0 * 16 >= a.cout) return;
+  const int64_t n = nb0 + sb * 16 + r;
+  const float* xl = xs + (size_t)(sb * 16 + r) * a.px;
+  const float* yl = ys + (size_t)(sb * 16 + r) * a.py;
+  const float* wl = a.wp + ((int64_t)wb0 * 64 + lane) * 4;
+
+  floatx4 acc[WB], A0[WB][KBI], A1[WB][KBI];
+  auto load_a = [&](const cgtp_uvt_item& it, floatx4 (&A)[WB][KBI]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < KBI; ++j)
+      if (j < it.nkb) {
+        const float* base = wl + ((int64_t)(it.p * a.kblocks + it.kb0 + j) * a.wbp) * 256;
+#pragma unroll
+        for (int wb = 0; wb < WB; ++wb) A[wb][j] = *reinterpret_cast<const floatx4*>(base + wb * 256);
+      }
+  };
+  auto process = [&](const cgtp_uvt_item& it, floatx4 (&Ac)[WB][KBI], floatx4 (&An)[WB][KBI], bool has_next,
+                     const cgtp_uvt_item& nx) __attribute__((always_inline)) {
+    if (has_next) load_a(nx, An);
+    if (it.flags & kUvtFirst) {
+#pragma unroll
+      for (int wb = 0; wb < WB; ++wb) acc[wb] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+    floatx4 bf[KBI];
+    uvt_mix<YC, KBI>(a, it, xl, yl, g, bf);
+#pragma unroll
+    for (int j = 0; j < KBI; ++j)
+      if (j < it.nkb) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int wb = 0; wb < WB; ++wb)
+            acc[wb] = __builtin_amdgcn_mfma_f32_16x16x4f32(Ac[wb][j][i], bf[j][i], acc[wb], 0, 0, 0);
+      }
+    if (it.flags & kUvtLast) {
+      // accumulator layout: lane (n = r, g) holds output channels 16 wb + 4 g .. + 3 of sample n
+      if (n < a.n_rows) {
+        float* orow = a.out + (n * a.dout + it.out_row) * a.cout;
+#pragma unroll
+        for (int wb = 0; wb < WB; ++wb) {
+          const int w = (wb0 + wb) * 16 + 4 * g;
+          if (w < a.cout) *reinterpret_cast<floatx4*>(orow + w) = acc[wb];
+        }
+      }
+    }
+  };
+
+  cgtp_uvt_item it = a.items[0];
+  load_a(it, A0);
+  for (int j = 0; j < a.n_items; j += 2) {
+    const cgtp_uvt_item it1 = a.items[min(j + 1, a.n_items - 1)];
+    process(it, A0, A1, j + 1 < a.n_items, it1);
+    if (j + 1 >= a.n_items) break;
+    const cgtp_uvt_item it2 = a.items[min(j + 2, a.n_items - 1)];
+    process(it1, A1, A0, j + 2 < a.n_items, it2);
+    it = it2;
+  }
+}
+
+// packed[((p * kblocks + kb) * wbp + wb) * 256 + lane * 4 + i] = W[p][16 kb + 4 (lane / 16) + i][16 wb + lane % 16]
+// (zero outside K x cout), W addressed with element strides so that the transposed weight of the backward needs no
+// copy of its own.
+__global__ void uvt_pack_kernel(const float* __restrict__ w, float* __restrict__ packed, int64_t n_vec, int K, int cout,
+                                int kblocks, int wbp, int64_t stride_p, int64_t stride_k, int64_t stride_c) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_vec) return;
+  const int lane = (int)(i & 63);
+  int64_t c = i >> 6;
+  const int wb = (int)(c % wbp); c /= wbp;
+  const int kb = (int)(c % kblocks);
+  const int64_t p = c / kblocks;
+  const int col = wb * 16 + (lane & 15);
+  floatx4 v = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int k = kb * 16 + 4 * (lane >> 4) + e;
+    if (k < K && col < cout) v[e] = w[p * stride_p + k * stride_k + col * stride_c];
+  }
+  *reinterpret_cast<floatx4*>(packed + i * 4) = v;
+}
+
+struct UvtPlan {
+  int sb_log2, wb, kbi, yc;
+  int64_t lds;
+  dim3 grid;
+  UvtDev dev;
+};
+
+static inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+// Launch shape from the extents alone: LDS pitches, sample blocks per workgroup, channel blocks per wavefront and the
+// chunk length the item list has to be cut for.
+static int uvt_shape(int64_t n_rows, int dx, int dy, int cx, int cy, int cout, UvtPlan* plan) {
+  if (n_rows < 0 || dx <= 0 || dy <= 0 || cx <= 0 || cy < 0 || cout <= 0) return CGTP_ERR_SHAPE;
+  if (cx % 4 || cout % 4 || cy % 4) return CGTP_ERR_SHAPE;
+  const bool yc = cy > 0;
+  if (yc && ((int64_t)cx * cy) % 16) return CGTP_ERR_SHAPE;
+  UvtDev& d = plan->dev;
+  d.n_rows = n_rows; d.dx = dx; d.dy = dy; d.cx = cx; d.cy = cy; d.cout = cout;
+  const int64_t K = yc ? (int64_t)cx * cy : cx;
+  d.kx = yc ? cx : round_up(cx, 16);
+  d.px = dx * d.kx + 4;
+  d.py = yc ? dy * cy + 4 : (dy | 1);
+  d.kblocks = (int)((K + 15) / 16);
+  const int wblocks = (cout + 15) / 16;
+  d.wbp = round_up(wblocks, 4);
+  const int64_t per_block = (int64_t)16 * (d.px + d.py) * 4;   // LDS bytes of one 16-sample block
+  if (per_block > kLdsBytes) return CGTP_ERR_LDS;
+  // sample blocks per workgroup: as many as keep two workgroups per compute unit, else as many as fit; fewer when the
+  // batch is too small to fill the chip with such workgroups
+  int sb_log2 = 2;
+  while (sb_log2 > 0 && (per_block << sb_log2) > kLdsBytes / 2 - 1024) --sb_log2;
+  const int64_t blocks16 = (n_rows + 15) / 16;
+  while (sb_log2 > 0 && (blocks16 >> sb_log2) < 512) --sb_log2;
+  d.sb_log2 = sb_log2;
+  const int wgroups = 4 >> sb_log2;
+  const int need = (wblocks + wgroups - 1) / wgroups;
+  const int wb = need >= 4 ? 4 : need >= 2 ? 2 : 1;
+  plan->sb_log2 = sb_log2; plan->wb = wb; plan->kbi = wb == 4 ? 4 : 8; plan->yc = yc;
+  plan->lds = per_block << sb_log2;
+  plan->grid = dim3((unsigned)((blocks16 + (1 << sb_log2) - 1) >> sb_log2),
+                    (unsigned)((wblocks + wgroups * wb - 1) / (wgroups * wb)));
+  return CGTP_OK;
+}
+
+static int uvt_plan(const cgtp_uvt_args* a, UvtPlan* plan) {
+  if (!a) return CGTP_ERR_NULL;
+  if (a->dtype != CGTP_F32) return CGTP_ERR_DTYPE;
+  if (a->n_items < 0 || a->dout <= 0) return CGTP_ERR_SHAPE;
+  const int st = uvt_shape(a->n_rows, a->dx, a->dy, a->cx, a->cy, a->cout, plan);
+  if (st != CGTP_OK) return st;
+  if (a->kbi != plan->kbi) return CGTP_ERR_SHAPE;   // the item list must be cut for this launch shape: cgtp_uvt_chunk()
+  if (!a->x || !a->y || !a->wp || !a->out || (a->n_items && (!a->items || !a->term_a || !a->term_b || !a->term_c)))
+    return CGTP_ERR_NULL;
+  const uintptr_t al = reinterpret_cast<uintptr_t>(a->x) | reinterpret_cast<uintptr_t>(a->wp) |
+                       reinterpret_cast<uintptr_t>(a->out) | (a->cy > 0 ? reinterpret_cast<uintptr_t>(a->y) : 0);
+  if (al & 15u) return CGTP_ERR_ALIGN;
+  UvtDev& d = plan->dev;
+  d.x = (const float*)a->x; d.y = (const float*)a->y; d.wp = (const float*)a->wp; d.out = (float*)a->out;
+  d.items = a->items; d.ta = a->term_a; d.tb = a->term_b; d.tc = (const float*)a->term_c;
+  d.n_items = a->n_items; d.dout = a->dout;
+  return CGTP_OK;
+}
+
+}  // namespace cgtp
+
+using namespace cgtp;
+
+extern "C" {
+
+int64_t cgtp_uvt_packed_elems(int32_t n_paths, int64_t K, int32_t cout) {
+  if (n_paths < 0 || K <= 0 || cout <= 0) return 0;
+  return (int64_t)n_paths * ((K + 15) / 16) * round_up((cout + 15) / 16, 4) * 256;
+}
+
+int cgtp_uvt_pack_weights(const void* w, void* packed, int32_t n_paths, int64_t K, int32_t cout, int64_t stride_p,
+                          int64_t stride_k, int64_t stride_c, int32_t dtype, void* stream) {
+  if (dtype != CGTP_F32) return CGTP_ERR_DTYPE;
+  if (!w || !packed) return CGTP_ERR_NULL;
+  if (n_paths < 0 || K <= 0 || cout <= 0 || K > (1 << 24)) return CGTP_ERR_SHAPE;
+  if (reinterpret_cast<uintptr_t>(packed) & 15u) return CGTP_ERR_ALIGN;
+  const int64_t n_vec = cgtp_uvt_packed_elems(n_paths, K, cout) / 4;
+  if (n_vec == 0) return CGTP_OK;
+  hipLaunchKernelGGL(uvt_pack_kernel, dim3((unsigned)((n_vec + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const float*)w, (float*)packed, n_vec, (int)K, (int)cout, (int)((K + 15) / 16),
+                     round_up((cout + 15) / 16, 4), stride_p, stride_k, stride_c);
+  return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
+}
+
+int cgtp_uvt_chunk(int64_t n_rows, int32_t dx, int32_t dy, int32_t cx, int32_t cy, int32_t cout) {
+  UvtPlan plan;
+  const int st = uvt_shape(n_rows, dx, dy, cx, cy, cout, &plan);
+  return st == CGTP_OK ? plan.kbi : -st;
+}
+
+int cgtp_uvt_validate(const cgtp_uvt_args* a) {
+  UvtPlan plan;
+  return uvt_plan(a, &plan);
+}
+
+int cgtp_uvt_apply(const cgtp_uvt_args* a, void* stream) {
+  UvtPlan plan;
+  const int st = uvt_plan(a, &plan);
+  if (st != CGTP_OK) return st;
+  if (a->n_rows == 0 || a->n_items == 0) return CGTP_OK;
+  void (*fn)(const UvtDev) = nullptr;
+  if (plan.yc) {
+    fn = plan.wb == 4 ? uvt_apply_kernel<true, 4, 4> : plan.wb == 2 ? uvt_apply_kernel<true, 2, 8> : uvt_apply_kernel<true, 1, 8>;
+  } else {
+    fn = plan.wb == 4 ? uvt_apply_kernel<false, 4, 4> : plan.wb == 2 ? uvt_apply_kernel<false, 2, 8> : uvt_apply_kernel<false, 1, 8>;
+  }
+  if (plan.lds > 48 * 1024 &&
+      hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds) != hipSuccess)
+    return CGTP_ERR_LDS;
+  hipLaunchKernelGGL(fn, plan.grid, dim3(256), (size_t)plan.lds, (hipStream_t)stream, plan.dev);
+  return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
+}
+
+}  // extern "C"

@@ -1,0 +1,231 @@
+"""Fully connected products in fp32 with a shared weight on the table-driven matrix-core kernels (``cgtp_uvt_*``):
+``tensor_product_u1v`` (``SO3Linear('uv')``) and ``tensor_product_uvw`` (``TensorProduct('uvw')``) for any irreps and
+normalisation, forward and first-order gradients, without the reference's ``(N, segments, C)`` intermediate
+(``equitorch/nn/functional/linears.py:257-336``, ``tensor_products.py:92-172``).
+
+The kernels walk a flat list of items (segment = (weight path, output row), chunk of the contracted channel axis)
+ordered by output row; this module cuts that list from the table for each of the roles a product is used in:
+
+    forward      out[M]   <- first operand rows M1, second operand rows M2, weight as stored
+    grad first   g1[M1]   <- rows M of grad_out,   second operand rows M2, weight transposed
+    ('uvw' only) g2[M2]   <- rows M of grad_out,   first operand rows M1,  weight permuted
+"""
+import ctypes as C
+from typing import Optional
+
+import numpy as np
+import torch
+from torch import Tensor
+from torch.autograd import Function
+
+from ... import _lib
+from ...ops import kernels
+
+FIRST, LAST = 1, 2
+
+
+class _Walk:
+    """Item list of one role of one table, cut for ``kblocks`` blocks of 16 contracted channels in chunks of ``kbi``."""
+
+    def __init__(self, out_idx, a_idx, b_idx, p_idx, coef, n_out: int, kblocks: int, kbi: int, device):
+        order = np.lexsort([b_idx, a_idx, p_idx, out_idx])
+        out_idx, a_idx, b_idx, p_idx = (np.asarray(v)[order] for v in (out_idx, a_idx, b_idx, p_idx))
+        coef = np.asarray(coef, dtype=np.float64)[order]
+        items = []
+        t, n_terms = 0, out_idx.shape[0]
+        for row in range(n_out):
+            first = len(items)
+            while t < n_terms and out_idx[t] == row:
+                t1 = t
+                while t1 < n_terms and out_idx[t1] == row and p_idx[t1] == p_idx[t]:
+                    t1 += 1
+                for kb0 in range(0, kblocks, kbi):
+                    items.append([int(p_idx[t]), kb0, min(kbi, kblocks - kb0), t, t1, row, 0, 0])
+                t = t1
+            if len(items) == first:                       # a row without terms is written as zeros
+                items.append([0, 0, 0, 0, 0, row, 0, 0])
+            items[first][6] |= FIRST
+            items[-1][6] |= LAST
+        self.n_items = len(items)
+        self.kbi = kbi
+        self.items = torch.tensor(items, dtype=torch.int32).to(device)
+        self.term_a = torch.from_numpy(a_idx.astype(np.int32)).to(device)
+        self.term_b = torch.from_numpy(b_idx.astype(np.int32)).to(device)
+        self.term_c = torch.from_numpy(coef.astype(np.float32)).to(device)
+
+
+def _walk(tp_info, role: str, kblocks: int, kbi: int, device) -> _Walk:
+    def build():
+        c = kernels.coo_of(tp_info)
+        if role == "out":        # rows of the first operand, rows of the second operand
+            return _Walk(c.M, c.M1, c.M2, c.p, c.coef, c.DO, kblocks, kbi, device)
+        if role == "in1":        # first operand of the launch = grad_out, second = input2
+            return _Walk(c.M1, c.M, c.M2, c.p, c.coef, c.D1, kblocks, kbi, device)
+        if role == "in1_uvw":    # first operand of the launch = input2, second = grad_out
+            return _Walk(c.M1, c.M2, c.M, c.p, c.coef, c.D1, kblocks, kbi, device)
+        if role == "in2_uvw":    # first operand of the launch = grad_out, second = input1
+            return _Walk(c.M2, c.M, c.M1, c.p, c.coef, c.D2, kblocks, kbi, device)
+        raise ValueError(role)
+    return kernels.cached(tp_info.info_Mij_fwd.scale, ("uvt_walk", role, kblocks, kbi, str(device)), build)
+
+
+def chunk_of(n_rows: int, dx: int, dy: int, cx: int, cy: int, cout: int) -> int:
+    """Chunk length (blocks of 16 contracted channels per item) of a launch with these extents; <= 0: the kernels do
+    not take them (channel counts not multiples of 4, rows of 16 samples beyond the LDS)."""
+    return int(_lib.lib.cgtp_uvt_chunk(n_rows, dx, dy, cx, cy, cout))
+
+
+def pack(w: Tensor, n_paths: int, k: int, cout: int, stride_p: int, stride_k: int, stride_c: int) -> Tensor:
+    """The weight viewed as ``(n_paths, k, cout)`` through element strides, in matrix-core fragment order."""
+    packed = torch.empty(int(_lib.lib.cgtp_uvt_packed_elems(n_paths, k, cout)), dtype=torch.float32, device=w.device)
+    _lib.check(_lib.lib.cgtp_uvt_pack_weights(w.data_ptr(), packed.data_ptr(), n_paths, k, cout, stride_p, stride_k,
+                                              stride_c, _lib.F32, _lib.stream_ptr(w.device)), "cgtp_uvt_pack_weights")
+    return packed
+
+
+def apply(x: Tensor, y: Tensor, wp: Tensor, tp_info, role: str, dout: int, cout: int) -> Tensor:
+    """One launch of ``cgtp_uvt_apply``: ``x (N, dx, cx)``, ``y (N, dy)`` or ``(N, dy, cy)`` -> ``(N, dout, cout)``."""
+    n, dx, cx = x.shape
+    dy = y.shape[1]
+    cy = y.shape[2] if y.ndim == 3 else 0
+    k = cx * cy if cy else cx
+    kbi = chunk_of(n, dx, dy, cx, cy, cout)
+    if kbi <= 0:
+        raise _lib.CgtpError(f"cgtp_uvt_apply does not take these extents (status {-kbi})")
+    walk = _walk(tp_info, role, (k + 15) // 16, kbi, x.device)
+    out = torch.empty((n, dout, cout), dtype=x.dtype, device=x.device)
+    if n == 0:
+        return out
+    a = _lib.UvtArgs()
+    a.x, a.y, a.wp, a.out = x.data_ptr(), y.data_ptr(), wp.data_ptr(), out.data_ptr()
+    a.items, a.term_a, a.term_b, a.term_c = (walk.items.data_ptr(), walk.term_a.data_ptr(), walk.term_b.data_ptr(),
+                                             walk.term_c.data_ptr())
+    a.n_rows, a.n_items = n, walk.n_items
+    a.dx, a.dy, a.dout, a.cx, a.cy, a.cout = dx, dy, dout, cx, cy, cout
+    a.kbi, a.dtype = kbi, _lib.F32
+    _lib.check(_lib.lib.cgtp_uvt_apply(C.byref(a), _lib.stream_ptr(x.device)), "cgtp_uvt_apply")
+    return out
+
+
+def _coo(tp_info):
+    return kernels.coo_of(tp_info)
+
+
+class _U1vNative(Function):
+    """u1v, shared fp32 weight ``(P, U, W)``.  The gradient of the first operand is the same kernel with the rows'
+    roles exchanged and the weight read transposed; the gradients of the second operand and of the weight come from
+    the differentiable two-stage route of ``_uv_gemm`` for now (library GEMMs), as does everything under
+    ``create_graph``."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, y: Tensor, w: Tensor, tp_info):
+        c = _coo(tp_info)
+        p, u, wc = w.shape
+        out = apply(x, y, pack(w, p, u, wc, u * wc, wc, 1), tp_info, "out", c.DO, wc)
+        ctx.save_for_backward(x, y, w)
+        ctx.tp_info = tp_info
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        from . import _uv_gemm
+        x, y, w = ctx.saved_tensors
+        need = ctx.needs_input_grad[:3]
+        tp_info = ctx.tp_info
+        if torch.is_grad_enabled():       # higher-order derivative: the differentiable route throughout
+            with torch.enable_grad():
+                out = _uv_gemm.u1v(x, y, w, tp_info)
+                wanted = [t for t, n in zip((x, y, w), need) if n]
+                got = iter(torch.autograd.grad(out, wanted, g, create_graph=True, allow_unused=True))
+            return tuple(next(got) if n else None for n in need) + (None,)
+        c = _coo(tp_info)
+        p, u, wc = w.shape
+        gx = gy = gw = None
+        g = g.contiguous()
+        if need[0]:
+            gx = apply(g, y, pack(w, p, wc, u, u * wc, 1, wc), tp_info, "in1", c.D1, u)
+        if need[1] or need[2]:
+            with torch.enable_grad():
+                yr, wr = y.detach().requires_grad_(need[1]), w.detach().requires_grad_(need[2])
+                out = _uv_gemm.u1v(x.detach(), yr, wr, tp_info)
+                wanted = [t for t, n in zip((yr, wr), need[1:]) if n]
+                got = iter(torch.autograd.grad(out, wanted, g))
+            gy = next(got) if need[1] else None
+            gw = next(got) if need[2] else None
+        return gx, gy, gw, None
+
+
+def u1v_supported(x: Tensor, y: Tensor, w: Tensor, tp_info) -> bool:
+    if not (x.dtype == y.dtype == w.dtype == torch.float32 and x.ndim == 3 and y.ndim == 2 and w.ndim == 3):
+        return False
+    if x.shape[0] == 0:
+        return False
+    c = _coo(tp_info)
+    _, u, wc = w.shape
+    n = x.shape[0]
+    return (chunk_of(n, c.D1, c.D2, u, 0, wc) > 0 and chunk_of(n, c.DO, c.D2, wc, 0, u) > 0
+            and x.data_ptr() % 16 == 0)
+
+
+def u1v(x: Tensor, y: Tensor, w: Tensor, tp_info) -> Tensor:
+    return _U1vNative.apply(x.contiguous(), y.contiguous(), w.contiguous(), tp_info)
+
+
+class _UvwNative(Function):
+    """uvw, shared fp32 weight ``(P, U, V, W)``: forward and the gradients of both operands on ``cgtp_uvt_apply``
+    (with the weight permuted as the reference permutes it, ``tensor_products.py:126-150``); the weight gradient and
+    higher orders from the two-stage route of ``_uvw_gemm``."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, y: Tensor, w: Tensor, tp_info):
+        c = _coo(tp_info)
+        p, u, v, wc = w.shape
+        out = apply(x, y, pack(w, p, u * v, wc, u * v * wc, wc, 1), tp_info, "out", c.DO, wc)
+        ctx.save_for_backward(x, y, w)
+        ctx.tp_info = tp_info
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        from . import _uvw_gemm
+        x, y, w = ctx.saved_tensors
+        need = ctx.needs_input_grad[:3]
+        tp_info = ctx.tp_info
+        if torch.is_grad_enabled():
+            with torch.enable_grad():
+                out = _uvw_gemm.uvw(x, y, w, tp_info)
+                wanted = [t for t, n in zip((x, y, w), need) if n]
+                got = iter(torch.autograd.grad(out, wanted, g, create_graph=True, allow_unused=True))
+            return tuple(next(got) if n else None for n in need) + (None,)
+        c = _coo(tp_info)
+        p, u, v, wc = w.shape
+        g = g.contiguous()
+        gx = gy = gw = None
+        if need[0]:     # first operand of the launch: y (channels v), second: grad_out (channels w); weight (P, V, W, U)
+            wt = w.permute(0, 2, 3, 1).contiguous()
+            gx = apply(y, g, pack(wt, p, v * wc, u, v * wc * u, u, 1), tp_info, "in1_uvw", c.D1, u)
+        if need[1]:     # first: grad_out (channels w), second: x (channels u); weight (P, W, U, V)
+            wt = w.permute(0, 3, 1, 2).contiguous()
+            gy = apply(g, x, pack(wt, p, wc * u, v, wc * u * v, v, 1), tp_info, "in2_uvw", c.D2, v)
+        if need[2]:
+            with torch.enable_grad():
+                wr = w.detach().requires_grad_(True)
+                out = _uvw_gemm.uvw(x.detach(), y.detach(), wr, tp_info)
+                (gw,) = torch.autograd.grad(out, (wr,), g)
+        return gx, gy, gw, None
+
+
+def uvw_supported(x: Tensor, y: Tensor, w: Tensor, tp_info) -> bool:
+    if not (x.dtype == y.dtype == w.dtype == torch.float32 and x.ndim == 3 and y.ndim == 3 and w.ndim == 4):
+        return False
+    if x.shape[0] == 0:
+        return False
+    c = _coo(tp_info)
+    _, u, v, wc = w.shape
+    n = x.shape[0]
+    return (chunk_of(n, c.D1, c.D2, u, v, wc) > 0 and chunk_of(n, c.D2, c.DO, v, wc, u) > 0
+            and chunk_of(n, c.DO, c.D1, wc, u, v) > 0 and x.data_ptr() % 16 == 0 and y.data_ptr() % 16 == 0)
+
+
+def uvw(x: Tensor, y: Tensor, w: Tensor, tp_info) -> Tensor:
+    return _UvwNative.apply(x.contiguous(), y.contiguous(), w.contiguous(), tp_info)

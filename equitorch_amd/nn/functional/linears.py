@@ -108,6 +108,10 @@ def tensor_product_u1v(input1: Tensor, input2: Tensor, weight: Tensor,
     if fast is not None:
         kernels.log_tier("tensor_product_u1v", "matrix-core kernel (compiled table)")
         return fast
+    from . import _uv_native
+    if _uv_native.u1v_supported(input1, input2, weight, tp_info_forward):
+        kernels.log_tier("tensor_product_u1v", "fp32 matrix-core kernel (table-driven)")
+        return _uv_native.u1v(input1, input2, weight, tp_info_forward)
     if input1.ndim == 3 and input2.ndim == 2 and _uv_gemm.supported(input1, input2, weight):
         kernels.log_tier("tensor_product_u1v", "library GEMM + table-driven kernel", str(input1.dtype))
         return _uv_gemm.u1v(input1, input2, weight, tp_info_forward)

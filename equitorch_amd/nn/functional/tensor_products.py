@@ -72,7 +72,11 @@ def tensor_product_uvw(input1: Tensor, input2: Tensor, weight: Tensor,
     if weight.ndim not in (4, 5) or input1.dtype != input2.dtype or input1.dtype != weight.dtype:
         raise _lib.CgtpError(f"tensor_product_uvw: operands {input1.dtype}, {input2.dtype}, {weight.dtype} with "
                              f"weight of {weight.ndim} dims")
-    from . import _uvw_gemm
+    from . import _uv_native, _uvw_gemm
+    if _uv_native.uvw_supported(input1, input2, weight, tp_info_forward):
+        kernels.log_tier("tensor_product_uvw", "fp32 matrix-core kernel (table-driven)")
+        return _uv_native.uvw(input1, input2, weight, tp_info_forward)
+    kernels.log_tier("tensor_product_uvw", "table-driven outer products + library GEMM", str(input1.dtype))
     return _uvw_gemm.uvw(input1.contiguous(), input2.contiguous(), weight, tp_info_forward)
 
 

@@ -442,7 +442,7 @@ class SegIndex:
     """Per-sorted-position index arrays of the segment mode (all int64, same device)."""
 
     def __init__(self, ptr: Tensor, perm: Optional[Tensor], seg_ids: Tensor, gather: Tensor,
-                 positions_per_wave: int = 32):
+                 positions_per_wave: int = int(__import__("os").environ.get("CGTP_POSITIONS_PER_WAVE", "32"))):
         self.ptr, self.perm, self.seg_ids, self.gather = ptr, perm, seg_ids, gather
         self.wave_seg = self.aligned_ranges(ptr, positions_per_wave)
 

@@ -41,7 +41,7 @@ int cgtp_version(void);
  * cgo, JNI) can check itself: which = CGTP_LAYOUT_*; writes sizeof(struct) followed by the byte offset of every field
  * in declaration order to out[0 .. capacity) and returns how many numbers the full description has (-1: bad id). */
 enum { CGTP_LAYOUT_OPERAND = 0, CGTP_LAYOUT_TRI_ARGS = 1, CGTP_LAYOUT_GEN_OPERAND = 2, CGTP_LAYOUT_GEN_ARGS = 3,
-       CGTP_LAYOUT_UVU_ARGS = 4 };
+       CGTP_LAYOUT_UVU_ARGS = 4, CGTP_LAYOUT_UVT_ITEM = 5, CGTP_LAYOUT_UVT_ARGS = 6 };
 int cgtp_abi_layout(int which, int64_t* out, int capacity);
 
 /* ---- generic sparse trilinear contraction -------------------------------------------------------------
@@ -289,6 +289,58 @@ int cgtp_uv_grad_y(int cfg, const void* x, const void* g, const void* wp, void* 
 int64_t cgtp_uv_grad_w_workspace_bytes(int cfg, int64_t n_rows, int32_t cin, int32_t cout);
 int cgtp_uv_grad_w(int cfg, const void* x, const void* y, const void* g, void* gw, void* workspace, int64_t n_rows,
                    int32_t cin, int32_t cout, int32_t dtype, const float* path_scale, void* stream);
+
+/* ---- fully connected products in fp32 on the matrix cores, any table --------------------------------------------
+ *
+ *   out[n, M, w] = sum_{segments s = (p, M)} sum_k inter_s[n, k] * W[p, k, w]
+ *   inter_s[n, k] = sum_{t in s} coef_t * x[n, a_t, k] * y[n, b_t]                       (cy == 0, K = cx)
+ *   inter_s[n, k] = sum_{t in s} coef_t * x[n, a_t, u] * y[n, b_t, v],  k = u * cy + v   (cy > 0, K = cx * cy)
+ *
+ * One fused launch for TensorProductU1VDummy.forward (equitorch/nn/functional/linears.py:257-280: vecsca, then vecmat
+ * with the (N, segments, C_in) intermediate in memory), for TensorProductUVWDummy.forward
+ * (equitorch/nn/functional/tensor_products.py:95-101: outer, then vecmat over the flattened (u, v) axis) and, with
+ * the rows' roles exchanged and the weight packed transposed, for the grad-input products of their backward passes
+ * (tensor_product_1vu / tensor_product_uvw with permuted weights, linears.py:290-293, tensor_products.py:126-150).
+ * Shared weights only.  The caller supplies the walk as a flat list of items ordered by output row: an item is one
+ * segment restricted to `nkb` blocks of 16 consecutive k starting at block kb0, with its terms t0..t1 in (term_a =
+ * row of x, term_b = row of y, term_c = coefficient); flags: 1 = first item of its output row, 2 = last.  Every output
+ * row needs at least one item (nkb = 0 for a row without terms: it is written as zeros).  nkb <= the chunk length
+ * cgtp_uvt_chunk() reports for the extents, which must also be passed as `kbi`.
+ * x (n_rows, dx, cx), y (n_rows, dy) or (n_rows, dy, cy), out (n_rows, dout, cout), all fp32 and contiguous; cx, cy,
+ * cout multiples of 4, cx * cy a multiple of 16 when cy > 0; 16-byte aligned pointers; the rows of 16 samples must
+ * fit the LDS (CGTP_ERR_LDS otherwise).  wp = cgtp_uvt_pack_weights(W): W (n_paths, K, cout) read through element
+ * strides (so that a transposed or flattened view needs no copy), rewritten in matrix-core fragment order, zero-padded;
+ * cgtp_uvt_packed_elems() elements.
+ */
+typedef struct cgtp_uvt_item {
+  int32_t p, kb0, nkb, t0, t1, out_row, flags, reserved_;
+} cgtp_uvt_item;
+
+typedef struct cgtp_uvt_args {
+  const void* x;
+  const void* y;
+  const void* wp;
+  void* out;
+  const cgtp_uvt_item* items;   /* device */
+  const int32_t* term_a;        /* device */
+  const int32_t* term_b;        /* device */
+  const void* term_c;           /* device, dtype */
+  int64_t n_rows;
+  int32_t n_items;
+  int32_t dx, dy, dout;
+  int32_t cx, cy, cout;
+  int32_t kbi;                  /* chunk length the items were cut for: cgtp_uvt_chunk() */
+  int32_t dtype;                /* CGTP_F32 */
+  int32_t reserved_;
+} cgtp_uvt_args;
+
+int64_t cgtp_uvt_packed_elems(int32_t n_paths, int64_t K, int32_t cout);
+int cgtp_uvt_pack_weights(const void* w, void* packed, int32_t n_paths, int64_t K, int32_t cout, int64_t stride_p,
+                          int64_t stride_k, int64_t stride_c, int32_t dtype, void* stream);
+/* Blocks of 16 k per item for these extents (4 or 8), or -status when the kernels do not take them.  Host only. */
+int cgtp_uvt_chunk(int64_t n_rows, int32_t dx, int32_t dy, int32_t cx, int32_t cy, int32_t cout);
+int cgtp_uvt_validate(const cgtp_uvt_args* args);
+int cgtp_uvt_apply(const cgtp_uvt_args* args, void* stream);
 
 /* ---- real spherical harmonics of vectors -----------------------------------------------------------------
  * Stands in for spherical_harmonics (equitorch/ops/spherical_harmonics.py:68-640: explicit polynomials per

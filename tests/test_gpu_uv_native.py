@@ -1,0 +1,107 @@
+"""GPU parity of the fully connected products in fp32 on the table-driven matrix-core kernels (``cgtp_uvt_*``):
+``SO3Linear('uv')`` / ``tensor_product_u1v`` and ``TensorProduct('uvw')`` / ``tensor_product_uvw`` with a shared
+weight, forward and all first-order gradients, against the dense float64 oracle (pinned on the CPU in
+tests/test_oracle_uv.py).  Results are sums over C_in (x C_2) channels and all paths of an output irrep of products
+of N(0,1) numbers: compared norm-wise (1e-5 of the tensor's largest magnitude)."""
+import pytest
+import torch
+
+from helpers import assert_close, unit_vectors
+from oracle import ref_ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _sh(lmax):
+    return "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+
+
+U1V_CASES = [  # irreps (out, in1, in2), C_in, C_out, N, module options
+    ((_sh(1),) * 3, 32, 32, 70, {}),
+    ((_sh(2),) * 3, 64, 128, 257, {}),
+    ((_sh(3),) * 3, 128, 128, 300, {}),
+    ((_sh(3),) * 3, 128, 64, 33, {"path_norm": False}),
+    ((_sh(2),) * 3, 20, 12, 1100, {}),                          # C_in padded to 32, C_out below one block of 16
+    ((_sh(2),) * 3, 32, 36, 515, {"channel_norm": True}),       # C_out = 2 blocks + 4
+    (("1o+2e+1e", "0e+1o+2e", "0e+1o"), 48, 40, 200, {}),       # irreps without a compiled table
+    (("0e+1e+2e+3e", "0e+1e+2e", "0e+1e+2e"), 16, 16, 64, {}),
+]
+
+
+@pytest.mark.parametrize("irreps,cin,cout,n,kw", U1V_CASES)
+def test_u1v_fp32_native(device, irreps, cin, cout, n, kw):
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import _uv_native
+    io, i1, i2 = irreps
+    mod = SO3Linear(i1, i2, io, cin, cout, internal_weights=False, feature_mode="uv", **kw).to(device)
+    d1, d2, do = Irreps(i1).dim, Irreps(i2).dim, Irreps(io).dim
+    g = torch.Generator().manual_seed(cin * 1000 + cout + n)
+    x = torch.randn(n, d1, cin, generator=g)
+    y = torch.randn(n, d2, generator=g)
+    w = torch.randn(mod.num_paths, cin, cout, generator=g) / cin ** 0.5
+    ct = torch.randn(n, do, cout, generator=g)
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    assert _uv_native.u1v_supported(xd, yd, wd, mod.tp_info_forward)
+    out = mod(xd, yd, wd)
+    gx, gy, gw = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
+    T = ref_ops.dense_coupling(io, i1, i2, path_norm=kw.get("path_norm", True),
+                               channel_norm=kw.get("channel_norm", False), channel_scale=cin ** -0.5).float().double()
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x, y, w), ct)
+    for name, a, b in zip(("out", "grad_x", "grad_y", "grad_w"), (out, gx, gy, gw), (ref_out, *ref_grads)):
+        assert_close(a, b, 1e-5, f"u1v {io} C={cin}->{cout} N={n} {name}", norm="max")
+
+
+UVW_CASES = [  # irreps, (U, V, W), N
+    ((_sh(2), _sh(2), "0e+1o"), (8, 16, 4), 301),
+    ((_sh(2), _sh(2), "0e+1o"), (32, 32, 8), 301),
+    ((_sh(2),) * 3, (32, 32, 32), 129),
+    ((_sh(2),) * 3, (16, 4, 64), 1000),
+    (("0e+1e+2e+3e", "0e+1e+2e", "0e+1e+2e"), (16, 16, 16), 256),   # the reference's comparison-test shape
+]
+
+
+@pytest.mark.parametrize("irreps,channels,n", UVW_CASES)
+def test_uvw_fp32_native(device, irreps, channels, n):
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.nn.functional import _uv_native
+    from equitorch_amd.utils import tp_infos
+    io, i1, i2 = irreps
+    infos = [t.to(device) for t in tp_infos(Irreps(io), Irreps(i1), Irreps(i2))[:3]]
+    T = ref_ops.dense_coupling(io, i1, i2).float().double()
+    u, v, wc = channels
+    g = torch.Generator().manual_seed(u * 100 + v * 10 + wc)
+    x = torch.randn(n, Irreps(i1).dim, u, generator=g)
+    y = torch.randn(n, Irreps(i2).dim, v, generator=g)
+    w = torch.randn(T.shape[0], u, v, wc, generator=g) / (u * v) ** 0.5
+    ct = torch.randn(n, Irreps(io).dim, wc, generator=g)
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    assert _uv_native.uvw_supported(xd, yd, wd, infos[0])
+    out = F.tensor_product_uvw(xd, yd, wd, *infos)
+    gx, gy, gw = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_uvw, T, (x, y, w), ct)
+    for name, a, b in zip(("out", "grad_x", "grad_y", "grad_w"), (out, gx, gy, gw), (ref_out, *ref_grads)):
+        assert_close(a, b, 1e-5, f"uvw {channels} N={n} {name}", norm="max")
+
+
+def test_u1v_fp32_native_full_size(device):
+    """The shapes of BASELINE configs[3] in fp32 (B = 32768, lmax = 3, C = 128): rows of a strided subset against
+    the oracle (each output row depends on its own sample only)."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.utils._sh import spherical_harmonics
+    irr, ch, n = _sh(3), 128, 32768
+    mod = SO3Linear(irr, irr, irr, ch, ch, internal_weights=False, feature_mode="uv").to(device)
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(n, 16, ch, generator=g)
+    y = spherical_harmonics(unit_vectors(n, g), 3)
+    w = torch.randn(mod.num_paths, ch, ch, generator=g) / (ch * mod.num_paths) ** 0.5
+    ct = torch.randn(n, 16, ch, generator=g)
+    sub = torch.arange(5, n, 257)
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    out = mod(xd, yd, wd)
+    (gx,) = torch.autograd.grad(out, (xd,), ct.to(device))
+    T = ref_ops.dense_coupling(irr, irr, irr).float().double()
+    ref_out, (rgx, _, _) = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x[sub], y[sub], w), ct[sub])
+    assert_close(out[sub.to(device)], ref_out, 1e-5, "full size out", norm="max")
+    assert_close(gx[sub.to(device)], rgx, 1e-5, "full size grad_x", norm="max")
