@@ -71,7 +71,7 @@ class UvtArgs(C.Structure):
                 ("n_rows", C.c_int64), ("n_items", C.c_int32),
                 ("dx", C.c_int32), ("dy", C.c_int32), ("dout", C.c_int32),
                 ("cx", C.c_int32), ("cy", C.c_int32), ("cout", C.c_int32),
-                ("kbi", C.c_int32), ("dtype", C.c_int32), ("reserved_", C.c_int32)]
+                ("kbi", C.c_int32), ("dtype", C.c_int32), ("n_terms", C.c_int32)]
 
 
 def _load():

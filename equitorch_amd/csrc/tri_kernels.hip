@@ -588,7 +588,7 @@ int cgtp_abi_layout(int which, int64_t* out, int capacity) {
                                 CGTP_OFF(cgtp_uvt_args, n_items), CGTP_OFF(cgtp_uvt_args, dx), CGTP_OFF(cgtp_uvt_args, dy),
                                 CGTP_OFF(cgtp_uvt_args, dout), CGTP_OFF(cgtp_uvt_args, cx), CGTP_OFF(cgtp_uvt_args, cy),
                                 CGTP_OFF(cgtp_uvt_args, cout), CGTP_OFF(cgtp_uvt_args, kbi), CGTP_OFF(cgtp_uvt_args, dtype),
-                                CGTP_OFF(cgtp_uvt_args, reserved_)};
+                                CGTP_OFF(cgtp_uvt_args, n_terms)};
 #undef CGTP_OFF
   const int64_t* tabs[] = {operand, tri, gen_operand, gen, uvu, uvt_item, uvt};
   const int counts[] = {(int)(sizeof(operand) / 8), (int)(sizeof(tri) / 8), (int)(sizeof(gen_operand) / 8),

@@ -25,6 +25,7 @@ namespace cgtp {
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kUvtFirst = 1, kUvtLast = 2;   // item flags: first / last item of its output row
+constexpr int64_t kUvtTableRoom = 24 * 1024;  // LDS kept free for the walk tables when the launch shape is chosen
 
 struct UvtDev {
   const float* x;
@@ -36,12 +37,13 @@ struct UvtDev {
   const int32_t* tb;
   const float* tc;
   int64_t n_rows;
-  int n_items, dx, dy, dout, cx, cy, cout;
+  int n_items, n_terms, dx, dy, dout, cx, cy, cout;
   int kx;        // y without channels: cx rounded up to 16 (row length of the staged x); with: cx
   int px, py;    // LDS pitch per sample of the x and y tiles, in elements
   int kblocks;   // K / 16 (K padded to 16)
   int wbp;       // blocks of 16 output channels, rounded up to a multiple of 4 (as packed)
   int sb_log2;   // log2 of the 16-sample blocks per workgroup (1, 2 or 4 blocks)
+  int zero_floats;  // zeros in LDS that the unused term slots of an item read
 };
 
 // Rows of the workgroup's samples into LDS: x as [sample][row][kx] (zero-padded channels), y as [sample][row] or
@@ -74,49 +76,148 @@ __device__ __forceinline__ void uvt_stage(const UvtDev& a, float* xs, float* ys,
   }
 }
 
-// This lane's part of the mixed operand of one item: bf[j][i] = inter_s[n, 16 (kb0 + j) + 4 g + i].
-template <bool YC, int KBI>
-__device__ __forceinline__ void uvt_mix(const UvtDev& a, const cgtp_uvt_item& it, const float* xl, const float* yl, int g,
-                                        floatx4 (&bf)[KBI]) {
-#pragma unroll
-  for (int j = 0; j < KBI; ++j) bf[j] = floatx4{0.f, 0.f, 0.f, 0.f};
-  int xo[KBI], yo[KBI];   // with a channelled y: offsets of (u) in a row of x and of (v .. v+3) in a row of y
-  if constexpr (YC) {
-#pragma unroll
-    for (int j = 0; j < KBI; ++j) {
-      const int k0 = (it.kb0 + j) * 16 + 4 * g;
-      xo[j] = k0 / a.cy;
-      yo[j] = k0 - xo[j] * a.cy;
-    }
+// The walk tables of a launch, copied to LDS by every workgroup (a few KB): reading them from memory with scalar loads
+// would put a memory round trip in front of every item, and a workgroup that fills the LDS with its samples' rows has
+// a single wavefront per SIMD to hide it behind.
+struct UvtTables {
+  const cgtp_uvt_item* items;
+  const int32_t* ta;
+  const int32_t* tb;
+  const float* tc;
+};
+
+__device__ __forceinline__ UvtTables uvt_stage_tables(const UvtDev& a, unsigned char* at) {
+  int32_t* dst = reinterpret_cast<int32_t*>(at);
+  const int32_t* src = reinterpret_cast<const int32_t*>(a.items);
+  for (int i = threadIdx.x; i < a.n_items * 8; i += blockDim.x) dst[i] = src[i];
+  int32_t* ta = dst + a.n_items * 8;
+  int32_t* tb = ta + a.n_terms;
+  float* tc = reinterpret_cast<float*>(tb + a.n_terms);
+  for (int i = threadIdx.x; i < a.n_terms; i += blockDim.x) {
+    ta[i] = a.ta[i];
+    tb[i] = a.tb[i];
+    tc[i] = a.tc[i];
   }
-  for (int t = it.t0; t < it.t1; ++t) {
-    const int ia = a.ta[t], ib = a.tb[t];
-    const float c = a.tc[t];
+  return UvtTables{reinterpret_cast<const cgtp_uvt_item*>(dst), ta, tb, tc};
+}
+
+__device__ __forceinline__ cgtp_uvt_item uvt_item_at(const UvtTables& tab, int j) {
+  const int32_t* p = reinterpret_cast<const int32_t*>(tab.items + j);
+  cgtp_uvt_item it;
+  it.p = __builtin_amdgcn_readfirstlane(p[0]); it.kb0 = __builtin_amdgcn_readfirstlane(p[1]);
+  it.nkb = __builtin_amdgcn_readfirstlane(p[2]); it.t0 = __builtin_amdgcn_readfirstlane(p[3]);
+  it.t1 = __builtin_amdgcn_readfirstlane(p[4]); it.out_row = __builtin_amdgcn_readfirstlane(p[5]);
+  it.flags = __builtin_amdgcn_readfirstlane(p[6]); it.reserved_ = 0;
+  return it;
+}
+
+// The first kUvtTerms terms of an item's segment in registers, read once per item: per lane the LDS address of the
+// term's row of x at the item's first block of k (so that block j is an immediate offset away: no address arithmetic
+// per read) and the factor coef * y[n, b]; with a channelled y the addresses of both rows and the coefficient.  Slots
+// past the end of the segment point at row 0 with a zero factor, so that the code has no branches around register
+// arrays (a conditional assignment to an array element costs the compiler a copy of the array).
+constexpr int kUvtTerms = 8;
+constexpr int kUvtKbi = 4;   // blocks of 16 k per item
+template <bool YC>
+struct UvtTerms {
+  const float* xr[kUvtTerms];
+  const float* yr[kUvtTerms];   // YC only
+  float s[kUvtTerms];
+  int n;
+};
+
+template <bool YC>
+__device__ __forceinline__ void uvt_terms(const UvtDev& a, const UvtTables& tab, const cgtp_uvt_item& it, const float* xl,
+                                          const float* yl, const float* zeros, int g, UvtTerms<YC>& T) {
+  T.n = min(it.t1 - it.t0, kUvtTerms);
+#pragma unroll
+  for (int k = 0; k < kUvtTerms; ++k) {
+    const bool live = k < T.n;
+    // a slot past the end of the segment reads a block of zeros in LDS (not a row of the input: 0 * inf would leak)
+    const int t = live ? it.t0 + k : it.t0;
+    const int ia = __builtin_amdgcn_readfirstlane(tab.ta[t]);
+    const int ib = __builtin_amdgcn_readfirstlane(tab.tb[t]);
+    const float c = live ? tab.tc[t] : 0.f;
     if constexpr (YC) {
-      const float* xr = xl + ia * a.cx;
-      const float* yr = yl + ib * a.cy;
-#pragma unroll
-      for (int j = 0; j < KBI; ++j)
-        if (j < it.nkb) bf[j] += (c * xr[xo[j]]) * *reinterpret_cast<const floatx4*>(yr + yo[j]);
+      T.xr[k] = live ? xl + ia * a.cx : zeros;
+      T.yr[k] = live ? yl + ib * a.cy : zeros;
+      T.s[k] = c;
     } else {
-      const float s = c * yl[ib];
-      const floatx4* xr = reinterpret_cast<const floatx4*>(xl + ia * a.kx + it.kb0 * 16 + 4 * g);
-#pragma unroll
-      for (int j = 0; j < KBI; ++j)
-        if (j < it.nkb) bf[j] += s * xr[j * 4];
+      T.xr[k] = live ? xl + ia * a.kx + it.kb0 * 16 + 4 * g : zeros;
+      T.s[k] = live ? c * yl[ib] : 0.f;
     }
   }
 }
 
-// WB: blocks of 16 output channels per wavefront; KBI: blocks of 16 k per item (the tables are built for it).
-template <bool YC, int WB, int KBI>
+// This lane's part of block j of 16 k of the mixed operand of an item: inter_s[n, 16 (kb0 + j) + 4 g + i], i < 4.
+// With a channelled y, lut[(kb0 + j) * 4 + g] holds the offsets (u, v) of k = 16 (kb0 + j) + 4 g = u * cy + v.
+template <bool YC>
+__device__ __forceinline__ floatx4 uvt_mix_block(const UvtTerms<YC>& T, int j, const int2* lut) {
+  floatx4 bf = {0.f, 0.f, 0.f, 0.f};
+  int2 o = make_int2(0, 0);
+  if constexpr (YC) o = lut[j * 4];
+#pragma unroll
+  for (int half = 0; half < kUvtTerms; half += 4) {
+    if (half == 0 || T.n > half) {      // wave-uniform; guards accumulation into one local only
+#pragma unroll
+      for (int k = half; k < half + 4; ++k) {
+        if constexpr (YC) {
+          bf += (T.s[k] * T.xr[k][o.x]) * *reinterpret_cast<const floatx4*>(T.yr[k] + o.y);
+        } else {
+          bf += T.s[k] * *reinterpret_cast<const floatx4*>(T.xr[k] + j * 16);
+        }
+      }
+    }
+  }
+  return bf;
+}
+
+// Terms beyond the first kUvtTerms of a segment (large irreps only): straight from the tables.
+template <bool YC>
+__device__ __forceinline__ floatx4 uvt_mix_tail(const UvtDev& a, const UvtTables& tab, const cgtp_uvt_item& it, int j,
+                                                const float* xl, const float* yl, int g, const int2* lut) {
+  floatx4 bf = {0.f, 0.f, 0.f, 0.f};
+  for (int t = it.t0 + kUvtTerms; t < it.t1; ++t) {
+    const int ia = tab.ta[t], ib = tab.tb[t];
+    const float c = tab.tc[t];
+    if constexpr (YC) {
+      const int2 o = lut[j * 4];
+      bf += (c * xl[ia * a.cx + o.x]) * *reinterpret_cast<const floatx4*>(yl + ib * a.cy + o.y);
+    } else {
+      bf += (c * yl[ib]) * *reinterpret_cast<const floatx4*>(xl + ia * a.kx + (it.kb0 + j) * 16 + 4 * g);
+    }
+  }
+  return bf;
+}
+
+// WB: blocks of 16 output channels per wavefront.  Every item covers exactly kUvtKbi blocks of 16 k (the packed
+// weights and the staged rows are zero-padded to whole items), so the body is straight-line code.
+// Software pipeline, by hand, because a workgroup whose rows fill the LDS leaves one wavefront per SIMD: while the
+// matrix instructions of block j of the current item run, the vector ALUs mix block j of the next item; the weight
+// fragments of the next item are requested before the current item starts (past the last item: the last item again).
+// Everything an item needs besides its operands is wave-uniform (scalar registers), and the operand reads use
+// immediate offsets: about 100 vector instructions per item next to its 16 * WB matrix instructions of 32 cycles.
+template <bool YC, int WB>
 __global__ void __launch_bounds__(256) uvt_apply_kernel(const UvtDev a) {
+  constexpr int KBI = kUvtKbi;
   extern __shared__ __align__(16) unsigned char smem[];
   const int sb_count = 1 << a.sb_log2;
   float* xs = reinterpret_cast<float*>(smem);
   float* ys = xs + (size_t)(16 * sb_count) * a.px;
   const int64_t nb0 = (int64_t)blockIdx.x * (16 * sb_count);
   uvt_stage<YC>(a, xs, ys, nb0, 16 * sb_count);
+  unsigned char* after = reinterpret_cast<unsigned char*>(ys + (size_t)(16 * sb_count) * a.py);
+  const UvtTables tab = uvt_stage_tables(a, after);
+  // (u, v) of k = 16 kb + 4 g for a channelled y; (0, 0) in the zero-padded tail of k
+  int2* lut_all = reinterpret_cast<int2*>(after + ((size_t)a.n_items * 32 + (size_t)a.n_terms * 12 + 15) / 16 * 16);
+  if constexpr (YC) {
+    for (int i = threadIdx.x; i < a.kblocks * 4; i += blockDim.x) {
+      const int k0 = i * 4, u = k0 / a.cy;
+      lut_all[i] = k0 < a.cx * a.cy ? make_int2(u, k0 - u * a.cy) : make_int2(0, 0);
+    }
+  }
+  float* zeros = reinterpret_cast<float*>(lut_all + (YC ? a.kblocks * 4 : 0));
+  for (int i = threadIdx.x; i < a.zero_floats; i += blockDim.x) zeros[i] = 0.f;
   __syncthreads();
 
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), r = lane & 15, g = lane >> 4;
@@ -126,36 +227,41 @@ __global__ void __launch_bounds__(256) uvt_apply_kernel(const UvtDev a) {
   const int64_t n = nb0 + sb * 16 + r;
   const float* xl = xs + (size_t)(sb * 16 + r) * a.px;
   const float* yl = ys + (size_t)(sb * 16 + r) * a.py;
-  const float* wl = a.wp + ((int64_t)wb0 * 64 + lane) * 4;
+  const int2* lut_g = lut_all + g;
 
-  floatx4 acc[WB], A0[WB][KBI], A1[WB][KBI];
+  floatx4 acc[WB], A0[WB][KBI], A1[WB][KBI], B0[KBI], B1[KBI];
   auto load_a = [&](const cgtp_uvt_item& it, floatx4 (&A)[WB][KBI]) __attribute__((always_inline)) {
+    // wave-uniform base of the item's fragments; a lane adds 16 bytes times its index
+    const float* base = a.wp + ((int64_t)(it.p * a.kblocks + it.kb0) * a.wbp + wb0) * 256;
 #pragma unroll
-    for (int j = 0; j < KBI; ++j)
-      if (j < it.nkb) {
-        const float* base = wl + ((int64_t)(it.p * a.kblocks + it.kb0 + j) * a.wbp) * 256;
+    for (int j = 0; j < KBI; ++j) {
+      const float* bj = base + (int64_t)j * a.wbp * 256;
 #pragma unroll
-        for (int wb = 0; wb < WB; ++wb) A[wb][j] = *reinterpret_cast<const floatx4*>(base + wb * 256);
-      }
-  };
-  auto process = [&](const cgtp_uvt_item& it, floatx4 (&Ac)[WB][KBI], floatx4 (&An)[WB][KBI], bool has_next,
-                     const cgtp_uvt_item& nx) __attribute__((always_inline)) {
-    if (has_next) load_a(nx, An);
-    if (it.flags & kUvtFirst) {
-#pragma unroll
-      for (int wb = 0; wb < WB; ++wb) acc[wb] = floatx4{0.f, 0.f, 0.f, 0.f};
+      for (int wb = 0; wb < WB; ++wb) A[wb][j] = *reinterpret_cast<const floatx4*>(bj + wb * 256 + lane * 4);
     }
-    floatx4 bf[KBI];
-    uvt_mix<YC, KBI>(a, it, xl, yl, g, bf);
+  };
+  auto mix_item = [&](const cgtp_uvt_item& it, const UvtTerms<YC>& T, int j) __attribute__((always_inline)) {
+    floatx4 b = uvt_mix_block<YC>(T, j, lut_g + it.kb0 * 4);
+    if (it.t1 - it.t0 > kUvtTerms) b += uvt_mix_tail<YC>(a, tab, it, j, xl, yl, g, lut_g + it.kb0 * 4);
+    return b;
+  };
+  auto process = [&](const cgtp_uvt_item& it, floatx4 (&Ac)[WB][KBI], floatx4 (&Bc)[KBI], floatx4 (&An)[WB][KBI],
+                     floatx4 (&Bn)[KBI], const cgtp_uvt_item& nx) __attribute__((always_inline)) {
+    load_a(nx, An);
+    const bool first = it.flags & kUvtFirst;
 #pragma unroll
-    for (int j = 0; j < KBI; ++j)
-      if (j < it.nkb) {
+    for (int wb = 0; wb < WB; ++wb) acc[wb] = first ? floatx4{0.f, 0.f, 0.f, 0.f} : acc[wb];
+    UvtTerms<YC> T;
+    uvt_terms<YC>(a, tab, nx, xl, yl, zeros, g, T);
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+    for (int j = 0; j < KBI; ++j) {
 #pragma unroll
-          for (int wb = 0; wb < WB; ++wb)
-            acc[wb] = __builtin_amdgcn_mfma_f32_16x16x4f32(Ac[wb][j][i], bf[j][i], acc[wb], 0, 0, 0);
-      }
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int wb = 0; wb < WB; ++wb)
+          acc[wb] = __builtin_amdgcn_mfma_f32_16x16x4f32(Ac[wb][j][i], Bc[j][i], acc[wb], 0, 0, 0);
+      Bn[j] = mix_item(nx, T, j);
+    }
     if (it.flags & kUvtLast) {
       // accumulator layout: lane (n = r, g) holds output channels 16 wb + 4 g .. + 3 of sample n
       if (n < a.n_rows) {
@@ -169,14 +275,22 @@ __global__ void __launch_bounds__(256) uvt_apply_kernel(const UvtDev a) {
     }
   };
 
-  cgtp_uvt_item it = a.items[0];
+  cgtp_uvt_item it = uvt_item_at(tab, 0);
   load_a(it, A0);
+  {
+    UvtTerms<YC> T;
+    uvt_terms<YC>(a, tab, it, xl, yl, zeros, g, T);
+#pragma unroll
+    for (int j = 0; j < KBI; ++j) B0[j] = mix_item(it, T, j);
+  }
+#pragma unroll
+  for (int wb = 0; wb < WB; ++wb) acc[wb] = floatx4{0.f, 0.f, 0.f, 0.f};
   for (int j = 0; j < a.n_items; j += 2) {
-    const cgtp_uvt_item it1 = a.items[min(j + 1, a.n_items - 1)];
-    process(it, A0, A1, j + 1 < a.n_items, it1);
+    const cgtp_uvt_item it1 = uvt_item_at(tab, min(j + 1, a.n_items - 1));
+    process(it, A0, B0, A1, B1, it1);
     if (j + 1 >= a.n_items) break;
-    const cgtp_uvt_item it2 = a.items[min(j + 2, a.n_items - 1)];
-    process(it1, A1, A0, j + 2 < a.n_items, it2);
+    const cgtp_uvt_item it2 = uvt_item_at(tab, min(j + 2, a.n_items - 1));
+    process(it1, A1, B1, A0, B0, it2);
     it = it2;
   }
 }
@@ -222,25 +336,25 @@ static int uvt_shape(int64_t n_rows, int dx, int dy, int cx, int cy, int cout, U
   UvtDev& d = plan->dev;
   d.n_rows = n_rows; d.dx = dx; d.dy = dy; d.cx = cx; d.cy = cy; d.cout = cout;
   const int64_t K = yc ? (int64_t)cx * cy : cx;
-  d.kx = yc ? cx : round_up(cx, 16);
+  d.kblocks = round_up((int)((K + 15) / 16), kUvtKbi);   // whole items: the tail is zero weights
+  d.kx = yc ? cx : d.kblocks * 16;
   d.px = dx * d.kx + 4;
   d.py = yc ? dy * cy + 4 : (dy | 1);
-  d.kblocks = (int)((K + 15) / 16);
   const int wblocks = (cout + 15) / 16;
   d.wbp = round_up(wblocks, 4);
   const int64_t per_block = (int64_t)16 * (d.px + d.py) * 4;   // LDS bytes of one 16-sample block
-  if (per_block > kLdsBytes) return CGTP_ERR_LDS;
+  if (per_block > kLdsBytes - kUvtTableRoom) return CGTP_ERR_LDS;
   // sample blocks per workgroup: as many as keep two workgroups per compute unit, else as many as fit; fewer when the
   // batch is too small to fill the chip with such workgroups
   int sb_log2 = 2;
-  while (sb_log2 > 0 && (per_block << sb_log2) > kLdsBytes / 2 - 1024) --sb_log2;
+  while (sb_log2 > 0 && (per_block << sb_log2) > kLdsBytes / 2 - kUvtTableRoom) --sb_log2;
   const int64_t blocks16 = (n_rows + 15) / 16;
   while (sb_log2 > 0 && (blocks16 >> sb_log2) < 512) --sb_log2;
   d.sb_log2 = sb_log2;
   const int wgroups = 4 >> sb_log2;
   const int need = (wblocks + wgroups - 1) / wgroups;
   const int wb = need >= 4 ? 4 : need >= 2 ? 2 : 1;
-  plan->sb_log2 = sb_log2; plan->wb = wb; plan->kbi = wb == 4 ? 4 : 8; plan->yc = yc;
+  plan->sb_log2 = sb_log2; plan->wb = wb; plan->kbi = kUvtKbi; plan->yc = yc;
   plan->lds = per_block << sb_log2;
   plan->grid = dim3((unsigned)((blocks16 + (1 << sb_log2) - 1) >> sb_log2),
                     (unsigned)((wblocks + wgroups * wb - 1) / (wgroups * wb)));
@@ -250,7 +364,7 @@ static int uvt_shape(int64_t n_rows, int dx, int dy, int cx, int cy, int cout, U
 static int uvt_plan(const cgtp_uvt_args* a, UvtPlan* plan) {
   if (!a) return CGTP_ERR_NULL;
   if (a->dtype != CGTP_F32) return CGTP_ERR_DTYPE;
-  if (a->n_items < 0 || a->dout <= 0) return CGTP_ERR_SHAPE;
+  if (a->n_items < 0 || a->n_terms < 0 || a->dout <= 0) return CGTP_ERR_SHAPE;
   const int st = uvt_shape(a->n_rows, a->dx, a->dy, a->cx, a->cy, a->cout, plan);
   if (st != CGTP_OK) return st;
   if (a->kbi != plan->kbi) return CGTP_ERR_SHAPE;   // the item list must be cut for this launch shape: cgtp_uvt_chunk()
@@ -262,7 +376,11 @@ static int uvt_plan(const cgtp_uvt_args* a, UvtPlan* plan) {
   UvtDev& d = plan->dev;
   d.x = (const float*)a->x; d.y = (const float*)a->y; d.wp = (const float*)a->wp; d.out = (float*)a->out;
   d.items = a->items; d.ta = a->term_a; d.tb = a->term_b; d.tc = (const float*)a->term_c;
-  d.n_items = a->n_items; d.dout = a->dout;
+  d.n_items = a->n_items; d.n_terms = a->n_terms; d.dout = a->dout;
+  d.zero_floats = a->cy > 0 ? round_up((a->cx > a->cy + 4 ? a->cx : a->cy + 4) + 4, 4) : kUvtKbi * 16 + 16;
+  plan->lds += ((int64_t)a->n_items * 32 + (int64_t)a->n_terms * 12 + 15) / 16 * 16 +
+               (a->cy > 0 ? (int64_t)d.kblocks * 32 : 0) + (int64_t)d.zero_floats * 4 + 16;
+  if (plan->lds > kLdsBytes) return CGTP_ERR_LDS;
   return CGTP_OK;
 }
 
@@ -274,7 +392,7 @@ extern "C" {
 
 int64_t cgtp_uvt_packed_elems(int32_t n_paths, int64_t K, int32_t cout) {
   if (n_paths < 0 || K <= 0 || cout <= 0) return 0;
-  return (int64_t)n_paths * ((K + 15) / 16) * round_up((cout + 15) / 16, 4) * 256;
+  return (int64_t)n_paths * round_up((int)((K + 15) / 16), kUvtKbi) * round_up((cout + 15) / 16, 4) * 256;
 }
 
 int cgtp_uvt_pack_weights(const void* w, void* packed, int32_t n_paths, int64_t K, int32_t cout, int64_t stride_p,
@@ -286,8 +404,8 @@ int cgtp_uvt_pack_weights(const void* w, void* packed, int32_t n_paths, int64_t 
   const int64_t n_vec = cgtp_uvt_packed_elems(n_paths, K, cout) / 4;
   if (n_vec == 0) return CGTP_OK;
   hipLaunchKernelGGL(uvt_pack_kernel, dim3((unsigned)((n_vec + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                     (const float*)w, (float*)packed, n_vec, (int)K, (int)cout, (int)((K + 15) / 16),
-                     round_up((cout + 15) / 16, 4), stride_p, stride_k, stride_c);
+                     (const float*)w, (float*)packed, n_vec, (int)K, (int)cout,
+                     round_up((int)((K + 15) / 16), kUvtKbi), round_up((cout + 15) / 16, 4), stride_p, stride_k, stride_c);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 
@@ -309,9 +427,9 @@ int cgtp_uvt_apply(const cgtp_uvt_args* a, void* stream) {
   if (a->n_rows == 0 || a->n_items == 0) return CGTP_OK;
   void (*fn)(const UvtDev) = nullptr;
   if (plan.yc) {
-    fn = plan.wb == 4 ? uvt_apply_kernel<true, 4, 4> : plan.wb == 2 ? uvt_apply_kernel<true, 2, 8> : uvt_apply_kernel<true, 1, 8>;
+    fn = plan.wb == 4 ? uvt_apply_kernel<true, 4> : plan.wb == 2 ? uvt_apply_kernel<true, 2> : uvt_apply_kernel<true, 1>;
   } else {
-    fn = plan.wb == 4 ? uvt_apply_kernel<false, 4, 4> : plan.wb == 2 ? uvt_apply_kernel<false, 2, 8> : uvt_apply_kernel<false, 1, 8>;
+    fn = plan.wb == 4 ? uvt_apply_kernel<false, 4> : plan.wb == 2 ? uvt_apply_kernel<false, 2> : uvt_apply_kernel<false, 1>;
   }
   if (plan.lds > 48 * 1024 &&
       hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds) != hipSuccess)

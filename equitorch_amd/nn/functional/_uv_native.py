@@ -40,10 +40,10 @@ class _Walk:
                 while t1 < n_terms and out_idx[t1] == row and p_idx[t1] == p_idx[t]:
                     t1 += 1
                 for kb0 in range(0, kblocks, kbi):
-                    items.append([int(p_idx[t]), kb0, min(kbi, kblocks - kb0), t, t1, row, 0, 0])
+                    items.append([int(p_idx[t]), kb0, kbi, t, t1, row, 0, 0])
                 t = t1
             if len(items) == first:                       # a row without terms is written as zeros
-                items.append([0, 0, 0, 0, 0, row, 0, 0])
+                items.append([0, 0, kbi, 0, 0, row, 0, 0])
             items[first][6] |= FIRST
             items[-1][6] |= LAST
         self.n_items = len(items)
@@ -92,7 +92,8 @@ def apply(x: Tensor, y: Tensor, wp: Tensor, tp_info, role: str, dout: int, cout:
     kbi = chunk_of(n, dx, dy, cx, cy, cout)
     if kbi <= 0:
         raise _lib.CgtpError(f"cgtp_uvt_apply does not take these extents (status {-kbi})")
-    walk = _walk(tp_info, role, (k + 15) // 16, kbi, x.device)
+    kblocks = ((k + 15) // 16 + kbi - 1) // kbi * kbi        # whole items; the tail of k is zero weights
+    walk = _walk(tp_info, role, kblocks, kbi, x.device)
     out = torch.empty((n, dout, cout), dtype=x.dtype, device=x.device)
     if n == 0:
         return out
@@ -100,7 +101,7 @@ def apply(x: Tensor, y: Tensor, wp: Tensor, tp_info, role: str, dout: int, cout:
     a.x, a.y, a.wp, a.out = x.data_ptr(), y.data_ptr(), wp.data_ptr(), out.data_ptr()
     a.items, a.term_a, a.term_b, a.term_c = (walk.items.data_ptr(), walk.term_a.data_ptr(), walk.term_b.data_ptr(),
                                              walk.term_c.data_ptr())
-    a.n_rows, a.n_items = n, walk.n_items
+    a.n_rows, a.n_items, a.n_terms = n, walk.n_items, walk.term_a.shape[0]
     a.dx, a.dy, a.dout, a.cx, a.cy, a.cout = dx, dy, dout, cx, cy, cout
     a.kbi, a.dtype = kbi, _lib.F32
     _lib.check(_lib.lib.cgtp_uvt_apply(C.byref(a), _lib.stream_ptr(x.device)), "cgtp_uvt_apply")

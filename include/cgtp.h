@@ -302,10 +302,10 @@ int cgtp_uv_grad_w(int cfg, const void* x, const void* y, const void* g, void* g
  * the rows' roles exchanged and the weight packed transposed, for the grad-input products of their backward passes
  * (tensor_product_1vu / tensor_product_uvw with permuted weights, linears.py:290-293, tensor_products.py:126-150).
  * Shared weights only.  The caller supplies the walk as a flat list of items ordered by output row: an item is one
- * segment restricted to `nkb` blocks of 16 consecutive k starting at block kb0, with its terms t0..t1 in (term_a =
- * row of x, term_b = row of y, term_c = coefficient); flags: 1 = first item of its output row, 2 = last.  Every output
- * row needs at least one item (nkb = 0 for a row without terms: it is written as zeros).  nkb <= the chunk length
- * cgtp_uvt_chunk() reports for the extents, which must also be passed as `kbi`.
+ * segment restricted to the `nkb` = cgtp_uvt_chunk() blocks of 16 consecutive k starting at block kb0 (K is padded
+ * with zero weights to whole items), with its terms t0..t1 in (term_a = row of x, term_b = row of y, term_c =
+ * coefficient); flags: 1 = first item of its output row, 2 = last.  Every output row needs at least one item (t0 = t1
+ * for a row without terms: it is written as zeros).  The chunk length must also be passed as `kbi`.
  * x (n_rows, dx, cx), y (n_rows, dy) or (n_rows, dy, cy), out (n_rows, dout, cout), all fp32 and contiguous; cx, cy,
  * cout multiples of 4, cx * cy a multiple of 16 when cy > 0; 16-byte aligned pointers; the rows of 16 samples must
  * fit the LDS (CGTP_ERR_LDS otherwise).  wp = cgtp_uvt_pack_weights(W): W (n_paths, K, cout) read through element
@@ -331,13 +331,14 @@ typedef struct cgtp_uvt_args {
   int32_t cx, cy, cout;
   int32_t kbi;                  /* chunk length the items were cut for: cgtp_uvt_chunk() */
   int32_t dtype;                /* CGTP_F32 */
-  int32_t reserved_;
+  int32_t n_terms;              /* entries of term_a / term_b / term_c (the tables are copied to LDS: 32 B per item +
+                                   12 B per term must fit next to the samples' rows, CGTP_ERR_LDS otherwise) */
 } cgtp_uvt_args;
 
 int64_t cgtp_uvt_packed_elems(int32_t n_paths, int64_t K, int32_t cout);
 int cgtp_uvt_pack_weights(const void* w, void* packed, int32_t n_paths, int64_t K, int32_t cout, int64_t stride_p,
                           int64_t stride_k, int64_t stride_c, int32_t dtype, void* stream);
-/* Blocks of 16 k per item for these extents (4 or 8), or -status when the kernels do not take them.  Host only. */
+/* Blocks of 16 k per item for these extents, or -status when the kernels do not take them.  Host only. */
 int cgtp_uvt_chunk(int64_t n_rows, int32_t dx, int32_t dy, int32_t cx, int32_t cy, int32_t cout);
 int cgtp_uvt_validate(const cgtp_uvt_args* args);
 int cgtp_uvt_apply(const cgtp_uvt_args* args, void* stream);
