@@ -317,6 +317,142 @@ __global__ void uvt_pack_kernel(const float* __restrict__ w, float* __restrict__
   *reinterpret_cast<floatx4*>(packed + i * 4) = v;
 }
 
+
+// ---- gradient of a shared weight ---------------------------------------------------------------------------------
+//   gW[p, k, w] = sum_n sum_{segments s = (p, M)} inter_s[n, k] * g[n, M, w]
+// The contraction runs over the samples: four per matrix instruction (A: lane (k = lane % 16, sample = lane / 16)
+// holds inter_s[n, k], formed from x and y as the lane needs it; B: lane (w = lane % 16, sample) holds g[n, M, w]).
+// A workgroup owns one weight path and one chunk of samples; its four wavefronts split a 128 (k) x 128 (w) block of
+// the path's gradient into 2 x 2 parts of 4 x 4 accumulator tiles.  Operands come straight from memory (no LDS), so
+// three wavefronts per SIMD hide the latency.  The chunks' partial results go to a workspace and are summed in chunk
+// order by uvt_gw_reduce_kernel (no atomics: the result does not depend on the launch).
+struct UvtGwDev {
+  const float* x;
+  const float* y;
+  const float* g;
+  float* part;                 // (n_chunks, n_paths, K, cout)
+  const cgtp_uvt_item* items;  // segments sorted by path: p, out_row = M, t0, t1
+  const int32_t* path_ptr;     // [n_paths + 1] into items
+  const int32_t* ta;
+  const int32_t* tb;
+  const float* tc;
+  int64_t n_rows;
+  int n_paths, dx, dy, dg, cx, cy, cout, K, chunk;
+};
+
+constexpr int kGwT = 4;   // accumulator tiles per wavefront and axis
+
+// Tile rows and columns are interleaved with the channels — row r of k-tile i is channel 4 r + i of the wavefront's
+// 64, column r of w-tile j is output channel 4 r + j — so that a lane's operands of the four tiles are four
+// consecutive channels: one 16-byte load per term instead of four 4-byte loads (the address units, shared by the
+// four SIMDs of a compute unit, are what this kernel would otherwise be bound by).
+template <bool YC>
+__global__ void __launch_bounds__(256, 4) uvt_grad_w_kernel(const UvtGwDev a) {
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), r = lane & 15, g4 = lane >> 4;
+  const int p = blockIdx.y;
+  const int kgroups = (a.K + 127) / 128;
+  const int kgrp = blockIdx.z % kgroups, wgrp = blockIdx.z / kgroups;
+  const int k0 = kgrp * 128 + (wave & 1) * 64 + 4 * r;    // this lane's four channels k0 .. k0 + 3 (tiles 0 .. 3)
+  const int w0 = wgrp * 128 + (wave >> 1) * 64 + 4 * r;   // and four output channels
+  const int64_t n_begin = (int64_t)blockIdx.x * a.chunk;
+  const int64_t n_end = n_begin + a.chunk < a.n_rows ? n_begin + a.chunk : a.n_rows;
+
+  floatx4 acc[kGwT][kGwT];
+#pragma unroll
+  for (int i = 0; i < kGwT; ++i)
+#pragma unroll
+    for (int j = 0; j < kGwT; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // K and cout are multiples of 4 (checked by the launcher), so a lane's four channels are all inside or all outside
+  const bool kok = k0 < a.K, wok = w0 < a.cout;
+  const int kc = kok ? k0 : 0, wc = wok ? w0 : 0;
+  int xo = kc, yo = 0;
+  if constexpr (YC) {
+    xo = kc / a.cy;
+    yo = kc - xo * a.cy;
+  }
+  const int s_begin = a.path_ptr[p], s_end = a.path_ptr[p + 1];
+  for (int s = s_begin; s < s_end; ++s) {
+    // the segment's terms (at most kUvtTerms per item: the caller splits longer segments) in scalar registers; slots
+    // past the end repeat the first term's rows — their loads are issued with the others and never used
+    const cgtp_uvt_item it = a.items[s];
+    const int n_t = it.t1 - it.t0;
+    int xrow[kUvtTerms], yrow[kUvtTerms];
+    float c[kUvtTerms];
+#pragma unroll
+    for (int k = 0; k < kUvtTerms; ++k) {
+      const int t = k < n_t ? it.t0 + k : it.t0;
+      xrow[k] = a.ta[t] * a.cx;
+      yrow[k] = a.tb[t] * (YC ? a.cy : 1);
+      c[k] = a.tc[t];
+    }
+    const int grow = it.out_row * a.cout;
+    for (int64_t n0 = n_begin; n0 < n_end; n0 += 4) {
+      const int64_t n = n0 + g4;
+      const bool live = n < n_end;
+      const int64_t nc = live ? n : n_end - 1;
+      const float* xn = a.x + nc * a.dx * a.cx + xo;
+      const float* yn = a.y + nc * a.dy * (YC ? a.cy : 1) + yo;
+      // all loads of the step first ...
+      const floatx4 bv4 = *reinterpret_cast<const floatx4*>(a.g + nc * a.dg * a.cout + grow + wc);
+      floatx4 v4[kUvtTerms];     // y without channels: four channels of x; with: four channels of y
+      float v1[kUvtTerms];       // y without channels: y[n, b]; with: x[n, a, u]
+#pragma unroll
+      for (int k = 0; k < kUvtTerms; ++k) {
+        if constexpr (YC) {
+          v1[k] = xn[xrow[k]];
+          v4[k] = *reinterpret_cast<const floatx4*>(yn + yrow[k]);
+        } else {
+          v4[k] = *reinterpret_cast<const floatx4*>(xn + xrow[k]);
+          v1[k] = yn[yrow[k]];
+        }
+      }
+      // ... then the mixing of the terms that exist (wave-uniform branches around arithmetic only)
+      floatx4 av = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int k = 0; k < kUvtTerms; ++k)
+        if (k < n_t) av += (c[k] * v1[k]) * v4[k];
+      const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+      av = (live && kok) ? av : zero;
+      const floatx4 bv = (live && wok) ? bv4 : zero;
+#pragma unroll
+      for (int i = 0; i < kGwT; ++i)
+#pragma unroll
+        for (int j = 0; j < kGwT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+    }
+  }
+  // accumulator layout: lane (column r, g4) holds rows 4 g4 .. + 3 of a tile; tile (i, j) row q is channel
+  // 4 q + i of the wavefront's 64, column r is output channel 4 r + j
+  float* out = a.part + ((int64_t)blockIdx.x * a.n_paths + p) * a.K * a.cout;
+  const int kbase = kgrp * 128 + (wave & 1) * 64;
+#pragma unroll
+  for (int i = 0; i < kGwT; ++i)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int k = kbase + 4 * (4 * g4 + e) + i;
+      if (k < a.K && wok) {
+        floatx4 v;
+#pragma unroll
+        for (int j = 0; j < kGwT; ++j) v[j] = acc[i][j][e];
+        *reinterpret_cast<floatx4*>(out + (int64_t)k * a.cout + w0) = v;
+      }
+    }
+}
+
+__global__ void uvt_gw_reduce_kernel(const float* __restrict__ part, float* __restrict__ gw, int64_t n_chunks, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float s = 0.f;
+  for (int64_t c = 0; c < n_chunks; ++c) s += part[c * n + i];
+  gw[i] = s;
+}
+
+static int64_t uvt_gw_chunk(int64_t n_rows) {
+  // samples per workgroup: enough workgroups to fill the chip at small batches, at most 128 partial results
+  int64_t chunk = 256;
+  while ((n_rows + chunk - 1) / chunk > 128) chunk *= 2;
+  return chunk;
+}
+
 struct UvtPlan {
   int sb_log2, wb, kbi, yc;
   int64_t lds;
@@ -435,6 +571,54 @@ int cgtp_uvt_apply(const cgtp_uvt_args* a, void* stream) {
       hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds) != hipSuccess)
     return CGTP_ERR_LDS;
   hipLaunchKernelGGL(fn, plan.grid, dim3(256), (size_t)plan.lds, (hipStream_t)stream, plan.dev);
+  return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
+}
+
+int64_t cgtp_uvt_grad_w_workspace_bytes(int64_t n_rows, int32_t n_paths, int64_t K, int32_t cout) {
+  if (n_rows <= 0 || n_paths <= 0 || K <= 0 || cout <= 0) return 0;
+  const int64_t chunk = uvt_gw_chunk(n_rows);
+  return ((n_rows + chunk - 1) / chunk) * n_paths * K * cout * (int64_t)sizeof(float);
+}
+
+int cgtp_uvt_grad_w(const cgtp_uvt_gw_args* a, void* stream) {
+  if (!a) return CGTP_ERR_NULL;
+  if (a->dtype != CGTP_F32) return CGTP_ERR_DTYPE;
+  if (a->n_rows < 0 || a->n_paths <= 0 || a->n_items < 0 || a->dx <= 0 || a->dy <= 0 || a->dg <= 0 || a->cx <= 0 ||
+      a->cy < 0 || a->cout <= 0)
+    return CGTP_ERR_SHAPE;
+  if (!a->x || !a->y || !a->g || !a->gw || !a->path_ptr || (a->n_items && (!a->items || !a->term_a || !a->term_b || !a->term_c)))
+    return CGTP_ERR_NULL;
+  const int64_t K = a->cy > 0 ? (int64_t)a->cx * a->cy : a->cx;
+  if (K > (1 << 24)) return CGTP_ERR_SHAPE;
+  if (K % 4 || a->cout % 4 || a->cy % 4) return CGTP_ERR_SHAPE;   // 16-byte operand loads
+  if ((reinterpret_cast<uintptr_t>(a->x) | reinterpret_cast<uintptr_t>(a->g) | reinterpret_cast<uintptr_t>(a->workspace) |
+       (a->cy > 0 ? reinterpret_cast<uintptr_t>(a->y) : 0)) & 15u)
+    return CGTP_ERR_ALIGN;
+  const int64_t n_out = (int64_t)a->n_paths * K * a->cout;
+  hipStream_t st = (hipStream_t)stream;
+  if (a->n_rows == 0) {   // no samples: the gradient is zero (written by the summation kernel over zero chunks)
+    hipLaunchKernelGGL(uvt_gw_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, st,
+                       (const float*)nullptr, (float*)a->gw, (int64_t)0, n_out);
+    return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
+  }
+  if (!a->workspace) return CGTP_ERR_WORKSPACE;
+  UvtGwDev d;
+  d.x = (const float*)a->x; d.y = (const float*)a->y; d.g = (const float*)a->g; d.part = (float*)a->workspace;
+  d.items = a->items; d.path_ptr = a->path_ptr; d.ta = a->term_a; d.tb = a->term_b; d.tc = (const float*)a->term_c;
+  d.n_rows = a->n_rows; d.n_paths = a->n_paths; d.dx = a->dx; d.dy = a->dy; d.dg = a->dg; d.cx = a->cx; d.cy = a->cy;
+  d.cout = a->cout; d.K = (int)K;
+  d.chunk = (int)uvt_gw_chunk(a->n_rows);
+  const int64_t n_chunks = (a->n_rows + d.chunk - 1) / d.chunk;
+  const int64_t zblocks = ((K + 127) / 128) * ((a->cout + 127) / 128);
+  if (zblocks > 65535 || a->n_paths > 65535) return CGTP_ERR_SHAPE;
+  dim3 grid((unsigned)n_chunks, (unsigned)a->n_paths, (unsigned)zblocks);
+  if (a->cy > 0)
+    hipLaunchKernelGGL(uvt_grad_w_kernel<true>, grid, dim3(256), 0, st, d);
+  else
+    hipLaunchKernelGGL(uvt_grad_w_kernel<false>, grid, dim3(256), 0, st, d);
+  if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
+  hipLaunchKernelGGL(uvt_gw_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, st,
+                     (const float*)a->workspace, (float*)a->gw, n_chunks, n_out);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 

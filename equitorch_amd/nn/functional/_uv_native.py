@@ -22,6 +22,7 @@ from ... import _lib
 from ...ops import kernels
 
 FIRST, LAST = 1, 2
+MAX_TERMS = 8      # terms of a segment the weight-gradient kernel holds in registers (kUvtTerms)
 
 
 class _Walk:
@@ -67,6 +68,56 @@ def _walk(tp_info, role: str, kblocks: int, kbi: int, device) -> _Walk:
             return _Walk(c.M2, c.M, c.M1, c.p, c.coef, c.D2, kblocks, kbi, device)
         raise ValueError(role)
     return kernels.cached(tp_info.info_Mij_fwd.scale, ("uvt_walk", role, kblocks, kbi, str(device)), build)
+
+
+class _PathWalk:
+    """Segments (weight path, output row) of a table sorted by path, with their terms: the walk of the weight-gradient
+    kernel, which owns one path per workgroup."""
+
+    def __init__(self, coo, device):
+        order = np.lexsort([coo.M2, coo.M1, coo.M, coo.p])
+        p_idx, m_idx, a_idx, b_idx = (np.asarray(v)[order] for v in (coo.p, coo.M, coo.M1, coo.M2))
+        coef = np.asarray(coo.coef, dtype=np.float64)[order]
+        items, path_ptr = [], [0]
+        t, n_terms = 0, p_idx.shape[0]
+        for p in range(coo.P):
+            while t < n_terms and p_idx[t] == p:
+                t1 = t
+                while t1 < n_terms and p_idx[t1] == p and m_idx[t1] == m_idx[t]:
+                    t1 += 1
+                for tb in range(t, t1, MAX_TERMS):       # the kernel keeps at most MAX_TERMS terms of an item
+                    items.append([p, 0, 0, tb, min(tb + MAX_TERMS, t1), int(m_idx[t]), 0, 0])
+                t = t1
+            path_ptr.append(len(items))
+        self.n_items, self.n_terms, self.n_paths = len(items), n_terms, coo.P
+        self.items = torch.tensor(items, dtype=torch.int32).reshape(-1, 8).to(device)
+        self.path_ptr = torch.tensor(path_ptr, dtype=torch.int32).to(device)
+        self.term_a = torch.from_numpy(a_idx.astype(np.int32)).to(device)
+        self.term_b = torch.from_numpy(b_idx.astype(np.int32)).to(device)
+        self.term_c = torch.from_numpy(coef.astype(np.float32)).to(device)
+
+
+def grad_w(x: Tensor, y: Tensor, g: Tensor, tp_info) -> Tensor:
+    """``gw[p, k, w] = sum_n sum_{(p, M)} inter[n, (p, M), k] g[n, M, w]`` (``cgtp_uvt_grad_w``): ``(P, K, C_out)`` with
+    ``K = C_x`` or ``C_x * C_y``; the caller reshapes."""
+    walk = kernels.cached(tp_info.info_Mij_fwd.scale, ("uvt_path_walk", str(x.device)),
+                          lambda: _PathWalk(kernels.coo_of(tp_info), x.device))
+    n, dx, cx = x.shape
+    dy = y.shape[1]
+    cy = y.shape[2] if y.ndim == 3 else 0
+    k = cx * cy if cy else cx
+    cout = g.shape[-1]
+    gw = torch.empty((walk.n_paths, k, cout), dtype=torch.float32, device=x.device)
+    ws = torch.empty(max(int(_lib.lib.cgtp_uvt_grad_w_workspace_bytes(n, walk.n_paths, k, cout)), 16), dtype=torch.uint8,
+                     device=x.device)
+    a = _lib.UvtGwArgs()
+    a.x, a.y, a.g, a.gw, a.workspace = x.data_ptr(), y.data_ptr(), g.data_ptr(), gw.data_ptr(), ws.data_ptr()
+    a.items, a.path_ptr = walk.items.data_ptr(), walk.path_ptr.data_ptr()
+    a.term_a, a.term_b, a.term_c = walk.term_a.data_ptr(), walk.term_b.data_ptr(), walk.term_c.data_ptr()
+    a.n_rows, a.n_items, a.n_terms, a.n_paths = n, walk.n_items, walk.n_terms, walk.n_paths
+    a.dx, a.dy, a.dg, a.cx, a.cy, a.cout, a.dtype = dx, dy, g.shape[1], cx, cy, cout, _lib.F32
+    _lib.check(_lib.lib.cgtp_uvt_grad_w(C.byref(a), _lib.stream_ptr(x.device)), "cgtp_uvt_grad_w")
+    return gw
 
 
 def chunk_of(n_rows: int, dx: int, dy: int, cx: int, cy: int, cout: int) -> int:
@@ -145,14 +196,13 @@ class _U1vNative(Function):
         g = g.contiguous()
         if need[0]:
             gx = apply(g, y, pack(w, p, wc, u, u * wc, 1, wc), tp_info, "in1", c.D1, u)
-        if need[1] or need[2]:
+        if need[2]:
+            gw = grad_w(x, y, g, tp_info)
+        if need[1]:
             with torch.enable_grad():
-                yr, wr = y.detach().requires_grad_(need[1]), w.detach().requires_grad_(need[2])
-                out = _uv_gemm.u1v(x.detach(), yr, wr, tp_info)
-                wanted = [t for t, n in zip((yr, wr), need[1:]) if n]
-                got = iter(torch.autograd.grad(out, wanted, g))
-            gy = next(got) if need[1] else None
-            gw = next(got) if need[2] else None
+                yr = y.detach().requires_grad_(True)
+                out = _uv_gemm.u1v(x.detach(), yr, w.detach(), tp_info)
+                (gy,) = torch.autograd.grad(out, (yr,), g)
         return gx, gy, gw, None
 
 
@@ -209,10 +259,7 @@ class _UvwNative(Function):
             wt = w.permute(0, 3, 1, 2).contiguous()
             gy = apply(g, x, pack(wt, p, wc * u, v, wc * u * v, v, 1), tp_info, "in2_uvw", c.D2, v)
         if need[2]:
-            with torch.enable_grad():
-                wr = w.detach().requires_grad_(True)
-                out = _uvw_gemm.uvw(x.detach(), y.detach(), wr, tp_info)
-                (gw,) = torch.autograd.grad(out, (wr,), g)
+            gw = grad_w(x, y, g, tp_info).view(p, u, v, wc)
         return gx, gy, gw, None
 
 

@@ -343,6 +343,39 @@ int cgtp_uvt_chunk(int64_t n_rows, int32_t dx, int32_t dy, int32_t cx, int32_t c
 int cgtp_uvt_validate(const cgtp_uvt_args* args);
 int cgtp_uvt_apply(const cgtp_uvt_args* args, void* stream);
 
+/* Gradient of the shared weight of the products above (the reference accumulates batch outer products with atomics:
+ * indexed_outer_scale_gather with out_accumulated, equitorch/nn/functional/linears.py:301-307,
+ * tensor_products.py:152-158):
+ *   gw[p, k, w] = sum_n sum_{segments s = (p, M)} inter_s[n, k] * g[n, M, w]
+ * with inter_s as in cgtp_uvt_apply (never written to memory).  items: the segments sorted by weight path (fields p,
+ * out_row = M, t0, t1 are read; at most 8 terms per item — a longer segment is given as several items),
+ * path_ptr[n_paths + 1] their ranges per path; x (n_rows, dx, cx), y (n_rows, dy) or
+ * (n_rows, dy, cy), g = grad_out (n_rows, dg, cout), gw (n_paths, K, cout) contiguous as the module stores the
+ * weight.  The samples are contracted on the matrix cores in chunks; the chunks' partial results live in `workspace`
+ * (cgtp_uvt_grad_w_workspace_bytes) and are added in chunk order.  Channel counts multiples of 4, 16-byte aligned
+ * pointers. */
+typedef struct cgtp_uvt_gw_args {
+  const void* x;
+  const void* y;
+  const void* g;
+  void* gw;
+  void* workspace;
+  const cgtp_uvt_item* items;   /* device */
+  const int32_t* path_ptr;      /* device */
+  const int32_t* term_a;        /* device */
+  const int32_t* term_b;        /* device */
+  const void* term_c;           /* device, dtype */
+  int64_t n_rows;
+  int32_t n_items, n_terms, n_paths;
+  int32_t dx, dy, dg;
+  int32_t cx, cy, cout;
+  int32_t dtype;                /* CGTP_F32 */
+  int32_t reserved_;
+} cgtp_uvt_gw_args;
+
+int64_t cgtp_uvt_grad_w_workspace_bytes(int64_t n_rows, int32_t n_paths, int64_t K, int32_t cout);
+int cgtp_uvt_grad_w(const cgtp_uvt_gw_args* args, void* stream);
+
 /* ---- real spherical harmonics of vectors -----------------------------------------------------------------
  * Stands in for spherical_harmonics (equitorch/ops/spherical_harmonics.py:68-640: explicit polynomials per
  * degree, TorchScript, differentiated by autograd) together with its callers' pre- and post-processing:
