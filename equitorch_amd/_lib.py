@@ -84,6 +84,14 @@ class UvtGwArgs(C.Structure):
                 ("reserved_", C.c_int32)]
 
 
+class UvtGyArgs(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("g", C.c_void_p), ("wp", C.c_void_p), ("gy", C.c_void_p),
+                ("items", C.c_void_p), ("term_m", C.c_void_p), ("term_b", C.c_void_p), ("term_c", C.c_void_p),
+                ("n_rows", C.c_int64), ("n_items", C.c_int32), ("n_terms", C.c_int32),
+                ("dx", C.c_int32), ("dy", C.c_int32), ("dg", C.c_int32),
+                ("cx", C.c_int32), ("cout", C.c_int32), ("dtype", C.c_int32)]
+
+
 def _load():
     if not os.path.exists(_LIB_PATH):
         raise ImportError(
@@ -140,6 +148,7 @@ def _load():
     lib.cgtp_uvt_grad_w_workspace_bytes.restype = C.c_int64
     lib.cgtp_uvt_grad_w_workspace_bytes.argtypes = [C.c_int64, C.c_int32, C.c_int64, C.c_int32]
     lib.cgtp_uvt_grad_w.argtypes = [C.POINTER(UvtGwArgs), C.c_void_p]
+    lib.cgtp_uvt_grad_y.argtypes = [C.POINTER(UvtGyArgs), C.c_void_p]
     lib.cgtp_sh_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_double, C.c_int,
                                     C.c_void_p]
     lib.cgtp_sh_backward.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_double,

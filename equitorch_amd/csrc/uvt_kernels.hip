@@ -86,7 +86,8 @@ struct UvtTables {
   const float* tc;
 };
 
-__device__ __forceinline__ UvtTables uvt_stage_tables(const UvtDev& a, unsigned char* at) {
+template <class Dev>
+__device__ __forceinline__ UvtTables uvt_stage_tables(const Dev& a, unsigned char* at) {
   int32_t* dst = reinterpret_cast<int32_t*>(at);
   const int32_t* src = reinterpret_cast<const int32_t*>(a.items);
   for (int i = threadIdx.x; i < a.n_items * 8; i += blockDim.x) dst[i] = src[i];
@@ -321,11 +322,15 @@ __global__ void uvt_pack_kernel(const float* __restrict__ w, float* __restrict__
 // ---- gradient of a shared weight ---------------------------------------------------------------------------------
 //   gW[p, k, w] = sum_n sum_{segments s = (p, M)} inter_s[n, k] * g[n, M, w]
 // The contraction runs over the samples: four per matrix instruction (A: lane (k = lane % 16, sample = lane / 16)
-// holds inter_s[n, k], formed from x and y as the lane needs it; B: lane (w = lane % 16, sample) holds g[n, M, w]).
-// A workgroup owns one weight path and one chunk of samples; its four wavefronts split a 128 (k) x 128 (w) block of
-// the path's gradient into 2 x 2 parts of 4 x 4 accumulator tiles.  Operands come straight from memory (no LDS), so
-// three wavefronts per SIMD hide the latency.  The chunks' partial results go to a workspace and are summed in chunk
-// order by uvt_gw_reduce_kernel (no atomics: the result does not depend on the launch).
+// holds inter_s[n, k]; B: lane (w = lane % 16, sample) holds g[n, M, w]).  A workgroup owns one weight path, one chunk
+// of samples and a 128 (k) x 128 (w) block of the path's gradient, which its four wavefronts split 2 x 2 into parts of
+// 4 x 4 accumulator tiles.  Two wavefronts need the same inter values and two the same g values, and the vector
+// memory path of a compute unit delivers about 64 bytes a cycle — loading every operand in the wavefront that uses it
+// took twice the time of the matrix instructions.  So the wavefronts load disjoint quarters of a step of eight
+// samples (sample pair = wavefront, four consecutive channels = lane), mix the terms, and exchange the results
+// through a double-buffered LDS stage; the loads of step i + 2 are in flight while step i is multiplied.
+// The chunks' partial results go to a workspace and are summed in chunk order by uvt_gw_reduce_kernel (no atomics:
+// the result does not depend on the launch).
 struct UvtGwDev {
   const float* x;
   const float* y;
@@ -340,102 +345,144 @@ struct UvtGwDev {
   int n_paths, dx, dy, dg, cx, cy, cout, K, chunk;
 };
 
-constexpr int kGwT = 4;   // accumulator tiles per wavefront and axis
+constexpr int kGwT = 4;        // accumulator tiles per wavefront and axis
+constexpr int kGwStep = 8;     // samples per step (two matrix instructions deep)
+constexpr int kGwPitch = 132;  // floats per sample row of the LDS stage: 128 channels, rows 4 banks apart
 
 // Tile rows and columns are interleaved with the channels — row r of k-tile i is channel 4 r + i of the wavefront's
 // 64, column r of w-tile j is output channel 4 r + j — so that a lane's operands of the four tiles are four
-// consecutive channels: one 16-byte load per term instead of four 4-byte loads (the address units, shared by the
-// four SIMDs of a compute unit, are what this kernel would otherwise be bound by).
+// consecutive channels: one 16-byte LDS read per operand and step.
 template <bool YC>
-__global__ void __launch_bounds__(256, 4) uvt_grad_w_kernel(const UvtGwDev a) {
+__global__ void __launch_bounds__(256, 3) uvt_grad_w_kernel(const UvtGwDev a) {
+  __shared__ __attribute__((aligned(16))) float lds_a[2][kGwStep][kGwPitch];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][kGwStep][kGwPitch];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), r = lane & 15, g4 = lane >> 4;
   const int p = blockIdx.y;
   const int kgroups = (a.K + 127) / 128;
   const int kgrp = blockIdx.z % kgroups, wgrp = blockIdx.z / kgroups;
-  const int k0 = kgrp * 128 + (wave & 1) * 64 + 4 * r;    // this lane's four channels k0 .. k0 + 3 (tiles 0 .. 3)
-  const int w0 = wgrp * 128 + (wave >> 1) * 64 + 4 * r;   // and four output channels
   const int64_t n_begin = (int64_t)blockIdx.x * a.chunk;
   const int64_t n_end = n_begin + a.chunk < a.n_rows ? n_begin + a.chunk : a.n_rows;
+
+  // loading role: sample ls of the step, channels lq .. lq + 3 of the block's 128 (both operands)
+  const int ls = 2 * wave + (lane >> 5), lq = 4 * (lane & 31);
+  // K and cout are multiples of 4 (checked by the launcher), so a lane's four channels are all inside or all outside
+  const bool kok = kgrp * 128 + lq < a.K, wok = wgrp * 128 + lq < a.cout;
+  const int kc = kok ? kgrp * 128 + lq : 0, wc = wok ? wgrp * 128 + lq : 0;
+  int xo = kc, yo = 0;
+  if constexpr (YC) {
+    xo = kc / a.cy;
+    yo = kc - xo * a.cy;
+  }
+  // multiplying role: channels kh * 64 .. + 63 by output channels wh * 64 .. + 63
+  const int kh = wave & 1, wh = wave >> 1;
 
   floatx4 acc[kGwT][kGwT];
 #pragma unroll
   for (int i = 0; i < kGwT; ++i)
 #pragma unroll
     for (int j = 0; j < kGwT; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
-  // K and cout are multiples of 4 (checked by the launcher), so a lane's four channels are all inside or all outside
-  const bool kok = k0 < a.K, wok = w0 < a.cout;
-  const int kc = kok ? k0 : 0, wc = wok ? w0 : 0;
-  int xo = kc, yo = 0;
-  if constexpr (YC) {
-    xo = kc / a.cy;
-    yo = kc - xo * a.cy;
-  }
+
   const int s_begin = a.path_ptr[p], s_end = a.path_ptr[p + 1];
-  for (int s = s_begin; s < s_end; ++s) {
-    // the segment's terms (at most kUvtTerms per item: the caller splits longer segments) in scalar registers; slots
-    // past the end repeat the first term's rows — their loads are issued with the others and never used
-    const cgtp_uvt_item it = a.items[s];
-    const int n_t = it.t1 - it.t0;
-    int xrow[kUvtTerms], yrow[kUvtTerms];
-    float c[kUvtTerms];
-#pragma unroll
-    for (int k = 0; k < kUvtTerms; ++k) {
-      const int t = k < n_t ? it.t0 + k : it.t0;
-      xrow[k] = a.ta[t] * a.cx;
-      yrow[k] = a.tb[t] * (YC ? a.cy : 1);
-      c[k] = a.tc[t];
-    }
-    const int grow = it.out_row * a.cout;
-    for (int64_t n0 = n_begin; n0 < n_end; n0 += 4) {
-      const int64_t n = n0 + g4;
-      const bool live = n < n_end;
-      const int64_t nc = live ? n : n_end - 1;
-      const float* xn = a.x + nc * a.dx * a.cx + xo;
-      const float* yn = a.y + nc * a.dy * (YC ? a.cy : 1) + yo;
-      // all loads of the step first ...
-      const floatx4 bv4 = *reinterpret_cast<const floatx4*>(a.g + nc * a.dg * a.cout + grow + wc);
-      floatx4 v4[kUvtTerms];     // y without channels: four channels of x; with: four channels of y
-      float v1[kUvtTerms];       // y without channels: y[n, b]; with: x[n, a, u]
+  const int steps = (int)((n_end - n_begin + kGwStep - 1) / kGwStep);
+  const int total = (s_end - s_begin) * steps;
+
+  // state of the loads in flight: the segment's terms in scalar registers (at most kUvtTerms per item: the caller
+  // splits longer segments; slots past the end repeat the first term's rows with coefficient zero)
+  int ld_item = s_begin - 1, ld_step = steps;
+  int xrow[kUvtTerms], yrow[kUvtTerms], grow = 0;
+  float c[kUvtTerms];
+  floatx4 v4[kUvtTerms];     // y without channels: four channels of x; with: four channels of y
+  float v1[kUvtTerms];       // y without channels: y[n, b]; with: x[n, a, u]
+  floatx4 bv4;
+  bool ld_live = false;
+
+  auto issue = [&]() __attribute__((always_inline)) {
+    if (ld_step == steps) {
+      ld_step = 0;
+      ++ld_item;
+      const cgtp_uvt_item it = a.items[ld_item];
+      const int n_t = it.t1 - it.t0;
 #pragma unroll
       for (int k = 0; k < kUvtTerms; ++k) {
-        if constexpr (YC) {
-          v1[k] = xn[xrow[k]];
-          v4[k] = *reinterpret_cast<const floatx4*>(yn + yrow[k]);
-        } else {
-          v4[k] = *reinterpret_cast<const floatx4*>(xn + xrow[k]);
-          v1[k] = yn[yrow[k]];
-        }
+        const int t = k < n_t ? it.t0 + k : it.t0;
+        xrow[k] = a.ta[t] * a.cx;
+        yrow[k] = a.tb[t] * (YC ? a.cy : 1);
+        c[k] = k < n_t ? a.tc[t] : 0.f;
       }
-      // ... then the mixing of the terms that exist (wave-uniform branches around arithmetic only)
-      floatx4 av = {0.f, 0.f, 0.f, 0.f};
+      grow = it.out_row * a.cout;
+    }
+    const int64_t n = n_begin + (int64_t)ld_step * kGwStep + ls;
+    ld_live = n < n_end;
+    const int64_t nc = ld_live ? n : n_end - 1;
+    const float* xn = a.x + nc * a.dx * a.cx + xo;
+    const float* yn = a.y + nc * a.dy * (YC ? a.cy : 1) + yo;
+    bv4 = *reinterpret_cast<const floatx4*>(a.g + nc * a.dg * a.cout + grow + wc);
 #pragma unroll
-      for (int k = 0; k < kUvtTerms; ++k)
-        if (k < n_t) av += (c[k] * v1[k]) * v4[k];
-      const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-      av = (live && kok) ? av : zero;
-      const floatx4 bv = (live && wok) ? bv4 : zero;
+    for (int k = 0; k < kUvtTerms; ++k) {
+      if constexpr (YC) {
+        v1[k] = xn[xrow[k]];
+        v4[k] = *reinterpret_cast<const floatx4*>(yn + yrow[k]);
+      } else {
+        v4[k] = *reinterpret_cast<const floatx4*>(xn + xrow[k]);
+        v1[k] = yn[yrow[k]];
+      }
+    }
+    ++ld_step;
+  };
+  // mixes the terms of the loads in flight and puts both operands into stage buf
+  auto commit = [&](int buf) __attribute__((always_inline)) {
+    floatx4 av = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < kGwT; ++i)
+    for (int k = 0; k < kUvtTerms; ++k) av += (c[k] * v1[k]) * v4[k];
+    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+    *reinterpret_cast<floatx4*>(&lds_a[buf][ls][lq]) = (ld_live && kok) ? av : zero;
+    *reinterpret_cast<floatx4*>(&lds_b[buf][ls][lq]) = (ld_live && wok) ? bv4 : zero;
+  };
+
+  if (total > 0) {
+    issue();
+    commit(0);
+    if (total > 1) issue();
+    __syncthreads();
+    for (int i = 0; i < total; ++i) {
+      const int buf = i & 1;
+      floatx4 af[2], bf[2];
 #pragma unroll
-        for (int j = 0; j < kGwT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+      for (int ks = 0; ks < 2; ++ks) {
+        af[ks] = *reinterpret_cast<const floatx4*>(&lds_a[buf][4 * ks + g4][kh * 64 + 4 * r]);
+        bf[ks] = *reinterpret_cast<const floatx4*>(&lds_b[buf][4 * ks + g4][wh * 64 + 4 * r]);
+      }
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int ti = 0; ti < kGwT; ++ti)
+#pragma unroll
+          for (int tj = 0; tj < kGwT; ++tj)
+            acc[ti][tj] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[ks][ti], bf[ks][tj], acc[ti][tj], 0, 0, 0);
+      if (i + 1 < total) commit(buf ^ 1);
+      if (i + 2 < total) issue();
+      __syncthreads();
     }
   }
   // accumulator layout: lane (column r, g4) holds rows 4 g4 .. + 3 of a tile; tile (i, j) row q is channel
   // 4 q + i of the wavefront's 64, column r is output channel 4 r + j
   float* out = a.part + ((int64_t)blockIdx.x * a.n_paths + p) * a.K * a.cout;
-  const int kbase = kgrp * 128 + (wave & 1) * 64;
+  const int kbase = kgrp * 128 + kh * 64;
+  const int w0 = wgrp * 128 + wh * 64 + 4 * r;
+  if (w0 < a.cout) {
 #pragma unroll
-  for (int i = 0; i < kGwT; ++i)
+    for (int i = 0; i < kGwT; ++i)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int k = kbase + 4 * (4 * g4 + e) + i;
-      if (k < a.K && wok) {
-        floatx4 v;
+      for (int e = 0; e < 4; ++e) {
+        const int k = kbase + 4 * (4 * g4 + e) + i;
+        if (k < a.K) {
+          floatx4 v;
 #pragma unroll
-        for (int j = 0; j < kGwT; ++j) v[j] = acc[i][j][e];
-        *reinterpret_cast<floatx4*>(out + (int64_t)k * a.cout + w0) = v;
+          for (int j = 0; j < kGwT; ++j) v[j] = acc[i][j][e];
+          *reinterpret_cast<floatx4*>(out + (int64_t)k * a.cout + w0) = v;
+        }
       }
-    }
+  }
 }
 
 __global__ void uvt_gw_reduce_kernel(const float* __restrict__ part, float* __restrict__ gw, int64_t n_chunks, int64_t n) {
@@ -451,6 +498,153 @@ static int64_t uvt_gw_chunk(int64_t n_rows) {
   int64_t chunk = 256;
   while ((n_rows + chunk - 1) / chunk > 128) chunk *= 2;
   return chunk;
+}
+
+// ---- gradient of a second operand without channels ("u1v") --------------------------------------------------------
+//   gy[n, b] = sum_{segments s = (p, a)} sum_{t in s} coef_t * sum_w g[n, M_t, w] * Z_s[n, w],
+//   Z_s[n, w] = sum_k x[n, a, k] * W[p, k, w]
+// The second operand is what is asked for, so nothing can be coupled before the channel contraction: a wavefront
+// forms Z_s for 16 samples and 32 output channels on the matrix cores (operands: the packed weight of the forward
+// and the plain row a of x staged in LDS), then takes the scalar products with the rows of g its segment's terms
+// name.  The accumulator lane (sample r, group q) holds four consecutive channels of its sample, so a term costs two
+// 16-byte loads of g (requested before the matrix instructions start), eight multiply-adds, a sum over the four
+// groups and one LDS add into the wavefront's own (sample, b) array — no atomics between wavefronts; the arrays are
+// added in wavefront order at the end.  Eight wavefronts share a workgroup's 16 samples: the segments are dealt round
+// robin to groups of wavefronts, the blocks of 32 output channels within a group.
+struct UvtGyDev {
+  const float* x;
+  const float* g;
+  const float* wp;
+  float* gy;
+  const cgtp_uvt_item* items;   // segments: p, out_row = a, t0, t1
+  const int32_t* ta;            // row M of g
+  const int32_t* tb;            // row b of gy
+  const float* tc;
+  int64_t n_rows;
+  int n_items, n_terms, dx, dy, dg, cx, cout;
+  int kx, px, kblocks, wbp;
+  int wchunks, wgroups;         // blocks of 32 output channels; wavefronts of a group that share a segment (1, 2, 4)
+};
+
+constexpr int kGyWB = 2;        // blocks of 16 output channels per pass
+constexpr int kGyWaves = 8;
+
+__global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGyDev a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* xs = reinterpret_cast<float*>(smem);
+  float* part = xs + (size_t)16 * a.px;                       // [wavefront][sample][b]
+  const int64_t nb0 = (int64_t)blockIdx.x * 16;
+  {
+    const int kx4 = a.kx / 4, per_sample = a.dx * kx4;
+    for (int i = threadIdx.x; i < 16 * per_sample; i += blockDim.x) {
+      const int s = i / per_sample, rem = i - s * per_sample, row = rem / kx4, c4 = rem - row * kx4;
+      const int64_t n = nb0 + s;
+      floatx4 v = {0.f, 0.f, 0.f, 0.f};
+      if (n < a.n_rows && c4 * 4 < a.cx) v = *reinterpret_cast<const floatx4*>(a.x + (n * a.dx + row) * a.cx + c4 * 4);
+      *reinterpret_cast<floatx4*>(xs + (size_t)s * a.px + row * a.kx + c4 * 4) = v;
+    }
+  }
+  for (int i = threadIdx.x; i < kGyWaves * 16 * a.dy; i += blockDim.x) part[i] = 0.f;
+  const UvtTables tab = uvt_stage_tables(a, reinterpret_cast<unsigned char*>(part + kGyWaves * 16 * a.dy));
+  __syncthreads();
+
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), r = lane & 15, q = lane >> 4;
+  const int wg = wave & (a.wgroups - 1), sg = wave / a.wgroups, sgroups = kGyWaves / a.wgroups;
+  const int64_t n = nb0 + r;
+  // samples past the end are staged as zeros (Z = 0); their rows of g are read from the last sample
+  const float* gn = a.g + (n < a.n_rows ? n : a.n_rows - 1) * a.dg * a.cout;
+  const float* xl = xs + (size_t)r * a.px + 4 * q;
+  float* mine = part + (size_t)(wave * 16 + r) * a.dy;
+  const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+
+  for (int s = sg; s < a.n_items; s += sgroups) {
+    const cgtp_uvt_item it = uvt_item_at(tab, s);
+    const int n_t = it.t1 - it.t0;
+    if (n_t <= 0) continue;
+    // the segment's first kUvtTerms terms in scalar registers; slots past the end repeat the first with factor zero
+    int mrow[kUvtTerms], brow[kUvtTerms];
+    float c[kUvtTerms];
+#pragma unroll
+    for (int k = 0; k < kUvtTerms; ++k) {
+      const int t = k < n_t ? it.t0 + k : it.t0;
+      mrow[k] = __builtin_amdgcn_readfirstlane(tab.ta[t]) * a.cout;
+      brow[k] = __builtin_amdgcn_readfirstlane(tab.tb[t]);
+      c[k] = k < n_t ? tab.tc[t] : 0.f;
+    }
+    const float* xrow = xl + it.out_row * a.kx;
+    for (int wc = wg; wc < a.wchunks; wc += a.wgroups) {
+      const int wb0 = wc * kGyWB;
+      int wcol[kGyWB];
+      bool wok[kGyWB];
+#pragma unroll
+      for (int wb = 0; wb < kGyWB; ++wb) {
+        const int w = (wb0 + wb) * 16 + 4 * q;       // cout is a multiple of 4: all four channels inside or outside
+        wok[wb] = w < a.cout;
+        wcol[wb] = wok[wb] ? w : 0;
+      }
+      floatx4 gv[kUvtTerms][kGyWB];
+#pragma unroll
+      for (int k = 0; k < kUvtTerms; ++k)
+#pragma unroll
+        for (int wb = 0; wb < kGyWB; ++wb) gv[k][wb] = *reinterpret_cast<const floatx4*>(gn + mrow[k] + wcol[wb]);
+
+      floatx4 acc[kGyWB], A0[kGyWB], A1[kGyWB], B0, B1;
+#pragma unroll
+      for (int wb = 0; wb < kGyWB; ++wb) acc[wb] = zero;
+      const float* base = a.wp + ((int64_t)it.p * a.kblocks * a.wbp + wb0) * 256 + lane * 4;
+      const int64_t kstride = (int64_t)a.wbp * 256;
+      auto load = [&](int kb, floatx4 (&A)[kGyWB], floatx4& B) __attribute__((always_inline)) {
+#pragma unroll
+        for (int wb = 0; wb < kGyWB; ++wb) A[wb] = *reinterpret_cast<const floatx4*>(base + kb * kstride + wb * 256);
+        B = *reinterpret_cast<const floatx4*>(xrow + kb * 16);
+      };
+      auto mult = [&](const floatx4 (&A)[kGyWB], const floatx4& B) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int wb = 0; wb < kGyWB; ++wb) acc[wb] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[wb][i], B[i], acc[wb], 0, 0, 0);
+      };
+      load(0, A0, B0);
+      for (int kb = 0; kb < a.kblocks; kb += 2) {     // kblocks is even (whole items of the packing)
+        load(kb + 1, A1, B1);
+        mult(A0, B0);
+        load(kb + 2 < a.kblocks ? kb + 2 : kb, A0, B0);
+        mult(A1, B1);
+      }
+      // accumulator: lane (sample r, q) holds Z[n, 16 (wb0 + wb) + 4 q + e]
+      auto add_term = [&](const floatx4 (&gt)[kGyWB], float coef, int b) __attribute__((always_inline)) {
+        float d = 0.f;
+#pragma unroll
+        for (int wb = 0; wb < kGyWB; ++wb) {
+          const floatx4 gg = wok[wb] ? gt[wb] : zero;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) d += gg[e] * acc[wb][e];
+        }
+        d += __shfl_xor(d, 16);
+        d += __shfl_xor(d, 32);
+        if (q == 0) atomicAdd(mine + b, coef * d);   // LDS, this wavefront's own array: in program order
+      };
+#pragma unroll
+      for (int k = 0; k < kUvtTerms; ++k) add_term(gv[k], c[k], brow[k]);
+      for (int t = it.t0 + kUvtTerms; t < it.t1; ++t) {   // longer segments (large irreps only)
+        floatx4 gt[kGyWB];
+        const int m = __builtin_amdgcn_readfirstlane(tab.ta[t]) * a.cout;
+#pragma unroll
+        for (int wb = 0; wb < kGyWB; ++wb) gt[wb] = *reinterpret_cast<const floatx4*>(gn + m + wcol[wb]);
+        add_term(gt, tab.tc[t], __builtin_amdgcn_readfirstlane(tab.tb[t]));
+      }
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 16 * a.dy; i += blockDim.x) {
+    const int64_t ni = nb0 + i / a.dy;
+    if (ni < a.n_rows) {
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < kGyWaves; ++w) sum += part[w * 16 * a.dy + i];
+      a.gy[nb0 * a.dy + i] = sum;
+    }
+  }
 }
 
 struct UvtPlan {
@@ -619,6 +813,40 @@ int cgtp_uvt_grad_w(const cgtp_uvt_gw_args* a, void* stream) {
   if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
   hipLaunchKernelGGL(uvt_gw_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, st,
                      (const float*)a->workspace, (float*)a->gw, n_chunks, n_out);
+  return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
+}
+
+int cgtp_uvt_grad_y(const cgtp_uvt_gy_args* a, void* stream) {
+  if (!a) return CGTP_ERR_NULL;
+  if (a->dtype != CGTP_F32) return CGTP_ERR_DTYPE;
+  if (a->n_rows < 0 || a->n_items < 0 || a->n_terms < 0 || a->dx <= 0 || a->dy <= 0 || a->dg <= 0 || a->cx <= 0 ||
+      a->cout <= 0)
+    return CGTP_ERR_SHAPE;
+  if (a->cx % 4 || a->cout % 4) return CGTP_ERR_SHAPE;
+  if (!a->x || !a->g || !a->wp || !a->gy || (a->n_items && (!a->items || !a->term_m || !a->term_b || !a->term_c)))
+    return CGTP_ERR_NULL;
+  if ((reinterpret_cast<uintptr_t>(a->x) | reinterpret_cast<uintptr_t>(a->g) | reinterpret_cast<uintptr_t>(a->wp)) & 15u)
+    return CGTP_ERR_ALIGN;
+  UvtGyDev d;
+  d.x = (const float*)a->x; d.g = (const float*)a->g; d.wp = (const float*)a->wp; d.gy = (float*)a->gy;
+  d.items = a->items; d.ta = a->term_m; d.tb = a->term_b; d.tc = (const float*)a->term_c;
+  d.n_rows = a->n_rows; d.n_items = a->n_items; d.n_terms = a->n_terms;
+  d.dx = a->dx; d.dy = a->dy; d.dg = a->dg; d.cx = a->cx; d.cout = a->cout;
+  d.kblocks = round_up((a->cx + 15) / 16, kUvtKbi);
+  d.kx = d.kblocks * 16;
+  d.px = a->dx * d.kx + 4;
+  d.wbp = round_up((a->cout + 15) / 16, 4);
+  d.wchunks = (a->cout + 16 * kGyWB - 1) / (16 * kGyWB);
+  d.wgroups = d.wchunks >= 4 ? 4 : d.wchunks >= 2 ? 2 : 1;
+  const int64_t lds = ((int64_t)16 * d.px + (int64_t)kGyWaves * 16 * a->dy) * 4 + (int64_t)a->n_items * 32 +
+                      (int64_t)a->n_terms * 12 + 16;
+  if (lds > kLdsBytes) return CGTP_ERR_LDS;
+  if (a->n_rows == 0) return CGTP_OK;
+  if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)uvt_grad_y_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             (int)lds) != hipSuccess)
+    return CGTP_ERR_LDS;
+  hipLaunchKernelGGL(uvt_grad_y_kernel, dim3((unsigned)((a->n_rows + 15) / 16)), dim3(kGyWaves * kWave), (size_t)lds,
+                     (hipStream_t)stream, d);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 

@@ -120,6 +120,56 @@ def grad_w(x: Tensor, y: Tensor, g: Tensor, tp_info) -> Tensor:
     return gw
 
 
+class _SegWalk:
+    """Segments (weight path, row of the first operand) with their terms (row of grad_out, row of the second operand):
+    the walk of ``cgtp_uvt_grad_y``.  Segments are not split: the kernel forms one matrix product per segment."""
+
+    def __init__(self, coo, device):
+        order = np.lexsort([coo.M, coo.M2, coo.M1, coo.p])
+        p_idx, a_idx, b_idx, m_idx = (np.asarray(v)[order] for v in (coo.p, coo.M1, coo.M2, coo.M))
+        coef = np.asarray(coo.coef, dtype=np.float64)[order]
+        items = []
+        t, n_terms = 0, p_idx.shape[0]
+        while t < n_terms:
+            t1 = t
+            while t1 < n_terms and p_idx[t1] == p_idx[t] and a_idx[t1] == a_idx[t]:
+                t1 += 1
+            items.append([int(p_idx[t]), 0, 0, t, t1, int(a_idx[t]), 0, 0])
+            t = t1
+        # longest segments first: the wavefront groups take segments round robin
+        items.sort(key=lambda it: it[3] - it[4])
+        self.n_items, self.n_terms = len(items), n_terms
+        self.items = torch.tensor(items, dtype=torch.int32).reshape(-1, 8).to(device)
+        self.term_m = torch.from_numpy(m_idx.astype(np.int32)).to(device)
+        self.term_b = torch.from_numpy(b_idx.astype(np.int32)).to(device)
+        self.term_c = torch.from_numpy(coef.astype(np.float32)).to(device)
+
+
+def grad_y_supported(n: int, dx: int, dy: int, cx: int, cout: int, tp_info) -> bool:
+    """Whether the 16 staged samples of a ``cgtp_uvt_grad_y`` workgroup and its tables fit the LDS."""
+    c = kernels.coo_of(tp_info)
+    kx = ((cx + 15) // 16 + 3) // 4 * 4 * 16
+    lds = (16 * (dx * kx + 4) + 8 * 16 * dy) * 4 + len(c.coef) * (32 + 12) + 16
+    return cx % 4 == 0 and cout % 4 == 0 and lds <= 160 * 1024
+
+
+def grad_y(x: Tensor, g: Tensor, wp: Tensor, tp_info, dy: int) -> Tensor:
+    """``gy[n, b] = sum_t c_t <g[n, M_t, :], x[n, a_t, :] @ W[p_t]>`` (``cgtp_uvt_grad_y``); ``wp``: the weight as packed
+    for the forward."""
+    walk = kernels.cached(tp_info.info_Mij_fwd.scale, ("uvt_seg_walk", str(x.device)),
+                          lambda: _SegWalk(kernels.coo_of(tp_info), x.device))
+    n, dx, cx = x.shape
+    gy = torch.empty((n, dy), dtype=torch.float32, device=x.device)
+    a = _lib.UvtGyArgs()
+    a.x, a.g, a.wp, a.gy = x.data_ptr(), g.data_ptr(), wp.data_ptr(), gy.data_ptr()
+    a.items, a.term_m, a.term_b, a.term_c = (walk.items.data_ptr(), walk.term_m.data_ptr(), walk.term_b.data_ptr(),
+                                             walk.term_c.data_ptr())
+    a.n_rows, a.n_items, a.n_terms = n, walk.n_items, walk.n_terms
+    a.dx, a.dy, a.dg, a.cx, a.cout, a.dtype = dx, dy, g.shape[1], cx, g.shape[2], _lib.F32
+    _lib.check(_lib.lib.cgtp_uvt_grad_y(C.byref(a), _lib.stream_ptr(x.device)), "cgtp_uvt_grad_y")
+    return gy
+
+
 def chunk_of(n_rows: int, dx: int, dy: int, cx: int, cy: int, cout: int) -> int:
     """Chunk length (blocks of 16 contracted channels per item) of a launch with these extents; <= 0: the kernels do
     not take them (channel counts not multiples of 4, rows of 16 samples beyond the LDS)."""
@@ -164,10 +214,10 @@ def _coo(tp_info):
 
 
 class _U1vNative(Function):
-    """u1v, shared fp32 weight ``(P, U, W)``.  The gradient of the first operand is the same kernel with the rows'
-    roles exchanged and the weight read transposed; the gradients of the second operand and of the weight come from
-    the differentiable two-stage route of ``_uv_gemm`` for now (library GEMMs), as does everything under
-    ``create_graph``."""
+    """u1v, shared fp32 weight ``(P, U, W)``.  The gradient of the first operand is the forward kernel with the rows'
+    roles exchanged and the weight read transposed; the gradients of the weight and of the second operand have
+    kernels of their own (``cgtp_uvt_grad_w``, ``cgtp_uvt_grad_y``).  Under ``create_graph`` the backward is the
+    differentiable two-stage route of ``_uv_gemm``."""
 
     @staticmethod
     def forward(ctx, x: Tensor, y: Tensor, w: Tensor, tp_info):
@@ -199,10 +249,7 @@ class _U1vNative(Function):
         if need[2]:
             gw = grad_w(x, y, g, tp_info)
         if need[1]:
-            with torch.enable_grad():
-                yr = y.detach().requires_grad_(True)
-                out = _uv_gemm.u1v(x.detach(), yr, w.detach(), tp_info)
-                (gy,) = torch.autograd.grad(out, (yr,), g)
+            gy = grad_y(x, g, pack(w, p, u, wc, u * wc, wc, 1), tp_info, c.D2)
         return gx, gy, gw, None
 
 
@@ -215,7 +262,7 @@ def u1v_supported(x: Tensor, y: Tensor, w: Tensor, tp_info) -> bool:
     _, u, wc = w.shape
     n = x.shape[0]
     return (chunk_of(n, c.D1, c.D2, u, 0, wc) > 0 and chunk_of(n, c.DO, c.D2, wc, 0, u) > 0
-            and x.data_ptr() % 16 == 0)
+            and grad_y_supported(n, c.D1, c.D2, u, wc, tp_info) and x.data_ptr() % 16 == 0)
 
 
 def u1v(x: Tensor, y: Tensor, w: Tensor, tp_info) -> Tensor:

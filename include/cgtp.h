@@ -376,6 +376,31 @@ typedef struct cgtp_uvt_gw_args {
 int64_t cgtp_uvt_grad_w_workspace_bytes(int64_t n_rows, int32_t n_paths, int64_t K, int32_t cout);
 int cgtp_uvt_grad_w(const cgtp_uvt_gw_args* args, void* stream);
 
+/* Gradient of a second operand without channels (u1v):
+ *   gy[n, b] = sum_t coef_t * sum_w grad_out[n, M_t, w] * (sum_k x[n, a_t, k] * W[p_t, k, w])
+ * (the reference obtains it from autograd through sparse_mul and the batched matmul,
+ * equitorch/nn/functional/linears.py:283-336).  wp: the weight as packed for the forward by cgtp_uvt_pack_weights.
+ * items: one per segment (p, a = out_row) with its terms t0 .. t1 (nkb, kb0, flags unused); term_m / term_b: rows of
+ * grad_out and of gy.  x (n_rows, dx, cx), grad_out (n_rows, dg, cout), gy (n_rows, dy); cx and cout multiples of 4,
+ * 16-byte aligned pointers.  The 16 staged samples of a workgroup must fit the LDS (CGTP_ERR_LDS otherwise). */
+typedef struct cgtp_uvt_gy_args {
+  const void* x;
+  const void* g;
+  const void* wp;
+  void* gy;
+  const cgtp_uvt_item* items;   /* device */
+  const int32_t* term_m;        /* device */
+  const int32_t* term_b;        /* device */
+  const void* term_c;           /* device, dtype */
+  int64_t n_rows;
+  int32_t n_items, n_terms;
+  int32_t dx, dy, dg;
+  int32_t cx, cout;
+  int32_t dtype;                /* CGTP_F32 */
+} cgtp_uvt_gy_args;
+
+int cgtp_uvt_grad_y(const cgtp_uvt_gy_args* args, void* stream);
+
 /* ---- real spherical harmonics of vectors -----------------------------------------------------------------
  * Stands in for spherical_harmonics (equitorch/ops/spherical_harmonics.py:68-640: explicit polynomials per
  * degree, TorchScript, differentiated by autograd) together with its callers' pre- and post-processing:
