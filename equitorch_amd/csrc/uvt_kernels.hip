@@ -528,6 +528,7 @@ struct UvtGyDev {
 
 constexpr int kGyWB = 2;        // blocks of 16 output channels per pass
 constexpr int kGyWaves = 8;
+constexpr int kGyRing = 4;       // blocks of 16 k in flight (= kUvtKbi: the packing pads k to whole multiples)
 
 __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGyDev a) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -557,83 +558,114 @@ __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGy
   float* mine = part + (size_t)(wave * 16 + r) * a.dy;
   const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
 
-  for (int s = sg; s < a.n_items; s += sgroups) {
-    const cgtp_uvt_item it = uvt_item_at(tab, s);
+  // The passes of this wavefront — (segment, block of 32 output channels) — form one sequence; the weight fragments
+  // and the rows of x run kGyRing blocks of 16 k ahead of the matrix instructions, across the ends of the passes
+  // (a weight fragment comes from the L2 in more cycles than one block's eight matrix instructions take).
+  const int64_t kstride = (int64_t)a.wbp * 256;
+  floatx4 A[kGyRing][kGyWB], B[kGyRing];
+  auto load = [&](const float* wbase, const float* xrow, int kb, floatx4 (&Aj)[kGyWB], floatx4& Bj) __attribute__((always_inline)) {
+#pragma unroll
+    for (int wb = 0; wb < kGyWB; ++wb) Aj[wb] = *reinterpret_cast<const floatx4*>(wbase + kb * kstride + wb * 256);
+    Bj = *reinterpret_cast<const floatx4*>(xrow + kb * 16);
+  };
+  auto wbase_of = [&](const cgtp_uvt_item& it, int wc) __attribute__((always_inline)) {
+    return a.wp + ((int64_t)it.p * a.kblocks * a.wbp + wc * kGyWB) * 256 + lane * 4;
+  };
+  int s = sg, wc = wg;
+  cgtp_uvt_item it = uvt_item_at(tab, s < a.n_items ? s : 0);
+  const float* wbase = wbase_of(it, wc);
+  const float* xrow = xl + it.out_row * a.kx;
+  if (s < a.n_items) {
+#pragma unroll
+    for (int j = 0; j < kGyRing; ++j) load(wbase, xrow, j, A[j], B[j]);   // kblocks is a multiple of kGyRing
+  }
+  while (s < a.n_items) {
+    // the pass after this one
+    int s2 = s, wc2 = wc + a.wgroups;
+    if (wc2 >= a.wchunks) {
+      wc2 = wg;
+      s2 = s + sgroups;
+    }
+    const bool more = s2 < a.n_items;
+    const cgtp_uvt_item it2 = uvt_item_at(tab, more ? s2 : s);
+    const float* wbase2 = more ? wbase_of(it2, wc2) : wbase;
+    const float* xrow2 = more ? xl + it2.out_row * a.kx : xrow;
+
     const int n_t = it.t1 - it.t0;
-    if (n_t <= 0) continue;
-    // the segment's first kUvtTerms terms in scalar registers; slots past the end repeat the first with factor zero
+    // the segment's first kUvtTerms terms in scalar registers (slots past the end: the first term again, never used)
     int mrow[kUvtTerms], brow[kUvtTerms];
     float c[kUvtTerms];
 #pragma unroll
     for (int k = 0; k < kUvtTerms; ++k) {
       const int t = k < n_t ? it.t0 + k : it.t0;
-      mrow[k] = __builtin_amdgcn_readfirstlane(tab.ta[t]) * a.cout;
+      mrow[k] = n_t > 0 ? __builtin_amdgcn_readfirstlane(tab.ta[t]) * a.cout : 0;
       brow[k] = __builtin_amdgcn_readfirstlane(tab.tb[t]);
-      c[k] = k < n_t ? tab.tc[t] : 0.f;
+      c[k] = tab.tc[t];
     }
-    const float* xrow = xl + it.out_row * a.kx;
-    for (int wc = wg; wc < a.wchunks; wc += a.wgroups) {
-      const int wb0 = wc * kGyWB;
-      int wcol[kGyWB];
-      bool wok[kGyWB];
+    const int wb0 = wc * kGyWB;
+    int wcol[kGyWB];
+    bool wok[kGyWB];
 #pragma unroll
-      for (int wb = 0; wb < kGyWB; ++wb) {
-        const int w = (wb0 + wb) * 16 + 4 * q;       // cout is a multiple of 4: all four channels inside or outside
-        wok[wb] = w < a.cout;
-        wcol[wb] = wok[wb] ? w : 0;
-      }
-      floatx4 gv[kUvtTerms][kGyWB];
+    for (int wb = 0; wb < kGyWB; ++wb) {
+      const int w = (wb0 + wb) * 16 + 4 * q;       // cout is a multiple of 4: all four channels inside or outside
+      wok[wb] = w < a.cout;
+      wcol[wb] = wok[wb] ? w : 0;
+    }
+    // rows of g of the terms, requested before the matrix instructions; the second half only for long segments
+    floatx4 gv[kUvtTerms][kGyWB];
 #pragma unroll
-      for (int k = 0; k < kUvtTerms; ++k)
+    for (int k = 0; k < kUvtTerms / 2; ++k)
+#pragma unroll
+      for (int wb = 0; wb < kGyWB; ++wb) gv[k][wb] = *reinterpret_cast<const floatx4*>(gn + mrow[k] + wcol[wb]);
+    if (n_t > kUvtTerms / 2) {
+#pragma unroll
+      for (int k = kUvtTerms / 2; k < kUvtTerms; ++k)
 #pragma unroll
         for (int wb = 0; wb < kGyWB; ++wb) gv[k][wb] = *reinterpret_cast<const floatx4*>(gn + mrow[k] + wcol[wb]);
+    }
 
-      floatx4 acc[kGyWB], A0[kGyWB], A1[kGyWB], B0, B1;
+    floatx4 acc[kGyWB];
 #pragma unroll
-      for (int wb = 0; wb < kGyWB; ++wb) acc[wb] = zero;
-      const float* base = a.wp + ((int64_t)it.p * a.kblocks * a.wbp + wb0) * 256 + lane * 4;
-      const int64_t kstride = (int64_t)a.wbp * 256;
-      auto load = [&](int kb, floatx4 (&A)[kGyWB], floatx4& B) __attribute__((always_inline)) {
+    for (int wb = 0; wb < kGyWB; ++wb) acc[wb] = zero;
+    for (int kb = 0; kb < a.kblocks; kb += kGyRing) {
+      const bool wrap = kb + kGyRing >= a.kblocks;   // the blocks requested now belong to the next pass
+      const float* wnext = wrap ? wbase2 : wbase;
+      const float* xnext = wrap ? xrow2 : xrow;
+      const int kbn = wrap ? 0 : kb + kGyRing;
 #pragma unroll
-        for (int wb = 0; wb < kGyWB; ++wb) A[wb] = *reinterpret_cast<const floatx4*>(base + kb * kstride + wb * 256);
-        B = *reinterpret_cast<const floatx4*>(xrow + kb * 16);
-      };
-      auto mult = [&](const floatx4 (&A)[kGyWB], const floatx4& B) __attribute__((always_inline)) {
+      for (int j = 0; j < kGyRing; ++j) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-          for (int wb = 0; wb < kGyWB; ++wb) acc[wb] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[wb][i], B[i], acc[wb], 0, 0, 0);
-      };
-      load(0, A0, B0);
-      for (int kb = 0; kb < a.kblocks; kb += 2) {     // kblocks is even (whole items of the packing)
-        load(kb + 1, A1, B1);
-        mult(A0, B0);
-        load(kb + 2 < a.kblocks ? kb + 2 : kb, A0, B0);
-        mult(A1, B1);
-      }
-      // accumulator: lane (sample r, q) holds Z[n, 16 (wb0 + wb) + 4 q + e]
-      auto add_term = [&](const floatx4 (&gt)[kGyWB], float coef, int b) __attribute__((always_inline)) {
-        float d = 0.f;
-#pragma unroll
-        for (int wb = 0; wb < kGyWB; ++wb) {
-          const floatx4 gg = wok[wb] ? gt[wb] : zero;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) d += gg[e] * acc[wb][e];
-        }
-        d += __shfl_xor(d, 16);
-        d += __shfl_xor(d, 32);
-        if (q == 0) atomicAdd(mine + b, coef * d);   // LDS, this wavefront's own array: in program order
-      };
-#pragma unroll
-      for (int k = 0; k < kUvtTerms; ++k) add_term(gv[k], c[k], brow[k]);
-      for (int t = it.t0 + kUvtTerms; t < it.t1; ++t) {   // longer segments (large irreps only)
-        floatx4 gt[kGyWB];
-        const int m = __builtin_amdgcn_readfirstlane(tab.ta[t]) * a.cout;
-#pragma unroll
-        for (int wb = 0; wb < kGyWB; ++wb) gt[wb] = *reinterpret_cast<const floatx4*>(gn + m + wcol[wb]);
-        add_term(gt, tab.tc[t], __builtin_amdgcn_readfirstlane(tab.tb[t]));
+          for (int wb = 0; wb < kGyWB; ++wb)
+            acc[wb] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[j][wb][i], B[j][i], acc[wb], 0, 0, 0);
+        load(wnext, xnext, kbn + j, A[j], B[j]);
       }
     }
+    // accumulator: lane (sample r, q) holds Z[n, 16 (wb0 + wb) + 4 q + e]
+    auto add_term = [&](const floatx4 (&gt)[kGyWB], float coef, int b) __attribute__((always_inline)) {
+      float d = 0.f;
+#pragma unroll
+      for (int wb = 0; wb < kGyWB; ++wb) {
+        const floatx4 gg = wok[wb] ? gt[wb] : zero;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) d += gg[e] * acc[wb][e];
+      }
+      d += __shfl_xor(d, 16);
+      d += __shfl_xor(d, 32);
+      if (q == 0) atomicAdd(mine + b, coef * d);   // LDS, this wavefront's own array: in program order
+    };
+#pragma unroll
+    for (int k = 0; k < kUvtTerms; ++k)
+      if (k < n_t) add_term(gv[k], c[k], brow[k]);
+    for (int t = it.t0 + kUvtTerms; t < it.t1; ++t) {   // longer segments (large irreps only)
+      floatx4 gt[kGyWB];
+      const int m = __builtin_amdgcn_readfirstlane(tab.ta[t]) * a.cout;
+#pragma unroll
+      for (int wb = 0; wb < kGyWB; ++wb) gt[wb] = *reinterpret_cast<const floatx4*>(gn + m + wcol[wb]);
+      add_term(gt, tab.tc[t], __builtin_amdgcn_readfirstlane(tab.tb[t]));
+    }
+    s = s2; wc = wc2; it = it2; wbase = wbase2; xrow = xrow2;
   }
   __syncthreads();
   for (int i = threadIdx.x; i < 16 * a.dy; i += blockDim.x) {
