@@ -71,7 +71,8 @@ class UvtArgs(C.Structure):
                 ("n_rows", C.c_int64), ("n_items", C.c_int32),
                 ("dx", C.c_int32), ("dy", C.c_int32), ("dout", C.c_int32),
                 ("cx", C.c_int32), ("cy", C.c_int32), ("cout", C.c_int32),
-                ("kbi", C.c_int32), ("dtype", C.c_int32), ("n_terms", C.c_int32)]
+                ("kbi", C.c_int32), ("dtype", C.c_int32), ("n_terms", C.c_int32),
+                ("n_groups", C.c_int32), ("group_ptr", C.c_int32 * 9)]
 
 
 class UvtGwArgs(C.Structure):
@@ -142,7 +143,8 @@ def _load():
     lib.cgtp_uvt_packed_elems.argtypes = [C.c_int32, C.c_int64, C.c_int32]
     lib.cgtp_uvt_pack_weights.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_int64, C.c_int64,
                                           C.c_int64, C.c_int32, C.c_void_p]
-    lib.cgtp_uvt_chunk.argtypes = [C.c_int64] + [C.c_int32] * 5
+    lib.cgtp_uvt_chunk.argtypes = [C.c_int64] + [C.c_int32] * 6
+    lib.cgtp_uvt_item_groups.argtypes = [C.c_int64] + [C.c_int32] * 6
     lib.cgtp_uvt_validate.argtypes = [C.POINTER(UvtArgs)]
     lib.cgtp_uvt_apply.argtypes = [C.POINTER(UvtArgs), C.c_void_p]
     lib.cgtp_uvt_grad_w_workspace_bytes.restype = C.c_int64

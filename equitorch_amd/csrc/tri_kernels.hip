@@ -588,13 +588,34 @@ int cgtp_abi_layout(int which, int64_t* out, int capacity) {
                                 CGTP_OFF(cgtp_uvt_args, n_items), CGTP_OFF(cgtp_uvt_args, dx), CGTP_OFF(cgtp_uvt_args, dy),
                                 CGTP_OFF(cgtp_uvt_args, dout), CGTP_OFF(cgtp_uvt_args, cx), CGTP_OFF(cgtp_uvt_args, cy),
                                 CGTP_OFF(cgtp_uvt_args, cout), CGTP_OFF(cgtp_uvt_args, kbi), CGTP_OFF(cgtp_uvt_args, dtype),
-                                CGTP_OFF(cgtp_uvt_args, n_terms)};
+                                CGTP_OFF(cgtp_uvt_args, n_terms), CGTP_OFF(cgtp_uvt_args, n_groups),
+                                CGTP_OFF(cgtp_uvt_args, group_ptr)};
+  static const int64_t uvt_gw[] = {sizeof(cgtp_uvt_gw_args), CGTP_OFF(cgtp_uvt_gw_args, x), CGTP_OFF(cgtp_uvt_gw_args, y),
+                                   CGTP_OFF(cgtp_uvt_gw_args, g), CGTP_OFF(cgtp_uvt_gw_args, gw),
+                                   CGTP_OFF(cgtp_uvt_gw_args, workspace), CGTP_OFF(cgtp_uvt_gw_args, items),
+                                   CGTP_OFF(cgtp_uvt_gw_args, path_ptr), CGTP_OFF(cgtp_uvt_gw_args, term_a),
+                                   CGTP_OFF(cgtp_uvt_gw_args, term_b), CGTP_OFF(cgtp_uvt_gw_args, term_c),
+                                   CGTP_OFF(cgtp_uvt_gw_args, n_rows), CGTP_OFF(cgtp_uvt_gw_args, n_items),
+                                   CGTP_OFF(cgtp_uvt_gw_args, n_terms), CGTP_OFF(cgtp_uvt_gw_args, n_paths),
+                                   CGTP_OFF(cgtp_uvt_gw_args, dx), CGTP_OFF(cgtp_uvt_gw_args, dy),
+                                   CGTP_OFF(cgtp_uvt_gw_args, dg), CGTP_OFF(cgtp_uvt_gw_args, cx),
+                                   CGTP_OFF(cgtp_uvt_gw_args, cy), CGTP_OFF(cgtp_uvt_gw_args, cout),
+                                   CGTP_OFF(cgtp_uvt_gw_args, dtype), CGTP_OFF(cgtp_uvt_gw_args, reserved_)};
+  static const int64_t uvt_gy[] = {sizeof(cgtp_uvt_gy_args), CGTP_OFF(cgtp_uvt_gy_args, x), CGTP_OFF(cgtp_uvt_gy_args, g),
+                                   CGTP_OFF(cgtp_uvt_gy_args, wp), CGTP_OFF(cgtp_uvt_gy_args, gy),
+                                   CGTP_OFF(cgtp_uvt_gy_args, items), CGTP_OFF(cgtp_uvt_gy_args, term_m),
+                                   CGTP_OFF(cgtp_uvt_gy_args, term_b), CGTP_OFF(cgtp_uvt_gy_args, term_c),
+                                   CGTP_OFF(cgtp_uvt_gy_args, n_rows), CGTP_OFF(cgtp_uvt_gy_args, n_items),
+                                   CGTP_OFF(cgtp_uvt_gy_args, n_terms), CGTP_OFF(cgtp_uvt_gy_args, dx),
+                                   CGTP_OFF(cgtp_uvt_gy_args, dy), CGTP_OFF(cgtp_uvt_gy_args, dg),
+                                   CGTP_OFF(cgtp_uvt_gy_args, cx), CGTP_OFF(cgtp_uvt_gy_args, cout),
+                                   CGTP_OFF(cgtp_uvt_gy_args, dtype)};
 #undef CGTP_OFF
-  const int64_t* tabs[] = {operand, tri, gen_operand, gen, uvu, uvt_item, uvt};
+  const int64_t* tabs[] = {operand, tri, gen_operand, gen, uvu, uvt_item, uvt, uvt_gw, uvt_gy};
   const int counts[] = {(int)(sizeof(operand) / 8), (int)(sizeof(tri) / 8), (int)(sizeof(gen_operand) / 8),
                         (int)(sizeof(gen) / 8), (int)(sizeof(uvu) / 8), (int)(sizeof(uvt_item) / 8),
-                        (int)(sizeof(uvt) / 8)};
-  if (which < 0 || which >= 7) return -1;
+                        (int)(sizeof(uvt) / 8), (int)(sizeof(uvt_gw) / 8), (int)(sizeof(uvt_gy) / 8)};
+  if (which < 0 || which >= 9) return -1;
   for (int i = 0; out && i < counts[which] && i < capacity; ++i) out[i] = tabs[which][i];
   return counts[which];
 }

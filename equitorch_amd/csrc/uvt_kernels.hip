@@ -9,12 +9,12 @@
 // for the whole batch) is formed on the vector ALUs directly in the layout of an MFMA B operand — lane (n, g) holds
 // k = 16 kb + 4 g + i of sample n — from the rows of x and y staged once per workgroup in LDS, and is contracted
 // with the weights by v_mfma_f32_16x16x4_f32 into a 16 (w) x 16 (n) accumulator tile per block of output channels.
-// The walk is a flat list of items (segment, chunk of k) ordered by output row, so a wavefront keeps only the
-// accumulators of the row it is working on.  fp32 matrix instructions are slow enough (32 cycles each) that the
-// table walk, the mixing (a few dozen FMAs per item) and the LDS reads disappear behind them; weight fragments come
-// from a copy of W repacked in fragment order (one contiguous KB per wavefront load) and are requested one item
-// ahead.  The gradient with respect to the channelled operand is the same kernel with the roles of the rows
-// exchanged and the weight packed transposed; the other two gradients have kernels of their own below.
+// The walk is a flat list of items (one per segment) ordered by output row, so a wavefront keeps only the
+// accumulators of the row it is working on.  A workgroup's wavefronts share the staged rows of its samples and split
+// the output rows (groups of items) and the output channels between them.  Weight fragments come from a copy of W
+// repacked in fragment order (one contiguous KB per wavefront load) and are requested four blocks of 16 k ahead.
+// The gradient with respect to the channelled operand is the same kernel with the roles of the rows exchanged and
+// the weight packed transposed; the other two gradients have kernels of their own below.
 #include "cgtp_device.h"
 #include "cgtp_host.h"
 
@@ -25,6 +25,7 @@ namespace cgtp {
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kUvtFirst = 1, kUvtLast = 2;   // item flags: first / last item of its output row
+constexpr int kUvtMaxGroups = 8;             // = wavefronts per workgroup
 constexpr int64_t kUvtTableRoom = 24 * 1024;  // LDS kept free for the walk tables when the launch shape is chosen
 
 struct UvtDev {
@@ -42,8 +43,11 @@ struct UvtDev {
   int px, py;    // LDS pitch per sample of the x and y tiles, in elements
   int kblocks;   // K / 16 (K padded to 16)
   int wbp;       // blocks of 16 output channels, rounded up to a multiple of 4 (as packed)
-  int sb_log2;   // log2 of the 16-sample blocks per workgroup (1, 2 or 4 blocks)
+  int sb_log2;   // log2 of the 16-sample blocks per workgroup
+  int wgroups;   // wavefronts of a sample block that split the output channels (power of two)
+  int igroups;   // groups of items (whole output rows) the remaining wavefronts of a sample block split
   int zero_floats;  // zeros in LDS that the unused term slots of an item read
+  int group_ptr[kUvtMaxGroups + 1];   // items of group i: group_ptr[i] .. group_ptr[i + 1]
 };
 
 // Rows of the workgroup's samples into LDS: x as [sample][row][kx] (zero-padded channels), y as [sample][row] or
@@ -144,14 +148,14 @@ __device__ __forceinline__ void uvt_terms(const UvtDev& a, const UvtTables& tab,
       T.yr[k] = live ? yl + ib * a.cy : zeros;
       T.s[k] = c;
     } else {
-      T.xr[k] = live ? xl + ia * a.kx + it.kb0 * 16 + 4 * g : zeros;
+      T.xr[k] = live ? xl + ia * a.kx + 4 * g : zeros;
       T.s[k] = live ? c * yl[ib] : 0.f;
     }
   }
 }
 
-// This lane's part of block j of 16 k of the mixed operand of an item: inter_s[n, 16 (kb0 + j) + 4 g + i], i < 4.
-// With a channelled y, lut[(kb0 + j) * 4 + g] holds the offsets (u, v) of k = 16 (kb0 + j) + 4 g = u * cy + v.
+// This lane's part of block j of 16 k of the mixed operand of an item: inter_s[n, 16 j + 4 g + i], i < 4.
+// With a channelled y, lut[j * 4 + g] holds the offsets (u, v) of k = 16 j + 4 g = u * cy + v.
 template <bool YC>
 __device__ __forceinline__ floatx4 uvt_mix_block(const UvtTerms<YC>& T, int j, const int2* lut) {
   floatx4 bf = {0.f, 0.f, 0.f, 0.f};
@@ -191,15 +195,15 @@ __device__ __forceinline__ floatx4 uvt_mix_tail(const UvtDev& a, const UvtTables
   return bf;
 }
 
-// WB: blocks of 16 output channels per wavefront.  Every item covers exactly kUvtKbi blocks of 16 k (the packed
-// weights and the staged rows are zero-padded to whole items), so the body is straight-line code.
-// Software pipeline, by hand, because a workgroup whose rows fill the LDS leaves one wavefront per SIMD: while the
-// matrix instructions of block j of the current item run, the vector ALUs mix block j of the next item; the weight
-// fragments of the next item are requested before the current item starts (past the last item: the last item again).
-// Everything an item needs besides its operands is wave-uniform (scalar registers), and the operand reads use
-// immediate offsets: about 100 vector instructions per item next to its 16 * WB matrix instructions of 32 cycles.
+// WB: blocks of 16 output channels per wavefront.  k is padded to whole multiples of kUvtKbi blocks of 16 (zero
+// weights, zero rows), so the ring of weight fragments turns in straight-line code.
+// While the matrix instructions of block j run, the vector ALUs mix block j + 1; the weight fragments of block j + 4
+// (of the next item past the end of this one) are requested as soon as block j's are consumed.  Everything an item
+// needs besides its operands is wave-uniform (scalar registers).  A wavefront issues one instruction every four
+// cycles, a matrix instruction keeps its pipeline busy for 32: with 4 WB matrix instructions per block next to
+// about 50 vector and LDS instructions, two wavefronts per SIMD keep the matrix pipeline fed when WB >= 2.
 template <bool YC, int WB>
-__global__ void __launch_bounds__(256) uvt_apply_kernel(const UvtDev a) {
+__global__ void __launch_bounds__(kUvtMaxGroups* kWave) uvt_apply_kernel(const UvtDev a) {
   constexpr int KBI = kUvtKbi;
   extern __shared__ __align__(16) unsigned char smem[];
   const int sb_count = 1 << a.sb_log2;
@@ -222,46 +226,66 @@ __global__ void __launch_bounds__(256) uvt_apply_kernel(const UvtDev a) {
   __syncthreads();
 
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), r = lane & 15, g = lane >> 4;
-  const int sb = wave & (sb_count - 1), wg = wave >> a.sb_log2, wgroups = 4 >> a.sb_log2;
-  const int wb0 = (blockIdx.y * wgroups + wg) * WB;
+  const int sb = wave & (sb_count - 1), rest = wave >> a.sb_log2;
+  const int wg = rest & (a.wgroups - 1), ig = rest / a.wgroups;
+  const int wb0 = (blockIdx.y * a.wgroups + wg) * WB;
   if (wb0 * 16 >= a.cout) return;
+  int j = a.group_ptr[ig];
+  const int j_end = a.group_ptr[ig + 1];
+  if (j >= j_end) return;
   const int64_t n = nb0 + sb * 16 + r;
   const float* xl = xs + (size_t)(sb * 16 + r) * a.px;
   const float* yl = ys + (size_t)(sb * 16 + r) * a.py;
   const int2* lut_g = lut_all + g;
 
-  floatx4 acc[WB], A0[WB][KBI], A1[WB][KBI], B0[KBI], B1[KBI];
-  auto load_a = [&](const cgtp_uvt_item& it, floatx4 (&A)[WB][KBI]) __attribute__((always_inline)) {
+  const int64_t kstride = (int64_t)a.wbp * 256;
+  auto wbase_of = [&](const cgtp_uvt_item& it) __attribute__((always_inline)) {
     // wave-uniform base of the item's fragments; a lane adds 16 bytes times its index
-    const float* base = a.wp + ((int64_t)(it.p * a.kblocks + it.kb0) * a.wbp + wb0) * 256;
-#pragma unroll
-    for (int j = 0; j < KBI; ++j) {
-      const float* bj = base + (int64_t)j * a.wbp * 256;
-#pragma unroll
-      for (int wb = 0; wb < WB; ++wb) A[wb][j] = *reinterpret_cast<const floatx4*>(bj + wb * 256 + lane * 4);
-    }
+    return a.wp + ((int64_t)it.p * a.kblocks * a.wbp + wb0) * 256 + lane * 4;
   };
-  auto mix_item = [&](const cgtp_uvt_item& it, const UvtTerms<YC>& T, int j) __attribute__((always_inline)) {
-    floatx4 b = uvt_mix_block<YC>(T, j, lut_g + it.kb0 * 4);
-    if (it.t1 - it.t0 > kUvtTerms) b += uvt_mix_tail<YC>(a, tab, it, j, xl, yl, g, lut_g + it.kb0 * 4);
-    return b;
+  floatx4 acc[WB], A[KBI][WB];
+  auto load_a = [&](const float* base, int kb, floatx4 (&Aj)[WB]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int wb = 0; wb < WB; ++wb) Aj[wb] = *reinterpret_cast<const floatx4*>(base + kb * kstride + wb * 256);
   };
-  auto process = [&](const cgtp_uvt_item& it, floatx4 (&Ac)[WB][KBI], floatx4 (&Bc)[KBI], floatx4 (&An)[WB][KBI],
-                     floatx4 (&Bn)[KBI], const cgtp_uvt_item& nx) __attribute__((always_inline)) {
-    load_a(nx, An);
+#pragma unroll
+  for (int wb = 0; wb < WB; ++wb) acc[wb] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  cgtp_uvt_item it = uvt_item_at(tab, j);
+  const float* base = wbase_of(it);
+#pragma unroll
+  for (int jj = 0; jj < KBI; ++jj) load_a(base, jj, A[jj]);
+  while (j < j_end) {
+    const bool more = j + 1 < j_end;
+    const cgtp_uvt_item it2 = uvt_item_at(tab, more ? j + 1 : j);
+    const float* base2 = wbase_of(it2);
+    UvtTerms<YC> T;
+    uvt_terms<YC>(a, tab, it, xl, yl, zeros, g, T);
+    const bool tail = it.t1 - it.t0 > kUvtTerms;
+    auto mix = [&](int kb) __attribute__((always_inline)) {
+      floatx4 b = uvt_mix_block<YC>(T, kb, lut_g);
+      if (tail) b += uvt_mix_tail<YC>(a, tab, it, kb, xl, yl, g, lut_g);
+      return b;
+    };
     const bool first = it.flags & kUvtFirst;
 #pragma unroll
     for (int wb = 0; wb < WB; ++wb) acc[wb] = first ? floatx4{0.f, 0.f, 0.f, 0.f} : acc[wb];
-    UvtTerms<YC> T;
-    uvt_terms<YC>(a, tab, nx, xl, yl, zeros, g, T);
+    floatx4 Bc = mix(0);
+    for (int kb = 0; kb < a.kblocks; kb += KBI) {
+      const bool wrap = kb + KBI >= a.kblocks;        // the fragments requested now belong to the next item
+      const float* wnext = wrap ? base2 : base;
+      const int kbn = wrap ? 0 : kb + KBI;
 #pragma unroll
-    for (int j = 0; j < KBI; ++j) {
+      for (int jj = 0; jj < KBI; ++jj) {
+        const floatx4 Bn = mix((jj + 1 < KBI || !wrap) ? kb + jj + 1 : kb + jj);
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int wb = 0; wb < WB; ++wb)
-          acc[wb] = __builtin_amdgcn_mfma_f32_16x16x4f32(Ac[wb][j][i], Bc[j][i], acc[wb], 0, 0, 0);
-      Bn[j] = mix_item(nx, T, j);
+          for (int wb = 0; wb < WB; ++wb)
+            acc[wb] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[jj][wb][i], Bc[i], acc[wb], 0, 0, 0);
+        load_a(wnext, kbn + jj, A[jj]);
+        Bc = Bn;
+      }
     }
     if (it.flags & kUvtLast) {
       // accumulator layout: lane (n = r, g) holds output channels 16 wb + 4 g .. + 3 of sample n
@@ -274,25 +298,9 @@ __global__ void __launch_bounds__(256) uvt_apply_kernel(const UvtDev a) {
         }
       }
     }
-  };
-
-  cgtp_uvt_item it = uvt_item_at(tab, 0);
-  load_a(it, A0);
-  {
-    UvtTerms<YC> T;
-    uvt_terms<YC>(a, tab, it, xl, yl, zeros, g, T);
-#pragma unroll
-    for (int j = 0; j < KBI; ++j) B0[j] = mix_item(it, T, j);
-  }
-#pragma unroll
-  for (int wb = 0; wb < WB; ++wb) acc[wb] = floatx4{0.f, 0.f, 0.f, 0.f};
-  for (int j = 0; j < a.n_items; j += 2) {
-    const cgtp_uvt_item it1 = uvt_item_at(tab, min(j + 1, a.n_items - 1));
-    process(it, A0, B0, A1, B1, it1);
-    if (j + 1 >= a.n_items) break;
-    const cgtp_uvt_item it2 = uvt_item_at(tab, min(j + 2, a.n_items - 1));
-    process(it1, A1, B1, A0, B0, it2);
+    ++j;
     it = it2;
+    base = base2;
   }
 }
 
@@ -680,68 +688,81 @@ __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGy
 }
 
 struct UvtPlan {
-  int sb_log2, wb, kbi, yc;
+  int wb, kbi, yc;
   int64_t lds;
   dim3 grid;
+  unsigned threads;
   UvtDev dev;
 };
 
 static inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
+static inline int pow2_floor(int v) { int p = 1; while (p * 2 <= v) p *= 2; return p; }
+static inline int pow2_ceil(int v) { int p = 1; while (p < v) p *= 2; return p; }
 
-// Launch shape from the extents alone: LDS pitches, sample blocks per workgroup, channel blocks per wavefront and the
-// chunk length the item list has to be cut for.
-static int uvt_shape(int64_t n_rows, int dx, int dy, int cx, int cy, int cout, UvtPlan* plan) {
-  if (n_rows < 0 || dx <= 0 || dy <= 0 || cx <= 0 || cy < 0 || cout <= 0) return CGTP_ERR_SHAPE;
+// Launch shape from the extents alone: LDS pitches, channel blocks per wavefront, and how a workgroup's (up to) eight
+// wavefronts are spent: on groups of output rows first (they share everything staged and repeat no arithmetic), on
+// blocks of output channels (they repeat the mixing), on further blocks of 16 samples when LDS and batch allow.
+static int uvt_shape(int64_t n_rows, int dx, int dy, int dout, int cx, int cy, int cout, UvtPlan* plan) {
+  if (n_rows < 0 || dx <= 0 || dy <= 0 || dout <= 0 || cx <= 0 || cy < 0 || cout <= 0) return CGTP_ERR_SHAPE;
   if (cx % 4 || cout % 4 || cy % 4) return CGTP_ERR_SHAPE;
   const bool yc = cy > 0;
   if (yc && ((int64_t)cx * cy) % 16) return CGTP_ERR_SHAPE;
   UvtDev& d = plan->dev;
-  d.n_rows = n_rows; d.dx = dx; d.dy = dy; d.cx = cx; d.cy = cy; d.cout = cout;
+  d.n_rows = n_rows; d.dx = dx; d.dy = dy; d.dout = dout; d.cx = cx; d.cy = cy; d.cout = cout;
   const int64_t K = yc ? (int64_t)cx * cy : cx;
-  d.kblocks = round_up((int)((K + 15) / 16), kUvtKbi);   // whole items: the tail is zero weights
+  if (K > (1 << 24)) return CGTP_ERR_SHAPE;
+  d.kblocks = round_up((int)((K + 15) / 16), kUvtKbi);   // whole turns of the fragment ring: the tail is zero weights
   d.kx = yc ? cx : d.kblocks * 16;
   d.px = dx * d.kx + 4;
   d.py = yc ? dy * cy + 4 : (dy | 1);
   const int wblocks = (cout + 15) / 16;
   d.wbp = round_up(wblocks, 4);
+  const int wb = wblocks >= 4 ? 4 : wblocks >= 2 ? 2 : 1;
+  const int need = (wblocks + wb - 1) / wb;             // wavefronts (or workgroups) that cover the output channels
+  int wgroups = need >= 2 ? 2 : 1;
+  int igroups = pow2_floor(dout < kUvtMaxGroups / wgroups ? dout : kUvtMaxGroups / wgroups);
+  while (wgroups < pow2_ceil(need) && wgroups * 2 * igroups <= kUvtMaxGroups) wgroups *= 2;
+  d.zero_floats = yc ? round_up((cx > cy + 4 ? cx : cy + 4) + 4, 4) : d.kblocks * 16 + 16;
   const int64_t per_block = (int64_t)16 * (d.px + d.py) * 4;   // LDS bytes of one 16-sample block
-  if (per_block > kLdsBytes - kUvtTableRoom) return CGTP_ERR_LDS;
-  // sample blocks per workgroup: as many as keep two workgroups per compute unit, else as many as fit; fewer when the
-  // batch is too small to fill the chip with such workgroups
-  int sb_log2 = 2;
-  while (sb_log2 > 0 && (per_block << sb_log2) > kLdsBytes / 2 - kUvtTableRoom) --sb_log2;
+  const int64_t fixed = (yc ? (int64_t)d.kblocks * 32 : 0) + (int64_t)d.zero_floats * 4 + 32;
+  if (per_block + fixed > kLdsBytes - kUvtTableRoom) return CGTP_ERR_LDS;
+  // further sample blocks: while wavefronts are left, two workgroups still fit a compute unit, and the batch is large
+  // enough to fill the chip with such workgroups
+  int sb_log2 = 0;
   const int64_t blocks16 = (n_rows + 15) / 16;
-  while (sb_log2 > 0 && (blocks16 >> sb_log2) < 512) --sb_log2;
-  d.sb_log2 = sb_log2;
-  const int wgroups = 4 >> sb_log2;
-  const int need = (wblocks + wgroups - 1) / wgroups;
-  const int wb = need >= 4 ? 4 : need >= 2 ? 2 : 1;
-  plan->sb_log2 = sb_log2; plan->wb = wb; plan->kbi = kUvtKbi; plan->yc = yc;
-  plan->lds = per_block << sb_log2;
-  plan->grid = dim3((unsigned)((blocks16 + (1 << sb_log2) - 1) >> sb_log2),
-                    (unsigned)((wblocks + wgroups * wb - 1) / (wgroups * wb)));
+  while ((wgroups * igroups) << (sb_log2 + 1) <= kUvtMaxGroups &&
+         (per_block << (sb_log2 + 1)) + fixed <= kLdsBytes / 2 - kUvtTableRoom && (blocks16 >> (sb_log2 + 1)) >= 512)
+    ++sb_log2;
+  d.sb_log2 = sb_log2; d.wgroups = wgroups; d.igroups = igroups;
+  plan->wb = wb; plan->kbi = kUvtKbi; plan->yc = yc;
+  plan->lds = (per_block << sb_log2) + fixed;
+  plan->threads = (unsigned)((wgroups * igroups) << sb_log2) * kWave;
+  plan->grid = dim3((unsigned)((blocks16 + (1 << sb_log2) - 1) >> sb_log2), (unsigned)((need + wgroups - 1) / wgroups));
   return CGTP_OK;
 }
 
 static int uvt_plan(const cgtp_uvt_args* a, UvtPlan* plan) {
   if (!a) return CGTP_ERR_NULL;
   if (a->dtype != CGTP_F32) return CGTP_ERR_DTYPE;
-  if (a->n_items < 0 || a->n_terms < 0 || a->dout <= 0) return CGTP_ERR_SHAPE;
-  const int st = uvt_shape(a->n_rows, a->dx, a->dy, a->cx, a->cy, a->cout, plan);
+  if (a->n_items < 0 || a->n_terms < 0) return CGTP_ERR_SHAPE;
+  const int st = uvt_shape(a->n_rows, a->dx, a->dy, a->dout, a->cx, a->cy, a->cout, plan);
   if (st != CGTP_OK) return st;
-  if (a->kbi != plan->kbi) return CGTP_ERR_SHAPE;   // the item list must be cut for this launch shape: cgtp_uvt_chunk()
+  UvtDev& d = plan->dev;
+  // the item list must be cut for this launch shape: cgtp_uvt_chunk(), cgtp_uvt_item_groups()
+  if (a->kbi != plan->kbi || a->n_groups != d.igroups) return CGTP_ERR_SHAPE;
+  if (a->group_ptr[0] != 0 || a->group_ptr[d.igroups] != a->n_items) return CGTP_ERR_SHAPE;
+  for (int i = 0; i < d.igroups; ++i)
+    if (a->group_ptr[i] > a->group_ptr[i + 1]) return CGTP_ERR_SHAPE;
   if (!a->x || !a->y || !a->wp || !a->out || (a->n_items && (!a->items || !a->term_a || !a->term_b || !a->term_c)))
     return CGTP_ERR_NULL;
   const uintptr_t al = reinterpret_cast<uintptr_t>(a->x) | reinterpret_cast<uintptr_t>(a->wp) |
                        reinterpret_cast<uintptr_t>(a->out) | (a->cy > 0 ? reinterpret_cast<uintptr_t>(a->y) : 0);
   if (al & 15u) return CGTP_ERR_ALIGN;
-  UvtDev& d = plan->dev;
   d.x = (const float*)a->x; d.y = (const float*)a->y; d.wp = (const float*)a->wp; d.out = (float*)a->out;
   d.items = a->items; d.ta = a->term_a; d.tb = a->term_b; d.tc = (const float*)a->term_c;
-  d.n_items = a->n_items; d.n_terms = a->n_terms; d.dout = a->dout;
-  d.zero_floats = a->cy > 0 ? round_up((a->cx > a->cy + 4 ? a->cx : a->cy + 4) + 4, 4) : kUvtKbi * 16 + 16;
-  plan->lds += ((int64_t)a->n_items * 32 + (int64_t)a->n_terms * 12 + 15) / 16 * 16 +
-               (a->cy > 0 ? (int64_t)d.kblocks * 32 : 0) + (int64_t)d.zero_floats * 4 + 16;
+  d.n_items = a->n_items; d.n_terms = a->n_terms;
+  for (int i = 0; i <= kUvtMaxGroups; ++i) d.group_ptr[i] = i <= d.igroups ? a->group_ptr[i] : a->n_items;
+  plan->lds += ((int64_t)a->n_items * 32 + (int64_t)a->n_terms * 12 + 15) / 16 * 16;
   if (plan->lds > kLdsBytes) return CGTP_ERR_LDS;
   return CGTP_OK;
 }
@@ -771,10 +792,16 @@ int cgtp_uvt_pack_weights(const void* w, void* packed, int32_t n_paths, int64_t 
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 
-int cgtp_uvt_chunk(int64_t n_rows, int32_t dx, int32_t dy, int32_t cx, int32_t cy, int32_t cout) {
+int cgtp_uvt_chunk(int64_t n_rows, int32_t dx, int32_t dy, int32_t dout, int32_t cx, int32_t cy, int32_t cout) {
   UvtPlan plan;
-  const int st = uvt_shape(n_rows, dx, dy, cx, cy, cout, &plan);
+  const int st = uvt_shape(n_rows, dx, dy, dout, cx, cy, cout, &plan);
   return st == CGTP_OK ? plan.kbi : -st;
+}
+
+int cgtp_uvt_item_groups(int64_t n_rows, int32_t dx, int32_t dy, int32_t dout, int32_t cx, int32_t cy, int32_t cout) {
+  UvtPlan plan;
+  const int st = uvt_shape(n_rows, dx, dy, dout, cx, cy, cout, &plan);
+  return st == CGTP_OK ? plan.dev.igroups : -st;
 }
 
 int cgtp_uvt_validate(const cgtp_uvt_args* a) {
@@ -796,7 +823,7 @@ int cgtp_uvt_apply(const cgtp_uvt_args* a, void* stream) {
   if (plan.lds > 48 * 1024 &&
       hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds) != hipSuccess)
     return CGTP_ERR_LDS;
-  hipLaunchKernelGGL(fn, plan.grid, dim3(256), (size_t)plan.lds, (hipStream_t)stream, plan.dev);
+  hipLaunchKernelGGL(fn, plan.grid, dim3(plan.threads), (size_t)plan.lds, (hipStream_t)stream, plan.dev);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 

@@ -26,48 +26,55 @@ MAX_TERMS = 8      # terms of a segment the weight-gradient kernel holds in regi
 
 
 class _Walk:
-    """Item list of one role of one table, cut for ``kblocks`` blocks of 16 contracted channels in chunks of ``kbi``."""
+    """Item list of one role of one table: one item per segment (weight path, output row), the items of a row
+    consecutive, the rows dealt to ``n_groups`` groups of about equal numbers of items (the wavefronts of a workgroup
+    take one group each)."""
 
-    def __init__(self, out_idx, a_idx, b_idx, p_idx, coef, n_out: int, kblocks: int, kbi: int, device):
+    def __init__(self, out_idx, a_idx, b_idx, p_idx, coef, n_out: int, n_groups: int, device):
         order = np.lexsort([b_idx, a_idx, p_idx, out_idx])
         out_idx, a_idx, b_idx, p_idx = (np.asarray(v)[order] for v in (out_idx, a_idx, b_idx, p_idx))
         coef = np.asarray(coef, dtype=np.float64)[order]
-        items = []
+        rows = []
         t, n_terms = 0, out_idx.shape[0]
         for row in range(n_out):
-            first = len(items)
+            items = []
             while t < n_terms and out_idx[t] == row:
                 t1 = t
                 while t1 < n_terms and out_idx[t1] == row and p_idx[t1] == p_idx[t]:
                     t1 += 1
-                for kb0 in range(0, kblocks, kbi):
-                    items.append([int(p_idx[t]), kb0, kbi, t, t1, row, 0, 0])
+                items.append([int(p_idx[t]), 0, 0, t, t1, row, 0, 0])
                 t = t1
-            if len(items) == first:                       # a row without terms is written as zeros
-                items.append([0, 0, kbi, 0, 0, row, 0, 0])
-            items[first][6] |= FIRST
+            if not items:                                  # a row without terms is written as zeros
+                items.append([0, 0, 0, 0, 0, row, 0, 0])
+            items[0][6] |= FIRST
             items[-1][6] |= LAST
-        self.n_items = len(items)
-        self.kbi = kbi
-        self.items = torch.tensor(items, dtype=torch.int32).to(device)
+            rows.append(items)
+        # longest rows first, each to the group with the fewest items so far
+        groups = [[] for _ in range(n_groups)]
+        for items in sorted(rows, key=len, reverse=True):
+            min(groups, key=len).extend(items)
+        flat = [it for grp in groups for it in grp]
+        self.n_items = len(flat)
+        self.group_ptr = np.cumsum([0] + [len(grp) for grp in groups]).tolist()
+        self.items = torch.tensor(flat, dtype=torch.int32).reshape(-1, 8).to(device)
         self.term_a = torch.from_numpy(a_idx.astype(np.int32)).to(device)
         self.term_b = torch.from_numpy(b_idx.astype(np.int32)).to(device)
         self.term_c = torch.from_numpy(coef.astype(np.float32)).to(device)
 
 
-def _walk(tp_info, role: str, kblocks: int, kbi: int, device) -> _Walk:
+def _walk(tp_info, role: str, n_groups: int, device) -> _Walk:
     def build():
         c = kernels.coo_of(tp_info)
         if role == "out":        # rows of the first operand, rows of the second operand
-            return _Walk(c.M, c.M1, c.M2, c.p, c.coef, c.DO, kblocks, kbi, device)
+            return _Walk(c.M, c.M1, c.M2, c.p, c.coef, c.DO, n_groups, device)
         if role == "in1":        # first operand of the launch = grad_out, second = input2
-            return _Walk(c.M1, c.M, c.M2, c.p, c.coef, c.D1, kblocks, kbi, device)
+            return _Walk(c.M1, c.M, c.M2, c.p, c.coef, c.D1, n_groups, device)
         if role == "in1_uvw":    # first operand of the launch = input2, second = grad_out
-            return _Walk(c.M1, c.M2, c.M, c.p, c.coef, c.D1, kblocks, kbi, device)
+            return _Walk(c.M1, c.M2, c.M, c.p, c.coef, c.D1, n_groups, device)
         if role == "in2_uvw":    # first operand of the launch = grad_out, second = input1
-            return _Walk(c.M2, c.M, c.M1, c.p, c.coef, c.D2, kblocks, kbi, device)
+            return _Walk(c.M2, c.M, c.M1, c.p, c.coef, c.D2, n_groups, device)
         raise ValueError(role)
-    return kernels.cached(tp_info.info_Mij_fwd.scale, ("uvt_walk", role, kblocks, kbi, str(device)), build)
+    return kernels.cached(tp_info.info_Mij_fwd.scale, ("uvt_walk", role, n_groups, str(device)), build)
 
 
 class _PathWalk:
@@ -170,10 +177,10 @@ def grad_y(x: Tensor, g: Tensor, wp: Tensor, tp_info, dy: int) -> Tensor:
     return gy
 
 
-def chunk_of(n_rows: int, dx: int, dy: int, cx: int, cy: int, cout: int) -> int:
-    """Chunk length (blocks of 16 contracted channels per item) of a launch with these extents; <= 0: the kernels do
-    not take them (channel counts not multiples of 4, rows of 16 samples beyond the LDS)."""
-    return int(_lib.lib.cgtp_uvt_chunk(n_rows, dx, dy, cx, cy, cout))
+def chunk_of(n_rows: int, dx: int, dy: int, dout: int, cx: int, cy: int, cout: int) -> int:
+    """Blocks of 16 contracted channels a launch with these extents pads to; <= 0: the kernels do not take them
+    (channel counts not multiples of 4, rows of 16 samples beyond the LDS)."""
+    return int(_lib.lib.cgtp_uvt_chunk(n_rows, dx, dy, dout, cx, cy, cout))
 
 
 def pack(w: Tensor, n_paths: int, k: int, cout: int, stride_p: int, stride_k: int, stride_c: int) -> Tensor:
@@ -190,11 +197,11 @@ def apply(x: Tensor, y: Tensor, wp: Tensor, tp_info, role: str, dout: int, cout:
     dy = y.shape[1]
     cy = y.shape[2] if y.ndim == 3 else 0
     k = cx * cy if cy else cx
-    kbi = chunk_of(n, dx, dy, cx, cy, cout)
+    kbi = chunk_of(n, dx, dy, dout, cx, cy, cout)
     if kbi <= 0:
         raise _lib.CgtpError(f"cgtp_uvt_apply does not take these extents (status {-kbi})")
-    kblocks = ((k + 15) // 16 + kbi - 1) // kbi * kbi        # whole items; the tail of k is zero weights
-    walk = _walk(tp_info, role, kblocks, kbi, x.device)
+    n_groups = int(_lib.lib.cgtp_uvt_item_groups(n, dx, dy, dout, cx, cy, cout))
+    walk = _walk(tp_info, role, n_groups, x.device)
     out = torch.empty((n, dout, cout), dtype=x.dtype, device=x.device)
     if n == 0:
         return out
@@ -205,6 +212,9 @@ def apply(x: Tensor, y: Tensor, wp: Tensor, tp_info, role: str, dout: int, cout:
     a.n_rows, a.n_items, a.n_terms = n, walk.n_items, walk.term_a.shape[0]
     a.dx, a.dy, a.dout, a.cx, a.cy, a.cout = dx, dy, dout, cx, cy, cout
     a.kbi, a.dtype = kbi, _lib.F32
+    a.n_groups = n_groups
+    for i, v in enumerate(walk.group_ptr):
+        a.group_ptr[i] = v
     _lib.check(_lib.lib.cgtp_uvt_apply(C.byref(a), _lib.stream_ptr(x.device)), "cgtp_uvt_apply")
     return out
 
@@ -261,7 +271,7 @@ def u1v_supported(x: Tensor, y: Tensor, w: Tensor, tp_info) -> bool:
     c = _coo(tp_info)
     _, u, wc = w.shape
     n = x.shape[0]
-    return (chunk_of(n, c.D1, c.D2, u, 0, wc) > 0 and chunk_of(n, c.DO, c.D2, wc, 0, u) > 0
+    return (chunk_of(n, c.D1, c.D2, c.DO, u, 0, wc) > 0 and chunk_of(n, c.DO, c.D2, c.D1, wc, 0, u) > 0
             and grad_y_supported(n, c.D1, c.D2, u, wc, tp_info) and x.data_ptr() % 16 == 0)
 
 
@@ -318,8 +328,8 @@ def uvw_supported(x: Tensor, y: Tensor, w: Tensor, tp_info) -> bool:
     c = _coo(tp_info)
     _, u, v, wc = w.shape
     n = x.shape[0]
-    return (chunk_of(n, c.D1, c.D2, u, v, wc) > 0 and chunk_of(n, c.D2, c.DO, v, wc, u) > 0
-            and chunk_of(n, c.DO, c.D1, wc, u, v) > 0 and x.data_ptr() % 16 == 0 and y.data_ptr() % 16 == 0)
+    return (chunk_of(n, c.D1, c.D2, c.DO, u, v, wc) > 0 and chunk_of(n, c.D2, c.DO, c.D1, v, wc, u) > 0
+            and chunk_of(n, c.DO, c.D1, c.D2, wc, u, v) > 0 and x.data_ptr() % 16 == 0 and y.data_ptr() % 16 == 0)
 
 
 def uvw(x: Tensor, y: Tensor, w: Tensor, tp_info) -> Tensor:

@@ -41,7 +41,8 @@ int cgtp_version(void);
  * cgo, JNI) can check itself: which = CGTP_LAYOUT_*; writes sizeof(struct) followed by the byte offset of every field
  * in declaration order to out[0 .. capacity) and returns how many numbers the full description has (-1: bad id). */
 enum { CGTP_LAYOUT_OPERAND = 0, CGTP_LAYOUT_TRI_ARGS = 1, CGTP_LAYOUT_GEN_OPERAND = 2, CGTP_LAYOUT_GEN_ARGS = 3,
-       CGTP_LAYOUT_UVU_ARGS = 4, CGTP_LAYOUT_UVT_ITEM = 5, CGTP_LAYOUT_UVT_ARGS = 6 };
+       CGTP_LAYOUT_UVU_ARGS = 4, CGTP_LAYOUT_UVT_ITEM = 5, CGTP_LAYOUT_UVT_ARGS = 6, CGTP_LAYOUT_UVT_GW_ARGS = 7,
+       CGTP_LAYOUT_UVT_GY_ARGS = 8 };
 int cgtp_abi_layout(int which, int64_t* out, int capacity);
 
 /* ---- generic sparse trilinear contraction -------------------------------------------------------------
@@ -301,11 +302,13 @@ int cgtp_uv_grad_w(int cfg, const void* x, const void* y, const void* g, void* g
  * (equitorch/nn/functional/tensor_products.py:95-101: outer, then vecmat over the flattened (u, v) axis) and, with
  * the rows' roles exchanged and the weight packed transposed, for the grad-input products of their backward passes
  * (tensor_product_1vu / tensor_product_uvw with permuted weights, linears.py:290-293, tensor_products.py:126-150).
- * Shared weights only.  The caller supplies the walk as a flat list of items ordered by output row: an item is one
- * segment restricted to the `nkb` = cgtp_uvt_chunk() blocks of 16 consecutive k starting at block kb0 (K is padded
- * with zero weights to whole items), with its terms t0..t1 in (term_a = row of x, term_b = row of y, term_c =
- * coefficient); flags: 1 = first item of its output row, 2 = last.  Every output row needs at least one item (t0 = t1
- * for a row without terms: it is written as zeros).  The chunk length must also be passed as `kbi`.
+ * Shared weights only.  The caller supplies the walk as a flat list of items, one per segment, with the segment's
+ * terms t0..t1 in (term_a = row of x, term_b = row of y, term_c = coefficient); flags: 1 = first item of its output
+ * row, 2 = last (kb0, nkb: 0, unused).  The items of an output row are consecutive, and every output row needs at
+ * least one item (t0 = t1 for a row without terms: it is written as zeros).  The wavefronts of a workgroup split the
+ * output rows: the list is ordered in cgtp_uvt_item_groups() groups of whole rows, group i being items group_ptr[i] ..
+ * group_ptr[i + 1] (groups of about equal length keep the wavefronts equally busy; empty groups are allowed).
+ * cgtp_uvt_chunk() (blocks of 16 k the kernels pad K to with zero weights) must be passed as `kbi`.
  * x (n_rows, dx, cx), y (n_rows, dy) or (n_rows, dy, cy), out (n_rows, dout, cout), all fp32 and contiguous; cx, cy,
  * cout multiples of 4, cx * cy a multiple of 16 when cy > 0; 16-byte aligned pointers; the rows of 16 samples must
  * fit the LDS (CGTP_ERR_LDS otherwise).  wp = cgtp_uvt_pack_weights(W): W (n_paths, K, cout) read through element
@@ -333,13 +336,17 @@ typedef struct cgtp_uvt_args {
   int32_t dtype;                /* CGTP_F32 */
   int32_t n_terms;              /* entries of term_a / term_b / term_c (the tables are copied to LDS: 32 B per item +
                                    12 B per term must fit next to the samples' rows, CGTP_ERR_LDS otherwise) */
+  int32_t n_groups;             /* cgtp_uvt_item_groups() */
+  int32_t group_ptr[9];         /* n_groups + 1 item offsets, group_ptr[0] = 0, group_ptr[n_groups] = n_items */
 } cgtp_uvt_args;
 
 int64_t cgtp_uvt_packed_elems(int32_t n_paths, int64_t K, int32_t cout);
 int cgtp_uvt_pack_weights(const void* w, void* packed, int32_t n_paths, int64_t K, int32_t cout, int64_t stride_p,
                           int64_t stride_k, int64_t stride_c, int32_t dtype, void* stream);
-/* Blocks of 16 k per item for these extents, or -status when the kernels do not take them.  Host only. */
-int cgtp_uvt_chunk(int64_t n_rows, int32_t dx, int32_t dy, int32_t cx, int32_t cy, int32_t cout);
+/* Launch shape for these extents, or -status when the kernels do not take them: blocks of 16 k that K is padded to
+ * a multiple of; groups of output rows the item list has to come in.  Host only. */
+int cgtp_uvt_chunk(int64_t n_rows, int32_t dx, int32_t dy, int32_t dout, int32_t cx, int32_t cy, int32_t cout);
+int cgtp_uvt_item_groups(int64_t n_rows, int32_t dx, int32_t dy, int32_t dout, int32_t cx, int32_t cy, int32_t cout);
 int cgtp_uvt_validate(const cgtp_uvt_args* args);
 int cgtp_uvt_apply(const cgtp_uvt_args* args, void* stream);
 

@@ -25,6 +25,8 @@ U1V_CASES = [  # irreps (out, in1, in2), C_in, C_out, N, module options
     ((_sh(2),) * 3, 32, 36, 515, {"channel_norm": True}),       # C_out = 2 blocks + 4
     (("1o+2e+1e", "0e+1o+2e", "0e+1o"), 48, 40, 200, {}),       # irreps without a compiled table
     (("0e+1e+2e+3e", "0e+1e+2e", "0e+1e+2e"), 16, 16, 64, {}),
+    (("0e", _sh(2), _sh(2)), 32, 64, 17000, {}),                # one output row: wavefronts spent on sample blocks
+    (("0e+1o", _sh(1), _sh(1)), 16, 256, 530, {}),              # output channels over two workgroups
 ]
 
 
