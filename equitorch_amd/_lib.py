@@ -57,7 +57,8 @@ class UvuArgs(C.Structure):
                 ("out", C.c_void_p),
                 ("grad_out", C.c_void_p), ("grad_x", C.c_void_p), ("grad_y", C.c_void_p),
                 ("grad_w", C.c_void_p), ("workspace", C.c_void_p), ("x_gather", C.c_void_p),
-                ("y_channels", C.c_int32), ("reserved_", C.c_int32), ("path_scale", C.c_void_p)]
+                ("y_channels", C.c_int32), ("reserved_", C.c_int32), ("path_scale", C.c_void_p),
+                ("radial_h", C.c_void_p), ("radial_w", C.c_void_p), ("radial_r", C.c_int32), ("reserved2_", C.c_int32)]
 
 
 class UvtItem(C.Structure):
@@ -118,6 +119,10 @@ def _load():
     lib.cgtp_uvu_describe.restype = C.c_uint64
     lib.cgtp_uvu_describe.argtypes = [C.c_int, C.POINTER(C.c_int32)]
     lib.cgtp_uvu_sh_degree.argtypes = [C.c_int]
+    lib.cgtp_uvu_radial_supported.argtypes = [C.c_int]
+    lib.cgtp_uvu_radial_grad_workspace_bytes.restype = C.c_int64
+    lib.cgtp_uvu_radial_grad_workspace_bytes.argtypes = [C.c_int64, C.c_int32, C.c_int32]
+    lib.cgtp_uvu_radial_grad.argtypes = [C.c_void_p] * 6 + [C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
     lib.cgtp_uvu_table.argtypes = [C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_int32)]
     lib.cgtp_uv_table.argtypes = [C.c_int, C.POINTER(C.c_int32), C.POINTER(C.c_float), C.POINTER(C.c_int32)]
     lib.cgtp_uvu_validate.argtypes = [C.POINTER(UvuArgs), C.c_int]

@@ -28,6 +28,10 @@ struct UvuDev {
   int C, lpe_log2, w_shared, pos_per_wave;
   int y_vec;  // segment mode: y holds edge vectors (kYUnitVector / kYRawVector) instead of harmonics
   const T* ps;  // optional factor of every weight path (the caller's table = compiled table x ps[p]); nullptr = ones
+  // weights produced in the kernel: w[e, p, c] = sum_r rh[e, r] * rw[r, p, c] (segment mode, fp32, C = 64)
+  const T* rh;   // (n_rows, R)
+  const T* rw;   // (R, P, C)
+  int R;
 };
 
 // Segment mode: which range of the sorted edge list a wavefront takes.  Workgroups are dispatched to the 8 XCDs
@@ -75,6 +79,17 @@ struct UvuBigEntry {
   void (*fwd_yc)(const UvuDev<float>);
   void (*bwd_yc[2])(const UvuDev<float>, int64_t);
 };
+// Segment-mode kernels that form the per-edge weights from per-edge features and a shared matrix (uvu_radial.hip);
+// [0]: second operand given as harmonics, [1]: as edge vectors (nullptr where the config has no such form).
+struct UvuRadialEntry {
+  void (*fwd[2])(const UvuDev<float>, int64_t);
+  void (*bwd[2][2])(const UvuDev<float>, int64_t);   // [.][weight gradient written per edge]
+  int lds_floats_per_r;   // LDS floats per row of the shared matrix
+};
+const UvuRadialEntry* uvu_radial_entries(int* count);
+constexpr int kRadialMaxR = 16;
+constexpr int kRadialC = 64;
+
 const UvuBigEntry* uvu_big_entries(int* count);
 const UvuBigEntry* uvu_big_entries_scaled(int* count);  // the same kernels applying UvuDev::ps
 

@@ -584,9 +584,11 @@ static const UvuEntry<T>* make_entries(int* count) {
 const UvuEntry<float>* uvu_entries_scaled_f32(int* count);
 const UvuEntry<double>* uvu_entries_scaled_f64(int* count);
 
-#ifdef CGTP_UVU_PS_UNIT
+#if defined(CGTP_UVU_PS_UNIT)
 const UvuEntry<float>* uvu_entries_scaled_f32(int* count) { return make_entries<float, true>(count); }
 const UvuEntry<double>* uvu_entries_scaled_f64(int* count) { return make_entries<double, true>(count); }
+}  // namespace cgtp
+#elif defined(CGTP_UVU_RADIAL_UNIT)
 }  // namespace cgtp
 #else
 template <typename T>
@@ -633,8 +635,20 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
   if (a->dtype != CGTP_F32 && a->dtype != CGTP_F64) return CGTP_ERR_DTYPE;
   if (a->cfg >= n_cfg && a->dtype != CGTP_F32) return CGTP_ERR_DTYPE;
   if (a->C <= 0 || a->n_rows < 0 || a->n_seg < 0 || a->n_x_rows < 0 || a->pos_per_wave < 0) return CGTP_ERR_SHAPE;
-  if (!a->x || !a->y || !a->w) return CGTP_ERR_NULL;
+  if (!a->x || !a->y || (!a->w && !a->radial_h)) return CGTP_ERR_NULL;
   const bool seg = a->n_seg > 0;
+  if (a->radial_h) {   // weights produced in the kernel
+    int n_rad = 0;
+    const UvuRadialEntry* rad = uvu_radial_entries(&n_rad);
+    if (big || a->cfg >= n_rad || !rad[a->cfg].fwd[0]) return CGTP_ERR_CONFIG;
+    if (a->y_vec && !rad[a->cfg].fwd[1]) return CGTP_ERR_CONFIG;
+    if (a->dtype != CGTP_F32) return CGTP_ERR_DTYPE;
+    if (!seg || a->w_shared || a->path_scale || a->C != kRadialC) return CGTP_ERR_SHAPE;
+    if (a->radial_r < 4 || a->radial_r > kRadialMaxR || a->radial_r % 4) return CGTP_ERR_SHAPE;
+    if (!a->radial_w) return CGTP_ERR_NULL;
+    if ((int64_t)rad[a->cfg].lds_floats_per_r * a->radial_r * 4 > kLdsBytes) return CGTP_ERR_LDS;
+    if (!aligned16(a->radial_h) || !aligned16(a->radial_w)) return CGTP_ERR_ALIGN;
+  }
   if (a->cfg >= n_cfg && seg) return CGTP_ERR_SHAPE;  // block-wise kernels only: row mode
   if (seg && (!a->ptr || !a->seg_ids || !a->gather)) return CGTP_ERR_NULL;
   if (!seg && (a->ptr || a->perm || a->seg_ids)) return CGTP_ERR_SHAPE;
@@ -665,7 +679,7 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
     const UvuEntry<double>* tab64 = entries<double>(&n64);
     vw = backward ? tab64[a->cfg].v_bwd : tab64[a->cfg].v_fwd;
   }
-  bool vec = vw > 1 && (a->C % vw) == 0 && aligned16(a->x) && aligned16(a->w);
+  bool vec = vw > 1 && (a->C % vw) == 0 && aligned16(a->x) && (aligned16(a->w) || a->radial_h);
   if (backward) {
     vec = vec && aligned16(a->grad_out) && (!a->grad_x || aligned16(a->grad_x)) &&
           (!a->grad_w || aligned16(a->grad_w));
@@ -673,6 +687,7 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
     vec = vec && aligned16(a->out);
   }
   if (a->workspace) vec = vec && aligned16(a->workspace);
+  if (a->radial_h && !(vec && vw == 4)) return CGTP_ERR_ALIGN;   // these kernels exist for four channels per lane only
   plan->V = vec ? vw : 1;
   const int lanes = (a->C + plan->V - 1) / plan->V;
   int lg = 0;
@@ -726,6 +741,7 @@ static UvuDev<T> to_dev(const cgtp_uvu_args* a, const UvuPlan& plan) {
   d.C = a->C; d.lpe_log2 = plan.lpe_log2; d.w_shared = a->w_shared; d.pos_per_wave = plan.pos_per_wave;
   d.y_vec = a->y_vec;
   d.ps = (const T*)a->path_scale;
+  d.rh = (const T*)a->radial_h; d.rw = (const T*)a->radial_w; d.R = a->radial_r;
   return d;
 }
 
@@ -781,6 +797,20 @@ static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward,
   return launched();
 }
 
+// Segment kernels that produce the weights themselves: the shared matrix lives in LDS.
+static int launch_radial(const cgtp_uvu_args* a, const UvuDev<float>& d, const UvuPlan& plan, int backward,
+                         hipStream_t stream) {
+  int n = 0;
+  const UvuRadialEntry& e = uvu_radial_entries(&n)[a->cfg];
+  void (*fn)(const UvuDev<float>, int64_t) = backward ? e.bwd[a->y_vec ? 1 : 0][a->grad_w ? 1 : 0] : e.fwd[a->y_vec ? 1 : 0];
+  const size_t lds = (size_t)e.lds_floats_per_r * a->radial_r * sizeof(float);
+  if (lds > 48 * 1024 &&
+      hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return CGTP_ERR_LDS;
+  hipLaunchKernelGGL(fn, dim3(seg_grid(plan.n_waves)), dim3(256), lds, stream, d, plan.n_waves);
+  return CGTP_OK;
+}
+
 template <typename T>
 static int launch_fwd(const cgtp_uvu_args* a, const UvuPlan& plan, hipStream_t stream) {
   int n = 0;
@@ -789,8 +819,18 @@ static int launch_fwd(const cgtp_uvu_args* a, const UvuPlan& plan, hipStream_t s
   const int vi = plan.V > 1;
   if (a->n_seg > 0) {
     if (plan.n_waves > 0) {
-      hipLaunchKernelGGL(a->y_vec ? e.seg_fwd_vec[vi] : e.seg_fwd[vi], dim3(seg_grid(plan.n_waves)), dim3(256), 0, stream,
-                         d, plan.n_waves);
+      if constexpr (sizeof(T) == 4) {
+        if (a->radial_h) {
+          const int st = launch_radial(a, d, plan, 0, stream);
+          if (st != CGTP_OK) return st;
+        } else {
+          hipLaunchKernelGGL(a->y_vec ? e.seg_fwd_vec[vi] : e.seg_fwd[vi], dim3(seg_grid(plan.n_waves)), dim3(256), 0,
+                             stream, d, plan.n_waves);
+        }
+      } else {
+        hipLaunchKernelGGL(a->y_vec ? e.seg_fwd_vec[vi] : e.seg_fwd[vi], dim3(seg_grid(plan.n_waves)), dim3(256), 0,
+                           stream, d, plan.n_waves);
+      }
       if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
     }
     return a->wave_seg ? CGTP_OK : launch_fixup<T>(d.out, d, (int64_t)e.dims[2] * a->C, stream);
@@ -815,9 +855,18 @@ static int launch_bwd(const cgtp_uvu_args* a, const UvuPlan& plan, hipStream_t s
     if (wred) launch_partial_sum<T>(nullptr, (T*)a->grad_w, 0, w_elems, stream);   // zero partials: writes 0
   } else {
     const int gwm = !a->grad_w ? kGwNone : (wred ? kGwReduce : kGwStore);
-    hipLaunchKernelGGL(seg ? (a->y_vec ? e.seg_bwd_vec[vi][gwm] : e.seg_bwd[vi][gwm]) : e.bwd[vi][gwm],
-                       dim3(seg ? seg_grid(plan.n_waves) : (unsigned)((plan.n_waves + 3) / 4)), dim3(256), 0, stream, d,
-                       plan.n_waves);
+    bool done = false;
+    if constexpr (sizeof(T) == 4) {
+      if (a->radial_h) {
+        const int st = launch_radial(a, d, plan, 1, stream);
+        if (st != CGTP_OK) return st;
+        done = true;
+      }
+    }
+    if (!done)
+      hipLaunchKernelGGL(seg ? (a->y_vec ? e.seg_bwd_vec[vi][gwm] : e.seg_bwd[vi][gwm]) : e.bwd[vi][gwm],
+                         dim3(seg ? seg_grid(plan.n_waves) : (unsigned)((plan.n_waves + 3) / 4)), dim3(256), 0, stream, d,
+                         plan.n_waves);
     if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
     if (wred) {
       launch_partial_sum<T>((const T*)d.wsw, (T*)a->grad_w, plan.n_waves, w_elems, stream);
@@ -897,6 +946,12 @@ int cgtp_uvu_sh_degree(int cfg) {
   return cfg >= 0 && cfg < n ? t[cfg].sh_lmax : -1;
 }
 
+int cgtp_uvu_radial_supported(int cfg) {
+  int n = 0;
+  const UvuRadialEntry* t = uvu_radial_entries(&n);
+  return cfg >= 0 && cfg < n && t[cfg].fwd[0] != nullptr;
+}
+
 int cgtp_uvu_validate(const cgtp_uvu_args* args, int backward) {
   UvuPlan plan;
   return uvu_plan(args, backward, false, &plan);
@@ -927,4 +982,4 @@ int cgtp_uvu_bwd(const cgtp_uvu_args* a, void* stream) {
 }
 
 }  // extern "C"
-#endif  // CGTP_UVU_PS_UNIT
+#endif  // CGTP_UVU_PS_UNIT / CGTP_UVU_RADIAL_UNIT

@@ -100,6 +100,27 @@ class _EdgeUvuVectors(Function):
         return (*res, None, None, None)
 
 
+class _EdgeUvuRadial(Function):
+    """The fused kernels with the per-edge weights ``h @ w_last`` formed inside them (``y_vec`` 0: the second operand
+    is given as harmonics, else as edge vectors)."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, y: Tensor, h: Tensor, w_eff: Tensor, plan: EdgePlan, cfg: int, y_vec: int):
+        dims = kernels.uvu_dims(cfg)
+        out = kernels.uvu_radial_forward(cfg, dims, x, y, h, w_eff, plan.fwd_index, y_vec)
+        ctx.save_for_backward(x, y, h, w_eff)
+        ctx.plan, ctx.cfg, ctx.dims, ctx.y_vec = plan, cfg, dims, y_vec
+        return out
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, g):
+        x, y, h, w_eff = ctx.saved_tensors
+        res = kernels.uvu_radial_backward(ctx.cfg, ctx.dims, x, y, h, w_eff, g.contiguous(), ctx.needs_input_grad[:4],
+                                          ctx.plan.bwd_index, ctx.y_vec)
+        return (*res, None, None, None)
+
+
 class _EdgeUvuRows(Function):
     """The same composition on the row-mode kernels, for tables the fused segment kernels do not cover: per-edge
     messages from the gathered node rows, then a segment sum over the dst-sorted list; the backward forms the
@@ -190,3 +211,32 @@ def edge_tensor_product_uu_vectors(x: Tensor, edge_vec: Tensor, weight: Tensor, 
         raise ValueError(f"second operand of the table has {d2} components: not a set of harmonics 0..l_max")
     sh = spherical_harmonics(edge_vec, l_max, normalize_input=normalize_input)
     return edge_tensor_product_uu(x, sh, weight, plan, tp_info_forward, tp_info_backward1, tp_info_backward2)
+
+
+def edge_tensor_product_uu_radial(x: Tensor, sh_or_vec: Tensor, h: Tensor, w_last: Tensor, plan: EdgePlan,
+                                  tp_info_forward: TensorProductInfo, edge_vectors: bool = False,
+                                  normalize_input: bool = True) -> Tensor:
+    """:func:`edge_tensor_product_uu` (or, with ``edge_vectors``, :func:`edge_tensor_product_uu_vectors`) with the
+    per-edge weights ``weight[e] = h[e] @ w_last`` — the last linear layer of the network that turns radial features
+    (``BesselBasis`` with a cutoff, ``equitorch/nn/radials.py:10-58``, ``nn/cutoffs.py:7-131``, and the user's MLP) into
+    tensor-product weights — formed inside the edge kernels, so that the ``(E, P, C)`` weight tensor is neither written
+    nor read in the forward.  ``h (E, R)``, ``w_last (R, P, C)`` (``nn.Linear(R, P * C, bias=False).weight.T`` viewed
+    that way; a bias is a constant feature).  fp32, ``C = 64``, ``R`` a multiple of 4 up to 16 on the fused path; other
+    shapes form ``h @ w_last`` with a matrix product and take the plain functions.
+    """
+    _lib.require_gpu(x, sh_or_vec, h, w_last)
+    if plan.num_src_nodes != x.shape[0]:
+        raise _lib.CgtpError(f"plan was built for {plan.num_src_nodes} source nodes, x has {x.shape[0]}")
+    cfg = kernels.uvu_config_of(tp_info_forward)
+    mode = 0 if not edge_vectors else (kernels.Y_UNIT_VECTOR if normalize_input else kernels.Y_RAW_VECTOR)
+    if (kernels.uvu_radial_supported(cfg, x, h, w_last) and sh_or_vec.dtype == x.dtype
+            and (not edge_vectors or kernels.uvu_sh_degree(cfg) >= 0)):
+        kernels.log_tier("edge_tensor_product_uu_radial", "fused gather / weights / product / segment sum",
+                         f"config {int(cfg)}")
+        w_eff = kernels.radial_effective_weight(w_last, cfg)       # differentiable: expands paths, folds factors
+        return _EdgeUvuRadial.apply(x.contiguous(), sh_or_vec.contiguous(), h.contiguous(), w_eff, plan, cfg, mode)
+    kernels.log_tier("edge_tensor_product_uu_radial", "weights by matrix product, then the plain edge product")
+    weight = (h @ w_last.reshape(w_last.shape[0], -1)).view(h.shape[0], *w_last.shape[1:])
+    if edge_vectors:
+        return edge_tensor_product_uu_vectors(x, sh_or_vec, weight, plan, tp_info_forward, normalize_input)
+    return edge_tensor_product_uu(x, sh_or_vec, weight, plan, tp_info_forward)

@@ -563,6 +563,69 @@ def uvu_backward(cfg: int, dims, x: Tensor, y: Tensor, w: Tensor, g: Tensor, nee
     return gx, gy, contract_paths(gw, cfg, -2)
 
 
+def radial_effective_weight(w_last: Tensor, cfg) -> Tensor:
+    """``w_last (R, P, C)`` of the caller's table laid out over the compiled paths with the table's per-path factors
+    folded in (the kernels that produce the per-edge weights themselves take no separate ``path_scale``)."""
+    w = expand_paths(w_last, cfg, -2)
+    scale = cfg.scale_tensor(w.dtype, w.device) if isinstance(cfg, Cfg) else None
+    if scale is not None:
+        w = w * scale.view(1, -1, 1)
+    return w.contiguous()
+
+
+def uvu_radial_supported(cfg: int, x: Tensor, h: Tensor, w_last: Tensor) -> bool:
+    """Whether the segment kernels of ``cfg`` can form the per-edge weights from ``h (E, R)`` and ``w_last (R, P, C)``
+    themselves: fp32, 64 channels, R a multiple of 4 up to 16, aligned operands."""
+    return (cfg >= 0 and bool(_lib.lib.cgtp_uvu_radial_supported(int(cfg))) and x.dtype == h.dtype == w_last.dtype
+            and x.dtype == torch.float32 and x.shape[-1] == 64 and h.ndim == 2 and w_last.ndim == 3
+            and h.shape[1] == w_last.shape[0] and h.shape[1] % 4 == 0 and 4 <= h.shape[1] <= 16
+            and 4 <= uvu_dims(int(cfg))[3] <= 16 and h.shape[0] > 0 and x.shape[0] > 0
+            and x.data_ptr() % 16 == 0 and h.data_ptr() % 16 == 0)
+
+
+def uvu_radial_forward(cfg: int, dims, x: Tensor, y: Tensor, h: Tensor, w_eff: Tensor, seg: SegIndex,
+                       y_vec: int = 0) -> Tensor:
+    """Segment-mode forward with the per-edge weights ``h @ w_eff`` formed inside the kernel (``w_eff`` from
+    :func:`radial_effective_weight`)."""
+    a = _uvu_args(Cfg(int(cfg)), x, y, h, seg, None, 0, y_vec)
+    a.w, a.w_shared, a.path_scale = None, 0, None
+    a.radial_h, a.radial_w, a.radial_r = h.data_ptr(), w_eff.data_ptr(), h.shape[1]
+    out = torch.empty((a.n_seg, dims[2], x.shape[-1]), dtype=x.dtype, device=x.device)
+    a.out = out.data_ptr()
+    ws = _workspace(a, 0, x.device)
+    _lib.check(_lib.lib.cgtp_uvu_fwd(C.byref(a), _lib.stream_ptr(x.device)), "cgtp_uvu_fwd (radial)")
+    return out
+
+
+def uvu_radial_backward(cfg: int, dims, x: Tensor, y: Tensor, h: Tensor, w_eff: Tensor, g: Tensor, need,
+                        seg: SegIndex, y_vec: int = 0):
+    """-> (grad_x, grad_y, grad_h, grad_w_eff).  The segment kernel regenerates the weights and writes the per-edge
+    weight gradient; ``cgtp_uvu_radial_grad`` contracts it with ``w_eff`` and ``h`` in one pass."""
+    a = _uvu_args(Cfg(int(cfg)), x, y, h, seg, None, 0, y_vec)
+    a.w, a.w_shared, a.path_scale = None, 0, None
+    a.radial_h, a.radial_w, a.radial_r = h.data_ptr(), w_eff.data_ptr(), h.shape[1]
+    a.grad_out = g.data_ptr()
+    gx = torch.empty_like(x) if need[0] else None
+    gy = torch.empty_like(y) if need[1] else None
+    want_w = need[2] or need[3]
+    n_paths = dims[3]
+    gw = torch.empty((y.shape[0], n_paths, x.shape[-1]), dtype=x.dtype, device=x.device) if want_w else None
+    a.grad_x, a.grad_y, a.grad_w = _lib.ptr(gx), _lib.ptr(gy), _lib.ptr(gw)
+    ws = _workspace(a, 1, x.device)
+    _lib.check(_lib.lib.cgtp_uvu_bwd(C.byref(a), _lib.stream_ptr(x.device)), "cgtp_uvu_bwd (radial)")
+    gh = gwl = None
+    if want_w:
+        r = h.shape[1]
+        gh = torch.empty_like(h)
+        gwl = torch.empty_like(w_eff)
+        nbytes = int(_lib.lib.cgtp_uvu_radial_grad_workspace_bytes(y.shape[0], r, n_paths))
+        ws2 = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+        _lib.check(_lib.lib.cgtp_uvu_radial_grad(gw.data_ptr(), h.data_ptr(), w_eff.data_ptr(), gh.data_ptr(),
+                                                 gwl.data_ptr(), ws2.data_ptr(), y.shape[0], r, n_paths, _lib.F32,
+                                                 _lib.stream_ptr(x.device)), "cgtp_uvu_radial_grad")
+    return gx, gy, gh, gwl
+
+
 def uvu_sh_degree(cfg: int) -> int:
     """Degree L when the fused kernels of ``cfg`` can evaluate the second operand from edge vectors, else -1."""
     return int(_lib.lib.cgtp_uvu_sh_degree(cfg))

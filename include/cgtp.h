@@ -230,7 +230,33 @@ typedef struct cgtp_uvu_args {
   const void* path_scale;  /* optional, device, P values of dtype: the caller's table is the compiled one with the
                               coefficients of weight path p multiplied by path_scale[p] (other path_norm / channel_norm
                               than the compiled default, equitorch/utils/_structs.py:177-206); NULL = all ones        */
+  /* Weights produced inside the segment kernels (w may then be NULL):
+   *   W[e, p, c] = sum_r radial_h[e, r] * radial_w[r, p, c]
+   * the last linear layer of the network that maps per-edge radial features (BesselBasis and cutoffs,
+   * equitorch/nn/radials.py:10-58, nn/cutoffs.py:7-131, then the user's MLP) to tensor-product weights — in the
+   * reference a separate linear whose (E, P, C) output the product then reads.  fp32, C = 64, segment mode, configs
+   * whose kernels keep four channels per lane (cgtp_uvu_radial_supported), radial_r in {4, 8, 12, 16}, no path_scale
+   * (fold it into radial_w), 16-byte aligned pointers.  Backward: grad_w (n_rows, P, C) is written when given;
+   * cgtp_uvu_radial_grad turns it into the gradients of radial_h and radial_w. */
+  const void* radial_h;    /* (n_rows, radial_r) or NULL                                          */
+  const void* radial_w;    /* (radial_r, P, C)                                                    */
+  int32_t radial_r;
+  int32_t reserved2_;
 } cgtp_uvu_args;
+
+/* 1 if config `cfg` has segment kernels that produce the weights themselves (cgtp_uvu_args.radial_h). */
+int cgtp_uvu_radial_supported(int cfg);
+/* The other two gradients of that mode, from the per-edge weight gradient grad_w (n_rows, n_paths, 64) the backward
+ * wrote, in one pass over it:
+ *   grad_radial_h[e, r]    = sum_{p, c} grad_w[e, p, c] * radial_w[r, p, c]
+ *   grad_radial_w[r, p, c] = sum_e radial_h[e, r] * grad_w[e, p, c]
+ * (in the reference: autograd through the linear layer that produced the weights).  fp32; 4 <= n_paths <= 16,
+ * radial_r <= 16; grad_w and radial_w 16-byte aligned.  The workgroups' partial sums over the edges live in `workspace`
+ * (cgtp_uvu_radial_grad_workspace_bytes) and are added in a fixed order. */
+int64_t cgtp_uvu_radial_grad_workspace_bytes(int64_t n_rows, int32_t radial_r, int32_t n_paths);
+int cgtp_uvu_radial_grad(const void* grad_w, const void* radial_h, const void* radial_w, void* grad_radial_h,
+                         void* grad_radial_w, void* workspace, int64_t n_rows, int32_t radial_r, int32_t n_paths,
+                         int32_t dtype, void* stream);
 
 int cgtp_uvu_validate(const cgtp_uvu_args* args, int backward);
 /* Bytes of workspace the forward (backward = 0) or backward (1) launch of `args` needs; 0 if none. */

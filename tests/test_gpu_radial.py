@@ -1,0 +1,86 @@
+"""GPU parity of the edge product whose per-edge weights are formed inside the kernels from per-edge features and a
+shared matrix (``edge_tensor_product_uu_radial``, ``cgtp_uvu_radial_grad``): output and all gradients against the
+dense float64 oracle with the weights formed by an explicit einsum (``W[e] = h[e] @ w_last``), gathered at src and
+summed at dst."""
+import pytest
+import torch
+
+from helpers import assert_close
+from oracle import ref_ops, ref_sh
+
+pytestmark = pytest.mark.gpu
+
+SH = {l: "+".join(f"{k}{'e' if k % 2 == 0 else 'o'}" for k in range(l + 1)) for l in range(5)}
+
+
+def _case(lmax, n_nodes, n_edges, r, seed, hub=False):
+    g = torch.Generator().manual_seed(seed)
+    d = (lmax + 1) ** 2
+    src = torch.randint(0, n_nodes, (n_edges,), generator=g)
+    dst = torch.randint(0, n_nodes, (n_edges,), generator=g)
+    dst[dst == 3] = 4                                           # an empty segment
+    if hub:
+        dst[50:400] = 11
+        src[200:500] = 2
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).float().double()
+    return src, dst, rd(n_nodes, d, 64), rd(n_edges, r), rd(n_nodes, d, 64), rd, g
+
+
+@pytest.mark.parametrize("lmax,r,vectors,hub", [(2, 16, False, False), (2, 8, False, True), (2, 16, True, False),
+                                                (2, 4, True, True), (1, 12, False, False), (1, 16, True, True)])
+def test_edge_product_with_weights_formed_in_the_kernel(device, lmax, r, vectors, hub):
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu_radial
+    from equitorch_amd.ops import kernels
+    n_nodes, n_edges = 70, 1303
+    irr = SH[lmax]
+    mod = SO3Linear(irr, irr, irr, internal_weights=False, feature_mode="uu").to(device)
+    src, dst, x, h, ct, rd, g = _case(lmax, n_nodes, n_edges, r, 300 + 10 * lmax + r, hub)
+    w_last = rd(r, mod.num_paths, 64) / r ** 0.5
+    d2 = (lmax + 1) ** 2
+    y = (rd(n_edges, 3) * (0.5 + torch.rand(n_edges, 1, generator=g, dtype=torch.float64))).float().double() if vectors \
+        else rd(n_edges, d2)
+    T = ref_ops.dense_coupling(irr, irr, irr)
+    xr, yr, hr, wr = (t.clone().requires_grad_(True) for t in (x, y, h, w_last))
+    sh = ref_sh.spherical_harmonics(ref_sh.normalize(yr), lmax) if vectors else yr
+    weights = torch.einsum("er,rpc->epc", hr, wr)
+    ref = ref_ops.scatter_sum(ref_ops.dense_u1u(T, xr[src], sh, weights), dst, n_nodes)
+    (ref * ct).sum().backward()
+
+    plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
+    xd, yd, hd, wd = (t.to(device, torch.float32).requires_grad_(True) for t in (x, y, h, w_last))
+    assert kernels.uvu_radial_supported(kernels.uvu_config_of(mod.tp_info_forward), xd, hd, wd)
+    out = edge_tensor_product_uu_radial(xd, yd, hd, wd, plan, mod.tp_info_forward, edge_vectors=vectors)
+    (out * ct.to(device, torch.float32)).sum().backward()
+    for name, a, b in (("out", out, ref), ("grad_x", xd.grad, xr.grad), ("grad_y", yd.grad, yr.grad),
+                       ("grad_h", hd.grad, hr.grad), ("grad_w_last", wd.grad, wr.grad)):
+        # grad_h sums over all paths and channels, grad_w_last over all edges, grad of vectors through the harmonics
+        long_sum = name in ("grad_h", "grad_w_last") or (vectors and name == "grad_y")
+        assert_close(a, b, tol=1e-5, what=f"radial lmax={lmax} R={r} vec={vectors} {name}",
+                     norm="max" if long_sum else "element")
+
+
+def test_radial_with_other_normalisation_and_fallback(device):
+    """A table that differs from the compiled one by per-path factors (path_norm off) keeps the fused kernels (the
+    factors are folded into the shared matrix); shapes the fused kernels do not take (R = 6) give the same numbers
+    through the plain functions."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu_radial
+    n_nodes, n_edges, lmax = 40, 500, 2
+    irr = SH[lmax]
+    mod = SO3Linear(irr, irr, irr, internal_weights=False, feature_mode="uu", path_norm=False).to(device)
+    T = ref_ops.dense_coupling(irr, irr, irr, path_norm=False)
+    for r in (8, 6):
+        src, dst, x, h, ct, rd, g = _case(lmax, n_nodes, n_edges, r, 77 + r)
+        w_last, y = rd(r, mod.num_paths, 64) / r ** 0.5, rd(n_edges, 9)
+        xr, yr, hr, wr = (t.clone().requires_grad_(True) for t in (x, y, h, w_last))
+        ref = ref_ops.scatter_sum(ref_ops.dense_u1u(T, xr[src], yr, torch.einsum("er,rpc->epc", hr, wr)), dst, n_nodes)
+        (ref * ct).sum().backward()
+        plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
+        xd, yd, hd, wd = (t.to(device, torch.float32).requires_grad_(True) for t in (x, y, h, w_last))
+        out = edge_tensor_product_uu_radial(xd, yd, hd, wd, plan, mod.tp_info_forward)
+        (out * ct.to(device, torch.float32)).sum().backward()
+        for name, a, b in (("out", out, ref), ("grad_x", xd.grad, xr.grad), ("grad_y", yd.grad, yr.grad),
+                           ("grad_h", hd.grad, hr.grad), ("grad_w_last", wd.grad, wr.grad)):
+            assert_close(a, b, tol=1e-5, what=f"radial path_norm=False R={r} {name}",
+                         norm="max" if name in ("grad_h", "grad_w_last") else "element")
