@@ -46,6 +46,7 @@ __device__ __forceinline__ void radial_weights(const float* lds, const float* __
   floatx4 hq[4];
 #pragma unroll
   for (int q = 0; q < 4; ++q) hq[q] = *reinterpret_cast<const floatx4*>(hrow + (4 * q < R ? 4 * q : 0));
+  // all paths side by side: P independent chains of matrix instructions keep the pipeline full
   floatx4 acc[P];
 #pragma unroll
   for (int p = 0; p < P; ++p) acc[p] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -63,8 +64,6 @@ __device__ __forceinline__ void radial_weights(const float* lds, const float* __
   for (int p = 0; p < P; ++p)
 #pragma unroll
     for (int v = 0; v < 4; ++v) w[p][v] = __shfl(acc[p][v], src, kWave);
-  // the loads of the tensor-product body stay below: issued earlier they would need registers that are not there
-  __builtin_amdgcn_sched_barrier(0);
 }
 
 template <class TP, bool YV>
@@ -133,19 +132,11 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_radial_kernel(const UvuDev
   zero_rows(acc);
   SegStep st;
   st.next_row = R.s0;
-  T x[D1][V];
-  zero_rows(x);
-  int x_seg = -1;
   for (int64_t cb = R.p0; cb < R.p1; cb += kWave) {
   const SegIndexRegs I(a.seg_ids, a.perm, a.gather, cb, cb + kWave < R.p1 ? cb + kWave : R.p1, L.lane);
   for (int off0 = 0; off0 < I.npos;) {
     int ei, oi;
     const bool valid = seg_step_begin<T, D1, V>(st, acc, a.gx, a.ws, I, off0, ei, oi, wave, R, L, 4, true, C, c0);
-    if (st.cur != x_seg) {   // the same for all lanes of the wavefront
-      x_seg = st.cur;
-#pragma unroll
-      for (int i = 0; i < D1; ++i) load_vec<T, V>(x[i], a.x + ((int64_t)x_seg * D1 + i) * C + c0);
-    }
     T w[P][V];
     radial_weights<TP>(rw_lds, a.rh, a.R, __shfl(ei, (L.lane & 3) << 4, kWave), L.lane, w);
     if (valid) {
@@ -164,6 +155,11 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_radial_kernel(const UvuDev
       for (int j = 0; j < D2; ++j) gy[j] = T(0);
 #pragma unroll
       for (int m = 0; m < DO; ++m) load_vec<T, V>(g[m], a.g + (gr * DO + m) * C + c0);
+      // the segment's rows of x are read again in every step (the plain kernel keeps them in registers over a
+      // segment; here the registers go to the weights' production, and the rows hit in the first-level cache)
+      T x[D1][V];
+#pragma unroll
+      for (int i = 0; i < D1; ++i) load_vec<T, V>(x[i], a.x + ((int64_t)st.cur * D1 + i) * C + c0);
       T* gwrow = a.gw + e * P * C + c0;
       TP::template bwd<T, V>(
           x, y, [&](int p, T (&wp)[V]) {
@@ -200,8 +196,8 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_radial_kernel(const UvuDev
 //   grad_h[e, r]    = sum_{p, c} grad_w[e, p, c] * W_last[r, p, c]
 //   grad_W[r, p, c] = sum_e h[e, r] * grad_w[e, p, c]
 // in one pass over grad_w (E, P, 64), the tensor the backward above wrote.  A workgroup walks tiles of 16 edges, staged
-// in LDS (double-buffered: the next tile is in flight while this one is multiplied); wavefront p owns the 64 columns
-// of path p.  Both products run on v_mfma_f32_16x16x4_f32:
+// in LDS (the next tile is requested into registers before this one is multiplied; three workgroups share a compute
+// unit and cover each other's waits); wavefront p owns the 64 columns of path p.  Both products run on v_mfma_f32_16x16x4_f32:
 //   grad_W^T tile: A = h^T (16 features x 4 edges), B = grad_w (4 edges x 16 columns): one LDS word per lane and step;
 //   grad_h tile:   A = W_last (16 features x 4 columns, held in registers for the whole kernel), B = grad_w^T
 //                  (4 columns x 16 edges): a lane's four columns of four steps are one 16-byte LDS read.
@@ -216,9 +212,9 @@ __global__ void __launch_bounds__(1024) uvu_radial_grad_kernel(const float* __re
                                                               int tiles_per_group) {
   extern __shared__ __align__(16) float rg_lds[];
   const int PC = P * kRadialC, pitch = PC + 16;
-  float* tile[2] = {rg_lds, rg_lds + kRgTile * pitch};
-  float* hs = rg_lds + 2 * kRgTile * pitch;                 // [2][16 edges][16 features]
-  float* ghs = hs + 2 * kRgTile * 16;                       // [P][16 features][16 edges + 1]
+  float* tile = rg_lds;                                     // [16 edges][pitch]
+  float* hs = rg_lds + kRgTile * pitch;                     // [16 edges][16 features]
+  float* ghs = hs + kRgTile * 16;                           // [P][16 features][16 edges + 1]
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), r = lane & 15, q = lane >> 4;
   const int nthreads = blockDim.x;
   const int64_t t_begin = (int64_t)blockIdx.x * tiles_per_group;
@@ -251,25 +247,24 @@ __global__ void __launch_bounds__(1024) uvu_radial_grad_kernel(const float* __re
       hstage = (e0 + e < n_rows && f < R) ? h[(e0 + e) * R + f] : 0.f;
     }
   };
-  auto commit = [&](int buf) __attribute__((always_inline)) {
+  auto commit = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const int idx = threadIdx.x + k * nthreads, e = idx / pc4, c4 = idx - e * pc4;
-      *reinterpret_cast<floatx4*>(tile[buf] + e * pitch + c4 * 4) = stage[k];
+      *reinterpret_cast<floatx4*>(tile + e * pitch + c4 * 4) = stage[k];
     }
-    if (threadIdx.x < kRgTile * 16) hs[buf * kRgTile * 16 + threadIdx.x] = hstage;
+    if (threadIdx.x < kRgTile * 16) hs[threadIdx.x] = hstage;
   };
 
   if (t_begin < t_end) {
     request(t_begin);
-    commit(0);
+    commit();
   }
   __syncthreads();
   for (int64_t t = t_begin; t < t_end; ++t) {
-    const int buf = (int)((t - t_begin) & 1);
     if (t + 1 < t_end) request(t + 1);
-    const float* tl = tile[buf] + wave * kRadialC;
-    const float* hl = hs + buf * kRgTile * 16;
+    const float* tl = tile + wave * kRadialC;
+    const float* hl = hs;
     // grad_W^T += grad_w^T h: contraction over the 16 edges, four per step
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
@@ -297,7 +292,7 @@ __global__ void __launch_bounds__(1024) uvu_radial_grad_kernel(const float* __re
       const int64_t row = t * kRgTile + e;
       if (row < n_rows && f < R) gh[row * R + f] = sum;
     }
-    if (t + 1 < t_end) commit(buf ^ 1);
+    if (t + 1 < t_end) commit();   // every wavefront is past its reads of the tile (barrier above)
     __syncthreads();
   }
   // this workgroup's partial grad_W: part[group][feature][column]
@@ -311,17 +306,29 @@ __global__ void __launch_bounds__(1024) uvu_radial_grad_kernel(const float* __re
     }
 }
 
-__global__ void radial_reduce_kernel(const float* __restrict__ part, float* __restrict__ out, int64_t n_groups, int64_t n) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
+// out[i] = sum over the groups of part[g][i]: 64 outputs per workgroup, 16 threads per output that each add every
+// 16th group in ascending order, then one thread adds the 16 sums in order (a fixed order whatever the launch).
+__global__ void __launch_bounds__(1024) radial_reduce_kernel(const float* __restrict__ part, float* __restrict__ out,
+                                                             int64_t n_groups, int64_t n) {
+  __shared__ float sums[16][64];
+  const int o = threadIdx.x & 63, gl = threadIdx.x >> 6;
+  const int64_t i = (int64_t)blockIdx.x * 64 + o;
   float s = 0.f;
-  for (int64_t g = 0; g < n_groups; ++g) s += part[g * n + i];
-  out[i] = s;
+  if (i < n)
+    for (int64_t g = gl; g < n_groups; g += 16) s += part[g * n + i];
+  sums[gl][o] = s;
+  __syncthreads();
+  if (gl == 0 && i < n) {
+    float t = 0.f;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) t += sums[k][o];
+    out[i] = t;
+  }
 }
 
 static int64_t radial_groups(int64_t n_rows) {
   const int64_t n_tiles = (n_rows + kRgTile - 1) / kRgTile;
-  return n_tiles < 256 ? (n_tiles > 0 ? n_tiles : 1) : 256;
+  return n_tiles < 512 ? (n_tiles > 0 ? n_tiles : 1) : 512;
 }
 
 template <class TP>
@@ -374,7 +381,7 @@ int cgtp_uvu_radial_grad(const void* grad_w, const void* radial_h, const void* r
   const int64_t n_out = (int64_t)radial_r * PC;
   hipStream_t st = (hipStream_t)stream;
   if (n_rows == 0) {
-    hipLaunchKernelGGL(radial_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, st,
+    hipLaunchKernelGGL(radial_reduce_kernel, dim3((unsigned)((n_out + 63) / 64)), dim3(1024), 0, st,
                        (const float*)nullptr, (float*)grad_radial_w, (int64_t)0, n_out);
     return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
   }
@@ -382,7 +389,7 @@ int cgtp_uvu_radial_grad(const void* grad_w, const void* radial_h, const void* r
   const int64_t groups = radial_groups(n_rows);
   const int64_t n_tiles = (n_rows + kRgTile - 1) / kRgTile;
   const int tiles_per_group = (int)((n_tiles + groups - 1) / groups);
-  const size_t lds = ((size_t)2 * kRgTile * (PC + 16) + 2 * kRgTile * 16 + (size_t)n_paths * 16 * 17) * sizeof(float);
+  const size_t lds = ((size_t)kRgTile * (PC + 16) + kRgTile * 16 + (size_t)n_paths * 16 * 17) * sizeof(float);
   if (lds > (size_t)kLdsBytes) return CGTP_ERR_LDS;
   if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)uvu_radial_grad_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                              (int)lds) != hipSuccess)
@@ -391,7 +398,7 @@ int cgtp_uvu_radial_grad(const void* grad_w, const void* radial_h, const void* r
                      (const float*)grad_w, (const float*)radial_h, (const float*)radial_w, (float*)grad_radial_h,
                      (float*)workspace, n_rows, (int)radial_r, (int)n_paths, tiles_per_group);
   if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
-  hipLaunchKernelGGL(radial_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, st,
+  hipLaunchKernelGGL(radial_reduce_kernel, dim3((unsigned)((n_out + 63) / 64)), dim3(1024), 0, st,
                      (const float*)workspace, (float*)grad_radial_w, groups, n_out);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
