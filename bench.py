@@ -870,11 +870,78 @@ def other_configs(args, headline):
     torch.cuda.empty_cache()
     sub.workload, sub.steps, sub.warmup = "edge_l6_fwd_bwd", 4, 2
     r = edge_rows_bench(sub)
+    torch.cuda.empty_cache()
+    out["cfg1_edge_weights_formed_in_kernel_R16"] = radial_record(16)
     out["cfg4_edge_fwd_bwd_lmax6_C32"] = {
         "Medges_s": r["value"], "step_ms": r["ms_per_step"], "fwd_ms": r["kernels"]["fwd_ms"],
         "bwd_ms": r["kernels"]["bwd_ms"], "bwd_hbm_frac": r["roofline"]["frac"],
         "bwd_fp32_frac": r["roofline"]["fp32_vector"]["frac"], "fwd_TFLOPs": r["kernels"]["fwd_TFLOPs"]}
     return out
+
+
+def radial_record(r):
+    """The headline edge workload with the per-edge weights formed inside the kernels from ``h (E, r)`` and a shared
+    ``(r, 11, 64)`` matrix (``edge_tensor_product_uu_radial``), next to the same step with the weights formed by a
+    matrix product and read back by the plain kernels.  Bytes per edge: compulsory traffic of the forward launch."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu, edge_tensor_product_uu_radial
+    from equitorch_amd.ops import kernels
+    lmax, ch, n_nodes, n_edges = WORKLOADS["edge_fwd_bwd"]
+    dev = torch.device("cuda:0")
+    irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+    mod = SO3Linear(irreps, irreps, irreps, ch, ch, internal_weights=False, feature_mode="uu").to(dev)
+    inp = make_inputs(lmax, ch, n_nodes, n_edges, 1, dev)
+    d, p, gen = inp["d"], mod.num_paths, inp["gen"]
+    plan = EdgePlan(inp["src"].to(dev), inp["dst"].to(dev), n_nodes)
+    x = inp["x"].to(dev).requires_grad_(True)
+    sh = inp["sh"].to(dev).requires_grad_(True)
+    hs = [torch.randn(n_edges, r, generator=gen).to(dev).requires_grad_(True) for _ in range(4)]
+    wl = (torch.randn(r, p, ch, generator=gen) / r ** 0.5).to(dev).requires_grad_(True)
+    ct = torch.randn(n_nodes, d, ch, generator=gen).to(dev)
+    cfg = kernels.uvu_config_of(mod.tp_info_forward)
+    dims = kernels.uvu_dims(cfg)
+
+    def wall(fn, steps=20, warm=3):
+        for i in range(warm):
+            fn(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            fn(i)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3
+
+    def events(fn, reps=12):
+        evs = []
+        for i in range(reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(); fn(i); b.record()
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        return sum(a.elapsed_time(b) for a, b in evs[2:]) / (reps - 2)
+
+    def fused(i):
+        out = edge_tensor_product_uu_radial(x, sh, hs[i % 4], wl, plan, mod.tp_info_forward)
+        return torch.autograd.grad(out, (x, sh, hs[i % 4], wl), ct)
+
+    def unfused(i):
+        w = (hs[i % 4] @ wl.view(r, -1)).view(n_edges, p, ch)
+        out = edge_tensor_product_uu(x, sh, w, plan, mod.tp_info_forward)
+        return torch.autograd.grad(out, (x, sh, hs[i % 4], wl), ct)
+    xd, shd, wld = x.detach(), sh.detach(), wl.detach()
+    fwd_ms = events(lambda i: kernels.uvu_radial_forward(cfg, dims, xd, shd, hs[i % 4].detach(), wld, plan.fwd_index))
+    bwd_ms = events(lambda i: kernels.uvu_radial_backward(cfg, dims, xd, shd, hs[i % 4].detach(), wld, ct,
+                                                          (True, True, True, True), plan.bwd_index))
+    node = n_nodes * d * ch * 4
+    idx = 2 * n_edges * 8 + (n_nodes + 1) * 8
+    fwd_bytes = n_edges * r * 4 + r * p * ch * 4 + n_edges * d * 4 + 2 * node + idx
+    plain_fwd_bytes, _ = algorithmic_bytes(n_nodes, n_edges, d, p, ch)
+    step_fused, step_unfused = wall(fused), wall(unfused)
+    return {"R": r, "fwd_ms": round(fwd_ms, 4), "bwd_all_grads_ms": round(bwd_ms, 4),
+            "fwd_bytes_per_edge": round(fwd_bytes / n_edges, 1),
+            "plain_fwd_bytes_per_edge": round(plain_fwd_bytes / n_edges, 1),
+            "step_ms": round(step_fused, 4), "step_ms_weights_by_matrix_product": round(step_unfused, 4),
+            "Medges_s": round(n_edges / (step_fused * 1e-3) / 1e6, 1)}
 
 
 def config0_record(with_cpu):

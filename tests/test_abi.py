@@ -245,3 +245,103 @@ def test_tables_of_a_module_in_reduced_precision_find_their_config():
             assert find(C.c_uint64(fp)) == -1                            # not an fp32 table
             assert find_rounded(C.c_uint64(fp), _lib.F32) == -1
         assert find_rounded(C.c_uint64(fingerprint(tp_coo(info), "bf16")), 3) == -1
+
+
+def test_table_driven_matrix_core_entry_points_validate_on_the_host():
+    """cgtp_uvt_*: launch shape queries and argument checks of the fp32 fully connected kernels, no launch."""
+    from equitorch_amd import _lib
+    L = _lib.lib
+    p16 = 4096
+    # lmax = 3, 128 -> 128 channels: four blocks of 16 k per ring turn; 16 output rows over 4 item groups (the other
+    # two wavefronts of a sample block split the 128 output channels)
+    assert L.cgtp_uvt_chunk(32768, 16, 16, 16, 128, 0, 128) == 4
+    assert L.cgtp_uvt_item_groups(32768, 16, 16, 16, 128, 0, 128) == 4
+    assert L.cgtp_uvt_item_groups(32768, 9, 9, 1, 32, 0, 64) == 1           # a single output row
+    assert L.cgtp_uvt_item_groups(32768, 9, 9, 9, 32, 0, 32) == 8           # one wavefront covers the channels
+    assert L.cgtp_uvt_chunk(100, 16, 16, 16, 130, 0, 128) == -2             # channels not a multiple of 4
+    assert L.cgtp_uvt_chunk(100, 49, 49, 49, 128, 0, 128) == -6             # 16 samples x 49 rows x 128 floats > LDS
+    assert L.cgtp_uvt_packed_elems(23, 128, 128) == 23 * 8 * 8 * 256
+    assert L.cgtp_uvt_packed_elems(2, 20, 12) == 2 * 4 * 4 * 256            # padded to whole ring turns / 4 blocks
+    a = _lib.UvtArgs()
+    a.dtype = _lib.BF16
+    assert L.cgtp_uvt_validate(C.byref(a)) == 4                             # fp32 only
+    a.dtype = _lib.F32
+    a.n_rows, a.dx, a.dy, a.dout, a.cx, a.cy, a.cout = 100, 9, 9, 9, 32, 0, 32
+    assert L.cgtp_uvt_validate(C.byref(a)) == 2                             # kbi / groups not set
+    a.kbi, a.n_groups = 4, 8
+    a.n_items, a.n_terms = 35, 83
+    for i in range(9):
+        a.group_ptr[i] = min(5 * i, 35)
+    assert L.cgtp_uvt_validate(C.byref(a)) == 1                             # null pointers
+    a.x = a.y = a.wp = a.out = a.items = a.term_a = a.term_b = a.term_c = p16
+    assert L.cgtp_uvt_validate(C.byref(a)) == 0
+    a.group_ptr[8] = 34
+    assert L.cgtp_uvt_validate(C.byref(a)) == 2                             # groups do not cover the items
+    a.group_ptr[8] = 35
+    a.x = p16 + 4
+    assert L.cgtp_uvt_validate(C.byref(a)) == 3                             # alignment
+    assert L.cgtp_uvt_pack_weights(p16, p16, 2, 0, 16, 1, 1, 1, _lib.F32, None) == 2
+    assert L.cgtp_uvt_pack_weights(None, p16, 2, 16, 16, 1, 1, 1, _lib.F32, None) == 1
+    # weight gradient: chunks of at least 256 samples, at most 128 of them
+    assert L.cgtp_uvt_grad_w_workspace_bytes(32768, 23, 128, 128) == 128 * 23 * 128 * 128 * 4
+    assert L.cgtp_uvt_grad_w_workspace_bytes(300, 4, 32, 16) == 2 * 4 * 32 * 16 * 4
+    g = _lib.UvtGwArgs()
+    g.dtype = _lib.F32
+    g.n_rows, g.n_paths, g.dx, g.dy, g.dg, g.cx, g.cy, g.cout = 10, 4, 9, 9, 9, 32, 0, 30
+    g.x = g.y = g.g = g.gw = g.path_ptr = g.items = g.term_a = g.term_b = g.term_c = p16
+    g.n_items = 1
+    assert L.cgtp_uvt_grad_w(C.byref(g), None) == 2                         # cout not a multiple of 4
+    g.cout = 32
+    assert L.cgtp_uvt_grad_w(C.byref(g), None) == 8                         # workspace missing
+    y = _lib.UvtGyArgs()
+    y.dtype = _lib.F32
+    y.n_rows, y.n_items, y.n_terms, y.dx, y.dy, y.dg, y.cx, y.cout = 0, 5, 9, 9, 9, 9, 32, 32
+    assert L.cgtp_uvt_grad_y(C.byref(y), None) == 1                         # null pointers
+    y.x = y.g = y.wp = y.gy = y.items = y.term_m = y.term_b = y.term_c = p16
+    assert L.cgtp_uvt_grad_y(C.byref(y), None) == 0                         # empty batch: no launch
+    y.dx, y.cx = 49, 128
+    assert L.cgtp_uvt_grad_y(C.byref(y), None) == 6                         # 16 samples do not fit the LDS
+
+
+def test_radial_mode_validates_on_the_host():
+    """Per-edge weights formed in the kernel: segment mode, fp32, 64 channels, 4 | R <= 16, configs that keep four
+    channels per lane (lmax <= 2 here)."""
+    from equitorch_amd import _lib
+    from equitorch_amd._tables import fingerprint, tp_coo
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    L = _lib.lib
+    p16 = 4096
+
+    def cfg_of(irr):
+        return L.cgtp_uvu_find(C.c_uint64(fingerprint(tp_coo(tp_infos(Irreps(irr), Irreps(irr), Irreps(irr))[0]))))
+    c2, c3 = cfg_of("0e+1o+2e"), cfg_of("0e+1o+2e+3o")
+    assert L.cgtp_uvu_radial_supported(c2) == 1 and L.cgtp_uvu_radial_supported(c3) == 0
+    assert L.cgtp_uvu_radial_supported(-1) == 0 and L.cgtp_uvu_radial_supported(999) == 0
+    a = _lib.UvuArgs()
+    a.cfg, a.dtype, a.C, a.n_rows, a.n_x_rows, a.n_seg = c2, _lib.F32, 64, 100, 10, 10
+    a.ptr = a.seg_ids = a.gather = a.x = a.y = a.out = p16
+    a.radial_h, a.radial_w, a.radial_r = p16, p16, 16
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 0                          # no weight tensor needed
+    a.radial_r = 6
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 2
+    a.radial_r, a.C = 8, 32
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 2                          # 64 channels only
+    a.C, a.dtype = 64, _lib.F64
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 4
+    a.dtype, a.radial_w = _lib.F32, None
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 1
+    a.radial_w, a.cfg = p16, c3
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 5                          # no such kernels for this table
+    a.cfg, a.path_scale = c2, p16
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 2                          # fold the factors into radial_w
+    a.path_scale, a.radial_h = None, p16 + 4
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 3
+    # gradients of the features and the shared matrix: at most 512 partial sums of (R, P, 64) floats
+    assert L.cgtp_uvu_radial_grad_workspace_bytes(65536, 16, 11) == 512 * 16 * 11 * 64 * 4
+    assert L.cgtp_uvu_radial_grad_workspace_bytes(100, 8, 4) == 7 * 8 * 4 * 64 * 4
+    assert L.cgtp_uvu_radial_grad(p16, p16, p16, p16, p16, None, 100, 16, 11, _lib.F32, None) == 8
+    assert L.cgtp_uvu_radial_grad(p16, p16, p16, p16, p16, p16, 100, 20, 11, _lib.F32, None) == 2
+    assert L.cgtp_uvu_radial_grad(p16, p16, p16, p16, p16, p16, 100, 16, 3, _lib.F32, None) == 2
+    assert L.cgtp_uvu_radial_grad(p16, p16, p16, None, p16, p16, 100, 16, 11, _lib.F32, None) == 1
+    assert L.cgtp_uvu_radial_grad(p16, p16, p16, p16, p16, p16, 100, 16, 11, _lib.F64, None) == 4
