@@ -277,16 +277,17 @@ int cgtp_layer_rms_backward(const void* x, const void* weight, const void* rsigm
   using namespace cgtp;
   NormSeg seg;
   if (int rc = norm_check(x, irrep_seg, irrep_rdims, n_irreps, n_rows, D, C, dtype, &seg)) return rc;
-  if (!rsigma || !grad_out) return n_rows ? CGTP_ERR_NULL : CGTP_OK;
-  if (grad_weight && !workspace) return CGTP_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
-  if (n_rows == 0) {   // no rows: the sum over them is zero (written by the summation kernel over zero partials)
+  if (n_rows == 0) {   // no rows (the operands may be null): the sum over them is zero, written by the summation
+                       // kernel over zero partials
     if (grad_weight) {
       if (dtype == CGTP_F32) launch_partial_sum<float>(nullptr, (float*)grad_weight, 0, (int64_t)n_irreps * C, s);
       else launch_partial_sum<double>(nullptr, (double*)grad_weight, 0, (int64_t)n_irreps * C, s);
     }
     return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
   }
+  if (!rsigma || !grad_out) return CGTP_ERR_NULL;
+  if (grad_weight && !workspace) return CGTP_ERR_WORKSPACE;
   return dtype == CGTP_F32
              ? bwd_launch<float>(x, weight, rsigma, grad_out, grad_x, grad_weight, workspace, seg, n_rows, D, C, scaled, s)
              : bwd_launch<double>(x, weight, rsigma, grad_out, grad_x, grad_weight, workspace, seg, n_rows, D, C, scaled, s);
