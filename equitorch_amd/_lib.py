@@ -58,7 +58,8 @@ class UvuArgs(C.Structure):
                 ("grad_out", C.c_void_p), ("grad_x", C.c_void_p), ("grad_y", C.c_void_p),
                 ("grad_w", C.c_void_p), ("workspace", C.c_void_p), ("x_gather", C.c_void_p),
                 ("y_channels", C.c_int32), ("reserved_", C.c_int32), ("path_scale", C.c_void_p),
-                ("radial_h", C.c_void_p), ("radial_w", C.c_void_p), ("radial_r", C.c_int32), ("reserved2_", C.c_int32)]
+                ("radial_h", C.c_void_p), ("radial_w", C.c_void_p), ("radial_r", C.c_int32), ("reserved2_", C.c_int32),
+                ("wave_pos", C.c_void_p)]
 
 
 class UvtItem(C.Structure):
@@ -120,6 +121,7 @@ def _load():
     lib.cgtp_uvu_describe.argtypes = [C.c_int, C.POINTER(C.c_int32)]
     lib.cgtp_uvu_sh_degree.argtypes = [C.c_int]
     lib.cgtp_uvu_radial_supported.argtypes = [C.c_int]
+    lib.cgtp_uvu_slots.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int]
     lib.cgtp_uvu_radial_grad_workspace_bytes.restype = C.c_int64
     lib.cgtp_uvu_radial_grad_workspace_bytes.argtypes = [C.c_int64, C.c_int32, C.c_int32]
     lib.cgtp_uvu_radial_grad.argtypes = [C.c_void_p] * 6 + [C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]

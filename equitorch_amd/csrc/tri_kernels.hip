@@ -578,7 +578,8 @@ int cgtp_abi_layout(int which, int64_t* out, int capacity) {
                                 CGTP_OFF(cgtp_uvu_args, x_gather), CGTP_OFF(cgtp_uvu_args, y_channels),
                                 CGTP_OFF(cgtp_uvu_args, reserved_), CGTP_OFF(cgtp_uvu_args, path_scale),
                                 CGTP_OFF(cgtp_uvu_args, radial_h), CGTP_OFF(cgtp_uvu_args, radial_w),
-                                CGTP_OFF(cgtp_uvu_args, radial_r), CGTP_OFF(cgtp_uvu_args, reserved2_)};
+                                CGTP_OFF(cgtp_uvu_args, radial_r), CGTP_OFF(cgtp_uvu_args, reserved2_),
+                                CGTP_OFF(cgtp_uvu_args, wave_pos)};
   static const int64_t uvt_item[] = {sizeof(cgtp_uvt_item), CGTP_OFF(cgtp_uvt_item, p), CGTP_OFF(cgtp_uvt_item, kb0),
                                      CGTP_OFF(cgtp_uvt_item, nkb), CGTP_OFF(cgtp_uvt_item, t0), CGTP_OFF(cgtp_uvt_item, t1),
                                      CGTP_OFF(cgtp_uvt_item, out_row), CGTP_OFF(cgtp_uvt_item, flags),

@@ -24,7 +24,8 @@ struct UvuDev {
   const int64_t* x_gather;  // row mode backward: optional row of x per batch row
   const int64_t* seg_ids;
   const int32_t* wave_seg;  // segment mode: optional wavefront -> first segment table (segment-aligned ranges)
-  int64_t n_rows, n_seg;
+  const int64_t* wave_pos;  // segment mode: optional wavefront -> first sorted position table (ranges cut anywhere)
+  int64_t n_rows, n_seg, n_waves;
   int C, lpe_log2, w_shared, pos_per_wave;
   int y_vec;  // segment mode: y holds edge vectors (kYUnitVector / kYRawVector) instead of harmonics
   const T* ps;  // optional factor of every weight path (the caller's table = compiled table x ps[p]); nullptr = ones

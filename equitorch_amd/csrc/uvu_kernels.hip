@@ -158,18 +158,21 @@ __global__ void __launch_bounds__(256, 2) uvu_bwd_kernel(const UvuDev<T> a, int6
 }
 
 // ---- segment mode ----------------------------------------------------------------------------------------------
-// Range [p0, p1) of sorted positions owned by one wavefront.  Two ways to cut the edge list:
+// Range [p0, p1) of sorted positions owned by one wavefront.  Three ways to cut the edge list:
 //  * aligned (wave_seg given): the wavefront owns the whole segments [s0, s1); every row it produces is final,
 //    and it also zero-fills the rows of empty segments in [s0, s1);
-//  * by position (wave_seg == nullptr): exactly per_wave positions each; the first / last segment of a range may
-//    continue in a neighbouring wavefront and then goes through a partial row (see uvu_fixup_kernel).
+//  * at given positions (wave_pos given): range k is [wave_pos[k], wave_pos[k + 1]) — the caller cuts where it
+//    likes, e.g. so that every wavefront has the same number of steps;
+//  * by position (neither): exactly per_wave positions each.
+// In the last two the first / last segment of a range may continue in a neighbouring wavefront and then goes
+// through a partial row (see uvu_fixup_kernel).
 struct SegRange {
   int64_t p0, p1;
   int s0, s1;                          // aligned mode: owned segments; else -1
   bool first_complete, last_complete;  // does the first / last segment of the range begin / end inside it?
   __device__ __forceinline__ SegRange(const int64_t* __restrict__ seg_ids, const int64_t* __restrict__ ptr,
-                                      const int32_t* __restrict__ wave_seg, int64_t wave, int per_wave,
-                                      int64_t n_rows) {
+                                      const int32_t* __restrict__ wave_seg, const int64_t* __restrict__ wave_pos,
+                                      int64_t wave, int per_wave, int64_t n_rows) {
     if (wave_seg) {
       s0 = wave_seg[wave];
       s1 = wave_seg[wave + 1];
@@ -178,8 +181,13 @@ struct SegRange {
       first_complete = last_complete = true;
     } else {
       s0 = s1 = -1;
-      p0 = wave * per_wave;
-      p1 = p0 + per_wave < n_rows ? p0 + per_wave : n_rows;
+      if (wave_pos) {
+        p0 = wave_pos[wave];
+        p1 = wave_pos[wave + 1];
+      } else {
+        p0 = wave * per_wave;
+        p1 = p0 + per_wave < n_rows ? p0 + per_wave : n_rows;
+      }
       first_complete = p0 == 0 || seg_ids[p0 - 1] != seg_ids[p0];
       last_complete = p1 == n_rows || seg_ids[p1 - 1] != seg_ids[p1];
     }
@@ -286,7 +294,7 @@ __global__ void __launch_bounds__(256) uvu_seg_fwd_kernel(const UvuDev<T> a, int
   const int c0 = L.cl * V;
   const bool cok = c0 < a.C;
   const int64_t C = a.C;
-  const SegRange R(a.seg_ids, a.ptr, a.wave_seg, wave, a.pos_per_wave, a.n_rows);
+  const SegRange R(a.seg_ids, a.ptr, a.wave_seg, a.wave_pos, wave, a.pos_per_wave, a.n_rows);
 
   T acc[DO][V];
   zero_rows(acc);
@@ -341,7 +349,7 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, 
   const int c0 = L.cl * V;
   const bool cok = c0 < a.C;
   const int64_t C = a.C;
-  const SegRange R(a.seg_ids, a.ptr, a.wave_seg, wave, a.pos_per_wave, a.n_rows);
+  const SegRange R(a.seg_ids, a.ptr, a.wave_seg, a.wave_pos, wave, a.pos_per_wave, a.n_rows);
 
   T gwacc[GW == kGwReduce ? P : 1][V], acc[D1][V];
   zero_rows(gwacc);
@@ -456,10 +464,23 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, 
 
 // Rows of segments cut by a wavefront boundary: rows[v] = sum of the partial rows of the wavefronts that
 // touch v, in ascending wavefront order; rows of empty segments are zeroed.  One wavefront per segment.
+// wave_pos (n_waves + 1 ascending positions) when the ranges were cut at given positions, else per_wave each.
+__device__ __forceinline__ int64_t range_of_position(const int64_t* __restrict__ wave_pos, int64_t n_waves, int per_wave,
+                                                     int64_t q) {
+  if (!wave_pos) return q / per_wave;
+  int64_t lo = 0, hi = n_waves - 1;   // largest k with wave_pos[k] <= q
+  while (lo < hi) {
+    const int64_t mid = (lo + hi + 1) >> 1;
+    if (wave_pos[mid] <= q) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256) uvu_fixup_kernel(T* __restrict__ rows, const T* __restrict__ ws,
                                                         const int64_t* __restrict__ ptr, int64_t n_seg,
-                                                        int64_t row_len, int per_wave) {
+                                                        int64_t row_len, int per_wave,
+                                                        const int64_t* __restrict__ wave_pos, int64_t n_waves) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t v = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
   if (v >= n_seg) return;
@@ -469,9 +490,11 @@ __global__ void __launch_bounds__(256) uvu_fixup_kernel(T* __restrict__ rows, co
     for (int64_t i = lane; i < row_len; i += kWave) dst[i] = T(0);
     return;
   }
-  const int64_t ka = b / per_wave, kb = (e - 1) / per_wave;
+  const int64_t ka = range_of_position(wave_pos, n_waves, per_wave, b);
+  const int64_t kb = range_of_position(wave_pos, n_waves, per_wave, e - 1);
   if (ka == kb) return;  // written in full by wavefront ka
-  const int64_t slot_a = (b % per_wave == 0) ? 0 : 1;
+  const int64_t first_a = wave_pos ? wave_pos[ka] : ka * per_wave;
+  const int64_t slot_a = (b == first_a) ? 0 : 1;
   for (int64_t i = lane; i < row_len; i += kWave) {
     T s = ws[(ka * 2 + slot_a) * row_len + i];
     for (int64_t k = ka + 1; k <= kb; ++k) s += ws[(k * 2) * row_len + i];
@@ -654,7 +677,8 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
   if (!seg && (a->ptr || a->perm || a->seg_ids)) return CGTP_ERR_SHAPE;
   if (seg && (a->n_seg >= (int64_t)1 << 31 || a->n_rows >= (int64_t)1 << 31 || a->n_x_rows >= (int64_t)1 << 31))
     return CGTP_ERR_SHAPE;  // segment mode keeps ids and rows in 32-bit registers
-  if (seg && a->wave_seg && a->n_waves <= 0) return CGTP_ERR_SHAPE;
+  if (seg && (a->wave_seg || a->wave_pos) && a->n_waves <= 0) return CGTP_ERR_SHAPE;
+  if (seg && a->wave_seg && a->wave_pos) return CGTP_ERR_SHAPE;
   if (a->y_vec) {  // harmonics evaluated in the kernel: fused segment kernels of a config laid out for them
     if (a->y_vec != kYUnitVector && a->y_vec != kYRawVector) return CGTP_ERR_SHAPE;
     if (!seg) return CGTP_ERR_SHAPE;
@@ -703,6 +727,9 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
   plan->pos_per_wave = 0;
   if (seg && a->wave_seg) {
     plan->n_waves = a->n_waves;  // segment-aligned ranges: every row is final, no partial rows
+  } else if (seg && a->wave_pos) {
+    plan->n_waves = a->n_waves;  // ranges cut at given positions: partial rows as for ranges by position
+    if (!backward || a->grad_x) plan->ws_elems = plan->n_waves * 2 * row_d * a->C;
   } else if (seg) {
     int ppw = a->pos_per_wave > 0 ? a->pos_per_wave : kDefaultPosPerWave;
     ppw = ((ppw + slots - 1) / slots) * slots;
@@ -737,6 +764,7 @@ static UvuDev<T> to_dev(const cgtp_uvu_args* a, const UvuPlan& plan) {
   d.ws = (T*)a->workspace;
   d.wsw = d.ws ? d.ws + plan.ws_elems : nullptr;
   d.ptr = a->ptr; d.perm = a->perm; d.gather = a->gather; d.x_gather = a->x_gather; d.seg_ids = a->seg_ids; d.wave_seg = a->wave_seg;
+  d.wave_pos = a->wave_pos; d.n_waves = plan.n_waves;
   d.n_rows = a->n_rows; d.n_seg = a->n_seg;
   d.C = a->C; d.lpe_log2 = plan.lpe_log2; d.w_shared = a->w_shared; d.pos_per_wave = plan.pos_per_wave;
   d.y_vec = a->y_vec;
@@ -756,7 +784,7 @@ static inline int launched() { return hipGetLastError() == hipSuccess ? CGTP_OK 
 template <typename T>
 static int launch_fixup(T* rows, const UvuDev<T>& d, int64_t row_len, hipStream_t stream) {
   hipLaunchKernelGGL(uvu_fixup_kernel<T>, dim3((unsigned)((d.n_seg + 3) / 4)), dim3(256), 0, stream, rows,
-                     (const T*)d.ws, d.ptr, d.n_seg, row_len, d.pos_per_wave);
+                     (const T*)d.ws, d.ptr, d.n_seg, row_len, d.pos_per_wave, d.wave_pos, d.n_waves);
   return launched();
 }
 
@@ -950,6 +978,20 @@ int cgtp_uvu_radial_supported(int cfg) {
   int n = 0;
   const UvuRadialEntry* t = uvu_radial_entries(&n);
   return cfg >= 0 && cfg < n && t[cfg].fwd[0] != nullptr;
+}
+
+int cgtp_uvu_slots(int cfg, int dtype, int C, int backward) {
+  int n = 0, n64 = 0;
+  const UvuEntry<float>* t = entries<float>(&n);
+  const UvuEntry<double>* t64 = entries<double>(&n64);
+  if (cfg < 0 || cfg >= n || C <= 0 || (dtype != CGTP_F32 && dtype != CGTP_F64)) return 0;
+  int vw = dtype == CGTP_F32 ? (backward ? t[cfg].v_bwd : t[cfg].v_fwd) : (backward ? t64[cfg].v_bwd : t64[cfg].v_fwd);
+  if (C % vw) vw = 1;
+  const int lanes = (C + vw - 1) / vw;
+  if (lanes > kWave) return 0;
+  int lg = 0;
+  while ((1 << lg) < lanes) ++lg;
+  return kWave >> lg;
 }
 
 int cgtp_uvu_validate(const cgtp_uvu_args* args, int backward) {

@@ -78,7 +78,7 @@ __global__ void __launch_bounds__(256) uvu_seg_fwd_radial_kernel(const UvuDev<fl
   if (wave < 0) return;
   const int c0 = L.cl * V;
   constexpr int64_t C = kRadialC;
-  const SegRange R(a.seg_ids, a.ptr, a.wave_seg, wave, a.pos_per_wave, a.n_rows);
+  const SegRange R(a.seg_ids, a.ptr, a.wave_seg, a.wave_pos, wave, a.pos_per_wave, a.n_rows);
 
   T acc[DO][V];
   zero_rows(acc);
@@ -126,7 +126,7 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_radial_kernel(const UvuDev
   if (wave < 0) return;
   const int c0 = L.cl * V;
   constexpr int64_t C = kRadialC;
-  const SegRange R(a.seg_ids, a.ptr, a.wave_seg, wave, a.pos_per_wave, a.n_rows);
+  const SegRange R(a.seg_ids, a.ptr, a.wave_seg, a.wave_pos, wave, a.pos_per_wave, a.n_rows);
 
   T acc[D1][V];
   zero_rows(acc);

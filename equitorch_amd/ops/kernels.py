@@ -438,13 +438,23 @@ def wigner_rotate_backward(x: Tensor, grad_out: Tensor, sincos, layout: Rotation
 
 
 # ---- specialised uvu ----------------------------------------------------------------------------------------
+# How the sorted edge list is cut into one range per wavefront: "aligned" (at segment boundaries, no partial rows),
+# "balanced" (after equal numbers of steps), "positions" (after equal numbers of positions), or "auto": measured on the
+# lmax = 2, C = 64 edge workload, the forward is fastest on aligned ranges (0.061 ms against 0.071 / 0.066) and the
+# backward, whose steps are three times as long, on balanced ones (0.115 ms against 0.122 / 0.118).
+_RANGE_MODE = __import__("os").environ.get("CGTP_RANGE_MODE", "auto")
+
+
 class SegIndex:
-    """Per-sorted-position index arrays of the segment mode (all int64, same device)."""
+    """Per-sorted-position index arrays of the segment mode (all int64, same device), and the tables that cut the
+    sorted list into one range per wavefront."""
 
     def __init__(self, ptr: Tensor, perm: Optional[Tensor], seg_ids: Tensor, gather: Tensor,
                  positions_per_wave: int = int(__import__("os").environ.get("CGTP_POSITIONS_PER_WAVE", "32"))):
         self.ptr, self.perm, self.seg_ids, self.gather = ptr, perm, seg_ids, gather
+        self.positions_per_wave = positions_per_wave
         self.wave_seg = self.aligned_ranges(ptr, positions_per_wave)
+        self._wave_pos = {}
 
     @staticmethod
     def aligned_ranges(ptr: Tensor, positions_per_wave: int) -> Optional[Tensor]:
@@ -462,9 +472,37 @@ class SegIndex:
         cuts = torch.unique_consecutive(torch.cat([cuts.new_zeros(1), cuts, cuts.new_full((1,), n_seg)]))
         return cuts.to(torch.int32).contiguous()
 
+    def balanced_positions(self, slots: int) -> Optional[Tensor]:
+        """Cut the sorted list after equal numbers of steps: a wavefront takes up to ``slots`` positions of one segment
+        per step, so a segment of n positions costs ceil(n / slots) steps wherever it lies, and a range that holds
+        whole steps only costs exactly its share.  int64 ``[n_ranges + 1]`` positions (first 0, last n_pos), cuts on
+        step boundaries; as many ranges as ``positions_per_wave`` positions each would give.  The time of a wavefront follows its number of
+        steps, and ranges cut at segment boundaries differ in it by a factor of up to five on a graph of average
+        degree 16."""
+        if slots <= 0:
+            return None
+        if slots not in self._wave_pos:
+            ptr = self.ptr
+            n_pos = int(ptr[-1])
+            if n_pos == 0:
+                self._wave_pos[slots] = None
+            else:
+                steps = (ptr[1:] - ptr[:-1] + slots - 1) // slots
+                last = torch.cumsum(steps, 0)                      # steps up to and including each segment
+                first = last - steps
+                # as many ranges as equal cuts by position would give (a launch sized for that many wavefronts
+                # stays resident in one round)
+                n_ranges = max(1, n_pos // self.positions_per_wave)
+                per_wave = max(1, -(-int(last[-1]) // n_ranges))
+                targets = torch.arange(0, int(last[-1]), per_wave, device=ptr.device, dtype=ptr.dtype)
+                seg = torch.searchsorted(last, targets, right=True)
+                pos = ptr[:-1][seg] + (targets - first[seg]) * slots
+                self._wave_pos[slots] = torch.cat([pos, pos.new_full((1,), n_pos)]).contiguous()
+        return self._wave_pos[slots]
+
 
 def _uvu_args(cfg: int, x: Tensor, y: Tensor, w: Tensor, seg: Optional[SegIndex], gather: Optional[Tensor],
-              pos_per_wave: int = 0, y_vec: int = 0) -> UvuArgs:
+              pos_per_wave: int = 0, y_vec: int = 0, backward: bool = False) -> UvuArgs:
     a = UvuArgs()
     a.y_vec = y_vec
     a.y_channels = int(y.ndim == 3)
@@ -476,8 +514,14 @@ def _uvu_args(cfg: int, x: Tensor, y: Tensor, w: Tensor, seg: Optional[SegIndex]
         a.ptr, a.perm, a.seg_ids, a.gather = seg.ptr.data_ptr(), _lib.ptr(seg.perm), seg.seg_ids.data_ptr(), \
             seg.gather.data_ptr()
         a.pos_per_wave = pos_per_wave
-        if seg.wave_seg is not None and pos_per_wave == 0:
-            a.wave_seg, a.n_waves = seg.wave_seg.data_ptr(), seg.wave_seg.shape[0] - 1
+        if pos_per_wave == 0:
+            wave_pos = None
+            if _RANGE_MODE == "balanced" or (_RANGE_MODE == "auto" and (backward or seg.wave_seg is None)):
+                wave_pos = seg.balanced_positions(int(_lib.lib.cgtp_uvu_slots(int(cfg), a.dtype, a.C, int(backward))))
+            if wave_pos is not None:
+                a.wave_pos, a.n_waves = wave_pos.data_ptr(), wave_pos.shape[0] - 1
+            elif seg.wave_seg is not None and _RANGE_MODE != "positions":
+                a.wave_seg, a.n_waves = seg.wave_seg.data_ptr(), seg.wave_seg.shape[0] - 1
     else:
         a.gather = _lib.ptr(gather)
     a.x, a.y, a.w = x.data_ptr(), y.data_ptr(), w.data_ptr()
@@ -546,7 +590,7 @@ def uvu_backward(cfg: int, dims, x: Tensor, y: Tensor, w: Tensor, g: Tensor, nee
     picks the row of ``g`` and ``x_gather`` the row of ``x`` of every batch row; with ``x_gather`` the returned
     grad_x is per batch row, ``(n_rows, D1, C)``."""
     w = expand_paths(w, cfg, -2)
-    a = _uvu_args(cfg, x, y, w, seg, gather, pos_per_wave, y_vec)
+    a = _uvu_args(cfg, x, y, w, seg, gather, pos_per_wave, y_vec, backward=True)
     a.grad_out = g.data_ptr()
     a.x_gather = _lib.ptr(x_gather)
     if not need[0]:
@@ -601,7 +645,7 @@ def uvu_radial_backward(cfg: int, dims, x: Tensor, y: Tensor, h: Tensor, w_eff: 
                         seg: SegIndex, y_vec: int = 0):
     """-> (grad_x, grad_y, grad_h, grad_w_eff).  The segment kernel regenerates the weights and writes the per-edge
     weight gradient; ``cgtp_uvu_radial_grad`` contracts it with ``w_eff`` and ``h`` in one pass."""
-    a = _uvu_args(Cfg(int(cfg)), x, y, h, seg, None, 0, y_vec)
+    a = _uvu_args(Cfg(int(cfg)), x, y, h, seg, None, 0, y_vec, backward=True)
     a.w, a.w_shared, a.path_scale = None, 0, None
     a.radial_h, a.radial_w, a.radial_r = h.data_ptr(), w_eff.data_ptr(), h.shape[1]
     a.grad_out = g.data_ptr()

@@ -167,8 +167,9 @@ int cgtp_segment_sum(const void* in, const void* scale, const int64_t* index, co
  * seg_ids.  The sorted list is cut into one range per wavefront in one of two ways.  With wave_seg (n_waves + 1
  * ascending segment indices, first 0, last n_seg) wavefront k owns the whole segments [wave_seg[k],
  * wave_seg[k+1]) and writes their rows directly (zero rows for empty segments); the caller balances the ranges
- * (about 32 positions each works well).  Without it every wavefront owns pos_per_wave consecutive positions and
- * segments cut by a range boundary go through partial rows in the workspace and a fix-up kernel.  Either way
+ * (about 32 positions each works well).  Without it every wavefront owns pos_per_wave consecutive positions, or the
+ * positions between two entries of wave_pos, and segments cut by a range boundary go through partial rows in the
+ * workspace and a fix-up kernel.  Either way
  * there are no atomics and results are deterministic.
  */
 int cgtp_uvu_num_configs(void);
@@ -242,6 +243,11 @@ typedef struct cgtp_uvu_args {
   const void* radial_w;    /* (radial_r, P, C)                                                    */
   int32_t radial_r;
   int32_t reserved2_;
+  const int64_t* wave_pos; /* segment mode, optional (not together with wave_seg): [n_waves + 1] ascending sorted
+                              positions, first 0, last n_rows, strictly increasing: wavefront k walks positions
+                              wave_pos[k] .. wave_pos[k + 1].  Cuts may fall inside segments (partial rows in the
+                              workspace, as without any table); cutting after equal numbers of steps —
+                              cgtp_uvu_slots() positions of one segment per step — keeps the wavefronts equally long */
 } cgtp_uvu_args;
 
 /* 1 if config `cfg` has segment kernels that produce the weights themselves (cgtp_uvu_args.radial_h). */
@@ -258,6 +264,9 @@ int cgtp_uvu_radial_grad(const void* grad_w, const void* radial_h, const void* r
                          void* grad_radial_w, void* workspace, int64_t n_rows, int32_t radial_r, int32_t n_paths,
                          int32_t dtype, void* stream);
 
+/* Positions of one segment a wavefront takes per step (64 / lanes per edge) in a segment-mode launch of config
+ * `cfg` with C channels and aligned operands; 0 if there is no such launch.  Host only. */
+int cgtp_uvu_slots(int cfg, int dtype, int C, int backward);
 int cgtp_uvu_validate(const cgtp_uvu_args* args, int backward);
 /* Bytes of workspace the forward (backward = 0) or backward (1) launch of `args` needs; 0 if none. */
 int64_t cgtp_uvu_workspace_bytes(const cgtp_uvu_args* args, int backward);

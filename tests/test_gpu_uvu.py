@@ -373,3 +373,42 @@ def test_u1u_so3_lmax4_reference_test_irreps(device):
             # up to 61 paths x hundreds of coefficients per element, inputs not normalised: norm-wise for the sums
             assert_close(a, b, 1e-5, f"so3 lmax=4 path_norm={path_norm} {name}",
                          norm="element" if name == "grad_w" else "max")
+
+
+@pytest.mark.parametrize("hub", [False, True])
+def test_edge_fused_ranges_balanced_by_steps(device, hub):
+    """Ranges cut after equal numbers of steps (``cgtp_uvu_args.wave_pos``; cuts inside segments, partial rows and
+    the fix-up kernel) give the rows of segment-aligned ranges, forward and backward, also with a hub node whose
+    segment spans many wavefronts and with empty segments."""
+    from equitorch_amd.nn.functional import EdgePlan
+    from equitorch_amd.ops import kernels
+    irreps = SH[2]
+    mod = _module(irreps, irreps, irreps).to(device)
+    cfg = kernels.uvu_config_of(mod.tp_info_forward)
+    dims = kernels.uvu_dims(cfg)
+    gen = torch.Generator().manual_seed(19)
+    n_nodes, n_edges, ch = 83, 2100, 64
+    src = torch.randint(0, n_nodes, (n_edges,), generator=gen)
+    dst = torch.randint(0, n_nodes - 2, (n_edges,), generator=gen)
+    if hub:
+        dst[100:900] = 17
+        src[300:1200] = 5
+    x, sh, w = tp_inputs(n_edges, 9, 2, 11, ch, False, seed=20)
+    x = x[:n_nodes].contiguous()
+    ct = torch.randn(n_nodes, 9, ch, generator=gen)
+    plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
+    xd, shd, wd, ctd = (t.to(device) for t in (x, sh, w, ct))
+    results = {}
+    for mode in ("aligned", "balanced"):
+        kernels._RANGE_MODE = mode
+        try:
+            out = kernels.uvu_forward(cfg, dims, xd, shd, wd, seg=plan.fwd_index)
+            grads = kernels.uvu_backward(cfg, dims, xd, shd, wd, ctd, (True, True, True), seg=plan.bwd_index)
+        finally:
+            kernels._RANGE_MODE = "auto"
+        results[mode] = (out, *grads)
+    wave_pos = plan.bwd_index.balanced_positions(4)
+    assert wave_pos[0] == 0 and wave_pos[-1] == n_edges and bool((wave_pos[1:] > wave_pos[:-1]).all())
+    for name, a, b in zip(("out", "grad_x", "grad_sh", "grad_w"), results["balanced"], results["aligned"]):
+        # per-edge results are the same numbers; node rows cut by a range boundary are summed in another order
+        assert_close(a, b, 1e-5, f"balanced vs aligned hub={hub} {name}")
