@@ -1,4 +1,7 @@
-"""Irreps-preserving channel mixing (``IrrepsLinear`` / ``IrrepWiseLinear``) as library GEMMs on strided views.
+"""Irreps-preserving channel mixing (``IrrepsLinear`` / ``IrrepWiseLinear``).  With a shared weight the layer runs on
+the hand-written matrix-core kernels of the fully connected product (bf16: compiled tables; fp32: table-driven) as a
+product with the scalar 1; per-sample weights, fp64, higher-order gradients and shapes those kernels do not take run
+as library GEMMs on strided views:
 
 The reference runs these layers on its table-driven vector-matrix kernels (``indexed_vecmat_scale_segment`` plus
 a scatter, ``equitorch/nn/functional/linears.py:494-571``).  The tables have a simple structure: a path couples
@@ -370,6 +373,41 @@ def _matrix_core_path(x: Tensor, weight: Tensor, plan: LinearPlan, in_size: int,
     return _uvw_mfma.try_forward(x, ones, weight, info)
 
 
+def _table_driven_path(x: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anchor: Tensor):
+    """fp32 with a shared weight: the layer as a fully connected product with the scalar 1 on the table-driven
+    matrix-core kernels (``cgtp_uvt_*``: forward, grad input and grad weight in one launch each, rows read and written
+    in place), when the product's table reproduces the plan's scales; None otherwise."""
+    from ...ops import kernels
+    from . import _uv_native
+    if x.dtype != torch.float32 or weight.ndim != 3 or x.shape[0] == 0:
+        return None
+
+    def build():
+        info = _as_tensor_product(plan, in_size)
+        if info is None:
+            return False
+        c = kernels.coo_of(info)
+        for m, m1, m2, p, coef in zip(c.M, c.M1, c.M2, c.p, c.coef):
+            path = plan.paths[int(p)]
+            if m2 != 0 or m - path.o0 != m1 - path.i0 or not 0 <= m - path.o0 < path.k:
+                return False
+            if abs(float(coef) - path.scale) > 1e-6 * max(1.0, abs(path.scale)):
+                return False
+        if len(c.coef) != sum(pt.k for pt in plan.paths):
+            return False
+        return info.to(x.device)
+
+    info = cached(anchor, ("linear_as_tp_fp32", in_size, str(x.device)), build)
+    if info is False:
+        return None
+    ones = cached(anchor, ("ones_fp32", x.shape[0], str(x.device)),
+                  lambda: torch.ones(x.shape[0], 1, dtype=torch.float32, device=x.device))
+    if not _uv_native.u1v_supported(x, ones, weight, info):
+        return None
+    kernels.log_tier("irreps_linear", "table-driven matrix-core kernels (fp32)")
+    return _uv_native.u1v(x, ones, weight, info)
+
+
 def mix(input: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anchor: Tensor = None) -> Tensor:
     """``(..., D_in, C_in) x (P, C_in, C_out) | (N, P, C_in, C_out) -> (..., D_out, C_out)``."""
     _lib.require_gpu(input, weight)
@@ -385,6 +423,8 @@ def mix(input: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anchor: T
     if weight.ndim == 4 and weight.shape[0] != x.shape[0]:
         raise _lib.CgtpError(f"per-sample weight has {weight.shape[0]} samples, input has {x.shape[0]}")
     out = _matrix_core_path(x, weight, plan, in_size, anchor) if anchor is not None else None
+    if out is None and anchor is not None:
+        out = _table_driven_path(x, weight, plan, in_size, anchor)
     if out is None:
         out = _Mix.apply(x, weight, plan, False, in_size)
     return out.reshape(*lead, plan.out_size, out.shape[-1])
