@@ -54,6 +54,12 @@ WORKLOADS = {
     # fully connected product on the matrix cores (BASELINE configs[3]): (lmax, C_in = C_out, batch)
     "uvw_fwd": (3, 128, 32768),
     "uvw_fwd_bwd": (3, 128, 32768),
+    # the same products in fp32 on the table-driven matrix-core kernels: SO3Linear('uv') at the configs[3] shape, and
+    # TensorProduct('uvw') with (lmax, U = V = W, batch)
+    "u1v_fp32_fwd_bwd": (3, 128, 32768),
+    "uvw_fp32_fwd_bwd": (2, 32, 32768),
+    # the headline edge workload with the per-edge weights formed inside the kernels from 16 features per edge
+    "edge_radial_fwd_bwd": (2, 64, 4096, 65536),
     # streaming kernels of known traffic (1 GiB): counter calibration and achievable-bandwidth reference
     "copy": None,
     "read": None,
@@ -746,6 +752,19 @@ def main():
     if args.workload == "edge_l6_fwd_bwd":
         print(json.dumps(edge_rows_bench(args)))
         return
+    if args.workload in ("u1v_fp32_fwd_bwd", "uvw_fp32_fwd_bwd"):
+        print(json.dumps(fp32_fully_connected_bench(args)))
+        return
+    if args.workload == "edge_radial_fwd_bwd":
+        r = radial_record(16)
+        print(json.dumps({
+            "metric": "edge-TP fwd+bwd Medges/s (lmax=2,C=64, weights formed in the kernels, R=16)",
+            "value": r["Medges_s"], "unit": "Medges/s", "n_gpus": 1, "steps": 20, "warmup": 3,
+            "ms_per_step": r["step_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "edge_radial_fwd_bwd: N=4096 nodes, E=65536 edges, irreps 0e+1o+2e, C=64, "
+                                   "h (E,16), W_last (16,11,64)"}, "kernels": r}))
+        return
 
     from equitorch_amd.nn import SO3Linear
     from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu
@@ -877,6 +896,96 @@ def other_configs(args, headline):
         "bwd_ms": r["kernels"]["bwd_ms"], "bwd_hbm_frac": r["roofline"]["frac"],
         "bwd_fp32_frac": r["roofline"]["fp32_vector"]["frac"], "fwd_TFLOPs": r["kernels"]["fwd_TFLOPs"]}
     return out
+
+
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X fp32 matrix, vendor figure
+
+
+def fp32_fully_connected_bench(args):
+    """``SO3Linear('uv')`` (u1v) or ``TensorProduct('uvw')`` with a shared fp32 weight, forward + backward through the
+    public autograd API, and every kernel of the step on its own.  Algorithmic flops per product: 2 * B * S * K * C_out
+    (S (path, output row) segments, K contracted channels; the coupling is not counted); the step has four."""
+    from equitorch_amd.nn import SO3Linear, TensorProduct
+    from equitorch_amd.nn.functional import _uv_native
+    from equitorch_amd.utils._sh import spherical_harmonics
+    lmax, ch, n = WORKLOADS[args.workload]
+    uvw = args.workload.startswith("uvw")
+    dev = torch.device("cuda:0")
+    irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+    d = (lmax + 1) ** 2
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(n, d, ch, generator=gen).to(dev)
+    ct = torch.randn(n, d, ch, generator=gen).to(dev)
+    if uvw:
+        mod = TensorProduct(irreps, irreps, irreps, ch, ch, ch, feature_mode="uvw", internal_weights=False).to(dev)
+        y = torch.randn(n, d, ch, generator=gen).to(dev)
+        w = (torch.randn(mod.num_paths, ch, ch, ch, generator=gen) / ch).to(dev)
+        k = ch * ch
+    else:
+        mod = SO3Linear(irreps, irreps, irreps, ch, ch, internal_weights=False, feature_mode="uv").to(dev)
+        vec = torch.randn(n, 3, generator=gen)
+        y = spherical_harmonics(vec / vec.norm(dim=-1, keepdim=True), lmax).to(dev)
+        w = (torch.randn(mod.num_paths, ch, ch, generator=gen) / (ch * mod.num_paths) ** 0.5).to(dev)
+        k = ch
+    info = mod.tp_info_forward
+    s1 = int(info.info_Mij_fwd.out_size)
+    flops = 2.0 * n * s1 * k * ch
+    xg, yg, wg = (t.clone().requires_grad_(True) for t in (x, y, w))
+
+    def step():
+        return torch.autograd.grad(mod(xg, yg, wg), (xg, yg, wg), ct)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) / args.steps * 1e3
+
+    def timed(fn):
+        evs = []
+        for _ in range(args.kernel_reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(); fn(); b.record()
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        return sum(a.elapsed_time(b) for a, b in evs[2:]) / (len(evs) - 2)
+    p = mod.num_paths
+    if uvw:
+        wp = _uv_native.pack(w, p, k, ch, k * ch, ch, 1)
+        wt1 = w.permute(0, 2, 3, 1).contiguous()
+        wp1 = _uv_native.pack(wt1, p, k, ch, k * ch, ch, 1)
+        wt2 = w.permute(0, 3, 1, 2).contiguous()
+        wp2 = _uv_native.pack(wt2, p, k, ch, k * ch, ch, 1)
+        kern = {
+            "fwd_ms": timed(lambda: _uv_native.apply(x, y, wp, info, "out", d, ch)),
+            "grad_x_ms": timed(lambda: _uv_native.apply(y, ct, wp1, info, "in1_uvw", d, ch)),
+            "grad_y_ms": timed(lambda: _uv_native.apply(ct, x, wp2, info, "in2_uvw", d, ch)),
+            "grad_w_ms": timed(lambda: _uv_native.grad_w(x, y, ct, info)),
+        }
+    else:
+        wp = _uv_native.pack(w, p, ch, ch, ch * ch, ch, 1)
+        wpt = _uv_native.pack(w, p, ch, ch, ch * ch, 1, ch)
+        kern = {
+            "fwd_ms": timed(lambda: _uv_native.apply(x, y, wp, info, "out", d, ch)),
+            "grad_x_ms": timed(lambda: _uv_native.apply(ct, y, wpt, info, "in1", d, ch)),
+            "grad_y_ms": timed(lambda: _uv_native.grad_y(x, ct, wp, info, d)),
+            "grad_w_ms": timed(lambda: _uv_native.grad_w(x, y, ct, info)),
+        }
+    tf = {key: flops / (v * 1e-3) / 1e12 for key, v in kern.items()}
+    name = "uvw" if uvw else "u1v"
+    return {
+        "metric": f"{name} fp32 fwd+bwd TFLOP/s (lmax={lmax},C={ch})", "value": round(4 * flops / (ms_step * 1e-3) / 1e12, 2),
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: B={n}, irreps {irreps}, channels {ch}, shared weight {tuple(w.shape)}, "
+                               f"forward + backward through the module"},
+        "roofline": {"bound": "mfma", "kernel": "cgtp::uvt_apply_kernel (forward)", "achieved": round(tf["fwd_ms"], 2),
+                     "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf["fwd_ms"] / FP32_MFMA_PEAK_TFLOPS, 4),
+                     "traffic": None, "algorithmic_flops": flops, "avg_ms": round(kern["fwd_ms"], 5)},
+        "kernels": {**{key: round(v, 5) for key, v in kern.items()},
+                    **{key.replace("_ms", "_mfma_frac"): round(v / FP32_MFMA_PEAK_TFLOPS, 4) for key, v in tf.items()}}}
 
 
 def radial_record(r):

@@ -465,9 +465,20 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, 
 // Rows of segments cut by a wavefront boundary: rows[v] = sum of the partial rows of the wavefronts that
 // touch v, in ascending wavefront order; rows of empty segments are zeroed.  One wavefront per segment.
 // wave_pos (n_waves + 1 ascending positions) when the ranges were cut at given positions, else per_wave each.
+// Called by all lanes of a wavefront with the same q.  Ranges cut at given positions are about equally long, so the
+// answer lies near q * n_waves / n_rows: the wavefront looks at 64 consecutive entries around that guess with one
+// coalesced load (a binary search is eleven dependent loads at 2048 ranges, and this kernel does little else) and
+// falls back to the search when the window misses.
 __device__ __forceinline__ int64_t range_of_position(const int64_t* __restrict__ wave_pos, int64_t n_waves, int per_wave,
-                                                     int64_t q) {
+                                                     int64_t n_rows, int64_t q, int lane) {
   if (!wave_pos) return q / per_wave;
+  int64_t base = q * n_waves / n_rows - 32;
+  if (base > n_waves - 63) base = n_waves - 63;
+  if (base < 0) base = 0;
+  const int64_t idx = base + lane;
+  const bool le = idx <= n_waves && wave_pos[idx] <= q;      // entries are ascending: a prefix of the lanes
+  const int cnt = __popcll(__ballot(le));
+  if (cnt > 0 && (cnt < kWave || base + kWave > n_waves)) return base + cnt - 1;
   int64_t lo = 0, hi = n_waves - 1;   // largest k with wave_pos[k] <= q
   while (lo < hi) {
     const int64_t mid = (lo + hi + 1) >> 1;
@@ -480,7 +491,8 @@ template <typename T>
 __global__ void __launch_bounds__(256) uvu_fixup_kernel(T* __restrict__ rows, const T* __restrict__ ws,
                                                         const int64_t* __restrict__ ptr, int64_t n_seg,
                                                         int64_t row_len, int per_wave,
-                                                        const int64_t* __restrict__ wave_pos, int64_t n_waves) {
+                                                        const int64_t* __restrict__ wave_pos, int64_t n_waves,
+                                                        int64_t n_rows) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t v = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
   if (v >= n_seg) return;
@@ -490,8 +502,8 @@ __global__ void __launch_bounds__(256) uvu_fixup_kernel(T* __restrict__ rows, co
     for (int64_t i = lane; i < row_len; i += kWave) dst[i] = T(0);
     return;
   }
-  const int64_t ka = range_of_position(wave_pos, n_waves, per_wave, b);
-  const int64_t kb = range_of_position(wave_pos, n_waves, per_wave, e - 1);
+  const int64_t ka = range_of_position(wave_pos, n_waves, per_wave, n_rows, b, lane);
+  const int64_t kb = range_of_position(wave_pos, n_waves, per_wave, n_rows, e - 1, lane);
   if (ka == kb) return;  // written in full by wavefront ka
   const int64_t first_a = wave_pos ? wave_pos[ka] : ka * per_wave;
   const int64_t slot_a = (b == first_a) ? 0 : 1;
@@ -784,7 +796,7 @@ static inline int launched() { return hipGetLastError() == hipSuccess ? CGTP_OK 
 template <typename T>
 static int launch_fixup(T* rows, const UvuDev<T>& d, int64_t row_len, hipStream_t stream) {
   hipLaunchKernelGGL(uvu_fixup_kernel<T>, dim3((unsigned)((d.n_seg + 3) / 4)), dim3(256), 0, stream, rows,
-                     (const T*)d.ws, d.ptr, d.n_seg, row_len, d.pos_per_wave, d.wave_pos, d.n_waves);
+                     (const T*)d.ws, d.ptr, d.n_seg, row_len, d.pos_per_wave, d.wave_pos, d.n_waves, d.n_rows);
   return launched();
 }
 
