@@ -376,36 +376,35 @@ def _matrix_core_path(x: Tensor, weight: Tensor, plan: LinearPlan, in_size: int,
 def _table_driven_path(x: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anchor: Tensor):
     """fp32 with a shared weight: the layer as a fully connected product with the scalar 1 on the table-driven
     matrix-core kernels (``cgtp_uvt_*``: forward, grad input and grad weight in one launch each, rows read and written
-    in place), when the product's table reproduces the plan's scales; None otherwise."""
+    in place): every path of the plan becomes ``k`` table entries (output row, input row, 0, weight, scale).  None
+    when the extents do not fit those kernels."""
+    import numpy as np
+
+    from ..._tables import TpCoo
     from ...ops import kernels
     from . import _uv_native
     if x.dtype != torch.float32 or weight.ndim != 3 or x.shape[0] == 0:
         return None
 
     def build():
-        info = _as_tensor_product(plan, in_size)
-        if info is None:
+        rows = [(p.o0 + j, p.i0 + j, p.w, p.scale) for p in plan.paths for j in range(p.k)]
+        if not rows:
             return False
-        c = kernels.coo_of(info)
-        for m, m1, m2, p, coef in zip(c.M, c.M1, c.M2, c.p, c.coef):
-            path = plan.paths[int(p)]
-            if m2 != 0 or m - path.o0 != m1 - path.i0 or not 0 <= m - path.o0 < path.k:
-                return False
-            if abs(float(coef) - path.scale) > 1e-6 * max(1.0, abs(path.scale)):
-                return False
-        if len(c.coef) != sum(pt.k for pt in plan.paths):
-            return False
-        return info.to(x.device)
+        m, m1, pw, sc = (np.asarray(v) for v in zip(*rows))
+        zeros = np.zeros(len(rows), dtype=np.int32)
+        coo = TpCoo(sc.astype(np.float64), m.astype(np.int32), m1.astype(np.int32), zeros, pw.astype(np.int32), zeros,
+                    int(in_size), 1, int(plan.out_size), int(plan.n_paths))
+        return _uv_native.CooTable(coo, anchor, lambda xx, yy, ww: _Mix.apply(xx, ww, plan, False, in_size) * yy[:, :, None])
 
-    info = cached(anchor, ("linear_as_tp_fp32", in_size, str(x.device)), build)
-    if info is False:
+    table = cached(anchor, ("linear_as_coo_table", in_size, plan.n_paths, plan.out_size), build)
+    if table is False:
         return None
     ones = cached(anchor, ("ones_fp32", x.shape[0], str(x.device)),
                   lambda: torch.ones(x.shape[0], 1, dtype=torch.float32, device=x.device))
-    if not _uv_native.u1v_supported(x, ones, weight, info):
+    if not _uv_native.u1v_supported(x, ones, weight, table):
         return None
     kernels.log_tier("irreps_linear", "table-driven matrix-core kernels (fp32)")
-    return _uv_native.u1v(x, ones, weight, info)
+    return _uv_native.u1v(x, ones, weight, table)
 
 
 def mix(input: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anchor: Tensor = None) -> Tensor:

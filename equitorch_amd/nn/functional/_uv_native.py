@@ -22,6 +22,20 @@ from ... import _lib
 from ...ops import kernels
 
 FIRST, LAST = 1, 2
+
+
+class CooTable:
+    """A product table given directly by its coordinates (``coo``: ``TpCoo`` fields M, M1, M2, p, coef and the extents)
+    instead of a ``TensorProductInfo`` — the tables of the channel-mixing layers, whose second operand is the scalar 1.
+    ``anchor``: a tensor that lives as long as the table (cache key); ``fallback(x, y, w)``: a differentiable
+    evaluation of the same product for gradients of higher order."""
+
+    def __init__(self, coo, anchor: Tensor, fallback):
+        self.coo, self.anchor, self.fallback = coo, anchor, fallback
+
+
+def _anchor(table) -> Tensor:
+    return table.anchor if isinstance(table, CooTable) else table.info_Mij_fwd.scale
 MAX_TERMS = 8      # terms of a segment the weight-gradient kernel holds in registers (kUvtTerms)
 
 
@@ -64,7 +78,7 @@ class _Walk:
 
 def _walk(tp_info, role: str, n_groups: int, device) -> _Walk:
     def build():
-        c = kernels.coo_of(tp_info)
+        c = _coo(tp_info)
         if role == "out":        # rows of the first operand, rows of the second operand
             return _Walk(c.M, c.M1, c.M2, c.p, c.coef, c.DO, n_groups, device)
         if role == "in1":        # first operand of the launch = grad_out, second = input2
@@ -74,7 +88,7 @@ def _walk(tp_info, role: str, n_groups: int, device) -> _Walk:
         if role == "in2_uvw":    # first operand of the launch = grad_out, second = input1
             return _Walk(c.M2, c.M, c.M1, c.p, c.coef, c.D2, n_groups, device)
         raise ValueError(role)
-    return kernels.cached(tp_info.info_Mij_fwd.scale, ("uvt_walk", role, n_groups, str(device)), build)
+    return kernels.cached(_anchor(tp_info), ("uvt_walk", role, n_groups, str(device)), build)
 
 
 class _PathWalk:
@@ -107,8 +121,8 @@ class _PathWalk:
 def grad_w(x: Tensor, y: Tensor, g: Tensor, tp_info) -> Tensor:
     """``gw[p, k, w] = sum_n sum_{(p, M)} inter[n, (p, M), k] g[n, M, w]`` (``cgtp_uvt_grad_w``): ``(P, K, C_out)`` with
     ``K = C_x`` or ``C_x * C_y``; the caller reshapes."""
-    walk = kernels.cached(tp_info.info_Mij_fwd.scale, ("uvt_path_walk", str(x.device)),
-                          lambda: _PathWalk(kernels.coo_of(tp_info), x.device))
+    walk = kernels.cached(_anchor(tp_info), ("uvt_path_walk", str(x.device)),
+                          lambda: _PathWalk(_coo(tp_info), x.device))
     n, dx, cx = x.shape
     dy = y.shape[1]
     cy = y.shape[2] if y.ndim == 3 else 0
@@ -154,7 +168,7 @@ class _SegWalk:
 
 def grad_y_supported(n: int, dx: int, dy: int, cx: int, cout: int, tp_info) -> bool:
     """Whether the 16 staged samples of a ``cgtp_uvt_grad_y`` workgroup and its tables fit the LDS."""
-    c = kernels.coo_of(tp_info)
+    c = _coo(tp_info)
     kx = ((cx + 15) // 16 + 3) // 4 * 4 * 16
     lds = (16 * (dx * kx + 4) + 8 * 16 * dy) * 4 + len(c.coef) * (32 + 12) + 16
     return cx % 4 == 0 and cout % 4 == 0 and lds <= 160 * 1024
@@ -163,8 +177,8 @@ def grad_y_supported(n: int, dx: int, dy: int, cx: int, cout: int, tp_info) -> b
 def grad_y(x: Tensor, g: Tensor, wp: Tensor, tp_info, dy: int) -> Tensor:
     """``gy[n, b] = sum_t c_t <g[n, M_t, :], x[n, a_t, :] @ W[p_t]>`` (``cgtp_uvt_grad_y``); ``wp``: the weight as packed
     for the forward."""
-    walk = kernels.cached(tp_info.info_Mij_fwd.scale, ("uvt_seg_walk", str(x.device)),
-                          lambda: _SegWalk(kernels.coo_of(tp_info), x.device))
+    walk = kernels.cached(_anchor(tp_info), ("uvt_seg_walk", str(x.device)),
+                          lambda: _SegWalk(_coo(tp_info), x.device))
     n, dx, cx = x.shape
     gy = torch.empty((n, dy), dtype=torch.float32, device=x.device)
     a = _lib.UvtGyArgs()
@@ -220,7 +234,7 @@ def apply(x: Tensor, y: Tensor, wp: Tensor, tp_info, role: str, dout: int, cout:
 
 
 def _coo(tp_info):
-    return kernels.coo_of(tp_info)
+    return tp_info.coo if isinstance(tp_info, CooTable) else kernels.coo_of(tp_info)
 
 
 class _U1vNative(Function):
@@ -246,7 +260,7 @@ class _U1vNative(Function):
         tp_info = ctx.tp_info
         if torch.is_grad_enabled():       # higher-order derivative: the differentiable route throughout
             with torch.enable_grad():
-                out = _uv_gemm.u1v(x, y, w, tp_info)
+                out = tp_info.fallback(x, y, w) if isinstance(tp_info, CooTable) else _uv_gemm.u1v(x, y, w, tp_info)
                 wanted = [t for t, n in zip((x, y, w), need) if n]
                 got = iter(torch.autograd.grad(out, wanted, g, create_graph=True, allow_unused=True))
             return tuple(next(got) if n else None for n in need) + (None,)

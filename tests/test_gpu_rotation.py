@@ -95,6 +95,42 @@ def test_so2_linear(device, mode, per_sample):
         assert_close(a, b, tol=1e-11, what=f"SO2Linear {mode} per_sample={per_sample} {name}")
 
 
+@pytest.mark.parametrize("cin,cout,n", [(32, 48, 300), (64, 64, 33)])
+def test_so2_linear_uv_fp32_on_the_matrix_core_kernels(device, cin, cout, n):
+    """fp32 with a shared weight: the table of the layer is handed to the table-driven kernels of the fully
+    connected product as it is (second operand = the scalar 1); out, grad_x and grad_w against the oracle, and the
+    second-order route (create_graph) still differentiates."""
+    from equitorch_amd.nn import SO2Linear
+    from equitorch_amd.nn.functional import _uv_native
+    irr_in, irr_out = "0e+1o+2e+3o", "0e+1o+2e"
+    info = _f32(ref_tables.so2_linear_infos(irr_out, irr_in)[0])
+    mod = SO2Linear(irr_in, irr_out, cin, cout, internal_weights=False, feature_mode="uv").to(device)
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(n, 16, cin, generator=g).double()
+    w = (torch.randn(mod.num_weights, cin, cout, generator=g) / cin ** 0.5).double()
+    ct = torch.randn(n, 9, cout, generator=g).double()
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    ref = ref_ops.cpu_so2_linear(xr, wr, info, per_sample=False)
+    rgx, rgw = torch.autograd.grad(ref, (xr, wr), ct)
+    xd, wd = x.float().to(device).requires_grad_(True), w.float().to(device).requires_grad_(True)
+    calls = []
+    orig = _uv_native.apply
+    _uv_native.apply = lambda *a, **k: (calls.append(1), orig(*a, **k))[1]
+    try:
+        out = mod(xd, wd)
+        gx, gw = torch.autograd.grad(out, (xd, wd), ct.float().to(device), create_graph=True)
+    finally:
+        _uv_native.apply = orig
+    assert calls, "the layer did not run on the table-driven kernels"
+    for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
+        # sums over C_in (x paths) products; grad_w also over the batch
+        assert_close(a, b, tol=1e-5, what=f"SO2Linear uv fp32 {cin}->{cout} {name}", norm="max")
+    (ggx,) = torch.autograd.grad(gw.sum(), (xd,))          # second order through the differentiable route
+    (rggx,) = torch.autograd.grad(torch.autograd.grad(ref_ops.cpu_so2_linear(xr, wr, info, per_sample=False), wr, ct,
+                                                      create_graph=True)[0].sum(), xr)
+    assert_close(ggx, rggx, tol=1e-5, what="SO2Linear uv fp32 d(grad_w)/dx", norm="max")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 @pytest.mark.parametrize("channels", [64, 10])
 def test_fused_rotation_kernel(device, dtype, channels):
