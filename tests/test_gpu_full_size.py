@@ -197,3 +197,53 @@ def test_row_mode_full_size_shared_weight(device):
         (gp,) = torch.autograd.grad(mod(xd[lo:hi].detach(), shd[lo:hi].detach(), ws), (ws,), ct[lo:hi].to(device))
         parts.append(gp)
     assert_close(gw, parts[0] + parts[1], 1e-5, "row mode grad_w additivity", norm="max")  # sums over 65536 rows
+
+
+def test_edge_radial_full_size(device):
+    """BASELINE configs[1] / configs[2] shapes with the per-edge weights formed inside the kernels (R = 16): output
+    rows, node gradients and per-edge gradients of seeded subsets against the float64 oracle evaluated on exactly the
+    edges those rows depend on; the gradient of the shared matrix (a sum over all edges) through additivity over two
+    halves of the edge list."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu_radial
+    n_nodes, n_edges, ch, r = 4096, 65536, 64, 16
+    irr = "0e+1o+2e"
+    mod = SO3Linear(irr, irr, irr, ch, ch, internal_weights=False, feature_mode="uu").to(device)
+    g = torch.Generator().manual_seed(23)
+    src = torch.randint(0, n_nodes, (n_edges,), generator=g)
+    dst = torch.randint(0, n_nodes, (n_edges,), generator=g)
+    x = torch.randn(n_nodes, 9, ch, generator=g)
+    sh = torch.randn(n_edges, 9, generator=g)
+    h = torch.randn(n_edges, r, generator=g)
+    wl = torch.randn(r, mod.num_paths, ch, generator=g) / r ** 0.5
+    ct = torch.randn(n_nodes, 9, ch, generator=g)
+    plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
+    xd, shd, hd, wd = (t.to(device).requires_grad_(True) for t in (x, sh, h, wl))
+    out = edge_tensor_product_uu_radial(xd, shd, hd, wd, plan, mod.tp_info_forward)
+    gx, gsh, gh, gwl = torch.autograd.grad(out, (xd, shd, hd, wd), ct.to(device))
+    T = ref_ops.dense_coupling(irr, irr, irr).float().double()
+    nodes = torch.arange(11, n_nodes, 173)
+    # output rows of the chosen nodes: all edges that end there
+    e_in = torch.nonzero(torch.isin(dst, nodes)).flatten()
+    w_in = torch.einsum("er,rpc->epc", h[e_in].double(), wl.double())
+    msg = ref_ops.dense_u1u(T, x[src[e_in]].double(), sh[e_in].double(), w_in)
+    ref_rows = ref_ops.scatter_sum(msg, dst[e_in], n_nodes)[nodes]
+    assert_close(out[nodes.to(device)], ref_rows, 1e-5, "radial full size out rows", norm="max")   # sums over ~16 edges
+    # gradients: node rows of grad_x need all edges that start there; per-edge gradients need their own edge only
+    e_out = torch.nonzero(torch.isin(src, nodes)).flatten()
+    xr = x.double().requires_grad_(True)
+    shr, hr = sh[e_out].double().requires_grad_(True), h[e_out].double().requires_grad_(True)
+    w_out = torch.einsum("er,rpc->epc", hr, wl.double())
+    loss = (ref_ops.dense_u1u(T, xr[src[e_out]], shr, w_out) * ct[dst[e_out]].double()).sum()
+    rgx, rgsh, rgh = torch.autograd.grad(loss, (xr, shr, hr))
+    assert_close(gx[nodes.to(device)], rgx[nodes], 1e-5, "radial full size grad_x rows", norm="max")
+    assert_close(gsh[e_out.to(device)], rgsh, 1e-5, "radial full size grad_sh rows", norm="max")   # 64 channels x coefficients
+    assert_close(gh[e_out.to(device)], rgh, 1e-5, "radial full size grad_h rows", norm="max")      # 11 paths x 64 channels
+    # grad of the shared matrix: additivity over two halves of the edge list (each half its own plan)
+    parts = []
+    for lo, hi in ((0, n_edges // 2), (n_edges // 2, n_edges)):
+        pl = EdgePlan(src[lo:hi].to(device), dst[lo:hi].to(device), n_nodes)
+        ws = wd.detach().requires_grad_(True)
+        o = edge_tensor_product_uu_radial(xd.detach(), shd[lo:hi].detach(), hd[lo:hi].detach(), ws, pl, mod.tp_info_forward)
+        parts.append(torch.autograd.grad(o, (ws,), ct.to(device))[0].double())
+    assert_close(gwl.double(), parts[0] + parts[1], 1e-5, "radial full size grad_w_last additivity", norm="max")

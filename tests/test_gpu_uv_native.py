@@ -107,3 +107,42 @@ def test_u1v_fp32_native_full_size(device):
     ref_out, (rgx, _, _) = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x[sub], y[sub], w), ct[sub])
     assert_close(out[sub.to(device)], ref_out, 1e-5, "full size out", norm="max")
     assert_close(gx[sub.to(device)], rgx, 1e-5, "full size grad_x", norm="max")
+
+
+def test_u1v_fp32_full_size_properties(device):
+    """The configs[3] shape in fp32 (B = 32768, lmax = 3, 128 -> 128) on the table-driven kernels.  out / grad_x /
+    grad_y of a strided subset of the rows against the dense oracle (a row depends on its own sample only); the weight
+    gradient, a sum over the batch, against the oracle's sum over the subset when every other output gradient is zero,
+    and through additivity over two halves of the batch."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import _uv_native
+    lmax, ch, n = 3, 128, 32768
+    irreps = _sh(lmax)
+    mod = SO3Linear(irreps, irreps, irreps, ch, ch, internal_weights=False, feature_mode="uv").to(device)
+    g = torch.Generator().manual_seed(17)
+    x = torch.randn(n, 16, ch, generator=g)
+    y = torch.randn(n, 16, generator=g)
+    w = torch.randn(mod.num_paths, ch, ch, generator=g) / (ch * mod.num_paths) ** 0.5
+    ct = torch.randn(n, 16, ch, generator=g)
+    sub = torch.arange(3, n, 331)                      # 99 rows spread over all workgroups
+    mask = torch.zeros(n, 1, 1)
+    mask[sub] = 1
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    assert _uv_native.u1v_supported(xd, yd, wd, mod.tp_info_forward)
+    out = mod(xd, yd, wd)
+    gx, gy, gw = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
+    T = ref_ops.dense_coupling(irreps, irreps, irreps).float().double()
+    ref_out, (rgx, rgy, rgw_sub) = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x[sub], y[sub], w), ct[sub])
+    sd = sub.to(device)
+    for name, a, b in (("out", out[sd], ref_out), ("grad_x", gx[sd], rgx), ("grad_y", gy[sd], rgy)):
+        assert_close(a, b, 1e-5, f"u1v fp32 full size {name} rows", norm="max")   # sums over 128 channels x paths
+    (gw_sub,) = torch.autograd.grad(mod(xd, yd, wd), (wd,), (ct * mask).to(device))
+    assert_close(gw_sub, rgw_sub, 1e-5, "u1v fp32 full size grad_w of the subset", norm="max")
+    half = n // 2
+    parts = []
+    for lo, hi in ((0, half), (half, n)):
+        ws = wd.detach().requires_grad_(True)
+        (gp,) = torch.autograd.grad(mod(xd[lo:hi].detach(), yd[lo:hi].detach(), ws), (ws,), ct[lo:hi].to(device))
+        parts.append(gp.double())
+    # a sum of 32768 x 16 products per element, in chunks: rounding of the three results bounds the difference
+    assert_close(gw.double(), parts[0] + parts[1], 1e-5, "u1v fp32 full size grad_w additivity", norm="max")
