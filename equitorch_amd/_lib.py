@@ -150,12 +150,12 @@ def _load():
     lib.cgtp_uvt_packed_elems.argtypes = [C.c_int32, C.c_int64, C.c_int32]
     lib.cgtp_uvt_pack_weights.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_int64, C.c_int64,
                                           C.c_int64, C.c_int32, C.c_void_p]
-    lib.cgtp_uvt_chunk.argtypes = [C.c_int64] + [C.c_int32] * 6
-    lib.cgtp_uvt_item_groups.argtypes = [C.c_int64] + [C.c_int32] * 6
+    lib.cgtp_uvt_chunk.argtypes = [C.c_int64] + [C.c_int32] * 7
+    lib.cgtp_uvt_item_groups.argtypes = [C.c_int64] + [C.c_int32] * 7
     lib.cgtp_uvt_validate.argtypes = [C.POINTER(UvtArgs)]
     lib.cgtp_uvt_apply.argtypes = [C.POINTER(UvtArgs), C.c_void_p]
     lib.cgtp_uvt_grad_w_workspace_bytes.restype = C.c_int64
-    lib.cgtp_uvt_grad_w_workspace_bytes.argtypes = [C.c_int64, C.c_int32, C.c_int64, C.c_int32]
+    lib.cgtp_uvt_grad_w_workspace_bytes.argtypes = [C.c_int64, C.c_int32, C.c_int64, C.c_int32, C.c_int32]
     lib.cgtp_uvt_grad_w.argtypes = [C.POINTER(UvtGwArgs), C.c_void_p]
     lib.cgtp_uvt_grad_y.argtypes = [C.POINTER(UvtGyArgs), C.c_void_p]
     lib.cgtp_sh_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_double, C.c_int,

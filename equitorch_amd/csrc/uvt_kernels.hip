@@ -15,28 +15,62 @@
 // repacked in fragment order (one contiguous KB per wavefront load) and are requested four blocks of 16 k ahead.
 // The gradient with respect to the channelled operand is the same kernel with the roles of the rows exchanged and
 // the weight packed transposed; the other two gradients have kernels of their own below.
+//
+// The file compiles twice: as it is for fp32 (v_mfma_f32_16x16x4_f32), and from uvt_kernels_f64.hip with CGTP_UVT_F64
+// defined for fp64 (v_mfma_f64_16x16x4_f64, same lane layouts); each set lives in its own namespace.
 #include "cgtp_device.h"
 #include "cgtp_host.h"
+
+#ifdef CGTP_UVT_F64
+#define UVT_NS uvt_f64
+typedef double real;
+#else
+#define UVT_NS uvt_f32
+typedef float real;
+#endif
 
 #pragma clang fp contract(fast)
 
 namespace cgtp {
+namespace UVT_NS {
 
-typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef real realx4 __attribute__((ext_vector_type(4)));
+#ifdef CGTP_UVT_F64
+constexpr int kDtype = CGTP_F64;
+#else
+constexpr int kDtype = CGTP_F32;
+#endif
+constexpr int kTermBytes = 8 + (int)sizeof(real);   // LDS bytes of one term: two row indices and a coefficient
+
+// D = A (16 x 4) * B (4 x 16) + C in the operands' own precision.  Operand layouts are the same for both instructions
+// (A: lane holds row lane % 16, k = lane / 16; B: column lane % 16, k = lane / 16); the accumulator's are not: lane
+// (column lane % 16, group g = lane / 16) holds in element e row 4 g + e in single and row g + 4 e in double precision.
+__host__ __device__ constexpr int acc_row(int g, int e) { return sizeof(real) == 8 ? g + 4 * e : 4 * g + e; }
+// Row of operand A that has to carry item c of 16 so that element e of group g ends up holding item 4 g + e (the
+// weight fragments are packed in this order: consumers then read four consecutive output channels per lane).
+__host__ __device__ constexpr int a_row_of(int c) { return sizeof(real) == 8 ? (c % 4) * 4 + c / 4 : c; }
+__device__ __forceinline__ realx4 mfma16(real a, real b, realx4 c, int, int, int) {
+#ifdef CGTP_UVT_F64
+  return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+#else
+  return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+#endif
+}
+
 
 constexpr int kUvtFirst = 1, kUvtLast = 2;   // item flags: first / last item of its output row
 constexpr int kUvtMaxGroups = 8;             // = wavefronts per workgroup
 constexpr int64_t kUvtTableRoom = 24 * 1024;  // LDS kept free for the walk tables when the launch shape is chosen
 
 struct UvtDev {
-  const float* x;
-  const float* y;
-  const float* wp;
-  float* out;
+  const real* x;
+  const real* y;
+  const real* wp;
+  real* out;
   const cgtp_uvt_item* items;
   const int32_t* ta;
   const int32_t* tb;
-  const float* tc;
+  const real* tc;
   int64_t n_rows;
   int n_items, n_terms, dx, dy, dout, cx, cy, cout;
   int kx;        // y without channels: cx rounded up to 16 (row length of the staged x); with: cx
@@ -53,23 +87,23 @@ struct UvtDev {
 // Rows of the workgroup's samples into LDS: x as [sample][row][kx] (zero-padded channels), y as [sample][row] or
 // [sample][row][cy].  Samples past the end of the batch are staged as zeros.
 template <bool YC>
-__device__ __forceinline__ void uvt_stage(const UvtDev& a, float* xs, float* ys, int64_t nb0, int n_samples) {
+__device__ __forceinline__ void uvt_stage(const UvtDev& a, real* xs, real* ys, int64_t nb0, int n_samples) {
   const int kx4 = a.kx / 4, per_sample = a.dx * kx4;
   for (int i = threadIdx.x; i < n_samples * per_sample; i += blockDim.x) {
     const int s = i / per_sample, rem = i - s * per_sample, row = rem / kx4, c4 = rem - row * kx4;
     const int64_t n = nb0 + s;
-    floatx4 v = {0.f, 0.f, 0.f, 0.f};
-    if (n < a.n_rows && c4 * 4 < a.cx) v = *reinterpret_cast<const floatx4*>(a.x + (n * a.dx + row) * a.cx + c4 * 4);
-    *reinterpret_cast<floatx4*>(xs + (size_t)s * a.px + row * a.kx + c4 * 4) = v;
+    realx4 v = {0.f, 0.f, 0.f, 0.f};
+    if (n < a.n_rows && c4 * 4 < a.cx) v = *reinterpret_cast<const realx4*>(a.x + (n * a.dx + row) * a.cx + c4 * 4);
+    *reinterpret_cast<realx4*>(xs + (size_t)s * a.px + row * a.kx + c4 * 4) = v;
   }
   if constexpr (YC) {
     const int cy4 = a.cy / 4, per_y = a.dy * cy4;
     for (int i = threadIdx.x; i < n_samples * per_y; i += blockDim.x) {
       const int s = i / per_y, rem = i - s * per_y;
       const int64_t n = nb0 + s;
-      floatx4 v = {0.f, 0.f, 0.f, 0.f};
-      if (n < a.n_rows) v = *reinterpret_cast<const floatx4*>(a.y + n * a.dy * a.cy + rem * 4);
-      *reinterpret_cast<floatx4*>(ys + (size_t)s * a.py + rem * 4) = v;
+      realx4 v = {0.f, 0.f, 0.f, 0.f};
+      if (n < a.n_rows) v = *reinterpret_cast<const realx4*>(a.y + n * a.dy * a.cy + rem * 4);
+      *reinterpret_cast<realx4*>(ys + (size_t)s * a.py + rem * 4) = v;
     }
   } else {
     for (int i = threadIdx.x; i < n_samples * a.dy; i += blockDim.x) {
@@ -87,7 +121,7 @@ struct UvtTables {
   const cgtp_uvt_item* items;
   const int32_t* ta;
   const int32_t* tb;
-  const float* tc;
+  const real* tc;
 };
 
 template <class Dev>
@@ -95,9 +129,9 @@ __device__ __forceinline__ UvtTables uvt_stage_tables(const Dev& a, unsigned cha
   int32_t* dst = reinterpret_cast<int32_t*>(at);
   const int32_t* src = reinterpret_cast<const int32_t*>(a.items);
   for (int i = threadIdx.x; i < a.n_items * 8; i += blockDim.x) dst[i] = src[i];
-  int32_t* ta = dst + a.n_items * 8;
+  real* tc = reinterpret_cast<real*>(dst + a.n_items * 8);   // first: items are 32 bytes, so this is aligned for doubles
+  int32_t* ta = reinterpret_cast<int32_t*>(tc + a.n_terms);
   int32_t* tb = ta + a.n_terms;
-  float* tc = reinterpret_cast<float*>(tb + a.n_terms);
   for (int i = threadIdx.x; i < a.n_terms; i += blockDim.x) {
     ta[i] = a.ta[i];
     tb[i] = a.tb[i];
@@ -125,15 +159,15 @@ constexpr int kUvtTerms = 8;
 constexpr int kUvtKbi = 4;   // blocks of 16 k per item
 template <bool YC>
 struct UvtTerms {
-  const float* xr[kUvtTerms];
-  const float* yr[kUvtTerms];   // YC only
-  float s[kUvtTerms];
+  const real* xr[kUvtTerms];
+  const real* yr[kUvtTerms];   // YC only
+  real s[kUvtTerms];
   int n;
 };
 
 template <bool YC>
-__device__ __forceinline__ void uvt_terms(const UvtDev& a, const UvtTables& tab, const cgtp_uvt_item& it, const float* xl,
-                                          const float* yl, const float* zeros, int g, UvtTerms<YC>& T) {
+__device__ __forceinline__ void uvt_terms(const UvtDev& a, const UvtTables& tab, const cgtp_uvt_item& it, const real* xl,
+                                          const real* yl, const real* zeros, int g, UvtTerms<YC>& T) {
   T.n = min(it.t1 - it.t0, kUvtTerms);
 #pragma unroll
   for (int k = 0; k < kUvtTerms; ++k) {
@@ -142,7 +176,7 @@ __device__ __forceinline__ void uvt_terms(const UvtDev& a, const UvtTables& tab,
     const int t = live ? it.t0 + k : it.t0;
     const int ia = __builtin_amdgcn_readfirstlane(tab.ta[t]);
     const int ib = __builtin_amdgcn_readfirstlane(tab.tb[t]);
-    const float c = live ? tab.tc[t] : 0.f;
+    const real c = live ? tab.tc[t] : 0.f;
     if constexpr (YC) {
       T.xr[k] = live ? xl + ia * a.cx : zeros;
       T.yr[k] = live ? yl + ib * a.cy : zeros;
@@ -157,8 +191,8 @@ __device__ __forceinline__ void uvt_terms(const UvtDev& a, const UvtTables& tab,
 // This lane's part of block j of 16 k of the mixed operand of an item: inter_s[n, 16 j + 4 g + i], i < 4.
 // With a channelled y, lut[j * 4 + g] holds the offsets (u, v) of k = 16 j + 4 g = u * cy + v.
 template <bool YC>
-__device__ __forceinline__ floatx4 uvt_mix_block(const UvtTerms<YC>& T, int j, const int2* lut) {
-  floatx4 bf = {0.f, 0.f, 0.f, 0.f};
+__device__ __forceinline__ realx4 uvt_mix_block(const UvtTerms<YC>& T, int j, const int2* lut) {
+  realx4 bf = {0.f, 0.f, 0.f, 0.f};
   int2 o = make_int2(0, 0);
   if constexpr (YC) o = lut[j * 4];
 #pragma unroll
@@ -167,9 +201,9 @@ __device__ __forceinline__ floatx4 uvt_mix_block(const UvtTerms<YC>& T, int j, c
 #pragma unroll
       for (int k = half; k < half + 4; ++k) {
         if constexpr (YC) {
-          bf += (T.s[k] * T.xr[k][o.x]) * *reinterpret_cast<const floatx4*>(T.yr[k] + o.y);
+          bf += (T.s[k] * T.xr[k][o.x]) * *reinterpret_cast<const realx4*>(T.yr[k] + o.y);
         } else {
-          bf += T.s[k] * *reinterpret_cast<const floatx4*>(T.xr[k] + j * 16);
+          bf += T.s[k] * *reinterpret_cast<const realx4*>(T.xr[k] + j * 16);
         }
       }
     }
@@ -179,17 +213,17 @@ __device__ __forceinline__ floatx4 uvt_mix_block(const UvtTerms<YC>& T, int j, c
 
 // Terms beyond the first kUvtTerms of a segment (large irreps only): straight from the tables.
 template <bool YC>
-__device__ __forceinline__ floatx4 uvt_mix_tail(const UvtDev& a, const UvtTables& tab, const cgtp_uvt_item& it, int j,
-                                                const float* xl, const float* yl, int g, const int2* lut) {
-  floatx4 bf = {0.f, 0.f, 0.f, 0.f};
+__device__ __forceinline__ realx4 uvt_mix_tail(const UvtDev& a, const UvtTables& tab, const cgtp_uvt_item& it, int j,
+                                                const real* xl, const real* yl, int g, const int2* lut) {
+  realx4 bf = {0.f, 0.f, 0.f, 0.f};
   for (int t = it.t0 + kUvtTerms; t < it.t1; ++t) {
     const int ia = tab.ta[t], ib = tab.tb[t];
-    const float c = tab.tc[t];
+    const real c = tab.tc[t];
     if constexpr (YC) {
       const int2 o = lut[j * 4];
-      bf += (c * xl[ia * a.cx + o.x]) * *reinterpret_cast<const floatx4*>(yl + ib * a.cy + o.y);
+      bf += (c * xl[ia * a.cx + o.x]) * *reinterpret_cast<const realx4*>(yl + ib * a.cy + o.y);
     } else {
-      bf += (c * yl[ib]) * *reinterpret_cast<const floatx4*>(xl + ia * a.kx + (it.kb0 + j) * 16 + 4 * g);
+      bf += (c * yl[ib]) * *reinterpret_cast<const realx4*>(xl + ia * a.kx + (it.kb0 + j) * 16 + 4 * g);
     }
   }
   return bf;
@@ -207,21 +241,21 @@ __global__ void __launch_bounds__(kUvtMaxGroups* kWave) uvt_apply_kernel(const U
   constexpr int KBI = kUvtKbi;
   extern __shared__ __align__(16) unsigned char smem[];
   const int sb_count = 1 << a.sb_log2;
-  float* xs = reinterpret_cast<float*>(smem);
-  float* ys = xs + (size_t)(16 * sb_count) * a.px;
+  real* xs = reinterpret_cast<real*>(smem);
+  real* ys = xs + (size_t)(16 * sb_count) * a.px;
   const int64_t nb0 = (int64_t)blockIdx.x * (16 * sb_count);
   uvt_stage<YC>(a, xs, ys, nb0, 16 * sb_count);
   unsigned char* after = reinterpret_cast<unsigned char*>(ys + (size_t)(16 * sb_count) * a.py);
   const UvtTables tab = uvt_stage_tables(a, after);
   // (u, v) of k = 16 kb + 4 g for a channelled y; (0, 0) in the zero-padded tail of k
-  int2* lut_all = reinterpret_cast<int2*>(after + ((size_t)a.n_items * 32 + (size_t)a.n_terms * 12 + 15) / 16 * 16);
+  int2* lut_all = reinterpret_cast<int2*>(after + ((size_t)a.n_items * 32 + (size_t)a.n_terms * kTermBytes + 15) / 16 * 16);
   if constexpr (YC) {
     for (int i = threadIdx.x; i < a.kblocks * 4; i += blockDim.x) {
       const int k0 = i * 4, u = k0 / a.cy;
       lut_all[i] = k0 < a.cx * a.cy ? make_int2(u, k0 - u * a.cy) : make_int2(0, 0);
     }
   }
-  float* zeros = reinterpret_cast<float*>(lut_all + (YC ? a.kblocks * 4 : 0));
+  real* zeros = reinterpret_cast<real*>(lut_all + (YC ? a.kblocks * 4 : 0));
   for (int i = threadIdx.x; i < a.zero_floats; i += blockDim.x) zeros[i] = 0.f;
   __syncthreads();
 
@@ -234,8 +268,8 @@ __global__ void __launch_bounds__(kUvtMaxGroups* kWave) uvt_apply_kernel(const U
   const int j_end = a.group_ptr[ig + 1];
   if (j >= j_end) return;
   const int64_t n = nb0 + sb * 16 + r;
-  const float* xl = xs + (size_t)(sb * 16 + r) * a.px;
-  const float* yl = ys + (size_t)(sb * 16 + r) * a.py;
+  const real* xl = xs + (size_t)(sb * 16 + r) * a.px;
+  const real* yl = ys + (size_t)(sb * 16 + r) * a.py;
   const int2* lut_g = lut_all + g;
 
   const int64_t kstride = (int64_t)a.wbp * 256;
@@ -243,46 +277,46 @@ __global__ void __launch_bounds__(kUvtMaxGroups* kWave) uvt_apply_kernel(const U
     // wave-uniform base of the item's fragments; a lane adds 16 bytes times its index
     return a.wp + ((int64_t)it.p * a.kblocks * a.wbp + wb0) * 256 + lane * 4;
   };
-  floatx4 acc[WB], A[KBI][WB];
-  auto load_a = [&](const float* base, int kb, floatx4 (&Aj)[WB]) __attribute__((always_inline)) {
+  realx4 acc[WB], A[KBI][WB];
+  auto load_a = [&](const real* base, int kb, realx4 (&Aj)[WB]) __attribute__((always_inline)) {
 #pragma unroll
-    for (int wb = 0; wb < WB; ++wb) Aj[wb] = *reinterpret_cast<const floatx4*>(base + kb * kstride + wb * 256);
+    for (int wb = 0; wb < WB; ++wb) Aj[wb] = *reinterpret_cast<const realx4*>(base + kb * kstride + wb * 256);
   };
 #pragma unroll
-  for (int wb = 0; wb < WB; ++wb) acc[wb] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int wb = 0; wb < WB; ++wb) acc[wb] = realx4{0.f, 0.f, 0.f, 0.f};
 
   cgtp_uvt_item it = uvt_item_at(tab, j);
-  const float* base = wbase_of(it);
+  const real* base = wbase_of(it);
 #pragma unroll
   for (int jj = 0; jj < KBI; ++jj) load_a(base, jj, A[jj]);
   while (j < j_end) {
     const bool more = j + 1 < j_end;
     const cgtp_uvt_item it2 = uvt_item_at(tab, more ? j + 1 : j);
-    const float* base2 = wbase_of(it2);
+    const real* base2 = wbase_of(it2);
     UvtTerms<YC> T;
     uvt_terms<YC>(a, tab, it, xl, yl, zeros, g, T);
     const bool tail = it.t1 - it.t0 > kUvtTerms;
     auto mix = [&](int kb) __attribute__((always_inline)) {
-      floatx4 b = uvt_mix_block<YC>(T, kb, lut_g);
+      realx4 b = uvt_mix_block<YC>(T, kb, lut_g);
       if (tail) b += uvt_mix_tail<YC>(a, tab, it, kb, xl, yl, g, lut_g);
       return b;
     };
     const bool first = it.flags & kUvtFirst;
 #pragma unroll
-    for (int wb = 0; wb < WB; ++wb) acc[wb] = first ? floatx4{0.f, 0.f, 0.f, 0.f} : acc[wb];
-    floatx4 Bc = mix(0);
+    for (int wb = 0; wb < WB; ++wb) acc[wb] = first ? realx4{0.f, 0.f, 0.f, 0.f} : acc[wb];
+    realx4 Bc = mix(0);
     for (int kb = 0; kb < a.kblocks; kb += KBI) {
       const bool wrap = kb + KBI >= a.kblocks;        // the fragments requested now belong to the next item
-      const float* wnext = wrap ? base2 : base;
+      const real* wnext = wrap ? base2 : base;
       const int kbn = wrap ? 0 : kb + KBI;
 #pragma unroll
       for (int jj = 0; jj < KBI; ++jj) {
-        const floatx4 Bn = mix((jj + 1 < KBI || !wrap) ? kb + jj + 1 : kb + jj);
+        const realx4 Bn = mix((jj + 1 < KBI || !wrap) ? kb + jj + 1 : kb + jj);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
           for (int wb = 0; wb < WB; ++wb)
-            acc[wb] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[jj][wb][i], Bc[i], acc[wb], 0, 0, 0);
+            acc[wb] = mfma16(A[jj][wb][i], Bc[i], acc[wb], 0, 0, 0);
         load_a(wnext, kbn + jj, A[jj]);
         Bc = Bn;
       }
@@ -290,11 +324,11 @@ __global__ void __launch_bounds__(kUvtMaxGroups* kWave) uvt_apply_kernel(const U
     if (it.flags & kUvtLast) {
       // accumulator layout: lane (n = r, g) holds output channels 16 wb + 4 g .. + 3 of sample n
       if (n < a.n_rows) {
-        float* orow = a.out + (n * a.dout + it.out_row) * a.cout;
+        real* orow = a.out + (n * a.dout + it.out_row) * a.cout;
 #pragma unroll
         for (int wb = 0; wb < WB; ++wb) {
           const int w = (wb0 + wb) * 16 + 4 * g;
-          if (w < a.cout) *reinterpret_cast<floatx4*>(orow + w) = acc[wb];
+          if (w < a.cout) *reinterpret_cast<realx4*>(orow + w) = acc[wb];
         }
       }
     }
@@ -307,7 +341,7 @@ __global__ void __launch_bounds__(kUvtMaxGroups* kWave) uvt_apply_kernel(const U
 // packed[((p * kblocks + kb) * wbp + wb) * 256 + lane * 4 + i] = W[p][16 kb + 4 (lane / 16) + i][16 wb + lane % 16]
 // (zero outside K x cout), W addressed with element strides so that the transposed weight of the backward needs no
 // copy of its own.
-__global__ void uvt_pack_kernel(const float* __restrict__ w, float* __restrict__ packed, int64_t n_vec, int K, int cout,
+__global__ void uvt_pack_kernel(const real* __restrict__ w, real* __restrict__ packed, int64_t n_vec, int K, int cout,
                                 int kblocks, int wbp, int64_t stride_p, int64_t stride_k, int64_t stride_c) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n_vec) return;
@@ -316,14 +350,15 @@ __global__ void uvt_pack_kernel(const float* __restrict__ w, float* __restrict__
   const int wb = (int)(c % wbp); c /= wbp;
   const int kb = (int)(c % kblocks);
   const int64_t p = c / kblocks;
-  const int col = wb * 16 + (lane & 15);
-  floatx4 v = {0.f, 0.f, 0.f, 0.f};
+  // row i of the fragment carries the output channel c with a_row_of(c) == i (the permutation is its own inverse)
+  const int col = wb * 16 + a_row_of(lane & 15);
+  realx4 v = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const int k = kb * 16 + 4 * (lane >> 4) + e;
     if (k < K && col < cout) v[e] = w[p * stride_p + k * stride_k + col * stride_c];
   }
-  *reinterpret_cast<floatx4*>(packed + i * 4) = v;
+  *reinterpret_cast<realx4*>(packed + i * 4) = v;
 }
 
 
@@ -340,15 +375,15 @@ __global__ void uvt_pack_kernel(const float* __restrict__ w, float* __restrict__
 // The chunks' partial results go to a workspace and are summed in chunk order by uvt_gw_reduce_kernel (no atomics:
 // the result does not depend on the launch).
 struct UvtGwDev {
-  const float* x;
-  const float* y;
-  const float* g;
-  float* part;                 // (n_chunks, n_paths, K, cout)
+  const real* x;
+  const real* y;
+  const real* g;
+  real* part;                 // (n_chunks, n_paths, K, cout)
   const cgtp_uvt_item* items;  // segments sorted by path: p, out_row = M, t0, t1
   const int32_t* path_ptr;     // [n_paths + 1] into items
   const int32_t* ta;
   const int32_t* tb;
-  const float* tc;
+  const real* tc;
   int64_t n_rows;
   int n_paths, dx, dy, dg, cx, cy, cout, K, chunk;
 };
@@ -361,9 +396,9 @@ constexpr int kGwPitch = 132;  // floats per sample row of the LDS stage: 128 ch
 // 64, column r of w-tile j is output channel 4 r + j — so that a lane's operands of the four tiles are four
 // consecutive channels: one 16-byte LDS read per operand and step.
 template <bool YC>
-__global__ void __launch_bounds__(256, 3) uvt_grad_w_kernel(const UvtGwDev a) {
-  __shared__ __attribute__((aligned(16))) float lds_a[2][kGwStep][kGwPitch];
-  __shared__ __attribute__((aligned(16))) float lds_b[2][kGwStep][kGwPitch];
+__global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : 3) uvt_grad_w_kernel(const UvtGwDev a) {
+  __shared__ __attribute__((aligned(16))) real lds_a[2][kGwStep][kGwPitch];
+  __shared__ __attribute__((aligned(16))) real lds_b[2][kGwStep][kGwPitch];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), r = lane & 15, g4 = lane >> 4;
   const int p = blockIdx.y;
   const int kgroups = (a.K + 127) / 128;
@@ -384,11 +419,11 @@ __global__ void __launch_bounds__(256, 3) uvt_grad_w_kernel(const UvtGwDev a) {
   // multiplying role: channels kh * 64 .. + 63 by output channels wh * 64 .. + 63
   const int kh = wave & 1, wh = wave >> 1;
 
-  floatx4 acc[kGwT][kGwT];
+  realx4 acc[kGwT][kGwT];
 #pragma unroll
   for (int i = 0; i < kGwT; ++i)
 #pragma unroll
-    for (int j = 0; j < kGwT; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < kGwT; ++j) acc[i][j] = realx4{0.f, 0.f, 0.f, 0.f};
 
   const int s_begin = a.path_ptr[p], s_end = a.path_ptr[p + 1];
   const int steps = (int)((n_end - n_begin + kGwStep - 1) / kGwStep);
@@ -398,10 +433,10 @@ __global__ void __launch_bounds__(256, 3) uvt_grad_w_kernel(const UvtGwDev a) {
   // splits longer segments; slots past the end repeat the first term's rows with coefficient zero)
   int ld_item = s_begin - 1, ld_step = steps;
   int xrow[kUvtTerms], yrow[kUvtTerms], grow = 0;
-  float c[kUvtTerms];
-  floatx4 v4[kUvtTerms];     // y without channels: four channels of x; with: four channels of y
-  float v1[kUvtTerms];       // y without channels: y[n, b]; with: x[n, a, u]
-  floatx4 bv4;
+  real c[kUvtTerms];
+  realx4 v4[kUvtTerms];     // y without channels: four channels of x; with: four channels of y
+  real v1[kUvtTerms];       // y without channels: y[n, b]; with: x[n, a, u]
+  realx4 bv4;
   bool ld_live = false;
 
   auto issue = [&]() __attribute__((always_inline)) {
@@ -422,16 +457,16 @@ __global__ void __launch_bounds__(256, 3) uvt_grad_w_kernel(const UvtGwDev a) {
     const int64_t n = n_begin + (int64_t)ld_step * kGwStep + ls;
     ld_live = n < n_end;
     const int64_t nc = ld_live ? n : n_end - 1;
-    const float* xn = a.x + nc * a.dx * a.cx + xo;
-    const float* yn = a.y + nc * a.dy * (YC ? a.cy : 1) + yo;
-    bv4 = *reinterpret_cast<const floatx4*>(a.g + nc * a.dg * a.cout + grow + wc);
+    const real* xn = a.x + nc * a.dx * a.cx + xo;
+    const real* yn = a.y + nc * a.dy * (YC ? a.cy : 1) + yo;
+    bv4 = *reinterpret_cast<const realx4*>(a.g + nc * a.dg * a.cout + grow + wc);
 #pragma unroll
     for (int k = 0; k < kUvtTerms; ++k) {
       if constexpr (YC) {
         v1[k] = xn[xrow[k]];
-        v4[k] = *reinterpret_cast<const floatx4*>(yn + yrow[k]);
+        v4[k] = *reinterpret_cast<const realx4*>(yn + yrow[k]);
       } else {
-        v4[k] = *reinterpret_cast<const floatx4*>(xn + xrow[k]);
+        v4[k] = *reinterpret_cast<const realx4*>(xn + xrow[k]);
         v1[k] = yn[yrow[k]];
       }
     }
@@ -439,12 +474,12 @@ __global__ void __launch_bounds__(256, 3) uvt_grad_w_kernel(const UvtGwDev a) {
   };
   // mixes the terms of the loads in flight and puts both operands into stage buf
   auto commit = [&](int buf) __attribute__((always_inline)) {
-    floatx4 av = {0.f, 0.f, 0.f, 0.f};
+    realx4 av = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int k = 0; k < kUvtTerms; ++k) av += (c[k] * v1[k]) * v4[k];
-    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-    *reinterpret_cast<floatx4*>(&lds_a[buf][ls][lq]) = (ld_live && kok) ? av : zero;
-    *reinterpret_cast<floatx4*>(&lds_b[buf][ls][lq]) = (ld_live && wok) ? bv4 : zero;
+    const realx4 zero = {0.f, 0.f, 0.f, 0.f};
+    *reinterpret_cast<realx4*>(&lds_a[buf][ls][lq]) = (ld_live && kok) ? av : zero;
+    *reinterpret_cast<realx4*>(&lds_b[buf][ls][lq]) = (ld_live && wok) ? bv4 : zero;
   };
 
   if (total > 0) {
@@ -454,11 +489,11 @@ __global__ void __launch_bounds__(256, 3) uvt_grad_w_kernel(const UvtGwDev a) {
     __syncthreads();
     for (int i = 0; i < total; ++i) {
       const int buf = i & 1;
-      floatx4 af[2], bf[2];
+      realx4 af[2], bf[2];
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
-        af[ks] = *reinterpret_cast<const floatx4*>(&lds_a[buf][4 * ks + g4][kh * 64 + 4 * r]);
-        bf[ks] = *reinterpret_cast<const floatx4*>(&lds_b[buf][4 * ks + g4][wh * 64 + 4 * r]);
+        af[ks] = *reinterpret_cast<const realx4*>(&lds_a[buf][4 * ks + g4][kh * 64 + 4 * r]);
+        bf[ks] = *reinterpret_cast<const realx4*>(&lds_b[buf][4 * ks + g4][wh * 64 + 4 * r]);
       }
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks)
@@ -466,7 +501,7 @@ __global__ void __launch_bounds__(256, 3) uvt_grad_w_kernel(const UvtGwDev a) {
         for (int ti = 0; ti < kGwT; ++ti)
 #pragma unroll
           for (int tj = 0; tj < kGwT; ++tj)
-            acc[ti][tj] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[ks][ti], bf[ks][tj], acc[ti][tj], 0, 0, 0);
+            acc[ti][tj] = mfma16(af[ks][ti], bf[ks][tj], acc[ti][tj], 0, 0, 0);
       if (i + 1 < total) commit(buf ^ 1);
       if (i + 2 < total) issue();
       __syncthreads();
@@ -474,7 +509,7 @@ __global__ void __launch_bounds__(256, 3) uvt_grad_w_kernel(const UvtGwDev a) {
   }
   // accumulator layout: lane (column r, g4) holds rows 4 g4 .. + 3 of a tile; tile (i, j) row q is channel
   // 4 q + i of the wavefront's 64, column r is output channel 4 r + j
-  float* out = a.part + ((int64_t)blockIdx.x * a.n_paths + p) * a.K * a.cout;
+  real* out = a.part + ((int64_t)blockIdx.x * a.n_paths + p) * a.K * a.cout;
   const int kbase = kgrp * 128 + kh * 64;
   const int w0 = wgrp * 128 + wh * 64 + 4 * r;
   if (w0 < a.cout) {
@@ -482,21 +517,21 @@ __global__ void __launch_bounds__(256, 3) uvt_grad_w_kernel(const UvtGwDev a) {
     for (int i = 0; i < kGwT; ++i)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const int k = kbase + 4 * (4 * g4 + e) + i;
+        const int k = kbase + 4 * acc_row(g4, e) + i;
         if (k < a.K) {
-          floatx4 v;
+          realx4 v;
 #pragma unroll
           for (int j = 0; j < kGwT; ++j) v[j] = acc[i][j][e];
-          *reinterpret_cast<floatx4*>(out + (int64_t)k * a.cout + w0) = v;
+          *reinterpret_cast<realx4*>(out + (int64_t)k * a.cout + w0) = v;
         }
       }
   }
 }
 
-__global__ void uvt_gw_reduce_kernel(const float* __restrict__ part, float* __restrict__ gw, int64_t n_chunks, int64_t n) {
+__global__ void uvt_gw_reduce_kernel(const real* __restrict__ part, real* __restrict__ gw, int64_t n_chunks, int64_t n) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  float s = 0.f;
+  real s = 0.f;
   for (int64_t c = 0; c < n_chunks; ++c) s += part[c * n + i];
   gw[i] = s;
 }
@@ -520,37 +555,37 @@ static int64_t uvt_gw_chunk(int64_t n_rows) {
 // added in wavefront order at the end.  Eight wavefronts share a workgroup's 16 samples: the segments are dealt round
 // robin to groups of wavefronts, the blocks of 32 output channels within a group.
 struct UvtGyDev {
-  const float* x;
-  const float* g;
-  const float* wp;
-  float* gy;
+  const real* x;
+  const real* g;
+  const real* wp;
+  real* gy;
   const cgtp_uvt_item* items;   // segments: p, out_row = a, t0, t1
   const int32_t* ta;            // row M of g
   const int32_t* tb;            // row b of gy
-  const float* tc;
+  const real* tc;
   int64_t n_rows;
   int n_items, n_terms, dx, dy, dg, cx, cout;
   int kx, px, kblocks, wbp;
   int wchunks, wgroups;         // blocks of 32 output channels; wavefronts of a group that share a segment (1, 2, 4)
 };
 
-constexpr int kGyWB = 2;        // blocks of 16 output channels per pass
+constexpr int kGyWB = sizeof(real) == 8 ? 1 : 2;   // blocks of 16 output channels per pass (registers: doubles take two)
 constexpr int kGyWaves = 8;
 constexpr int kGyRing = 4;       // blocks of 16 k in flight (= kUvtKbi: the packing pads k to whole multiples)
 
 __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGyDev a) {
   extern __shared__ __align__(16) unsigned char smem[];
-  float* xs = reinterpret_cast<float*>(smem);
-  float* part = xs + (size_t)16 * a.px;                       // [wavefront][sample][b]
+  real* xs = reinterpret_cast<real*>(smem);
+  real* part = xs + (size_t)16 * a.px;                       // [wavefront][sample][b]
   const int64_t nb0 = (int64_t)blockIdx.x * 16;
   {
     const int kx4 = a.kx / 4, per_sample = a.dx * kx4;
     for (int i = threadIdx.x; i < 16 * per_sample; i += blockDim.x) {
       const int s = i / per_sample, rem = i - s * per_sample, row = rem / kx4, c4 = rem - row * kx4;
       const int64_t n = nb0 + s;
-      floatx4 v = {0.f, 0.f, 0.f, 0.f};
-      if (n < a.n_rows && c4 * 4 < a.cx) v = *reinterpret_cast<const floatx4*>(a.x + (n * a.dx + row) * a.cx + c4 * 4);
-      *reinterpret_cast<floatx4*>(xs + (size_t)s * a.px + row * a.kx + c4 * 4) = v;
+      realx4 v = {0.f, 0.f, 0.f, 0.f};
+      if (n < a.n_rows && c4 * 4 < a.cx) v = *reinterpret_cast<const realx4*>(a.x + (n * a.dx + row) * a.cx + c4 * 4);
+      *reinterpret_cast<realx4*>(xs + (size_t)s * a.px + row * a.kx + c4 * 4) = v;
     }
   }
   for (int i = threadIdx.x; i < kGyWaves * 16 * a.dy; i += blockDim.x) part[i] = 0.f;
@@ -561,28 +596,28 @@ __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGy
   const int wg = wave & (a.wgroups - 1), sg = wave / a.wgroups, sgroups = kGyWaves / a.wgroups;
   const int64_t n = nb0 + r;
   // samples past the end are staged as zeros (Z = 0); their rows of g are read from the last sample
-  const float* gn = a.g + (n < a.n_rows ? n : a.n_rows - 1) * a.dg * a.cout;
-  const float* xl = xs + (size_t)r * a.px + 4 * q;
-  float* mine = part + (size_t)(wave * 16 + r) * a.dy;
-  const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+  const real* gn = a.g + (n < a.n_rows ? n : a.n_rows - 1) * a.dg * a.cout;
+  const real* xl = xs + (size_t)r * a.px + 4 * q;
+  real* mine = part + (size_t)(wave * 16 + r) * a.dy;
+  const realx4 zero = {0.f, 0.f, 0.f, 0.f};
 
   // The passes of this wavefront — (segment, block of 32 output channels) — form one sequence; the weight fragments
   // and the rows of x run kGyRing blocks of 16 k ahead of the matrix instructions, across the ends of the passes
   // (a weight fragment comes from the L2 in more cycles than one block's eight matrix instructions take).
   const int64_t kstride = (int64_t)a.wbp * 256;
-  floatx4 A[kGyRing][kGyWB], B[kGyRing];
-  auto load = [&](const float* wbase, const float* xrow, int kb, floatx4 (&Aj)[kGyWB], floatx4& Bj) __attribute__((always_inline)) {
+  realx4 A[kGyRing][kGyWB], B[kGyRing];
+  auto load = [&](const real* wbase, const real* xrow, int kb, realx4 (&Aj)[kGyWB], realx4& Bj) __attribute__((always_inline)) {
 #pragma unroll
-    for (int wb = 0; wb < kGyWB; ++wb) Aj[wb] = *reinterpret_cast<const floatx4*>(wbase + kb * kstride + wb * 256);
-    Bj = *reinterpret_cast<const floatx4*>(xrow + kb * 16);
+    for (int wb = 0; wb < kGyWB; ++wb) Aj[wb] = *reinterpret_cast<const realx4*>(wbase + kb * kstride + wb * 256);
+    Bj = *reinterpret_cast<const realx4*>(xrow + kb * 16);
   };
   auto wbase_of = [&](const cgtp_uvt_item& it, int wc) __attribute__((always_inline)) {
     return a.wp + ((int64_t)it.p * a.kblocks * a.wbp + wc * kGyWB) * 256 + lane * 4;
   };
   int s = sg, wc = wg;
   cgtp_uvt_item it = uvt_item_at(tab, s < a.n_items ? s : 0);
-  const float* wbase = wbase_of(it, wc);
-  const float* xrow = xl + it.out_row * a.kx;
+  const real* wbase = wbase_of(it, wc);
+  const real* xrow = xl + it.out_row * a.kx;
   if (s < a.n_items) {
 #pragma unroll
     for (int j = 0; j < kGyRing; ++j) load(wbase, xrow, j, A[j], B[j]);   // kblocks is a multiple of kGyRing
@@ -596,13 +631,13 @@ __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGy
     }
     const bool more = s2 < a.n_items;
     const cgtp_uvt_item it2 = uvt_item_at(tab, more ? s2 : s);
-    const float* wbase2 = more ? wbase_of(it2, wc2) : wbase;
-    const float* xrow2 = more ? xl + it2.out_row * a.kx : xrow;
+    const real* wbase2 = more ? wbase_of(it2, wc2) : wbase;
+    const real* xrow2 = more ? xl + it2.out_row * a.kx : xrow;
 
     const int n_t = it.t1 - it.t0;
     // the segment's first kUvtTerms terms in scalar registers (slots past the end: the first term again, never used)
     int mrow[kUvtTerms], brow[kUvtTerms];
-    float c[kUvtTerms];
+    real c[kUvtTerms];
 #pragma unroll
     for (int k = 0; k < kUvtTerms; ++k) {
       const int t = k < n_t ? it.t0 + k : it.t0;
@@ -620,25 +655,25 @@ __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGy
       wcol[wb] = wok[wb] ? w : 0;
     }
     // rows of g of the terms, requested before the matrix instructions; the second half only for long segments
-    floatx4 gv[kUvtTerms][kGyWB];
+    realx4 gv[kUvtTerms][kGyWB];
 #pragma unroll
     for (int k = 0; k < kUvtTerms / 2; ++k)
 #pragma unroll
-      for (int wb = 0; wb < kGyWB; ++wb) gv[k][wb] = *reinterpret_cast<const floatx4*>(gn + mrow[k] + wcol[wb]);
+      for (int wb = 0; wb < kGyWB; ++wb) gv[k][wb] = *reinterpret_cast<const realx4*>(gn + mrow[k] + wcol[wb]);
     if (n_t > kUvtTerms / 2) {
 #pragma unroll
       for (int k = kUvtTerms / 2; k < kUvtTerms; ++k)
 #pragma unroll
-        for (int wb = 0; wb < kGyWB; ++wb) gv[k][wb] = *reinterpret_cast<const floatx4*>(gn + mrow[k] + wcol[wb]);
+        for (int wb = 0; wb < kGyWB; ++wb) gv[k][wb] = *reinterpret_cast<const realx4*>(gn + mrow[k] + wcol[wb]);
     }
 
-    floatx4 acc[kGyWB];
+    realx4 acc[kGyWB];
 #pragma unroll
     for (int wb = 0; wb < kGyWB; ++wb) acc[wb] = zero;
     for (int kb = 0; kb < a.kblocks; kb += kGyRing) {
       const bool wrap = kb + kGyRing >= a.kblocks;   // the blocks requested now belong to the next pass
-      const float* wnext = wrap ? wbase2 : wbase;
-      const float* xnext = wrap ? xrow2 : xrow;
+      const real* wnext = wrap ? wbase2 : wbase;
+      const real* xnext = wrap ? xrow2 : xrow;
       const int kbn = wrap ? 0 : kb + kGyRing;
 #pragma unroll
       for (int j = 0; j < kGyRing; ++j) {
@@ -646,16 +681,16 @@ __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGy
         for (int i = 0; i < 4; ++i)
 #pragma unroll
           for (int wb = 0; wb < kGyWB; ++wb)
-            acc[wb] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[j][wb][i], B[j][i], acc[wb], 0, 0, 0);
+            acc[wb] = mfma16(A[j][wb][i], B[j][i], acc[wb], 0, 0, 0);
         load(wnext, xnext, kbn + j, A[j], B[j]);
       }
     }
     // accumulator: lane (sample r, q) holds Z[n, 16 (wb0 + wb) + 4 q + e]
-    auto add_term = [&](const floatx4 (&gt)[kGyWB], float coef, int b) __attribute__((always_inline)) {
-      float d = 0.f;
+    auto add_term = [&](const realx4 (&gt)[kGyWB], real coef, int b) __attribute__((always_inline)) {
+      real d = 0.f;
 #pragma unroll
       for (int wb = 0; wb < kGyWB; ++wb) {
-        const floatx4 gg = wok[wb] ? gt[wb] : zero;
+        const realx4 gg = wok[wb] ? gt[wb] : zero;
 #pragma unroll
         for (int e = 0; e < 4; ++e) d += gg[e] * acc[wb][e];
       }
@@ -667,10 +702,10 @@ __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGy
     for (int k = 0; k < kUvtTerms; ++k)
       if (k < n_t) add_term(gv[k], c[k], brow[k]);
     for (int t = it.t0 + kUvtTerms; t < it.t1; ++t) {   // longer segments (large irreps only)
-      floatx4 gt[kGyWB];
+      realx4 gt[kGyWB];
       const int m = __builtin_amdgcn_readfirstlane(tab.ta[t]) * a.cout;
 #pragma unroll
-      for (int wb = 0; wb < kGyWB; ++wb) gt[wb] = *reinterpret_cast<const floatx4*>(gn + m + wcol[wb]);
+      for (int wb = 0; wb < kGyWB; ++wb) gt[wb] = *reinterpret_cast<const realx4*>(gn + m + wcol[wb]);
       add_term(gt, tab.tc[t], __builtin_amdgcn_readfirstlane(tab.tb[t]));
     }
     s = s2; wc = wc2; it = it2; wbase = wbase2; xrow = xrow2;
@@ -679,7 +714,7 @@ __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGy
   for (int i = threadIdx.x; i < 16 * a.dy; i += blockDim.x) {
     const int64_t ni = nb0 + i / a.dy;
     if (ni < a.n_rows) {
-      float sum = 0.f;
+      real sum = 0.f;
 #pragma unroll
       for (int w = 0; w < kGyWaves; ++w) sum += part[w * 16 * a.dy + i];
       a.gy[nb0 * a.dy + i] = sum;
@@ -717,14 +752,15 @@ static int uvt_shape(int64_t n_rows, int dx, int dy, int dout, int cx, int cy, i
   d.py = yc ? dy * cy + 4 : (dy | 1);
   const int wblocks = (cout + 15) / 16;
   d.wbp = round_up(wblocks, 4);
-  const int wb = wblocks >= 4 ? 4 : wblocks >= 2 ? 2 : 1;
+  // blocks of 16 output channels per wavefront; in double precision four blocks do not fit the registers
+  const int wb = (wblocks >= 4 && sizeof(real) == 4) ? 4 : wblocks >= 2 ? 2 : 1;
   const int need = (wblocks + wb - 1) / wb;             // wavefronts (or workgroups) that cover the output channels
   int wgroups = need >= 2 ? 2 : 1;
   int igroups = pow2_floor(dout < kUvtMaxGroups / wgroups ? dout : kUvtMaxGroups / wgroups);
   while (wgroups < pow2_ceil(need) && wgroups * 2 * igroups <= kUvtMaxGroups) wgroups *= 2;
   d.zero_floats = yc ? round_up((cx > cy + 4 ? cx : cy + 4) + 4, 4) : d.kblocks * 16 + 16;
-  const int64_t per_block = (int64_t)16 * (d.px + d.py) * 4;   // LDS bytes of one 16-sample block
-  const int64_t fixed = (yc ? (int64_t)d.kblocks * 32 : 0) + (int64_t)d.zero_floats * 4 + 32;
+  const int64_t per_block = (int64_t)16 * (d.px + d.py) * (int64_t)sizeof(real);   // LDS bytes of one 16-sample block
+  const int64_t fixed = (yc ? (int64_t)d.kblocks * 32 : 0) + (int64_t)d.zero_floats * (int64_t)sizeof(real) + 32;
   if (per_block + fixed > kLdsBytes - kUvtTableRoom) return CGTP_ERR_LDS;
   // further sample blocks: while wavefronts are left, two workgroups still fit a compute unit, and the batch is large
   // enough to fill the chip with such workgroups
@@ -743,7 +779,7 @@ static int uvt_shape(int64_t n_rows, int dx, int dy, int dout, int cx, int cy, i
 
 static int uvt_plan(const cgtp_uvt_args* a, UvtPlan* plan) {
   if (!a) return CGTP_ERR_NULL;
-  if (a->dtype != CGTP_F32) return CGTP_ERR_DTYPE;
+  if (a->dtype != kDtype) return CGTP_ERR_DTYPE;
   if (a->n_items < 0 || a->n_terms < 0) return CGTP_ERR_SHAPE;
   const int st = uvt_shape(a->n_rows, a->dx, a->dy, a->dout, a->cx, a->cy, a->cout, plan);
   if (st != CGTP_OK) return st;
@@ -758,68 +794,67 @@ static int uvt_plan(const cgtp_uvt_args* a, UvtPlan* plan) {
   const uintptr_t al = reinterpret_cast<uintptr_t>(a->x) | reinterpret_cast<uintptr_t>(a->wp) |
                        reinterpret_cast<uintptr_t>(a->out) | (a->cy > 0 ? reinterpret_cast<uintptr_t>(a->y) : 0);
   if (al & 15u) return CGTP_ERR_ALIGN;
-  d.x = (const float*)a->x; d.y = (const float*)a->y; d.wp = (const float*)a->wp; d.out = (float*)a->out;
-  d.items = a->items; d.ta = a->term_a; d.tb = a->term_b; d.tc = (const float*)a->term_c;
+  d.x = (const real*)a->x; d.y = (const real*)a->y; d.wp = (const real*)a->wp; d.out = (real*)a->out;
+  d.items = a->items; d.ta = a->term_a; d.tb = a->term_b; d.tc = (const real*)a->term_c;
   d.n_items = a->n_items; d.n_terms = a->n_terms;
   for (int i = 0; i <= kUvtMaxGroups; ++i) d.group_ptr[i] = i <= d.igroups ? a->group_ptr[i] : a->n_items;
-  plan->lds += ((int64_t)a->n_items * 32 + (int64_t)a->n_terms * 12 + 15) / 16 * 16;
+  plan->lds += ((int64_t)a->n_items * 32 + (int64_t)a->n_terms * kTermBytes + 15) / 16 * 16;
   if (plan->lds > kLdsBytes) return CGTP_ERR_LDS;
   return CGTP_OK;
 }
 
-}  // namespace cgtp
+// ---- entry points of this precision (the C entry points below dispatch on dtype) ------------------------------
 
-using namespace cgtp;
-
-extern "C" {
-
-int64_t cgtp_uvt_packed_elems(int32_t n_paths, int64_t K, int32_t cout) {
+int64_t packed_elems(int32_t n_paths, int64_t K, int32_t cout) {
   if (n_paths < 0 || K <= 0 || cout <= 0) return 0;
   return (int64_t)n_paths * round_up((int)((K + 15) / 16), kUvtKbi) * round_up((cout + 15) / 16, 4) * 256;
 }
 
-int cgtp_uvt_pack_weights(const void* w, void* packed, int32_t n_paths, int64_t K, int32_t cout, int64_t stride_p,
+int pack_weights(const void* w, void* packed, int32_t n_paths, int64_t K, int32_t cout, int64_t stride_p,
                           int64_t stride_k, int64_t stride_c, int32_t dtype, void* stream) {
-  if (dtype != CGTP_F32) return CGTP_ERR_DTYPE;
+  if (dtype != kDtype) return CGTP_ERR_DTYPE;
   if (!w || !packed) return CGTP_ERR_NULL;
   if (n_paths < 0 || K <= 0 || cout <= 0 || K > (1 << 24)) return CGTP_ERR_SHAPE;
   if (reinterpret_cast<uintptr_t>(packed) & 15u) return CGTP_ERR_ALIGN;
-  const int64_t n_vec = cgtp_uvt_packed_elems(n_paths, K, cout) / 4;
+  const int64_t n_vec = packed_elems(n_paths, K, cout) / 4;
   if (n_vec == 0) return CGTP_OK;
   hipLaunchKernelGGL(uvt_pack_kernel, dim3((unsigned)((n_vec + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                     (const float*)w, (float*)packed, n_vec, (int)K, (int)cout,
+                     (const real*)w, (real*)packed, n_vec, (int)K, (int)cout,
                      round_up((int)((K + 15) / 16), kUvtKbi), round_up((cout + 15) / 16, 4), stride_p, stride_k, stride_c);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 
-int cgtp_uvt_chunk(int64_t n_rows, int32_t dx, int32_t dy, int32_t dout, int32_t cx, int32_t cy, int32_t cout) {
+int chunk(int64_t n_rows, int32_t dx, int32_t dy, int32_t dout, int32_t cx, int32_t cy, int32_t cout) {
   UvtPlan plan;
   const int st = uvt_shape(n_rows, dx, dy, dout, cx, cy, cout, &plan);
   return st == CGTP_OK ? plan.kbi : -st;
 }
 
-int cgtp_uvt_item_groups(int64_t n_rows, int32_t dx, int32_t dy, int32_t dout, int32_t cx, int32_t cy, int32_t cout) {
+int item_groups(int64_t n_rows, int32_t dx, int32_t dy, int32_t dout, int32_t cx, int32_t cy, int32_t cout) {
   UvtPlan plan;
   const int st = uvt_shape(n_rows, dx, dy, dout, cx, cy, cout, &plan);
   return st == CGTP_OK ? plan.dev.igroups : -st;
 }
 
-int cgtp_uvt_validate(const cgtp_uvt_args* a) {
+int validate(const cgtp_uvt_args* a) {
   UvtPlan plan;
   return uvt_plan(a, &plan);
 }
 
-int cgtp_uvt_apply(const cgtp_uvt_args* a, void* stream) {
+int apply(const cgtp_uvt_args* a, void* stream) {
   UvtPlan plan;
   const int st = uvt_plan(a, &plan);
   if (st != CGTP_OK) return st;
   if (a->n_rows == 0 || a->n_items == 0) return CGTP_OK;
   void (*fn)(const UvtDev) = nullptr;
   if (plan.yc) {
-    fn = plan.wb == 4 ? uvt_apply_kernel<true, 4> : plan.wb == 2 ? uvt_apply_kernel<true, 2> : uvt_apply_kernel<true, 1>;
+    fn = plan.wb == 2 ? uvt_apply_kernel<true, 2> : uvt_apply_kernel<true, 1>;
   } else {
-    fn = plan.wb == 4 ? uvt_apply_kernel<false, 4> : plan.wb == 2 ? uvt_apply_kernel<false, 2> : uvt_apply_kernel<false, 1>;
+    fn = plan.wb == 2 ? uvt_apply_kernel<false, 2> : uvt_apply_kernel<false, 1>;
   }
+#ifndef CGTP_UVT_F64
+  if (plan.wb == 4) fn = plan.yc ? uvt_apply_kernel<true, 4> : uvt_apply_kernel<false, 4>;
+#endif
   if (plan.lds > 48 * 1024 &&
       hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds) != hipSuccess)
     return CGTP_ERR_LDS;
@@ -827,15 +862,15 @@ int cgtp_uvt_apply(const cgtp_uvt_args* a, void* stream) {
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 
-int64_t cgtp_uvt_grad_w_workspace_bytes(int64_t n_rows, int32_t n_paths, int64_t K, int32_t cout) {
+int64_t grad_w_workspace_bytes(int64_t n_rows, int32_t n_paths, int64_t K, int32_t cout) {
   if (n_rows <= 0 || n_paths <= 0 || K <= 0 || cout <= 0) return 0;
   const int64_t chunk = uvt_gw_chunk(n_rows);
-  return ((n_rows + chunk - 1) / chunk) * n_paths * K * cout * (int64_t)sizeof(float);
+  return ((n_rows + chunk - 1) / chunk) * n_paths * K * cout * (int64_t)sizeof(real);
 }
 
-int cgtp_uvt_grad_w(const cgtp_uvt_gw_args* a, void* stream) {
+int grad_w(const cgtp_uvt_gw_args* a, void* stream) {
   if (!a) return CGTP_ERR_NULL;
-  if (a->dtype != CGTP_F32) return CGTP_ERR_DTYPE;
+  if (a->dtype != kDtype) return CGTP_ERR_DTYPE;
   if (a->n_rows < 0 || a->n_paths <= 0 || a->n_items < 0 || a->dx <= 0 || a->dy <= 0 || a->dg <= 0 || a->cx <= 0 ||
       a->cy < 0 || a->cout <= 0)
     return CGTP_ERR_SHAPE;
@@ -851,13 +886,13 @@ int cgtp_uvt_grad_w(const cgtp_uvt_gw_args* a, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   if (a->n_rows == 0) {   // no samples: the gradient is zero (written by the summation kernel over zero chunks)
     hipLaunchKernelGGL(uvt_gw_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, st,
-                       (const float*)nullptr, (float*)a->gw, (int64_t)0, n_out);
+                       (const real*)nullptr, (real*)a->gw, (int64_t)0, n_out);
     return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
   }
   if (!a->workspace) return CGTP_ERR_WORKSPACE;
   UvtGwDev d;
-  d.x = (const float*)a->x; d.y = (const float*)a->y; d.g = (const float*)a->g; d.part = (float*)a->workspace;
-  d.items = a->items; d.path_ptr = a->path_ptr; d.ta = a->term_a; d.tb = a->term_b; d.tc = (const float*)a->term_c;
+  d.x = (const real*)a->x; d.y = (const real*)a->y; d.g = (const real*)a->g; d.part = (real*)a->workspace;
+  d.items = a->items; d.path_ptr = a->path_ptr; d.ta = a->term_a; d.tb = a->term_b; d.tc = (const real*)a->term_c;
   d.n_rows = a->n_rows; d.n_paths = a->n_paths; d.dx = a->dx; d.dy = a->dy; d.dg = a->dg; d.cx = a->cx; d.cy = a->cy;
   d.cout = a->cout; d.K = (int)K;
   d.chunk = (int)uvt_gw_chunk(a->n_rows);
@@ -871,13 +906,13 @@ int cgtp_uvt_grad_w(const cgtp_uvt_gw_args* a, void* stream) {
     hipLaunchKernelGGL(uvt_grad_w_kernel<false>, grid, dim3(256), 0, st, d);
   if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
   hipLaunchKernelGGL(uvt_gw_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, st,
-                     (const float*)a->workspace, (float*)a->gw, n_chunks, n_out);
+                     (const real*)a->workspace, (real*)a->gw, n_chunks, n_out);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 
-int cgtp_uvt_grad_y(const cgtp_uvt_gy_args* a, void* stream) {
+int grad_y(const cgtp_uvt_gy_args* a, void* stream) {
   if (!a) return CGTP_ERR_NULL;
-  if (a->dtype != CGTP_F32) return CGTP_ERR_DTYPE;
+  if (a->dtype != kDtype) return CGTP_ERR_DTYPE;
   if (a->n_rows < 0 || a->n_items < 0 || a->n_terms < 0 || a->dx <= 0 || a->dy <= 0 || a->dg <= 0 || a->cx <= 0 ||
       a->cout <= 0)
     return CGTP_ERR_SHAPE;
@@ -887,8 +922,8 @@ int cgtp_uvt_grad_y(const cgtp_uvt_gy_args* a, void* stream) {
   if ((reinterpret_cast<uintptr_t>(a->x) | reinterpret_cast<uintptr_t>(a->g) | reinterpret_cast<uintptr_t>(a->wp)) & 15u)
     return CGTP_ERR_ALIGN;
   UvtGyDev d;
-  d.x = (const float*)a->x; d.g = (const float*)a->g; d.wp = (const float*)a->wp; d.gy = (float*)a->gy;
-  d.items = a->items; d.ta = a->term_m; d.tb = a->term_b; d.tc = (const float*)a->term_c;
+  d.x = (const real*)a->x; d.g = (const real*)a->g; d.wp = (const real*)a->wp; d.gy = (real*)a->gy;
+  d.items = a->items; d.ta = a->term_m; d.tb = a->term_b; d.tc = (const real*)a->term_c;
   d.n_rows = a->n_rows; d.n_items = a->n_items; d.n_terms = a->n_terms;
   d.dx = a->dx; d.dy = a->dy; d.dg = a->dg; d.cx = a->cx; d.cout = a->cout;
   d.kblocks = round_up((a->cx + 15) / 16, kUvtKbi);
@@ -897,8 +932,8 @@ int cgtp_uvt_grad_y(const cgtp_uvt_gy_args* a, void* stream) {
   d.wbp = round_up((a->cout + 15) / 16, 4);
   d.wchunks = (a->cout + 16 * kGyWB - 1) / (16 * kGyWB);
   d.wgroups = d.wchunks >= 4 ? 4 : d.wchunks >= 2 ? 2 : 1;
-  const int64_t lds = ((int64_t)16 * d.px + (int64_t)kGyWaves * 16 * a->dy) * 4 + (int64_t)a->n_items * 32 +
-                      (int64_t)a->n_terms * 12 + 16;
+  const int64_t lds = ((int64_t)16 * d.px + (int64_t)kGyWaves * 16 * a->dy) * (int64_t)sizeof(real) +
+                      (int64_t)a->n_items * 32 + (int64_t)a->n_terms * kTermBytes + 16;
   if (lds > kLdsBytes) return CGTP_ERR_LDS;
   if (a->n_rows == 0) return CGTP_OK;
   if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)uvt_grad_y_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -909,4 +944,72 @@ int cgtp_uvt_grad_y(const cgtp_uvt_gy_args* a, void* stream) {
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 
+
+}  // namespace UVT_NS
+}  // namespace cgtp
+
+#ifndef CGTP_UVT_F64
+// The double-precision set of the same kernels and entry points: uvt_kernels_f64.hip compiles this file with
+// CGTP_UVT_F64 defined.
+namespace cgtp {
+namespace uvt_f64 {
+int pack_weights(const void* w, void* packed, int32_t n_paths, int64_t K, int32_t cout, int64_t stride_p, int64_t stride_k,
+                 int64_t stride_c, int32_t dtype, void* stream);
+int chunk(int64_t n_rows, int32_t dx, int32_t dy, int32_t dout, int32_t cx, int32_t cy, int32_t cout);
+int item_groups(int64_t n_rows, int32_t dx, int32_t dy, int32_t dout, int32_t cx, int32_t cy, int32_t cout);
+int validate(const cgtp_uvt_args* a);
+int apply(const cgtp_uvt_args* a, void* stream);
+int64_t grad_w_workspace_bytes(int64_t n_rows, int32_t n_paths, int64_t K, int32_t cout);
+int grad_w(const cgtp_uvt_gw_args* a, void* stream);
+int grad_y(const cgtp_uvt_gy_args* a, void* stream);
+}  // namespace uvt_f64
+}  // namespace cgtp
+
+using namespace cgtp;
+
+extern "C" {
+
+int64_t cgtp_uvt_packed_elems(int32_t n_paths, int64_t K, int32_t cout) { return uvt_f32::packed_elems(n_paths, K, cout); }
+
+int cgtp_uvt_pack_weights(const void* w, void* packed, int32_t n_paths, int64_t K, int32_t cout, int64_t stride_p,
+                          int64_t stride_k, int64_t stride_c, int32_t dtype, void* stream) {
+  return dtype == CGTP_F64 ? uvt_f64::pack_weights(w, packed, n_paths, K, cout, stride_p, stride_k, stride_c, dtype, stream)
+                           : uvt_f32::pack_weights(w, packed, n_paths, K, cout, stride_p, stride_k, stride_c, dtype, stream);
+}
+
+int cgtp_uvt_chunk(int64_t n_rows, int32_t dx, int32_t dy, int32_t dout, int32_t cx, int32_t cy, int32_t cout,
+                   int32_t dtype) {
+  if (dtype != CGTP_F32 && dtype != CGTP_F64) return -CGTP_ERR_DTYPE;
+  return dtype == CGTP_F64 ? uvt_f64::chunk(n_rows, dx, dy, dout, cx, cy, cout) : uvt_f32::chunk(n_rows, dx, dy, dout, cx, cy, cout);
+}
+
+int cgtp_uvt_item_groups(int64_t n_rows, int32_t dx, int32_t dy, int32_t dout, int32_t cx, int32_t cy, int32_t cout,
+                         int32_t dtype) {
+  if (dtype != CGTP_F32 && dtype != CGTP_F64) return -CGTP_ERR_DTYPE;
+  return dtype == CGTP_F64 ? uvt_f64::item_groups(n_rows, dx, dy, dout, cx, cy, cout)
+                           : uvt_f32::item_groups(n_rows, dx, dy, dout, cx, cy, cout);
+}
+
+int cgtp_uvt_validate(const cgtp_uvt_args* a) {
+  return a && a->dtype == CGTP_F64 ? uvt_f64::validate(a) : uvt_f32::validate(a);
+}
+
+int cgtp_uvt_apply(const cgtp_uvt_args* a, void* stream) {
+  return a && a->dtype == CGTP_F64 ? uvt_f64::apply(a, stream) : uvt_f32::apply(a, stream);
+}
+
+int64_t cgtp_uvt_grad_w_workspace_bytes(int64_t n_rows, int32_t n_paths, int64_t K, int32_t cout, int32_t dtype) {
+  return dtype == CGTP_F64 ? uvt_f64::grad_w_workspace_bytes(n_rows, n_paths, K, cout)
+                           : uvt_f32::grad_w_workspace_bytes(n_rows, n_paths, K, cout);
+}
+
+int cgtp_uvt_grad_w(const cgtp_uvt_gw_args* a, void* stream) {
+  return a && a->dtype == CGTP_F64 ? uvt_f64::grad_w(a, stream) : uvt_f32::grad_w(a, stream);
+}
+
+int cgtp_uvt_grad_y(const cgtp_uvt_gy_args* a, void* stream) {
+  return a && a->dtype == CGTP_F64 ? uvt_f64::grad_y(a, stream) : uvt_f32::grad_y(a, stream);
+}
+
 }  // extern "C"
+#endif  // CGTP_UVT_F64

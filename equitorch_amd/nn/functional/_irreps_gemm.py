@@ -383,7 +383,7 @@ def _table_driven_path(x: Tensor, weight: Tensor, plan: LinearPlan, in_size: int
     from ..._tables import TpCoo
     from ...ops import kernels
     from . import _uv_native
-    if x.dtype != torch.float32 or weight.ndim != 3 or x.shape[0] == 0:
+    if x.dtype not in (torch.float32, torch.float64) or weight.ndim != 3 or x.shape[0] == 0:
         return None
 
     def build():
@@ -399,11 +399,11 @@ def _table_driven_path(x: Tensor, weight: Tensor, plan: LinearPlan, in_size: int
     table = cached(anchor, ("linear_as_coo_table", in_size, plan.n_paths, plan.out_size), build)
     if table is False:
         return None
-    ones = cached(anchor, ("ones_fp32", x.shape[0], str(x.device)),
-                  lambda: torch.ones(x.shape[0], 1, dtype=torch.float32, device=x.device))
+    ones = cached(anchor, ("ones", x.dtype, x.shape[0], str(x.device)),
+                  lambda: torch.ones(x.shape[0], 1, dtype=x.dtype, device=x.device))
     if not _uv_native.u1v_supported(x, ones, weight, table):
         return None
-    kernels.log_tier("irreps_linear", "table-driven matrix-core kernels (fp32)")
+    kernels.log_tier("irreps_linear", "table-driven matrix-core kernels")
     return _uv_native.u1v(x, ones, weight, table)
 
 

@@ -39,7 +39,17 @@ def _anchor(table) -> Tensor:
 MAX_TERMS = 8      # terms of a segment the weight-gradient kernel holds in registers (kUvtTerms)
 
 
-class _Walk:
+class _Coefficients:
+    """The coefficients of a walk's terms as a device tensor of the launch's dtype (made on first use)."""
+
+    def term_c(self, dtype: torch.dtype) -> Tensor:
+        if dtype not in self._term_c:
+            self._term_c[dtype] = torch.from_numpy(np.ascontiguousarray(self._coef, dtype=np.float64)).to(
+                device=self._device, dtype=dtype)
+        return self._term_c[dtype]
+
+
+class _Walk(_Coefficients):
     """Item list of one role of one table: one item per segment (weight path, output row), the items of a row
     consecutive, the rows dealt to ``n_groups`` groups of about equal numbers of items (the wavefronts of a workgroup
     take one group each)."""
@@ -73,7 +83,7 @@ class _Walk:
         self.items = torch.tensor(flat, dtype=torch.int32).reshape(-1, 8).to(device)
         self.term_a = torch.from_numpy(a_idx.astype(np.int32)).to(device)
         self.term_b = torch.from_numpy(b_idx.astype(np.int32)).to(device)
-        self.term_c = torch.from_numpy(coef.astype(np.float32)).to(device)
+        self._coef, self._device, self._term_c = coef, device, {}
 
 
 def _walk(tp_info, role: str, n_groups: int, device) -> _Walk:
@@ -91,7 +101,7 @@ def _walk(tp_info, role: str, n_groups: int, device) -> _Walk:
     return kernels.cached(_anchor(tp_info), ("uvt_walk", role, n_groups, str(device)), build)
 
 
-class _PathWalk:
+class _PathWalk(_Coefficients):
     """Segments (weight path, output row) of a table sorted by path, with their terms: the walk of the weight-gradient
     kernel, which owns one path per workgroup."""
 
@@ -115,7 +125,7 @@ class _PathWalk:
         self.path_ptr = torch.tensor(path_ptr, dtype=torch.int32).to(device)
         self.term_a = torch.from_numpy(a_idx.astype(np.int32)).to(device)
         self.term_b = torch.from_numpy(b_idx.astype(np.int32)).to(device)
-        self.term_c = torch.from_numpy(coef.astype(np.float32)).to(device)
+        self._coef, self._device, self._term_c = coef, device, {}
 
 
 def grad_w(x: Tensor, y: Tensor, g: Tensor, tp_info) -> Tensor:
@@ -128,20 +138,20 @@ def grad_w(x: Tensor, y: Tensor, g: Tensor, tp_info) -> Tensor:
     cy = y.shape[2] if y.ndim == 3 else 0
     k = cx * cy if cy else cx
     cout = g.shape[-1]
-    gw = torch.empty((walk.n_paths, k, cout), dtype=torch.float32, device=x.device)
-    ws = torch.empty(max(int(_lib.lib.cgtp_uvt_grad_w_workspace_bytes(n, walk.n_paths, k, cout)), 16), dtype=torch.uint8,
+    gw = torch.empty((walk.n_paths, k, cout), dtype=x.dtype, device=x.device)
+    ws = torch.empty(max(int(_lib.lib.cgtp_uvt_grad_w_workspace_bytes(n, walk.n_paths, k, cout, _lib.dtype_code(x.dtype))), 16), dtype=torch.uint8,
                      device=x.device)
     a = _lib.UvtGwArgs()
     a.x, a.y, a.g, a.gw, a.workspace = x.data_ptr(), y.data_ptr(), g.data_ptr(), gw.data_ptr(), ws.data_ptr()
     a.items, a.path_ptr = walk.items.data_ptr(), walk.path_ptr.data_ptr()
-    a.term_a, a.term_b, a.term_c = walk.term_a.data_ptr(), walk.term_b.data_ptr(), walk.term_c.data_ptr()
+    a.term_a, a.term_b, a.term_c = walk.term_a.data_ptr(), walk.term_b.data_ptr(), walk.term_c(x.dtype).data_ptr()
     a.n_rows, a.n_items, a.n_terms, a.n_paths = n, walk.n_items, walk.n_terms, walk.n_paths
-    a.dx, a.dy, a.dg, a.cx, a.cy, a.cout, a.dtype = dx, dy, g.shape[1], cx, cy, cout, _lib.F32
+    a.dx, a.dy, a.dg, a.cx, a.cy, a.cout, a.dtype = dx, dy, g.shape[1], cx, cy, cout, _lib.dtype_code(x.dtype)
     _lib.check(_lib.lib.cgtp_uvt_grad_w(C.byref(a), _lib.stream_ptr(x.device)), "cgtp_uvt_grad_w")
     return gw
 
 
-class _SegWalk:
+class _SegWalk(_Coefficients):
     """Segments (weight path, row of the first operand) with their terms (row of grad_out, row of the second operand):
     the walk of ``cgtp_uvt_grad_y``.  Segments are not split: the kernel forms one matrix product per segment."""
 
@@ -163,14 +173,14 @@ class _SegWalk:
         self.items = torch.tensor(items, dtype=torch.int32).reshape(-1, 8).to(device)
         self.term_m = torch.from_numpy(m_idx.astype(np.int32)).to(device)
         self.term_b = torch.from_numpy(b_idx.astype(np.int32)).to(device)
-        self.term_c = torch.from_numpy(coef.astype(np.float32)).to(device)
+        self._coef, self._device, self._term_c = coef, device, {}
 
 
-def grad_y_supported(n: int, dx: int, dy: int, cx: int, cout: int, tp_info) -> bool:
+def grad_y_supported(n: int, dx: int, dy: int, cx: int, cout: int, tp_info, itemsize: int = 4) -> bool:
     """Whether the 16 staged samples of a ``cgtp_uvt_grad_y`` workgroup and its tables fit the LDS."""
     c = _coo(tp_info)
     kx = ((cx + 15) // 16 + 3) // 4 * 4 * 16
-    lds = (16 * (dx * kx + 4) + 8 * 16 * dy) * 4 + len(c.coef) * (32 + 12) + 16
+    lds = (16 * (dx * kx + 4) + 8 * 16 * dy) * itemsize + len(c.coef) * (32 + 8 + itemsize) + 16
     return cx % 4 == 0 and cout % 4 == 0 and lds <= 160 * 1024
 
 
@@ -180,28 +190,28 @@ def grad_y(x: Tensor, g: Tensor, wp: Tensor, tp_info, dy: int) -> Tensor:
     walk = kernels.cached(_anchor(tp_info), ("uvt_seg_walk", str(x.device)),
                           lambda: _SegWalk(_coo(tp_info), x.device))
     n, dx, cx = x.shape
-    gy = torch.empty((n, dy), dtype=torch.float32, device=x.device)
+    gy = torch.empty((n, dy), dtype=x.dtype, device=x.device)
     a = _lib.UvtGyArgs()
     a.x, a.g, a.wp, a.gy = x.data_ptr(), g.data_ptr(), wp.data_ptr(), gy.data_ptr()
     a.items, a.term_m, a.term_b, a.term_c = (walk.items.data_ptr(), walk.term_m.data_ptr(), walk.term_b.data_ptr(),
-                                             walk.term_c.data_ptr())
+                                             walk.term_c(x.dtype).data_ptr())
     a.n_rows, a.n_items, a.n_terms = n, walk.n_items, walk.n_terms
-    a.dx, a.dy, a.dg, a.cx, a.cout, a.dtype = dx, dy, g.shape[1], cx, g.shape[2], _lib.F32
+    a.dx, a.dy, a.dg, a.cx, a.cout, a.dtype = dx, dy, g.shape[1], cx, g.shape[2], _lib.dtype_code(x.dtype)
     _lib.check(_lib.lib.cgtp_uvt_grad_y(C.byref(a), _lib.stream_ptr(x.device)), "cgtp_uvt_grad_y")
     return gy
 
 
-def chunk_of(n_rows: int, dx: int, dy: int, dout: int, cx: int, cy: int, cout: int) -> int:
+def chunk_of(n_rows: int, dx: int, dy: int, dout: int, cx: int, cy: int, cout: int, dtype=torch.float32) -> int:
     """Blocks of 16 contracted channels a launch with these extents pads to; <= 0: the kernels do not take them
     (channel counts not multiples of 4, rows of 16 samples beyond the LDS)."""
-    return int(_lib.lib.cgtp_uvt_chunk(n_rows, dx, dy, dout, cx, cy, cout))
+    return int(_lib.lib.cgtp_uvt_chunk(n_rows, dx, dy, dout, cx, cy, cout, _lib.dtype_code(dtype)))
 
 
 def pack(w: Tensor, n_paths: int, k: int, cout: int, stride_p: int, stride_k: int, stride_c: int) -> Tensor:
     """The weight viewed as ``(n_paths, k, cout)`` through element strides, in matrix-core fragment order."""
-    packed = torch.empty(int(_lib.lib.cgtp_uvt_packed_elems(n_paths, k, cout)), dtype=torch.float32, device=w.device)
+    packed = torch.empty(int(_lib.lib.cgtp_uvt_packed_elems(n_paths, k, cout)), dtype=w.dtype, device=w.device)
     _lib.check(_lib.lib.cgtp_uvt_pack_weights(w.data_ptr(), packed.data_ptr(), n_paths, k, cout, stride_p, stride_k,
-                                              stride_c, _lib.F32, _lib.stream_ptr(w.device)), "cgtp_uvt_pack_weights")
+                                              stride_c, _lib.dtype_code(w.dtype), _lib.stream_ptr(w.device)), "cgtp_uvt_pack_weights")
     return packed
 
 
@@ -211,10 +221,10 @@ def apply(x: Tensor, y: Tensor, wp: Tensor, tp_info, role: str, dout: int, cout:
     dy = y.shape[1]
     cy = y.shape[2] if y.ndim == 3 else 0
     k = cx * cy if cy else cx
-    kbi = chunk_of(n, dx, dy, dout, cx, cy, cout)
+    kbi = chunk_of(n, dx, dy, dout, cx, cy, cout, x.dtype)
     if kbi <= 0:
         raise _lib.CgtpError(f"cgtp_uvt_apply does not take these extents (status {-kbi})")
-    n_groups = int(_lib.lib.cgtp_uvt_item_groups(n, dx, dy, dout, cx, cy, cout))
+    n_groups = int(_lib.lib.cgtp_uvt_item_groups(n, dx, dy, dout, cx, cy, cout, _lib.dtype_code(x.dtype)))
     walk = _walk(tp_info, role, n_groups, x.device)
     out = torch.empty((n, dout, cout), dtype=x.dtype, device=x.device)
     if n == 0:
@@ -222,10 +232,10 @@ def apply(x: Tensor, y: Tensor, wp: Tensor, tp_info, role: str, dout: int, cout:
     a = _lib.UvtArgs()
     a.x, a.y, a.wp, a.out = x.data_ptr(), y.data_ptr(), wp.data_ptr(), out.data_ptr()
     a.items, a.term_a, a.term_b, a.term_c = (walk.items.data_ptr(), walk.term_a.data_ptr(), walk.term_b.data_ptr(),
-                                             walk.term_c.data_ptr())
+                                             walk.term_c(x.dtype).data_ptr())
     a.n_rows, a.n_items, a.n_terms = n, walk.n_items, walk.term_a.shape[0]
     a.dx, a.dy, a.dout, a.cx, a.cy, a.cout = dx, dy, dout, cx, cy, cout
-    a.kbi, a.dtype = kbi, _lib.F32
+    a.kbi, a.dtype = kbi, _lib.dtype_code(x.dtype)
     a.n_groups = n_groups
     for i, v in enumerate(walk.group_ptr):
         a.group_ptr[i] = v
@@ -278,15 +288,17 @@ class _U1vNative(Function):
 
 
 def u1v_supported(x: Tensor, y: Tensor, w: Tensor, tp_info) -> bool:
-    if not (x.dtype == y.dtype == w.dtype == torch.float32 and x.ndim == 3 and y.ndim == 2 and w.ndim == 3):
+    if not (x.dtype == y.dtype == w.dtype and x.dtype in (torch.float32, torch.float64) and x.ndim == 3 and y.ndim == 2
+            and w.ndim == 3):
         return False
     if x.shape[0] == 0:
         return False
     c = _coo(tp_info)
     _, u, wc = w.shape
     n = x.shape[0]
-    return (chunk_of(n, c.D1, c.D2, c.DO, u, 0, wc) > 0 and chunk_of(n, c.DO, c.D2, c.D1, wc, 0, u) > 0
-            and grad_y_supported(n, c.D1, c.D2, u, wc, tp_info) and x.data_ptr() % 16 == 0)
+    dt = x.dtype
+    return (chunk_of(n, c.D1, c.D2, c.DO, u, 0, wc, dt) > 0 and chunk_of(n, c.DO, c.D2, c.D1, wc, 0, u, dt) > 0
+            and grad_y_supported(n, c.D1, c.D2, u, wc, tp_info, x.element_size()) and x.data_ptr() % 16 == 0)
 
 
 def u1v(x: Tensor, y: Tensor, w: Tensor, tp_info) -> Tensor:
@@ -335,15 +347,17 @@ class _UvwNative(Function):
 
 
 def uvw_supported(x: Tensor, y: Tensor, w: Tensor, tp_info) -> bool:
-    if not (x.dtype == y.dtype == w.dtype == torch.float32 and x.ndim == 3 and y.ndim == 3 and w.ndim == 4):
+    if not (x.dtype == y.dtype == w.dtype and x.dtype in (torch.float32, torch.float64) and x.ndim == 3 and y.ndim == 3
+            and w.ndim == 4):
         return False
     if x.shape[0] == 0:
         return False
     c = _coo(tp_info)
     _, u, v, wc = w.shape
     n = x.shape[0]
-    return (chunk_of(n, c.D1, c.D2, c.DO, u, v, wc) > 0 and chunk_of(n, c.D2, c.DO, c.D1, v, wc, u) > 0
-            and chunk_of(n, c.DO, c.D1, c.D2, wc, u, v) > 0 and x.data_ptr() % 16 == 0 and y.data_ptr() % 16 == 0)
+    dt = x.dtype
+    return (chunk_of(n, c.D1, c.D2, c.DO, u, v, wc, dt) > 0 and chunk_of(n, c.D2, c.DO, c.D1, v, wc, u, dt) > 0
+            and chunk_of(n, c.DO, c.D1, c.D2, wc, u, v, dt) > 0 and x.data_ptr() % 16 == 0 and y.data_ptr() % 16 == 0)
 
 
 def uvw(x: Tensor, y: Tensor, w: Tensor, tp_info) -> Tensor:

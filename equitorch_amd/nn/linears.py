@@ -276,7 +276,7 @@ class SO2Linear(nn.Module):
                 and weight.shape[-3] == self.num_weights and input.ndim >= 3):
             if weight.ndim == 3:
                 _lib_require(input, weight)
-                if input.dtype == torch.float32:
+                if input.dtype in (torch.float32, torch.float64):
                     # every table entry is one (C_in, C_out) product on one component: the table-driven matrix-core
                     # kernels of the fully connected product take the table as it is
                     from .functional import _irreps_gemm as G

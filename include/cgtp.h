@@ -326,7 +326,7 @@ int64_t cgtp_uv_grad_w_workspace_bytes(int cfg, int64_t n_rows, int32_t cin, int
 int cgtp_uv_grad_w(int cfg, const void* x, const void* y, const void* g, void* gw, void* workspace, int64_t n_rows,
                    int32_t cin, int32_t cout, int32_t dtype, const float* path_scale, void* stream);
 
-/* ---- fully connected products in fp32 on the matrix cores, any table --------------------------------------------
+/* ---- fully connected products in fp32 / fp64 on the matrix cores, any table --------------------------------------
  *
  *   out[n, M, w] = sum_{segments s = (p, M)} sum_k inter_s[n, k] * W[p, k, w]
  *   inter_s[n, k] = sum_{t in s} coef_t * x[n, a_t, k] * y[n, b_t]                       (cy == 0, K = cx)
@@ -344,7 +344,8 @@ int cgtp_uv_grad_w(int cfg, const void* x, const void* y, const void* g, void* g
  * output rows: the list is ordered in cgtp_uvt_item_groups() groups of whole rows, group i being items group_ptr[i] ..
  * group_ptr[i + 1] (groups of about equal length keep the wavefronts equally busy; empty groups are allowed).
  * cgtp_uvt_chunk() (blocks of 16 k the kernels pad K to with zero weights) must be passed as `kbi`.
- * x (n_rows, dx, cx), y (n_rows, dy) or (n_rows, dy, cy), out (n_rows, dout, cout), all fp32 and contiguous; cx, cy,
+ * x (n_rows, dx, cx), y (n_rows, dy) or (n_rows, dy, cy), out (n_rows, dout, cout), all of one dtype (CGTP_F32 |
+ * CGTP_F64) and contiguous; cx, cy,
  * cout multiples of 4, cx * cy a multiple of 16 when cy > 0; 16-byte aligned pointers; the rows of 16 samples must
  * fit the LDS (CGTP_ERR_LDS otherwise).  wp = cgtp_uvt_pack_weights(W): W (n_paths, K, cout) read through element
  * strides (so that a transposed or flattened view needs no copy), rewritten in matrix-core fragment order, zero-padded;
@@ -368,7 +369,7 @@ typedef struct cgtp_uvt_args {
   int32_t dx, dy, dout;
   int32_t cx, cy, cout;
   int32_t kbi;                  /* chunk length the items were cut for: cgtp_uvt_chunk() */
-  int32_t dtype;                /* CGTP_F32 */
+  int32_t dtype;                /* CGTP_F32 | CGTP_F64 */
   int32_t n_terms;              /* entries of term_a / term_b / term_c (the tables are copied to LDS: 32 B per item +
                                    12 B per term must fit next to the samples' rows, CGTP_ERR_LDS otherwise) */
   int32_t n_groups;             /* cgtp_uvt_item_groups() */
@@ -380,8 +381,10 @@ int cgtp_uvt_pack_weights(const void* w, void* packed, int32_t n_paths, int64_t 
                           int64_t stride_k, int64_t stride_c, int32_t dtype, void* stream);
 /* Launch shape for these extents, or -status when the kernels do not take them: blocks of 16 k that K is padded to
  * a multiple of; groups of output rows the item list has to come in.  Host only. */
-int cgtp_uvt_chunk(int64_t n_rows, int32_t dx, int32_t dy, int32_t dout, int32_t cx, int32_t cy, int32_t cout);
-int cgtp_uvt_item_groups(int64_t n_rows, int32_t dx, int32_t dy, int32_t dout, int32_t cx, int32_t cy, int32_t cout);
+int cgtp_uvt_chunk(int64_t n_rows, int32_t dx, int32_t dy, int32_t dout, int32_t cx, int32_t cy, int32_t cout,
+                   int32_t dtype);
+int cgtp_uvt_item_groups(int64_t n_rows, int32_t dx, int32_t dy, int32_t dout, int32_t cx, int32_t cy, int32_t cout,
+                         int32_t dtype);
 int cgtp_uvt_validate(const cgtp_uvt_args* args);
 int cgtp_uvt_apply(const cgtp_uvt_args* args, void* stream);
 
@@ -411,11 +414,11 @@ typedef struct cgtp_uvt_gw_args {
   int32_t n_items, n_terms, n_paths;
   int32_t dx, dy, dg;
   int32_t cx, cy, cout;
-  int32_t dtype;                /* CGTP_F32 */
+  int32_t dtype;                /* CGTP_F32 | CGTP_F64 */
   int32_t reserved_;
 } cgtp_uvt_gw_args;
 
-int64_t cgtp_uvt_grad_w_workspace_bytes(int64_t n_rows, int32_t n_paths, int64_t K, int32_t cout);
+int64_t cgtp_uvt_grad_w_workspace_bytes(int64_t n_rows, int32_t n_paths, int64_t K, int32_t cout, int32_t dtype);
 int cgtp_uvt_grad_w(const cgtp_uvt_gw_args* args, void* stream);
 
 /* Gradient of a second operand without channels (u1v):
@@ -438,7 +441,7 @@ typedef struct cgtp_uvt_gy_args {
   int32_t n_items, n_terms;
   int32_t dx, dy, dg;
   int32_t cx, cout;
-  int32_t dtype;                /* CGTP_F32 */
+  int32_t dtype;                /* CGTP_F32 | CGTP_F64 */
 } cgtp_uvt_gy_args;
 
 int cgtp_uvt_grad_y(const cgtp_uvt_gy_args* args, void* stream);

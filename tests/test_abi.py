@@ -254,12 +254,15 @@ def test_table_driven_matrix_core_entry_points_validate_on_the_host():
     p16 = 4096
     # lmax = 3, 128 -> 128 channels: four blocks of 16 k per ring turn; 16 output rows over 4 item groups (the other
     # two wavefronts of a sample block split the 128 output channels)
-    assert L.cgtp_uvt_chunk(32768, 16, 16, 16, 128, 0, 128) == 4
-    assert L.cgtp_uvt_item_groups(32768, 16, 16, 16, 128, 0, 128) == 4
-    assert L.cgtp_uvt_item_groups(32768, 9, 9, 1, 32, 0, 64) == 1           # a single output row
-    assert L.cgtp_uvt_item_groups(32768, 9, 9, 9, 32, 0, 32) == 8           # one wavefront covers the channels
-    assert L.cgtp_uvt_chunk(100, 16, 16, 16, 130, 0, 128) == -2             # channels not a multiple of 4
-    assert L.cgtp_uvt_chunk(100, 49, 49, 49, 128, 0, 128) == -6             # 16 samples x 49 rows x 128 floats > LDS
+    assert L.cgtp_uvt_chunk(32768, 16, 16, 16, 128, 0, 128, _lib.F32) == 4
+    assert L.cgtp_uvt_item_groups(32768, 16, 16, 16, 128, 0, 128, _lib.F32) == 4
+    assert L.cgtp_uvt_item_groups(32768, 9, 9, 1, 32, 0, 64, _lib.F32) == 1           # a single output row
+    assert L.cgtp_uvt_item_groups(32768, 9, 9, 9, 32, 0, 32, _lib.F64) == 8           # one wavefront covers the channels
+    assert L.cgtp_uvt_chunk(100, 16, 16, 16, 130, 0, 128, _lib.F32) == -2             # channels not a multiple of 4
+    assert L.cgtp_uvt_chunk(100, 49, 49, 49, 128, 0, 128, _lib.F32) == -6   # 16 samples x 49 rows x 128 floats > LDS
+    assert L.cgtp_uvt_chunk(100, 16, 16, 16, 128, 0, 128, _lib.F64) == -6   # the same rows as doubles do not fit either
+    assert L.cgtp_uvt_chunk(100, 16, 16, 16, 64, 0, 128, _lib.F64) == 4
+    assert L.cgtp_uvt_chunk(100, 16, 16, 16, 64, 0, 128, _lib.BF16) == -4
     assert L.cgtp_uvt_packed_elems(23, 128, 128) == 23 * 8 * 8 * 256
     assert L.cgtp_uvt_packed_elems(2, 20, 12) == 2 * 4 * 4 * 256            # padded to whole ring turns / 4 blocks
     a = _lib.UvtArgs()
@@ -283,8 +286,8 @@ def test_table_driven_matrix_core_entry_points_validate_on_the_host():
     assert L.cgtp_uvt_pack_weights(p16, p16, 2, 0, 16, 1, 1, 1, _lib.F32, None) == 2
     assert L.cgtp_uvt_pack_weights(None, p16, 2, 16, 16, 1, 1, 1, _lib.F32, None) == 1
     # weight gradient: chunks of at least 256 samples, at most 128 of them
-    assert L.cgtp_uvt_grad_w_workspace_bytes(32768, 23, 128, 128) == 128 * 23 * 128 * 128 * 4
-    assert L.cgtp_uvt_grad_w_workspace_bytes(300, 4, 32, 16) == 2 * 4 * 32 * 16 * 4
+    assert L.cgtp_uvt_grad_w_workspace_bytes(32768, 23, 128, 128, _lib.F32) == 128 * 23 * 128 * 128 * 4
+    assert L.cgtp_uvt_grad_w_workspace_bytes(300, 4, 32, 16, _lib.F64) == 2 * 4 * 32 * 16 * 8
     g = _lib.UvtGwArgs()
     g.dtype = _lib.F32
     g.n_rows, g.n_paths, g.dx, g.dy, g.dg, g.cx, g.cy, g.cout = 10, 4, 9, 9, 9, 32, 0, 30

@@ -30,6 +30,51 @@ U1V_CASES = [  # irreps (out, in1, in2), C_in, C_out, N, module options
 ]
 
 
+@pytest.mark.parametrize("irreps,cin,cout,n", [((_sh(2),) * 3, 64, 32, 300), ((_sh(2), _sh(3), _sh(2)), 32, 48, 70),
+                                              (("1o+2e+1e", "0e+1o+2e", "0e+1o"), 20, 12, 515)])
+def test_u1v_fp64_native(device, irreps, cin, cout, n):
+    """The same kernels in double precision (v_mfma_f64_16x16x4_f64): forward and all gradients to 1e-11 of the
+    tensor's largest magnitude (sums over C_in x paths products)."""
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import _uv_native
+    io, i1, i2 = irreps
+    mod = SO3Linear(i1, i2, io, cin, cout, internal_weights=False, feature_mode="uv").to(device)
+    d1, d2, do = Irreps(i1).dim, Irreps(i2).dim, Irreps(io).dim
+    g = torch.Generator().manual_seed(cin + cout + n)
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64)
+    x, y, w, ct = rd(n, d1, cin), rd(n, d2), rd(mod.num_paths, cin, cout) / cin ** 0.5, rd(n, do, cout)
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    assert _uv_native.u1v_supported(xd, yd, wd, mod.tp_info_forward)
+    out = mod(xd, yd, wd)
+    gx, gy, gw = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
+    T = ref_ops.dense_coupling(io, i1, i2, channel_scale=cin ** -0.5).float().double()   # tables hold fp32 coefficients
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x, y, w), ct)
+    for name, a, b in zip(("out", "grad_x", "grad_y", "grad_w"), (out, gx, gy, gw), (ref_out, *ref_grads)):
+        assert_close(a, b, 1e-11, f"u1v fp64 {io} C={cin}->{cout} N={n} {name}", norm="max")
+
+
+def test_uvw_fp64_native(device):
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.nn.functional import _uv_native
+    from equitorch_amd.utils import tp_infos
+    io, i1, i2 = _sh(2), _sh(2), "0e+1o"
+    infos = [t.to(device) for t in tp_infos(Irreps(io), Irreps(i1), Irreps(i2))[:3]]
+    T = ref_ops.dense_coupling(io, i1, i2).float().double()
+    u, v, wc, n = 16, 8, 12, 301
+    g = torch.Generator().manual_seed(4)
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64)
+    x, y, w, ct = rd(n, 9, u), rd(n, 4, v), rd(T.shape[0], u, v, wc) / (u * v) ** 0.5, rd(n, 9, wc)
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    assert _uv_native.uvw_supported(xd, yd, wd, infos[0])
+    out = F.tensor_product_uvw(xd, yd, wd, *infos)
+    gx, gy, gw = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_uvw, T, (x, y, w), ct)
+    for name, a, b in zip(("out", "grad_x", "grad_y", "grad_w"), (out, gx, gy, gw), (ref_out, *ref_grads)):
+        assert_close(a, b, 1e-11, f"uvw fp64 {name}", norm="max")
+
+
 @pytest.mark.parametrize("irreps,cin,cout,n,kw", U1V_CASES)
 def test_u1v_fp32_native(device, irreps, cin, cout, n, kw):
     from equitorch_amd.irreps import Irreps
