@@ -294,8 +294,12 @@ __global__ void __launch_bounds__(256, 1) uv_gw_kernel(const __bf16* __restrict_
   prefetch_begin(n_begin);
 #pragma unroll
   for (int r = 0; r < MR; ++r) prefetch_row(r);
-  const unsigned char* xa = xt + (8 * lq + (ls >> 2)) * pu + (ls & 3) * 8;
-  const unsigned char* gb = gt + (8 * lq + (ls >> 2)) * pw + (ls & 3) * 8;
+  // The 32 samples of a step are contracted in the order the transpose reads like best: k-slots 8q..8q+3 of lane
+  // group q are samples 4q..4q+3, slots 8q+4..8q+7 samples 16+4q..16+4q+3 (the same for both operands, so the sum
+  // is unchanged): the four groups of one read then touch 16 consecutive tile rows, which the row pitch spreads
+  // over all banks (groups 8 rows apart share theirs).
+  const unsigned char* xa = xt + (4 * lq + (ls >> 2)) * pu + (ls & 3) * 8;
+  const unsigned char* gb = gt + (4 * lq + (ls >> 2)) * pw + (ls & 3) * 8;
   for (int64_t nb = n_begin; nb < n_end; nb += kGwStep) {
     __syncthreads();  // the previous step's fragment reads are done
 #pragma unroll
@@ -344,8 +348,8 @@ __global__ void __launch_bounds__(256, 1) uv_gw_kernel(const __bf16* __restrict_
           // tiles past the channel count repeat the last one; their products are never stored.  No branches
           // here: a branch per read would make every read wait for the one before.
           const int ut = min(vu * 4 + i, cin / 16 - 1), wt = min(vw * 4 + i, cout / 16 - 1);
-          fa[i] = lds_read_tr(xr + ut * 32, xr + ut * 32 + 4 * pu);
-          fb[i] = lds_read_tr(gr + wt * 32, gr + wt * 32 + 4 * pw);
+          fa[i] = lds_read_tr(xr + ut * 32, xr + ut * 32 + 16 * pu);
+          fb[i] = lds_read_tr(gr + wt * 32, gr + wt * 32 + 16 * pw);
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i)
