@@ -102,6 +102,75 @@ def _gen_contract(spec: "TriSpec", ops, axes, out_axes: str, out_shared: bool, n
     return out
 
 
+def _matrix_core_route(spec: "TriSpec", ops, axes, out_axes: str, out_shared: bool, n_rows: int,
+                       dtype) -> Optional[Tensor]:
+    """Two of the two-axis contractions have matrix-core kernels (``cgtp_uvt_apply`` / ``cgtp_uvt_grad_w``, any
+    table): a batched vector operand times a shared matrix operand, with or without a channel-less third operand
+    (``indexed_vecmat_scale_gather`` / ``indexed_mat_t_vec_scale_gather`` with a shared ``input2``; reference
+    ``ops/batched_sparse_dense_op.py:1200-1534``), and the outer product of two batched vector operands summed over
+    the rows (``indexed_outer_scale_gather(..., out_accumulated=True)``, ``:436-579``: the gradient of such a shared
+    matrix).  Returns None where they do not apply (other operand shapes, channel counts that are not multiples of
+    4, rows of 16 samples beyond the LDS); the caller then takes the general kernel."""
+    from ..._tables import TpCoo
+    from . import _uv_native as nat
+    if dtype not in (torch.float32, torch.float64) or n_rows <= 0:
+        return None
+    slot = {}
+    for i, ax in enumerate(axes):
+        if ax is None:
+            continue
+        if ax in slot:
+            return None
+        slot[ax] = i
+    nnz = spec.out_idx.shape[0]
+    if nnz == 0:
+        return None
+    coef = np.ones(nnz) if spec.coef is None else spec.coef
+    zeros = np.zeros(nnz, dtype=np.int64)
+
+    def rows_of(ax):           # (batched, contiguous) rows of a vector / channel-less operand
+        t = ops[slot[ax]]
+        return t.contiguous() if t.ndim == 2 + len(ax) else None
+
+    def table(key, build):
+        fast = spec.__dict__.setdefault("_matrix_core_tables", {})
+        if key not in fast:
+            fast[key] = nat.CooTable(build(), torch.empty(0), None)
+        return fast[key]
+
+    if not out_shared and "uw" in slot and len(out_axes) == 1 and set(slot) - {""} == {"uw", "uw".replace(out_axes, "")}:
+        vec_ax = "uw".replace(out_axes, "")
+        mat, x = ops[slot["uw"]], rows_of(vec_ax)
+        y = rows_of("") if "" in slot else torch.ones((n_rows, 1), dtype=dtype, device=mat.device)
+        if mat.ndim != 3 or x is None or y is None or x.data_ptr() % 16:
+            return None
+        n_paths, d1, d2 = mat.shape[0], x.shape[1], y.shape[1]
+        k, cout = (mat.shape[1], mat.shape[2]) if vec_ax == "u" else (mat.shape[2], mat.shape[1])
+        if nat.chunk_of(n_rows, d1, d2, spec.out_size, k, 0, cout, dtype) <= 0:
+            return None
+        tab = table(("apply", vec_ax, "" in slot), lambda: TpCoo(
+            coef, spec.out_idx, spec.idx[slot[vec_ax]], spec.idx[slot[""]] if "" in slot else zeros,
+            spec.idx[slot["uw"]], zeros, d1, d2, spec.out_size, n_paths))
+        sp, su, sw = mat.stride()
+        wp = nat.pack(mat, n_paths, k, cout, sp, *((su, sw) if vec_ax == "u" else (sw, su)))
+        kernels.log_tier("sparse matrix product", "table-driven matrix-core kernel (shared matrix)", str(dtype))
+        return nat.apply(x, y, wp, tab, "out", spec.out_size, cout)
+    if out_shared and out_axes == "uw" and set(slot) - {""} == {"u", "w"}:
+        x, g = rows_of("u"), rows_of("w")
+        y = rows_of("") if "" in slot else torch.ones((n_rows, 1), dtype=dtype, device=ops[slot["u"]].device)
+        if x is None or g is None or y is None or x.shape[2] % 4 or g.shape[2] % 4:
+            return None
+        if (x.data_ptr() | g.data_ptr()) % 16:
+            return None
+        tab = table(("grad_w", "" in slot), lambda: TpCoo(
+            coef, spec.idx[slot["w"]], spec.idx[slot["u"]], spec.idx[slot[""]] if "" in slot else zeros,
+            spec.out_idx, zeros, x.shape[1], y.shape[1], g.shape[1], spec.out_size))
+        kernels.log_tier("sparse matrix product", "table-driven matrix-core kernel (outer product summed over rows)",
+                         str(dtype))
+        return nat.grad_w(x, y, g, tab)
+    return None
+
+
 class TriContract(Function):
     """forward(spec, kinds, out_kind, out_shared, a, b, w) -> out.
 
@@ -155,8 +224,10 @@ class TriContract(Function):
                                        n_rows, ext["u"], dtype, device,
                                        reduce_c=(out_axes == ""), reduce_rows=out_shared)
         else:
-            out = _gen_contract(spec, ops, axes, out_axes, out_shared, n_rows, ext["u"] or 1, ext["w"] or 1, dtype,
-                                device)
+            out = _matrix_core_route(spec, ops, axes, out_axes, out_shared, n_rows, dtype) if any_batched else None
+            if out is None:
+                out = _gen_contract(spec, ops, axes, out_axes, out_shared, n_rows, ext["u"] or 1, ext["w"] or 1,
+                                    dtype, device)
         if not out_shared and not any_batched:
             out = out.squeeze(0)  # every operand shared -> result has no batch axis either
         ctx.spec, ctx.axes, ctx.out_axes = spec, axes, out_axes

@@ -150,6 +150,54 @@ def test_matrix_ops_sweep(device, tables13, op, shared1, shared2, acc):
     assert_close(gy, rgy, 1e-5, f"{op} grad2", norm="max" if shared2 else "element")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("op", ["vecmat", "mat_t_vec"])
+def test_shared_matrix_ops_on_the_matrix_core_kernels(device, monkeypatch, op, dtype):
+    """``sparse_vecmat`` / ``sparse_mat_t_vec`` with a shared matrix operand and channel counts that are multiples of
+    4 run on the table-driven matrix-core kernels, and so do their gradients (vector operand: the same kernel with
+    the matrix transposed; matrix operand: the outer product summed over the rows); the route is asserted, results
+    against the dense contraction in float64.  The table is a random one (11 output rows, 9 vector rows, 6
+    matrices, 60 entries, one output row without entries)."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.ops import kernels
+    from equitorch_amd.structs import SparseProductInfo
+    ax1, ax2, axo, eq = MAT[op]
+    g = torch.Generator().manual_seed(stable_seed(op, str(dtype)))
+    n, n_out, ext = 203, 11, {"u": 24, "w": 16}
+    size = {"vecmat": (9, 6), "mat_t_vec": (6, 9)}[op]
+    nnz = 60
+    out_idx = torch.sort(torch.randint(0, n_out - 1, (nnz,), generator=g)).values     # row 10 stays empty
+    seg = torch.searchsorted(out_idx, torch.arange(n_out + 1))
+    i1, i2 = (torch.randint(0, sz, (nnz,), generator=g) for sz in size)
+    scale = torch.randn(nnz, generator=g)
+    info = SparseProductInfo(scale, i1, i2, seg, None, None, n_out).to(device)
+    T = torch.zeros(n_out, *size, dtype=torch.float64)
+    T.index_put_((out_idx, i1, i2), scale.double(), accumulate=True)
+    shared = {"vecmat": (False, True), "mat_t_vec": (True, False)}[op]
+
+    def mk(axes, sh, d):
+        return torch.randn(*((() if sh else (n,)) + (d,) + tuple(ext[a] for a in axes)), generator=g,
+                           dtype=torch.float64)
+    x, y = mk(ax1, shared[0], size[0]), mk(ax2, shared[1], size[1])
+    seen = []
+    monkeypatch.setattr(kernels, "log_tier", lambda op_, tier, detail="": seen.append(tier))
+    xd, yd = (t.to(dtype).to(device).requires_grad_(True) for t in (x, y))
+    out = getattr(F, f"sparse_{op}")(xd, yd, info)
+    xr, yr = (t.to(dtype).double().requires_grad_(True) for t in (x, y))
+    ref_out = torch.einsum(eq.format(a="" if shared[0] else "n", b="" if shared[1] else "n", o="n"), T, xr, yr)
+    tol = 1e-5 if dtype == torch.float32 else 1e-11
+    # sums over 16 or 24 channels and several entries per element: norm-wise in fp32
+    assert_close(out, ref_out, tol, f"{op} forward", norm="max")
+    assert out[:, n_out - 1].abs().max().item() == 0.0
+    ct = torch.randn(ref_out.shape, generator=g, dtype=torch.float64)
+    gx, gy = torch.autograd.grad(out, (xd, yd), ct.to(dtype).to(device))
+    rgx, rgy = torch.autograd.grad(ref_out, (xr, yr), ct.to(dtype).double())
+    assert_close(gx, rgx, tol, f"{op} grad1", norm="max")
+    assert_close(gy, rgy, tol, f"{op} grad2", norm="max")
+    assert sum("shared matrix" in t for t in seen) == 2, seen          # forward and the vector operand's gradient
+    assert sum("summed over rows" in t for t in seen) == 1, seen       # the matrix operand's gradient
+
+
 @pytest.mark.parametrize("scaled,indexed,segmented", [(True, True, True), (False, True, True), (True, False, True),
                                                       (True, True, False), (False, False, False)])
 def test_indexed_scale_segment(device, scaled, indexed, segmented):
