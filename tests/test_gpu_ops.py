@@ -198,6 +198,45 @@ def test_shared_matrix_ops_on_the_matrix_core_kernels(device, monkeypatch, op, d
     assert sum("summed over rows" in t for t in seen) == 1, seen       # the matrix operand's gradient
 
 
+@pytest.mark.parametrize("case", range(16))
+def test_matrix_core_route_random_shapes(device, case):
+    """The same route on seeded random tables and extents: batches below and across the 16-sample blocks (1 .. 700
+    rows), channel counts from 4 that are no multiples of 16, weight paths and output rows without entries, repeated
+    (row, row, path) entries, fp32 and fp64; forward and both gradients against the dense contraction in float64."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.structs import SparseProductInfo
+    g = torch.Generator().manual_seed(stable_seed("matrix core route", case))
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    dtype = torch.float64 if case % 4 == 3 else torch.float32
+    n = [1, 15, 16, 17, 33, 100, 257, 700][case % 8]
+    n_out, d_vec, n_mat = ri(1, 12), ri(1, 10), ri(1, 7)
+    cu, cw = 4 * ri(1, 10), 4 * ri(1, 10)
+    nnz = ri(1, 50)
+    out_idx = torch.sort(torch.randint(0, n_out, (nnz,), generator=g)).values
+    seg = torch.searchsorted(out_idx, torch.arange(n_out + 1))
+    i1 = torch.randint(0, d_vec, (nnz,), generator=g)
+    i2 = torch.randint(0, n_mat, (nnz,), generator=g)
+    scale = torch.randn(nnz, generator=g)
+    info = SparseProductInfo(scale, i1, i2, seg, None, None, n_out).to(device)
+    T = torch.zeros(n_out, d_vec, n_mat, dtype=torch.float64)
+    T.index_put_((out_idx, i1, i2), scale.double(), accumulate=True)
+    x = torch.randn(n, d_vec, cu, generator=g, dtype=torch.float64).to(dtype)
+    m = torch.randn(n_mat, cu, cw, generator=g, dtype=torch.float64).to(dtype)
+    xd, md = (t.to(device).requires_grad_(True) for t in (x, m))
+    out = F.sparse_vecmat(xd, md, info)
+    xr, mr = (t.double().requires_grad_(True) for t in (x, m))
+    ref_out = torch.einsum("mab,nau,buw->nmw", T, xr, mr)
+    tol = 1e-5 if dtype == torch.float32 else 1e-11
+    what = f"case {case}: n={n} out={n_out} rows={d_vec} paths={n_mat} {cu}->{cw} nnz={nnz} {dtype}"
+    # sums over up to 40 channels and several entries per element, and over the batch for the matrix: norm-wise
+    assert_close(out, ref_out, tol, what + " forward", norm="max")
+    ct = torch.randn(ref_out.shape, generator=g, dtype=torch.float64).to(dtype)
+    gx, gm = torch.autograd.grad(out, (xd, md), ct.to(device))
+    rgx, rgm = torch.autograd.grad(ref_out, (xr, mr), ct.double())
+    assert_close(gx, rgx, tol, what + " grad vector", norm="max")
+    assert_close(gm, rgm, tol, what + " grad matrix", norm="max")
+
+
 @pytest.mark.parametrize("scaled,indexed,segmented", [(True, True, True), (False, True, True), (True, False, True),
                                                       (True, True, False), (False, False, False)])
 def test_indexed_scale_segment(device, scaled, indexed, segmented):
