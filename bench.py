@@ -63,6 +63,8 @@ WORKLOADS = {
     # streaming kernels of known traffic (1 GiB): counter calibration and achievable-bandwidth reference
     "copy": None,
     "read": None,
+    # rate of LDS reads by instruction, tile layout and wavefronts per compute unit
+    "lds": None,
     # indexed scale-segment reduction alone: the messages of BASELINE configs[1] summed to their destination nodes
     "scatter": None,
     # spherical harmonics of 2^20 vectors up to degree 6 (forward and gradient kernels), normalisation fused
@@ -318,6 +320,45 @@ def scatter_bench(steps, warmup):
                       "roofline": {"bound": "hbm", "kernel": "cgtp::segment_sum_kernel<float,4>", "achieved": round(gbs, 1),
                                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                                    "traffic": None, "algorithmic_bytes": nbytes, "avg_ms": round(ms, 5)}}))
+
+
+def lds_read_rates(steps, warmup):
+    """Rate of LDS reads per compute unit by instruction, tile layout and wavefronts per CU (4, 8, 16): the numbers
+    behind the layout of the bf16 weight-gradient kernel's transpose reads.  One JSON line."""
+    import ctypes
+    from equitorch_amd import _lib
+    blib = ctypes.CDLL(os.path.join(ROOT, "equitorch_amd", "lib", "libcgtp_bench.so"))
+    blib.cgtpbench_lds_read.argtypes = [ctypes.c_int] * 6 + [ctypes.c_void_p, ctypes.c_void_p]
+    dev = torch.device("cuda:0")
+    n_cu = torch.cuda.get_device_properties(dev).multi_processor_count
+    out = torch.empty(4 * n_cu * 256, dtype=torch.int32, device=dev)
+    stream = _lib.stream_ptr(dev)
+    iters = 4000
+    cases = [("ds_read_b128 contiguous", 2, 2, 256), ("ds_read_b64 contiguous", 1, 2, 256),
+             ("ds_read_b64_tr_b16 rows 8q..8q+3 pitch 288", 0, 0, 288), ("ds_read_b64_tr_b16 rows 4q..4q+3 pitch 288", 0, 1, 288),
+             ("ds_read_b64_tr_b16 rows 4q..4q+3 pitch 272", 0, 1, 272), ("ds_read_b64_tr_b16 rows 4q..4q+3 pitch 256", 0, 1, 256)]
+    rows = {}
+    for name, kind, row_mode, pitch in cases:
+        rates = {}
+        for per_cu, lds in ((1, 100000), (2, 70000), (4, 36000)):
+            def launch():
+                _lib.check(blib.cgtpbench_lds_read(kind, row_mode, pitch, per_cu * n_cu, lds, iters, out.data_ptr(), stream))
+            for _ in range(max(warmup, 1)):
+                launch()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(steps):
+                launch()
+            b.record()
+            torch.cuda.synchronize()
+            ms = a.elapsed_time(b) / steps
+            bytes_per_cu = iters * 8 * 64 * (16 if kind == 2 else 8) * 4 * per_cu
+            rates[f"{4 * per_cu}_waves_per_cu_bytes_per_ns"] = round(bytes_per_cu / (ms * 1e6), 1)
+        rows[name] = rates
+    print(json.dumps({"metric": "lds_read_rate", "value": rows["ds_read_b128 contiguous"]["16_waves_per_cu_bytes_per_ns"],
+                      "unit": "B/ns per CU", "n_gpus": 1, "steps": steps, "warmup": warmup,
+                      "config": {"workload": "eight reads per wavefront, then s_waitcnt; four wavefronts per workgroup"},
+                      "rates": rows}))
 
 
 def membench(kind, steps, warmup):
@@ -725,6 +766,9 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
+    if args.workload == "lds":
+        lds_read_rates(args.steps, args.warmup)
+        return
     if args.workload in ("copy", "read"):
         membench(args.workload, args.steps, args.warmup)
         return
