@@ -390,34 +390,41 @@ struct UvtGwDev {
 
 constexpr int kGwT = 4;        // accumulator tiles per wavefront and axis
 constexpr int kGwStep = 8;     // samples per step (two matrix instructions deep)
-constexpr int kGwPitch = 132;  // floats per sample row of the LDS stage: 128 channels, rows 4 banks apart
 
 // Tile rows and columns are interleaved with the channels — row r of k-tile i is channel 4 r + i of the wavefront's
 // 64, column r of w-tile j is output channel 4 r + j — so that a lane's operands of the four tiles are four
 // consecutive channels: one 16-byte LDS read per operand and step.
-template <bool YC>
-__global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : 3) uvt_grad_w_kernel(const UvtGwDev a) {
-  __shared__ __attribute__((aligned(16))) real lds_a[2][kGwStep][kGwPitch];
-  __shared__ __attribute__((aligned(16))) real lds_b[2][kGwStep][kGwPitch];
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), r = lane & 15, g4 = lane >> 4;
+// NARROW (few output channels): the block is 256 (k) x 64 (w), the four wavefronts split k four ways and share the
+// w columns, a thread loads and mixes two samples of its four k channels per step; with 128 columns for 32 or 64
+// output channels most of the matrix instructions would multiply zeros.
+template <bool YC, bool NARROW>
+__global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : NARROW ? 2 : 3) uvt_grad_w_kernel(const UvtGwDev a) {
+  constexpr int KT = NARROW ? 256 : 128, WT = NARROW ? 64 : 128, NA = NARROW ? 2 : 1;
+  __shared__ __attribute__((aligned(16))) real lds_a[2][kGwStep][KT + 4];   // rows 4 banks apart
+  __shared__ __attribute__((aligned(16))) real lds_b[2][kGwStep][WT + 4];
+  const int tid = threadIdx.x;
+  const int wave = tid / kWave, lane = tid & (kWave - 1), r = lane & 15, g4 = lane >> 4;
   const int p = blockIdx.y;
-  const int kgroups = (a.K + 127) / 128;
+  const int kgroups = (a.K + KT - 1) / KT;
   const int kgrp = blockIdx.z % kgroups, wgrp = blockIdx.z / kgroups;
   const int64_t n_begin = (int64_t)blockIdx.x * a.chunk;
   const int64_t n_end = n_begin + a.chunk < a.n_rows ? n_begin + a.chunk : a.n_rows;
 
-  // loading role: sample ls of the step, channels lq .. lq + 3 of the block's 128 (both operands)
-  const int ls = 2 * wave + (lane >> 5), lq = 4 * (lane & 31);
+  // loading role: channels lq .. lq + 3 of the block's k range for sample ls (and ls + 4 if NARROW), channels
+  // lqb .. lqb + 3 of its w range for sample lsb (NARROW: the first 128 threads only)
+  const int ls = NARROW ? tid >> 6 : 2 * wave + (lane >> 5), lq = NARROW ? 4 * (tid & 63) : 4 * (lane & 31);
+  const int lsb = NARROW ? (tid >> 4) & 7 : ls, lqb = NARROW ? 4 * (tid & 15) : lq;
+  const bool b_thread = !NARROW || tid < 128;
   // K and cout are multiples of 4 (checked by the launcher), so a lane's four channels are all inside or all outside
-  const bool kok = kgrp * 128 + lq < a.K, wok = wgrp * 128 + lq < a.cout;
-  const int kc = kok ? kgrp * 128 + lq : 0, wc = wok ? wgrp * 128 + lq : 0;
+  const bool kok = kgrp * KT + lq < a.K, wok = b_thread && wgrp * WT + lqb < a.cout;
+  const int kc = kok ? kgrp * KT + lq : 0, wc = wok ? wgrp * WT + lqb : 0;
   int xo = kc, yo = 0;
   if constexpr (YC) {
     xo = kc / a.cy;
     yo = kc - xo * a.cy;
   }
   // multiplying role: channels kh * 64 .. + 63 by output channels wh * 64 .. + 63
-  const int kh = wave & 1, wh = wave >> 1;
+  const int kh = NARROW ? wave : wave & 1, wh = NARROW ? 0 : wave >> 1;
 
   realx4 acc[kGwT][kGwT];
 #pragma unroll
@@ -434,10 +441,10 @@ __global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : 3) uvt_grad_w_ker
   int ld_item = s_begin - 1, ld_step = steps;
   int xrow[kUvtTerms], yrow[kUvtTerms], grow = 0;
   real c[kUvtTerms];
-  realx4 v4[kUvtTerms];     // y without channels: four channels of x; with: four channels of y
-  real v1[kUvtTerms];       // y without channels: y[n, b]; with: x[n, a, u]
+  realx4 v4[NA][kUvtTerms];     // y without channels: four channels of x; with: four channels of y
+  real v1[NA][kUvtTerms];       // y without channels: y[n, b]; with: x[n, a, u]
   realx4 bv4;
-  bool ld_live = false;
+  bool ld_live[NA] = {}, ldb_live = false;
 
   auto issue = [&]() __attribute__((always_inline)) {
     if (ld_step == steps) {
@@ -454,32 +461,43 @@ __global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : 3) uvt_grad_w_ker
       }
       grow = it.out_row * a.cout;
     }
-    const int64_t n = n_begin + (int64_t)ld_step * kGwStep + ls;
-    ld_live = n < n_end;
-    const int64_t nc = ld_live ? n : n_end - 1;
-    const real* xn = a.x + nc * a.dx * a.cx + xo;
-    const real* yn = a.y + nc * a.dy * (YC ? a.cy : 1) + yo;
-    bv4 = *reinterpret_cast<const realx4*>(a.g + nc * a.dg * a.cout + grow + wc);
+    const int64_t n0 = n_begin + (int64_t)ld_step * kGwStep;
+    {
+      const int64_t n = n0 + lsb;
+      ldb_live = n < n_end;
+      bv4 = *reinterpret_cast<const realx4*>(a.g + (ldb_live ? n : n_end - 1) * a.dg * a.cout + grow + wc);
+    }
 #pragma unroll
-    for (int k = 0; k < kUvtTerms; ++k) {
-      if constexpr (YC) {
-        v1[k] = xn[xrow[k]];
-        v4[k] = *reinterpret_cast<const realx4*>(yn + yrow[k]);
-      } else {
-        v4[k] = *reinterpret_cast<const realx4*>(xn + xrow[k]);
-        v1[k] = yn[yrow[k]];
+    for (int j = 0; j < NA; ++j) {
+      const int64_t n = n0 + ls + 4 * j;
+      ld_live[j] = n < n_end;
+      const int64_t nc = ld_live[j] ? n : n_end - 1;
+      const real* xn = a.x + nc * a.dx * a.cx + xo;
+      const real* yn = a.y + nc * a.dy * (YC ? a.cy : 1) + yo;
+#pragma unroll
+      for (int k = 0; k < kUvtTerms; ++k) {
+        if constexpr (YC) {
+          v1[j][k] = xn[xrow[k]];
+          v4[j][k] = *reinterpret_cast<const realx4*>(yn + yrow[k]);
+        } else {
+          v4[j][k] = *reinterpret_cast<const realx4*>(xn + xrow[k]);
+          v1[j][k] = yn[yrow[k]];
+        }
       }
     }
     ++ld_step;
   };
   // mixes the terms of the loads in flight and puts both operands into stage buf
   auto commit = [&](int buf) __attribute__((always_inline)) {
-    realx4 av = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int k = 0; k < kUvtTerms; ++k) av += (c[k] * v1[k]) * v4[k];
     const realx4 zero = {0.f, 0.f, 0.f, 0.f};
-    *reinterpret_cast<realx4*>(&lds_a[buf][ls][lq]) = (ld_live && kok) ? av : zero;
-    *reinterpret_cast<realx4*>(&lds_b[buf][ls][lq]) = (ld_live && wok) ? bv4 : zero;
+#pragma unroll
+    for (int j = 0; j < NA; ++j) {
+      realx4 av = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int k = 0; k < kUvtTerms; ++k) av += (c[k] * v1[j][k]) * v4[j][k];
+      *reinterpret_cast<realx4*>(&lds_a[buf][ls + 4 * j][lq]) = (ld_live[j] && kok) ? av : zero;
+    }
+    if (b_thread) *reinterpret_cast<realx4*>(&lds_b[buf][lsb][lqb]) = (ldb_live && wok) ? bv4 : zero;
   };
 
   if (total > 0) {
@@ -510,8 +528,8 @@ __global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : 3) uvt_grad_w_ker
   // accumulator layout: lane (column r, g4) holds rows 4 g4 .. + 3 of a tile; tile (i, j) row q is channel
   // 4 q + i of the wavefront's 64, column r is output channel 4 r + j
   real* out = a.part + ((int64_t)blockIdx.x * a.n_paths + p) * a.K * a.cout;
-  const int kbase = kgrp * 128 + kh * 64;
-  const int w0 = wgrp * 128 + wh * 64 + 4 * r;
+  const int kbase = kgrp * KT + kh * 64;
+  const int w0 = wgrp * WT + wh * 64 + 4 * r;
   if (w0 < a.cout) {
 #pragma unroll
     for (int i = 0; i < kGwT; ++i)
@@ -897,13 +915,18 @@ int grad_w(const cgtp_uvt_gw_args* a, void* stream) {
   d.cout = a->cout; d.K = (int)K;
   d.chunk = (int)uvt_gw_chunk(a->n_rows);
   const int64_t n_chunks = (a->n_rows + d.chunk - 1) / d.chunk;
-  const int64_t zblocks = ((K + 127) / 128) * ((a->cout + 127) / 128);
+  // few output channels and a long contracted axis: 256 x 64 blocks (single precision; in double precision the
+  // second set of operands in flight does not fit the registers)
+  const bool narrow = sizeof(real) == 4 && a->cout <= 64 && K >= 256;
+  const int64_t kt = narrow ? 256 : 128, wt = narrow ? 64 : 128;
+  const int64_t zblocks = ((K + kt - 1) / kt) * ((a->cout + wt - 1) / wt);
   if (zblocks > 65535 || a->n_paths > 65535) return CGTP_ERR_SHAPE;
   dim3 grid((unsigned)n_chunks, (unsigned)a->n_paths, (unsigned)zblocks);
-  if (a->cy > 0)
-    hipLaunchKernelGGL(uvt_grad_w_kernel<true>, grid, dim3(256), 0, st, d);
-  else
-    hipLaunchKernelGGL(uvt_grad_w_kernel<false>, grid, dim3(256), 0, st, d);
+  void (*fn)(const UvtGwDev) = a->cy > 0 ? uvt_grad_w_kernel<true, false> : uvt_grad_w_kernel<false, false>;
+#ifndef CGTP_UVT_F64
+  if (narrow) fn = a->cy > 0 ? uvt_grad_w_kernel<true, true> : uvt_grad_w_kernel<false, true>;
+#endif
+  hipLaunchKernelGGL(fn, grid, dim3(256), 0, st, d);
   if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
   hipLaunchKernelGGL(uvt_gw_reduce_kernel, dim3((unsigned)((n_out + 255) / 256)), dim3(256), 0, st,
                      (const real*)a->workspace, (real*)a->gw, n_chunks, n_out);
