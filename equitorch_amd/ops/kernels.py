@@ -531,6 +531,9 @@ def _uvu_args(cfg: int, x: Tensor, y: Tensor, w: Tensor, seg: Optional[SegIndex]
     return a
 
 
+_GW_WORKSPACE_BYTES = 512 << 20      # largest per-row weight-gradient workspace of one row-mode backward launch
+
+
 def _workspace(a: UvuArgs, backward: int, device):
     nbytes = int(_lib.lib.cgtp_uvu_workspace_bytes(C.byref(a), backward))
     if nbytes == 0:
@@ -589,10 +592,37 @@ def uvu_backward(cfg: int, dims, x: Tensor, y: Tensor, w: Tensor, g: Tensor, nee
     """Compiled-table backward -> (grad_x, grad_y, grad_w), None where ``need`` is False.  Row mode: ``gather``
     picks the row of ``g`` and ``x_gather`` the row of ``x`` of every batch row; with ``x_gather`` the returned
     grad_x is per batch row, ``(n_rows, D1, C)``."""
+    w_given = w
     w = expand_paths(w, cfg, -2)
     a = _uvu_args(cfg, x, y, w, seg, gather, pos_per_wave, y_vec, backward=True)
     a.grad_out = g.data_ptr()
     a.x_gather = _lib.ptr(x_gather)
+    n = y.shape[0]
+    if seg is None and need[2] and w.ndim == 2 and n > 1:
+        # Row mode with a shared weight: some kernels write one weight gradient per row into the workspace and sum
+        # afterwards ((rows + chunks) * paths * channels elements).  Past _GW_WORKSPACE_BYTES the rows are taken in
+        # equal parts, each with a workspace of its own size, and the parts' gradients are added in order.
+        a.grad_w = w.data_ptr()       # any non-null pointer: the query only asks whether the gradient is wanted
+        nbytes = int(_lib.lib.cgtp_uvu_workspace_bytes(C.byref(a), 1))
+        if nbytes > _GW_WORKSPACE_BYTES:
+            parts = min(n, -(-nbytes // _GW_WORKSPACE_BYTES))
+            step = -(-n // parts)
+            gx = (torch.empty((n,) + x.shape[1:], dtype=x.dtype, device=x.device) if x_gather is not None
+                  else torch.empty_like(x)) if need[0] else None
+            gy = torch.empty_like(y) if need[1] else None
+            gw = None
+            rows = lambda t, i0, i1: None if t is None else t[i0:i1]
+            for i0 in range(0, n, step):
+                i1 = min(i0 + step, n)
+                px, py, pw = uvu_backward(cfg, dims, x if x_gather is not None else x[i0:i1], y[i0:i1], w_given,
+                                          g if gather is not None else g[i0:i1], need, None, rows(gather, i0, i1),
+                                          pos_per_wave, rows(x_gather, i0, i1), y_vec)
+                if gx is not None:
+                    gx[i0:i1] = px
+                if gy is not None:
+                    gy[i0:i1] = py
+                gw = pw if gw is None else gw + pw
+            return gx, gy, gw
     if not need[0]:
         gx = None
     elif x_gather is not None:

@@ -182,6 +182,32 @@ def test_u1u_block_wise_shared_weight(device, lmax, n, ch):
         assert_close(g, r, 1e-5, f"lmax={lmax} shared {name}")
 
 
+@pytest.mark.parametrize("lmax,n,ch", [(4, 700, 32), (2, 5000, 64)])
+def test_shared_weight_backward_in_row_parts(device, monkeypatch, lmax, n, ch):
+    """The same gradients when the rows are taken in parts because the per-row weight-gradient workspace would pass
+    its limit (set to 1 MB here: several parts with an uneven tail), against the dense oracle and against the single
+    launch."""
+    from equitorch_amd.ops import kernels
+    irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+    d = (lmax + 1) ** 2
+    mod = _module(irreps, irreps, irreps).to(device)
+    x, sh, w = tp_inputs(n, d, lmax, mod.num_paths, ch, True, seed=166 + lmax)
+    ct = torch.randn(n, d, ch, generator=torch.Generator().manual_seed(8))
+    whole = _run(mod, x, sh, w, ct, device)
+    calls = []
+    real = kernels._lib.lib.cgtp_uvu_bwd
+    monkeypatch.setattr(kernels, "_GW_WORKSPACE_BYTES", 1 << 20)
+    monkeypatch.setattr(kernels._lib.lib, "cgtp_uvu_bwd", lambda a, s: (calls.append(1), real(a, s))[1])
+    parts = _run(mod, x, sh, w, ct, device)
+    assert len(calls) > 1, "the backward was not split"
+    T = ref_ops.dense_coupling(irreps, irreps, irreps)
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1u, T, (x, sh, w), ct)
+    for name, g, h, r in zip(("out", "grad_x", "grad_sh", "grad_w"), parts, whole, (ref_out, *ref_grads)):
+        assert_close(g, r, 1e-5, f"lmax={lmax} rows in parts {name}", norm="max" if name == "grad_w" else "element")
+        if name != "grad_w":            # per-row results do not depend on the split
+            assert torch.equal(g, h), name
+
+
 def test_edge_large_table(device):
     """Edge message passing at lmax = 6, C = 32 (BASELINE configs[4] shapes, small graph): gathered row-mode
     kernels plus segment sums against the dense oracle."""
