@@ -65,6 +65,8 @@ WORKLOADS = {
     "read": None,
     # rate of LDS reads by instruction, tile layout and wavefronts per compute unit
     "lds": None,
+    # vector FMAs next to matrix instructions on one SIMD: same wavefront, two wavefronts, split roles
+    "coissue": None,
     # indexed scale-segment reduction alone: the messages of BASELINE configs[1] summed to their destination nodes
     "scatter": None,
     # spherical harmonics of 2^20 vectors up to degree 6 (forward and gradient kernels), normalisation fused
@@ -320,6 +322,50 @@ def scatter_bench(steps, warmup):
                       "roofline": {"bound": "hbm", "kernel": "cgtp::segment_sum_kernel<float,4>", "achieved": round(gbs, 1),
                                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                                    "traffic": None, "algorithmic_bytes": nbytes, "avg_ms": round(ms, 5)}}))
+
+
+def coissue_rates(steps, warmup):
+    """Time of 8 matrix instructions + the FMAs that fit their run time (32 with the bf16 instruction, 64 with the fp32
+    one) per SIMD, issued by one wavefront, by two, or split between two wavefronts: how much vector work hides behind
+    matrix work on this chip.  One JSON line, ns per such unit of work."""
+    import ctypes
+    from equitorch_amd import _lib
+    blib = ctypes.CDLL(os.path.join(ROOT, "equitorch_amd", "lib", "libcgtp_bench.so"))
+    blib.cgtpbench_coissue.argtypes = [ctypes.c_int] * 5 + [ctypes.c_void_p, ctypes.c_void_p]
+    dev = torch.device("cuda:0")
+    n_cu = torch.cuda.get_device_properties(dev).multi_processor_count
+    out = torch.empty(n_cu * 512, dtype=torch.float32, device=dev)
+    stream = _lib.stream_ptr(dev)
+    iters = 20000
+    names = {0: "matrix only", 1: "fma only", 2: "one by one (1 matrix : R fma)", 3: "in blocks (8 matrix, 8 R fma)",
+             4: "split: one wavefront matrix, one fma"}
+    table = {}
+    for f32 in (0, 1):
+        rows = {}
+        for threads in (256, 512):
+            for mode in range(5):
+                if mode == 4 and threads != 512:
+                    continue
+                def launch():
+                    _lib.check(blib.cgtpbench_coissue(mode, f32, threads, n_cu, iters, out.data_ptr(), stream))
+                for _ in range(max(warmup, 1)):
+                    launch()
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                for _ in range(steps):
+                    launch()
+                b.record()
+                torch.cuda.synchronize()
+                ns = a.elapsed_time(b) / steps * 1e6 / iters
+                # work per iteration and SIMD: every wavefront that issues a kind issues 8 matrix / 8 R fma
+                waves = threads // 256
+                units = 1 if mode == 4 else waves
+                rows[f"{waves} wavefront(s) per SIMD, {names[mode]}"] = round(ns / units, 1)
+        table["v_mfma_f32_16x16x4_f32 + 64 fma" if f32 else "v_mfma_f32_16x16x32_bf16 + 32 fma"] = rows
+    print(json.dumps({"metric": "coissue_ns_per_unit", "value": None, "unit": "ns per (8 matrix instructions + their FMAs) per SIMD",
+                      "n_gpus": 1, "steps": steps, "warmup": warmup,
+                      "config": {"workload": "register-only loops; 'matrix only' / 'fma only' rows count their own kind only"},
+                      "rates": table}))
 
 
 def lds_read_rates(steps, warmup):
@@ -768,6 +814,9 @@ def main():
 
     if args.workload == "lds":
         lds_read_rates(args.steps, args.warmup)
+        return
+    if args.workload == "coissue":
+        coissue_rates(args.steps, args.warmup)
         return
     if args.workload in ("copy", "read"):
         membench(args.workload, args.steps, args.warmup)

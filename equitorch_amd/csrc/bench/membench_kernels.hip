@@ -4,6 +4,8 @@
 // multiple of 16 and the pointers 16-byte aligned; status codes as in cgtp.h.
 // lds_read: the rate at which wavefronts read LDS with ds_read_b128, ds_read_b64 or ds_read_b64_tr_b16 (the transpose
 // read the bf16 weight-gradient kernel forms its matrix operands with), in the tile layouts that kernel can use.
+// coissue: how much vector-ALU work (independent fp32 FMAs) hides behind matrix instructions on one SIMD, issued by
+// the same wavefront (interleaved or in blocks) or by another wavefront of the SIMD.
 #include "cgtp_device.h"
 #include "cgtp_host.h"
 
@@ -59,6 +61,67 @@ __global__ void __launch_bounds__(256) lds_read_kernel(int* __restrict__ out, in
   out[blockIdx.x * 256 + threadIdx.x] = acc[0] + acc[1] + acc[2] + acc[3];
 }
 
+// MODE 0: matrix instructions only; 1: FMAs only; 2: one matrix instruction then R FMAs, eight times per iteration;
+// 3: eight matrix instructions then 8 R FMAs; 4: wavefronts 0-3 of the workgroup matrix instructions only,
+// wavefronts 4-7 FMAs only (512 threads: one of each per SIMD).  F32: v_mfma_f32_16x16x4_f32, else
+// v_mfma_f32_16x16x32_bf16.  All operands in registers; 32 independent FMA chains.
+template <int MODE, int R, bool F32>
+__global__ void __launch_bounds__(512) coissue_kernel(float* __restrict__ out, int iters) {
+  typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+  typedef float floatx4 __attribute__((ext_vector_type(4)));
+  const int wave = threadIdx.x >> 6;
+  floatx4 acc[8];
+  float v[32];
+  for (int i = 0; i < 8; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < 32; ++i) v[i] = threadIdx.x * 0.001f + i;
+  bf16x8 a, b;
+  for (int e = 0; e < 8; ++e) { a[e] = (__bf16)(float)(threadIdx.x & 7); b[e] = (__bf16)1.0f; }
+  const float fa = (float)(threadIdx.x & 7), fb = 1.0f, m = 1.0001f, c = 0.5f;
+  const bool do_m = MODE == 0 || MODE == 3 || (MODE == 4 && (wave & 4) == 0);
+  const bool do_v = MODE == 1 || MODE == 3 || (MODE == 4 && (wave & 4) != 0);
+  for (int it = 0; it < iters; ++it) {
+    if (MODE == 2) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (F32) acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa, fb, acc[i], 0, 0, 0);
+        else acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < R; ++j) v[(i * R + j) & 31] = __builtin_fmaf(v[(i * R + j) & 31], m, c);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+      if (do_m) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          if (F32) acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa, fb, acc[i], 0, 0, 0);
+          else acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (do_v) {
+#pragma unroll
+        for (int j = 0; j < 8 * R; ++j) v[j & 31] = __builtin_fmaf(v[j & 31], m, c);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+  float s = 0.f;
+  for (int i = 0; i < 8; ++i) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+  for (int i = 0; i < 32; ++i) s += v[i];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+template <bool F32, int R>
+static void (*coissue_fn(int mode))(float*, int) {
+  switch (mode) {
+    case 0: return coissue_kernel<0, R, F32>;
+    case 1: return coissue_kernel<1, R, F32>;
+    case 2: return coissue_kernel<2, R, F32>;
+    case 3: return coissue_kernel<3, R, F32>;
+    default: return coissue_kernel<4, R, F32>;
+  }
+}
+
 }  // namespace cgtp
 
 using namespace cgtp;
@@ -98,6 +161,18 @@ int cgtpbench_lds_read(int kind, int row_mode, int pitch, int workgroups, int ld
     return CGTP_ERR_LDS;
   hipLaunchKernelGGL(fn, dim3((unsigned)workgroups), dim3(256), (size_t)lds_bytes, (hipStream_t)stream, (int*)out, iters,
                      pitch, row_mode);
+  return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
+}
+
+// One launch of one workgroup per compute unit (`workgroups`), 256 or 512 threads (one or two wavefronts per SIMD),
+// `iters` iterations of 8 matrix instructions and / or 8 * fma_per_mfma FMAs per wavefront (fma_per_mfma 4 with the
+// bf16 instruction, 8 with the fp32 one: the instruction's run time in issue slots); out: workgroups * threads floats.
+int cgtpbench_coissue(int mode, int f32, int threads, int workgroups, int iters, void* out, void* stream) {
+  if (!out) return CGTP_ERR_NULL;
+  if (mode < 0 || mode > 4 || (threads != 256 && threads != 512) || workgroups <= 0 || iters <= 0) return CGTP_ERR_SHAPE;
+  if (mode == 4 && threads != 512) return CGTP_ERR_SHAPE;
+  void (*fn)(float*, int) = f32 ? coissue_fn<true, 8>(mode) : coissue_fn<false, 4>(mode);
+  hipLaunchKernelGGL(fn, dim3((unsigned)workgroups), dim3((unsigned)threads), 0, (hipStream_t)stream, (float*)out, iters);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 
