@@ -793,8 +793,8 @@ def layer_bench(steps, warmup):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="edge_fwd_bwd", choices=sorted(WORKLOADS))
     ap.add_argument("--rotate", type=int, default=4, help="number of weight buffers cycled through")
     ap.add_argument("--graph", default="uniform", choices=["uniform", "local"],
@@ -805,7 +805,7 @@ def main():
     ap.add_argument("--cpu-sample-edges", type=int, default=16384)
     ap.add_argument("--pos-per-wave", type=int, default=0,
                     help="sorted positions per wavefront in the per-kernel timing (0 = library default)")
-    ap.add_argument("--kernel-reps", type=int, default=30, help="launches per kernel for the roofline timing")
+    ap.add_argument("--kernel-reps", type=int, default=100, help="launches per kernel for the roofline timing")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on exactly one GPU (the path has no multi-GPU part); use --gpus 1",
@@ -892,6 +892,7 @@ def main():
     t0 = time.perf_counter()
     for i in range(args.steps):
         step(i)
+    host_elapsed = time.perf_counter() - t0        # the host has issued every launch; the GPU may still be running
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
@@ -903,17 +904,25 @@ def main():
     xd, shd = x.detach(), sh.detach()
 
     def time_kernel(fn):
+        """(average, median) launch duration in ms.  Average: one pair of events around all launches, issued back
+        to back as in the step loop (a pair per launch adds the events' own ~1 us to every launch); median: of
+        launches bracketed one by one."""
+        wd = [w.detach() for w in ws]
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for i in range(args.kernel_reps):
+            fn(wd[i % args.rotate])
+        b.record()
         evs = []
         for i in range(args.kernel_reps):
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            w = ws[i % args.rotate].detach()
-            a.record()
-            fn(w)
-            b.record()
-            evs.append((a, b))
+            c, d_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            c.record()
+            fn(wd[i % args.rotate])
+            d_.record()
+            evs.append((c, d_))
         torch.cuda.synchronize()
-        ts = sorted(a.elapsed_time(b) for a, b in evs)
-        return sum(ts) / len(ts), ts[len(ts) // 2]
+        ts = sorted(c.elapsed_time(d_) for c, d_ in evs)
+        return a.elapsed_time(b) / args.kernel_reps, ts[len(ts) // 2]
 
     ppw = args.pos_per_wave
     fwd_fn = lambda w: kernels.uvu_forward(cfg, dims, xd, shd, w, seg=plan.fwd_index, pos_per_wave=ppw)
@@ -933,7 +942,8 @@ def main():
     rec = {
         "metric": "edge-TP fwd+bwd Medges/s (lmax=2,C=64)" if backward else "edge-TP fwd Medges/s (lmax=2,C=64)",
         "value": round(medges, 2), "unit": "Medges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_per_step, 4), "host_issue_ms_per_step": round(host_elapsed / args.steps * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"{args.workload}: N={n_nodes} nodes, E={n_edges} edges, irreps {irreps}, "
                                f"C={ch}, per-edge weights (E,{p},{ch}), {args.rotate} rotating weight buffers"
