@@ -216,10 +216,7 @@ template <typename T, int D, int V>
 __device__ __forceinline__ void flush_segment(SegStep& st, T (&acc)[D][V], T* __restrict__ final_rows,
                                               T* __restrict__ ws, int64_t wave, bool complete, const SegRange& R,
                                               const Lanes& L, bool cok, int64_t C, int c0) {
-#pragma unroll
-  for (int m = 0; m < D; ++m)
-#pragma unroll
-    for (int v = 0; v < V; ++v) acc[m][v] = cross_group_sum(acc[m][v], L.lpe);
+  cross_group_sum_rows<T, D, V>(acc, L.lpe);
   T* dst = complete ? final_rows + (int64_t)st.cur * D * C : ws + (wave * 2 + (st.first ? 0 : 1)) * D * C;
   if (L.slot == 0 && cok && final_rows) {  // final_rows == nullptr: this result was not requested
 #pragma unroll
