@@ -133,4 +133,51 @@ __device__ __forceinline__ void cross_group_sum_rows(T (&acc)[D][V], int width) 
   }
 }
 
+// Sums of N values over groups of `width` consecutive lanes, left spread over the group's lanes: `done(s)` receives
+// an array s with s[i] = the group's sum of val[i * width + cl] in the lane whose place in the group is cl (fewer
+// entries the wider the group; entries past N are zero).  Stage b halves the values a lane still carries: the lane
+// keeps those whose index has bit b equal to its own, hands the others to its partner cl ^ (1 << b) and adds what
+// the partner hands over, so N values over 16 lanes take N/2 + N/4 + N/8 + N/16 exchanges in four dependent stages
+// (11 for N = 9) where a butterfly sum of every value takes 4 N, and one lane-contiguous store can follow instead
+// of N single-lane ones.  The first two stages stay inside quads (DPP), the others go through ds_bpermute, issued
+// together per stage.  All lanes of a group must be active; the order of the additions is fixed.
+template <int B>
+__device__ __forceinline__ float lane_xor_exchange(float v, int lane) {
+  if constexpr (B == 0)
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+  else if constexpr (B == 1)
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+  else
+    return lane_exchange(v, (lane ^ (1 << B)) << 2);
+}
+template <int B>
+__device__ __forceinline__ double lane_xor_exchange(double v, int lane) {
+  return lane_exchange(v, (lane ^ (1 << B)) << 2);
+}
+template <typename T, int N, int B = 0, typename Done>
+__device__ __forceinline__ void group_sum_scatter(const T (&val)[N], int width, Done&& done) {
+  if constexpr (B < 6) {
+    if ((1 << B) < width) {   // the same for every lane
+      constexpr int M = (N + 1) / 2;
+      const int lane = threadIdx.x & (kWave - 1);
+      const bool upper = (lane >> B) & 1;
+      T keep[M], recv[M];
+#pragma unroll
+      for (int i = 0; i < M; ++i) {
+        const T lo = val[2 * i];
+        const T hi = 2 * i + 1 < N ? val[2 * i + 1] : T(0);
+        keep[i] = upper ? hi : lo;
+        recv[i] = lane_xor_exchange<B>(upper ? lo : hi, lane);
+      }
+#pragma unroll
+      for (int i = 0; i < M; ++i) keep[i] += recv[i];
+      group_sum_scatter<T, M, B + 1>(keep, width, done);
+      return;
+    }
+  }
+  done(val);
+}
+template <typename T, int N>
+__device__ __forceinline__ constexpr int array_len(const T (&)[N]) { return N; }
+
 }  // namespace cgtp

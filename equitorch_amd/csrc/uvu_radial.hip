@@ -179,11 +179,13 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_radial_kernel(const UvuDev
           pt.pull_back(vx, vy, vz, a.y_vec == kYUnitVector);
           if (L.cl == 0) { a.gy[e * 3] = vx; a.gy[e * 3 + 1] = vy; a.gy[e * 3 + 2] = vz; }
         } else {
+          group_sum_scatter<T, D2>(gy, L.lpe, [&](const auto& s) {   // lane cl ends up with components cl, cl + lpe, ...
 #pragma unroll
-          for (int j = 0; j < D2; ++j) {
-            const T s = group_sum(gy[j], L.lpe);
-            if (L.cl == (j & (L.lpe - 1))) a.gy[e * D2 + j] = s;
-          }
+            for (int i = 0; i < array_len(s); ++i) {
+              const int j = i * L.lpe + L.cl;
+              if (j < D2) a.gy[e * D2 + j] = s[i];
+            }
+          });
         }
       }
     }
