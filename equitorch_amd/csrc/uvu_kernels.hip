@@ -245,6 +245,11 @@ struct SegIndexRegs {
     sid = (int)seg_ids[p];
     edge = (int)(perm ? perm[p] : p);
     other = (int)gather[p];
+    // The step loop reads these registers through the cross-lane unit in every step.  While the loads are still
+    // pending when the loop is entered, the compiler's wait for them sits inside the loop, where the counter it
+    // waits on also counts the stores of the step before: every step then begins by draining them.  Passing the
+    // values through an (empty) instruction here puts the wait in front of the loop.
+    asm volatile("" : "+v"(sid), "+v"(edge), "+v"(other));
   }
 };
 
