@@ -630,13 +630,17 @@ def edge_rows_bench(args):
             evs.append((a, b))
         torch.cuda.synchronize()
         return sum(a.elapsed_time(b) for a, b in evs) / len(evs)
-    fwd_ms = timed(lambda w: kernels.uvu_forward(cfg, dims, xd, shd, w, gather=plan.src))
-    bwd_ms = timed(lambda w: kernels.uvu_backward(cfg, dims, xd, shd, w, ct, (True, True, True), gather=plan.dst,
-                                                  x_gather=plan.src))
+    # the launches of the step: gather, product and segment sum fused (kernel + fix-up of the cut segments)
+    fwd_ms = timed(lambda w: kernels.uvu_forward(cfg, dims, xd, shd, w, seg=plan.fwd_index))
+    bwd_ms = timed(lambda w: kernels.uvu_backward(cfg, dims, xd, shd, w, ct, (True, True, True), seg=plan.bwd_index))
+    # for comparison: the same products per edge row, without the segment sums that would have to follow
+    rows_fwd_ms = timed(lambda w: kernels.uvu_forward(cfg, dims, xd, shd, w, gather=plan.src))
+    rows_bwd_ms = timed(lambda w: kernels.uvu_backward(cfg, dims, xd, shd, w, ct, (True, True, True), gather=plan.dst,
+                                                       x_gather=plan.src))
     nnz, s1 = dims[4], int(mod.tp_info_forward.info_Mij_fwd.out_size)
     flops_fwd = 2.0 * (nnz + s1) * ch * n_edges
     fwd_bytes, bwd_bytes = algorithmic_bytes(n_nodes, n_edges, d, p, ch)
-    msg = n_edges * d * ch * 4  # the unfused path also writes the per-edge rows once
+    msg = 0                     # per-edge rows stay in LDS
     tf = 3 * flops_fwd / (bwd_ms * 1e-3) / 1e12
     gbs = (bwd_bytes + msg) / (bwd_ms * 1e-3) / 1e9
     rec = {
@@ -645,13 +649,14 @@ def edge_rows_bench(args):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"{args.workload}: N={n_nodes} nodes, E={n_edges} edges, irreps {irreps}, C={ch}, "
                                f"per-edge weights (E,{p},{ch}), {n_rot} rotating weight buffers"},
-        "roofline": {"bound": "hbm", "kernel": "cgtp::uvu_big_bwd_kernel<TPB_sh6,1>", "achieved": round(gbs, 1),
+        "roofline": {"bound": "hbm", "kernel": "cgtp::uvu_big_seg_bwd_kernel<TPB_sh6,1>", "achieved": round(gbs, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
                      "algorithmic_bytes": bwd_bytes + msg, "avg_ms": round(bwd_ms, 4),
                      "fp32_vector": {"achieved": round(tf, 2), "peak": FP32_VECTOR_PEAK_TFLOPS, "unit": "TFLOP/s",
                                      "frac": round(tf / FP32_VECTOR_PEAK_TFLOPS, 4),
                                      "algorithmic_flops": 3 * flops_fwd}},
         "kernels": {"fwd_ms": round(fwd_ms, 4), "bwd_ms": round(bwd_ms, 4),
+                    "rows_fwd_ms": round(rows_fwd_ms, 4), "rows_bwd_ms": round(rows_bwd_ms, 4),
                     "fwd_TFLOPs": round(flops_fwd / (fwd_ms * 1e-3) / 1e12, 2),
                     "fwd_GBs": round((fwd_bytes + msg) / (fwd_ms * 1e-3) / 1e9, 1)},
     }

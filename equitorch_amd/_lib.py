@@ -122,6 +122,8 @@ def _load():
     lib.cgtp_uvu_sh_degree.argtypes = [C.c_int]
     lib.cgtp_uvu_radial_supported.argtypes = [C.c_int]
     lib.cgtp_uvu_slots.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int]
+    lib.cgtp_uvu_blockwise_only.argtypes = [C.c_int]
+    lib.cgtp_uvu_blockwise_only.restype = C.c_int
     lib.cgtp_uvu_radial_grad_workspace_bytes.restype = C.c_int64
     lib.cgtp_uvu_radial_grad_workspace_bytes.argtypes = [C.c_int64, C.c_int32, C.c_int32]
     lib.cgtp_uvu_radial_grad.argtypes = [C.c_void_p] * 6 + [C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]

@@ -97,11 +97,210 @@ __global__ void __launch_bounds__(256, 2) uvu_big_bwd_kernel(const UvuDev<float>
     // several channel chunks: each writes its partial sums to the workspace, the host sums them in chunk order
     float* gyrow = (gridDim.y > 1 ? a.ws + (int64_t)blockIdx.y * a.n_rows * D2 : a.gy) + r * D2;
 #pragma unroll
+    for (int j = 0; j < D2; ++j) gy[j] *= keep;
+    group_sum_scatter<float, D2>(gy, L.lpe, [&](const auto& s) {   // lane cl ends up with components cl, cl + lpe, ...
+#pragma unroll
+      for (int i = 0; i < array_len(s); ++i) {
+        const int j = i * L.lpe + L.cl;
+        if (row_ok && j < D2) gyrow[j] = s[i];
+      }
+    });
+  }
+}
+
+// ---- segment mode: gather, product and segment sum in one launch ------------------------------------------------
+// The sorted edge list is cut into ranges of `per_range` consecutive positions, one range per slot (group of lanes
+// that handles one edge).  A slot walks its range one position at a time and adds the finished rows of every edge to
+// an accumulator row in LDS (rows x 64 floats per wavefront, lane-private columns: no conflicts; plain read-add-write,
+// which measured 15 % faster per launch than ds_add_f32); when the
+// segment id changes it stores the row and clears it.  A segment that lies inside the range goes to its row of the
+// result; the (at most two) segments that continue in a neighbouring range go to the range's partial rows
+// ws[range][0 | 1], which uvu_fixup_kernel adds in range order.  Per-edge messages never reach memory.
+struct BigSegRange {   // positions and ranges fit 32 bits (the host checks n_rows < 2^31)
+  int p0, p1;
+  bool first_complete, last_complete;
+  __device__ __forceinline__ BigSegRange(const int64_t* __restrict__ seg_ids, int range, int per_range, int n_rows) {
+    const int64_t b = (int64_t)range * per_range;
+    p0 = b < n_rows ? (int)b : n_rows;
+    p1 = b + per_range < n_rows ? (int)(b + per_range) : n_rows;
+    first_complete = p0 >= p1 || p0 == 0 || seg_ids[p0 - 1] != seg_ids[p0];
+    last_complete = p0 >= p1 || p1 == n_rows || seg_ids[p1 - 1] != seg_ids[p1];
+  }
+};
+
+// The channel count as a value the compiler cannot follow from one loop iteration to the next.  The generated bodies
+// address row p of an operand at p * C; with C invariant over the loop, all of these products (one per weight path
+// and row: more than a hundred) are computed once in front of the loop and kept, which takes more scalar registers
+// than there are: they end up parked in vector registers, and those in scratch.  Used in the backward (lmax = 6: 3.19
+// -> 2.87 ms per launch); the forward, with fewer rows to address, is faster without (1.68 against 1.72 ms).
+__device__ __forceinline__ int opaque_copy(int v) {
+  asm volatile("" : "+s"(v));
+  return v;
+}
+
+// Segment id, edge and gathered row of the k-th position of a range; past the end of the range, those of its last
+// position (of position 0 for an empty range), so that every slot runs the same loads.
+struct BigSegIndex {
+  int sid, edge, other;
+  __device__ __forceinline__ BigSegIndex(const UvuDev<float>& a, const BigSegRange& R, int k) {
+    const int q = R.p0 + k;
+    const int qq = q < R.p1 ? q : (R.p1 > R.p0 ? R.p1 - 1 : 0);
+    sid = (int)a.seg_ids[qq];
+    edge = a.perm ? (int)a.perm[qq] : qq;
+    other = (int)a.gather[qq];
+  }
+};
+
+// Store the slot's accumulator row (D rows of one channel per lane) as the row of segment `seg` and clear it.
+template <int D>
+__device__ __forceinline__ void big_seg_flush(float* __restrict__ acc, float* __restrict__ rows, float* __restrict__ ws,
+                                              int seg, int range, bool first, bool complete, int64_t C, int c,
+                                              bool c_ok) {
+  float* dst = (complete ? rows + (int64_t)seg * D * C : ws + ((int64_t)range * 2 + (first ? 0 : 1)) * D * C) + c;
+#pragma unroll
+  for (int m = 0; m < D; ++m) {
+    const float v = acc[m * kWave];
+    acc[m * kWave] = 0.f;
+    if (c_ok) dst[m * C] = v;
+  }
+}
+
+template <class TP, bool PS>
+__global__ void __launch_bounds__(256, 2) uvu_big_seg_fwd_kernel(const UvuDev<float> a, int64_t n_waves) {
+  constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
+  extern __shared__ float big_seg_lds[];
+  const Lanes L(a.lpe_log2);
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (wave >= n_waves) return;
+  float* acc = big_seg_lds + (threadIdx.x / kWave) * DO * kWave + L.lane;
+#pragma unroll
+  for (int m = 0; m < DO; ++m) acc[m * kWave] = 0.f;
+  const int64_t C = a.C;
+  const int c_raw = blockIdx.y * L.lpe + L.cl;
+  const bool c_ok = c_raw < a.C;
+  const int c = min(c_raw, a.C - 1);
+  const int range = (int)wave * L.slots + L.slot;
+  const BigSegRange R(a.seg_ids, range, a.pos_per_wave, (int)a.n_rows);
+  const float* __restrict__ ps = a.ps;
+  int cur = -1;
+  bool first = true;
+  BigSegIndex I(a, R, 0);
+  for (int k = 0; k < a.pos_per_wave; ++k) {       // the same trip count in every slot; `live` masks the tail
+    const bool live = R.p0 + k < R.p1;
+    const int sid = I.sid;
+    const int64_t e = I.edge, xr = I.other;
+    if (k + 1 < a.pos_per_wave) I = BigSegIndex(a, R, k + 1);   // in flight during this position's arithmetic
+    if (live && sid != cur) {
+      if (cur >= 0) {
+        big_seg_flush<DO>(acc, a.out, a.ws, cur, range, first, first ? R.first_complete : true, C, c, c_ok);
+        first = false;
+      }
+      cur = sid;
+    }
+    float x[D1], y[D2];
+#pragma unroll
+    for (int j = 0; j < D2; ++j) y[j] = a.y[e * D2 + j];
+#pragma unroll
+    for (int i = 0; i < D1; ++i) x[i] = a.x[(xr * D1 + i) * C + c];
+    const float* wrow = a.w + (a.w_shared ? 0 : e) * P * C + c;
+    TP::fwd(
+        x, y,
+        [&](int p) __attribute__((always_inline)) {
+          const float w = __builtin_nontemporal_load(wrow + p * C);
+          if constexpr (PS) return w * ps[p]; else return w;
+        },
+        [&](int m, float v) __attribute__((always_inline)) {
+          acc[m * kWave] += live ? v : 0.f;   // no branch: the reads can be issued early
+        });
+  }
+  if (cur >= 0)
+    big_seg_flush<DO>(acc, a.out, a.ws, cur, range, first, (first ? R.first_complete : true) && R.last_complete, C, c,
+                      c_ok);
+}
+
+// Backward of the above over the list sorted by the other end: a segment is a row of x, its gradient is summed in
+// LDS; grad_out rows are gathered, grad_y and the weight gradient are written per edge.
+template <class TP, int GW, bool PS>
+__global__ void __launch_bounds__(256, 2) uvu_big_seg_bwd_kernel(const UvuDev<float> a, int64_t n_waves) {
+  constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
+  extern __shared__ float big_seg_lds[];
+  const Lanes L(a.lpe_log2);
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (wave >= n_waves) return;
+  float* acc = big_seg_lds + (threadIdx.x / kWave) * D1 * kWave + L.lane;
+#pragma unroll
+  for (int i = 0; i < D1; ++i) acc[i * kWave] = 0.f;
+  const int64_t C0 = a.C;
+  const int c_raw = blockIdx.y * L.lpe + L.cl;
+  const bool c_ok = c_raw < a.C;
+  const int c = min(c_raw, a.C - 1);
+  const int range = (int)wave * L.slots + L.slot;
+  const BigSegRange R(a.seg_ids, range, a.pos_per_wave, (int)a.n_rows);
+  const float* __restrict__ ps = a.ps;
+  const bool want_gx = a.gx != nullptr;
+  int cur = -1;
+  bool first = true;
+  BigSegIndex I(a, R, 0);
+  for (int k = 0; k < a.pos_per_wave; ++k) {
+    const int64_t C = opaque_copy(a.C);
+    const bool live = R.p0 + k < R.p1;
+    const int sid = I.sid;
+    const int64_t e = I.edge, gr = I.other;
+    if (k + 1 < a.pos_per_wave) I = BigSegIndex(a, R, k + 1);   // in flight during this position's arithmetic
+    if (live && sid != cur) {
+      if (cur >= 0) {
+        if (want_gx)
+          big_seg_flush<D1>(acc, a.gx, a.ws, cur, range, first, first ? R.first_complete : true, C, c, c_ok);
+        first = false;
+      }
+      cur = sid;
+    }
+    float y[D2], gy[D2], g[DO];
+#pragma unroll
     for (int j = 0; j < D2; ++j) {
-      const float s = group_sum(gy[j] * keep, L.lpe);
-      if (row_ok && L.cl == (j & (L.lpe - 1))) gyrow[j] = s;
+      y[j] = a.y[e * D2 + j];
+      gy[j] = 0.f;
+    }
+    const float* grow = a.g + gr * DO * C + c;
+#pragma unroll
+    for (int m = 0; m < DO; ++m) g[m] = grow[m * C];
+    const float* xrow = a.x + (int64_t)sid * D1 * C + c;
+    const float* wrow = a.w + (a.w_shared ? 0 : e) * P * C + c;
+    float* gwrow = a.gw + e * P * C + c;
+    const bool store = live && c_ok;
+    TP::bwd(
+        [&](int i) __attribute__((always_inline)) { return xrow[i * C]; }, y,
+        [&](int p) __attribute__((always_inline)) {
+          const float w = __builtin_nontemporal_load(wrow + p * C);
+          if constexpr (PS) return w * ps[p]; else return w;
+        },
+        g,
+        [&](int i, float v) __attribute__((always_inline)) {
+          if (live) acc[i * kWave] += v;   // under a branch on purpose: hoisted reads would not fit the registers here
+        },
+        gy,
+        [&](int p, float v) __attribute__((always_inline)) {
+          if constexpr (GW == kGwStore) {
+            if (store) __builtin_nontemporal_store(PS ? v * ps[p] : v, gwrow + p * C);
+          }
+        });
+    if (a.gy) {
+      const float keep = c_ok ? 1.f : 0.f;  // duplicate channels of the padding lanes do not count
+      float* gyrow = a.gy + e * D2;
+#pragma unroll
+      for (int j = 0; j < D2; ++j) gy[j] *= keep;
+      group_sum_scatter<float, D2>(gy, L.lpe, [&](const auto& s) {   // lane cl ends up with components cl, cl + lpe, ...
+#pragma unroll
+        for (int i = 0; i < array_len(s); ++i) {
+          const int j = i * L.lpe + L.cl;
+          if (live && j < D2) gyrow[j] = s[i];
+        }
+      });
     }
   }
+  if (cur >= 0 && want_gx)
+    big_seg_flush<D1>(acc, a.gx, a.ws, cur, range, first, (first ? R.first_complete : true) && R.last_complete, C0, c,
+                      c_ok);
 }
 
 template <class TP, bool PS>
@@ -118,6 +317,9 @@ static UvuBigEntry make_big_entry() {
   e.fwd_yc = uvu_big_fwd_kernel<TP, PS, true>;
   e.bwd_yc[kGwNone] = uvu_big_bwd_kernel<TP, kGwNone, PS, true>;
   e.bwd_yc[kGwStore] = uvu_big_bwd_kernel<TP, kGwStore, PS, true>;
+  e.seg_fwd = uvu_big_seg_fwd_kernel<TP, PS>;
+  e.seg_bwd[kGwNone] = uvu_big_seg_bwd_kernel<TP, kGwNone, PS>;
+  e.seg_bwd[kGwStore] = uvu_big_seg_bwd_kernel<TP, kGwStore, PS>;
   return e;
 }
 

@@ -79,6 +79,9 @@ struct UvuBigEntry {
   // the same with a channelled second operand, y (n_rows, D2, C) ("uuu"): grad_y is then per channel as well
   void (*fwd_yc)(const UvuDev<float>);
   void (*bwd_yc[2])(const UvuDev<float>, int64_t);
+  // segment mode (gather, product and segment sum fused); dynamic LDS: 4 x rows x 64 floats per workgroup
+  void (*seg_fwd)(const UvuDev<float>, int64_t);
+  void (*seg_bwd[2])(const UvuDev<float>, int64_t);
 };
 // Segment-mode kernels that form the per-edge weights from per-edge features and a shared matrix (uvu_radial.hip);
 // [0]: second operand given as harmonics, [1]: as edge vectors (nullptr where the config has no such form).

@@ -690,7 +690,13 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
     if ((int64_t)rad[a->cfg].lds_floats_per_r * a->radial_r * 4 > kLdsBytes) return CGTP_ERR_LDS;
     if (!aligned16(a->radial_h) || !aligned16(a->radial_w)) return CGTP_ERR_ALIGN;
   }
-  if (a->cfg >= n_cfg && seg) return CGTP_ERR_SHAPE;  // block-wise kernels only: row mode
+  if (big && seg) {
+    // block-wise kernels in segment mode: ranges by position only, harmonics given, per-edge weights (or no weight
+    // gradient), rows no wider than one wavefront
+    if (a->wave_seg || a->wave_pos || a->y_vec || a->y_channels) return CGTP_ERR_SHAPE;
+    if (backward && a->w_shared && a->grad_w) return CGTP_ERR_SHAPE;
+    if (a->C > kWave) return CGTP_ERR_SHAPE;
+  }
   if (seg && (!a->ptr || !a->seg_ids || !a->gather)) return CGTP_ERR_NULL;
   if (!seg && (a->ptr || a->perm || a->seg_ids)) return CGTP_ERR_SHAPE;
   if (seg && (a->n_seg >= (int64_t)1 << 31 || a->n_rows >= (int64_t)1 << 31 || a->n_x_rows >= (int64_t)1 << 31))
@@ -748,6 +754,16 @@ static int uvu_plan(const cgtp_uvu_args* a, int backward, bool need_ws, UvuPlan*
   } else if (seg && a->wave_pos) {
     plan->n_waves = a->n_waves;  // ranges cut at given positions: partial rows as for ranges by position
     if (!backward || a->grad_x) plan->ws_elems = plan->n_waves * 2 * row_d * a->C;
+  } else if (seg && big) {
+    // one range per slot; by default as many ranges as fill the resident wavefronts once (two per SIMD), but no
+    // fewer than 4 positions each.  pos_per_wave here counts the positions of a range.
+    int64_t per = a->pos_per_wave > 0 ? a->pos_per_wave : (a->n_rows + kMaxRowWaves * slots - 1) / (kMaxRowWaves * slots);
+    if (a->pos_per_wave <= 0 && per < 4) per = 4;
+    if (per >= (int64_t)1 << 30) return CGTP_ERR_SHAPE;
+    plan->pos_per_wave = (int)per;
+    const int64_t n_ranges = (a->n_rows + per - 1) / per;
+    plan->n_waves = (n_ranges + slots - 1) / slots;
+    if (!backward || a->grad_x) plan->ws_elems = plan->n_waves * slots * 2 * row_d * a->C;
   } else if (seg) {
     int ppw = a->pos_per_wave > 0 ? a->pos_per_wave : kDefaultPosPerWave;
     ppw = ((ppw + slots - 1) / slots) * slots;
@@ -811,6 +827,24 @@ static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward,
   const UvuBigEntry& e = (a->path_scale ? uvu_big_entries_scaled(&n_big) : uvu_big_entries(&n_big))[plan.big_idx];
   const bool wred = backward && a->w_shared && a->grad_w;
   const int64_t w_elems = (int64_t)e.dims[3] * a->C;
+  if (a->n_seg > 0) {   // fused gather / product / segment sum; the fix-up sees one range per slot
+    UvuDev<float> d = to_dev<float>(a, plan);
+    const int rows = backward ? e.dims[0] : e.dims[2];
+    if (plan.n_waves > 0) {
+      void (*fn)(const UvuDev<float>, int64_t) = backward ? e.seg_bwd[a->grad_w ? kGwStore : kGwNone] : e.seg_fwd;
+      const size_t lds = (size_t)4 * rows * kWave * sizeof(float);
+      if (lds > (size_t)kLdsBytes) return CGTP_ERR_LDS;
+      if (lds > 48 * 1024 &&
+          hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return CGTP_ERR_LDS;
+      hipLaunchKernelGGL(fn, dim3((unsigned)((plan.n_waves + 3) / 4)), dim3(256), lds, stream, d, plan.n_waves);
+      if (launched() != CGTP_OK) return CGTP_ERR_LAUNCH;
+    }
+    float* out_rows = backward ? d.gx : d.out;
+    if (!out_rows) return CGTP_OK;
+    d.n_waves = plan.n_waves * (kWave >> plan.lpe_log2);
+    return launch_fixup<float>(out_rows, d, (int64_t)rows * a->C, stream);   // also zeroes the rows of empty segments
+  }
   if (plan.n_waves == 0) {
     if (wred) launch_partial_sum<float>(nullptr, (float*)a->grad_w, 0, w_elems, stream);   // zero partials: writes 0
     return CGTP_OK;
@@ -1010,6 +1044,13 @@ int cgtp_uvu_slots(int cfg, int dtype, int C, int backward) {
   int lg = 0;
   while ((1 << lg) < lanes) ++lg;
   return kWave >> lg;
+}
+
+int cgtp_uvu_blockwise_only(int cfg) {
+  int n = 0, n_big = 0;
+  entries<float>(&n);
+  uvu_big_entries(&n_big);
+  return cfg >= n && cfg < n + n_big;
 }
 
 int cgtp_uvu_validate(const cgtp_uvu_args* args, int backward) {

@@ -514,7 +514,7 @@ def _uvu_args(cfg: int, x: Tensor, y: Tensor, w: Tensor, seg: Optional[SegIndex]
         a.ptr, a.perm, a.seg_ids, a.gather = seg.ptr.data_ptr(), _lib.ptr(seg.perm), seg.seg_ids.data_ptr(), \
             seg.gather.data_ptr()
         a.pos_per_wave = pos_per_wave
-        if pos_per_wave == 0:
+        if pos_per_wave == 0 and not _lib.lib.cgtp_uvu_blockwise_only(int(cfg)):   # those cut ranges by position
             wave_pos = None
             if _RANGE_MODE == "balanced" or (_RANGE_MODE == "auto" and (backward or seg.wave_seg is None)):
                 wave_pos = seg.balanced_positions(int(_lib.lib.cgtp_uvu_slots(int(cfg), a.dtype, a.C, int(backward))))

@@ -171,6 +171,12 @@ int cgtp_segment_sum(const void* in, const void* scale, const int64_t* index, co
  * positions between two entries of wave_pos, and segments cut by a range boundary go through partial rows in the
  * workspace and a fix-up kernel.  Either way
  * there are no atomics and results are deterministic.
+ *
+ * Configs whose tables are too large for a register-resident body (cgtp_uvu_blockwise_only(): e.g. lmax = 6, 6460
+ * coefficients) run segment mode on their block-wise kernels: fp32, C <= 64, harmonics given, per-edge weights (or
+ * no weight gradient), ranges by position only (wave_seg and wave_pos must be NULL); one range per group of lanes
+ * that handles an edge, pos_per_wave then counts the positions of such a range (0 = as many ranges as fill the GPU
+ * once), and the sums over a segment are kept in LDS.
  */
 int cgtp_uvu_num_configs(void);
 int cgtp_uvu_find(uint64_t fingerprint);
@@ -201,7 +207,7 @@ typedef struct cgtp_uvu_args {
   const int64_t* seg_ids;  /* segment mode: [n_rows] sorted position -> segment id, ascending      */
   const int64_t* gather;   /* [n_rows] row of the gathered operand (fwd: x, bwd: grad_out); row mode: per
                               row, optional; segment mode: per sorted position, required           */
-  int32_t pos_per_wave;    /* segment mode without wave_seg: positions per wavefront; 0 = 32       */
+  int32_t pos_per_wave;    /* segment mode without wave_seg: positions per wavefront; 0 = 32 (block-wise-only configs: see above) */
   int32_t y_vec;           /* segment mode: 0 = y holds harmonics (n_rows, D2); 1 / 2 = y holds edge vectors
                               (n_rows, 3) and the kernel evaluates the harmonics of degrees 0..sqrt(D2)-1 itself,
                               of y / max(|y|, 1e-12) (1) or of y as it is (2); grad_y is then (n_rows, 3).  Needs a
@@ -267,6 +273,8 @@ int cgtp_uvu_radial_grad(const void* grad_w, const void* radial_h, const void* r
 /* Positions of one segment a wavefront takes per step (64 / lanes per edge) in a segment-mode launch of config
  * `cfg` with C channels and aligned operands; 0 if there is no such launch.  Host only. */
 int cgtp_uvu_slots(int cfg, int dtype, int C, int backward);
+/* 1 if config `cfg` exists only as block-wise kernels (one channel per lane, fp32), else 0. */
+int cgtp_uvu_blockwise_only(int cfg);
 int cgtp_uvu_validate(const cgtp_uvu_args* args, int backward);
 /* Bytes of workspace the forward (backward = 0) or backward (1) launch of `args` needs; 0 if none. */
 int64_t cgtp_uvu_workspace_bytes(const cgtp_uvu_args* args, int backward);

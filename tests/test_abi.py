@@ -138,7 +138,21 @@ def test_large_table_configs_and_row_gathers_validate_on_the_host():
     assert L.cgtp_uvu_workspace_bytes(C.byref(a), 1) == (10 + 1) * 106 * 32 * 4
     assert L.cgtp_uvu_bwd(C.byref(a), None) == 8                    # workspace missing, nothing launched
     a.w_shared, a.grad_w, a.n_seg, a.ptr, a.seg_ids, a.gather = 0, 4096, 10, 4096, 4096, 4096
-    assert L.cgtp_uvu_validate(C.byref(a), 0) == 2                  # no segment mode
+    # segment mode on the block-wise kernels: one range per group of 32 lanes (C = 32: two per wavefront), at least
+    # 4 positions each -> 3 ranges, 2 wavefronts, 2 partial rows per range slot
+    assert L.cgtp_uvu_blockwise_only(cfg) == 1 and L.cgtp_uvu_blockwise_only(0) == 0
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 0 and L.cgtp_uvu_validate(C.byref(a), 1) == 0
+    assert L.cgtp_uvu_workspace_bytes(C.byref(a), 0) == 2 * 2 * 2 * 49 * 32 * 4
+    a.pos_per_wave = 1                                              # here: positions per range -> 10 ranges, 5 wavefronts
+    assert L.cgtp_uvu_workspace_bytes(C.byref(a), 1) == 5 * 2 * 2 * 49 * 32 * 4
+    a.pos_per_wave = 0
+    a.w_shared = 1
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 0 and L.cgtp_uvu_validate(C.byref(a), 1) == 2   # no shared-weight gradient
+    a.w_shared, a.C = 0, 65
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 2                  # one wavefront wide at most
+    a.C, a.wave_seg, a.n_waves = 32, 4096, 3
+    assert L.cgtp_uvu_validate(C.byref(a), 0) == 2                  # ranges by position only
+    a.wave_seg, a.n_waves = None, 0
     # row-mode backward with gathered x rows: x may then have any number of rows
     a.n_seg, a.ptr, a.seg_ids = 0, None, None
     a.n_x_rows = 4

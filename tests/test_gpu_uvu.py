@@ -208,13 +208,15 @@ def test_shared_weight_backward_in_row_parts(device, monkeypatch, lmax, n, ch):
             assert torch.equal(g, h), name
 
 
-def test_edge_large_table(device):
-    """Edge message passing at lmax = 6, C = 32 (BASELINE configs[4] shapes, small graph): gathered row-mode
-    kernels plus segment sums against the dense oracle."""
+@pytest.mark.parametrize("ch", [32, 20, 64])
+def test_edge_large_table(device, ch):
+    """Edge message passing at lmax = 6 (BASELINE configs[4] shapes, small graph) through the public path: the
+    block-wise kernels in segment mode (gather, product and segment sum in one launch) against the dense oracle."""
     from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu
+    from equitorch_amd.ops import kernels
     mod = _module(SH6, SH6, SH6).to(device)
     gen = torch.Generator().manual_seed(15)
-    n_nodes, n_edges, ch = 41, 333, 32
+    n_nodes, n_edges = 41, 333
     src = torch.randint(0, n_nodes, (n_edges,), generator=gen)
     dst = torch.randint(0, n_nodes - 2, (n_edges,), generator=gen)
     x, sh, w = tp_inputs(n_edges, 49, 6, mod.num_paths, ch, False, seed=16)
@@ -222,6 +224,8 @@ def test_edge_large_table(device):
     ct = torch.randn(n_nodes, 49, ch, generator=gen)
     plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
     xd, shd, wd = (t.to(device).requires_grad_(True) for t in (x, sh, w))
+    cfg = kernels.uvu_config_of(mod.tp_info_forward)
+    assert kernels.uvu_launchable(cfg, xd.detach(), shd.detach(), wd.detach(), segments=True), "fused path expected"
     out = edge_tensor_product_uu(xd, shd, wd, plan, mod.tp_info_forward)
     (out * ct.to(device)).sum().backward()
     T = ref_ops.dense_coupling(SH6, SH6, SH6)
@@ -231,7 +235,48 @@ def test_edge_large_table(device):
     ref_out, ref_grads = ref_ops.dense_grads(ref_fn, T, (x, sh, w), ct)
     for name, g, r in zip(("out", "grad_x", "grad_sh", "grad_w"), (out, xd.grad, shd.grad, wd.grad),
                           (ref_out, *ref_grads)):
-        assert_close(g, r, 1e-5, f"edge lmax=6 {name}")
+        assert_close(g, r, 1e-5, f"edge lmax=6 C={ch} {name}")
+
+
+@pytest.mark.parametrize("lmax,ch,per", [(4, 32, 1), (4, 16, 3), (4, 32, 7), (6, 32, 64), (4, 8, 5), (4, 32, 5000)])
+def test_edge_large_table_ranges(device, lmax, ch, per):
+    """The same kernels with ranges of `per` sorted positions: a hub node whose segment spans many ranges, nodes
+    without edges, a last range that is not full, and one range that holds everything."""
+    from equitorch_amd.nn.functional import EdgePlan
+    from equitorch_amd.ops import kernels
+    irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+    mod = _module(irreps, irreps, irreps).to(device)
+    d = (lmax + 1) ** 2
+    gen = torch.Generator().manual_seed(100 + per)
+    n_nodes, n_edges = 37, 301
+    src = torch.randint(0, n_nodes, (n_edges,), generator=gen)
+    dst = torch.randint(0, n_nodes - 3, (n_edges,), generator=gen)
+    dst[::3] = 5                                           # hub: a third of all edges end at node 5
+    src[1::4] = 11                                         # and a quarter start at node 11
+    x, sh, w = tp_inputs(n_edges, d, lmax, mod.num_paths, ch, False, seed=17)
+    x = x[:n_nodes].contiguous()
+    ct = torch.randn(n_nodes, d, ch, generator=gen)
+    plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
+    cfg = kernels.uvu_config_of(mod.tp_info_forward)
+    dims = kernels.uvu_dims(cfg)
+    xd, shd, wd, ctd = (t.to(device) for t in (x, sh, w, ct))
+    out = kernels.uvu_forward(cfg, dims, xd, shd, wd, seg=plan.fwd_index, pos_per_wave=per)
+    gx, gy, gw = kernels.uvu_backward(cfg, dims, xd, shd, wd, ctd, (True, True, True), seg=plan.bwd_index,
+                                      pos_per_wave=per)
+    T = ref_ops.dense_coupling(irreps, irreps, irreps)
+
+    def ref_fn(T, x, sh, w):
+        return ref_ops.scatter_sum(ref_ops.dense_u1u(T, x.index_select(0, src), sh, w), dst, n_nodes)
+    ref_out, ref_grads = ref_ops.dense_grads(ref_fn, T, (x, sh, w), ct)
+    for name, g, r in zip(("out", "grad_x", "grad_sh", "grad_w"), (out, gx, gy, gw), (ref_out, *ref_grads)):
+        assert_close(g, r, 1e-5, f"edge lmax={lmax} C={ch} per={per} {name}")
+    # only some gradients requested
+    gx2, gy2, gw2 = kernels.uvu_backward(cfg, dims, xd, shd, wd, ctd, (True, False, False), seg=plan.bwd_index,
+                                         pos_per_wave=per)
+    assert gy2 is None and gw2 is None and torch.equal(gx2, gx)
+    gx3, gy3, gw3 = kernels.uvu_backward(cfg, dims, xd, shd, wd, ctd, (False, True, True), seg=plan.bwd_index,
+                                         pos_per_wave=per)
+    assert gx3 is None and torch.equal(gy3, gy) and torch.equal(gw3, gw)
 
 
 @pytest.mark.parametrize("lmax,n,ch", [(3, 130, 128), (2, 257, 200), (2, 33, 65)])
