@@ -159,8 +159,8 @@ def edge_tensor_product_uu(x: Tensor, sh: Tensor, weight: Tensor, plan: EdgePlan
     """``out[v] = sum_{e: dst[e]=v} TP_uu(x[src[e]], sh[e], W[e])``.
 
     ``x (N_src, D1, C)``, ``sh (E, D2)``, ``weight (E, P, C) | (P, C)`` -> ``(N, DO, C)``.  Uses the fused
-    kernel when the table of ``tp_info_forward`` is compiled in and one wavefront slot covers the channels;
-    otherwise runs the same three steps as separate launches.
+    kernel when the table of ``tp_info_forward`` is compiled in and one wavefront slot covers the channels (large
+    tables, e.g. lmax = 6: fp32 with per-edge weights); otherwise runs the same three steps as separate launches.
     """
     _lib.require_gpu(x, sh, weight)
     if plan.num_src_nodes != x.shape[0]:

@@ -147,7 +147,8 @@ def test_edge_fused_full_size_vectors(device):
 
 def test_edge_full_size_lmax6(device):
     """BASELINE configs[4] shapes: N = 20000, E = 200000, lmax = 6, C = 32, per-edge weights (2.7 GB), forward and
-    all gradients through the public autograd path (block-wise row-mode kernels + segment sums over 200000 rows)."""
+    all gradients through the public autograd path (block-wise kernels in segment mode: 4082 ranges of 49 sorted
+    positions, segment sums in LDS)."""
     from equitorch_amd.nn import SO3Linear
     from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu
     irr = _sh_irreps(6)
