@@ -431,14 +431,19 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, 
       }
       if (a.gy) {
         if constexpr (YV) {
-          // chain rule through the harmonics (and the normalisation): three values per edge instead of D2
-#pragma unroll
-          for (int j = 0; j < D2; ++j) gy[j] = group_sum(gy[j], L.lpe);
+          // chain rule through the harmonics (and the normalisation): linear in grad_y, so every lane applies it
+          // to its own channels' share first and three values per edge are summed over the channels instead of D2
           const ShPoint<T> pt(ux, uy, uz, a.y_vec == kYUnitVector);
-          T vx, vy, vz;
-          sh_pull_back<T, TP::SH_LMAX>(pt.x, pt.y, pt.z, gy, vx, vy, vz);
-          pt.pull_back(vx, vy, vz, a.y_vec == kYUnitVector);
-          if (L.cl == 0) { a.gy[e * 3] = vx; a.gy[e * 3 + 1] = vy; a.gy[e * 3 + 2] = vz; }
+          T v3[3];
+          sh_pull_back<T, TP::SH_LMAX>(pt.x, pt.y, pt.z, gy, v3[0], v3[1], v3[2]);
+          pt.pull_back(v3[0], v3[1], v3[2], a.y_vec == kYUnitVector);
+          group_sum_scatter<T, 3>(v3, L.lpe, [&](const auto& s) {
+#pragma unroll
+            for (int i = 0; i < array_len(s); ++i) {
+              const int j = i * L.lpe + L.cl;
+              if (j < 3) a.gy[e * 3 + j] = s[i];
+            }
+          });
         } else {
           group_sum_scatter<T, D2>(gy, L.lpe, [&](const auto& s) {   // lane cl ends up with components cl, cl + lpe, ...
 #pragma unroll
