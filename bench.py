@@ -798,8 +798,8 @@ def layer_bench(steps, warmup):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="edge_fwd_bwd", choices=sorted(WORKLOADS))
     ap.add_argument("--rotate", type=int, default=4, help="number of weight buffers cycled through")
     ap.add_argument("--graph", default="uniform", choices=["uniform", "local"],
@@ -984,7 +984,7 @@ def other_configs(args, headline):
                                       "Medges_s": round(65536 / (k["fwd_avg_ms"] * 1e-3) / 1e6, 1)}
     out["cfg0_uvu_B1024_C16_shared_w"] = config0_record(not args.no_cpu_baseline)
     sub = copy.copy(args)
-    sub.steps, sub.warmup, sub.kernel_reps, sub.no_cpu_baseline = 10, 3, 12, True
+    sub.steps, sub.warmup, sub.kernel_reps, sub.no_cpu_baseline = 50, 10, 30, True
     sub.workload = "uvw_fwd_bwd"
     r = uvw_bench(sub)
     flops = r["roofline"]["algorithmic_flops"]
@@ -995,7 +995,7 @@ def other_configs(args, headline):
         "grad_x_ms": r["kernels"]["grad_x_ms"], "grad_sh_ms": r["kernels"]["grad_sh_ms"],
         "grad_w_ms": r["kernels"]["grad_w_ms"]}
     torch.cuda.empty_cache()
-    sub.workload, sub.steps, sub.warmup = "edge_l6_fwd_bwd", 4, 2
+    sub.workload, sub.steps, sub.warmup = "edge_l6_fwd_bwd", 20, 4
     r = edge_rows_bench(sub)
     torch.cuda.empty_cache()
     out["cfg1_edge_weights_formed_in_kernel_R16"] = radial_record(16)
