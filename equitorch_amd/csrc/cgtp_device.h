@@ -140,7 +140,9 @@ __device__ __forceinline__ void cross_group_sum_rows(T (&acc)[D][V], int width) 
 // the partner hands over, so N values over 16 lanes take N/2 + N/4 + N/8 + N/16 exchanges in four dependent stages
 // (11 for N = 9) where a butterfly sum of every value takes 4 N, and one lane-contiguous store can follow instead
 // of N single-lane ones.  The first two stages stay inside quads (DPP), the others go through ds_bpermute, issued
-// together per stage.  All lanes of a group must be active; the order of the additions is fixed.
+// together per stage.  All lanes of a group must be active; the order of the additions is fixed.  In a kernel close to
+// a register boundary the few extra live values can cost a wavefront per SIMD: check the resource usage of every
+// instantiation that adopts it.
 template <int B>
 __device__ __forceinline__ float lane_xor_exchange(float v, int lane) {
   if constexpr (B == 0)

@@ -135,13 +135,11 @@ __global__ void __launch_bounds__(256, 2) uvu_bwd_kernel(const UvuDev<T> a, int6
       zero_rows(gx);
     }
     if (a.gy) {
-      group_sum_scatter<T, D2>(gy, L.lpe, [&](const auto& s) {   // lane cl ends up with components cl, cl + lpe, ...
 #pragma unroll
-        for (int i = 0; i < array_len(s); ++i) {
-          const int j = i * L.lpe + L.cl;
-          if (j < D2) a.gy[r * D2 + j] = s[i];
-        }
-      });
+      for (int j = 0; j < D2; ++j) {
+        const T s = group_sum(gy[j], L.lpe);
+        if (L.cl == (j & (L.lpe - 1))) a.gy[r * D2 + j] = s;
+      }
     }
   }
   if constexpr (GW == kGwReduce) {
@@ -430,7 +428,12 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, 
             });
       }
       if (a.gy) {
-        if constexpr (YV) {
+        // Sums over the channels of an edge.  kSpread: the halving exchange (group_sum_scatter) — a quarter of the
+        // cross-lane moves, issued together, one store.  It keeps a few more values live at once; in the
+        // instantiations named by kSpread that costs nothing, in most others it costs a wavefront per SIMD or
+        // scratch, and those sum one component at a time as before.
+        constexpr bool kSpread = sizeof(T) == 4 && V == 4 && GW != kGwReduce && D2 >= 9;
+        if constexpr (YV && kSpread) {
           // chain rule through the harmonics (and the normalisation): linear in grad_y, so every lane applies it
           // to its own channels' share first and three values per edge are summed over the channels instead of D2
           const ShPoint<T> pt(ux, uy, uz, a.y_vec == kYUnitVector);
@@ -444,7 +447,15 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, 
               if (j < 3) a.gy[e * 3 + j] = s[i];
             }
           });
-        } else {
+        } else if constexpr (YV) {
+#pragma unroll
+          for (int j = 0; j < D2; ++j) gy[j] = group_sum(gy[j], L.lpe);
+          const ShPoint<T> pt(ux, uy, uz, a.y_vec == kYUnitVector);
+          T vx, vy, vz;
+          sh_pull_back<T, TP::SH_LMAX>(pt.x, pt.y, pt.z, gy, vx, vy, vz);
+          pt.pull_back(vx, vy, vz, a.y_vec == kYUnitVector);
+          if (L.cl == 0) { a.gy[e * 3] = vx; a.gy[e * 3 + 1] = vy; a.gy[e * 3 + 2] = vz; }
+        } else if constexpr (kSpread) {
           group_sum_scatter<T, D2>(gy, L.lpe, [&](const auto& s) {   // lane cl ends up with components cl, cl + lpe, ...
 #pragma unroll
             for (int i = 0; i < array_len(s); ++i) {
@@ -452,6 +463,12 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, 
               if (j < D2) a.gy[e * D2 + j] = s[i];
             }
           });
+        } else {
+#pragma unroll
+          for (int j = 0; j < D2; ++j) {
+            const T s = group_sum(gy[j], L.lpe);
+            if (L.cl == (j & (L.lpe - 1))) a.gy[e * D2 + j] = s;
+          }
         }
       }
     }

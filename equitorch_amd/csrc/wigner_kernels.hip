@@ -260,17 +260,11 @@ __global__ void __launch_bounds__(256) wigner_rotate_bwd_kernel(
 #pragma unroll
   for (int a = 0; a < 3; ++a) {
     if (!outs[a]) continue;
-    T vals[NACC];
 #pragma unroll
-    for (int i = 0; i < NACC; ++i) vals[i] = ok ? accs[a][i] : T(0);
-    T* dst = outs[a] + r * cs_dim;
-    group_sum_scatter<T, NACC>(vals, lpr, [&](const auto& s) {   // lane `sub` ends up with columns sub, sub + lpr, ...
-#pragma unroll
-      for (int i = 0; i < array_len(s); ++i) {
-        const int j = i * lpr + sub;
-        if (r < n_rows && j < NACC && j < cs_dim) dst[j] = s[i];
-      }
-    });
+    for (int i = 0; i < NACC; ++i) {
+      const T total = group_sum(ok ? accs[a][i] : T(0), lpr);
+      if (r < n_rows && sub == 0 && i < cs_dim) outs[a][r * cs_dim + i] = total;
+    }
     if (r < n_rows && sub == 0)
       for (int i = NACC; i < cs_dim; ++i) outs[a][r * cs_dim + i] = T(0);
   }
