@@ -220,40 +220,88 @@ __global__ void __launch_bounds__(256, 2) uvu_big_seg_fwd_kernel(const UvuDev<fl
 
 // Backward of the above over the list sorted by the other end: a segment is a row of x, its gradient is summed in
 // LDS; grad_out rows are gathered, grad_y and the weight gradient are written per edge.
+//
+// The body needs all 256 registers, so nothing may stay in a register from one position to the next: whatever the
+// compiler carries across the body it spills to scratch, and a reload from scratch waits on the counter that also
+// counts the 106 weight-gradient stores of the position before (they would otherwise drain in the background).
+// Therefore
+//  * everything that follows from the thread index and the kernel arguments (lane roles, range, channel, pointers)
+//    is derived again in every iteration from a copy of the thread index the compiler cannot follow (opaque_lane);
+//  * the two values that do change (open segment, "nothing flushed yet") live in LDS (kBigSegStateInts per lane);
+//  * the indices of the next positions are staged in LDS a chunk at a time: every `lanes per edge` iterations the
+//    lanes of a slot load segment id, edge and gathered row of that many positions with one coalesced load each
+//    (kBigSegIndexInts per wavefront), and an iteration reads its three values from there.
+constexpr int kBigSegIndexInts = kWave * 3;
+constexpr int kBigSegStateInts = 2;
+__device__ __forceinline__ int opaque_lane() {
+  int v = threadIdx.x;
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
 template <class TP, int GW, bool PS>
 __global__ void __launch_bounds__(256, 2) uvu_big_seg_bwd_kernel(const UvuDev<float> a, int64_t n_waves) {
   constexpr int D1 = TP::D1, D2 = TP::D2, DO = TP::DO, P = TP::P;
   extern __shared__ float big_seg_lds[];
-  const Lanes L(a.lpe_log2);
-  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
-  if (wave >= n_waves) return;
-  float* acc = big_seg_lds + (threadIdx.x / kWave) * D1 * kWave + L.lane;
+  if ((int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave >= n_waves) return;
+  int* const idx_all = reinterpret_cast<int*>(big_seg_lds + 4 * D1 * kWave);
+  volatile int* const state = reinterpret_cast<volatile int*>(idx_all + 4 * kBigSegIndexInts) + threadIdx.x;
+  {
+    float* acc = big_seg_lds + (threadIdx.x / kWave) * D1 * kWave + (threadIdx.x & (kWave - 1));
 #pragma unroll
-  for (int i = 0; i < D1; ++i) acc[i * kWave] = 0.f;
-  const int64_t C0 = a.C;
-  const int c_raw = blockIdx.y * L.lpe + L.cl;
-  const bool c_ok = c_raw < a.C;
-  const int c = min(c_raw, a.C - 1);
-  const int range = (int)wave * L.slots + L.slot;
-  const BigSegRange R(a.seg_ids, range, a.pos_per_wave, (int)a.n_rows);
+    for (int i = 0; i < D1; ++i) acc[i * kWave] = 0.f;
+    state[0] = -1;    // open segment
+    state[256] = 1;   // no segment of the range flushed yet
+  }
   const float* __restrict__ ps = a.ps;
-  const bool want_gx = a.gx != nullptr;
-  int cur = -1;
-  bool first = true;
-  BigSegIndex I(a, R, 0);
-  for (int k = 0; k < a.pos_per_wave; ++k) {
+  const int per = a.pos_per_wave, n_rows = (int)a.n_rows;
+  for (int k = 0; k <= per; ++k) {      // iteration `per` only closes the range
+    const int tid = opaque_lane();
+    const int lane = tid & (kWave - 1), wv = tid >> 6;
+    const int lpe = 1 << a.lpe_log2, slot = lane >> a.lpe_log2, cl = lane & (lpe - 1);
     const int64_t C = opaque_copy(a.C);
-    const bool live = R.p0 + k < R.p1;
-    const int sid = I.sid;
-    const int64_t e = I.edge, gr = I.other;
-    if (k + 1 < a.pos_per_wave) I = BigSegIndex(a, R, k + 1);   // in flight during this position's arithmetic
+    const int c_raw = blockIdx.y * lpe + cl;
+    const bool c_ok = c_raw < a.C;
+    const int c = min(c_raw, a.C - 1);
+    const int range = ((int)blockIdx.x * 4 + wv) * (kWave >> a.lpe_log2) + slot;
+    const int64_t b0 = (int64_t)range * per;
+    const int p0 = b0 < n_rows ? (int)b0 : n_rows;
+    const int p1 = b0 + per < n_rows ? (int)(b0 + per) : n_rows;
+    float* acc = big_seg_lds + wv * D1 * kWave + lane;
+    int* idx = idx_all + wv * kBigSegIndexInts;
+    const int cur = state[0];
+    const bool first = state[256] != 0;
+    if (k == per) {
+      if (cur >= 0 && a.gx) {
+        const bool first_complete = p0 == 0 || a.seg_ids[p0 - 1] != a.seg_ids[p0];
+        const bool last_complete = p1 == n_rows || a.seg_ids[p1 - 1] != a.seg_ids[p1];
+        big_seg_flush<D1>(acc, a.gx, a.ws, cur, range, first, (first ? first_complete : true) && last_complete, C, c,
+                          c_ok);
+      }
+      break;
+    }
+    const int kk = k & (lpe - 1);
+    if (kk == 0) {   // the same in every lane: stage the indices of the next lpe positions of every slot
+      const int q = p0 + k + cl;
+      const int qq = q < p1 ? q : (p1 > p0 ? p1 - 1 : 0);
+      idx[lane * 3 + 0] = (int)a.seg_ids[qq];
+      idx[lane * 3 + 1] = a.perm ? (int)a.perm[qq] : qq;
+      idx[lane * 3 + 2] = (int)a.gather[qq];
+      __builtin_amdgcn_wave_barrier();
+    }
+    const int ent = (slot * lpe + kk) * 3;
+    const int sid = idx[ent];
+    const int64_t e = idx[ent + 1], gr = idx[ent + 2];
+    const bool live = p0 + k < p1;
     if (live && sid != cur) {
       if (cur >= 0) {
-        if (want_gx)
-          big_seg_flush<D1>(acc, a.gx, a.ws, cur, range, first, first ? R.first_complete : true, C, c, c_ok);
-        first = false;
+        if (a.gx) {
+          const bool first_complete = p0 == 0 || a.seg_ids[p0 - 1] != a.seg_ids[p0];
+          big_seg_flush<D1>(acc, a.gx, a.ws, cur, range, first, first ? first_complete : true, C, c, c_ok);
+        }
+        state[256] = 0;
       }
-      cur = sid;
+      state[0] = sid;
     }
     float y[D2], gy[D2], g[DO];
 #pragma unroll
@@ -289,18 +337,15 @@ __global__ void __launch_bounds__(256, 2) uvu_big_seg_bwd_kernel(const UvuDev<fl
       float* gyrow = a.gy + e * D2;
 #pragma unroll
       for (int j = 0; j < D2; ++j) gy[j] *= keep;
-      group_sum_scatter<float, D2>(gy, L.lpe, [&](const auto& s) {   // lane cl ends up with components cl, cl + lpe, ...
+      group_sum_scatter<float, D2>(gy, lpe, [&](const auto& s) {   // lane cl ends up with components cl, cl + lpe, ...
 #pragma unroll
         for (int i = 0; i < array_len(s); ++i) {
-          const int j = i * L.lpe + L.cl;
+          const int j = i * lpe + cl;
           if (live && j < D2) gyrow[j] = s[i];
         }
       });
     }
   }
-  if (cur >= 0 && want_gx)
-    big_seg_flush<D1>(acc, a.gx, a.ws, cur, range, first, (first ? R.first_complete : true) && R.last_complete, C0, c,
-                      c_ok);
 }
 
 template <class TP, bool PS>

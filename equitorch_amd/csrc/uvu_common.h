@@ -79,7 +79,8 @@ struct UvuBigEntry {
   // the same with a channelled second operand, y (n_rows, D2, C) ("uuu"): grad_y is then per channel as well
   void (*fwd_yc)(const UvuDev<float>);
   void (*bwd_yc[2])(const UvuDev<float>, int64_t);
-  // segment mode (gather, product and segment sum fused); dynamic LDS: 4 x rows x 64 floats per workgroup
+  // segment mode (gather, product and segment sum fused); dynamic LDS: 4 x rows x 64 floats per workgroup, the
+  // backward 5120 bytes more (staged indices and per-lane state)
   void (*seg_fwd)(const UvuDev<float>, int64_t);
   void (*seg_bwd[2])(const UvuDev<float>, int64_t);
 };

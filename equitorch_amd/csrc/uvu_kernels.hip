@@ -854,7 +854,9 @@ static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward,
     const int rows = backward ? e.dims[0] : e.dims[2];
     if (plan.n_waves > 0) {
       void (*fn)(const UvuDev<float>, int64_t) = backward ? e.seg_bwd[a->grad_w ? kGwStore : kGwNone] : e.seg_fwd;
-      const size_t lds = (size_t)4 * rows * kWave * sizeof(float);
+      // accumulator rows of the four wavefronts; the backward also stages indices (64 x 3 ints per wavefront) and
+      // keeps two ints of state per lane there
+      const size_t lds = (size_t)4 * rows * kWave * sizeof(float) + (backward ? (4 * kWave * 3 + 256 * 2) * sizeof(int) : 0);
       if (lds > (size_t)kLdsBytes) return CGTP_ERR_LDS;
       if (lds > 48 * 1024 &&
           hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
