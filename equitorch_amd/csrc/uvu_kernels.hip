@@ -497,21 +497,32 @@ __global__ void __launch_bounds__(256, 2) uvu_seg_bwd_kernel(const UvuDev<T> a, 
 // answer lies near q * n_waves / n_rows: the wavefront looks at 64 consecutive entries around that guess with one
 // coalesced load (a binary search is eleven dependent loads at 2048 ranges, and this kernel does little else) and
 // falls back to the search when the window misses.
+// `first` receives the first position of the range found (from the window, not from another load).
 __device__ __forceinline__ int64_t range_of_position(const int64_t* __restrict__ wave_pos, int64_t n_waves, int per_wave,
-                                                     int64_t n_rows, int64_t q, int lane) {
-  if (!wave_pos) return q / per_wave;
+                                                     int64_t n_rows, int64_t q, int lane, int64_t* first) {
+  if (!wave_pos) {
+    const int64_t k = q / per_wave;
+    *first = k * per_wave;
+    return k;
+  }
   int64_t base = q * n_waves / n_rows - 32;
   if (base > n_waves - 63) base = n_waves - 63;
   if (base < 0) base = 0;
   const int64_t idx = base + lane;
-  const bool le = idx <= n_waves && wave_pos[idx] <= q;      // entries are ascending: a prefix of the lanes
+  const int64_t pos = idx <= n_waves ? wave_pos[idx] : INT64_MAX;
+  const bool le = pos <= q;                                   // entries are ascending: a prefix of the lanes
   const int cnt = __popcll(__ballot(le));
-  if (cnt > 0 && (cnt < kWave || base + kWave > n_waves)) return base + cnt - 1;
+  if (cnt > 0 && (cnt < kWave || base + kWave > n_waves)) {
+    // positions fit 32 bits in segment mode
+    *first = (int64_t)(unsigned)__shfl((int)pos, cnt - 1, kWave);
+    return base + cnt - 1;
+  }
   int64_t lo = 0, hi = n_waves - 1;   // largest k with wave_pos[k] <= q
   while (lo < hi) {
     const int64_t mid = (lo + hi + 1) >> 1;
     if (wave_pos[mid] <= q) lo = mid; else hi = mid - 1;
   }
+  *first = wave_pos[lo];
   return lo;
 }
 
@@ -530,11 +541,41 @@ __global__ void __launch_bounds__(256) uvu_fixup_kernel(T* __restrict__ rows, co
     for (int64_t i = lane; i < row_len; i += kWave) dst[i] = T(0);
     return;
   }
-  const int64_t ka = range_of_position(wave_pos, n_waves, per_wave, n_rows, b, lane);
-  const int64_t kb = range_of_position(wave_pos, n_waves, per_wave, n_rows, e - 1, lane);
+  int64_t first_a, first_b;
+  const int64_t ka = range_of_position(wave_pos, n_waves, per_wave, n_rows, b, lane, &first_a);
+  const int64_t kb = range_of_position(wave_pos, n_waves, per_wave, n_rows, e - 1, lane, &first_b);
   if (ka == kb) return;  // written in full by wavefront ka
-  const int64_t first_a = wave_pos ? wave_pos[ka] : ka * per_wave;
-  const int64_t slot_a = (b == first_a) ? 0 : 1;
+  const int slot_a = (b == first_a) ? 0 : 1;
+  // 16 bytes per lane and three groups of lanes' worth in flight: a row of 9 x 64 floats is one round trip
+  constexpr int N = 16 / sizeof(T);
+  const bool wide = row_len % N == 0 && ((reinterpret_cast<uintptr_t>(rows) | reinterpret_cast<uintptr_t>(ws)) & 15) == 0;
+  if (wide) {
+    constexpr int U = 3;
+    for (int64_t i0 = (int64_t)lane * N; i0 < row_len; i0 += (int64_t)U * kWave * N) {
+      T s[U][N];
+      const T* src = ws + (ka * 2 + slot_a) * row_len;
+      for (int64_t k = ka;;) {           // all loads of a partial row are issued before any is added
+        T t[U][N];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int64_t i = i0 + (int64_t)u * kWave * N;
+          load_vec<T, N>(t[u], src + (i < row_len ? i : i0));
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int n = 0; n < N; ++n) s[u][n] = k == ka ? t[u][n] : s[u][n] + t[u][n];
+        if (++k > kb) break;
+        src = ws + (k * 2) * row_len;
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t i = i0 + (int64_t)u * kWave * N;
+        if (i < row_len) store_vec<T, N>(dst + i, s[u]);
+      }
+    }
+    return;
+  }
   for (int64_t i = lane; i < row_len; i += kWave) {
     T s = ws[(ka * 2 + slot_a) * row_len + i];
     for (int64_t k = ka + 1; k <= kb; ++k) s += ws[(k * 2) * row_len + i];
