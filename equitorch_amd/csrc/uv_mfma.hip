@@ -174,10 +174,15 @@ __global__ void __launch_bounds__(256, 2) uv_gy_kernel(const __bf16* __restrict_
             g1[i] = (float)v[4 + i];
           }
         });
+    // the four lanes of a sample: all values of a stage are exchanged before any is added (one wait per stage
+    // instead of one per value); same operands per addition as value-by-value
 #pragma unroll
-    for (int j = 0; j < D2; ++j) {
-      part[j] += __shfl_xor(part[j], 16, kWave);
-      part[j] += __shfl_xor(part[j], 32, kWave);
+    for (int off = 16; off < kWave; off <<= 1) {
+      float t[D2];
+#pragma unroll
+      for (int j = 0; j < D2; ++j) t[j] = lane_exchange(part[j], (lane ^ off) << 2);
+#pragma unroll
+      for (int j = 0; j < D2; ++j) part[j] += t[j];
     }
   }
   __syncthreads();  // every wavefront is done with the staged rows; reuse the front of LDS for the partial sums
