@@ -45,7 +45,9 @@ __device__ __forceinline__ int64_t seg_wave_index(int64_t n_waves) {
   const int64_t per_xcd = (blocks + 7) / 8;
   const int64_t block = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if ((int64_t)(blockIdx.x >> 3) >= per_xcd || block >= blocks) return -1;
-  const int64_t wave = block * waves_per_block + threadIdx.x / kWave;
+  // the wavefront's number within the workgroup as a scalar: everything derived from it (range, segment ids,
+  // flags) then lives in scalar registers
+  const int64_t wave = block * waves_per_block + __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
   return wave < n_waves ? wave : -1;
 }
 

@@ -264,7 +264,7 @@ __device__ __forceinline__ bool seg_step_begin(SegStep& st, T (&acc)[D][V], T* _
   const int sid = __shfl(I.sid, src, kWave);
   edge = __shfl(I.edge, src, kWave);
   other = __shfl(I.other, src, kWave);
-  const int lead = __shfl(I.sid, off0, kWave);
+  const int lead = __builtin_amdgcn_readlane(I.sid, off0);   // off0 is the same in every lane: a scalar read, no wait
   if (lead != st.cur) {
     if (st.cur >= 0)
       flush_segment<T, D, V>(st, acc, final_rows, ws, wave, st.first ? R.first_complete : true, R, L, cok, C, c0);
