@@ -100,11 +100,12 @@ def test_edge_fused_small(device, shared_w):
         assert_close(g, r, 1e-5, f"edge fused shared={shared_w} {name}")
 
 
-@pytest.mark.parametrize("pos_per_wave", [4, 8, 32, 60])
+@pytest.mark.parametrize("pos_per_wave,ch", [(4, 32), (8, 32), (32, 32), (60, 32), (8, 7), (12, 18), (8, 64)])
 @pytest.mark.parametrize("hub", [False, True])
-def test_edge_fused_range_modes(device, pos_per_wave, hub):
+def test_edge_fused_range_modes(device, pos_per_wave, ch, hub):
     """Ranges cut by position (partial rows + fix-up kernel) must give the same rows as segment-aligned ranges,
-    including with a hub node whose segment spans many wavefronts and with empty segments."""
+    including with a hub node whose segment spans many wavefronts and with empty segments.  7 and 18 channels: rows
+    whose length is no multiple of four, which the fix-up kernel adds element by element."""
     from equitorch_amd.nn.functional import EdgePlan
     from equitorch_amd.ops import kernels
     irreps = SH[2]
@@ -112,7 +113,7 @@ def test_edge_fused_range_modes(device, pos_per_wave, hub):
     cfg = kernels.uvu_config_of(mod.tp_info_forward)
     dims = kernels.uvu_dims(cfg)
     gen = torch.Generator().manual_seed(9)
-    n_nodes, n_edges, ch = 61, 900, 32
+    n_nodes, n_edges = 61, 900
     src = torch.randint(0, n_nodes, (n_edges,), generator=gen)
     dst = torch.randint(0, n_nodes, (n_edges,), generator=gen)
     if hub:
@@ -132,7 +133,7 @@ def test_edge_fused_range_modes(device, pos_per_wave, hub):
     gx, gy, gw = kernels.uvu_backward(cfg, dims, xd, shd, wd, ctd, (True, True, True), seg=plan.bwd_index,
                                       pos_per_wave=pos_per_wave)
     for name, g, r in zip(("out", "grad_x", "grad_sh", "grad_w"), (out, gx, gy, gw), (ref_out, *ref_grads)):
-        assert_close(g, r, 1e-5, f"ppw={pos_per_wave} hub={hub} {name}")
+        assert_close(g, r, 1e-5, f"ppw={pos_per_wave} C={ch} hub={hub} {name}")
     if not hub:
         assert plan.fwd_index.wave_seg is not None
     out_a = kernels.uvu_forward(cfg, dims, xd, shd, wd, seg=plan.fwd_index)
@@ -338,8 +339,8 @@ def test_uuu_on_the_block_wise_kernels(device, lmax, channels, shared_w):
 
 @pytest.mark.parametrize("hub", [False, True])
 def test_edge_large_table_hub_and_shared_weight(device, hub):
-    """lmax = 4, C = 48 (no fused kernels: gathered row-mode launches plus segment sums), with and without a hub node
-    and with per-edge and shared weights, against the dense oracle."""
+    """lmax = 4, C = 48 on the block-wise kernels, with and without a hub node: per-edge weights take the fused segment
+    mode, a shared weight the gathered row-mode launches plus segment sums; both against the dense oracle."""
     from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu
     irr = "0e+1o+2e+3o+4e"
     mod = _module(irr, irr, irr).to(device)
