@@ -45,6 +45,53 @@ def profiled_traffic(workload):
     return None, "no counter run on record"
 
 
+def measured_traffic(workload):
+    """HBM bytes per launch of the dominant kernel, measured now: this script is run four times as a child process
+    under ``rocprofv3 --pmc`` (one counter per run: FETCH_SIZE, WRITE_SIZE; the workload with a few steps, and the
+    streaming copy of 1 GiB whose true traffic is known and gives the scale of each counter).  The backward's figure
+    includes its fix-up kernel.  Returns (bytes or None, description)."""
+    import csv, glob, shutil, subprocess, tempfile
+    if shutil.which("rocprofv3") is None:
+        return None, "rocprofv3 not found"
+    me = os.path.abspath(__file__)
+    runs = {"work": ["--workload", workload, "--no-cpu-baseline", "--no-configs", "--no-measure-traffic", "--steps", "5",
+                     "--warmup", "2", "--kernel-reps", "5"],
+            "copy": ["--workload", "copy", "--steps", "5", "--warmup", "2"]}
+    env = dict(os.environ, TMPDIR="/tmp")
+    raw = {}
+    out_dir = tempfile.mkdtemp(prefix="cgtp_pmc_", dir="/tmp")
+    try:
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            for tag, extra in runs.items():
+                d = os.path.join(out_dir, f"{counter}_{tag}")
+                cmd = ["timeout", "-s", "KILL", "90", "rocprofv3", "--pmc", counter, "--output-format", "csv",
+                       "-d", d, "-o", "t", "--", "python3", me, *extra]
+                res = subprocess.run(cmd, cwd="/tmp", env=env, capture_output=True, text=True)
+                files = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)
+                if res.returncode != 0 or not files:
+                    return None, f"counter run failed ({counter}, {tag}, exit {res.returncode})"
+                acc = {}
+                with open(files[0]) as f:
+                    for row in csv.DictReader(f):
+                        if row["Counter_Name"] != counter:
+                            continue
+                        for key in ("uvu_seg_bwd_kernel", "uvu_seg_fwd_kernel", "uvu_fixup_kernel", "copy_kernel"):
+                            if key in row["Kernel_Name"]:
+                                acc.setdefault(key, []).append(float(row["Counter_Value"]))
+                raw[(counter, tag)] = {k: sum(v) / len(v) for k, v in acc.items()}
+    finally:
+        shutil.rmtree(out_dir, ignore_errors=True)
+    try:
+        gib_kib = float(1 << 20)                                   # the copy kernel reads and writes 1 GiB
+        scale = {c: gib_kib / raw[(c, "copy")]["copy_kernel"] for c in ("FETCH_SIZE", "WRITE_SIZE")}
+        names = ["uvu_seg_bwd_kernel", "uvu_fixup_kernel"] if workload == "edge_fwd_bwd" else ["uvu_seg_fwd_kernel"]
+        kib = sum(raw[(c, "work")].get(n, 0.0) * scale[c] for c in scale for n in names)
+    except (KeyError, ZeroDivisionError):
+        return None, "counter run gave no rows for the kernels"
+    return int(kib * 1024), ("measured by this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE in child processes, scaled by "
+                             f"the copy kernel (x{scale['FETCH_SIZE']:.3f} / x{scale['WRITE_SIZE']:.3f})")
+
+
 WORKLOADS = {
     # name: (lmax, channels, nodes, edges)
     "edge_fwd_bwd": (2, 64, 4096, 65536),
@@ -811,6 +858,9 @@ def main():
     ap.add_argument("--pos-per-wave", type=int, default=0,
                     help="sorted positions per wavefront in the per-kernel timing (0 = library default)")
     ap.add_argument("--kernel-reps", type=int, default=100, help="launches per kernel for the roofline timing")
+    ap.add_argument("--no-measure-traffic", action="store_true",
+                    help="edge workloads: take roofline.traffic from the committed profile summary instead of measuring "
+                         "it now with four short child runs under rocprofv3 --pmc (10-20 s)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on exactly one GPU (the path has no multi-GPU part); use --gpus 1",
@@ -949,6 +999,15 @@ def main():
         dom, dom_bytes, dom_ms = "cgtp::uvu_seg_fwd_kernel<TP_sh2,float,4>", fwd_bytes, fwd_avg
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
     traffic, traffic_source = profiled_traffic(args.workload) if args.graph == "uniform" else (None, "not profiled")
+    # measured now unless told otherwise, or unless this process itself runs under a profiler (its children would be
+    # profiled twice)
+    profiled = any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ) or "rocprof" in os.environ.get("LD_PRELOAD", "")
+    if not args.no_measure_traffic and not profiled and args.graph == "uniform":
+        live, live_source = measured_traffic(args.workload)
+        if live is not None:
+            traffic, traffic_source = live, live_source
+        else:
+            traffic_source += f" (live measurement unavailable: {live_source})"
 
     rec = {
         "metric": "edge-TP fwd+bwd Medges/s (lmax=2,C=64)" if backward else "edge-TP fwd Medges/s (lmax=2,C=64)",
