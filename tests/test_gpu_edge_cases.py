@@ -153,3 +153,50 @@ def test_converted_module_runs_on_the_compiled_kernels(device):
     # the channel-wise product of a float16 module finds its compiled table as well
     half = enn.SO3Linear("0e+1o+2e", "0e+1o+2e", "0e+1o+2e", c, c, feature_mode="uu").to(device).half()
     assert kernels.uvu_config_of(half.tp_info_forward) >= 0
+
+
+def test_baseline_configurations_take_their_kernels(device, monkeypatch):
+    """The five benchmark configurations, at small sizes, must reach the kernels written for them: the fused segment
+    kernels for the edge products (lmax = 2 and lmax = 6), the compiled channel-wise kernel for the row product with a
+    shared weight, the bf16 matrix-core kernel for the fully connected product."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu
+    from equitorch_amd.ops import kernels
+    from equitorch_amd.utils._sh import spherical_harmonics
+    seen = []
+    monkeypatch.setattr(kernels, "log_tier", lambda op, tier, detail="": seen.append((op, tier)))
+    g = torch.Generator().manual_seed(3)
+
+    def irreps(lmax):
+        return "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+
+    def unit(n):
+        v = torch.randn(n, 3, generator=g)
+        return v / v.norm(dim=1, keepdim=True)
+    # configs 1-2 (lmax = 2, C = 64) and 4 (lmax = 6, C = 32): per-edge weights on a graph
+    for lmax, ch in ((2, 64), (6, 32)):
+        irr, d = irreps(lmax), (lmax + 1) ** 2
+        mod = SO3Linear(irr, irr, irr, ch, ch, internal_weights=False, feature_mode="uu").to(device)
+        n_nodes, n_edges = 50, 400
+        plan = EdgePlan(torch.randint(0, n_nodes, (n_edges,), generator=g).to(device),
+                        torch.randint(0, n_nodes, (n_edges,), generator=g).to(device), n_nodes)
+        x = torch.randn(n_nodes, d, ch, generator=g).to(device).requires_grad_(True)
+        sh = spherical_harmonics(unit(n_edges), lmax).to(device)
+        w = torch.randn(n_edges, mod.num_paths, ch, generator=g).to(device)
+        edge_tensor_product_uu(x, sh, w, plan, mod.tp_info_forward).sum().backward()
+        assert seen[-1] == ("edge_tensor_product_uu", "fused gather / product / segment sum"), (lmax, seen)
+    # config 0: B = 1024, C = 16, shared weight
+    irr = irreps(2)
+    mod = SO3Linear(irr, irr, irr, 16, 16, internal_weights=False, feature_mode="uu").to(device)
+    x = torch.randn(1024, 9, 16, generator=g).to(device)
+    mod(x, spherical_harmonics(unit(1024), 2).to(device), torch.randn(mod.num_paths, 16, generator=g).to(device))
+    assert seen[-1] == ("tensor_product_u1u", "compiled table"), seen
+    # config 3: bf16, 128 -> 128 channels, lmax = 3, shared weight
+    irr = irreps(3)
+    mod = SO3Linear(irr, irr, irr, 128, 128, internal_weights=False, feature_mode="uv").to(device)
+    x = torch.randn(256, 16, 128, generator=g).to(device).bfloat16()
+    y = spherical_harmonics(unit(256), 3).to(device).bfloat16()
+    w = (torch.randn(mod.num_paths, 128, 128, generator=g) / 40).to(device).bfloat16()
+    mod(x, y, w)
+    assert seen[-1] == ("tensor_product_u1v", "matrix-core kernel (compiled table)"), seen
