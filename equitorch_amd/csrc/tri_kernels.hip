@@ -314,36 +314,37 @@ __global__ void __launch_bounds__(256) segment_sum_kernel(const T* __restrict__ 
   const int64_t c = ((wave % chunks) * kWave + lane) * V;
   const int64_t n = row / out_size, m = row % out_size;
   const int64_t tb = seg ? seg[m] : m, te = seg ? seg[m + 1] : m + 1;
-  const T* base = in + n * in_size * C + c;
+  const T* base = in + n * in_size * C + (c < C ? c : 0);
   const bool ok = c < C;
   T acc[V];
 #pragma unroll
   for (int v = 0; v < V; ++v) acc[v] = T(0);
-  int64_t t0 = tb;
-  for (; t0 + U <= te; t0 += U) {
-    int64_t idx[U];
-    T sc[U];
+  // Terms four at a time.  The positions and scales of the next four are requested while the rows of these four are
+  // on their way (a group then costs one round trip to memory, not two), and a last group of one to three terms
+  // takes the same path with its missing terms pointed at the last one and left out of the sum.  Additions in
+  // position order, whatever the launch shape.
+  auto fetch = [&](int64_t t0, int64_t (&idx)[U], T (&sc)[U]) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      idx[u] = index ? index[t0 + u] : t0 + u;
-      sc[u] = scale ? scale[t0 + u] : T(1);
+      const int64_t t = t0 + u < te ? t0 + u : te - 1;
+      idx[u] = index ? index[t] : t;
+      sc[u] = scale ? scale[t] : T(1);
     }
+  };
+  int64_t idx[U];
+  T sc[U];
+  if (tb < te) fetch(tb, idx, sc);
+  for (int64_t t0 = tb; t0 < te; t0 += U) {
     T x[U][V];
-    if (ok) {
 #pragma unroll
-      for (int u = 0; u < U; ++u) load_vec<T, V>(x[u], base + idx[u] * C);
+    for (int u = 0; u < U; ++u) load_vec<T, V>(x[u], base + idx[u] * C);
+    T scn[U];
 #pragma unroll
-      for (int u = 0; u < U; ++u) fmav<T, V>(acc, sc[u], x[u]);
-    }
-  }
-  for (; t0 < te; ++t0) {
-    const int64_t i = index ? index[t0] : t0;
-    const T sc = scale ? scale[t0] : T(1);
-    if (ok) {
-      T x[V];
-      load_vec<T, V>(x, base + i * C);
-      fmav<T, V>(acc, sc, x);
-    }
+    for (int u = 0; u < U; ++u) scn[u] = sc[u];
+    if (t0 + U < te) fetch(t0 + U, idx, sc);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (t0 + u < te) fmav<T, V>(acc, scn[u], x[u]);     // the same in every lane
   }
   if (ok) store_vec<T, V>(out + (n * out_size + m) * C + c, acc);
 }
