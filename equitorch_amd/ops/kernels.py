@@ -543,6 +543,9 @@ def _workspace(a: UvuArgs, backward: int, device):
     return ws
 
 
+_LAUNCHABLE = {}
+
+
 def uvu_launchable(cfg: int, x: Tensor, y: Tensor, w: Tensor, segments: bool = False, gathered: bool = False,
                    y_vec: int = 0) -> bool:
     """True when both the specialised forward and backward accept these operands (dtype, channel count,
@@ -550,6 +553,13 @@ def uvu_launchable(cfg: int, x: Tensor, y: Tensor, w: Tensor, segments: bool = F
     of ``x`` picked by an index."""
     if x.shape[0] == 0 or y.shape[0] == 0:
         return False
+    # the answer depends on these only (pointers enter through their 16-byte alignment)
+    key = (int(cfg), x.dtype, x.shape[-1], w.ndim, y.ndim, segments, gathered, y_vec,
+           x.data_ptr() % 16, y.data_ptr() % 16, w.data_ptr() % 16, x.shape[0] == y.shape[0],
+           max(x.shape[0], y.shape[0]) >= 1 << 31)
+    hit = _LAUNCHABLE.get(key)
+    if hit is not None:
+        return hit
     a = UvuArgs()
     a.cfg, a.dtype, a.C = cfg, _lib.dtype_code(x.dtype), x.shape[-1]
     a.w_shared = int(w.ndim == 2)
@@ -564,7 +574,10 @@ def uvu_launchable(cfg: int, x: Tensor, y: Tensor, w: Tensor, segments: bool = F
         a.gather = a.x_gather = dummy
     a.x, a.y, a.w = x.data_ptr() or dummy, y.data_ptr() or dummy, w.data_ptr() or dummy
     a.out = a.grad_out = a.grad_x = a.grad_y = a.grad_w = dummy
-    return _lib.lib.cgtp_uvu_validate(C.byref(a), 1) == 0
+    ok = _lib.lib.cgtp_uvu_validate(C.byref(a), 1) == 0
+    if len(_LAUNCHABLE) < 4096:
+        _LAUNCHABLE[key] = ok
+    return ok
 
 
 Y_HARMONICS, Y_UNIT_VECTOR, Y_RAW_VECTOR = 0, 1, 2
