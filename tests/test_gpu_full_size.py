@@ -248,3 +248,44 @@ def test_edge_radial_full_size(device):
         o = edge_tensor_product_uu_radial(xd.detach(), shd[lo:hi].detach(), hd[lo:hi].detach(), ws, pl, mod.tp_info_forward)
         parts.append(torch.autograd.grad(o, (ws,), ct.to(device))[0].double())
     assert_close(gwl.double(), parts[0] + parts[1], 1e-5, "radial full size grad_w_last additivity", norm="max")
+
+
+@pytest.mark.parametrize("lmax,ch,n_nodes,n_edges", [(2, 64, 100_000, 3_200_000), (6, 32, 50_000, 700_000)])
+def test_edge_kernels_past_two_to_the_31_weight_elements(device, lmax, ch, n_nodes, n_edges):
+    """3.2 million edges x 11 paths x 64 channels = 2.25e9 weight elements (9 GB; its gradient as much), and 700 000
+    edges x 106 paths x 32 channels at lmax = 6: every element offset past 2^31 must be formed in 64 bits.  No oracle at this size: the fused segment kernels (forward and all
+    gradients) against the row-mode kernels followed by segment sums, which share no addressing code with them;
+    1e-5 of the tensor's scale (the two paths add in different orders)."""
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import EdgePlan
+    from equitorch_amd.ops import kernels
+    if torch.cuda.get_device_properties(0).total_memory < 80 * 2 ** 30:
+        pytest.skip("needs about 50 GB of device memory")
+    irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+    d = (lmax + 1) ** 2
+    mod = SO3Linear(irreps, irreps, irreps, ch, ch, internal_weights=False, feature_mode="uu").to(device)
+    g = torch.Generator(device=device).manual_seed(1)
+    src = torch.randint(0, n_nodes, (n_edges,), generator=g, device=device)
+    dst = torch.randint(0, n_nodes, (n_edges,), generator=g, device=device)
+    plan = EdgePlan(src, dst, n_nodes)
+    x = torch.randn(n_nodes, d, ch, generator=g, device=device)
+    sh = torch.randn(n_edges, d, generator=g, device=device)
+    w = torch.randn(n_edges, mod.num_paths, ch, generator=g, device=device)
+    ct = torch.randn(n_nodes, d, ch, generator=g, device=device)
+    assert w.numel() > 2 ** 31
+    cfg = kernels.uvu_config_of(mod.tp_info_forward)
+    dims = kernels.uvu_dims(cfg)
+    out = kernels.uvu_forward(cfg, dims, x, sh, w, seg=plan.fwd_index)
+    gx, gy, gw = kernels.uvu_backward(cfg, dims, x, sh, w, ct, (True, True, True), seg=plan.bwd_index)
+    msg = kernels.uvu_forward(cfg, dims, x, sh, w, gather=plan.src)
+    out2 = kernels.segment_sum(msg.view(1, n_edges, -1), None, plan.perm_dst, plan.ptr_dst, n_nodes).view(n_nodes, d, ch)
+    del msg
+    gxe, gy2, gw2 = kernels.uvu_backward(cfg, dims, x, sh, w, ct, (True, True, True), gather=plan.dst,
+                                         x_gather=plan.src)
+    gx2 = kernels.segment_sum(gxe.view(1, n_edges, -1), None, plan.perm_src, plan.ptr_src, n_nodes).view(n_nodes, d, ch)
+    del gxe
+    for name, a, b in (("out", out, out2), ("grad_x", gx, gx2), ("grad_sh", gy, gy2), ("grad_w", gw, gw2)):
+        scale = max(1.0, b.abs().max().item())
+        assert (a - b).abs().max().item() <= 1e-5 * scale, name
+    del out, out2, gx, gx2, gy, gy2, gw, gw2, w, sh
+    torch.cuda.empty_cache()
