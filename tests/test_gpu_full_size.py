@@ -289,3 +289,41 @@ def test_edge_kernels_past_two_to_the_31_weight_elements(device, lmax, ch, n_nod
         assert (a - b).abs().max().item() <= 1e-5 * scale, name
     del out, out2, gx, gx2, gy, gy2, gw, gw2, w, sh
     torch.cuda.empty_cache()
+
+
+def test_fully_connected_bf16_past_two_to_the_31_elements(device):
+    """1.2 million samples x 16 x 128 bf16 = 2.46e9 elements per operand: rows at both ends of the batch (the last ones
+    lie past 2^31 elements) must come out bit-equal to the same rows computed as a small batch of their own (a row's
+    result depends on nothing else), for the output and the gradients of both per-sample operands; the weight
+    gradient, a sum over all samples, must be the sum over the two halves of the batch (rel 1e-2, bf16)."""
+    from equitorch_amd.nn import SO3Linear
+    if torch.cuda.get_device_properties(0).total_memory < 80 * 2 ** 30:
+        pytest.skip("needs about 40 GB of device memory")
+    irreps, ch, n = "0e+1o+2e+3o", 128, 1_200_000
+    mod = SO3Linear(irreps, irreps, irreps, ch, ch, internal_weights=False, feature_mode="uv").to(device)
+    g = torch.Generator(device=device).manual_seed(2)
+    x = torch.randn(n, 16, ch, generator=g, device=device).bfloat16().requires_grad_(True)
+    y = torch.randn(n, 16, generator=g, device=device).bfloat16().requires_grad_(True)
+    w = (torch.randn(mod.num_paths, ch, ch, generator=g, device=device) / 40).bfloat16().requires_grad_(True)
+    ct = torch.randn(n, 16, ch, generator=g, device=device).bfloat16()
+    assert x.numel() > 2 ** 31
+    out = mod(x, y, w)
+    gx, gy, gw = torch.autograd.grad(out, (x, y, w), ct)
+    idx = torch.cat([torch.arange(0, 64, device=device), torch.arange(n - 1100, n - 1000, device=device),
+                     torch.arange(n - 64, n, device=device)])
+    xs, ys = (t.detach()[idx].clone().requires_grad_(True) for t in (x, y))
+    gxs, gys, _ = torch.autograd.grad(mod(xs, ys, w), (xs, ys, w), ct[idx])
+    assert torch.equal(out[idx], mod(xs, ys, w)), "out"
+    assert torch.equal(gx[idx], gxs), "grad_x"
+    assert torch.equal(gy[idx], gys), "grad_sh"
+    del out, gx, gy
+    half = n // 2
+    parts = []
+    for lo, hi in ((0, half), (half, n)):
+        xh, yh = x.detach()[lo:hi], y.detach()[lo:hi]
+        (gwh,) = torch.autograd.grad(mod(xh, yh, w), (w,), ct[lo:hi])
+        parts.append(gwh.float())
+    ref = parts[0] + parts[1]
+    assert (gw.float() - ref).abs().max().item() <= 1e-2 * ref.abs().max().item(), "grad_w"
+    del x, y, ct
+    torch.cuda.empty_cache()
