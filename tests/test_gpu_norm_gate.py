@@ -253,3 +253,35 @@ def test_layer_rms_second_order_and_fallback(device):
     xb = torch.randn(5, 16, 8, generator=g, dtype=torch.float64)
     ref = ref_ops.cpu_layer_rms_norm(xb, ref_tables.irreps_info("0e+7o"), None)
     assert_close(layer_rms_norm(xb.to(device), big, None), ref, tol=1e-6, what="composed path")
+
+
+def test_rows_past_two_to_the_31_elements(device):
+    """3.8 million rows x 9 x 64 fp32 = 2.19e9 elements: gate, layer norm and squared norm, forward and gradients.
+    A row's result depends on its own row only, so rows from both ends of the batch (the last ones lie past 2^31
+    elements) must be bit-equal to the same rows computed as a batch of their own."""
+    from equitorch_amd.nn import Gate, LayerRMSNorm, SquaredNorm
+    if torch.cuda.get_device_properties(0).total_memory < 80 * 2 ** 30:
+        pytest.skip("needs about 50 GB of device memory")
+    n, ch = 3_800_000, 64
+    g = torch.Generator(device=device).manual_seed(3)
+    x = torch.randn(n, 9, ch, generator=g, device=device).requires_grad_(True)
+    assert x.numel() > 2 ** 31
+    gate = torch.randn(n, 3, ch, generator=g, device=device).requires_grad_(True)
+    ct = torch.randn(n, 9, ch, generator=g, device=device)
+    idx = torch.cat([torch.arange(0, 50, device=device), torch.arange(n - 2000, n - 1950, device=device),
+                     torch.arange(n - 50, n, device=device)])
+
+    def check(name, fn, inputs, cot):
+        out = fn(*inputs)
+        grads = torch.autograd.grad(out, inputs, cot)
+        small = [t.detach()[idx].clone().requires_grad_(True) for t in inputs]
+        outs = fn(*small)
+        gs = torch.autograd.grad(outs, small, cot[idx])
+        assert torch.equal(out[idx], outs), name
+        for a, b in zip(grads, gs):
+            assert torch.equal(a[idx], b), name
+    check("gate", Gate("0e+1o+2e").to(device), (x, gate), ct)
+    check("layer rms norm", LayerRMSNorm("0e+1o+2e", ch).to(device), (x,), ct)
+    check("squared norm", SquaredNorm("0e+1o+2e", True).to(device), (x,), torch.randn(n, 3, ch, generator=g, device=device))
+    del x, gate, ct
+    torch.cuda.empty_cache()
