@@ -166,3 +166,28 @@ def test_add_spherical_harmonics_transform(device):
     assert_close(out.edge_norm, v.norm(dim=-1), tol=1e-12, what="edge_norm")
     scaled = AddSphericalHarmonics(2, sh_attr="y", integral_normalize=True)(data)
     assert_close(scaled.y, ref_sh.spherical_harmonics(v, 2) / math.sqrt(4 * math.pi), tol=1e-12, what="scaled")
+
+
+def test_harmonics_past_two_to_the_31_elements(device):
+    """44 million vectors x 49 components (lmax = 6) = 2.16e9 output elements: the first and the last thousand rows and
+    their gradients must be bit-equal to the same vectors evaluated as a batch of their own."""
+    from equitorch_amd.nn import SphericalHarmonics
+    if torch.cuda.get_device_properties(0).total_memory < 80 * 2 ** 30:
+        pytest.skip("needs about 30 GB of device memory")
+    n = 44_000_000
+    g = torch.Generator(device=device).manual_seed(4)
+    v = torch.randn(n, 3, generator=g, device=device).requires_grad_(True)
+    sh = SphericalHarmonics(6).to(device)
+    out = sh(v)
+    assert out.numel() > 2 ** 31
+    idx = torch.cat([torch.arange(0, 1000, device=device), torch.arange(n - 1000, n, device=device)])
+    ct = torch.randn(2000, 49, generator=g, device=device)
+    full_ct = torch.zeros_like(out)
+    full_ct[idx] = ct
+    (gv,) = torch.autograd.grad(out, v, full_ct)
+    vs = v.detach()[idx].clone().requires_grad_(True)
+    outs = sh(vs)
+    (gvs,) = torch.autograd.grad(outs, vs, ct)
+    assert torch.equal(out[idx], outs) and torch.equal(gv[idx], gvs)
+    del out, full_ct, gv, v
+    torch.cuda.empty_cache()

@@ -191,3 +191,36 @@ def test_u1v_fp32_full_size_properties(device):
         parts.append(gp.double())
     # a sum of 32768 x 16 products per element, in chunks: rounding of the three results bounds the difference
     assert_close(gw.double(), parts[0] + parts[1], 1e-5, "u1v fp32 full size grad_w additivity", norm="max")
+
+
+def test_fp32_fully_connected_past_two_to_the_31_elements(device):
+    """1.1 million samples x 16 x 128 fp32 = 2.25e9 elements per operand on the table-driven matrix-core kernels: rows
+    at both ends of the batch against the same rows as a batch of their own (1e-5), the weight gradient against the
+    sum over the two halves of the batch (1e-4 norm-wise: sums of a million terms in different groupings)."""
+    from equitorch_amd.nn import SO3Linear
+    if torch.cuda.get_device_properties(0).total_memory < 80 * 2 ** 30:
+        pytest.skip("needs about 50 GB of device memory")
+    n, ch, irreps = 1_100_000, 128, "0e+1o+2e+3o"
+    mod = SO3Linear(irreps, irreps, irreps, ch, ch, internal_weights=False, feature_mode="uv").to(device)
+    g = torch.Generator(device=device).manual_seed(5)
+    x = torch.randn(n, 16, ch, generator=g, device=device).requires_grad_(True)
+    y = torch.randn(n, 16, generator=g, device=device).requires_grad_(True)
+    w = (torch.randn(mod.num_paths, ch, ch, generator=g, device=device) / 40).requires_grad_(True)
+    ct = torch.randn(n, 16, ch, generator=g, device=device)
+    assert x.numel() > 2 ** 31
+    out = mod(x, y, w)
+    gx, gy, gw = torch.autograd.grad(out, (x, y, w), ct)
+    idx = torch.cat([torch.arange(0, 64, device=device), torch.arange(n - 64, n, device=device)])
+    xs, ys = (t.detach()[idx].clone().requires_grad_(True) for t in (x, y))
+    outs = mod(xs, ys, w)
+    gxs, gys, _ = torch.autograd.grad(outs, (xs, ys, w), ct[idx])
+    for name, a, b in (("out", out[idx], outs), ("grad_x", gx[idx], gxs), ("grad_sh", gy[idx], gys)):
+        assert (a - b).abs().max().item() <= 1e-5 * max(1.0, b.abs().max().item()), name
+    del out, gx, gy
+    half = n // 2
+    parts = [torch.autograd.grad(mod(x.detach()[lo:hi], y.detach()[lo:hi], w), (w,), ct[lo:hi])[0]
+             for lo, hi in ((0, half), (half, n))]
+    ref = parts[0] + parts[1]
+    assert (gw - ref).abs().max().item() <= 1e-4 * ref.abs().max().item(), "grad_w"
+    del x, y, ct
+    torch.cuda.empty_cache()
