@@ -285,3 +285,41 @@ def test_rows_past_two_to_the_31_elements(device):
     check("squared norm", SquaredNorm("0e+1o+2e", True).to(device), (x,), torch.randn(n, 3, ch, generator=g, device=device))
     del x, gate, ct
     torch.cuda.empty_cache()
+
+
+def test_node_layers_past_two_to_the_31_elements(device):
+    """The same check (rows at both ends of 3.8 million rows x 9 x 64 fp32 bit-equal to the same rows as a batch of their
+    own, forward and input gradient) for the fused Wigner rotation, the channel-wise SO(2) map, the irrep-wise linear
+    layer and the batch norm in evaluation mode."""
+    import math
+    import equitorch_amd.nn as enn
+    from equitorch_amd.nn.functional import sincos
+    if torch.cuda.get_device_properties(0).total_memory < 80 * 2 ** 30:
+        pytest.skip("needs about 50 GB of device memory")
+    irr, n, ch = "0e+1o+2e", 3_800_000, 64
+    g = torch.Generator(device=device).manual_seed(6)
+    x = torch.randn(n, 9, ch, generator=g, device=device).requires_grad_(True)
+    ct = torch.randn(n, 9, ch, generator=g, device=device)
+    assert x.numel() > 2 ** 31
+    idx = torch.cat([torch.arange(0, 50, device=device), torch.arange(n - 50, n, device=device)])
+
+    def check(name, fn):
+        out = fn(x, slice(None))
+        (gx,) = torch.autograd.grad(out, x, ct)
+        xs = x.detach()[idx].clone().requires_grad_(True)
+        outs = fn(xs, idx)
+        (gxs,) = torch.autograd.grad(outs, xs, ct[idx])
+        assert torch.equal(out[idx], outs) and torch.equal(gx[idx], gxs), name
+        del out, gx
+        torch.cuda.empty_cache()
+    sc = [sincos(torch.rand(n, generator=g, device=device) * 2 * math.pi, 2) for _ in range(3)]
+    rot = enn.SparseWignerRotation(irr).to(device)
+    check("rotation", lambda t, i: rot(t, *(s[i] for s in sc)))
+    so2 = enn.SO2Linear(irr, irr, ch, ch, feature_mode="uu").to(device)
+    check("so2 uu", lambda t, i: so2(t))
+    lin = enn.IrrepsLinear(irr, irr, ch, ch).to(device)
+    check("irreps linear", lambda t, i: lin(t))
+    bn = enn.BatchRMSNorm(irr, ch).to(device).eval()
+    check("batch rms norm (eval)", lambda t, i: bn(t))
+    del x, ct
+    torch.cuda.empty_cache()
