@@ -84,3 +84,36 @@ def test_radial_with_other_normalisation_and_fallback(device):
                            ("grad_h", hd.grad, hr.grad), ("grad_w_last", wd.grad, wr.grad)):
             assert_close(a, b, tol=1e-5, what=f"radial path_norm=False R={r} {name}",
                          norm="max" if name in ("grad_h", "grad_w_last") else "element")
+
+
+def test_weights_formed_in_the_kernel_at_3_2_million_edges(device):
+    """3.2 million edges (the weight tensor that is never formed would have 2.25e9 elements; the per-edge weight
+    gradient, which is written, has): harmonics and weights both produced inside the edge kernels, all five gradients,
+    against the composition harmonics kernel -> matrix product -> plain fused edge product.  1e-4 of each tensor's
+    scale (sums over 32 to 3.2 million terms in different orders)."""
+    from equitorch_amd.nn import SO3Linear, SphericalHarmonics
+    from equitorch_amd.nn.functional import (EdgePlan, edge_tensor_product_uu, edge_tensor_product_uu_radial)
+    if torch.cuda.get_device_properties(0).total_memory < 80 * 2 ** 30:
+        pytest.skip("needs about 60 GB of device memory")
+    irreps, ch, n_nodes, n_edges, r = "0e+1o+2e", 64, 100_000, 3_200_000, 16
+    mod = SO3Linear(irreps, irreps, irreps, ch, ch, internal_weights=False, feature_mode="uu").to(device)
+    g = torch.Generator(device=device).manual_seed(7)
+    src = torch.randint(0, n_nodes, (n_edges,), generator=g, device=device)
+    dst = torch.randint(0, n_nodes, (n_edges,), generator=g, device=device)
+    plan = EdgePlan(src, dst, n_nodes)
+    x = torch.randn(n_nodes, 9, ch, generator=g, device=device).requires_grad_(True)
+    vec = torch.randn(n_edges, 3, generator=g, device=device).requires_grad_(True)
+    h = torch.randn(n_edges, r, generator=g, device=device).requires_grad_(True)
+    wl = (torch.randn(r, 11, ch, generator=g, device=device) / 4).requires_grad_(True)
+    ct = torch.randn(n_nodes, 9, ch, generator=g, device=device)
+    out = edge_tensor_product_uu_radial(x, vec, h, wl, plan, mod.tp_info_forward, edge_vectors=True)
+    grads = torch.autograd.grad(out, (x, vec, h, wl), ct)
+    sh = SphericalHarmonics(2)(vec)
+    w = (h @ wl.view(r, -1)).view(n_edges, 11, ch)
+    assert w.numel() > 2 ** 31
+    out2 = edge_tensor_product_uu(x, sh, w, plan, mod.tp_info_forward)
+    grads2 = torch.autograd.grad(out2, (x, vec, h, wl), ct)
+    for name, a, b in zip(("out", "grad_x", "grad_vec", "grad_h", "grad_w_last"), (out, *grads), (out2, *grads2)):
+        assert (a - b).abs().max().item() <= 1e-4 * max(1.0, b.abs().max().item()), name
+    del w, sh, out, out2, grads, grads2
+    torch.cuda.empty_cache()
