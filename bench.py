@@ -54,6 +54,8 @@ def measured_traffic(workload):
     if shutil.which("rocprofv3") is None:
         return None, "rocprofv3 not found"
     me = os.path.abspath(__file__)
+    # the interpreter binary itself goes after "--": no launcher, shell or env hop between the profiler and the program
+    interpreter = os.path.realpath(sys.executable)
     runs = {"work": ["--workload", workload, "--no-cpu-baseline", "--no-configs", "--no-measure-traffic", "--steps", "5",
                      "--warmup", "2", "--kernel-reps", "5"],
             "copy": ["--workload", "copy", "--steps", "5", "--warmup", "2"]}
@@ -65,7 +67,7 @@ def measured_traffic(workload):
             for tag, extra in runs.items():
                 d = os.path.join(out_dir, f"{counter}_{tag}")
                 cmd = ["timeout", "-s", "KILL", "90", "rocprofv3", "--pmc", counter, "--output-format", "csv",
-                       "-d", d, "-o", "t", "--", "python3", me, *extra]
+                       "-d", d, "-o", "t", "--", interpreter, me, *extra]
                 res = subprocess.run(cmd, cwd="/tmp", env=env, capture_output=True, text=True)
                 files = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)
                 if res.returncode != 0 or not files:
@@ -110,10 +112,6 @@ WORKLOADS = {
     # streaming kernels of known traffic (1 GiB): counter calibration and achievable-bandwidth reference
     "copy": None,
     "read": None,
-    # rate of LDS reads by instruction, tile layout and wavefronts per compute unit
-    "lds": None,
-    # vector FMAs next to matrix instructions on one SIMD: same wavefront, two wavefronts, split roles
-    "coissue": None,
     # indexed scale-segment reduction alone: the messages of BASELINE configs[1] summed to their destination nodes
     "scatter": None,
     # spherical harmonics of 2^20 vectors up to degree 6 (forward and gradient kernels), normalisation fused
@@ -371,91 +369,8 @@ def scatter_bench(steps, warmup):
                                    "traffic": None, "algorithmic_bytes": nbytes, "avg_ms": round(ms, 5)}}))
 
 
-def coissue_rates(steps, warmup):
-    """Time of 8 matrix instructions + the FMAs that fit their run time (32 with the bf16 instruction, 64 with the fp32
-    one) per SIMD, issued by one wavefront, by two, or split between two wavefronts: how much vector work hides behind
-    matrix work on this chip.  One JSON line, ns per such unit of work."""
-    import ctypes
-    from equitorch_amd import _lib
-    blib = ctypes.CDLL(os.path.join(ROOT, "equitorch_amd", "lib", "libcgtp_bench.so"))
-    blib.cgtpbench_coissue.argtypes = [ctypes.c_int] * 5 + [ctypes.c_void_p, ctypes.c_void_p]
-    dev = torch.device("cuda:0")
-    n_cu = torch.cuda.get_device_properties(dev).multi_processor_count
-    out = torch.empty(n_cu * 512, dtype=torch.float32, device=dev)
-    stream = _lib.stream_ptr(dev)
-    iters = 20000
-    names = {0: "matrix only", 1: "fma only", 2: "one by one (1 matrix : R fma)", 3: "in blocks (8 matrix, 8 R fma)",
-             4: "split: one wavefront matrix, one fma"}
-    table = {}
-    for f32 in (0, 1):
-        rows = {}
-        for threads in (256, 512):
-            for mode in range(5):
-                if mode == 4 and threads != 512:
-                    continue
-                def launch():
-                    _lib.check(blib.cgtpbench_coissue(mode, f32, threads, n_cu, iters, out.data_ptr(), stream))
-                for _ in range(max(warmup, 1)):
-                    launch()
-                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                a.record()
-                for _ in range(steps):
-                    launch()
-                b.record()
-                torch.cuda.synchronize()
-                ns = a.elapsed_time(b) / steps * 1e6 / iters
-                # work per iteration and SIMD: every wavefront that issues a kind issues 8 matrix / 8 R fma
-                waves = threads // 256
-                units = 1 if mode == 4 else waves
-                rows[f"{waves} wavefront(s) per SIMD, {names[mode]}"] = round(ns / units, 1)
-        table["v_mfma_f32_16x16x4_f32 + 64 fma" if f32 else "v_mfma_f32_16x16x32_bf16 + 32 fma"] = rows
-    print(json.dumps({"metric": "coissue_ns_per_unit", "value": None, "unit": "ns per (8 matrix instructions + their FMAs) per SIMD",
-                      "n_gpus": 1, "steps": steps, "warmup": warmup,
-                      "config": {"workload": "register-only loops; 'matrix only' / 'fma only' rows count their own kind only"},
-                      "rates": table}))
-
-
-def lds_read_rates(steps, warmup):
-    """Rate of LDS reads per compute unit by instruction, tile layout and wavefronts per CU (4, 8, 16): the numbers
-    behind the layout of the bf16 weight-gradient kernel's transpose reads.  One JSON line."""
-    import ctypes
-    from equitorch_amd import _lib
-    blib = ctypes.CDLL(os.path.join(ROOT, "equitorch_amd", "lib", "libcgtp_bench.so"))
-    blib.cgtpbench_lds_read.argtypes = [ctypes.c_int] * 6 + [ctypes.c_void_p, ctypes.c_void_p]
-    dev = torch.device("cuda:0")
-    n_cu = torch.cuda.get_device_properties(dev).multi_processor_count
-    out = torch.empty(4 * n_cu * 256, dtype=torch.int32, device=dev)
-    stream = _lib.stream_ptr(dev)
-    iters = 4000
-    cases = [("ds_read_b128 contiguous", 2, 2, 256), ("ds_read_b64 contiguous", 1, 2, 256),
-             ("ds_read_b64_tr_b16 rows 8q..8q+3 pitch 288", 0, 0, 288), ("ds_read_b64_tr_b16 rows 4q..4q+3 pitch 288", 0, 1, 288),
-             ("ds_read_b64_tr_b16 rows 4q..4q+3 pitch 272", 0, 1, 272), ("ds_read_b64_tr_b16 rows 4q..4q+3 pitch 256", 0, 1, 256)]
-    rows = {}
-    for name, kind, row_mode, pitch in cases:
-        rates = {}
-        for per_cu, lds in ((1, 100000), (2, 70000), (4, 36000)):
-            def launch():
-                _lib.check(blib.cgtpbench_lds_read(kind, row_mode, pitch, per_cu * n_cu, lds, iters, out.data_ptr(), stream))
-            for _ in range(max(warmup, 1)):
-                launch()
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-            for _ in range(steps):
-                launch()
-            b.record()
-            torch.cuda.synchronize()
-            ms = a.elapsed_time(b) / steps
-            bytes_per_cu = iters * 8 * 64 * (16 if kind == 2 else 8) * 4 * per_cu
-            rates[f"{4 * per_cu}_waves_per_cu_bytes_per_ns"] = round(bytes_per_cu / (ms * 1e6), 1)
-        rows[name] = rates
-    print(json.dumps({"metric": "lds_read_rate", "value": rows["ds_read_b128 contiguous"]["16_waves_per_cu_bytes_per_ns"],
-                      "unit": "B/ns per CU", "n_gpus": 1, "steps": steps, "warmup": warmup,
-                      "config": {"workload": "eight reads per wavefront, then s_waitcnt; four wavefronts per workgroup"},
-                      "rates": rows}))
-
-
-def membench(kind, steps, warmup):
-    """Plain 1 GiB device copy (reads 1 GiB, writes 1 GiB) or read; one JSON line with the achieved GB/s."""
+def stream_rate(kind, steps, warmup):
+    """(GB/s, ms per launch) of a plain 1 GiB device copy (reads 1 GiB, writes 1 GiB) or read on this box."""
     import ctypes
     from equitorch_amd import _lib
     blib = ctypes.CDLL(os.path.join(ROOT, "equitorch_amd", "lib", "libcgtp_bench.so"))
@@ -482,7 +397,15 @@ def membench(kind, steps, warmup):
     torch.cuda.synchronize()
     ms = sum(a.elapsed_time(b) for a, b in evs) / steps
     moved = n_bytes * (2 if kind == "copy" else 1)
-    print(json.dumps({"metric": f"membench_{kind}", "value": round(moved / ms / 1e6, 1), "unit": "GB/s",
+    del src, dst
+    return moved / ms / 1e6, ms
+
+
+def membench(kind, steps, warmup):
+    """The streaming kernels as a workload of their own; one JSON line with the achieved GB/s."""
+    n_bytes = 1 << 30
+    gbs, ms = stream_rate(kind, steps, warmup)
+    print(json.dumps({"metric": f"membench_{kind}", "value": round(gbs, 1), "unit": "GB/s",
                       "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 5),
                       "bytes_read": n_bytes, "bytes_written": n_bytes if kind == "copy" else 0,
                       "config": {"workload": f"{kind} of 1 GiB, float4 grid-stride, 4096 workgroups"}}))
@@ -867,12 +790,6 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
-    if args.workload == "lds":
-        lds_read_rates(args.steps, args.warmup)
-        return
-    if args.workload == "coissue":
-        coissue_rates(args.steps, args.warmup)
-        return
     if args.workload in ("copy", "read"):
         membench(args.workload, args.steps, args.warmup)
         return
@@ -1002,12 +919,17 @@ def main():
     # measured now unless told otherwise, or unless this process itself runs under a profiler (its children would be
     # profiled twice)
     profiled = any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ) or "rocprof" in os.environ.get("LD_PRELOAD", "")
+    traffic_measured = False
     if not args.no_measure_traffic and not profiled and args.graph == "uniform":
         live, live_source = measured_traffic(args.workload)
         if live is not None:
-            traffic, traffic_source = live, live_source
+            traffic, traffic_source, traffic_measured = live, live_source, True
         else:
             traffic_source += f" (live measurement unavailable: {live_source})"
+    # what this box itself delivers for plain streaming kernels, next to the vendor peak: the denominators a tuned
+    # bandwidth-bound kernel can actually be held against
+    copy_gbs, _ = stream_rate("copy", 10, 3)
+    read_gbs, _ = stream_rate("read", 10, 3)
 
     rec = {
         "metric": "edge-TP fwd+bwd Medges/s (lmax=2,C=64)" if backward else "edge-TP fwd Medges/s (lmax=2,C=64)",
@@ -1020,8 +942,13 @@ def main():
                                + ("" if args.graph == "uniform" else f", {args.graph} graph")},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": traffic, "traffic_source": traffic_source,
-                     "algorithmic_bytes": dom_bytes, "avg_ms": round(dom_ms, 5)},
+                     "traffic": traffic, "traffic_source": traffic_source, "traffic_measured": traffic_measured,
+                     "algorithmic_bytes": dom_bytes, "avg_ms": round(dom_ms, 5),
+                     "achievable": {"copy_GBs": round(copy_gbs, 1), "read_GBs": round(read_gbs, 1),
+                                    "what": "1 GiB streaming copy (read + write bytes) and read kernels, same run",
+                                    "frac_of_copy": round(achieved / copy_gbs, 4),
+                                    "frac_of_read": round(achieved / read_gbs, 4),
+                                    "traffic_GBs": None if traffic is None else round(traffic / dom_ms / 1e6, 1)}},
         "kernels": {"fwd_avg_ms": round(fwd_avg, 5), "fwd_med_ms": round(fwd_med, 5),
                     "fwd_GBs": round(fwd_bytes / fwd_avg / 1e6, 1),
                     "bwd_avg_ms": round(bwd_avg, 5), "bwd_med_ms": round(bwd_med, 5),

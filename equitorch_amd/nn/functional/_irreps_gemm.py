@@ -373,6 +373,20 @@ def _matrix_core_path(x: Tensor, weight: Tensor, plan: LinearPlan, in_size: int,
     return _uvw_mfma.try_forward(x, ones, weight, info)
 
 
+_ONES = {}
+
+
+def _ones_column(n: int, dtype, device) -> Tensor:
+    """``(n, 1)`` ones: one buffer per dtype and device, grown geometrically to the largest batch seen and sliced, so
+    that graphs of varying size do not leave one buffer per distinct size behind."""
+    key = (dtype, str(device))
+    buf = _ONES.get(key)
+    if buf is None or buf.shape[0] < n:
+        buf = torch.ones(max(n, 2 * (0 if buf is None else buf.shape[0])), 1, dtype=dtype, device=device)
+        _ONES[key] = buf
+    return buf[:n]
+
+
 def _table_driven_path(x: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anchor: Tensor):
     """fp32 with a shared weight: the layer as a fully connected product with the scalar 1 on the table-driven
     matrix-core kernels (``cgtp_uvt_*``: forward, grad input and grad weight in one launch each, rows read and written
@@ -399,8 +413,7 @@ def _table_driven_path(x: Tensor, weight: Tensor, plan: LinearPlan, in_size: int
     table = cached(anchor, ("linear_as_coo_table", in_size, plan.n_paths, plan.out_size), build)
     if table is False:
         return None
-    ones = cached(anchor, ("ones", x.dtype, x.shape[0], str(x.device)),
-                  lambda: torch.ones(x.shape[0], 1, dtype=x.dtype, device=x.device))
+    ones = _ones_column(x.shape[0], x.dtype, x.device)
     if not _uv_native.u1v_supported(x, ones, weight, table):
         return None
     kernels.log_tier("irreps_linear", "table-driven matrix-core kernels")

@@ -34,6 +34,8 @@ class TriSpec:
         self.coef = None if coef is None else np.asarray(coef, dtype=np.float64)
         self.out_size = int(out_size)
         self.sizes = list(sizes)
+        # rows an operand must have for every index of the table to land inside it
+        self.min_rows = [0 if i is None or i.size == 0 else int(i.max()) + 1 for i in self.idx]
         self._grad = {}
         self._packed = {}
 
@@ -195,12 +197,16 @@ class TriContract(Function):
         ops = [None if ax is None else (t.to(dtype).contiguous() if single_axis else t.to(dtype))
                for t, ax in zip(ops, axes)]
         n_rows, ext = None, {"u": None, "w": None}
-        for t, ax in zip(ops, axes):
+        for slot, (t, ax) in enumerate(zip(ops, axes)):
             if ax is None:
                 continue
             if t.ndim not in (1 + len(ax), 2 + len(ax)):
                 raise _lib.CgtpError(f"operand with axes '{ax}' must have {1 + len(ax)} or {2 + len(ax)} dims, "
                                      f"got {t.ndim}")
+            have = t.shape[t.ndim - len(ax) - 1]
+            if have < spec.min_rows[slot]:
+                raise _lib.CgtpError(f"operand {slot} has {have} rows along its indexed axis, the table reaches row "
+                                     f"{spec.min_rows[slot] - 1}")
             if not _is_shared(t, ax):
                 if n_rows not in (None, t.shape[0]):
                     raise _lib.CgtpError(f"batch size mismatch: {n_rows} vs {t.shape[0]}")

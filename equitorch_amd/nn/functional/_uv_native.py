@@ -297,6 +297,9 @@ def u1v_supported(x: Tensor, y: Tensor, w: Tensor, tp_info) -> bool:
     _, u, wc = w.shape
     n = x.shape[0]
     dt = x.dtype
+    if tuple(x.shape) != (n, c.D1, u) or tuple(y.shape) != (n, c.D2) or w.shape[0] != c.P:
+        raise _lib.CgtpError(f"operands {tuple(x.shape)}, {tuple(y.shape)}, {tuple(w.shape)} do not fit the table: "
+                             f"expected (N, {c.D1}, U), (N, {c.D2}), ({c.P}, U, W)")
     return (chunk_of(n, c.D1, c.D2, c.DO, u, 0, wc, dt) > 0 and chunk_of(n, c.DO, c.D2, c.D1, wc, 0, u, dt) > 0
             and grad_y_supported(n, c.D1, c.D2, u, wc, tp_info, x.element_size()) and x.data_ptr() % 16 == 0)
 
@@ -356,6 +359,9 @@ def uvw_supported(x: Tensor, y: Tensor, w: Tensor, tp_info) -> bool:
     _, u, v, wc = w.shape
     n = x.shape[0]
     dt = x.dtype
+    if tuple(x.shape) != (n, c.D1, u) or tuple(y.shape) != (n, c.D2, v) or w.shape[0] != c.P:
+        raise _lib.CgtpError(f"operands {tuple(x.shape)}, {tuple(y.shape)}, {tuple(w.shape)} do not fit the table: "
+                             f"expected (N, {c.D1}, U), (N, {c.D2}, V), ({c.P}, U, V, W)")
     return (chunk_of(n, c.D1, c.D2, c.DO, u, v, wc, dt) > 0 and chunk_of(n, c.D2, c.DO, c.D1, v, wc, u, dt) > 0
             and chunk_of(n, c.DO, c.D1, c.D2, wc, u, v, dt) > 0 and x.data_ptr() % 16 == 0 and y.data_ptr() % 16 == 0)
 

@@ -61,6 +61,33 @@ class EdgePlan:
                 SparseScaleInfo(None, self.dst, None, None, self.num_edges))
 
 
+def _check_edge_operands(x: Tensor, y: Tensor, plan: EdgePlan, tp_info: TensorProductInfo, weight: Optional[Tensor] = None,
+                         h: Optional[Tensor] = None, w_last: Optional[Tensor] = None, edge_vectors: bool = False) -> None:
+    """Operand extents against the edge list and the table, before any kernel sees them: the fused kernels read
+    ``P * C`` weights and ``D2`` (or 3) values of the second operand for every edge of the plan, and ``D1 * C`` values
+    of every source node, whatever the tensors hold."""
+    coo = kernels.coo_of(tp_info)
+    e = plan.num_edges
+    if plan.num_src_nodes != x.shape[0]:
+        raise _lib.CgtpError(f"plan was built for {plan.num_src_nodes} source nodes, x has {x.shape[0]}")
+    if x.ndim != 3 or x.shape[1] != coo.D1:
+        raise _lib.CgtpError(f"x must be (N_src, {coo.D1}, C) for this table, got {tuple(x.shape)}")
+    d2 = 3 if edge_vectors else coo.D2
+    if y.ndim != 2 or y.shape[0] != e or y.shape[1] != d2:
+        raise _lib.CgtpError(f"the second operand must be ({e}, {d2}) for this plan and table, got {tuple(y.shape)}")
+    c = x.shape[2]
+    if weight is not None:
+        ok = (weight.ndim == 2 and tuple(weight.shape) == (coo.P, c)) or \
+             (weight.ndim == 3 and tuple(weight.shape) == (e, coo.P, c))
+        if not ok:
+            raise _lib.CgtpError(f"weight must be ({coo.P}, {c}) or ({e}, {coo.P}, {c}), got {tuple(weight.shape)}")
+    if h is not None:
+        if h.ndim != 2 or h.shape[0] != e:
+            raise _lib.CgtpError(f"h must be ({e}, R), got {tuple(h.shape)}")
+        if w_last.ndim != 3 or tuple(w_last.shape) != (h.shape[1], coo.P, c):
+            raise _lib.CgtpError(f"w_last must be ({h.shape[1]}, {coo.P}, {c}), got {tuple(w_last.shape)}")
+
+
 class _EdgeUvuCompiled(Function):
     @staticmethod
     def forward(ctx, x: Tensor, sh: Tensor, w: Tensor, plan: EdgePlan, tp_info: TensorProductInfo, cfg: int):
@@ -163,8 +190,7 @@ def edge_tensor_product_uu(x: Tensor, sh: Tensor, weight: Tensor, plan: EdgePlan
     tables, e.g. lmax = 6: fp32 with per-edge weights); otherwise runs the same three steps as separate launches.
     """
     _lib.require_gpu(x, sh, weight)
-    if plan.num_src_nodes != x.shape[0]:
-        raise _lib.CgtpError(f"plan was built for {plan.num_src_nodes} source nodes, x has {x.shape[0]}")
+    _check_edge_operands(x, sh, plan, tp_info_forward, weight=weight)
     cfg = kernels.uvu_config_of(tp_info_forward)
     if cfg >= 0 and x.dtype == sh.dtype == weight.dtype and x.dtype in (torch.float32, torch.float64):
         xc, yc, wc = x.contiguous(), sh.contiguous(), weight.contiguous()
@@ -196,8 +222,7 @@ def edge_tensor_product_uu_vectors(x: Tensor, edge_vec: Tensor, weight: Tensor, 
     _lib.require_gpu(x, edge_vec, weight)
     if edge_vec.ndim != 2 or edge_vec.shape[1] != 3:
         raise ValueError(f"edge_vec must be (E, 3), got {tuple(edge_vec.shape)}")
-    if plan.num_src_nodes != x.shape[0]:
-        raise _lib.CgtpError(f"plan was built for {plan.num_src_nodes} source nodes, x has {x.shape[0]}")
+    _check_edge_operands(x, edge_vec, plan, tp_info_forward, weight=weight, edge_vectors=True)
     cfg = kernels.uvu_config_of(tp_info_forward)
     mode = kernels.Y_UNIT_VECTOR if normalize_input else kernels.Y_RAW_VECTOR
     if (cfg >= 0 and kernels.uvu_sh_degree(cfg) >= 0 and x.dtype == edge_vec.dtype == weight.dtype
@@ -225,16 +250,17 @@ def edge_tensor_product_uu_radial(x: Tensor, sh_or_vec: Tensor, h: Tensor, w_las
     shapes form ``h @ w_last`` with a matrix product and take the plain functions.
     """
     _lib.require_gpu(x, sh_or_vec, h, w_last)
-    if plan.num_src_nodes != x.shape[0]:
-        raise _lib.CgtpError(f"plan was built for {plan.num_src_nodes} source nodes, x has {x.shape[0]}")
+    _check_edge_operands(x, sh_or_vec, plan, tp_info_forward, h=h, w_last=w_last, edge_vectors=edge_vectors)
     cfg = kernels.uvu_config_of(tp_info_forward)
     mode = 0 if not edge_vectors else (kernels.Y_UNIT_VECTOR if normalize_input else kernels.Y_RAW_VECTOR)
-    if (kernels.uvu_radial_supported(cfg, x, h, w_last) and sh_or_vec.dtype == x.dtype
+    xc, yc, hc = x.contiguous(), sh_or_vec.contiguous(), h.contiguous()
+    # a misaligned operand (a view at an odd offset) takes the matrix-product route below instead of an error
+    if (kernels.uvu_radial_supported(cfg, xc, hc, w_last) and yc.dtype == xc.dtype and yc.data_ptr() % 16 == 0
             and (not edge_vectors or kernels.uvu_sh_degree(cfg) >= 0)):
         kernels.log_tier("edge_tensor_product_uu_radial", "fused gather / weights / product / segment sum",
                          f"config {int(cfg)}")
         w_eff = kernels.radial_effective_weight(w_last, cfg)       # differentiable: expands paths, folds factors
-        return _EdgeUvuRadial.apply(x.contiguous(), sh_or_vec.contiguous(), h.contiguous(), w_eff, plan, cfg, mode)
+        return _EdgeUvuRadial.apply(xc, yc, hc, w_eff, plan, cfg, mode)
     kernels.log_tier("edge_tensor_product_uu_radial", "weights by matrix product, then the plain edge product")
     weight = (h @ w_last.reshape(w_last.shape[0], -1)).view(h.shape[0], *w_last.shape[1:])
     if edge_vectors:

@@ -68,5 +68,8 @@ def sparse_vecmat(input1: Tensor, input2: Tensor, info_fwd: SparseProductInfo,
 def sparse_mat_t_vec(input1: Tensor, input2: Tensor, info_fwd: SparseProductInfo,
                      info_bwd1: Optional[SparseProductInfo] = None, info_bwd2: Optional[SparseProductInfo] = None,
                      out_accumulated: bool = False) -> Tensor:
-    """``z[n,M,u] = sum_t s_t sum_w Y[(n),i1_t,u,w] x[n,i2_t,w]`` (reference ``:434-500``)."""
-    return _binary("uw", "w", "u", input1, input2, info_fwd, out_accumulated)
+    """``z[n,M,w] = sum_t s_t sum_u Y[(n),i1_t,u,w] x[n,i2_t,u]``: the matrix ``(.., M1, C_in, C_out)`` first, the vector
+    ``(.., M2, C_in)`` second, contracted over the matrix's first channel axis — ``input1.T @ input2`` entry by entry
+    (reference ``:434-500``, which calls the vector-matrix product with the operands exchanged,
+    ``ops/batched_sparse_dense_op.py:1200-1238``)."""
+    return _binary("uw", "u", "w", input1, input2, info_fwd, out_accumulated)

@@ -8,8 +8,11 @@ table-driven HIP kernels: the element-wise members below on the single-axis kern
     inner  : z[n,M]   = sum_t s_t sum_c x[n,i1_t,c] y[n,i2_t,c]    (:713-855)
 
 An operand without its batch axis is shared over the batch; ``out_accumulated`` sums the result over the
-batch (gradient of a shared operand).  ``gather_index`` / ``index_out`` are never produced by the table
-builders and are rejected.
+batch (gradient of a shared operand).  ``gather_index`` (position inside a segment -> table entry, ``:103-106``)
+and ``index_out`` (segment -> output row, ``:138-144``) are never produced by the table builders; they are
+honoured by rewriting the table (entries permuted on the way in, result rows placed on the way out).  ``out=`` is
+written as the reference's kernels write it: the rows of the segments only, added to when ``out_accumulated``
+(``kernel_utils.py:139-155``: an atomic add onto what the tensor holds) and stored otherwise.
 """
 from typing import Optional
 
@@ -21,12 +24,48 @@ from .._lib import OPERAND_SCALAR, OPERAND_VEC
 from . import kernels
 
 
+def _gathered(scale, index1, index2, gather_index):
+    """The table with its entries read through ``gather_index``: entry t of the new table is entry
+    ``gather_index[t]`` of the old one (an operand without an index column is indexed by the entry number)."""
+    if gather_index is None:
+        return scale, index1, index2
+    pick = lambda t: gather_index if t is None else t.index_select(0, gather_index)
+    return (None if scale is None else scale.index_select(0, gather_index)), pick(index1), pick(index2)
+
+
+def _finish(res: Tensor, dim: int, out: Optional[Tensor], out_accumulated: bool, out_size: Optional[int],
+            index_out: Optional[Tensor]) -> Tensor:
+    """Place the ``n_seg`` result rows: into a fresh zero tensor of ``out_size`` rows (rows past the segments and
+    rows no segment names stay zero) or into ``out``, at rows ``0 .. n_seg-1`` or ``index_out``; ``dim`` is the axis
+    of ``res`` that runs over the segments."""
+    n_seg = res.shape[dim]
+    fresh = out is None
+    if fresh:
+        size = n_seg if out_size is None else int(out_size)
+        if index_out is None and size == n_seg:
+            return res
+        shape = list(res.shape)
+        shape[dim] = size
+        out = torch.zeros(shape, dtype=res.dtype, device=res.device)
+    need = n_seg if index_out is None else (int(index_out.max()) + 1 if index_out.numel() else 0)
+    if out.shape[dim] < need:
+        raise _lib.CgtpError(f"the output has {out.shape[dim]} rows, the table writes row {need - 1}")
+    res = res.to(out.dtype)
+    if index_out is None:
+        target = out.narrow(dim, 0, n_seg)
+        target.add_(res) if (out_accumulated and not fresh) else target.copy_(res)
+    elif out_accumulated:
+        out.index_add_(dim, index_out, res)
+    else:
+        out.index_copy_(dim, index_out, res)
+    return out
+
+
 def _product(input1: Tensor, kind1: int, input2: Tensor, kind2: int, scale, index1, index2, seg,
              gather_index, index_out, out, out_accumulated: bool, out_size: Optional[int],
              reduce_c: bool) -> Tensor:
-    if gather_index is not None or index_out is not None:
-        raise NotImplementedError("gather_index / index_out tables are not supported")
-    _lib.require_gpu(input1, input2, scale, index1, index2, seg)
+    _lib.require_gpu(input1, input2, scale, index1, index2, seg, gather_index, index_out)
+    scale, index1, index2 = _gathered(scale, index1, index2, gather_index)
     dtype = torch.result_type(input1, input2)
     input1, input2 = input1.to(dtype).contiguous(), input2.to(dtype).contiguous()
     full1 = 3 if kind1 == OPERAND_VEC else 2
@@ -49,17 +88,7 @@ def _product(input1: Tensor, kind1: int, input2: Tensor, kind2: int, scale, inde
     table, n_seg = kernels.product_tri_table(scale, index1, index2, seg, n_entries, dtype, input1.device)
     res = kernels.tri_contract(table, n_seg, (input1, kind1), (input2, kind2), (None, 0), n_rows, channels,
                                dtype, input1.device, reduce_c=reduce_c, reduce_rows=out_accumulated)
-    if out_size is not None and out_size != n_seg:
-        sparse_dim = 0 if out_accumulated else 1
-        shape = list(res.shape)
-        shape[sparse_dim] = out_size
-        full = torch.zeros(shape, dtype=res.dtype, device=res.device)
-        full.narrow(sparse_dim, 0, min(n_seg, out_size)).copy_(res.narrow(sparse_dim, 0, min(n_seg, out_size)))
-        res = full
-    if out is not None:
-        out.copy_(res)
-        return out
-    return res
+    return _finish(res, 0 if out_accumulated else 1, out, out_accumulated, out_size, index_out)
 
 
 def indexed_mul_scale_gather(input1, input2, scale=None, index1=None, index2=None, seg=None,
@@ -96,19 +125,17 @@ def indexed_inner_scale_gather(input1, input2, scale=None, index1=None, index2=N
 def _matrix_product(input1, axes1, input2, axes2, out_axes, scale, index1, index2, seg, gather_index, index_out,
                     out, out_accumulated, out_size):
     """Matrix members of the family on the two-axis contraction kernel (no autograd at this layer)."""
-    if gather_index is not None or index_out is not None:
-        raise NotImplementedError("gather_index / index_out tables are not supported")
     from ..nn.functional._tri import spec_from_product_info, tri
     from ..structs import SparseProductInfo
-    info = SparseProductInfo(scale, index1, index2, seg, None, None, out_size)
+    _lib.require_gpu(input1, input2, scale, index1, index2, seg, gather_index, index_out)
+    scale, index1, index2 = _gathered(scale, index1, index2, gather_index)
+    info = SparseProductInfo(scale, index1, index2, seg, None, None, None)
     size1, size2 = input1.shape[-1 - len(axes1)], input2.shape[-1 - len(axes2)]
     with torch.no_grad():
         res = tri(spec_from_product_info(info, size1, size2), (axes1, axes2, None), out_axes, input1, input2,
                   None, out_shared=out_accumulated)
-    if out is not None:
-        out.copy_(res)
-        return out
-    return res
+    batched = res.ndim == 2 + len(out_axes)          # no batch axis when summed over it or when both operands are shared
+    return _finish(res, 1 if batched else 0, out, out_accumulated, out_size, index_out)
 
 
 def indexed_outer_scale_gather(input1, input2, scale=None, index1=None, index2=None, seg=None,
@@ -132,6 +159,8 @@ def indexed_mat_t_vec_scale_gather(input1, input2, scale=None, index1=None, inde
                                    gather_index=None, index_out=None, out=None, out_accumulated=False,
                                    out_size=None, block_size_n=8, block_size_c_out=32, block_size_c_in=32,
                                    num_stages=1, loop_unroll_factor=4):
-    """``z[n,M,u] = sum_t s_t sum_w Y[(n),i1_t,u,w] x[n,i2_t,w]`` (reference ``:1200-1238``)."""
-    return _matrix_product(input1, "uw", input2, "w", "u", scale, index1, index2, seg, gather_index, index_out,
+    """``z[n,M,w] = sum_t s_t sum_u Y[(n),i1_t,u,w] x[n,i2_t,u]``: matrix ``(.., M1, C_in, C_out)`` first, vector
+    ``(.., M2, C_in)`` second (reference ``:1200-1238``: the vector-matrix product with operands and index columns
+    exchanged)."""
+    return _matrix_product(input1, "uw", input2, "u", "w", scale, index1, index2, seg, gather_index, index_out,
                            out, out_accumulated, out_size)

@@ -666,6 +666,7 @@ def uvu_radial_supported(cfg: int, x: Tensor, h: Tensor, w_last: Tensor) -> bool
     return (cfg >= 0 and bool(_lib.lib.cgtp_uvu_radial_supported(int(cfg))) and x.dtype == h.dtype == w_last.dtype
             and x.dtype == torch.float32 and x.shape[-1] == 64 and h.ndim == 2 and w_last.ndim == 3
             and h.shape[1] == w_last.shape[0] and h.shape[1] % 4 == 0 and 4 <= h.shape[1] <= 16
+            and w_last.shape[2] == x.shape[-1]
             and 4 <= uvu_dims(int(cfg))[3] <= 16 and h.shape[0] > 0 and x.shape[0] > 0
             and x.data_ptr() % 16 == 0 and h.data_ptr() % 16 == 0)
 

@@ -8,7 +8,7 @@ import itertools
 import pytest
 import torch
 
-from helpers import assert_close, stable_seed
+from helpers import assert_close, fp32_twin, stable_seed
 from oracle import ref_ops, ref_tables
 
 pytestmark = pytest.mark.gpu
@@ -96,23 +96,28 @@ def test_row_sums_beyond_1024_rows(device, tables13, table, n, channels, dtype):
                           ("vecsca", ref_ops.cpu_vecsca, torch.randn(n, d2, generator=g, dtype=torch.float64))):
         y = y.to(dtype)
         out = getattr(F, f"sparse_{op}")(x.to(device), y.to(device), info_m, out_accumulated=True)
-        # sums of n products of N(0,1) numbers: magnitude sqrt(n) * coefficients; compared norm-wise
+        # sums of n products of N(0,1) numbers: magnitude sqrt(n) * coefficients; compared norm-wise, and against what
+        # the same CPU function loses in fp32
+        r32 = fp32_twin(oracle, x, y, info_r, out_accumulated=True) if dtype == torch.float32 else None
         assert_close(out, oracle(x.double(), y.double(), info_r, out_accumulated=True), tol, f"{op} row sum",
-                     norm="max")
+                     norm="max", fp32_ref=r32)
     # gradient of a shared second operand (the sum over rows happens in the backward launch)
     w = torch.randn(d2, channels, generator=g, dtype=torch.float64).to(dtype)
     wd = w.to(device).requires_grad_(True)
     ct = torch.randn(n, info_r["seg_out"].shape[0] - 1, channels, generator=g, dtype=torch.float64).to(dtype)
     (gw,) = torch.autograd.grad(F.sparse_mul(x.to(device), wd, info_m), (wd,), ct.to(device))
-    wr = w.double().requires_grad_(True)
-    (rgw,) = torch.autograd.grad(ref_ops.cpu_mul(x.double(), wr, info_r), (wr,), ct.double())
-    assert_close(gw, rgw, tol, "shared-operand gradient", norm="max")
+    def shared_grad(dt):
+        wr = w.to(dt).requires_grad_(True)
+        info = {k: (v.to(dt) if v is not None and v.is_floating_point() else v) for k, v in info_r.items()}
+        return torch.autograd.grad(ref_ops.cpu_mul(x.to(dt), wr, info), (wr,), ct.to(dt))[0]
+    assert_close(gw, shared_grad(torch.float64), tol, "shared-operand gradient", norm="max",
+                 fp32_ref=shared_grad(torch.float32) if dtype == torch.float32 else None)
 
 
 MAT = {  # name: (axes1, axes2, out axes, einsum)
     "outer": ("u", "w", "uw", "mab,{a}au,{b}bw->{o}muw"),
     "vecmat": ("u", "uw", "w", "mab,{a}au,{b}buw->{o}mw"),
-    "mat_t_vec": ("uw", "w", "u", "mab,{a}auw,{b}bw->{o}mu"),
+    "mat_t_vec": ("uw", "u", "w", "mab,{a}auw,{b}bu->{o}mw"),
 }
 
 
@@ -135,19 +140,23 @@ def test_matrix_ops_sweep(device, tables13, op, shared1, shared2, acc):
     x, y = mk(ax1, shared1), mk(ax2, shared2)
     xd, yd = (t.float().to(device).requires_grad_(True) for t in (x, y))
     out = getattr(F, f"sparse_{op}")(xd, yd, info_m, out_accumulated=acc)
-    xr, yr = (t.float().double().requires_grad_(True) for t in (x, y))
     eq = eq.format(a="" if shared1 else "n", b="" if shared2 else "n", o="" if (shared1 and shared2) else "n")
-    ref_out = torch.einsum(eq, T, xr, yr)
-    if acc:
-        ref_out = ref_out.sum(0)
+
+    def dense(dt):      # the dense contraction in float64 (the arbiter) and in float32 (what fp32 arithmetic loses)
+        xr, yr = (t.float().to(dt).requires_grad_(True) for t in (x, y))
+        o = torch.einsum(eq, T.to(dt), xr, yr)
+        return (o.sum(0) if acc else o), xr, yr
+    ref_out, xr, yr = dense(torch.float64)
+    out32, x32, y32 = dense(torch.float32)
     # results summed over the batch (accumulated output, gradient of a shared operand) and over up to 21 channels
     # and ~40 coefficients per element: norm-wise; per-row results element-wise
-    assert_close(out, ref_out, 1e-5, f"{op} forward", norm="max" if acc else "element")
+    assert_close(out, ref_out, 1e-5, f"{op} forward", norm="max" if acc else "element", fp32_ref=out32)
     ct = torch.randn(ref_out.shape, generator=g, dtype=torch.float64)
     gx, gy = torch.autograd.grad(out, (xd, yd), ct.float().to(device))
     rgx, rgy = torch.autograd.grad(ref_out, (xr, yr), ct.float().double())
-    assert_close(gx, rgx, 1e-5, f"{op} grad1", norm="max" if shared1 else "element")
-    assert_close(gy, rgy, 1e-5, f"{op} grad2", norm="max" if shared2 else "element")
+    gx32, gy32 = torch.autograd.grad(out32, (x32, y32), ct.float())
+    assert_close(gx, rgx, 1e-5, f"{op} grad1", norm="max" if shared1 else "element", fp32_ref=gx32)
+    assert_close(gy, rgy, 1e-5, f"{op} grad2", norm="max" if shared2 else "element", fp32_ref=gy32)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
@@ -183,17 +192,25 @@ def test_shared_matrix_ops_on_the_matrix_core_kernels(device, monkeypatch, op, d
     monkeypatch.setattr(kernels, "log_tier", lambda op_, tier, detail="": seen.append(tier))
     xd, yd = (t.to(dtype).to(device).requires_grad_(True) for t in (x, y))
     out = getattr(F, f"sparse_{op}")(xd, yd, info)
-    xr, yr = (t.to(dtype).double().requires_grad_(True) for t in (x, y))
-    ref_out = torch.einsum(eq.format(a="" if shared[0] else "n", b="" if shared[1] else "n", o="n"), T, xr, yr)
+    eq = eq.format(a="" if shared[0] else "n", b="" if shared[1] else "n", o="n")
+    ct = None
+
+    def dense(dt):      # (out, grad1, grad2) of the dense contraction carried out in ``dt``
+        nonlocal ct
+        xr, yr = (t.to(dtype).to(dt).requires_grad_(True) for t in (x, y))
+        o = torch.einsum(eq, T.to(dt), xr, yr)
+        if ct is None:
+            ct = torch.randn(o.shape, generator=g, dtype=torch.float64).to(dtype)
+        return (o, *torch.autograd.grad(o, (xr, yr), ct.to(dt)))
+    ref_out, rgx, rgy = dense(torch.float64)
+    r32 = dense(torch.float32) if dtype == torch.float32 else (None, None, None)
     tol = 1e-5 if dtype == torch.float32 else 1e-11
-    # sums over 16 or 24 channels and several entries per element: norm-wise in fp32
-    assert_close(out, ref_out, tol, f"{op} forward", norm="max")
+    # sums over 16 or 24 channels and several entries per element: norm-wise in fp32, and against fp32 arithmetic
+    assert_close(out, ref_out, tol, f"{op} forward", norm="max", fp32_ref=r32[0])
     assert out[:, n_out - 1].abs().max().item() == 0.0
-    ct = torch.randn(ref_out.shape, generator=g, dtype=torch.float64)
-    gx, gy = torch.autograd.grad(out, (xd, yd), ct.to(dtype).to(device))
-    rgx, rgy = torch.autograd.grad(ref_out, (xr, yr), ct.to(dtype).double())
-    assert_close(gx, rgx, tol, f"{op} grad1", norm="max")
-    assert_close(gy, rgy, tol, f"{op} grad2", norm="max")
+    gx, gy = torch.autograd.grad(out, (xd, yd), ct.to(device))
+    assert_close(gx, rgx, tol, f"{op} grad1", norm="max", fp32_ref=r32[1])
+    assert_close(gy, rgy, tol, f"{op} grad2", norm="max", fp32_ref=r32[2])
     assert sum("shared matrix" in t for t in seen) == 2, seen          # forward and the vector operand's gradient
     assert sum("summed over rows" in t for t in seen) == 1, seen       # the matrix operand's gradient
 
@@ -224,17 +241,22 @@ def test_matrix_core_route_random_shapes(device, case):
     m = torch.randn(n_mat, cu, cw, generator=g, dtype=torch.float64).to(dtype)
     xd, md = (t.to(device).requires_grad_(True) for t in (x, m))
     out = F.sparse_vecmat(xd, md, info)
-    xr, mr = (t.double().requires_grad_(True) for t in (x, m))
-    ref_out = torch.einsum("mab,nau,buw->nmw", T, xr, mr)
+    ct = torch.randn(n, n_out, cw, generator=g, dtype=torch.float64).to(dtype)
+
+    def dense(dt):      # (out, grad vector, grad matrix) of the dense contraction carried out in ``dt``
+        xr, mr = (t.to(dt).requires_grad_(True) for t in (x, m))
+        o = torch.einsum("mab,nau,buw->nmw", T.to(dt), xr, mr)
+        return (o, *torch.autograd.grad(o, (xr, mr), ct.to(dt)))
+    ref_out, rgx, rgm = dense(torch.float64)
+    r32 = dense(torch.float32) if dtype == torch.float32 else (None, None, None)
     tol = 1e-5 if dtype == torch.float32 else 1e-11
     what = f"case {case}: n={n} out={n_out} rows={d_vec} paths={n_mat} {cu}->{cw} nnz={nnz} {dtype}"
-    # sums over up to 40 channels and several entries per element, and over the batch for the matrix: norm-wise
-    assert_close(out, ref_out, tol, what + " forward", norm="max")
-    ct = torch.randn(ref_out.shape, generator=g, dtype=torch.float64).to(dtype)
+    # sums over up to 40 channels and several entries per element, and over the batch for the matrix: norm-wise, and
+    # against what the same contraction loses in fp32
+    assert_close(out, ref_out, tol, what + " forward", norm="max", fp32_ref=r32[0])
     gx, gm = torch.autograd.grad(out, (xd, md), ct.to(device))
-    rgx, rgm = torch.autograd.grad(ref_out, (xr, mr), ct.double())
-    assert_close(gx, rgx, tol, what + " grad vector", norm="max")
-    assert_close(gm, rgm, tol, what + " grad matrix", norm="max")
+    assert_close(gx, rgx, tol, what + " grad vector", norm="max", fp32_ref=r32[1])
+    assert_close(gm, rgm, tol, what + " grad matrix", norm="max", fp32_ref=r32[2])
 
 
 @pytest.mark.parametrize("scaled,indexed,segmented", [(True, True, True), (False, True, True), (True, False, True),

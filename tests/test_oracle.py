@@ -35,7 +35,7 @@ def test_dot_and_cross_product_paths():
 
 def _wigner_from_harmonics(rot, lmax):
     """Block-diagonal D with Y(R v) = D Y(v), solved by least squares from the harmonics themselves."""
-    from equitorch_amd.utils._sh import spherical_harmonics
+    from oracle.ref_sh import spherical_harmonics
     v = unit_vectors(400, torch.Generator().manual_seed(11)).double()
     y, yr = spherical_harmonics(v, lmax), spherical_harmonics(v @ rot.T, lmax)
     d = torch.zeros((lmax + 1) ** 2, (lmax + 1) ** 2, dtype=torch.float64)
@@ -49,7 +49,7 @@ def test_dense_oracle_is_equivariant():
     q, _ = torch.linalg.qr(torch.randn(3, 3, generator=torch.Generator().manual_seed(5), dtype=torch.float64))
     for rot in (q * torch.sign(torch.linalg.det(q)), -q * torch.sign(torch.linalg.det(q))):  # proper, improper
         d = _wigner_from_harmonics(rot, 2)
-        from equitorch_amd.utils._sh import spherical_harmonics
+        from oracle.ref_sh import spherical_harmonics
         g = torch.Generator().manual_seed(6)
         v = unit_vectors(9, g).double()
         x = torch.randn(9, 9, 4, generator=g, dtype=torch.float64)

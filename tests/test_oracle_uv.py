@@ -159,7 +159,7 @@ def test_structural_uvw_and_uuu_chains_match_dense(irreps, shared_w):
 
 def test_dense_u1v_is_equivariant():
     """O(3) equivariance of the fully connected product for arbitrary weights (Wigner-D from the harmonics)."""
-    from equitorch_amd.utils._sh import spherical_harmonics
+    from oracle.ref_sh import spherical_harmonics
     from test_oracle import _wigner_from_harmonics
     q, _ = torch.linalg.qr(torch.randn(3, 3, generator=torch.Generator().manual_seed(9), dtype=torch.float64))
     rot = -q * torch.sign(torch.linalg.det(q))       # improper: parities matter

@@ -40,3 +40,38 @@ def test_cutoffs_boundary_behaviour():
     assert cos[4] == 0
     mol = MollifierCutoff(r_max=4.0, eps=1e-7)(r.detach())
     assert abs(float(mol[0]) - 1) < 1e-6 and float(mol[3]) < 1e-12 and float(mol[2]) == math.exp(1 - 1 / (1 - 0.625 ** 2 + 1e-7))
+
+
+def test_edge_operand_extents_are_checked_before_any_launch():
+    """The fused edge kernels read P * C weights, D2 harmonics (or 3 vector components) and R radial features for
+    every edge of the plan whatever the tensors hold, so a short operand has to be a Python error, not a read past
+    the allocation.  The check runs on the host; no GPU is needed to see it refuse."""
+    import types
+
+    import pytest
+    import torch
+    from equitorch_amd import _lib
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.nn.functional import edge
+    from equitorch_amd.utils._structs import tp_infos
+
+    irreps = Irreps("0e+1o+2e")
+    info = tp_infos(irreps, irreps, irreps)[0]
+    n, e, c, r, p = 5, 12, 64, 8, 11
+    plan = types.SimpleNamespace(num_edges=e, num_src_nodes=n, num_nodes=n)
+    x, sh, vec = torch.zeros(n, 9, c), torch.zeros(e, 9), torch.zeros(e, 3)
+    h, w_last, w = torch.zeros(e, r), torch.zeros(r, p, c), torch.zeros(e, p, c)
+    edge._check_edge_operands(x, sh, plan, info, weight=w)
+    edge._check_edge_operands(x, sh, plan, info, weight=w[0])
+    edge._check_edge_operands(x, vec, plan, info, h=h, w_last=w_last, edge_vectors=True)
+    bad = [dict(x=x[:4]), dict(x=x[:, :8]), dict(y=sh[:-1]), dict(y=sh[:, :8]), dict(weight=w[:-1]),
+           dict(weight=w[:, :10]), dict(weight=w[..., :32]), dict(h=h[:-1], w_last=w_last, weight=None),
+           dict(h=h, w_last=w_last[:-1], weight=None), dict(h=h, w_last=w_last[:, :10], weight=None),
+           dict(h=h, w_last=w_last[..., :32], weight=None), dict(y=vec)]
+    for change in bad:
+        kw = dict(x=x, y=sh, weight=w, h=None, w_last=None)
+        kw.update(change)
+        with pytest.raises(_lib.CgtpError):
+            edge._check_edge_operands(kw["x"], kw["y"], plan, info, weight=kw["weight"], h=kw["h"], w_last=kw["w_last"])
+    with pytest.raises(_lib.CgtpError):
+        edge._check_edge_operands(x, sh, plan, info, h=h, w_last=w_last, edge_vectors=True)
