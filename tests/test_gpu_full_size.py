@@ -48,10 +48,13 @@ def _check_subsets(T, src, dst, x, sh, w, ct, got, n_dst, n_src, n_edge, tol=1e-
     mask = torch.zeros(n_nodes, dtype=torch.bool)
     mask[nodes] = True
     e_in = torch.nonzero(mask[dst]).flatten()
-    msg = ref_ops.dense_u1u(T, x[src[e_in]], sh[e_in], w[e_in])
-    ref_out = ref_ops.scatter_sum(msg, dst[e_in], n_nodes)[nodes]
-    # rows summed over ~16 (up to hundreds at a hub) edges x all coefficients: element-wise where it holds
-    assert_close(out[nodes], ref_out, tol, f"{tag} out rows", norm="max")
+    def out_rows(dt):   # float64: the arbiter; float32: what the same sums lose in the reference's own arithmetic
+        msg = ref_ops.dense_u1u(T, x[src[e_in]], sh[e_in], w[e_in], dtype=dt)
+        return ref_ops.scatter_sum(msg, dst[e_in], n_nodes)[nodes]
+    # rows summed over ~16 (up to hundreds at a hub) edges x all coefficients: norm-wise, and within three times the fp32
+    # restatement's own error
+    assert_close(out[nodes], out_rows(torch.float64), tol, f"{tag} out rows", norm="max",
+                 fp32_ref=out_rows(torch.float32))
     # grad_x rows: all out-edges of a strided set of nodes; grad_sh / grad_w: those edges and a strided set of edges
     nodes = torch.unique(torch.cat([torch.arange(5, n_nodes, max(1, n_nodes // n_src)), torch.tensor([0, n_nodes - 1])]))
     mask = torch.zeros(n_nodes, dtype=torch.bool)
@@ -60,12 +63,15 @@ def _check_subsets(T, src, dst, x, sh, w, ct, got, n_dst, n_src, n_edge, tol=1e-
     emask[torch.arange(7, n_edges, max(1, n_edges // n_edge))] = True
     emask[0] = emask[n_edges - 1] = True
     e_sub = torch.nonzero(emask).flatten()
-    xr = x.double().requires_grad_(True)
-    shr, wr = sh[e_sub].double().requires_grad_(True), w[e_sub].double().requires_grad_(True)
-    loss = (ref_ops.dense_u1u(T, xr[src[e_sub]], shr, wr) * ct[dst[e_sub]].double()).sum()
-    rgx, rgsh, rgw = torch.autograd.grad(loss, (xr, shr, wr))
-    assert_close(gx[nodes], rgx[nodes], tol, f"{tag} grad_x rows", norm="max")
-    assert_close(gsh[e_sub], rgsh, tol, f"{tag} grad_sh rows", norm="max")
+    def grads(dt):
+        xr = x.detach().to(dt).clone().requires_grad_(True)
+        shr, wr = sh[e_sub].detach().to(dt).clone().requires_grad_(True), w[e_sub].detach().to(dt).clone().requires_grad_(True)
+        loss = (ref_ops.dense_u1u(T, xr[src[e_sub]], shr, wr, dtype=dt) * ct[dst[e_sub]].to(dt)).sum()
+        return torch.autograd.grad(loss, (xr, shr, wr))
+    rgx, rgsh, rgw = grads(torch.float64)
+    gx32, gsh32, _ = grads(torch.float32)
+    assert_close(gx[nodes], rgx[nodes], tol, f"{tag} grad_x rows", norm="max", fp32_ref=gx32[nodes])
+    assert_close(gsh[e_sub], rgsh, tol, f"{tag} grad_sh rows", norm="max", fp32_ref=gsh32)
     assert_close(gw[e_sub], rgw, tol, f"{tag} grad_w rows")
 
 
@@ -128,21 +134,24 @@ def test_edge_fused_full_size_vectors(device):
     out = edge_tensor_product_uu_vectors(xd, vd, wd, plan, mod.tp_info_forward)
     (out * ct.to(device)).sum().backward()
     from oracle import ref_sh
-    vr = vec.double().requires_grad_(True)
-    shr = ref_sh.spherical_harmonics(vr / vr.norm(dim=-1, keepdim=True), 2)
     T = ref_ops.dense_coupling(irr, irr, irr)
     e_sub = torch.arange(7, n_edges, 128)
-    xr, wr = x.double(), w[e_sub].double()
-    loss = (ref_ops.dense_u1u(T, xr[src[e_sub]], shr[e_sub], wr) * ct[dst[e_sub]].double()).sum()
-    (rgv,) = torch.autograd.grad(loss, vr)
-    assert_close(vd.grad.cpu()[e_sub], rgv[e_sub], 1e-5, "grad_vec rows", norm="max")
     nodes = torch.arange(3, n_nodes, 64)
     mask = torch.zeros(n_nodes, dtype=torch.bool)
     mask[nodes] = True
     e_in = torch.nonzero(mask[dst]).flatten()
-    msg = ref_ops.dense_u1u(T, xr[src[e_in]], shr.detach()[e_in], w[e_in])
-    assert_close(out.detach().cpu()[nodes], ref_ops.scatter_sum(msg, dst[e_in], n_nodes)[nodes], 1e-5,
-                 "out rows (vectors)", norm="max")
+
+    def oracle(dt):     # (grad_vec rows, out rows) with the harmonics of the oracle, in float64 and restated in float32
+        vr = vec.detach().to(dt).clone().requires_grad_(True)
+        shr = ref_sh.spherical_harmonics(vr / vr.norm(dim=-1, keepdim=True), 2)
+        loss = (ref_ops.dense_u1u(T, x.to(dt)[src[e_sub]], shr[e_sub], w[e_sub], dtype=dt) * ct[dst[e_sub]].to(dt)).sum()
+        (rgv,) = torch.autograd.grad(loss, vr)
+        msg = ref_ops.dense_u1u(T, x[src[e_in]], shr.detach()[e_in], w[e_in], dtype=dt)
+        return rgv[e_sub], ref_ops.scatter_sum(msg, dst[e_in], n_nodes)[nodes]
+    rgv, rout = oracle(torch.float64)
+    gv32, out32 = oracle(torch.float32)
+    assert_close(vd.grad.cpu()[e_sub], rgv, 1e-5, "grad_vec rows", norm="max", fp32_ref=gv32)
+    assert_close(out.detach().cpu()[nodes], rout, 1e-5, "out rows (vectors)", norm="max", fp32_ref=out32)
 
 
 def test_edge_full_size_lmax6(device):
@@ -183,13 +192,15 @@ def test_row_mode_full_size_shared_weight(device):
     gx, gsh, gw = torch.autograd.grad(out, (xd, shd, wd), ct.to(device))
     T = ref_ops.dense_coupling(irr, irr, irr)
     ref_out, (rgx, rgsh, rgw_sub) = ref_ops.dense_grads(ref_ops.dense_u1u, T, (x[sub], sh[sub], w), ct[sub])
+    _, (_, gsh32, gw32) = ref_ops.dense_grads(ref_ops.dense_u1u, T, (x[sub], sh[sub], w), ct[sub], dtype=torch.float32)
     assert_close(out[sub.to(device)], ref_out, 1e-5, "row mode out")
     assert_close(gx[sub.to(device)], rgx, 1e-5, "row mode grad_x")
-    assert_close(gsh[sub.to(device)], rgsh, 1e-5, "row mode grad_sh", norm="max")   # sums over 64 channels x 83 terms
+    # sums over 64 channels x 83 terms: norm-wise, and within three times the fp32 contraction's own loss
+    assert_close(gsh[sub.to(device)], rgsh, 1e-5, "row mode grad_sh", norm="max", fp32_ref=gsh32)
     masked = torch.zeros_like(ct)
     masked[sub] = ct[sub]
     (gw_sub,) = torch.autograd.grad(mod(xd, shd, wd), (wd,), masked.to(device))
-    assert_close(gw_sub, rgw_sub, 1e-5, "row mode grad_w of the subset", norm="max")      # sum over 256 rows
+    assert_close(gw_sub, rgw_sub, 1e-5, "row mode grad_w of the subset", norm="max", fp32_ref=gw32)   # sum over 256 rows
     # the full gradient is additive over two halves of the batch
     half = n // 2
     parts = []
@@ -226,20 +237,27 @@ def test_edge_radial_full_size(device):
     nodes = torch.arange(11, n_nodes, 173)
     # output rows of the chosen nodes: all edges that end there
     e_in = torch.nonzero(torch.isin(dst, nodes)).flatten()
-    w_in = torch.einsum("er,rpc->epc", h[e_in].double(), wl.double())
-    msg = ref_ops.dense_u1u(T, x[src[e_in]].double(), sh[e_in].double(), w_in)
-    ref_rows = ref_ops.scatter_sum(msg, dst[e_in], n_nodes)[nodes]
-    assert_close(out[nodes.to(device)], ref_rows, 1e-5, "radial full size out rows", norm="max")   # sums over ~16 edges
-    # gradients: node rows of grad_x need all edges that start there; per-edge gradients need their own edge only
     e_out = torch.nonzero(torch.isin(src, nodes)).flatten()
-    xr = x.double().requires_grad_(True)
-    shr, hr = sh[e_out].double().requires_grad_(True), h[e_out].double().requires_grad_(True)
-    w_out = torch.einsum("er,rpc->epc", hr, wl.double())
-    loss = (ref_ops.dense_u1u(T, xr[src[e_out]], shr, w_out) * ct[dst[e_out]].double()).sum()
-    rgx, rgsh, rgh = torch.autograd.grad(loss, (xr, shr, hr))
-    assert_close(gx[nodes.to(device)], rgx[nodes], 1e-5, "radial full size grad_x rows", norm="max")
-    assert_close(gsh[e_out.to(device)], rgsh, 1e-5, "radial full size grad_sh rows", norm="max")   # 64 channels x coefficients
-    assert_close(gh[e_out.to(device)], rgh, 1e-5, "radial full size grad_h rows", norm="max")      # 11 paths x 64 channels
+
+    def oracle(dt):     # out rows, grad_x rows, grad_sh and grad_h of the edges that start at the chosen nodes, in ``dt``
+        w_in = torch.einsum("er,rpc->epc", h[e_in].to(dt), wl.to(dt))
+        msg = ref_ops.dense_u1u(T, x[src[e_in]], sh[e_in], w_in, dtype=dt)
+        rows = ref_ops.scatter_sum(msg, dst[e_in], n_nodes)[nodes]
+        # gradients: node rows of grad_x need all edges that start there; per-edge gradients their own edge only
+        xr = x.detach().to(dt).clone().requires_grad_(True)
+        shr, hr = sh[e_out].detach().to(dt).clone().requires_grad_(True), h[e_out].detach().to(dt).clone().requires_grad_(True)
+        w_out = torch.einsum("er,rpc->epc", hr, wl.to(dt))
+        loss = (ref_ops.dense_u1u(T, xr[src[e_out]], shr, w_out, dtype=dt) * ct[dst[e_out]].to(dt)).sum()
+        rgx, rgsh, rgh = torch.autograd.grad(loss, (xr, shr, hr))
+        return rows, rgx[nodes], rgsh, rgh
+    ref_rows, rgx, rgsh, rgh = oracle(torch.float64)
+    rows32, gx32, gsh32, gh32 = oracle(torch.float32)
+    # sums over ~16 edges (rows), 64 channels x coefficients (grad_sh), 11 paths x 64 channels (grad_h): norm-wise, and
+    # within three times what the same computation loses in fp32
+    assert_close(out[nodes.to(device)], ref_rows, 1e-5, "radial full size out rows", norm="max", fp32_ref=rows32)
+    assert_close(gx[nodes.to(device)], rgx, 1e-5, "radial full size grad_x rows", norm="max", fp32_ref=gx32)
+    assert_close(gsh[e_out.to(device)], rgsh, 1e-5, "radial full size grad_sh rows", norm="max", fp32_ref=gsh32)
+    assert_close(gh[e_out.to(device)], rgh, 1e-5, "radial full size grad_h rows", norm="max", fp32_ref=gh32)
     # grad of the shared matrix: additivity over two halves of the edge list (each half its own plan)
     parts = []
     for lo, hi in ((0, n_edges // 2), (n_edges // 2, n_edges)):

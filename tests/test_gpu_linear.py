@@ -46,11 +46,16 @@ def test_irreps_linear_matches_oracle(device, io, ii, kw, shared, dtype):
     out = mod(xd, wd)
     gx, gw = _grads(out, (xd, wd), ct.to(device, dtype))
     tol = 1e-5 if dtype == torch.float32 else 1e-12
-    for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
+    # the same CPU function on float32 tensors: what the reference's own fp32 arithmetic loses
+    x32, w32 = x.float().requires_grad_(True), w.float().requires_grad_(True)
+    ref32 = ref_ops.cpu_irreps_linear(x32, w32, info)
+    r32 = (ref32, *_grads(ref32, (x32, w32), ct.float()))
+    for (name, a, b), b32 in zip((("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)), r32):
         # channel_norm as the reference passes it (channel_scale = C_in) gives terms of order 10^2 that cancel:
-        # that case is compared norm-wise in fp32
+        # that case is compared norm-wise in fp32, and held to three times the fp32 restatement's own error
         big = bool(kw.get("channel_norm")) and dtype == torch.float32
-        assert_close(a, b, tol=tol, what=f"{io}<-{ii} shared={shared} {name}", norm="max" if big else "element")
+        assert_close(a, b, tol=tol, what=f"{io}<-{ii} shared={shared} {name}", norm="max" if big else "element",
+                     fp32_ref=b32 if big else None)
 
 
 @pytest.mark.parametrize("shared", [True, False])

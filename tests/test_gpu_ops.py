@@ -107,8 +107,8 @@ def test_row_sums_beyond_1024_rows(device, tables13, table, n, channels, dtype):
     ct = torch.randn(n, info_r["seg_out"].shape[0] - 1, channels, generator=g, dtype=torch.float64).to(dtype)
     (gw,) = torch.autograd.grad(F.sparse_mul(x.to(device), wd, info_m), (wd,), ct.to(device))
     def shared_grad(dt):
-        wr = w.to(dt).requires_grad_(True)
-        info = {k: (v.to(dt) if v is not None and v.is_floating_point() else v) for k, v in info_r.items()}
+        wr = w.detach().to(dt).clone().requires_grad_(True)
+        info = {k: (v.to(dt) if isinstance(v, torch.Tensor) and v.is_floating_point() else v) for k, v in info_r.items()}
         return torch.autograd.grad(ref_ops.cpu_mul(x.to(dt), wr, info), (wr,), ct.to(dt))[0]
     assert_close(gw, shared_grad(torch.float64), tol, "shared-operand gradient", norm="max",
                  fp32_ref=shared_grad(torch.float32) if dtype == torch.float32 else None)
@@ -143,7 +143,7 @@ def test_matrix_ops_sweep(device, tables13, op, shared1, shared2, acc):
     eq = eq.format(a="" if shared1 else "n", b="" if shared2 else "n", o="" if (shared1 and shared2) else "n")
 
     def dense(dt):      # the dense contraction in float64 (the arbiter) and in float32 (what fp32 arithmetic loses)
-        xr, yr = (t.float().to(dt).requires_grad_(True) for t in (x, y))
+        xr, yr = (t.float().detach().to(dt).clone().requires_grad_(True) for t in (x, y))
         o = torch.einsum(eq, T.to(dt), xr, yr)
         return (o.sum(0) if acc else o), xr, yr
     ref_out, xr, yr = dense(torch.float64)
@@ -197,7 +197,7 @@ def test_shared_matrix_ops_on_the_matrix_core_kernels(device, monkeypatch, op, d
 
     def dense(dt):      # (out, grad1, grad2) of the dense contraction carried out in ``dt``
         nonlocal ct
-        xr, yr = (t.to(dtype).to(dt).requires_grad_(True) for t in (x, y))
+        xr, yr = (t.to(dtype).detach().to(dt).clone().requires_grad_(True) for t in (x, y))
         o = torch.einsum(eq, T.to(dt), xr, yr)
         if ct is None:
             ct = torch.randn(o.shape, generator=g, dtype=torch.float64).to(dtype)
@@ -244,7 +244,7 @@ def test_matrix_core_route_random_shapes(device, case):
     ct = torch.randn(n, n_out, cw, generator=g, dtype=torch.float64).to(dtype)
 
     def dense(dt):      # (out, grad vector, grad matrix) of the dense contraction carried out in ``dt``
-        xr, mr = (t.to(dt).requires_grad_(True) for t in (x, m))
+        xr, mr = (t.detach().to(dt).clone().requires_grad_(True) for t in (x, m))
         o = torch.einsum("mab,nau,buw->nmw", T.to(dt), xr, mr)
         return (o, *torch.autograd.grad(o, (xr, mr), ct.to(dt)))
     ref_out, rgx, rgm = dense(torch.float64)

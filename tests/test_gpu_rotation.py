@@ -122,13 +122,19 @@ def test_so2_linear_uv_fp32_on_the_matrix_core_kernels(device, cin, cout, n):
     finally:
         _uv_native.apply = orig
     assert calls, "the layer did not run on the table-driven kernels"
-    for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
+    def second_order(xs, ws, cts):
+        return torch.autograd.grad(torch.autograd.grad(ref_ops.cpu_so2_linear(xs, ws, info, per_sample=False), ws, cts,
+                                                       create_graph=True)[0].sum(), xs)[0]
+    # the same CPU function on float32 tensors: what the reference's own fp32 arithmetic loses
+    x32, w32 = x.float().requires_grad_(True), w.float().requires_grad_(True)
+    ref32 = ref_ops.cpu_so2_linear(x32, w32, info, per_sample=False)
+    r32 = (ref32, *torch.autograd.grad(ref32, (x32, w32), ct.float()))
+    for (name, a, b), b32 in zip((("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)), r32):
         # sums over C_in (x paths) products; grad_w also over the batch
-        assert_close(a, b, tol=1e-5, what=f"SO2Linear uv fp32 {cin}->{cout} {name}", norm="max")
+        assert_close(a, b, tol=1e-5, what=f"SO2Linear uv fp32 {cin}->{cout} {name}", norm="max", fp32_ref=b32)
     (ggx,) = torch.autograd.grad(gw.sum(), (xd,))          # second order through the differentiable route
-    (rggx,) = torch.autograd.grad(torch.autograd.grad(ref_ops.cpu_so2_linear(xr, wr, info, per_sample=False), wr, ct,
-                                                      create_graph=True)[0].sum(), xr)
-    assert_close(ggx, rggx, tol=1e-5, what="SO2Linear uv fp32 d(grad_w)/dx", norm="max")
+    assert_close(ggx, second_order(xr, wr, ct), tol=1e-5, what="SO2Linear uv fp32 d(grad_w)/dx", norm="max",
+                 fp32_ref=second_order(x32, w32, ct.float()))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])

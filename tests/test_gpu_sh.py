@@ -56,9 +56,15 @@ def test_backward_matches_oracle_autograd(device, l_max, normalize, dtype):
     (out * ct.to(device, dtype)).sum().backward()
     tol = 1e-11 if dtype == torch.float64 else 1e-5
     assert_close(out, ref, tol=tol, what="Y")
-    # the gradient sums (l_max + 1)^2 polynomial derivatives per component: norm-wise above degree 8 in fp32
-    assert_close(vd.grad, v.grad, tol=tol, what="grad_xyz",
-                 norm="max" if (l_max > 8 and dtype == torch.float32) else "element")
+    # the gradient sums (l_max + 1)^2 polynomial derivatives per component: norm-wise above degree 8 in fp32, and
+    # within three times what the oracle's own recursion loses when it runs in fp32
+    long_sum = l_max > 8 and dtype == torch.float32
+    g32 = None
+    if long_sum:
+        v32 = v.detach().float().requires_grad_(True)
+        (scale * ref_sh.spherical_harmonics(ref_sh.normalize(v32) if normalize else v32, l_max) * ct.float()).sum().backward()
+        g32 = v32.grad
+    assert_close(vd.grad, v.grad, tol=tol, what="grad_xyz", norm="max" if long_sum else "element", fp32_ref=g32)
 
 
 def test_module_layout_options_and_edge_cases(device):
@@ -137,19 +143,24 @@ def test_edge_product_with_harmonics_evaluated_in_the_kernel(device, lmax, chann
     if dtype == torch.float64:
         T = T.float().double()          # the compiled tables hold the reference's fp32 coefficients
     x, ct, w = rd(n_nodes, d, channels), rd(n_nodes, d, channels), rd(n_edges, mod.num_paths, channels)
-    xr, vr, wr = (t.clone().requires_grad_(True) for t in (x, vec, w))
-    sh = ref_sh.spherical_harmonics(ref_sh.normalize(vr) if normalize else vr, lmax)
-    ref = ref_ops.scatter_sum(ref_ops.dense_u1u(T, xr[src], sh, wr), dst, n_nodes)
-    (ref * ct).sum().backward()
+    def oracle(dt):
+        xs, vs, ws = (t.detach().to(dt).clone().requires_grad_(True) for t in (x, vec, w))
+        ys = ref_sh.spherical_harmonics(ref_sh.normalize(vs) if normalize else vs, lmax)
+        res = ref_ops.scatter_sum(ref_ops.dense_u1u(T, xs[src], ys, ws, dtype=dt), dst, n_nodes)
+        (res * ct.to(dt)).sum().backward()
+        return res.detach(), xs.grad, vs.grad, ws.grad
+    want = oracle(torch.float64)
+    gv32 = oracle(torch.float32)[2] if dtype == torch.float32 else None
     plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
     xd, vd, wd = (t.to(device, dtype).requires_grad_(True) for t in (x, vec, w))
     out = edge_tensor_product_uu_vectors(xd, vd, wd, plan, mod.tp_info_forward, normalize_input=normalize)
     (out * ct.to(device, dtype)).sum().backward()
     tol = 1e-5 if dtype == torch.float32 else 1e-11
-    for name, a, b in (("out", out, ref), ("grad_x", xd.grad, xr.grad), ("grad_vec", vd.grad, vr.grad),
-                       ("grad_w", wd.grad, wr.grad)):
-        # grad_vec: a sum over all channels and coefficients pushed through the harmonics' derivative
-        assert_close(a, b, tol=tol, what=f"lmax={lmax} {name}", norm="max" if name == "grad_vec" else "element")
+    for name, a, b in zip(("out", "grad_x", "grad_vec", "grad_w"), (out, xd.grad, vd.grad, wd.grad), want):
+        # grad_vec: a sum over all channels and coefficients pushed through the harmonics' derivative — norm-wise, and
+        # within three times what the oracle's own chain loses in fp32
+        assert_close(a, b, tol=tol, what=f"lmax={lmax} {name}", norm="max" if name == "grad_vec" else "element",
+                     fp32_ref=gv32 if name == "grad_vec" else None)
 
 
 def test_add_spherical_harmonics_transform(device):

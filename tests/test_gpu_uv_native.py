@@ -95,8 +95,12 @@ def test_u1v_fp32_native(device, irreps, cin, cout, n, kw):
     T = ref_ops.dense_coupling(io, i1, i2, path_norm=kw.get("path_norm", True),
                                channel_norm=kw.get("channel_norm", False), channel_scale=cin ** -0.5).float().double()
     ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x, y, w), ct)
-    for name, a, b in zip(("out", "grad_x", "grad_y", "grad_w"), (out, gx, gy, gw), (ref_out, *ref_grads)):
-        assert_close(a, b, 1e-5, f"u1v {io} C={cin}->{cout} N={n} {name}", norm="max")
+    out32, grads32 = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x, y, w), ct, dtype=torch.float32)
+    for name, a, b, r in zip(("out", "grad_x", "grad_y", "grad_w"), (out, gx, gy, gw), (ref_out, *ref_grads),
+                             (out32, *grads32)):
+        # sums over C_in x paths products (the weight's over the batch too): norm-wise, and within three times what the
+        # same contraction loses in fp32 arithmetic
+        assert_close(a, b, 1e-5, f"u1v {io} C={cin}->{cout} N={n} {name}", norm="max", fp32_ref=r)
 
 
 UVW_CASES = [  # irreps, (U, V, W), N
@@ -128,8 +132,10 @@ def test_uvw_fp32_native(device, irreps, channels, n):
     out = F.tensor_product_uvw(xd, yd, wd, *infos)
     gx, gy, gw = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
     ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_uvw, T, (x, y, w), ct)
-    for name, a, b in zip(("out", "grad_x", "grad_y", "grad_w"), (out, gx, gy, gw), (ref_out, *ref_grads)):
-        assert_close(a, b, 1e-5, f"uvw {channels} N={n} {name}", norm="max")
+    out32, grads32 = ref_ops.dense_grads(ref_ops.dense_uvw, T, (x, y, w), ct, dtype=torch.float32)
+    for name, a, b, r in zip(("out", "grad_x", "grad_y", "grad_w"), (out, gx, gy, gw), (ref_out, *ref_grads),
+                             (out32, *grads32)):
+        assert_close(a, b, 1e-5, f"uvw {channels} N={n} {name}", norm="max", fp32_ref=r)
 
 
 def test_u1v_fp32_native_full_size(device):
@@ -150,8 +156,9 @@ def test_u1v_fp32_native_full_size(device):
     (gx,) = torch.autograd.grad(out, (xd,), ct.to(device))
     T = ref_ops.dense_coupling(irr, irr, irr).float().double()
     ref_out, (rgx, _, _) = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x[sub], y[sub], w), ct[sub])
-    assert_close(out[sub.to(device)], ref_out, 1e-5, "full size out", norm="max")
-    assert_close(gx[sub.to(device)], rgx, 1e-5, "full size grad_x", norm="max")
+    out32, (gx32, _, _) = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x[sub], y[sub], w), ct[sub], dtype=torch.float32)
+    assert_close(out[sub.to(device)], ref_out, 1e-5, "full size out", norm="max", fp32_ref=out32)
+    assert_close(gx[sub.to(device)], rgx, 1e-5, "full size grad_x", norm="max", fp32_ref=gx32)
 
 
 def test_u1v_fp32_full_size_properties(device):
@@ -178,11 +185,15 @@ def test_u1v_fp32_full_size_properties(device):
     gx, gy, gw = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
     T = ref_ops.dense_coupling(irreps, irreps, irreps).float().double()
     ref_out, (rgx, rgy, rgw_sub) = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x[sub], y[sub], w), ct[sub])
+    out32, (gx32, gy32, gw32) = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x[sub], y[sub], w), ct[sub],
+                                                    dtype=torch.float32)
     sd = sub.to(device)
-    for name, a, b in (("out", out[sd], ref_out), ("grad_x", gx[sd], rgx), ("grad_y", gy[sd], rgy)):
-        assert_close(a, b, 1e-5, f"u1v fp32 full size {name} rows", norm="max")   # sums over 128 channels x paths
+    for name, a, b, r in (("out", out[sd], ref_out, out32), ("grad_x", gx[sd], rgx, gx32),
+                          ("grad_y", gy[sd], rgy, gy32)):
+        # sums over 128 channels x paths: norm-wise, and within three times the fp32 contraction's own loss
+        assert_close(a, b, 1e-5, f"u1v fp32 full size {name} rows", norm="max", fp32_ref=r)
     (gw_sub,) = torch.autograd.grad(mod(xd, yd, wd), (wd,), (ct * mask).to(device))
-    assert_close(gw_sub, rgw_sub, 1e-5, "u1v fp32 full size grad_w of the subset", norm="max")
+    assert_close(gw_sub, rgw_sub, 1e-5, "u1v fp32 full size grad_w of the subset", norm="max", fp32_ref=gw32)
     half = n // 2
     parts = []
     for lo, hi in ((0, half), (half, n)):
