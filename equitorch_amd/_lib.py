@@ -62,6 +62,12 @@ class UvuArgs(C.Structure):
                 ("wave_pos", C.c_void_p)]
 
 
+class UvuTab(C.Structure):
+    _fields_ = [("coef", C.c_void_p), ("idx", C.c_void_p), ("paths", C.c_void_p),
+                ("nnz", C.c_int32), ("n_segments", C.c_int32),
+                ("D1", C.c_int32), ("D2", C.c_int32), ("DO", C.c_int32), ("P", C.c_int32)]
+
+
 class UvtItem(C.Structure):
     _fields_ = [("p", C.c_int32), ("kb0", C.c_int32), ("nkb", C.c_int32), ("t0", C.c_int32), ("t1", C.c_int32),
                 ("out_row", C.c_int32), ("flags", C.c_int32), ("reserved_", C.c_int32)]
@@ -134,6 +140,11 @@ def _load():
     lib.cgtp_uvu_workspace_bytes.argtypes = [C.POINTER(UvuArgs), C.c_int]
     lib.cgtp_uvu_fwd.argtypes = [C.POINTER(UvuArgs), C.c_void_p]
     lib.cgtp_uvu_bwd.argtypes = [C.POINTER(UvuArgs), C.c_void_p]
+    lib.cgtp_uvu_tab_workspace_bytes.restype = C.c_int64
+    lib.cgtp_uvu_tab_workspace_bytes.argtypes = [C.POINTER(UvuArgs), C.POINTER(UvuTab), C.c_int]
+    lib.cgtp_uvu_tab_validate.argtypes = [C.POINTER(UvuArgs), C.POINTER(UvuTab), C.c_int]
+    lib.cgtp_uvu_tab_fwd.argtypes = [C.POINTER(UvuArgs), C.POINTER(UvuTab), C.c_void_p]
+    lib.cgtp_uvu_tab_bwd.argtypes = [C.POINTER(UvuArgs), C.POINTER(UvuTab), C.c_void_p]
     lib.cgtp_uv_find.argtypes = [C.c_uint64]
     lib.cgtp_uv_find_rounded.argtypes = [C.c_uint64, C.c_int]
     _uv = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32,

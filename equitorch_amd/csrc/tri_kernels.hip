@@ -614,12 +614,18 @@ int cgtp_abi_layout(int which, int64_t* out, int capacity) {
                                    CGTP_OFF(cgtp_uvt_gy_args, dy), CGTP_OFF(cgtp_uvt_gy_args, dg),
                                    CGTP_OFF(cgtp_uvt_gy_args, cx), CGTP_OFF(cgtp_uvt_gy_args, cout),
                                    CGTP_OFF(cgtp_uvt_gy_args, dtype)};
+  static const int64_t uvu_tab[] = {sizeof(cgtp_uvu_tab), CGTP_OFF(cgtp_uvu_tab, coef), CGTP_OFF(cgtp_uvu_tab, idx),
+                                    CGTP_OFF(cgtp_uvu_tab, paths),
+                                    CGTP_OFF(cgtp_uvu_tab, nnz), CGTP_OFF(cgtp_uvu_tab, n_segments),
+                                    CGTP_OFF(cgtp_uvu_tab, D1), CGTP_OFF(cgtp_uvu_tab, D2),
+                                    CGTP_OFF(cgtp_uvu_tab, DO), CGTP_OFF(cgtp_uvu_tab, P)};
 #undef CGTP_OFF
-  const int64_t* tabs[] = {operand, tri, gen_operand, gen, uvu, uvt_item, uvt, uvt_gw, uvt_gy};
+  const int64_t* tabs[] = {operand, tri, gen_operand, gen, uvu, uvt_item, uvt, uvt_gw, uvt_gy, uvu_tab};
   const int counts[] = {(int)(sizeof(operand) / 8), (int)(sizeof(tri) / 8), (int)(sizeof(gen_operand) / 8),
                         (int)(sizeof(gen) / 8), (int)(sizeof(uvu) / 8), (int)(sizeof(uvt_item) / 8),
-                        (int)(sizeof(uvt) / 8), (int)(sizeof(uvt_gw) / 8), (int)(sizeof(uvt_gy) / 8)};
-  if (which < 0 || which >= 9) return -1;
+                        (int)(sizeof(uvt) / 8), (int)(sizeof(uvt_gw) / 8), (int)(sizeof(uvt_gy) / 8),
+                        (int)(sizeof(uvu_tab) / 8)};
+  if (which < 0 || which >= 10) return -1;
   for (int i = 0; out && i < counts[which] && i < capacity; ++i) out[i] = tabs[which][i];
   return counts[which];
 }

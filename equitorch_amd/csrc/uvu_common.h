@@ -97,6 +97,12 @@ const UvuRadialEntry* uvu_radial_entries(int* count);
 constexpr int kRadialMaxR = 16;
 constexpr int kRadialC = 64;
 
+// The fix-up pass of the segment kernels for callers outside their translation unit: adds the partial rows
+// ws[(range, 2, row_len)] of the segments that span several ranges (ranges of `per_range` sorted positions each) in
+// range order, and writes zero rows for empty segments.  Status code.
+int uvu_fixup_rows_f32(float* rows, const float* ws, const int64_t* ptr, int64_t n_seg, int64_t row_len, int per_range,
+                       int64_t n_ranges, int64_t n_rows, hipStream_t stream);
+
 const UvuBigEntry* uvu_big_entries(int* count);
 const UvuBigEntry* uvu_big_entries_scaled(int* count);  // the same kernels applying UvuDev::ps
 

@@ -885,6 +885,13 @@ static int launch_fixup(T* rows, const UvuDev<T>& d, int64_t row_len, hipStream_
   return launched();
 }
 
+int uvu_fixup_rows_f32(float* rows, const float* ws, const int64_t* ptr, int64_t n_seg, int64_t row_len, int per_range,
+                       int64_t n_ranges, int64_t n_rows, hipStream_t stream) {
+  hipLaunchKernelGGL(uvu_fixup_kernel<float>, dim3((unsigned)((n_seg + 3) / 4)), dim3(256), 0, stream, rows, ws, ptr,
+                     n_seg, row_len, per_range, (const int64_t*)nullptr, n_ranges, n_rows);
+  return launched();
+}
+
 static int launch_big(const cgtp_uvu_args* a, const UvuPlan& plan, int backward, hipStream_t stream) {
   int n_big = 0;
   const UvuBigEntry& e = (a->path_scale ? uvu_big_entries_scaled(&n_big) : uvu_big_entries(&n_big))[plan.big_idx];

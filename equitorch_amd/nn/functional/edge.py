@@ -148,6 +148,26 @@ class _EdgeUvuRadial(Function):
         return (*res, None, None, None)
 
 
+class _EdgeUvuTable(Function):
+    """Gather, product and segment sum in one launch for a table that is not compiled in: the table-driven segment
+    kernels (``cgtp_uvu_tab_fwd`` / ``cgtp_uvu_tab_bwd``), tables read through the scalar cache, the per-edge
+    operands and the segment sums in LDS."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, sh: Tensor, w: Tensor, plan: EdgePlan, tab):
+        out = kernels.uvu_tab_forward(tab, x, sh, w, plan.fwd_index)
+        ctx.save_for_backward(x, sh, w)
+        ctx.plan, ctx.tab = plan, tab
+        return out
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, g):
+        x, sh, w = ctx.saved_tensors
+        res = kernels.uvu_tab_backward(ctx.tab, x, sh, w, g.contiguous(), ctx.needs_input_grad[:3], ctx.plan.bwd_index)
+        return (*res, None, None)
+
+
 class _EdgeUvuRows(Function):
     """The same composition on the row-mode kernels, for tables the fused segment kernels do not cover: per-edge
     messages from the gathered node rows, then a segment sum over the dst-sorted list; the backward forms the
@@ -200,6 +220,13 @@ def edge_tensor_product_uu(x: Tensor, sh: Tensor, weight: Tensor, plan: EdgePlan
         if kernels.uvu_launchable(cfg, xc, yc, wc, gathered=True):
             kernels.log_tier("edge_tensor_product_uu", "block-wise row kernels + segment sums", f"config {int(cfg)}")
             return _EdgeUvuRows.apply(xc, yc, wc, plan, tp_info_forward, cfg)
+    if x.dtype == sh.dtype == weight.dtype == torch.float32:
+        tab = kernels.uvu_table_of(tp_info_forward, x.device)
+        xc, yc, wc = x.contiguous(), sh.contiguous(), weight.contiguous()
+        if kernels.uvu_tab_launchable(tab, xc, yc, wc, weight.requires_grad and torch.is_grad_enabled()):
+            kernels.log_tier("edge_tensor_product_uu", "table-driven fused gather / product / segment sum",
+                             f"{tab.nnz} coefficients")
+            return _EdgeUvuTable.apply(xc, yc, wc, plan, tab)
     kernels.log_tier("edge_tensor_product_uu", "index_select + tensor_product_u1u + sparse_scale")
     msg = tensor_product_u1u(x.index_select(0, plan.src), sh, weight, tp_info_forward)
     e, d, c = msg.shape

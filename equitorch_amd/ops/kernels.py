@@ -714,6 +714,114 @@ def uvu_radial_backward(cfg: int, dims, x: Tensor, y: Tensor, h: Tensor, w_eff: 
     return gx, gy, gh, gwl
 
 
+# ---- channel-wise product over an edge list for a table that is not compiled in ------------------------------------
+class UvuTable:
+    """A ``TensorProductInfo`` as the data the table-driven segment kernels read: entries sorted by (path, output
+    row), one (path, output row) segment per run; device arrays and the ``cgtp_uvu_tab`` descriptor over them."""
+
+    def __init__(self, coo, device):
+        order = np.lexsort((coo.M2, coo.M1, coo.M, coo.p))          # by path, then output row, then table order
+        p, m = coo.p[order].astype(np.int64), coo.M[order].astype(np.int64)
+        nnz = int(order.shape[0])
+        padded = (nnz + 63) // 64 * 64 + 128         # whole 64-entry chunks, and two more the walk reads ahead into
+        key = p * (int(coo.DO) + 1) + m
+        last_of_seg = np.concatenate([key[1:] != key[:-1], [True]])
+        last_of_path = np.concatenate([p[1:] != p[:-1], [True]])
+        idx = np.zeros(padded, dtype=np.uint32)
+        idx[:nnz] = (coo.M1[order].astype(np.uint32) | (coo.M2[order].astype(np.uint32) << 8)
+                     | (last_of_seg.astype(np.uint32) << 16) | (last_of_path.astype(np.uint32) << 17)
+                     | (m.astype(np.uint32) << 18))
+        coef = np.zeros(padded, dtype=np.float32)
+        coef[:nnz] = coo.coef[order]
+        walk = p[np.concatenate([[True], p[1:] != p[:-1]])]          # the paths in walk order
+        paths = np.concatenate([walk, [0xffff, 0xffff]]).astype(np.uint32)
+        self.dims = (int(coo.D1), int(coo.D2), int(coo.DO), int(coo.P))
+        self.nnz, self.n_segments = nnz, int(last_of_seg.sum())
+        self.coef = torch.from_numpy(coef).to(device)
+        self.idx = torch.from_numpy(idx.view(np.int32).copy()).to(device)
+        self.paths = torch.from_numpy(paths.view(np.int32).copy()).to(device)
+        t = _lib.UvuTab()
+        t.coef, t.idx, t.paths = (v.data_ptr() for v in (self.coef, self.idx, self.paths))
+        t.nnz, t.n_segments = self.nnz, self.n_segments
+        t.D1, t.D2, t.DO, t.P = self.dims
+        self.c = t
+
+
+def uvu_table_of(tp_info, device) -> Optional[UvuTable]:
+    """The table of ``tp_info`` for the table-driven segment kernels (cached on the info), or None when it does not
+    fit them (a row index past 255, more than 8192 entries)."""
+    def build():
+        coo = coo_of(tp_info)
+        if max(coo.D1, coo.D2, coo.DO) > 255 or coo.P > 65534 or coo.coef.shape[0] > 8192 \
+                or coo.coef.shape[0] == 0:
+            return False
+        return UvuTable(coo, device)
+    tab = cached(tp_info.info_Mij_fwd.scale, ("uvu_table", str(device)), build)
+    return tab or None
+
+
+def _uvu_tab_args(x: Tensor, y: Tensor, w: Tensor, seg: SegIndex) -> UvuArgs:
+    a = UvuArgs()
+    a.cfg, a.dtype, a.C = -1, _lib.dtype_code(x.dtype), x.shape[-1]
+    a.w_shared = int(w.ndim == 2)
+    a.n_rows, a.n_x_rows = y.shape[0], x.shape[0]
+    a.n_seg = seg.ptr.shape[0] - 1
+    a.ptr, a.perm, a.seg_ids, a.gather = seg.ptr.data_ptr(), _lib.ptr(seg.perm), seg.seg_ids.data_ptr(), \
+        seg.gather.data_ptr()
+    a.x, a.y, a.w = x.data_ptr(), y.data_ptr(), w.data_ptr()
+    return a
+
+
+def uvu_tab_launchable(tab: Optional[UvuTable], x: Tensor, y: Tensor, w: Tensor, need_grad_w: bool) -> bool:
+    """Whether the table-driven segment kernels take these operands in both directions (fp32, up to 256 channels — 64
+    unless a multiple of 4 and aligned —, per-edge weights or a shared weight that needs no gradient)."""
+    if tab is None or x.dtype != torch.float32 or not (x.dtype == y.dtype == w.dtype):
+        return False
+    if x.shape[0] == 0 or y.shape[0] == 0 or y.ndim != 2 or (w.ndim == 2 and need_grad_w):
+        return False
+    a = UvuArgs()
+    a.dtype, a.C, a.w_shared = _lib.F32, x.shape[-1], int(w.ndim == 2)
+    a.n_rows, a.n_x_rows, a.n_seg = y.shape[0], x.shape[0], x.shape[0]
+    dummy = 256
+    a.ptr = a.seg_ids = a.gather = a.out = a.grad_out = a.grad_x = a.grad_y = dummy
+    a.x, a.y, a.w = x.data_ptr() or dummy, y.data_ptr() or dummy, w.data_ptr() or dummy
+    return all(_lib.lib.cgtp_uvu_tab_validate(C.byref(a), C.byref(tab.c), d) == 0 for d in (0, 1))
+
+
+def _uvu_tab_workspace(a: UvuArgs, tab: UvuTable, backward: int, device):
+    nbytes = int(_lib.lib.cgtp_uvu_tab_workspace_bytes(C.byref(a), C.byref(tab.c), backward))
+    if nbytes < 0:
+        _lib.check(_lib.lib.cgtp_uvu_tab_validate(C.byref(a), C.byref(tab.c), backward), "cgtp_uvu_tab_validate")
+    if nbytes <= 0:
+        return None
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    a.workspace = ws.data_ptr()
+    return ws
+
+
+def uvu_tab_forward(tab: UvuTable, x: Tensor, y: Tensor, w: Tensor, seg: SegIndex) -> Tensor:
+    """``out[s] = sum_{q in segment s} TP(x[seg.gather[q]], y[e_q], w[e_q])`` for any table, one launch."""
+    a = _uvu_tab_args(x, y, w, seg)
+    out = torch.empty((a.n_seg, tab.dims[2], x.shape[-1]), dtype=x.dtype, device=x.device)
+    a.out = out.data_ptr()
+    ws = _uvu_tab_workspace(a, tab, 0, x.device)
+    _lib.check(_lib.lib.cgtp_uvu_tab_fwd(C.byref(a), C.byref(tab.c), _lib.stream_ptr(x.device)), "cgtp_uvu_tab_fwd")
+    return out
+
+
+def uvu_tab_backward(tab: UvuTable, x: Tensor, y: Tensor, w: Tensor, g: Tensor, need, seg: SegIndex):
+    """-> (grad_x, grad_y, grad_w) over the list sorted by the other end (``seg``: segments = rows of x)."""
+    a = _uvu_tab_args(x, y, w, seg)
+    a.grad_out = g.data_ptr()
+    gx = torch.empty_like(x) if need[0] else None
+    gy = torch.empty_like(y) if need[1] else None
+    gw = torch.empty_like(w) if need[2] else None
+    a.grad_x, a.grad_y, a.grad_w = _lib.ptr(gx), _lib.ptr(gy), _lib.ptr(gw)
+    ws = _uvu_tab_workspace(a, tab, 1, x.device)
+    _lib.check(_lib.lib.cgtp_uvu_tab_bwd(C.byref(a), C.byref(tab.c), _lib.stream_ptr(x.device)), "cgtp_uvu_tab_bwd")
+    return gx, gy, gw
+
+
 def uvu_sh_degree(cfg: int) -> int:
     """Degree L when the fused kernels of ``cfg`` can evaluate the second operand from edge vectors, else -1."""
     return int(_lib.lib.cgtp_uvu_sh_degree(cfg))

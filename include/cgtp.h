@@ -42,7 +42,7 @@ int cgtp_version(void);
  * in declaration order to out[0 .. capacity) and returns how many numbers the full description has (-1: bad id). */
 enum { CGTP_LAYOUT_OPERAND = 0, CGTP_LAYOUT_TRI_ARGS = 1, CGTP_LAYOUT_GEN_OPERAND = 2, CGTP_LAYOUT_GEN_ARGS = 3,
        CGTP_LAYOUT_UVU_ARGS = 4, CGTP_LAYOUT_UVT_ITEM = 5, CGTP_LAYOUT_UVT_ARGS = 6, CGTP_LAYOUT_UVT_GW_ARGS = 7,
-       CGTP_LAYOUT_UVT_GY_ARGS = 8 };
+       CGTP_LAYOUT_UVT_GY_ARGS = 8, CGTP_LAYOUT_UVU_TABLE = 9 };
 int cgtp_abi_layout(int which, int64_t* out, int capacity);
 
 /* ---- generic sparse trilinear contraction -------------------------------------------------------------
@@ -269,6 +269,39 @@ int64_t cgtp_uvu_radial_grad_workspace_bytes(int64_t n_rows, int32_t radial_r, i
 int cgtp_uvu_radial_grad(const void* grad_w, const void* radial_h, const void* radial_w, void* grad_radial_h,
                          void* grad_radial_w, void* workspace, int64_t n_rows, int32_t radial_r, int32_t n_paths,
                          int32_t dtype, void* stream);
+
+/* ---- channel-wise product over an edge list for a table that is not compiled in ---------------------------
+ *
+ * The same fused launch as cgtp_uvu_fwd / cgtp_uvu_bwd in segment mode — gather at one end of the edge, product,
+ * segment sum at the other, no per-edge messages in memory, no atomics — for ANY table, handed over as data and
+ * read by the kernels through the scalar cache, with the per-edge operands and the segment sums in LDS.  Replaces,
+ * for irreps without a compiled table, the reference's composition of index_select, the table-driven product
+ * kernels (equitorch/ops/batched_sparse_dense_op.py:63-152, 1578-1662 behind equitorch/nn/functional/linears.py:16-93)
+ * and indexed_scale_segment (equitorch/ops/indexed_scale_segment_op.py:7-108).
+ *
+ * `a` is read as in segment mode with ranges by position: dtype CGTP_F32, n_seg > 0, ptr / seg_ids / gather (and
+ * perm) given, C <= 256 (<= 64 unless C is a multiple of 4 and the operands are 16-byte aligned), harmonics given
+ * (y_vec, y_channels, radial_*, path_scale, wave_seg, wave_pos, x_gather unused and zero); cfg is ignored.  Per-edge
+ * or shared weights; a shared weight's gradient is not formed here (CGTP_ERR_SHAPE with w_shared and grad_w).
+ * pos_per_wave counts the sorted positions of one range (one range per group of lanes that handles an edge); 0 = as
+ * many ranges as fill the GPU once.  workspace: cgtp_uvu_tab_workspace_bytes() bytes (partial rows of the segments a
+ * range boundary cuts). */
+typedef struct cgtp_uvu_tab {
+  const float* coef;        /* [nnz64 + 128] device, nnz64 = nnz rounded up to a multiple of 64: coefficients, entries
+                               sorted by (path, output row); zeros past nnz                                     */
+  const uint32_t* idx;      /* [nnz64 + 128] device, one word per entry: row of x | row of y << 8 | 1 << 16 on the last
+                               entry of a (path, output row) segment | 1 << 17 on the last entry of a path | output row
+                               << 18 (rows < 256); zeros past nnz                                              */
+  const uint32_t* paths;    /* [n_paths_walked + 2] device: the weight path of every run of entries in walk order, then
+                               0xffff twice                                                                    */
+  int32_t nnz, n_segments;  /* nnz <= 8192; n_segments = number of (path, output row) runs                      */
+  int32_t D1, D2, DO, P;    /* rows of x, y, out (each < 256) and number of weight paths                        */
+} cgtp_uvu_tab;
+int64_t cgtp_uvu_tab_workspace_bytes(const cgtp_uvu_args* a, const cgtp_uvu_tab* t, int backward);
+/* Status the launch would return for these arguments (pointers are only tested for NULL and alignment). Host only. */
+int cgtp_uvu_tab_validate(const cgtp_uvu_args* a, const cgtp_uvu_tab* t, int backward);
+int cgtp_uvu_tab_fwd(const cgtp_uvu_args* a, const cgtp_uvu_tab* t, void* stream);
+int cgtp_uvu_tab_bwd(const cgtp_uvu_args* a, const cgtp_uvu_tab* t, void* stream);
 
 /* Positions of one segment a wavefront takes per step (64 / lanes per edge) in a segment-mode launch of config
  * `cfg` with C channels and aligned operands; 0 if there is no such launch.  Host only. */
