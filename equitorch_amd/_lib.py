@@ -68,6 +68,19 @@ class UvuTab(C.Structure):
                 ("D1", C.c_int32), ("D2", C.c_int32), ("DO", C.c_int32), ("P", C.c_int32)]
 
 
+class PswTable(C.Structure):
+    _fields_ = [("entries", C.c_void_p), ("coef", C.c_void_p), ("slots", C.c_void_p), ("blocks", C.c_void_p),
+                ("n_entries", C.c_int32), ("n_slots", C.c_int32), ("n_blocks", C.c_int32), ("max_rows", C.c_int32),
+                ("D1", C.c_int32), ("D2", C.c_int32), ("DO", C.c_int32), ("P", C.c_int32)]
+
+
+class PswArgs(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("y", C.c_void_p), ("w", C.c_void_p), ("out", C.c_void_p),
+                ("g", C.c_void_p), ("gx", C.c_void_p), ("gy", C.c_void_p), ("gw", C.c_void_p),
+                ("n_rows", C.c_int64), ("cx", C.c_int32), ("cy", C.c_int32), ("cout", C.c_int32),
+                ("dtype", C.c_int32)]
+
+
 class UvtItem(C.Structure):
     _fields_ = [("p", C.c_int32), ("kb0", C.c_int32), ("nkb", C.c_int32), ("t0", C.c_int32), ("t1", C.c_int32),
                 ("out_row", C.c_int32), ("flags", C.c_int32), ("reserved_", C.c_int32)]
@@ -145,6 +158,9 @@ def _load():
     lib.cgtp_uvu_tab_validate.argtypes = [C.POINTER(UvuArgs), C.POINTER(UvuTab), C.c_int]
     lib.cgtp_uvu_tab_fwd.argtypes = [C.POINTER(UvuArgs), C.POINTER(UvuTab), C.c_void_p]
     lib.cgtp_uvu_tab_bwd.argtypes = [C.POINTER(UvuArgs), C.POINTER(UvuTab), C.c_void_p]
+    lib.cgtp_psw_validate.argtypes = [C.POINTER(PswArgs), C.POINTER(PswTable), C.c_int]
+    lib.cgtp_psw_fwd.argtypes = [C.POINTER(PswArgs), C.POINTER(PswTable), C.c_void_p]
+    lib.cgtp_psw_bwd.argtypes = [C.POINTER(PswArgs), C.POINTER(PswTable), C.c_void_p]
     lib.cgtp_uv_find.argtypes = [C.c_uint64]
     lib.cgtp_uv_find_rounded.argtypes = [C.c_uint64, C.c_int]
     _uv = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32,

@@ -619,13 +619,28 @@ int cgtp_abi_layout(int which, int64_t* out, int capacity) {
                                     CGTP_OFF(cgtp_uvu_tab, nnz), CGTP_OFF(cgtp_uvu_tab, n_segments),
                                     CGTP_OFF(cgtp_uvu_tab, D1), CGTP_OFF(cgtp_uvu_tab, D2),
                                     CGTP_OFF(cgtp_uvu_tab, DO), CGTP_OFF(cgtp_uvu_tab, P)};
+  static const int64_t psw_table[] = {sizeof(cgtp_psw_table), CGTP_OFF(cgtp_psw_table, entries),
+                                      CGTP_OFF(cgtp_psw_table, coef), CGTP_OFF(cgtp_psw_table, slots),
+                                      CGTP_OFF(cgtp_psw_table, blocks), CGTP_OFF(cgtp_psw_table, n_entries),
+                                      CGTP_OFF(cgtp_psw_table, n_slots), CGTP_OFF(cgtp_psw_table, n_blocks),
+                                      CGTP_OFF(cgtp_psw_table, max_rows), CGTP_OFF(cgtp_psw_table, D1),
+                                      CGTP_OFF(cgtp_psw_table, D2), CGTP_OFF(cgtp_psw_table, DO),
+                                      CGTP_OFF(cgtp_psw_table, P)};
+  static const int64_t psw_args[] = {sizeof(cgtp_psw_args), CGTP_OFF(cgtp_psw_args, x), CGTP_OFF(cgtp_psw_args, y),
+                                     CGTP_OFF(cgtp_psw_args, w), CGTP_OFF(cgtp_psw_args, out),
+                                     CGTP_OFF(cgtp_psw_args, g), CGTP_OFF(cgtp_psw_args, gx),
+                                     CGTP_OFF(cgtp_psw_args, gy), CGTP_OFF(cgtp_psw_args, gw),
+                                     CGTP_OFF(cgtp_psw_args, n_rows), CGTP_OFF(cgtp_psw_args, cx),
+                                     CGTP_OFF(cgtp_psw_args, cy), CGTP_OFF(cgtp_psw_args, cout),
+                                     CGTP_OFF(cgtp_psw_args, dtype)};
 #undef CGTP_OFF
-  const int64_t* tabs[] = {operand, tri, gen_operand, gen, uvu, uvt_item, uvt, uvt_gw, uvt_gy, uvu_tab};
+  const int64_t* tabs[] = {operand, tri, gen_operand, gen, uvu, uvt_item, uvt, uvt_gw, uvt_gy, uvu_tab, psw_table,
+                           psw_args};
   const int counts[] = {(int)(sizeof(operand) / 8), (int)(sizeof(tri) / 8), (int)(sizeof(gen_operand) / 8),
                         (int)(sizeof(gen) / 8), (int)(sizeof(uvu) / 8), (int)(sizeof(uvt_item) / 8),
                         (int)(sizeof(uvt) / 8), (int)(sizeof(uvt_gw) / 8), (int)(sizeof(uvt_gy) / 8),
-                        (int)(sizeof(uvu_tab) / 8)};
-  if (which < 0 || which >= 10) return -1;
+                        (int)(sizeof(uvu_tab) / 8), (int)(sizeof(psw_table) / 8), (int)(sizeof(psw_args) / 8)};
+  if (which < 0 || which >= 12) return -1;
   for (int i = 0; out && i < counts[which] && i < capacity; ++i) out[i] = tabs[which][i];
   return counts[which];
 }

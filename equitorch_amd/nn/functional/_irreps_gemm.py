@@ -420,6 +420,31 @@ def _table_driven_path(x: Tensor, weight: Tensor, plan: LinearPlan, in_size: int
     return _uv_native.u1v(x, ones, weight, table)
 
 
+def _streaming_path(x: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anchor: Tensor):
+    """A weight per sample: the streaming kernels of the fully connected products (``_psw``), with the scalar 1 as the
+    second operand.  None when the plan or the extents do not fit them."""
+    import numpy as np
+
+    from ...ops import kernels
+    from . import _psw
+
+    def build():
+        rows = [(p.o0 + j, p.i0 + j, p.w, p.scale) for p in plan.paths for j in range(p.k)]
+        if not rows or in_size > 255:
+            return False
+        m, m1, pw, sc = (np.asarray(v) for v in zip(*rows))
+        try:
+            return _psw.PswTable(m, m1, np.zeros_like(m), pw, sc, in_size, 1, plan.out_size, plan.n_paths, x.device)
+        except ValueError:
+            return False
+
+    table = cached(anchor, ("linear_as_psw_table", in_size, plan.n_paths, plan.out_size, str(x.device)), build)
+    if table is False or not _psw.launchable(table, x, None, weight):
+        return None
+    kernels.log_tier("irreps_linear", "per-sample weight streaming kernel", str(x.dtype))
+    return _psw.product(table, x, None, weight, lambda xx, _y, ww: _Mix.apply(xx, ww, plan, False, in_size))
+
+
 def mix(input: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anchor: Tensor = None) -> Tensor:
     """``(..., D_in, C_in) x (P, C_in, C_out) | (N, P, C_in, C_out) -> (..., D_out, C_out)``."""
     _lib.require_gpu(input, weight)
@@ -437,6 +462,8 @@ def mix(input: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anchor: T
     out = _matrix_core_path(x, weight, plan, in_size, anchor) if anchor is not None else None
     if out is None and anchor is not None:
         out = _table_driven_path(x, weight, plan, in_size, anchor)
+    if out is None and weight.ndim == 4 and anchor is not None:
+        out = _streaming_path(x, weight, plan, in_size, anchor)
     if out is None:
         out = _Mix.apply(x, weight, plan, False, in_size)
     return out.reshape(*lead, plan.out_size, out.shape[-1])

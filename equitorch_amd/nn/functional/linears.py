@@ -112,6 +112,13 @@ def tensor_product_u1v(input1: Tensor, input2: Tensor, weight: Tensor,
     if _uv_native.u1v_supported(input1, input2, weight, tp_info_forward):
         kernels.log_tier("tensor_product_u1v", "fp32 matrix-core kernel (table-driven)")
         return _uv_native.u1v(input1, input2, weight, tp_info_forward)
+    if weight.ndim == 4:
+        from . import _psw
+        table = _psw.table_of_coo(kernels.coo_of(tp_info_forward), tp_info_forward.info_Mij_fwd.scale, 1, input1.device)
+        if _psw.launchable(table, input1, input2, weight):
+            kernels.log_tier("tensor_product_u1v", "per-sample weight streaming kernel", str(input1.dtype))
+            return _psw.product(table, input1, input2, weight,
+                                lambda x, y, w: _uv_gemm.u1v(x, y, w, tp_info_forward))
     if input1.ndim == 3 and input2.ndim == 2 and _uv_gemm.supported(input1, input2, weight):
         kernels.log_tier("tensor_product_u1v", "library GEMM + table-driven kernel", str(input1.dtype))
         return _uv_gemm.u1v(input1, input2, weight, tp_info_forward)
@@ -129,7 +136,15 @@ def tensor_product_1vu(input1: Tensor, input2: Tensor, weight: Tensor,
     """``input1 (N, D1)``, ``input2 (N, D2, C_in)`` -> ``(N, DO, C_out)`` (reference ``:338-412``)."""
     _check_batch(input1, input2, weight)
     from . import _uv_gemm
+    if weight.ndim == 4 and input1.ndim == 2 and input2.ndim == 3:
+        from . import _psw
+        table = _psw.table_of_coo(kernels.coo_of(tp_info_forward), tp_info_forward.info_Mij_fwd.scale, 2, input1.device)
+        if _psw.launchable(table, input2, input1, weight):
+            kernels.log_tier("tensor_product_1vu", "per-sample weight streaming kernel", str(input1.dtype))
+            return _psw.product(table, input2, input1, weight,
+                                lambda x, y, w: _uv_gemm.one_vu(y, x, w, tp_info_forward))
     if input1.ndim == 2 and input2.ndim == 3 and _uv_gemm.supported(input1, input2, weight):
+        kernels.log_tier("tensor_product_1vu", "library GEMM + table-driven kernel", str(input1.dtype))
         return _uv_gemm.one_vu(input1, input2, weight, tp_info_forward)
     return tri(spec_from_tp_info(tp_info_forward), ("", "u", "uw"), "w", input1, input2, weight)
 

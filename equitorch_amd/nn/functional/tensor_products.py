@@ -76,6 +76,15 @@ def tensor_product_uvw(input1: Tensor, input2: Tensor, weight: Tensor,
     if _uv_native.uvw_supported(input1, input2, weight, tp_info_forward):
         kernels.log_tier("tensor_product_uvw", "fp32 matrix-core kernel (table-driven)")
         return _uv_native.uvw(input1, input2, weight, tp_info_forward)
+    if weight.ndim == 5 and input1.ndim == 3 and input2.ndim == 3:
+        from . import _psw
+        table = _psw.table_of_coo(kernels.coo_of(tp_info_forward), tp_info_forward.info_Mij_fwd.scale, 1, input1.device)
+        w4 = weight.contiguous().flatten(2, 3)
+        if _psw.launchable(table, input1, input2, w4):
+            kernels.log_tier("tensor_product_uvw", "per-sample weight streaming kernel", str(input1.dtype))
+            u, v = weight.shape[2:4]
+            return _psw.product(table, input1, input2, w4,
+                                lambda x, y, w: _uvw_gemm.uvw(x, y, w.unflatten(2, (u, v)), tp_info_forward))
     kernels.log_tier("tensor_product_uvw", "table-driven outer products + library GEMM", str(input1.dtype))
     return _uvw_gemm.uvw(input1.contiguous(), input2.contiguous(), weight, tp_info_forward)
 

@@ -42,7 +42,7 @@ int cgtp_version(void);
  * in declaration order to out[0 .. capacity) and returns how many numbers the full description has (-1: bad id). */
 enum { CGTP_LAYOUT_OPERAND = 0, CGTP_LAYOUT_TRI_ARGS = 1, CGTP_LAYOUT_GEN_OPERAND = 2, CGTP_LAYOUT_GEN_ARGS = 3,
        CGTP_LAYOUT_UVU_ARGS = 4, CGTP_LAYOUT_UVT_ITEM = 5, CGTP_LAYOUT_UVT_ARGS = 6, CGTP_LAYOUT_UVT_GW_ARGS = 7,
-       CGTP_LAYOUT_UVT_GY_ARGS = 8, CGTP_LAYOUT_UVU_TABLE = 9 };
+       CGTP_LAYOUT_UVT_GY_ARGS = 8, CGTP_LAYOUT_UVU_TABLE = 9, CGTP_LAYOUT_PSW_TABLE = 10, CGTP_LAYOUT_PSW_ARGS = 11 };
 int cgtp_abi_layout(int which, int64_t* out, int capacity);
 
 /* ---- generic sparse trilinear contraction -------------------------------------------------------------
@@ -461,6 +461,57 @@ typedef struct cgtp_uvt_gw_args {
 
 int64_t cgtp_uvt_grad_w_workspace_bytes(int64_t n_rows, int32_t n_paths, int64_t K, int32_t cout, int32_t dtype);
 int cgtp_uvt_grad_w(const cgtp_uvt_gw_args* args, void* stream);
+
+/* ---- fully connected products with a weight per sample ---------------------------------------------------
+ *
+ *   out[n, M, w] = sum_t coef_t * sum_{u, v} x[n, a_t, u] * y[n, b_t, v] * W[n, p_t, u * cy + v, w]
+ *
+ * One streaming launch over the per-sample weight W (n_rows, n_paths, cx * cy, cout), each element read once, for
+ * the products the reference runs as two launches with the (N, segments, C_in) intermediate in memory when the
+ * weight has a batch axis (per-sample detection: equitorch/nn/tensor_products.py:152-155; u1v / 1vu:
+ * equitorch/nn/functional/linears.py:254-412; uvw: equitorch/nn/functional/tensor_products.py:95-158; channel mixing
+ * between irreps with y = NULL: linears.py:494-571; kernel ops/batched_sparse_dense_op.py:1289-1381).  The backward
+ * writes grad_W in the same stream (read W, write grad_W) and sums grad_x / grad_y per sample in LDS; any of gx / gy
+ * / gw may be NULL.  The table is data: the paths are walked output irrep by output irrep.
+ *   blocks  [n_blocks][4]  (first output row, rows L, first slot, one past the last slot); the rows of different
+ *                          blocks do not overlap; output rows outside every block are not written
+ *   slots   [n_slots][3]   (weight path p, first entry, one past the last entry) of a walked path
+ *   entries [n_entries]    j | a << 8 | b << 16 | 1 << 24 on the last entry of a run of equal j; j = output row - the
+ *                          block's first row; sorted by j inside a slot; every j < L occurs in every slot of the
+ *                          block (with coefficient 0 where the path has no term for it)
+ *   coef    [n_entries]    dtype
+ * x (n_rows, D1, cx), y (n_rows, D2, cy) or NULL (then cy = 1, D2 = 1 and y = 1), out / g (n_rows, DO, cout), all
+ * contiguous, dtype CGTP_F32 | CGTP_F64.  cout <= 64 vector lanes: cout <= 256 (fp32) / 128 (fp64) when it is a
+ * multiple of 4 / 2 and W, out, g, gw are 16-byte aligned, cout <= 64 otherwise (CGTP_ERR_SHAPE beyond); D1, D2,
+ * max_rows < 256; one sample's rows must fit 64 KB of LDS (CGTP_ERR_LDS otherwise). */
+typedef struct cgtp_psw_table {
+  const uint32_t* entries;  /* device */
+  const void* coef;         /* device, dtype */
+  const int32_t* slots;     /* device */
+  const int32_t* blocks;    /* device */
+  int32_t n_entries, n_slots, n_blocks;
+  int32_t max_rows;         /* largest L of a block */
+  int32_t D1, D2, DO, P;
+} cgtp_psw_table;
+
+typedef struct cgtp_psw_args {
+  const void* x;
+  const void* y;
+  const void* w;
+  void* out;       /* forward */
+  const void* g;   /* backward: grad_out */
+  void* gx;
+  void* gy;
+  void* gw;
+  int64_t n_rows;
+  int32_t cx, cy, cout;
+  int32_t dtype;
+} cgtp_psw_args;
+
+/* Status the launch would return for these arguments. Host only. */
+int cgtp_psw_validate(const cgtp_psw_args* a, const cgtp_psw_table* t, int backward);
+int cgtp_psw_fwd(const cgtp_psw_args* a, const cgtp_psw_table* t, void* stream);
+int cgtp_psw_bwd(const cgtp_psw_args* a, const cgtp_psw_table* t, void* stream);
 
 /* Gradient of a second operand without channels (u1v):
  *   gy[n, b] = sum_t coef_t * sum_w grad_out[n, M_t, w] * (sum_k x[n, a_t, k] * W[p_t, k, w])

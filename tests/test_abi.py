@@ -30,7 +30,8 @@ def test_struct_layouts_match_the_ctypes_mirror():
     field offset as compiled, in declaration order."""
     from equitorch_amd import _lib
     for which, cls in enumerate((_lib.Operand, _lib.TriArgs, _lib.GenOperand, _lib.GenArgs, _lib.UvuArgs, _lib.UvtItem,
-                                _lib.UvtArgs, _lib.UvtGwArgs, _lib.UvtGyArgs, _lib.UvuTab)):
+                                _lib.UvtArgs, _lib.UvtGwArgs, _lib.UvtGyArgs, _lib.UvuTab, _lib.PswTable,
+                                _lib.PswArgs)):
         n = _lib.lib.cgtp_abi_layout(which, None, 0)
         assert n == 1 + len(cls._fields_), f"{cls.__name__}: {n - 1} fields in the library, {len(cls._fields_)} here"
         buf = (C.c_int64 * n)()

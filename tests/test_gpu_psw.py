@@ -1,0 +1,248 @@
+"""Fully connected products with a weight per sample (``cgtp_psw_fwd`` / ``cgtp_psw_bwd``: one streaming launch each way,
+no library GEMM, no intermediate in memory) against the dense float64 oracle: u1v, 1vu, uvw and the channel mixing
+between irreps, forward and all first-order gradients.  The reference takes a weight with a batch axis through its
+table-driven kernels like a shared one (``equitorch/nn/tensor_products.py:152-155``,
+``equitorch/nn/functional/linears.py:254-412``).  While the product and its backward run, ``torch.matmul`` / ``bmm``
+/ ``baddbmm`` raise."""
+import pytest
+import torch
+
+from helpers import assert_close, fp32_twin, stable_seed
+from oracle import ref_ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _sh(lmax):
+    return "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+
+
+@pytest.fixture
+def no_library_gemm():
+    """Context manager: inside it ``torch.matmul`` / ``bmm`` / ``baddbmm`` / ``einsum`` raise."""
+    import contextlib
+
+    @contextlib.contextmanager
+    def guard():
+        def refuse(*a, **k):
+            raise AssertionError("a library GEMM was called")
+        names = ("matmul", "bmm", "baddbmm", "einsum")
+        saved = {name: getattr(torch, name) for name in names}
+        for name in names:
+            setattr(torch, name, refuse)
+        try:
+            yield
+        finally:
+            for name, fn in saved.items():
+                setattr(torch, name, fn)
+    return guard
+
+
+def _tiers(monkeypatch):
+    from equitorch_amd.ops import kernels
+    seen = []
+    monkeypatch.setattr(kernels, "log_tier", lambda op, tier, detail="": seen.append(tier))
+    return seen
+
+
+U1V = [  # irreps (out, in1, in2), C_in, C_out, N, dtype
+    ((_sh(2),) * 3, 32, 32, 300, torch.float32),          # 8 lanes a row, one sample a wavefront, 8 row slices
+    ((_sh(2),) * 3, 16, 16, 20000, torch.float32),        # several samples a wavefront
+    ((_sh(3),) * 3, 64, 64, 70, torch.float32),           # blocks of 7 rows
+    ((_sh(2),) * 3, 5, 20, 129, torch.float32),           # 5 lanes of 4 channels, C_in below a chunk
+    ((_sh(2),) * 3, 33, 7, 1000, torch.float32),          # one channel a lane, chunks of 32 + 1
+    ((_sh(1),) * 3, 100, 128, 77, torch.float32),         # 32 lanes a row, chunks of 64 + 36
+    ((_sh(1),) * 3, 8, 256, 40, torch.float32),           # a row over the whole wavefront
+    (("1o+2e+1e", "0e+1o+2e", "0e+1o"), 24, 40, 200, torch.float32),
+    (("2x0e+1o+1e", "0e+2x1o", "0e+1o+1e"), 12, 12, 64, torch.float32),
+    (("0e+4e", "2e+3o", "2e+3o"), 8, 16, 50, torch.float32),      # a block of 9 rows: the 16-row pass
+    ((_sh(2),) * 3, 32, 32, 300, torch.float64),
+    ((_sh(3), _sh(2), _sh(3)), 20, 6, 45, torch.float64),
+]
+
+
+@pytest.mark.parametrize("irreps,cin,cout,n,dtype", U1V)
+def test_u1v_per_sample_weight(device, monkeypatch, no_library_gemm, irreps, cin, cout, n, dtype):
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    io, i1, i2 = irreps
+    infos = [t.to(device) for t in tp_infos(Irreps(io), Irreps(i1), Irreps(i2))[:3]]
+    T = ref_ops.dense_coupling(io, i1, i2).float().double()
+    g = torch.Generator().manual_seed(stable_seed("psw u1v", irreps, cin, cout, n))
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).to(dtype)
+    x, y, w = rd(n, T.shape[2], cin), rd(n, T.shape[3]), rd(n, T.shape[0], cin, cout) / cin ** 0.5
+    ct = rd(n, T.shape[1], cout)
+    seen = _tiers(monkeypatch)
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    with no_library_gemm():
+        out = F.tensor_product_u1v(xd, yd, wd, *infos)
+        grads = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
+    assert seen and "per-sample weight streaming" in seen[-1], seen
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x, y, w), ct)
+    tol = 1e-5 if dtype == torch.float32 else 1e-12
+    twin = (None,) * 4
+    if dtype == torch.float32:
+        o32, g32 = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x, y, w), ct, dtype=torch.float32)
+        twin = (o32, *g32)
+    for name, a, b, b32 in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads), twin):
+        assert_close(a, b, tol, f"u1v per-sample {io} {cin}->{cout} N={n} {dtype} {name}", norm="max", fp32_ref=b32)
+
+
+@pytest.mark.parametrize("irreps,cin,cout,n", [((_sh(2),) * 3, 32, 32, 300), (("1o+2e+1e", "0e+1o", "0e+1o+2e"), 10, 24, 99)])
+def test_1vu_per_sample_weight(device, monkeypatch, no_library_gemm, irreps, cin, cout, n):
+    """The channels on the second operand: the same kernels with the operands' places exchanged."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    io, i1, i2 = irreps
+    infos = [t.to(device) for t in tp_infos(Irreps(io), Irreps(i1), Irreps(i2))[:3]]
+    T = ref_ops.dense_coupling(io, i1, i2).float().double()
+    g = torch.Generator().manual_seed(stable_seed("psw 1vu", irreps, cin, cout, n))
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).float()
+    x, y, w = rd(n, T.shape[2]), rd(n, T.shape[3], cin), rd(n, T.shape[0], cin, cout) / cin ** 0.5
+    ct = rd(n, T.shape[1], cout)
+    seen = _tiers(monkeypatch)
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    with no_library_gemm():
+        out = F.tensor_product_1vu(xd, yd, wd, *infos)
+        grads = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
+    assert seen and "per-sample weight streaming" in seen[-1], seen
+
+    def dense_1vu(T, x, y, w, dtype=torch.float64):
+        return ref_ops.dense_u1v(T.transpose(2, 3), y, x, w, dtype=dtype)
+    ref_out, ref_grads = ref_ops.dense_grads(dense_1vu, T, (x, y, w), ct)
+    o32, g32 = ref_ops.dense_grads(dense_1vu, T, (x, y, w), ct, dtype=torch.float32)
+    for name, a, b, b32 in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads), (o32, *g32)):
+        assert_close(a, b, 1e-5, f"1vu per-sample {io} {cin}->{cout} {name}", norm="max", fp32_ref=b32)
+
+
+UVW = [  # irreps, U, V, C_out, N, dtype
+    ((_sh(2), _sh(2), "0e+1o"), 16, 8, 12, 301, torch.float32),      # chunks of 8 u
+    ((_sh(1),) * 3, 4, 64, 32, 90, torch.float32),                   # chunks of one u
+    ((_sh(2),) * 3, 6, 3, 5, 2000, torch.float32),                   # chunks of 21 u > U, one channel a lane
+    ((_sh(1),) * 3, 3, 100, 16, 33, torch.float32),                  # V beyond the lanes of a sample
+    ((_sh(2), _sh(2), "0e+1o"), 8, 8, 8, 64, torch.float64),
+]
+
+
+@pytest.mark.parametrize("irreps,u,v,cout,n,dtype", UVW)
+def test_uvw_per_sample_weight(device, monkeypatch, no_library_gemm, irreps, u, v, cout, n, dtype):
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    io, i1, i2 = irreps
+    infos = [t.to(device) for t in tp_infos(Irreps(io), Irreps(i1), Irreps(i2))[:3]]
+    T = ref_ops.dense_coupling(io, i1, i2).float().double()
+    g = torch.Generator().manual_seed(stable_seed("psw uvw", irreps, u, v, cout, n))
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).to(dtype)
+    x, y, w = rd(n, T.shape[2], u), rd(n, T.shape[3], v), rd(n, T.shape[0], u, v, cout) / (u * v) ** 0.5
+    ct = rd(n, T.shape[1], cout)
+    seen = _tiers(monkeypatch)
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    with no_library_gemm():
+        out = F.tensor_product_uvw(xd, yd, wd, *infos)
+        grads = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
+    assert seen and "per-sample weight streaming" in seen[-1], seen
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_uvw, T, (x, y, w), ct)
+    tol = 1e-5 if dtype == torch.float32 else 1e-12
+    twin = (None,) * 4
+    if dtype == torch.float32:
+        o32, g32 = ref_ops.dense_grads(ref_ops.dense_uvw, T, (x, y, w), ct, dtype=torch.float32)
+        twin = (o32, *g32)
+    for name, a, b, b32 in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads), twin):
+        assert_close(a, b, tol, f"uvw per-sample {io} {u}x{v}->{cout} N={n} {dtype} {name}", norm="max", fp32_ref=b32)
+
+
+def test_only_some_gradients(device, no_library_gemm):
+    """Operands that need no gradient: the backward forms only what is asked for."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    irr = _sh(2)
+    infos = [t.to(device) for t in tp_infos(Irreps(irr), Irreps(irr), Irreps(irr))[:3]]
+    T = ref_ops.dense_coupling(irr, irr, irr).float().double()
+    g = torch.Generator().manual_seed(3)
+    n, cin, cout = 150, 16, 24
+    x, y, w, ct = (torch.randn(*s, generator=g) for s in ((n, 9, cin), (n, 9), (n, T.shape[0], cin, cout), (n, 9, cout)))
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x, y, w), ct)
+    for need in ((True, False, False), (False, True, False), (False, False, True), (True, True, False)):
+        leaves = [t.to(device).requires_grad_(r) for t, r in zip((x, y, w), need)]
+        with no_library_gemm():
+            out = F.tensor_product_u1v(*leaves, *infos)
+            grads = torch.autograd.grad(out, [t for t, r in zip(leaves, need) if r], ct.to(device))
+        for a, b in zip(grads, [b for b, r in zip(ref_grads, need) if r]):
+            assert_close(a, b, 1e-5, f"u1v per-sample, gradients {need}", norm="max")
+
+
+def test_second_order_goes_through_the_differentiable_route(device):
+    """A gradient of the gradient: the backward re-expresses the product through differentiable pieces."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    irr = _sh(1)
+    infos = [t.to(device) for t in tp_infos(Irreps(irr), Irreps(irr), Irreps(irr))[:3]]
+    T = ref_ops.dense_coupling(irr, irr, irr).float().double()
+    g = torch.Generator().manual_seed(5)
+    n, cin, cout = 20, 8, 8
+    x, y, w, ct = (torch.randn(*s, generator=g, dtype=torch.float64)
+                   for s in ((n, 4, cin), (n, 4), (n, T.shape[0], cin, cout), (n, 4, cout)))
+
+    def second(fn, x, y, w, ct):
+        x, y, w = (t.clone().requires_grad_(True) for t in (x, y, w))
+        gx, = torch.autograd.grad(fn(x, y, w), x, ct, create_graph=True)
+        return torch.autograd.grad(gx.square().sum(), (y, w))
+    got = second(lambda a, b, c: F.tensor_product_u1v(a, b, c, *infos), *(t.to(device) for t in (x, y, w, ct)))
+    ref = second(lambda a, b, c: ref_ops.dense_u1v(T, a, b, c), x, y, w, ct)
+    for name, a, b in zip(("d/dy", "d/dw"), got, ref):
+        assert_close(a, b, 1e-11, f"u1v per-sample second order {name}", norm="max")
+
+
+@pytest.mark.parametrize("io,ii,dtype", [("0e+1o+2e", "0e+1o+1o+2e+0e", torch.float32),
+                                         ("2x0e+1o+3x2e", "0e+2x1o+2e+3e", torch.float32),
+                                         ("0e+1o", "0e+1e+2e", torch.float64)])
+def test_channel_mixing_per_sample_weight(device, monkeypatch, no_library_gemm, io, ii, dtype):
+    """``IrrepsLinear`` with a weight per sample: the same kernels with the scalar 1 as second operand (several input
+    irreps feeding one output irrep share its rows; an output irrep without a source stays zero)."""
+    from equitorch_amd.nn import IrrepsLinear
+    from oracle import ref_tables
+    n, cin, cout = 210, 24, 40
+    mod = IrrepsLinear(ii, io, cin, cout, internal_weights=False).to(device)
+    info = ref_tables.irreps_linear_infos(io, ii)[0]
+    info["scale_MM0"] = torch.tensor(info["scale_MM0"]).double().tolist()    # the tables hold fp32 values
+    g = torch.Generator().manual_seed(8)
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).to(dtype).double()
+    x, w, ct = rd(n, mod.irreps_in_dim, cin), rd(n, mod.num_paths, cin, cout), rd(n, mod.irreps_out_dim, cout)
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    ref = ref_ops.cpu_irreps_linear(xr, wr, info)
+    rgx, rgw = torch.autograd.grad(ref, (xr, wr), ct)
+    seen = _tiers(monkeypatch)
+    xd, wd = (t.to(device, dtype).requires_grad_(True) for t in (x, w))
+    with no_library_gemm():
+        out = mod(xd, wd)
+        gx, gw = torch.autograd.grad(out, (xd, wd), ct.to(device, dtype))
+    assert seen and "per-sample weight streaming" in seen[-1], seen
+    tol = 1e-5 if dtype == torch.float32 else 1e-12
+    for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
+        assert_close(a, b, tol, f"IrrepsLinear per-sample {io}<-{ii} {dtype} {name}")
+
+
+def test_irrep_wise_per_sample_weight(device, monkeypatch, no_library_gemm):
+    from equitorch_amd.nn import IrrepWiseLinear
+    from oracle import ref_tables
+    irr, cin, cout, n = "0e+1o+2e+1o", 16, 8, 333
+    mod = IrrepWiseLinear(irr, cin, cout, internal_weights=False).to(device)
+    info = ref_tables.irreps_info(irr)
+    g = torch.Generator().manual_seed(2)
+    x, w, ct = (torch.randn(*s, generator=g, dtype=torch.float64) for s in ((n, 12, cin), (n, 4, cin, cout), (n, 12, cout)))
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    ref = ref_ops.cpu_irrep_wise_linear(xr, wr, info)
+    rgx, rgw = torch.autograd.grad(ref, (xr, wr), ct)
+    seen = _tiers(monkeypatch)
+    xd, wd = (t.to(device).requires_grad_(True) for t in (x, w))
+    with no_library_gemm():
+        out = mod(xd, wd)
+        gx, gw = torch.autograd.grad(out, (xd, wd), ct.to(device))
+    assert seen and "per-sample weight streaming" in seen[-1], seen
+    for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
+        assert_close(a, b, 1e-12, f"IrrepWiseLinear per-sample {name}")
