@@ -141,38 +141,61 @@ __device__ __forceinline__ void psw_fwd_block(const PswDev<T>& a, const PswLayou
   for (int j = 0; j < JB; ++j)
 #pragma unroll
     for (int v = 0; v < V; ++v) acc[j][v] = T(0);
-  for (int q = q0; q < q1; ++q) {
-    const int p = slots[3 * q], e0 = slots[3 * q + 1], e1 = slots[3 * q + 2];
-    const T* wp = a.w + ((n * a.P + p) * (int64_t)a.K) * a.Wc + L.wl * V;
-    for (int k0 = 0; k0 < a.K; k0 += a.TK) {
-      const int TKc = a.K - k0 < a.TK ? a.K - k0 : a.TK;
-      psw_wave_sync();   // the previous chunk's rows have been read
-      psw_form_t(a, t, xs, ys, e0, e1, k0, TKc, L);
-      psw_wave_sync();
-      const T* wrow = wp + (int64_t)k0 * a.Wc;
-      for (int kk0 = 0; kk0 < TKc; kk0 += 4 * L.KS) {
-        T wv[4][V];
-        int row[4];
+  // The walk over (path, chunk of rows, batch of 4 rows a lane) is flat: the rows of the next batch are requested
+  // before the current ones are used, across chunk and path boundaries, so forming a chunk's t overlaps the loads.
+  const auto load_batch = [&](T (&wv)[4][V], int q, int k0, int kk0) {
+    const int p = slots[3 * q];
+    const int TKc = a.K - k0 < a.TK ? a.K - k0 : a.TK;
+    const T* wrow = a.w + ((n * a.P + p) * (int64_t)a.K + k0) * a.Wc + L.wl * V;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int kk = kk0 + i * L.KS + L.ks;
-          row[i] = kk < TKc ? kk : TKc - 1;
-          if (lane_ok && kk < TKc) {
-            load_vec_stream<T, V>(wv[i], wrow + (int64_t)kk * a.Wc);
-          } else {
+    for (int i = 0; i < 4; ++i) {
+      const int kk = kk0 + i * L.KS + L.ks;
+      if (lane_ok && kk < TKc) {
+        load_vec_stream<T, V>(wv[i], wrow + (int64_t)kk * a.Wc);
+      } else {
 #pragma unroll
-            for (int v = 0; v < V; ++v) wv[i][v] = T(0);
-          }
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          T tj[JB];
-          psw_read_row<T, JB>(tj, t + row[i] * a.JP + j0);
-#pragma unroll
-          for (int j = 0; j < JB; ++j) fmav<T, V>(acc[j], tj[j], wv[i]);
-        }
+        for (int v = 0; v < V; ++v) wv[i][v] = T(0);
       }
     }
+  };
+  int q = q0, k0 = 0, kk0 = 0;
+  T cur[4][V];
+  if (q < q1) load_batch(cur, q, k0, kk0);
+  while (q < q1) {
+    const int TKc = a.K - k0 < a.TK ? a.K - k0 : a.TK;
+    if (kk0 == 0) {
+      psw_wave_sync();   // the previous chunk's rows have been read
+      psw_form_t(a, t, xs, ys, slots[3 * q + 1], slots[3 * q + 2], k0, TKc, L);
+      psw_wave_sync();
+    }
+    int nq = q, nk0 = k0, nkk0 = kk0 + 4 * L.KS;
+    if (nkk0 >= TKc) {
+      nkk0 = 0;
+      nk0 = k0 + a.TK;
+      if (nk0 >= a.K) { nk0 = 0; ++nq; }
+    }
+    T nxt[4][V];
+    if (nq < q1) {
+      load_batch(nxt, nq, nk0, nkk0);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int v = 0; v < V; ++v) nxt[i][v] = T(0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int kk = kk0 + i * L.KS + L.ks;
+      T tj[JB];
+      psw_read_row<T, JB>(tj, t + (kk < TKc ? kk : TKc - 1) * a.JP + j0);
+#pragma unroll
+      for (int j = 0; j < JB; ++j) fmav<T, V>(acc[j], tj[j], cur[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int v = 0; v < V; ++v) cur[i][v] = nxt[i][v];
+    q = nq; k0 = nk0; kk0 = nkk0;
   }
   // add the row slices: lanes that differ in ks
   for (int off = L.LPS; off < L.LS; off <<= 1) {
@@ -203,7 +226,7 @@ __device__ __forceinline__ void psw_stage(const PswDev<T>& a, const PswLayout& l
   for (int i = L.li; i < ny; i += L.LS) lds[lay.ys + i] = a.y == nullptr ? T(1) : (sample_ok ? a.y[n * ny + i] : T(0));
 }
 
-template <typename T, int V>
+template <typename T, int V, bool BIG>
 __global__ void __launch_bounds__(kWave) psw_fwd_kernel(const PswDev<T> a) {
   extern __shared__ __align__(16) unsigned char psw_lds_raw[];
   const PswLane L(a.s_log2, a.lps_log2);
@@ -220,8 +243,8 @@ __global__ void __launch_bounds__(kWave) psw_fwd_kernel(const PswDev<T> a) {
       if (rows <= 1) { psw_fwd_block<T, V, 1>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 1; }
       else if (rows <= 3) { psw_fwd_block<T, V, 3>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 3; }
       else if (rows <= 5) { psw_fwd_block<T, V, 5>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 5; }
-      else if (rows <= 8) { psw_fwd_block<T, V, 8>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 8; }
-      else { psw_fwd_block<T, V, 16>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 16; }
+      else if (!BIG || rows <= 8) { psw_fwd_block<T, V, 8>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 8; }
+      else if constexpr (BIG) { psw_fwd_block<T, V, 16>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 16; }
     }
   }
 }
@@ -313,74 +336,98 @@ __device__ __forceinline__ void psw_bwd_block(const PswDev<T>& a, const PswLayou
       }
     }
   }
-  for (int q = q0; q < q1; ++q) {
+  // flat walk as in the forward, two rows a lane per batch
+  const auto load_batch = [&](T (&wv)[2][V], int q, int k0, int kk0) {
+    const int p = slots[3 * q];
+    const int TKc = a.K - k0 < a.TK ? a.K - k0 : a.TK;
+    const T* wrow = a.w + ((n * a.P + p) * (int64_t)a.K + k0) * a.Wc + L.wl * V;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int kk = kk0 + i * L.KS + L.ks;
+      if (want_t && lane_ok && kk < TKc) {
+        load_vec_stream<T, V>(wv[i], wrow + (int64_t)kk * a.Wc);
+      } else {
+#pragma unroll
+        for (int v = 0; v < V; ++v) wv[i][v] = T(0);
+      }
+    }
+  };
+  int q = q0, k0 = 0, kk0 = 0;
+  T cur[2][V];
+  if (q < q1) load_batch(cur, q, k0, kk0);
+  while (q < q1) {
     const int p = slots[3 * q], e0 = slots[3 * q + 1], e1 = slots[3 * q + 2];
-    const int64_t wbase = ((n * a.P + p) * (int64_t)a.K) * a.Wc + L.wl * V;
-    for (int k0 = 0; k0 < a.K; k0 += a.TK) {
-      const int TKc = a.K - k0 < a.TK ? a.K - k0 : a.TK;
+    const int TKc = a.K - k0 < a.TK ? a.K - k0 : a.TK;
+    if (kk0 == 0) {
       psw_wave_sync();   // the previous chunk's t and gt have been read
       if (want_w) psw_form_t(a, t, xs, ys, e0, e1, k0, TKc, L);
       psw_wave_sync();
-      const T* wrow = a.w + wbase + (int64_t)k0 * a.Wc;
-      T* gwrow = want_w ? a.gw + wbase + (int64_t)k0 * a.Wc : nullptr;
-      for (int kk0 = 0; kk0 < TKc; kk0 += 2 * L.KS) {
-        T wv[2][V];
+    }
+    int nq = q, nk0 = k0, nkk0 = kk0 + 2 * L.KS;
+    if (nkk0 >= TKc) {
+      nkk0 = 0;
+      nk0 = k0 + a.TK;
+      if (nk0 >= a.K) { nk0 = 0; ++nq; }
+    }
+    T nxt[2][V];
+    if (nq < q1) {
+      load_batch(nxt, nq, nk0, nkk0);
+    } else {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          const int kk = kk0 + i * L.KS + L.ks;
-          if (want_t && lane_ok && kk < TKc) {
-            load_vec_stream<T, V>(wv[i], wrow + (int64_t)kk * a.Wc);
-          } else {
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int v = 0; v < V; ++v) wv[i][v] = T(0);
+        for (int v = 0; v < V; ++v) nxt[i][v] = T(0);
+    }
+    T* gwrow = want_w ? a.gw + ((n * a.P + p) * (int64_t)a.K + k0) * a.Wc + L.wl * V : nullptr;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int kk = kk0 + i * L.KS + L.ks;
+      const bool active = kk < TKc;
+      const int row = active ? kk : TKc - 1;
+      if (want_w) {
+        T tj[JB], o[V];
+        psw_read_row<T, JB>(tj, t + row * a.JP + j0);
+        mulv<T, V>(o, tj[0], gr[0]);
+#pragma unroll
+        for (int j = 1; j < JB; ++j) fmav<T, V>(o, tj[j], gr[j]);
+        if (lane_ok && active) {
+          T* dst = gwrow + (int64_t)kk * a.Wc;
+          if (j0 > 0) {   // a block wider than one pass: the earlier rows' part is there already
+            T old[V];
+            load_vec<T, V>(old, dst);
+#pragma unroll
+            for (int v = 0; v < V; ++v) o[v] += old[v];
           }
-        }
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          const int kk = kk0 + i * L.KS + L.ks;
-          const bool active = kk < TKc;
-          const int row = active ? kk : TKc - 1;
-          if (want_w) {
-            T tj[JB], o[V];
-            psw_read_row<T, JB>(tj, t + row * a.JP + j0);
-            mulv<T, V>(o, tj[0], gr[0]);
-#pragma unroll
-            for (int j = 1; j < JB; ++j) fmav<T, V>(o, tj[j], gr[j]);
-            if (lane_ok && active) {
-              T* dst = gwrow + (int64_t)kk * a.Wc;
-              if (j0 > 0) {   // a block wider than one pass: the earlier rows' part is there already
-                T old[V];
-                load_vec<T, V>(old, dst);
-#pragma unroll
-                for (int v = 0; v < V; ++v) o[v] += old[v];
-              }
-              store_vec_stream<T, V>(dst, o);
-            }
-          }
-          if (want_t) {
-            T d[JB];
-#pragma unroll
-            for (int j = 0; j < JB; ++j) d[j] = dotv<T, V>(wv[i], gr[j]);
-            T* grow = gt + row * a.JP + j0;
-            group_sum_scatter<T, JB>(d, L.LPS, [&](const auto& sums) {
-#pragma unroll
-              for (int i2 = 0; i2 < array_len(sums); ++i2) {
-                const int j = i2 * L.LPS + L.wl;
-                if (active && j < jb) grow[j] = sums[i2];
-              }
-            });
-          }
+          store_vec_stream<T, V>(dst, o);
         }
       }
       if (want_t) {
-        psw_wave_sync();
-        psw_carry_back(a, lay, lds, L, e0, e1, k0, TKc, j0, jb);
+        T d[JB];
+#pragma unroll
+        for (int j = 0; j < JB; ++j) d[j] = dotv<T, V>(cur[i], gr[j]);
+        T* grow = gt + row * a.JP + j0;
+        group_sum_scatter<T, JB>(d, L.LPS, [&](const auto& sums) {
+#pragma unroll
+          for (int i2 = 0; i2 < array_len(sums); ++i2) {
+            const int j = i2 * L.LPS + L.wl;
+            if (active && j < jb) grow[j] = sums[i2];
+          }
+        });
       }
     }
+    if (want_t && nkk0 == 0) {   // the chunk's last batch
+      psw_wave_sync();
+      psw_carry_back(a, lay, lds, L, e0, e1, k0, TKc, j0, jb);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int v = 0; v < V; ++v) cur[i][v] = nxt[i][v];
+    q = nq; k0 = nk0; kk0 = nkk0;
   }
 }
 
-template <typename T, int V>
+template <typename T, int V, bool BIG>
 __global__ void __launch_bounds__(kWave) psw_bwd_kernel(const PswDev<T> a) {
   extern __shared__ __align__(16) unsigned char psw_lds_raw[];
   const PswLane L(a.s_log2, a.lps_log2);
@@ -401,8 +448,8 @@ __global__ void __launch_bounds__(kWave) psw_bwd_kernel(const PswDev<T> a) {
       if (rows <= 1) { psw_bwd_block<T, V, 1>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 1; }
       else if (rows <= 3) { psw_bwd_block<T, V, 3>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 3; }
       else if (rows <= 5) { psw_bwd_block<T, V, 5>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 5; }
-      else if (rows <= 8) { psw_bwd_block<T, V, 8>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 8; }
-      else { psw_bwd_block<T, V, 16>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 16; }
+      else if (!BIG || rows <= 8) { psw_bwd_block<T, V, 8>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 8; }
+      else if constexpr (BIG) { psw_bwd_block<T, V, 16>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 16; }
     }
   }
   psw_wave_sync();
@@ -451,10 +498,15 @@ int psw_plan(const cgtp_psw_args* a, const cgtp_psw_table* tab, bool backward, P
   if (lanes > kWave) return CGTP_ERR_SHAPE;
   plan->lps_log2 = 0;
   while ((1 << plan->lps_log2) < lanes) ++plan->lps_log2;
-  // as many samples per wavefront as leave the GPU a few thousand wavefronts
+  // as many samples per wavefront as leave the GPU sixteen thousand wavefronts or more
   const int s_max_log2 = 6 - plan->lps_log2;
   plan->s_log2 = 0;
-  while (plan->s_log2 < s_max_log2 && (a->n_rows >> (plan->s_log2 + 1)) >= 4096) ++plan->s_log2;
+  // a batch is four rows a lane: with fewer than 4 x row slices rows in a weight matrix most of its loads would be
+  // idle, so short matrices get more samples per wavefront instead of more slices
+  const int64_t rows_k = (int64_t)a->cx * a->cy;
+  while (plan->s_log2 < s_max_log2 && 4 * (kWave >> (plan->s_log2 + plan->lps_log2)) > (rows_k > 4 ? rows_k : 4))
+    ++plan->s_log2;
+  while (plan->s_log2 < s_max_log2 && (a->n_rows >> (plan->s_log2 + 1)) >= 16384) ++plan->s_log2;
   const int64_t K = (int64_t)a->cx * a->cy;
   if (K > (1 << 24)) return CGTP_ERR_SHAPE;
   plan->JP = (tab->max_rows + 3) & ~3;
@@ -492,12 +544,15 @@ int psw_launch_t(const cgtp_psw_args* a, const cgtp_psw_table* tab, bool backwar
   d.s_log2 = plan.s_log2; d.lps_log2 = plan.lps_log2; d.TK = plan.TK; d.JP = plan.JP;
   const dim3 grid((unsigned)plan.groups), block(kWave);
   constexpr int VEC = 16 / sizeof(T);
+  // blocks of at most 8 rows (l <= 3): kernels without the 16-row pass, which would set their register count
+  const bool big = tab->max_rows > 8;
+  const auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, block, plan.lds_bytes, stream, d); };
   if (!backward) {
-    if (plan.V == 1) hipLaunchKernelGGL((psw_fwd_kernel<T, 1>), grid, block, plan.lds_bytes, stream, d);
-    else hipLaunchKernelGGL((psw_fwd_kernel<T, VEC>), grid, block, plan.lds_bytes, stream, d);
+    if (plan.V == 1) big ? go(psw_fwd_kernel<T, 1, true>) : go(psw_fwd_kernel<T, 1, false>);
+    else big ? go(psw_fwd_kernel<T, VEC, true>) : go(psw_fwd_kernel<T, VEC, false>);
   } else {
-    if (plan.V == 1) hipLaunchKernelGGL((psw_bwd_kernel<T, 1>), grid, block, plan.lds_bytes, stream, d);
-    else hipLaunchKernelGGL((psw_bwd_kernel<T, VEC>), grid, block, plan.lds_bytes, stream, d);
+    if (plan.V == 1) big ? go(psw_bwd_kernel<T, 1, true>) : go(psw_bwd_kernel<T, 1, false>);
+    else big ? go(psw_bwd_kernel<T, VEC, true>) : go(psw_bwd_kernel<T, VEC, false>);
   }
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }

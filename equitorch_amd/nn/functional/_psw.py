@@ -7,8 +7,8 @@ The reference takes a weight with a batch axis through the same two launches as 
 ``equitorch/nn/functional/tensor_products.py:95-158`` for uvw, ``linears.py:494-571`` for the channel mixing between
 irreps).
 
-A table qualifies when every weight path writes the consecutive rows of one output irrep and the irreps of different
-paths coincide or are disjoint — true for every table ``tp_infos`` / ``irreps_linear_infos`` / ``irreps_info`` build.
+A table qualifies when the row ranges that different weight paths write (one output irrep each) coincide or are
+disjoint — true for every table ``tp_infos`` / ``irreps_linear_infos`` / ``irreps_info`` build.
 """
 import ctypes as C
 from typing import Callable, Optional
@@ -35,10 +35,8 @@ class PswTable:
             raise ValueError("operand rows beyond 255")
         blocks_of = {}
         for p in np.unique(path):
-            rows = np.unique(out_row[path == p])
-            if not np.array_equal(rows, np.arange(rows[0], rows[0] + rows.size)):
-                raise ValueError("the output rows of a path must be consecutive (one irrep)")
-            blocks_of.setdefault((int(rows[0]), int(rows.size)), []).append(int(p))
+            rows = out_row[path == p]             # a row in between without a term gets a zero entry below
+            blocks_of.setdefault((int(rows.min()), int(rows.max() - rows.min() + 1)), []).append(int(p))
         end = 0
         for m0, rows in sorted(blocks_of):
             if m0 < end:
