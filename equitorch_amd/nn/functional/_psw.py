@@ -7,8 +7,9 @@ The reference takes a weight with a batch axis through the same two launches as 
 ``equitorch/nn/functional/tensor_products.py:95-158`` for uvw, ``linears.py:494-571`` for the channel mixing between
 irreps).
 
-A table qualifies when the row ranges that different weight paths write (one output irrep each) coincide or are
-disjoint — true for every table ``tp_infos`` / ``irreps_linear_infos`` / ``irreps_info`` build.
+The kernels walk the table in blocks of output rows: the row ranges of the weight paths, overlapping ranges merged.
+For the tables ``tp_infos`` / ``irreps_linear_infos`` / ``irreps_info`` build a block is one output irrep; a table
+whose blocks exceed ``MAX_BLOCK_ROWS`` rows is left to the library route.
 """
 import ctypes as C
 from typing import Callable, Optional
@@ -22,6 +23,7 @@ from ... import _lib
 from ...ops import kernels
 
 _END_ROW = 1 << 24
+MAX_BLOCK_ROWS = 32      # 16 rows per pass; every further pass streams the block's weights again
 
 
 class PswTable:
@@ -33,17 +35,20 @@ class PswTable:
         coef = np.asarray(coef, dtype=np.float64)
         if max(d1, d2) > 255:
             raise ValueError("operand rows beyond 255")
+        # blocks: row ranges of the paths, ranges that overlap merged into one (an output irrep and all paths into it;
+        # for the SO(2) tables, whose weights couple the rows +m and -m, all orders of an output irrep)
+        spans = sorted((int(out_row[path == p].min()), int(out_row[path == p].max()) + 1, int(p)) for p in np.unique(path))
         blocks_of = {}
-        for p in np.unique(path):
-            rows = out_row[path == p]             # a row in between without a term gets a zero entry below
-            blocks_of.setdefault((int(rows.min()), int(rows.max() - rows.min() + 1)), []).append(int(p))
-        end = 0
-        for m0, rows in sorted(blocks_of):
-            if m0 < end:
-                raise ValueError("output irreps of different paths overlap")
-            end = m0 + rows
-        if max(rows for _, rows in blocks_of) > 255:
-            raise ValueError("an output irrep of more than 255 rows")
+        lo, hi, members = spans[0][0], spans[0][1], []
+        for a0, a1, p in spans:
+            if a0 >= hi:
+                blocks_of[(lo, hi - lo)] = members
+                lo, hi, members = a0, a1, []
+            hi = max(hi, a1)
+            members.append(p)
+        blocks_of[(lo, hi - lo)] = members
+        if max(rows for _, rows in blocks_of) > MAX_BLOCK_ROWS:
+            raise ValueError("a block of more rows than the kernels take in two passes")
         words, coefs, slots, blocks = [], [], [], []
         for (m0, rows), paths in sorted(blocks_of.items()):
             q0 = len(slots)

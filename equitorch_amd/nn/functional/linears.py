@@ -157,7 +157,18 @@ def tensor_product_vu1(input1: Tensor, input2: Tensor, weight: Tensor,
     ``input2 (N, D2, C2)``, ``weight (P, C1, C2)`` -> ``(N, DO)`` (reference ``:414-492``)."""
     _check_batch(input1, input2, weight)
     from . import _uv_gemm
+    if weight.ndim == 4 and input1.ndim == 3 and input2.ndim == 3:
+        # a weight per sample: the uvw product with one output channel, W read as (N, P, C1 * C2, 1)
+        from . import _psw
+        table = _psw.table_of_coo(kernels.coo_of(tp_info_forward), tp_info_forward.info_Mij_fwd.scale, 1, input1.device)
+        w4 = weight.contiguous().flatten(2, 3).unsqueeze(-1)
+        if _psw.launchable(table, input1, input2, w4):
+            kernels.log_tier("tensor_product_vu1", "per-sample weight streaming kernel", str(input1.dtype))
+            shape = weight.shape
+            return _psw.product(table, input1, input2, w4, lambda x, y, w: _uv_gemm.vu1(
+                x, y, w.reshape(shape), tp_info_forward).unsqueeze(-1)).squeeze(-1)
     if input1.ndim == 3 and input2.ndim == 3 and _uv_gemm.supported(input1, input2, weight):
+        kernels.log_tier("tensor_product_vu1", "library GEMM + table-driven kernel", str(input1.dtype))
         return _uv_gemm.vu1(input1, input2, weight, tp_info_forward)
     return tri(spec_from_tp_info(tp_info_forward), ("u", "w", "uw"), "", input1, input2, weight)
 

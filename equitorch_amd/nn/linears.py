@@ -293,7 +293,9 @@ class SO2Linear(nn.Module):
             # per-sample weights: every table entry is a (C_in, C_out) GEMM on one component, batched over samples
             from .functional import _irreps_gemm as G
             plan = G.plan_of_product_info(self.info_forward, self.irreps_in.dim, self.num_weights)
-            return G.mix(input, weight, plan, self.irreps_in.dim)
+            anchor = next(t for t in (self.info_forward.seg_out, self.info_forward.index1,
+                                      self.info_forward.index2, self.info_forward.scale) if t is not None)
+            return G.mix(input, weight, plan, self.irreps_in.dim, anchor=anchor)
         return sparse_vecmat(input, weight, self.info_forward, self.info_backward1, self.info_backward2)
 
     def _apply(self, *args, **kwargs):

@@ -246,3 +246,62 @@ def test_irrep_wise_per_sample_weight(device, monkeypatch, no_library_gemm):
     assert seen and "per-sample weight streaming" in seen[-1], seen
     for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
         assert_close(a, b, 1e-12, f"IrrepWiseLinear per-sample {name}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_so2_linear_uv_per_sample_weight(device, monkeypatch, no_library_gemm, dtype):
+    """``SO2Linear('uv')`` with a weight per sample: a weight couples the rows +m and -m of an output irrep, so the
+    blocks of the walk are whole output irreps with most (path, row) pairs empty."""
+    from equitorch_amd.nn import SO2Linear
+    from oracle import ref_tables
+    irr_in, irr_out, n, cin, cout = "0e+1o+2e+3o", "0e+1o+2e", 130, 8, 12
+    info = ref_tables.so2_linear_infos(irr_out, irr_in)[0]
+    info["scale"] = None if info.get("scale") is None else torch.tensor(info["scale"]).double().tolist()
+    mod = SO2Linear(irr_in, irr_out, cin, cout, internal_weights=False, feature_mode="uv").to(device)
+    g = torch.Generator().manual_seed(12)
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).to(dtype).double()
+    x, w, ct = rd(n, 16, cin), rd(n, mod.num_weights, cin, cout), rd(n, 9, cout)
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    ref = ref_ops.cpu_so2_linear(xr, wr, info, per_sample=True)
+    rgx, rgw = torch.autograd.grad(ref, (xr, wr), ct)
+    seen = _tiers(monkeypatch)
+    xd, wd = (t.to(device, dtype).requires_grad_(True) for t in (x, w))
+    with no_library_gemm():
+        out = mod(xd, wd)
+        gx, gw = torch.autograd.grad(out, (xd, wd), ct.to(device, dtype))
+    assert seen and "per-sample weight streaming" in seen[-1], seen
+    tol = 1e-5 if dtype == torch.float32 else 1e-12
+    for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
+        assert_close(a, b, tol, f"SO2Linear uv per-sample {dtype} {name}")
+
+
+@pytest.mark.parametrize("c1,c2,n,dtype", [(16, 8, 301, torch.float32), (5, 70, 64, torch.float32), (8, 8, 50, torch.float64)])
+def test_vu1_per_sample_weight(device, monkeypatch, no_library_gemm, c1, c2, n, dtype):
+    """``out[n,M] = sum c x[n,a,u] W[n,p,u,w] y[n,b,w]``: the uvw product with a single output channel — a weight row is
+    one element, the lanes of a sample run over the rows."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    io, i1, i2 = _sh(2), _sh(2), "0e+1o"
+    infos = [t.to(device) for t in tp_infos(Irreps(io), Irreps(i1), Irreps(i2))[:3]]
+    T = ref_ops.dense_coupling(io, i1, i2).float().double()
+    g = torch.Generator().manual_seed(stable_seed("psw vu1", c1, c2, n))
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).to(dtype)
+    x, y, w, ct = rd(n, 9, c1), rd(n, 4, c2), rd(n, T.shape[0], c1, c2) / (c1 * c2) ** 0.5, rd(n, 9)
+
+    def dense_vu1(T, x, y, w, dtype=torch.float64):
+        return ref_ops.dense_uvw(T, x, y, w.unsqueeze(-1), dtype=dtype).squeeze(-1)
+    seen = _tiers(monkeypatch)
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    with no_library_gemm():
+        out = F.tensor_product_vu1(xd, yd, wd, *infos)
+        grads = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
+    assert seen and "per-sample weight streaming" in seen[-1], seen
+    ref_out, ref_grads = ref_ops.dense_grads(dense_vu1, T, (x, y, w), ct)
+    tol = 1e-5 if dtype == torch.float32 else 1e-12
+    twin = (None,) * 4
+    if dtype == torch.float32:
+        o32, g32 = ref_ops.dense_grads(dense_vu1, T, (x, y, w), ct, dtype=torch.float32)
+        twin = (o32, *g32)
+    for name, a, b, b32 in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads), twin):
+        assert_close(a, b, tol, f"vu1 per-sample {c1}x{c2} N={n} {dtype} {name}", norm="max", fp32_ref=b32)

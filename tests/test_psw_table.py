@@ -69,14 +69,18 @@ def test_walk_reproduces_the_dense_product(irreps, channelled):
 
 def test_rows_without_a_term_and_tables_the_kernels_do_not_walk():
     """A (path, row) pair without a coefficient gets a zero entry, so the coupled operand's row is defined; row ranges
-    of different paths that overlap partly are refused."""
+    of different paths that overlap are merged into one block; a block beyond two passes of rows is refused."""
     from equitorch_amd.nn.functional._psw import PswTable
     # path 0 writes rows 0..2 but has no term for row 1
     t = PswTable([0, 2], [0, 1], [0, 0], [0, 0], [1.0, 2.0], 2, 1, 3, 1, "cpu")
     assert t.entries.tolist() == [0 | 1 << 24, 1 | 1 << 24, 2 | 1 << 8 | 1 << 24]
     assert t.coef(torch.float64).tolist() == [1.0, 0.0, 2.0]
     assert t.blocks.tolist() == [[0, 3, 0, 1]] and t.slots.tolist() == [[0, 0, 3]]
-    with pytest.raises(ValueError):     # rows 0..1 and 1..2 overlap without coinciding
-        PswTable([0, 1, 1, 2], [0, 0, 0, 0], [0, 0, 0, 0], [0, 0, 1, 1], [1.0] * 4, 1, 1, 3, 2, "cpu")
+    # rows 0..1 and 1..2 overlap without coinciding: one block of three rows, zero entries where a path has no term
+    t = PswTable([0, 1, 1, 2], [0, 0, 0, 0], [0, 0, 0, 0], [0, 0, 1, 1], [1.0] * 4, 1, 1, 3, 2, "cpu")
+    assert t.blocks.tolist() == [[0, 3, 0, 2]] and t.slots.tolist() == [[0, 0, 3], [1, 3, 6]]
+    assert t.coef(torch.float64).tolist() == [1.0, 1.0, 0.0, 0.0, 1.0, 1.0]
+    with pytest.raises(ValueError):     # a block of more rows than two passes take
+        PswTable([0, 40], [0, 0], [0, 0], [0, 0], [1.0, 1.0], 1, 1, 41, 1, "cpu")
     t = PswTable([2, 0], [0, 0], [0, 0], [0, 0], [1.0, 1.0], 1, 1, 4, 1, "cpu")     # row 3 is never written
     assert not t.covers_output and t.blocks.tolist() == [[0, 3, 0, 1]]
