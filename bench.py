@@ -107,6 +107,10 @@ WORKLOADS = {
     # TensorProduct('uvw') with (lmax, U = V = W, batch)
     "u1v_fp32_fwd_bwd": (3, 128, 32768),
     "uvw_fp32_fwd_bwd": (2, 32, 32768),
+    # SO3Linear('uv') with a weight per sample on the streaming kernels: (lmax, C_in = C_out, batch); W is 738 MB
+    "u1v_per_sample_fwd_bwd": (2, 16, 65536),
+    # the edge step for irreps without a compiled table (0e+1o+2e+3o <- 1o+2e+3o x 0e+1o+2e), fused table-driven kernels
+    "edge_table_fwd_bwd": (None, 64, 4096, 65536),
     # the headline edge workload with the per-edge weights formed inside the kernels from 16 features per edge
     "edge_radial_fwd_bwd": (2, 64, 4096, 65536),
     # streaming kernels of known traffic (1 GiB): counter calibration and achievable-bandwidth reference
@@ -820,6 +824,12 @@ def main():
     if args.workload in ("u1v_fp32_fwd_bwd", "uvw_fp32_fwd_bwd"):
         print(json.dumps(fp32_fully_connected_bench(args)))
         return
+    if args.workload == "u1v_per_sample_fwd_bwd":
+        print(json.dumps(per_sample_bench(args)))
+        return
+    if args.workload == "edge_table_fwd_bwd":
+        print(json.dumps(edge_table_bench(args)))
+        return
     if args.workload == "edge_radial_fwd_bwd":
         r = radial_record(16)
         print(json.dumps({
@@ -1086,6 +1096,141 @@ def fp32_fully_connected_bench(args):
                      "traffic": None, "algorithmic_flops": flops, "avg_ms": round(kern["fwd_ms"], 5)},
         "kernels": {**{key: round(v, 5) for key, v in kern.items()},
                     **{key.replace("_ms", "_mfma_frac"): round(v / FP32_MFMA_PEAK_TFLOPS, 4) for key, v in tf.items()}}}
+
+
+def _events_ms(fn, reps):
+    """Average duration of ``fn`` from one pair of events around ``reps`` back-to-back calls on the current stream."""
+    for _ in range(3):
+        fn()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps
+
+
+def per_sample_bench(args):
+    """``tensor_product_u1v`` with a weight per sample (N, P, C, C), fp32, forward + backward through autograd on the
+    streaming kernels.  HBM-bound: the weight is read once forward; backward it is read once and its gradient written
+    once.  Algorithmic bytes: N * P * C * C * 4 per pass over the weight (operands and output are 2-10 % more and are
+    not counted).  The weight tensors rotate over two buffers (1.5 GB: past the last-level cache)."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.ops import kernels
+    from equitorch_amd.utils import tp_infos
+    lmax, ch, n = WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    irreps = "+".join(f"{l}{'e' if l % 2 == 0 else 'o'}" for l in range(lmax + 1))
+    infos = [t.to(dev) for t in tp_infos(Irreps(irreps), Irreps(irreps), Irreps(irreps))[:3]]
+    d, p = (lmax + 1) ** 2, kernels.coo_of(infos[0]).P
+    gen = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn(n, d, ch, device=dev, generator=gen).requires_grad_(True)
+    y = torch.randn(n, d, device=dev, generator=gen).requires_grad_(True)
+    ws = [torch.randn(n, p, ch, ch, device=dev, generator=gen).requires_grad_(True) for _ in range(2)]
+    ct = torch.randn(n, d, ch, device=dev, generator=gen)
+    w_bytes = ws[0].numel() * 4
+    seen = []
+    log, kernels.log_tier = kernels.log_tier, lambda op, tier, detail="": seen.append(tier)
+    F.tensor_product_u1v(x, y, ws[0], *infos)
+    kernels.log_tier = log
+    if not seen or "streaming" not in seen[-1]:
+        raise RuntimeError(f"the per-sample product did not take the streaming kernels: {seen}")
+    count = [0]
+
+    def fwd():
+        count[0] += 1
+        return F.tensor_product_u1v(x, y, ws[count[0] % 2], *infos)
+
+    def step():
+        out = fwd()
+        torch.autograd.grad(out, (x, y, ws[count[0] % 2]), ct)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) / args.steps * 1e3
+    with torch.no_grad():
+        fwd_ms = _events_ms(fwd, args.kernel_reps)
+    outs = [F.tensor_product_u1v(x, y, w, *infos) for w in ws]
+
+    def bwd():
+        count[0] += 1
+        i = count[0] % 2
+        torch.autograd.grad(outs[i], (x, y, ws[i]), ct, retain_graph=True)
+    bwd_ms = _events_ms(bwd, args.kernel_reps)
+    rate = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
+    copy_gbs, read_gbs = stream_rate("copy", 20, 3)[0], stream_rate("read", 20, 3)[0]
+    return {
+        "metric": f"u1v per-sample weight fwd+bwd Msamples/s (lmax={lmax},C={ch})", "value": round(n / (ms_step * 1e-3) / 1e6, 2),
+        "unit": "Msamples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: N={n}, irreps {irreps}, {ch} -> {ch} channels, weight {tuple(ws[0].shape)} "
+                               f"per sample ({w_bytes / 1e6:.0f} MB), forward + backward through autograd"},
+        "roofline": {"bound": "hbm", "kernel": "cgtp::psw_bwd_kernel<float,4,false>", "achieved": round(rate(2 * w_bytes, bwd_ms), 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(rate(2 * w_bytes, bwd_ms) / HBM_PEAK_GBS, 4),
+                     "traffic": None, "algorithmic_bytes": 2 * w_bytes, "avg_ms": round(bwd_ms, 5),
+                     "achievable": {"copy_GBs": round(copy_gbs, 1), "read_GBs": round(read_gbs, 1),
+                                    "frac_of_copy": round(rate(2 * w_bytes, bwd_ms) / copy_gbs, 4)}},
+        "kernels": {"fwd_ms": round(fwd_ms, 5), "fwd_GBs": round(rate(w_bytes, fwd_ms), 1),
+                    "fwd_frac_of_peak": round(rate(w_bytes, fwd_ms) / HBM_PEAK_GBS, 4),
+                    "fwd_frac_of_read": round(rate(w_bytes, fwd_ms) / read_gbs, 4),
+                    "bwd_ms": round(bwd_ms, 5), "bwd_GBs": round(rate(2 * w_bytes, bwd_ms), 1)}}
+
+
+def edge_table_bench(args):
+    """The edge step (gather, channel-wise product, segment sum; forward + backward) for an irreps triple without a
+    compiled table, on the fused table-driven kernels, next to the three separate launches they replace and to the
+    compiled lmax = 2 table on the same graph."""
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu
+    from equitorch_amd.ops import kernels
+    _, ch, n_nodes, n_edges = WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    gen = torch.Generator().manual_seed(0)
+    src = torch.randint(0, n_nodes, (n_edges,), generator=gen)
+    dst = torch.randint(0, n_nodes, (n_edges,), generator=gen)
+    plan = EdgePlan(src.to(dev), dst.to(dev), n_nodes)
+    triple = ("0e+1o+2e+3o", "1o+2e+3o", "0e+1o+2e")
+    fused_table = kernels.uvu_table_of
+    res, nnz = {}, {}
+    for name, (io, i1, i2), table_of in (("table", triple, fused_table), ("separate", triple, lambda *a: None),
+                                         ("compiled", ("0e+1o+2e",) * 3, fused_table)):
+        kernels.uvu_table_of = table_of
+        try:
+            mod = SO3Linear(i1, i2, io, ch, ch, internal_weights=False, feature_mode="uu").to(dev)
+            nnz[name] = int(kernels.coo_of(mod.tp_info_forward).coef.shape[0])
+            x = torch.randn(n_nodes, Irreps(i1).dim, ch, device=dev, requires_grad=True)
+            y = torch.randn(n_edges, Irreps(i2).dim, device=dev, requires_grad=True)
+            w = torch.randn(n_edges, mod.num_paths, ch, device=dev, requires_grad=True)
+            ct = torch.randn(n_nodes, Irreps(io).dim, ch, device=dev)
+
+            def fwd():
+                return edge_tensor_product_uu(x, y, w, plan, mod.tp_info_forward)
+
+            def step():
+                torch.autograd.grad(fwd(), (x, y, w), ct)
+            with torch.no_grad():
+                f = _events_ms(fwd, args.kernel_reps)
+            res[name] = {"fwd_ms": round(f, 4), "step_ms": round(_events_ms(step, args.kernel_reps), 4)}
+        finally:
+            kernels.uvu_table_of = fused_table
+    ms_step = res["table"]["step_ms"]
+    per_coef = {k: v["step_ms"] / nnz[k] for k, v in res.items()}
+    return {
+        "metric": "edge-TP fwd+bwd Medges/s (irreps without a compiled table, C=64)", "value": round(n_edges / (ms_step * 1e-3) / 1e6, 2),
+        "unit": "Medges/s", "n_gpus": 1, "steps": args.kernel_reps, "warmup": 3, "ms_per_step": ms_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: N={n_nodes} nodes, E={n_edges} edges, {triple[0]} <- {triple[1]} x {triple[2]} "
+                               f"({nnz['table']} coefficients), C={ch}, per-edge weights"},
+        "kernels": {**res, "coefficients": nnz,
+                    "per_coefficient_vs_compiled": round(per_coef["table"] / per_coef["compiled"], 2),
+                    "fused_vs_separate": round(res["separate"]["step_ms"] / ms_step, 2)}}
 
 
 def radial_record(r):
