@@ -552,7 +552,11 @@ def algorithmic_bytes(n_nodes, n_edges, d, p, ch):
     return fwd, bwd
 
 
-FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X fp32, vendor figure
+FP32_VECTOR_PEAK_TFLOPS = 157.3  # MI355X fp32, vendor figure (packed instructions: two values per lane and issue)
+FP32_UNPACKED_PEAK_TFLOPS = 78.6  # the same with one value per lane: what code built with packed fp32 off can issue at most
+# per the data sheet; a register-only loop of independent v_fma_f32 on this chip issues one every 1.15 ns per SIMD from
+# two wavefronts per SIMD up (2.07 ns from one): 114 TFLOP/s over 1024 SIMDs
+FP32_MEASURED_ISSUE_TFLOPS = 114.0
 
 
 def edge_rows_bench(args):
@@ -628,10 +632,15 @@ def edge_rows_bench(args):
                      "algorithmic_bytes": bwd_bytes + msg, "avg_ms": round(bwd_ms, 4),
                      "fp32_vector": {"achieved": round(tf, 2), "peak": FP32_VECTOR_PEAK_TFLOPS, "unit": "TFLOP/s",
                                      "frac": round(tf / FP32_VECTOR_PEAK_TFLOPS, 4),
+                                     "unpacked_peak": FP32_UNPACKED_PEAK_TFLOPS,
+                                     "frac_of_unpacked": round(tf / FP32_UNPACKED_PEAK_TFLOPS, 4),
+                                     "measured_issue_rate": FP32_MEASURED_ISSUE_TFLOPS,
+                                     "frac_of_measured_issue_rate": round(tf / FP32_MEASURED_ISSUE_TFLOPS, 4),
                                      "algorithmic_flops": 3 * flops_fwd}},
         "kernels": {"fwd_ms": round(fwd_ms, 4), "bwd_ms": round(bwd_ms, 4),
                     "rows_fwd_ms": round(rows_fwd_ms, 4), "rows_bwd_ms": round(rows_bwd_ms, 4),
                     "fwd_TFLOPs": round(flops_fwd / (fwd_ms * 1e-3) / 1e12, 2),
+                    "fwd_fp32_frac_of_unpacked": round(flops_fwd / (fwd_ms * 1e-3) / 1e12 / FP32_UNPACKED_PEAK_TFLOPS, 4),
                     "fwd_GBs": round((fwd_bytes + msg) / (fwd_ms * 1e-3) / 1e9, 1)},
     }
     if not args.no_cpu_baseline:
@@ -1004,7 +1013,10 @@ def other_configs(args, headline):
     out["cfg4_edge_fwd_bwd_lmax6_C32"] = {
         "Medges_s": r["value"], "step_ms": r["ms_per_step"], "fwd_ms": r["kernels"]["fwd_ms"],
         "bwd_ms": r["kernels"]["bwd_ms"], "bwd_hbm_frac": r["roofline"]["frac"],
-        "bwd_fp32_frac": r["roofline"]["fp32_vector"]["frac"], "fwd_TFLOPs": r["kernels"]["fwd_TFLOPs"]}
+        "bwd_fp32_frac": r["roofline"]["fp32_vector"]["frac"],
+        "bwd_fp32_frac_of_unpacked": r["roofline"]["fp32_vector"]["frac_of_unpacked"],
+        "fwd_TFLOPs": r["kernels"]["fwd_TFLOPs"],
+        "fwd_fp32_frac_of_unpacked": r["kernels"]["fwd_fp32_frac_of_unpacked"]}
     return out
 
 
