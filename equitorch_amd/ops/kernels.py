@@ -454,7 +454,32 @@ class SegIndex:
         self.ptr, self.perm, self.seg_ids, self.gather = ptr, perm, seg_ids, gather
         self.positions_per_wave = positions_per_wave
         self.wave_seg = self.aligned_ranges(ptr, positions_per_wave)
+        # the step-balanced cuts for every slot count a launch can have (64 / lanes per edge), built here, where a host
+        # sync is expected, and not on the first backward (inside autograd, possibly under graph capture)
         self._wave_pos = {}
+        self._build_balanced(self.SLOT_COUNTS)
+
+    SLOT_COUNTS = (1, 2, 4, 8, 16, 32, 64)
+
+    def _build_balanced(self, slot_counts) -> None:
+        import numpy as np
+        ptr = self.ptr.detach().cpu().numpy()
+        n_pos = int(ptr[-1]) if ptr.shape[0] else 0
+        for slots in slot_counts:
+            if n_pos == 0:
+                self._wave_pos[slots] = None
+                continue
+            steps = (np.diff(ptr) + slots - 1) // slots
+            last = np.cumsum(steps)                            # steps up to and including each segment
+            first = last - steps
+            # as many ranges as equal cuts by position would give (a launch sized for that many wavefronts stays
+            # resident in one round)
+            n_ranges = max(1, n_pos // self.positions_per_wave)
+            per_wave = max(1, -(-int(last[-1]) // n_ranges))
+            targets = np.arange(0, int(last[-1]), per_wave, dtype=np.int64)
+            seg = np.searchsorted(last, targets, side="right")
+            pos = ptr[:-1][seg] + (targets - first[seg]) * slots
+            self._wave_pos[slots] = torch.from_numpy(np.concatenate([pos, [n_pos]]).astype(np.int64)).to(self.ptr.device)
 
     @staticmethod
     def aligned_ranges(ptr: Tensor, positions_per_wave: int) -> Optional[Tensor]:
@@ -481,23 +506,8 @@ class SegIndex:
         degree 16."""
         if slots <= 0:
             return None
-        if slots not in self._wave_pos:
-            ptr = self.ptr
-            n_pos = int(ptr[-1])
-            if n_pos == 0:
-                self._wave_pos[slots] = None
-            else:
-                steps = (ptr[1:] - ptr[:-1] + slots - 1) // slots
-                last = torch.cumsum(steps, 0)                      # steps up to and including each segment
-                first = last - steps
-                # as many ranges as equal cuts by position would give (a launch sized for that many wavefronts
-                # stays resident in one round)
-                n_ranges = max(1, n_pos // self.positions_per_wave)
-                per_wave = max(1, -(-int(last[-1]) // n_ranges))
-                targets = torch.arange(0, int(last[-1]), per_wave, device=ptr.device, dtype=ptr.dtype)
-                seg = torch.searchsorted(last, targets, right=True)
-                pos = ptr[:-1][seg] + (targets - first[seg]) * slots
-                self._wave_pos[slots] = torch.cat([pos, pos.new_full((1,), n_pos)]).contiguous()
+        if slots not in self._wave_pos:      # a slot count outside SLOT_COUNTS: built now (reads ptr back: a host sync)
+            self._build_balanced((slots,))
         return self._wave_pos[slots]
 
 
