@@ -89,21 +89,28 @@ __global__ void __launch_bounds__(256) uvu_seg_fwd_radial_kernel(const UvuDev<fl
   for (int off0 = 0; off0 < I.npos;) {
     int ei, oi;
     const bool valid = seg_step_begin<T, DO, V>(st, acc, a.out, a.ws, I, off0, ei, oi, wave, R, L, 4, true, C, c0);
-    // slots past the segment boundary carry the position the step started at: their weights are formed and dropped
-    T w[P][V];
-    radial_weights<TP>(rw_lds, a.rh, a.R, __shfl(ei, (L.lane & 3) << 4, kWave), L.lane, w);
+    // the edge's operands are requested first: the gathers are in flight while the weights are formed
+    T x[D1][V], y[D2], yv[3];
     if (valid) {
       const int64_t e = ei, xr = oi;
-      T x[D1][V], y[D2];
       if constexpr (YV) {
-        const ShPoint<T> pt(a.y[e * 3], a.y[e * 3 + 1], a.y[e * 3 + 2], a.y_vec == kYUnitVector);
-        sh_values<T, TP::SH_LMAX>(pt.x, pt.y, pt.z, y);
+#pragma unroll
+        for (int j = 0; j < 3; ++j) yv[j] = a.y[e * 3 + j];
       } else {
 #pragma unroll
         for (int j = 0; j < D2; ++j) y[j] = a.y[e * D2 + j];
       }
 #pragma unroll
       for (int i = 0; i < D1; ++i) load_vec<T, V>(x[i], a.x + (xr * D1 + i) * C + c0);
+    }
+    // slots past the segment boundary carry the position the step started at: their weights are formed and dropped
+    T w[P][V];
+    radial_weights<TP>(rw_lds, a.rh, a.R, __shfl(ei, (L.lane & 3) << 4, kWave), L.lane, w);
+    if (valid) {
+      if constexpr (YV) {
+        const ShPoint<T> pt(yv[0], yv[1], yv[2], a.y_vec == kYUnitVector);
+        sh_values<T, TP::SH_LMAX>(pt.x, pt.y, pt.z, y);
+      }
       TP::template fwd<T, V>(x, y, [&](int p, T (&wp)[V]) {
 #pragma unroll
         for (int v = 0; v < V; ++v) wp[v] = w[p][v];
