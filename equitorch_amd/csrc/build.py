@@ -60,7 +60,33 @@ def build(jobs: int = 8) -> str:
         res = subprocess.run(cmd, capture_output=True, text=True)
         if res.returncode != 0:
             raise RuntimeError(f"link of {path} failed:\n{res.stdout}\n{res.stderr}")
+    build_torch_shim()
     return LIB_PATH
+
+
+SHIM_PATH = os.path.join(LIB_DIR, "_cgtp_torch.so")
+
+
+def build_torch_shim() -> str:
+    """The PyTorch C++ extension over the C ABI (``torch_shim/cgtp_torch.cpp``: autograd node, argument block and
+    allocation of the fused edge product), compiled with the host compiler against this interpreter's torch and
+    linked to ``libcgtp.so`` next to it.  No device code."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension
+    src = os.path.join(HERE, "torch_shim", "cgtp_torch.cpp")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-fPIC", "-shared", "-std=c++17", src, "-o", SHIM_PATH,
+           "-DTORCH_EXTENSION_NAME=_cgtp_torch", "-DTORCH_API_INCLUDE_EXTENSION_H", "-DUSE_ROCM",
+           "-D__HIP_PLATFORM_AMD__=1", f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           *[f"-I{d}" for d in cpp_extension.include_paths()], f"-I{sysconfig.get_paths()['include']}",
+           "-I/opt/rocm/include", f"-I{os.path.join(ROOT, 'include')}",
+           *[f"-L{d}" for d in cpp_extension.library_paths()], "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip",
+           "-ltorch_hip", "-ltorch_python", f"-L{LIB_DIR}", "-lcgtp", "-Wl,-rpath,$ORIGIN"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"build of {SHIM_PATH} failed:\n{res.stdout}\n{res.stderr}")
+    return SHIM_PATH
 
 
 if __name__ == "__main__":

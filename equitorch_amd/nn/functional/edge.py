@@ -88,6 +88,28 @@ def _check_edge_operands(x: Tensor, y: Tensor, plan: EdgePlan, tp_info: TensorPr
             raise _lib.CgtpError(f"w_last must be ({h.shape[1]}, {coo.P}, {c}), got {tuple(w_last.shape)}")
 
 
+def _shim_handle(plan: EdgePlan, cfg, x: Tensor, y_vec: int):
+    """The C++ extension's handle of this plan for one compiled table, dtype and channel count (it holds the sorted
+    views and the range tables of both directions), or None when the extension is not there or the table needs the
+    weights rearranged (a subset of the compiled paths)."""
+    from ... import _shim
+    mod = _shim.module()
+    if mod is None or getattr(cfg, "w_rows", None) is not None:
+        return None
+    scale_np = getattr(cfg, "path_scale", None)
+    key = (int(cfg), x.dtype, x.shape[-1], y_vec, None if scale_np is None else scale_np.tobytes())
+    handles = plan.__dict__.setdefault("_shim_handles", {})
+    if key not in handles:
+        code = _lib.dtype_code(x.dtype)
+        scale = cfg.scale_tensor(x.dtype, x.device) if isinstance(cfg, kernels.Cfg) else None
+        views = []
+        for seg, backward in ((plan.fwd_index, False), (plan.bwd_index, True)):
+            wave_seg, wave_pos = kernels.seg_ranges(cfg, seg, code, x.shape[-1], backward)
+            views += [seg.ptr, seg.perm, seg.seg_ids, seg.gather, wave_seg, wave_pos]
+        handles[key] = mod.EdgeHandle(int(cfg), int(kernels.uvu_dims(cfg)[2]), int(y_vec), scale, *views)
+    return handles[key]
+
+
 class _EdgeUvuCompiled(Function):
     @staticmethod
     def forward(ctx, x: Tensor, sh: Tensor, w: Tensor, plan: EdgePlan, tp_info: TensorProductInfo, cfg: int):
@@ -216,6 +238,10 @@ def edge_tensor_product_uu(x: Tensor, sh: Tensor, weight: Tensor, plan: EdgePlan
         xc, yc, wc = x.contiguous(), sh.contiguous(), weight.contiguous()
         if kernels.uvu_launchable(cfg, xc, yc, wc, segments=True):
             kernels.log_tier("edge_tensor_product_uu", "fused gather / product / segment sum", f"config {int(cfg)}")
+            handle = _shim_handle(plan, cfg, xc, 0)
+            if handle is not None:
+                from ... import _shim
+                return _shim.module().edge_uvu(xc, yc, wc, handle)
             return _EdgeUvuCompiled.apply(xc, yc, wc, plan, tp_info_forward, cfg)
         if kernels.uvu_launchable(cfg, xc, yc, wc, gathered=True):
             kernels.log_tier("edge_tensor_product_uu", "block-wise row kernels + segment sums", f"config {int(cfg)}")
@@ -256,6 +282,10 @@ def edge_tensor_product_uu_vectors(x: Tensor, edge_vec: Tensor, weight: Tensor, 
             and x.dtype in (torch.float32, torch.float64)):
         xc, vc, wc = x.contiguous(), edge_vec.contiguous(), weight.contiguous()
         if kernels.uvu_launchable(cfg, xc, vc, wc, segments=True, y_vec=mode):
+            handle = _shim_handle(plan, cfg, xc, mode)
+            if handle is not None:
+                from ... import _shim
+                return _shim.module().edge_uvu(xc, vc, wc, handle)
             return _EdgeUvuVectors.apply(xc, vc, wc, plan, cfg, mode)
     d2 = int(kernels.coo_of(tp_info_forward).D2)
     l_max = int(round(d2 ** 0.5)) - 1

@@ -511,6 +511,22 @@ class SegIndex:
         return self._wave_pos[slots]
 
 
+def seg_ranges(cfg: int, seg: SegIndex, dtype_code: int, channels: int, backward: bool):
+    """``(wave_seg, wave_pos)``, at most one of them a tensor: how a segment-mode launch of ``cfg`` cuts the sorted list
+    into one range per wavefront (``_RANGE_MODE``); both None = ranges of equal numbers of positions, which is also all
+    the block-wise kernels of the large tables take."""
+    if _lib.lib.cgtp_uvu_blockwise_only(int(cfg)):
+        return None, None
+    wave_pos = None
+    if _RANGE_MODE == "balanced" or (_RANGE_MODE == "auto" and (backward or seg.wave_seg is None)):
+        wave_pos = seg.balanced_positions(int(_lib.lib.cgtp_uvu_slots(int(cfg), dtype_code, channels, int(backward))))
+    if wave_pos is not None:
+        return None, wave_pos
+    if seg.wave_seg is not None and _RANGE_MODE != "positions":
+        return seg.wave_seg, None
+    return None, None
+
+
 def _uvu_args(cfg: int, x: Tensor, y: Tensor, w: Tensor, seg: Optional[SegIndex], gather: Optional[Tensor],
               pos_per_wave: int = 0, y_vec: int = 0, backward: bool = False) -> UvuArgs:
     a = UvuArgs()
@@ -524,14 +540,12 @@ def _uvu_args(cfg: int, x: Tensor, y: Tensor, w: Tensor, seg: Optional[SegIndex]
         a.ptr, a.perm, a.seg_ids, a.gather = seg.ptr.data_ptr(), _lib.ptr(seg.perm), seg.seg_ids.data_ptr(), \
             seg.gather.data_ptr()
         a.pos_per_wave = pos_per_wave
-        if pos_per_wave == 0 and not _lib.lib.cgtp_uvu_blockwise_only(int(cfg)):   # those cut ranges by position
-            wave_pos = None
-            if _RANGE_MODE == "balanced" or (_RANGE_MODE == "auto" and (backward or seg.wave_seg is None)):
-                wave_pos = seg.balanced_positions(int(_lib.lib.cgtp_uvu_slots(int(cfg), a.dtype, a.C, int(backward))))
+        if pos_per_wave == 0:
+            wave_seg, wave_pos = seg_ranges(cfg, seg, a.dtype, a.C, backward)
             if wave_pos is not None:
                 a.wave_pos, a.n_waves = wave_pos.data_ptr(), wave_pos.shape[0] - 1
-            elif seg.wave_seg is not None and _RANGE_MODE != "positions":
-                a.wave_seg, a.n_waves = seg.wave_seg.data_ptr(), seg.wave_seg.shape[0] - 1
+            elif wave_seg is not None:
+                a.wave_seg, a.n_waves = wave_seg.data_ptr(), wave_seg.shape[0] - 1
     else:
         a.gather = _lib.ptr(gather)
     a.x, a.y, a.w = x.data_ptr(), y.data_ptr(), w.data_ptr()

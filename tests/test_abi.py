@@ -363,3 +363,16 @@ def test_radial_mode_validates_on_the_host():
     assert L.cgtp_uvu_radial_grad(p16, p16, p16, p16, p16, p16, 100, 16, 3, _lib.F32, None) == 2
     assert L.cgtp_uvu_radial_grad(p16, p16, p16, None, p16, p16, 100, 16, 11, _lib.F32, None) == 1
     assert L.cgtp_uvu_radial_grad(p16, p16, p16, p16, p16, p16, 100, 16, 11, _lib.F64, None) == 4
+
+
+def test_torch_extension_loads_and_matches_the_library():
+    """The PyTorch C++ extension over the C ABI imports without a GPU, was built against this libcgtp (ABI version),
+    and takes a plan's index tensors as they are."""
+    import torch
+
+    from equitorch_amd import _lib, _shim
+    mod = _shim.module()
+    assert mod is not None, "equitorch_amd/lib/_cgtp_torch.so is not built"
+    assert mod.abi_version() == _lib.lib.cgtp_version()
+    i = torch.zeros(3, dtype=torch.int64)
+    mod.EdgeHandle(0, 9, 0, None, i, None, i, i, None, i, i, i, i, i, torch.zeros(2, dtype=torch.int32), None)
