@@ -305,3 +305,53 @@ def test_vu1_per_sample_weight(device, monkeypatch, no_library_gemm, c1, c2, n, 
         twin = (o32, *g32)
     for name, a, b, b32 in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads), twin):
         assert_close(a, b, tol, f"vu1 per-sample {c1}x{c2} N={n} {dtype} {name}", norm="max", fp32_ref=b32)
+
+
+@pytest.mark.parametrize("n", [1, 2, 63, 4097])
+def test_sample_counts_at_the_edges_of_a_wavefront(device, monkeypatch, no_library_gemm, n):
+    """One sample, fewer samples than a wavefront takes, and a count that leaves the last wavefront partly empty
+    (16 -> 8 channels: 16 samples a wavefront at 4097)."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    irr = _sh(2)
+    infos = [t.to(device) for t in tp_infos(Irreps(irr), Irreps(irr), Irreps(irr))[:3]]
+    T = ref_ops.dense_coupling(irr, irr, irr).float().double()
+    g = torch.Generator().manual_seed(n)
+    x, y, w, ct = (torch.randn(*s, generator=g) for s in ((n, 9, 16), (n, 9), (n, T.shape[0], 16, 8), (n, 9, 8)))
+    seen = _tiers(monkeypatch)
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    with no_library_gemm():
+        out = F.tensor_product_u1v(xd, yd, wd, *infos)
+        grads = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
+    assert "per-sample weight streaming" in seen[-1], seen
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x, y, w), ct)
+    for name, a, b in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads)):
+        assert_close(a, b, 1e-5, f"u1v per-sample N={n} {name}", norm="max")
+
+
+def test_no_samples_and_operands_the_kernels_do_not_take(device, monkeypatch):
+    """An empty batch, a weight view that is not contiguous, and more output channels than a wavefront covers: the
+    product still returns the right result (an empty tensor; a copy; the library route)."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    irr = _sh(1)
+    infos = [t.to(device) for t in tp_infos(Irreps(irr), Irreps(irr), Irreps(irr))[:3]]
+    T = ref_ops.dense_coupling(irr, irr, irr).float().double()
+    p = T.shape[0]
+    out = F.tensor_product_u1v(torch.zeros(0, 4, 8, device=device), torch.zeros(0, 4, device=device),
+                               torch.zeros(0, p, 8, 8, device=device), *infos)
+    assert out.shape == (0, 4, 8)
+    g = torch.Generator().manual_seed(0)
+    n = 33
+    x, y = torch.randn(n, 4, 8, generator=g), torch.randn(n, 4, generator=g)
+    w_t = torch.randn(n, p, 12, 8, generator=g)                    # the product sees its transpose: a strided view
+    seen = _tiers(monkeypatch)
+    out = F.tensor_product_u1v(x.to(device), y.to(device), w_t.to(device).transpose(2, 3), *infos)
+    assert "per-sample weight streaming" in seen[-1], seen
+    assert_close(out, ref_ops.dense_u1v(T, x, y, w_t.transpose(2, 3)), 1e-5, "u1v per-sample, strided weight", norm="max")
+    w_wide = torch.randn(n, p, 8, 260, generator=g)                # 260 channels: beyond 64 lanes of four
+    out = F.tensor_product_u1v(x.to(device), y.to(device), w_wide.to(device), *infos)
+    assert "per-sample weight streaming" not in seen[-1], seen
+    assert_close(out, ref_ops.dense_u1v(T, x, y, w_wide), 1e-5, "u1v per-sample, 260 output channels", norm="max")
