@@ -312,7 +312,7 @@ __device__ __forceinline__ void psw_carry_back(const PswDev<T>& a, const PswLayo
   }
 }
 
-template <typename T, int V, int JB>
+template <typename T, int V, int JB, int NB>
 __device__ __forceinline__ void psw_bwd_block(const PswDev<T>& a, const PswLayout& lay, T* lds, const PswLane& L,
                                               int64_t n, bool sample_ok, int m0, int rows, int j0, int q0, int q1) {
   const auto slots = psw_constant(a.slots);
@@ -336,13 +336,13 @@ __device__ __forceinline__ void psw_bwd_block(const PswDev<T>& a, const PswLayou
       }
     }
   }
-  // flat walk as in the forward, two rows a lane per batch
-  const auto load_batch = [&](T (&wv)[2][V], int q, int k0, int kk0) {
+  // flat walk as in the forward, NB rows a lane per batch
+  const auto load_batch = [&](T (&wv)[NB][V], int q, int k0, int kk0) {
     const int p = slots[3 * q];
     const int TKc = a.K - k0 < a.TK ? a.K - k0 : a.TK;
     const T* wrow = a.w + ((n * a.P + p) * (int64_t)a.K + k0) * a.Wc + L.wl * V;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NB; ++i) {
       const int kk = kk0 + i * L.KS + L.ks;
       if (want_t && lane_ok && kk < TKc) {
         load_vec_stream<T, V>(wv[i], wrow + (int64_t)kk * a.Wc);
@@ -353,7 +353,7 @@ __device__ __forceinline__ void psw_bwd_block(const PswDev<T>& a, const PswLayou
     }
   };
   int q = q0, k0 = 0, kk0 = 0;
-  T cur[2][V];
+  T cur[NB][V];
   if (q < q1) load_batch(cur, q, k0, kk0);
   while (q < q1) {
     const int p = slots[3 * q], e0 = slots[3 * q + 1], e1 = slots[3 * q + 2];
@@ -363,24 +363,24 @@ __device__ __forceinline__ void psw_bwd_block(const PswDev<T>& a, const PswLayou
       if (want_w) psw_form_t(a, t, xs, ys, e0, e1, k0, TKc, L);
       psw_wave_sync();
     }
-    int nq = q, nk0 = k0, nkk0 = kk0 + 2 * L.KS;
+    int nq = q, nk0 = k0, nkk0 = kk0 + NB * L.KS;
     if (nkk0 >= TKc) {
       nkk0 = 0;
       nk0 = k0 + a.TK;
       if (nk0 >= a.K) { nk0 = 0; ++nq; }
     }
-    T nxt[2][V];
+    T nxt[NB][V];
     if (nq < q1) {
       load_batch(nxt, nq, nk0, nkk0);
     } else {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < NB; ++i)
 #pragma unroll
         for (int v = 0; v < V; ++v) nxt[i][v] = T(0);
     }
     T* gwrow = want_w ? a.gw + ((n * a.P + p) * (int64_t)a.K + k0) * a.Wc + L.wl * V : nullptr;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NB; ++i) {
       const int kk = kk0 + i * L.KS + L.ks;
       const bool active = kk < TKc;
       const int row = active ? kk : TKc - 1;
@@ -420,14 +420,14 @@ __device__ __forceinline__ void psw_bwd_block(const PswDev<T>& a, const PswLayou
       psw_carry_back(a, lay, lds, L, e0, e1, k0, TKc, j0, jb);
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < NB; ++i)
 #pragma unroll
       for (int v = 0; v < V; ++v) cur[i][v] = nxt[i][v];
     q = nq; k0 = nk0; kk0 = nkk0;
   }
 }
 
-template <typename T, int V, bool BIG>
+template <typename T, int V, bool BIG, int NB>
 __global__ void __launch_bounds__(kWave) psw_bwd_kernel(const PswDev<T> a) {
   extern __shared__ __align__(16) unsigned char psw_lds_raw[];
   const PswLane L(a.s_log2, a.lps_log2);
@@ -445,11 +445,11 @@ __global__ void __launch_bounds__(kWave) psw_bwd_kernel(const PswDev<T> a) {
     const int m0 = blocks[4 * b], rows_all = blocks[4 * b + 1], q0 = blocks[4 * b + 2], q1 = blocks[4 * b + 3];
     for (int j0 = 0; j0 < rows_all;) {
       const int rows = rows_all - j0;
-      if (rows <= 1) { psw_bwd_block<T, V, 1>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 1; }
-      else if (rows <= 3) { psw_bwd_block<T, V, 3>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 3; }
-      else if (rows <= 5) { psw_bwd_block<T, V, 5>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 5; }
-      else if (!BIG || rows <= 8) { psw_bwd_block<T, V, 8>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 8; }
-      else if constexpr (BIG) { psw_bwd_block<T, V, 16>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 16; }
+      if (rows <= 1) { psw_bwd_block<T, V, 1, NB>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 1; }
+      else if (rows <= 3) { psw_bwd_block<T, V, 3, NB>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 3; }
+      else if (rows <= 5) { psw_bwd_block<T, V, 5, NB>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 5; }
+      else if (!BIG || rows <= 8) { psw_bwd_block<T, V, 8, NB>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 8; }
+      else if constexpr (BIG) { psw_bwd_block<T, V, 16, NB>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 16; }
     }
   }
   psw_wave_sync();
@@ -551,8 +551,14 @@ int psw_launch_t(const cgtp_psw_args* a, const cgtp_psw_table* tab, bool backwar
     if (plan.V == 1) big ? go(psw_fwd_kernel<T, 1, true>) : go(psw_fwd_kernel<T, 1, false>);
     else big ? go(psw_fwd_kernel<T, VEC, true>) : go(psw_fwd_kernel<T, VEC, false>);
   } else {
-    if (plan.V == 1) big ? go(psw_bwd_kernel<T, 1, true>) : go(psw_bwd_kernel<T, 1, false>);
-    else big ? go(psw_bwd_kernel<T, VEC, true>) : go(psw_bwd_kernel<T, VEC, false>);
+    // rows of W a lane has in flight per batch: four when the weights come from HBM (bytes in flight are what the
+    // rate follows: 0.50 -> 0.42 ms at 738 MB), two when they fit the 256 MB last-level cache (loads return sooner
+    // and the fourth wavefront per SIMD that the smaller batch leaves room for counts more: 0.10 against 0.14 ms at
+    // 185 MB) and in the kernels with the 16-row pass (registers)
+    const int64_t w_bytes = a->n_rows * (int64_t)tab->P * d.K * d.Wc * (int64_t)sizeof(T);
+    const bool deep = !big && w_bytes > (256LL << 20);
+    if (plan.V == 1) big ? go(psw_bwd_kernel<T, 1, true, 2>) : deep ? go(psw_bwd_kernel<T, 1, false, 4>) : go(psw_bwd_kernel<T, 1, false, 2>);
+    else big ? go(psw_bwd_kernel<T, VEC, true, 2>) : deep ? go(psw_bwd_kernel<T, VEC, false, 4>) : go(psw_bwd_kernel<T, VEC, false, 2>);
   }
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
