@@ -128,7 +128,7 @@ __device__ __forceinline__ void psw_form_t(const PswDev<T>& a, T* t, const T* xs
 }
 
 // ---- forward --------------------------------------------------------------------------------------------
-template <typename T, int V, int JB>
+template <typename T, int V, int JB, int NB>
 __device__ __forceinline__ void psw_fwd_block(const PswDev<T>& a, const PswLayout& lay, T* lds, const PswLane& L,
                                               int64_t n, bool sample_ok, int m0, int rows, int j0, int q0, int q1) {
   const auto slots = psw_constant(a.slots);
@@ -141,14 +141,14 @@ __device__ __forceinline__ void psw_fwd_block(const PswDev<T>& a, const PswLayou
   for (int j = 0; j < JB; ++j)
 #pragma unroll
     for (int v = 0; v < V; ++v) acc[j][v] = T(0);
-  // The walk over (path, chunk of rows, batch of 4 rows a lane) is flat: the rows of the next batch are requested
+  // The walk over (path, chunk of rows, batch of NB rows a lane) is flat: the rows of the next batch are requested
   // before the current ones are used, across chunk and path boundaries, so forming a chunk's t overlaps the loads.
-  const auto load_batch = [&](T (&wv)[4][V], int q, int k0, int kk0) {
+  const auto load_batch = [&](T (&wv)[NB][V], int q, int k0, int kk0) {
     const int p = slots[3 * q];
     const int TKc = a.K - k0 < a.TK ? a.K - k0 : a.TK;
     const T* wrow = a.w + ((n * a.P + p) * (int64_t)a.K + k0) * a.Wc + L.wl * V;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < NB; ++i) {
       const int kk = kk0 + i * L.KS + L.ks;
       if (lane_ok && kk < TKc) {
         load_vec_stream<T, V>(wv[i], wrow + (int64_t)kk * a.Wc);
@@ -159,7 +159,7 @@ __device__ __forceinline__ void psw_fwd_block(const PswDev<T>& a, const PswLayou
     }
   };
   int q = q0, k0 = 0, kk0 = 0;
-  T cur[4][V];
+  T cur[NB][V];
   if (q < q1) load_batch(cur, q, k0, kk0);
   while (q < q1) {
     const int TKc = a.K - k0 < a.TK ? a.K - k0 : a.TK;
@@ -168,23 +168,23 @@ __device__ __forceinline__ void psw_fwd_block(const PswDev<T>& a, const PswLayou
       psw_form_t(a, t, xs, ys, slots[3 * q + 1], slots[3 * q + 2], k0, TKc, L);
       psw_wave_sync();
     }
-    int nq = q, nk0 = k0, nkk0 = kk0 + 4 * L.KS;
+    int nq = q, nk0 = k0, nkk0 = kk0 + NB * L.KS;
     if (nkk0 >= TKc) {
       nkk0 = 0;
       nk0 = k0 + a.TK;
       if (nk0 >= a.K) { nk0 = 0; ++nq; }
     }
-    T nxt[4][V];
+    T nxt[NB][V];
     if (nq < q1) {
       load_batch(nxt, nq, nk0, nkk0);
     } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < NB; ++i)
 #pragma unroll
         for (int v = 0; v < V; ++v) nxt[i][v] = T(0);
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < NB; ++i) {
       const int kk = kk0 + i * L.KS + L.ks;
       T tj[JB];
       psw_read_row<T, JB>(tj, t + (kk < TKc ? kk : TKc - 1) * a.JP + j0);
@@ -192,7 +192,7 @@ __device__ __forceinline__ void psw_fwd_block(const PswDev<T>& a, const PswLayou
       for (int j = 0; j < JB; ++j) fmav<T, V>(acc[j], tj[j], cur[i]);
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < NB; ++i)
 #pragma unroll
       for (int v = 0; v < V; ++v) cur[i][v] = nxt[i][v];
     q = nq; k0 = nk0; kk0 = nkk0;
@@ -226,7 +226,7 @@ __device__ __forceinline__ void psw_stage(const PswDev<T>& a, const PswLayout& l
   for (int i = L.li; i < ny; i += L.LS) lds[lay.ys + i] = a.y == nullptr ? T(1) : (sample_ok ? a.y[n * ny + i] : T(0));
 }
 
-template <typename T, int V, bool BIG>
+template <typename T, int V, bool BIG, int NB>
 __global__ void __launch_bounds__(kWave) psw_fwd_kernel(const PswDev<T> a) {
   extern __shared__ __align__(16) unsigned char psw_lds_raw[];
   const PswLane L(a.s_log2, a.lps_log2);
@@ -240,11 +240,11 @@ __global__ void __launch_bounds__(kWave) psw_fwd_kernel(const PswDev<T> a) {
     const int m0 = blocks[4 * b], rows_all = blocks[4 * b + 1], q0 = blocks[4 * b + 2], q1 = blocks[4 * b + 3];
     for (int j0 = 0; j0 < rows_all;) {
       const int rows = rows_all - j0;
-      if (rows <= 1) { psw_fwd_block<T, V, 1>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 1; }
-      else if (rows <= 3) { psw_fwd_block<T, V, 3>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 3; }
-      else if (rows <= 5) { psw_fwd_block<T, V, 5>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 5; }
-      else if (!BIG || rows <= 8) { psw_fwd_block<T, V, 8>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 8; }
-      else if constexpr (BIG) { psw_fwd_block<T, V, 16>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 16; }
+      if (rows <= 1) { psw_fwd_block<T, V, 1, NB>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 1; }
+      else if (rows <= 3) { psw_fwd_block<T, V, 3, NB>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 3; }
+      else if (rows <= 5) { psw_fwd_block<T, V, 5, NB>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 5; }
+      else if (!BIG || rows <= 8) { psw_fwd_block<T, V, 8, NB>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 8; }
+      else if constexpr (BIG) { psw_fwd_block<T, V, 16, NB>(a, lay, lds, L, n, sample_ok, m0, rows, j0, q0, q1); j0 += 16; }
     }
   }
 }
@@ -548,8 +548,12 @@ int psw_launch_t(const cgtp_psw_args* a, const cgtp_psw_table* tab, bool backwar
   const bool big = tab->max_rows > 8;
   const auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, block, plan.lds_bytes, stream, d); };
   if (!backward) {
-    if (plan.V == 1) big ? go(psw_fwd_kernel<T, 1, true>) : go(psw_fwd_kernel<T, 1, false>);
-    else big ? go(psw_fwd_kernel<T, VEC, true>) : go(psw_fwd_kernel<T, VEC, false>);
+    // rows of W a lane has in flight per batch: eight when a weight matrix has that many rows per row slice (142
+    // registers, three wavefronts per SIMD, 24 rows in flight per SIMD: 0.158 -> 0.137 ms at lmax = 3, 64 -> 64
+    // channels), four otherwise (a batch of eight would be half idle) and in the kernels with the 16-row pass
+    const bool deep = !big && d.K >= 8 * (kWave >> (plan.s_log2 + plan.lps_log2));
+    if (plan.V == 1) big ? go(psw_fwd_kernel<T, 1, true, 4>) : deep ? go(psw_fwd_kernel<T, 1, false, 8>) : go(psw_fwd_kernel<T, 1, false, 4>);
+    else big ? go(psw_fwd_kernel<T, VEC, true, 4>) : deep ? go(psw_fwd_kernel<T, VEC, false, 8>) : go(psw_fwd_kernel<T, VEC, false, 4>);
   } else {
     // rows of W a lane has in flight per batch: four when the weights come from HBM (bytes in flight are what the
     // rate follows: 0.50 -> 0.42 ms at 738 MB), two when they fit the 256 MB last-level cache (loads return sooner
