@@ -355,3 +355,32 @@ def test_no_samples_and_operands_the_kernels_do_not_take(device, monkeypatch):
     out = F.tensor_product_u1v(x.to(device), y.to(device), w_wide.to(device), *infos)
     assert "per-sample weight streaming" not in seen[-1], seen
     assert_close(out, ref_ops.dense_u1v(T, x, y, w_wide), 1e-5, "u1v per-sample, 260 output channels", norm="max")
+
+
+def test_weights_beyond_the_last_level_cache(device, monkeypatch, no_library_gemm):
+    """1.08 GB of per-sample weights (N = 24 000, 32 -> 32 channels): the launcher then keeps four rows of W per lane
+    in flight in the backward.  Samples are independent, so a strided subset of them is compared with the dense
+    oracle evaluated on exactly those samples (output, and every gradient including the subset's rows of grad_W)."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    irr, n, ch = _sh(2), 24000, 32
+    infos = [t.to(device) for t in tp_infos(Irreps(irr), Irreps(irr), Irreps(irr))[:3]]
+    T = ref_ops.dense_coupling(irr, irr, irr).float().double()
+    g = torch.Generator(device=device).manual_seed(1)
+    x = torch.randn(n, 9, ch, device=device, generator=g).requires_grad_(True)
+    y = torch.randn(n, 9, device=device, generator=g).requires_grad_(True)
+    w = (torch.randn(n, T.shape[0], ch, ch, device=device, generator=g) / ch ** 0.5).requires_grad_(True)
+    ct = torch.randn(n, 9, ch, device=device, generator=g)
+    assert w.numel() * 4 > 256 << 20
+    seen = _tiers(monkeypatch)
+    with no_library_gemm():
+        out = F.tensor_product_u1v(x, y, w, *infos)
+        grads = torch.autograd.grad(out, (x, y, w), ct)
+    assert "per-sample weight streaming" in seen[-1], seen
+    rows = torch.arange(5, n, 371, device=device)
+    sub = lambda t: t.detach()[rows].cpu()
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1v, T, (sub(x), sub(y), sub(w)), sub(ct))
+    o32, g32 = ref_ops.dense_grads(ref_ops.dense_u1v, T, (sub(x), sub(y), sub(w)), sub(ct), dtype=torch.float32)
+    for name, a, b, b32 in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads), (o32, *g32)):
+        assert_close(sub(a), b, 1e-5, f"u1v per-sample, 1.08 GB of weights, {name}", norm="max", fp32_ref=b32)
