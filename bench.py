@@ -1017,6 +1017,23 @@ def other_configs(args, headline):
         "bwd_fp32_frac_of_unpacked": r["roofline"]["fp32_vector"]["frac_of_unpacked"],
         "fwd_TFLOPs": r["kernels"]["fwd_TFLOPs"],
         "fwd_fp32_frac_of_unpacked": r["kernels"]["fwd_fp32_frac_of_unpacked"]}
+    torch.cuda.empty_cache()
+    # beside the BASELINE configurations: a weight per sample on the streaming kernels, and an edge step for irreps
+    # without a compiled table on the fused table-driven kernels
+    sub.workload, sub.steps, sub.warmup, sub.kernel_reps = "u1v_per_sample_fwd_bwd", 20, 3, 20
+    r = per_sample_bench(sub)
+    out["u1v_per_sample_weight_N65536_C16"] = {
+        "step_ms": r["ms_per_step"], "Msamples_s": r["value"], "fwd_ms": r["kernels"]["fwd_ms"],
+        "fwd_hbm_frac": r["kernels"]["fwd_frac_of_peak"], "fwd_frac_of_read_rate": r["kernels"]["fwd_frac_of_read"],
+        "bwd_ms": r["kernels"]["bwd_ms"], "bwd_hbm_frac": r["roofline"]["frac"],
+        "bwd_frac_of_copy_rate": r["roofline"]["achievable"]["frac_of_copy"]}
+    torch.cuda.empty_cache()
+    sub.workload, sub.kernel_reps = "edge_table_fwd_bwd", 10
+    r = edge_table_bench(sub)
+    out["edge_fwd_bwd_irreps_without_compiled_table"] = {
+        "Medges_s": r["value"], "step_ms": r["ms_per_step"], "separate_launches_step_ms": r["kernels"]["separate"]["step_ms"],
+        "per_coefficient_vs_compiled": r["kernels"]["per_coefficient_vs_compiled"]}
+    torch.cuda.empty_cache()
     return out
 
 
