@@ -554,9 +554,24 @@ __global__ void uvt_gw_reduce_kernel(const real* __restrict__ part, real* __rest
   gw[i] = s;
 }
 
-static int64_t uvt_gw_chunk(int64_t n_rows) {
-  // samples per workgroup: enough workgroups to fill the chip at small batches, at most 128 partial results
+// few output channels and a long contracted axis: 256 x 64 blocks (single precision; in double precision the second
+// set of operands in flight does not fit the registers)
+static bool uvt_gw_narrow(int64_t K, int32_t cout) { return sizeof(real) == 4 && cout <= 64 && K >= 256; }
+
+static int64_t uvt_gw_blocks(int64_t K, int32_t cout) {
+  const bool narrow = uvt_gw_narrow(K, cout);
+  const int64_t kt = narrow ? 256 : 128, wt = narrow ? 64 : 128;
+  return ((K + kt - 1) / kt) * ((cout + wt - 1) / wt);
+}
+
+static int64_t uvt_gw_chunk(int64_t n_rows, int32_t n_paths, int64_t K, int32_t cout) {
+  // samples per workgroup: at most 128 partial results; 256 samples, fewer (down to 32: four steps) while the launch
+  // would have less than three workgroups per compute unit — a node-level layer has a few thousand samples and a
+  // handful of paths, and with 256 samples per workgroup its 48 workgroups took 100 us for 0.3 GFLOP
+  const int64_t per_chunk = n_paths * uvt_gw_blocks(K, cout);
   int64_t chunk = 256;
+  while (chunk > 32 && ((n_rows + chunk - 1) / chunk) * per_chunk < 768 && (n_rows + chunk / 2 - 1) / (chunk / 2) <= 128)
+    chunk /= 2;
   while ((n_rows + chunk - 1) / chunk > 128) chunk *= 2;
   return chunk;
 }
@@ -882,7 +897,7 @@ int apply(const cgtp_uvt_args* a, void* stream) {
 
 int64_t grad_w_workspace_bytes(int64_t n_rows, int32_t n_paths, int64_t K, int32_t cout) {
   if (n_rows <= 0 || n_paths <= 0 || K <= 0 || cout <= 0) return 0;
-  const int64_t chunk = uvt_gw_chunk(n_rows);
+  const int64_t chunk = uvt_gw_chunk(n_rows, n_paths, K, cout);
   return ((n_rows + chunk - 1) / chunk) * n_paths * K * cout * (int64_t)sizeof(real);
 }
 
@@ -913,13 +928,10 @@ int grad_w(const cgtp_uvt_gw_args* a, void* stream) {
   d.items = a->items; d.path_ptr = a->path_ptr; d.ta = a->term_a; d.tb = a->term_b; d.tc = (const real*)a->term_c;
   d.n_rows = a->n_rows; d.n_paths = a->n_paths; d.dx = a->dx; d.dy = a->dy; d.dg = a->dg; d.cx = a->cx; d.cy = a->cy;
   d.cout = a->cout; d.K = (int)K;
-  d.chunk = (int)uvt_gw_chunk(a->n_rows);
+  d.chunk = (int)uvt_gw_chunk(a->n_rows, a->n_paths, K, a->cout);
   const int64_t n_chunks = (a->n_rows + d.chunk - 1) / d.chunk;
-  // few output channels and a long contracted axis: 256 x 64 blocks (single precision; in double precision the
-  // second set of operands in flight does not fit the registers)
-  const bool narrow = sizeof(real) == 4 && a->cout <= 64 && K >= 256;
-  const int64_t kt = narrow ? 256 : 128, wt = narrow ? 64 : 128;
-  const int64_t zblocks = ((K + kt - 1) / kt) * ((a->cout + wt - 1) / wt);
+  const bool narrow = uvt_gw_narrow(K, a->cout);
+  const int64_t zblocks = uvt_gw_blocks(K, a->cout);
   if (zblocks > 65535 || a->n_paths > 65535) return CGTP_ERR_SHAPE;
   dim3 grid((unsigned)n_chunks, (unsigned)a->n_paths, (unsigned)zblocks);
   void (*fn)(const UvtGwDev) = a->cy > 0 ? uvt_grad_w_kernel<true, false> : uvt_grad_w_kernel<false, false>;
