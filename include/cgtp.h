@@ -438,8 +438,8 @@ int cgtp_uvt_apply(const cgtp_uvt_args* args, void* stream);
  * path_ptr[n_paths + 1] their ranges per path; x (n_rows, dx, cx), y (n_rows, dy) or
  * (n_rows, dy, cy), g = grad_out (n_rows, dg, cout), gw (n_paths, K, cout) contiguous as the module stores the
  * weight.  The samples are contracted on the matrix cores in chunks; the chunks' partial results live in `workspace`
- * (cgtp_uvt_grad_w_workspace_bytes) and are added in chunk order.  Channel counts multiples of 4, 16-byte aligned
- * pointers. */
+ * (cgtp_uvt_grad_w_workspace_bytes) and are added in a fixed order.  Channel counts multiples of 4, 16-byte aligned
+ * pointers; gw and workspace aligned to four elements (16 bytes fp32, 32 bytes fp64). */
 typedef struct cgtp_uvt_gw_args {
   const void* x;
   const void* y;
