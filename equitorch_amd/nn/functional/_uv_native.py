@@ -300,8 +300,17 @@ def u1v_supported(x: Tensor, y: Tensor, w: Tensor, tp_info) -> bool:
     if tuple(x.shape) != (n, c.D1, u) or tuple(y.shape) != (n, c.D2) or w.shape[0] != c.P:
         raise _lib.CgtpError(f"operands {tuple(x.shape)}, {tuple(y.shape)}, {tuple(w.shape)} do not fit the table: "
                              f"expected (N, {c.D1}, U), (N, {c.D2}), ({c.P}, U, W)")
-    return (chunk_of(n, c.D1, c.D2, c.DO, u, 0, wc, dt) > 0 and chunk_of(n, c.DO, c.D2, c.D1, wc, 0, u, dt) > 0
-            and grad_y_supported(n, c.D1, c.D2, u, wc, tp_info, x.element_size()) and x.data_ptr() % 16 == 0)
+    return u1v_fits(n, u, wc, tp_info, dt) and x.data_ptr() % 16 == 0
+
+
+def u1v_fits(n: int, u: int, wc: int, tp_info, dtype: torch.dtype) -> bool:
+    """Whether the forward, the gradient of the channelled operand and the gradient of the second operand have a launch
+    shape for ``n`` samples, ``u -> wc`` channels in ``dtype`` (float32 | float64): extents only, no tensors."""
+    c = _coo(tp_info)
+    size = torch.empty(0, dtype=dtype).element_size()
+    return (n > 0 and chunk_of(n, c.D1, c.D2, c.DO, u, 0, wc, dtype) > 0
+            and chunk_of(n, c.DO, c.D2, c.D1, wc, 0, u, dtype) > 0
+            and grad_y_supported(n, c.D1, c.D2, u, wc, tp_info, size))
 
 
 def u1v(x: Tensor, y: Tensor, w: Tensor, tp_info) -> Tensor:
@@ -362,8 +371,14 @@ def uvw_supported(x: Tensor, y: Tensor, w: Tensor, tp_info) -> bool:
     if tuple(x.shape) != (n, c.D1, u) or tuple(y.shape) != (n, c.D2, v) or w.shape[0] != c.P:
         raise _lib.CgtpError(f"operands {tuple(x.shape)}, {tuple(y.shape)}, {tuple(w.shape)} do not fit the table: "
                              f"expected (N, {c.D1}, U), (N, {c.D2}, V), ({c.P}, U, V, W)")
-    return (chunk_of(n, c.D1, c.D2, c.DO, u, v, wc, dt) > 0 and chunk_of(n, c.D2, c.DO, c.D1, v, wc, u, dt) > 0
-            and chunk_of(n, c.DO, c.D1, c.D2, wc, u, v, dt) > 0 and x.data_ptr() % 16 == 0 and y.data_ptr() % 16 == 0)
+    return uvw_fits(n, u, v, wc, tp_info, dt) and x.data_ptr() % 16 == 0 and y.data_ptr() % 16 == 0
+
+
+def uvw_fits(n: int, u: int, v: int, wc: int, tp_info, dtype: torch.dtype) -> bool:
+    """The same for the product with channels on both operands."""
+    c = _coo(tp_info)
+    return (n > 0 and chunk_of(n, c.D1, c.D2, c.DO, u, v, wc, dtype) > 0
+            and chunk_of(n, c.D2, c.DO, c.D1, v, wc, u, dtype) > 0 and chunk_of(n, c.DO, c.D1, c.D2, wc, u, v, dtype) > 0)
 
 
 def uvw(x: Tensor, y: Tensor, w: Tensor, tp_info) -> Tensor:

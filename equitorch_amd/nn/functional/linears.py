@@ -57,6 +57,11 @@ def _check_batch(input1, input2, weight):
     _lib.require_gpu(input1, input2, weight)
 
 
+def _widen(*tensors: Tensor) -> bool:
+    """All operands in one 16-bit floating type."""
+    return tensors[0].dtype in (torch.bfloat16, torch.float16) and all(t.dtype == tensors[0].dtype for t in tensors)
+
+
 def tensor_product_u1u(input1: Tensor, input2: Tensor, weight: Tensor,
                        tp_info_forward: TensorProductInfo,
                        tp_info_backward1: Optional[TensorProductInfo] = None,
@@ -112,6 +117,14 @@ def tensor_product_u1v(input1: Tensor, input2: Tensor, weight: Tensor,
     if _uv_native.u1v_supported(input1, input2, weight, tp_info_forward):
         kernels.log_tier("tensor_product_u1v", "fp32 matrix-core kernel (table-driven)")
         return _uv_native.u1v(input1, input2, weight, tp_info_forward)
+    if _widen(input1, input2, weight) and input1.ndim == 3 and input2.ndim == 2 and (
+            weight.ndim == 4 or (weight.ndim == 3 and _uv_native.u1v_fits(
+                input1.shape[0], weight.shape[1], weight.shape[2], tp_info_forward, torch.float32))):
+        # 16-bit operands on a table without compiled matrix-core kernels: the table-driven kernels in fp32
+        # arithmetic on widened copies (at 4096 samples, 64 channels, 0e+1e+2e+3e: 0.10 against 0.78 ms for the
+        # library route in bf16), the result rounded once
+        kernels.log_tier("tensor_product_u1v", "operands widened to fp32", str(input1.dtype))
+        return tensor_product_u1v(input1.float(), input2.float(), weight.float(), tp_info_forward).to(input1.dtype)
     if weight.ndim == 4:
         from . import _psw
         table = _psw.table_of_coo(kernels.coo_of(tp_info_forward), tp_info_forward.info_Mij_fwd.scale, 1, input1.device)

@@ -76,6 +76,12 @@ def tensor_product_uvw(input1: Tensor, input2: Tensor, weight: Tensor,
     if _uv_native.uvw_supported(input1, input2, weight, tp_info_forward):
         kernels.log_tier("tensor_product_uvw", "fp32 matrix-core kernel (table-driven)")
         return _uv_native.uvw(input1, input2, weight, tp_info_forward)
+    if (input1.dtype in (torch.bfloat16, torch.float16) and input1.ndim == 3 and input2.ndim == 3 and (
+            weight.ndim == 5 or _uv_native.uvw_fits(input1.shape[0], weight.shape[1], weight.shape[2], weight.shape[3],
+                                                    tp_info_forward, torch.float32))):
+        # 16-bit operands: the table-driven kernels in fp32 arithmetic on widened copies, the result rounded once
+        kernels.log_tier("tensor_product_uvw", "operands widened to fp32", str(input1.dtype))
+        return tensor_product_uvw(input1.float(), input2.float(), weight.float(), tp_info_forward).to(input1.dtype)
     if weight.ndim == 5 and input1.ndim == 3 and input2.ndim == 3:
         from . import _psw
         table = _psw.table_of_coo(kernels.coo_of(tp_info_forward), tp_info_forward.info_Mij_fwd.scale, 1, input1.device)

@@ -235,3 +235,34 @@ def test_fp32_fully_connected_past_two_to_the_31_elements(device):
     assert (gw - ref).abs().max().item() <= 1e-4 * ref.abs().max().item(), "grad_w"
     del x, y, ct
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("per_sample", [False, True])
+def test_16_bit_operands_without_a_compiled_table(device, monkeypatch, dtype, per_sample):
+    """bf16 / fp16 operands on irreps whose table has no compiled matrix-core kernels (the reference's own comparison
+    irreps ``0e+1e+2e+3e``): the table-driven kernels in fp32 arithmetic on widened copies, the result rounded once —
+    no ``(N, segments, C)`` intermediate and no library GEMM.  Against the float64 oracle on the rounded inputs."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.ops import kernels
+    from equitorch_amd.utils import tp_infos
+    irr, n, cin, cout = "0e+1e+2e+3e", 300, 32, 48
+    infos = [t.to(device) for t in tp_infos(Irreps(irr), Irreps(irr), Irreps(irr))[:3]]
+    T = ref_ops.dense_coupling(irr, irr, irr).float().double()
+    g = torch.Generator().manual_seed(3)
+    rd = lambda *s: torch.randn(*s, generator=g).to(dtype)
+    x, y = rd(n, 16, cin), rd(n, 16)
+    w = (torch.randn(*((n,) if per_sample else ()), T.shape[0], cin, cout, generator=g) / (cin * T.shape[0]) ** 0.5).to(dtype)
+    ct = rd(n, 16, cout)
+    seen = []
+    monkeypatch.setattr(kernels, "log_tier", lambda op, tier, detail="": seen.append(tier))
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    out = F.tensor_product_u1v(xd, yd, wd, *infos)
+    assert out.dtype == dtype
+    assert "widened" in seen[0] and ("streaming" in seen[-1] if per_sample else "matrix-core" in seen[-1]), seen
+    grads = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x.double(), y.double(), w.double()), ct.double())
+    for name, a, b in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads)):
+        assert a.dtype == dtype
+        assert_close(a.float(), b, 1e-2, f"u1v {dtype} widened per_sample={per_sample} {name}", norm="max")
