@@ -180,7 +180,10 @@ def grad_y_supported(n: int, dx: int, dy: int, cx: int, cout: int, tp_info, item
     """Whether the 16 staged samples of a ``cgtp_uvt_grad_y`` workgroup and its tables fit the LDS."""
     c = _coo(tp_info)
     kx = ((cx + 15) // 16 + 3) // 4 * 4 * 16
-    lds = (16 * (dx * kx + 4) + 8 * 16 * dy) * itemsize + len(c.coef) * (32 + 8 + itemsize) + 16
+    # one 32-byte item per (weight path, row of the first operand) segment, 8 bytes + a coefficient per term
+    n_items = kernels.cached(_anchor(tp_info), "uvt_seg_count",
+                             lambda: len(set(zip(np.asarray(c.p).tolist(), np.asarray(c.M1).tolist()))))
+    lds = (16 * (dx * kx + 4) + 8 * 16 * dy) * itemsize + n_items * 32 + len(c.coef) * (8 + itemsize) + 16
     return cx % 4 == 0 and cout % 4 == 0 and lds <= 160 * 1024
 
 

@@ -266,3 +266,32 @@ def test_16_bit_operands_without_a_compiled_table(device, monkeypatch, dtype, pe
     for name, a, b in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads)):
         assert a.dtype == dtype
         assert_close(a.float(), b, 1e-2, f"u1v {dtype} widened per_sample={per_sample} {name}", norm="max")
+
+
+def test_all_even_table_at_128_channels(device, monkeypatch):
+    """``0e+1e+2e+3e`` (34 paths, 611 coefficients) at 128 -> 128 channels, fp32 and bf16: the 16 staged samples and the
+    walk tables of every kernel of the step fit the LDS (the host's estimate for the gradient of the second operand
+    used to count an item per coefficient and sent this shape to the library route)."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.ops import kernels
+    from equitorch_amd.utils import tp_infos
+    irr, n, ch = "0e+1e+2e+3e", 1000, 128
+    infos = [t.to(device) for t in tp_infos(Irreps(irr), Irreps(irr), Irreps(irr))[:3]]
+    T = ref_ops.dense_coupling(irr, irr, irr).float().double()
+    g = torch.Generator().manual_seed(9)
+    x, y, ct = (torch.randn(*s, generator=g) for s in ((n, 16, ch), (n, 16), (n, 16, ch)))
+    w = torch.randn(T.shape[0], ch, ch, generator=g) / (ch * T.shape[0]) ** 0.5
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x, y, w), ct)
+    for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 1e-2)):
+        seen = []
+        monkeypatch.setattr(kernels, "log_tier", lambda op, tier, detail="": seen.append(tier))
+        xd, yd, wd = (t.to(device, dtype).requires_grad_(True) for t in (x, y, w))
+        out = F.tensor_product_u1v(xd, yd, wd, *infos)
+        assert "fp32 matrix-core kernel (table-driven)" in seen[-1], seen
+        grads = torch.autograd.grad(out, (xd, yd, wd), ct.to(device, dtype))
+        if dtype == torch.bfloat16:      # the oracle on the rounded inputs
+            r = lambda t: t.to(dtype).double()
+            ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1v, T, (r(x), r(y), r(w)), r(ct))
+        for name, a, b in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads)):
+            assert_close(a.float(), b, tol, f"u1v {irr} 128 -> 128 {dtype} {name}", norm="max")
