@@ -117,6 +117,18 @@ def tensor_product_u1v(input1: Tensor, input2: Tensor, weight: Tensor,
     if _uv_native.u1v_supported(input1, input2, weight, tp_info_forward):
         kernels.log_tier("tensor_product_u1v", "fp32 matrix-core kernel (table-driven)")
         return _uv_native.u1v(input1, input2, weight, tp_info_forward)
+    if (weight.ndim == 3 and input1.ndim == 3 and input2.ndim == 2 and input1.dtype == input2.dtype == weight.dtype
+            and input1.dtype in (torch.float32, torch.float64) and (weight.shape[1] % 4 or weight.shape[2] % 4)):
+        # channel counts that are not multiples of 4 (the kernels move 16 bytes per lane): zero channels appended to
+        # the operand and the weight, the result cut back
+        u, wc = weight.shape[1:]
+        u4, w4 = -(-u // 4) * 4, -(-wc // 4) * 4
+        if _uv_native.u1v_fits(input1.shape[0], u4, w4, tp_info_forward, input1.dtype):
+            kernels.log_tier("tensor_product_u1v", "channel counts padded to multiples of 4", f"{u} -> {wc}")
+            pad = torch.nn.functional.pad
+            out = tensor_product_u1v(pad(input1, (0, u4 - u)), input2, pad(weight, (0, w4 - wc, 0, u4 - u)),
+                                     tp_info_forward)
+            return out[..., :wc].contiguous()
     if _widen(input1, input2, weight) and input1.ndim == 3 and input2.ndim == 2 and (
             weight.ndim == 4 or (weight.ndim == 3 and _uv_native.u1v_fits(
                 input1.shape[0], weight.shape[1], weight.shape[2], tp_info_forward, torch.float32))):

@@ -76,6 +76,18 @@ def tensor_product_uvw(input1: Tensor, input2: Tensor, weight: Tensor,
     if _uv_native.uvw_supported(input1, input2, weight, tp_info_forward):
         kernels.log_tier("tensor_product_uvw", "fp32 matrix-core kernel (table-driven)")
         return _uv_native.uvw(input1, input2, weight, tp_info_forward)
+    if (weight.ndim == 4 and input1.ndim == 3 and input2.ndim == 3 and input1.dtype in (torch.float32, torch.float64)
+            and any(c % 4 for c in weight.shape[1:])):
+        # channel counts that are not multiples of 4: zero channels appended to the operands and the weight, the result
+        # cut back
+        u, v, wc = weight.shape[1:]
+        u4, v4, w4 = (-(-c // 4) * 4 for c in (u, v, wc))
+        if _uv_native.uvw_fits(input1.shape[0], u4, v4, w4, tp_info_forward, input1.dtype):
+            kernels.log_tier("tensor_product_uvw", "channel counts padded to multiples of 4", f"{u} x {v} -> {wc}")
+            pad = torch.nn.functional.pad
+            out = tensor_product_uvw(pad(input1, (0, u4 - u)), pad(input2, (0, v4 - v)),
+                                     pad(weight, (0, w4 - wc, 0, v4 - v, 0, u4 - u)), tp_info_forward)
+            return out[..., :wc].contiguous()
     if (input1.dtype in (torch.bfloat16, torch.float16) and input1.ndim == 3 and input2.ndim == 3 and (
             weight.ndim == 5 or _uv_native.uvw_fits(input1.shape[0], weight.shape[1], weight.shape[2], weight.shape[3],
                                                     tp_info_forward, torch.float32))):

@@ -295,3 +295,33 @@ def test_all_even_table_at_128_channels(device, monkeypatch):
             ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1v, T, (r(x), r(y), r(w)), r(ct))
         for name, a, b in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads)):
             assert_close(a.float(), b, tol, f"u1v {irr} 128 -> 128 {dtype} {name}", norm="max")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_channel_counts_that_are_not_multiples_of_four(device, monkeypatch, dtype):
+    """10 -> 7 channels (u1v) and 5 x 6 -> 9 (uvw) with a shared weight: zero channels are appended up to multiples of
+    4 and the same kernels run; forward and all gradients against the dense oracle."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.ops import kernels
+    from equitorch_amd.utils import tp_infos
+    irr, n = _sh(2), 211
+    infos = [t.to(device) for t in tp_infos(Irreps(irr), Irreps(irr), Irreps(irr))[:3]]
+    T = ref_ops.dense_coupling(irr, irr, irr).float().double()
+    g = torch.Generator().manual_seed(10)
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).to(dtype)
+    tol = 1e-5 if dtype == torch.float32 else 1e-11
+    cases = (("u1v", F.tensor_product_u1v, ref_ops.dense_u1v, (rd(n, 9, 10), rd(n, 9), rd(T.shape[0], 10, 7) / 3), rd(n, 9, 7)),
+             ("uvw", F.tensor_product_uvw, ref_ops.dense_uvw, (rd(n, 9, 5), rd(n, 9, 6), rd(T.shape[0], 5, 6, 9) / 5), rd(n, 9, 9)))
+    for name, fn, ref_fn, ops, ct in cases:
+        seen = []
+        monkeypatch.setattr(kernels, "log_tier", lambda op, tier, detail="": seen.append(tier))
+        leaves = [t.to(device).requires_grad_(True) for t in ops]
+        out = fn(*leaves, *infos)
+        assert "padded" in seen[0] and "matrix-core" in seen[-1], seen
+        assert out.shape == ct.shape and out.is_contiguous()
+        grads = torch.autograd.grad(out, leaves, ct.to(device))
+        ref_out, ref_grads = ref_ops.dense_grads(ref_fn, T, ops, ct)
+        for what, a, b in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads)):
+            assert a.shape == b.shape
+            assert_close(a, b, tol, f"{name} {dtype} odd channel counts {what}", norm="max")
