@@ -445,6 +445,29 @@ def _streaming_path(x: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, a
     return _psw.product(table, x, None, weight, lambda xx, _y, ww: _Mix.apply(xx, ww, plan, False, in_size))
 
 
+def _adapted_path(x: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anchor: Tensor):
+    """Operands the native kernels do not take as they are, adapted to them: bf16 / fp16 widened to fp32 (the result
+    rounded once), channel counts of a shared weight that are not multiples of 4 filled up with zero channels (the
+    result cut back).  None when the kernels still have no launch shape for the adapted operands."""
+    dtype, cin, cout = x.dtype, weight.shape[-2], weight.shape[-1]
+    xa, wa = x, weight
+    if dtype in (torch.bfloat16, torch.float16):
+        xa, wa = xa.float(), wa.float()
+    elif dtype not in (torch.float32, torch.float64):
+        return None
+    if wa.ndim == 3 and (cin % 4 or cout % 4):
+        pad = torch.nn.functional.pad
+        xa, wa = pad(xa, (0, -cin % 4)), pad(wa, (0, -cout % 4, 0, -cin % 4))
+    if xa is x:
+        return None
+    out = _table_driven_path(xa, wa, plan, in_size, anchor) if wa.ndim == 3 else _streaming_path(xa, wa, plan, in_size, anchor)
+    if out is None:
+        return None
+    if out.shape[-1] != cout:
+        out = out[..., :cout]
+    return out.to(dtype).contiguous()
+
+
 def mix(input: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anchor: Tensor = None) -> Tensor:
     """``(..., D_in, C_in) x (P, C_in, C_out) | (N, P, C_in, C_out) -> (..., D_out, C_out)``."""
     _lib.require_gpu(input, weight)
@@ -464,6 +487,8 @@ def mix(input: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anchor: T
         out = _table_driven_path(x, weight, plan, in_size, anchor)
     if out is None and weight.ndim == 4 and anchor is not None:
         out = _streaming_path(x, weight, plan, in_size, anchor)
+    if out is None and anchor is not None and x.shape[0] > 0:
+        out = _adapted_path(x, weight, plan, in_size, anchor)
     if out is None:
         out = _Mix.apply(x, weight, plan, False, in_size)
     return out.reshape(*lead, plan.out_size, out.shape[-1])

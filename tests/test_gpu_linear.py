@@ -123,3 +123,38 @@ def test_bf16_shared_weight_runs_on_the_matrix_core_kernels(device, irr, cin, co
     for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
         assert a.dtype == torch.bfloat16
         assert_close(a.float(), b, tol=1e-2, what=f"bf16 {irr} {name}")
+
+
+@pytest.mark.parametrize("dtype,cin,cout,shared", [(torch.float32, 10, 7, True), (torch.float64, 6, 9, True),
+                                                    (torch.bfloat16, 24, 40, True), (torch.bfloat16, 10, 7, True),
+                                                    (torch.float16, 16, 8, False)])
+def test_operands_adapted_to_the_native_kernels(device, monkeypatch, dtype, cin, cout, shared):
+    """Channel counts that are not multiples of 4 (zero channels appended) and 16-bit operands without a compiled
+    matrix-core table (widened to fp32, the result rounded once) run on the table-driven / streaming kernels instead of
+    the library GEMMs; against the oracle on the rounded inputs."""
+    from equitorch_amd.nn import IrrepsLinear
+    from equitorch_amd.ops import kernels
+    io, ii, n = "0e+1o+2e", "0e+1o+1o+2e+0e", 130
+    mod = IrrepsLinear(ii, io, cin, cout, internal_weights=False).to(device)
+    info = ref_tables.irreps_linear_infos(io, ii)[0]
+    info["scale_MM0"] = torch.tensor(info["scale_MM0"]).double().tolist()
+    g = torch.Generator().manual_seed(4)
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).to(dtype).double()
+    x, ct = rd(n, mod.irreps_in_dim, cin), rd(n, mod.irreps_out_dim, cout)
+    w = rd(*(() if shared else (n,)), mod.num_paths, cin, cout) / cin ** 0.5
+    w = w.to(dtype).double()
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    ref = ref_ops.cpu_irreps_linear(xr, wr, info)
+    rgx, rgw = _grads(ref, (xr, wr), ct)
+    seen = []
+    monkeypatch.setattr(kernels, "log_tier", lambda op, tier, detail="": seen.append(tier))
+    xd, wd = (t.to(device, dtype).requires_grad_(True) for t in (x, w))
+    out = mod(xd, wd)
+    assert seen and ("table-driven matrix-core" in seen[-1] or "streaming" in seen[-1]), seen
+    assert out.dtype == dtype and out.shape == ref.shape and out.is_contiguous()
+    gx, gw = _grads(out, (xd, wd), ct.to(device, dtype))
+    tol = {torch.float32: 1e-5, torch.float64: 1e-12}.get(dtype, 1e-2)
+    for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
+        assert a.dtype == dtype and a.shape == b.shape
+        assert_close(a.double(), b, tol, f"IrrepsLinear {dtype} {cin}->{cout} shared={shared} {name}",
+                     norm="element" if dtype in (torch.float32, torch.float64) else "max")
