@@ -300,9 +300,11 @@ def test_table_driven_matrix_core_entry_points_validate_on_the_host():
     assert L.cgtp_uvt_validate(C.byref(a)) == 3                             # alignment
     assert L.cgtp_uvt_pack_weights(p16, p16, 2, 0, 16, 1, 1, 1, _lib.F32, None) == 2
     assert L.cgtp_uvt_pack_weights(None, p16, 2, 16, 16, 1, 1, 1, _lib.F32, None) == 1
-    # weight gradient: chunks of at least 256 samples, at most 128 of them
+    # weight gradient: at most 128 chunks of samples; chunks of 256 samples, down to 32 while the launch would have
+    # fewer than three workgroups per compute unit
     assert L.cgtp_uvt_grad_w_workspace_bytes(32768, 23, 128, 128, _lib.F32) == 128 * 23 * 128 * 128 * 4
-    assert L.cgtp_uvt_grad_w_workspace_bytes(300, 4, 32, 16, _lib.F64) == 2 * 4 * 32 * 16 * 8
+    assert L.cgtp_uvt_grad_w_workspace_bytes(300, 4, 32, 16, _lib.F64) == 10 * 4 * 32 * 16 * 8
+    assert L.cgtp_uvt_grad_w_workspace_bytes(8192, 23, 128, 128, _lib.F32) == 64 * 23 * 128 * 128 * 4
     g = _lib.UvtGwArgs()
     g.dtype = _lib.F32
     g.n_rows, g.n_paths, g.dx, g.dy, g.dg, g.cx, g.cy, g.cout = 10, 4, 9, 9, 9, 32, 0, 30
