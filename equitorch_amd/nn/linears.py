@@ -276,17 +276,19 @@ class SO2Linear(nn.Module):
                 and weight.shape[-3] == self.num_weights and input.ndim >= 3):
             if weight.ndim == 3:
                 _lib_require(input, weight)
-                if input.dtype in (torch.float32, torch.float64):
-                    # every table entry is one (C_in, C_out) product on one component: the table-driven matrix-core
-                    # kernels of the fully connected product take the table as it is
-                    from .functional import _irreps_gemm as G
-                    plan = G.plan_of_product_info(self.info_forward, self.irreps_in.dim, self.num_weights)
-                    anchor = next(t for t in (self.info_forward.seg_out, self.info_forward.index1,
-                                              self.info_forward.index2, self.info_forward.scale) if t is not None)
-                    x3 = input.reshape(-1, *input.shape[-2:]).contiguous()
-                    out = G._table_driven_path(x3, weight.contiguous(), plan, self.irreps_in.dim, anchor)
-                    if out is not None:
-                        return out.reshape(*input.shape[:-2], plan.out_size, out.shape[-1])
+                # every table entry is one (C_in, C_out) product on one component: the table-driven matrix-core
+                # kernels of the fully connected product take the table as it is (16-bit operands widened, channel
+                # counts filled up to multiples of 4)
+                from .functional import _irreps_gemm as G
+                plan = G.plan_of_product_info(self.info_forward, self.irreps_in.dim, self.num_weights)
+                anchor = next(t for t in (self.info_forward.seg_out, self.info_forward.index1,
+                                          self.info_forward.index2, self.info_forward.scale) if t is not None)
+                x3 = input.reshape(-1, *input.shape[-2:]).contiguous()
+                out = G._table_driven_path(x3, weight.contiguous(), plan, self.irreps_in.dim, anchor)
+                if out is None and x3.shape[0] > 0:
+                    out = G._adapted_path(x3, weight.contiguous(), plan, self.irreps_in.dim, anchor)
+                if out is not None:
+                    return out.reshape(*input.shape[:-2], plan.out_size, out.shape[-1])
                 # one GEMM per order |m| over the components of that order side by side
                 from .functional._so2_gemm import so2_linear_uv_shared
                 return so2_linear_uv_shared(input, weight, self.info_forward, self.irreps_in.dim, self.num_weights)

@@ -227,3 +227,32 @@ def test_fused_rotation_gradients_of_the_sincos_tensors(device, dtype, irr, chan
     cr = [cs[0][:, :1 + 2 * max_l].clone().requires_grad_(True), cs[1][:, :1 + 2 * max_l]]
     (ra,) = torch.autograd.grad(ref_ops.cpu_wigner_rotation(x, cr[0], cr[1], None, z, j), cr[0], ct)
     assert_close(ga[:, :1 + 2 * max_l], ra, tol=tol * 10, what="grad of alpha alone")
+
+
+@pytest.mark.parametrize("dtype,cin,cout", [(torch.bfloat16, 16, 24), (torch.float32, 6, 5)])
+def test_so2_linear_uv_adapted_operands(device, monkeypatch, dtype, cin, cout):
+    """bf16 operands (widened to fp32) and channel counts that are not multiples of 4 (zero channels appended) on the
+    table-driven kernels; against the oracle on the rounded inputs."""
+    from equitorch_amd.nn import SO2Linear
+    from equitorch_amd.ops import kernels
+    irr_in, irr_out, n = "0e+1o+2e+3o", "0e+1o+2e", 77
+    info = _f32(ref_tables.so2_linear_infos(irr_out, irr_in)[0])
+    mod = SO2Linear(irr_in, irr_out, cin, cout, internal_weights=False, feature_mode="uv").to(device)
+    g = torch.Generator().manual_seed(6)
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).to(dtype).double()
+    x, w, ct = rd(n, 16, cin), rd(mod.num_weights, cin, cout) / cin ** 0.5, rd(n, 9, cout)
+    w = w.to(dtype).double()
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    ref = ref_ops.cpu_so2_linear(xr, wr, info)
+    rgx, rgw = torch.autograd.grad(ref, (xr, wr), ct)
+    seen = []
+    monkeypatch.setattr(kernels, "log_tier", lambda op, tier, detail="": seen.append(tier))
+    xd, wd = (t.to(device, dtype).requires_grad_(True) for t in (x, w))
+    out = mod(xd, wd)
+    assert seen and "table-driven matrix-core" in seen[-1], seen
+    gx, gw = torch.autograd.grad(out, (xd, wd), ct.to(device, dtype))
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
+        assert a.dtype == dtype and a.shape == b.shape
+        assert_close(a.double(), b, tol, f"SO2Linear uv {dtype} {cin}->{cout} {name}",
+                     norm="element" if dtype == torch.float32 else "max")
