@@ -154,6 +154,94 @@ at::Tensor edge_uvu(const at::Tensor& x, const at::Tensor& y, const at::Tensor& 
   return EdgeUvu::apply(x, y, w, &h);
 }
 
+// ---- row mode: the channel-wise product on a plain batch (SO3Linear('uu') on its compiled table) -----------------
+// Gradients of higher order are re-expressed in Python through the differentiable contraction family; the callables
+// that do it are registered once per table and looked up by number when a backward runs with gradient mode on.
+std::vector<py::object>& fallbacks() {
+  static std::vector<py::object>* v = new std::vector<py::object>();   // never destroyed: outlives the interpreter's teardown
+  return *v;
+}
+
+cgtp_uvu_args row_args(const at::Tensor& x, const at::Tensor& y, const at::Tensor& w, const at::Tensor& path_scale,
+                       int64_t cfg) {
+  TORCH_CHECK(x.is_cuda() && y.is_cuda() && w.is_cuda(), "cgtp: operands must live on the GPU");
+  TORCH_CHECK(x.is_contiguous() && y.is_contiguous() && w.is_contiguous(), "cgtp: operands must be contiguous");
+  TORCH_CHECK(x.scalar_type() == y.scalar_type() && x.scalar_type() == w.scalar_type() &&
+                  (x.scalar_type() == at::kFloat || x.scalar_type() == at::kDouble),
+              "cgtp: operands must share one dtype, float32 or float64");
+  TORCH_CHECK(x.dim() == 3 && y.dim() == 2 && x.size(0) == y.size(0) && (w.dim() == 2 || (w.dim() == 3 && w.size(0) == x.size(0))),
+              "cgtp: x (N, D1, C), y (N, D2), w (N, P, C) | (P, C)");
+  cgtp_uvu_args a{};
+  a.cfg = (int32_t)cfg;
+  a.dtype = x.scalar_type() == at::kFloat ? CGTP_F32 : CGTP_F64;
+  a.C = (int32_t)x.size(2);
+  a.w_shared = w.dim() == 2;
+  a.n_rows = y.size(0);
+  a.n_x_rows = x.size(0);
+  a.x = x.data_ptr();
+  a.y = y.data_ptr();
+  a.w = w.data_ptr();
+  a.path_scale = ptr_or_null(path_scale);
+  return a;
+}
+
+class RowUvu : public torch::autograd::Function<RowUvu> {
+ public:
+  // scale: handed over by address, not as an argument tensor (it is no input of the node, and may be undefined)
+  static at::Tensor forward(AutogradContext* ctx, const at::Tensor& x, const at::Tensor& y, const at::Tensor& w,
+                            const at::Tensor* scale, int64_t cfg, int64_t d_out, int64_t fallback) {
+    const at::Tensor& path_scale = *scale;
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+    cgtp_uvu_args a = row_args(x, y, w, path_scale, cfg);
+    at::Tensor out = at::empty({x.size(0), d_out, x.size(2)}, x.options());
+    a.out = out.data_ptr();
+    at::Tensor ws = workspace_for(a, 0, x);
+    check_status(cgtp_uvu_fwd(&a, current_stream(x)), "cgtp_uvu_fwd");
+    ctx->save_for_backward({x, y, w, path_scale});
+    ctx->saved_data["cfg"] = cfg;
+    ctx->saved_data["fallback"] = fallback;
+    return out;
+  }
+
+  static variable_list backward(AutogradContext* ctx, variable_list grad_outputs) {
+    const variable_list s = ctx->get_saved_variables();
+    const bool need_x = ctx->needs_input_grad(0), need_y = ctx->needs_input_grad(1), need_w = ctx->needs_input_grad(2);
+    if (at::GradMode::is_enabled()) {   // a gradient of the gradient is wanted: the differentiable route, in Python
+      py::gil_scoped_acquire gil;
+      const py::object fn = fallbacks().at((size_t)ctx->saved_data["fallback"].toInt());
+      const py::tuple r = fn(grad_outputs[0], s[0], s[1], s[2], need_x, need_y, need_w);
+      variable_list out(7);
+      for (int i = 0; i < 3; ++i)
+        if (!r[i].is_none()) out[i] = r[i].cast<at::Tensor>();
+      return out;
+    }
+    const at::Tensor& x = s[0];
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+    cgtp_uvu_args a = row_args(x, s[1], s[2], s[3], ctx->saved_data["cfg"].toInt());
+    const at::Tensor g = grad_outputs[0].contiguous();
+    a.grad_out = g.data_ptr();
+    at::Tensor gx, gy, gw;
+    if (need_x) gx = at::empty_like(x);
+    if (need_y) gy = at::empty_like(s[1]);
+    if (need_w) gw = at::empty_like(s[2]);
+    a.grad_x = const_cast<void*>(ptr_or_null(gx));
+    a.grad_y = const_cast<void*>(ptr_or_null(gy));
+    a.grad_w = const_cast<void*>(ptr_or_null(gw));
+    at::Tensor ws = workspace_for(a, 1, x);
+    check_status(cgtp_uvu_bwd(&a, current_stream(x)), "cgtp_uvu_bwd");
+    return {gx, gy, gw, at::Tensor(), at::Tensor(), at::Tensor(), at::Tensor()};
+  }
+};
+
+// Bytes of workspace the row-mode backward with all gradients would ask for (the Python side splits batches whose
+// per-row weight gradients exceed its budget before it comes here).
+int64_t row_backward_workspace(const at::Tensor& x, const at::Tensor& y, const at::Tensor& w, int64_t cfg) {
+  cgtp_uvu_args a = row_args(x, y, w, at::Tensor(), cfg);
+  a.grad_out = a.x;                      // any non-null pointers: the query asks which gradients are wanted
+  a.grad_w = const_cast<void*>(a.w);
+  return cgtp_uvu_workspace_bytes(&a, 1);
+}
+
 at::Tensor opt(const c10::optional<at::Tensor>& t) { return t.has_value() ? *t : at::Tensor(); }
 
 }  // namespace
@@ -173,5 +261,15 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         return h;
       }));
   m.def("edge_uvu", &edge_uvu, "fused edge product with its autograd node: x (N, D1, C), y (E, D2 | 3), w (E, P, C) | (P, C)");
+  m.def("row_uvu", [](const at::Tensor& x, const at::Tensor& y, const at::Tensor& w, c10::optional<at::Tensor> path_scale,
+                      int64_t cfg, int64_t d_out, int64_t fallback) {
+    const at::Tensor scale = opt(path_scale);
+    return RowUvu::apply(x, y, w, &scale, cfg, d_out, fallback);
+  }, "channel-wise product on a batch with its autograd node: x (N, D1, C), y (N, D2), w (N, P, C) | (P, C)");
+  m.def("row_backward_workspace", &row_backward_workspace);
+  m.def("register_fallback", [](py::object fn) {
+    fallbacks().push_back(std::move(fn));
+    return (int64_t)fallbacks().size() - 1;
+  }, "keeps a callable (grad_out, x, y, w, need_x, need_y, need_w) -> (gx, gy, gw) for gradients of higher order");
   m.def("abi_version", []() { return cgtp_version(); });
 }

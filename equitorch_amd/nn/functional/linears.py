@@ -53,6 +53,31 @@ class _UvuCompiled(Function):
         return (*res, None, None)
 
 
+def _row_uvu_extension(x: Tensor, y: Tensor, w: Tensor, tp_info: TensorProductInfo, cfg):
+    """The same launches issued by the C++ extension (autograd node and argument block in C++), or None: extension
+    not there, a table that needs its weights rearranged, or a shared weight whose per-row gradient workspace the
+    Python side would split."""
+    from ... import _shim
+    mod = _shim.module()
+    if mod is None or getattr(cfg, "w_rows", None) is not None:
+        return None
+    if w.ndim == 2 and w.requires_grad and mod.row_backward_workspace(x, y, w, int(cfg)) > kernels._GW_WORKSPACE_BYTES:
+        return None
+
+    def register():
+        def second_order(g, x_, y_, w_, need_x, need_y, need_w):
+            with torch.enable_grad():
+                spec = spec_from_tp_info(tp_info)
+                gx = tri(spec.grad_spec(0), (V, S, V), V, g, y_, w_) if need_x else None
+                gy = tri(spec.grad_spec(1), (V, V, V), S, x_, g, w_) if need_y else None
+                gw = tri(spec.grad_spec(2), (V, S, V), V, x_, y_, g, out_shared=(w_.ndim == 2)) if need_w else None
+            return gx, gy, gw
+        return mod.register_fallback(second_order)
+    fallback = kernels.cached(tp_info.info_Mij_fwd.scale, "row_uvu_fallback", register)
+    scale = cfg.scale_tensor(x.dtype, x.device) if isinstance(cfg, kernels.Cfg) else None
+    return mod.row_uvu(x, y, w, scale, int(cfg), int(kernels.uvu_dims(cfg)[2]), fallback)
+
+
 def _check_batch(input1, input2, weight):
     _lib.require_gpu(input1, input2, weight)
 
@@ -74,6 +99,9 @@ def tensor_product_u1u(input1: Tensor, input2: Tensor, weight: Tensor,
         x, y, w = input1.contiguous(), input2.contiguous(), weight.contiguous()
         if cfg >= 0 and kernels.uvu_launchable(cfg, x, y, w):
             kernels.log_tier("tensor_product_u1u", "compiled table", f"config {int(cfg)}")
+            out = _row_uvu_extension(x, y, w, tp_info_forward, cfg)
+            if out is not None:
+                return out
             return _UvuCompiled.apply(x, y, w, tp_info_forward, cfg)
     kernels.log_tier("tensor_product_u1u", "table-driven kernel", str(input1.dtype))
     return tri(spec_from_tp_info(tp_info_forward), (V, S, V), V, input1, input2, weight)

@@ -71,3 +71,43 @@ def test_gradient_subsets_and_no_grad(device):
         out = edge_tensor_product_uu(torch.randn(50, 9, 64, device=device), torch.randn(400, 9, device=device),
                                      torch.randn(400, 11, 64, device=device), plan, mod.tp_info_forward)
     assert out.shape == (50, 9, 64) and out.grad_fn is None and torch.isfinite(out).all()
+
+
+@pytest.mark.parametrize("lmax,ch,dtype,shared_w,kw", [
+    (2, 16, torch.float32, True, {}),
+    (2, 64, torch.float32, False, {}),
+    (3, 32, torch.float64, True, {}),
+    (2, 20, torch.float32, True, {"path_norm": False}),
+])
+def test_row_mode_through_the_extension(device, lmax, ch, dtype, shared_w, kw):
+    """``SO3Linear('uu')`` on a batch: first-order results bit-equal to the ``ctypes`` route; a gradient of the
+    gradient goes back to Python's differentiable route and agrees with it."""
+    from equitorch_amd import _shim
+    from equitorch_amd.nn import SO3Linear
+    assert _shim.module() is not None
+    irr, n, d = _sh(lmax), 700, (lmax + 1) ** 2
+    mod = SO3Linear(irr, irr, irr, ch, ch, internal_weights=False, feature_mode="uu", **kw).to(device)
+    g = torch.Generator().manual_seed(lmax * 100 + ch)
+    x, y = torch.randn(n, d, ch, generator=g, dtype=dtype), torch.randn(n, d, generator=g, dtype=dtype)
+    w = torch.randn(*(() if shared_w else (n,)), mod.num_paths, ch, generator=g, dtype=dtype)
+    ct = torch.randn(n, d, ch, generator=g, dtype=dtype).to(device)
+    first, second = [], []
+    for use_shim in (True, False):
+        saved = _shim._module
+        if not use_shim:
+            _shim._module = None
+        try:
+            xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+            out = mod(xd, yd, wd)
+            assert ("Cpp" in type(out.grad_fn).__name__) == use_shim, type(out.grad_fn).__name__
+            grads = torch.autograd.grad(out, (xd, yd, wd), ct, retain_graph=True)
+            gx, = torch.autograd.grad(out, xd, ct, create_graph=True)
+            gg = torch.autograd.grad(gx.square().sum(), (yd, wd))
+        finally:
+            _shim._module = saved
+        first.append((out, *grads))
+        second.append(gg)
+    for a, b in zip(*first):
+        assert torch.equal(a, b)
+    for a, b in zip(*second):
+        assert torch.allclose(a, b, rtol=1e-5 if dtype == torch.float32 else 1e-12, atol=1e-5 if dtype == torch.float32 else 1e-12)
