@@ -388,8 +388,10 @@ __device__ __forceinline__ void psw_bwd_block(const PswDev<T>& a, const PswLayou
         T tj[JB], o[V];
         psw_read_row<T, JB>(tj, t + row * a.JP + j0);
         mulv<T, V>(o, tj[0], gr[0]);
+        // rows past the block's own (a pass holds JB >= rows) were never written in t: whatever the LDS holds there
+        // must not reach the sum, not even multiplied by the zero rows of grad_out (it may be NaN)
 #pragma unroll
-        for (int j = 1; j < JB; ++j) fmav<T, V>(o, tj[j], gr[j]);
+        for (int j = 1; j < JB; ++j) fmav<T, V>(o, j < jb ? tj[j] : T(0), gr[j]);
         if (lane_ok && active) {
           T* dst = gwrow + (int64_t)kk * a.Wc;
           if (j0 > 0) {   // a block wider than one pass: the earlier rows' part is there already

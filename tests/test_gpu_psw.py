@@ -384,3 +384,29 @@ def test_weights_beyond_the_last_level_cache(device, monkeypatch, no_library_gem
     o32, g32 = ref_ops.dense_grads(ref_ops.dense_u1v, T, (sub(x), sub(y), sub(w)), sub(ct), dtype=torch.float32)
     for name, a, b, b32 in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads), (o32, *g32)):
         assert_close(sub(a), b, 1e-5, f"u1v per-sample, 1.08 GB of weights, {name}", norm="max", fp32_ref=b32)
+
+
+def test_gradcheck_and_gradgradcheck_with_a_weight_per_sample(device):
+    """The reference checks ``gradcheck`` and ``gradgradcheck`` of all four modes with shared and with per-sample
+    weights in float64 (``test/test_tp/test_grad_tp.py:57-103``, ``0e+1e+2e x 0e+1e+2e -> 0e+1e+2e+3e``); here for
+    the weight per sample: first order on the streaming kernels (uv, uvw) and the compiled / table-driven kernels
+    (uu, uuu), second order through the differentiable route behind them."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    io, i1, i2 = "0e+1e+2e+3e", "0e+1e+2e", "0e+1e+2e"
+    info = tp_infos(Irreps(io), Irreps(i1), Irreps(i2))[0].to(device)
+    from equitorch_amd.ops import kernels
+    p = kernels.coo_of(info).P
+    g = torch.Generator().manual_seed(2)
+    n = 5
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).to(device).requires_grad_(True)
+    cases = (("u1u", F.tensor_product_u1u, rd(n, 9, 3), rd(n, 9), rd(n, p, 3)),
+             ("u1v", F.tensor_product_u1v, rd(n, 9, 3), rd(n, 9), rd(n, p, 3, 4)),
+             ("uuu", F.tensor_product_uuu, rd(n, 9, 3), rd(n, 9, 3), rd(n, p, 3)),
+             ("uvw", F.tensor_product_uvw, rd(n, 9, 3), rd(n, 9, 2), rd(n, p, 3, 2, 4)))
+    for name, op, x, y, w in cases:
+        fn = lambda x, y, w: op(x, y, w, info)
+        assert fn(x, y, w).shape[:2] == (n, 16), name
+        assert torch.autograd.gradcheck(fn, (x, y, w), eps=1e-6, atol=1e-5, rtol=1e-5, nondet_tol=1e-9), name
+        assert torch.autograd.gradgradcheck(fn, (x, y, w), eps=1e-6, atol=1e-5, rtol=1e-5, nondet_tol=1e-9), name
