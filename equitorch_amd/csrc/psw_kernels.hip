@@ -40,12 +40,13 @@ __device__ __forceinline__ void psw_wave_sync() {
 }
 
 constexpr unsigned kPswEndRow = 1u << 24;   // entry word: last entry of its (path, output row) run
+constexpr unsigned kPswNoTerm = 1u << 25;   // entry word: the path has no term for this row (the row of t is zero)
 
 template <typename T>
 struct PswDev {
   const T* x; const T* y; const T* w; T* out;
   const T* g; T* gx; T* gy; T* gw;
-  const uint32_t* entries;   // j | a << 8 | b << 16 | kPswEndRow
+  const uint32_t* entries;   // j | a << 8 | b << 16 | kPswEndRow | kPswNoTerm
   const T* coef;
   const int32_t* slots;      // (path, e0, e1) per walked path
   const int32_t* blocks;     // (m0, L, q0, q1) per output irrep
@@ -118,7 +119,7 @@ __device__ __forceinline__ void psw_form_t(const PswDev<T>& a, T* t, const T* xs
     for (int e = e0; e < e1; ++e) {
       const unsigned wd = ent[e];
       const T c = cf[e];
-      val = fma(c * xu[(int)((wd >> 8) & 255u) * a.U], yv[(int)((wd >> 16) & 255u) * a.Vy], val);
+      if (!(wd & kPswNoTerm)) val = fma(c * xu[(int)((wd >> 8) & 255u) * a.U], yv[(int)((wd >> 16) & 255u) * a.Vy], val);
       if (wd & kPswEndRow) {
         row[wd & 255u] = val;
         val = T(0);
@@ -270,7 +271,7 @@ __device__ __forceinline__ void psw_carry_back(const PswDev<T>& a, const PswLayo
       for (int e = e0; e < e1; ++e) {
         const unsigned wd = ent[e];
         const int j = (int)(wd & 255u) - j0;
-        if (j < 0 || j >= jb) continue;
+        if (j < 0 || j >= jb || (wd & kPswNoTerm)) continue;
         const int ia = (int)((wd >> 8) & 255u) * a.U + u, ib = (int)((wd >> 16) & 255u);
         const T cg = cf[e] * gr[j + j0];
         if (want_x) gxl[ia] = fma(cg, ys[ib], gxl[ia]);
@@ -286,7 +287,7 @@ __device__ __forceinline__ void psw_carry_back(const PswDev<T>& a, const PswLayo
       for (int e = e0; e < e1; ++e) {
         const unsigned wd = ent[e];
         const int j = (int)(wd & 255u);
-        if (j < j0 || j >= j0 + jb) continue;
+        if (j < j0 || j >= j0 + jb || (wd & kPswNoTerm)) continue;
         const T* yb = ys + (int)((wd >> 16) & 255u) * a.Vy;
         T sum = T(0);
         for (int v = 0; v < a.Vy; ++v) sum = fma(yb[v], gr[v * a.JP + j], sum);
@@ -301,7 +302,7 @@ __device__ __forceinline__ void psw_carry_back(const PswDev<T>& a, const PswLayo
       for (int e = e0; e < e1; ++e) {
         const unsigned wd = ent[e];
         const int j = (int)(wd & 255u);
-        if (j < j0 || j >= j0 + jb) continue;
+        if (j < j0 || j >= j0 + jb || (wd & kPswNoTerm)) continue;
         const T* xa = xs + (int)((wd >> 8) & 255u) * a.U + u0;
         T sum = T(0);
         for (int ul = 0; ul < uc; ++ul) sum = fma(xa[ul], gr[(int64_t)ul * a.Vy * a.JP + j], sum);

@@ -23,6 +23,7 @@ from ... import _lib
 from ...ops import kernels
 
 _END_ROW = 1 << 24
+_NO_TERM = 1 << 25       # the path has no term for this row: the entry only closes the (zero) row
 MAX_BLOCK_ROWS = 32      # 16 rows per pass; every further pass streams the block's weights again
 
 
@@ -58,7 +59,7 @@ class PswTable:
                 for j in range(rows):
                     hit = sel[out_row[sel] == m0 + j]
                     if hit.size == 0:                      # keeps the row of the coupled operand defined: zero
-                        words.append(j | _END_ROW)
+                        words.append(j | _END_ROW | _NO_TERM)
                         coefs.append(0.0)
                         continue
                     for i, t in enumerate(hit):

@@ -478,7 +478,8 @@ int cgtp_uvt_grad_w(const cgtp_uvt_gw_args* args, void* stream);
  *   slots   [n_slots][3]   (weight path p, first entry, one past the last entry) of a walked path
  *   entries [n_entries]    j | a << 8 | b << 16 | 1 << 24 on the last entry of a run of equal j; j = output row - the
  *                          block's first row; sorted by j inside a slot; every j < L occurs in every slot of the
- *                          block (with coefficient 0 where the path has no term for it)
+ *                          block (where the path has no term for it: one entry j | 1 << 24 | 1 << 25, no operand is
+ *                          read for it)
  *   coef    [n_entries]    dtype
  * x (n_rows, D1, cx), y (n_rows, D2, cy) or NULL (then cy = 1, D2 = 1 and y = 1), out / g (n_rows, DO, cout), all
  * contiguous, dtype CGTP_F32 | CGTP_F64.  cout <= 64 vector lanes: cout <= 256 (fp32) / 128 (fp64) when it is a

@@ -73,7 +73,7 @@ def test_rows_without_a_term_and_tables_the_kernels_do_not_walk():
     from equitorch_amd.nn.functional._psw import PswTable
     # path 0 writes rows 0..2 but has no term for row 1
     t = PswTable([0, 2], [0, 1], [0, 0], [0, 0], [1.0, 2.0], 2, 1, 3, 1, "cpu")
-    assert t.entries.tolist() == [0 | 1 << 24, 1 | 1 << 24, 2 | 1 << 8 | 1 << 24]
+    assert t.entries.tolist() == [0 | 1 << 24, 1 | 1 << 24 | 1 << 25, 2 | 1 << 8 | 1 << 24]
     assert t.coef(torch.float64).tolist() == [1.0, 0.0, 2.0]
     assert t.blocks.tolist() == [[0, 3, 0, 1]] and t.slots.tolist() == [[0, 0, 3]]
     # rows 0..1 and 1..2 overlap without coinciding: one block of three rows, zero entries where a path has no term
