@@ -76,6 +76,7 @@ class PswTable:
         self.blocks = torch.tensor(blocks, dtype=torch.int32).reshape(-1, 4).to(device)
         self.dims = (int(d1), int(d2), int(d_out), int(n_paths))
         self.max_rows = max(rows for _, rows, _, _ in blocks)
+        self.launchable = {}                 # memo of launchable(): extents and dtype -> bool
 
     def coef(self, dtype) -> Tensor:
         if dtype not in self._coef:
@@ -130,10 +131,18 @@ def launchable(table: Optional[PswTable], x: Tensor, y: Optional[Tensor], w: Ten
     cy = 1 if y is None or y.ndim == 2 else y.shape[2]
     if x.shape[1] != d1 or tuple(w.shape[:3]) != (x.shape[0], n_paths, x.shape[2] * cy):
         return False
-    args, c_table = _args(table, x, y, w), table.c_table(x.dtype)
-    args.out = args.g = 256                    # the real buffers are fresh allocations (aligned)
-    return (_lib.lib.cgtp_psw_validate(C.byref(args), C.byref(c_table), 0) == 0
-            and _lib.lib.cgtp_psw_validate(C.byref(args), C.byref(c_table), 1) == 0)
+    # the answer depends on the extents, the dtype and the 16-byte alignment of the weight only
+    key = (x.dtype, x.shape[0], x.shape[2], cy, w.shape[-1], y is None, w.data_ptr() % 16)
+    hit = table.launchable.get(key)
+    if hit is None:
+        args, c_table = _args(table, x, y, w), table.c_table(x.dtype)
+        args.out = args.g = 256                # the real buffers are fresh allocations (aligned)
+        hit = (_lib.lib.cgtp_psw_validate(C.byref(args), C.byref(c_table), 0) == 0
+               and _lib.lib.cgtp_psw_validate(C.byref(args), C.byref(c_table), 1) == 0)
+        if len(table.launchable) > 256:
+            table.launchable.clear()
+        table.launchable[key] = hit
+    return hit
 
 
 class _Product(Function):

@@ -320,6 +320,65 @@ def u1v(x: Tensor, y: Tensor, w: Tensor, tp_info) -> Tensor:
     return _U1vNative.apply(x.contiguous(), y.contiguous(), w.contiguous(), tp_info)
 
 
+# ---- vu1: out[n, M] = sum_t c_t <y[n, b_t, :], x[n, a_t, :] @ W[p_t]> ---------------------------------------------
+# With the table's output rows and second-operand rows exchanged (T'), this is the gradient of u1v_T' with respect to
+# its channel-less operand for the cotangent y — the kernel cgtp_uvt_grad_y — and its own gradients are the forward
+# (grad y), the input gradient (grad x) and the weight gradient of u1v_T' with the cotangent of vu1 as the channel-less
+# operand.  The reference computes it in three stages, weight first (equitorch/nn/functional/linears.py:414-492).
+def _swapped(tp_info) -> CooTable:
+    def build():
+        c = _coo(tp_info)
+        return CooTable(c._replace(M=c.M2, M2=c.M, D2=c.DO, DO=c.D2), torch.zeros(1), None)
+    return kernels.cached(_anchor(tp_info), "vu1_table", build)
+
+
+class _Vu1Native(Function):
+    @staticmethod
+    def forward(ctx, x: Tensor, y: Tensor, w: Tensor, tp_info):
+        t = _swapped(tp_info)
+        p, u, wc = w.shape
+        out = grad_y(x, y, pack(w, p, u, wc, u * wc, wc, 1), t, t.coo.D2)
+        ctx.save_for_backward(x, y, w)
+        ctx.tp_info = tp_info
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        from . import _uv_gemm
+        x, y, w = ctx.saved_tensors
+        need = ctx.needs_input_grad[:3]
+        if torch.is_grad_enabled():       # higher-order derivative: the differentiable route throughout
+            with torch.enable_grad():
+                out = _uv_gemm.vu1(x, y, w, ctx.tp_info)
+                wanted = [v for v, n in zip((x, y, w), need) if n]
+                got = iter(torch.autograd.grad(out, wanted, g, create_graph=True, allow_unused=True))
+            return tuple(next(got) if n else None for n in need) + (None,)
+        t = _swapped(ctx.tp_info)
+        c = t.coo
+        p, u, wc = w.shape
+        g = g.contiguous()
+        gx = apply(y, g, pack(w, p, wc, u, u * wc, 1, wc), t, "in1", c.D1, u) if need[0] else None
+        gy = apply(x, g, pack(w, p, u, wc, u * wc, wc, 1), t, "out", c.DO, wc) if need[1] else None
+        gw = grad_w(x, g, y, t) if need[2] else None
+        return gx, gy, gw, None
+
+
+def vu1_supported(x: Tensor, y: Tensor, w: Tensor, tp_info) -> bool:
+    if not (x.dtype == y.dtype == w.dtype and x.dtype in (torch.float32, torch.float64) and x.ndim == 3 and y.ndim == 3
+            and w.ndim == 3 and x.shape[0] > 0):
+        return False
+    c = _coo(tp_info)
+    n, (_, u, wc) = x.shape[0], w.shape
+    if tuple(x.shape) != (n, c.D1, u) or tuple(y.shape) != (n, c.D2, wc) or w.shape[0] != c.P:
+        raise _lib.CgtpError(f"operands {tuple(x.shape)}, {tuple(y.shape)}, {tuple(w.shape)} do not fit the table: "
+                             f"expected (N, {c.D1}, C1), (N, {c.D2}, C2), ({c.P}, C1, C2)")
+    return u1v_fits(n, u, wc, _swapped(tp_info), x.dtype) and x.data_ptr() % 16 == 0 and y.data_ptr() % 16 == 0
+
+
+def vu1(x: Tensor, y: Tensor, w: Tensor, tp_info) -> Tensor:
+    return _Vu1Native.apply(x.contiguous(), y.contiguous(), w.contiguous(), tp_info)
+
+
 class _UvwNative(Function):
     """uvw, shared fp32 weight ``(P, U, V, W)``: forward and the gradients of both operands on ``cgtp_uvt_apply``
     (with the weight permuted as the reference permutes it, ``tensor_products.py:126-150``); the weight gradient and

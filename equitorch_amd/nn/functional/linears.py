@@ -220,6 +220,10 @@ def tensor_product_vu1(input1: Tensor, input2: Tensor, weight: Tensor,
             shape = weight.shape
             return _psw.product(table, input1, input2, w4, lambda x, y, w: _uv_gemm.vu1(
                 x, y, w.reshape(shape), tp_info_forward).unsqueeze(-1)).squeeze(-1)
+    from . import _uv_native
+    if _uv_native.vu1_supported(input1, input2, weight, tp_info_forward):
+        kernels.log_tier("tensor_product_vu1", "fp32 matrix-core kernel (table-driven)")
+        return _uv_native.vu1(input1, input2, weight, tp_info_forward)
     if input1.ndim == 3 and input2.ndim == 3 and _uv_gemm.supported(input1, input2, weight):
         kernels.log_tier("tensor_product_vu1", "library GEMM + table-driven kernel", str(input1.dtype))
         return _uv_gemm.vu1(input1, input2, weight, tp_info_forward)

@@ -325,3 +325,40 @@ def test_channel_counts_that_are_not_multiples_of_four(device, monkeypatch, dtyp
         for what, a, b in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads)):
             assert a.shape == b.shape
             assert_close(a, b, tol, f"{name} {dtype} odd channel counts {what}", norm="max")
+
+
+@pytest.mark.parametrize("irreps,c1,c2,n,dtype", [((_sh(2),) * 3, 32, 48, 300, torch.float32),
+                                                   (("1o+2e+1e", "0e+1o+2e", "0e+1o"), 16, 64, 515, torch.float32),
+                                                   ((_sh(3), _sh(2), _sh(3)), 20, 12, 70, torch.float64)])
+def test_vu1_native(device, monkeypatch, irreps, c1, c2, n, dtype):
+    """``out[n,M] = sum c <y[n,b,:], x[n,a,:] @ W[p]>`` with a shared weight on the table-driven matrix-core kernels
+    (the kernel of the second operand's gradient of u1v, run on the table with output and second-operand rows
+    exchanged), forward and all gradients against the dense oracle."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.ops import kernels
+    from equitorch_amd.utils import tp_infos
+    io, i1, i2 = irreps
+    infos = [t.to(device) for t in tp_infos(Irreps(io), Irreps(i1), Irreps(i2))[:3]]
+    T = ref_ops.dense_coupling(io, i1, i2).float().double()
+    g = torch.Generator().manual_seed(c1 + c2 + n)
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).to(dtype)
+    x, y, w = rd(n, T.shape[2], c1), rd(n, T.shape[3], c2), rd(T.shape[0], c1, c2) / (c1 * c2) ** 0.5
+    ct = rd(n, T.shape[1])
+
+    def dense_vu1(T, x, y, w, dtype=torch.float64):
+        return ref_ops.dense_uvw(T, x, y, w.unsqueeze(-1), dtype=dtype).squeeze(-1)
+    seen = []
+    monkeypatch.setattr(kernels, "log_tier", lambda op, tier, detail="": seen.append(tier))
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    out = F.tensor_product_vu1(xd, yd, wd, *infos)
+    assert "matrix-core" in seen[-1], seen
+    grads = torch.autograd.grad(out, (xd, yd, wd), ct.to(device))
+    ref_out, ref_grads = ref_ops.dense_grads(dense_vu1, T, (x, y, w), ct)
+    tol = 1e-5 if dtype == torch.float32 else 1e-11
+    twin = (None,) * 4
+    if dtype == torch.float32:
+        o32, g32 = ref_ops.dense_grads(dense_vu1, T, (x, y, w), ct, dtype=torch.float32)
+        twin = (o32, *g32)
+    for name, a, b, b32 in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads), twin):
+        assert_close(a, b, tol, f"vu1 {io} {c1}x{c2} N={n} {dtype} {name}", norm="max", fp32_ref=b32)
