@@ -320,6 +320,16 @@ def u1v(x: Tensor, y: Tensor, w: Tensor, tp_info) -> Tensor:
     return _U1vNative.apply(x.contiguous(), y.contiguous(), w.contiguous(), tp_info)
 
 
+# ---- 1vu: the channels on the second operand — u1v on the table with the operands' rows exchanged -------------------
+def operands_exchanged(tp_info) -> CooTable:
+    def build():
+        from . import _uv_gemm
+        c = _coo(tp_info)
+        return CooTable(c._replace(M1=c.M2, M2=c.M1, D1=c.D2, D2=c.D1), torch.zeros(1),
+                        lambda xx, yy, ww: _uv_gemm.one_vu(yy, xx, ww, tp_info))
+    return kernels.cached(_anchor(tp_info), "1vu_table", build)
+
+
 # ---- vu1: out[n, M] = sum_t c_t <y[n, b_t, :], x[n, a_t, :] @ W[p_t]> ---------------------------------------------
 # With the table's output rows and second-operand rows exchanged (T'), this is the gradient of u1v_T' with respect to
 # its channel-less operand for the cotangent y — the kernel cgtp_uvt_grad_y — and its own gradients are the forward

@@ -196,6 +196,12 @@ def tensor_product_1vu(input1: Tensor, input2: Tensor, weight: Tensor,
             kernels.log_tier("tensor_product_1vu", "per-sample weight streaming kernel", str(input1.dtype))
             return _psw.product(table, input2, input1, weight,
                                 lambda x, y, w: _uv_gemm.one_vu(y, x, w, tp_info_forward))
+    if input1.ndim == 2 and input2.ndim == 3 and weight.ndim == 3:
+        from . import _uv_native
+        table = _uv_native.operands_exchanged(tp_info_forward)
+        if _uv_native.u1v_supported(input2, input1, weight, table):
+            kernels.log_tier("tensor_product_1vu", "fp32 matrix-core kernel (table-driven)")
+            return _uv_native.u1v(input2, input1, weight, table)
     if input1.ndim == 2 and input2.ndim == 3 and _uv_gemm.supported(input1, input2, weight):
         kernels.log_tier("tensor_product_1vu", "library GEMM + table-driven kernel", str(input1.dtype))
         return _uv_gemm.one_vu(input1, input2, weight, tp_info_forward)

@@ -362,3 +362,41 @@ def test_vu1_native(device, monkeypatch, irreps, c1, c2, n, dtype):
         twin = (o32, *g32)
     for name, a, b, b32 in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads), twin):
         assert_close(a, b, tol, f"vu1 {io} {c1}x{c2} N={n} {dtype} {name}", norm="max", fp32_ref=b32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_1vu_native(device, monkeypatch, dtype):
+    """The channels on the second operand with a shared weight: the u1v kernels on the table with the operands' rows
+    exchanged; forward, all gradients and a gradient of the gradient."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.ops import kernels
+    from equitorch_amd.utils import tp_infos
+    io, i1, i2 = "1o+2e+1e", "0e+1o", "0e+1o+2e"
+    infos = [t.to(device) for t in tp_infos(Irreps(io), Irreps(i1), Irreps(i2))[:3]]
+    T = ref_ops.dense_coupling(io, i1, i2).float().double()
+    n, cin, cout = 333, 24, 40
+    g = torch.Generator().manual_seed(21)
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64).to(dtype)
+    x, y, w, ct = rd(n, T.shape[2]), rd(n, T.shape[3], cin), rd(T.shape[0], cin, cout) / cin ** 0.5, rd(n, T.shape[1], cout)
+
+    def dense_1vu(T, x, y, w, dtype=torch.float64):
+        return ref_ops.dense_u1v(T.transpose(2, 3), y, x, w, dtype=dtype)
+    seen = []
+    monkeypatch.setattr(kernels, "log_tier", lambda op, tier, detail="": seen.append(tier))
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    out = F.tensor_product_1vu(xd, yd, wd, *infos)
+    assert "matrix-core" in seen[-1], seen
+    grads = torch.autograd.grad(out, (xd, yd, wd), ct.to(device), retain_graph=True)
+    ref_out, ref_grads = ref_ops.dense_grads(dense_1vu, T, (x, y, w), ct)
+    tol = 1e-5 if dtype == torch.float32 else 1e-11
+    for name, a, b in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads)):
+        assert_close(a, b, tol, f"1vu {dtype} {name}", norm="max")
+    if dtype == torch.float64:
+        gy, = torch.autograd.grad(out, yd, ct.to(device), create_graph=True)
+        gg = torch.autograd.grad(gy.square().sum(), (xd, wd))
+        xr, yr, wr = (t.clone().requires_grad_(True) for t in (x, y, w))
+        rgy, = torch.autograd.grad(dense_1vu(T, xr, yr, wr), yr, ct, create_graph=True)
+        rgg = torch.autograd.grad(rgy.square().sum(), (xr, wr))
+        for name, a, b in zip(("d/dx", "d/dw"), gg, rgg):
+            assert_close(a, b, 1e-10, f"1vu second order {name}", norm="max")
