@@ -53,6 +53,33 @@ class _UvuCompiled(Function):
         return (*res, None, None)
 
 
+class _UvuTableRows(Function):
+    """u1u for a table that is not compiled in, on the table-driven segment kernels (``cgtp_uvu_tab_fwd`` / ``_bwd``)
+    with the batch as an edge list of one edge per node."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, y: Tensor, w: Tensor, tp_info: TensorProductInfo, tab):
+        out = kernels.uvu_tab_forward(tab, x, y, w, kernels.identity_segments(x.shape[0], x.device))
+        ctx.save_for_backward(x, y, w)
+        ctx.tp_info, ctx.tab = tp_info, tab
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        x, y, w = ctx.saved_tensors
+        need = ctx.needs_input_grad[:3]
+        if torch.is_grad_enabled():   # higher-order derivative requested: the differentiable contraction
+            with torch.enable_grad():
+                spec = spec_from_tp_info(ctx.tp_info)
+                gx = tri(spec.grad_spec(0), (V, S, V), V, g, y, w) if need[0] else None
+                gy = tri(spec.grad_spec(1), (V, V, V), S, x, g, w) if need[1] else None
+                gw = tri(spec.grad_spec(2), (V, S, V), V, x, y, g, out_shared=(w.ndim == 2)) if need[2] else None
+            return gx, gy, gw, None, None
+        res = kernels.uvu_tab_backward(ctx.tab, x, y, w, g.contiguous(), need,
+                                       kernels.identity_segments(x.shape[0], x.device))
+        return (*res, None, None)
+
+
 def _row_uvu_extension(x: Tensor, y: Tensor, w: Tensor, tp_info: TensorProductInfo, cfg):
     """The same launches issued by the C++ extension (autograd node and argument block in C++), or None: extension
     not there, a table that needs its weights rearranged, or a shared weight whose per-row gradient workspace the
@@ -103,6 +130,16 @@ def tensor_product_u1u(input1: Tensor, input2: Tensor, weight: Tensor,
             if out is not None:
                 return out
             return _UvuCompiled.apply(x, y, w, tp_info_forward, cfg)
+    if (input1.ndim == 3 and input2.ndim == 2 and input1.dtype == input2.dtype == weight.dtype == torch.float32
+            and input1.shape[0] == input2.shape[0] and input1.shape[0] > 0):
+        # no compiled table: the table-driven segment kernels of the edge products, the batch seen as an edge list in
+        # which every row is a node with one edge (entries walked from registers, operands in LDS: about a third of the
+        # time of the general contraction kernel below, which reads every operand of every coefficient from memory)
+        tab = kernels.uvu_table_of(tp_info_forward, input1.device)
+        x, y, w = input1.contiguous(), input2.contiguous(), weight.contiguous()
+        if kernels.uvu_tab_launchable(tab, x, y, w, weight.requires_grad and torch.is_grad_enabled()):
+            kernels.log_tier("tensor_product_u1u", "table-driven segment kernels on the batch", f"{tab.nnz} coefficients")
+            return _UvuTableRows.apply(x, y, w, tp_info_forward, tab)
     kernels.log_tier("tensor_product_u1u", "table-driven kernel", str(input1.dtype))
     return tri(spec_from_tp_info(tp_info_forward), (V, S, V), V, input1, input2, weight)
 

@@ -527,6 +527,30 @@ def seg_ranges(cfg: int, seg: SegIndex, dtype_code: int, channels: int, backward
     return None, None
 
 
+class IdentitySegments:
+    """A plain batch seen as an edge list in which row r is the only edge of node r: what the table-driven segment
+    kernels need (``ptr``, ``perm``, ``seg_ids``, ``gather``) to run a product on a batch.  ``fwd_index`` and
+    ``bwd_index`` are this object itself, as on an ``EdgePlan``."""
+
+    def __init__(self, n: int, device):
+        ids = torch.arange(n + 1, dtype=torch.int64, device=device)
+        self.ptr, self.perm, self.seg_ids, self.gather = ids, None, ids[:n], ids[:n]
+        self.fwd_index = self.bwd_index = self
+
+
+_IDENTITY = {}
+
+
+def identity_segments(n: int, device) -> IdentitySegments:
+    key = (n, str(device))
+    seg = _IDENTITY.get(key)
+    if seg is None:
+        if len(_IDENTITY) >= 8:
+            _IDENTITY.pop(next(iter(_IDENTITY)))
+        seg = _IDENTITY[key] = IdentitySegments(n, device)
+    return seg
+
+
 def _uvu_args(cfg: int, x: Tensor, y: Tensor, w: Tensor, seg: Optional[SegIndex], gather: Optional[Tensor],
               pos_per_wave: int = 0, y_vec: int = 0, backward: bool = False) -> UvuArgs:
     a = UvuArgs()

@@ -127,3 +127,36 @@ def test_speed_next_to_the_other_routes(device, monkeypatch):
         print(f"{name}: {nnz[name]} coefficients, {ms[name]:.3f} ms per forward + backward")
     assert ms["table"] < ms["separate"], ms
     assert ms["table"] / nnz["table"] <= 6.0 * ms["compiled"] / nnz["compiled"], (ms, nnz)
+
+
+@pytest.mark.parametrize("irreps,channels", [(TABLES[0], 64), (TABLES[2], 20), (("0e+2e+4e",) * 3, 32)])
+def test_plain_batch_without_a_compiled_table(device, monkeypatch, irreps, channels):
+    """``SO3Linear('uu')`` on a batch for irreps without a compiled table: the segment kernels with every row a node of
+    one edge; forward, all gradients and a gradient of the gradient (which goes to the differentiable contraction)."""
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.ops import kernels
+    io, i1, i2 = irreps
+    mod = SO3Linear(i1, i2, io, channels, channels, internal_weights=False, feature_mode="uu").to(device)
+    assert int(kernels.uvu_config_of(mod.tp_info_forward)) < 0
+    n = 777
+    gen = torch.Generator().manual_seed(stable_seed("row table", irreps, channels))
+    x, y = torch.randn(n, Irreps(i1).dim, channels, generator=gen), torch.randn(n, Irreps(i2).dim, generator=gen)
+    w, ct = torch.randn(n, mod.num_paths, channels, generator=gen), torch.randn(n, Irreps(io).dim, channels, generator=gen)
+    seen = []
+    monkeypatch.setattr(kernels, "log_tier", lambda op, tier, detail="": seen.append(tier))
+    xd, yd, wd = (t.to(device).requires_grad_(True) for t in (x, y, w))
+    out = mod(xd, yd, wd)
+    assert "segment kernels on the batch" in seen[-1], seen
+    grads = torch.autograd.grad(out, (xd, yd, wd), ct.to(device), retain_graph=True)
+    T = ref_ops.dense_coupling(io, i1, i2).float().double()
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1u, T, (x, y, w), ct)
+    for name, a, b in zip(("out", "grad_x", "grad_y", "grad_w"), (out, *grads), (ref_out, *ref_grads)):
+        assert_close(a, b, 1e-5, f"{io} C={channels} batch {name}")
+    gx, = torch.autograd.grad(out, xd, ct.to(device), create_graph=True)
+    gg = torch.autograd.grad(gx.square().sum(), (yd, wd))
+    xr, yr, wr = (t.double().requires_grad_(True) for t in (x, y, w))
+    rgx, = torch.autograd.grad(ref_ops.dense_u1u(T, xr, yr, wr), xr, ct.double(), create_graph=True)
+    rgg = torch.autograd.grad(rgx.square().sum(), (yr, wr))
+    for name, a, b in zip(("d/dy", "d/dw"), gg, rgg):
+        assert_close(a, b, 1e-5, f"{io} batch second order {name}", norm="max")
