@@ -410,3 +410,34 @@ def test_gradcheck_and_gradgradcheck_with_a_weight_per_sample(device):
         assert fn(x, y, w).shape[:2] == (n, 16), name
         assert torch.autograd.gradcheck(fn, (x, y, w), eps=1e-6, atol=1e-5, rtol=1e-5, nondet_tol=1e-9), name
         assert torch.autograd.gradgradcheck(fn, (x, y, w), eps=1e-6, atol=1e-5, rtol=1e-5, nondet_tol=1e-9), name
+
+
+def test_weight_tensor_past_two_to_the_31_elements(device, monkeypatch, no_library_gemm):
+    """N = 70 000 samples, 64 -> 64 channels, lmax = 2: the per-sample weight has 3.15e9 elements (12.6 GB), so every
+    offset into it and into its gradient past sample 47 662 exceeds 32 bits.  Samples from the far end, and a strided
+    subset, against the dense oracle on exactly those samples."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.utils import tp_infos
+    irr, n, ch = _sh(2), 70000, 64
+    infos = [t.to(device) for t in tp_infos(Irreps(irr), Irreps(irr), Irreps(irr))[:3]]
+    T = ref_ops.dense_coupling(irr, irr, irr).float().double()
+    g = torch.Generator(device=device).manual_seed(2)
+    x = torch.randn(n, 9, ch, device=device, generator=g).requires_grad_(True)
+    y = torch.randn(n, 9, device=device, generator=g).requires_grad_(True)
+    w = torch.randn(n, T.shape[0], ch, ch, device=device, generator=g).mul_(ch ** -0.5).requires_grad_(True)
+    ct = torch.randn(n, 9, ch, device=device, generator=g)
+    assert w.numel() > 2 ** 31
+    seen = _tiers(monkeypatch)
+    with no_library_gemm():
+        out = F.tensor_product_u1v(x, y, w, *infos)
+        gx, gy, gw = torch.autograd.grad(out, (x, y, w), ct)
+    assert "per-sample weight streaming" in seen[-1], seen
+    rows = torch.cat([torch.arange(3, n, 5000, device=device), torch.arange(n - 8, n, device=device)])
+    sub = lambda t: t.detach()[rows].cpu()
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1v, T, (sub(x), sub(y), sub(w)), sub(ct))
+    o32, g32 = ref_ops.dense_grads(ref_ops.dense_u1v, T, (sub(x), sub(y), sub(w)), sub(ct), dtype=torch.float32)
+    for name, a, b, b32 in zip(("out", "grad_x", "grad_y", "grad_w"), (out, gx, gy, gw), (ref_out, *ref_grads), (o32, *g32)):
+        assert_close(sub(a), b, 1e-5, f"u1v per-sample, 3.15e9 weights, {name}", norm="max", fp32_ref=b32)
+    del w, gw
+    torch.cuda.empty_cache()
