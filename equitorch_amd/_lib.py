@@ -158,6 +158,11 @@ def _load():
     lib.cgtp_uvu_tab_validate.argtypes = [C.POINTER(UvuArgs), C.POINTER(UvuTab), C.c_int]
     lib.cgtp_uvu_tab_fwd.argtypes = [C.POINTER(UvuArgs), C.POINTER(UvuTab), C.c_void_p]
     lib.cgtp_uvu_tab_bwd.argtypes = [C.POINTER(UvuArgs), C.POINTER(UvuTab), C.c_void_p]
+    lib.cgtp_bessel.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_double, C.c_int32, C.c_void_p]
+    lib.cgtp_bessel_grad.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32,
+                                     C.c_double, C.c_int32, C.c_void_p]
+    lib.cgtp_cutoff.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_double, C.c_double, C.c_double,
+                                C.c_int32, C.c_void_p]
     lib.cgtp_psw_validate.argtypes = [C.POINTER(PswArgs), C.POINTER(PswTable), C.c_int]
     lib.cgtp_psw_fwd.argtypes = [C.POINTER(PswArgs), C.POINTER(PswTable), C.c_void_p]
     lib.cgtp_psw_bwd.argtypes = [C.POINTER(PswArgs), C.POINTER(PswTable), C.c_void_p]

@@ -1,7 +1,9 @@
 """Cutoff modules (``equitorch/nn/cutoffs.py``): the edge length mapped to [0, 1] over ``[r_min, r_max]``, then one
-of the envelopes of ``functional.cutoffs``."""
+of the envelopes of ``functional.cutoffs``.  The functions there are tensor expressions, as in the reference; the modules
+here take one kernel each way for fp32 / fp64 tensors on the GPU (``functional/_radial.py``)."""
 from torch import Tensor, nn
 
+from .functional import _radial
 from .functional.cutoffs import cosine_cutoff, mollifier_cutoff, polynomial_cutoff, radial_standarize
 
 
@@ -14,6 +16,13 @@ class _Cutoff(nn.Module):
     def _unit(self, input: Tensor) -> Tensor:
         return radial_standarize(input, self.range, self.r_min)
 
+    def _apply_envelope(self, input: Tensor, kind: int, param: float, expression) -> Tensor:
+        """fp32 / fp64 tensors on the GPU: standardisation, envelope and (in the backward) their derivative in one
+        launch; everything else the tensor expression."""
+        if _radial.fused(input):
+            return _radial.cutoff(input, kind, self.r_min, self.range, param, expression)
+        return expression(input)
+
 
 class PolynomialCutoff(_Cutoff):
     """Polynomial envelope of order ``p >= 2`` (reference ``:7-42``)."""
@@ -25,7 +34,7 @@ class PolynomialCutoff(_Cutoff):
         self.p = float(p)
 
     def forward(self, input: Tensor) -> Tensor:
-        return polynomial_cutoff(self._unit(input), p=self.p)
+        return self._apply_envelope(input, _radial.POLYNOMIAL, self.p, lambda r: polynomial_cutoff(self._unit(r), p=self.p))
 
 
 class CosineCutoff(_Cutoff):
@@ -36,7 +45,7 @@ class CosineCutoff(_Cutoff):
         super().__init__(r_max, r_min)
 
     def forward(self, input: Tensor) -> Tensor:
-        return cosine_cutoff(self._unit(input))
+        return self._apply_envelope(input, _radial.COSINE, 0.0, lambda r: cosine_cutoff(self._unit(r)))
 
 
 class MollifierCutoff(_Cutoff):
@@ -48,4 +57,4 @@ class MollifierCutoff(_Cutoff):
         self.eps = eps
 
     def forward(self, input: Tensor) -> Tensor:
-        return mollifier_cutoff(self._unit(input), eps=self.eps)
+        return self._apply_envelope(input, _radial.MOLLIFIER, self.eps, lambda r: mollifier_cutoff(self._unit(r), eps=self.eps))

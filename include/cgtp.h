@@ -367,6 +367,27 @@ int64_t cgtp_uv_grad_w_workspace_bytes(int cfg, int64_t n_rows, int32_t cin, int
 int cgtp_uv_grad_w(int cfg, const void* x, const void* y, const void* g, void* gw, void* workspace, int64_t n_rows,
                    int32_t cin, int32_t cout, int32_t dtype, const float* path_scale, void* stream);
 
+/* ---- radial basis and cutoff envelopes ---------------------------------------------------------------------------
+ *
+ * Element-wise functions of the edge length r (n values), fp32 / fp64, one launch forward and one for the gradient.
+ * The reference writes them as tensor expressions: BesselBasis.forward (equitorch/nn/radials.py:46-58) and
+ * radial_standarize / polynomial_cutoff / cosine_cutoff / mollifier_cutoff (equitorch/nn/functional/cutoffs.py:4-25,
+ * :30-49, :52-64, :67-80) behind the cutoff modules (equitorch/nn/cutoffs.py:7-131).
+ *
+ *   cgtp_bessel:       out[i, k] = (2 / r_max) * sin(freq[k] * r[i] / r_max) / r[i]          out (n, num_basis)
+ *   cgtp_bessel_grad:  gr[i] = sum_k g[i, k] * d out[i, k] / d r[i]                             (NULL: not wanted)
+ *                      gfreq_rows[i, k] = g[i, k] * d out[i, k] / d freq[k]                     (NULL: not wanted;
+ *                      the caller sums it over i: the gradient of trainable frequencies)
+ *   cgtp_cutoff:       u = clamp((r - r_min) / range, 0, 1);  kind 0: polynomial envelope of order param,
+ *                      1: cosine, 2: mollifier with eps = param.  g == NULL: out[i] = envelope(u);
+ *                      else out[i] = g[i] * d envelope / d r[i] (zero where the clamp is active). */
+int cgtp_bessel(const void* r, const void* freq, void* out, int64_t n, int32_t num_basis, double r_max, int32_t dtype,
+                void* stream);
+int cgtp_bessel_grad(const void* r, const void* freq, const void* g, void* gr, void* gfreq_rows, int64_t n,
+                     int32_t num_basis, double r_max, int32_t dtype, void* stream);
+int cgtp_cutoff(int kind, const void* r, const void* g, void* out, int64_t n, double r_min, double range, double param,
+                int32_t dtype, void* stream);
+
 /* ---- fully connected products in fp32 / fp64 on the matrix cores, any table --------------------------------------
  *
  *   out[n, M, w] = sum_{segments s = (p, M)} sum_k inter_s[n, k] * W[p, k, w]
