@@ -6,6 +6,7 @@ import pytest
 import torch
 
 from helpers import assert_close
+from oracle import ref_ops
 
 pytestmark = pytest.mark.gpu
 
@@ -200,3 +201,36 @@ def test_baseline_configurations_take_their_kernels(device, monkeypatch):
     w = (torch.randn(mod.num_paths, 128, 128, generator=g) / 40).to(device).bfloat16()
     mod(x, y, w)
     assert seen[-1] == ("tensor_product_u1v", "matrix-core kernel (compiled table)"), seen
+
+
+@pytest.mark.parametrize("irreps", [("2e+0e", "0e", "0e"), ("0e+1o+2e", "0e+1e+2e", "1o"), ("0e+1o+2e", "0e+1e+2e", "0e")])
+def test_output_irreps_that_no_path_reaches_follow_the_reference_tables(device, irreps):
+    """The reference numbers the rows of its second-stage table ``info_M_fwd`` by their rank among the output rows
+    that some path reaches (``equitorch/utils/_structs.py:228-231``: the batch index of ``extract_batch_segments``, not
+    the row it stands for), and every product Function takes its output rows from that table
+    (``nn/functional/linears.py:24-25, :262-263``, ``tensor_products.py:17-18, :100-101``).  When an output irrep that
+    no path reaches precedes one that is reached — ``0e x 0e -> 2e+0e`` — the reference therefore writes the result
+    into the first rows of the output and leaves the last ones zero.  The tables of this package are the reference's
+    bit for bit, so the kernels do the same: the product here must equal the reference's algorithm on the reference's
+    tables (the CPU oracle), which differs from the dense contraction with the Clebsch-Gordan tensor in exactly the
+    rows that moved."""
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.nn import SO3Linear
+    from oracle import ref_tables
+    io, i1, i2 = irreps
+    c, n = 8, 33
+    fwd = ref_ops.tables_to_torch(ref_tables.tp_infos(io, i1, i2)[0], torch.float64)
+    g = torch.Generator().manual_seed(5)
+    d1, d2, do = Irreps(i1).dim, Irreps(i2).dim, Irreps(io).dim
+    x = torch.randn(n, d1, c, generator=g, dtype=torch.float64)
+    y = torch.randn(n, d2, generator=g, dtype=torch.float64)
+    for mode, oracle in (("uu", ref_ops.cpu_u1u_forward), ("uv", ref_ops.cpu_u1v_forward)):
+        mod = SO3Linear(i1, i2, io, c, c, internal_weights=False, feature_mode=mode).to(device)
+        w = torch.randn(*((mod.num_paths, c) if mode == "uu" else (mod.num_paths, c, c)), generator=g, dtype=torch.float64)
+        out = mod(x.float().to(device), y.float().to(device), w.float().to(device))
+        ref, _ = oracle(x, y, w, fwd)
+        assert out.shape == (n, do, c)
+        assert_close(out, ref, 1e-5, f"{mode} {i1} x {i2} -> {io}: the reference's algorithm on its tables", norm="max")
+        T = ref_ops.dense_coupling(io, i1, i2, **({"channel_scale": c ** -0.5} if mode == "uv" else {})).double()
+        dense = (ref_ops.dense_u1u if mode == "uu" else ref_ops.dense_u1v)(T, x, y, w)
+        assert float((dense - ref).abs().max()) > 0.1, "the dense contraction places these rows elsewhere"
