@@ -103,7 +103,9 @@ def tables_to_torch(info: dict, float_dtype=torch.float32) -> dict:
         if isinstance(v, dict):
             out[k] = tables_to_torch(v, float_dtype)
         elif isinstance(v, list):
-            out[k] = torch.tensor(v, dtype=float_dtype if k == "scale" else torch.int64)
+            # coefficient lists ("scale" of the product tables, "scale_MM0" / "scales_ii0" of the channel-mixing tables)
+            # are floating point, everything else an index
+            out[k] = torch.tensor(v, dtype=float_dtype if k.startswith("scale") else torch.int64)
         else:
             out[k] = v
     return out
