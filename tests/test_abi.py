@@ -367,6 +367,27 @@ def test_radial_mode_validates_on_the_host():
     assert L.cgtp_uvu_radial_grad(p16, p16, p16, p16, p16, p16, 100, 16, 11, _lib.F64, None) == 4
 
 
+def test_radial_basis_and_cutoff_entry_points_validate_on_the_host():
+    """``cgtp_bessel`` / ``cgtp_bessel_grad`` / ``cgtp_cutoff``: argument checks return before any launch."""
+    from equitorch_amd import _lib
+    L = _lib.lib
+    p = 4096
+    assert L.cgtp_bessel(p, p, p, 0, 8, 4.0, _lib.F32, None) == 0                 # nothing to do
+    assert L.cgtp_bessel(None, p, p, 10, 8, 4.0, _lib.F32, None) == 1             # null
+    assert L.cgtp_bessel(p, None, p, 10, 8, 4.0, _lib.F64, None) == 1
+    assert L.cgtp_bessel(p, p, p, 10, 8, 4.0, _lib.BF16, None) == 4               # dtype
+    assert L.cgtp_bessel(p, p, p, 10, 0, 4.0, _lib.F32, None) == 2                # no basis functions
+    assert L.cgtp_bessel(p, p, p, 10, 8, 0.0, _lib.F32, None) == 2                # r_max
+    assert L.cgtp_bessel(p, p, p, -1, 8, 4.0, _lib.F32, None) == 2
+    assert L.cgtp_bessel_grad(p, p, p, None, None, 10, 8, 4.0, _lib.F32, None) == 0   # no gradient wanted
+    assert L.cgtp_bessel_grad(p, p, None, p, None, 10, 8, 4.0, _lib.F32, None) == 1
+    assert L.cgtp_cutoff(0, p, None, p, 0, 0.0, 4.0, 6.0, _lib.F64, None) == 0
+    assert L.cgtp_cutoff(3, p, None, p, 10, 0.0, 4.0, 6.0, _lib.F32, None) == 2   # kind
+    assert L.cgtp_cutoff(1, p, None, p, 10, 0.0, 0.0, 0.0, _lib.F32, None) == 2   # empty interval
+    assert L.cgtp_cutoff(1, p, None, None, 10, 0.0, 4.0, 0.0, _lib.F32, None) == 1
+    assert L.cgtp_cutoff(2, p, None, p, 10, 0.0, 4.0, 1e-7, _lib.F16, None) == 4
+
+
 def test_torch_extension_loads_and_matches_the_library():
     """The PyTorch C++ extension over the C ABI imports without a GPU, was built against this libcgtp (ABI version),
     and takes a plan's index tensors as they are."""
