@@ -35,6 +35,7 @@ namespace cgtp {
 namespace UVT_NS {
 
 typedef real realx4 __attribute__((ext_vector_type(4)));
+typedef real realx2 __attribute__((ext_vector_type(2)));
 #ifdef CGTP_UVT_F64
 constexpr int kDtype = CGTP_F64;
 #else
@@ -396,10 +397,12 @@ constexpr int kGwStep = 8;     // samples per step (two matrix instructions deep
 // consecutive channels: one 16-byte LDS read per operand and step.
 // NARROW (few output channels): the block is 256 (k) x 64 (w), the four wavefronts split k four ways and share the
 // w columns, a thread loads and mixes two samples of its four k channels per step; with 128 columns for 32 or 64
-// output channels most of the matrix instructions would multiply zeros.
-template <bool YC, bool NARROW>
+// output channels most of the matrix instructions would multiply zeros.  NARROW = 2 (at most 32 output channels):
+// 256 (k) x 32 (w), two w tiles per wavefront, column r of tile j is output channel 2 r + j.
+template <bool YC, int NARROW>
 __global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : NARROW ? 2 : 3) uvt_grad_w_kernel(const UvtGwDev a) {
-  constexpr int KT = NARROW ? 256 : 128, WT = NARROW ? 64 : 128, NA = NARROW ? 2 : 1;
+  constexpr int KT = NARROW ? 256 : 128, WT = NARROW == 2 ? 32 : NARROW ? 64 : 128, NA = NARROW ? 2 : 1;
+  constexpr int TW = NARROW == 2 ? 2 : kGwT;      // w tiles per wavefront
   __shared__ __attribute__((aligned(16))) real lds_a[2][kGwStep][KT + 4];   // rows 4 banks apart
   __shared__ __attribute__((aligned(16))) real lds_b[2][kGwStep][WT + 4];
   const int tid = threadIdx.x;
@@ -413,8 +416,9 @@ __global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : NARROW ? 2 : 3) u
   // loading role: channels lq .. lq + 3 of the block's k range for sample ls (and ls + 4 if NARROW), channels
   // lqb .. lqb + 3 of its w range for sample lsb (NARROW: the first 128 threads only)
   const int ls = NARROW ? tid >> 6 : 2 * wave + (lane >> 5), lq = NARROW ? 4 * (tid & 63) : 4 * (lane & 31);
-  const int lsb = NARROW ? (tid >> 4) & 7 : ls, lqb = NARROW ? 4 * (tid & 15) : lq;
-  const bool b_thread = !NARROW || tid < 128;
+  const int lsb = NARROW == 2 ? (tid >> 3) & 7 : NARROW ? (tid >> 4) & 7 : ls;
+  const int lqb = NARROW == 2 ? 4 * (tid & 7) : NARROW ? 4 * (tid & 15) : lq;
+  const bool b_thread = !NARROW || tid < (NARROW == 2 ? 64 : 128);
   // K and cout are multiples of 4 (checked by the launcher), so a lane's four channels are all inside or all outside
   const bool kok = kgrp * KT + lq < a.K, wok = b_thread && wgrp * WT + lqb < a.cout;
   const int kc = kok ? kgrp * KT + lq : 0, wc = wok ? wgrp * WT + lqb : 0;
@@ -426,11 +430,11 @@ __global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : NARROW ? 2 : 3) u
   // multiplying role: channels kh * 64 .. + 63 by output channels wh * 64 .. + 63
   const int kh = NARROW ? wave : wave & 1, wh = NARROW ? 0 : wave >> 1;
 
-  realx4 acc[kGwT][kGwT];
+  realx4 acc[kGwT][TW];
 #pragma unroll
   for (int i = 0; i < kGwT; ++i)
 #pragma unroll
-    for (int j = 0; j < kGwT; ++j) acc[i][j] = realx4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < TW; ++j) acc[i][j] = realx4{0.f, 0.f, 0.f, 0.f};
 
   const int s_begin = a.path_ptr[p], s_end = a.path_ptr[p + 1];
   const int steps = (int)((n_end - n_begin + kGwStep - 1) / kGwStep);
@@ -507,18 +511,25 @@ __global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : NARROW ? 2 : 3) u
     __syncthreads();
     for (int i = 0; i < total; ++i) {
       const int buf = i & 1;
-      realx4 af[2], bf[2];
+      realx4 af[2];
+      real bf[2][TW];
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
         af[ks] = *reinterpret_cast<const realx4*>(&lds_a[buf][4 * ks + g4][kh * 64 + 4 * r]);
-        bf[ks] = *reinterpret_cast<const realx4*>(&lds_b[buf][4 * ks + g4][wh * 64 + 4 * r]);
+        if constexpr (TW == 4) {
+          const realx4 b = *reinterpret_cast<const realx4*>(&lds_b[buf][4 * ks + g4][wh * 64 + 4 * r]);
+          bf[ks][0] = b[0]; bf[ks][1] = b[1]; bf[ks][2] = b[2]; bf[ks][3] = b[3];
+        } else {
+          const realx2 b = *reinterpret_cast<const realx2*>(&lds_b[buf][4 * ks + g4][2 * r]);
+          bf[ks][0] = b[0]; bf[ks][1] = b[1];
+        }
       }
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
         for (int ti = 0; ti < kGwT; ++ti)
 #pragma unroll
-          for (int tj = 0; tj < kGwT; ++tj)
+          for (int tj = 0; tj < TW; ++tj)
             acc[ti][tj] = mfma16(af[ks][ti], bf[ks][tj], acc[ti][tj], 0, 0, 0);
       if (i + 1 < total) commit(buf ^ 1);
       if (i + 2 < total) issue();
@@ -529,7 +540,7 @@ __global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : NARROW ? 2 : 3) u
   // 4 q + i of the wavefront's 64, column r is output channel 4 r + j
   real* out = a.part + ((int64_t)blockIdx.x * a.n_paths + p) * a.K * a.cout;
   const int kbase = kgrp * KT + kh * 64;
-  const int w0 = wgrp * WT + wh * 64 + 4 * r;
+  const int w0 = wgrp * WT + wh * 64 + TW * r;
   if (w0 < a.cout) {
 #pragma unroll
     for (int i = 0; i < kGwT; ++i)
@@ -537,10 +548,15 @@ __global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : NARROW ? 2 : 3) u
       for (int e = 0; e < 4; ++e) {
         const int k = kbase + 4 * acc_row(g4, e) + i;
         if (k < a.K) {
-          realx4 v;
+          if constexpr (TW == 4) {
+            realx4 v;
 #pragma unroll
-          for (int j = 0; j < kGwT; ++j) v[j] = acc[i][j][e];
-          *reinterpret_cast<realx4*>(out + (int64_t)k * a.cout + w0) = v;
+            for (int j = 0; j < 4; ++j) v[j] = acc[i][j][e];
+            *reinterpret_cast<realx4*>(out + (int64_t)k * a.cout + w0) = v;
+          } else {
+            const realx2 v = {acc[i][0][e], acc[i][1][e]};
+            *reinterpret_cast<realx2*>(out + (int64_t)k * a.cout + w0) = v;
+          }
         }
       }
   }
@@ -579,11 +595,13 @@ uvt_gw_reduce_kernel(const real* __restrict__ part, real* __restrict__ gw, int64
 
 // few output channels and a long contracted axis: 256 x 64 blocks (single precision; in double precision the second
 // set of operands in flight does not fit the registers)
-static bool uvt_gw_narrow(int64_t K, int32_t cout) { return sizeof(real) == 4 && cout <= 64 && K >= 256; }
+static int uvt_gw_narrow(int64_t K, int32_t cout) {
+  return sizeof(real) == 4 && cout <= 64 && K >= 256 ? (cout <= 32 ? 2 : 1) : 0;
+}
 
 static int64_t uvt_gw_blocks(int64_t K, int32_t cout) {
-  const bool narrow = uvt_gw_narrow(K, cout);
-  const int64_t kt = narrow ? 256 : 128, wt = narrow ? 64 : 128;
+  const int narrow = uvt_gw_narrow(K, cout);
+  const int64_t kt = narrow ? 256 : 128, wt = narrow == 2 ? 32 : narrow ? 64 : 128;
   return ((K + kt - 1) / kt) * ((cout + wt - 1) / wt);
 }
 
@@ -955,13 +973,14 @@ int grad_w(const cgtp_uvt_gw_args* a, void* stream) {
   d.cout = a->cout; d.K = (int)K;
   d.chunk = (int)uvt_gw_chunk(a->n_rows, a->n_paths, K, a->cout);
   const int64_t n_chunks = (a->n_rows + d.chunk - 1) / d.chunk;
-  const bool narrow = uvt_gw_narrow(K, a->cout);
+  const int narrow = uvt_gw_narrow(K, a->cout);
   const int64_t zblocks = uvt_gw_blocks(K, a->cout);
   if (zblocks > 65535 || a->n_paths > 65535) return CGTP_ERR_SHAPE;
   dim3 grid((unsigned)n_chunks, (unsigned)a->n_paths, (unsigned)zblocks);
-  void (*fn)(const UvtGwDev) = a->cy > 0 ? uvt_grad_w_kernel<true, false> : uvt_grad_w_kernel<false, false>;
+  void (*fn)(const UvtGwDev) = a->cy > 0 ? uvt_grad_w_kernel<true, 0> : uvt_grad_w_kernel<false, 0>;
 #ifndef CGTP_UVT_F64
-  if (narrow) fn = a->cy > 0 ? uvt_grad_w_kernel<true, true> : uvt_grad_w_kernel<false, true>;
+  if (narrow == 1) fn = a->cy > 0 ? uvt_grad_w_kernel<true, 1> : uvt_grad_w_kernel<false, 1>;
+  if (narrow == 2) fn = a->cy > 0 ? uvt_grad_w_kernel<true, 2> : uvt_grad_w_kernel<false, 2>;
 #endif
   hipLaunchKernelGGL(fn, grid, dim3(256), 0, st, d);
   if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;

@@ -108,6 +108,8 @@ UVW_CASES = [  # irreps, (U, V, W), N
     ((_sh(2), _sh(2), "0e+1o"), (32, 32, 8), 301),
     ((_sh(2),) * 3, (32, 32, 32), 129),
     ((_sh(2),) * 3, (16, 4, 64), 1000),
+    ((_sh(1), _sh(2), _sh(1)), (32, 8, 20), 700),      # weight gradient in 256 x 32 blocks, 20 of the 32 columns used
+    ((_sh(1), _sh(2), _sh(1)), (32, 16, 48), 515),     # 256 x 64 blocks
     (("0e+1e+2e+3e", "0e+1e+2e", "0e+1e+2e"), (16, 16, 16), 256),   # the reference's comparison-test shape
 ]
 
