@@ -197,10 +197,11 @@ __device__ __forceinline__ realx4 uvt_mix_block(const UvtTerms<YC>& T, int j, co
   int2 o = make_int2(0, 0);
   if constexpr (YC) o = lut[j * 4];
 #pragma unroll
-  for (int half = 0; half < kUvtTerms; half += 4) {
-    if (half == 0 || T.n > half) {      // wave-uniform; guards accumulation into one local only
+  for (int half = 0; half < kUvtTerms; half += 2) {
+    if (half == 0 || T.n > half) {      // wave-uniform; guards accumulation into one local only.  Pairs of slots: most
+                                        // segments of the tables up to lmax = 3 have one or two terms
 #pragma unroll
-      for (int k = half; k < half + 4; ++k) {
+      for (int k = half; k < half + 2; ++k) {
         if constexpr (YC) {
           bf += (T.s[k] * T.xr[k][o.x]) * *reinterpret_cast<const realx4*>(T.yr[k] + o.y);
         } else {
@@ -443,6 +444,7 @@ __global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : NARROW ? 2 : 3) u
   // state of the loads in flight: the segment's terms in scalar registers (at most kUvtTerms per item: the caller
   // splits longer segments; slots past the end repeat the first term's rows with coefficient zero)
   int ld_item = s_begin - 1, ld_step = steps;
+  int n_slots = 0;              // the item's term count rounded up to a pair: pairs of slots past it are skipped
   int xrow[kUvtTerms], yrow[kUvtTerms], grow = 0;
   real c[kUvtTerms];
   realx4 v4[NA][kUvtTerms];     // y without channels: four channels of x; with: four channels of y
@@ -456,6 +458,7 @@ __global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : NARROW ? 2 : 3) u
       ++ld_item;
       const cgtp_uvt_item it = a.items[ld_item];
       const int n_t = it.t1 - it.t0;
+      n_slots = __builtin_amdgcn_readfirstlane((n_t + 1) & ~1);
 #pragma unroll
       for (int k = 0; k < kUvtTerms; ++k) {
         const int t = k < n_t ? it.t0 + k : it.t0;
@@ -479,13 +482,18 @@ __global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : NARROW ? 2 : 3) u
       const real* xn = a.x + nc * a.dx * a.cx + xo;
       const real* yn = a.y + nc * a.dy * (YC ? a.cy : 1) + yo;
 #pragma unroll
-      for (int k = 0; k < kUvtTerms; ++k) {
-        if constexpr (YC) {
-          v1[j][k] = xn[xrow[k]];
-          v4[j][k] = *reinterpret_cast<const realx4*>(yn + yrow[k]);
-        } else {
-          v4[j][k] = *reinterpret_cast<const realx4*>(xn + xrow[k]);
-          v1[j][k] = yn[yrow[k]];
+      for (int h = 0; h < kUvtTerms; h += 2) {
+        if (h < n_slots) {            // the same in every lane: a scalar branch
+#pragma unroll
+          for (int k = h; k < h + 2; ++k) {
+            if constexpr (YC) {
+              v1[j][k] = xn[xrow[k]];
+              v4[j][k] = *reinterpret_cast<const realx4*>(yn + yrow[k]);
+            } else {
+              v4[j][k] = *reinterpret_cast<const realx4*>(xn + xrow[k]);
+              v1[j][k] = yn[yrow[k]];
+            }
+          }
         }
       }
     }
@@ -498,7 +506,12 @@ __global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : NARROW ? 2 : 3) u
     for (int j = 0; j < NA; ++j) {
       realx4 av = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int k = 0; k < kUvtTerms; ++k) av += (c[k] * v1[j][k]) * v4[j][k];
+      for (int h = 0; h < kUvtTerms; h += 2) {
+        if (h < n_slots) {            // slots of the loads in flight: commit runs before the next issue
+          av += (c[h] * v1[j][h]) * v4[j][h];
+          av += (c[h + 1] * v1[j][h + 1]) * v4[j][h + 1];
+        }
+      }
       *reinterpret_cast<realx4*>(&lds_a[buf][ls + 4 * j][lq]) = (ld_live[j] && kok) ? av : zero;
     }
     if (b_thread) *reinterpret_cast<realx4*>(&lds_b[buf][lsb][lqb]) = (ldb_live && wok) ? bv4 : zero;
