@@ -741,17 +741,16 @@ __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGy
       wok[wb] = w < a.cout;
       wcol[wb] = wok[wb] ? w : 0;
     }
-    // rows of g of the terms, requested before the matrix instructions; the second half only for long segments
+    // rows of g of the terms, requested before the matrix instructions: slots in pairs up to the segment's term count
     realx4 gv[kUvtTerms][kGyWB];
 #pragma unroll
-    for (int k = 0; k < kUvtTerms / 2; ++k)
+    for (int h = 0; h < kUvtTerms; h += 2) {
+      if (h == 0 || n_t > h) {
 #pragma unroll
-      for (int wb = 0; wb < kGyWB; ++wb) gv[k][wb] = *reinterpret_cast<const realx4*>(gn + mrow[k] + wcol[wb]);
-    if (n_t > kUvtTerms / 2) {
+        for (int k = h; k < h + 2; ++k)
 #pragma unroll
-      for (int k = kUvtTerms / 2; k < kUvtTerms; ++k)
-#pragma unroll
-        for (int wb = 0; wb < kGyWB; ++wb) gv[k][wb] = *reinterpret_cast<const realx4*>(gn + mrow[k] + wcol[wb]);
+          for (int wb = 0; wb < kGyWB; ++wb) gv[k][wb] = *reinterpret_cast<const realx4*>(gn + mrow[k] + wcol[wb]);
+      }
     }
 
     realx4 acc[kGyWB];
