@@ -575,6 +575,102 @@ __global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : NARROW ? 2 : 3) u
   }
 }
 
+// Weights of at most 64 x 64 (K <= 64 and at most 64 output channels — the channel mixing of 64-channel models): one
+// block, and the block of the kernel above would be three quarters zeros.  Here a wavefront owns the whole block and a
+// chunk of samples by itself: the operands' layout in memory is the matrix instructions' own (lane (r, g) holds the
+// four channels 4 r .. 4 r + 3 of sample g of four: one 16-byte load, element i = tile i), so nothing is exchanged
+// through LDS and there is no barrier; two steps of eight samples are loaded before the first is multiplied, and
+// several wavefronts per SIMD cover each other's load latency.
+template <bool YC>
+__global__ void __launch_bounds__(kWave) uvt_grad_w_small_kernel(const UvtGwDev a) {
+  const int lane = threadIdx.x, r = lane & 15, g4 = lane >> 4;
+  const int p = blockIdx.y;
+  const int64_t n_begin = (int64_t)blockIdx.x * a.chunk;
+  const int64_t n_end = n_begin + a.chunk < a.n_rows ? n_begin + a.chunk : a.n_rows;
+  const bool kok = 4 * r < a.K, wok = 4 * r < a.cout;
+  const int kc = kok ? 4 * r : 0, wc = wok ? 4 * r : 0;
+  int xo = kc, yo = 0;
+  if constexpr (YC) {
+    xo = kc / a.cy;
+    yo = kc - xo * a.cy;
+  }
+  realx4 acc[kGwT][kGwT];
+#pragma unroll
+  for (int i = 0; i < kGwT; ++i)
+#pragma unroll
+    for (int j = 0; j < kGwT; ++j) acc[i][j] = realx4{0.f, 0.f, 0.f, 0.f};
+  constexpr int NS = 4;          // groups of four samples in flight: two steps of eight
+  const realx4 zero = {0.f, 0.f, 0.f, 0.f};
+  for (int s = a.path_ptr[p]; s < a.path_ptr[p + 1]; ++s) {
+    const cgtp_uvt_item it = a.items[s];
+    const int n_t = __builtin_amdgcn_readfirstlane(it.t1 - it.t0);
+    const int grow = __builtin_amdgcn_readfirstlane(it.out_row) * a.cout;
+    for (int64_t n0 = n_begin; n0 < n_end; n0 += 4 * NS) {
+      realx4 av[NS], bv[NS];
+      const real* xn[NS];
+      const real* yn[NS];
+      bool live[NS];
+#pragma unroll
+      for (int q = 0; q < NS; ++q) {
+        const int64_t n = n0 + 4 * q + g4;
+        live[q] = n < n_end;
+        const int64_t nc = live[q] ? n : n_end - 1;
+        xn[q] = a.x + nc * a.dx * a.cx + xo;
+        yn[q] = a.y + nc * a.dy * (YC ? a.cy : 1) + yo;
+        bv[q] = *reinterpret_cast<const realx4*>(a.g + nc * a.dg * a.cout + grow + wc);
+        av[q] = zero;
+      }
+      for (int t0 = 0; t0 < n_t; t0 += 2) {          // the segment's terms, two at a time (most have one or two)
+        const bool two = t0 + 1 < n_t;
+        const int ta0 = a.ta[it.t0 + t0] * a.cx, tb0 = a.tb[it.t0 + t0] * (YC ? a.cy : 1);
+        const int ta1 = a.ta[it.t0 + (two ? t0 + 1 : t0)] * a.cx, tb1 = a.tb[it.t0 + (two ? t0 + 1 : t0)] * (YC ? a.cy : 1);
+        const real c0 = a.tc[it.t0 + t0], c1 = two ? a.tc[it.t0 + t0 + 1] : real(0);
+        realx4 v4[NS][2];
+        real v1[NS][2];
+#pragma unroll
+        for (int q = 0; q < NS; ++q) {
+          if constexpr (YC) {
+            v1[q][0] = xn[q][ta0]; v4[q][0] = *reinterpret_cast<const realx4*>(yn[q] + tb0);
+            v1[q][1] = xn[q][ta1]; v4[q][1] = *reinterpret_cast<const realx4*>(yn[q] + tb1);
+          } else {
+            v4[q][0] = *reinterpret_cast<const realx4*>(xn[q] + ta0); v1[q][0] = yn[q][tb0];
+            v4[q][1] = *reinterpret_cast<const realx4*>(xn[q] + ta1); v1[q][1] = yn[q][tb1];
+          }
+        }
+#pragma unroll
+        for (int q = 0; q < NS; ++q) {
+          av[q] += (c0 * v1[q][0]) * v4[q][0];
+          av[q] += (c1 * v1[q][1]) * v4[q][1];
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < NS; ++q) {
+        const realx4 af = (live[q] && kok) ? av[q] : zero;
+        const realx4 bf = (live[q] && wok) ? bv[q] : zero;
+#pragma unroll
+        for (int ti = 0; ti < kGwT; ++ti)
+#pragma unroll
+          for (int tj = 0; tj < kGwT; ++tj) acc[ti][tj] = mfma16(af[ti], bf[tj], acc[ti][tj], 0, 0, 0);
+      }
+    }
+  }
+  real* out = a.part + ((int64_t)blockIdx.x * a.n_paths + p) * a.K * a.cout;
+  if (wok) {
+#pragma unroll
+    for (int i = 0; i < kGwT; ++i)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int k = 4 * acc_row(g4, e) + i;
+        if (k < a.K) {
+          realx4 v;
+#pragma unroll
+          for (int j = 0; j < kGwT; ++j) v[j] = acc[i][j][e];
+          *reinterpret_cast<realx4*>(out + (int64_t)k * a.cout + 4 * r) = v;
+        }
+      }
+  }
+}
+
 // gw[i] = sum over the chunks c of part[c * n + i], in a fixed order: a thread owns four consecutive elements (n is a
 // multiple of 4) and every fourth chunk, four loads in flight; the four slices of a column are added in slice order.
 // (One thread per element walking all chunks one after the other took 33 us for 128 chunks of 12 288 elements: 128
@@ -618,7 +714,18 @@ static int64_t uvt_gw_blocks(int64_t K, int32_t cout) {
   return ((K + kt - 1) / kt) * ((cout + wt - 1) / wt);
 }
 
+// one wavefront per (path, chunk of samples) with the whole weight block in its registers
+static bool uvt_gw_small(int64_t K, int32_t cout) { return sizeof(real) == 4 && K <= 64 && cout <= 64; }   // doubles: 312 registers
+
 static int64_t uvt_gw_chunk(int64_t n_rows, int32_t n_paths, int64_t K, int32_t cout) {
+  if (uvt_gw_small(K, cout)) {
+    // wavefronts, not workgroups of four: chunks of 32 samples or more, at most 8192 wavefronts and 512 partial
+    // results (three paths over 65 536 samples: 641 us for the layer's step with at most 128, 442 with 512, 492 with
+    // 2048 — the partial results are 16 KB each and the reduction reads them all)
+    int64_t chunk = 32;
+    while ((n_rows + chunk - 1) / chunk > 512 || ((n_rows + chunk - 1) / chunk) * n_paths > 8192) chunk *= 2;
+    return chunk;
+  }
   // samples per workgroup: at most 128 partial results; 256 samples, fewer (down to 32: four steps) while the launch
   // would have less than three workgroups per compute unit — a node-level layer has a few thousand samples and a
   // handful of paths, and with 256 samples per workgroup its 48 workgroups took 100 us for 0.3 GFLOP
@@ -989,6 +1096,15 @@ int grad_w(const cgtp_uvt_gw_args* a, void* stream) {
   const int64_t zblocks = uvt_gw_blocks(K, a->cout);
   if (zblocks > 65535 || a->n_paths > 65535) return CGTP_ERR_SHAPE;
   dim3 grid((unsigned)n_chunks, (unsigned)a->n_paths, (unsigned)zblocks);
+  if (uvt_gw_small(K, a->cout)) {
+    hipLaunchKernelGGL(a->cy > 0 ? uvt_grad_w_small_kernel<true> : uvt_grad_w_small_kernel<false>,
+                       dim3((unsigned)n_chunks, (unsigned)a->n_paths), dim3(kWave), 0, st, d);
+    if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
+    hipLaunchKernelGGL(uvt_gw_reduce_kernel, dim3((unsigned)((n_out / 4 + kGwReduceCols - 1) / kGwReduceCols)),
+                       dim3(kGwReduceCols * kGwReduceSlices), 0, st, (const real*)a->workspace, (real*)a->gw, n_chunks,
+                       n_out / 4);
+    return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
+  }
   void (*fn)(const UvtGwDev) = a->cy > 0 ? uvt_grad_w_kernel<true, 0> : uvt_grad_w_kernel<false, 0>;
 #ifndef CGTP_UVT_F64
   if (narrow == 1) fn = a->cy > 0 ? uvt_grad_w_kernel<true, 1> : uvt_grad_w_kernel<false, 1>;

@@ -305,6 +305,12 @@ def test_table_driven_matrix_core_entry_points_validate_on_the_host():
     assert L.cgtp_uvt_grad_w_workspace_bytes(32768, 23, 128, 128, _lib.F32) == 128 * 23 * 128 * 128 * 4
     assert L.cgtp_uvt_grad_w_workspace_bytes(300, 4, 32, 16, _lib.F64) == 10 * 4 * 32 * 16 * 8
     assert L.cgtp_uvt_grad_w_workspace_bytes(8192, 23, 128, 128, _lib.F32) == 64 * 23 * 128 * 128 * 4
+    # single precision weights of at most 64 x 64: one wavefront per (path, chunk), chunks of 32 samples or more, at
+    # most 512 chunks and 8192 wavefronts
+    assert L.cgtp_uvt_grad_w_workspace_bytes(4096, 3, 64, 64, _lib.F32) == 128 * 3 * 64 * 64 * 4
+    assert L.cgtp_uvt_grad_w_workspace_bytes(65536, 3, 64, 64, _lib.F32) == 512 * 3 * 64 * 64 * 4
+    assert L.cgtp_uvt_grad_w_workspace_bytes(4096, 100, 32, 48, _lib.F32) == 64 * 100 * 32 * 48 * 4
+    assert L.cgtp_uvt_grad_w_workspace_bytes(4096, 3, 64, 64, _lib.F64) == 128 * 3 * 64 * 64 * 8
     g = _lib.UvtGwArgs()
     g.dtype = _lib.F32
     g.n_rows, g.n_paths, g.dx, g.dy, g.dg, g.cx, g.cy, g.cout = 10, 4, 9, 9, 9, 32, 0, 30

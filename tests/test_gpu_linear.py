@@ -125,6 +125,30 @@ def test_bf16_shared_weight_runs_on_the_matrix_core_kernels(device, irr, cin, co
         assert_close(a.float(), b, tol=1e-2, what=f"bf16 {irr} {name}")
 
 
+@pytest.mark.parametrize("cin,cout,n", [(64, 64, 20003), (48, 24, 1001), (16, 64, 70001), (64, 8, 31)])
+def test_weight_gradient_of_weights_up_to_64_by_64(device, cin, cout, n):
+    """fp32 shared weights of at most 64 x 64: the weight gradient has a wavefront per (path, chunk of samples) that keeps
+    the whole block in its registers.  Sample counts that leave a ragged last chunk (and a last group of fewer than
+    four samples) and that make the chunks 32, 64 and 256 samples long; sums over up to 70 001 samples in fp32 are
+    compared norm-wise, with the fp32 restatement beside them."""
+    from equitorch_amd.nn import IrrepsLinear
+    io, ii = "0e+1o+2e", "0e+1o+1o+2e"
+    mod = IrrepsLinear(ii, io, cin, cout, internal_weights=False).to(device)
+    info = ref_tables.irreps_linear_infos(io, ii)[0]
+    info["scale_MM0"] = torch.tensor(info["scale_MM0"]).double().tolist()
+    g = torch.Generator().manual_seed(n)
+    rd = lambda *s: torch.randn(*s, generator=g).double()
+    x, ct, w = rd(n, mod.irreps_in_dim, cin), rd(n, mod.irreps_out_dim, cout), rd(mod.num_paths, cin, cout)
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    ref = ref_ops.cpu_irreps_linear(xr, wr, info)
+    rgw, = _grads(ref, (wr,), ct)
+    x32, w32 = x.float(), w.float().requires_grad_(True)
+    r32, = _grads(ref_ops.cpu_irreps_linear(x32, w32, info), (w32,), ct.float())
+    xd, wd = x.to(device, torch.float32), w.to(device, torch.float32).requires_grad_(True)
+    gw, = _grads(mod(xd, wd), (wd,), ct.to(device, torch.float32))
+    assert_close(gw, rgw, tol=1e-5, what=f"grad_w {cin}->{cout} n={n}", norm="max", fp32_ref=r32)
+
+
 @pytest.mark.parametrize("dtype,cin,cout,shared", [(torch.float32, 10, 7, True), (torch.float64, 6, 9, True),
                                                     (torch.bfloat16, 24, 40, True), (torch.bfloat16, 10, 7, True),
                                                     (torch.float16, 16, 8, False)])
