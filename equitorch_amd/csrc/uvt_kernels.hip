@@ -157,7 +157,10 @@ __device__ __forceinline__ cgtp_uvt_item uvt_item_at(const UvtTables& tab, int j
 // past the end of the segment point at row 0 with a zero factor, so that the code has no branches around register
 // arrays (a conditional assignment to an array element costs the compiler a copy of the array).
 constexpr int kUvtTerms = 8;
-constexpr int kUvtKbi = 4;   // blocks of 16 k per item
+// Blocks of 16 k in the ring of weight fragments; k is padded to whole turns of it (zero weights, zero rows of the
+// staged tiles).  Four blocks cover the round trip to L2; with at most 32 contracted channels a ring of four would be
+// half padding — twice the LDS per sample and twice the matrix instructions — so those get a ring of two.
+__host__ __device__ constexpr int uvt_kbi(int64_t K) { return K <= 32 ? 2 : 4; }
 template <bool YC>
 struct UvtTerms {
   const real* xr[kUvtTerms];
@@ -231,16 +234,15 @@ __device__ __forceinline__ realx4 uvt_mix_tail(const UvtDev& a, const UvtTables&
   return bf;
 }
 
-// WB: blocks of 16 output channels per wavefront.  k is padded to whole multiples of kUvtKbi blocks of 16 (zero
+// WB: blocks of 16 output channels per wavefront.  k is padded to whole multiples of KBI blocks of 16 (zero
 // weights, zero rows), so the ring of weight fragments turns in straight-line code.
 // While the matrix instructions of block j run, the vector ALUs mix block j + 1; the weight fragments of block j + 4
 // (of the next item past the end of this one) are requested as soon as block j's are consumed.  Everything an item
 // needs besides its operands is wave-uniform (scalar registers).  A wavefront issues one instruction every four
 // cycles, a matrix instruction keeps its pipeline busy for 32: with 4 WB matrix instructions per block next to
 // about 50 vector and LDS instructions, two wavefronts per SIMD keep the matrix pipeline fed when WB >= 2.
-template <bool YC, int WB>
+template <bool YC, int WB, int KBI>
 __global__ void __launch_bounds__(kUvtMaxGroups* kWave) uvt_apply_kernel(const UvtDev a) {
-  constexpr int KBI = kUvtKbi;
   extern __shared__ __align__(16) unsigned char smem[];
   const int sb_count = 1 << a.sb_log2;
   real* xs = reinterpret_cast<real*>(smem);
@@ -765,8 +767,9 @@ struct UvtGyDev {
 
 constexpr int kGyWB = sizeof(real) == 8 ? 1 : 2;   // blocks of 16 output channels per pass (registers: doubles take two)
 constexpr int kGyWaves = 8;
-constexpr int kGyRing = 4;       // blocks of 16 k in flight (= kUvtKbi: the packing pads k to whole multiples)
+// kGyRing (template argument): blocks of 16 k in flight = uvt_kbi(K), the packing pads k to whole multiples
 
+template <int kGyRing>
 __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGyDev a) {
   extern __shared__ __align__(16) unsigned char smem[];
   real* xs = reinterpret_cast<real*>(smem);
@@ -939,7 +942,8 @@ static int uvt_shape(int64_t n_rows, int dx, int dy, int dout, int cx, int cy, i
   d.n_rows = n_rows; d.dx = dx; d.dy = dy; d.dout = dout; d.cx = cx; d.cy = cy; d.cout = cout;
   const int64_t K = yc ? (int64_t)cx * cy : cx;
   if (K > (1 << 24)) return CGTP_ERR_SHAPE;
-  d.kblocks = round_up((int)((K + 15) / 16), kUvtKbi);   // whole turns of the fragment ring: the tail is zero weights
+  const int kbi = uvt_kbi(K);
+  d.kblocks = round_up((int)((K + 15) / 16), kbi);   // whole turns of the fragment ring: the tail is zero weights
   d.kx = yc ? cx : d.kblocks * 16;
   d.px = dx * d.kx + 4;
   d.py = yc ? dy * cy + 4 : (dy | 1);
@@ -963,7 +967,7 @@ static int uvt_shape(int64_t n_rows, int dx, int dy, int dout, int cx, int cy, i
          (per_block << (sb_log2 + 1)) + fixed <= kLdsBytes / 2 - kUvtTableRoom && (blocks16 >> (sb_log2 + 1)) >= 512)
     ++sb_log2;
   d.sb_log2 = sb_log2; d.wgroups = wgroups; d.igroups = igroups;
-  plan->wb = wb; plan->kbi = kUvtKbi; plan->yc = yc;
+  plan->wb = wb; plan->kbi = kbi; plan->yc = yc;
   plan->lds = (per_block << sb_log2) + fixed;
   plan->threads = (unsigned)((wgroups * igroups) << sb_log2) * kWave;
   plan->grid = dim3((unsigned)((blocks16 + (1 << sb_log2) - 1) >> sb_log2), (unsigned)((need + wgroups - 1) / wgroups));
@@ -1000,7 +1004,7 @@ static int uvt_plan(const cgtp_uvt_args* a, UvtPlan* plan) {
 
 int64_t packed_elems(int32_t n_paths, int64_t K, int32_t cout) {
   if (n_paths < 0 || K <= 0 || cout <= 0) return 0;
-  return (int64_t)n_paths * round_up((int)((K + 15) / 16), kUvtKbi) * round_up((cout + 15) / 16, 4) * 256;
+  return (int64_t)n_paths * round_up((int)((K + 15) / 16), uvt_kbi(K)) * round_up((cout + 15) / 16, 4) * 256;
 }
 
 int pack_weights(const void* w, void* packed, int32_t n_paths, int64_t K, int32_t cout, int64_t stride_p,
@@ -1013,7 +1017,7 @@ int pack_weights(const void* w, void* packed, int32_t n_paths, int64_t K, int32_
   if (n_vec == 0) return CGTP_OK;
   hipLaunchKernelGGL(uvt_pack_kernel, dim3((unsigned)((n_vec + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
                      (const real*)w, (real*)packed, n_vec, (int)K, (int)cout,
-                     round_up((int)((K + 15) / 16), kUvtKbi), round_up((cout + 15) / 16, 4), stride_p, stride_k, stride_c);
+                     round_up((int)((K + 15) / 16), uvt_kbi(K)), round_up((cout + 15) / 16, 4), stride_p, stride_k, stride_c);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 
@@ -1040,14 +1044,25 @@ int apply(const cgtp_uvt_args* a, void* stream) {
   if (st != CGTP_OK) return st;
   if (a->n_rows == 0 || a->n_items == 0) return CGTP_OK;
   void (*fn)(const UvtDev) = nullptr;
-  if (plan.yc) {
-    fn = plan.wb == 2 ? uvt_apply_kernel<true, 2> : uvt_apply_kernel<true, 1>;
-  } else {
-    fn = plan.wb == 2 ? uvt_apply_kernel<false, 2> : uvt_apply_kernel<false, 1>;
-  }
+  if (plan.kbi == 4) {
+    if (plan.yc) {
+      fn = plan.wb == 2 ? uvt_apply_kernel<true, 2, 4> : uvt_apply_kernel<true, 1, 4>;
+    } else {
+      fn = plan.wb == 2 ? uvt_apply_kernel<false, 2, 4> : uvt_apply_kernel<false, 1, 4>;
+    }
 #ifndef CGTP_UVT_F64
-  if (plan.wb == 4) fn = plan.yc ? uvt_apply_kernel<true, 4> : uvt_apply_kernel<false, 4>;
+    if (plan.wb == 4) fn = plan.yc ? uvt_apply_kernel<true, 4, 4> : uvt_apply_kernel<false, 4, 4>;
 #endif
+  } else {
+    if (plan.yc) {
+      fn = plan.wb == 2 ? uvt_apply_kernel<true, 2, 2> : uvt_apply_kernel<true, 1, 2>;
+    } else {
+      fn = plan.wb == 2 ? uvt_apply_kernel<false, 2, 2> : uvt_apply_kernel<false, 1, 2>;
+    }
+#ifndef CGTP_UVT_F64
+    if (plan.wb == 4) fn = plan.yc ? uvt_apply_kernel<true, 4, 2> : uvt_apply_kernel<false, 4, 2>;
+#endif
+  }
   if (plan.lds > 48 * 1024 &&
       hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds) != hipSuccess)
     return CGTP_ERR_LDS;
@@ -1134,7 +1149,8 @@ int grad_y(const cgtp_uvt_gy_args* a, void* stream) {
   d.items = a->items; d.ta = a->term_m; d.tb = a->term_b; d.tc = (const real*)a->term_c;
   d.n_rows = a->n_rows; d.n_items = a->n_items; d.n_terms = a->n_terms;
   d.dx = a->dx; d.dy = a->dy; d.dg = a->dg; d.cx = a->cx; d.cout = a->cout;
-  d.kblocks = round_up((a->cx + 15) / 16, kUvtKbi);
+  const int ring = uvt_kbi(a->cx);
+  d.kblocks = round_up((a->cx + 15) / 16, ring);
   d.kx = d.kblocks * 16;
   d.px = a->dx * d.kx + 4;
   d.wbp = round_up((a->cout + 15) / 16, 4);
@@ -1144,11 +1160,10 @@ int grad_y(const cgtp_uvt_gy_args* a, void* stream) {
                       (int64_t)a->n_items * 32 + (int64_t)a->n_terms * kTermBytes + 16;
   if (lds > kLdsBytes) return CGTP_ERR_LDS;
   if (a->n_rows == 0) return CGTP_OK;
-  if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)uvt_grad_y_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                             (int)lds) != hipSuccess)
+  void (*fn)(const UvtGyDev) = ring == 4 ? uvt_grad_y_kernel<4> : uvt_grad_y_kernel<2>;
+  if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
     return CGTP_ERR_LDS;
-  hipLaunchKernelGGL(uvt_grad_y_kernel, dim3((unsigned)((a->n_rows + 15) / 16)), dim3(kGyWaves * kWave), (size_t)lds,
-                     (hipStream_t)stream, d);
+  hipLaunchKernelGGL(fn, dim3((unsigned)((a->n_rows + 15) / 16)), dim3(kGyWaves * kWave), (size_t)lds, (hipStream_t)stream, d);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 
