@@ -27,6 +27,8 @@ U1V_CASES = [  # irreps (out, in1, in2), C_in, C_out, N, module options
     (("0e+1e+2e+3e", "0e+1e+2e", "0e+1e+2e"), 16, 16, 64, {}),
     (("0e", _sh(2), _sh(2)), 32, 64, 17000, {}),                # one output row: wavefronts spent on sample blocks
     (("0e+1o", _sh(1), _sh(1)), 16, 256, 530, {}),              # output channels over two workgroups
+    ((_sh(2),) * 3, 8, 8, 515, {}),                             # a fragment ring of two blocks, half of it padding
+    ((_sh(3), _sh(2), _sh(3)), 16, 40, 333, {}),                # ... one block of k, output channels 2 blocks + 8
 ]
 
 
@@ -111,6 +113,8 @@ UVW_CASES = [  # irreps, (U, V, W), N
     ((_sh(1), _sh(2), _sh(1)), (32, 8, 20), 700),      # weight gradient in 256 x 32 blocks, 20 of the 32 columns used
     ((_sh(1), _sh(2), _sh(1)), (32, 16, 48), 515),     # 256 x 64 blocks
     (("0e+1e+2e+3e", "0e+1e+2e", "0e+1e+2e"), (16, 16, 16), 256),   # the reference's comparison-test shape
+    ((_sh(2), _sh(2), _sh(1)), (4, 8, 16), 515),       # 32 contracted channel pairs: a fragment ring of two blocks
+    ((_sh(1), _sh(1), _sh(2)), (4, 4, 8), 130),        # 16 pairs: half of that ring is padding
 ]
 
 
