@@ -6,6 +6,9 @@
 // index_select and indexed_scale_segment, equitorch/ops/indexed_scale_segment_op.py:143-170).
 #include <torch/extension.h>
 
+#include <memory>
+#include <unordered_map>
+
 // torch's ROCm build presents its HIP devices as device type "cuda": the guard and stream types that follow that
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
@@ -23,10 +26,32 @@ struct SegView {
   at::Tensor ptr, perm, seg_ids, gather, wave_seg, wave_pos;
 };
 
+// Callables (grad_out, x, y, w, need_x, need_y, need_w) -> (gx, gy, gw) that evaluate the gradients of an edge product
+// through differentiable functions, for a backward that runs with gradient mode on (a gradient of the gradient is
+// wanted).  One per EdgeHandle, looked up by number when the backward runs, dropped with the last copy of the handle.
+std::unordered_map<int64_t, py::object>& edge_fallbacks() {
+  static auto* m = new std::unordered_map<int64_t, py::object>();   // never destroyed: outlives the interpreter's teardown
+  return *m;
+}
+
 struct EdgeHandle {
   SegView fwd, bwd;
   at::Tensor path_scale;   // undefined = all ones
   int64_t cfg, d_out, y_vec;
+  int64_t fallback = -1;
+  std::shared_ptr<void> fallback_guard;
+
+  void set_fallback(py::object fn) {
+    static int64_t next = 0;
+    const int64_t id = next++;
+    edge_fallbacks()[id] = std::move(fn);
+    fallback = id;
+    fallback_guard = std::shared_ptr<void>(nullptr, [id](void*) {
+      if (!Py_IsInitialized()) return;
+      py::gil_scoped_acquire gil;
+      edge_fallbacks().erase(id);
+    });
+  }
 };
 
 const void* ptr_or_null(const at::Tensor& t) { return t.defined() ? t.data_ptr() : nullptr; }
@@ -126,7 +151,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> seg_backward(const at::Tensor& x,
   return {gx, gy, gw};
 }
 
-// The autograd node of the fused edge product.  Differentiable once, like the Python Functions it stands in for.
+// The autograd node of the fused edge product.  A backward under gradient mode hands over to the handle's callable.
 class EdgeUvu : public torch::autograd::Function<EdgeUvu> {
  public:
   static at::Tensor forward(AutogradContext* ctx, const at::Tensor& x, const at::Tensor& y, const at::Tensor& w,
@@ -136,11 +161,24 @@ class EdgeUvu : public torch::autograd::Function<EdgeUvu> {
                             h->bwd.wave_pos, h->path_scale});
     ctx->saved_data["cfg"] = h->cfg;
     ctx->saved_data["y_vec"] = h->y_vec;
+    ctx->saved_data["fallback"] = h->fallback;
     return out;
   }
 
   static variable_list backward(AutogradContext* ctx, variable_list grad_outputs) {
     const variable_list s = ctx->get_saved_variables();
+    if (at::GradMode::is_enabled()) {
+      py::gil_scoped_acquire gil;
+      const auto it = edge_fallbacks().find(ctx->saved_data["fallback"].toInt());
+      TORCH_CHECK(it != edge_fallbacks().end(),
+                  "cgtp: a gradient of higher order of an edge product was asked for after its EdgePlan was released");
+      const py::tuple r = it->second(grad_outputs[0], s[0], s[1], s[2], ctx->needs_input_grad(0),
+                                     ctx->needs_input_grad(1), ctx->needs_input_grad(2));
+      variable_list out(4);
+      for (int i = 0; i < 3; ++i)
+        if (!r[i].is_none()) out[i] = r[i].cast<at::Tensor>();
+      return out;
+    }
     const SegView bwd{s[3], s[4], s[5], s[6], s[7], s[8]};
     at::NoGradGuard no_grad;
     auto [gx, gy, gw] = seg_backward(s[0], s[1], s[2], grad_outputs[0], bwd, s[9], ctx->saved_data["cfg"].toInt(),
@@ -259,7 +297,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         h.fwd = SegView{f_ptr, opt(f_perm), f_seg_ids, f_gather, opt(f_wave_seg), opt(f_wave_pos)};
         h.bwd = SegView{b_ptr, opt(b_perm), b_seg_ids, b_gather, opt(b_wave_seg), opt(b_wave_pos)};
         return h;
-      }));
+      }))
+      .def("set_fallback", &EdgeHandle::set_fallback,
+           "callable (grad_out, x, y, w, need_x, need_y, need_w) -> (gx, gy, gw) for gradients of higher order");
   m.def("edge_uvu", &edge_uvu, "fused edge product with its autograd node: x (N, D1, C), y (E, D2 | 3), w (E, P, C) | (P, C)");
   m.def("row_uvu", [](const at::Tensor& x, const at::Tensor& y, const at::Tensor& w, c10::optional<at::Tensor> path_scale,
                       int64_t cfg, int64_t d_out, int64_t fallback) {

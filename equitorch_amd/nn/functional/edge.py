@@ -88,7 +88,34 @@ def _check_edge_operands(x: Tensor, y: Tensor, plan: EdgePlan, tp_info: TensorPr
             raise _lib.CgtpError(f"w_last must be ({h.shape[1]}, {coo.P}, {c}), got {tuple(w_last.shape)}")
 
 
-def _shim_handle(plan: EdgePlan, cfg, x: Tensor, y_vec: int):
+def _unfused(plan: EdgePlan, tp_info: TensorProductInfo, y_vec: int = 0):
+    """``expression(x, y, w)``: the same result from the three steps the fused kernels replace — gather, product on the
+    batch of edges, segment sum — each of which autograd differentiates to any order (``y``: harmonics, or edge vectors
+    when ``y_vec`` says so).  The fused kernels' backward evaluates it when a gradient of the gradient is asked for
+    (forces in the loss), as the reference's composition of differentiable functions would be.  Holds the plan's
+    tensors, not the plan."""
+    src, infos, num_nodes = plan.src, plan.scale_infos(), plan.num_nodes
+    d2 = int(kernels.coo_of(tp_info).D2)
+
+    def expression(x: Tensor, y: Tensor, w: Tensor) -> Tensor:
+        if y_vec:
+            from .sphericals import spherical_harmonics
+            y = spherical_harmonics(y, int(round(d2 ** 0.5)) - 1, normalize_input=(y_vec == kernels.Y_UNIT_VECTOR))
+        msg = tensor_product_u1u(x.index_select(0, src), y, w, tp_info)
+        e, d, c = msg.shape
+        return sparse_scale(msg.view(1, e, d * c), *infos).view(num_nodes, d, c)
+    return expression
+
+
+def _higher_order(expression, inputs, need, g: Tensor):
+    """Gradients of ``expression(*inputs)`` for the inputs ``need`` marks, themselves differentiable."""
+    with torch.enable_grad():
+        wanted = [t for t, n in zip(inputs, need) if n]
+        grads = iter(torch.autograd.grad(expression(*inputs), wanted, g, create_graph=True, allow_unused=True))
+    return tuple(next(grads) if n else None for n in need)
+
+
+def _shim_handle(plan: EdgePlan, cfg, x: Tensor, y_vec: int, tp_info: TensorProductInfo):
     """The C++ extension's handle of this plan for one compiled table, dtype and channel count (it holds the sorted
     views and the range tables of both directions), or None when the extension is not there or the table needs the
     weights rearranged (a subset of the compiled paths)."""
@@ -107,6 +134,8 @@ def _shim_handle(plan: EdgePlan, cfg, x: Tensor, y_vec: int):
             wave_seg, wave_pos = kernels.seg_ranges(cfg, seg, code, x.shape[-1], backward)
             views += [seg.ptr, seg.perm, seg.seg_ids, seg.gather, wave_seg, wave_pos]
         handles[key] = mod.EdgeHandle(int(cfg), int(kernels.uvu_dims(cfg)[2]), int(y_vec), scale, *views)
+        expression = _unfused(plan, tp_info, y_vec)
+        handles[key].set_fallback(lambda g, x_, y_, w_, *need: _higher_order(expression, (x_, y_, w_), need, g))
     return handles[key]
 
 
@@ -116,14 +145,15 @@ class _EdgeUvuCompiled(Function):
         dims = kernels.uvu_dims(cfg)
         out = kernels.uvu_forward(cfg, dims, x, sh, w, seg=plan.fwd_index)
         ctx.save_for_backward(x, sh, w)
-        ctx.plan, ctx.cfg, ctx.dims = plan, cfg, dims
+        ctx.plan, ctx.cfg, ctx.dims, ctx.tp_info = plan, cfg, dims, tp_info
         return out
 
     @staticmethod
-    @torch.autograd.function.once_differentiable
     def backward(ctx, g):
         x, sh, w = ctx.saved_tensors
         plan = ctx.plan
+        if torch.is_grad_enabled():
+            return (*_higher_order(_unfused(plan, ctx.tp_info), (x, sh, w), ctx.needs_input_grad[:3], g), None, None, None)
         res = kernels.uvu_backward(ctx.cfg, ctx.dims, x, sh, w, g.contiguous(), ctx.needs_input_grad[:3],
                                    seg=plan.bwd_index)
         return (*res, None, None, None)
@@ -133,20 +163,22 @@ class _EdgeUvuVectors(Function):
     """The fused kernels with the harmonics evaluated inside them: the second operand is the edge vector."""
 
     @staticmethod
-    def forward(ctx, x: Tensor, vec: Tensor, w: Tensor, plan: EdgePlan, cfg: int, y_vec: int):
+    def forward(ctx, x: Tensor, vec: Tensor, w: Tensor, plan: EdgePlan, cfg: int, y_vec: int, tp_info: TensorProductInfo):
         dims = kernels.uvu_dims(cfg)
         out = kernels.uvu_forward(cfg, dims, x, vec, w, seg=plan.fwd_index, y_vec=y_vec)
         ctx.save_for_backward(x, vec, w)
-        ctx.plan, ctx.cfg, ctx.dims, ctx.y_vec = plan, cfg, dims, y_vec
+        ctx.plan, ctx.cfg, ctx.dims, ctx.y_vec, ctx.tp_info = plan, cfg, dims, y_vec, tp_info
         return out
 
     @staticmethod
-    @torch.autograd.function.once_differentiable
     def backward(ctx, g):
         x, vec, w = ctx.saved_tensors
+        if torch.is_grad_enabled():
+            expression = _unfused(ctx.plan, ctx.tp_info, ctx.y_vec)
+            return (*_higher_order(expression, (x, vec, w), ctx.needs_input_grad[:3], g), None, None, None, None)
         res = kernels.uvu_backward(ctx.cfg, ctx.dims, x, vec, w, g.contiguous(), ctx.needs_input_grad[:3],
                                    seg=ctx.plan.bwd_index, y_vec=ctx.y_vec)
-        return (*res, None, None, None)
+        return (*res, None, None, None, None)
 
 
 class _EdgeUvuRadial(Function):
@@ -154,20 +186,34 @@ class _EdgeUvuRadial(Function):
     is given as harmonics, else as edge vectors)."""
 
     @staticmethod
-    def forward(ctx, x: Tensor, y: Tensor, h: Tensor, w_eff: Tensor, plan: EdgePlan, cfg: int, y_vec: int):
+    def forward(ctx, x: Tensor, y: Tensor, h: Tensor, w_last: Tensor, plan: EdgePlan, cfg: int, y_vec: int,
+                tp_info: TensorProductInfo):
         dims = kernels.uvu_dims(cfg)
+        w_eff = kernels.radial_effective_weight(w_last, cfg)       # over the compiled paths, the table's factors folded in
         out = kernels.uvu_radial_forward(cfg, dims, x, y, h, w_eff, plan.fwd_index, y_vec)
-        ctx.save_for_backward(x, y, h, w_eff)
-        ctx.plan, ctx.cfg, ctx.dims, ctx.y_vec = plan, cfg, dims, y_vec
+        ctx.save_for_backward(x, y, h, w_last, w_eff)
+        ctx.plan, ctx.cfg, ctx.dims, ctx.y_vec, ctx.tp_info = plan, cfg, dims, y_vec, tp_info
         return out
 
     @staticmethod
-    @torch.autograd.function.once_differentiable
     def backward(ctx, g):
-        x, y, h, w_eff = ctx.saved_tensors
-        res = kernels.uvu_radial_backward(ctx.cfg, ctx.dims, x, y, h, w_eff, g.contiguous(), ctx.needs_input_grad[:4],
-                                          ctx.plan.bwd_index, ctx.y_vec)
-        return (*res, None, None, None)
+        x, y, h, w_last, w_eff = ctx.saved_tensors
+        need = ctx.needs_input_grad[:4]
+        if torch.is_grad_enabled():
+            plain = _unfused(ctx.plan, ctx.tp_info, ctx.y_vec)
+
+            def expression(x_, y_, h_, w_):
+                return plain(x_, y_, (h_ @ w_.reshape(w_.shape[0], -1)).view(h_.shape[0], *w_.shape[1:]))
+            return (*_higher_order(expression, (x, y, h, w_last), need, g), None, None, None, None)
+        gx, gy, gh, gwe = kernels.uvu_radial_backward(ctx.cfg, ctx.dims, x, y, h, w_eff, g.contiguous(), need,
+                                                      ctx.plan.bwd_index, ctx.y_vec)
+        gwl = None
+        if need[3]:       # back through the rearrangement of the paths (linear in w_last)
+            with torch.enable_grad():
+                wl = w_last.detach().requires_grad_(True)
+                we = kernels.radial_effective_weight(wl, ctx.cfg)
+            (gwl,) = torch.autograd.grad(we, wl, gwe)
+        return gx, gy, gh, gwl, None, None, None, None
 
 
 class _EdgeUvuTable(Function):
@@ -176,18 +222,19 @@ class _EdgeUvuTable(Function):
     operands and the segment sums in LDS."""
 
     @staticmethod
-    def forward(ctx, x: Tensor, sh: Tensor, w: Tensor, plan: EdgePlan, tab):
+    def forward(ctx, x: Tensor, sh: Tensor, w: Tensor, plan: EdgePlan, tab, tp_info: TensorProductInfo):
         out = kernels.uvu_tab_forward(tab, x, sh, w, plan.fwd_index)
         ctx.save_for_backward(x, sh, w)
-        ctx.plan, ctx.tab = plan, tab
+        ctx.plan, ctx.tab, ctx.tp_info = plan, tab, tp_info
         return out
 
     @staticmethod
-    @torch.autograd.function.once_differentiable
     def backward(ctx, g):
         x, sh, w = ctx.saved_tensors
+        if torch.is_grad_enabled():
+            return (*_higher_order(_unfused(ctx.plan, ctx.tp_info), (x, sh, w), ctx.needs_input_grad[:3], g), None, None, None)
         res = kernels.uvu_tab_backward(ctx.tab, x, sh, w, g.contiguous(), ctx.needs_input_grad[:3], ctx.plan.bwd_index)
-        return (*res, None, None)
+        return (*res, None, None, None)
 
 
 class _EdgeUvuRows(Function):
@@ -202,15 +249,16 @@ class _EdgeUvuRows(Function):
         e, d, c = msg.shape
         out = kernels.segment_sum(msg.view(1, e, d * c), None, plan.perm_dst, plan.ptr_dst, plan.num_nodes)
         ctx.save_for_backward(x, sh, w)
-        ctx.plan, ctx.cfg, ctx.dims = plan, cfg, dims
+        ctx.plan, ctx.cfg, ctx.dims, ctx.tp_info = plan, cfg, dims, tp_info
         return out.view(plan.num_nodes, d, c)
 
     @staticmethod
-    @torch.autograd.function.once_differentiable
     def backward(ctx, g):
         x, sh, w = ctx.saved_tensors
         plan = ctx.plan
         need = ctx.needs_input_grad[:3]
+        if torch.is_grad_enabled():
+            return (*_higher_order(_unfused(plan, ctx.tp_info), (x, sh, w), need, g), None, None, None)
         gxe, gy, gw = kernels.uvu_backward(ctx.cfg, ctx.dims, x, sh, w, g.contiguous(), need, gather=plan.dst,
                                            x_gather=plan.src)
         gx = None
@@ -238,7 +286,7 @@ def edge_tensor_product_uu(x: Tensor, sh: Tensor, weight: Tensor, plan: EdgePlan
         xc, yc, wc = x.contiguous(), sh.contiguous(), weight.contiguous()
         if kernels.uvu_launchable(cfg, xc, yc, wc, segments=True):
             kernels.log_tier("edge_tensor_product_uu", "fused gather / product / segment sum", f"config {int(cfg)}")
-            handle = _shim_handle(plan, cfg, xc, 0)
+            handle = _shim_handle(plan, cfg, xc, 0, tp_info_forward)
             if handle is not None:
                 from ... import _shim
                 return _shim.module().edge_uvu(xc, yc, wc, handle)
@@ -252,7 +300,7 @@ def edge_tensor_product_uu(x: Tensor, sh: Tensor, weight: Tensor, plan: EdgePlan
         if kernels.uvu_tab_launchable(tab, xc, yc, wc, weight.requires_grad and torch.is_grad_enabled()):
             kernels.log_tier("edge_tensor_product_uu", "table-driven fused gather / product / segment sum",
                              f"{tab.nnz} coefficients")
-            return _EdgeUvuTable.apply(xc, yc, wc, plan, tab)
+            return _EdgeUvuTable.apply(xc, yc, wc, plan, tab, tp_info_forward)
     kernels.log_tier("edge_tensor_product_uu", "index_select + tensor_product_u1u + sparse_scale")
     msg = tensor_product_u1u(x.index_select(0, plan.src), sh, weight, tp_info_forward)
     e, d, c = msg.shape
@@ -282,11 +330,11 @@ def edge_tensor_product_uu_vectors(x: Tensor, edge_vec: Tensor, weight: Tensor, 
             and x.dtype in (torch.float32, torch.float64)):
         xc, vc, wc = x.contiguous(), edge_vec.contiguous(), weight.contiguous()
         if kernels.uvu_launchable(cfg, xc, vc, wc, segments=True, y_vec=mode):
-            handle = _shim_handle(plan, cfg, xc, mode)
+            handle = _shim_handle(plan, cfg, xc, mode, tp_info_forward)
             if handle is not None:
                 from ... import _shim
                 return _shim.module().edge_uvu(xc, vc, wc, handle)
-            return _EdgeUvuVectors.apply(xc, vc, wc, plan, cfg, mode)
+            return _EdgeUvuVectors.apply(xc, vc, wc, plan, cfg, mode, tp_info_forward)
     d2 = int(kernels.coo_of(tp_info_forward).D2)
     l_max = int(round(d2 ** 0.5)) - 1
     if (l_max + 1) ** 2 != d2:
@@ -316,8 +364,7 @@ def edge_tensor_product_uu_radial(x: Tensor, sh_or_vec: Tensor, h: Tensor, w_las
             and (not edge_vectors or kernels.uvu_sh_degree(cfg) >= 0)):
         kernels.log_tier("edge_tensor_product_uu_radial", "fused gather / weights / product / segment sum",
                          f"config {int(cfg)}")
-        w_eff = kernels.radial_effective_weight(w_last, cfg)       # differentiable: expands paths, folds factors
-        return _EdgeUvuRadial.apply(xc, yc, hc, w_eff, plan, cfg, mode)
+        return _EdgeUvuRadial.apply(xc, yc, hc, w_last, plan, cfg, mode, tp_info_forward)
     kernels.log_tier("edge_tensor_product_uu_radial", "weights by matrix product, then the plain edge product")
     weight = (h @ w_last.reshape(w_last.shape[0], -1)).view(h.shape[0], *w_last.shape[1:])
     if edge_vectors:

@@ -8,6 +8,16 @@ from .. import _lib
 MAX_DEGREE = 17
 
 
+def _expression(xyz: Tensor, l_max: int, normalize: bool, scale: float) -> Tensor:
+    """The same function as a tensor expression that autograd differentiates to any order (as the reference's
+    TorchScript polynomials are, ``equitorch/ops/spherical_harmonics.py:68-640``): the Clebsch-Gordan recursion
+    ``Y_l ~ C(l; l-1, 1) Y_(l-1) (x) Y_1``, whose degree-l block is the harmonic polynomial homogeneous of degree l."""
+    from ..utils._sh import spherical_harmonics as recursion
+    v = xyz / xyz.norm(dim=-1, keepdim=True).clamp_min(1e-12) if normalize else xyz
+    out = recursion(v, l_max)
+    return out if scale == 1.0 else out * scale
+
+
 class _SphericalHarmonics(torch.autograd.Function):
     """``(n, 3) -> (n, (l_max+1)^2)``; optional fused normalisation of the input and overall scale."""
 
@@ -22,10 +32,14 @@ class _SphericalHarmonics(torch.autograd.Function):
         return out
 
     @staticmethod
-    @torch.autograd.function.once_differentiable
     def backward(ctx, grad_out: Tensor):
         (xyz,) = ctx.saved_tensors
         l_max, normalize, scale = ctx.args
+        if torch.is_grad_enabled():   # a gradient of the gradient is wanted (forces in the loss): the tensor expression
+            with torch.enable_grad():
+                (grad,) = torch.autograd.grad(_expression(xyz, l_max, normalize, scale), (xyz,), grad_out,
+                                              create_graph=True)
+            return grad, None, None, None
         grad_out = grad_out.contiguous()
         grad = torch.empty_like(xyz)
         _lib.check(_lib.lib.cgtp_sh_backward(_lib.ptr(xyz), _lib.ptr(grad_out), _lib.ptr(grad), xyz.shape[0], l_max,
