@@ -14,7 +14,7 @@ def _expression(xyz: Tensor, l_max: int, normalize: bool, scale: float) -> Tenso
     ``Y_l ~ C(l; l-1, 1) Y_(l-1) (x) Y_1``, whose degree-l block is the harmonic polynomial homogeneous of degree l."""
     from ..utils._sh import spherical_harmonics as recursion
     v = xyz / xyz.norm(dim=-1, keepdim=True).clamp_min(1e-12) if normalize else xyz
-    out = recursion(v, l_max)
+    out = recursion(v, l_max, dtype=xyz.dtype)
     return out if scale == 1.0 else out * scale
 
 
