@@ -101,3 +101,48 @@ def test_forces_in_the_loss_through_the_fused_edge_products(device, monkeypatch,
     names = ("x", "second operand", "h", "w_last") if radial else ("x", "second operand", "w")
     for name, a, b in zip(names, gg, ref_gg):
         assert_close(a, b, tol, f"{mode}: d loss / d {name} with the force in the loss", norm="max")
+
+
+@pytest.mark.parametrize("case", ["shared weight", "table that is not compiled in", "row kernels + segment sums"])
+def test_forces_in_the_loss_on_the_other_routes_of_the_edge_product(device, monkeypatch, case):
+    """The same check where ``edge_tensor_product_uu`` takes another route: a shared weight (its gradient is a sum over
+    the edges), a table without compiled kernels (table-driven fused kernels) and a table whose fused kernels do not
+    take 128 channels (row kernels followed by segment sums)."""
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu
+    from equitorch_amd.ops import kernels
+    io, i1, i2, ch, dtype, want = {
+        "shared weight": ("0e+1o+2e", "0e+1o+2e", "0e+1o+2e", 64, torch.float64, "fused gather / product / segment sum"),
+        "table that is not compiled in": ("1o+2e+1e", "0e+1o+2e", "0e+1o", 32, torch.float32, "table-driven fused"),
+        "row kernels + segment sums": ("0e+1o+2e+3o+4e",) * 3 + (128, torch.float32, "block-wise row kernels"),
+    }[case]
+    n_nodes, n_edges = 30, 300
+    mod = SO3Linear(i1, i2, io, ch, ch, internal_weights=False, feature_mode="uu").to(device)
+    gen = torch.Generator().manual_seed(len(case))
+    src, dst = torch.randint(0, n_nodes, (n_edges,), generator=gen), torch.randint(0, n_nodes, (n_edges,), generator=gen)
+    rd = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float64).to(dtype).double()
+    d1, d2, do = Irreps(i1).dim, Irreps(i2).dim, Irreps(io).dim
+    x, sh, ct, ct2, cf = rd(n_nodes, d1, ch), rd(n_edges, d2), rd(n_nodes, do, ch), rd(n_nodes, do, ch), rd(n_edges, d2)
+    w = rd(mod.num_paths, ch) if case == "shared weight" else rd(n_edges, mod.num_paths, ch)
+    T = ref_ops.dense_coupling(io, i1, i2).float().double()
+    plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
+    seen = []
+    monkeypatch.setattr(kernels, "log_tier", lambda op, tier, detail="": seen.append(tier))
+
+    def twice(fn, inputs, cts):
+        ct, cf, ct2 = cts
+        out = fn(*inputs)
+        (force,) = torch.autograd.grad(out, inputs[1], ct, create_graph=True)
+        return out, force, torch.autograd.grad((force * cf).sum() + (out * ct2).sum(), inputs)
+
+    reference = lambda x, sh, w: ref_ops.scatter_sum(ref_ops.dense_u1u(T, x.index_select(0, src), sh, w), dst, n_nodes)
+    ref = twice(reference, [t.clone().requires_grad_(True) for t in (x, sh, w)], (ct, cf, ct2))
+    got = twice(lambda x, sh, w: edge_tensor_product_uu(x, sh, w, plan, mod.tp_info_forward),
+                [t.to(device, dtype).requires_grad_(True) for t in (x, sh, w)], [t.to(device, dtype) for t in (ct, cf, ct2)])
+    assert want in seen[0], seen
+    tol = 1e-5 if dtype == torch.float32 else 1e-11
+    assert_close(got[0], ref[0], tol, f"{case}: out", norm="max")
+    assert_close(got[1], ref[1], tol, f"{case}: gradient under create_graph", norm="max")
+    for name, a, b in zip(("x", "harmonics", "w"), got[2], ref[2]):
+        assert_close(a, b, tol, f"{case}: d loss / d {name} with the force in the loss", norm="max")
