@@ -45,13 +45,17 @@ class Cfg(int):
     compiled ones times one factor per weight path — what ``path_norm`` / ``channel_norm`` / ``channel_scale`` change
     (``equitorch/utils/_structs.py:177-206``).  ``w_rows`` (int array over the compiled paths, or None = identity): the
     caller's weight row of every compiled path, -1 for a path the caller's table does not have (an explicit ``path=``
-    subset); such weights are expanded with zero rows before the launch (:func:`expand_paths`)."""
+    subset); such weights are expanded with zero rows before the launch (:func:`expand_paths`).  ``exact``: every
+    coefficient of the caller's table is the compiled one times its path's factor to the last bit.  The tables hold
+    fp32 products of coupling and normalisation, so with another normalisation the ratios of a path's entries scatter
+    by an fp32 rounding (1e-7): nothing in fp32 arithmetic, but seven digits short of what float64 operands are held
+    to — those take the compiled kernels for exact matches only (:func:`uvu_launchable`)."""
     path_scale: Optional[np.ndarray]
     w_rows: Optional[np.ndarray]
 
-    def __new__(cls, value: int, path_scale=None, w_rows=None):
+    def __new__(cls, value: int, path_scale=None, w_rows=None, exact=True):
         obj = super().__new__(cls, value)
-        obj.path_scale, obj.w_rows = path_scale, w_rows
+        obj.path_scale, obj.w_rows, obj.exact = path_scale, w_rows, exact
         obj._dev = {}
         return obj
 
@@ -134,6 +138,7 @@ def _match_config(tp_info, family: str) -> Cfg:
         if any(len(r) != count[pc] for pc, r in ratios.items()):
             continue
         scale = np.zeros(dims[3], dtype=np.float64)
+        exact = True
         for pc, r in ratios.items():
             r = np.asarray(r)
             mid = float(np.median(r))
@@ -141,13 +146,14 @@ def _match_config(tp_info, family: str) -> Cfg:
                 ok = False
                 break
             scale[pc] = mid
+            exact = exact and bool(np.all(r == mid))
         if not ok:
             continue
         full = len(ratios) == dims[3]
         identity = full and all(row_of[pc] == pc for pc in range(dims[3]))
         ones = full and np.all(np.abs(scale - 1.0) <= tol)
         rows = None if identity else np.array([row_of.get(pc, -1) for pc in range(dims[3])], dtype=np.int64)
-        return Cfg(cfg, None if ones else scale, rows)
+        return Cfg(cfg, None if ones else scale, rows, exact)
     return Cfg(-1)
 
 
@@ -600,6 +606,8 @@ def uvu_launchable(cfg: int, x: Tensor, y: Tensor, w: Tensor, segments: bool = F
     alignment); outputs are torch allocations and therefore always aligned.  ``gathered``: row mode with the rows
     of ``x`` picked by an index."""
     if x.shape[0] == 0 or y.shape[0] == 0:
+        return False
+    if x.dtype == torch.float64 and not getattr(cfg, "exact", True):
         return False
     # the answer depends on these only (pointers enter through their 16-byte alignment)
     key = (int(cfg), x.dtype, x.shape[-1], w.ndim, y.ndim, segments, gathered, y_vec,

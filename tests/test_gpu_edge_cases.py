@@ -234,3 +234,52 @@ def test_output_irreps_that_no_path_reaches_follow_the_reference_tables(device, 
         T = ref_ops.dense_coupling(io, i1, i2, **({"channel_scale": c ** -0.5} if mode == "uv" else {})).double()
         dense = (ref_ops.dense_u1u if mode == "uu" else ref_ops.dense_u1v)(T, x, y, w)
         assert float((dense - ref).abs().max()) > 0.1, "the dense contraction places these rows elsewhere"
+
+
+@pytest.mark.parametrize("irreps,kw", [(("0e+1o+2e", "0e+1o+2e", "0e+1o+2e+3o"), {}),
+                                       (("0e+1o+2e", "0e+1o+2e", "0e+1o+2e"), {"path_norm": False}),
+                                       (("0e+1o+2e", "0e+1o+2e", "0e+1o+2e"), {})])
+def test_float64_on_a_table_that_matches_a_compiled_one_up_to_rounding(device, monkeypatch, irreps, kw):
+    """The reference's tables hold the fp32 product of coupling and normalisation.  A table that is a compiled one
+    times a factor per path (a subset of its paths, another normalisation) matches it entry by entry only to an fp32
+    rounding: good enough for fp32 operands, 1e-8 off for float64 ones.  float64 operands take the compiled kernels
+    for bit-exact matches only and the table-driven kernels otherwise — 1e-11 against the dense oracle built from the
+    module's own fp32 coefficients either way, on a batch and over an edge list."""
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.nn import SO3Linear
+    from equitorch_amd.nn.functional import EdgePlan, edge_tensor_product_uu
+    from equitorch_amd.ops import kernels
+    i1, i2, io = irreps
+    ch, n_nodes, n_edges = 8, 40, 333
+    mod = SO3Linear(i1, i2, io, ch, ch, internal_weights=False, feature_mode="uu", **kw).to(device)
+    cfg = kernels.uvu_config_of(mod.tp_info_forward)
+    assert int(cfg) >= 0
+    if io != i1:
+        assert not cfg.exact        # a subset of the paths of a larger compiled table, renormalised
+    elif not kw:
+        assert cfg.exact and cfg.path_scale is None
+    T = ref_ops.dense_coupling(io, i1, i2, **kw).float().double()
+    g = torch.Generator().manual_seed(len(io) + len(kw))
+    rd = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64)
+    src, dst = torch.randint(0, n_nodes, (n_edges,), generator=g), torch.randint(0, n_nodes, (n_edges,), generator=g)
+    x, sh, w = rd(n_nodes, Irreps(i1).dim, ch), rd(n_edges, Irreps(i2).dim), rd(n_edges, mod.num_paths, ch)
+    ct = rd(n_nodes, Irreps(io).dim, ch)
+    seen = []
+    monkeypatch.setattr(kernels, "log_tier", lambda op, tier, detail="": seen.append(tier))
+    plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
+    dev = [t.to(device).requires_grad_(True) for t in (x, sh, w)]
+    out = edge_tensor_product_uu(*dev, plan, mod.tp_info_forward)
+    assert ("fused gather / product / segment sum" == seen[0]) == cfg.exact, seen
+    grads = torch.autograd.grad(out, dev, ct.to(device))
+    ref_fn = lambda T, x, sh, w: ref_ops.scatter_sum(ref_ops.dense_u1u(T, x.index_select(0, src), sh, w), dst, n_nodes)
+    ref_out, ref_grads = ref_ops.dense_grads(ref_fn, T, (x, sh, w), ct)
+    for name, a, b in zip(("out", "grad_x", "grad_sh", "grad_w"), (out, *grads), (ref_out, *ref_grads)):
+        assert_close(a, b, 1e-11, f"{io} {kw} edge list {name}", norm="max")
+    xe = x.index_select(0, src)
+    dev = [t.to(device).requires_grad_(True) for t in (xe, sh, w)]
+    cte = rd(n_edges, Irreps(io).dim, ch)
+    out = mod(*dev)
+    grads = torch.autograd.grad(out, dev, cte.to(device))
+    ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1u, T, (xe, sh, w), cte)
+    for name, a, b in zip(("out", "grad_x", "grad_sh", "grad_w"), (out, *grads), (ref_out, *ref_grads)):
+        assert_close(a, b, 1e-11, f"{io} {kw} batch {name}", norm="max")
