@@ -468,6 +468,27 @@ def _adapted_path(x: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anc
     return out.to(dtype).contiguous()
 
 
+class _NoPaths(Function):
+    """A table without a reachable entry: the result is zero whatever the operands hold, and so are their gradients.
+    (The reference's builder can produce one: ``sparse_product_info``, ``equitorch/utils/_structs.py:105-123``, shifts
+    its segment pointers when the first output row has no entry, e.g. ``SO2Linear('0e' -> '2e+0e')``; its kernels then
+    walk no segment and return the zero-filled output.)"""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, weight: Tensor, out_size: int):
+        ctx.save_for_backward(x, weight)
+        return x.new_zeros(x.shape[0], out_size, weight.shape[-1])
+
+    @staticmethod
+    def backward(ctx, g):
+        x, weight = ctx.saved_tensors
+        return torch.zeros_like(x), torch.zeros_like(weight), None
+
+
+def no_paths(x: Tensor, weight: Tensor, plan: LinearPlan) -> Tensor:
+    return _NoPaths.apply(x, weight, plan.out_size)
+
+
 def mix(input: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anchor: Tensor = None) -> Tensor:
     """``(..., D_in, C_in) x (P, C_in, C_out) | (N, P, C_in, C_out) -> (..., D_out, C_out)``."""
     _lib.require_gpu(input, weight)
@@ -482,6 +503,8 @@ def mix(input: Tensor, weight: Tensor, plan: LinearPlan, in_size: int, anchor: T
     x = input.reshape(-1, *input.shape[-2:]).contiguous()
     if weight.ndim == 4 and weight.shape[0] != x.shape[0]:
         raise _lib.CgtpError(f"per-sample weight has {weight.shape[0]} samples, input has {x.shape[0]}")
+    if not plan.paths:
+        return no_paths(x, weight, plan).reshape(*lead, plan.out_size, weight.shape[-1])
     out = _matrix_core_path(x, weight, plan, in_size, anchor) if anchor is not None else None
     if out is None and anchor is not None:
         out = _table_driven_path(x, weight, plan, in_size, anchor)

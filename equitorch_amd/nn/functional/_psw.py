@@ -68,6 +68,10 @@ class PswTable:
                 slots.append((p, e0, len(words)))
             blocks.append((m0, rows, q0, len(slots)))
         self.covers_output = sum(rows for _, rows, _, _ in blocks) == d_out
+        # weight paths without an entry (the reference's tables can leave one out: `sparse_product_info`,
+        # `equitorch/utils/_structs.py:105-123`, shifts its segments when the first output row has no entry): the
+        # kernels never visit them, so their gradient is written here
+        self.unwalked_paths = sorted(set(range(int(n_paths))) - set(int(p) for p in np.unique(path)))
         self.device = device
         self.entries = torch.tensor(words, dtype=torch.int64).to(torch.int32).to(device)     # bit 24 at most: fits
         self._coef64 = torch.tensor(coefs, dtype=torch.float64)
@@ -177,6 +181,9 @@ class _Product(Function):
         gx = torch.empty_like(x) if need[0] else None
         gy = torch.empty_like(y) if need[1] and y is not None else None
         gw = torch.empty_like(w) if need[2] else None
+        if gw is not None:
+            for p in ctx.table.unwalked_paths:
+                gw[:, p].zero_()
         args, c_table = _args(ctx.table, x, y, w), ctx.table.c_table(x.dtype)
         args.g = g.data_ptr()
         args.gx, args.gy, args.gw = (0 if t is None else t.data_ptr() for t in (gx, gy, gw))

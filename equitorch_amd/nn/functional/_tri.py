@@ -97,6 +97,8 @@ def _gen_contract(spec: "TriSpec", ops, axes, out_axes: str, out_shared: bool, n
     out = torch.empty(shape, dtype=dtype, device=device)
     if n_rows == 0 or out.numel() == 0:      # empty batch: nothing to launch; a sum over no rows is zero
         return out.zero_()
+    if a.nnz == 0:                           # a table without entries: a sum over no terms
+        return out.zero_()
     a.out, a.n_rows, a.U, a.W = out.data_ptr(), n_rows, U, W
     a.out_has_u, a.out_has_w = int("u" in out_axes), int("w" in out_axes)
     a.reduce_rows, a.dtype = int(out_shared), _lib.dtype_code(dtype)
@@ -289,9 +291,14 @@ def spec_from_product_info(info, size1: int, size2: int) -> TriSpec:
             s = info.seg_out.detach().cpu().numpy().astype(np.int64)
             n_out = s.shape[0] - 1
             out_idx = np.repeat(np.arange(n_out, dtype=np.int64), np.diff(s))
+            # entries past the last segment are reached by no output row.  The reference's builder leaves such
+            # entries behind when the first output row has none (`sparse_product_info`,
+            # `equitorch/utils/_structs.py:105-123`, shifts its segment pointers by one row then); its kernels walk
+            # the segments and never see them
+            i1, i2 = i1[:out_idx.shape[0]], i2[:out_idx.shape[0]]
         if info.out_size is not None:
             n_out = max(n_out, int(info.out_size))
-        coef = None if info.scale is None else info.scale.detach().cpu().double().numpy()
+        coef = None if info.scale is None else info.scale.detach().cpu().double().numpy()[:out_idx.shape[0]]
         return TriSpec(out_idx, [i1, i2, None], coef, n_out, [size1, size2, None])
 
     if anchor is None:

@@ -284,6 +284,8 @@ class SO2Linear(nn.Module):
                 anchor = next(t for t in (self.info_forward.seg_out, self.info_forward.index1,
                                           self.info_forward.index2, self.info_forward.scale) if t is not None)
                 x3 = input.reshape(-1, *input.shape[-2:]).contiguous()
+                if not plan.paths:
+                    return G.no_paths(x3, weight, plan).reshape(*input.shape[:-2], plan.out_size, weight.shape[-1])
                 out = G._table_driven_path(x3, weight.contiguous(), plan, self.irreps_in.dim, anchor)
                 if out is None and x3.shape[0] > 0:
                     out = G._adapted_path(x3, weight.contiguous(), plan, self.irreps_in.dim, anchor)

@@ -250,6 +250,8 @@ def tri_contract(table: dict, n_out: int, a: Tuple[Optional[Tensor], int], b: Tu
         raise _lib.CgtpError(f"out must be a contiguous {dtype} tensor of shape {shape}")
     if n_rows == 0 or out.numel() == 0:      # empty batch: nothing to launch; a sum over no rows is zero
         return out.zero_()
+    if table["idx"].shape[0] == 0:           # a table without entries: a sum over no terms
+        return out.zero_()
     args = TriArgs()
     args.a, args.b, args.w = _operand(*a, rows_a), _operand(*b, rows_b), _operand(*w, rows_w)
     args.coef, args.idx, args.seg = _lib.ptr(table["coef"]), table["idx"].data_ptr(), table["seg"].data_ptr()

@@ -496,7 +496,8 @@ int cgtp_uvt_grad_w(const cgtp_uvt_gw_args* args, void* stream);
  * / gw may be NULL.  The table is data: the paths are walked output irrep by output irrep.
  *   blocks  [n_blocks][4]  (first output row, rows L, first slot, one past the last slot); the rows of different
  *                          blocks do not overlap; output rows outside every block are not written
- *   slots   [n_slots][3]   (weight path p, first entry, one past the last entry) of a walked path
+ *   slots   [n_slots][3]   (weight path p, first entry, one past the last entry) of a walked path; the rows of gw
+ *                          that belong to a path without a slot are not written (the caller zeroes them)
  *   entries [n_entries]    j | a << 8 | b << 16 | 1 << 24 on the last entry of a run of equal j; j = output row - the
  *                          block's first row; sorted by j inside a slot; every j < L occurs in every slot of the
  *                          block (where the path has no term for it: one entry j | 1 << 24 | 1 << 25, no operand is

@@ -256,3 +256,37 @@ def test_so2_linear_uv_adapted_operands(device, monkeypatch, dtype, cin, cout):
         assert a.dtype == dtype and a.shape == b.shape
         assert_close(a.double(), b, tol, f"SO2Linear uv {dtype} {cin}->{cout} {name}",
                      norm="element" if dtype == torch.float32 else "max")
+
+
+@pytest.mark.parametrize("irr_in,irr_out", [("0e", "1o+2e"), ("1o+1e", "2e+0e"), ("0e", "2e+0e"), ("0e", "1o")])
+@pytest.mark.parametrize("mode,per_sample", [("uu", False), ("uu", True), ("uv", False), ("uv", True)])
+def test_so2_linear_on_tables_the_reference_builder_leaves_incomplete(device, irr_in, irr_out, mode, per_sample):
+    """When the first output component has no entry (no input component of its order), the reference's
+    ``sparse_product_info`` (``equitorch/utils/_structs.py:105-123``) shifts its segment pointers by a row: entries
+    move to the wrong output rows, the last ones are reached by no row, and with ``0e -> 2e+0e`` none is reached at
+    all.  The tables here are the reference's bit for bit, so the modules follow them — result and gradients of the
+    reference's algorithm on those tables, zero gradient for a weight no row uses (not whatever the allocator
+    returned: the buffers are dirtied first), zeros with zero gradients for a table without a reachable entry."""
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.nn import SO2Linear
+    info = _f32(ref_tables.so2_linear_infos(irr_out, irr_in)[0])
+    n, cin = 17, 33 if mode == "uv" else 8
+    cout = 4 if mode == "uv" else cin
+    mod = SO2Linear(irr_in, irr_out, cin, cout, internal_weights=False, feature_mode=mode).to(device)
+    g = torch.Generator().manual_seed(len(irr_in) + len(irr_out))
+    x = torch.randn(n, Irreps(irr_in).dim, cin, generator=g, dtype=torch.float64)
+    wshape = (mod.num_weights, cout) if mode == "uu" else (mod.num_weights, cin, cout)
+    w = torch.randn(*((n,) if per_sample else ()), *wshape, generator=g, dtype=torch.float64)
+    ct = torch.randn(n, Irreps(irr_out).dim, cout, generator=g, dtype=torch.float64)
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    ref = ref_ops.cpu_so2_linear(xr, wr, info, per_sample=per_sample)
+    rgx, rgw = torch.autograd.grad(ref, (xr, wr), ct)
+    for dtype, tol in ((torch.float64, 1e-11), (torch.float32, 1e-5)):
+        xd, wd = x.to(device, dtype).requires_grad_(True), w.to(device, dtype).requires_grad_(True)
+        dirt = [torch.full_like(t, 1e3) for t in (xd, wd, wd)]
+        del dirt
+        out = mod(xd, wd)
+        gx, gw = torch.autograd.grad(out, (xd, wd), ct.to(device, dtype))
+        for name, a, b in (("out", out, ref), ("grad_x", gx, rgx), ("grad_w", gw, rgw)):
+            assert_close(a, b, tol=tol, what=f"SO2Linear {irr_in} -> {irr_out} {mode} per_sample={per_sample} {dtype} {name}",
+                         norm="max")
