@@ -117,6 +117,9 @@ def segment_csr(src: torch.Tensor, ptr: torch.Tensor, dim: int) -> torch.Tensor:
     ids = torch.repeat_interleave(torch.arange(n_seg), ptr[1:] - ptr[:-1])
     shape = list(src.shape)
     shape[dim] = n_seg
+    # entries past the last pointer belong to no segment (the reference's builders can leave some behind,
+    # equitorch/utils/_structs.py:105-123); a pointer-driven sum never reads them
+    src = src.narrow(dim, int(ptr[0]), int(ptr[-1]) - int(ptr[0]))
     return torch.zeros(shape, dtype=src.dtype).index_add_(dim, ids, src)
 
 
@@ -433,6 +436,9 @@ def cpu_z_rotation(x, cs, info):
 def cpu_j(x, info):
     """``sparse_scale(x, j_matrix_info)``: ``out[n, M] = sum_{t in seg M} scale_t x[n, index_t]``."""
     seg, idx, sc = info["seg_out"], info["index"], info["scale"]
+    n = len(sc)
+    seg = seg if seg is not None else list(range(n + 1))       # the builders store an identity as None
+    idx = idx if idx is not None else list(range(n))
     return torch.stack([sum(sc[t] * x[:, idx[t]] for t in range(seg[m], seg[m + 1])) for m in range(len(seg) - 1)],
                        dim=1)
 
