@@ -250,6 +250,13 @@ def _coo(tp_info):
     return tp_info.coo if isinstance(tp_info, CooTable) else kernels.coo_of(tp_info)
 
 
+def _aligned(g: Tensor) -> Tensor:
+    """The incoming gradient as the kernels want it: contiguous and on a 16-byte boundary.  Autograd may hand over a
+    view into a larger buffer (the gradient of a ``cat`` or of a slice), contiguous but at any element offset."""
+    g = g.contiguous()
+    return g.clone() if g.data_ptr() % 16 else g
+
+
 class _U1vNative(Function):
     """u1v, shared fp32 weight ``(P, U, W)``.  The gradient of the first operand is the forward kernel with the rows'
     roles exchanged and the weight read transposed; the gradients of the weight and of the second operand have
@@ -280,7 +287,7 @@ class _U1vNative(Function):
         c = _coo(tp_info)
         p, u, wc = w.shape
         gx = gy = gw = None
-        g = g.contiguous()
+        g = _aligned(g)
         if need[0]:
             gx = apply(g, y, pack(w, p, wc, u, u * wc, 1, wc), tp_info, "in1", c.D1, u)
         if need[2]:
@@ -366,7 +373,7 @@ class _Vu1Native(Function):
         t = _swapped(ctx.tp_info)
         c = t.coo
         p, u, wc = w.shape
-        g = g.contiguous()
+        g = _aligned(g)
         gx = apply(y, g, pack(w, p, wc, u, u * wc, 1, wc), t, "in1", c.D1, u) if need[0] else None
         gy = apply(x, g, pack(w, p, u, wc, u * wc, wc, 1), t, "out", c.DO, wc) if need[1] else None
         gw = grad_w(x, g, y, t) if need[2] else None
@@ -417,7 +424,7 @@ class _UvwNative(Function):
             return tuple(next(got) if n else None for n in need) + (None,)
         c = _coo(tp_info)
         p, u, v, wc = w.shape
-        g = g.contiguous()
+        g = _aligned(g)
         gx = gy = gw = None
         if need[0]:     # first operand of the launch: y (channels v), second: grad_out (channels w); weight (P, V, W, U)
             wt = w.permute(0, 2, 3, 1).contiguous()

@@ -414,3 +414,37 @@ def test_1vu_native(device, monkeypatch, dtype):
         rgg = torch.autograd.grad(rgy.square().sum(), (xr, wr))
         for name, a, b in zip(("d/dx", "d/dw"), gg, rgg):
             assert_close(a, b, 1e-10, f"1vu second order {name}", norm="max")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_incoming_gradient_at_an_odd_offset_of_a_larger_buffer(device, dtype):
+    """Autograd hands the backward whatever view the consumer produced: the gradient of a slice or of a ``cat`` is
+    contiguous but starts at any element of a larger buffer.  The kernels want 16-byte boundaries; the Functions copy
+    such a gradient first.  Same results as with an aligned gradient, for the u1v product, the uvw product and the
+    channel mixing that runs on them."""
+    import equitorch_amd.nn.functional as F
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.nn import IrrepsLinear, SO3Linear
+    from equitorch_amd.utils import tp_infos
+    irr, n = _sh(2), 130
+    g = torch.Generator().manual_seed(5)
+    rd = lambda *s: torch.randn(*s, generator=g).to(device, dtype)
+    uv = SO3Linear(irr, irr, irr, 8, 12, internal_weights=False, feature_mode="uv").to(device)
+    lin = IrrepsLinear("1o+2e", "1o+2e", 4, 12, internal_weights=False).to(device)
+    infos = [t.to(device) for t in tp_infos(Irreps(irr), Irreps(irr), Irreps(irr))[:3]]
+    cases = [("u1v", lambda x, y, w: uv(x, y, w), (rd(n, 9, 8), rd(n, 9), rd(uv.num_paths, 8, 12))),
+             ("uvw", lambda x, y, w: F.tensor_product_uvw(x, y, w, *infos), (rd(n, 9, 4), rd(n, 9, 4), rd(11, 4, 4, 8))),
+             ("linear", lambda x, w: lin(x, w), (rd(n, 8, 4), rd(lin.num_paths, 4, 12)))]
+    for name, fn, ops in cases:
+        leaves = [t.clone().requires_grad_(True) for t in ops]
+        out = fn(*leaves)
+        ct = torch.randn(out.shape, generator=g).to(device, dtype)
+        want = torch.autograd.grad(out, leaves, ct, retain_graph=True)
+        for k in (1, 3):
+            buf = torch.empty(ct.numel() + 3, dtype=dtype, device=device)
+            buf[k:k + ct.numel()] = ct.reshape(-1)
+            odd = buf[k:k + ct.numel()].view(ct.shape)
+            assert odd.is_contiguous() and odd.data_ptr() % 16 != 0
+            got = torch.autograd.grad(out, leaves, odd, retain_graph=True)
+            for a, b in zip(got, want):
+                assert torch.equal(a, b), f"{name}: gradient differs with the cotangent {k} elements off"
