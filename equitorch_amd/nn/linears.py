@@ -73,8 +73,7 @@ class SO3Linear(nn.Module):
         if None in shape:  # channels were not given at construction: take them from the input
             shape = ((self.num_paths, input1.shape[-1], weight.shape[-1]) if self.feature_mode == 'uv'
                      else (self.num_paths, input1.shape[-1]))
-        numel = math.prod(shape)
-        return weight.view(-1, *shape) if weight.numel() > numel else weight.view(*shape)
+        return _view_weight(weight, shape, math.prod(shape))
 
     def forward(self, input1: Tensor, input2: Tensor, weight: Optional[Tensor] = None):
         assert input1.shape[-2] == self.irreps_in1_dim, \
@@ -109,6 +108,11 @@ class SO3Linear(nn.Module):
 
 
 def _view_weight(weight: Tensor, shape, numel: int) -> Tensor:
+    """The reference's rule (``equitorch/nn/linears.py:163-168``): more elements than one set of weights means a set
+    per sample.  A weight without elements (an empty batch with per-sample weights, which the reference's ``view``
+    rejects as ambiguous) is per-sample with zero samples."""
+    if weight.numel() == 0 and numel > 0:
+        return weight.view(0, *shape)
     return weight.view(-1, *shape) if weight.numel() > numel else weight.view(*shape)
 
 

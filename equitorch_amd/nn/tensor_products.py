@@ -12,6 +12,7 @@ from ..irreps import check_irreps
 from ..structs import IrrepsInfo, TensorProductInfo
 from ..utils._structs import tp_infos
 from ._irreps_module import IrrepsModule
+from .linears import _view_weight
 from .functional.tensor_products import tensor_dot_uu, tensor_dot_uv, tensor_product_uuu, tensor_product_uvw
 from .init import initialize_tensor_product
 
@@ -76,7 +77,7 @@ class TensorProduct(nn.Module):
             if None in shape:
                 shape = ((self.num_paths, input1.shape[-1], input2.shape[-1], weight.shape[-1])
                          if self.feature_mode == 'uvw' else (self.num_paths, input1.shape[-1]))
-            weight = weight.view(-1, *shape) if weight.numel() > math.prod(shape) else weight.view(*shape)
+            weight = _view_weight(weight, shape, math.prod(shape))
         infos = (self.tp_info_forward, self.tp_info_backward1, self.tp_info_backward2)
         if self.feature_mode == 'uuu':
             return tensor_product_uuu(input1, input2, weight, *infos)

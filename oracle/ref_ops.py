@@ -476,6 +476,6 @@ def cpu_so2_linear(x, w, info, per_sample=False):
         rows[o] = term if rows[o] is None else rows[o] + term
     # a row no entry reaches is zero; a table none of whose entries is reachable gives zeros that still hang on the
     # operands (the reference's kernel returns its zero-filled output and zero gradients)
-    blank = 0.0 * (x[:, 0, :1] * (w[:, 0].reshape(w.shape[0], -1)[:, :1] if per_sample else w[0].reshape(-1)[:1]))
+    blank = 0.0 * (x[:, 0, :1] * (w[:, 0].flatten(1)[:, :1] if per_sample else w[0].reshape(-1)[:1]))
     blank = blank.expand(x.shape[0], w.shape[-1])
     return torch.stack([r if r is not None else blank for r in rows], dim=1)

@@ -283,3 +283,33 @@ def test_float64_on_a_table_that_matches_a_compiled_one_up_to_rounding(device, m
     ref_out, ref_grads = ref_ops.dense_grads(ref_ops.dense_u1u, T, (xe, sh, w), cte)
     for name, a, b in zip(("out", "grad_x", "grad_sh", "grad_w"), (out, *grads), (ref_out, *ref_grads)):
         assert_close(a, b, 1e-11, f"{io} {kw} batch {name}", norm="max")
+
+
+def test_empty_batch_with_a_weight_per_sample(device):
+    """No samples and a weight with a sample axis: the weight has no elements, which the reference's per-sample rule
+    (``weight.numel() > weight_numel`` then ``view(-1, ...)``, ``equitorch/nn/linears.py:163-168``) cannot tell from a
+    malformed shared weight.  Taken as zero sets of weights here: empty result, empty gradients of the right shapes."""
+    from equitorch_amd import nn as enn
+    irr = "0e+1o+2e"
+    mods = [
+        (enn.IrrepsLinear(irr, irr, 8, 12, internal_weights=False), lambda m: [(0, 9, 8), (0, m.num_paths, 8, 12)], (0, 9, 12)),
+        (enn.IrrepWiseLinear(irr, 8, 12, internal_weights=False), lambda m: [(0, 9, 8), (0, 3, 8, 12)], (0, 9, 12)),
+        (enn.SO2Linear(irr, irr, 8, 12, internal_weights=False, feature_mode="uv"),
+         lambda m: [(0, 9, 8), (0, m.num_weights, 8, 12)], (0, 9, 12)),
+        (enn.SO2Linear(irr, irr, 8, 8, internal_weights=False, feature_mode="uu"),
+         lambda m: [(0, 9, 8), (0, m.num_weights, 8)], (0, 9, 8)),
+        (enn.SO3Linear(irr, irr, irr, 8, 8, internal_weights=False, feature_mode="uu"),
+         lambda m: [(0, 9, 8), (0, 9), (0, m.num_paths, 8)], (0, 9, 8)),
+        (enn.SO3Linear(irr, irr, irr, 8, 12, internal_weights=False, feature_mode="uv"),
+         lambda m: [(0, 9, 8), (0, 9), (0, m.num_paths, 8, 12)], (0, 9, 12)),
+        (enn.TensorProduct(irr, irr, irr, 4, 4, 8, internal_weights=False, feature_mode="uvw"),
+         lambda m: [(0, 9, 4), (0, 9, 4), (0, m.num_paths, 4, 4, 8)], (0, 9, 8)),
+    ]
+    for mod, shapes, out_shape in mods:
+        mod = mod.to(device)
+        ops = [torch.zeros(*s, device=device, requires_grad=True) for s in shapes(mod)]
+        out = mod(*ops)
+        assert tuple(out.shape) == out_shape, (type(mod).__name__, out.shape)
+        grads = torch.autograd.grad(out, ops, torch.zeros_like(out), allow_unused=True)
+        for t, g in zip(ops, grads):
+            assert g is None or g.shape == t.shape
