@@ -64,10 +64,10 @@ def test_forces_in_the_loss_through_the_fused_edge_products(device, monkeypatch,
     weights = (rd(n_edges, R), rd(R, P, ch) / R ** 0.5) if radial else (rd(n_edges, P, ch),)
     T = ref_ops.dense_coupling(irreps, irreps, irreps).float().double()
 
-    def reference(x, second, *weights):
+    def reference(x, second, *weights):      # in the precision of its operands
         sh = ref_sh.spherical_harmonics(ref_sh.normalize(second), l_max) if vectors else second
         w = (weights[0] @ weights[1].reshape(R, -1)).view(n_edges, P, ch) if radial else weights[0]
-        return ref_ops.scatter_sum(ref_ops.dense_u1u(T, x.index_select(0, src), sh, w), dst, n_nodes)
+        return ref_ops.scatter_sum(ref_ops.dense_u1u(T, x.index_select(0, src), sh, w, dtype=x.dtype), dst, n_nodes)
 
     plan = EdgePlan(src.to(device), dst.to(device), n_nodes)
     seen = []
@@ -96,11 +96,16 @@ def test_forces_in_the_loss_through_the_fused_edge_products(device, monkeypatch,
         assert "fused gather / product / segment sum" in seen[0], seen
     assert ("Cpp" in type(out.grad_fn).__name__) == (use_shim and not radial), type(out.grad_fn).__name__
     tol = 1e-5 if dtype == torch.float32 else 1e-11
-    assert_close(out, ref_out, tol, f"{mode}: out", norm="max")
-    assert_close(force, ref_force, tol, f"{mode}: gradient under create_graph", norm="max")
+    # fp32: the same computation restated in fp32 arithmetic beside every norm-wise comparison
+    r32 = (None, None, (None,) * len(ref_gg))
+    if dtype == torch.float32:
+        r32 = twice(reference, [t.float().requires_grad_(True) for t in (x, second, *weights)],
+                    [t.float() for t in (ct, cf, ct2)])
+    assert_close(out, ref_out, tol, f"{mode}: out", norm="max", fp32_ref=r32[0])
+    assert_close(force, ref_force, tol, f"{mode}: gradient under create_graph", norm="max", fp32_ref=r32[1])
     names = ("x", "second operand", "h", "w_last") if radial else ("x", "second operand", "w")
-    for name, a, b in zip(names, gg, ref_gg):
-        assert_close(a, b, tol, f"{mode}: d loss / d {name} with the force in the loss", norm="max")
+    for name, a, b, b32 in zip(names, gg, ref_gg, r32[2]):
+        assert_close(a, b, tol, f"{mode}: d loss / d {name} with the force in the loss", norm="max", fp32_ref=b32)
 
 
 @pytest.mark.parametrize("case", ["shared weight", "table that is not compiled in", "row kernels + segment sums"])
@@ -136,13 +141,17 @@ def test_forces_in_the_loss_on_the_other_routes_of_the_edge_product(device, monk
         (force,) = torch.autograd.grad(out, inputs[1], ct, create_graph=True)
         return out, force, torch.autograd.grad((force * cf).sum() + (out * ct2).sum(), inputs)
 
-    reference = lambda x, sh, w: ref_ops.scatter_sum(ref_ops.dense_u1u(T, x.index_select(0, src), sh, w), dst, n_nodes)
+    reference = lambda x, sh, w: ref_ops.scatter_sum(ref_ops.dense_u1u(T, x.index_select(0, src), sh, w, dtype=x.dtype),
+                                                     dst, n_nodes)
     ref = twice(reference, [t.clone().requires_grad_(True) for t in (x, sh, w)], (ct, cf, ct2))
+    r32 = (None, None, (None,) * 3)
+    if dtype == torch.float32:
+        r32 = twice(reference, [t.float().requires_grad_(True) for t in (x, sh, w)], [t.float() for t in (ct, cf, ct2)])
     got = twice(lambda x, sh, w: edge_tensor_product_uu(x, sh, w, plan, mod.tp_info_forward),
                 [t.to(device, dtype).requires_grad_(True) for t in (x, sh, w)], [t.to(device, dtype) for t in (ct, cf, ct2)])
     assert want in seen[0], seen
     tol = 1e-5 if dtype == torch.float32 else 1e-11
-    assert_close(got[0], ref[0], tol, f"{case}: out", norm="max")
-    assert_close(got[1], ref[1], tol, f"{case}: gradient under create_graph", norm="max")
-    for name, a, b in zip(("x", "harmonics", "w"), got[2], ref[2]):
-        assert_close(a, b, tol, f"{case}: d loss / d {name} with the force in the loss", norm="max")
+    assert_close(got[0], ref[0], tol, f"{case}: out", norm="max", fp32_ref=r32[0])
+    assert_close(got[1], ref[1], tol, f"{case}: gradient under create_graph", norm="max", fp32_ref=r32[1])
+    for name, a, b, b32 in zip(("x", "harmonics", "w"), got[2], ref[2], r32[2]):
+        assert_close(a, b, tol, f"{case}: d loss / d {name} with the force in the loss", norm="max", fp32_ref=b32)
