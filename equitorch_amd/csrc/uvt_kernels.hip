@@ -158,9 +158,12 @@ __device__ __forceinline__ cgtp_uvt_item uvt_item_at(const UvtTables& tab, int j
 // arrays (a conditional assignment to an array element costs the compiler a copy of the array).
 constexpr int kUvtTerms = 8;
 // Blocks of 16 k in the ring of weight fragments; k is padded to whole turns of it (zero weights, zero rows of the
-// staged tiles).  Four blocks cover the round trip to L2; with at most 32 contracted channels a ring of four would be
-// half padding — twice the LDS per sample and twice the matrix instructions — so those get a ring of two.
-__host__ __device__ constexpr int uvt_kbi(int64_t K) { return K <= 32 ? 2 : 4; }
+// staged tiles).  Four blocks cover the round trip to L2 by themselves, which the large products need (their rows fill
+// the LDS: one workgroup per compute unit).  Up to 64 contracted channels the ring is two blocks: with at most 32 a
+// ring of four would be half padding (twice the LDS per sample, twice the matrix instructions), and at 64 the 32
+// registers it saves let a second workgroup onto the compute unit, which covers the latency better than the deeper
+// ring did (64 -> 64 channels, lmax = 3, 32768 samples: forward 415 -> 355 us, grad y 734 -> 561 us).
+__host__ __device__ constexpr int uvt_kbi(int64_t K) { return K <= 64 ? 2 : 4; }
 template <bool YC>
 struct UvtTerms {
   const real* xr[kUvtTerms];

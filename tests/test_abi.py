@@ -276,14 +276,16 @@ def test_table_driven_matrix_core_entry_points_validate_on_the_host():
     assert L.cgtp_uvt_chunk(100, 16, 16, 16, 130, 0, 128, _lib.F32) == -2             # channels not a multiple of 4
     assert L.cgtp_uvt_chunk(100, 49, 49, 49, 128, 0, 128, _lib.F32) == -6   # 16 samples x 49 rows x 128 floats > LDS
     assert L.cgtp_uvt_chunk(100, 16, 16, 16, 128, 0, 128, _lib.F64) == -6   # the same rows as doubles do not fit either
-    assert L.cgtp_uvt_chunk(100, 16, 16, 16, 64, 0, 128, _lib.F64) == 4
+    assert L.cgtp_uvt_chunk(100, 16, 16, 16, 64, 0, 128, _lib.F64) == 2
     assert L.cgtp_uvt_chunk(100, 16, 16, 16, 64, 0, 128, _lib.BF16) == -4
     assert L.cgtp_uvt_packed_elems(23, 128, 128) == 23 * 8 * 8 * 256
     assert L.cgtp_uvt_packed_elems(2, 20, 12) == 2 * 2 * 4 * 256            # padded to whole ring turns / 4 blocks
-    assert L.cgtp_uvt_packed_elems(2, 40, 12) == 2 * 4 * 4 * 256            # a ring of four past 32 contracted channels
+    assert L.cgtp_uvt_packed_elems(2, 40, 12) == 2 * 4 * 4 * 256            # three blocks of k: two turns of a ring of two
+    assert L.cgtp_uvt_packed_elems(2, 72, 12) == 2 * 8 * 4 * 256            # a ring of four past 64 contracted channels
     assert L.cgtp_uvt_chunk(32768, 16, 16, 16, 32, 0, 128, _lib.F32) == 2
     assert L.cgtp_uvt_chunk(32768, 9, 9, 9, 4, 8, 16, _lib.F32) == 2         # K = 4 x 8
-    assert L.cgtp_uvt_chunk(32768, 9, 9, 9, 8, 8, 16, _lib.F64) == 4
+    assert L.cgtp_uvt_chunk(32768, 9, 9, 9, 8, 8, 16, _lib.F64) == 2         # K = 64
+    assert L.cgtp_uvt_chunk(32768, 9, 9, 9, 8, 16, 16, _lib.F64) == 4
     a = _lib.UvtArgs()
     a.dtype = _lib.BF16
     assert L.cgtp_uvt_validate(C.byref(a)) == 4                             # fp32 only
@@ -291,7 +293,7 @@ def test_table_driven_matrix_core_entry_points_validate_on_the_host():
     a.n_rows, a.dx, a.dy, a.dout, a.cx, a.cy, a.cout = 100, 9, 9, 9, 32, 0, 32
     assert L.cgtp_uvt_validate(C.byref(a)) == 2                             # kbi / groups not set
     a.kbi, a.n_groups = 4, 8
-    assert L.cgtp_uvt_validate(C.byref(a)) == 2                             # 32 contracted channels: a ring of two
+    assert L.cgtp_uvt_validate(C.byref(a)) == 2                             # up to 64 contracted channels: a ring of two
     a.kbi = 2
     a.n_items, a.n_terms = 35, 83
     for i in range(9):
