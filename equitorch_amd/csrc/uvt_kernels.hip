@@ -585,33 +585,48 @@ __global__ void __launch_bounds__(256, sizeof(real) == 8 ? 1 : NARROW ? 2 : 3) u
 // chunk of samples by itself: the operands' layout in memory is the matrix instructions' own (lane (r, g) holds the
 // four channels 4 r .. 4 r + 3 of sample g of four: one 16-byte load, element i = tile i), so nothing is exchanged
 // through LDS and there is no barrier; two steps of eight samples are loaded before the first is multiplied, and
-// several wavefronts per SIMD cover each other's load latency.
-template <bool YC>
+// several wavefronts per SIMD cover each other's load latency.  An axis of at most 32 channels takes two channels a
+// lane and two tiles (32 x 32 weights, lmax = 3, 32768 samples: 461 -> 226 us).
+template <int N> struct UvtVec;
+template <> struct UvtVec<2> { typedef realx2 type; };
+template <> struct UvtVec<4> { typedef realx4 type; };
+
+// TI / TJ: channels a lane holds of the contracted and of the output axis = accumulator tiles along each (4: up to 64
+// channels, 2: up to 32 — a 32 x 32 weight in 4 x 4 tiles would multiply three quarters zeros).
+template <bool YC, int TI, int TJ>
 __global__ void __launch_bounds__(kWave) uvt_grad_w_small_kernel(const UvtGwDev a) {
+  typedef typename UvtVec<TI>::type VI;
+  typedef typename UvtVec<TJ>::type VJ;
   const int lane = threadIdx.x, r = lane & 15, g4 = lane >> 4;
   const int p = blockIdx.y;
   const int64_t n_begin = (int64_t)blockIdx.x * a.chunk;
   const int64_t n_end = n_begin + a.chunk < a.n_rows ? n_begin + a.chunk : a.n_rows;
-  const bool kok = 4 * r < a.K, wok = 4 * r < a.cout;
-  const int kc = kok ? 4 * r : 0, wc = wok ? 4 * r : 0;
+  const bool kok = TI * r < a.K, wok = TJ * r < a.cout;
+  const int kc = kok ? TI * r : 0, wc = wok ? TJ * r : 0;
   int xo = kc, yo = 0;
   if constexpr (YC) {
     xo = kc / a.cy;
     yo = kc - xo * a.cy;
   }
-  realx4 acc[kGwT][kGwT];
+  realx4 acc[TI][TJ];
 #pragma unroll
-  for (int i = 0; i < kGwT; ++i)
+  for (int i = 0; i < TI; ++i)
 #pragma unroll
-    for (int j = 0; j < kGwT; ++j) acc[i][j] = realx4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < TJ; ++j) acc[i][j] = realx4{0.f, 0.f, 0.f, 0.f};
   constexpr int NS = 4;          // groups of four samples in flight: two steps of eight
-  const realx4 zero = {0.f, 0.f, 0.f, 0.f};
+  VI zi;
+  VJ zj;
+#pragma unroll
+  for (int i = 0; i < TI; ++i) zi[i] = 0.f;
+#pragma unroll
+  for (int j = 0; j < TJ; ++j) zj[j] = 0.f;
   for (int s = a.path_ptr[p]; s < a.path_ptr[p + 1]; ++s) {
     const cgtp_uvt_item it = a.items[s];
     const int n_t = __builtin_amdgcn_readfirstlane(it.t1 - it.t0);
     const int grow = __builtin_amdgcn_readfirstlane(it.out_row) * a.cout;
     for (int64_t n0 = n_begin; n0 < n_end; n0 += 4 * NS) {
-      realx4 av[NS], bv[NS];
+      VI av[NS];
+      VJ bv[NS];
       const real* xn[NS];
       const real* yn[NS];
       bool live[NS];
@@ -622,24 +637,24 @@ __global__ void __launch_bounds__(kWave) uvt_grad_w_small_kernel(const UvtGwDev 
         const int64_t nc = live[q] ? n : n_end - 1;
         xn[q] = a.x + nc * a.dx * a.cx + xo;
         yn[q] = a.y + nc * a.dy * (YC ? a.cy : 1) + yo;
-        bv[q] = *reinterpret_cast<const realx4*>(a.g + nc * a.dg * a.cout + grow + wc);
-        av[q] = zero;
+        bv[q] = *reinterpret_cast<const VJ*>(a.g + nc * a.dg * a.cout + grow + wc);
+        av[q] = zi;
       }
       for (int t0 = 0; t0 < n_t; t0 += 2) {          // the segment's terms, two at a time (most have one or two)
         const bool two = t0 + 1 < n_t;
         const int ta0 = a.ta[it.t0 + t0] * a.cx, tb0 = a.tb[it.t0 + t0] * (YC ? a.cy : 1);
         const int ta1 = a.ta[it.t0 + (two ? t0 + 1 : t0)] * a.cx, tb1 = a.tb[it.t0 + (two ? t0 + 1 : t0)] * (YC ? a.cy : 1);
         const real c0 = a.tc[it.t0 + t0], c1 = two ? a.tc[it.t0 + t0 + 1] : real(0);
-        realx4 v4[NS][2];
+        VI v4[NS][2];
         real v1[NS][2];
 #pragma unroll
         for (int q = 0; q < NS; ++q) {
           if constexpr (YC) {
-            v1[q][0] = xn[q][ta0]; v4[q][0] = *reinterpret_cast<const realx4*>(yn[q] + tb0);
-            v1[q][1] = xn[q][ta1]; v4[q][1] = *reinterpret_cast<const realx4*>(yn[q] + tb1);
+            v1[q][0] = xn[q][ta0]; v4[q][0] = *reinterpret_cast<const VI*>(yn[q] + tb0);
+            v1[q][1] = xn[q][ta1]; v4[q][1] = *reinterpret_cast<const VI*>(yn[q] + tb1);
           } else {
-            v4[q][0] = *reinterpret_cast<const realx4*>(xn[q] + ta0); v1[q][0] = yn[q][tb0];
-            v4[q][1] = *reinterpret_cast<const realx4*>(xn[q] + ta1); v1[q][1] = yn[q][tb1];
+            v4[q][0] = *reinterpret_cast<const VI*>(xn[q] + ta0); v1[q][0] = yn[q][tb0];
+            v4[q][1] = *reinterpret_cast<const VI*>(xn[q] + ta1); v1[q][1] = yn[q][tb1];
           }
         }
 #pragma unroll
@@ -650,27 +665,27 @@ __global__ void __launch_bounds__(kWave) uvt_grad_w_small_kernel(const UvtGwDev 
       }
 #pragma unroll
       for (int q = 0; q < NS; ++q) {
-        const realx4 af = (live[q] && kok) ? av[q] : zero;
-        const realx4 bf = (live[q] && wok) ? bv[q] : zero;
+        const VI af = (live[q] && kok) ? av[q] : zi;
+        const VJ bf = (live[q] && wok) ? bv[q] : zj;
 #pragma unroll
-        for (int ti = 0; ti < kGwT; ++ti)
+        for (int ti = 0; ti < TI; ++ti)
 #pragma unroll
-          for (int tj = 0; tj < kGwT; ++tj) acc[ti][tj] = mfma16(af[ti], bf[tj], acc[ti][tj], 0, 0, 0);
+          for (int tj = 0; tj < TJ; ++tj) acc[ti][tj] = mfma16(af[ti], bf[tj], acc[ti][tj], 0, 0, 0);
       }
     }
   }
   real* out = a.part + ((int64_t)blockIdx.x * a.n_paths + p) * a.K * a.cout;
   if (wok) {
 #pragma unroll
-    for (int i = 0; i < kGwT; ++i)
+    for (int i = 0; i < TI; ++i)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const int k = 4 * acc_row(g4, e) + i;
+        const int k = TI * acc_row(g4, e) + i;
         if (k < a.K) {
-          realx4 v;
+          VJ v;
 #pragma unroll
-          for (int j = 0; j < kGwT; ++j) v[j] = acc[i][j][e];
-          *reinterpret_cast<realx4*>(out + (int64_t)k * a.cout + 4 * r) = v;
+          for (int j = 0; j < TJ; ++j) v[j] = acc[i][j][e];
+          *reinterpret_cast<VJ*>(out + (int64_t)k * a.cout + TJ * r) = v;
         }
       }
   }
@@ -1115,8 +1130,13 @@ int grad_w(const cgtp_uvt_gw_args* a, void* stream) {
   if (zblocks > 65535 || a->n_paths > 65535) return CGTP_ERR_SHAPE;
   dim3 grid((unsigned)n_chunks, (unsigned)a->n_paths, (unsigned)zblocks);
   if (uvt_gw_small(K, a->cout)) {
-    hipLaunchKernelGGL(a->cy > 0 ? uvt_grad_w_small_kernel<true> : uvt_grad_w_small_kernel<false>,
-                       dim3((unsigned)n_chunks, (unsigned)a->n_paths), dim3(kWave), 0, st, d);
+    const bool yc = a->cy > 0, ki = K <= 32, wj = a->cout <= 32;      // two channels a lane where 32 cover the axis
+    void (*small)(const UvtGwDev) =
+        ki ? (wj ? (yc ? uvt_grad_w_small_kernel<true, 2, 2> : uvt_grad_w_small_kernel<false, 2, 2>)
+                 : (yc ? uvt_grad_w_small_kernel<true, 2, 4> : uvt_grad_w_small_kernel<false, 2, 4>))
+           : (wj ? (yc ? uvt_grad_w_small_kernel<true, 4, 2> : uvt_grad_w_small_kernel<false, 4, 2>)
+                 : (yc ? uvt_grad_w_small_kernel<true, 4, 4> : uvt_grad_w_small_kernel<false, 4, 4>));
+    hipLaunchKernelGGL(small, dim3((unsigned)n_chunks, (unsigned)a->n_paths), dim3(kWave), 0, st, d);
     if (hipGetLastError() != hipSuccess) return CGTP_ERR_LAUNCH;
     hipLaunchKernelGGL(uvt_gw_reduce_kernel, dim3((unsigned)((n_out / 4 + kGwReduceCols - 1) / kGwReduceCols)),
                        dim3(kGwReduceCols * kGwReduceSlices), 0, st, (const real*)a->workspace, (real*)a->gw, n_chunks,

@@ -125,10 +125,12 @@ def test_bf16_shared_weight_runs_on_the_matrix_core_kernels(device, irr, cin, co
         assert_close(a.float(), b, tol=1e-2, what=f"bf16 {irr} {name}")
 
 
-@pytest.mark.parametrize("cin,cout,n", [(64, 64, 20003), (48, 24, 1001), (16, 64, 70001), (64, 8, 31)])
+@pytest.mark.parametrize("cin,cout,n", [(64, 64, 20003), (48, 24, 1001), (16, 64, 70001), (64, 8, 31), (32, 32, 4099),
+                                        (8, 24, 515)])
 def test_weight_gradient_of_weights_up_to_64_by_64(device, cin, cout, n):
     """fp32 shared weights of at most 64 x 64: the weight gradient has a wavefront per (path, chunk of samples) that keeps
-    the whole block in its registers.  Sample counts that leave a ragged last chunk (and a last group of fewer than
+    the whole block in its registers (four channels a lane along an axis of up to 64 channels, two along one of up
+    to 32: all four combinations).  Sample counts that leave a ragged last chunk (and a last group of fewer than
     four samples) and that make the chunks 32, 64 and 256 samples long; sums over up to 70 001 samples in fp32 are
     compared norm-wise, with the fp32 restatement beside them."""
     from equitorch_amd.nn import IrrepsLinear
