@@ -75,3 +75,43 @@ def test_other_tables_do_not_match():
     assert kernels.uvu_config_of(info) == -1 and kernels.uv_config_of(info) == -1
     # same dims as sh2 but other parities: entries differ
     assert kernels.uv_config_of(_infos("0e+1e+2e")) == -1
+
+
+def test_exactness_of_a_match_decides_what_float64_operands_run_on():
+    """``Cfg.exact``: every coefficient equals the compiled one times its path's factor to the last bit.  The default
+    tables are exact; a subset of the paths of a larger table with another normalisation matches only to an fp32
+    rounding (ratios within 1e-6 of each other, not equal), which float64 operands are not given."""
+    from equitorch_amd.irreps import Irreps
+    from equitorch_amd.ops import kernels
+    from equitorch_amd.utils import tp_infos
+    assert kernels.uvu_config_of(_infos(SH2)).exact and kernels.uvu_config_of(_infos(SH3)).exact
+    sub = kernels.uvu_config_of(tp_infos(Irreps(SH3), Irreps(SH2), Irreps(SH2))[0])
+    assert sub >= 0 and sub.w_rows is not None and sub.path_scale is not None and not sub.exact
+    x = torch.zeros(4, 9, 8, dtype=torch.float64)
+    assert not kernels.uvu_launchable(sub, x, torch.zeros(4, 9, dtype=torch.float64), torch.zeros(4, 13, 8, dtype=torch.float64))
+
+
+def test_host_logic_for_tables_the_reference_builder_leaves_incomplete():
+    """``sparse_product_info`` (``equitorch/utils/_structs.py:105-123``) shifts its segments when the first output row
+    has no entry: the general contraction's spec keeps what the segments reach, the streaming kernels' walk lists the
+    weight paths it never visits, and a weight without elements is a weight per sample of an empty batch."""
+    from equitorch_amd.nn import SO2Linear
+    from equitorch_amd.nn.functional import _irreps_gemm as G, _psw
+    from equitorch_amd.nn.functional._tri import spec_from_product_info
+    from equitorch_amd.nn.linears import _view_weight
+    mod = SO2Linear("1o+1e", "2e+0e", 4, 4, internal_weights=False, feature_mode="uu")
+    info = mod.info_forward
+    spec = spec_from_product_info(info, mod.irreps_in.dim, mod.num_weights)
+    reached, entries = int(info.seg_out[-1]), info.scale.shape[0]
+    assert reached < entries and spec.out_idx.shape[0] == reached == spec.idx[0].shape[0] == spec.coef.shape[0]
+    mod = SO2Linear("0e", "1o+2e", 4, 4, internal_weights=False, feature_mode="uv")
+    plan = G.plan_of_product_info(mod.info_forward, 1, mod.num_weights)
+    assert len(plan.paths) == 1 and plan.n_paths == 2                      # the second weight is used by no row
+    table = _psw.PswTable([p.o0 for p in plan.paths], [p.i0 for p in plan.paths], [0] * len(plan.paths),
+                          [p.w for p in plan.paths], [p.scale for p in plan.paths], 1, 1, plan.out_size, plan.n_paths, "cpu")
+    assert table.unwalked_paths == [1]
+    empty = SO2Linear("0e", "2e+0e", 4, 4, internal_weights=False, feature_mode="uv")
+    assert not G.plan_of_product_info(empty.info_forward, 1, empty.num_weights).paths
+    assert _view_weight(torch.zeros(0, 3, 4, 5), (3, 4, 5), 60).shape == (0, 3, 4, 5)
+    assert _view_weight(torch.zeros(60), (3, 4, 5), 60).shape == (3, 4, 5)
+    assert _view_weight(torch.zeros(2, 60), (3, 4, 5), 60).shape == (2, 3, 4, 5)
