@@ -163,7 +163,12 @@ constexpr int kUvtTerms = 8;
 // ring of four would be half padding (twice the LDS per sample, twice the matrix instructions), and at 64 the 32
 // registers it saves let a second workgroup onto the compute unit, which covers the latency better than the deeper
 // ring did (64 -> 64 channels, lmax = 3, 32768 samples: forward 415 -> 355 us, grad y 734 -> 561 us).
-__host__ __device__ constexpr int uvt_kbi(int64_t K) { return K <= 64 ? 2 : 4; }
+// Past 64 channels the ring is also two where four would pad k by two or three blocks (80, 96, 144, 160 ... channels:
+// 96 -> 96, lmax = 2, 32768 samples: forward 475 -> 348 us, grad y 586 -> 346 us).
+__host__ __device__ constexpr int uvt_kbi(int64_t K) {
+  const int64_t kb = (K + 15) / 16;
+  return K <= 64 || kb % 4 == 1 || kb % 4 == 2 ? 2 : 4;
+}
 template <bool YC>
 struct UvtTerms {
   const real* xr[kUvtTerms];

@@ -281,7 +281,8 @@ def test_table_driven_matrix_core_entry_points_validate_on_the_host():
     assert L.cgtp_uvt_packed_elems(23, 128, 128) == 23 * 8 * 8 * 256
     assert L.cgtp_uvt_packed_elems(2, 20, 12) == 2 * 2 * 4 * 256            # padded to whole ring turns / 4 blocks
     assert L.cgtp_uvt_packed_elems(2, 40, 12) == 2 * 4 * 4 * 256            # three blocks of k: two turns of a ring of two
-    assert L.cgtp_uvt_packed_elems(2, 72, 12) == 2 * 8 * 4 * 256            # a ring of four past 64 contracted channels
+    assert L.cgtp_uvt_packed_elems(2, 72, 12) == 2 * 6 * 4 * 256            # five blocks of k: three turns of a ring of two
+    assert L.cgtp_uvt_packed_elems(2, 104, 12) == 2 * 8 * 4 * 256           # seven blocks: two turns of a ring of four
     assert L.cgtp_uvt_chunk(32768, 16, 16, 16, 32, 0, 128, _lib.F32) == 2
     assert L.cgtp_uvt_chunk(32768, 9, 9, 9, 4, 8, 16, _lib.F32) == 2         # K = 4 x 8
     assert L.cgtp_uvt_chunk(32768, 9, 9, 9, 8, 8, 16, _lib.F64) == 2         # K = 64

@@ -29,6 +29,9 @@ U1V_CASES = [  # irreps (out, in1, in2), C_in, C_out, N, module options
     (("0e+1o", _sh(1), _sh(1)), 16, 256, 530, {}),              # output channels over two workgroups
     ((_sh(2),) * 3, 8, 8, 515, {}),                             # a fragment ring of two blocks, half of it padding
     ((_sh(3), _sh(2), _sh(3)), 16, 40, 333, {}),                # ... one block of k, output channels 2 blocks + 8
+    ((_sh(2),) * 3, 96, 80, 300, {}),                           # six blocks of k: a ring of two past 64 channels
+    ((_sh(1), _sh(2), _sh(1)), 160, 96, 130, {}),               # ten blocks
+    ((_sh(2),) * 3, 112, 48, 77, {}),                           # seven blocks: padded to eight, a ring of four
 ]
 
 
