@@ -792,15 +792,20 @@ constexpr int kGyWB = sizeof(real) == 8 ? 1 : 2;   // blocks of 16 output channe
 constexpr int kGyWaves = 8;
 // kGyRing (template argument): blocks of 16 k in flight = uvt_kbi(K), the packing pads k to whole multiples
 
-template <int kGyRing>
+// kGyHalves: sets of 16 samples per workgroup (1 or 2).  With two, a wavefront multiplies every weight fragment with
+// the rows of both sets (two accumulator sets), which halves the requests to the L2 per matrix instruction — the
+// rate of those requests, not the matrix pipeline, is what bounds this kernel.  Taken where the rows of 32 samples
+// fit the LDS and the batch still fills the chip.
+template <int kGyRing, int kGyHalves>
 __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGyDev a) {
+  constexpr int SW = 16 * kGyHalves;
   extern __shared__ __align__(16) unsigned char smem[];
   real* xs = reinterpret_cast<real*>(smem);
-  real* part = xs + (size_t)16 * a.px;                       // [wavefront][sample][b]
-  const int64_t nb0 = (int64_t)blockIdx.x * 16;
+  real* part = xs + (size_t)SW * a.px;                       // [wavefront][sample][b]
+  const int64_t nb0 = (int64_t)blockIdx.x * SW;
   {
     const int kx4 = a.kx / 4, per_sample = a.dx * kx4;
-    for (int i = threadIdx.x; i < 16 * per_sample; i += blockDim.x) {
+    for (int i = threadIdx.x; i < SW * per_sample; i += blockDim.x) {
       const int s = i / per_sample, rem = i - s * per_sample, row = rem / kx4, c4 = rem - row * kx4;
       const int64_t n = nb0 + s;
       realx4 v = {0.f, 0.f, 0.f, 0.f};
@@ -808,28 +813,35 @@ __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGy
       *reinterpret_cast<realx4*>(xs + (size_t)s * a.px + row * a.kx + c4 * 4) = v;
     }
   }
-  for (int i = threadIdx.x; i < kGyWaves * 16 * a.dy; i += blockDim.x) part[i] = 0.f;
-  const UvtTables tab = uvt_stage_tables(a, reinterpret_cast<unsigned char*>(part + kGyWaves * 16 * a.dy));
+  for (int i = threadIdx.x; i < kGyWaves * SW * a.dy; i += blockDim.x) part[i] = 0.f;
+  const UvtTables tab = uvt_stage_tables(a, reinterpret_cast<unsigned char*>(part + kGyWaves * SW * a.dy));
   __syncthreads();
 
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), r = lane & 15, q = lane >> 4;
   const int wg = wave & (a.wgroups - 1), sg = wave / a.wgroups, sgroups = kGyWaves / a.wgroups;
-  const int64_t n = nb0 + r;
   // samples past the end are staged as zeros (Z = 0); their rows of g are read from the last sample
-  const real* gn = a.g + (n < a.n_rows ? n : a.n_rows - 1) * a.dg * a.cout;
-  const real* xl = xs + (size_t)r * a.px + 4 * q;
-  real* mine = part + (size_t)(wave * 16 + r) * a.dy;
+  const real* gn[kGyHalves];
+  real* mine[kGyHalves];
+#pragma unroll
+  for (int h = 0; h < kGyHalves; ++h) {
+    const int64_t n = nb0 + 16 * h + r;
+    gn[h] = a.g + (n < a.n_rows ? n : a.n_rows - 1) * a.dg * a.cout;
+    mine[h] = part + (size_t)(wave * SW + 16 * h + r) * a.dy;
+  }
+  const real* xl = xs + (size_t)r * a.px + 4 * q;    // set h: 16 h px further
+  const size_t xhalf = (size_t)16 * a.px;
   const realx4 zero = {0.f, 0.f, 0.f, 0.f};
 
   // The passes of this wavefront — (segment, block of 32 output channels) — form one sequence; the weight fragments
   // and the rows of x run kGyRing blocks of 16 k ahead of the matrix instructions, across the ends of the passes
   // (a weight fragment comes from the L2 in more cycles than one block's eight matrix instructions take).
   const int64_t kstride = (int64_t)a.wbp * 256;
-  realx4 A[kGyRing][kGyWB], B[kGyRing];
-  auto load = [&](const real* wbase, const real* xrow, int kb, realx4 (&Aj)[kGyWB], realx4& Bj) __attribute__((always_inline)) {
+  realx4 A[kGyRing][kGyWB], B[kGyRing][kGyHalves];
+  auto load = [&](const real* wbase, const real* xrow, int kb, realx4 (&Aj)[kGyWB], realx4 (&Bj)[kGyHalves]) __attribute__((always_inline)) {
 #pragma unroll
     for (int wb = 0; wb < kGyWB; ++wb) Aj[wb] = *reinterpret_cast<const realx4*>(wbase + kb * kstride + wb * 256);
-    Bj = *reinterpret_cast<const realx4*>(xrow + kb * 16);
+#pragma unroll
+    for (int h = 0; h < kGyHalves; ++h) Bj[h] = *reinterpret_cast<const realx4*>(xrow + h * xhalf + kb * 16);
   };
   auto wbase_of = [&](const cgtp_uvt_item& it, int wc) __attribute__((always_inline)) {
     return a.wp + ((int64_t)it.p * a.kblocks * a.wbp + wc * kGyWB) * 256 + lane * 4;
@@ -875,20 +887,25 @@ __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGy
       wcol[wb] = wok[wb] ? w : 0;
     }
     // rows of g of the terms, requested before the matrix instructions: slots in pairs up to the segment's term count
-    realx4 gv[kUvtTerms][kGyWB];
+    realx4 gv[kGyHalves][kUvtTerms][kGyWB];
 #pragma unroll
     for (int h = 0; h < kUvtTerms; h += 2) {
       if (h == 0 || n_t > h) {
 #pragma unroll
         for (int k = h; k < h + 2; ++k)
 #pragma unroll
-          for (int wb = 0; wb < kGyWB; ++wb) gv[k][wb] = *reinterpret_cast<const realx4*>(gn + mrow[k] + wcol[wb]);
+          for (int hs = 0; hs < kGyHalves; ++hs)
+#pragma unroll
+            for (int wb = 0; wb < kGyWB; ++wb)
+              gv[hs][k][wb] = *reinterpret_cast<const realx4*>(gn[hs] + mrow[k] + wcol[wb]);
       }
     }
 
-    realx4 acc[kGyWB];
+    realx4 acc[kGyHalves][kGyWB];
 #pragma unroll
-    for (int wb = 0; wb < kGyWB; ++wb) acc[wb] = zero;
+    for (int hs = 0; hs < kGyHalves; ++hs)
+#pragma unroll
+      for (int wb = 0; wb < kGyWB; ++wb) acc[hs][wb] = zero;
     for (int kb = 0; kb < a.kblocks; kb += kGyRing) {
       const bool wrap = kb + kGyRing >= a.kblocks;   // the blocks requested now belong to the next pass
       const real* wnext = wrap ? wbase2 : wbase;
@@ -899,43 +916,53 @@ __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGy
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-          for (int wb = 0; wb < kGyWB; ++wb)
-            acc[wb] = mfma16(A[j][wb][i], B[j][i], acc[wb], 0, 0, 0);
+          for (int hs = 0; hs < kGyHalves; ++hs)
+#pragma unroll
+            for (int wb = 0; wb < kGyWB; ++wb)
+              acc[hs][wb] = mfma16(A[j][wb][i], B[j][hs][i], acc[hs][wb], 0, 0, 0);
         load(wnext, xnext, kbn + j, A[j], B[j]);
       }
     }
     // accumulator: lane (sample r, q) holds Z[n, 16 (wb0 + wb) + 4 q + e]
-    auto add_term = [&](const realx4 (&gt)[kGyWB], real coef, int b) __attribute__((always_inline)) {
+    auto add_term = [&](const realx4 (&gt)[kGyWB], const realx4 (&z)[kGyWB], real* to, real coef, int b) __attribute__((always_inline)) {
       real d = 0.f;
 #pragma unroll
       for (int wb = 0; wb < kGyWB; ++wb) {
         const realx4 gg = wok[wb] ? gt[wb] : zero;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) d += gg[e] * acc[wb][e];
+        for (int e = 0; e < 4; ++e) d += gg[e] * z[wb][e];
       }
       d += __shfl_xor(d, 16);
       d += __shfl_xor(d, 32);
-      if (q == 0) atomicAdd(mine + b, coef * d);   // LDS, this wavefront's own array: in program order
+      if (q == 0) atomicAdd(to + b, coef * d);   // LDS, this wavefront's own array: in program order
     };
 #pragma unroll
     for (int k = 0; k < kUvtTerms; ++k)
-      if (k < n_t) add_term(gv[k], c[k], brow[k]);
-    for (int t = it.t0 + kUvtTerms; t < it.t1; ++t) {   // longer segments (large irreps only)
-      realx4 gt[kGyWB];
-      const int m = __builtin_amdgcn_readfirstlane(tab.ta[t]) * a.cout;
+      if (k < n_t) {
 #pragma unroll
-      for (int wb = 0; wb < kGyWB; ++wb) gt[wb] = *reinterpret_cast<const realx4*>(gn + m + wcol[wb]);
-      add_term(gt, tab.tc[t], __builtin_amdgcn_readfirstlane(tab.tb[t]));
+        for (int hs = 0; hs < kGyHalves; ++hs) add_term(gv[hs][k], acc[hs], mine[hs], c[k], brow[k]);
+      }
+    for (int t = it.t0 + kUvtTerms; t < it.t1; ++t) {   // longer segments (large irreps only)
+      const int m = __builtin_amdgcn_readfirstlane(tab.ta[t]) * a.cout;
+      const int b = __builtin_amdgcn_readfirstlane(tab.tb[t]);
+      const real coef = tab.tc[t];
+#pragma unroll
+      for (int hs = 0; hs < kGyHalves; ++hs) {
+        realx4 gt[kGyWB];
+#pragma unroll
+        for (int wb = 0; wb < kGyWB; ++wb) gt[wb] = *reinterpret_cast<const realx4*>(gn[hs] + m + wcol[wb]);
+        add_term(gt, acc[hs], mine[hs], coef, b);
+      }
     }
     s = s2; wc = wc2; it = it2; wbase = wbase2; xrow = xrow2;
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < 16 * a.dy; i += blockDim.x) {
+  for (int i = threadIdx.x; i < SW * a.dy; i += blockDim.x) {
     const int64_t ni = nb0 + i / a.dy;
     if (ni < a.n_rows) {
       real sum = 0.f;
 #pragma unroll
-      for (int w = 0; w < kGyWaves; ++w) sum += part[w * 16 * a.dy + i];
+      for (int w = 0; w < kGyWaves; ++w) sum += part[w * SW * a.dy + i];
       a.gy[nb0 * a.dy + i] = sum;
     }
   }
@@ -1184,14 +1211,28 @@ int grad_y(const cgtp_uvt_gy_args* a, void* stream) {
   d.wbp = round_up((a->cout + 15) / 16, 4);
   d.wchunks = (a->cout + 16 * kGyWB - 1) / (16 * kGyWB);
   d.wgroups = d.wchunks >= 4 ? 4 : d.wchunks >= 2 ? 2 : 1;
-  const int64_t lds = ((int64_t)16 * d.px + (int64_t)kGyWaves * 16 * a->dy) * (int64_t)sizeof(real) +
-                      (int64_t)a->n_items * 32 + (int64_t)a->n_terms * kTermBytes + 16;
+  auto lds_of = [&](int halves) {
+    return ((int64_t)16 * halves * d.px + (int64_t)kGyWaves * 16 * halves * a->dy) * (int64_t)sizeof(real) +
+           (int64_t)a->n_items * 32 + (int64_t)a->n_terms * kTermBytes + 16;
+  };
+  // Two sets of 16 samples per workgroup: single precision (the doubles' registers do not take a second set of g
+  // rows), the rows of 32 samples fit the LDS, at least two workgroups per compute unit remain — and the kernel with
+  // one set would not have two workgroups on a compute unit to gain from: a ring of four (151 registers), or walk
+  // tables, which every workgroup copies, a third as large as its rows of x.  lmax = 2, 32768 samples, 128 -> 128
+  // channels: 590 -> 518 us; lmax = 4, 16384 samples, 32 -> 32: 463 -> 372 us; where two workgroups of the one-set
+  // kernel fit, they are faster (64 -> 64, lmax = 3: 563 against 616 us).
+  const int64_t table_bytes = (int64_t)a->n_items * 32 + (int64_t)a->n_terms * kTermBytes;
+  const bool one_wg_anyway = ring == 4 || 3 * table_bytes >= (int64_t)16 * d.px * (int64_t)sizeof(real);
+  const int halves = sizeof(real) == 4 && one_wg_anyway && lds_of(2) <= kLdsBytes && a->n_rows >= 32 * 512 ? 2 : 1;
+  const int64_t lds = lds_of(halves);
   if (lds > kLdsBytes) return CGTP_ERR_LDS;
   if (a->n_rows == 0) return CGTP_OK;
-  void (*fn)(const UvtGyDev) = ring == 4 ? uvt_grad_y_kernel<4> : uvt_grad_y_kernel<2>;
+  void (*fn)(const UvtGyDev) = halves == 2 ? (ring == 4 ? uvt_grad_y_kernel<4, 2> : uvt_grad_y_kernel<2, 2>)
+                                           : (ring == 4 ? uvt_grad_y_kernel<4, 1> : uvt_grad_y_kernel<2, 1>);
   if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
     return CGTP_ERR_LDS;
-  hipLaunchKernelGGL(fn, dim3((unsigned)((a->n_rows + 15) / 16)), dim3(kGyWaves * kWave), (size_t)lds, (hipStream_t)stream, d);
+  const int64_t per_wg = 16 * halves;
+  hipLaunchKernelGGL(fn, dim3((unsigned)((a->n_rows + per_wg - 1) / per_wg)), dim3(kGyWaves * kWave), (size_t)lds, (hipStream_t)stream, d);
   return hipGetLastError() == hipSuccess ? CGTP_OK : CGTP_ERR_LAUNCH;
 }
 
