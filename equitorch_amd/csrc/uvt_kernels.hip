@@ -79,6 +79,7 @@ struct UvtDev {
   int kblocks;   // K / 16 (K padded to 16)
   int wbp;       // blocks of 16 output channels, rounded up to a multiple of 4 (as packed)
   int sb_log2;   // log2 of the 16-sample blocks per workgroup
+  int ns;        // sets of 16 samples per wavefront (1 or 2)
   int wgroups;   // wavefronts of a sample block that split the output channels (power of two)
   int igroups;   // groups of items (whole output rows) the remaining wavefronts of a sample block split
   int zero_floats;  // zeros in LDS that the unused term slots of an item read
@@ -249,10 +250,15 @@ __device__ __forceinline__ realx4 uvt_mix_tail(const UvtDev& a, const UvtTables&
 // needs besides its operands is wave-uniform (scalar registers).  A wavefront issues one instruction every four
 // cycles, a matrix instruction keeps its pipeline busy for 32: with 4 WB matrix instructions per block next to
 // about 50 vector and LDS instructions, two wavefronts per SIMD keep the matrix pipeline fed when WB >= 2.
-template <bool YC, int WB, int KBI>
+// NS = 2 (y without channels, WB = KBI = 4 only): the wavefront multiplies each weight fragment with the mixed rows
+// of two sets of 16 samples (two accumulator sets), which halves the requests to the L2 per matrix instruction —
+// at 128 channels the rate of those requests bounds the kernel, not the matrix pipeline.  Taken where the rows of
+// 32 samples fit the LDS.
+template <bool YC, int WB, int KBI, int NS = 1>
 __global__ void __launch_bounds__(kUvtMaxGroups* kWave) uvt_apply_kernel(const UvtDev a) {
+  static_assert(NS == 1 || (NS == 2 && !YC), "two sample sets: y without channels");
   extern __shared__ __align__(16) unsigned char smem[];
-  const int sb_count = 1 << a.sb_log2;
+  const int sb_count = (1 << a.sb_log2) * NS;
   real* xs = reinterpret_cast<real*>(smem);
   real* ys = xs + (size_t)(16 * sb_count) * a.px;
   const int64_t nb0 = (int64_t)blockIdx.x * (16 * sb_count);
@@ -272,7 +278,7 @@ __global__ void __launch_bounds__(kUvtMaxGroups* kWave) uvt_apply_kernel(const U
   __syncthreads();
 
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), r = lane & 15, g = lane >> 4;
-  const int sb = wave & (sb_count - 1), rest = wave >> a.sb_log2;
+  const int sb = (wave & ((1 << a.sb_log2) - 1)) * NS, rest = wave >> a.sb_log2;   // first set of this wavefront
   const int wg = rest & (a.wgroups - 1), ig = rest / a.wgroups;
   const int wb0 = (blockIdx.y * a.wgroups + wg) * WB;
   if (wb0 * 16 >= a.cout) return;
@@ -290,12 +296,20 @@ __global__ void __launch_bounds__(kUvtMaxGroups* kWave) uvt_apply_kernel(const U
     return a.wp + ((int64_t)it.p * a.kblocks * a.wbp + wb0) * 256 + lane * 4;
   };
   realx4 acc[WB], A[KBI][WB];
+  // second set of samples (NS = 2): rows 16 further in the staged tiles
+  realx4 acc2[NS == 2 ? WB : 1];
+  const int x2 = 16 * a.px;
+  const real* yl2 = yl + (size_t)16 * a.py;
   auto load_a = [&](const real* base, int kb, realx4 (&Aj)[WB]) __attribute__((always_inline)) {
 #pragma unroll
     for (int wb = 0; wb < WB; ++wb) Aj[wb] = *reinterpret_cast<const realx4*>(base + kb * kstride + wb * 256);
   };
 #pragma unroll
   for (int wb = 0; wb < WB; ++wb) acc[wb] = realx4{0.f, 0.f, 0.f, 0.f};
+  if constexpr (NS == 2) {
+#pragma unroll
+    for (int wb = 0; wb < WB; ++wb) acc2[wb] = realx4{0.f, 0.f, 0.f, 0.f};
+  }
 
   cgtp_uvt_item it = uvt_item_at(tab, j);
   const real* base = wbase_of(it);
@@ -313,22 +327,59 @@ __global__ void __launch_bounds__(kUvtMaxGroups* kWave) uvt_apply_kernel(const U
       if (tail) b += uvt_mix_tail<YC>(a, tab, it, kb, xl, yl, g, lut_g);
       return b;
     };
+    // second set: its factors coef * y[n + 16, b]; the rows of x are those of the first set x2 further (slots past
+    // the end stay on the block of zeros)
+    real s2[NS == 2 ? kUvtTerms : 1];
+    int xo[NS == 2 ? kUvtTerms : 1];
+    if constexpr (NS == 2) {
+#pragma unroll
+      for (int k = 0; k < kUvtTerms; ++k) {
+        const bool live = k < T.n;
+        const int t = live ? it.t0 + k : it.t0;
+        const int ib = __builtin_amdgcn_readfirstlane(tab.tb[t]);
+        s2[k] = live ? tab.tc[t] * yl2[ib] : 0.f;
+        xo[k] = live ? x2 : 0;
+      }
+    }
+    auto mix2 = [&](int kb) __attribute__((always_inline)) {
+      realx4 b = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (NS == 2) {
+#pragma unroll
+        for (int half = 0; half < kUvtTerms; half += 2) {
+          if (half == 0 || T.n > half) {
+#pragma unroll
+            for (int k = half; k < half + 2; ++k) b += s2[k] * *reinterpret_cast<const realx4*>(T.xr[k] + xo[k] + kb * 16);
+          }
+        }
+        if (tail) b += uvt_mix_tail<YC>(a, tab, it, kb, xl + x2, yl2, g, lut_g);
+      }
+      return b;
+    };
     const bool first = it.flags & kUvtFirst;
 #pragma unroll
     for (int wb = 0; wb < WB; ++wb) acc[wb] = first ? realx4{0.f, 0.f, 0.f, 0.f} : acc[wb];
+    if constexpr (NS == 2) {
+#pragma unroll
+      for (int wb = 0; wb < WB; ++wb) acc2[wb] = first ? realx4{0.f, 0.f, 0.f, 0.f} : acc2[wb];
+    }
     realx4 Bc = mix(0);
+    realx4 Bc2 = mix2(0);
     for (int kb = 0; kb < a.kblocks; kb += KBI) {
       const bool wrap = kb + KBI >= a.kblocks;        // the fragments requested now belong to the next item
       const real* wnext = wrap ? base2 : base;
       const int kbn = wrap ? 0 : kb + KBI;
 #pragma unroll
       for (int jj = 0; jj < KBI; ++jj) {
-        const realx4 Bn = mix((jj + 1 < KBI || !wrap) ? kb + jj + 1 : kb + jj);
+        const int kb_next = (jj + 1 < KBI || !wrap) ? kb + jj + 1 : kb + jj;
+        const realx4 Bn = mix(kb_next);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-          for (int wb = 0; wb < WB; ++wb)
+          for (int wb = 0; wb < WB; ++wb) {
             acc[wb] = mfma16(A[jj][wb][i], Bc[i], acc[wb], 0, 0, 0);
+            if constexpr (NS == 2) acc2[wb] = mfma16(A[jj][wb][i], Bc2[i], acc2[wb], 0, 0, 0);
+          }
+        if constexpr (NS == 2) Bc2 = mix2(kb_next);
         load_a(wnext, kbn + jj, A[jj]);
         Bc = Bn;
       }
@@ -341,6 +392,16 @@ __global__ void __launch_bounds__(kUvtMaxGroups* kWave) uvt_apply_kernel(const U
         for (int wb = 0; wb < WB; ++wb) {
           const int w = (wb0 + wb) * 16 + 4 * g;
           if (w < a.cout) *reinterpret_cast<realx4*>(orow + w) = acc[wb];
+        }
+      }
+      if constexpr (NS == 2) {
+        if (n + 16 < a.n_rows) {
+          real* orow = a.out + ((n + 16) * a.dout + it.out_row) * a.cout;
+#pragma unroll
+          for (int wb = 0; wb < WB; ++wb) {
+            const int w = (wb0 + wb) * 16 + 4 * g;
+            if (w < a.cout) *reinterpret_cast<realx4*>(orow + w) = acc2[wb];
+          }
         }
       }
     }
@@ -970,6 +1031,8 @@ __global__ void __launch_bounds__(kGyWaves* kWave) uvt_grad_y_kernel(const UvtGy
 
 struct UvtPlan {
   int wb, kbi, yc;
+  bool two_sets_ok;
+  int64_t per_block, fixed;
   int64_t lds;
   dim3 grid;
   unsigned threads;
@@ -1016,7 +1079,12 @@ static int uvt_shape(int64_t n_rows, int dx, int dy, int dout, int cx, int cy, i
   while ((wgroups * igroups) << (sb_log2 + 1) <= kUvtMaxGroups &&
          (per_block << (sb_log2 + 1)) + fixed <= kLdsBytes / 2 - kUvtTableRoom && (blocks16 >> (sb_log2 + 1)) >= 512)
     ++sb_log2;
-  d.sb_log2 = sb_log2; d.wgroups = wgroups; d.igroups = igroups;
+  // Two sets of samples per wavefront: the widest form of the kernel only (single precision, y without channels, 64
+  // output channels per wavefront, a ring of four: one workgroup per compute unit anyway), where two workgroups per
+  // compute unit remain in the batch; uvt_plan() takes it if the rows of 32 samples fit the LDS beside the tables.
+  plan->two_sets_ok = sizeof(real) == 4 && !yc && wb == 4 && kbi == 4 && sb_log2 == 0 && blocks16 / 2 >= 512;
+  plan->per_block = per_block; plan->fixed = fixed;
+  d.sb_log2 = sb_log2; d.ns = 1; d.wgroups = wgroups; d.igroups = igroups;
   plan->wb = wb; plan->kbi = kbi; plan->yc = yc;
   plan->lds = (per_block << sb_log2) + fixed;
   plan->threads = (unsigned)((wgroups * igroups) << sb_log2) * kWave;
@@ -1045,7 +1113,13 @@ static int uvt_plan(const cgtp_uvt_args* a, UvtPlan* plan) {
   d.items = a->items; d.ta = a->term_a; d.tb = a->term_b; d.tc = (const real*)a->term_c;
   d.n_items = a->n_items; d.n_terms = a->n_terms;
   for (int i = 0; i <= kUvtMaxGroups; ++i) d.group_ptr[i] = i <= d.igroups ? a->group_ptr[i] : a->n_items;
-  plan->lds += ((int64_t)a->n_items * 32 + (int64_t)a->n_terms * kTermBytes + 15) / 16 * 16;
+  const int64_t tables = ((int64_t)a->n_items * 32 + (int64_t)a->n_terms * kTermBytes + 15) / 16 * 16;
+  if (plan->two_sets_ok && 2 * plan->per_block + plan->fixed + tables <= kLdsBytes) {
+    d.ns = 2;
+    plan->lds = 2 * plan->per_block + plan->fixed;
+    plan->grid.x = (unsigned)(((a->n_rows + 15) / 16 + 1) / 2);
+  }
+  plan->lds += tables;
   if (plan->lds > kLdsBytes) return CGTP_ERR_LDS;
   return CGTP_OK;
 }
@@ -1101,7 +1175,7 @@ int apply(const cgtp_uvt_args* a, void* stream) {
       fn = plan.wb == 2 ? uvt_apply_kernel<false, 2, 4> : uvt_apply_kernel<false, 1, 4>;
     }
 #ifndef CGTP_UVT_F64
-    if (plan.wb == 4) fn = plan.yc ? uvt_apply_kernel<true, 4, 4> : uvt_apply_kernel<false, 4, 4>;
+    if (plan.wb == 4) fn = plan.yc ? uvt_apply_kernel<true, 4, 4> : plan.dev.ns == 2 ? uvt_apply_kernel<false, 4, 4, 2> : uvt_apply_kernel<false, 4, 4>;
 #endif
   } else {
     if (plan.yc) {

@@ -170,17 +170,22 @@ def test_u1v_fp32_native_full_size(device):
     assert_close(gx[sub.to(device)], rgx, 1e-5, "full size grad_x", norm="max", fp32_ref=gx32)
 
 
-@pytest.mark.parametrize("lmax,cin,cout,n", [(2, 128, 128, 16384 + 21), (1, 128, 96, 32768), (4, 32, 32, 16384 + 5)])
-def test_u1v_fp32_second_operand_gradient_of_large_batches(device, lmax, cin, cout, n):
-    """From 16384 samples on, where the rows of 32 samples fit the LDS, the gradient of the second operand takes
-    workgroups of 32 samples (a weight fragment multiplied with two sets of 16); below that, and in every other test
+@pytest.mark.parametrize("irr1,lmax,cin,cout,n", [
+    (None, 2, 128, 128, 16384 + 21), (None, 1, 128, 96, 32768), (None, 1, 112, 128, 16384 + 16), (None, 4, 32, 32, 16384 + 5),
+    ("4e", 4, 128, 64, 16384 + 3),          # segments of more than eight terms: the part of a segment read from the tables
+])
+def test_u1v_fp32_large_batches_in_workgroups_of_32_samples(device, irr1, lmax, cin, cout, n):
+    """From 16384 samples on, where the rows of 32 samples fit the LDS, the gradient of the second operand and (with
+    a fragment ring of four and 64 or more output channels) the forward and the gradient of the first operand take
+    workgroups of 32 samples, a weight fragment multiplied with two sets of 16; below that, and in every other test
     of this file, 16.  Rows of a strided subset, the last samples of a ragged batch among them, against the oracle
-    (each row of the result depends on its own sample only)."""
+    (each row of the results depends on its own sample only)."""
     from equitorch_amd.nn import SO3Linear
     from equitorch_amd.utils._sh import spherical_harmonics
     irr = _sh(lmax)
-    mod = SO3Linear(irr, irr, irr, cin, cout, internal_weights=False, feature_mode="uv").to(device)
-    d = (lmax + 1) ** 2
+    irr1 = irr1 or irr
+    mod = SO3Linear(irr1, irr, irr1, cin, cout, internal_weights=False, feature_mode="uv").to(device)
+    d = mod.irreps_in1_dim
     g = torch.Generator().manual_seed(11 + lmax)
     x = torch.randn(n, d, cin, generator=g)
     y = spherical_harmonics(unit_vectors(n, g), lmax)
@@ -188,12 +193,17 @@ def test_u1v_fp32_second_operand_gradient_of_large_batches(device, lmax, cin, co
     ct = torch.randn(n, d, cout, generator=g)
     sub = torch.cat([torch.arange(3, n, 509), torch.arange(n - 40, n)])
     xd, yd, wd = (t.to(device) for t in (x, y, w))
-    yd.requires_grad_(True)
-    (gy,) = torch.autograd.grad(mod(xd, yd, wd), (yd,), ct.to(device))
-    T = ref_ops.dense_coupling(irr, irr, irr).float().double()
-    _, (_, rgy, _) = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x[sub], y[sub], w), ct[sub])
-    _, (_, gy32, _) = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x[sub], y[sub], w), ct[sub], dtype=torch.float32)
-    assert_close(gy[sub.to(device)], rgy, 1e-5, f"lmax {lmax} {cin}->{cout} N={n} grad_y", norm="max", fp32_ref=gy32)
+    xd.requires_grad_(True), yd.requires_grad_(True)
+    out = mod(xd, yd, wd)
+    gx, gy = torch.autograd.grad(out, (xd, yd), ct.to(device))
+    T = ref_ops.dense_coupling(irr1, irr1, irr).float().double()
+    ref_out, (rgx, rgy, _) = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x[sub], y[sub], w), ct[sub])
+    out32, (gx32, gy32, _) = ref_ops.dense_grads(ref_ops.dense_u1v, T, (x[sub], y[sub], w), ct[sub], dtype=torch.float32)
+    on = sub.to(device)
+    tag = f"{irr1} lmax {lmax} {cin}->{cout} N={n}"
+    assert_close(out[on], ref_out, 1e-5, tag + " out", norm="max", fp32_ref=out32)
+    assert_close(gx[on], rgx, 1e-5, tag + " grad_x", norm="max", fp32_ref=gx32)
+    assert_close(gy[on], rgy, 1e-5, tag + " grad_y", norm="max", fp32_ref=gy32)
 
 
 def test_u1v_fp32_full_size_properties(device):
